@@ -1,0 +1,146 @@
+/*
+ * vecops_hip.h - C ABI of libvecops_hip.so, the gfx950 (MI355X) kernels behind
+ * the vecops matmul path.
+ *
+ * Every entry point takes plain device pointers, element extents and element
+ * strides; none allocates, none synchronises: work is enqueued on `stream`
+ * (a hipStream_t passed as void*, null = the default stream) and the call
+ * returns.  The artifact DSOs that plug into vecops::runtime::Executable call
+ * these functions from their `run` callback and then wait for the stream,
+ * because the vecops kernel ABI is synchronous (runtime/CallAbi.h:7-16).
+ *
+ * Return values are VecopsStatusCode numbers (runtime/CallAbi.h:34-51):
+ * 0 ok, 1 invalid argument, 2 not applicable, 6 execution error.  A failing
+ * call leaves a message readable with vecops_hip_last_error() on the same
+ * host thread.
+ *
+ * dtype codes are VecopsDType numbers (runtime/CallAbi.h:62-91):
+ * 2 i8, 3 u8, 6 i32, 11 bf16, 12 f32.
+ */
+#ifndef VECOPS_HIP_H
+#define VECOPS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VECOPS_HIP_EXPORT __attribute__((visibility("default")))
+
+#define VECOPS_HIP_ABI_VERSION 1u
+
+/* One operand of a matmul: `data` addresses logical element zero in device
+ * memory.  rank 2 = [rows, cols]; rank 3 = [batch, rows, cols].  Strides are in
+ * elements; a zero batch stride broadcasts the operand over the batch
+ * (planning/families/ArchitectureFamily.h:393-421). */
+typedef struct VecopsHipOperand {
+  void* data;
+  uint32_t dtype;
+  uint32_t rank;
+  int64_t sizes[3];
+  int64_t strides[3];
+} VecopsHipOperand;
+
+/* How fp32 operands are multiplied (bf16 and int8 operands ignore it).
+ *   BF16: round each fp32 operand element to bf16 (nearest even) on load and use
+ *         the bf16 matrix cores - what vecops' x86 path does, which has no fp32
+ *         atom (matmul/details/kernel/amx/Atoms.h:51-60).
+ *   F32 : multiply in fp32 on the fp32 matrix cores - vecops' SME_F32F32 atom
+ *         (matmul/details/kernel/sme/Atoms.h:65-76). */
+typedef enum VecopsHipCompute { VECOPS_HIP_COMPUTE_BF16 = 0, VECOPS_HIP_COMPUTE_F32 = 1 } VecopsHipCompute;
+
+/* Kernel families of the GPU rule table (vecops_hip_select_kernel). */
+typedef enum VecopsHipKernelFamily {
+  VECOPS_HIP_FAMILY_NONE = 0,          /* empty problem: nothing to launch */
+  VECOPS_HIP_FAMILY_TILE_256 = 1,      /* 256x256 workgroup tile, MFMA */
+  VECOPS_HIP_FAMILY_TILE_128 = 2,      /* 128x128 workgroup tile, MFMA */
+  VECOPS_HIP_FAMILY_TILE_64 = 3,       /* 64x64 workgroup tile, MFMA */
+  VECOPS_HIP_FAMILY_SKINNY = 4,        /* wavefront split-K dot products */
+  VECOPS_HIP_FAMILY_ZERO_K = 5         /* K == 0: C = Cin or zeros */
+} VecopsHipKernelFamily;
+
+typedef struct VecopsHipPlan {
+  uint32_t family;     /* VecopsHipKernelFamily */
+  uint32_t split_k;    /* >= 1; > 1 needs workspace */
+  uint32_t vector_a;   /* 1 = 16-byte loads along K usable for A */
+  uint32_t vector_b;   /* 1 = 16-byte loads usable for B */
+  uint32_t b_layout;   /* 0 = K contiguous, 1 = N contiguous, 2 = generic */
+  uint32_t reserved;
+  uint64_t workspace_bytes;
+} VecopsHipPlan;
+
+/* ABI version of the loaded library. */
+VECOPS_HIP_EXPORT uint32_t vecops_hip_abi_version(void);
+
+/* Message of the last failing call on this host thread ("" if none). */
+VECOPS_HIP_EXPORT const char* vecops_hip_last_error(void);
+
+/* Number of HIP devices visible, or a negative number when the HIP runtime
+ * cannot be initialised. */
+VECOPS_HIP_EXPORT int32_t vecops_hip_device_count(void);
+
+/*
+ * GPU counterpart of vecops' runtime shape selector
+ * (matmul/details/kernel/RuntimeDispatch.h:24-83,
+ * src/MatmulRuntimeDispatch.cpp:12-32 and its call sites
+ * matmul/details/kernel/amx/Backend.h:2724-2757): a pure function of the
+ * operand metadata that chooses the kernel family, the split-K factor and the
+ * external workspace a call needs.  No device access.
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                 const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                 uint32_t compute, VecopsHipPlan* plan);
+
+/*
+ * C[..,M,N] = C_in + A[..,M,K] . B[..,N,K]^T  - replaces
+ * ops::Matmul<Config>::operator() (ops/Matmul.h:530-570) for
+ *   a,b bf16 -> c f32|bf16      (AMX_BF16F32)
+ *   a,b f32  -> c f32|bf16      (bf16 or fp32 compute, see VecopsHipCompute)
+ *   a,b i8   -> c i32           (AMX_I8I32<int8,int8>; accumulators wrap mod 2^32)
+ * c_in may be null (zero accumulator); otherwise it has c's dtype class (f32,
+ * bf16 or i32) and may alias c element for element.  K == 0 writes zeros or
+ * C_in; zero M, N or batch writes nothing (ops/Matmul.h:41-43).  Operand
+ * metadata is validated as planning/families/ArchitectureFamily.h:1590-1652
+ * does.  `workspace` must hold vecops_hip_plan_matmul(...).workspace_bytes.
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                            const VecopsHipOperand* c_in, const VecopsHipOperand* c, uint32_t compute,
+                                            void* workspace, uint64_t workspace_size, void* stream);
+
+/*
+ * c[i,j] = (float(acc[i,j]) * row_scales[i]) * column_scales[j],
+ * acc = sum_k a[i,k]*b[j,k] (+ correction[j]) in wrapping int32 - replaces
+ * ops::matmul with AMX_I8I32<int8,int8> and an output carrying
+ * RuntimePerRowColumnDequantizeTransform (matmul/Quantization.h:195-250); the
+ * optional correction row is the stride-0 int32 C-input of
+ * tests/ops/MatmulConversionTestCommon.h:1467-1472.  a is [M,K] with row
+ * stride lda, b is [N,K] with row stride ldb (both K contiguous), c is fp32
+ * [M,N] with row stride ldc.  Bit-exact.
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_i8_dequant(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                                                       const float* row_scales, const float* column_scales,
+                                                       const int32_t* correction, float* c, int64_t ldc, int64_t m,
+                                                       int64_t n, int64_t k, void* workspace, uint64_t workspace_size,
+                                                       void* stream);
+
+/* Workspace bytes vecops_hip_matmul_i8_dequant needs for these extents. */
+VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int64_t n, int64_t k);
+
+/*
+ * y[m,n] = bf16( sum_g scales[n,g] * sum_{k in group g} float(x[m,k]) * float(w[n,k]) )
+ * x bf16 [M,K] (row stride ldx), w int8 [N,K] (row stride ldw), scales fp32
+ * [N, K/group] dense, y bf16 [M,N] (row stride ldy); fp32 accumulation.
+ * No counterpart in vecops (it has no weight-only group-scaled matmul); this
+ * is the decode-shaped GEMV / skinny GEMM of the north-star workload.  m <= 16,
+ * k a multiple of `group`, group a multiple of 16.
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t ldx, const int8_t* w, int64_t ldw,
+                                                        const float* scales, void* y, int64_t ldy, int64_t m,
+                                                        int64_t n, int64_t k, int64_t group, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VECOPS_HIP_H */

@@ -1,0 +1,185 @@
+// TEST INFRASTRUCTURE ONLY.  A caller of the real vecops CPU matmul
+// (ops::matmul, include/vecops/ops/Matmul.h:530-586) exposed through a C ABI so
+// the Python tests can hold the oracle restatement and the gfx950 kernels
+// against the reference itself.  It is compiled by oracle/Makefile from the
+// vecops sources where they lie (never copied) into oracle/_ref/, and needs an
+// x86 host with AMX (the only x86 matmul backend,
+// include/vecops/matmul/details/kernel/Backend.h:57-72).
+//
+// Every tensor is passed with fully dynamic extents and strides (meta::Any), the
+// most general form the reference accepts (tests/ops/MatmulTest.cpp:220-279).
+#include <cpuid.h>
+#include <sys/syscall.h>
+#include <unistd.h>
+
+#include <cstdint>
+#include <vector>
+
+#include "vecops/matmul/Quantization.h"
+#include "vecops/ops/Matmul.h"
+
+using namespace vecops;
+using namespace vecops::meta;
+using namespace vecops::tensor;
+
+namespace {
+
+bool g_amx_ready = false;
+
+// tests/ops/MatmulTestArch.h:22-27: AMX tile data must be requested from the
+// kernel before the first tile instruction.
+bool enable_amx() {
+  if (g_amx_ready) return true;
+  unsigned eax = 0, ebx = 0, ecx = 0, edx = 0;
+  if (!__get_cpuid_count(7, 0, &eax, &ebx, &ecx, &edx)) return false;
+  const bool amx_bf16 = (edx >> 22) & 1, amx_tile = (edx >> 24) & 1, amx_int8 = (edx >> 25) & 1;
+  const bool avx512f = (ebx >> 16) & 1;
+  if (!(amx_bf16 && amx_tile && amx_int8 && avx512f)) return false;
+  if (syscall(SYS_arch_prctl, 0x1023, 18) != 0) return false;
+  g_amx_ready = true;
+  return true;
+}
+
+template <typename T>
+auto view2(T* p, int64_t rows, int64_t cols, int64_t s0, int64_t s1) {
+  return make_tensor(p, make_layout(make_shape(Any{rows}, Any{cols}), make_strides(Any{s0}, Any{s1})));
+}
+
+template <typename T>
+auto view3(T* p, int64_t batch, int64_t rows, int64_t cols, int64_t sb, int64_t s0, int64_t s1) {
+  return make_tensor(
+    p, make_layout(make_shape(Any{batch}, Any{rows}, Any{cols}), make_strides(Any{sb}, Any{s0}, Any{s1})));
+}
+
+template <typename Atom, typename TA, typename TB, typename TC>
+int run2(const TA* a, const TB* b, TC* c, const TC* cin, int64_t m, int64_t n, int64_t k, const int64_t* sa,
+         const int64_t* sb, const int64_t* sc) {
+  if (!enable_amx()) return -1;
+  auto at = view2(const_cast<TA*>(a), m, k, sa[0], sa[1]);
+  auto bt = view2(const_cast<TB*>(b), n, k, sb[0], sb[1]);
+  auto ct = view2(c, m, n, sc[0], sc[1]);
+  auto op = ops::matmul(ops::MatmulConfig<Atom>{});
+  if (cin) {
+    auto cit = view2(const_cast<TC*>(cin), m, n, sc[0], sc[1]);
+    const nint_t bytes = op.required_workspace(Any{m}, Any{n}, Any{k}, at, bt, cit, ct);
+    kernel::Workspace ws(bytes);
+    auto v = ws.view();
+    op(v, Any{m}, Any{n}, Any{k}, at, bt, cit, ct);
+  } else {
+    const nint_t bytes = op.required_workspace(Any{m}, Any{n}, Any{k}, at, bt, ct);
+    kernel::Workspace ws(bytes);
+    auto v = ws.view();
+    op(v, Any{m}, Any{n}, Any{k}, at, bt, ct);
+  }
+  return 0;
+}
+
+template <typename Atom, typename TA, typename TB, typename TC>
+int run3(const TA* a, const TB* b, TC* c, int64_t batch, int64_t m, int64_t n, int64_t k, const int64_t* sa,
+         const int64_t* sb, const int64_t* sc) {
+  if (!enable_amx()) return -1;
+  auto at = view3(const_cast<TA*>(a), batch, m, k, sa[0], sa[1], sa[2]);
+  auto bt = view3(const_cast<TB*>(b), batch, n, k, sb[0], sb[1], sb[2]);
+  auto ct = view3(c, batch, m, n, sc[0], sc[1], sc[2]);
+  auto op = ops::matmul(ops::MatmulConfig<Atom>{});
+  const nint_t bytes = op.required_workspace(Any{m}, Any{n}, Any{k}, at, bt, ct);
+  kernel::Workspace ws(bytes);
+  auto v = ws.view();
+  op(v, Any{m}, Any{n}, Any{k}, at, bt, ct);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+#define VREF_EXPORT __attribute__((visibility("default")))
+
+VREF_EXPORT int vref_available(void) { return enable_amx() ? 1 : 0; }
+
+// bf16 x bf16 -> fp32 / bf16, fp32 memory -> bf16 compute -> fp32 / bf16 (AMX_BF16F32).
+VREF_EXPORT int vref_matmul_bf16_f32(const uint16_t* a, const uint16_t* b, float* c, const float* cin, int64_t m,
+                                     int64_t n, int64_t k, const int64_t* sa, const int64_t* sb, const int64_t* sc) {
+  return run2<matmul::AMX_BF16F32>(reinterpret_cast<const bfloat16_t*>(a), reinterpret_cast<const bfloat16_t*>(b), c,
+                                   cin, m, n, k, sa, sb, sc);
+}
+VREF_EXPORT int vref_matmul_bf16_bf16(const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t m, int64_t n,
+                                      int64_t k, const int64_t* sa, const int64_t* sb, const int64_t* sc) {
+  return run2<matmul::AMX_BF16F32>(reinterpret_cast<const bfloat16_t*>(a), reinterpret_cast<const bfloat16_t*>(b),
+                                   reinterpret_cast<bfloat16_t*>(c), static_cast<const bfloat16_t*>(nullptr), m, n, k,
+                                   sa, sb, sc);
+}
+VREF_EXPORT int vref_matmul_f32_f32(const float* a, const float* b, float* c, const float* cin, int64_t m, int64_t n,
+                                    int64_t k, const int64_t* sa, const int64_t* sb, const int64_t* sc) {
+  return run2<matmul::AMX_BF16F32>(a, b, c, cin, m, n, k, sa, sb, sc);
+}
+VREF_EXPORT int vref_matmul_f32_bf16(const float* a, const float* b, uint16_t* c, int64_t m, int64_t n, int64_t k,
+                                     const int64_t* sa, const int64_t* sb, const int64_t* sc) {
+  return run2<matmul::AMX_BF16F32>(a, b, reinterpret_cast<bfloat16_t*>(c), static_cast<const bfloat16_t*>(nullptr), m,
+                                   n, k, sa, sb, sc);
+}
+// Rank-3 batch (stride 0 on the batch axis = broadcast operand).
+VREF_EXPORT int vref_matmul_bf16_f32_batched(const uint16_t* a, const uint16_t* b, float* c, int64_t batch, int64_t m,
+                                             int64_t n, int64_t k, const int64_t* sa, const int64_t* sb,
+                                             const int64_t* sc) {
+  return run3<matmul::AMX_BF16F32>(reinterpret_cast<const bfloat16_t*>(a), reinterpret_cast<const bfloat16_t*>(b), c,
+                                   batch, m, n, k, sa, sb, sc);
+}
+// int8 x int8 -> int32 (wraps) and u8 x i8 -> int32.
+VREF_EXPORT int vref_matmul_i8_i32(const int8_t* a, const int8_t* b, int32_t* c, const int32_t* cin, int64_t m,
+                                   int64_t n, int64_t k, const int64_t* sa, const int64_t* sb, const int64_t* sc) {
+  return run2<matmul::AMX_I8I32<int8_t, int8_t>>(a, b, c, cin, m, n, k, sa, sb, sc);
+}
+VREF_EXPORT int vref_matmul_u8i8_i32(const uint8_t* a, const int8_t* b, int32_t* c, int64_t m, int64_t n, int64_t k,
+                                     const int64_t* sa, const int64_t* sb, const int64_t* sc) {
+  return run2<matmul::AMX_I8I32<uint8_t, int8_t>>(a, b, c, static_cast<const int32_t*>(nullptr), m, n, k, sa, sb, sc);
+}
+
+// int8 x int8 with the fused per-row x per-column dequantisation epilogue
+// (matmul/Quantization.h:195-250).  column_scales must be readable 64 floats
+// past n (unmasked vector load, Quantization.h:229-231).  correction (may be
+// null) is the stride-0 int32 C-input row of
+// tests/ops/MatmulConversionTestCommon.h:1467-1472.
+VREF_EXPORT int vref_matmul_i8_dequant(const int8_t* a, const int8_t* b, const float* row_scales,
+                                       const float* column_scales, const int32_t* correction, float* c, int64_t m,
+                                       int64_t n, int64_t k) {
+  if (!enable_amx()) return -1;
+  using Atom = matmul::AMX_I8I32<int8_t, int8_t>;
+  auto at = view2(const_cast<int8_t*>(a), m, k, k, 1);
+  auto bt = view2(const_cast<int8_t*>(b), n, k, k, 1);
+  auto ct = view2(c, m, n, n, 1);
+  auto deq = matmul::make_runtime_per_row_column_dequantize_transform({row_scales, column_scales, 0});
+  auto cout = tensor::output<int32_t>(ct, deq);
+  auto op = ops::matmul(ops::MatmulConfig<Atom>{});
+  if (correction) {
+    auto cit = view2(const_cast<int32_t*>(correction), m, n, 0, 1);
+    const nint_t bytes = op.required_workspace(Any{m}, Any{n}, Any{k}, at, bt, cit, cout);
+    kernel::Workspace ws(bytes);
+    auto v = ws.view();
+    op(v, Any{m}, Any{n}, Any{k}, at, bt, cit, cout);
+  } else {
+    const nint_t bytes = op.required_workspace(Any{m}, Any{n}, Any{k}, at, bt, cout);
+    kernel::Workspace ws(bytes);
+    auto v = ws.view();
+    op(v, Any{m}, Any{n}, Any{k}, at, bt, cout);
+  }
+  return 0;
+}
+
+// The non-inline dispatch predicates of src/MatmulRuntimeDispatch.cpp:12-32.
+VREF_EXPORT int vref_amx_small_vector_profitable(int shape, int64_t m, int64_t n, int64_t k) {
+  return kernel::matmul_details::runtime_amx_small_vector_profitable(
+    static_cast<kernel::matmul_details::SmallVectorShape>(shape), m, n, k);
+}
+VREF_EXPORT int vref_sme_small_vector_profitable(int shape, int64_t m, int64_t n, int64_t k) {
+  return kernel::matmul_details::runtime_sme_small_vector_profitable(
+    static_cast<kernel::matmul_details::SmallVectorShape>(shape), m, n, k);
+}
+VREF_EXPORT int vref_small_area_profitable(int64_t m, int64_t n, int64_t k, int64_t limit) {
+  return kernel::matmul_details::runtime_small_area_profitable(m, n, k, limit);
+}
+VREF_EXPORT int vref_amx_residual_split_profitable(int64_t m, int64_t n, int64_t k) {
+  return kernel::matmul_details::runtime_amx_residual_split_profitable(m, n, k);
+}
+
+}  // extern "C"

@@ -1,0 +1,155 @@
+"""ctypes binding of ``libvecops_hip.so`` (``include/vecops_hip.h``).
+
+There is no CPU fallback: loading fails loudly when the HIP library has not been
+built, and every call goes to the GPU kernels.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libvecops_hip.so")
+
+# VecopsDType numbers
+I8, U8, I32, F16, BF16, F32 = 2, 3, 6, 10, 11, 12
+COMPUTE_BF16, COMPUTE_F32 = 0, 1
+FAMILY_NAMES = {0: "none", 1: "tile_256", 2: "tile_128", 3: "tile_64", 4: "skinny", 5: "zero_k"}
+STATUS_NAMES = {0: "Ok", 1: "InvalidArgument", 2: "NotApplicable", 3: "NotFound", 4: "AbiMismatch", 5: "LoadError",
+                6: "ExecutionError", 7: "InternalError"}
+
+EXPORTS = [
+    "vecops_hip_abi_version", "vecops_hip_last_error", "vecops_hip_device_count", "vecops_hip_plan_matmul",
+    "vecops_hip_matmul", "vecops_hip_matmul_i8_dequant", "vecops_hip_matmul_i8_dequant_workspace",
+    "vecops_hip_matmul_w8a16_group",
+]
+
+
+class Operand(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("dtype", C.c_uint32), ("rank", C.c_uint32), ("sizes", C.c_int64 * 3),
+                ("strides", C.c_int64 * 3)]
+
+
+class Plan(C.Structure):
+    _fields_ = [("family", C.c_uint32), ("split_k", C.c_uint32), ("vector_a", C.c_uint32), ("vector_b", C.c_uint32),
+                ("b_layout", C.c_uint32), ("reserved", C.c_uint32), ("workspace_bytes", C.c_uint64)]
+
+
+class VecopsHipError(RuntimeError):
+    def __init__(self, code: int, message: str) -> None:
+        super().__init__(f"{STATUS_NAMES.get(code, code)}: {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: build it with vecops_amd.build.build_all() "
+                               "(there is no CPU fallback for the HIP path)")
+        L = C.CDLL(LIB_PATH)
+        L.vecops_hip_abi_version.restype = C.c_uint32
+        L.vecops_hip_last_error.restype = C.c_char_p
+        L.vecops_hip_device_count.restype = C.c_int32
+        P = C.POINTER(Operand)
+        L.vecops_hip_plan_matmul.argtypes = [P, P, P, P, C.c_uint32, C.POINTER(Plan)]
+        L.vecops_hip_matmul.argtypes = [P, P, P, P, C.c_uint32, C.c_void_p, C.c_uint64, C.c_void_p]
+        L.vecops_hip_matmul_i8_dequant.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p,
+                                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
+                                                   C.c_int64, C.c_int64, C.c_void_p, C.c_uint64, C.c_void_p]
+        L.vecops_hip_matmul_i8_dequant_workspace.restype = C.c_uint64
+        L.vecops_hip_matmul_i8_dequant_workspace.argtypes = [C.c_int64] * 3
+        L.vecops_hip_matmul_w8a16_group.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p,
+                                                    C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                                                    C.c_int64, C.c_void_p]
+        _lib = L
+    return _lib
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise VecopsHipError(rc, lib().vecops_hip_last_error().decode())
+
+
+def _torch_dtype_code(t) -> int:
+    import torch
+    return {torch.int8: I8, torch.uint8: U8, torch.int32: I32, torch.float16: F16, torch.bfloat16: BF16,
+            torch.float32: F32}[t.dtype]
+
+
+def operand(t) -> Operand:
+    """Describe a torch tensor (rank 2 or 3, any strides) living in device memory."""
+    o = Operand()
+    o.data = t.data_ptr()
+    o.dtype = _torch_dtype_code(t)
+    o.rank = t.dim()
+    for i in range(t.dim()):
+        o.sizes[i] = t.shape[i]
+        o.strides[i] = t.stride(i)
+    return o
+
+
+def _stream_handle(stream) -> int:
+    import torch
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return s.cuda_stream
+
+
+def plan_matmul(a, b, c, c_in=None, compute=COMPUTE_BF16) -> Plan:
+    plan = Plan()
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    _check(lib().vecops_hip_plan_matmul(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None,
+                                        C.byref(oc), compute, C.byref(plan)))
+    return plan
+
+
+def matmul(a, b, c, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None):
+    """c[..,M,N] = c_in + a[..,M,K] . b[..,N,K]^T on the GPU; returns c.
+
+    Mirrors ``ops::matmul(config)(workspace, m, n, k, A, B[, Cin], C)``: the caller
+    allocates the output; a workspace tensor is allocated here when the plan needs
+    one and none is passed.
+    """
+    import torch
+    plan = plan_matmul(a, b, c, c_in, compute)
+    if plan.workspace_bytes and (workspace is None or workspace.numel() * workspace.element_size()
+                                 < plan.workspace_bytes):
+        workspace = torch.empty(plan.workspace_bytes, dtype=torch.uint8, device=c.device)
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None, C.byref(oc),
+                                   compute, ws_ptr, ws_size, _stream_handle(stream)))
+    return c
+
+
+def matmul_i8_dequant(a, b, row_scales, column_scales, c, correction=None, workspace=None, stream=None):
+    import torch
+    m, k = a.shape
+    n = b.shape[0]
+    assert a.stride(1) == 1 and b.stride(1) == 1 and c.stride(1) == 1
+    need = lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k)
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=c.device)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_i8_dequant(
+        a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), row_scales.data_ptr(), column_scales.data_ptr(),
+        correction.data_ptr() if correction is not None else None, c.data_ptr(), c.stride(0), m, n, k, ws_ptr,
+        ws_size, _stream_handle(stream)))
+    return c
+
+
+def matmul_w8a16_group(x, w, scales, y, group: int, stream=None):
+    m, k = x.shape
+    n = w.shape[0]
+    assert x.stride(1) == 1 and w.stride(1) == 1 and y.stride(1) == 1 and scales.is_contiguous()
+    _check(lib().vecops_hip_matmul_w8a16_group(x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
+                                               scales.data_ptr(), y.data_ptr(), y.stride(0), m, n, k, group,
+                                               _stream_handle(stream)))
+    return y

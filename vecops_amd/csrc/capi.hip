@@ -1,0 +1,380 @@
+// C ABI of libvecops_hip.so (declared in include/vecops_hip.h): operand
+// validation, the GPU kernel-selection rule table and the kernel launches.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "skinny_w8a16.h"
+#include "tile_gemm_launch.h"
+#include "vecops_hip.h"
+
+namespace {
+
+using namespace vecops_hip;
+
+enum : int32_t { ST_OK = 0, ST_INVALID = 1, ST_NOT_APPLICABLE = 2, ST_EXEC = 6 };
+enum : uint32_t { DT_I8 = 2, DT_U8 = 3, DT_I32 = 6, DT_F16 = 10, DT_BF16 = 11, DT_F32 = 12 };
+
+thread_local char g_error[512] = "";
+
+int32_t fail(int32_t code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int64_t dtype_bytes(uint32_t dt) {
+  switch (dt) {
+    case DT_I8: case DT_U8: return 1;
+    case DT_F16: case DT_BF16: return 2;
+    case DT_I32: case DT_F32: return 4;
+    default: return 0;
+  }
+}
+
+struct View {  // rank-3 normalised operand
+  void* data;
+  uint32_t dtype;
+  int64_t batch, rows, cols;
+  int64_t bs, rs, cs;
+};
+
+bool normalise(const VecopsHipOperand* o, View* v) {
+  if (o == nullptr || (o->rank != 2 && o->rank != 3)) return false;
+  const int base = o->rank == 3 ? 1 : 0;
+  v->data = o->data;
+  v->dtype = o->dtype;
+  v->batch = o->rank == 3 ? o->sizes[0] : 1;
+  v->bs = o->rank == 3 ? o->strides[0] : 0;
+  v->rows = o->sizes[base];
+  v->cols = o->sizes[base + 1];
+  v->rs = o->strides[base];
+  v->cs = o->strides[base + 1];
+  return v->batch >= 0 && v->rows >= 0 && v->cols >= 0;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// 16-byte loads along K: unit K stride, row and batch strides and base all multiples of 16 bytes.
+bool k_vector_ok(const View& v) {
+  const int64_t eb = dtype_bytes(v.dtype);
+  const int64_t per = 16 / eb;
+  return v.cs == 1 && v.rs % per == 0 && v.bs % per == 0 && aligned16(v.data);
+}
+
+struct Problem {
+  View a, b, c, cin;
+  bool has_cin;
+  int src;       // SrcKind
+  int out_kind;  // OutKind
+  int cin_kind;
+  int64_t batch, m, n, k;
+};
+
+// Same rules as vecops' validate() (planning/families/ArchitectureFamily.h:1590-1652,
+// planning/families/GenericTiled.h:100-154) plus the dtype combinations this library implements.
+int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* cin,
+                 const VecopsHipOperand* c, uint32_t compute, Problem* pr) {
+  if (!normalise(a, &pr->a) || !normalise(b, &pr->b) || !normalise(c, &pr->c))
+    return fail(ST_INVALID, "matmul: operands must be rank 2 or 3 with non-negative extents");
+  pr->has_cin = cin != nullptr;
+  if (pr->has_cin && !normalise(cin, &pr->cin)) return fail(ST_INVALID, "matmul: malformed c_in");
+  if (a->rank != b->rank || a->rank != c->rank || (pr->has_cin && cin->rank != c->rank))
+    return fail(ST_INVALID, "matmul: operand ranks differ");
+  if (pr->a.cols != pr->b.cols)
+    return fail(ST_INVALID, "matmul: K of a (%lld) and b (%lld) differ", (long long)pr->a.cols, (long long)pr->b.cols);
+  if (pr->c.rows != pr->a.rows || pr->c.cols != pr->b.rows)
+    return fail(ST_INVALID, "matmul: c must be [M=%lld, N=%lld]", (long long)pr->a.rows, (long long)pr->b.rows);
+  if (pr->a.batch != pr->b.batch || pr->a.batch != pr->c.batch)
+    return fail(ST_INVALID, "matmul: batch extents differ");
+  if (pr->has_cin && (pr->cin.rows != pr->c.rows || pr->cin.cols != pr->c.cols || pr->cin.batch != pr->c.batch))
+    return fail(ST_INVALID, "matmul: c_in extents differ from c");
+  pr->batch = pr->a.batch;
+  pr->m = pr->a.rows;
+  pr->n = pr->b.rows;
+  pr->k = pr->a.cols;
+  if (pr->m > INT32_MAX || pr->n > INT32_MAX || pr->k > INT32_MAX - 256 || pr->batch > 65535 * 16)
+    return fail(ST_INVALID, "matmul: extent too large");
+
+  const uint32_t da = pr->a.dtype, db = pr->b.dtype, dc = pr->c.dtype;
+  if (da != db) return fail(ST_NOT_APPLICABLE, "matmul: a and b dtypes differ (%u, %u)", da, db);
+  if (da == DT_BF16) {
+    pr->src = SRC_BF16;
+  } else if (da == DT_F32) {
+    if (compute != VECOPS_HIP_COMPUTE_BF16)
+      return fail(ST_NOT_APPLICABLE, "matmul: fp32 compute on fp32 operands is not built; use bf16 compute");
+    pr->src = SRC_F32_AS_BF16;
+  } else if (da == DT_I8) {
+    pr->src = SRC_I8;
+  } else {
+    return fail(ST_NOT_APPLICABLE, "matmul: operand dtype %u not supported", da);
+  }
+  if (pr->src == SRC_I8) {
+    if (dc != DT_I32) return fail(ST_NOT_APPLICABLE, "matmul: int8 operands need an int32 c");
+    pr->out_kind = OUT_I32;
+  } else {
+    if (dc == DT_F32) pr->out_kind = OUT_F32;
+    else if (dc == DT_BF16) pr->out_kind = OUT_BF16;
+    else return fail(ST_NOT_APPLICABLE, "matmul: floating operands need an f32 or bf16 c");
+  }
+  pr->cin_kind = pr->out_kind;
+  if (pr->has_cin) {
+    const uint32_t di = pr->cin.dtype;
+    if (pr->src == SRC_I8) {
+      if (di != DT_I32) return fail(ST_NOT_APPLICABLE, "matmul: c_in must be int32");
+      pr->cin_kind = OUT_I32;
+    } else if (di == DT_F32) {
+      pr->cin_kind = OUT_F32;
+    } else if (di == DT_BF16) {
+      pr->cin_kind = OUT_BF16;
+    } else {
+      return fail(ST_NOT_APPLICABLE, "matmul: c_in must be f32 or bf16");
+    }
+  }
+  return ST_OK;
+}
+
+constexpr int kComputeUnits = 256;
+
+// The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure
+// integer function of (operand class, m, n, k); it picks the workgroup tile by
+// how many tiles the problem yields against the 256 compute units and splits K
+// when even the smallest tile leaves most of them idle.
+void choose(const Problem& pr, VecopsHipPlan* plan) {
+  memset(plan, 0, sizeof(*plan));
+  plan->split_k = 1;
+  if (pr.batch == 0 || pr.m == 0 || pr.n == 0) {
+    plan->family = VECOPS_HIP_FAMILY_NONE;
+    return;
+  }
+  if (pr.k == 0) {
+    plan->family = VECOPS_HIP_FAMILY_ZERO_K;
+    return;
+  }
+  plan->vector_a = k_vector_ok(pr.a) ? 1 : 0;
+  plan->vector_b = k_vector_ok(pr.b) ? 1 : 0;
+  plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
+
+  auto tiles = [&](int64_t t) { return ((pr.m + t - 1) / t) * ((pr.n + t - 1) / t) * pr.batch; };
+  uint32_t family;
+  int64_t tile;
+  if (pr.m > 128 && pr.n > 128 && tiles(256) >= kComputeUnits * 3 / 4) {
+    family = VECOPS_HIP_FAMILY_TILE_256;
+    tile = 256;
+  } else if (pr.m > 64 && pr.n > 64 && tiles(128) >= kComputeUnits / 2) {
+    family = VECOPS_HIP_FAMILY_TILE_128;
+    tile = 128;
+  } else {
+    family = VECOPS_HIP_FAMILY_TILE_64;
+    tile = 64;
+    if (pr.m > 64 && pr.n > 64 && tiles(64) > 4 * kComputeUnits) {
+      family = VECOPS_HIP_FAMILY_TILE_128;
+      tile = 128;
+    }
+  }
+  plan->family = family;
+  const int64_t ktile = pr.src == SRC_I8 ? 128 : 64;
+  const int64_t k_tiles = (pr.k + ktile - 1) / ktile;
+  const int64_t wgs = tiles(tile);
+  int64_t split = 1;
+  if (wgs < kComputeUnits / 2 && k_tiles >= 8) {
+    split = kComputeUnits / wgs;
+    if (split > k_tiles / 4) split = k_tiles / 4;
+    if (split > 64) split = 64;
+    if (split < 1) split = 1;
+  }
+  plan->split_k = static_cast<uint32_t>(split);
+  if (split > 1) plan->workspace_bytes = static_cast<uint64_t>(split) * pr.batch * pr.m * pr.n * 4u;
+}
+
+int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* row_scales, const float* column_scales,
+                    const int32_t* correction, void* workspace, uint64_t workspace_size, hipStream_t stream) {
+  if (plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
+  if (pr.a.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: a has no storage");
+  if (pr.b.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: b has no storage");
+  if (pr.c.data == nullptr) return fail(ST_INVALID, "matmul: c has no storage");
+  if (plan.workspace_bytes > workspace_size || (plan.workspace_bytes > 0 && workspace == nullptr))
+    return fail(ST_INVALID, "matmul: workspace of %llu bytes required, %llu supplied",
+                (unsigned long long)plan.workspace_bytes, (unsigned long long)workspace_size);
+
+  TileGemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.a = pr.a.data;
+  p.b = pr.b.data;
+  p.c = pr.c.data;
+  p.cin = pr.has_cin ? pr.cin.data : nullptr;
+  p.partial = workspace;
+  p.row_scales = row_scales;
+  p.column_scales = column_scales;
+  p.correction = correction;
+  p.m = static_cast<int32_t>(pr.m);
+  p.n = static_cast<int32_t>(pr.n);
+  p.k = static_cast<int32_t>(pr.k);
+  p.batch = static_cast<int32_t>(pr.batch);
+  p.out_kind = pr.out_kind;
+  p.cin_kind = pr.cin_kind;
+  p.a_rs = pr.a.rs; p.a_ks = pr.a.cs; p.a_bs = pr.a.bs;
+  p.b_rs = pr.b.rs; p.b_ks = pr.b.cs; p.b_bs = pr.b.bs;
+  p.c_rs = pr.c.rs; p.c_cs = pr.c.cs; p.c_bs = pr.c.bs;
+  if (pr.has_cin) { p.cin_rs = pr.cin.rs; p.cin_cs = pr.cin.cs; p.cin_bs = pr.cin.bs; }
+  const bool is_int = pr.src == SRC_I8;
+
+  if (plan.family == VECOPS_HIP_FAMILY_ZERO_K) {
+    p.split_k = 0;  // empty sum: the reduce kernel emits epilogue(0)
+    hipError_t e = launch_splitk_reduce(p, is_int, stream);
+    if (e != hipSuccess) return fail(ST_EXEC, "zero-K kernel launch: %s", hipGetErrorString(e));
+    return ST_OK;
+  }
+
+  const int tile = plan.family == VECOPS_HIP_FAMILY_TILE_256 ? 256 : plan.family == VECOPS_HIP_FAMILY_TILE_128 ? 128 : 64;
+  const int ktile = is_int ? 128 : 64;
+  p.tiles_m = static_cast<int32_t>((pr.m + tile - 1) / tile);
+  p.tiles_n = static_cast<int32_t>((pr.n + tile - 1) / tile);
+  const int k_tiles = static_cast<int>((pr.k + ktile - 1) / ktile);
+  p.split_k = static_cast<int32_t>(plan.split_k);
+  p.k_tiles_per_split = (k_tiles + p.split_k - 1) / p.split_k;
+  const bool vec = plan.vector_a && plan.vector_b;
+
+  hipError_t e;
+  switch (pr.src) {
+    case SRC_BF16: e = launch_tile_gemm_bf16(p, tile, vec, stream); break;
+    case SRC_F32_AS_BF16: e = launch_tile_gemm_f32_as_bf16(p, tile, vec, stream); break;
+    default: e = launch_tile_gemm_i8(p, tile, vec, stream); break;
+  }
+  if (e != hipSuccess) return fail(ST_EXEC, "tile kernel launch: %s", hipGetErrorString(e));
+  if (p.split_k > 1) {
+    e = launch_splitk_reduce(p, is_int, stream);
+    if (e != hipSuccess) return fail(ST_EXEC, "split-K reduce launch: %s", hipGetErrorString(e));
+  }
+  return ST_OK;
+}
+
+void make_operand(VecopsHipOperand* o, const void* data, uint32_t dtype, int64_t rows, int64_t cols, int64_t rs) {
+  memset(o, 0, sizeof(*o));
+  o->data = const_cast<void*>(data);
+  o->dtype = dtype;
+  o->rank = 2;
+  o->sizes[0] = rows;
+  o->sizes[1] = cols;
+  o->strides[0] = rs;
+  o->strides[1] = 1;
+}
+
+template <int MB, int ROWS>
+void launch_skinny(const SkinnyW8A16Params& p, hipStream_t stream) {
+  const int64_t waves = (p.n + ROWS - 1) / ROWS;
+  const int64_t blocks = (waves + 3) / 4;
+  hipLaunchKernelGGL((skinny_w8a16_kernel<MB, ROWS>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p);
+}
+
+}  // namespace
+
+extern "C" {
+
+uint32_t vecops_hip_abi_version(void) { return VECOPS_HIP_ABI_VERSION; }
+
+const char* vecops_hip_last_error(void) { return g_error; }
+
+int32_t vecops_hip_device_count(void) {
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess) {
+    fail(ST_EXEC, "hipGetDeviceCount: %s", hipGetErrorString(e));
+    return -1;
+  }
+  return n;
+}
+
+int32_t vecops_hip_plan_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                               const VecopsHipOperand* c, uint32_t compute, VecopsHipPlan* plan) {
+  if (plan == nullptr) return fail(ST_INVALID, "plan_matmul: null plan");
+  Problem pr;
+  int32_t rc = describe(a, b, c_in, c, compute, &pr);
+  if (rc != ST_OK) return rc;
+  choose(pr, plan);
+  return ST_OK;
+}
+
+int32_t vecops_hip_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                          const VecopsHipOperand* c, uint32_t compute, void* workspace, uint64_t workspace_size,
+                          void* stream) {
+  Problem pr;
+  int32_t rc = describe(a, b, c_in, c, compute, &pr);
+  if (rc != ST_OK) return rc;
+  VecopsHipPlan plan;
+  choose(pr, &plan);
+  return run_problem(pr, plan, nullptr, nullptr, nullptr, workspace, workspace_size, static_cast<hipStream_t>(stream));
+}
+
+uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int64_t n, int64_t k) {
+  VecopsHipOperand a, b, c;
+  make_operand(&a, reinterpret_cast<void*>(16), DT_I8, m, k, k);
+  make_operand(&b, reinterpret_cast<void*>(16), DT_I8, n, k, k);
+  make_operand(&c, reinterpret_cast<void*>(16), DT_I32, m, n, n);
+  VecopsHipPlan plan;
+  if (vecops_hip_plan_matmul(&a, &b, nullptr, &c, 0, &plan) != ST_OK) return 0;
+  return plan.workspace_bytes;
+}
+
+int32_t vecops_hip_matmul_i8_dequant(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                                     const float* row_scales, const float* column_scales, const int32_t* correction,
+                                     float* c, int64_t ldc, int64_t m, int64_t n, int64_t k, void* workspace,
+                                     uint64_t workspace_size, void* stream) {
+  if (m < 0 || n < 0 || k < 0) return fail(ST_INVALID, "matmul_i8_dequant: negative extent");
+  if (m > 0 && n > 0 && (row_scales == nullptr || column_scales == nullptr))
+    return fail(ST_INVALID, "matmul_i8_dequant: scales are required");
+  VecopsHipOperand oa, ob, oc;
+  make_operand(&oa, a, DT_I8, m, k, lda);
+  make_operand(&ob, b, DT_I8, n, k, ldb);
+  make_operand(&oc, c, DT_I32, m, n, ldc);  // accumulator class; the epilogue writes fp32
+  Problem pr;
+  int32_t rc = describe(&oa, &ob, nullptr, &oc, 0, &pr);
+  if (rc != ST_OK) return rc;
+  VecopsHipPlan plan;
+  choose(pr, &plan);
+  return run_problem(pr, plan, row_scales, column_scales, correction, workspace, workspace_size,
+                     static_cast<hipStream_t>(stream));
+}
+
+int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t ldx, const int8_t* w, int64_t ldw, const float* scales,
+                                      void* y, int64_t ldy, int64_t m, int64_t n, int64_t k, int64_t group,
+                                      void* stream) {
+  if (m < 0 || n < 0 || k < 0) return fail(ST_INVALID, "matmul_w8a16_group: negative extent");
+  if (m > 16) return fail(ST_NOT_APPLICABLE, "matmul_w8a16_group: m = %lld exceeds 16", (long long)m);
+  if (group <= 0 || group % 16 != 0 || k % group != 0)
+    return fail(ST_INVALID, "matmul_w8a16_group: group must be a multiple of 16 that divides k");
+  if (m == 0 || n == 0) return ST_OK;
+  if (x == nullptr || w == nullptr || scales == nullptr || y == nullptr)
+    return fail(ST_INVALID, "matmul_w8a16_group: null operand");
+  if (!aligned16(x) || !aligned16(w) || ldx % 8 != 0 || ldw % 16 != 0)
+    return fail(ST_INVALID, "matmul_w8a16_group: x and w rows must be 16-byte aligned");
+  if (n > INT32_MAX || k > INT32_MAX) return fail(ST_INVALID, "matmul_w8a16_group: extent too large");
+  SkinnyW8A16Params p;
+  p.x = static_cast<const uint16_t*>(x);
+  p.w = w;
+  p.scales = scales;
+  p.y = static_cast<uint16_t*>(y);
+  p.ldx = ldx;
+  p.ldw = ldw;
+  p.ldy = ldy;
+  p.m = static_cast<int32_t>(m);
+  p.n = static_cast<int32_t>(n);
+  p.k = static_cast<int32_t>(k);
+  p.group = static_cast<int32_t>(group);
+  p.groups = static_cast<int32_t>(k / group);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (m == 1) launch_skinny<1, 8>(p, s);
+  else if (m == 2) launch_skinny<2, 8>(p, s);
+  else if (m <= 4) launch_skinny<4, 4>(p, s);
+  else if (m <= 8) launch_skinny<8, 2>(p, s);
+  else launch_skinny<16, 2>(p, s);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(ST_EXEC, "skinny kernel launch: %s", hipGetErrorString(e));
+  return ST_OK;
+}
+
+}  // extern "C"

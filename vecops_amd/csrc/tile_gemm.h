@@ -1,0 +1,526 @@
+// MFMA workgroup-tile GEMM for gfx950: C[M,N] (+)= A[M,K] . B[N,K]^T.
+//
+// Geometry (identical in bytes for every operand type):
+//   * a K tile is 128 bytes of operand per row = eight 16-byte chunks
+//     (64 bf16 or 128 int8 elements);
+//   * one MFMA k-step consumes two chunks: lanes 0-31 take the even chunk,
+//     lanes 32-63 the odd one, each lane holding 16 contiguous bytes of its row
+//     (v_mfma_f32_32x32x16_bf16: 8 bf16; v_mfma_i32_32x32x32_i8: 16 int8);
+//   * a workgroup is 4 wavefronts in a 2x2 grid; each wavefront owns
+//     WM x WN accumulator tiles of 32x32, so the workgroup tile is
+//     (64*WM) x (64*WN);
+//   * LDS holds two stages of (BM + BN) rows x 128 bytes; chunk c of row r lives
+//     at r*128 + ((c ^ (r & 7)) * 16), which makes the 16-byte reads of eight
+//     consecutive rows hit eight different bank groups.
+//
+// fp32 operands in "bf16 compute" mode are rounded to bf16 (nearest even) while
+// they are staged into LDS, so the inner loop is the bf16 one.
+#ifndef VECOPS_HIP_TILE_GEMM_H
+#define VECOPS_HIP_TILE_GEMM_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+namespace vecops_hip {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+
+enum SrcKind : int { SRC_BF16 = 0, SRC_F32_AS_BF16 = 1, SRC_I8 = 2 };
+enum OutKind : int { OUT_F32 = 0, OUT_BF16 = 1, OUT_I32 = 2 };
+// How an operand tile is fetched from global memory.
+enum LoadKind : int {
+  LOAD_KVEC = 0,     // K contiguous, rows and base 16-byte aligned: one 16-byte load per chunk
+  LOAD_GENERIC = 1,  // any strides / alignment: one load per element
+  LOAD_NVEC = 2      // spatial index contiguous (B given as [K,N] row-major), 16-byte aligned rows
+};
+
+struct TileGemmParams {
+  const void* a;
+  const void* b;
+  const void* cin;  // null = zero accumulator
+  void* c;
+  void* partial;    // split-K partial sums [split][batch][M][N] in accumulator type
+  const float* row_scales;     // int8 dequant epilogue (null = none)
+  const float* column_scales;
+  const int32_t* correction;   // int32 row added to every accumulator row (null = none)
+  int32_t m, n, k;
+  int32_t batch;
+  int32_t tiles_m, tiles_n;
+  int32_t split_k;
+  int32_t k_tiles_per_split;
+  int32_t out_kind;
+  int32_t cin_kind;
+  int64_t a_rs, a_ks, a_bs;  // row, k and batch strides in elements
+  int64_t b_rs, b_ks, b_bs;
+  int64_t c_rs, c_cs, c_bs;
+  int64_t cin_rs, cin_cs, cin_bs;
+};
+
+template <int SRC>
+struct SrcTraits;
+template <>
+struct SrcTraits<SRC_BF16> {
+  static constexpr int kElemsPerChunk = 8;
+  static constexpr int kSrcBytes = 2;
+  static constexpr bool kInt = false;
+};
+template <>
+struct SrcTraits<SRC_F32_AS_BF16> {
+  static constexpr int kElemsPerChunk = 8;
+  static constexpr int kSrcBytes = 4;
+  static constexpr bool kInt = false;
+};
+template <>
+struct SrcTraits<SRC_I8> {
+  static constexpr int kElemsPerChunk = 16;
+  static constexpr int kSrcBytes = 1;
+  static constexpr bool kInt = true;
+};
+
+// fp32 -> bf16 bits, round to nearest even; NaN -> 0x7fc0 (vecops util/BFloat16.h:25-37).
+__device__ __forceinline__ uint32_t bf16_bits_rne(float x) {
+  uint32_t bits = __float_as_uint(x);
+  uint32_t rounded = (bits + (((bits >> 16) & 1u) + 0x7fffu)) >> 16;
+  return (x != x) ? 0x7fc0u : rounded;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return bf16_bits_rne(lo) | (bf16_bits_rne(hi) << 16);
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+__device__ __forceinline__ int lds_chunk_offset(int row, int chunk) { return row * 128 + (((chunk ^ row) & 7) << 4); }
+
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+// Two fp32 -> packed bf16 pair with the hardware converter (round to nearest even).
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
+  f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
+// Fast path: one whole 16-byte chunk, no bounds checks (the caller guarantees
+// that the row exists and that the chunk lies inside K).
+template <int SRC>
+__device__ __forceinline__ u32x4 load_chunk_fast(const char* src) {
+  if constexpr (SRC == SRC_F32_AS_BF16) {
+    const f32x4* p = reinterpret_cast<const f32x4*>(src);
+    const f32x4 lo = p[0], hi = p[1];
+    u32x4 out;
+    out.x = cvt_pk_bf16(lo.x, lo.y);
+    out.y = cvt_pk_bf16(lo.z, lo.w);
+    out.z = cvt_pk_bf16(hi.x, hi.y);
+    out.w = cvt_pk_bf16(hi.z, hi.w);
+    return out;
+  } else {
+    return *reinterpret_cast<const u32x4*>(src);
+  }
+}
+
+// Slow path: element by element with bounds checks and arbitrary K stride; used
+// for the K tail of the vector path and for every chunk of the generic path.
+template <int SRC>
+__device__ __noinline__ u32x4 load_chunk_checked(const void* base, int64_t row_off, int64_t kstep, int k0, int k_end,
+                                                 bool row_ok) {
+  constexpr int EPC = SrcTraits<SRC>::kElemsPerChunk;
+  uint32_t w0 = 0u, w1 = 0u, w2 = 0u, w3 = 0u;
+  if (row_ok) {
+#pragma unroll
+    for (int e = 0; e < EPC; ++e) {
+      const int k = k0 + e;
+      uint32_t v = 0u;
+      if (k < k_end) {
+        if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
+        else if constexpr (SRC == SRC_F32_AS_BF16) v = cvt_pk_bf16(static_cast<const float*>(base)[row_off + k * kstep], 0.0f) & 0xffffu;
+        else v = static_cast<const uint8_t*>(base)[row_off + k * kstep];
+      }
+      constexpr int per_word = EPC / 4;
+      const uint32_t shifted = v << ((e % per_word) * (32 / per_word));
+      const int word = e / per_word;
+      if (word == 0) w0 |= shifted;
+      else if (word == 1) w1 |= shifted;
+      else if (word == 2) w2 |= shifted;
+      else w3 |= shifted;
+    }
+  }
+  return u32x4{w0, w1, w2, w3};
+}
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+// Accumulator tile type per operand class.
+template <bool INT>
+struct AccTile {
+  using type = f32x16;
+};
+template <>
+struct AccTile<true> {
+  using type = i32x16;
+};
+
+template <int SRC>
+__device__ __forceinline__ void mfma_step(typename AccTile<SrcTraits<SRC>::kInt>::type& acc, const u32x4& a,
+                                          const u32x4& b) {
+  if constexpr (SrcTraits<SRC>::kInt) {
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a), __builtin_bit_cast(i32x4, b), acc, 0, 0,
+                                                0);
+  } else {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc,
+                                                  0, 0, 0);
+  }
+}
+
+// Final value of one output element: accumulator (+ correction) (+ Cin), then
+// the optional dequantisation, then conversion to the memory dtype of C.
+//   fp :  c = convert(acc + cin)
+//   int:  v = acc + correction[col] + cin  (wrapping);  c = v  or
+//         c = (float(v) * row_scales[row]) * column_scales[col]
+//         (vecops matmul/Quantization.h:224-231: two multiplies, row first).
+template <bool INT, typename AccScalar>
+__device__ __forceinline__ void store_output(const TileGemmParams& p, int batch, int row, int col, AccScalar acc) {
+  const int64_t c_off = batch * p.c_bs + row * p.c_rs + col * p.c_cs;
+  if constexpr (INT) {
+    uint32_t v = static_cast<uint32_t>(acc);
+    if (p.correction) v += static_cast<uint32_t>(p.correction[col]);
+    if (p.cin) v += static_cast<uint32_t>(
+                 static_cast<const int32_t*>(p.cin)[batch * p.cin_bs + row * p.cin_rs + col * p.cin_cs]);
+    const int32_t s = static_cast<int32_t>(v);
+    if (p.row_scales) {
+      const float t = static_cast<float>(s) * p.row_scales[row];
+      static_cast<float*>(p.c)[c_off] = t * p.column_scales[col];
+    } else if (p.out_kind == OUT_I32) {
+      static_cast<int32_t*>(p.c)[c_off] = s;
+    } else {
+      static_cast<float*>(p.c)[c_off] = static_cast<float>(s);
+    }
+  } else {
+    float v = acc;
+    if (p.cin) {
+      const int64_t ci = batch * p.cin_bs + row * p.cin_rs + col * p.cin_cs;
+      v += (p.cin_kind == OUT_BF16) ? bf16_bits_to_f32(static_cast<const uint16_t*>(p.cin)[ci])
+                                    : static_cast<const float*>(p.cin)[ci];
+    }
+    if (p.out_kind == OUT_BF16) {
+      static_cast<uint16_t*>(p.c)[c_off] = static_cast<uint16_t>(bf16_bits_rne(v));
+    } else {
+      static_cast<float*>(p.c)[c_off] = v;
+    }
+  }
+}
+
+// One lane's 16 accumulators of a 32x32 tile through the full epilogue, with
+// bounds checks; out of line to keep the kernels small (edge tiles, split-K
+// partials, C-input and strided C only).
+template <bool INT>
+__device__ __noinline__ void store_tile_general(const TileGemmParams& p, int batch, int split, int row0, int col,
+                                                typename AccTile<INT>::type tile) {
+  using AccScalar = typename std::conditional<INT, int32_t, float>::type;
+  if (col >= p.n) return;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = row0 + (r >> 2) * 8 + (r & 3);
+    if (row < p.m) {
+      if (p.split_k > 1) {
+        AccScalar* part = static_cast<AccScalar*>(p.partial);
+        part[((static_cast<int64_t>(split) * p.batch + batch) * p.m + row) * p.n + col] = tile[r];
+      } else {
+        store_output<INT, AccScalar>(p, batch, row, col, tile[r]);
+      }
+    }
+  }
+}
+
+// Workgroup id -> (batch, split, tile_m, tile_n).  Workgroups are dealt to the
+// eight XCDs round-robin, each XCD with its own L2: renumber so that an XCD
+// receives a contiguous run of tiles, then walk tiles in bands of 8 tile rows so
+// that a run shares A rows and B columns.
+__device__ __forceinline__ void map_workgroup(const TileGemmParams& p, int& batch, int& split, int& tm, int& tn) {
+  int pid = blockIdx.x;
+  const int total = gridDim.x;
+  if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int tile = pid % tiles;
+  const int rest = pid / tiles;
+  split = rest % p.split_k;
+  batch = rest / p.split_k;
+  constexpr int kBand = 8;
+  const int band_size = kBand * p.tiles_n;
+  const int band = tile / band_size;
+  const int first_m = band * kBand;
+  const int rows_in_band = min(p.tiles_m - first_m, kBand);
+  const int in_band = tile - band * band_size;
+  tm = first_m + in_band % rows_in_band;
+  tn = in_band / rows_in_band;
+}
+
+// Per-thread staging plan for one operand: thread t stages chunk (t & 7) of rows
+// (t >> 3) + 32*i.  Rows past the operand's extent are clamped to its last row:
+// they are loaded but only feed accumulator rows/columns that are never stored.
+template <int SRC, int LOAD, int CHUNKS>
+struct OperandStager {
+  const char* base;     // operand base for this batch
+  int64_t row_bytes[CHUNKS];  // byte offset of each staged row (fast path)
+  int64_t rs, ks;       // element strides (checked path)
+  int first_row, extent, k_end;
+
+  __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
+                                       int k_end_, int ld_row, int ld_chunk) {
+    using T = SrcTraits<SRC>;
+    base = static_cast<const char*>(base_);
+    rs = rs_;
+    ks = ks_;
+    first_row = first_row_;
+    extent = extent_;
+    k_end = k_end_;
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int row = min(first_row + ld_row + i * 32, extent - 1);
+      row_bytes[i] = (static_cast<int64_t>(row) * rs + ld_chunk * T::kElemsPerChunk) * T::kSrcBytes;
+    }
+  }
+
+  // Whole K tile inside [0, K): unconditional 16-byte loads.
+  __device__ __forceinline__ void fetch_fast(u32x4 (&stage)[CHUNKS], int kt) const {
+    using T = SrcTraits<SRC>;
+    const int64_t k_bytes = static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes);
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) stage[i] = load_chunk_fast<SRC>(base + row_bytes[i] + k_bytes);
+  }
+
+  __device__ __forceinline__ void fetch_checked(u32x4 (&stage)[CHUNKS], int kt, int ld_row, int ld_chunk) const {
+    using T = SrcTraits<SRC>;
+    const int k0 = kt * 8 * T::kElemsPerChunk + ld_chunk * T::kElemsPerChunk;
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int row = first_row + ld_row + i * 32;
+      stage[i] = load_chunk_checked<SRC>(base, static_cast<int64_t>(row) * rs, ks, k0, k_end, row < extent);
+    }
+  }
+
+  __device__ __forceinline__ void fetch(u32x4 (&stage)[CHUNKS], int kt, int full_k_tiles, int ld_row,
+                                        int ld_chunk) const {
+    if constexpr (LOAD == LOAD_KVEC) {
+      if (kt < full_k_tiles) {
+        fetch_fast(stage, kt);
+        return;
+      }
+    }
+    fetch_checked(stage, kt, ld_row, ld_chunk);
+  }
+};
+
+template <int SRC, int WM, int WN, int LOAD_A, int LOAD_B>
+__global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) {
+  using T = SrcTraits<SRC>;
+  constexpr bool INT = T::kInt;
+  using Acc = typename AccTile<INT>::type;
+  constexpr int EPC = T::kElemsPerChunk;
+  constexpr int KTILE = 8 * EPC;  // elements per K tile
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int A_CHUNKS = BM / 32, B_CHUNKS = BN / 32;  // 16-byte chunks each thread stages per tile
+  constexpr int STAGE_BYTES = (BM + BN) * 128;
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  int batch, split, tm, tn;
+  map_workgroup(p, batch, split, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int total_k_tiles = (p.k + KTILE - 1) / KTILE;
+  const int full_k_tiles = p.k / KTILE;
+  const int kt_begin = split * p.k_tiles_per_split;
+  const int kt_end = min(total_k_tiles, kt_begin + p.k_tiles_per_split);
+
+  // staging assignment: thread -> (chunk column, 32-row stripe)
+  const int ld_chunk = tid & 7;
+  const int ld_row = tid >> 3;
+
+  OperandStager<SRC, LOAD_A, A_CHUNKS> stager_a;
+  OperandStager<SRC, LOAD_B, B_CHUNKS> stager_b;
+  stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, ld_row,
+                ld_chunk);
+  stager_b.init(static_cast<const char*>(p.b) + batch * p.b_bs * T::kSrcBytes, p.b_rs, p.b_ks, n0, p.n, p.k, ld_row,
+                ld_chunk);
+
+  Acc acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  u32x4 stage_a[A_CHUNKS], stage_b[B_CHUNKS];
+
+  // LDS byte offsets this thread writes (stage 0) and reads (stage 0, k-step 0)
+  const int st_off = lds_chunk_offset(ld_row, ld_chunk);  // + i*32*128 per chunk row
+  const int frag_row = lane & 31;
+  const int frag_half = lane >> 5;
+
+  if (kt_begin < kt_end) {
+    stager_a.fetch(stage_a, kt_begin, full_k_tiles, ld_row, ld_chunk);
+    stager_b.fetch(stage_b, kt_begin, full_k_tiles, ld_row, ld_chunk);
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<u32x4*>(lds + st_off + i * 4096) = stage_a[i];
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<u32x4*>(lds + BM * 128 + st_off + i * 4096) = stage_b[i];
+  }
+  __syncthreads();
+
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    const int stage = (kt - kt_begin) & 1;
+    const bool more = kt + 1 < kt_end;
+    if (more) {
+      stager_a.fetch(stage_a, kt + 1, full_k_tiles, ld_row, ld_chunk);
+      stager_b.fetch(stage_b, kt + 1, full_k_tiles, ld_row, ld_chunk);
+    }
+
+    const char* sa = lds + stage * STAGE_BYTES + (wm * WM * 32) * 128;
+    const char* sb = lds + stage * STAGE_BYTES + BM * 128 + (wn * WN * 32) * 128;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      // rows i*32 + frag_row keep (row & 7) == (frag_row & 7): one swizzled offset per k-step
+      const int off = lds_chunk_offset(frag_row, ks * 2 + frag_half);
+      u32x4 fa[WM], fb[WN];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) fa[i] = *reinterpret_cast<const u32x4*>(sa + off + i * 4096);
+#pragma unroll
+      for (int j = 0; j < WN; ++j) fb[j] = *reinterpret_cast<const u32x4*>(sb + off + j * 4096);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) mfma_step<SRC>(acc[i][j], fa[i], fb[j]);
+    }
+
+    if (more) {
+      char* dst = lds + (stage ^ 1) * STAGE_BYTES + st_off;
+#pragma unroll
+      for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<u32x4*>(dst + i * 4096) = stage_a[i];
+#pragma unroll
+      for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<u32x4*>(dst + BM * 128 + i * 4096) = stage_b[i];
+    }
+    __syncthreads();
+  }
+
+  // Epilogue.  Accumulator register r of lane l is C[(r/4)*8 + (l/32)*4 + r%4][l%32]
+  // of its 32x32 tile.  Tiles that lie wholly inside C and need no C-input or
+  // split-K take one of three inline store loops; everything else goes through
+  // the general out-of-line routine.
+  const bool interior = m0 + BM <= p.m && n0 + BN <= p.n;
+  const bool simple = interior && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1;
+  char* c_base = static_cast<char*>(p.c);
+  if (simple && !INT && p.out_kind == OUT_BF16) {
+    static_for<WM>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      static_for<WN>([&](auto cj) {
+        constexpr int j = decltype(cj)::value;
+        const int col = n0 + (wn * WN + j) * 32 + frag_row;
+        const int row0 = m0 + (wm * WM + i) * 32 + frag_half * 4;
+        uint16_t* dst = reinterpret_cast<uint16_t*>(c_base) + batch * p.c_bs + row0 * p.c_rs + col;
+        static_for<16>([&](auto cr) {
+          constexpr int r = decltype(cr)::value;
+          if constexpr (!INT) {
+            dst[((r >> 2) * 8 + (r & 3)) * p.c_rs] =
+              static_cast<uint16_t>(cvt_pk_bf16(acc[i][j][r], 0.0f));
+          }
+        });
+      });
+    });
+  } else if (simple && (INT ? (p.out_kind == OUT_I32 && p.row_scales == nullptr && p.correction == nullptr)
+                            : p.out_kind == OUT_F32)) {
+    static_for<WM>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      static_for<WN>([&](auto cj) {
+        constexpr int j = decltype(cj)::value;
+        const int col = n0 + (wn * WN + j) * 32 + frag_row;
+        const int row0 = m0 + (wm * WM + i) * 32 + frag_half * 4;
+        auto* dst = reinterpret_cast<typename std::conditional<INT, int32_t, float>::type*>(c_base) +
+                    batch * p.c_bs + row0 * p.c_rs + col;
+        static_for<16>([&](auto cr) {
+          constexpr int r = decltype(cr)::value;
+          dst[((r >> 2) * 8 + (r & 3)) * p.c_rs] = acc[i][j][r];
+        });
+      });
+    });
+  } else if (simple && INT && p.row_scales != nullptr) {
+    static_for<WM>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      float rs[16];
+      const int row0 = m0 + (wm * WM + i) * 32 + frag_half * 4;
+      static_for<16>([&](auto cr) {
+        constexpr int r = decltype(cr)::value;
+        rs[r] = p.row_scales[row0 + (r >> 2) * 8 + (r & 3)];
+      });
+      static_for<WN>([&](auto cj) {
+        constexpr int j = decltype(cj)::value;
+        const int col = n0 + (wn * WN + j) * 32 + frag_row;
+        const float cs = p.column_scales[col];
+        const uint32_t corr = p.correction ? static_cast<uint32_t>(p.correction[col]) : 0u;
+        float* dst = reinterpret_cast<float*>(c_base) + batch * p.c_bs + row0 * p.c_rs + col;
+        static_for<16>([&](auto cr) {
+          constexpr int r = decltype(cr)::value;
+          if constexpr (INT) {
+            const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(acc[i][j][r]) + corr);
+            const float t = static_cast<float>(v) * rs[r];
+            dst[((r >> 2) * 8 + (r & 3)) * p.c_rs] = t * cs;
+          }
+        });
+      });
+    });
+  } else {
+    static_for<WM>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      static_for<WN>([&](auto cj) {
+        constexpr int j = decltype(cj)::value;
+        store_tile_general<INT>(p, batch, split, m0 + (wm * WM + i) * 32 + frag_half * 4,
+                                n0 + (wn * WN + j) * 32 + frag_row, acc[i][j]);
+      });
+    });
+  }
+}
+
+// Sums the split-K partials and applies the same epilogue as the tile kernel.
+template <bool INT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const TileGemmParams p) {
+  using AccScalar = typename std::conditional<INT, int32_t, float>::type;
+  const int64_t per_batch = static_cast<int64_t>(p.m) * p.n;
+  const int64_t total = per_batch * p.batch;
+  const AccScalar* part = static_cast<const AccScalar*>(p.partial);
+  for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += gridDim.x * 256ll) {
+    const int batch = static_cast<int>(idx / per_batch);
+    const int64_t rem = idx - batch * per_batch;
+    const int row = static_cast<int>(rem / p.n), col = static_cast<int>(rem - static_cast<int64_t>(row) * p.n);
+    AccScalar sum = 0;
+    for (int s = 0; s < p.split_k; ++s) {
+      if constexpr (INT)
+        sum = static_cast<int32_t>(static_cast<uint32_t>(sum) + static_cast<uint32_t>(part[s * total + idx]));
+      else
+        sum += part[s * total + idx];
+    }
+    store_output<INT, AccScalar>(p, batch, row, col, sum);
+  }
+}
+
+}  // namespace vecops_hip
+#endif

@@ -1,0 +1,53 @@
+// Host-side launchers of the tile GEMM kernels, one translation unit per operand
+// class so the kernels compile in parallel.
+#ifndef VECOPS_HIP_TILE_GEMM_LAUNCH_H
+#define VECOPS_HIP_TILE_GEMM_LAUNCH_H
+
+#include <hip/hip_runtime.h>
+
+#include "tile_gemm.h"
+
+namespace vecops_hip {
+
+// tile: 256, 128 or 64 (workgroup tile edge).  vec: operands allow 16-byte loads
+// along K.  Returns the HIP error of the launch (hipSuccess when enqueued).
+hipError_t launch_tile_gemm_bf16(const TileGemmParams& p, int tile, bool vec, hipStream_t stream);
+hipError_t launch_tile_gemm_f32_as_bf16(const TileGemmParams& p, int tile, bool vec, hipStream_t stream);
+hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile, bool vec, hipStream_t stream);
+hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
+
+// Shared by the per-class translation units.
+template <int SRC, int WM, int WN, int LA, int LB>
+hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
+  constexpr int kLds = 2 * (64 * WM + 64 * WN) * 128;
+  auto kernel = tile_gemm_kernel<SRC, WM, WN, LA, LB>;
+  // > 64 KiB of dynamic LDS has to be enabled once per device; cheap enough to repeat per thread.
+  static thread_local int configured_device = -1;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  if (configured_device != device) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return e;
+    configured_device = device;
+  }
+  const int64_t grid = static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.batch * p.split_k;
+  if (grid <= 0 || grid > INT32_MAX) return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(256), kLds, stream, p);
+  return hipGetLastError();
+}
+
+template <int SRC>
+hipError_t launch_tile_class(const TileGemmParams& p, int tile, bool vec, hipStream_t stream) {
+  if (tile == 256)
+    return vec ? launch_tile_instance<SRC, 4, 4, LOAD_KVEC, LOAD_KVEC>(p, stream)
+               : launch_tile_instance<SRC, 4, 4, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
+  if (tile == 128)
+    return vec ? launch_tile_instance<SRC, 2, 2, LOAD_KVEC, LOAD_KVEC>(p, stream)
+               : launch_tile_instance<SRC, 2, 2, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
+  return vec ? launch_tile_instance<SRC, 1, 1, LOAD_KVEC, LOAD_KVEC>(p, stream)
+             : launch_tile_instance<SRC, 1, 1, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
+}
+
+}  // namespace vecops_hip
+#endif
