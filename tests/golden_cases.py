@@ -1,0 +1,101 @@
+"""Case table shared by tests/golden/make_golden.py (which ran the real vecops CPU
+matmul on these inputs) and the tests that compare the oracle and the GPU kernels
+with the stored outputs.  Inputs come from vecops_amd.synth seeds; shapes follow
+the reference's own tests (file:line per case)."""
+import os
+
+import numpy as np
+
+from vecops_amd import synth
+
+GOLDEN_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vecops_matmul_golden.npz")
+
+CASES = [
+    # tests/ops/MatmulTest.cpp:434-452 (microkernel shapes and K tails)
+    {"name": "bf16_37x51x79", "kind": "bf16_f32", "m": 37, "n": 51, "k": 79},
+    {"name": "bf16_1x128x65", "kind": "bf16_f32", "m": 1, "n": 128, "k": 65},
+    {"name": "bf16_512x1x256", "kind": "bf16_f32", "m": 512, "n": 1, "k": 256},
+    {"name": "bf16_96x16x67", "kind": "bf16_f32", "m": 96, "n": 16, "k": 67},
+    {"name": "bf16_130x270x1000", "kind": "bf16_f32", "m": 130, "n": 270, "k": 1000},
+    # BASELINE config 3 shapes scaled to fixture size (ragged M/N/K)
+    {"name": "bf16_77x100x301", "kind": "bf16_f32", "m": 77, "n": 100, "k": 301},
+    {"name": "bf16_255x63x819", "kind": "bf16_f32", "m": 255, "n": 63, "k": 819},
+    {"name": "bf16_300x300x17", "kind": "bf16_f32", "m": 300, "n": 300, "k": 17},
+    # bf16 output: RNE of the fp32 accumulator (tests/ops/MatmulConversionTestCommon.h:87-145)
+    {"name": "bf16out_64x96x160", "kind": "bf16_bf16", "m": 64, "n": 96, "k": 160},
+    # fp32 memory -> bf16 compute (the only fp32 path of the x86 backend)
+    {"name": "f32mem_33x65x257", "kind": "f32_f32", "m": 33, "n": 65, "k": 257},
+    {"name": "f32mem_bf16out_33x65x257", "kind": "f32_bf16", "m": 33, "n": 65, "k": 257},
+    # B handed over as [K,N] row-major (tests/ops/MatmulOrientationTest.cpp:65-70)
+    {"name": "bf16_nn_70x90x130", "kind": "bf16_f32", "m": 70, "n": 90, "k": 130, "b_layout": "kn"},
+    # A transposed in memory as well
+    {"name": "bf16_tn_70x90x130", "kind": "bf16_f32", "m": 70, "n": 90, "k": 130, "a_layout": "km"},
+    # inner stride 2, padded rows (tests/ops/MatmulTest.cpp:220-279)
+    {"name": "bf16_inner2_19x21x35", "kind": "bf16_f32", "m": 19, "n": 21, "k": 35, "inner": 2},
+    # rank 3, broadcast B / broadcast A (tests/ops/MatmulBatchTest.cpp:176-335)
+    {"name": "bf16_batch3_sharedB", "kind": "bf16_f32", "m": 19, "n": 21, "k": 35, "batch": 3, "share": "b"},
+    {"name": "bf16_batch3_sharedA", "kind": "bf16_f32", "m": 19, "n": 21, "k": 35, "batch": 3, "share": "a"},
+    {"name": "bf16_batch4", "kind": "bf16_f32", "m": 40, "n": 33, "k": 72, "batch": 4},
+    # explicit C input (ops/Matmul.h:144-146)
+    {"name": "bf16_cin_37x51x79", "kind": "bf16_f32", "m": 37, "n": 51, "k": 79, "cin": True},
+    # int8 (tests/ops/MatmulTest.cpp:1005-1023)
+    {"name": "i8_19x21x69", "kind": "i8_i32", "m": 19, "n": 21, "k": 69},
+    {"name": "i8_1x128x65", "kind": "i8_i32", "m": 1, "n": 128, "k": 65},
+    {"name": "i8_130x140x515", "kind": "i8_i32", "m": 130, "n": 140, "k": 515},
+    {"name": "i8_cin_35x53x257", "kind": "i8_i32", "m": 35, "n": 53, "k": 257, "cin": True},
+    {"name": "u8i8_19x21x69", "kind": "u8i8_i32", "m": 19, "n": 21, "k": 69},
+    # fused per-row x per-column dequantisation (tests/ops/MatmulConversionTestCommon.h:1437-1540)
+    {"name": "deq_67x129x515", "kind": "i8_dequant", "m": 67, "n": 129, "k": 515},
+    {"name": "deq_corr_67x129x515", "kind": "i8_dequant", "m": 67, "n": 129, "k": 515, "correction": True},
+    {"name": "deq_256x384x1024", "kind": "i8_dequant", "m": 256, "n": 384, "k": 1024},
+]
+
+
+def make_inputs(case: dict) -> dict:
+    m, n, k = case["m"], case["n"], case["k"]
+    kind = case["kind"]
+    batch = case.get("batch")
+    out = {}
+    if kind in ("bf16_f32", "bf16_bf16"):
+        gen = lambda seed, shape: synth.bf16_round(synth.uniform_pm1(seed, shape))  # noqa: E731
+    elif kind in ("f32_f32", "f32_bf16"):
+        gen = synth.uniform_pm1
+    else:
+        gen = synth.int8_sym
+    inner = case.get("inner", 1)
+    if batch:
+        share = case.get("share")
+        a = gen(1, (m, k)) if share == "a" else gen(1, (batch, m, k))
+        b = gen(2, (n, k)) if share == "b" else gen(2, (batch, n, k))
+        if share == "a":
+            a = np.broadcast_to(a, (batch, m, k))
+        if share == "b":
+            b = np.broadcast_to(b, (batch, n, k))
+        out["c_shape"] = (batch, m, n)
+    elif inner > 1:
+        a = gen(1, (m, inner * k + 3))[:, 0:inner * k:inner]
+        b = gen(2, (n, inner * k + 5))[:, 0:inner * k:inner]
+        out["c_shape"] = (m, n)
+    else:
+        a = gen(1, (m, k))
+        b = gen(2, (n, k))
+        if kind == "u8i8_i32":
+            a = (synth.draws(1, m * k) % np.uint64(256)).astype(np.uint8).reshape(m, k)
+        if case.get("a_layout") == "km":
+            a = np.ascontiguousarray(a.T).T
+        if case.get("b_layout") == "kn":
+            b = np.ascontiguousarray(b.T).T
+        out["c_shape"] = (m, n)
+    out["a"], out["b"] = a, b
+    if case.get("cin"):
+        if kind == "i8_i32":
+            out["cin"] = ((synth.draws(3, m * n) % np.uint64(200001)).astype(np.int64) - 100000).astype(
+                np.int32).reshape(m, n)
+        else:
+            out["cin"] = synth.uniform_pm1(3, (m, n))
+    if kind == "i8_dequant":
+        out["row_scales"] = synth.scales(3, m)
+        out["column_scales"] = synth.scales(4, n)
+        if case.get("correction"):
+            out["correction"] = ((synth.draws(5, n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32)
+    return out

@@ -1,0 +1,90 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header
+declares, and the kernel-selection rule table (a pure function) gives known answers."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from vecops_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "vecops_hip.h")).read()
+    return sorted(set(re.findall(r"VECOPS_HIP_EXPORT[^;(]*?\b(vecops_hip_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = capi.lib()
+    names = declared_symbols()
+    assert sorted(names) == sorted(capi.EXPORTS)
+    for name in names:
+        assert getattr(lib, name) is not None
+    assert lib.vecops_hip_abi_version() == 1
+
+
+def _operand(dtype, shape, strides=None, data=0x1000):
+    o = capi.Operand()
+    o.data, o.dtype, o.rank = data, dtype, len(shape)
+    if strides is None:
+        strides, acc = [], 1
+        for s in reversed(shape):
+            strides.insert(0, acc)
+            acc *= s
+    for i, (s, st) in enumerate(zip(shape, strides)):
+        o.sizes[i], o.strides[i] = s, st
+    return o
+
+
+def _plan(a, b, c, compute=0):
+    plan = capi.Plan()
+    rc = capi.lib().vecops_hip_plan_matmul(C.byref(a), C.byref(b), None, C.byref(c), compute, C.byref(plan))
+    return rc, plan
+
+
+def test_rule_table_known_answers():
+    # BASELINE config 2: 256 tiles of 256x256, one per compute unit
+    rc, p = _plan(_operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (4096, 4096)),
+                  _operand(capi.BF16, (4096, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256" and p.split_k == 1 and p.workspace_bytes == 0
+    assert p.vector_a == 1 and p.vector_b == 1
+    # config 4
+    rc, p = _plan(_operand(capi.I8, (2048, 4096)), _operand(capi.I8, (11008, 4096)),
+                  _operand(capi.I32, (2048, 11008)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256" and p.split_k == 1
+    # tiny output, long K (config 3's 255x63x8191): small tile and split-K with workspace
+    rc, p = _plan(_operand(capi.BF16, (255, 8191)), _operand(capi.BF16, (63, 8191)), _operand(capi.F32, (255, 63)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k > 1
+    assert p.workspace_bytes == p.split_k * 255 * 63 * 4
+    assert p.vector_a == 0                                   # 8191-element rows are not 16-byte aligned
+    # empty problems
+    rc, p = _plan(_operand(capi.BF16, (0, 64)), _operand(capi.BF16, (8, 64)), _operand(capi.F32, (0, 8)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "none"
+    rc, p = _plan(_operand(capi.BF16, (4, 0)), _operand(capi.BF16, (8, 0)), _operand(capi.F32, (4, 8)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "zero_k"
+    # B handed over as [K,N] row-major
+    rc, p = _plan(_operand(capi.BF16, (512, 512)), _operand(capi.BF16, (512, 512), (1, 512)),
+                  _operand(capi.F32, (512, 512)))
+    assert rc == 0 and p.b_layout == 1
+
+
+def test_plan_validation():
+    rc, _ = _plan(_operand(capi.BF16, (4, 8)), _operand(capi.BF16, (5, 9)), _operand(capi.F32, (4, 5)))
+    assert rc == 1 and b"K of a" in capi.lib().vecops_hip_last_error()
+    rc, _ = _plan(_operand(capi.BF16, (4, 8)), _operand(capi.BF16, (5, 8)), _operand(capi.F32, (4, 6)))
+    assert rc == 1
+    rc, _ = _plan(_operand(capi.BF16, (2, 4, 8)), _operand(capi.BF16, (3, 5, 8)), _operand(capi.F32, (2, 4, 5)))
+    assert rc == 1                                           # batch extents differ
+    rc, _ = _plan(_operand(capi.BF16, (4, 8)), _operand(capi.I8, (5, 8)), _operand(capi.F32, (4, 5)))
+    assert rc == 2                                           # NotApplicable: another recipe may take it
+    rc, _ = _plan(_operand(capi.I8, (4, 8)), _operand(capi.I8, (5, 8)), _operand(capi.F32, (4, 5)))
+    assert rc == 2
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIB_PATH", "/nonexistent/libvecops_hip.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        capi.lib()

@@ -1,0 +1,400 @@
+"""Parity of the gfx950 kernels, called through the C ABI (include/vecops_hip.h),
+with the CPU oracle on the same seeded inputs, plus size-independent properties
+at the full BASELINE sizes.
+
+Tolerances: integer paths and the dequantisation epilogue are bit-exact.  fp32
+outputs may differ from the oracle (fp64 accumulation) only through fp32
+summation order: |got - want| <= 2e-6 * max(1, K/32) * max(1, |want|, |got|),
+well inside the reference's own 8e-4 for fp32 outputs
+(tests/ops/MatmulConversionTestCommon.h:79-83).  bf16 outputs: one bf16 ulp
+(2^-7 relative; the reference allows 2e-2).
+"""
+import numpy as np
+import pytest
+
+from conftest import rel_err
+from oracle import oracle as O
+from vecops_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def fp32_tol(k):
+    return 2e-6 * max(1.0, k / 32)
+
+
+def dev_bf16(x_bits, device):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x_bits).view(np.int16)).to(device).view(torch.bfloat16)
+
+
+def host_bits(t):
+    import torch
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+REF_SHAPES = [(16, 16, 35), (16, 32, 67), (16, 48, 79), (1, 48, 79), (32, 16, 33), (48, 16, 65), (32, 32, 97),
+              (16, 64, 67), (16, 80, 67), (16, 96, 67), (64, 16, 67), (80, 16, 67), (96, 16, 67), (37, 51, 79),
+              (1, 128, 65), (512, 1, 256)]  # tests/ops/MatmulTest.cpp:434-452
+TILE_SHAPES = [(256, 256, 64), (257, 255, 65), (512, 768, 1024), (300, 520, 1000), (1000, 130, 2048),
+               (129, 129, 129), (64, 64, 8), (1024, 1024, 1024), (2048, 2048, 512)]
+
+
+@pytest.mark.parametrize("m,n,k", REF_SHAPES + TILE_SHAPES)
+def test_bf16_gemm_fp32_out(device, oracle, m, n, k):
+    import torch
+    from vecops_amd import capi
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul(dev_bf16(a, device), dev_bf16(b, device), c)
+    torch.cuda.synchronize()
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, acc_f64=True)
+    assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+
+
+@pytest.mark.parametrize("m,n,k", [(37, 51, 79), (256, 256, 256), (300, 520, 1000), (1024, 512, 2048)])
+def test_bf16_out_is_rne_of_fp32_out(device, oracle, m, n, k):
+    """Same kernel, same summation order: the bf16 output must be exactly the
+    round-to-nearest-even of the fp32 output (docs/Tensor.md:253-299)."""
+    import torch
+    from vecops_amd import capi
+    a = dev_bf16(synth.bf16_round(synth.uniform_pm1(1, (m, k))), device)
+    b = dev_bf16(synth.bf16_round(synth.uniform_pm1(2, (n, k))), device)
+    c32 = torch.empty((m, n), dtype=torch.float32, device=device)
+    c16 = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    capi.matmul(a, b, c32)
+    capi.matmul(a, b, c16)
+    torch.cuda.synchronize()
+    assert np.array_equal(host_bits(c16), oracle.bf16_from_f32(c32.cpu().numpy()))
+
+
+def test_fp32_memory_bf16_compute(device, oracle):
+    import torch
+    from vecops_amd import capi
+    for (m, n, k) in [(33, 65, 257), (256, 384, 512), (1024, 1024, 1024)]:
+        a, b = synth.uniform_pm1(1, (m, k)), synth.uniform_pm1(2, (n, k))
+        c = torch.empty((m, n), dtype=torch.float32, device=device)
+        capi.matmul(torch.from_numpy(a).to(device), torch.from_numpy(b).to(device), c, compute=capi.COMPUTE_BF16)
+        torch.cuda.synchronize()
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want, atom=O.ATOM_BF16F32, acc_f64=True)
+        assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+        # B as [K,N] row-major (BASELINE config 1 layout)
+        b_kn = torch.from_numpy(np.ascontiguousarray(b.T)).to(device)
+        c2 = torch.empty((m, n), dtype=torch.float32, device=device)
+        capi.matmul(torch.from_numpy(a).to(device), b_kn.t(), c2)
+        torch.cuda.synchronize()
+        assert rel_err(c2.cpu().numpy(), want) <= fp32_tol(k)
+
+
+@pytest.mark.parametrize("layout", ["nn", "tn", "tt", "inner2", "padded", "c_transposed", "offset2"])
+def test_layouts(device, oracle, layout):
+    """Strided views give the values of dense copies (tests/ops/MatmulOrientationTest.cpp:139,249;
+    tests/ops/MatmulTest.cpp:220-279)."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = 70, 90, 130
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, acc_f64=True)
+    ta, tb = dev_bf16(a, device), dev_bf16(b, device)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    if layout in ("nn", "tt"):
+        tb = tb.t().contiguous().t()
+    if layout in ("tn", "tt"):
+        ta = ta.t().contiguous().t()
+    if layout == "inner2":
+        big_a = torch.zeros((m, 2 * k + 3), dtype=torch.bfloat16, device=device)
+        big_b = torch.zeros((n, 2 * k + 5), dtype=torch.bfloat16, device=device)
+        big_a[:, 0:2 * k:2] = ta
+        big_b[:, 0:2 * k:2] = tb
+        ta, tb = big_a[:, 0:2 * k:2], big_b[:, 0:2 * k:2]
+    if layout == "padded":
+        big_a = torch.zeros((m, k + 8), dtype=torch.bfloat16, device=device)
+        big_a[:, :k] = ta
+        ta = big_a[:, :k]
+    if layout == "offset2":  # rows start 2 bytes off a 16-byte boundary
+        flat = torch.zeros(m * k + 1, dtype=torch.bfloat16, device=device)
+        flat[1:] = ta.reshape(-1)
+        ta = flat[1:].view(m, k)
+    if layout == "c_transposed":
+        c = torch.full((n, m), float("nan"), dtype=torch.float32, device=device).t()
+    capi.matmul(ta, tb, c)
+    torch.cuda.synchronize()
+    assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+
+
+def test_batched_and_broadcast(device, oracle):
+    """Rank 3: independent products over the batch; stride 0 broadcasts an operand
+    (tests/ops/MatmulBatchTest.cpp:176-335)."""
+    import torch
+    from vecops_amd import capi
+    batch, m, n, k = 5, 45, 67, 200
+    a = synth.bf16_round(synth.uniform_pm1(1, (batch, m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (batch, n, k)))
+    for share in (None, "a", "b"):
+        ha = np.broadcast_to(a[0], a.shape) if share == "a" else a
+        hb = np.broadcast_to(b[0], b.shape) if share == "b" else b
+        ta = dev_bf16(a[0], device).expand(batch, m, k) if share == "a" else dev_bf16(a, device)
+        tb = dev_bf16(b[0], device).expand(batch, n, k) if share == "b" else dev_bf16(b, device)
+        c = torch.full((batch, m, n), float("nan"), dtype=torch.float32, device=device)
+        capi.matmul(ta, tb, c)
+        torch.cuda.synchronize()
+        want = np.zeros((batch, m, n), np.float32)
+        oracle.matmul(ha, hb, want, acc_f64=True)
+        assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+    # batch == 0: nothing to do, no error (ArchitectureFamily.h:1935-1938)
+    capi.matmul(torch.empty((0, m, k), dtype=torch.bfloat16, device=device),
+                torch.empty((0, n, k), dtype=torch.bfloat16, device=device),
+                torch.empty((0, m, n), dtype=torch.float32, device=device))
+
+
+@pytest.mark.parametrize("m,n,k", [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)])
+def test_config3_irregular_batch8(device, oracle, m, n, k):
+    """BASELINE config 3 at full size: batch 8, bf16 in, fp32 out.  All eight
+    products run on the GPU; the oracle checks batches 0 and 7 in full."""
+    import torch
+    from vecops_amd import capi
+    batch = 8
+    a = synth.bf16_round(synth.uniform_pm1(1, (batch, m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (batch, n, k)))
+    c = torch.full((batch, m, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul(dev_bf16(a, device), dev_bf16(b, device), c)
+    torch.cuda.synchronize()
+    got = c.cpu().numpy()
+    assert np.isfinite(got).all()
+    for bi in (0, 7):
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a[bi], b[bi], want, acc_f64=True)
+        assert rel_err(got[bi], want) <= fp32_tol(k)
+
+
+def test_explicit_c_input_and_aliasing(device, oracle):
+    import torch
+    from vecops_amd import capi
+    for (m, n, k) in [(37, 51, 79), (300, 260, 512)]:
+        a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+        b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+        cin = synth.uniform_pm1(3, (m, n))
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want, cin=cin, acc_f64=True)
+        c = torch.from_numpy(cin.copy()).to(device)
+        capi.matmul(dev_bf16(a, device), dev_bf16(b, device), c, c_in=c)   # Cin aliases Cout
+        torch.cuda.synchronize()
+        assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+        # a broadcast row as C input (bias): stride 0 over rows
+        bias = torch.from_numpy(cin[0].copy()).to(device)
+        c2 = torch.empty((m, n), dtype=torch.float32, device=device)
+        capi.matmul(dev_bf16(a, device), dev_bf16(b, device), c2, c_in=bias.expand(m, n))
+        torch.cuda.synchronize()
+        want2 = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want2, cin=np.broadcast_to(cin[0], (m, n)), acc_f64=True)
+        assert rel_err(c2.cpu().numpy(), want2) <= fp32_tol(k)
+
+
+def test_zero_extents(device):
+    """K == 0 writes zeros (single C) or C_in (explicit C); zero M or N writes nothing
+    (ops/Matmul.h:41-43; tests/ops/MatmulTest.cpp:456-457)."""
+    import torch
+    from vecops_amd import capi
+    bf = torch.bfloat16
+    c = torch.full((4, 5), 3.0, dtype=torch.float32, device=device)
+    capi.matmul(torch.empty((4, 0), dtype=bf, device=device), torch.empty((5, 0), dtype=bf, device=device), c)
+    torch.cuda.synchronize()
+    assert torch.equal(c, torch.zeros_like(c))
+    cin = torch.full((4, 5), 2.5, dtype=torch.float32, device=device)
+    capi.matmul(torch.empty((4, 0), dtype=bf, device=device), torch.empty((5, 0), dtype=bf, device=device), c,
+                c_in=cin)
+    torch.cuda.synchronize()
+    assert torch.equal(c, cin)
+    capi.matmul(torch.empty((0, 16), dtype=bf, device=device), torch.empty((5, 16), dtype=bf, device=device),
+                torch.empty((0, 5), dtype=torch.float32, device=device))
+    capi.matmul(torch.empty((4, 16), dtype=bf, device=device), torch.empty((0, 16), dtype=bf, device=device),
+                torch.empty((4, 0), dtype=torch.float32, device=device))
+    torch.cuda.synchronize()
+
+
+def test_invalid_arguments_are_rejected(device):
+    import torch
+    from vecops_amd import capi
+    bf = torch.bfloat16
+    a = torch.zeros((4, 8), dtype=bf, device=device)
+    with pytest.raises(capi.VecopsHipError) as e:
+        capi.matmul(a, torch.zeros((5, 9), dtype=bf, device=device), torch.zeros((4, 5), device=device))
+    assert e.value.code == 1
+    with pytest.raises(capi.VecopsHipError) as e:
+        capi.matmul(a, torch.zeros((5, 8), dtype=bf, device=device), torch.zeros((4, 6), device=device))
+    assert e.value.code == 1
+    with pytest.raises(capi.VecopsHipError) as e:  # dtype combination outside the path
+        capi.matmul(a, torch.zeros((5, 8), dtype=torch.int8, device=device), torch.zeros((4, 5), device=device))
+    assert e.value.code == 2
+
+
+# --- int8 -------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("m,n,k", [(19, 21, 69), (1, 128, 65), (128, 1, 65), (1, 16, 129), (35, 53, 257),
+                                   (256, 256, 128), (300, 520, 1000), (1024, 768, 4096), (130, 140, 515)])
+def test_int8_gemm_bit_exact(device, oracle, m, n, k):
+    import torch
+    from vecops_amd import capi
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    c = torch.full((m, n), -1, dtype=torch.int32, device=device)
+    capi.matmul(torch.from_numpy(a).to(device), torch.from_numpy(b).to(device), c)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy(), oracle.matmul_i8_dense(a, b))
+
+
+def test_int32_accumulator_wraps(device):
+    """tests/ops/MatmulTest.cpp:1025-1055: 262145 products of 127*127 wrap mod 2^32."""
+    import torch
+    from vecops_amd import capi
+    K = 262145
+    a = torch.full((1, K), 127, dtype=torch.int8, device=device)
+    c = torch.zeros((1, 1), dtype=torch.int32, device=device)
+    capi.matmul(a, a.clone(), c)
+    torch.cuda.synchronize()
+    assert int(c.item()) == int(np.uint32((127 * 127 * K) % 2 ** 32).astype(np.int32))
+    # a full tile of wrapping accumulators
+    m = n = 64
+    am = torch.full((m, K), 127, dtype=torch.int8, device=device)
+    cm = torch.zeros((m, n), dtype=torch.int32, device=device)
+    capi.matmul(am, am.clone(), cm)
+    torch.cuda.synchronize()
+    assert (cm.cpu().numpy() == np.uint32((127 * 127 * K) % 2 ** 32).astype(np.int32)).all()
+
+
+def test_int8_c_input(device, oracle):
+    import torch
+    from vecops_amd import capi
+    m, n, k = 35, 53, 257
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    cin = ((synth.draws(3, m * n) % np.uint64(200001)).astype(np.int64) - 100000).astype(np.int32).reshape(m, n)
+    c = torch.zeros((m, n), dtype=torch.int32, device=device)
+    capi.matmul(torch.from_numpy(a).to(device), torch.from_numpy(b).to(device), c,
+                c_in=torch.from_numpy(cin).to(device))
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy(), oracle.matmul_i8_dense(a, b) + cin)
+
+
+@pytest.mark.parametrize("m,n,k,corr", [(67, 129, 515, False), (67, 129, 515, True), (256, 384, 1024, False),
+                                        (300, 1000, 2048, True), (1, 300, 4096, False), (16, 64, 100, True)])
+def test_int8_dequant_bit_exact(device, oracle, m, n, k, corr):
+    import torch
+    from vecops_amd import capi
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    rs, cs = synth.scales(3, m), synth.scales(4, n)
+    correction = ((synth.draws(5, n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32) if corr else None
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul_i8_dequant(torch.from_numpy(a).to(device), torch.from_numpy(b).to(device),
+                           torch.from_numpy(rs).to(device), torch.from_numpy(cs).to(device), c,
+                           correction=torch.from_numpy(correction).to(device) if corr else None)
+    torch.cuda.synchronize()
+    want = oracle.matmul_i8_dequant(a, b, rs, cs, correction)
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+# --- full BASELINE sizes: size-independent properties -------------------------------------
+
+def test_config2_bf16_4096_sampled_and_linear(device, oracle):
+    """bf16 4096^3, B given as [K,N] row-major, bf16 out: 4096 sampled outputs
+    against the oracle, and the whole output against fp32-out of the same kernel."""
+    import torch
+    from vecops_amd import capi
+    n = 4096
+    a = synth.bf16_round(synth.normal(1, (n, n), 0.02))
+    b_kn = synth.bf16_round(synth.normal(2, (n, n), 0.02))      # [K, N]
+    ta, tb = dev_bf16(a, device), dev_bf16(b_kn, device).t()    # strided [N, K] view
+    c16 = torch.empty((n, n), dtype=torch.bfloat16, device=device)
+    c32 = torch.empty((n, n), dtype=torch.float32, device=device)
+    capi.matmul(ta, tb, c16)
+    capi.matmul(ta, tb, c32)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(7)
+    rows, cols = rng.integers(0, n, 4096), rng.integers(0, n, 4096)
+    rows[:8] = [0, 0, n - 1, n - 1, 255, 256, 2047, 2048]
+    cols[:8] = [0, n - 1, 0, n - 1, 256, 255, 2048, 2047]
+    want = oracle.matmul_sampled(a, b_kn.T, rows, cols)
+    got32 = c32.cpu().numpy()
+    assert rel_err(got32[rows, cols], want) <= fp32_tol(n)
+    assert np.array_equal(host_bits(c16), oracle.bf16_from_f32(got32))
+    # linearity: (2A) B == 2 (A B) exactly in binary floating point
+    c32b = torch.empty_like(c32)
+    capi.matmul(ta * 2, tb, c32b)
+    torch.cuda.synchronize()
+    assert torch.equal(c32b, c32 * 2)
+
+
+def test_config4_int8_full_size_checksum(device, oracle):
+    """int8 2048x4096x11008: every int32 accumulator is checked by a checksum of
+    checksums that is exact mod 2^32 (C v == A (B^T v) for a random integer v), the
+    dequantised output is checked bit-for-bit against the epilogue applied to those
+    accumulators, and 64 whole rows are compared with the oracle."""
+    import torch
+    from vecops_amd import capi
+    m, k, n = 2048, 4096, 11008
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    rs, cs = synth.scales(3, m), synth.scales(4, n)
+    ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    acc = torch.empty((m, n), dtype=torch.int32, device=device)
+    capi.matmul(ta, tb, acc)
+    out = torch.empty((m, n), dtype=torch.float32, device=device)
+    trs, tcs = torch.from_numpy(rs).to(device), torch.from_numpy(cs).to(device)
+    capi.matmul_i8_dequant(ta, tb, trs, tcs, out)
+    torch.cuda.synchronize()
+    # checksum of checksums in int64 (no overflow: |v| < 2^15, |sum| < 2^63), reduced mod 2^32
+    v = torch.from_numpy((synth.draws(9, n) % np.uint64(32768)).astype(np.int64)).to(device)
+    lhs = (acc.to(torch.int64) * v[None, :]).sum(dim=1)
+    btv = (tb.to(torch.int64) * v[:, None]).sum(dim=0)          # [K]
+    rhs = (ta.to(torch.int64) * btv[None, :]).sum(dim=1)
+    assert torch.equal(lhs & 0xFFFFFFFF, rhs & 0xFFFFFFFF)
+    w = torch.from_numpy((synth.draws(10, m) % np.uint64(32768)).astype(np.int64)).to(device)
+    lhs2 = (acc.to(torch.int64) * w[:, None]).sum(dim=0)
+    atw = (ta.to(torch.int64) * w[:, None]).sum(dim=0)
+    rhs2 = (tb.to(torch.int64) * atw[None, :]).sum(dim=1)
+    assert torch.equal(lhs2 & 0xFFFFFFFF, rhs2 & 0xFFFFFFFF)
+    # epilogue: two IEEE fp32 multiplies, row scale first
+    expect = (acc.to(torch.float32) * trs[:, None]) * tcs[None, :]
+    assert torch.equal(out.view(torch.int32), expect.view(torch.int32))
+    rows = np.r_[0:32, m - 32:m]
+    want = oracle.matmul_i8_dequant(a[rows], b, rs[rows], cs)
+    assert np.array_equal(out[torch.from_numpy(rows).to(device)].cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+# --- weight-only int8, per-group scales (no reference counterpart: parity unpinned) ------------
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 8, 16])
+@pytest.mark.parametrize("n,k,group", [(14336, 4096, 128), (300, 512, 64), (17, 1024, 128), (4096, 11008, 128)])
+def test_w8a16_group(device, oracle, m, n, k, group):
+    """Checked against the fp64 brute force of the stated contract: fp32 accumulation
+    over K=4096 plus the final bf16 rounding stay within one bf16 ulp (2^-7) of it."""
+    import torch
+    from vecops_amd import capi
+    if n * k > 20e6 and m not in (1, 4, 16):
+        pytest.skip("large case only at the BASELINE M values")
+    x = synth.bf16_round(synth.normal(1, (m, k)))
+    w = synth.int8_sym(2, (n, k))
+    s = synth.scales(3, (n, k // group))
+    y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=device)
+    capi.matmul_w8a16_group(dev_bf16(x, device), torch.from_numpy(w).to(device), torch.from_numpy(s).to(device), y,
+                            group)
+    torch.cuda.synchronize()
+    _, want = oracle.matmul_w8a16_group(x, w, s, group)
+    assert rel_err(synth.bf16_to_f32(host_bits(y)), want) <= 2 ** -7
+
+
+def test_w8a16_rejects_bad_arguments(device):
+    import torch
+    from vecops_amd import capi
+    x = torch.zeros((17, 256), dtype=torch.bfloat16, device=device)
+    w = torch.zeros((8, 256), dtype=torch.int8, device=device)
+    s = torch.zeros((8, 2), device=device)
+    y = torch.zeros((17, 8), dtype=torch.bfloat16, device=device)
+    with pytest.raises(capi.VecopsHipError) as e:
+        capi.matmul_w8a16_group(x, w, s, y, 128)
+    assert e.value.code == 2                                   # m > 16 is another kernel family
+    with pytest.raises(capi.VecopsHipError) as e:
+        capi.matmul_w8a16_group(x[:4], w, s, y[:4], 100)
+    assert e.value.code == 1
