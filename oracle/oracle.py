@@ -94,6 +94,8 @@ class Oracle:
         for name in ("vo_amx_small_vector_profitable", "vo_sme_small_vector_profitable"):
             getattr(L, name).argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64]
         L.vo_small_area_profitable.argtypes = [C.c_int64] * 4
+        L.vo_threads.restype = C.c_int
+        L.vo_matmul_bf16_dense.argtypes = [C.c_void_p] * 4 + [C.c_int64] * 3
         L.vo_amx_residual_split_profitable.argtypes = [C.c_int64] * 3
 
     # -- conversions ---------------------------------------------------------
@@ -128,6 +130,20 @@ class Oracle:
         if rc != 0:
             raise ValueError("vo_matmul_sampled rejected the operand shapes")
         return out
+
+    def threads(self) -> int:
+        return int(self.lib.vo_threads())
+
+    def matmul_bf16_dense(self, a_bits: np.ndarray, b_bits: np.ndarray, out_bf16: bool = False) -> np.ndarray:
+        """Vectorised all-core bf16 product on dense operands (CPU-baseline kernel)."""
+        a_bits = np.ascontiguousarray(a_bits, dtype=np.uint16)
+        b_bits = np.ascontiguousarray(b_bits, dtype=np.uint16)
+        m, k = a_bits.shape
+        n = b_bits.shape[0]
+        c = np.empty((m, n), dtype=np.uint16 if out_bf16 else np.float32)
+        self.lib.vo_matmul_bf16_dense(a_bits.ctypes.data, b_bits.ctypes.data, None if out_bf16 else c.ctypes.data,
+                                      c.ctypes.data if out_bf16 else None, m, n, k)
+        return c
 
     def matmul_i8_dense(self, a: np.ndarray, b: np.ndarray) -> np.ndarray:
         a = np.ascontiguousarray(a, dtype=np.int8)

@@ -375,3 +375,37 @@ VO_EXPORT int vo_amx_residual_split_profitable(int64_t m, int64_t n, int64_t k) 
   const int tm = n == 17 || n == 18 || n == 20, tn = m == 33 || m == 47 || m == 48;
   return ((sm && sn) || (tm && tn)) && k == 1024;
 }
+
+/* ---- CPU-baseline kernels (timed by the benchmark, never used as a checker of
+ * themselves): the same semantics as vo_matmul on dense K-contiguous operands,
+ * written so the compiler vectorises them across all host cores. -------------- */
+#include <omp.h>
+
+VO_EXPORT int vo_threads(void) { return omp_get_max_threads(); }
+
+/* bf16 x bf16 -> fp32 accumulate -> fp32 or bf16 out (AMX_BF16F32 semantics,
+ * vectorised summation order). */
+VO_EXPORT void vo_matmul_bf16_dense(const uint16_t* a, const uint16_t* b, float* c_f32, uint16_t* c_bf16, int64_t M,
+                                    int64_t N, int64_t K) {
+  float* bf = (float*)malloc((size_t)N * K * sizeof(float));
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < N * K; ++i) bf[i] = vo_f32_from_bf16(b[i]);
+#pragma omp parallel
+  {
+    float* ar = (float*)malloc((size_t)K * sizeof(float));
+#pragma omp for schedule(dynamic, 1)
+    for (int64_t i = 0; i < M; ++i) {
+      for (int64_t k = 0; k < K; ++k) ar[k] = vo_f32_from_bf16(a[i * K + k]);
+      for (int64_t j = 0; j < N; ++j) {
+        const float* br = bf + j * K;
+        float acc = 0.0f;
+#pragma omp simd reduction(+ : acc)
+        for (int64_t k = 0; k < K; ++k) acc += ar[k] * br[k];
+        if (c_f32) c_f32[i * N + j] = acc;
+        if (c_bf16) c_bf16[i * N + j] = vo_bf16_from_f32(acc);
+      }
+    }
+    free(ar);
+  }
+  free(bf);
+}

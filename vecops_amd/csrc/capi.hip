@@ -66,6 +66,14 @@ bool k_vector_ok(const View& v) {
   return v.cs == 1 && v.rs % per == 0 && v.bs % per == 0 && aligned16(v.data);
 }
 
+// B stored [K,N] row-major: unit stride along N, N a multiple of 8 elements, K stride,
+// batch stride and base multiples of 16 bytes (16-bit or 32-bit source elements).
+bool n_vector_ok(const View& v) {
+  const int64_t eb = dtype_bytes(v.dtype);
+  const int64_t per = 16 / eb;
+  return v.rs == 1 && v.rows % 8 == 0 && v.rows >= 8 && v.cs % per == 0 && v.bs % per == 0 && aligned16(v.data);
+}
+
 struct Problem {
   View a, b, c, cin;
   bool has_cin;
@@ -156,7 +164,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     return;
   }
   plan->vector_a = k_vector_ok(pr.a) ? 1 : 0;
-  plan->vector_b = k_vector_ok(pr.b) ? 1 : 0;
+  plan->vector_b = (k_vector_ok(pr.b) || (pr.b.rs == 1 && pr.b.cs != 1 && n_vector_ok(pr.b) && pr.src != SRC_I8)) ? 1 : 0;
   plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
 
   auto tiles = [&](int64_t t) { return ((pr.m + t - 1) / t) * ((pr.n + t - 1) / t) * pr.batch; };
@@ -237,13 +245,15 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   const int k_tiles = static_cast<int>((pr.k + ktile - 1) / ktile);
   p.split_k = static_cast<int32_t>(plan.split_k);
   p.k_tiles_per_split = (k_tiles + p.split_k - 1) / p.split_k;
-  const bool vec = plan.vector_a && plan.vector_b;
+  int mode = MODE_GENERIC;
+  if (plan.vector_a && k_vector_ok(pr.b)) mode = MODE_KVEC;
+  else if (plan.vector_a && plan.vector_b && plan.b_layout == 1) mode = MODE_NVEC_B;
 
   hipError_t e;
   switch (pr.src) {
-    case SRC_BF16: e = launch_tile_gemm_bf16(p, tile, vec, stream); break;
-    case SRC_F32_AS_BF16: e = launch_tile_gemm_f32_as_bf16(p, tile, vec, stream); break;
-    default: e = launch_tile_gemm_i8(p, tile, vec, stream); break;
+    case SRC_BF16: e = launch_tile_gemm_bf16(p, tile, mode, stream); break;
+    case SRC_F32_AS_BF16: e = launch_tile_gemm_f32_as_bf16(p, tile, mode, stream); break;
+    default: e = launch_tile_gemm_i8(p, tile, mode, stream); break;
   }
   if (e != hipSuccess) return fail(ST_EXEC, "tile kernel launch: %s", hipGetErrorString(e));
   if (p.split_k > 1) {

@@ -98,7 +98,14 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-__device__ __forceinline__ int lds_chunk_offset(int row, int chunk) { return row * 128 + (((chunk ^ row) & 7) << 4); }
+// LDS byte offset of 16-byte chunk `chunk` (0..7) of tile row `row`.  The chunk
+// slot is XOR-swizzled with (row ^ row/8): eight consecutive rows at one logical
+// chunk (the MFMA fragment read), the eight chunks of one row (the K-contiguous
+// staging write) and eight rows 8 apart at one chunk (the transposing staging
+// write) all land in eight different 16-byte slots of the 128-byte bank period.
+__device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
+  return row * 128 + (((chunk ^ row ^ (row >> 3)) & 7) << 4);
+}
 
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
@@ -269,25 +276,33 @@ __device__ __forceinline__ void map_workgroup(const TileGemmParams& p, int& batc
   tn = in_band / rows_in_band;
 }
 
-// Per-thread staging plan for one operand: thread t stages chunk (t & 7) of rows
-// (t >> 3) + 32*i.  Rows past the operand's extent are clamped to its last row:
-// they are loaded but only feed accumulator rows/columns that are never stored.
-template <int SRC, int LOAD, int CHUNKS>
-struct OperandStager {
-  const char* base;     // operand base for this batch
-  int64_t row_bytes[CHUNKS];  // byte offset of each staged row (fast path)
-  int64_t rs, ks;       // element strides (checked path)
-  int first_row, extent, k_end;
+// Staging of one operand tile (ROWS rows x 128 bytes) from global memory into
+// LDS.  A stager owns the registers that hold a fetched tile between fetch() and
+// commit().  Rows past the operand's extent are clamped to its last row on the
+// fast paths: they are loaded but only feed accumulator rows/columns that are
+// never stored.
+//
+// LOAD_KVEC / LOAD_GENERIC: thread t stages chunk (t & 7) of rows (t >> 3) + 32*i.
+template <int SRC, int LOAD, int ROWS>
+struct Stager {
+  using T = SrcTraits<SRC>;
+  static constexpr int CHUNKS = ROWS / 32;
+  const char* base;
+  int64_t row_bytes[CHUNKS];  // byte offset of each staged row, chunk included (fast path)
+  int64_t rs, ks;             // element strides (checked path)
+  int first_row, extent, k_end, ld_row, ld_chunk;
+  u32x4 regs[CHUNKS];
 
   __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
-                                       int k_end_, int ld_row, int ld_chunk) {
-    using T = SrcTraits<SRC>;
+                                       int k_end_, int tid) {
     base = static_cast<const char*>(base_);
     rs = rs_;
     ks = ks_;
     first_row = first_row_;
     extent = extent_;
     k_end = k_end_;
+    ld_chunk = tid & 7;
+    ld_row = tid >> 3;
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int row = min(first_row + ld_row + i * 32, extent - 1);
@@ -295,33 +310,105 @@ struct OperandStager {
     }
   }
 
-  // Whole K tile inside [0, K): unconditional 16-byte loads.
-  __device__ __forceinline__ void fetch_fast(u32x4 (&stage)[CHUNKS], int kt) const {
-    using T = SrcTraits<SRC>;
-    const int64_t k_bytes = static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes);
+  __device__ __forceinline__ void fetch(int kt, int full_k_tiles) {
+    if constexpr (LOAD == LOAD_KVEC) {
+      if (kt < full_k_tiles) {  // whole K tile inside [0, K): unconditional 16-byte loads
+        const int64_t k_bytes = static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes);
 #pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) stage[i] = load_chunk_fast<SRC>(base + row_bytes[i] + k_bytes);
-  }
-
-  __device__ __forceinline__ void fetch_checked(u32x4 (&stage)[CHUNKS], int kt, int ld_row, int ld_chunk) const {
-    using T = SrcTraits<SRC>;
+        for (int i = 0; i < CHUNKS; ++i) regs[i] = load_chunk_fast<SRC>(base + row_bytes[i] + k_bytes);
+        return;
+      }
+    }
     const int k0 = kt * 8 * T::kElemsPerChunk + ld_chunk * T::kElemsPerChunk;
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int row = first_row + ld_row + i * 32;
-      stage[i] = load_chunk_checked<SRC>(base, static_cast<int64_t>(row) * rs, ks, k0, k_end, row < extent);
+      regs[i] = load_chunk_checked<SRC>(base, static_cast<int64_t>(row) * rs, ks, k0, k_end, row < extent);
     }
   }
 
-  __device__ __forceinline__ void fetch(u32x4 (&stage)[CHUNKS], int kt, int full_k_tiles, int ld_row,
-                                        int ld_chunk) const {
-    if constexpr (LOAD == LOAD_KVEC) {
-      if (kt < full_k_tiles) {
-        fetch_fast(stage, kt);
-        return;
-      }
+  __device__ __forceinline__ void commit(char* lds_tile) const {
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i)
+      *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(ld_row + i * 32, ld_chunk)) = regs[i];
+  }
+};
+
+// LOAD_NVEC: the operand is stored with its spatial index contiguous (B handed
+// over as [K,N] row-major).  Thread t < ROWS owns one 8(k) x 8(n) block of the
+// tile: it loads eight 16-byte rows along n, transposes the block in registers
+// with byte permutes and writes eight K-contiguous chunks.  16-bit compute
+// elements only (bf16, or fp32 rounded to bf16 on load).
+template <int SRC, int ROWS>
+struct Stager<SRC, LOAD_NVEC, ROWS> {
+  using T = SrcTraits<SRC>;
+  static_assert(T::kElemsPerChunk == 8, "transposing stager handles 16-bit compute elements");
+  static constexpr int NBLOCKS = ROWS / 8;
+  const char* base;
+  const char* block_ptr;  // address of (k-block row 0, n-block) for K tile 0
+  int64_t rs, ks;         // rs == 1; ks = elements between consecutive k
+  int first_row, extent, k_end, nb, kb, tid_;
+  bool active;
+  u32x4 regs[8];
+
+  __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
+                                       int k_end_, int tid) {
+    base = static_cast<const char*>(base_);
+    rs = rs_;
+    ks = ks_;
+    first_row = first_row_;
+    extent = extent_;
+    k_end = k_end_;
+    tid_ = tid;
+    active = tid < ROWS;
+    nb = tid % NBLOCKS;
+    kb = (tid / NBLOCKS) & 7;
+    const int n = min(first_row + nb * 8, extent - 8);  // extent is a multiple of 8 on this path
+    block_ptr = base + (static_cast<int64_t>(kb) * 8 * ks + n) * T::kSrcBytes;
+  }
+
+  __device__ __forceinline__ void fetch(int kt, int full_k_tiles) {
+    if (!active) return;
+    if (kt < full_k_tiles) {
+      const char* p = block_ptr + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) regs[r] = load_chunk_fast<SRC>(p + r * ks * T::kSrcBytes);
+      return;
     }
-    fetch_checked(stage, kt, ld_row, ld_chunk);
+    // K tail: rows k >= K read as zero, columns n >= N as zero
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int k = kt * 64 + kb * 8 + r;
+      uint32_t w[4] = {0u, 0u, 0u, 0u};
+      if (k < k_end) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int n = first_row + nb * 8 + e;
+          if (n < extent) {
+            uint32_t v;
+            if constexpr (SRC == SRC_BF16) v = reinterpret_cast<const uint16_t*>(base)[k * ks + n];
+            else v = cvt_pk_bf16(reinterpret_cast<const float*>(base)[k * ks + n], 0.0f) & 0xffffu;
+            w[e >> 1] |= v << ((e & 1) * 16);
+          }
+        }
+      }
+      regs[r] = u32x4{w[0], w[1], w[2], w[3]};
+    }
+  }
+
+  __device__ __forceinline__ void commit(char* lds_tile) const {
+    if (!active) return;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      // output chunk for n-row e: dword j = (regs[2j][e], regs[2j+1][e])
+      const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+      u32x4 out;
+      out.x = __builtin_amdgcn_perm(regs[1][e >> 1], regs[0][e >> 1], sel);
+      out.y = __builtin_amdgcn_perm(regs[3][e >> 1], regs[2][e >> 1], sel);
+      out.z = __builtin_amdgcn_perm(regs[5][e >> 1], regs[4][e >> 1], sel);
+      out.w = __builtin_amdgcn_perm(regs[7][e >> 1], regs[6][e >> 1], sel);
+      *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(nb * 8 + e, kb)) = out;
+    }
   }
 };
 
@@ -333,7 +420,6 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
   constexpr int EPC = T::kElemsPerChunk;
   constexpr int KTILE = 8 * EPC;  // elements per K tile
   constexpr int BM = 64 * WM, BN = 64 * WN;
-  constexpr int A_CHUNKS = BM / 32, B_CHUNKS = BN / 32;  // 16-byte chunks each thread stages per tile
   constexpr int STAGE_BYTES = (BM + BN) * 128;
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -352,16 +438,10 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
   const int kt_begin = split * p.k_tiles_per_split;
   const int kt_end = min(total_k_tiles, kt_begin + p.k_tiles_per_split);
 
-  // staging assignment: thread -> (chunk column, 32-row stripe)
-  const int ld_chunk = tid & 7;
-  const int ld_row = tid >> 3;
-
-  OperandStager<SRC, LOAD_A, A_CHUNKS> stager_a;
-  OperandStager<SRC, LOAD_B, B_CHUNKS> stager_b;
-  stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, ld_row,
-                ld_chunk);
-  stager_b.init(static_cast<const char*>(p.b) + batch * p.b_bs * T::kSrcBytes, p.b_rs, p.b_ks, n0, p.n, p.k, ld_row,
-                ld_chunk);
+  Stager<SRC, LOAD_A, BM> stager_a;
+  Stager<SRC, LOAD_B, BN> stager_b;
+  stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, tid);
+  stager_b.init(static_cast<const char*>(p.b) + batch * p.b_bs * T::kSrcBytes, p.b_rs, p.b_ks, n0, p.n, p.k, tid);
 
   Acc acc[WM][WN];
 #pragma unroll
@@ -371,20 +451,20 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-  u32x4 stage_a[A_CHUNKS], stage_b[B_CHUNKS];
-
-  // LDS byte offsets this thread writes (stage 0) and reads (stage 0, k-step 0)
-  const int st_off = lds_chunk_offset(ld_row, ld_chunk);  // + i*32*128 per chunk row
   const int frag_row = lane & 31;
   const int frag_half = lane >> 5;
+  // LDS offsets of this lane's fragments at k-step 0; k-step ks flips bits 5-6: off ^ (ks << 5)
+  int off_a[WM], off_b[WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i) off_a[i] = lds_chunk_offset((wm * WM + i) * 32 + frag_row, frag_half);
+#pragma unroll
+  for (int j = 0; j < WN; ++j) off_b[j] = BM * 128 + lds_chunk_offset((wn * WN + j) * 32 + frag_row, frag_half);
 
   if (kt_begin < kt_end) {
-    stager_a.fetch(stage_a, kt_begin, full_k_tiles, ld_row, ld_chunk);
-    stager_b.fetch(stage_b, kt_begin, full_k_tiles, ld_row, ld_chunk);
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<u32x4*>(lds + st_off + i * 4096) = stage_a[i];
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<u32x4*>(lds + BM * 128 + st_off + i * 4096) = stage_b[i];
+    stager_a.fetch(kt_begin, full_k_tiles);
+    stager_b.fetch(kt_begin, full_k_tiles);
+    stager_a.commit(lds);
+    stager_b.commit(lds + BM * 128);
   }
   __syncthreads();
 
@@ -392,21 +472,18 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
     const int stage = (kt - kt_begin) & 1;
     const bool more = kt + 1 < kt_end;
     if (more) {
-      stager_a.fetch(stage_a, kt + 1, full_k_tiles, ld_row, ld_chunk);
-      stager_b.fetch(stage_b, kt + 1, full_k_tiles, ld_row, ld_chunk);
+      stager_a.fetch(kt + 1, full_k_tiles);
+      stager_b.fetch(kt + 1, full_k_tiles);
     }
 
-    const char* sa = lds + stage * STAGE_BYTES + (wm * WM * 32) * 128;
-    const char* sb = lds + stage * STAGE_BYTES + BM * 128 + (wn * WN * 32) * 128;
+    const char* tile = lds + stage * STAGE_BYTES;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      // rows i*32 + frag_row keep (row & 7) == (frag_row & 7): one swizzled offset per k-step
-      const int off = lds_chunk_offset(frag_row, ks * 2 + frag_half);
       u32x4 fa[WM], fb[WN];
 #pragma unroll
-      for (int i = 0; i < WM; ++i) fa[i] = *reinterpret_cast<const u32x4*>(sa + off + i * 4096);
+      for (int i = 0; i < WM; ++i) fa[i] = *reinterpret_cast<const u32x4*>(tile + (off_a[i] ^ (ks << 5)));
 #pragma unroll
-      for (int j = 0; j < WN; ++j) fb[j] = *reinterpret_cast<const u32x4*>(sb + off + j * 4096);
+      for (int j = 0; j < WN; ++j) fb[j] = *reinterpret_cast<const u32x4*>(tile + (off_b[j] ^ (ks << 5)));
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
@@ -414,11 +491,9 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
     }
 
     if (more) {
-      char* dst = lds + (stage ^ 1) * STAGE_BYTES + st_off;
-#pragma unroll
-      for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<u32x4*>(dst + i * 4096) = stage_a[i];
-#pragma unroll
-      for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<u32x4*>(dst + BM * 128 + i * 4096) = stage_b[i];
+      char* next = lds + (stage ^ 1) * STAGE_BYTES;
+      stager_a.commit(next);
+      stager_b.commit(next + BM * 128);
     }
     __syncthreads();
   }

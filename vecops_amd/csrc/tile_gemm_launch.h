@@ -9,11 +9,18 @@
 
 namespace vecops_hip {
 
-// tile: 256, 128 or 64 (workgroup tile edge).  vec: operands allow 16-byte loads
-// along K.  Returns the HIP error of the launch (hipSuccess when enqueued).
-hipError_t launch_tile_gemm_bf16(const TileGemmParams& p, int tile, bool vec, hipStream_t stream);
-hipError_t launch_tile_gemm_f32_as_bf16(const TileGemmParams& p, int tile, bool vec, hipStream_t stream);
-hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile, bool vec, hipStream_t stream);
+// How the operand pair is fetched.
+enum LoadMode : int {
+  MODE_GENERIC = 0,  // element loads, any strides
+  MODE_KVEC = 1,     // A and B K-contiguous and 16-byte aligned
+  MODE_NVEC_B = 2    // A K-contiguous; B stored [K,N] row-major, 16-byte aligned (16-bit compute types)
+};
+
+// tile: 256, 128 or 64 (workgroup tile edge).  Returns the HIP error of the
+// launch (hipSuccess when enqueued).
+hipError_t launch_tile_gemm_bf16(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
+hipError_t launch_tile_gemm_f32_as_bf16(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
+hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
 
 // Shared by the per-class translation units.
@@ -37,16 +44,20 @@ hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <int SRC, int WM, int WN>
+hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t stream) {
+  if (mode == MODE_KVEC) return launch_tile_instance<SRC, WM, WN, LOAD_KVEC, LOAD_KVEC>(p, stream);
+  if constexpr (SrcTraits<SRC>::kElemsPerChunk == 8) {
+    if (mode == MODE_NVEC_B) return launch_tile_instance<SRC, WM, WN, LOAD_KVEC, LOAD_NVEC>(p, stream);
+  }
+  return launch_tile_instance<SRC, WM, WN, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
+}
+
 template <int SRC>
-hipError_t launch_tile_class(const TileGemmParams& p, int tile, bool vec, hipStream_t stream) {
-  if (tile == 256)
-    return vec ? launch_tile_instance<SRC, 4, 4, LOAD_KVEC, LOAD_KVEC>(p, stream)
-               : launch_tile_instance<SRC, 4, 4, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
-  if (tile == 128)
-    return vec ? launch_tile_instance<SRC, 2, 2, LOAD_KVEC, LOAD_KVEC>(p, stream)
-               : launch_tile_instance<SRC, 2, 2, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
-  return vec ? launch_tile_instance<SRC, 1, 1, LOAD_KVEC, LOAD_KVEC>(p, stream)
-             : launch_tile_instance<SRC, 1, 1, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
+hipError_t launch_tile_class(const TileGemmParams& p, int tile, int mode, hipStream_t stream) {
+  if (tile == 256) return launch_tile_mode<SRC, 4, 4>(p, mode, stream);
+  if (tile == 128) return launch_tile_mode<SRC, 2, 2>(p, mode, stream);
+  return launch_tile_mode<SRC, 1, 1>(p, mode, stream);
 }
 
 }  // namespace vecops_hip
