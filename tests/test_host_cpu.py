@@ -1,0 +1,233 @@
+"""The C++ host layer without a GPU: ABI layout, artifact loading, schema
+validation, dispatch, provider behaviour and error mapping - the checks vecops
+runs against its fake backend in tests/runtime/RuntimeTest.cpp:302-347,468,
+502-506,557-562, here against the real HIP artifacts (whose run() stops at
+"no HIP device" on a host without one).  Every test runs against the restated
+runtime and, where oracle/_ref holds it, against the plug-in compiled into the
+vecops tree's own runtime."""
+import ctypes as C
+import os
+import shutil
+import subprocess
+import threading
+
+import numpy as np
+import pytest
+
+from vecops_amd import host_api as H
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FLAVORS = [H.HOST_LIB] + ([H.UPSTREAM_LIB] if os.path.exists(H.UPSTREAM_LIB) else [])
+
+
+@pytest.fixture(scope="module", params=FLAVORS, ids=lambda p: "upstream" if "upstream" in p else "restated")
+def host(request):
+    return H.HostLibrary(request.param)
+
+
+def bf16(shape):
+    return np.zeros(shape, np.uint16)
+
+
+ABI_PROBE = r"""
+#include <stdio.h>
+#include <stddef.h>
+#include HEADER_CALL
+#include HEADER_KERNEL
+#define S(T) printf(#T " %zu\n", sizeof(T))
+#define O(T, F) printf(#T "." #F " %zu\n", offsetof(T, F))
+int main(void) {
+  S(VecopsError); O(VecopsError, code); O(VecopsError, message); O(VecopsError, message_capacity); O(VecopsError, message_required);
+  S(VecopsTensorView); O(VecopsTensorView, data); O(VecopsTensorView, byte_offset); O(VecopsTensorView, device_type);
+  O(VecopsTensorView, device_index); O(VecopsTensorView, dtype); O(VecopsTensorView, rank); O(VecopsTensorView, sizes);
+  O(VecopsTensorView, strides); O(VecopsTensorView, flags);
+  S(VecopsScalar); O(VecopsScalar, dtype); O(VecopsScalar, value);
+  S(VecopsValue); O(VecopsValue, kind); O(VecopsValue, value);
+  S(VecopsExecutionContext); O(VecopsExecutionContext, requested_threads); O(VecopsExecutionContext, stream);
+  O(VecopsExecutionContext, user_data); O(VecopsExecutionContext, flags); O(VecopsExecutionContext, workspace_provider);
+  O(VecopsExecutionContext, thread_pool); O(VecopsExecutionContext, allocation_observer);
+  S(VecopsCall); O(VecopsCall, num_values); O(VecopsCall, values); O(VecopsCall, workspace); O(VecopsCall, workspace_size);
+  O(VecopsCall, context);
+  S(VecopsDimensionConstraint); O(VecopsDimensionConstraint, kind); O(VecopsDimensionConstraint, value);
+  O(VecopsDimensionConstraint, lower_bound); O(VecopsDimensionConstraint, upper_bound); O(VecopsDimensionConstraint, alignment);
+  S(VecopsTensorParameter); O(VecopsTensorParameter, dtype_mask); O(VecopsTensorParameter, device_type);
+  O(VecopsTensorParameter, device_index); O(VecopsTensorParameter, rank); O(VecopsTensorParameter, optional);
+  O(VecopsTensorParameter, dimension_constraint_stride); O(VecopsTensorParameter, sizes); O(VecopsTensorParameter, strides);
+  O(VecopsTensorParameter, required_flags);
+  S(VecopsScalarParameter); S(VecopsParameterDescriptor); O(VecopsParameterDescriptor, kind); O(VecopsParameterDescriptor, name);
+  O(VecopsParameterDescriptor, constraint);
+  S(VecopsKernelDescriptorV1); O(VecopsKernelDescriptorV1, abi_version_major); O(VecopsKernelDescriptorV1, abi_version_minor);
+  O(VecopsKernelDescriptorV1, operator_name); O(VecopsKernelDescriptorV1, specialization_key);
+  O(VecopsKernelDescriptorV1, num_parameters); O(VecopsKernelDescriptorV1, parameter_stride); O(VecopsKernelDescriptorV1, parameters);
+  O(VecopsKernelDescriptorV1, workspace); O(VecopsKernelDescriptorV1, run); O(VecopsKernelDescriptorV1, flags);
+  printf("enum %d %d %d %d %d %d %d %d\n", VECOPS_STATUS_EXECUTION_ERROR, VECOPS_DEVICE_PRIVATE, VECOPS_DTYPE_BF16,
+         VECOPS_DTYPE_F32, VECOPS_DTYPE_I8, VECOPS_VALUE_TENSOR, (int)VECOPS_TENSOR_WRITE, VECOPS_DIM_DYNAMIC);
+  printf("symbol %s %u %u\n", VECOPS_KERNEL_QUERY_SYMBOL_V1, VECOPS_KERNEL_ABI_VERSION_MAJOR, VECOPS_KERNEL_ABI_VERSION_MINOR);
+  return 0;
+}
+"""
+
+
+def _probe(tmp_path, tag, include_dir, call_header, kernel_header):
+    src = tmp_path / f"probe_{tag}.c"
+    src.write_text(ABI_PROBE)
+    exe = tmp_path / f"probe_{tag}"
+    subprocess.run(["gcc", "-I", include_dir, f'-DHEADER_CALL="{call_header}"', f'-DHEADER_KERNEL="{kernel_header}"',
+                    str(src), "-o", str(exe)], check=True)
+    return subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+
+
+def test_abi_layout(tmp_path):
+    ours = _probe(tmp_path, "ours", os.path.join(ROOT, "vecops_amd", "host", "include"), "vecops_rt/abi.h",
+                  "vecops_rt/abi.h")
+    facts = dict(line.rsplit(" ", 1) for line in ours.splitlines() if not line.startswith(("enum", "symbol")))
+    for name, size in H.ABI_SIZES.items():
+        assert int(facts[name]) == size == C.sizeof({"VecopsTensorView": H.TensorView, "VecopsScalar": H.Scalar,
+                                                     "VecopsValue": H.Value,
+                                                     "VecopsExecutionContext": H.ExecutionContext}[name])
+    assert "symbol vecops_kernel_query_v1 1 1" in ours
+    assert "enum 6 255 11 12 2 1 2 2" in ours
+    if os.path.isdir("/root/reference/include/vecops/runtime"):
+        # byte-for-byte the same layout as vecops' own runtime/CallAbi.h and runtime/KernelAbi.h
+        theirs = _probe(tmp_path, "ref", "/root/reference/include", "vecops/runtime/CallAbi.h",
+                        "vecops/runtime/KernelAbi.h")
+        assert ours == theirs
+
+
+def test_every_artifact_loads_with_its_key(host):
+    files = sorted(os.listdir(H.ARTIFACT_DIR))
+    assert len(files) == 12
+    for f in files:
+        name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
+        assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
+        assert f == "".join(ch if (ch.isalnum() or ch in "_.=-") else "_" for ch in key) + ".so"
+    # exactly one exported symbol of ours per artifact
+    out = subprocess.run(["nm", "-D", "--defined-only", os.path.join(H.ARTIFACT_DIR, files[0])], capture_output=True,
+                         text=True).stdout
+    assert [l.split()[-1] for l in out.splitlines() if " T " in l] == ["vecops_kernel_query_v1"]
+
+
+def test_loader_error_mapping(host, tmp_path):
+    with pytest.raises(H.HostError) as e:       # unloadable -> LoadError (Executable.cpp:208-218)
+        host.load_artifact(str(tmp_path / "missing.so"))
+    assert e.value.code == 5
+    with pytest.raises(H.HostError) as e:       # a DSO without the query symbol -> AbiMismatch (:219-229)
+        host.load_artifact(os.path.join(ROOT, "oracle", "libvecops_oracle.so"))
+    assert e.value.code == 4 and "vecops_kernel_query_v1" in e.value.message
+
+
+def test_resolve_picks_recipe_by_dtype_and_placement(host):
+    op = host.operator("vecops::matmul")
+    a32, b32, c32 = np.zeros((4, 8), np.float32), np.zeros((5, 8), np.float32), np.zeros((4, 5), np.float32)
+    assert op.resolve(H.Frame([a32, b32, None, c32], outputs=(3,))) == \
+        "vecops::matmul;operands=f32;compute=bf16;memory=host;backend=hip-gfx950"
+    assert op.resolve(H.Frame([bf16((4, 8)), bf16((5, 8)), None, c32], outputs=(3,))) == \
+        "vecops::matmul;operands=bf16;compute=bf16;memory=host;backend=hip-gfx950"
+    ai, bi, ci = np.zeros((4, 8), np.int8), np.zeros((5, 8), np.int8), np.zeros((4, 5), np.int32)
+    assert op.resolve(H.Frame([ai, bi, None, ci], outputs=(3,))) == \
+        "vecops::matmul;operands=i8;compute=i32;memory=host;backend=hip-gfx950"
+    dev = lambda dtype, shape: {"data": 0x10000, "dtype": dtype, "shape": shape,  # noqa: E731
+                                "strides": (shape[-1], 1) if len(shape) == 2 else (shape[1] * shape[2], shape[2], 1),
+                                "device_type": H.DEVICE_PRIVATE}
+    f = H.Frame([dev(H.BF16, (2, 4, 8)), dev(H.BF16, (2, 5, 8)), None, dev(H.BF16, (2, 4, 5))], outputs=(3,))
+    assert op.resolve(f) == "vecops::matmul;operands=bf16;compute=bf16;memory=device;backend=hip-gfx950"
+    # explicit ComputeType specialization (bf16 is what the x86 reference path computes in)
+    assert "compute=bf16" in op.resolve(H.Frame([a32, b32, None, c32], outputs=(3,)), {"ComputeType": ("dtype", H.BF16)})
+    with pytest.raises(H.HostError) as e:       # true fp32 compute is a recipe that is not built
+        op.resolve(H.Frame([a32, b32, None, c32], outputs=(3,)), {"ComputeType": ("dtype", H.F32)})
+    assert e.value.code == 2
+    w = host.operator("vecops::matmul_w8a16_group")
+    x, wq, s, y = bf16((4, 256)), np.zeros((8, 256), np.int8), np.zeros((8, 2), np.float32), bf16((4, 8))
+    assert w.resolve(H.Frame([x, wq, s, y], outputs=(3,))) == \
+        "vecops::matmul_w8a16_group;G=128;memory=host;backend=hip-gfx950"
+    s4 = np.zeros((8, 4), np.float32)
+    assert "G=64" in w.resolve(H.Frame([x, wq, s4, y], outputs=(3,)), {"G": 64})
+    with pytest.raises(H.HostError) as e:       # valid call, no artifact for G=32 -> NotFound from the provider
+        w.resolve(H.Frame([x, wq, np.zeros((8, 8), np.float32), y], outputs=(3,)), {"G": 32})
+    assert e.value.code == 3
+
+
+def test_schema_validation(host):
+    op = host.operator("vecops::matmul")
+    c = np.zeros((4, 5), np.float32)
+    ok = [bf16((4, 8)), bf16((5, 8)), None, c]
+    op.resolve(H.Frame(ok, outputs=(3,)))
+    cases = [
+        ([bf16((4, 8)), bf16((5, 9)), None, c], "K"),                            # K mismatch
+        ([bf16((4, 8)), bf16((5, 8)), None, np.zeros((4, 6), np.float32)], "c must be"),
+        ([bf16((4, 8)), bf16((5, 8)), np.zeros((4, 6), np.float32), c], "c_in"),
+        ([bf16((2, 4, 8)), bf16((3, 5, 8)), None, np.zeros((2, 4, 5), np.float32)], "batch"),
+        ([bf16((4, 8)), bf16((2, 5, 8)), None, c], "rank"),
+        ([bf16((4, 8)), bf16((5, 8)), None, None], "not optional"),
+        ([bf16((4, 8)), bf16((5, 8)), c], "expects 4 arguments"),
+        ([np.zeros((4, 8), np.int32), bf16((5, 8)), None, c], "dtype"),
+    ]
+    for args, needle in cases:
+        with pytest.raises(H.HostError) as e:
+            op.resolve(H.Frame(args, outputs=(len(args) - 1,)))
+        assert e.value.code == 1 and needle in e.value.message, (needle, e.value.message)
+    with pytest.raises(H.HostError) as e:       # output without write access
+        op.resolve(H.Frame(ok, outputs=()))
+    assert e.value.code == 1 and "access" in e.value.message
+    with pytest.raises(H.HostError) as e:       # operand dtypes no recipe takes
+        op.resolve(H.Frame([bf16((4, 8)), np.zeros((5, 8), np.int8), None, c], outputs=(3,)))
+    assert e.value.code in (2, 3)
+    deq = host.operator("vecops::matmul_i8_dequant")
+    a, b = np.zeros((4, 8), np.int8), np.zeros((5, 8), np.int8)
+    with pytest.raises(H.HostError) as e:
+        deq.resolve(H.Frame([a, b, np.zeros(3, np.float32), np.zeros(5, np.float32), None, c], outputs=(5,)))
+    assert e.value.code == 1 and "row_scales" in e.value.message
+
+
+def test_provider_without_artifacts_reports_not_found(host, tmp_path):
+    op = host.operator("vecops::matmul", str(tmp_path))
+    with pytest.raises(H.HostError) as e:
+        op.resolve(H.Frame([bf16((4, 8)), bf16((5, 8)), None, np.zeros((4, 5), np.float32)], outputs=(3,)))
+    assert e.value.code == 3 and "no HIP artifact" in e.value.message
+
+
+def test_artifact_with_the_wrong_key_is_rejected(host, tmp_path):
+    """A file in the bf16 slot that is really the int8 artifact: the provider (and
+    Operator.cpp:250-253 behind it) must refuse it with AbiMismatch (RuntimeTest.cpp:502-506)."""
+    bf = "vecops__matmul_operands=bf16_compute=bf16_memory=host_backend=hip-gfx950.so"
+    i8 = "vecops__matmul_operands=i8_compute=i32_memory=host_backend=hip-gfx950.so"
+    shutil.copy(os.path.join(H.ARTIFACT_DIR, i8), tmp_path / bf)
+    op = host.operator("vecops::matmul", str(tmp_path))
+    with pytest.raises(H.HostError) as e:
+        op.resolve(H.Frame([bf16((4, 8)), bf16((5, 8)), None, np.zeros((4, 5), np.float32)], outputs=(3,)))
+    assert e.value.code == 4
+
+
+def test_concurrent_resolution(host):
+    """Provider thread-safety (RuntimeTest.cpp:512-547): many threads resolving the same and different keys."""
+    op = host.operator("vecops::matmul")
+    frames = [H.Frame([bf16((4, 8)), bf16((5, 8)), None, np.zeros((4, 5), np.float32)], outputs=(3,)),
+              H.Frame([np.zeros((4, 8), np.int8), np.zeros((5, 8), np.int8), None, np.zeros((4, 5), np.int32)],
+                      outputs=(3,))]
+    keys, errors = [], []
+
+    def work(i):
+        try:
+            for _ in range(20):
+                keys.append(op.resolve(frames[i % 2]))
+        except Exception as exc:  # pragma: no cover
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(8)]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    assert not errors and len(keys) == 160 and len(set(keys)) == 2
+
+
+def test_invoke_without_a_gpu_is_an_execution_error(host):
+    """On a host with no HIP device the artifact's run() reports
+    VECOPS_STATUS_EXECUTION_ERROR through VecopsError; nothing falls back to the CPU."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    op = host.operator("vecops::matmul")
+    c = np.full((4, 5), 7.0, np.float32)
+    with pytest.raises(H.HostError) as e:
+        op.invoke(H.Frame([bf16((4, 8)), bf16((5, 8)), None, c], outputs=(3,)))
+    assert e.value.code == 6 and "no HIP device" in e.value.message
+    assert (c == 7.0).all()

@@ -1,0 +1,150 @@
+"""The whole drop-in path on the GPU: vecops Operator -> dispatch policy -> recipe
+-> HipExecutableProvider -> Executable -> artifact DSO -> C ABI -> gfx950 kernel,
+with host tensors (staged inside the artifact) and with device tensors (used in
+place), checked against the oracle.  Runs against the restated runtime and against
+the plug-in compiled into the vecops tree's own runtime where oracle/_ref holds it."""
+import os
+
+import numpy as np
+import pytest
+
+from conftest import rel_err
+from oracle import oracle as O
+from vecops_amd import host_api as H
+from vecops_amd import synth
+
+pytestmark = pytest.mark.gpu
+FLAVORS = [H.HOST_LIB] + ([H.UPSTREAM_LIB] if os.path.exists(H.UPSTREAM_LIB) else [])
+
+
+@pytest.fixture(scope="module", params=FLAVORS, ids=lambda p: "upstream" if "upstream" in p else "restated")
+def host(request, device):
+    return H.HostLibrary(request.param)
+
+
+def fp32_tol(k):
+    return 2e-6 * max(1.0, k / 32)
+
+
+@pytest.mark.parametrize("m,n,k", [(37, 51, 79), (300, 260, 1000), (255, 63, 8191)])
+def test_matmul_bf16_host_tensors(host, oracle, m, n, k):
+    op = host.operator("vecops::matmul")
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    c = np.full((m, n), np.nan, np.float32)
+    frame = H.Frame([a, b, None, c], outputs=(3,))
+    assert op.workspace(frame) == 0          # host callers cannot supply device scratch
+    op.invoke(frame)
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, acc_f64=True)
+    assert rel_err(c, want) <= fp32_tol(k)
+
+
+def test_matmul_host_strided_views_and_aliased_c_input(host, oracle):
+    op = host.operator("vecops::matmul")
+    m, n, k = 33, 47, 130
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b_kn = np.ascontiguousarray(synth.bf16_round(synth.uniform_pm1(2, (n, k))).T)   # [K,N] row-major
+    b = b_kn.T
+    store = np.full((m, 2 * n), -5.0, np.float32)
+    store[:, 0:2 * n:2] = synth.uniform_pm1(3, (m, n))
+    c = store[:, 0:2 * n:2]                                                        # every other column
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, cin=c.copy(), acc_f64=True)
+    op.invoke(H.Frame([a, b, c, c], outputs=(3,)))                                   # C input aliases the output
+    assert rel_err(c, want) <= fp32_tol(k)
+    assert (store[:, 1:2 * n:2] == -5.0).all()                                       # gaps untouched
+
+
+def test_matmul_device_tensors_and_workspace(host, oracle, device):
+    import torch
+    op = host.operator("vecops::matmul")
+    m, n, k = 255, 63, 8191                   # tiny output, long K: split-K needs caller workspace
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    ta = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+    tb = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    frame = H.Frame([ta, tb, None, c], outputs=(3,))
+    assert op.resolve(frame).endswith("memory=device;backend=hip-gfx950")
+    need = op.workspace(frame)
+    assert need > 0
+    with pytest.raises(H.HostError) as e:     # Executable::invoke rejects too little workspace (Executable.cpp:291-295)
+        op.invoke(frame)
+    assert e.value.code == 1 and "workspace bytes" in e.value.message
+    ws = torch.empty(need, dtype=torch.uint8, device=device)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        op.invoke(frame, workspace=ws.data_ptr(), workspace_size=need, stream=stream.cuda_stream)
+    # the ABI is synchronous: the result is visible as soon as invoke returns
+    got = c.cpu().numpy()
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, acc_f64=True)
+    assert rel_err(got, want) <= fp32_tol(k)
+
+
+def test_matmul_rank3_fp32_and_int8(host, oracle, device):
+    import torch
+    op = host.operator("vecops::matmul")
+    batch, m, n, k = 3, 40, 56, 96
+    a, b = synth.uniform_pm1(1, (batch, m, k)), synth.uniform_pm1(2, (n, k))
+    c = np.zeros((batch, m, n), np.float32)
+    bb = np.broadcast_to(b, (batch, n, k))    # stride-0 batch
+    op.invoke(H.Frame([a, bb, None, c], outputs=(3,)))
+    want = np.zeros((batch, m, n), np.float32)
+    oracle.matmul(a, bb, want, atom=O.ATOM_BF16F32, acc_f64=True)
+    assert rel_err(c, want) <= fp32_tol(k)
+    ai, bi = synth.int8_sym(3, (130, 515)), synth.int8_sym(4, (140, 515))
+    ci = torch.zeros((130, 140), dtype=torch.int32, device=device)
+    op.invoke(H.Frame([torch.from_numpy(ai).to(device), torch.from_numpy(bi).to(device), None, ci], outputs=(3,)))
+    assert np.array_equal(ci.cpu().numpy(), oracle.matmul_i8_dense(ai, bi))
+
+
+def test_matmul_i8_dequant_operator(host, oracle, device):
+    import torch
+    op = host.operator("vecops::matmul_i8_dequant")
+    m, n, k = 67, 129, 515
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    rs, cs = synth.scales(3, m), synth.scales(4, n)
+    corr = ((synth.draws(5, n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32)
+    want = oracle.matmul_i8_dequant(a, b, rs, cs, corr)
+    c = np.zeros((m, n), np.float32)
+    op.invoke(H.Frame([a, b, rs, cs, corr, c], outputs=(5,)))
+    assert np.array_equal(c.view(np.uint32), want.view(np.uint32))
+    tc = torch.zeros((m, n), dtype=torch.float32, device=device)
+    to = lambda x: torch.from_numpy(x).to(device)  # noqa: E731
+    op.invoke(H.Frame([to(a), to(b), to(rs), to(cs), None, tc], outputs=(5,)))
+    assert np.array_equal(tc.cpu().numpy().view(np.uint32), oracle.matmul_i8_dequant(a, b, rs, cs).view(np.uint32))
+
+
+def test_matmul_w8a16_group_operator(host, oracle, device):
+    import torch
+    op = host.operator("vecops::matmul_w8a16_group")
+    for m, n, k, g in [(1, 512, 1024, 128), (4, 300, 512, 64)]:
+        x = synth.bf16_round(synth.normal(1, (m, k)))
+        w = synth.int8_sym(2, (n, k))
+        s = synth.scales(3, (n, k // g))
+        _, want = oracle.matmul_w8a16_group(x, w, s, g)
+        y = np.zeros((m, n), np.uint16)
+        op.invoke(H.Frame([x, w, s, y], outputs=(3,)), {"G": g})
+        assert rel_err(synth.bf16_to_f32(y), want) <= 2 ** -7
+        ty = torch.zeros((m, n), dtype=torch.bfloat16, device=device)
+        tx = torch.from_numpy(x.view(np.int16)).to(device).view(torch.bfloat16)
+        op.invoke(H.Frame([tx, torch.from_numpy(w).to(device), torch.from_numpy(s).to(device), ty], outputs=(3,)),
+                  {"G": g})
+        got = ty.view(torch.int16).cpu().numpy().view(np.uint16)
+        assert np.array_equal(got, y)         # host-staged and in-place runs agree bit for bit
+    with pytest.raises(H.HostError) as e:     # M > 16 is not the skinny family
+        op.invoke(H.Frame([np.zeros((17, 256), np.uint16), np.zeros((8, 256), np.int8), np.zeros((8, 2), np.float32),
+                           np.zeros((17, 8), np.uint16)], outputs=(3,)))
+    assert e.value.code in (2, 3)
+
+
+def test_mixed_placement_is_refused(host, device):
+    import torch
+    op = host.operator("vecops::matmul")
+    a = np.zeros((4, 8), np.uint16)
+    tb = torch.zeros((5, 8), dtype=torch.bfloat16, device=device)
+    with pytest.raises(H.HostError) as e:
+        op.invoke(H.Frame([a, tb, None, np.zeros((4, 5), np.float32)], outputs=(3,)))
+    assert e.value.code in (2, 3)

@@ -1,0 +1,527 @@
+// Source of the HIP kernel-artifact DSOs for the vecops matmul operators.  One
+// DSO per (operator, operand class, memory placement); the build compiles this
+// file once per artifact with
+//   -DVECOPS_ARTIFACT_KIND=<0..4>   0 matmul bf16, 1 matmul f32 (bf16 compute), 2 matmul i8,
+//                                   3 matmul_i8_dequant, 4 matmul_w8a16_group
+//   -DVECOPS_ARTIFACT_DEVICE=<0|1>  0: tensors are host memory, staged through HBM here
+//                                   1: tensors are HIP device pointers, used in place
+//   -DVECOPS_ARTIFACT_GROUP=<G>     group size of kind 4
+//
+// Each DSO exports exactly vecops_kernel_query_v1 (vecops runtime/KernelAbi.h:176)
+// and follows the callback contract of runtime/KernelAbi.h:129-131: status codes
+// out, message into the caller's VecopsError, no exception crosses, everything in
+// the call record is borrowed, and run() returns only when the result is visible
+// to the caller (the ABI is synchronous, runtime/CallAbi.h:16).  The context's
+// `stream` is read as a hipStream_t (null = the default stream).
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "vecops_hip.h"
+#include "vecops_rt/abi.h"
+
+#ifndef VECOPS_ARTIFACT_KIND
+#error "VECOPS_ARTIFACT_KIND must be defined"
+#endif
+#ifndef VECOPS_ARTIFACT_DEVICE
+#error "VECOPS_ARTIFACT_DEVICE must be defined"
+#endif
+#ifndef VECOPS_ARTIFACT_GROUP
+#define VECOPS_ARTIFACT_GROUP 128
+#endif
+
+#define VSTR2(x) #x
+#define VSTR(x) VSTR2(x)
+
+namespace {
+
+#if VECOPS_ARTIFACT_DEVICE
+#define MEMORY_NAME "device"
+constexpr uint32_t kDeviceType = VECOPS_DEVICE_PRIVATE;
+#else
+#define MEMORY_NAME "host"
+constexpr uint32_t kDeviceType = VECOPS_DEVICE_CPU;
+#endif
+
+constexpr uint64_t bit(uint32_t dtype) { return uint64_t{1} << (dtype - 1); }
+
+// ---- error reporting (same convention as vecops' generated adapters,
+// src/compiler/KernelCompiler.cpp:272-278) ---------------------------------------
+int32_t report(VecopsError* error, int32_t code, const std::string& message) {
+  if (error != nullptr && error->struct_size >= sizeof(VecopsError)) {
+    error->code = code;
+    error->message_required = message.size() + 1;
+    if (error->message != nullptr && error->message_capacity > 0) {
+      const size_t n = message.size() < error->message_capacity - 1 ? message.size() : error->message_capacity - 1;
+      memcpy(error->message, message.data(), n);
+      error->message[n] = '\0';
+    }
+  }
+  return code;
+}
+
+int32_t report_hip(VecopsError* error, const char* what, hipError_t e) {
+  return report(error, VECOPS_STATUS_EXECUTION_ERROR, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+int32_t report_kernel(VecopsError* error, int32_t rc) { return report(error, rc, vecops_hip_last_error()); }
+
+size_t dtype_bytes(uint32_t dt) {
+  switch (dt) {
+    case VECOPS_DTYPE_I8: case VECOPS_DTYPE_U8: case VECOPS_DTYPE_BOOL: return 1;
+    case VECOPS_DTYPE_I16: case VECOPS_DTYPE_U16: case VECOPS_DTYPE_F16: case VECOPS_DTYPE_BF16: return 2;
+    case VECOPS_DTYPE_I32: case VECOPS_DTYPE_U32: case VECOPS_DTYPE_F32: return 4;
+    default: return 8;
+  }
+}
+
+const VecopsTensorView* tensor_arg(const VecopsCall* call, uint32_t index) {
+  if (index >= call->num_values) return nullptr;
+  const VecopsValue& v = call->values[index];
+  return v.kind == VECOPS_VALUE_TENSOR ? &v.value.tensor : nullptr;
+}
+
+hipStream_t stream_of(const VecopsCall* call) {
+  const VecopsExecutionContext* ctx = call->context;
+  if (ctx == nullptr || ctx->struct_size < offsetof(VecopsExecutionContext, stream) + sizeof(void*)) return nullptr;
+  return static_cast<hipStream_t>(ctx->stream);
+}
+
+// Logical element zero of a view.
+char* origin(const VecopsTensorView* t) { return static_cast<char*>(t->data) + t->byte_offset; }
+
+bool fill_operand(const VecopsTensorView* t, void* data, VecopsHipOperand* o) {
+  if (t->rank != 2 && t->rank != 3) return false;
+  memset(o, 0, sizeof(*o));
+  o->data = data;
+  o->dtype = t->dtype;
+  o->rank = t->rank;
+  for (uint32_t i = 0; i < t->rank; ++i) {
+    o->sizes[i] = t->sizes[i];
+    o->strides[i] = t->strides[i];
+  }
+  return true;
+}
+
+// ---- host staging --------------------------------------------------------------------------
+// A host view is mirrored as the smallest byte range that holds all of its
+// elements; strides carry over unchanged.  Views with the same origin share one
+// device buffer, so a C input that aliases the output stays aliased.
+struct Staged {
+  const VecopsTensorView* view = nullptr;
+  void* device = nullptr;
+  size_t bytes = 0;
+  bool write_back = false;
+  bool owner = true;
+};
+
+class Staging {
+public:
+  explicit Staging(hipStream_t stream) : stream_(stream) {}
+  ~Staging() {
+    for (auto& s : items_)
+      if (s.owner && s.device != nullptr) (void)hipFree(s.device);
+    if (workspace_ != nullptr) (void)hipFree(workspace_);
+  }
+
+  // Returns the device address of the view's logical element zero (null for an empty view).
+  hipError_t add(const VecopsTensorView* t, bool write_back, void** device_origin, std::string* why) {
+    *device_origin = nullptr;
+    size_t span = 1;
+    for (uint32_t i = 0; i < t->rank; ++i) {
+      if (t->sizes[i] == 0) return hipSuccess;
+      if (t->strides[i] < 0) {
+        *why = "negative strides are not supported by the HIP artifacts";
+        return hipErrorInvalidValue;
+      }
+      span += static_cast<size_t>(t->sizes[i] - 1) * static_cast<size_t>(t->strides[i]);
+    }
+    const size_t bytes = span * dtype_bytes(t->dtype);
+    for (auto& s : items_) {
+      if (origin(s.view) == origin(t) && s.bytes >= bytes) {
+        s.write_back = s.write_back || write_back;
+        *device_origin = s.device;
+        return hipSuccess;
+      }
+    }
+    Staged s;
+    s.view = t;
+    s.bytes = bytes;
+    s.write_back = write_back;
+    hipError_t e = hipMalloc(&s.device, bytes);
+    if (e != hipSuccess) return e;
+    items_.push_back(s);
+    // outputs are uploaded too: a strided output must keep the bytes between its elements
+    e = hipMemcpyAsync(s.device, origin(t), bytes, hipMemcpyHostToDevice, stream_);
+    *device_origin = s.device;
+    return e;
+  }
+
+  hipError_t workspace(uint64_t bytes, void** out) {
+    *out = nullptr;
+    if (bytes == 0) return hipSuccess;
+    hipError_t e = hipMalloc(&workspace_, bytes);
+    *out = workspace_;
+    return e;
+  }
+
+  hipError_t finish() {
+    for (auto& s : items_) {
+      if (!s.write_back) continue;
+      hipError_t e = hipMemcpyAsync(origin(s.view), s.device, s.bytes, hipMemcpyDeviceToHost, stream_);
+      if (e != hipSuccess) return e;
+    }
+    return hipStreamSynchronize(stream_);
+  }
+
+private:
+  hipStream_t stream_;
+  std::vector<Staged> items_;
+  void* workspace_ = nullptr;
+};
+
+// Resolves the device address of each tensor argument: in place for device
+// artifacts, through `staging` for host artifacts.
+int32_t device_address(const VecopsTensorView* t, bool is_output, Staging* staging, void** out, VecopsError* error) {
+#if VECOPS_ARTIFACT_DEVICE
+  (void)is_output;
+  (void)staging;
+  (void)error;
+  *out = origin(t);
+  return VECOPS_STATUS_OK;
+#else
+  std::string why;
+  hipError_t e = staging->add(t, is_output, out, &why);
+  if (e != hipSuccess) {
+    if (!why.empty()) return report(error, VECOPS_STATUS_INVALID_ARGUMENT, why);
+    return report_hip(error, "staging a host tensor in device memory", e);
+  }
+  return VECOPS_STATUS_OK;
+#endif
+}
+
+int32_t finish(Staging* staging, hipStream_t stream, VecopsError* error) {
+#if VECOPS_ARTIFACT_DEVICE
+  (void)staging;
+  hipError_t e = hipStreamSynchronize(stream);
+#else
+  (void)stream;
+  hipError_t e = staging->finish();
+#endif
+  if (e != hipSuccess) return report_hip(error, "waiting for the kernels", e);
+  return VECOPS_STATUS_OK;
+}
+
+int32_t check_call(const VecopsCall* call, uint32_t expected, VecopsError* error) {
+  if (call == nullptr || call->struct_size < offsetof(VecopsCall, context) + sizeof(void*))
+    return report(error, VECOPS_STATUS_ABI_MISMATCH, "call record is smaller than ABI v1");
+  if (call->num_values != expected || (expected != 0 && call->values == nullptr))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "wrong number of arguments for this artifact");
+  return VECOPS_STATUS_OK;
+}
+
+// =================================================================================================
+#if VECOPS_ARTIFACT_KIND <= 2  // vecops::matmul (a, b, c_in?, c)
+// =================================================================================================
+
+#if VECOPS_ARTIFACT_KIND == 0
+#define OPERANDS "bf16"
+#define COMPUTE "bf16"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16);
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
+#elif VECOPS_ARTIFACT_KIND == 1
+#define OPERANDS "f32"
+#define COMPUTE "bf16"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
+#else
+#define OPERANDS "i8"
+#define COMPUTE "i32"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8);
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_I32);
+#endif
+
+constexpr const char* kOperatorName = "vecops::matmul";
+constexpr const char* kKey =
+  "vecops::matmul;operands=" OPERANDS ";compute=" COMPUTE ";memory=" MEMORY_NAME ";backend=hip-gfx950";
+
+#define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
+   {.tensor = {sizeof(VecopsTensorParameter), MASK, kDeviceType, -1, RANK, OPTIONAL,                          \
+               sizeof(VecopsDimensionConstraint), nullptr, nullptr, FLAGS}}}
+
+const VecopsParameterDescriptor kParameters[] = {
+  TENSOR_PARAM("a", kInMask, -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("b", kInMask, -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("c_in", kOutMask, -1, 1, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("c", kOutMask, -1, 0, VECOPS_TENSOR_WRITE),
+};
+
+int32_t plan(const VecopsCall* call, VecopsHipOperand ops[4], bool* has_cin, VecopsHipPlan* out, VecopsError* error) {
+  if (int32_t rc = check_call(call, 4, error); rc != VECOPS_STATUS_OK) return rc;
+  const VecopsTensorView* a = tensor_arg(call, 0);
+  const VecopsTensorView* b = tensor_arg(call, 1);
+  const VecopsTensorView* cin = tensor_arg(call, 2);
+  const VecopsTensorView* c = tensor_arg(call, 3);
+  if (a == nullptr || b == nullptr || c == nullptr)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "a, b and c must be tensors");
+  *has_cin = cin != nullptr;
+  // 16 is a stand-in address with the alignment real allocations have; plan() only reads metadata
+  if (!fill_operand(a, reinterpret_cast<void*>(16), &ops[0]) || !fill_operand(b, reinterpret_cast<void*>(16), &ops[1]) ||
+      !fill_operand(c, reinterpret_cast<void*>(16), &ops[3]) ||
+      (cin != nullptr && !fill_operand(cin, reinterpret_cast<void*>(16), &ops[2])))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "tensors must have rank 2 or 3");
+#if VECOPS_ARTIFACT_DEVICE
+  ops[0].data = origin(a);
+  ops[1].data = origin(b);
+  ops[3].data = origin(c);
+  if (cin != nullptr) ops[2].data = origin(cin);
+#endif
+  int32_t rc = vecops_hip_plan_matmul(&ops[0], &ops[1], *has_cin ? &ops[2] : nullptr, &ops[3],
+                                      VECOPS_HIP_COMPUTE_BF16, out);
+  if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
+  return VECOPS_STATUS_OK;
+}
+
+int32_t workspace_impl(const VecopsCall* call, uint64_t* bytes, VecopsError* error) {
+  VecopsHipOperand ops[4];
+  bool has_cin = false;
+  VecopsHipPlan p;
+  if (int32_t rc = plan(call, ops, &has_cin, &p, error); rc != VECOPS_STATUS_OK) return rc;
+#if VECOPS_ARTIFACT_DEVICE
+  *bytes = p.workspace_bytes;  // device scratch the caller must hand in
+#else
+  *bytes = 0;  // host callers cannot supply device scratch; run() allocates it
+#endif
+  return VECOPS_STATUS_OK;
+}
+
+int32_t run_impl(const VecopsCall* call, VecopsError* error) {
+  VecopsHipOperand ops[4];
+  bool has_cin = false;
+  VecopsHipPlan p;
+  if (int32_t rc = plan(call, ops, &has_cin, &p, error); rc != VECOPS_STATUS_OK) return rc;
+  if (p.family == VECOPS_HIP_FAMILY_NONE) return VECOPS_STATUS_OK;
+  hipStream_t stream = stream_of(call);
+  Staging staging(stream);
+  void* ws = call->workspace;
+  uint64_t ws_size = call->workspace_size;
+#if !VECOPS_ARTIFACT_DEVICE
+  // c first: if c_in aliases c they share the staged buffer and the write-back flag
+  const uint32_t order[4] = {3, 2, 0, 1};
+  for (uint32_t idx : order) {
+    const VecopsTensorView* t = tensor_arg(call, idx);
+    if (t == nullptr) continue;
+    void* dev = nullptr;
+    if (int32_t rc = device_address(t, idx == 3, &staging, &dev, error); rc != VECOPS_STATUS_OK) return rc;
+    ops[idx].data = dev;
+  }
+  if (hipError_t e = staging.workspace(p.workspace_bytes, &ws); e != hipSuccess)
+    return report_hip(error, "allocating split-K scratch", e);
+  ws_size = p.workspace_bytes;
+#endif
+  int32_t rc = vecops_hip_matmul(&ops[0], &ops[1], has_cin ? &ops[2] : nullptr, &ops[3], VECOPS_HIP_COMPUTE_BF16, ws,
+                                 ws_size, stream);
+  if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
+  return finish(&staging, stream, error);
+}
+
+// =================================================================================================
+#elif VECOPS_ARTIFACT_KIND == 3  // vecops::matmul_i8_dequant (a, b, row_scales, column_scales, correction?, c)
+// =================================================================================================
+
+constexpr const char* kOperatorName = "vecops::matmul_i8_dequant";
+constexpr const char* kKey =
+  "vecops::matmul_i8_dequant;operands=i8;epilogue=row_col_dequant;memory=" MEMORY_NAME ";backend=hip-gfx950";
+
+#define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
+   {.tensor = {sizeof(VecopsTensorParameter), MASK, kDeviceType, -1, RANK, OPTIONAL,                          \
+               sizeof(VecopsDimensionConstraint), nullptr, nullptr, FLAGS}}}
+
+const VecopsParameterDescriptor kParameters[] = {
+  TENSOR_PARAM("a", bit(VECOPS_DTYPE_I8), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("b", bit(VECOPS_DTYPE_I8), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("row_scales", bit(VECOPS_DTYPE_F32), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("column_scales", bit(VECOPS_DTYPE_F32), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("correction", bit(VECOPS_DTYPE_I32), -1, 1, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("c", bit(VECOPS_DTYPE_F32), -1, 0, VECOPS_TENSOR_WRITE),
+};
+
+struct DequantArgs {
+  const VecopsTensorView *a, *b, *rs, *cs, *corr, *c;
+  int64_t m, n, k;
+};
+
+int32_t decode(const VecopsCall* call, DequantArgs* d, VecopsError* error) {
+  if (int32_t rc = check_call(call, 6, error); rc != VECOPS_STATUS_OK) return rc;
+  d->a = tensor_arg(call, 0);
+  d->b = tensor_arg(call, 1);
+  d->rs = tensor_arg(call, 2);
+  d->cs = tensor_arg(call, 3);
+  d->corr = tensor_arg(call, 4);
+  d->c = tensor_arg(call, 5);
+  if (!d->a || !d->b || !d->rs || !d->cs || !d->c)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "a, b, row_scales, column_scales and c must be tensors");
+  if (d->a->rank != 2 || d->b->rank != 2 || d->c->rank != 2 || d->rs->rank != 1 || d->cs->rank != 1 ||
+      (d->corr && d->corr->rank != 1))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "matmul_i8_dequant takes rank-2 matrices and rank-1 vectors");
+  d->m = d->a->sizes[0];
+  d->k = d->a->sizes[1];
+  d->n = d->b->sizes[0];
+  if (d->b->sizes[1] != d->k || d->c->sizes[0] != d->m || d->c->sizes[1] != d->n || d->rs->sizes[0] != d->m ||
+      d->cs->sizes[0] != d->n || (d->corr && d->corr->sizes[0] != d->n))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "matmul_i8_dequant: extents disagree");
+  auto unit = [](const VecopsTensorView* t, uint32_t axis) { return t->sizes[axis] <= 1 || t->strides[axis] == 1; };
+  if (!unit(d->a, 1) || !unit(d->b, 1) || !unit(d->c, 1) || !unit(d->rs, 0) || !unit(d->cs, 0) ||
+      (d->corr && !unit(d->corr, 0)))
+    return report(error, VECOPS_STATUS_NOT_APPLICABLE, "matmul_i8_dequant: last axes must be contiguous");
+  return VECOPS_STATUS_OK;
+}
+
+int32_t workspace_impl(const VecopsCall* call, uint64_t* bytes, VecopsError* error) {
+  DequantArgs d;
+  if (int32_t rc = decode(call, &d, error); rc != VECOPS_STATUS_OK) return rc;
+#if VECOPS_ARTIFACT_DEVICE
+  *bytes = vecops_hip_matmul_i8_dequant_workspace(d.m, d.n, d.k);
+#else
+  *bytes = 0;
+#endif
+  return VECOPS_STATUS_OK;
+}
+
+int32_t run_impl(const VecopsCall* call, VecopsError* error) {
+  DequantArgs d;
+  if (int32_t rc = decode(call, &d, error); rc != VECOPS_STATUS_OK) return rc;
+  if (d.m == 0 || d.n == 0) return VECOPS_STATUS_OK;
+  hipStream_t stream = stream_of(call);
+  Staging staging(stream);
+  void *a = nullptr, *b = nullptr, *rs = nullptr, *cs = nullptr, *corr = nullptr, *c = nullptr;
+  int32_t rc;
+  if ((rc = device_address(d.c, true, &staging, &c, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(d.a, false, &staging, &a, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(d.b, false, &staging, &b, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(d.rs, false, &staging, &rs, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(d.cs, false, &staging, &cs, error)) != VECOPS_STATUS_OK) return rc;
+  if (d.corr && (rc = device_address(d.corr, false, &staging, &corr, error)) != VECOPS_STATUS_OK) return rc;
+  void* ws = call->workspace;
+  uint64_t ws_size = call->workspace_size;
+#if !VECOPS_ARTIFACT_DEVICE
+  ws_size = vecops_hip_matmul_i8_dequant_workspace(d.m, d.n, d.k);
+  if (hipError_t e = staging.workspace(ws_size, &ws); e != hipSuccess)
+    return report_hip(error, "allocating split-K scratch", e);
+#endif
+  rc = vecops_hip_matmul_i8_dequant(static_cast<const int8_t*>(a), d.a->strides[0], static_cast<const int8_t*>(b),
+                                    d.b->strides[0], static_cast<const float*>(rs), static_cast<const float*>(cs),
+                                    static_cast<const int32_t*>(corr), static_cast<float*>(c), d.c->strides[0], d.m,
+                                    d.n, d.k, ws, ws_size, stream);
+  if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
+  return finish(&staging, stream, error);
+}
+
+// =================================================================================================
+#else  // vecops::matmul_w8a16_group (x, w, scales, y)
+// =================================================================================================
+
+constexpr const char* kOperatorName = "vecops::matmul_w8a16_group";
+constexpr const char* kKey = "vecops::matmul_w8a16_group;G=" VSTR(VECOPS_ARTIFACT_GROUP) ";memory=" MEMORY_NAME
+                             ";backend=hip-gfx950";
+
+#define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
+   {.tensor = {sizeof(VecopsTensorParameter), MASK, kDeviceType, -1, RANK, OPTIONAL,                          \
+               sizeof(VecopsDimensionConstraint), nullptr, nullptr, FLAGS}}}
+
+const VecopsParameterDescriptor kParameters[] = {
+  TENSOR_PARAM("x", bit(VECOPS_DTYPE_BF16), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("w", bit(VECOPS_DTYPE_I8), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("scales", bit(VECOPS_DTYPE_F32), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("y", bit(VECOPS_DTYPE_BF16), -1, 0, VECOPS_TENSOR_WRITE),
+};
+
+int32_t workspace_impl(const VecopsCall* call, uint64_t* bytes, VecopsError* error) {
+  if (int32_t rc = check_call(call, 4, error); rc != VECOPS_STATUS_OK) return rc;
+  *bytes = 0;
+  return VECOPS_STATUS_OK;
+}
+
+int32_t run_impl(const VecopsCall* call, VecopsError* error) {
+  if (int32_t rc = check_call(call, 4, error); rc != VECOPS_STATUS_OK) return rc;
+  const VecopsTensorView* x = tensor_arg(call, 0);
+  const VecopsTensorView* w = tensor_arg(call, 1);
+  const VecopsTensorView* s = tensor_arg(call, 2);
+  const VecopsTensorView* y = tensor_arg(call, 3);
+  if (!x || !w || !s || !y || x->rank != 2 || w->rank != 2 || s->rank != 2 || y->rank != 2)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "x, w, scales and y must be rank-2 tensors");
+  const int64_t m = x->sizes[0], k = x->sizes[1], n = w->sizes[0], g = VECOPS_ARTIFACT_GROUP;
+  if (w->sizes[1] != k || y->sizes[0] != m || y->sizes[1] != n || k % g != 0 || s->sizes[0] != n ||
+      s->sizes[1] != k / g)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "matmul_w8a16_group: extents disagree");
+  auto unit = [](const VecopsTensorView* t) { return t->sizes[1] <= 1 || t->strides[1] == 1; };
+  if (!unit(x) || !unit(w) || !unit(y) || !unit(s) || (s->sizes[0] > 1 && s->strides[0] != s->sizes[1]))
+    return report(error, VECOPS_STATUS_NOT_APPLICABLE, "matmul_w8a16_group: rows must be contiguous, scales dense");
+  if (m == 0 || n == 0) return VECOPS_STATUS_OK;
+  hipStream_t stream = stream_of(call);
+  Staging staging(stream);
+  void *dx = nullptr, *dw = nullptr, *ds = nullptr, *dy = nullptr;
+  int32_t rc;
+  if ((rc = device_address(y, true, &staging, &dy, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(x, false, &staging, &dx, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(w, false, &staging, &dw, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(s, false, &staging, &ds, error)) != VECOPS_STATUS_OK) return rc;
+  rc = vecops_hip_matmul_w8a16_group(dx, x->strides[0], static_cast<const int8_t*>(dw), w->strides[0],
+                                     static_cast<const float*>(ds), dy, y->strides[0], m, n, k, g, stream);
+  if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
+  return finish(&staging, stream, error);
+}
+
+#endif
+
+// ---- callbacks: nothing may escape as an exception --------------------------------------------------
+int32_t workspace_entry(const VecopsCall* call, uint64_t* bytes, VecopsError* error) {
+  try {
+    if (bytes == nullptr) return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "null workspace size pointer");
+    return workspace_impl(call, bytes, error);
+  } catch (const std::exception& e) {
+    return report(error, VECOPS_STATUS_EXECUTION_ERROR, e.what());
+  } catch (...) {
+    return report(error, VECOPS_STATUS_EXECUTION_ERROR, "unknown exception in the workspace query");
+  }
+}
+
+int32_t run_entry(const VecopsCall* call, VecopsError* error) {
+  try {
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+      return report(error, VECOPS_STATUS_EXECUTION_ERROR,
+                    std::string("no HIP device available: ") + (e != hipSuccess ? hipGetErrorString(e) : "0 devices"));
+    return run_impl(call, error);
+  } catch (const std::exception& e) {
+    return report(error, VECOPS_STATUS_EXECUTION_ERROR, e.what());
+  } catch (...) {
+    return report(error, VECOPS_STATUS_EXECUTION_ERROR, "unknown exception in the kernel artifact");
+  }
+}
+
+const VecopsKernelDescriptorV1 kDescriptor = {
+  sizeof(VecopsKernelDescriptorV1),
+  VECOPS_KERNEL_ABI_VERSION_MAJOR,
+  VECOPS_KERNEL_ABI_VERSION_MINOR,
+  kOperatorName,
+  kKey,
+  static_cast<uint32_t>(sizeof(kParameters) / sizeof(kParameters[0])),
+  sizeof(VecopsParameterDescriptor),
+  kParameters,
+  workspace_entry,
+  run_entry,
+  0,
+};
+
+}  // namespace
+
+extern "C" VECOPS_RUNTIME_EXPORT const VecopsKernelDescriptorV1* vecops_kernel_query_v1(void) { return &kDescriptor; }

@@ -1,0 +1,373 @@
+#include "matmul_plugin.hpp"
+
+#include <algorithm>
+
+namespace vecops::hip {
+
+namespace {
+
+using rt::DType;
+using rt::Status;
+using rt::StatusCode;
+using rt::TensorView;
+using rt::Value;
+
+Status invalid(std::string m) { return Status(StatusCode::InvalidArgument, std::move(m)); }
+Status not_applicable(std::string m) { return Status(StatusCode::NotApplicable, std::move(m)); }
+
+const TensorView* tensor_at(std::span<const Value> values, std::size_t i) {
+  return i < values.size() ? std::get_if<TensorView>(&values[i]) : nullptr;
+}
+
+rt::ParameterSchema tensor_param(std::string name, std::uint64_t dtypes, std::optional<std::uint32_t> rank,
+                                 std::uint64_t flags, bool optional = false) {
+  rt::TensorConstraint c;
+  c.dtype_mask = dtypes;
+  c.rank = rank;
+  c.required_flags = flags;
+  c.optional = optional;
+  return rt::ParameterSchema{std::move(name), std::move(c)};
+}
+
+std::int64_t rows(const TensorView& t) { return t.sizes[t.sizes.size() - 2]; }
+std::int64_t cols(const TensorView& t) { return t.sizes[t.sizes.size() - 1]; }
+
+// A = [..,M,K], B = [..,N,K], C_in / C = [..,M,N]; ranks 2 or 3 and all equal;
+// batch extents equal (planning/families/ArchitectureFamily.h:1590-1652).
+Status matmul_relations(std::span<const Value> v) {
+  const TensorView* a = tensor_at(v, 0);
+  const TensorView* b = tensor_at(v, 1);
+  const TensorView* cin = tensor_at(v, 2);
+  const TensorView* c = tensor_at(v, 3);
+  if (a == nullptr || b == nullptr || c == nullptr) return invalid("vecops::matmul needs a, b and c tensors");
+  const std::size_t rank = a->sizes.size();
+  if (rank != 2 && rank != 3) return invalid("a must have rank 2 or 3");
+  if (b->sizes.size() != rank || c->sizes.size() != rank || (cin && cin->sizes.size() != rank))
+    return invalid("a, b, c_in and c must have the same rank");
+  if (cols(*a) != cols(*b)) return invalid("a and b disagree on K");
+  if (rows(*c) != rows(*a) || cols(*c) != rows(*b)) return invalid("c must be [.., M, N]");
+  if (cin && (rows(*cin) != rows(*c) || cols(*cin) != cols(*c))) return invalid("c_in must be [.., M, N]");
+  if (rank == 3) {
+    if (a->sizes[0] != b->sizes[0] || a->sizes[0] != c->sizes[0] || (cin && cin->sizes[0] != c->sizes[0]))
+      return invalid("batch extents differ");
+  }
+  return Status::success();
+}
+
+Status dequant_relations(std::span<const Value> v) {
+  const TensorView* a = tensor_at(v, 0);
+  const TensorView* b = tensor_at(v, 1);
+  const TensorView* rs = tensor_at(v, 2);
+  const TensorView* cs = tensor_at(v, 3);
+  const TensorView* corr = tensor_at(v, 4);
+  const TensorView* c = tensor_at(v, 5);
+  if (!a || !b || !rs || !cs || !c) return invalid("vecops::matmul_i8_dequant needs a, b, both scale vectors and c");
+  if (a->sizes[1] != b->sizes[1]) return invalid("a and b disagree on K");
+  if (c->sizes[0] != a->sizes[0] || c->sizes[1] != b->sizes[0]) return invalid("c must be [M, N]");
+  if (rs->sizes[0] != a->sizes[0]) return invalid("row_scales must have M entries");
+  if (cs->sizes[0] != b->sizes[0]) return invalid("column_scales must have N entries");
+  if (corr && corr->sizes[0] != b->sizes[0]) return invalid("correction must have N entries");
+  return Status::success();
+}
+
+Status w8a16_relations(std::span<const Value> v) {
+  const TensorView* x = tensor_at(v, 0);
+  const TensorView* w = tensor_at(v, 1);
+  const TensorView* s = tensor_at(v, 2);
+  const TensorView* y = tensor_at(v, 3);
+  if (!x || !w || !s || !y) return invalid("vecops::matmul_w8a16_group needs x, w, scales and y");
+  if (x->sizes[1] != w->sizes[1]) return invalid("x and w disagree on K");
+  if (y->sizes[0] != x->sizes[0] || y->sizes[1] != w->sizes[0]) return invalid("y must be [M, N]");
+  if (s->sizes[0] != w->sizes[0]) return invalid("scales must have N rows");
+  return Status::success();
+}
+
+// Placement of a call: all tensors on the host, or all on the device.
+rt::Result<Placement> placement_of(const rt::KernelCall& call) {
+  bool host = false, device = false;
+  for (const Value& v : call.arguments().values()) {
+    if (const auto* t = std::get_if<TensorView>(&v)) {
+      if (t->device_type == VECOPS_DEVICE_CPU) host = true;
+      else if (t->device_type == VECOPS_DEVICE_PRIVATE) device = true;
+      else return not_applicable("tensors must be host (CPU) or HIP device (PRIVATE) memory");
+    }
+  }
+  if (host && device) return not_applicable("tensors of one call must all be host or all be device memory");
+  return device ? Placement::Device : Placement::Host;
+}
+
+const char* placement_name(Placement p) { return p == Placement::Device ? "device" : "host"; }
+
+rt::Result<DType> compute_type(const rt::KernelCall& call) {
+  auto it = call.values().find("ComputeType");
+  if (it == call.values().end()) return DType::BFloat16;
+  if (const auto* d = std::get_if<DType>(&it->second)) return *d;
+  return invalid("ComputeType must be a DType");
+}
+
+rt::Result<std::int64_t> group_size(const rt::KernelCall& call) {
+  auto it = call.values().find("G");
+  if (it == call.values().end()) return std::int64_t{128};
+  if (const auto* g = std::get_if<std::int64_t>(&it->second)) return *g;
+  return invalid("G must be an integer");
+}
+
+constexpr const char* kBackend = "backend=hip-gfx950";
+
+std::shared_ptr<rt::Operator> assemble(rt::OperatorSchema schema,
+                                       std::vector<std::shared_ptr<const rt::KernelRecipe>> recipes,
+                                       const std::filesystem::path& dir) {
+  return std::make_shared<rt::Operator>(std::move(schema), std::move(recipes),
+                                        std::make_shared<MatmulDispatchPolicy>(),
+                                        std::make_shared<HipExecutableProvider>(dir));
+}
+
+}  // namespace
+
+// ---- schemas -----------------------------------------------------------------------------------
+
+rt::OperatorSchema make_matmul_schema() {
+  using rt::dtype_bit;
+  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8);
+  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int32);
+  std::vector<rt::ParameterSchema> params;
+  params.push_back(tensor_param("a", in, std::nullopt, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("b", in, std::nullopt, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("c_in", out, std::nullopt, VECOPS_TENSOR_READ, /*optional=*/true));
+  params.push_back(tensor_param("c", out, std::nullopt, VECOPS_TENSOR_WRITE));
+  return rt::OperatorSchema(kMatmulName, std::move(params), matmul_relations);
+}
+
+rt::OperatorSchema make_matmul_i8_dequant_schema() {
+  using rt::dtype_bit;
+  std::vector<rt::ParameterSchema> params;
+  params.push_back(tensor_param("a", dtype_bit(DType::Int8), 2u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("b", dtype_bit(DType::Int8), 2u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("row_scales", dtype_bit(DType::Float32), 1u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("column_scales", dtype_bit(DType::Float32), 1u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("correction", dtype_bit(DType::Int32), 1u, VECOPS_TENSOR_READ, /*optional=*/true));
+  params.push_back(tensor_param("c", dtype_bit(DType::Float32), 2u, VECOPS_TENSOR_WRITE));
+  return rt::OperatorSchema(kMatmulI8DequantName, std::move(params), dequant_relations);
+}
+
+rt::OperatorSchema make_matmul_w8a16_group_schema() {
+  using rt::dtype_bit;
+  std::vector<rt::ParameterSchema> params;
+  params.push_back(tensor_param("x", dtype_bit(DType::BFloat16), 2u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("w", dtype_bit(DType::Int8), 2u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("scales", dtype_bit(DType::Float32), 2u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("y", dtype_bit(DType::BFloat16), 2u, VECOPS_TENSOR_WRITE));
+  return rt::OperatorSchema(kMatmulW8A16GroupName, std::move(params), w8a16_relations);
+}
+
+// ---- recipes ------------------------------------------------------------------------------------
+
+MatmulRecipe::MatmulRecipe(OperandClass operands) : operands_(operands) {
+  id_ = operands == OperandClass::BF16 ? "hip.matmul.bf16.tile"
+        : operands == OperandClass::F32 ? "hip.matmul.f32.tile"
+                                        : "hip.matmul.i8.tile";
+}
+
+Status MatmulRecipe::match(const rt::KernelCall& call) const {
+  const auto values = call.arguments().values();
+  const TensorView* a = tensor_at(values, 0);
+  const TensorView* b = tensor_at(values, 1);
+  const TensorView* cin = tensor_at(values, 2);
+  const TensorView* c = tensor_at(values, 3);
+  if (a == nullptr || b == nullptr || c == nullptr) return invalid("vecops::matmul needs a, b and c tensors");
+  const DType want = operands_ == OperandClass::BF16 ? DType::BFloat16
+                     : operands_ == OperandClass::F32 ? DType::Float32
+                                                      : DType::Int8;
+  if (a->dtype != want || b->dtype != want) return not_applicable("operand dtypes belong to another recipe");
+  const bool int_out = operands_ == OperandClass::I8;
+  if (int_out ? c->dtype != DType::Int32 : (c->dtype != DType::Float32 && c->dtype != DType::BFloat16))
+    return not_applicable("output dtype does not fit these operands");
+  if (cin != nullptr &&
+      (int_out ? cin->dtype != DType::Int32 : (cin->dtype != DType::Float32 && cin->dtype != DType::BFloat16)))
+    return not_applicable("c_in dtype does not fit these operands");
+  auto compute = compute_type(call);
+  if (!compute) return compute.status();
+  if (operands_ == OperandClass::F32) {
+    // fp32 memory: bf16 compute is built (what vecops' x86 path does); true fp32 compute is not
+    if (compute.value() != DType::BFloat16) return not_applicable("ComputeType=Float32 is not built for fp32 operands");
+  }
+  auto place = placement_of(call);
+  if (!place) return place.status();
+  return Status::success();
+}
+
+rt::Result<rt::BoundKernelRecipe> MatmulRecipe::bind(const rt::KernelCall& call) const {
+  if (Status st = match(call); !st.ok()) return st;
+  const Placement place = placement_of(call).value();
+  const char* operands = operands_ == OperandClass::BF16 ? "bf16" : operands_ == OperandClass::F32 ? "f32" : "i8";
+  const char* compute = operands_ == OperandClass::I8 ? "i32" : "bf16";
+  rt::BoundKernelRecipe bound;
+  bound.recipe_id = id_;
+  bound.specialization_key = std::string(kMatmulName) + ";operands=" + operands + ";compute=" + compute +
+                             ";memory=" + placement_name(place) + ";" + kBackend;
+  bound.artifact_key = id_ + ";" + bound.specialization_key;
+  return bound;
+}
+
+Status MatmulI8DequantRecipe::match(const rt::KernelCall& call) const {
+  auto place = placement_of(call);
+  if (!place) return place.status();
+  const auto values = call.arguments().values();
+  for (std::size_t i : {std::size_t{0}, std::size_t{1}, std::size_t{5}}) {
+    const TensorView* t = tensor_at(values, i);
+    if (t == nullptr) return invalid("vecops::matmul_i8_dequant needs a, b and c tensors");
+    if (t->strides.size() != 2 || (t->sizes[1] > 1 && t->strides[1] != 1))
+      return not_applicable("a, b and c must be contiguous along their last axis");
+  }
+  return Status::success();
+}
+
+rt::Result<rt::BoundKernelRecipe> MatmulI8DequantRecipe::bind(const rt::KernelCall& call) const {
+  if (Status st = match(call); !st.ok()) return st;
+  rt::BoundKernelRecipe bound;
+  bound.recipe_id = std::string(id());
+  bound.specialization_key = std::string(kMatmulI8DequantName) + ";operands=i8;epilogue=row_col_dequant;memory=" +
+                             placement_name(placement_of(call).value()) + ";" + kBackend;
+  bound.artifact_key = bound.recipe_id + ";" + bound.specialization_key;
+  return bound;
+}
+
+Status MatmulW8A16GroupRecipe::match(const rt::KernelCall& call) const {
+  auto place = placement_of(call);
+  if (!place) return place.status();
+  auto g = group_size(call);
+  if (!g) return g.status();
+  const auto values = call.arguments().values();
+  const TensorView* x = tensor_at(values, 0);
+  const TensorView* w = tensor_at(values, 1);
+  const TensorView* s = tensor_at(values, 2);
+  if (x == nullptr || w == nullptr || s == nullptr) return invalid("vecops::matmul_w8a16_group needs x, w and scales");
+  if (g.value() <= 0 || g.value() % 16 != 0) return invalid("G must be a positive multiple of 16");
+  if (x->sizes[1] % g.value() != 0) return invalid("K must be a multiple of G");
+  if (s->sizes[1] != x->sizes[1] / g.value()) return invalid("scales must be [N, K/G]");
+  if (x->sizes[0] > 16) return not_applicable("the skinny family takes at most 16 activation rows");
+  return Status::success();
+}
+
+rt::Result<rt::BoundKernelRecipe> MatmulW8A16GroupRecipe::bind(const rt::KernelCall& call) const {
+  if (Status st = match(call); !st.ok()) return st;
+  rt::BoundKernelRecipe bound;
+  bound.recipe_id = std::string(id());
+  bound.specialization_key = std::string(kMatmulW8A16GroupName) + ";G=" + std::to_string(group_size(call).value()) +
+                             ";memory=" + placement_name(placement_of(call).value()) + ";" + kBackend;
+  bound.artifact_key = bound.recipe_id + ";" + bound.specialization_key;
+  return bound;
+}
+
+// ---- dispatch policy --------------------------------------------------------------------------------
+
+rt::Result<std::vector<std::size_t>>
+MatmulDispatchPolicy::candidates(const rt::KernelCall& call,
+                                 std::span<const std::shared_ptr<const rt::KernelRecipe>> recipes) const {
+  std::vector<std::size_t> order;
+  const auto values = call.arguments().values();
+  const TensorView* a = tensor_at(values, 0);
+  for (std::size_t i = 0; i < recipes.size(); ++i) {
+    if (recipes[i] == nullptr) continue;
+    if (const auto* mm = dynamic_cast<const MatmulRecipe*>(recipes[i].get()); mm != nullptr && a != nullptr) {
+      const DType want = mm->operands() == OperandClass::BF16 ? DType::BFloat16
+                         : mm->operands() == OperandClass::F32 ? DType::Float32
+                                                               : DType::Int8;
+      if (a->dtype != want) continue;
+    }
+    order.push_back(i);
+  }
+  if (order.empty())
+    return Status(StatusCode::NotFound, "no recipe of this operator takes operands of this dtype");
+  return order;
+}
+
+// ---- provider -----------------------------------------------------------------------------------------
+
+std::string artifact_file_name(std::string_view key) {
+  std::string name;
+  name.reserve(key.size() + 3);
+  for (const char ch : key) {
+    const bool keep = (ch >= 'A' && ch <= 'Z') || (ch >= 'a' && ch <= 'z') || (ch >= '0' && ch <= '9') || ch == '_' ||
+                      ch == '.' || ch == '=' || ch == '-';
+    name.push_back(keep ? ch : '_');
+  }
+  return name + ".so";
+}
+
+HipExecutableProvider::HipExecutableProvider(std::filesystem::path artifact_directory)
+  : directory_(std::move(artifact_directory)) {}
+
+std::filesystem::path HipExecutableProvider::artifact_path(std::string_view specialization_key) const {
+  return directory_ / artifact_file_name(specialization_key);
+}
+
+std::size_t HipExecutableProvider::loads() const {
+  std::lock_guard<std::mutex> lock(mutex_);
+  return loads_;
+}
+
+rt::Result<std::shared_ptr<rt::Executable>> HipExecutableProvider::resolve(const rt::BoundKernelRecipe& recipe) {
+  const std::string& key = recipe.specialization_key;
+  std::shared_ptr<Pending> mine;
+  {
+    std::unique_lock<std::mutex> lock(mutex_);
+    for (;;) {
+      if (auto it = loaded_.find(key); it != loaded_.end()) return it->second;
+      auto waiting = pending_.find(key);
+      if (waiting == pending_.end()) break;
+      auto other = waiting->second;  // another thread is loading this key: wait for it
+      other->ready.wait(lock, [&] { return other->done; });
+    }
+    mine = std::make_shared<Pending>();
+    pending_.emplace(key, mine);
+  }
+  auto finish = [&](std::shared_ptr<rt::Executable> executable) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (executable != nullptr) {
+      loaded_.emplace(key, std::move(executable));
+      ++loads_;
+    }
+    pending_.erase(key);
+    mine->done = true;
+    mine->ready.notify_all();
+  };
+  const std::filesystem::path path = artifact_path(key);
+  std::error_code ec;
+  if (!std::filesystem::exists(path, ec)) {
+    finish(nullptr);
+    return Status(StatusCode::NotFound, "no HIP artifact for " + key + " (expected " + path.string() + ")");
+  }
+  auto executable = rt::Executable::load(path);
+  if (!executable) {
+    finish(nullptr);
+    return executable.status();
+  }
+  if (executable.value()->specialization_key() != key) {
+    finish(nullptr);
+    return Status(StatusCode::AbiMismatch, path.string() + " carries specialization key '" +
+                                             std::string(executable.value()->specialization_key()) + "', wanted '" +
+                                             key + "'");
+  }
+  finish(executable.value());
+  return executable;
+}
+
+// ---- operators ---------------------------------------------------------------------------------------------
+
+std::shared_ptr<rt::Operator> make_matmul_operator(const std::filesystem::path& dir) {
+  return assemble(make_matmul_schema(),
+                  {std::make_shared<MatmulRecipe>(OperandClass::BF16), std::make_shared<MatmulRecipe>(OperandClass::F32),
+                   std::make_shared<MatmulRecipe>(OperandClass::I8)},
+                  dir);
+}
+
+std::shared_ptr<rt::Operator> make_matmul_i8_dequant_operator(const std::filesystem::path& dir) {
+  return assemble(make_matmul_i8_dequant_schema(), {std::make_shared<MatmulI8DequantRecipe>()}, dir);
+}
+
+std::shared_ptr<rt::Operator> make_matmul_w8a16_group_operator(const std::filesystem::path& dir) {
+  return assemble(make_matmul_w8a16_group_schema(), {std::make_shared<MatmulW8A16GroupRecipe>()}, dir);
+}
+
+}  // namespace vecops::hip

@@ -1,0 +1,139 @@
+// The MI355X drop-in for the vecops matmul path: operator schemas, kernel
+// recipes, the shape-class dispatch policy and the executable provider that
+// hands out ahead-of-time built HIP artifact DSOs.  Everything here implements
+// vecops' own plug-in interfaces (runtime/Operator.h:67-191); an application
+// builds `Operator(schema, recipes, policy, provider)` exactly as it would for
+// any other vecops backend.
+//
+// Logical operators (vecops ships no matmul OperatorSchema; at its C++ level the
+// scales ride on tensor specs as functor transforms, matmul/Quantization.h:91-250,
+// which cannot cross the C ABI, so they are positional tensors here; outputs
+// last and caller-allocated, runtime/KernelDefinition.h:217-229):
+//
+//   vecops::matmul              (a[..,M,K], b[..,N,K], c_in?[..,M,N], c[..,M,N] out)
+//       specialization value  ComputeType : DType   (BFloat16 default, Float32)
+//   vecops::matmul_i8_dequant   (a i8[M,K], b i8[N,K], row_scales f32[M],
+//                                column_scales f32[N], correction? i32[N], c f32[M,N] out)
+//   vecops::matmul_w8a16_group  (x bf16[M,K], w i8[N,K], scales f32[N,K/G], y bf16[M,N] out)
+//       specialization value  G : ConstInt          (128 default)
+#ifndef VECOPS_HIP_MATMUL_PLUGIN_HPP
+#define VECOPS_HIP_MATMUL_PLUGIN_HPP
+
+#include <condition_variable>
+#include <filesystem>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "vecops_rt/surface.hpp"
+
+namespace vecops::hip {
+
+namespace rt = ::vecops::runtime;
+
+inline constexpr const char* kMatmulName = "vecops::matmul";
+inline constexpr const char* kMatmulI8DequantName = "vecops::matmul_i8_dequant";
+inline constexpr const char* kMatmulW8A16GroupName = "vecops::matmul_w8a16_group";
+
+// Schemas.  Ranks are left open on vecops::matmul (rank 2 and rank 3 go through
+// one operator); the relation validator enforces what the CPU path asserts in
+// validate() (planning/families/ArchitectureFamily.h:1590-1652,
+// planning/families/GenericTiled.h:100-154): equal ranks, A=[..,M,K], B=[..,N,K],
+// C=[..,M,N], equal batch extents.
+rt::OperatorSchema make_matmul_schema();
+rt::OperatorSchema make_matmul_i8_dequant_schema();
+rt::OperatorSchema make_matmul_w8a16_group_schema();
+
+// Operand classes of vecops::matmul, one artifact each.
+enum class OperandClass { BF16, F32, I8 };
+
+// Kernel families a recipe stands for: the MFMA workgroup-tile kernels or the
+// wavefront split-K dot-product kernels for skinny shapes.
+enum class KernelFamily { Tile, Skinny };
+
+// Where the tensors of a call live.  Host tensors are staged through device
+// memory inside the artifact; device tensors (VECOPS_DEVICE_PRIVATE carrying HIP
+// device pointers) are used in place.
+enum class Placement { Host, Device };
+
+// Recipe of vecops::matmul for one operand class.  match() is metadata-only:
+// dtype class, ComputeType, uniform placement.  bind() yields
+//   vecops::matmul;operands=<bf16|f32|i8>;compute=<bf16|f32|i32>;memory=<host|device>;backend=hip-gfx950
+class MatmulRecipe final : public rt::KernelRecipe {
+public:
+  explicit MatmulRecipe(OperandClass operands);
+  [[nodiscard]] std::string_view id() const override { return id_; }
+  [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
+  [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
+  [[nodiscard]] OperandClass operands() const { return operands_; }
+
+private:
+  OperandClass operands_;
+  std::string id_;
+};
+
+// vecops::matmul_i8_dequant:  ...;operands=i8;epilogue=row_col_dequant;memory=..;backend=hip-gfx950
+class MatmulI8DequantRecipe final : public rt::KernelRecipe {
+public:
+  [[nodiscard]] std::string_view id() const override { return "hip.matmul_i8_dequant.tile"; }
+  [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
+  [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
+};
+
+// vecops::matmul_w8a16_group, skinny family (M <= 16):  ...;G=<group>;memory=..;backend=hip-gfx950
+class MatmulW8A16GroupRecipe final : public rt::KernelRecipe {
+public:
+  [[nodiscard]] std::string_view id() const override { return "hip.matmul_w8a16_group.skinny"; }
+  [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
+  [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
+};
+
+// GPU counterpart of the call sites of vecops' runtime shape predicates
+// (matmul/details/kernel/amx/Backend.h:2724-2757 consulting
+// src/MatmulRuntimeDispatch.cpp:12-32): orders the recipes of an operator for
+// one call.  Recipes whose operand class cannot take the call are dropped (they
+// would answer NotApplicable anyway); the rest keep declaration order.
+class MatmulDispatchPolicy final : public rt::DispatchPolicy {
+public:
+  [[nodiscard]] rt::Result<std::vector<std::size_t>>
+  candidates(const rt::KernelCall& call, std::span<const std::shared_ptr<const rt::KernelRecipe>> recipes) const override;
+};
+
+// Resolves bound recipes to artifact DSOs found in one directory
+// (<directory>/<file name derived from the specialization key>.so).  Never
+// builds: a missing artifact is NotFound, like vecops' provider in CacheOnly
+// mode (src/runtime/Provider.cpp:175-236).  Thread-safe; identical concurrent
+// requests load the DSO once.
+class HipExecutableProvider final : public rt::ExecutableProvider {
+public:
+  explicit HipExecutableProvider(std::filesystem::path artifact_directory);
+  [[nodiscard]] rt::Result<std::shared_ptr<rt::Executable>> resolve(const rt::BoundKernelRecipe& recipe) override;
+  // File an artifact with this key is expected under.
+  [[nodiscard]] std::filesystem::path artifact_path(std::string_view specialization_key) const;
+  [[nodiscard]] std::size_t loads() const;  // DSOs actually loaded so far (tests)
+
+private:
+  struct Pending {
+    std::condition_variable ready;
+    bool done = false;
+  };
+  std::filesystem::path directory_;
+  mutable std::mutex mutex_;
+  std::map<std::string, std::shared_ptr<rt::Executable>, std::less<>> loaded_;
+  std::map<std::string, std::shared_ptr<Pending>, std::less<>> pending_;
+  std::size_t loads_ = 0;
+};
+
+// File name (without directory) of the artifact for a specialization key:
+// characters outside [A-Za-z0-9_.=-] become '_', plus ".so".
+std::string artifact_file_name(std::string_view specialization_key);
+
+// Ready-made operators over one artifact directory.
+std::shared_ptr<rt::Operator> make_matmul_operator(const std::filesystem::path& artifact_directory);
+std::shared_ptr<rt::Operator> make_matmul_i8_dequant_operator(const std::filesystem::path& artifact_directory);
+std::shared_ptr<rt::Operator> make_matmul_w8a16_group_operator(const std::filesystem::path& artifact_directory);
+
+}  // namespace vecops::hip
+#endif
