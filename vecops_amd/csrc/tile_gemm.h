@@ -118,10 +118,14 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
 
 // Fast path: one whole 16-byte chunk, no bounds checks (the caller guarantees
 // that the row exists and that the chunk lies inside K).
+#define VECOPS_GLOBAL __attribute__((address_space(1)))
+
 template <int SRC>
 __device__ __forceinline__ u32x4 load_chunk_fast(const char* src) {
+  // global address space spelled out: a generic (flat) load would also count
+  // against the LDS counter and stall the LDS-only waits of the main loop
   if constexpr (SRC == SRC_F32_AS_BF16) {
-    const f32x4* p = reinterpret_cast<const f32x4*>(src);
+    const VECOPS_GLOBAL f32x4* p = (const VECOPS_GLOBAL f32x4*)(src);
     const f32x4 lo = p[0], hi = p[1];
     u32x4 out;
     out.x = cvt_pk_bf16(lo.x, lo.y);
@@ -130,7 +134,7 @@ __device__ __forceinline__ u32x4 load_chunk_fast(const char* src) {
     out.w = cvt_pk_bf16(hi.z, hi.w);
     return out;
   } else {
-    return *reinterpret_cast<const u32x4*>(src);
+    return *(const VECOPS_GLOBAL u32x4*)(src);
   }
 }
 
@@ -169,6 +173,24 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for<N - 1>(f);
     f(std::integral_constant<int, N - 1>{});
   }
+}
+
+// Scheduling hint for one k-step of the main loop: spread N_A instructions of
+// class MASK_A and N_B of class MASK_B evenly between the N_MFMA matrix
+// instructions, so that each memory instruction issues in the shadow of an MFMA
+// instead of in a clump that leaves the matrix pipe idle.
+// Classes (llvm.amdgcn.sched.group.barrier): 0x008 MFMA, 0x020 VMEM read,
+// 0x100 LDS read, 0x200 LDS write.
+template <int N_MFMA, int N_A, int MASK_A, int N_B, int MASK_B>
+__device__ __forceinline__ void interleave_hint() {
+  static_for<N_MFMA>([&](auto ci) {
+    constexpr int i = decltype(ci)::value;
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    constexpr int a = (i + 1) * N_A / N_MFMA - i * N_A / N_MFMA;
+    constexpr int b = (i + 1) * N_B / N_MFMA - i * N_B / N_MFMA;
+    if constexpr (a > 0) __builtin_amdgcn_sched_group_barrier(MASK_A, a, 0);
+    if constexpr (b > 0) __builtin_amdgcn_sched_group_barrier(MASK_B, b, 0);
+  });
 }
 
 // Accumulator tile type per operand class.
@@ -287,6 +309,8 @@ template <int SRC, int LOAD, int ROWS>
 struct Stager {
   using T = SrcTraits<SRC>;
   static constexpr int CHUNKS = ROWS / 32;
+  static constexpr int kLdsStores = CHUNKS;  // per thread and K tile
+  static constexpr int kGlobalLoads = (LOAD == LOAD_KVEC) ? CHUNKS * (SRC == SRC_F32_AS_BF16 ? 2 : 1) : 0;
   const char* base;
   int64_t row_bytes[CHUNKS];  // byte offset of each staged row, chunk included (fast path)
   int64_t rs, ks;             // element strides (checked path)
@@ -310,12 +334,22 @@ struct Stager {
     }
   }
 
+  // K tile kt lies wholly inside [0, K): unconditional 16-byte loads on the vector
+  // path (the generic path has no such shortcut and checks every element).
+  __device__ __forceinline__ void fetch_full(int kt) {
+    if constexpr (LOAD == LOAD_KVEC) {
+      const int64_t k_bytes = static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes);
+#pragma unroll
+      for (int i = 0; i < CHUNKS; ++i) regs[i] = load_chunk_fast<SRC>(base + row_bytes[i] + k_bytes);
+    } else {
+      fetch(kt, 0);
+    }
+  }
+
   __device__ __forceinline__ void fetch(int kt, int full_k_tiles) {
     if constexpr (LOAD == LOAD_KVEC) {
-      if (kt < full_k_tiles) {  // whole K tile inside [0, K): unconditional 16-byte loads
-        const int64_t k_bytes = static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes);
-#pragma unroll
-        for (int i = 0; i < CHUNKS; ++i) regs[i] = load_chunk_fast<SRC>(base + row_bytes[i] + k_bytes);
+      if (kt < full_k_tiles) {
+        fetch_full(kt);
         return;
       }
     }
@@ -344,6 +378,8 @@ struct Stager<SRC, LOAD_NVEC, ROWS> {
   using T = SrcTraits<SRC>;
   static_assert(T::kElemsPerChunk == 8, "transposing stager handles 16-bit compute elements");
   static constexpr int NBLOCKS = ROWS / 8;
+  static constexpr int kLdsStores = 8;
+  static constexpr int kGlobalLoads = 8 * (SRC == SRC_F32_AS_BF16 ? 2 : 1);
   const char* base;
   const char* block_ptr;  // address of (k-block row 0, n-block) for K tile 0
   int64_t rs, ks;         // rs == 1; ks = elements between consecutive k
@@ -367,12 +403,17 @@ struct Stager<SRC, LOAD_NVEC, ROWS> {
     block_ptr = base + (static_cast<int64_t>(kb) * 8 * ks + n) * T::kSrcBytes;
   }
 
+  __device__ __forceinline__ void fetch_full(int kt) {
+    if (!active) return;
+    const char* p = block_ptr + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) regs[r] = load_chunk_fast<SRC>(p + r * ks * T::kSrcBytes);
+  }
+
   __device__ __forceinline__ void fetch(int kt, int full_k_tiles) {
     if (!active) return;
     if (kt < full_k_tiles) {
-      const char* p = block_ptr + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes;
-#pragma unroll
-      for (int r = 0; r < 8; ++r) regs[r] = load_chunk_fast<SRC>(p + r * ks * T::kSrcBytes);
+      fetch_full(kt);
       return;
     }
     // K tail: rows k >= K read as zero, columns n >= N as zero
@@ -431,6 +472,12 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
 
   int batch, split, tm, tn;
   map_workgroup(p, batch, split, tm, tn);
+  // workgroup-uniform by construction; say so, or every loop bound derived from
+  // them is treated as divergent
+  batch = __builtin_amdgcn_readfirstlane(batch);
+  split = __builtin_amdgcn_readfirstlane(split);
+  tm = __builtin_amdgcn_readfirstlane(tm);
+  tn = __builtin_amdgcn_readfirstlane(tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int total_k_tiles = (p.k + KTILE - 1) / KTILE;
@@ -460,42 +507,99 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
 #pragma unroll
   for (int j = 0; j < WN; ++j) off_b[j] = BM * 128 + lds_chunk_offset((wn * WN + j) * 32 + frag_row, frag_half);
 
-  if (kt_begin < kt_end) {
-    stager_a.fetch(kt_begin, full_k_tiles);
-    stager_b.fetch(kt_begin, full_k_tiles);
+  // The K tiles of this workgroup are walked as a sequence seq(0..nk-1): a partial
+  // last tile of K (if this split owns it) comes FIRST, so that only the prologue
+  // needs bounds-checked loads and the steady-state loop issues nothing but whole
+  // 16-byte loads (sums may be taken in any order).
+  const int nk = __builtin_amdgcn_readfirstlane(kt_end - kt_begin);
+  const int has_tail = __builtin_amdgcn_readfirstlane((nk > 0 && kt_end > full_k_tiles) ? 1 : 0);
+  auto seq = [&](int j) { return (has_tail && j == 0) ? kt_end - 1 : kt_begin + j - has_tail; };
+
+  // Software pipeline over K tiles, two LDS stages, two fragment register sets:
+  //   k-step 0 : read fragments(ks=1)                                  | MFMA on fragments(ks=0)
+  //   k-step 1 : read fragments(ks=2), store tile it+1 into other stage | MFMA
+  //   k-step 2 : read fragments(ks=3), issue global loads of tile it+2   | MFMA
+  //   barrier  : every wave's reads of this stage and stores into the other are done
+  //   k-step 3 : read fragments(ks=0) of tile it+1 from the other stage  | MFMA
+  // Global loads get a whole tile of MFMA work to land; LDS reads one k-step.
+  u32x4 fa[2][WM], fb[2][WN];
+  auto read_frags = [&](int set, const char* tile, int ks) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) fa[set][i] = *reinterpret_cast<const u32x4*>(tile + (off_a[i] ^ (ks << 5)));
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb[set][j] = *reinterpret_cast<const u32x4*>(tile + (off_b[j] ^ (ks << 5)));
+  };
+  auto mfma_all = [&](int set) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j) mfma_step<SRC>(acc[i][j], fa[set][i], fb[set][j]);
+  };
+  // workgroup barrier that waits only for this wave's LDS traffic, not for the
+  // global prefetch in flight
+  auto lds_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0), vmcnt / expcnt untouched
+    __builtin_amdgcn_s_barrier();
+  };
+
+  if (nk > 0) {
+    stager_a.fetch(seq(0), full_k_tiles);
+    stager_b.fetch(seq(0), full_k_tiles);
     stager_a.commit(lds);
     stager_b.commit(lds + BM * 128);
-  }
-  __syncthreads();
-
-  for (int kt = kt_begin; kt < kt_end; ++kt) {
-    const int stage = (kt - kt_begin) & 1;
-    const bool more = kt + 1 < kt_end;
-    if (more) {
-      stager_a.fetch(kt + 1, full_k_tiles);
-      stager_b.fetch(kt + 1, full_k_tiles);
-    }
-
-    const char* tile = lds + stage * STAGE_BYTES;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      u32x4 fa[WM], fb[WN];
-#pragma unroll
-      for (int i = 0; i < WM; ++i) fa[i] = *reinterpret_cast<const u32x4*>(tile + (off_a[i] ^ (ks << 5)));
-#pragma unroll
-      for (int j = 0; j < WN; ++j) fb[j] = *reinterpret_cast<const u32x4*>(tile + (off_b[j] ^ (ks << 5)));
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j) mfma_step<SRC>(acc[i][j], fa[i], fb[j]);
-    }
-
-    if (more) {
-      char* next = lds + (stage ^ 1) * STAGE_BYTES;
-      stager_a.commit(next);
-      stager_b.commit(next + BM * 128);
+    const int full_in_range = nk - has_tail;  // whole K tiles this workgroup owns
+    if (nk > 1) {
+      stager_a.fetch_full(seq(1));
+      stager_b.fetch_full(seq(1));
     }
     __syncthreads();
+    read_frags(0, lds, 0);
+
+    // The loop body is one straight-line block: stores into the other stage,
+    // prefetches (tile index clamped to the last one) and the fragment reads of the
+    // next tile are issued unconditionally; the surplus ones of the final
+    // iterations touch valid memory and are never consumed.
+    auto main_loop = [&](auto prefetch_tag) {
+      constexpr bool PREFETCH = decltype(prefetch_tag)::value;
+      for (int it = 0; it < nk; ++it) {
+        const char* tile = lds + (it & 1) * STAGE_BYTES;
+        char* other = lds + ((it & 1) ^ 1) * STAGE_BYTES;
+
+        constexpr int N_MFMA = WM * WN, N_READ = WM + WN;
+        constexpr int N_STORE = Stager<SRC, LOAD_A, BM>::kLdsStores + Stager<SRC, LOAD_B, BN>::kLdsStores;
+        constexpr int N_LOAD = Stager<SRC, LOAD_A, BM>::kGlobalLoads + Stager<SRC, LOAD_B, BN>::kGlobalLoads;
+
+        read_frags(1, tile, 1);
+        mfma_all(0);
+        interleave_hint<N_MFMA, N_READ, 0x100, 0, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+
+        read_frags(0, tile, 2);
+        stager_a.commit(other);
+        stager_b.commit(other + BM * 128);
+        mfma_all(1);
+        interleave_hint<N_MFMA, N_READ, 0x100, N_STORE, 0x200>();
+        __builtin_amdgcn_sched_barrier(0);
+
+        read_frags(1, tile, 3);
+        if constexpr (PREFETCH) {
+          const int t2 = seq(max(has_tail, min(it + 2, nk - 1)));
+          stager_a.fetch_full(t2);
+          stager_b.fetch_full(t2);
+        }
+        mfma_all(0);
+        interleave_hint<N_MFMA, N_READ, 0x100, PREFETCH ? N_LOAD : 0, 0x020>();
+        __builtin_amdgcn_sched_barrier(0);
+
+        lds_barrier();
+        read_frags(0, other, 0);
+        mfma_all(1);
+        interleave_hint<N_MFMA, N_READ, 0x100, 0, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    if (full_in_range > 0) main_loop(std::true_type{});
+    else main_loop(std::false_type{});
   }
 
   // Epilogue.  Accumulator register r of lane l is C[(r/4)*8 + (l/32)*4 + r%4][l%32]
