@@ -274,11 +274,20 @@ void make_operand(VecopsHipOperand* o, const void* data, uint32_t dtype, int64_t
   o->strides[1] = 1;
 }
 
-template <int MB, int ROWS>
+template <int MB, int ROWS, int UNROLL>
 void launch_skinny(const SkinnyW8A16Params& p, hipStream_t stream) {
   const int64_t waves = (p.n + ROWS - 1) / ROWS;
   const int64_t blocks = (waves + 3) / 4;
-  hipLaunchKernelGGL((skinny_w8a16_kernel<MB, ROWS>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL((skinny_w8a16_kernel<MB, ROWS, UNROLL>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                     p);
+}
+
+template <int SPG, int TILES>
+void launch_skinny_mfma(const SkinnyW8A16Params& p, hipStream_t stream) {
+  constexpr int kWaves = 8;
+  const int64_t blocks = (p.n + 16 * TILES - 1) / (16 * TILES);
+  hipLaunchKernelGGL((skinny_w8a16_mfma_kernel<kWaves, SPG, TILES>), dim3(static_cast<unsigned>(blocks)),
+                     dim3(64 * kWaves), 0, stream, p);
 }
 
 }  // namespace
@@ -377,11 +386,19 @@ int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t ldx, const int8_t* 
   p.group = static_cast<int32_t>(group);
   p.groups = static_cast<int32_t>(k / group);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (m == 1) launch_skinny<1, 8>(p, s);
-  else if (m == 2) launch_skinny<2, 8>(p, s);
-  else if (m <= 4) launch_skinny<4, 4>(p, s);
-  else if (m <= 8) launch_skinny<8, 2>(p, s);
-  else launch_skinny<16, 2>(p, s);
+  // GPU rule table of the skinny family: matrix cores once the widening of a weight
+  // byte can be shared by three or more activation rows
+  const bool mfma_ok = group % 64 == 0 && (group == 64 || group == 128 || group == 256);
+  if (m >= 3 && mfma_ok) {
+    const int tiles = m > 4 ? 2 : 1;  // more weight rows per workgroup = fewer activation reloads
+    if (group == 64) { if (tiles == 2) launch_skinny_mfma<1, 2>(p, s); else launch_skinny_mfma<1, 1>(p, s); }
+    else if (group == 128) { if (tiles == 2) launch_skinny_mfma<2, 2>(p, s); else launch_skinny_mfma<2, 1>(p, s); }
+    else { if (tiles == 2) launch_skinny_mfma<4, 2>(p, s); else launch_skinny_mfma<4, 1>(p, s); }
+  } else if (m == 1) launch_skinny<1, 2, 2>(p, s);
+  else if (m == 2) launch_skinny<2, 2, 2>(p, s);
+  else if (m <= 4) launch_skinny<4, 2, 1>(p, s);
+  else if (m <= 8) launch_skinny<8, 2, 1>(p, s);
+  else launch_skinny<16, 1, 1>(p, s);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(ST_EXEC, "skinny kernel launch: %s", hipGetErrorString(e));
   return ST_OK;

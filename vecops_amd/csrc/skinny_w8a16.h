@@ -1,15 +1,17 @@
 // Decode-shaped weight-only int8 matmul for gfx950 (HBM-bound):
 //   y[m,n] = bf16( sum_g S[n,g] * sum_{k in g} float(x[m,k]) * float(W[n,k]) ),  M <= 16.
 //
-// The weight matrix is read exactly once, 16 bytes per lane per load, a whole
-// wavefront reading 1 KiB contiguous of one weight row.  A wavefront owns ROWS
-// consecutive weight rows and walks K in steps of 1024 elements; the activation
-// chunk a lane needs (the same k range for every row) is loaded once per step
-// and reused for all ROWS rows, so activations cost 1/ROWS of the weight
-// traffic from cache.  Products and sums are fp32 (fmaf); the group scale
-// multiplies the 16-element partial sum of a lane, which never straddles a group
-// because the group size is a multiple of 16.  The per-lane sums are reduced
-// across the wavefront with DPP-free shuffles at the end.
+// The weight matrix is read exactly once.  Two kernel families:
+//  * dot-product (M <= 2, or group sizes that are not multiples of 64): a
+//    wavefront owns ROWS consecutive weight rows and reads 1 KiB contiguous of one
+//    row per load instruction (16 bytes per lane); products and sums in fp32 on the
+//    vector ALU.
+//  * matrix-core (M = 3..16): 16 weight rows x 16 activation rows per
+//    v_mfma_f32_16x16x32_bf16, so the cost of widening a weight byte is paid once
+//    for all activation rows.
+// Both widen weights with the unsigned-byte converter, u = w xor 0x80 = w + 128, and
+// use  sum_k x_k*w_k = sum_k x_k*u_k - 128 * sum_k x_k  per scale group; a lane's
+// 16-element chunk never straddles a group because group sizes are multiples of 16.
 #ifndef VECOPS_HIP_SKINNY_W8A16_H
 #define VECOPS_HIP_SKINNY_W8A16_H
 
@@ -36,13 +38,17 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-template <int MB, int ROWS>
+// ---- dot-product family (VALU): one wavefront owns ROWS consecutive weight rows ----------
+template <int MB, int ROWS, int UNROLL>
 __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const SkinnyW8A16Params p) {
   const int lane = threadIdx.x & 63;
-  const int wave_in_block = threadIdx.x >> 6;
-  const int64_t wave_id = static_cast<int64_t>(blockIdx.x) * 4 + wave_in_block;
-  const int64_t n0 = wave_id * ROWS;
+  const int wave = threadIdx.x >> 6;
+  const int64_t n0 = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * ROWS;
   if (n0 >= p.n) return;
+  const int chunks = p.k >> 4;  // 16-element chunks per row
+  const VECOPS_GLOBAL char* wbase = (const VECOPS_GLOBAL char*)p.w;
+  const VECOPS_GLOBAL uint16_t* xbase = (const VECOPS_GLOBAL uint16_t*)p.x;
+  const VECOPS_GLOBAL float* sbase = (const VECOPS_GLOBAL float*)p.scales;
 
   float acc[ROWS][MB];
 #pragma unroll
@@ -50,56 +56,67 @@ __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const SkinnyW8A16Para
 #pragma unroll
     for (int mm = 0; mm < MB; ++mm) acc[r][mm] = 0.0f;
 
-  const int chunks = p.k >> 4;
-  for (int c0 = 0; c0 < chunks; c0 += 64) {
-    const int c = c0 + lane;
-    const bool active = c < chunks;
-    const int k0 = c << 4;
-    // weights first: ROWS independent 16-byte loads in flight per lane
-    u32x4 wq[ROWS];
+  for (int c0 = 0; c0 < chunks; c0 += 64 * UNROLL) {
+    // all weight loads of this step first
+    u32x4 wq[UNROLL][ROWS];
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const int64_t n = n0 + r;
-      wq[r] = u32x4{0u, 0u, 0u, 0u};
-      if (active && n < p.n) wq[r] = *reinterpret_cast<const u32x4*>(p.w + n * p.ldw + k0);
-    }
-    const int g = active ? k0 / p.group : 0;
-    float sc[ROWS];
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * 64 + lane;
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const int64_t n = n0 + r;
-      sc[r] = (active && n < p.n) ? p.scales[n * p.groups + g] : 0.0f;
-    }
-    // activations: 16 bf16 per row of x, widened to fp32
-    float xf[MB][16];
-#pragma unroll
-    for (int mm = 0; mm < MB; ++mm) {
-      u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
-      if (active && mm < p.m) {
-        const u32x4* px = reinterpret_cast<const u32x4*>(p.x + mm * p.ldx + k0);
-        lo = px[0];
-        hi = px[1];
-      }
-      const uint32_t words[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        xf[mm][2 * e] = __uint_as_float(words[e] << 16);
-        xf[mm][2 * e + 1] = __uint_as_float(words[e] & 0xffff0000u);
+      for (int r = 0; r < ROWS; ++r) {
+        const int64_t n = n0 + r;
+        wq[u][r] = u32x4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};  // reads as w == 0
+        if (c < chunks && n < p.n)
+          wq[u][r] = *(const VECOPS_GLOBAL u32x4*)(wbase + n * p.ldw + (static_cast<int64_t>(c) << 4));
       }
     }
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const uint32_t words[4] = {wq[r].x, wq[r].y, wq[r].z, wq[r].w};
-      float wf[16];
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * 64 + lane;
+      const bool active = c < chunks;
+      const int k0 = c << 4;
+      const int g = active ? k0 / p.group : 0;
+      float sc[ROWS];
 #pragma unroll
-      for (int e = 0; e < 16; ++e)
-        wf[e] = static_cast<float>(static_cast<int8_t>((words[e >> 2] >> ((e & 3) * 8)) & 0xffu));
+      for (int r = 0; r < ROWS; ++r) {
+        const int64_t n = n0 + r;
+        sc[r] = (active && n < p.n) ? sbase[n * p.groups + g] : 0.0f;
+      }
+      // activations: 16 bf16 per row of x, widened to fp32, and their sum
+      float xf[MB][16], xsum[MB];
 #pragma unroll
       for (int mm = 0; mm < MB; ++mm) {
-        float part = 0.0f;
+        u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
+        if (active && mm < p.m) {
+          const VECOPS_GLOBAL u32x4* px = (const VECOPS_GLOBAL u32x4*)(xbase + mm * p.ldx + k0);
+          lo = px[0];
+          hi = px[1];
+        }
+        const uint32_t words[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        float s = 0.0f;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) part = fmaf(xf[mm][e], wf[e], part);
-        acc[r][mm] = fmaf(sc[r], part, acc[r][mm]);
+        for (int e = 0; e < 8; ++e) {
+          xf[mm][2 * e] = __uint_as_float(words[e] << 16);
+          xf[mm][2 * e + 1] = __uint_as_float(words[e] & 0xffff0000u);
+          s += xf[mm][2 * e];
+          s += xf[mm][2 * e + 1];
+        }
+        xsum[mm] = s;
+      }
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        const uint32_t words[4] = {wq[u][r].x ^ 0x80808080u, wq[u][r].y ^ 0x80808080u, wq[u][r].z ^ 0x80808080u,
+                                   wq[u][r].w ^ 0x80808080u};
+        float wf[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) wf[e] = static_cast<float>((words[e >> 2] >> ((e & 3) * 8)) & 0xffu);
+#pragma unroll
+        for (int mm = 0; mm < MB; ++mm) {
+          float part = -128.0f * xsum[mm];
+#pragma unroll
+          for (int e = 0; e < 16; ++e) part = fmaf(xf[mm][e], wf[e], part);
+          acc[r][mm] = fmaf(sc[r], part, acc[r][mm]);
+        }
       }
     }
   }
@@ -112,6 +129,142 @@ __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const SkinnyW8A16Para
       const int64_t n = n0 + r;
       if (lane == 0 && mm < p.m && n < p.n) p.y[mm * p.ldy + n] = static_cast<uint16_t>(bf16_bits_rne(total));
     }
+  }
+}
+
+// ---- matrix-core family: a workgroup owns TILES x 16 weight rows, its WAVES wavefronts
+// split K by scale groups --------------------------------------------------------------------
+// One v_mfma_f32_16x16x32_bf16 multiplies 16 weight rows x 32 k by 32 k x 16
+// activation rows (M padded to 16 with zeros).  Lane l holds weight row l % 16 and
+// the 16 consecutive k of quarter l / 16 of a 64-element step (one 16-byte load),
+// which feed two MFMAs; the activation operand uses the same k order.  Weights are
+// widened byte -> fp32 -> bf16 (exact for 0..255) as u = w + 128, and a second
+// MFMA against an all-ones operand accumulates sum_k x[m,k] of the group, so that
+//   acc += S[n,g] * (sum_k u*x - 128 * sum_k x).
+// Loads run D = 4 steps ahead of their use (flat software pipeline across groups).
+// SPG = 64-element steps per scale group (group size / 64).
+template <int WAVES, int SPG, int TILES>
+__global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_mfma_kernel(const SkinnyW8A16Params p) {
+  constexpr int D = 4;
+  static_assert(D % SPG == 0, "pipeline depth must hold whole groups");
+  __shared__ float red[WAVES][TILES][16 * 16];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * (16 * TILES);
+  const int row = lane & 15, quarter = lane >> 4;
+  const int gpw = (p.groups + WAVES - 1) / WAVES;
+  const int g_begin = min(p.groups, wave * gpw), g_end = min(p.groups, g_begin + gpw);
+  const int total = (g_end - g_begin) * SPG;  // steps of this wavefront
+  // rows past N are clamped: computed, never stored
+  const VECOPS_GLOBAL char* wrow[TILES];
+  const VECOPS_GLOBAL float* srow[TILES][4];
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) {
+    const int64_t n = min(n0 + t * 16 + row, static_cast<int64_t>(p.n) - 1);
+    wrow[t] = (const VECOPS_GLOBAL char*)p.w + n * p.ldw + quarter * 16 + static_cast<int64_t>(g_begin) * SPG * 64;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      srow[t][r] = (const VECOPS_GLOBAL float*)p.scales +
+                   min(n0 + t * 16 + quarter * 4 + r, static_cast<int64_t>(p.n) - 1) * p.groups + g_begin;
+  }
+  const VECOPS_GLOBAL char* xrow = (const VECOPS_GLOBAL char*)(p.x + static_cast<int64_t>(min(row, p.m - 1)) * p.ldx) +
+                                   quarter * 32 + static_cast<int64_t>(g_begin) * SPG * 128;
+  const bool x_ok = row < p.m;
+
+  f32x4 acc[TILES], dot[TILES], xs = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) {
+    acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    dot[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};  // eight bf16 1.0
+  u32x4 wq[D][TILES], x1[D], x2[D];
+  float sc[D / SPG][TILES][4];
+
+  auto issue = [&](auto slot_tag, int step) {
+    constexpr int slot = decltype(slot_tag)::value;
+    if (step < total) {
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) wq[slot][t] = *(const VECOPS_GLOBAL u32x4*)(wrow[t] + static_cast<int64_t>(step) * 64);
+      x1[slot] = u32x4{0u, 0u, 0u, 0u};
+      x2[slot] = u32x4{0u, 0u, 0u, 0u};
+      if (x_ok) {
+        const VECOPS_GLOBAL u32x4* px = (const VECOPS_GLOBAL u32x4*)(xrow + static_cast<int64_t>(step) * 128);
+        x1[slot] = px[0];
+        x2[slot] = px[1];
+      }
+      // the group's scales ride with its last step: consumed there, free when the slot is reissued
+      if constexpr (slot % SPG == SPG - 1) {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sc[slot / SPG][t][r] = srow[t][r][step / SPG];
+      }
+    }
+  };
+  auto consume = [&](auto slot_tag, int step) {
+    constexpr int slot = decltype(slot_tag)::value;
+    if (step < total) {
+      const bf16x8 b1 = __builtin_bit_cast(bf16x8, x1[slot]), b2 = __builtin_bit_cast(bf16x8, x2[slot]);
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) {
+        uint32_t a[8];
+        const uint32_t wd[4] = {wq[slot][t].x ^ 0x80808080u, wq[slot][t].y ^ 0x80808080u, wq[slot][t].z ^ 0x80808080u,
+                                wq[slot][t].w ^ 0x80808080u};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float f0 = static_cast<float>(wd[q] & 0xffu), f1 = static_cast<float>((wd[q] >> 8) & 0xffu);
+          const float f2 = static_cast<float>((wd[q] >> 16) & 0xffu), f3 = static_cast<float>(wd[q] >> 24);
+          // upper halves of two fp32 = two bf16 (exact: the values are integers below 256)
+          a[2 * q] = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+          a[2 * q + 1] = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+        }
+        const u32x4 a1 = {a[0], a[1], a[2], a[3]}, a2 = {a[4], a[5], a[6], a[7]};
+        dot[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a1), b1, dot[t], 0, 0, 0);
+        dot[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a2), b2, dot[t], 0, 0, 0);
+      }
+      xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones), b1, xs, 0, 0, 0);
+      xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones), b2, xs, 0, 0, 0);
+      if constexpr (slot % SPG == SPG - 1) {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            acc[t][r] = fmaf(sc[slot / SPG][t][r], fmaf(-128.0f, xs[r], dot[t][r]), acc[t][r]);
+            dot[t][r] = 0.0f;
+          }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) xs[r] = 0.0f;
+      }
+    }
+  };
+
+  static_for<D>([&](auto u) { issue(u, decltype(u)::value); });
+  for (int s = 0; s < total; s += D) {
+    static_for<D>([&](auto u) {
+      consume(u, s + decltype(u)::value);
+      issue(u, s + D + decltype(u)::value);
+    });
+  }
+
+  // Sum the K slices through LDS.  Accumulator register r of lane l is output
+  // (weight row quarter*4 + r, activation row l % 16) of its 16x16 tile.
+#pragma unroll
+  for (int t = 0; t < TILES; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][t][(quarter * 4 + r) * 16 + row] = acc[t][r];
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float total_sum = 0.0f;
+        for (int w = 0; w < WAVES; ++w) total_sum += red[w][t][(quarter * 4 + r) * 16 + row];
+        const int64_t n = n0 + t * 16 + quarter * 4 + r;
+        if (row < p.m && n < p.n)
+          p.y[static_cast<int64_t>(row) * p.ldy + n] = static_cast<uint16_t>(bf16_bits_rne(total_sum));
+      }
   }
 }
 

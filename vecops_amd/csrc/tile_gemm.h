@@ -186,7 +186,9 @@ __device__ __forceinline__ void interleave_hint() {
   static_for<N_MFMA>([&](auto ci) {
     constexpr int i = decltype(ci)::value;
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    constexpr int a = (i + 1) * N_A / N_MFMA - i * N_A / N_MFMA;
+    // class A (fragment reads for the next k-step) is front-loaded, one per MFMA,
+    // so the data has landed when the next k-step starts; class B is spread evenly
+    constexpr int a = i < N_A ? 1 : 0;
     constexpr int b = (i + 1) * N_B / N_MFMA - i * N_B / N_MFMA;
     if constexpr (a > 0) __builtin_amdgcn_sched_group_barrier(MASK_A, a, 0);
     if constexpr (b > 0) __builtin_amdgcn_sched_group_barrier(MASK_B, b, 0);
@@ -304,11 +306,13 @@ __device__ __forceinline__ void map_workgroup(const TileGemmParams& p, int& batc
 // fast paths: they are loaded but only feed accumulator rows/columns that are
 // never stored.
 //
-// LOAD_KVEC / LOAD_GENERIC: thread t stages chunk (t & 7) of rows (t >> 3) + 32*i.
-template <int SRC, int LOAD, int ROWS>
+// LOAD_KVEC / LOAD_GENERIC: thread t stages chunk (t & 7) of rows (t >> 3) + (THREADS/8)*i.
+template <int SRC, int LOAD, int ROWS, int THREADS>
 struct Stager {
   using T = SrcTraits<SRC>;
-  static constexpr int CHUNKS = ROWS / 32;
+  static constexpr int ROWS_PER_PASS = THREADS / 8;  // eight threads stage one 128-byte row
+  static constexpr int CHUNKS = ROWS / ROWS_PER_PASS;
+  static_assert(CHUNKS >= 1, "tile too small for this many threads");
   static constexpr int kLdsStores = CHUNKS;  // per thread and K tile
   static constexpr int kGlobalLoads = (LOAD == LOAD_KVEC) ? CHUNKS * (SRC == SRC_F32_AS_BF16 ? 2 : 1) : 0;
   const char* base;
@@ -329,7 +333,7 @@ struct Stager {
     ld_row = tid >> 3;
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
-      const int row = min(first_row + ld_row + i * 32, extent - 1);
+      const int row = min(first_row + ld_row + i * ROWS_PER_PASS, extent - 1);
       row_bytes[i] = (static_cast<int64_t>(row) * rs + ld_chunk * T::kElemsPerChunk) * T::kSrcBytes;
     }
   }
@@ -356,7 +360,7 @@ struct Stager {
     const int k0 = kt * 8 * T::kElemsPerChunk + ld_chunk * T::kElemsPerChunk;
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
-      const int row = first_row + ld_row + i * 32;
+      const int row = first_row + ld_row + i * ROWS_PER_PASS;
       regs[i] = load_chunk_checked<SRC>(base, static_cast<int64_t>(row) * rs, ks, k0, k_end, row < extent);
     }
   }
@@ -364,7 +368,7 @@ struct Stager {
   __device__ __forceinline__ void commit(char* lds_tile) const {
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i)
-      *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(ld_row + i * 32, ld_chunk)) = regs[i];
+      *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(ld_row + i * ROWS_PER_PASS, ld_chunk)) = regs[i];
   }
 };
 
@@ -373,8 +377,9 @@ struct Stager {
 // tile: it loads eight 16-byte rows along n, transposes the block in registers
 // with byte permutes and writes eight K-contiguous chunks.  16-bit compute
 // elements only (bf16, or fp32 rounded to bf16 on load).
-template <int SRC, int ROWS>
-struct Stager<SRC, LOAD_NVEC, ROWS> {
+template <int SRC, int ROWS, int THREADS>
+struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
+  static_assert(ROWS <= THREADS, "one 8x8 block per thread at most");
   using T = SrcTraits<SRC>;
   static_assert(T::kElemsPerChunk == 8, "transposing stager handles 16-bit compute elements");
   static constexpr int NBLOCKS = ROWS / 8;
@@ -453,22 +458,26 @@ struct Stager<SRC, LOAD_NVEC, ROWS> {
   }
 };
 
-template <int SRC, int WM, int WN, int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) {
+// Workgroup shapes: WAVES_M x WAVES_N wavefronts, each owning WM x WN accumulator
+// tiles of 32x32.  The 256x256 tile runs 8 wavefronts (two per SIMD, so one
+// wavefront's waits are covered by the other's MFMAs); the small tiles run 4.
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const TileGemmParams p) {
   using T = SrcTraits<SRC>;
   constexpr bool INT = T::kInt;
   using Acc = typename AccTile<INT>::type;
   constexpr int EPC = T::kElemsPerChunk;
   constexpr int KTILE = 8 * EPC;  // elements per K tile
-  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int THREADS = 64 * WAVES_M * WAVES_N;
+  constexpr int BM = 32 * WAVES_M * WM, BN = 32 * WAVES_N * WN;
   constexpr int STAGE_BYTES = (BM + BN) * 128;
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
   int batch, split, tm, tn;
   map_workgroup(p, batch, split, tm, tn);
@@ -485,8 +494,8 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
   const int kt_begin = split * p.k_tiles_per_split;
   const int kt_end = min(total_k_tiles, kt_begin + p.k_tiles_per_split);
 
-  Stager<SRC, LOAD_A, BM> stager_a;
-  Stager<SRC, LOAD_B, BN> stager_b;
+  Stager<SRC, LOAD_A, BM, THREADS> stager_a;
+  Stager<SRC, LOAD_B, BN, THREADS> stager_b;
   stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, tid);
   stager_b.init(static_cast<const char*>(p.b) + batch * p.b_bs * T::kSrcBytes, p.b_rs, p.b_ks, n0, p.n, p.k, tid);
 
@@ -523,11 +532,13 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
   //   k-step 3 : read fragments(ks=0) of tile it+1 from the other stage  | MFMA
   // Global loads get a whole tile of MFMA work to land; LDS reads one k-step.
   u32x4 fa[2][WM], fb[2][WN];
+  // read in the order the MFMAs consume: A fragment 0, every B fragment, the other A fragments
   auto read_frags = [&](int set, const char* tile, int ks) {
-#pragma unroll
-    for (int i = 0; i < WM; ++i) fa[set][i] = *reinterpret_cast<const u32x4*>(tile + (off_a[i] ^ (ks << 5)));
+    fa[set][0] = *reinterpret_cast<const u32x4*>(tile + (off_a[0] ^ (ks << 5)));
 #pragma unroll
     for (int j = 0; j < WN; ++j) fb[set][j] = *reinterpret_cast<const u32x4*>(tile + (off_b[j] ^ (ks << 5)));
+#pragma unroll
+    for (int i = 1; i < WM; ++i) fa[set][i] = *reinterpret_cast<const u32x4*>(tile + (off_a[i] ^ (ks << 5)));
   };
   auto mfma_all = [&](int set) {
 #pragma unroll
@@ -566,8 +577,8 @@ __global__ __launch_bounds__(256) void tile_gemm_kernel(const TileGemmParams p) 
         char* other = lds + ((it & 1) ^ 1) * STAGE_BYTES;
 
         constexpr int N_MFMA = WM * WN, N_READ = WM + WN;
-        constexpr int N_STORE = Stager<SRC, LOAD_A, BM>::kLdsStores + Stager<SRC, LOAD_B, BN>::kLdsStores;
-        constexpr int N_LOAD = Stager<SRC, LOAD_A, BM>::kGlobalLoads + Stager<SRC, LOAD_B, BN>::kGlobalLoads;
+        constexpr int N_STORE = decltype(stager_a)::kLdsStores + decltype(stager_b)::kLdsStores;
+        constexpr int N_LOAD = decltype(stager_a)::kGlobalLoads + decltype(stager_b)::kGlobalLoads;
 
         read_frags(1, tile, 1);
         mfma_all(0);

@@ -24,10 +24,11 @@ hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile, int mode, hipS
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
 
 // Shared by the per-class translation units.
-template <int SRC, int WM, int WN, int LA, int LB>
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB>
 hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
-  constexpr int kLds = 2 * (64 * WM + 64 * WN) * 128;
-  auto kernel = tile_gemm_kernel<SRC, WM, WN, LA, LB>;
+  constexpr int kLds = 2 * 32 * (WAVES_M * WM + WAVES_N * WN) * 128;
+  constexpr int kThreads = 64 * WAVES_M * WAVES_N;
+  auto kernel = tile_gemm_kernel<SRC, WAVES_M, WAVES_N, WM, WN, LA, LB>;
   // > 64 KiB of dynamic LDS has to be enabled once per device; cheap enough to repeat per thread.
   static thread_local int configured_device = -1;
   int device = 0;
@@ -40,24 +41,25 @@ hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
   }
   const int64_t grid = static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.batch * p.split_k;
   if (grid <= 0 || grid > INT32_MAX) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(256), kLds, stream, p);
+  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kThreads), kLds, stream, p);
   return hipGetLastError();
 }
 
-template <int SRC, int WM, int WN>
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN>
 hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t stream) {
-  if (mode == MODE_KVEC) return launch_tile_instance<SRC, WM, WN, LOAD_KVEC, LOAD_KVEC>(p, stream);
+  if (mode == MODE_KVEC) return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_KVEC>(p, stream);
   if constexpr (SrcTraits<SRC>::kElemsPerChunk == 8) {
-    if (mode == MODE_NVEC_B) return launch_tile_instance<SRC, WM, WN, LOAD_KVEC, LOAD_NVEC>(p, stream);
+    if (mode == MODE_NVEC_B)
+      return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_NVEC>(p, stream);
   }
-  return launch_tile_instance<SRC, WM, WN, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
+  return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
 }
 
 template <int SRC>
 hipError_t launch_tile_class(const TileGemmParams& p, int tile, int mode, hipStream_t stream) {
-  if (tile == 256) return launch_tile_mode<SRC, 4, 4>(p, mode, stream);
-  if (tile == 128) return launch_tile_mode<SRC, 2, 2>(p, mode, stream);
-  return launch_tile_mode<SRC, 1, 1>(p, mode, stream);
+  if (tile == 256) return launch_tile_mode<SRC, 2, 4, 4, 2>(p, mode, stream);  // 8 wavefronts of 128x64
+  if (tile == 128) return launch_tile_mode<SRC, 2, 2, 2, 2>(p, mode, stream);  // 4 wavefronts of 64x64
+  return launch_tile_mode<SRC, 2, 2, 1, 1>(p, mode, stream);                    // 4 wavefronts of 32x32
 }
 
 }  // namespace vecops_hip
