@@ -257,16 +257,17 @@ __device__ __forceinline__ void store_output(const TileGemmParams& p, int batch,
 
 // One lane's 16 accumulators of a 32x32 tile through the full epilogue, with
 // bounds checks; out of line to keep the kernels small (edge tiles, split-K
-// partials, C-input and strided C only).
+// partials, C-input and strided C only).  The lane owns output row `row` and
+// columns col0 + (r/4)*8 + r%4.
 template <bool INT>
-__device__ __noinline__ void store_tile_general(const TileGemmParams& p, int batch, int split, int row0, int col,
+__device__ __noinline__ void store_tile_general(const TileGemmParams& p, int batch, int split, int row, int col0,
                                                 typename AccTile<INT>::type tile) {
   using AccScalar = typename std::conditional<INT, int32_t, float>::type;
-  if (col >= p.n) return;
+  if (row >= p.m) return;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const int row = row0 + (r >> 2) * 8 + (r & 3);
-    if (row < p.m) {
+    const int col = col0 + (r >> 2) * 8 + (r & 3);
+    if (col < p.n) {
       if (p.split_k > 1) {
         AccScalar* part = static_cast<AccScalar*>(p.partial);
         part[((static_cast<int64_t>(split) * p.batch + batch) * p.m + row) * p.n + col] = tile[r];
@@ -458,6 +459,15 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
   }
 };
 
+// Dynamic LDS one workgroup is launched with: two staging stages, or the bf16
+// epilogue's row-major tiles if those are larger.
+template <int WAVES_M, int WAVES_N, int WM, int WN>
+constexpr int kTileLdsBytes() {
+  const int stages = 2 * 32 * (WAVES_M * WM + WAVES_N * WN) * 128;
+  const int epilogue = (WN * 32 * 2 + 16) * (WM * 32) * WAVES_M * WAVES_N;
+  return stages > epilogue ? stages : epilogue;
+}
+
 // Workgroup shapes: WAVES_M x WAVES_N wavefronts, each owning WM x WN accumulator
 // tiles of 32x32.  The 256x256 tile runs 8 wavefronts (two per SIMD, so one
 // wavefront's waits are covered by the other's MFMAs); the small tiles run 4.
@@ -544,7 +554,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
 #pragma unroll
     for (int i = 0; i < WM; ++i)
 #pragma unroll
-      for (int j = 0; j < WN; ++j) mfma_step<SRC>(acc[i][j], fa[set][i], fb[set][j]);
+      for (int j = 0; j < WN; ++j) mfma_step<SRC>(acc[i][j], fb[set][j], fa[set][i]);  // B rows first: see the epilogue
   };
   // workgroup barrier that waits only for this wave's LDS traffic, not for the
   // global prefetch in flight
@@ -613,67 +623,101 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
     else main_loop(std::false_type{});
   }
 
-  // Epilogue.  Accumulator register r of lane l is C[(r/4)*8 + (l/32)*4 + r%4][l%32]
-  // of its 32x32 tile.  Tiles that lie wholly inside C and need no C-input or
-  // split-K take one of three inline store loops; everything else goes through
-  // the general out-of-line routine.
+  // Epilogue.  The MFMAs were issued with the B tile as first operand, so the
+  // accumulators hold C transposed: register r of lane l is
+  //   C[row = l % 32][col = (r/4)*8 + (l/32)*4 + r%4]
+  // of its 32x32 tile, i.e. four consecutive columns per register quad, which
+  // become one 8-byte (bf16) or 16-byte (fp32 / int32) store.  Tiles that lie
+  // wholly inside C, need no C-input or split-K and have 16-byte aligned rows take
+  // one of three inline store loops; everything else goes through the general
+  // out-of-line routine.
   const bool interior = m0 + BM <= p.m && n0 + BN <= p.n;
-  const bool simple = interior && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1;
+  const bool aligned = (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
+  const bool simple = interior && aligned && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1;
   char* c_base = static_cast<char*>(p.c);
   if (simple && !INT && p.out_kind == OUT_BF16) {
+    // bf16: 8-byte pieces scattered over 32 rows would waste most of every memory
+    // transaction, so each wavefront first lays its tile out row-major in LDS (the
+    // staging buffers are dead by now) and then stores whole 16-byte row segments.
+    constexpr int TILE_COLS = WN * 32, TILE_ROWS = WM * 32;
+    constexpr int PITCH = TILE_COLS * 2 + 16;  // bytes; the pad staggers rows across banks
+    static_assert(PITCH * TILE_ROWS * WAVES_M * WAVES_N <= kTileLdsBytes<WAVES_M, WAVES_N, WM, WN>(),
+                  "epilogue staging must fit the launch's LDS");
+    __syncthreads();  // every wavefront is done reading fragments
+    char* mine = lds + wave * (PITCH * TILE_ROWS);
     static_for<WM>([&](auto ci) {
       constexpr int i = decltype(ci)::value;
       static_for<WN>([&](auto cj) {
         constexpr int j = decltype(cj)::value;
-        const int col = n0 + (wn * WN + j) * 32 + frag_row;
-        const int row0 = m0 + (wm * WM + i) * 32 + frag_half * 4;
-        uint16_t* dst = reinterpret_cast<uint16_t*>(c_base) + batch * p.c_bs + row0 * p.c_rs + col;
-        static_for<16>([&](auto cr) {
-          constexpr int r = decltype(cr)::value;
+        static_for<4>([&](auto cq) {
+          constexpr int q = decltype(cq)::value;
           if constexpr (!INT) {
-            dst[((r >> 2) * 8 + (r & 3)) * p.c_rs] =
-              static_cast<uint16_t>(cvt_pk_bf16(acc[i][j][r], 0.0f));
+            u32x2 v;
+            v.x = cvt_pk_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]);
+            v.y = cvt_pk_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            *reinterpret_cast<u32x2*>(mine + (i * 32 + frag_row) * PITCH + (j * 32 + q * 8 + frag_half * 4) * 2) = v;
           }
         });
       });
     });
+    // the wavefront reads back only what it wrote itself: its own LDS traffic is ordered
+    constexpr int SEGS = TILE_COLS / 8;        // 16-byte segments per row
+    constexpr int ROWS_PER_PASS = 64 / SEGS;   // rows one load/store instruction covers
+    const int seg = lane % SEGS, sub = lane / SEGS;
+    uint16_t* out = reinterpret_cast<uint16_t*>(c_base) + batch * p.c_bs +
+                    static_cast<int64_t>(m0 + wm * TILE_ROWS) * p.c_rs + n0 + wn * TILE_COLS + seg * 8;
+#pragma unroll
+    for (int r0 = 0; r0 < TILE_ROWS; r0 += ROWS_PER_PASS) {
+      const int r = r0 + sub;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + seg * 16);
+      *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs) = v;
+    }
   } else if (simple && (INT ? (p.out_kind == OUT_I32 && p.row_scales == nullptr && p.correction == nullptr)
                             : p.out_kind == OUT_F32)) {
     static_for<WM>([&](auto ci) {
       constexpr int i = decltype(ci)::value;
+      const int row = m0 + (wm * WM + i) * 32 + frag_row;
       static_for<WN>([&](auto cj) {
         constexpr int j = decltype(cj)::value;
-        const int col = n0 + (wn * WN + j) * 32 + frag_row;
-        const int row0 = m0 + (wm * WM + i) * 32 + frag_half * 4;
-        auto* dst = reinterpret_cast<typename std::conditional<INT, int32_t, float>::type*>(c_base) +
-                    batch * p.c_bs + row0 * p.c_rs + col;
-        static_for<16>([&](auto cr) {
-          constexpr int r = decltype(cr)::value;
-          dst[((r >> 2) * 8 + (r & 3)) * p.c_rs] = acc[i][j][r];
+        const int col0 = n0 + (wn * WN + j) * 32 + frag_half * 4;
+        uint32_t* dst = reinterpret_cast<uint32_t*>(c_base) + batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col0;
+        static_for<4>([&](auto cq) {
+          constexpr int q = decltype(cq)::value;
+          // four consecutive accumulator registers as one 16-byte vector of their own type
+          const auto v = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
+          *reinterpret_cast<typename std::remove_const<decltype(v)>::type*>(dst + q * 8) = v;
         });
       });
     });
   } else if (simple && INT && p.row_scales != nullptr) {
-    static_for<WM>([&](auto ci) {
-      constexpr int i = decltype(ci)::value;
-      float rs[16];
-      const int row0 = m0 + (wm * WM + i) * 32 + frag_half * 4;
-      static_for<16>([&](auto cr) {
-        constexpr int r = decltype(cr)::value;
-        rs[r] = p.row_scales[row0 + (r >> 2) * 8 + (r & 3)];
+    float rs[WM];
+    static_for<WM>([&](auto ci) { rs[decltype(ci)::value] = p.row_scales[m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row]; });
+    static_for<WN>([&](auto cj) {
+      constexpr int j = decltype(cj)::value;
+      const int col0 = n0 + (wn * WN + j) * 32 + frag_half * 4;
+      f32x4 cs[4];
+      i32x4 corr[4];
+      static_for<4>([&](auto cq) {
+        constexpr int q = decltype(cq)::value;
+        cs[q] = *reinterpret_cast<const f32x4*>(p.column_scales + col0 + q * 8);
+        corr[q] = p.correction ? *reinterpret_cast<const i32x4*>(p.correction + col0 + q * 8) : i32x4{0, 0, 0, 0};
       });
-      static_for<WN>([&](auto cj) {
-        constexpr int j = decltype(cj)::value;
-        const int col = n0 + (wn * WN + j) * 32 + frag_row;
-        const float cs = p.column_scales[col];
-        const uint32_t corr = p.correction ? static_cast<uint32_t>(p.correction[col]) : 0u;
-        float* dst = reinterpret_cast<float*>(c_base) + batch * p.c_bs + row0 * p.c_rs + col;
-        static_for<16>([&](auto cr) {
-          constexpr int r = decltype(cr)::value;
+      static_for<WM>([&](auto ci) {
+        constexpr int i = decltype(ci)::value;
+        const int row = m0 + (wm * WM + i) * 32 + frag_row;
+        float* dst = reinterpret_cast<float*>(c_base) + batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col0;
+        static_for<4>([&](auto cq) {
+          constexpr int q = decltype(cq)::value;
           if constexpr (INT) {
-            const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(acc[i][j][r]) + corr);
-            const float t = static_cast<float>(v) * rs[r];
-            dst[((r >> 2) * 8 + (r & 3)) * p.c_rs] = t * cs;
+            const auto a4 = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
+            f32x4 out;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(a4[e]) + static_cast<uint32_t>(corr[q][e]));
+              const float t = static_cast<float>(v) * rs[i];  // row scale first, then column scale:
+              out[e] = t * cs[q][e];                          // two separately rounded multiplies
+            }
+            *reinterpret_cast<f32x4*>(dst + q * 8) = out;
           }
         });
       });
@@ -683,8 +727,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
       constexpr int i = decltype(ci)::value;
       static_for<WN>([&](auto cj) {
         constexpr int j = decltype(cj)::value;
-        store_tile_general<INT>(p, batch, split, m0 + (wm * WM + i) * 32 + frag_half * 4,
-                                n0 + (wn * WN + j) * 32 + frag_row, acc[i][j]);
+        store_tile_general<INT>(p, batch, split, m0 + (wm * WM + i) * 32 + frag_row,
+                                n0 + (wn * WN + j) * 32 + frag_half * 4, acc[i][j]);
       });
     });
   }

@@ -26,7 +26,7 @@ hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_
 // Shared by the per-class translation units.
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB>
 hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
-  constexpr int kLds = 2 * 32 * (WAVES_M * WM + WAVES_N * WN) * 128;
+  constexpr int kLds = kTileLdsBytes<WAVES_M, WAVES_N, WM, WN>();
   constexpr int kThreads = 64 * WAVES_M * WAVES_N;
   auto kernel = tile_gemm_kernel<SRC, WAVES_M, WAVES_N, WM, WN, LA, LB>;
   // > 64 KiB of dynamic LDS has to be enabled once per device; cheap enough to repeat per thread.
@@ -57,7 +57,11 @@ hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t strea
 
 template <int SRC>
 hipError_t launch_tile_class(const TileGemmParams& p, int tile, int mode, hipStream_t stream) {
-  if (tile == 256) return launch_tile_mode<SRC, 2, 4, 4, 2>(p, mode, stream);  // 8 wavefronts of 128x64
+  if (tile == 256) {
+    // 8 wavefronts of 128x64; the transposing B loader needs the registers of 4 wavefronts of 128x128
+    if (mode == MODE_NVEC_B) return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
+    return launch_tile_mode<SRC, 2, 4, 4, 2>(p, mode, stream);
+  }
   if (tile == 128) return launch_tile_mode<SRC, 2, 2, 2, 2>(p, mode, stream);  // 4 wavefronts of 64x64
   return launch_tile_mode<SRC, 2, 2, 1, 1>(p, mode, stream);                    // 4 wavefronts of 32x32
 }
