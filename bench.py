@@ -26,6 +26,14 @@ PEAK_BF16_TFLOPS = 2500.0
 PEAK_INT8_TOPS = 5000.0
 PEAK_HBM_GBPS = 8000.0
 
+# HBM-side bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes kept under
+# profiles/ (KiB per dispatch x 1024, FETCH scaled by 2.000 and WRITE by 1.000: what the
+# same counters read for a 1 GiB device copy, `--only copy`).  Counters cannot be read
+# from inside this process, so these are the recorded figures for exactly these workloads.
+TRAFFIC_BF16_4096 = int((101935 * 2.000 + 45568 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT = int((110595 * 2.000 + 124570 * 1.000) * 1024)
+TRAFFIC_GEMV_M1 = int((29702.9 * 2.000 + 56.0 * 1.000) * 1024)
+
 
 def _device_tensors_bf16_gemm(dev):
     import numpy as np
@@ -70,8 +78,9 @@ def bench_bf16_gemm(dev, steps, warmup):
     return {
         "wall_ms": wall_ms, "event_ms": ev_ms, "value": flops / (wall_ms * 1e-3) / 1e12,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
-                     "kernel": "tile_gemm_kernel<bf16,256x256>", "algorithmic_flops_per_launch": flops},
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BF16_4096,
+                     "kernel": "vecops_hip::tile_gemm_kernel<bf16, 256x256x64, B as [K,N]>",
+                     "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": 3 * 2 * n * n},
         "host": (a, b_kn),
     }
 
@@ -91,7 +100,10 @@ def bench_int8_dequant(dev, steps, warmup):
     return {"metric": "int8_quantized_matmul_tops", "workload": "int8 2048x4096x11008, per-token x per-channel "
             "dequant fused, fp32 out", "value": tops, "unit": "TOP/s", "ms_per_step": wall_ms, "dtype": "int8",
             "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                         "frac": tops / PEAK_INT8_TOPS, "traffic": None}}
+                         "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT,
+                         "kernel": "vecops_hip::tile_gemm_kernel<int8, 256x256x128, dequant epilogue>",
+                         "algorithmic_ops_per_launch": ops,
+                         "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
 
 
 def bench_gemv(dev, steps, warmup, m=1):
@@ -113,7 +125,21 @@ def bench_gemv(dev, steps, warmup, m=1):
             "bf16 activations, bf16 out, weights rotated through 8 buffers", "value": gbps, "unit": "GB/s",
             "us_per_step": wall_ms * 1e3, "dtype": "int8 x bf16 -> f32",
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                         "frac": gbps / PEAK_HBM_GBPS, "traffic": None, "algorithmic_bytes_per_launch": nbytes}}
+                         "frac": gbps / PEAK_HBM_GBPS, "traffic": TRAFFIC_GEMV_M1 if m == 1 else None,
+                         "kernel": "vecops_hip::skinny_w8a16_kernel", "algorithmic_bytes_per_launch": nbytes}}
+
+
+def bench_copy(dev, steps, warmup):
+    """A plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
+    counters of the other workloads are scaled by."""
+    import torch
+    nbytes = 1 << 30
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    wall_ms, ev_ms = _time_launches(lambda i: dst.copy_(src), steps, warmup)
+    return {"metric": "device_copy_gbps", "workload": "torch copy_ of 1 GiB (reads 1 GiB, writes 1 GiB)",
+            "bytes_read_per_launch": nbytes, "bytes_written_per_launch": nbytes,
+            "value": 2.0 * nbytes / (ev_ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall_ms}
 
 
 def cpu_baseline(a, b_kn):
@@ -125,26 +151,32 @@ def cpu_baseline(a, b_kn):
     n = 4096
     b_nk = np.ascontiguousarray(b_kn.T)
     ref = Reference.load()
+    budget_s = 12.0
     if ref is not None:
         c = np.zeros((n, n), np.uint16)
-        t0 = time.perf_counter()
-        ref.matmul_bf16_bf16(a, b_nk, c)
-        dt = time.perf_counter() - t0
+        reps, t0 = 0, time.perf_counter()
+        while reps == 0 or time.perf_counter() - t0 < budget_s:
+            ref.matmul_bf16_bf16(a, b_nk, c)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
         return {"value": 2.0 * n ** 3 / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "reference",
-                "sample": "full 4096^3 product, vecops ops::matmul<AMX_BF16F32>, one call on one thread "
-                          f"({dt * 1e3:.0f} ms, B pre-transposed to [N,K])"}
+                "sample": f"full 4096^3 product x {reps}, vecops ops::matmul<AMX_BF16F32> on one thread "
+                          f"({dt * 1e3:.0f} ms each, B pre-transposed to [N,K])"}
     oracle = Oracle()
-    rows = 64
+    rows = 256
     t0 = time.perf_counter()
     oracle.matmul_bf16_dense(a[:rows], b_nk, out_bf16=True)
     probe = time.perf_counter() - t0
-    rows = int(min(n, max(64, 64 * (12.0 / max(probe, 1e-3)))))
-    rows -= rows % 64
-    t0 = time.perf_counter()
-    oracle.matmul_bf16_dense(a[:rows], b_nk, out_bf16=True)
-    dt = time.perf_counter() - t0
+    rows = int(min(n, max(256, 256 * (budget_s / max(probe, 1e-3)))))
+    rows -= rows % 256
+    reps, t0 = 0, time.perf_counter()
+    while reps == 0 or time.perf_counter() - t0 < budget_s:
+        oracle.matmul_bf16_dense(a[:rows], b_nk, out_bf16=True)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
     return {"value": 2.0 * rows * n * n / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.threads(), "kind": "port",
-            "sample": f"first {rows} of 4096 rows of A against all of B ({dt:.1f} s), oracle C port, OpenMP"}
+            "sample": f"first {rows} of 4096 rows of A against all of B, {reps} times ({dt:.2f} s each), "
+                      "oracle C port, OpenMP"}
 
 
 def main() -> int:
@@ -153,7 +185,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["bf16", "int8", "gemv"], help="run a single workload (for profiling)")
+    ap.add_argument("--only", choices=["bf16", "int8", "gemv", "copy"], help="run a single workload (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the matmul path is built and measured on a single MI355X "
@@ -171,6 +203,9 @@ def main() -> int:
 
     if args.only == "int8":
         print(json.dumps(bench_int8_dequant(dev, args.steps, args.warmup)))
+        return 0
+    if args.only == "copy":
+        print(json.dumps(bench_copy(dev, args.steps, args.warmup)))
         return 0
     if args.only == "gemv":
         print(json.dumps(bench_gemv(dev, args.steps, args.warmup)))
