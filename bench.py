@@ -94,7 +94,9 @@ def bench_int8_dequant(dev, steps, warmup):
     rs = torch.from_numpy(synth.scales(3, m)).to(dev)
     cs = torch.from_numpy(synth.scales(4, n)).to(dev)
     c = torch.empty((m, n), dtype=torch.float32, device=dev)
-    wall_ms, ev_ms = _time_launches(lambda i: capi.matmul_i8_dequant(a, b, rs, cs, c), steps, warmup)
+    need = capi.lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k)   # the caller owns the scratch
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    wall_ms, ev_ms = _time_launches(lambda i: capi.matmul_i8_dequant(a, b, rs, cs, c, workspace=ws), steps, warmup)
     ops = 2.0 * m * n * k
     tops = ops / (ev_ms * 1e-3) / 1e12
     return {"metric": "int8_quantized_matmul_tops", "workload": "int8 2048x4096x11008, per-token x per-channel "

@@ -133,7 +133,7 @@ VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int
  * x bf16 [M,K] (row stride ldx), w int8 [N,K] (row stride ldw), scales fp32
  * [N, K/group] dense, y bf16 [M,N] (row stride ldy); fp32 accumulation.
  * No counterpart in vecops (it has no weight-only group-scaled matmul); this
- * is the decode-shaped GEMV / skinny GEMM of the north-star workload.  m <= 16,
+ * is the decode-shaped GEMV / skinny GEMM.  m <= 16,
  * k a multiple of `group`, group a multiple of 16.
  */
 VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t ldx, const int8_t* w, int64_t ldw,
