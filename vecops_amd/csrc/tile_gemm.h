@@ -6,11 +6,11 @@
 //   * one MFMA k-step consumes two chunks: lanes 0-31 take the even chunk,
 //     lanes 32-63 the odd one, each lane holding 16 contiguous bytes of its row
 //     (v_mfma_f32_32x32x16_bf16: 8 bf16; v_mfma_i32_32x32x32_i8: 16 int8);
-//   * a workgroup is 4 wavefronts in a 2x2 grid; each wavefront owns
+//   * a workgroup is WAVES_M x WAVES_N wavefronts; each wavefront owns
 //     WM x WN accumulator tiles of 32x32, so the workgroup tile is
-//     (64*WM) x (64*WN);
+//     (32*WAVES_M*WM) x (32*WAVES_N*WN);
 //   * LDS holds two stages of (BM + BN) rows x 128 bytes; chunk c of row r lives
-//     at r*128 + ((c ^ (r & 7)) * 16), which makes the 16-byte reads of eight
+//     at r*128 + (((c ^ r ^ r/8) & 7) * 16), which makes the 16-byte reads of eight
 //     consecutive rows hit eight different bank groups.
 //
 // fp32 operands in "bf16 compute" mode are rounded to bf16 (nearest even) while
@@ -116,16 +116,28 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
-// Fast path: one whole 16-byte chunk, no bounds checks (the caller guarantees
-// that the row exists and that the chunk lies inside K).
 #define VECOPS_GLOBAL __attribute__((address_space(1)))
 
+// Tells the compiler that a global pointer is the same in every lane, so that it is
+// kept in scalar registers and loads through it take the scalar-base form.
+__device__ __forceinline__ const VECOPS_GLOBAL char* uniform_ptr(const VECOPS_GLOBAL char* p) {
+  const uint64_t bits = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
+  return reinterpret_cast<const VECOPS_GLOBAL char*>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+// Fast path: one whole 16-byte chunk, no bounds checks (the caller guarantees
+// that the row exists and that the chunk lies inside K).
+
 template <int SRC>
-__device__ __forceinline__ u32x4 load_chunk_fast(const char* src) {
-  // global address space spelled out: a generic (flat) load would also count
-  // against the LDS counter and stall the LDS-only waits of the main loop
+__device__ __forceinline__ u32x4 load_chunk_fast(const VECOPS_GLOBAL char* base, uint32_t offset) {
+  // Global address space spelled out: a generic (flat) load would also count
+  // against the LDS counter and stall the LDS-only waits of the main loop.  `base`
+  // is wavefront-uniform, `offset` per lane: the load takes its base from scalar
+  // registers and the lane holds one 32-bit offset instead of a 64-bit pointer.
   if constexpr (SRC == SRC_F32_AS_BF16) {
-    const VECOPS_GLOBAL f32x4* p = (const VECOPS_GLOBAL f32x4*)(src);
+    const VECOPS_GLOBAL f32x4* p = (const VECOPS_GLOBAL f32x4*)(base + offset);
     const f32x4 lo = p[0], hi = p[1];
     u32x4 out;
     out.x = cvt_pk_bf16(lo.x, lo.y);
@@ -134,7 +146,7 @@ __device__ __forceinline__ u32x4 load_chunk_fast(const char* src) {
     out.w = cvt_pk_bf16(hi.z, hi.w);
     return out;
   } else {
-    return *(const VECOPS_GLOBAL u32x4*)(src);
+    return *(const VECOPS_GLOBAL u32x4*)(base + offset);
   }
 }
 
@@ -173,26 +185,6 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for<N - 1>(f);
     f(std::integral_constant<int, N - 1>{});
   }
-}
-
-// Scheduling hint for one k-step of the main loop: spread N_A instructions of
-// class MASK_A and N_B of class MASK_B evenly between the N_MFMA matrix
-// instructions, so that each memory instruction issues in the shadow of an MFMA
-// instead of in a clump that leaves the matrix pipe idle.
-// Classes (llvm.amdgcn.sched.group.barrier): 0x008 MFMA, 0x020 VMEM read,
-// 0x100 LDS read, 0x200 LDS write.
-template <int N_MFMA, int N_A, int MASK_A, int N_B, int MASK_B>
-__device__ __forceinline__ void interleave_hint() {
-  static_for<N_MFMA>([&](auto ci) {
-    constexpr int i = decltype(ci)::value;
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    // class A (fragment reads for the next k-step) is front-loaded, one per MFMA,
-    // so the data has landed when the next k-step starts; class B is spread evenly
-    constexpr int a = i < N_A ? 1 : 0;
-    constexpr int b = (i + 1) * N_B / N_MFMA - i * N_B / N_MFMA;
-    if constexpr (a > 0) __builtin_amdgcn_sched_group_barrier(MASK_A, a, 0);
-    if constexpr (b > 0) __builtin_amdgcn_sched_group_barrier(MASK_B, b, 0);
-  });
 }
 
 // Accumulator tile type per operand class.
@@ -302,23 +294,29 @@ __device__ __forceinline__ void map_workgroup(const TileGemmParams& p, int& batc
 }
 
 // Staging of one operand tile (ROWS rows x 128 bytes) from global memory into
-// LDS.  A stager owns the registers that hold a fetched tile between fetch() and
-// commit().  Rows past the operand's extent are clamped to its last row on the
-// fast paths: they are loaded but only feed accumulator rows/columns that are
-// never stored.
+// LDS.  A stager owns the registers that hold a fetched tile between fetch and
+// commit.  The registers form kParts groups that are stored and refilled
+// independently, so the main loop can spread a tile's LDS writes (the scarce
+// resource: a 16-byte LDS write costs about three times a 16-byte read) evenly
+// over its k-steps and refill each group right after it has been stored.  Rows
+// past the operand's extent are clamped to its last row on the fast paths: they
+// are loaded but only feed accumulator rows/columns that are never stored.
 //
-// LOAD_KVEC / LOAD_GENERIC: thread t stages chunk (t & 7) of rows (t >> 3) + (THREADS/8)*i.
+// LOAD_KVEC / LOAD_GENERIC: thread t stages chunk (t & 7) of rows (t >> 3) + (THREADS/8)*i;
+// part i is that one chunk.
 template <int SRC, int LOAD, int ROWS, int THREADS>
 struct Stager {
   using T = SrcTraits<SRC>;
   static constexpr int ROWS_PER_PASS = THREADS / 8;  // eight threads stage one 128-byte row
   static constexpr int CHUNKS = ROWS / ROWS_PER_PASS;
   static_assert(CHUNKS >= 1, "tile too small for this many threads");
-  static constexpr int kLdsStores = CHUNKS;  // per thread and K tile
-  static constexpr int kGlobalLoads = (LOAD == LOAD_KVEC) ? CHUNKS * (SRC == SRC_F32_AS_BF16 ? 2 : 1) : 0;
+  static constexpr int kParts = CHUNKS;
+  static constexpr int kStoreOps = 1;  // schedulable operations per part: one LDS write,
+  static constexpr int kLoadOps = 1;   // one refill (one or two load instructions)
   const char* base;
-  int64_t row_bytes[CHUNKS];  // byte offset of each staged row, chunk included (fast path)
-  int64_t rs, ks;             // element strides (checked path)
+  const VECOPS_GLOBAL char* tile_base;  // first row of the tile, k = 0 (wavefront-uniform)
+  uint32_t row_bytes[CHUNKS];  // byte offset of each staged row from tile_base, chunk included (fast path)
+  int64_t rs, ks;              // element strides (checked path)
   int first_row, extent, k_end, ld_row, ld_chunk;
   u32x4 regs[CHUNKS];
 
@@ -332,32 +330,59 @@ struct Stager {
     k_end = k_end_;
     ld_chunk = tid & 7;
     ld_row = tid >> 3;
+    tile_base = (const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * rs * T::kSrcBytes);
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
-      const int row = min(first_row + ld_row + i * ROWS_PER_PASS, extent - 1);
-      row_bytes[i] = (static_cast<int64_t>(row) * rs + ld_chunk * T::kElemsPerChunk) * T::kSrcBytes;
+      const int row = min(first_row + ld_row + i * ROWS_PER_PASS, extent - 1) - first_row;
+      // the launcher admits this path only when a tile's rows span less than 4 GiB
+      row_bytes[i] = static_cast<uint32_t>((static_cast<int64_t>(row) * rs + ld_chunk * T::kElemsPerChunk) * T::kSrcBytes);
     }
   }
 
-  // K tile kt lies wholly inside [0, K): unconditional 16-byte loads on the vector
-  // path (the generic path has no such shortcut and checks every element).
-  __device__ __forceinline__ void fetch_full(int kt) {
+  // Part PART of K tile kt, which lies wholly inside [0, K): an unconditional
+  // 16-byte load on the vector path (the generic path checks every element).
+  template <int PART>
+  __device__ __forceinline__ void fetch_part(int kt) {
     if constexpr (LOAD == LOAD_KVEC) {
-      const int64_t k_bytes = static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes);
-#pragma unroll
-      for (int i = 0; i < CHUNKS; ++i) regs[i] = load_chunk_fast<SRC>(base + row_bytes[i] + k_bytes);
+      const VECOPS_GLOBAL char* k_base =
+          uniform_ptr(tile_base + static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes));
+      regs[PART] = load_chunk_fast<SRC>(k_base, row_bytes[PART]);
     } else {
-      fetch(kt, 0);
+      const int k0 = kt * 8 * T::kElemsPerChunk + ld_chunk * T::kElemsPerChunk;
+      const int row = first_row + ld_row + PART * ROWS_PER_PASS;
+      regs[PART] = load_chunk_checked<SRC>(base, static_cast<int64_t>(row) * rs, ks, k0, k_end, row < extent);
     }
   }
 
-  __device__ __forceinline__ void fetch(int kt, int full_k_tiles) {
+  // Whole tile kt, which lies wholly inside [0, K).
+  __device__ __forceinline__ void fetch_full(int kt) {
+    static_for<CHUNKS>([&](auto ci) { fetch_part<decltype(ci)::value>(kt); });
+  }
+
+  // A second register set for the start of the pipeline: the tile after the first
+  // one is requested while the first is still in flight, and moved into the
+  // staging registers once the first has been stored.
+  struct Spare {
+    u32x4 regs[CHUNKS];
+  };
+  __device__ __forceinline__ void fetch_full_spare(Spare& spare, int kt) {
     if constexpr (LOAD == LOAD_KVEC) {
-      if (kt < full_k_tiles) {
-        fetch_full(kt);
-        return;
-      }
+      const VECOPS_GLOBAL char* k_base =
+          uniform_ptr(tile_base + static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes));
+#pragma unroll
+      for (int i = 0; i < CHUNKS; ++i) spare.regs[i] = load_chunk_fast<SRC>(k_base, row_bytes[i]);
     }
+  }
+  __device__ __forceinline__ void take_spare(const Spare& spare) {
+    if constexpr (LOAD == LOAD_KVEC) {
+#pragma unroll
+      for (int i = 0; i < CHUNKS; ++i) regs[i] = spare.regs[i];
+    }
+  }
+  static constexpr bool kHasSpare = LOAD == LOAD_KVEC;
+
+  // Whole tile, every element bounds-checked: the partial last K tile.
+  __device__ __forceinline__ void fetch_checked(int kt) {
     const int k0 = kt * 8 * T::kElemsPerChunk + ld_chunk * T::kElemsPerChunk;
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
@@ -366,32 +391,51 @@ struct Stager {
     }
   }
 
+  template <int PART>
+  __device__ __forceinline__ void commit_part(char* lds_tile) const {
+    *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(ld_row + PART * ROWS_PER_PASS, ld_chunk)) = regs[PART];
+  }
+
+  // the main loop's view: part PART as numbered store / load operations
+  template <int PART, int OP>
+  __device__ __forceinline__ void store_op(char* lds_tile) const {
+    commit_part<PART>(lds_tile);
+  }
+  template <int PART, int OP>
+  __device__ __forceinline__ void load_op(int kt) {
+    fetch_part<PART>(kt);
+  }
+
   __device__ __forceinline__ void commit(char* lds_tile) const {
-#pragma unroll
-    for (int i = 0; i < CHUNKS; ++i)
-      *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(ld_row + i * ROWS_PER_PASS, ld_chunk)) = regs[i];
+    static_for<CHUNKS>([&](auto ci) { commit_part<decltype(ci)::value>(lds_tile); });
   }
 };
 
 // LOAD_NVEC: the operand is stored with its spatial index contiguous (B handed
-// over as [K,N] row-major).  Thread t < ROWS owns one 8(k) x 8(n) block of the
-// tile: it loads eight 16-byte rows along n, transposes the block in registers
-// with byte permutes and writes eight K-contiguous chunks.  16-bit compute
-// elements only (bf16, or fp32 rounded to bf16 on load).
+// over as [K,N] row-major).  The tile is cut into units of 8(k) x 4(n)
+// elements; a thread owns UNITS of them (its parts).  For a unit it loads eight
+// 8-byte rows along n, transposes them in registers with byte permutes and
+// writes four K-contiguous 16-byte chunks.  Consecutive threads take consecutive
+// n, so a wavefront's load covers 512 contiguous bytes of one k row.  16-bit
+// compute elements only (bf16, or fp32 rounded to bf16 on load).
 template <int SRC, int ROWS, int THREADS>
 struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
-  static_assert(ROWS <= THREADS, "one 8x8 block per thread at most");
   using T = SrcTraits<SRC>;
   static_assert(T::kElemsPerChunk == 8, "transposing stager handles 16-bit compute elements");
-  static constexpr int NBLOCKS = ROWS / 8;
-  static constexpr int kLdsStores = 8;
-  static constexpr int kGlobalLoads = 8 * (SRC == SRC_F32_AS_BF16 ? 2 : 1);
+  static constexpr int UNITS_TOTAL = 2 * ROWS;  // (ROWS / 4) along n  x  8 along k
+  static constexpr int UNITS = UNITS_TOTAL >= THREADS ? UNITS_TOTAL / THREADS : 1;
+  static constexpr bool kAllActive = UNITS_TOTAL >= THREADS;
+  static constexpr int kParts = UNITS;
+  static constexpr int kStoreOps = 4;  // schedulable operations per part: four LDS writes
+  static constexpr int kLoadOps = 8;   // (each with its permutes), eight row loads
   const char* base;
-  const char* block_ptr;  // address of (k-block row 0, n-block) for K tile 0
-  int64_t rs, ks;         // rs == 1; ks = elements between consecutive k
-  int first_row, extent, k_end, nb, kb, tid_;
+  const VECOPS_GLOBAL char* tile_base;  // (k = 0, first n of the tile), wavefront-uniform
+  uint32_t unit_bytes[UNITS];  // byte offset of (first k of the unit, its first n) from tile_base
+  int64_t rs, ks;              // rs == 1; ks = elements between consecutive k
+  int first_row, extent, k_end;
+  int n_local[UNITS], kb[UNITS];
   bool active;
-  u32x4 regs[8];
+  uint32_t regs[UNITS][8][2];
 
   __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
                                        int k_end_, int tid) {
@@ -401,61 +445,174 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
     first_row = first_row_;
     extent = extent_;
     k_end = k_end_;
-    tid_ = tid;
-    active = tid < ROWS;
-    nb = tid % NBLOCKS;
-    kb = (tid / NBLOCKS) & 7;
-    const int n = min(first_row + nb * 8, extent - 8);  // extent is a multiple of 8 on this path
-    block_ptr = base + (static_cast<int64_t>(kb) * 8 * ks + n) * T::kSrcBytes;
+    active = kAllActive || tid < UNITS_TOTAL;
+    tile_base = (const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * T::kSrcBytes);
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+      const int unit = u * THREADS + tid;
+      n_local[u] = (unit % (ROWS / 4)) * 4;
+      kb[u] = (unit / (ROWS / 4)) & 7;
+      // extent is a multiple of 8 on this path: clamp whole 8-column blocks, keep the offset inside the block
+      const int n = min(first_row + n_local[u], extent - 8 + (n_local[u] & 4)) - first_row;
+      // the launcher admits this path only when a K tile's 64 rows span less than 4 GiB
+      unit_bytes[u] = static_cast<uint32_t>((static_cast<int64_t>(kb[u]) * 8 * ks + n) * T::kSrcBytes);
+    }
+  }
+
+  // row R (k = 8*kb + R) of unit PART
+  template <int PART, int R>
+  __device__ __forceinline__ void load_op(int kt) {
+    if (!kAllActive && !active) return;
+    const VECOPS_GLOBAL char* row = tile_base + (static_cast<int64_t>(kt) * 64 + R) * ks * T::kSrcBytes;
+    const VECOPS_GLOBAL char* src = uniform_ptr(row) + unit_bytes[PART];
+    if constexpr (SRC == SRC_F32_AS_BF16) {
+      const f32x4 v = *(const VECOPS_GLOBAL f32x4*)(src);
+      regs[PART][R][0] = cvt_pk_bf16(v.x, v.y);
+      regs[PART][R][1] = cvt_pk_bf16(v.z, v.w);
+    } else {
+      const u32x2 v = *(const VECOPS_GLOBAL u32x2*)(src);
+      regs[PART][R][0] = v.x;
+      regs[PART][R][1] = v.y;
+    }
+  }
+
+  template <int PART>
+  __device__ __forceinline__ void fetch_part(int kt) {
+    static_for<8>([&](auto cr) { load_op<PART, decltype(cr)::value>(kt); });
   }
 
   __device__ __forceinline__ void fetch_full(int kt) {
-    if (!active) return;
-    const char* p = block_ptr + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes;
-#pragma unroll
-    for (int r = 0; r < 8; ++r) regs[r] = load_chunk_fast<SRC>(p + r * ks * T::kSrcBytes);
+    static_for<UNITS>([&](auto cu) { fetch_part<decltype(cu)::value>(kt); });
   }
 
-  __device__ __forceinline__ void fetch(int kt, int full_k_tiles) {
-    if (!active) return;
-    if (kt < full_k_tiles) {
-      fetch_full(kt);
-      return;
-    }
-    // K tail: rows k >= K read as zero, columns n >= N as zero
+  // second register set for the start of the pipeline (see the chunk stager)
+  struct Spare {
+    uint32_t regs[UNITS][8][2];
+  };
+  __device__ __forceinline__ void fetch_full_spare(Spare& spare, int kt) {
+    Stager tmp = *this;  // addresses only: its registers are overwritten before any use
+    tmp.fetch_full(kt);
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const int k = kt * 64 + kb * 8 + r;
-      uint32_t w[4] = {0u, 0u, 0u, 0u};
-      if (k < k_end) {
+    for (int u = 0; u < UNITS; ++u)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int n = first_row + nb * 8 + e;
-          if (n < extent) {
-            uint32_t v;
-            if constexpr (SRC == SRC_BF16) v = reinterpret_cast<const uint16_t*>(base)[k * ks + n];
-            else v = cvt_pk_bf16(reinterpret_cast<const float*>(base)[k * ks + n], 0.0f) & 0xffffu;
-            w[e >> 1] |= v << ((e & 1) * 16);
+      for (int r = 0; r < 8; ++r) {
+        spare.regs[u][r][0] = tmp.regs[u][r][0];
+        spare.regs[u][r][1] = tmp.regs[u][r][1];
+      }
+  }
+  __device__ __forceinline__ void take_spare(const Spare& spare) {
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        regs[u][r][0] = spare.regs[u][r][0];
+        regs[u][r][1] = spare.regs[u][r][1];
+      }
+  }
+  static constexpr bool kHasSpare = true;
+
+  // Whole tile with bounds checks (the partial last K tile): rows k >= K read as
+  // zero, columns n >= N as zero.
+  __device__ __forceinline__ void fetch_checked(int kt) {
+    if (!kAllActive && !active) return;
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const int k = kt * 64 + kb[u] * 8 + r;
+        regs[u][r][0] = 0u;
+        regs[u][r][1] = 0u;
+        if (k < k_end) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int n = first_row + n_local[u] + e;
+            if (n < extent) {
+              uint32_t v;
+              if constexpr (SRC == SRC_BF16) v = reinterpret_cast<const uint16_t*>(base)[k * ks + n];
+              else v = cvt_pk_bf16(reinterpret_cast<const float*>(base)[k * ks + n], 0.0f) & 0xffffu;
+              regs[u][r][e >> 1] |= v << ((e & 1) * 16);
+            }
           }
         }
       }
-      regs[r] = u32x4{w[0], w[1], w[2], w[3]};
     }
   }
 
+  // output chunk for n-row E of unit PART: dword j = (regs[2j][E], regs[2j+1][E])
+  template <int PART, int E>
+  __device__ __forceinline__ void store_op(char* lds_tile) const {
+    if (!kAllActive && !active) return;
+    constexpr uint32_t sel = (E & 1) ? 0x07060302u : 0x05040100u;
+    u32x4 out;
+    out.x = __builtin_amdgcn_perm(regs[PART][1][E >> 1], regs[PART][0][E >> 1], sel);
+    out.y = __builtin_amdgcn_perm(regs[PART][3][E >> 1], regs[PART][2][E >> 1], sel);
+    out.z = __builtin_amdgcn_perm(regs[PART][5][E >> 1], regs[PART][4][E >> 1], sel);
+    out.w = __builtin_amdgcn_perm(regs[PART][7][E >> 1], regs[PART][6][E >> 1], sel);
+    *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(n_local[PART] + E, kb[PART])) = out;
+  }
+
+  template <int PART>
+  __device__ __forceinline__ void commit_part(char* lds_tile) const {
+    static_for<4>([&](auto ce) { store_op<PART, decltype(ce)::value>(lds_tile); });
+  }
+
   __device__ __forceinline__ void commit(char* lds_tile) const {
-    if (!active) return;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      // output chunk for n-row e: dword j = (regs[2j][e], regs[2j+1][e])
-      const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
-      u32x4 out;
-      out.x = __builtin_amdgcn_perm(regs[1][e >> 1], regs[0][e >> 1], sel);
-      out.y = __builtin_amdgcn_perm(regs[3][e >> 1], regs[2][e >> 1], sel);
-      out.z = __builtin_amdgcn_perm(regs[5][e >> 1], regs[4][e >> 1], sel);
-      out.w = __builtin_amdgcn_perm(regs[7][e >> 1], regs[6][e >> 1], sel);
-      *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(nb * 8 + e, kb)) = out;
+    static_for<UNITS>([&](auto cu) { commit_part<decltype(cu)::value>(lds_tile); });
+  }
+};
+
+// One schedulable staging operation: store operation `op` or load operation `op`
+// of part `part` of operand A (0) or B (1); operand -1 = none.
+struct StagingOp {
+  int operand, part, is_load, op;
+};
+
+// Which of the four k-steps of a K tile stores (and then refills) which staging
+// parts, and in what order.  Chunk parts (one LDS write, one refill) are dealt out
+// evenly, A's first; a transposing B stager has one or two heavy parts (four
+// writes, eight loads), which take k-steps 0 and 2 while A's chunks share the
+// others.
+template <typename SA, typename SB, bool B_TRANSPOSING>
+struct StagingSchedule {
+  static constexpr int PARTS_A = SA::kParts, PARTS_B = SB::kParts;
+  static constexpr int step_a(int part) {
+    if constexpr (!B_TRANSPOSING) return part * 4 / (PARTS_A + PARTS_B);
+    else if constexpr (PARTS_B == 2) return part * 2 < PARTS_A ? 1 : 3;
+    else return 1 + part * 3 / PARTS_A;
+  }
+  static constexpr int step_b(int part) {
+    if constexpr (!B_TRANSPOSING) return (PARTS_A + part) * 4 / (PARTS_A + PARTS_B);
+    else return part * 2;
+  }
+  // number of operations of k-step `step`
+  static constexpr int ops(int step) {
+    int n = 0;
+    for (int q = 0; q < PARTS_A; ++q) n += step_a(q) == step ? SA::kStoreOps + SA::kLoadOps : 0;
+    for (int q = 0; q < PARTS_B; ++q) n += step_b(q) == step ? SB::kStoreOps + SB::kLoadOps : 0;
+    return n;
+  }
+  // Operation number g of k-step `step`.  Part by part (a part's stores, then its
+  // loads), or, with stores_first, every store of the step before any load: the
+  // order for the k-step whose stores are followed by the barrier.
+  static constexpr StagingOp op(int step, int g, bool stores_first) {
+    int n = 0;
+    for (int pass = 0; pass < (stores_first ? 2 : 1); ++pass) {
+      for (int operand = 0; operand < 2; ++operand) {
+        const int parts = operand == 0 ? PARTS_A : PARTS_B;
+        const int n_st = operand == 0 ? SA::kStoreOps : SB::kStoreOps;
+        const int n_ld = operand == 0 ? SA::kLoadOps : SB::kLoadOps;
+        for (int q = 0; q < parts; ++q) {
+          if ((operand == 0 ? step_a(q) : step_b(q)) != step) continue;
+          if (!stores_first || pass == 0)
+            for (int e = 0; e < n_st; ++e)
+              if (n++ == g) return StagingOp{operand, q, 0, e};
+          if (!stores_first || pass == 1)
+            for (int r = 0; r < n_ld; ++r)
+              if (n++ == g) return StagingOp{operand, q, 1, r};
+        }
+      }
     }
+    return StagingOp{-1, 0, 0, 0};
   }
 };
 
@@ -469,8 +626,9 @@ constexpr int kTileLdsBytes() {
 }
 
 // Workgroup shapes: WAVES_M x WAVES_N wavefronts, each owning WM x WN accumulator
-// tiles of 32x32.  The 256x256 tile runs 8 wavefronts (two per SIMD, so one
-// wavefront's waits are covered by the other's MFMAs); the small tiles run 4.
+// tiles of 32x32.  Every shape in use runs 4 wavefronts, one per SIMD: the 256x256
+// tile with 128x128 per wavefront (256 accumulator registers in the AGPR half of
+// the unified file), the small tiles with 64x64 or 32x32.
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const TileGemmParams p) {
   using T = SrcTraits<SRC>;
@@ -509,14 +667,6 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, tid);
   stager_b.init(static_cast<const char*>(p.b) + batch * p.b_bs * T::kSrcBytes, p.b_rs, p.b_ks, n0, p.n, p.k, tid);
 
-  Acc acc[WM][WN];
-#pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
   const int frag_row = lane & 31;
   const int frag_half = lane >> 5;
   // LDS offsets of this lane's fragments at k-step 0; k-step ks flips bits 5-6: off ^ (ks << 5)
@@ -534,27 +684,32 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   const int has_tail = __builtin_amdgcn_readfirstlane((nk > 0 && kt_end > full_k_tiles) ? 1 : 0);
   auto seq = [&](int j) { return (has_tail && j == 0) ? kt_end - 1 : kt_begin + j - has_tail; };
 
-  // Software pipeline over K tiles, two LDS stages, two fragment register sets:
-  //   k-step 0 : read fragments(ks=1)                                  | MFMA on fragments(ks=0)
-  //   k-step 1 : read fragments(ks=2), store tile it+1 into other stage | MFMA
-  //   k-step 2 : read fragments(ks=3), issue global loads of tile it+2   | MFMA
-  //   barrier  : every wave's reads of this stage and stores into the other are done
-  //   k-step 3 : read fragments(ks=0) of tile it+1 from the other stage  | MFMA
-  // Global loads get a whole tile of MFMA work to land; LDS reads one k-step.
+  // Software pipeline over K tiles, two LDS stages, two fragment register sets.
+  // K tile `it` is multiplied in four k-steps; k-step s
+  //   * reads the fragments of k-step s+1 (for s = 3: of k-step 0 of tile it+1, from
+  //     the other stage, after the barrier),
+  //   * stores its share of the staging registers (tile it+1) into the other stage
+  //     and refills them with global loads of tile it+2,
+  //   * issues the MFMAs of k-step s.
+  // A k-step is written out as slots: one MFMA followed by the memory operations
+  // dealt to that slot, each slot fenced against reordering, so that every memory
+  // instruction issues in the shadow of an MFMA and the LDS pipe sees an even
+  // stream instead of bursts (all wavefronts of a workgroup run in step).  The
+  // barrier sits in the middle of k-step 3: its stores and a first half of its
+  // MFMAs before, the fragment reads and the other half after.  A global load has a
+  // whole K tile of MFMA work to land before its registers are stored; an LDS read
+  // has most of a k-step.
   u32x4 fa[2][WM], fb[2][WN];
-  // read in the order the MFMAs consume: A fragment 0, every B fragment, the other A fragments
-  auto read_frags = [&](int set, const char* tile, int ks) {
-    fa[set][0] = *reinterpret_cast<const u32x4*>(tile + (off_a[0] ^ (ks << 5)));
-#pragma unroll
-    for (int j = 0; j < WN; ++j) fb[set][j] = *reinterpret_cast<const u32x4*>(tile + (off_b[j] ^ (ks << 5)));
-#pragma unroll
-    for (int i = 1; i < WM; ++i) fa[set][i] = *reinterpret_cast<const u32x4*>(tile + (off_a[i] ^ (ks << 5)));
+  constexpr int N_MFMA = WM * WN, N_READ = WM + WN;
+  // fragment reads in the order the MFMAs consume them: A fragment 0, every B fragment, the other A fragments
+  auto read_frag = [&](int set, const char* tile, int ks, auto r_tag) {
+    constexpr int r = decltype(r_tag)::value;
+    if constexpr (r == 0) fa[set][0] = *reinterpret_cast<const u32x4*>(tile + (off_a[0] ^ (ks << 5)));
+    else if constexpr (r <= WN) fb[set][r - 1] = *reinterpret_cast<const u32x4*>(tile + (off_b[r - 1] ^ (ks << 5)));
+    else fa[set][r - WN] = *reinterpret_cast<const u32x4*>(tile + (off_a[r - WN] ^ (ks << 5)));
   };
-  auto mfma_all = [&](int set) {
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-      for (int j = 0; j < WN; ++j) mfma_step<SRC>(acc[i][j], fb[set][j], fa[set][i]);  // B rows first: see the epilogue
+  auto read_frags = [&](int set, const char* tile, int ks) {
+    static_for<N_READ>([&](auto cr) { read_frag(set, tile, ks, cr); });
   };
   // workgroup barrier that waits only for this wave's LDS traffic, not for the
   // global prefetch in flight
@@ -563,17 +718,51 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
     __builtin_amdgcn_s_barrier();
   };
 
+  using SA = decltype(stager_a);
+  using SB = decltype(stager_b);
+  using Sched = StagingSchedule<SA, SB, LOAD_B == LOAD_NVEC>;
+
+  // Start of the pipeline: tile 0 into the staging registers and, without waiting
+  // for it, tile 1 into a spare set (position 1 is never the partial tile: one
+  // straight path also keeps the count of loads in flight, which the waits of the
+  // loop are derived from, exact); tile 0 to LDS; tile 1 into the staging registers.
   if (nk > 0) {
-    stager_a.fetch(seq(0), full_k_tiles);
-    stager_b.fetch(seq(0), full_k_tiles);
+    // one branch for both operands: a wait in front of the out-of-line checked
+    // loader must not separate A's loads from B's
+    if (seq(0) < full_k_tiles) {
+      stager_a.fetch_full(seq(0));
+      stager_b.fetch_full(seq(0));
+    } else {
+      stager_a.fetch_checked(seq(0));
+      stager_b.fetch_checked(seq(0));
+    }
+    typename SA::Spare spare_a;
+    typename SB::Spare spare_b;
+    if (nk > 1) {
+      if constexpr (SA::kHasSpare) stager_a.fetch_full_spare(spare_a, seq(1));
+      if constexpr (SB::kHasSpare) stager_b.fetch_full_spare(spare_b, seq(1));
+    }
     stager_a.commit(lds);
     stager_b.commit(lds + BM * 128);
-    const int full_in_range = nk - has_tail;  // whole K tiles this workgroup owns
     if (nk > 1) {
-      stager_a.fetch_full(seq(1));
-      stager_b.fetch_full(seq(1));
+      if constexpr (SA::kHasSpare) stager_a.take_spare(spare_a);
+      else stager_a.fetch_full(seq(1));
+      if constexpr (SB::kHasSpare) stager_b.take_spare(spare_b);
+      else stager_b.fetch_full(seq(1));
     }
-    __syncthreads();
+  }
+
+  Acc acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  if (nk > 0) {
+    const int full_in_range = nk - has_tail;  // whole K tiles this workgroup owns
+    lds_barrier();  // tile 0 is in LDS
     read_frags(0, lds, 0);
 
     // The loop body is one straight-line block: stores into the other stage,
@@ -585,38 +774,56 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
       for (int it = 0; it < nk; ++it) {
         const char* tile = lds + (it & 1) * STAGE_BYTES;
         char* other = lds + ((it & 1) ^ 1) * STAGE_BYTES;
+        // K tile to prefetch: seq(min(it + 2, nk - 1)), never the tail tile (position 0)
+        const int t2 = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(it + 2, nk - 1)));
 
-        constexpr int N_MFMA = WM * WN, N_READ = WM + WN;
-        constexpr int N_STORE = decltype(stager_a)::kLdsStores + decltype(stager_b)::kLdsStores;
-        constexpr int N_LOAD = decltype(stager_a)::kGlobalLoads + decltype(stager_b)::kGlobalLoads;
+        auto stage_op = [&](auto step_tag, auto g_tag, auto order_tag) {
+          constexpr StagingOp o = Sched::op(decltype(step_tag)::value, decltype(g_tag)::value, decltype(order_tag)::value);
+          if constexpr (o.operand == 0 && o.is_load == 0) stager_a.template store_op<o.part, o.op>(other);
+          if constexpr (o.operand == 0 && o.is_load == 1 && PREFETCH) stager_a.template load_op<o.part, o.op>(t2);
+          if constexpr (o.operand == 1 && o.is_load == 0) stager_b.template store_op<o.part, o.op>(other + BM * 128);
+          if constexpr (o.operand == 1 && o.is_load == 1 && PREFETCH) stager_b.template load_op<o.part, o.op>(t2);
+        };
+        // Slots [S0, S1) of k-step STEP: MFMA x on fragment set mfma_set, then this
+        // slot's share of the N_RD fragment reads (k-step read_ks of read_tile into
+        // the other set; dealt front-biased) and of the step's staging operations
+        // (if STAGE).
+        auto slots = [&](auto step_tag, auto s0_tag, auto s1_tag, auto nrd_tag, auto stage_tag, auto order_tag,
+                         int mfma_set, const char* read_tile, int read_ks) {
+          constexpr int STEP = decltype(step_tag)::value, S0 = decltype(s0_tag)::value, S1 = decltype(s1_tag)::value;
+          constexpr int NS = S1 - S0, N_RD = decltype(nrd_tag)::value;
+          constexpr int G = decltype(stage_tag)::value ? Sched::ops(STEP) : 0;
+          if constexpr (NS == 0) {
+            static_for<G>([&](auto cg) { stage_op(step_tag, cg, order_tag); });
+          }
+          static_for<NS>([&](auto ci) {
+            constexpr int i = decltype(ci)::value, x = S0 + i;
+            mfma_step<SRC>(acc[x / WN][x % WN], fb[mfma_set][x % WN], fa[mfma_set][x / WN]);  // B rows first: see the epilogue
+            constexpr int r0 = (i * N_RD + NS - 1) / NS, r1 = ((i + 1) * N_RD + NS - 1) / NS;
+            static_for<r1 - r0>([&](auto cr) {
+              read_frag(mfma_set ^ 1, read_tile, read_ks, std::integral_constant<int, r0 + decltype(cr)::value>{});
+            });
+            constexpr int g0 = i * G / NS, g1 = (i + 1) * G / NS;
+            static_for<g1 - g0>([&](auto cg) {
+              stage_op(step_tag, std::integral_constant<int, g0 + decltype(cg)::value>{}, order_tag);
+            });
+            __builtin_amdgcn_sched_barrier(0);
+          });
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I3 = std::integral_constant<int, 3>;
+        using All = std::integral_constant<int, N_MFMA>;
+        using Half = std::integral_constant<int, N_MFMA / 2>;
+        using Reads = std::integral_constant<int, N_READ>;
 
-        read_frags(1, tile, 1);
-        mfma_all(0);
-        interleave_hint<N_MFMA, N_READ, 0x100, 0, 0>();
-        __builtin_amdgcn_sched_barrier(0);
-
-        read_frags(0, tile, 2);
-        stager_a.commit(other);
-        stager_b.commit(other + BM * 128);
-        mfma_all(1);
-        interleave_hint<N_MFMA, N_READ, 0x100, N_STORE, 0x200>();
-        __builtin_amdgcn_sched_barrier(0);
-
-        read_frags(1, tile, 3);
-        if constexpr (PREFETCH) {
-          const int t2 = seq(max(has_tail, min(it + 2, nk - 1)));
-          stager_a.fetch_full(t2);
-          stager_b.fetch_full(t2);
-        }
-        mfma_all(0);
-        interleave_hint<N_MFMA, N_READ, 0x100, PREFETCH ? N_LOAD : 0, 0x020>();
-        __builtin_amdgcn_sched_barrier(0);
-
+        slots(I0{}, I0{}, All{}, Reads{}, std::true_type{}, std::false_type{}, 0, tile, 1);
+        slots(I1{}, I0{}, All{}, Reads{}, std::true_type{}, std::false_type{}, 1, tile, 2);
+        slots(I2{}, I0{}, All{}, Reads{}, std::true_type{}, std::false_type{}, 0, tile, 3);
+        slots(I3{}, I0{}, Half{}, I0{}, std::true_type{}, std::true_type{}, 1, tile, 0);
         lds_barrier();
-        read_frags(0, other, 0);
-        mfma_all(1);
-        interleave_hint<N_MFMA, N_READ, 0x100, 0, 0>();
-        __builtin_amdgcn_sched_barrier(0);
+        slots(I3{}, Half{}, All{}, Reads{}, std::false_type{}, std::false_type{}, 1, other, 0);
       }
     };
     if (full_in_range > 0) main_loop(std::true_type{});

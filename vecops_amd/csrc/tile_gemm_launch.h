@@ -58,9 +58,9 @@ hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t strea
 template <int SRC>
 hipError_t launch_tile_class(const TileGemmParams& p, int tile, int mode, hipStream_t stream) {
   if (tile == 256) {
-    // 8 wavefronts of 128x64; the transposing B loader needs the registers of 4 wavefronts of 128x128
-    if (mode == MODE_NVEC_B) return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
-    return launch_tile_mode<SRC, 2, 4, 4, 2>(p, mode, stream);
+    // 4 wavefronts of 128x128, one per SIMD: a third less LDS read traffic than 8 wavefronts of 128x64,
+    // which matters because the LDS pipe, not the MFMA pipe, is what the 8-wavefront shape saturates
+    return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
   }
   if (tile == 128) return launch_tile_mode<SRC, 2, 2, 2, 2>(p, mode, stream);  // 4 wavefronts of 64x64
   return launch_tile_mode<SRC, 2, 2, 1, 1>(p, mode, stream);                    // 4 wavefronts of 32x32
