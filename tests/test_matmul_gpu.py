@@ -327,6 +327,32 @@ def test_config2_bf16_4096_sampled_and_linear(device, oracle):
     assert torch.equal(c32b, c32 * 2)
 
 
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+def test_wide_ragged_bf16_sampled(device, oracle, layout):
+    """Many 256-wide tiles with ragged N and a K tail: sampled outputs against the
+    oracle, bf16 output against RNE of the fp32 output."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = 2048, 11000, 264
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    ta = dev_bf16(a, device)
+    tb = dev_bf16(b, device) if layout == "nt" else dev_bf16(np.ascontiguousarray(b.T), device).t()
+    c32 = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    c16 = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    capi.matmul(ta, tb, c32)
+    capi.matmul(ta, tb, c16)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(11)
+    rows, cols = rng.integers(0, m, 8192), rng.integers(0, n, 8192)
+    rows[:6] = [0, 0, m - 1, m - 1, 255, 256]
+    cols[:6] = [0, n - 1, 0, n - 1, 255, 256]
+    got32 = c32.cpu().numpy()
+    assert not np.isnan(got32).any()
+    assert rel_err(got32[rows, cols], oracle.matmul_sampled(a, b, rows, cols)) <= fp32_tol(k)
+    assert np.array_equal(host_bits(c16), oracle.bf16_from_f32(got32))
+
+
 def test_config4_int8_full_size_checksum(device, oracle):
     """int8 2048x4096x11008: every int32 accumulator is checked by a checksum of
     checksums that is exact mod 2^32 (C v == A (B^T v) for a random integer v), the

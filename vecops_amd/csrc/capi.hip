@@ -154,7 +154,10 @@ constexpr int kComputeUnits = 256;
 // The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure
 // integer function of (operand class, m, n, k); it picks the workgroup tile by
 // how many tiles the problem yields against the 256 compute units and splits K
-// when even the smallest tile leaves most of them idle.
+// when even the smallest tile leaves most of them idle.  A part-filled last round
+// of big tiles is not worth avoiding: the chip runs against its power limit on real
+// data, a lightly loaded round clocks higher, and narrower tiles (256x192 was
+// measured) cost more LDS and L2 traffic per flop than the better balance saves.
 void choose(const Problem& pr, VecopsHipPlan* plan) {
   memset(plan, 0, sizeof(*plan));
   plan->split_k = 1;

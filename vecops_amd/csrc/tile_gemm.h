@@ -423,8 +423,8 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
   using T = SrcTraits<SRC>;
   static_assert(T::kElemsPerChunk == 8, "transposing stager handles 16-bit compute elements");
   static constexpr int UNITS_TOTAL = 2 * ROWS;  // (ROWS / 4) along n  x  8 along k
-  static constexpr int UNITS = UNITS_TOTAL >= THREADS ? UNITS_TOTAL / THREADS : 1;
-  static constexpr bool kAllActive = UNITS_TOTAL >= THREADS;
+  static constexpr int UNITS = (UNITS_TOTAL + THREADS - 1) / THREADS;
+  static constexpr bool kAllActive = UNITS_TOTAL % THREADS == 0;  // else the last unit of some threads is idle
   static constexpr int kParts = UNITS;
   static constexpr int kStoreOps = 4;  // schedulable operations per part: four LDS writes
   static constexpr int kLoadOps = 8;   // (each with its permutes), eight row loads
@@ -434,8 +434,10 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
   int64_t rs, ks;              // rs == 1; ks = elements between consecutive k
   int first_row, extent, k_end;
   int n_local[UNITS], kb[UNITS];
-  bool active;
+  int tid_;
   uint32_t regs[UNITS][8][2];
+
+  __device__ __forceinline__ bool active(int u) const { return kAllActive || u * THREADS + tid_ < UNITS_TOTAL; }
 
   __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
                                        int k_end_, int tid) {
@@ -445,7 +447,7 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
     first_row = first_row_;
     extent = extent_;
     k_end = k_end_;
-    active = kAllActive || tid < UNITS_TOTAL;
+    tid_ = tid;
     tile_base = (const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * T::kSrcBytes);
 #pragma unroll
     for (int u = 0; u < UNITS; ++u) {
@@ -462,7 +464,7 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
   // row R (k = 8*kb + R) of unit PART
   template <int PART, int R>
   __device__ __forceinline__ void load_op(int kt) {
-    if (!kAllActive && !active) return;
+    if (!active(PART)) return;
     const VECOPS_GLOBAL char* row = tile_base + (static_cast<int64_t>(kt) * 64 + R) * ks * T::kSrcBytes;
     const VECOPS_GLOBAL char* src = uniform_ptr(row) + unit_bytes[PART];
     if constexpr (SRC == SRC_F32_AS_BF16) {
@@ -514,9 +516,9 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
   // Whole tile with bounds checks (the partial last K tile): rows k >= K read as
   // zero, columns n >= N as zero.
   __device__ __forceinline__ void fetch_checked(int kt) {
-    if (!kAllActive && !active) return;
 #pragma unroll
     for (int u = 0; u < UNITS; ++u) {
+      if (!active(u)) continue;
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
         const int k = kt * 64 + kb[u] * 8 + r;
@@ -541,7 +543,7 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
   // output chunk for n-row E of unit PART: dword j = (regs[2j][E], regs[2j+1][E])
   template <int PART, int E>
   __device__ __forceinline__ void store_op(char* lds_tile) const {
-    if (!kAllActive && !active) return;
+    if (!active(PART)) return;
     constexpr uint32_t sel = (E & 1) ? 0x07060302u : 0x05040100u;
     u32x4 out;
     out.x = __builtin_amdgcn_perm(regs[PART][1][E >> 1], regs[PART][0][E >> 1], sel);
@@ -869,15 +871,15 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
     });
     // the wavefront reads back only what it wrote itself: its own LDS traffic is ordered
     constexpr int SEGS = TILE_COLS / 8;        // 16-byte segments per row
-    constexpr int ROWS_PER_PASS = 64 / SEGS;   // rows one load/store instruction covers
-    const int seg = lane % SEGS, sub = lane / SEGS;
+    constexpr int TOTAL = TILE_ROWS * SEGS;    // 16-byte segments of this wavefront's tile
+    static_assert(TOTAL % 64 == 0, "whole store instructions");
     uint16_t* out = reinterpret_cast<uint16_t*>(c_base) + batch * p.c_bs +
-                    static_cast<int64_t>(m0 + wm * TILE_ROWS) * p.c_rs + n0 + wn * TILE_COLS + seg * 8;
+                    static_cast<int64_t>(m0 + wm * TILE_ROWS) * p.c_rs + n0 + wn * TILE_COLS;
 #pragma unroll
-    for (int r0 = 0; r0 < TILE_ROWS; r0 += ROWS_PER_PASS) {
-      const int r = r0 + sub;
+    for (int base = 0; base < TOTAL; base += 64) {
+      const int idx = base + lane, r = idx / SEGS, seg = idx % SEGS;
       const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + seg * 16);
-      *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs) = v;
+      *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + seg * 8) = v;
     }
   } else if (simple && (INT ? (p.out_kind == OUT_I32 && p.row_scales == nullptr && p.correction == nullptr)
                             : p.out_kind == OUT_F32)) {
