@@ -66,8 +66,6 @@ def test_gpu_reproduces_golden(device, case):
     import torch
     from vecops_amd import capi
     kind = case["kind"]
-    if kind == "u8i8_i32":
-        pytest.skip("u8 operands are not built yet")
     inp = make_inputs(case)
     in_bf16 = kind in ("bf16_f32", "bf16_bf16")
     a = _to_device(inp["a"], device, in_bf16)
@@ -81,7 +79,7 @@ def test_gpu_reproduces_golden(device, case):
         got = c.cpu().numpy()
     else:
         out_dt = {"bf16_f32": torch.float32, "f32_f32": torch.float32, "bf16_bf16": torch.bfloat16,
-                  "f32_bf16": torch.bfloat16, "i8_i32": torch.int32}[kind]
+                  "f32_bf16": torch.bfloat16, "i8_i32": torch.int32, "u8i8_i32": torch.int32}[kind]
         c = torch.zeros(inp["c_shape"], dtype=out_dt, device=device)
         cin = torch.from_numpy(inp["cin"]).to(device) if "cin" in inp else None
         capi.matmul(a, b, c, c_in=cin)

@@ -247,6 +247,49 @@ def test_int8_gemm_bit_exact(device, oracle, m, n, k):
     assert np.array_equal(c.cpu().numpy(), oracle.matmul_i8_dense(a, b))
 
 
+@pytest.mark.parametrize("signs", ["us", "su", "uu"])
+@pytest.mark.parametrize("m,n,k", [(19, 21, 69), (1, 128, 65), (300, 520, 1000), (256, 256, 128), (64, 48, 8191)])
+def test_unsigned_byte_operands_bit_exact(device, oracle, signs, m, n, k):
+    """AMX_I8I32<A, B> with uint8 on either side (matmul/details/kernel/amx/Atoms.h:73-86): the
+    unsigned side is staged as u - 128 and restored with row / column sums in the epilogue;
+    every int32 must equal the oracle's plain integer sum (tile, split-K and ragged shapes)."""
+    import torch
+    from vecops_amd import capi
+    def gen(seed, shape, unsigned):
+        if unsigned:
+            return (synth.draws(seed, shape[0] * shape[1]) % np.uint64(256)).astype(np.uint8).reshape(shape)
+        return synth.int8_sym(seed, shape)
+    a, b = gen(1, (m, k), signs[0] == "u"), gen(2, (n, k), signs[1] == "u")
+    c = torch.full((m, n), -1, dtype=torch.int32, device=device)
+    capi.matmul(torch.from_numpy(a).to(device), torch.from_numpy(b).to(device), c)
+    torch.cuda.synchronize()
+    want = np.zeros((m, n), np.int32)
+    oracle.matmul(a, b, want, atom=2)
+    assert np.array_equal(c.cpu().numpy(), want)
+    assert np.array_equal(want, (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.int32))
+
+
+def test_unsigned_bytes_batched_cin_and_wrap(device, oracle):
+    """uint8 x uint8 with a rank-3 batch, a broadcast B, an int32 C input and accumulators that
+    wrap (255 * 255 * K > 2^31)."""
+    import torch
+    from vecops_amd import capi
+    batch, m, n, k = 3, 70, 33, 40000
+    a = np.full((batch, m, k), 255, np.uint8)
+    a[1] = (synth.draws(1, m * k) % np.uint64(256)).astype(np.uint8).reshape(m, k)
+    b = np.full((n, k), 255, np.uint8)
+    b[::2] = (synth.draws(2, ((n + 1) // 2) * k) % np.uint64(256)).astype(np.uint8).reshape(-1, k)
+    cin = ((synth.draws(3, batch * m * n) % np.uint64(200001)).astype(np.int64) - 100000).astype(np.int32)
+    cin = cin.reshape(batch, m, n)
+    tb = torch.from_numpy(b).to(device)[None].expand(batch, n, k)          # stride-0 batch
+    c = torch.zeros((batch, m, n), dtype=torch.int32, device=device)
+    capi.matmul(torch.from_numpy(a).to(device), tb, c, c_in=torch.from_numpy(cin).to(device))
+    torch.cuda.synchronize()
+    want = (np.einsum("bmk,nk->bmn", a.astype(np.int64), b.astype(np.int64)) + cin).astype(np.uint64)
+    want = (want & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.int32)
+    assert np.array_equal(c.cpu().numpy(), want)
+
+
 def test_int32_accumulator_wraps(device):
     """tests/ops/MatmulTest.cpp:1025-1055: 262145 products of 127*127 wrap mod 2^32."""
     import torch

@@ -81,6 +81,7 @@ struct Problem {
   View a, b, c, cin;
   bool has_cin;
   int src;       // SrcKind
+  bool a_unsigned, b_unsigned;  // 8-bit integer operands only
   int out_kind;  // OutKind
   int cin_kind;
   int64_t batch, m, n, k;
@@ -112,19 +113,25 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
     return fail(ST_INVALID, "matmul: extent too large");
 
   const uint32_t da = pr->a.dtype, db = pr->b.dtype, dc = pr->c.dtype;
-  if (da != db) return fail(ST_NOT_APPLICABLE, "matmul: a and b dtypes differ (%u, %u)", da, db);
-  if (da == DT_BF16) {
+  const bool bytes_a = da == DT_I8 || da == DT_U8, bytes_b = db == DT_I8 || db == DT_U8;
+  pr->a_unsigned = da == DT_U8;
+  pr->b_unsigned = db == DT_U8;
+  if (da != db && !(bytes_a && bytes_b))
+    return fail(ST_NOT_APPLICABLE, "matmul: a and b dtypes differ (%u, %u)", da, db);
+  if (bytes_a) {
+    // AMX_I8I32<A, B> with A, B in {int8, uint8} (matmul/details/kernel/amx/Atoms.h:73-86)
+    pr->src = (pr->a_unsigned || pr->b_unsigned) ? SRC_I8_FLIP : SRC_I8;
+  } else if (da == DT_BF16) {
     pr->src = SRC_BF16;
   } else if (da == DT_F32) {
     if (compute != VECOPS_HIP_COMPUTE_BF16)
       return fail(ST_NOT_APPLICABLE, "matmul: fp32 compute on fp32 operands is not built; use bf16 compute");
     pr->src = SRC_F32_AS_BF16;
-  } else if (da == DT_I8) {
-    pr->src = SRC_I8;
   } else {
     return fail(ST_NOT_APPLICABLE, "matmul: operand dtype %u not supported", da);
   }
-  if (pr->src == SRC_I8) {
+  const bool is_int = pr->src == SRC_I8 || pr->src == SRC_I8_FLIP;
+  if (is_int) {
     if (dc != DT_I32) return fail(ST_NOT_APPLICABLE, "matmul: int8 operands need an int32 c");
     pr->out_kind = OUT_I32;
   } else {
@@ -135,7 +142,7 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
   pr->cin_kind = pr->out_kind;
   if (pr->has_cin) {
     const uint32_t di = pr->cin.dtype;
-    if (pr->src == SRC_I8) {
+    if (is_int) {
       if (di != DT_I32) return fail(ST_NOT_APPLICABLE, "matmul: c_in must be int32");
       pr->cin_kind = OUT_I32;
     } else if (di == DT_F32) {
@@ -170,7 +177,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     return;
   }
   plan->vector_a = k_vector_ok(pr.a) ? 1 : 0;
-  plan->vector_b = (k_vector_ok(pr.b) || (pr.b.rs == 1 && pr.b.cs != 1 && n_vector_ok(pr.b) && pr.src != SRC_I8)) ? 1 : 0;
+  plan->vector_b = (k_vector_ok(pr.b) || (pr.b.rs == 1 && pr.b.cs != 1 && n_vector_ok(pr.b) && dtype_bytes(pr.b.dtype) != 1)) ? 1 : 0;
   plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
 
   auto tiles = [&](int64_t t) { return ((pr.m + t - 1) / t) * ((pr.n + t - 1) / t) * pr.batch; };
@@ -191,7 +198,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     }
   }
   plan->family = family;
-  const int64_t ktile = pr.src == SRC_I8 ? 128 : 64;
+  const int64_t ktile = dtype_bytes(pr.a.dtype) == 1 ? 128 : 64;
   const int64_t k_tiles = (pr.k + ktile - 1) / ktile;
   const int64_t wgs = tiles(tile);
   int64_t split = 1;
@@ -203,6 +210,8 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
   }
   plan->split_k = static_cast<uint32_t>(split);
   if (split > 1) plan->workspace_bytes = static_cast<uint64_t>(split) * pr.batch * pr.m * pr.n * 4u;
+  // an unsigned 8-bit operand needs the sums of the other operand's rows: after the partials
+  if (pr.src == SRC_I8_FLIP) plan->workspace_bytes += static_cast<uint64_t>(pr.batch) * (pr.m + pr.n) * 4u;
 }
 
 int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* row_scales, const float* column_scales,
@@ -235,7 +244,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   p.b_rs = pr.b.rs; p.b_ks = pr.b.cs; p.b_bs = pr.b.bs;
   p.c_rs = pr.c.rs; p.c_cs = pr.c.cs; p.c_bs = pr.c.bs;
   if (pr.has_cin) { p.cin_rs = pr.cin.rs; p.cin_cs = pr.cin.cs; p.cin_bs = pr.cin.bs; }
-  const bool is_int = pr.src == SRC_I8;
+  const bool is_int = pr.src == SRC_I8 || pr.src == SRC_I8_FLIP;
 
   if (plan.family == VECOPS_HIP_FAMILY_ZERO_K) {
     p.split_k = 0;  // empty sum: the reduce kernel emits epilogue(0)
@@ -256,7 +265,27 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   else if (plan.vector_a && plan.vector_b && plan.b_layout == 1) mode = MODE_NVEC_B;
 
   hipError_t e;
+  if (pr.src == SRC_I8_FLIP) {
+    // terms of the unsigned side(s), kept behind the split-K partials in the workspace
+    const uint64_t partial_bytes = plan.split_k > 1 ? static_cast<uint64_t>(plan.split_k) * pr.batch * pr.m * pr.n * 4u : 0;
+    int32_t* row_term = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + partial_bytes);
+    int32_t* col_term = row_term + pr.batch * pr.m;
+    p.a_flip = pr.a_unsigned ? 0x80808080u : 0u;
+    p.b_flip = pr.b_unsigned ? 0x80808080u : 0u;
+    if (pr.b_unsigned) {  // + 128 * sum_k a'[m,k] per row
+      e = launch_byte_row_sums(pr.a.data, p.batch, p.m, p.k, pr.a.bs, pr.a.rs, pr.a.cs, p.a_flip, 128u, row_term, stream);
+      if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
+      p.row_term = row_term;
+    }
+    if (pr.a_unsigned) {  // + 128 * sum_k b'[n,k] per column
+      e = launch_byte_row_sums(pr.b.data, p.batch, p.n, p.k, pr.b.bs, pr.b.rs, pr.b.cs, p.b_flip, 128u, col_term, stream);
+      if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
+      p.col_term = col_term;
+    }
+    if (pr.a_unsigned && pr.b_unsigned) p.const_term = 16384u * static_cast<uint32_t>(pr.k);
+  }
   switch (pr.src) {
+    case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile, mode, stream); break;
     case SRC_BF16: e = launch_tile_gemm_bf16(p, tile, mode, stream); break;
     case SRC_F32_AS_BF16: e = launch_tile_gemm_f32_as_bf16(p, tile, mode, stream); break;
     default: e = launch_tile_gemm_i8(p, tile, mode, stream); break;

@@ -33,7 +33,14 @@ typedef __attribute__((ext_vector_type(16))) int i32x16;
 typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
 
-enum SrcKind : int { SRC_BF16 = 0, SRC_F32_AS_BF16 = 1, SRC_I8 = 2 };
+// SRC_I8_FLIP: 8-bit integer operands of which at least one is unsigned.  The
+// matrix cores multiply signed bytes only, so an unsigned operand is staged as
+// s = u xor 0x80 = u - 128 and the difference is added back in the epilogue:
+//   sum_k ua*b  = sum_k sa*b  + 128 * sum_k b          (per output column)
+//   sum_k a*ub  = sum_k a*sb  + 128 * sum_k a          (per output row)
+//   sum_k ua*ub = sum_k sa*sb + 128 * sum_k sb + 128 * sum_k sa + 16384 * K
+// all in wrapping 32-bit arithmetic, like the accumulators themselves.
+enum SrcKind : int { SRC_BF16 = 0, SRC_F32_AS_BF16 = 1, SRC_I8 = 2, SRC_I8_FLIP = 3 };
 enum OutKind : int { OUT_F32 = 0, OUT_BF16 = 1, OUT_I32 = 2 };
 // How an operand tile is fetched from global memory.
 enum LoadKind : int {
@@ -51,6 +58,11 @@ struct TileGemmParams {
   const float* row_scales;     // int8 dequant epilogue (null = none)
   const float* column_scales;
   const int32_t* correction;   // int32 row added to every accumulator row (null = none)
+  // unsigned-operand terms (SRC_I8_FLIP; null / zero = none), added to the accumulator first
+  const int32_t* row_term;     // [batch][M]
+  const int32_t* col_term;     // [batch][N]
+  uint32_t const_term;
+  uint32_t a_flip, b_flip;     // 0x80808080 for an unsigned operand, else 0
   int32_t m, n, k;
   int32_t batch;
   int32_t tiles_m, tiles_n;
@@ -130,6 +142,9 @@ __device__ __forceinline__ const VECOPS_GLOBAL char* uniform_ptr(const VECOPS_GL
 // Fast path: one whole 16-byte chunk, no bounds checks (the caller guarantees
 // that the row exists and that the chunk lies inside K).
 
+template <>
+struct SrcTraits<SRC_I8_FLIP> : SrcTraits<SRC_I8> {};
+
 template <int SRC>
 __device__ __forceinline__ u32x4 load_chunk_fast(const VECOPS_GLOBAL char* base, uint32_t offset) {
   // Global address space spelled out: a generic (flat) load would also count
@@ -154,27 +169,27 @@ __device__ __forceinline__ u32x4 load_chunk_fast(const VECOPS_GLOBAL char* base,
 // for the K tail of the vector path and for every chunk of the generic path.
 template <int SRC>
 __device__ __noinline__ u32x4 load_chunk_checked(const void* base, int64_t row_off, int64_t kstep, int k0, int k_end,
-                                                 bool row_ok) {
+                                                 bool row_ok, uint32_t pad) {
+  // `pad` is what an element outside the operand reads as: 0, or for an operand
+  // that is xor-flipped on its way into LDS the flip byte, so that it ends up 0
   constexpr int EPC = SrcTraits<SRC>::kElemsPerChunk;
   uint32_t w0 = 0u, w1 = 0u, w2 = 0u, w3 = 0u;
-  if (row_ok) {
 #pragma unroll
-    for (int e = 0; e < EPC; ++e) {
-      const int k = k0 + e;
-      uint32_t v = 0u;
-      if (k < k_end) {
-        if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
-        else if constexpr (SRC == SRC_F32_AS_BF16) v = cvt_pk_bf16(static_cast<const float*>(base)[row_off + k * kstep], 0.0f) & 0xffffu;
-        else v = static_cast<const uint8_t*>(base)[row_off + k * kstep];
-      }
-      constexpr int per_word = EPC / 4;
-      const uint32_t shifted = v << ((e % per_word) * (32 / per_word));
-      const int word = e / per_word;
-      if (word == 0) w0 |= shifted;
-      else if (word == 1) w1 |= shifted;
-      else if (word == 2) w2 |= shifted;
-      else w3 |= shifted;
+  for (int e = 0; e < EPC; ++e) {
+    const int k = k0 + e;
+    uint32_t v = pad;
+    if (row_ok && k < k_end) {
+      if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
+      else if constexpr (SRC == SRC_F32_AS_BF16) v = cvt_pk_bf16(static_cast<const float*>(base)[row_off + k * kstep], 0.0f) & 0xffffu;
+      else v = static_cast<const uint8_t*>(base)[row_off + k * kstep];
     }
+    constexpr int per_word = EPC / 4;
+    const uint32_t shifted = v << ((e % per_word) * (32 / per_word));
+    const int word = e / per_word;
+    if (word == 0) w0 |= shifted;
+    else if (word == 1) w1 |= shifted;
+    else if (word == 2) w2 |= shifted;
+    else w3 |= shifted;
   }
   return u32x4{w0, w1, w2, w3};
 }
@@ -219,7 +234,9 @@ template <bool INT, typename AccScalar>
 __device__ __forceinline__ void store_output(const TileGemmParams& p, int batch, int row, int col, AccScalar acc) {
   const int64_t c_off = batch * p.c_bs + row * p.c_rs + col * p.c_cs;
   if constexpr (INT) {
-    uint32_t v = static_cast<uint32_t>(acc);
+    uint32_t v = static_cast<uint32_t>(acc) + p.const_term;
+    if (p.row_term) v += static_cast<uint32_t>(p.row_term[static_cast<int64_t>(batch) * p.m + row]);
+    if (p.col_term) v += static_cast<uint32_t>(p.col_term[static_cast<int64_t>(batch) * p.n + col]);
     if (p.correction) v += static_cast<uint32_t>(p.correction[col]);
     if (p.cin) v += static_cast<uint32_t>(
                  static_cast<const int32_t*>(p.cin)[batch * p.cin_bs + row * p.cin_rs + col * p.cin_cs]);
@@ -318,16 +335,18 @@ struct Stager {
   uint32_t row_bytes[CHUNKS];  // byte offset of each staged row from tile_base, chunk included (fast path)
   int64_t rs, ks;              // element strides (checked path)
   int first_row, extent, k_end, ld_row, ld_chunk;
+  uint32_t flip;  // SRC_I8_FLIP: xor mask applied on the way into LDS
   u32x4 regs[CHUNKS];
 
   __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
-                                       int k_end_, int tid) {
+                                       int k_end_, int tid, uint32_t flip_) {
     base = static_cast<const char*>(base_);
     rs = rs_;
     ks = ks_;
     first_row = first_row_;
     extent = extent_;
     k_end = k_end_;
+    flip = flip_;
     ld_chunk = tid & 7;
     ld_row = tid >> 3;
     tile_base = (const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * rs * T::kSrcBytes);
@@ -350,7 +369,7 @@ struct Stager {
     } else {
       const int k0 = kt * 8 * T::kElemsPerChunk + ld_chunk * T::kElemsPerChunk;
       const int row = first_row + ld_row + PART * ROWS_PER_PASS;
-      regs[PART] = load_chunk_checked<SRC>(base, static_cast<int64_t>(row) * rs, ks, k0, k_end, row < extent);
+      regs[PART] = load_chunk_checked<SRC>(base, static_cast<int64_t>(row) * rs, ks, k0, k_end, row < extent, flip & 0xffu);
     }
   }
 
@@ -387,13 +406,15 @@ struct Stager {
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int row = first_row + ld_row + i * ROWS_PER_PASS;
-      regs[i] = load_chunk_checked<SRC>(base, static_cast<int64_t>(row) * rs, ks, k0, k_end, row < extent);
+      regs[i] = load_chunk_checked<SRC>(base, static_cast<int64_t>(row) * rs, ks, k0, k_end, row < extent, flip & 0xffu);
     }
   }
 
   template <int PART>
   __device__ __forceinline__ void commit_part(char* lds_tile) const {
-    *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(ld_row + PART * ROWS_PER_PASS, ld_chunk)) = regs[PART];
+    u32x4 v = regs[PART];
+    if constexpr (SRC == SRC_I8_FLIP) v ^= u32x4{flip, flip, flip, flip};
+    *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(ld_row + PART * ROWS_PER_PASS, ld_chunk)) = v;
   }
 
   // the main loop's view: part PART as numbered store / load operations
@@ -440,7 +461,7 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
   __device__ __forceinline__ bool active(int u) const { return kAllActive || u * THREADS + tid_ < UNITS_TOTAL; }
 
   __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
-                                       int k_end_, int tid) {
+                                       int k_end_, int tid, uint32_t /*flip*/) {
     base = static_cast<const char*>(base_);
     rs = rs_;
     ks = ks_;
@@ -666,8 +687,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
 
   Stager<SRC, LOAD_A, BM, THREADS> stager_a;
   Stager<SRC, LOAD_B, BN, THREADS> stager_b;
-  stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, tid);
-  stager_b.init(static_cast<const char*>(p.b) + batch * p.b_bs * T::kSrcBytes, p.b_rs, p.b_ks, n0, p.n, p.k, tid);
+  stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, tid, p.a_flip);
+  stager_b.init(static_cast<const char*>(p.b) + batch * p.b_bs * T::kSrcBytes, p.b_rs, p.b_ks, n0, p.n, p.k, tid, p.b_flip);
 
   const int frag_row = lane & 31;
   const int frag_half = lane >> 5;
@@ -842,7 +863,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   // out-of-line routine.
   const bool interior = m0 + BM <= p.m && n0 + BN <= p.n;
   const bool aligned = (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
-  const bool simple = interior && aligned && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1;
+  const bool simple = interior && aligned && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1 && SRC != SRC_I8_FLIP;
   char* c_base = static_cast<char*>(p.c);
   if (simple && !INT && p.out_kind == OUT_BF16) {
     // bf16: 8-byte pieces scattered over 32 rows would waste most of every memory

@@ -21,6 +21,11 @@ enum LoadMode : int {
 hipError_t launch_tile_gemm_bf16(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_f32_as_bf16(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
+// 8-bit operands of which at least one is unsigned (p.a_flip / p.b_flip and the epilogue terms set)
+hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
+// out[b][r] = scale * sum_k int8(x[b][r][k] xor flip): the epilogue terms of an unsigned operand
+hipError_t launch_byte_row_sums(const void* x, int32_t batch, int32_t rows, int32_t k, int64_t bs, int64_t rs,
+                                int64_t ks, uint32_t flip, uint32_t scale, int32_t* out, hipStream_t stream);
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
 
 // Shared by the per-class translation units.

@@ -241,7 +241,7 @@ constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
 #else
 #define OPERANDS "i8"
 #define COMPUTE "i32"
-constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8);
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);  // either side may be unsigned
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_I32);
 #endif
 

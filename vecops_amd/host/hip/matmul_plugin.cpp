@@ -128,7 +128,8 @@ std::shared_ptr<rt::Operator> assemble(rt::OperatorSchema schema,
 
 rt::OperatorSchema make_matmul_schema() {
   using rt::dtype_bit;
-  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8);
+  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8) |
+                           dtype_bit(DType::UInt8);
   const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int32);
   std::vector<rt::ParameterSchema> params;
   params.push_back(tensor_param("a", in, std::nullopt, VECOPS_TENSOR_READ));
@@ -162,6 +163,16 @@ rt::OperatorSchema make_matmul_w8a16_group_schema() {
 
 // ---- recipes ------------------------------------------------------------------------------------
 
+// Operand dtypes of a class: the 8-bit integer class takes signed and unsigned
+// bytes on either side (AMX_I8I32<A, B>, matmul/details/kernel/amx/Atoms.h:73-86).
+static bool takes(OperandClass operands, DType dtype) {
+  switch (operands) {
+    case OperandClass::BF16: return dtype == DType::BFloat16;
+    case OperandClass::F32: return dtype == DType::Float32;
+    default: return dtype == DType::Int8 || dtype == DType::UInt8;
+  }
+}
+
 MatmulRecipe::MatmulRecipe(OperandClass operands) : operands_(operands) {
   id_ = operands == OperandClass::BF16 ? "hip.matmul.bf16.tile"
         : operands == OperandClass::F32 ? "hip.matmul.f32.tile"
@@ -175,10 +186,8 @@ Status MatmulRecipe::match(const rt::KernelCall& call) const {
   const TensorView* cin = tensor_at(values, 2);
   const TensorView* c = tensor_at(values, 3);
   if (a == nullptr || b == nullptr || c == nullptr) return invalid("vecops::matmul needs a, b and c tensors");
-  const DType want = operands_ == OperandClass::BF16 ? DType::BFloat16
-                     : operands_ == OperandClass::F32 ? DType::Float32
-                                                      : DType::Int8;
-  if (a->dtype != want || b->dtype != want) return not_applicable("operand dtypes belong to another recipe");
+  if (!takes(operands_, a->dtype) || !takes(operands_, b->dtype))
+    return not_applicable("operand dtypes belong to another recipe");
   const bool int_out = operands_ == OperandClass::I8;
   if (int_out ? c->dtype != DType::Int32 : (c->dtype != DType::Float32 && c->dtype != DType::BFloat16))
     return not_applicable("output dtype does not fit these operands");
@@ -270,10 +279,7 @@ MatmulDispatchPolicy::candidates(const rt::KernelCall& call,
   for (std::size_t i = 0; i < recipes.size(); ++i) {
     if (recipes[i] == nullptr) continue;
     if (const auto* mm = dynamic_cast<const MatmulRecipe*>(recipes[i].get()); mm != nullptr && a != nullptr) {
-      const DType want = mm->operands() == OperandClass::BF16 ? DType::BFloat16
-                         : mm->operands() == OperandClass::F32 ? DType::Float32
-                                                               : DType::Int8;
-      if (a->dtype != want) continue;
+      if (!takes(mm->operands(), a->dtype)) continue;
     }
     order.push_back(i);
   }
