@@ -98,7 +98,8 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul(const VecopsHipOperand* a, cons
  * ops::Matmul<Config>::operator() (ops/Matmul.h:530-570) for
  *   a,b bf16 -> c f32|bf16      (AMX_BF16F32)
  *   a,b f32  -> c f32|bf16      (bf16 or fp32 compute, see VecopsHipCompute)
- *   a,b i8   -> c i32           (AMX_I8I32<int8,int8>; accumulators wrap mod 2^32)
+ *   a,b i8|u8 -> c i32          (AMX_I8I32<A,B>, either side signed or unsigned;
+ *                                accumulators wrap mod 2^32)
  * c_in may be null (zero accumulator); otherwise it has c's dtype class (f32,
  * bf16 or i32) and may alias c element for element.  K == 0 writes zeros or
  * C_in; zero M, N or batch writes nothing (ops/Matmul.h:41-43).  Operand

@@ -96,7 +96,7 @@ def test_abi_layout(tmp_path):
 
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
-    assert len(files) == 12
+    assert len(files) == 14
     for f in files:
         name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
         assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
@@ -133,9 +133,13 @@ def test_resolve_picks_recipe_by_dtype_and_placement(host):
     assert op.resolve(f) == "vecops::matmul;operands=bf16;compute=bf16;memory=device;backend=hip-gfx950"
     # explicit ComputeType specialization (bf16 is what the x86 reference path computes in)
     assert "compute=bf16" in op.resolve(H.Frame([a32, b32, None, c32], outputs=(3,)), {"ComputeType": ("dtype", H.BF16)})
-    with pytest.raises(H.HostError) as e:       # true fp32 compute is a recipe that is not built
-        op.resolve(H.Frame([a32, b32, None, c32], outputs=(3,)), {"ComputeType": ("dtype", H.F32)})
-    assert e.value.code == 2
+    # true fp32 compute (the SME_F32F32 atom) is a specialization of its own
+    assert op.resolve(H.Frame([a32, b32, None, c32], outputs=(3,)), {"ComputeType": ("dtype", H.F32)}) == \
+        "vecops::matmul;operands=f32;compute=f32;memory=host;backend=hip-gfx950"
+    with pytest.raises(H.HostError) as e:       # bf16 operands cannot ask for fp32 compute
+        op.resolve(H.Frame([bf16((8, 16)), bf16((8, 16)), None, np.zeros((8, 8), np.float32)], outputs=(3,)),
+                   {"ComputeType": ("dtype", H.F32)})
+    assert e.value.code in (2, 3)
     w = host.operator("vecops::matmul_w8a16_group")
     x, wq, s, y = bf16((4, 256)), np.zeros((8, 256), np.int8), np.zeros((8, 2), np.float32), bf16((4, 8))
     assert w.resolve(H.Frame([x, wq, s, y], outputs=(3,))) == \

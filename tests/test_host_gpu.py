@@ -98,6 +98,25 @@ def test_matmul_rank3_fp32_and_int8(host, oracle, device):
     ci = torch.zeros((130, 140), dtype=torch.int32, device=device)
     op.invoke(H.Frame([torch.from_numpy(ai).to(device), torch.from_numpy(bi).to(device), None, ci], outputs=(3,)))
     assert np.array_equal(ci.cpu().numpy(), oracle.matmul_i8_dense(ai, bi))
+    # unsigned activations against signed weights, host tensors: the same recipe and artifact
+    au = (synth.draws(5, 130 * 515) % np.uint64(256)).astype(np.uint8).reshape(130, 515)
+    cu = np.zeros((130, 140), np.int32)
+    op.invoke(H.Frame([au, bi, None, cu], outputs=(3,)))
+    assert np.array_equal(cu, (au.astype(np.int64) @ bi.astype(np.int64).T).astype(np.int32))
+
+
+def test_matmul_fp32_compute_operator(host, oracle):
+    """ComputeType=Float32 selects the fp32-compute artifact: operands are not rounded to bf16."""
+    op = host.operator("vecops::matmul")
+    m, n, k = 96, 80, 300
+    a, b = synth.uniform_pm1(1, (m, k)), synth.uniform_pm1(2, (n, k))
+    c = np.zeros((m, n), np.float32)
+    op.invoke(H.Frame([a, b, None, c], outputs=(3,)), {"ComputeType": ("dtype", H.F32)})
+    exact = a.astype(np.float64) @ b.astype(np.float64).T
+    assert rel_err(c, exact) <= 1.2e-7 * k
+    c_bf16_compute = np.zeros((m, n), np.float32)
+    op.invoke(H.Frame([a, b, None, c_bf16_compute], outputs=(3,)))
+    assert rel_err(c_bf16_compute, exact) > 1e-3        # the default rounds the operands to bf16
 
 
 def test_matmul_i8_dequant_operator(host, oracle, device):

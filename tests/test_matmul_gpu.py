@@ -89,6 +89,45 @@ def test_fp32_memory_bf16_compute(device, oracle):
         assert rel_err(c2.cpu().numpy(), want) <= fp32_tol(k)
 
 
+def fp32_compute_tol(k):
+    """fp32 products summed in fp32 in an unspecified order: a random walk of K roundings of
+    half an ulp at the size of the partial sums (~sqrt(K)/3 for U[-1,1) operands), scaled like
+    rel_err by max(1, |c|); a few sigma over a million outputs.  Operands rounded to bf16 would
+    be off by 2^-9 * sqrt(K) - a hundred times more."""
+    return max(2e-6, 1.2e-7 * k)
+
+
+@pytest.mark.parametrize("m,n,k,layout", [(1024, 1024, 1024, "nn"), (1024, 1024, 1024, "nt"), (37, 51, 79, "nt"),
+                                          (300, 520, 1001, "nn"), (257, 255, 65, "tn"), (64, 48, 4099, "nt"),
+                                          (512, 768, 96, "nn")])
+def test_fp32_compute(device, oracle, m, n, k, layout):
+    """fp32 operands multiplied in fp32 (the SME_F32F32 atom, matmul/details/kernel/sme/Atoms.h:65-76;
+    1024^3 with B as [K,N] is BASELINE configs[0]): operands must NOT be rounded to bf16."""
+    import torch
+    from vecops_amd import capi
+    a, b = synth.uniform_pm1(1, (m, k)), synth.uniform_pm1(2, (n, k))
+    ta = torch.from_numpy(a).to(device)
+    if layout[0] == "t":
+        ta = torch.from_numpy(np.ascontiguousarray(a.T)).to(device).t()
+    tb = torch.from_numpy(b).to(device)
+    if layout[1] == "n":
+        tb = torch.from_numpy(np.ascontiguousarray(b.T)).to(device).t()       # B stored [K, N]
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul(ta, tb, c, compute=capi.COMPUTE_F32)
+    torch.cuda.synchronize()
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, atom=1, acc_f64=True)
+    assert rel_err(c.cpu().numpy(), want) <= fp32_compute_tol(k)
+    assert rel_err(want, (a.astype(np.float64) @ b.astype(np.float64).T)) <= 1e-6   # the oracle itself: plain fp64 product
+    # accumulate into an fp32 C input, bf16 output
+    cin = synth.uniform_pm1(3, (m, n))
+    c16 = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    capi.matmul(ta, tb, c16, c_in=torch.from_numpy(cin).to(device), compute=capi.COMPUTE_F32)
+    torch.cuda.synchronize()
+    got16 = synth.bf16_to_f32(host_bits(c16))
+    assert rel_err(got16, want + cin) <= 2.0 ** -8
+
+
 @pytest.mark.parametrize("layout", ["nn", "tn", "tt", "inner2", "padded", "c_transposed", "offset2"])
 def test_layouts(device, oracle, layout):
     """Strided views give the values of dense copies (tests/ops/MatmulOrientationTest.cpp:139,249;

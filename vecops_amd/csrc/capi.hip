@@ -124,9 +124,9 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
   } else if (da == DT_BF16) {
     pr->src = SRC_BF16;
   } else if (da == DT_F32) {
-    if (compute != VECOPS_HIP_COMPUTE_BF16)
-      return fail(ST_NOT_APPLICABLE, "matmul: fp32 compute on fp32 operands is not built; use bf16 compute");
-    pr->src = SRC_F32_AS_BF16;
+    if (compute != VECOPS_HIP_COMPUTE_BF16 && compute != VECOPS_HIP_COMPUTE_F32)
+      return fail(ST_INVALID, "matmul: unknown compute type %u", compute);
+    pr->src = compute == VECOPS_HIP_COMPUTE_F32 ? SRC_F32 : SRC_F32_AS_BF16;
   } else {
     return fail(ST_NOT_APPLICABLE, "matmul: operand dtype %u not supported", da);
   }
@@ -157,6 +157,9 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
 }
 
 constexpr int kComputeUnits = 256;
+
+// elements of K in one 128-byte K tile of the compute type
+int k_tile_elements(int src) { return src == SRC_I8 || src == SRC_I8_FLIP ? 128 : src == SRC_F32 ? 32 : 64; }
 
 // The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure
 // integer function of (operand class, m, n, k); it picks the workgroup tile by
@@ -198,7 +201,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     }
   }
   plan->family = family;
-  const int64_t ktile = dtype_bytes(pr.a.dtype) == 1 ? 128 : 64;
+  const int64_t ktile = k_tile_elements(pr.src);
   const int64_t k_tiles = (pr.k + ktile - 1) / ktile;
   const int64_t wgs = tiles(tile);
   int64_t split = 1;
@@ -254,7 +257,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   }
 
   const int tile = plan.family == VECOPS_HIP_FAMILY_TILE_256 ? 256 : plan.family == VECOPS_HIP_FAMILY_TILE_128 ? 128 : 64;
-  const int ktile = is_int ? 128 : 64;
+  const int ktile = k_tile_elements(pr.src);
   p.tiles_m = static_cast<int32_t>((pr.m + tile - 1) / tile);
   p.tiles_n = static_cast<int32_t>((pr.n + tile - 1) / tile);
   const int k_tiles = static_cast<int>((pr.k + ktile - 1) / ktile);
@@ -288,6 +291,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile, mode, stream); break;
     case SRC_BF16: e = launch_tile_gemm_bf16(p, tile, mode, stream); break;
     case SRC_F32_AS_BF16: e = launch_tile_gemm_f32_as_bf16(p, tile, mode, stream); break;
+    case SRC_F32: e = launch_tile_gemm_f32(p, tile, mode, stream); break;
     default: e = launch_tile_gemm_i8(p, tile, mode, stream); break;
   }
   if (e != hipSuccess) return fail(ST_EXEC, "tile kernel launch: %s", hipGetErrorString(e));

@@ -40,7 +40,10 @@ typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
 //   sum_k a*ub  = sum_k a*sb  + 128 * sum_k a          (per output row)
 //   sum_k ua*ub = sum_k sa*sb + 128 * sum_k sb + 128 * sum_k sa + 16384 * K
 // all in wrapping 32-bit arithmetic, like the accumulators themselves.
-enum SrcKind : int { SRC_BF16 = 0, SRC_F32_AS_BF16 = 1, SRC_I8 = 2, SRC_I8_FLIP = 3 };
+// SRC_F32: fp32 operands multiplied in fp32 on the fp32 matrix cores
+// (v_mfma_f32_32x32x2_f32); a 16-byte chunk holds four k, a k-step (two chunks)
+// feeds four MFMAs per accumulator tile, a K tile is 32 elements.
+enum SrcKind : int { SRC_BF16 = 0, SRC_F32_AS_BF16 = 1, SRC_I8 = 2, SRC_I8_FLIP = 3, SRC_F32 = 4 };
 enum OutKind : int { OUT_F32 = 0, OUT_BF16 = 1, OUT_I32 = 2 };
 // How an operand tile is fetched from global memory.
 enum LoadKind : int {
@@ -144,6 +147,12 @@ __device__ __forceinline__ const VECOPS_GLOBAL char* uniform_ptr(const VECOPS_GL
 
 template <>
 struct SrcTraits<SRC_I8_FLIP> : SrcTraits<SRC_I8> {};
+template <>
+struct SrcTraits<SRC_F32> {
+  static constexpr int kElemsPerChunk = 4;
+  static constexpr int kSrcBytes = 4;
+  static constexpr bool kInt = false;
+};
 
 template <int SRC>
 __device__ __forceinline__ u32x4 load_chunk_fast(const VECOPS_GLOBAL char* base, uint32_t offset) {
@@ -181,6 +190,7 @@ __device__ __noinline__ u32x4 load_chunk_checked(const void* base, int64_t row_o
     if (row_ok && k < k_end) {
       if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
       else if constexpr (SRC == SRC_F32_AS_BF16) v = cvt_pk_bf16(static_cast<const float*>(base)[row_off + k * kstep], 0.0f) & 0xffffu;
+      else if constexpr (SRC == SRC_F32) v = __float_as_uint(static_cast<const float*>(base)[row_off + k * kstep]);
       else v = static_cast<const uint8_t*>(base)[row_off + k * kstep];
     }
     constexpr int per_word = EPC / 4;
@@ -215,7 +225,12 @@ struct AccTile<true> {
 template <int SRC>
 __device__ __forceinline__ void mfma_step(typename AccTile<SrcTraits<SRC>::kInt>::type& acc, const u32x4& a,
                                           const u32x4& b) {
-  if constexpr (SrcTraits<SRC>::kInt) {
+  if constexpr (SRC == SRC_F32) {
+    // lanes 0-31 hold k0..k3 of their row, lanes 32-63 k4..k7: MFMA e multiplies the pair (k_e, k_{4+e})
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[e]), __uint_as_float(b[e]), acc, 0, 0, 0);
+  } else if constexpr (SrcTraits<SRC>::kInt) {
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a), __builtin_bit_cast(i32x4, b), acc, 0, 0,
                                                 0);
   } else {
@@ -579,6 +594,102 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
     static_for<4>([&](auto ce) { store_op<PART, decltype(ce)::value>(lds_tile); });
   }
 
+  __device__ __forceinline__ void commit(char* lds_tile) const {
+    static_for<UNITS>([&](auto cu) { commit_part<decltype(cu)::value>(lds_tile); });
+  }
+};
+
+// LOAD_NVEC for 32-bit compute elements: units of 4(k) x 4(n); a thread loads four
+// 16-byte rows along n and writes four K-contiguous chunks, the transposition being
+// a mere choice of registers.
+template <int ROWS, int THREADS>
+struct Stager<SRC_F32, LOAD_NVEC, ROWS, THREADS> {
+  using T = SrcTraits<SRC_F32>;
+  static constexpr int UNITS_TOTAL = 2 * ROWS;  // (ROWS / 4) along n  x  8 along k
+  static constexpr int UNITS = (UNITS_TOTAL + THREADS - 1) / THREADS;
+  static constexpr bool kAllActive = UNITS_TOTAL % THREADS == 0;
+  static constexpr int kParts = UNITS;
+  static constexpr int kStoreOps = 4;
+  static constexpr int kLoadOps = 4;
+  static constexpr bool kHasSpare = false;
+  struct Spare {};
+  const char* base;
+  const VECOPS_GLOBAL char* tile_base;
+  uint32_t unit_bytes[UNITS];
+  int64_t rs, ks;
+  int first_row, extent, k_end;
+  int n_local[UNITS], kb[UNITS];
+  int tid_;
+  uint32_t regs[UNITS][4][4];  // [k row][n]
+
+  __device__ __forceinline__ bool active(int u) const { return kAllActive || u * THREADS + tid_ < UNITS_TOTAL; }
+
+  __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
+                                       int k_end_, int tid, uint32_t /*flip*/) {
+    base = static_cast<const char*>(base_);
+    rs = rs_;
+    ks = ks_;
+    first_row = first_row_;
+    extent = extent_;
+    k_end = k_end_;
+    tid_ = tid;
+    tile_base = (const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * 4);
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+      const int unit = u * THREADS + tid;
+      n_local[u] = (unit % (ROWS / 4)) * 4;
+      kb[u] = (unit / (ROWS / 4)) & 7;  // chunk of the K tile: k = 4*kb .. 4*kb+3
+      const int n = min(first_row + n_local[u], extent - 4) - first_row;  // extent is a multiple of 4 on this path
+      unit_bytes[u] = static_cast<uint32_t>((static_cast<int64_t>(kb[u]) * 4 * ks + n) * 4);
+    }
+  }
+
+  template <int PART, int R>
+  __device__ __forceinline__ void load_op(int kt) {
+    if (!active(PART)) return;
+    const VECOPS_GLOBAL char* row = tile_base + (static_cast<int64_t>(kt) * 32 + R) * ks * 4;
+    const u32x4 v = *(const VECOPS_GLOBAL u32x4*)(uniform_ptr(row) + unit_bytes[PART]);
+    regs[PART][R][0] = v.x;
+    regs[PART][R][1] = v.y;
+    regs[PART][R][2] = v.z;
+    regs[PART][R][3] = v.w;
+  }
+  template <int PART>
+  __device__ __forceinline__ void fetch_part(int kt) {
+    static_for<4>([&](auto cr) { load_op<PART, decltype(cr)::value>(kt); });
+  }
+  __device__ __forceinline__ void fetch_full(int kt) {
+    static_for<UNITS>([&](auto cu) { fetch_part<decltype(cu)::value>(kt); });
+  }
+  __device__ __forceinline__ void fetch_full_spare(Spare&, int) {}
+  __device__ __forceinline__ void take_spare(const Spare&) {}
+
+  __device__ __forceinline__ void fetch_checked(int kt) {
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+      if (!active(u)) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int k = kt * 32 + kb[u] * 4 + r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int n = first_row + n_local[u] + e;
+          regs[u][r][e] = (k < k_end && n < extent) ? __float_as_uint(reinterpret_cast<const float*>(base)[k * ks + n]) : 0u;
+        }
+      }
+    }
+  }
+
+  template <int PART, int E>
+  __device__ __forceinline__ void store_op(char* lds_tile) const {
+    if (!active(PART)) return;
+    const u32x4 out = {regs[PART][0][E], regs[PART][1][E], regs[PART][2][E], regs[PART][3][E]};
+    *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(n_local[PART] + E, kb[PART])) = out;
+  }
+  template <int PART>
+  __device__ __forceinline__ void commit_part(char* lds_tile) const {
+    static_for<4>([&](auto ce) { store_op<PART, decltype(ce)::value>(lds_tile); });
+  }
   __device__ __forceinline__ void commit(char* lds_tile) const {
     static_for<UNITS>([&](auto cu) { commit_part<decltype(cu)::value>(lds_tile); });
   }

@@ -13,13 +13,14 @@ namespace vecops_hip {
 enum LoadMode : int {
   MODE_GENERIC = 0,  // element loads, any strides
   MODE_KVEC = 1,     // A and B K-contiguous and 16-byte aligned
-  MODE_NVEC_B = 2    // A K-contiguous; B stored [K,N] row-major, 16-byte aligned (16-bit compute types)
+  MODE_NVEC_B = 2    // A K-contiguous; B stored [K,N] row-major, 16-byte aligned (16- and 32-bit compute types)
 };
 
 // tile: 256, 128 or 64 (workgroup tile edge).  Returns the HIP error of the
 // launch (hipSuccess when enqueued).
 hipError_t launch_tile_gemm_bf16(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_f32_as_bf16(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
+hipError_t launch_tile_gemm_f32(const TileGemmParams& p, int tile, int mode, hipStream_t stream);  // fp32 compute
 hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
 // 8-bit operands of which at least one is unsigned (p.a_flip / p.b_flip and the epilogue terms set)
 hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
@@ -53,7 +54,7 @@ hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN>
 hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t stream) {
   if (mode == MODE_KVEC) return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_KVEC>(p, stream);
-  if constexpr (SrcTraits<SRC>::kElemsPerChunk == 8) {
+  if constexpr (SrcTraits<SRC>::kElemsPerChunk == 8 || SRC == SRC_F32) {
     if (mode == MODE_NVEC_B)
       return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_NVEC>(p, stream);
   }

@@ -1,7 +1,7 @@
 // Source of the HIP kernel-artifact DSOs for the vecops matmul operators.  One
 // DSO per (operator, operand class, memory placement); the build compiles this
 // file once per artifact with
-//   -DVECOPS_ARTIFACT_KIND=<0..4>   0 matmul bf16, 1 matmul f32 (bf16 compute), 2 matmul i8,
+//   -DVECOPS_ARTIFACT_KIND=<0..5>   0 matmul bf16, 1 matmul f32 (bf16 compute), 5 matmul f32 (fp32 compute), 2 matmul i8,
 //                                   3 matmul_i8_dequant, 4 matmul_w8a16_group
 //   -DVECOPS_ARTIFACT_DEVICE=<0|1>  0: tensors are host memory, staged through HBM here
 //                                   1: tensors are HIP device pointers, used in place
@@ -225,7 +225,7 @@ int32_t check_call(const VecopsCall* call, uint32_t expected, VecopsError* error
 }
 
 // =================================================================================================
-#if VECOPS_ARTIFACT_KIND <= 2  // vecops::matmul (a, b, c_in?, c)
+#if VECOPS_ARTIFACT_KIND <= 2 || VECOPS_ARTIFACT_KIND == 5  // vecops::matmul (a, b, c_in?, c)
 // =================================================================================================
 
 #if VECOPS_ARTIFACT_KIND == 0
@@ -238,6 +238,12 @@ constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
 #define COMPUTE "bf16"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
+#elif VECOPS_ARTIFACT_KIND == 5
+#define OPERANDS "f32"
+#define COMPUTE "f32"
+#define COMPUTE_CODE VECOPS_HIP_COMPUTE_F32
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
 #else
 #define OPERANDS "i8"
 #define COMPUTE "i32"
@@ -245,6 +251,9 @@ constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);  // ei
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_I32);
 #endif
 
+#ifndef COMPUTE_CODE
+#define COMPUTE_CODE VECOPS_HIP_COMPUTE_BF16
+#endif
 constexpr const char* kOperatorName = "vecops::matmul";
 constexpr const char* kKey =
   "vecops::matmul;operands=" OPERANDS ";compute=" COMPUTE ";memory=" MEMORY_NAME ";backend=hip-gfx950";
@@ -281,8 +290,7 @@ int32_t plan(const VecopsCall* call, VecopsHipOperand ops[4], bool* has_cin, Vec
   ops[3].data = origin(c);
   if (cin != nullptr) ops[2].data = origin(cin);
 #endif
-  int32_t rc = vecops_hip_plan_matmul(&ops[0], &ops[1], *has_cin ? &ops[2] : nullptr, &ops[3],
-                                      VECOPS_HIP_COMPUTE_BF16, out);
+  int32_t rc = vecops_hip_plan_matmul(&ops[0], &ops[1], *has_cin ? &ops[2] : nullptr, &ops[3], COMPUTE_CODE, out);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
   return VECOPS_STATUS_OK;
 }
@@ -324,8 +332,8 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
     return report_hip(error, "allocating split-K scratch", e);
   ws_size = p.workspace_bytes;
 #endif
-  int32_t rc = vecops_hip_matmul(&ops[0], &ops[1], has_cin ? &ops[2] : nullptr, &ops[3], VECOPS_HIP_COMPUTE_BF16, ws,
-                                 ws_size, stream);
+  int32_t rc = vecops_hip_matmul(&ops[0], &ops[1], has_cin ? &ops[2] : nullptr, &ops[3], COMPUTE_CODE, ws, ws_size,
+                                 stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
   return finish(&staging, stream, error);
 }

@@ -197,8 +197,12 @@ Status MatmulRecipe::match(const rt::KernelCall& call) const {
   auto compute = compute_type(call);
   if (!compute) return compute.status();
   if (operands_ == OperandClass::F32) {
-    // fp32 memory: bf16 compute is built (what vecops' x86 path does); true fp32 compute is not
-    if (compute.value() != DType::BFloat16) return not_applicable("ComputeType=Float32 is not built for fp32 operands");
+    // fp32 memory: bf16 compute (what vecops' x86 path does, AMX_BF16F32 on converted operands) or
+    // fp32 compute (the SME_F32F32 atom, matmul/details/kernel/sme/Atoms.h:65-76)
+    if (compute.value() != DType::BFloat16 && compute.value() != DType::Float32)
+      return not_applicable("ComputeType must be BFloat16 or Float32 for fp32 operands");
+  } else if (operands_ == OperandClass::BF16 && compute.value() != DType::BFloat16) {
+    return not_applicable("bf16 operands are multiplied in bf16");
   }
   auto place = placement_of(call);
   if (!place) return place.status();
@@ -209,7 +213,8 @@ rt::Result<rt::BoundKernelRecipe> MatmulRecipe::bind(const rt::KernelCall& call)
   if (Status st = match(call); !st.ok()) return st;
   const Placement place = placement_of(call).value();
   const char* operands = operands_ == OperandClass::BF16 ? "bf16" : operands_ == OperandClass::F32 ? "f32" : "i8";
-  const char* compute = operands_ == OperandClass::I8 ? "i32" : "bf16";
+  const bool f32_compute = operands_ == OperandClass::F32 && compute_type(call).value() == DType::Float32;
+  const char* compute = operands_ == OperandClass::I8 ? "i32" : f32_compute ? "f32" : "bf16";
   rt::BoundKernelRecipe bound;
   bound.recipe_id = id_;
   bound.specialization_key = std::string(kMatmulName) + ";operands=" + operands + ";compute=" + compute +
