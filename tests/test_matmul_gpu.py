@@ -474,7 +474,8 @@ def test_config4_int8_full_size_checksum(device, oracle):
 # --- weight-only int8, per-group scales (no reference counterpart: parity unpinned) ------------
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 8, 16])
-@pytest.mark.parametrize("n,k,group", [(14336, 4096, 128), (300, 512, 64), (17, 1024, 128), (4096, 11008, 128)])
+@pytest.mark.parametrize("n,k,group", [(14336, 4096, 128), (300, 512, 64), (17, 1024, 128), (4096, 11008, 128),
+                                       (2064, 4096, 256), (2100, 4096, 128)])
 def test_w8a16_group(device, oracle, m, n, k, group):
     """Checked against the fp64 brute force of the stated contract: fp32 accumulation
     over K=4096 plus the final bf16 rounding stay within one bf16 ulp (2^-7) of it."""

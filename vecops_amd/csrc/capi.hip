@@ -329,6 +329,15 @@ void launch_skinny_mfma(const SkinnyW8A16Params& p, hipStream_t stream) {
                      dim3(64 * kWaves), 0, stream, p);
 }
 
+// The register-resident variant: K must be exactly 8 wavefronts x 8 steps x 64.
+template <int SPG, int TILES>
+void launch_skinny_mfma_resident(const SkinnyW8A16Params& p, int passes, hipStream_t stream) {
+  const int64_t rows_per_wg = static_cast<int64_t>(16) * TILES * passes;
+  const int64_t blocks = (p.n + rows_per_wg - 1) / rows_per_wg;
+  hipLaunchKernelGGL((skinny_w8a16_mfma_resident_kernel<SPG, TILES>), dim3(static_cast<unsigned>(blocks)), dim3(512), 0,
+                     stream, p, passes);
+}
+
 }  // namespace
 
 extern "C" {
@@ -428,7 +437,13 @@ int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t ldx, const int8_t* 
   // GPU rule table of the skinny family: matrix cores once the widening of a weight
   // byte can be shared by three or more activation rows
   const bool mfma_ok = group % 64 == 0 && (group == 64 || group == 128 || group == 256);
-  if (m >= 3 && mfma_ok) {
+  if (m >= 2 && k == 4096 && (group == 128 || group == 256) && n >= 2048) {
+    // activations resident in registers; a workgroup walks two blocks of 32 rows (224 workgroups at
+    // N = 14336).  More passes reuse the activations further but leave too few workgroups to pull
+    // the bandwidth: 4 passes measured 50 % slower.
+    if (group == 128) launch_skinny_mfma_resident<2, 2>(p, 2, s);
+    else launch_skinny_mfma_resident<4, 2>(p, 2, s);
+  } else if (m >= 3 && mfma_ok) {
     const int tiles = m > 4 ? 2 : 1;  // more weight rows per workgroup = fewer activation reloads
     if (group == 64) { if (tiles == 2) launch_skinny_mfma<1, 2>(p, s); else launch_skinny_mfma<1, 1>(p, s); }
     else if (group == 128) { if (tiles == 2) launch_skinny_mfma<2, 2>(p, s); else launch_skinny_mfma<2, 1>(p, s); }

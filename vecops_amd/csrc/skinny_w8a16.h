@@ -268,5 +268,158 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_mfma_kernel(const Ski
   }
 }
 
+// ---- matrix-core family, activations resident in registers -------------------------------------
+// Same arithmetic and operand layout as skinny_w8a16_mfma_kernel, for K = 8 wavefronts
+// x 8 steps x 64 (4096).  In that kernel every step carries, besides its weight loads,
+// two activation loads and its share of the scale loads - four of five memory
+// instructions fetch data that is not weights.  Here a wavefront loads the activation
+// fragments of its K slice once (64 registers) and keeps them while the workgroup walks
+// `passes` consecutive blocks of TILES x 16 weight rows; the scales of a block arrive as
+// one coalesced 4-byte load per lane (lane = row + 16 * group) and are handed to the
+// lanes that need them with lane permutes.  The steps of all passes form one flat
+// sequence with loads D = 4 steps ahead; the K slices are summed through LDS once per
+// pass (double-buffered, one barrier per pass).
+template <int SPG, int TILES>
+__global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const SkinnyW8A16Params p, int passes) {
+  constexpr int WAVES = 8, S = 8, D = 4;  // a deeper pipeline (D = 8) measured no faster
+  constexpr int GPW = S / SPG;                      // scale groups of a wavefront's K slice
+  constexpr int NSC = (16 * GPW + 63) / 64;         // scale registers per tile
+  static_assert(S % SPG == 0 && D % SPG == 0, "whole groups per pipeline round");
+  __shared__ float red[2][WAVES][TILES][16 * 16];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int row = lane & 15, quarter = lane >> 4;
+  const int64_t wg_row0 = static_cast<int64_t>(blockIdx.x) * passes * (16 * TILES);
+  const int64_t last_row = static_cast<int64_t>(p.n) - 1;
+  const int g_begin = wave * GPW;
+  const VECOPS_GLOBAL char* wbase = (const VECOPS_GLOBAL char*)p.w + quarter * 16 + static_cast<int64_t>(wave) * S * 64;
+  const VECOPS_GLOBAL float* sbase = (const VECOPS_GLOBAL float*)p.scales;
+
+  // activation fragments of this K slice, resident for the whole kernel
+  u32x4 x1[S], x2[S];
+  {
+    const VECOPS_GLOBAL char* xrow = (const VECOPS_GLOBAL char*)(p.x + static_cast<int64_t>(min(row, p.m - 1)) * p.ldx) +
+                                     quarter * 32 + static_cast<int64_t>(wave) * S * 128;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      x1[s] = u32x4{0u, 0u, 0u, 0u};
+      x2[s] = u32x4{0u, 0u, 0u, 0u};
+      if (row < p.m) {
+        const VECOPS_GLOBAL u32x4* px = (const VECOPS_GLOBAL u32x4*)(xrow + s * 128);
+        x1[s] = px[0];
+        x2[s] = px[1];
+      }
+    }
+  }
+
+  const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};  // eight bf16 1.0
+  u32x4 wq[D][TILES];
+  float sc_cur[TILES][NSC], sc_nxt[TILES][NSC] = {};
+  f32x4 acc[TILES], dot[TILES], xs = {0.f, 0.f, 0.f, 0.f};
+  const int total = passes * S;
+
+  // rows past N are clamped: computed, never stored
+  auto weight_row = [&](int pass, int t) { return min(wg_row0 + (pass * TILES + t) * 16 + row, last_row); };
+  auto load_scales = [&](float (&dst)[TILES][NSC], int pass) {
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int i = 0; i < NSC; ++i) {
+        const int h = i * 64 + lane;  // holder index = row + 16 * group
+        const int g = min(h >> 4, GPW - 1);
+        dst[t][i] = sbase[weight_row(pass, t) * p.groups + g_begin + g];
+      }
+  };
+  auto issue = [&](auto slot_tag, int step) {
+    constexpr int slot = decltype(slot_tag)::value;
+    if (step < total) {
+      const int pass = step / S, s = step - pass * S;
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+        wq[slot][t] = *(const VECOPS_GLOBAL u32x4*)(wbase + weight_row(pass, t) * p.ldw + s * 64);
+    }
+  };
+  // S is a multiple of D: slot `slot` always holds step s = slot or slot + D of its pass
+  auto consume = [&](auto slot_tag, auto s_tag, int pass) {
+    constexpr int slot = decltype(slot_tag)::value, s = decltype(s_tag)::value;
+    const bf16x8 b1 = __builtin_bit_cast(bf16x8, x1[s]), b2 = __builtin_bit_cast(bf16x8, x2[s]);
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+      uint32_t a[8];
+      const uint32_t wd[4] = {wq[slot][t].x ^ 0x80808080u, wq[slot][t].y ^ 0x80808080u, wq[slot][t].z ^ 0x80808080u,
+                              wq[slot][t].w ^ 0x80808080u};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float f0 = static_cast<float>(wd[q] & 0xffu), f1 = static_cast<float>((wd[q] >> 8) & 0xffu);
+        const float f2 = static_cast<float>((wd[q] >> 16) & 0xffu), f3 = static_cast<float>(wd[q] >> 24);
+        // upper halves of two fp32 = two bf16 (exact: the values are integers below 256)
+        a[2 * q] = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+        a[2 * q + 1] = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+      }
+      const u32x4 a1 = {a[0], a[1], a[2], a[3]}, a2 = {a[4], a[5], a[6], a[7]};
+      dot[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a1), b1, dot[t], 0, 0, 0);
+      dot[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a2), b2, dot[t], 0, 0, 0);
+    }
+    xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones), b1, xs, 0, 0, 0);
+    xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones), b2, xs, 0, 0, 0);
+    if constexpr (s % SPG == SPG - 1) {
+      constexpr int g = s / SPG;
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          // the scale of (weight row quarter*4 + r, group g) sits in lane (quarter*4 + r) + 16*g of its register
+          const int h = quarter * 4 + r + 16 * g;
+          const float scale = __shfl(sc_cur[t][(16 * g) / 64], h & 63, 64);
+          acc[t][r] = fmaf(scale, fmaf(-128.0f, xs[r], dot[t][r]), acc[t][r]);
+          dot[t][r] = 0.0f;
+        }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) xs[r] = 0.0f;
+    }
+    (void)pass;
+  };
+
+  load_scales(sc_cur, 0);
+  static_for<D>([&](auto u) { issue(u, decltype(u)::value); });
+  for (int pass = 0; pass < passes; ++pass) {
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+      acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      dot[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (pass + 1 < passes) load_scales(sc_nxt, pass + 1);
+    static_for<S>([&](auto cs) {
+      constexpr int s = decltype(cs)::value;
+      consume(std::integral_constant<int, s % D>{}, cs, pass);
+      issue(std::integral_constant<int, s % D>{}, pass * S + s + D);
+    });
+    // Sum the K slices through LDS.  Accumulator register r of lane l is output
+    // (weight row quarter*4 + r, activation row l % 16) of its 16x16 tile.
+    float (*mine)[TILES][16 * 16] = red[pass & 1];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mine[wave][t][(quarter * 4 + r) * 16 + row] = acc[t][r];
+    __syncthreads();
+    if (wave < TILES) {  // wavefront t finishes tile t
+      const int t = wave;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float total_sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) total_sum += mine[w][t][(quarter * 4 + r) * 16 + row];
+        const int64_t n = wg_row0 + (pass * TILES + t) * 16 + quarter * 4 + r;
+        if (row < p.m && n < p.n)
+          p.y[static_cast<int64_t>(row) * p.ldy + n] = static_cast<uint16_t>(bf16_bits_rne(total_sum));
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int i = 0; i < NSC; ++i) sc_cur[t][i] = sc_nxt[t][i];
+  }
+}
+
 }  // namespace vecops_hip
 #endif
