@@ -30,9 +30,9 @@ PEAK_HBM_GBPS = 8000.0
 # profiles/ (KiB per dispatch x 1024, FETCH scaled by 2.000 and WRITE by 1.000: what the
 # same counters read for a 1 GiB device copy, `--only copy`).  Counters cannot be read
 # from inside this process, so these are the recorded figures for exactly these workloads.
-TRAFFIC_BF16_4096 = int((101935 * 2.000 + 45568 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT = int((110595 * 2.000 + 124570 * 1.000) * 1024)
-TRAFFIC_GEMV_M1 = int((29702.9 * 2.000 + 56.0 * 1.000) * 1024)
+TRAFFIC_BF16_4096 = int((102033 * 2.000 + 47616 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT = int((103713 * 2.000 + 112200 * 1.000) * 1024)
+TRAFFIC_GEMV_M1 = int((29683.3 * 2.000 + 56.0 * 1.000) * 1024)
 
 
 def _device_tensors_bf16_gemm(dev):
@@ -128,7 +128,9 @@ def bench_gemv(dev, steps, warmup, m=1):
             "us_per_step": wall_ms * 1e3, "dtype": "int8 x bf16 -> f32",
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                          "frac": gbps / PEAK_HBM_GBPS, "traffic": TRAFFIC_GEMV_M1 if m == 1 else None,
-                         "kernel": "vecops_hip::skinny_w8a16_kernel", "algorithmic_bytes_per_launch": nbytes}}
+                         "kernel": "vecops_hip::skinny_w8a16_kernel" if m == 1 else
+                                   "vecops_hip::skinny_w8a16_mfma_resident_kernel",
+                         "algorithmic_bytes_per_launch": nbytes}}
 
 
 def bench_copy(dev, steps, warmup):
@@ -188,6 +190,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", choices=["bf16", "int8", "gemv", "copy"], help="run a single workload (for profiling)")
+    ap.add_argument("--gemv-m", type=int, default=1, help="activation rows of the --only gemv workload (1..16)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the matmul path is built and measured on a single MI355X "
@@ -210,7 +213,7 @@ def main() -> int:
         print(json.dumps(bench_copy(dev, args.steps, args.warmup)))
         return 0
     if args.only == "gemv":
-        print(json.dumps(bench_gemv(dev, args.steps, args.warmup)))
+        print(json.dumps(bench_gemv(dev, args.steps, args.warmup, m=args.gemv_m)))
         return 0
 
     main_res = bench_bf16_gemm(dev, args.steps, args.warmup)
