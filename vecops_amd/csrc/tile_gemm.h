@@ -49,7 +49,10 @@ enum OutKind : int { OUT_F32 = 0, OUT_BF16 = 1, OUT_I32 = 2 };
 enum LoadKind : int {
   LOAD_KVEC = 0,     // K contiguous, rows and base 16-byte aligned: one 16-byte load per chunk
   LOAD_GENERIC = 1,  // any strides / alignment: one load per element
-  LOAD_NVEC = 2      // spatial index contiguous (B given as [K,N] row-major), 16-byte aligned rows
+  LOAD_NVEC = 2,     // spatial index contiguous (B given as [K,N] row-major), 16-byte aligned rows:
+                     // transposed in registers on the way into LDS (32-bit compute elements)
+  LOAD_NTR = 3       // the same operand layout for 16-bit compute elements: stored in LDS as it
+                     // lies in memory ([k][n]) and transposed by the LDS read (ds_read_b64_tr_b16)
 };
 
 struct TileGemmParams {
@@ -447,33 +450,41 @@ struct Stager {
   }
 };
 
-// LOAD_NVEC: the operand is stored with its spatial index contiguous (B handed
-// over as [K,N] row-major).  The tile is cut into units of 8(k) x 4(n)
-// elements; a thread owns UNITS of them (its parts).  For a unit it loads eight
-// 8-byte rows along n, transposes them in registers with byte permutes and
-// writes four K-contiguous 16-byte chunks.  Consecutive threads take consecutive
-// n, so a wavefront's load covers 512 contiguous bytes of one k row.  16-bit
-// compute elements only (bf16, or fp32 rounded to bf16 on load).
+// LOAD_NTR: the operand is stored with its spatial index contiguous (B handed over
+// as [K,N] row-major) and goes into LDS untransposed: row k of the K tile holds the
+// tile's ROWS spatial positions, kPitch bytes apart.  Thread t stages 16-byte chunk
+// idx % (ROWS/8) of k row idx / (ROWS/8), idx = t + THREADS * i; part i is that one
+// chunk, exactly like the K-contiguous stager.  16-bit compute elements (bf16, or
+// fp32 rounded to bf16 on load).  The matching fragment read is ds_read_b64_tr_b16:
+// within 16 lanes, lane s supplies the address of four consecutive n of row
+// k0 + s/4 at column n0 + 4*(s%4), and lane j receives column n0 + j of rows
+// k0 .. k0+3 - four consecutive k of one spatial position, half an MFMA operand.
+// The pitch is 64 bytes more than a row so that the four rows of such a read fall
+// into different bank groups.
 template <int SRC, int ROWS, int THREADS>
-struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
+struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
   using T = SrcTraits<SRC>;
-  static_assert(T::kElemsPerChunk == 8, "transposing stager handles 16-bit compute elements");
-  static constexpr int UNITS_TOTAL = 2 * ROWS;  // (ROWS / 4) along n  x  8 along k
-  static constexpr int UNITS = (UNITS_TOTAL + THREADS - 1) / THREADS;
-  static constexpr bool kAllActive = UNITS_TOTAL % THREADS == 0;  // else the last unit of some threads is idle
-  static constexpr int kParts = UNITS;
-  static constexpr int kStoreOps = 4;  // schedulable operations per part: four LDS writes
-  static constexpr int kLoadOps = 8;   // (each with its permutes), eight row loads
+  static_assert(T::kElemsPerChunk == 8, "transposing LDS reads handle 16-bit compute elements");
+  static constexpr int kPitch = ROWS * 2 + 64;
+  static constexpr int CHUNKS_PER_ROW = ROWS / 8;
+  static constexpr int CHUNKS = 64 * CHUNKS_PER_ROW / THREADS;
+  static_assert(CHUNKS >= 1 && 64 * CHUNKS_PER_ROW % THREADS == 0, "whole chunks per thread");
+  static constexpr int kParts = CHUNKS;
+  static constexpr int kStoreOps = 1;
+  static constexpr int kLoadOps = 1;
+  static constexpr bool kHasSpare = true;
   const char* base;
   const VECOPS_GLOBAL char* tile_base;  // (k = 0, first n of the tile), wavefront-uniform
-  uint32_t unit_bytes[UNITS];  // byte offset of (first k of the unit, its first n) from tile_base
-  int64_t rs, ks;              // rs == 1; ks = elements between consecutive k
-  int first_row, extent, k_end;
-  int n_local[UNITS], kb[UNITS];
-  int tid_;
-  uint32_t regs[UNITS][8][2];
+  uint32_t chunk_bytes[CHUNKS];  // byte offset of (k row, first n of the chunk) from tile_base
+  int64_t rs, ks;                // rs == 1; ks = elements between consecutive k
+  int first_row, extent, k_end, tid_;
+  u32x4 regs[CHUNKS];
+  struct Spare {
+    u32x4 regs[CHUNKS];
+  };
 
-  __device__ __forceinline__ bool active(int u) const { return kAllActive || u * THREADS + tid_ < UNITS_TOTAL; }
+  __device__ __forceinline__ static int k_row(int part, int tid) { return (part * THREADS + tid) / CHUNKS_PER_ROW; }
+  __device__ __forceinline__ static int chunk(int part, int tid) { return (part * THREADS + tid) % CHUNKS_PER_ROW; }
 
   __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
                                        int k_end_, int tid, uint32_t /*flip*/) {
@@ -486,116 +497,71 @@ struct Stager<SRC, LOAD_NVEC, ROWS, THREADS> {
     tid_ = tid;
     tile_base = (const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * T::kSrcBytes);
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-      const int unit = u * THREADS + tid;
-      n_local[u] = (unit % (ROWS / 4)) * 4;
-      kb[u] = (unit / (ROWS / 4)) & 7;
-      // extent is a multiple of 8 on this path: clamp whole 8-column blocks, keep the offset inside the block
-      const int n = min(first_row + n_local[u], extent - 8 + (n_local[u] & 4)) - first_row;
+    for (int i = 0; i < CHUNKS; ++i) {
+      // extent is a multiple of 8 on this path: a chunk past it is clamped onto the last one
+      const int n = min(first_row + chunk(i, tid) * 8, extent - 8) - first_row;
       // the launcher admits this path only when a K tile's 64 rows span less than 4 GiB
-      unit_bytes[u] = static_cast<uint32_t>((static_cast<int64_t>(kb[u]) * 8 * ks + n) * T::kSrcBytes);
+      chunk_bytes[i] = static_cast<uint32_t>((static_cast<int64_t>(k_row(i, tid)) * ks + n) * T::kSrcBytes);
     }
   }
 
-  // row R (k = 8*kb + R) of unit PART
-  template <int PART, int R>
-  __device__ __forceinline__ void load_op(int kt) {
-    if (!active(PART)) return;
-    const VECOPS_GLOBAL char* row = tile_base + (static_cast<int64_t>(kt) * 64 + R) * ks * T::kSrcBytes;
-    const VECOPS_GLOBAL char* src = uniform_ptr(row) + unit_bytes[PART];
-    if constexpr (SRC == SRC_F32_AS_BF16) {
-      const f32x4 v = *(const VECOPS_GLOBAL f32x4*)(src);
-      regs[PART][R][0] = cvt_pk_bf16(v.x, v.y);
-      regs[PART][R][1] = cvt_pk_bf16(v.z, v.w);
-    } else {
-      const u32x2 v = *(const VECOPS_GLOBAL u32x2*)(src);
-      regs[PART][R][0] = v.x;
-      regs[PART][R][1] = v.y;
-    }
+  __device__ __forceinline__ const VECOPS_GLOBAL char* k_tile_base(int kt) const {
+    return uniform_ptr(tile_base + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes);
   }
-
   template <int PART>
   __device__ __forceinline__ void fetch_part(int kt) {
-    static_for<8>([&](auto cr) { load_op<PART, decltype(cr)::value>(kt); });
+    regs[PART] = load_chunk_fast<SRC>(k_tile_base(kt), chunk_bytes[PART]);
   }
-
   __device__ __forceinline__ void fetch_full(int kt) {
-    static_for<UNITS>([&](auto cu) { fetch_part<decltype(cu)::value>(kt); });
+    static_for<CHUNKS>([&](auto ci) { fetch_part<decltype(ci)::value>(kt); });
   }
-
-  // second register set for the start of the pipeline (see the chunk stager)
-  struct Spare {
-    uint32_t regs[UNITS][8][2];
-  };
   __device__ __forceinline__ void fetch_full_spare(Spare& spare, int kt) {
-    Stager tmp = *this;  // addresses only: its registers are overwritten before any use
-    tmp.fetch_full(kt);
+    const VECOPS_GLOBAL char* k_base = k_tile_base(kt);
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u)
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        spare.regs[u][r][0] = tmp.regs[u][r][0];
-        spare.regs[u][r][1] = tmp.regs[u][r][1];
-      }
+    for (int i = 0; i < CHUNKS; ++i) spare.regs[i] = load_chunk_fast<SRC>(k_base, chunk_bytes[i]);
   }
   __device__ __forceinline__ void take_spare(const Spare& spare) {
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u)
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        regs[u][r][0] = spare.regs[u][r][0];
-        regs[u][r][1] = spare.regs[u][r][1];
-      }
+    for (int i = 0; i < CHUNKS; ++i) regs[i] = spare.regs[i];
   }
-  static constexpr bool kHasSpare = true;
 
   // Whole tile with bounds checks (the partial last K tile): rows k >= K read as
   // zero, columns n >= N as zero.
   __device__ __forceinline__ void fetch_checked(int kt) {
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-      if (!active(u)) continue;
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int k = kt * 64 + k_row(i, tid_);
+      uint32_t w[4] = {0u, 0u, 0u, 0u};
+      if (k < k_end) {
 #pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const int k = kt * 64 + kb[u] * 8 + r;
-        regs[u][r][0] = 0u;
-        regs[u][r][1] = 0u;
-        if (k < k_end) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int n = first_row + n_local[u] + e;
-            if (n < extent) {
-              uint32_t v;
-              if constexpr (SRC == SRC_BF16) v = reinterpret_cast<const uint16_t*>(base)[k * ks + n];
-              else v = cvt_pk_bf16(reinterpret_cast<const float*>(base)[k * ks + n], 0.0f) & 0xffffu;
-              regs[u][r][e >> 1] |= v << ((e & 1) * 16);
-            }
+        for (int e = 0; e < 8; ++e) {
+          const int n = first_row + chunk(i, tid_) * 8 + e;
+          if (n < extent) {
+            uint32_t v;
+            if constexpr (SRC == SRC_BF16) v = reinterpret_cast<const uint16_t*>(base)[k * ks + n];
+            else v = cvt_pk_bf16(reinterpret_cast<const float*>(base)[k * ks + n], 0.0f) & 0xffffu;
+            w[e >> 1] |= v << ((e & 1) * 16);
           }
         }
       }
+      regs[i] = u32x4{w[0], w[1], w[2], w[3]};
     }
-  }
-
-  // output chunk for n-row E of unit PART: dword j = (regs[2j][E], regs[2j+1][E])
-  template <int PART, int E>
-  __device__ __forceinline__ void store_op(char* lds_tile) const {
-    if (!active(PART)) return;
-    constexpr uint32_t sel = (E & 1) ? 0x07060302u : 0x05040100u;
-    u32x4 out;
-    out.x = __builtin_amdgcn_perm(regs[PART][1][E >> 1], regs[PART][0][E >> 1], sel);
-    out.y = __builtin_amdgcn_perm(regs[PART][3][E >> 1], regs[PART][2][E >> 1], sel);
-    out.z = __builtin_amdgcn_perm(regs[PART][5][E >> 1], regs[PART][4][E >> 1], sel);
-    out.w = __builtin_amdgcn_perm(regs[PART][7][E >> 1], regs[PART][6][E >> 1], sel);
-    *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(n_local[PART] + E, kb[PART])) = out;
   }
 
   template <int PART>
   __device__ __forceinline__ void commit_part(char* lds_tile) const {
-    static_for<4>([&](auto ce) { store_op<PART, decltype(ce)::value>(lds_tile); });
+    *reinterpret_cast<u32x4*>(lds_tile + k_row(PART, tid_) * kPitch + chunk(PART, tid_) * 16) = regs[PART];
   }
-
   __device__ __forceinline__ void commit(char* lds_tile) const {
-    static_for<UNITS>([&](auto cu) { commit_part<decltype(cu)::value>(lds_tile); });
+    static_for<CHUNKS>([&](auto ci) { commit_part<decltype(ci)::value>(lds_tile); });
+  }
+  template <int PART, int OP>
+  __device__ __forceinline__ void store_op(char* lds_tile) const {
+    commit_part<PART>(lds_tile);
+  }
+  template <int PART, int OP>
+  __device__ __forceinline__ void load_op(int kt) {
+    fetch_part<PART>(kt);
   }
 };
 
@@ -750,11 +716,19 @@ struct StagingSchedule {
   }
 };
 
+// Bytes of one LDS stage: the A tile (rows x 128) and the B tile, which in its
+// untransposed form is 64 k rows of (columns x 2 + 64) bytes.
+template <int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_B>
+constexpr int kStageBytes() {
+  const int bm = 32 * WAVES_M * WM, bn = 32 * WAVES_N * WN;
+  return bm * 128 + (LOAD_B == LOAD_NTR ? 64 * (bn * 2 + 64) : bn * 128);
+}
+
 // Dynamic LDS one workgroup is launched with: two staging stages, or the bf16
 // epilogue's row-major tiles if those are larger.
-template <int WAVES_M, int WAVES_N, int WM, int WN>
+template <int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_B>
 constexpr int kTileLdsBytes() {
-  const int stages = 2 * 32 * (WAVES_M * WM + WAVES_N * WN) * 128;
+  const int stages = 2 * kStageBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>();
   const int epilogue = (WN * 32 * 2 + 16) * (WM * 32) * WAVES_M * WAVES_N;
   return stages > epilogue ? stages : epilogue;
 }
@@ -772,7 +746,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   constexpr int KTILE = 8 * EPC;  // elements per K tile
   constexpr int THREADS = 64 * WAVES_M * WAVES_N;
   constexpr int BM = 32 * WAVES_M * WM, BN = 32 * WAVES_N * WN;
-  constexpr int STAGE_BYTES = (BM + BN) * 128;
+  constexpr int STAGE_BYTES = kStageBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>();
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -808,7 +782,17 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
 #pragma unroll
   for (int i = 0; i < WM; ++i) off_a[i] = lds_chunk_offset((wm * WM + i) * 32 + frag_row, frag_half);
 #pragma unroll
-  for (int j = 0; j < WN; ++j) off_b[j] = BM * 128 + lds_chunk_offset((wn * WN + j) * 32 + frag_row, frag_half);
+  for (int j = 0; j < WN; ++j) {
+    if constexpr (LOAD_B == LOAD_NTR) {
+      // transposing read: 16-lane group g = lane / 16 serves columns (g & 1) * 16 .. + 15 of the fragment and
+      // the k half g / 2; lane s of the group addresses row s / 4, columns 4 * (s % 4) .. + 3
+      constexpr int PITCH_B = Stager<SRC, LOAD_NTR, BN, THREADS>::kPitch;
+      const int s = lane & 15, g = lane >> 4;
+      off_b[j] = BM * 128 + ((g >> 1) * 8 + (s >> 2)) * PITCH_B + ((wn * WN + j) * 32 + (g & 1) * 16 + (s & 3) * 4) * 2;
+    } else {
+      off_b[j] = BM * 128 + lds_chunk_offset((wn * WN + j) * 32 + frag_row, frag_half);
+    }
+  }
 
   // The K tiles of this workgroup are walked as a sequence seq(0..nk-1): a partial
   // last tile of K (if this split owns it) comes FIRST, so that only the prologue
@@ -839,7 +823,20 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   auto read_frag = [&](int set, const char* tile, int ks, auto r_tag) {
     constexpr int r = decltype(r_tag)::value;
     if constexpr (r == 0) fa[set][0] = *reinterpret_cast<const u32x4*>(tile + (off_a[0] ^ (ks << 5)));
-    else if constexpr (r <= WN) fb[set][r - 1] = *reinterpret_cast<const u32x4*>(tile + (off_b[r - 1] ^ (ks << 5)));
+    else if constexpr (r <= WN) {
+      if constexpr (LOAD_B == LOAD_NTR) {
+        // k-step ks covers rows 16*ks .. 16*ks+15 of the tile; the two reads give k 0-3 and 4-7 of the lane's half
+        constexpr int PITCH_B = Stager<SRC, LOAD_NTR, BN, THREADS>::kPitch;
+        typedef __attribute__((ext_vector_type(4))) short s16x4;
+        typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+        const char* at = tile + off_b[r - 1] + ks * 16 * PITCH_B;
+        const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at)));
+        const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * PITCH_B)));
+        fb[set][r - 1] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      } else {
+        fb[set][r - 1] = *reinterpret_cast<const u32x4*>(tile + (off_b[r - 1] ^ (ks << 5)));
+      }
+    }
     else fa[set][r - WN] = *reinterpret_cast<const u32x4*>(tile + (off_a[r - WN] ^ (ks << 5)));
   };
   auto read_frags = [&](int set, const char* tile, int ks) {
@@ -982,7 +979,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
     // staging buffers are dead by now) and then stores whole 16-byte row segments.
     constexpr int TILE_COLS = WN * 32, TILE_ROWS = WM * 32;
     constexpr int PITCH = TILE_COLS * 2 + 16;  // bytes; the pad staggers rows across banks
-    static_assert(PITCH * TILE_ROWS * WAVES_M * WAVES_N <= kTileLdsBytes<WAVES_M, WAVES_N, WM, WN>(),
+    static_assert(PITCH * TILE_ROWS * WAVES_M * WAVES_N <= kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>(),
                   "epilogue staging must fit the launch's LDS");
     __syncthreads();  // every wavefront is done reading fragments
     char* mine = lds + wave * (PITCH * TILE_ROWS);

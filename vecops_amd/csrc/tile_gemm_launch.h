@@ -32,7 +32,7 @@ hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_
 // Shared by the per-class translation units.
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB>
 hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
-  constexpr int kLds = kTileLdsBytes<WAVES_M, WAVES_N, WM, WN>();
+  constexpr int kLds = kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LB>();
   constexpr int kThreads = 64 * WAVES_M * WAVES_N;
   auto kernel = tile_gemm_kernel<SRC, WAVES_M, WAVES_N, WM, WN, LA, LB>;
   // > 64 KiB of dynamic LDS has to be enabled once per device; cheap enough to repeat per thread.
@@ -54,7 +54,10 @@ hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN>
 hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t stream) {
   if (mode == MODE_KVEC) return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_KVEC>(p, stream);
-  if constexpr (SrcTraits<SRC>::kElemsPerChunk == 8 || SRC == SRC_F32) {
+  if constexpr (SrcTraits<SRC>::kElemsPerChunk == 8) {  // 16-bit compute: B untransposed in LDS, transposing reads
+    if (mode == MODE_NVEC_B)
+      return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_NTR>(p, stream);
+  } else if constexpr (SRC == SRC_F32) {                // 32-bit compute: transposed in registers
     if (mode == MODE_NVEC_B)
       return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_NVEC>(p, stream);
   }
