@@ -102,6 +102,14 @@ struct SrcTraits<SRC_I8> {
   static constexpr int kSrcBytes = 1;
   static constexpr bool kInt = true;
 };
+template <>
+struct SrcTraits<SRC_I8_FLIP> : SrcTraits<SRC_I8> {};
+template <>
+struct SrcTraits<SRC_F32> {
+  static constexpr int kElemsPerChunk = 4;
+  static constexpr int kSrcBytes = 4;
+  static constexpr bool kInt = false;
+};
 
 // fp32 -> bf16 bits, round to nearest even; NaN -> 0x7fc0 (vecops util/BFloat16.h:25-37).
 __device__ __forceinline__ uint32_t bf16_bits_rne(float x) {
@@ -137,7 +145,7 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
 #define VECOPS_GLOBAL __attribute__((address_space(1)))
 
 // Tells the compiler that a global pointer is the same in every lane, so that it is
-// kept in scalar registers and loads through it take the scalar-base form.
+// kept in scalar registers.
 __device__ __forceinline__ const VECOPS_GLOBAL char* uniform_ptr(const VECOPS_GLOBAL char* p) {
   const uint64_t bits = reinterpret_cast<uint64_t>(p);
   const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
@@ -145,35 +153,32 @@ __device__ __forceinline__ const VECOPS_GLOBAL char* uniform_ptr(const VECOPS_GL
   return reinterpret_cast<const VECOPS_GLOBAL char*>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
+// Buffer descriptor over [base, base + 4 GiB): loads through it take the base from
+// four scalar registers, a 32-bit per-lane byte offset and a scalar byte offset,
+// so a load costs no vector ALU work for its address.  `base` must be the same in
+// every lane.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_buffer(const VECOPS_GLOBAL char* base) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)uniform_ptr(base), 0, 0x7fffffff, 0x00020000);
+}
+
 // Fast path: one whole 16-byte chunk, no bounds checks (the caller guarantees
-// that the row exists and that the chunk lies inside K).
-
-template <>
-struct SrcTraits<SRC_I8_FLIP> : SrcTraits<SRC_I8> {};
-template <>
-struct SrcTraits<SRC_F32> {
-  static constexpr int kElemsPerChunk = 4;
-  static constexpr int kSrcBytes = 4;
-  static constexpr bool kInt = false;
-};
-
+// that the row exists and that the chunk lies inside K).  `uniform_offset` (same in
+// every lane) and `lane_offset` are byte offsets from the descriptor's base; their
+// sum stays below 2^31.
 template <int SRC>
-__device__ __forceinline__ u32x4 load_chunk_fast(const VECOPS_GLOBAL char* base, uint32_t offset) {
-  // Global address space spelled out: a generic (flat) load would also count
-  // against the LDS counter and stall the LDS-only waits of the main loop.  `base`
-  // is wavefront-uniform, `offset` per lane: the load takes its base from scalar
-  // registers and the lane holds one 32-bit offset instead of a 64-bit pointer.
+__device__ __forceinline__ u32x4 load_chunk_fast(__amdgpu_buffer_rsrc_t buffer, uint32_t lane_offset,
+                                                 uint32_t uniform_offset) {
   if constexpr (SRC == SRC_F32_AS_BF16) {
-    const VECOPS_GLOBAL f32x4* p = (const VECOPS_GLOBAL f32x4*)(base + offset);
-    const f32x4 lo = p[0], hi = p[1];
+    const u32x4 lo = __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset, uniform_offset, 0);
+    const u32x4 hi = __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset + 16, uniform_offset, 0);
     u32x4 out;
-    out.x = cvt_pk_bf16(lo.x, lo.y);
-    out.y = cvt_pk_bf16(lo.z, lo.w);
-    out.z = cvt_pk_bf16(hi.x, hi.y);
-    out.w = cvt_pk_bf16(hi.z, hi.w);
+    out.x = cvt_pk_bf16(__uint_as_float(lo.x), __uint_as_float(lo.y));
+    out.y = cvt_pk_bf16(__uint_as_float(lo.z), __uint_as_float(lo.w));
+    out.z = cvt_pk_bf16(__uint_as_float(hi.x), __uint_as_float(hi.y));
+    out.w = cvt_pk_bf16(__uint_as_float(hi.z), __uint_as_float(hi.w));
     return out;
   } else {
-    return *(const VECOPS_GLOBAL u32x4*)(base + offset);
+    return __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset, uniform_offset, 0);
   }
 }
 
@@ -349,8 +354,8 @@ struct Stager {
   static constexpr int kStoreOps = 1;  // schedulable operations per part: one LDS write,
   static constexpr int kLoadOps = 1;   // one refill (one or two load instructions)
   const char* base;
-  const VECOPS_GLOBAL char* tile_base;  // first row of the tile, k = 0 (wavefront-uniform)
-  uint32_t row_bytes[CHUNKS];  // byte offset of each staged row from tile_base, chunk included (fast path)
+  __amdgpu_buffer_rsrc_t tile_buf;  // descriptor based at the first row of the tile, k = 0 (fast path)
+  uint32_t row_bytes[CHUNKS];  // byte offset of each staged row from that base, chunk included (fast path)
   int64_t rs, ks;              // element strides (checked path)
   int first_row, extent, k_end, ld_row, ld_chunk;
   uint32_t flip;  // SRC_I8_FLIP: xor mask applied on the way into LDS
@@ -367,11 +372,11 @@ struct Stager {
     flip = flip_;
     ld_chunk = tid & 7;
     ld_row = tid >> 3;
-    tile_base = (const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * rs * T::kSrcBytes);
+    tile_buf = tile_buffer((const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * rs * T::kSrcBytes));
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int row = min(first_row + ld_row + i * ROWS_PER_PASS, extent - 1) - first_row;
-      // the launcher admits this path only when a tile's rows span less than 4 GiB
+      // the launcher admits this path only when a tile's rows plus one row's K span less than 2 GiB
       row_bytes[i] = static_cast<uint32_t>((static_cast<int64_t>(row) * rs + ld_chunk * T::kElemsPerChunk) * T::kSrcBytes);
     }
   }
@@ -381,9 +386,7 @@ struct Stager {
   template <int PART>
   __device__ __forceinline__ void fetch_part(int kt) {
     if constexpr (LOAD == LOAD_KVEC) {
-      const VECOPS_GLOBAL char* k_base =
-          uniform_ptr(tile_base + static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes));
-      regs[PART] = load_chunk_fast<SRC>(k_base, row_bytes[PART]);
+      regs[PART] = load_chunk_fast<SRC>(tile_buf, row_bytes[PART], kt * (8 * T::kElemsPerChunk * T::kSrcBytes));
     } else {
       const int k0 = kt * 8 * T::kElemsPerChunk + ld_chunk * T::kElemsPerChunk;
       const int row = first_row + ld_row + PART * ROWS_PER_PASS;
@@ -404,10 +407,9 @@ struct Stager {
   };
   __device__ __forceinline__ void fetch_full_spare(Spare& spare, int kt) {
     if constexpr (LOAD == LOAD_KVEC) {
-      const VECOPS_GLOBAL char* k_base =
-          uniform_ptr(tile_base + static_cast<int64_t>(kt) * (8 * T::kElemsPerChunk * T::kSrcBytes));
 #pragma unroll
-      for (int i = 0; i < CHUNKS; ++i) spare.regs[i] = load_chunk_fast<SRC>(k_base, row_bytes[i]);
+      for (int i = 0; i < CHUNKS; ++i)
+        spare.regs[i] = load_chunk_fast<SRC>(tile_buf, row_bytes[i], kt * (8 * T::kElemsPerChunk * T::kSrcBytes));
     }
   }
   __device__ __forceinline__ void take_spare(const Spare& spare) {
@@ -495,30 +497,31 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
     extent = extent_;
     k_end = k_end_;
     tid_ = tid;
-    tile_base = (const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * T::kSrcBytes);
+    tile_base = uniform_ptr((const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * T::kSrcBytes));
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       // extent is a multiple of 8 on this path: a chunk past it is clamped onto the last one
       const int n = min(first_row + chunk(i, tid) * 8, extent - 8) - first_row;
-      // the launcher admits this path only when a K tile's 64 rows span less than 4 GiB
+      // the launcher admits this path only when a K tile's 64 rows span less than 2 GiB
       chunk_bytes[i] = static_cast<uint32_t>((static_cast<int64_t>(k_row(i, tid)) * ks + n) * T::kSrcBytes);
     }
   }
 
-  __device__ __forceinline__ const VECOPS_GLOBAL char* k_tile_base(int kt) const {
-    return uniform_ptr(tile_base + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes);
+  // descriptor based at row 0 of K tile kt (scalar arithmetic: every term is wavefront-uniform)
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t k_tile_buffer(int kt) const {
+    return tile_buffer(tile_base + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes);
   }
   template <int PART>
   __device__ __forceinline__ void fetch_part(int kt) {
-    regs[PART] = load_chunk_fast<SRC>(k_tile_base(kt), chunk_bytes[PART]);
+    regs[PART] = load_chunk_fast<SRC>(k_tile_buffer(kt), chunk_bytes[PART], 0u);
   }
   __device__ __forceinline__ void fetch_full(int kt) {
     static_for<CHUNKS>([&](auto ci) { fetch_part<decltype(ci)::value>(kt); });
   }
   __device__ __forceinline__ void fetch_full_spare(Spare& spare, int kt) {
-    const VECOPS_GLOBAL char* k_base = k_tile_base(kt);
+    const __amdgpu_buffer_rsrc_t k_buf = k_tile_buffer(kt);
 #pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) spare.regs[i] = load_chunk_fast<SRC>(k_base, chunk_bytes[i]);
+    for (int i = 0; i < CHUNKS; ++i) spare.regs[i] = load_chunk_fast<SRC>(k_buf, chunk_bytes[i], 0u);
   }
   __device__ __forceinline__ void take_spare(const Spare& spare) {
 #pragma unroll
