@@ -57,7 +57,7 @@ typedef enum VecopsHipKernelFamily {
   VECOPS_HIP_FAMILY_TILE_256 = 1,      /* 256x256 workgroup tile, MFMA */
   VECOPS_HIP_FAMILY_TILE_128 = 2,      /* 128x128 workgroup tile, MFMA */
   VECOPS_HIP_FAMILY_TILE_64 = 3,       /* 64x64 workgroup tile, MFMA */
-  VECOPS_HIP_FAMILY_SKINNY = 4,        /* wavefront split-K dot products */
+  VECOPS_HIP_FAMILY_SKINNY = 4,        /* one side <= 16 rows: wavefronts split K, the wide operand is read once */
   VECOPS_HIP_FAMILY_ZERO_K = 5         /* K == 0: C = Cin or zeros */
 } VecopsHipKernelFamily;
 

@@ -272,6 +272,49 @@ def test_invalid_arguments_are_rejected(device):
     assert e.value.code == 2
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 14336, 4096), (16, 14336, 4096), (4, 4096, 11008), (3, 1000, 520),
+                                   (2048, 7, 264), (5, 513, 64), (16, 600, 8200)])
+def test_skinny_bf16_family(device, oracle, m, n, k):
+    """One side at most 16 rows, the other long (the small-vector shapes of
+    matmul/details/kernel/RuntimeDispatch.h:24-83): the skinny kernel, fp32 and bf16 outputs."""
+    import torch
+    from vecops_amd import capi
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    ta, tb = dev_bf16(a, device), dev_bf16(b, device)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    assert capi.FAMILY_NAMES[capi.plan_matmul(ta, tb, c).family] == "skinny"
+    capi.matmul(ta, tb, c)
+    c16 = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    capi.matmul(ta, tb, c16)
+    torch.cuda.synchronize()
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, acc_f64=True)
+    got = c.cpu().numpy()
+    assert rel_err(got, want) <= fp32_tol(k)
+    assert np.array_equal(host_bits(c16), oracle.bf16_from_f32(got))
+
+
+def test_skinny_bf16_batched_strided(device, oracle):
+    """Rank-3 batch with a broadcast narrow operand, padded rows of the wide operand and a
+    transposed (column-major) output."""
+    import torch
+    from vecops_amd import capi
+    batch, m, n, k = 3, 6, 1100, 776
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b_pad = synth.bf16_round(synth.uniform_pm1(2, (batch, n, k + 24)))
+    tb = dev_bf16(b_pad, device)[:, :, :k]                              # row stride k + 24
+    ta = dev_bf16(a, device)[None].expand(batch, m, k)                  # stride-0 batch
+    c_t = torch.full((batch, n, m), float("nan"), dtype=torch.float32, device=device)
+    c = c_t.transpose(1, 2)                                             # [batch, m, n] view, n stride m
+    assert capi.FAMILY_NAMES[capi.plan_matmul(ta, tb, c).family] == "skinny"
+    capi.matmul(ta, tb, c)
+    torch.cuda.synchronize()
+    want = np.zeros((batch, m, n), np.float32)
+    oracle.matmul(np.broadcast_to(a, (batch, m, k)), b_pad[:, :, :k], want, acc_f64=True)
+    assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+
+
 # --- int8 -------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("m,n,k", [(19, 21, 69), (1, 128, 65), (128, 1, 65), (1, 16, 129), (35, 53, 257),

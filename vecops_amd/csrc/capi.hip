@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstring>
 
+#include "skinny_dense.h"
 #include "skinny_w8a16.h"
 #include "tile_gemm_launch.h"
 #include "vecops_hip.h"
@@ -159,6 +160,14 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
 
 constexpr int kComputeUnits = 256;
 
+// bf16 x bf16 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
+bool skinny_applies(const Problem& pr) {
+  if (pr.src != SRC_BF16 || pr.has_cin) return false;
+  if (!k_vector_ok(pr.a) || !k_vector_ok(pr.b) || pr.k % 8 != 0 || pr.k < 64) return false;
+  const int64_t narrow = pr.m < pr.n ? pr.m : pr.n, wide = pr.m < pr.n ? pr.n : pr.m;
+  return narrow <= 16 && wide >= 512 && pr.batch <= 65535;
+}
+
 // elements of K in one 128-byte K tile of the compute type
 int k_tile_elements(int src) { return src == SRC_I8 || src == SRC_I8_FLIP ? 128 : src == SRC_F32 ? 32 : 64; }
 
@@ -183,6 +192,14 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
   plan->vector_a = k_vector_ok(pr.a) ? 1 : 0;
   plan->vector_b = (k_vector_ok(pr.b) || (pr.b.rs == 1 && pr.b.cs != 1 && n_vector_ok(pr.b) && dtype_bytes(pr.b.dtype) != 1)) ? 1 : 0;
   plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
+
+  // Skinny family: one operand has at most 16 rows and the other is long - the GPU reading of
+  // vecops' small-vector shapes (runtime_dispatch_rules::skinny_at_most / large_m1 / large_n1,
+  // matmul/details/kernel/RuntimeDispatch.h:24-83): HBM-bound, the wide operand is read once.
+  if (skinny_applies(pr)) {
+    plan->family = VECOPS_HIP_FAMILY_SKINNY;
+    return;
+  }
 
   auto tiles = [&](int64_t t) { return ((pr.m + t - 1) / t) * ((pr.n + t - 1) / t) * pr.batch; };
   uint32_t family;
@@ -254,6 +271,43 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     p.split_k = 0;  // empty sum: the reduce kernel emits epilogue(0)
     hipError_t e = launch_splitk_reduce(p, is_int, stream);
     if (e != hipSuccess) return fail(ST_EXEC, "zero-K kernel launch: %s", hipGetErrorString(e));
+    return ST_OK;
+  }
+
+  if (plan.family == VECOPS_HIP_FAMILY_SKINNY) {
+    const bool a_narrow = pr.m < pr.n;  // else b is the narrow side
+    const View& wide = a_narrow ? pr.b : pr.a;
+    const View& narrow = a_narrow ? pr.a : pr.b;
+    SkinnyDenseParams q;
+    q.w = static_cast<const uint16_t*>(wide.data);
+    q.x = static_cast<const uint16_t*>(narrow.data);
+    q.y = pr.c.data;
+    q.ldw = wide.rs;
+    q.ldx = narrow.rs;
+    q.w_bs = wide.bs;
+    q.x_bs = narrow.bs;
+    q.y_bs = pr.c.bs;
+    q.y_stride_r = a_narrow ? pr.c.cs : pr.c.rs;
+    q.y_stride_s = a_narrow ? pr.c.rs : pr.c.cs;
+    q.rows = static_cast<int32_t>(wide.rows);
+    q.s = static_cast<int32_t>(narrow.rows);
+    q.k = static_cast<int32_t>(pr.k);
+    q.out_bf16 = pr.out_kind == OUT_BF16 ? 1 : 0;
+    // 64 wide rows per workgroup when that still leaves most compute units a workgroup, else 32 or 16
+    const int64_t wgs64 = (wide.rows + 63) / 64 * pr.batch;
+    const dim3 block(512);
+    if (wgs64 >= 200) {
+      hipLaunchKernelGGL((skinny_dense_kernel<2, 2>), dim3(static_cast<unsigned>((wide.rows + 63) / 64), p.batch), block, 0,
+                         stream, q);
+    } else if (wgs64 * 2 >= 200) {
+      hipLaunchKernelGGL((skinny_dense_kernel<1, 2>), dim3(static_cast<unsigned>((wide.rows + 31) / 32), p.batch), block, 0,
+                         stream, q);
+    } else {
+      hipLaunchKernelGGL((skinny_dense_kernel<1, 1>), dim3(static_cast<unsigned>((wide.rows + 15) / 16), p.batch), block, 0,
+                         stream, q);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(ST_EXEC, "skinny kernel launch: %s", hipGetErrorString(e));
     return ST_OK;
   }
 
