@@ -161,55 +161,82 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_buffer(const VECOPS_GLOBA
   return __builtin_amdgcn_make_buffer_rsrc((void*)uniform_ptr(base), 0, 0x7fffffff, 0x00020000);
 }
 
-// Fast path: one whole 16-byte chunk, no bounds checks (the caller guarantees
-// that the row exists and that the chunk lies inside K).  `uniform_offset` (same in
-// every lane) and `lane_offset` are byte offsets from the descriptor's base; their
-// sum stays below 2^31.
+// What the staging registers hold for one 16-byte chunk of compute elements between
+// its global load and its LDS store.  fp32 operands that are multiplied as bf16 are
+// held as loaded (32 bytes) and rounded only when they are stored: a conversion right
+// behind the load would wait for the load and expose the memory latency of every chunk.
 template <int SRC>
-__device__ __forceinline__ u32x4 load_chunk_fast(__amdgpu_buffer_rsrc_t buffer, uint32_t lane_offset,
-                                                 uint32_t uniform_offset) {
-  if constexpr (SRC == SRC_F32_AS_BF16) {
-    const u32x4 lo = __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset, uniform_offset, 0);
-    const u32x4 hi = __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset + 16, uniform_offset, 0);
+struct Staged {
+  u32x4 v;
+  __device__ __forceinline__ u32x4 chunk() const { return v; }
+};
+template <>
+struct Staged<SRC_F32_AS_BF16> {
+  u32x4 lo, hi;  // eight fp32 values
+  __device__ __forceinline__ u32x4 chunk() const {
     u32x4 out;
     out.x = cvt_pk_bf16(__uint_as_float(lo.x), __uint_as_float(lo.y));
     out.y = cvt_pk_bf16(__uint_as_float(lo.z), __uint_as_float(lo.w));
     out.z = cvt_pk_bf16(__uint_as_float(hi.x), __uint_as_float(hi.y));
     out.w = cvt_pk_bf16(__uint_as_float(hi.z), __uint_as_float(hi.w));
     return out;
+  }
+};
+
+// Fast path: one whole 16-byte chunk, no bounds checks (the caller guarantees
+// that the row exists and that the chunk lies inside K).  `uniform_offset` (same in
+// every lane) and `lane_offset` are byte offsets from the descriptor's base; their
+// sum stays below 2^31.
+template <int SRC>
+__device__ __forceinline__ Staged<SRC> load_chunk_fast(__amdgpu_buffer_rsrc_t buffer, uint32_t lane_offset,
+                                                       uint32_t uniform_offset) {
+  if constexpr (SRC == SRC_F32_AS_BF16) {
+    Staged<SRC> out;
+    out.lo = __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset, uniform_offset, 0);
+    out.hi = __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset + 16, uniform_offset, 0);
+    return out;
   } else {
-    return __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset, uniform_offset, 0);
+    return Staged<SRC>{__builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset, uniform_offset, 0)};
   }
 }
 
 // Slow path: element by element with bounds checks and arbitrary K stride; used
 // for the K tail of the vector path and for every chunk of the generic path.
 template <int SRC>
-__device__ __noinline__ u32x4 load_chunk_checked(const void* base, int64_t row_off, int64_t kstep, int k0, int k_end,
-                                                 bool row_ok, uint32_t pad) {
+__device__ __noinline__ Staged<SRC> load_chunk_checked(const void* base, int64_t row_off, int64_t kstep, int k0,
+                                                       int k_end, bool row_ok, uint32_t pad) {
   // `pad` is what an element outside the operand reads as: 0, or for an operand
   // that is xor-flipped on its way into LDS the flip byte, so that it ends up 0
   constexpr int EPC = SrcTraits<SRC>::kElemsPerChunk;
-  uint32_t w0 = 0u, w1 = 0u, w2 = 0u, w3 = 0u;
+  if constexpr (SRC == SRC_F32_AS_BF16) {
+    uint32_t w[8];
 #pragma unroll
-  for (int e = 0; e < EPC; ++e) {
-    const int k = k0 + e;
-    uint32_t v = pad;
-    if (row_ok && k < k_end) {
-      if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
-      else if constexpr (SRC == SRC_F32_AS_BF16) v = cvt_pk_bf16(static_cast<const float*>(base)[row_off + k * kstep], 0.0f) & 0xffffu;
-      else if constexpr (SRC == SRC_F32) v = __float_as_uint(static_cast<const float*>(base)[row_off + k * kstep]);
-      else v = static_cast<const uint8_t*>(base)[row_off + k * kstep];
+    for (int e = 0; e < 8; ++e) {
+      const int k = k0 + e;
+      w[e] = (row_ok && k < k_end) ? __float_as_uint(static_cast<const float*>(base)[row_off + k * kstep]) : 0u;
     }
-    constexpr int per_word = EPC / 4;
-    const uint32_t shifted = v << ((e % per_word) * (32 / per_word));
-    const int word = e / per_word;
-    if (word == 0) w0 |= shifted;
-    else if (word == 1) w1 |= shifted;
-    else if (word == 2) w2 |= shifted;
-    else w3 |= shifted;
+    return Staged<SRC>{u32x4{w[0], w[1], w[2], w[3]}, u32x4{w[4], w[5], w[6], w[7]}};
+  } else {
+    uint32_t w0 = 0u, w1 = 0u, w2 = 0u, w3 = 0u;
+#pragma unroll
+    for (int e = 0; e < EPC; ++e) {
+      const int k = k0 + e;
+      uint32_t v = pad;
+      if (row_ok && k < k_end) {
+        if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
+        else if constexpr (SRC == SRC_F32) v = __float_as_uint(static_cast<const float*>(base)[row_off + k * kstep]);
+        else v = static_cast<const uint8_t*>(base)[row_off + k * kstep];
+      }
+      constexpr int per_word = EPC / 4;
+      const uint32_t shifted = v << ((e % per_word) * (32 / per_word));
+      const int word = e / per_word;
+      if (word == 0) w0 |= shifted;
+      else if (word == 1) w1 |= shifted;
+      else if (word == 2) w2 |= shifted;
+      else w3 |= shifted;
+    }
+    return Staged<SRC>{u32x4{w0, w1, w2, w3}};
   }
-  return u32x4{w0, w1, w2, w3};
 }
 
 template <int N, typename F>
@@ -353,13 +380,15 @@ struct Stager {
   static constexpr int kParts = CHUNKS;
   static constexpr int kStoreOps = 1;  // schedulable operations per part: one LDS write,
   static constexpr int kLoadOps = 1;   // one refill (one or two load instructions)
+  // a second register set for the start of the pipeline (fp32 held as loaded is twice the registers: no room)
+  static constexpr bool kHasSpare = LOAD == LOAD_KVEC && SRC != SRC_F32_AS_BF16;
   const char* base;
   __amdgpu_buffer_rsrc_t tile_buf;  // descriptor based at the first row of the tile, k = 0 (fast path)
   uint32_t row_bytes[CHUNKS];  // byte offset of each staged row from that base, chunk included (fast path)
   int64_t rs, ks;              // element strides (checked path)
   int first_row, extent, k_end, ld_row, ld_chunk;
   uint32_t flip;  // SRC_I8_FLIP: xor mask applied on the way into LDS
-  u32x4 regs[CHUNKS];
+  Staged<SRC> regs[CHUNKS];
 
   __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
                                        int k_end_, int tid, uint32_t flip_) {
@@ -403,22 +432,21 @@ struct Stager {
   // one is requested while the first is still in flight, and moved into the
   // staging registers once the first has been stored.
   struct Spare {
-    u32x4 regs[CHUNKS];
+    Staged<SRC> regs[kHasSpare ? CHUNKS : 1];
   };
   __device__ __forceinline__ void fetch_full_spare(Spare& spare, int kt) {
-    if constexpr (LOAD == LOAD_KVEC) {
+    if constexpr (kHasSpare) {
 #pragma unroll
       for (int i = 0; i < CHUNKS; ++i)
         spare.regs[i] = load_chunk_fast<SRC>(tile_buf, row_bytes[i], kt * (8 * T::kElemsPerChunk * T::kSrcBytes));
     }
   }
   __device__ __forceinline__ void take_spare(const Spare& spare) {
-    if constexpr (LOAD == LOAD_KVEC) {
+    if constexpr (kHasSpare) {
 #pragma unroll
       for (int i = 0; i < CHUNKS; ++i) regs[i] = spare.regs[i];
     }
   }
-  static constexpr bool kHasSpare = LOAD == LOAD_KVEC;
 
   // Whole tile, every element bounds-checked: the partial last K tile.
   __device__ __forceinline__ void fetch_checked(int kt) {
@@ -432,7 +460,7 @@ struct Stager {
 
   template <int PART>
   __device__ __forceinline__ void commit_part(char* lds_tile) const {
-    u32x4 v = regs[PART];
+    u32x4 v = regs[PART].chunk();
     if constexpr (SRC == SRC_I8_FLIP) v ^= u32x4{flip, flip, flip, flip};
     *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(ld_row + PART * ROWS_PER_PASS, ld_chunk)) = v;
   }
@@ -474,15 +502,17 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
   static constexpr int kParts = CHUNKS;
   static constexpr int kStoreOps = 1;
   static constexpr int kLoadOps = 1;
-  static constexpr bool kHasSpare = true;
+  static constexpr bool kHasSpare = SRC != SRC_F32_AS_BF16;
   const char* base;
   const VECOPS_GLOBAL char* tile_base;  // (k = 0, first n of the tile), wavefront-uniform
-  uint32_t chunk_bytes[CHUNKS];  // byte offset of (k row, first n of the chunk) from tile_base
+  static_assert(THREADS % CHUNKS_PER_ROW == 0, "every part of a thread is the same chunk, THREADS / CHUNKS_PER_ROW k rows on");
+  static constexpr int K_ROWS_PER_PART = THREADS / CHUNKS_PER_ROW;
+  uint32_t chunk_bytes;  // byte offset of (k row of part 0, first n of the chunk) from tile_base
   int64_t rs, ks;                // rs == 1; ks = elements between consecutive k
   int first_row, extent, k_end, tid_;
-  u32x4 regs[CHUNKS];
+  Staged<SRC> regs[CHUNKS];
   struct Spare {
-    u32x4 regs[CHUNKS];
+    Staged<SRC> regs[kHasSpare ? CHUNKS : 1];
   };
 
   __device__ __forceinline__ static int k_row(int part, int tid) { return (part * THREADS + tid) / CHUNKS_PER_ROW; }
@@ -498,13 +528,14 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
     k_end = k_end_;
     tid_ = tid;
     tile_base = uniform_ptr((const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * T::kSrcBytes));
-#pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) {
-      // extent is a multiple of 8 on this path: a chunk past it is clamped onto the last one
-      const int n = min(first_row + chunk(i, tid) * 8, extent - 8) - first_row;
-      // the launcher admits this path only when a K tile's 64 rows span less than 2 GiB
-      chunk_bytes[i] = static_cast<uint32_t>((static_cast<int64_t>(k_row(i, tid)) * ks + n) * T::kSrcBytes);
-    }
+    // extent is a multiple of 8 on this path: a chunk past it is clamped onto the last one
+    const int n = min(first_row + chunk(0, tid) * 8, extent - 8) - first_row;
+    // the launcher admits this path only when a K tile's 64 rows span less than 2 GiB
+    chunk_bytes = static_cast<uint32_t>((static_cast<int64_t>(k_row(0, tid)) * ks + n) * T::kSrcBytes);
+  }
+  // byte offset of part PART's k rows from part 0's (wavefront-uniform)
+  __device__ __forceinline__ uint32_t part_offset(int part) const {
+    return __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(part * K_ROWS_PER_PART * ks * T::kSrcBytes));
   }
 
   // descriptor based at row 0 of K tile kt (scalar arithmetic: every term is wavefront-uniform)
@@ -513,19 +544,23 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
   }
   template <int PART>
   __device__ __forceinline__ void fetch_part(int kt) {
-    regs[PART] = load_chunk_fast<SRC>(k_tile_buffer(kt), chunk_bytes[PART], 0u);
+    regs[PART] = load_chunk_fast<SRC>(k_tile_buffer(kt), chunk_bytes, part_offset(PART));
   }
   __device__ __forceinline__ void fetch_full(int kt) {
     static_for<CHUNKS>([&](auto ci) { fetch_part<decltype(ci)::value>(kt); });
   }
   __device__ __forceinline__ void fetch_full_spare(Spare& spare, int kt) {
-    const __amdgpu_buffer_rsrc_t k_buf = k_tile_buffer(kt);
+    if constexpr (kHasSpare) {
+      const __amdgpu_buffer_rsrc_t k_buf = k_tile_buffer(kt);
 #pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) spare.regs[i] = load_chunk_fast<SRC>(k_buf, chunk_bytes[i], 0u);
+      for (int i = 0; i < CHUNKS; ++i) spare.regs[i] = load_chunk_fast<SRC>(k_buf, chunk_bytes, part_offset(i));
+    }
   }
   __device__ __forceinline__ void take_spare(const Spare& spare) {
+    if constexpr (kHasSpare) {
 #pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) regs[i] = spare.regs[i];
+      for (int i = 0; i < CHUNKS; ++i) regs[i] = spare.regs[i];
+    }
   }
 
   // Whole tile with bounds checks (the partial last K tile): rows k >= K read as
@@ -534,26 +569,31 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int k = kt * 64 + k_row(i, tid_);
-      uint32_t w[4] = {0u, 0u, 0u, 0u};
-      if (k < k_end) {
+      if constexpr (SRC == SRC_BF16) {
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        if (k < k_end) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int n = first_row + chunk(i, tid_) * 8 + e;
+            if (n < extent) w[e >> 1] |= static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(base)[k * ks + n]) << ((e & 1) * 16);
+          }
+        }
+        regs[i] = Staged<SRC>{u32x4{w[0], w[1], w[2], w[3]}};
+      } else {
+        uint32_t w[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int n = first_row + chunk(i, tid_) * 8 + e;
-          if (n < extent) {
-            uint32_t v;
-            if constexpr (SRC == SRC_BF16) v = reinterpret_cast<const uint16_t*>(base)[k * ks + n];
-            else v = cvt_pk_bf16(reinterpret_cast<const float*>(base)[k * ks + n], 0.0f) & 0xffffu;
-            w[e >> 1] |= v << ((e & 1) * 16);
-          }
+          w[e] = (k < k_end && n < extent) ? __float_as_uint(reinterpret_cast<const float*>(base)[k * ks + n]) : 0u;
         }
+        regs[i] = Staged<SRC>{u32x4{w[0], w[1], w[2], w[3]}, u32x4{w[4], w[5], w[6], w[7]}};
       }
-      regs[i] = u32x4{w[0], w[1], w[2], w[3]};
     }
   }
 
   template <int PART>
   __device__ __forceinline__ void commit_part(char* lds_tile) const {
-    *reinterpret_cast<u32x4*>(lds_tile + k_row(PART, tid_) * kPitch + chunk(PART, tid_) * 16) = regs[PART];
+    *reinterpret_cast<u32x4*>(lds_tile + k_row(PART, tid_) * kPitch + chunk(PART, tid_) * 16) = regs[PART].chunk();
   }
   __device__ __forceinline__ void commit(char* lds_tile) const {
     static_for<CHUNKS>([&](auto ci) { commit_part<decltype(ci)::value>(lds_tile); });
@@ -736,6 +776,126 @@ constexpr int kTileLdsBytes() {
   return stages > epilogue ? stages : epilogue;
 }
 
+// Epilogue of the tile kernels: the accumulators of one wavefront to C.
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LDS_BYTES>
+__device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char* lds,
+                                                   typename AccTile<SrcTraits<SRC>::kInt>::type (&acc)[WM][WN], int batch,
+                                                   int split, int m0, int n0, int wm, int wn, int wave, int lane) {
+  constexpr bool INT = SrcTraits<SRC>::kInt;
+  constexpr int BM = 32 * WAVES_M * WM, BN = 32 * WAVES_N * WN;
+  const int frag_row = lane & 31;
+  const int frag_half = lane >> 5;
+  // Epilogue.  The MFMAs were issued with the B tile as first operand, so the
+  // accumulators hold C transposed: register r of lane l is
+  //   C[row = l % 32][col = (r/4)*8 + (l/32)*4 + r%4]
+  // of its 32x32 tile, i.e. four consecutive columns per register quad, which
+  // become one 8-byte (bf16) or 16-byte (fp32 / int32) store.  Tiles that lie
+  // wholly inside C, need no C-input or split-K and have 16-byte aligned rows take
+  // one of three inline store loops; everything else goes through the general
+  // out-of-line routine.
+  const bool interior = m0 + BM <= p.m && n0 + BN <= p.n;
+  const bool aligned = (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
+  const bool simple = interior && aligned && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1 && SRC != SRC_I8_FLIP;
+  char* c_base = static_cast<char*>(p.c);
+  if (simple && !INT && p.out_kind == OUT_BF16) {
+    // bf16: 8-byte pieces scattered over 32 rows would waste most of every memory
+    // transaction, so each wavefront first lays its tile out row-major in LDS (the
+    // staging buffers are dead by now) and then stores whole 16-byte row segments.
+    constexpr int TILE_COLS = WN * 32, TILE_ROWS = WM * 32;
+    constexpr int PITCH = TILE_COLS * 2 + 16;  // bytes; the pad staggers rows across banks
+    static_assert(PITCH * TILE_ROWS * WAVES_M * WAVES_N <= LDS_BYTES,
+                  "epilogue staging must fit the launch's LDS");
+    __syncthreads();  // every wavefront is done reading fragments
+    char* mine = lds + wave * (PITCH * TILE_ROWS);
+    static_for<WM>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      static_for<WN>([&](auto cj) {
+        constexpr int j = decltype(cj)::value;
+        static_for<4>([&](auto cq) {
+          constexpr int q = decltype(cq)::value;
+          if constexpr (!INT) {
+            u32x2 v;
+            v.x = cvt_pk_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]);
+            v.y = cvt_pk_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            *reinterpret_cast<u32x2*>(mine + (i * 32 + frag_row) * PITCH + (j * 32 + q * 8 + frag_half * 4) * 2) = v;
+          }
+        });
+      });
+    });
+    // the wavefront reads back only what it wrote itself: its own LDS traffic is ordered
+    constexpr int SEGS = TILE_COLS / 8;        // 16-byte segments per row
+    constexpr int TOTAL = TILE_ROWS * SEGS;    // 16-byte segments of this wavefront's tile
+    static_assert(TOTAL % 64 == 0, "whole store instructions");
+    uint16_t* out = reinterpret_cast<uint16_t*>(c_base) + batch * p.c_bs +
+                    static_cast<int64_t>(m0 + wm * TILE_ROWS) * p.c_rs + n0 + wn * TILE_COLS;
+#pragma unroll
+    for (int base = 0; base < TOTAL; base += 64) {
+      const int idx = base + lane, r = idx / SEGS, seg = idx % SEGS;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + seg * 16);
+      *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + seg * 8) = v;
+    }
+  } else if (simple && (INT ? (p.out_kind == OUT_I32 && p.row_scales == nullptr && p.correction == nullptr)
+                            : p.out_kind == OUT_F32)) {
+    static_for<WM>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      const int row = m0 + (wm * WM + i) * 32 + frag_row;
+      static_for<WN>([&](auto cj) {
+        constexpr int j = decltype(cj)::value;
+        const int col0 = n0 + (wn * WN + j) * 32 + frag_half * 4;
+        uint32_t* dst = reinterpret_cast<uint32_t*>(c_base) + batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col0;
+        static_for<4>([&](auto cq) {
+          constexpr int q = decltype(cq)::value;
+          // four consecutive accumulator registers as one 16-byte vector of their own type
+          const auto v = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
+          *reinterpret_cast<typename std::remove_const<decltype(v)>::type*>(dst + q * 8) = v;
+        });
+      });
+    });
+  } else if (simple && INT && p.row_scales != nullptr) {
+    float rs[WM];
+    static_for<WM>([&](auto ci) { rs[decltype(ci)::value] = p.row_scales[m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row]; });
+    static_for<WN>([&](auto cj) {
+      constexpr int j = decltype(cj)::value;
+      const int col0 = n0 + (wn * WN + j) * 32 + frag_half * 4;
+      f32x4 cs[4];
+      i32x4 corr[4];
+      static_for<4>([&](auto cq) {
+        constexpr int q = decltype(cq)::value;
+        cs[q] = *reinterpret_cast<const f32x4*>(p.column_scales + col0 + q * 8);
+        corr[q] = p.correction ? *reinterpret_cast<const i32x4*>(p.correction + col0 + q * 8) : i32x4{0, 0, 0, 0};
+      });
+      static_for<WM>([&](auto ci) {
+        constexpr int i = decltype(ci)::value;
+        const int row = m0 + (wm * WM + i) * 32 + frag_row;
+        float* dst = reinterpret_cast<float*>(c_base) + batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col0;
+        static_for<4>([&](auto cq) {
+          constexpr int q = decltype(cq)::value;
+          if constexpr (INT) {
+            const auto a4 = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
+            f32x4 out;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(a4[e]) + static_cast<uint32_t>(corr[q][e]));
+              const float t = static_cast<float>(v) * rs[i];  // row scale first, then column scale:
+              out[e] = t * cs[q][e];                          // two separately rounded multiplies
+            }
+            *reinterpret_cast<f32x4*>(dst + q * 8) = out;
+          }
+        });
+      });
+    });
+  } else {
+    static_for<WM>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      static_for<WN>([&](auto cj) {
+        constexpr int j = decltype(cj)::value;
+        store_tile_general<INT>(p, batch, split, m0 + (wm * WM + i) * 32 + frag_row,
+                                n0 + (wn * WN + j) * 32 + frag_half * 4, acc[i][j]);
+      });
+    });
+  }
+}
+
 // Workgroup shapes: WAVES_M x WAVES_N wavefronts, each owning WM x WN accumulator
 // tiles of 32x32.  Every shape in use runs 4 wavefronts, one per SIMD: the 256x256
 // tile with 128x128 per wavefront (256 accumulator registers in the AGPR half of
@@ -863,26 +1023,29 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   if (nk > 0) {
     // one branch for both operands: a wait in front of the out-of-line checked
     // loader must not separate A's loads from B's
-    if (seq(0) < full_k_tiles) {
-      stager_a.fetch_full(seq(0));
-      stager_b.fetch_full(seq(0));
+    // (scalar tile indices: a load whose uniform offset sits in a vector register is wrapped in a loop)
+    const int first = __builtin_amdgcn_readfirstlane(seq(0));
+    const int second = __builtin_amdgcn_readfirstlane(seq(nk > 1 ? 1 : 0));
+    if (first < full_k_tiles) {
+      stager_a.fetch_full(first);
+      stager_b.fetch_full(first);
     } else {
-      stager_a.fetch_checked(seq(0));
-      stager_b.fetch_checked(seq(0));
+      stager_a.fetch_checked(first);
+      stager_b.fetch_checked(first);
     }
     typename SA::Spare spare_a;
     typename SB::Spare spare_b;
     if (nk > 1) {
-      if constexpr (SA::kHasSpare) stager_a.fetch_full_spare(spare_a, seq(1));
-      if constexpr (SB::kHasSpare) stager_b.fetch_full_spare(spare_b, seq(1));
+      if constexpr (SA::kHasSpare) stager_a.fetch_full_spare(spare_a, second);
+      if constexpr (SB::kHasSpare) stager_b.fetch_full_spare(spare_b, second);
     }
     stager_a.commit(lds);
     stager_b.commit(lds + BM * 128);
     if (nk > 1) {
       if constexpr (SA::kHasSpare) stager_a.take_spare(spare_a);
-      else stager_a.fetch_full(seq(1));
+      else stager_a.fetch_full(second);
       if constexpr (SB::kHasSpare) stager_b.take_spare(spare_b);
-      else stager_b.fetch_full(seq(1));
+      else stager_b.fetch_full(second);
     }
   }
 
@@ -896,6 +1059,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
 
   if (nk > 0) {
     const int full_in_range = nk - has_tail;  // whole K tiles this workgroup owns
+    if constexpr (SRC == SRC_F32_AS_BF16) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
     lds_barrier();  // tile 0 is in LDS
     read_frags(0, lds, 0);
 
@@ -964,115 +1128,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
     else main_loop(std::false_type{});
   }
 
-  // Epilogue.  The MFMAs were issued with the B tile as first operand, so the
-  // accumulators hold C transposed: register r of lane l is
-  //   C[row = l % 32][col = (r/4)*8 + (l/32)*4 + r%4]
-  // of its 32x32 tile, i.e. four consecutive columns per register quad, which
-  // become one 8-byte (bf16) or 16-byte (fp32 / int32) store.  Tiles that lie
-  // wholly inside C, need no C-input or split-K and have 16-byte aligned rows take
-  // one of three inline store loops; everything else goes through the general
-  // out-of-line routine.
-  const bool interior = m0 + BM <= p.m && n0 + BN <= p.n;
-  const bool aligned = (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
-  const bool simple = interior && aligned && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1 && SRC != SRC_I8_FLIP;
-  char* c_base = static_cast<char*>(p.c);
-  if (simple && !INT && p.out_kind == OUT_BF16) {
-    // bf16: 8-byte pieces scattered over 32 rows would waste most of every memory
-    // transaction, so each wavefront first lays its tile out row-major in LDS (the
-    // staging buffers are dead by now) and then stores whole 16-byte row segments.
-    constexpr int TILE_COLS = WN * 32, TILE_ROWS = WM * 32;
-    constexpr int PITCH = TILE_COLS * 2 + 16;  // bytes; the pad staggers rows across banks
-    static_assert(PITCH * TILE_ROWS * WAVES_M * WAVES_N <= kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>(),
-                  "epilogue staging must fit the launch's LDS");
-    __syncthreads();  // every wavefront is done reading fragments
-    char* mine = lds + wave * (PITCH * TILE_ROWS);
-    static_for<WM>([&](auto ci) {
-      constexpr int i = decltype(ci)::value;
-      static_for<WN>([&](auto cj) {
-        constexpr int j = decltype(cj)::value;
-        static_for<4>([&](auto cq) {
-          constexpr int q = decltype(cq)::value;
-          if constexpr (!INT) {
-            u32x2 v;
-            v.x = cvt_pk_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]);
-            v.y = cvt_pk_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-            *reinterpret_cast<u32x2*>(mine + (i * 32 + frag_row) * PITCH + (j * 32 + q * 8 + frag_half * 4) * 2) = v;
-          }
-        });
-      });
-    });
-    // the wavefront reads back only what it wrote itself: its own LDS traffic is ordered
-    constexpr int SEGS = TILE_COLS / 8;        // 16-byte segments per row
-    constexpr int TOTAL = TILE_ROWS * SEGS;    // 16-byte segments of this wavefront's tile
-    static_assert(TOTAL % 64 == 0, "whole store instructions");
-    uint16_t* out = reinterpret_cast<uint16_t*>(c_base) + batch * p.c_bs +
-                    static_cast<int64_t>(m0 + wm * TILE_ROWS) * p.c_rs + n0 + wn * TILE_COLS;
-#pragma unroll
-    for (int base = 0; base < TOTAL; base += 64) {
-      const int idx = base + lane, r = idx / SEGS, seg = idx % SEGS;
-      const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + seg * 16);
-      *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + seg * 8) = v;
-    }
-  } else if (simple && (INT ? (p.out_kind == OUT_I32 && p.row_scales == nullptr && p.correction == nullptr)
-                            : p.out_kind == OUT_F32)) {
-    static_for<WM>([&](auto ci) {
-      constexpr int i = decltype(ci)::value;
-      const int row = m0 + (wm * WM + i) * 32 + frag_row;
-      static_for<WN>([&](auto cj) {
-        constexpr int j = decltype(cj)::value;
-        const int col0 = n0 + (wn * WN + j) * 32 + frag_half * 4;
-        uint32_t* dst = reinterpret_cast<uint32_t*>(c_base) + batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col0;
-        static_for<4>([&](auto cq) {
-          constexpr int q = decltype(cq)::value;
-          // four consecutive accumulator registers as one 16-byte vector of their own type
-          const auto v = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
-          *reinterpret_cast<typename std::remove_const<decltype(v)>::type*>(dst + q * 8) = v;
-        });
-      });
-    });
-  } else if (simple && INT && p.row_scales != nullptr) {
-    float rs[WM];
-    static_for<WM>([&](auto ci) { rs[decltype(ci)::value] = p.row_scales[m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row]; });
-    static_for<WN>([&](auto cj) {
-      constexpr int j = decltype(cj)::value;
-      const int col0 = n0 + (wn * WN + j) * 32 + frag_half * 4;
-      f32x4 cs[4];
-      i32x4 corr[4];
-      static_for<4>([&](auto cq) {
-        constexpr int q = decltype(cq)::value;
-        cs[q] = *reinterpret_cast<const f32x4*>(p.column_scales + col0 + q * 8);
-        corr[q] = p.correction ? *reinterpret_cast<const i32x4*>(p.correction + col0 + q * 8) : i32x4{0, 0, 0, 0};
-      });
-      static_for<WM>([&](auto ci) {
-        constexpr int i = decltype(ci)::value;
-        const int row = m0 + (wm * WM + i) * 32 + frag_row;
-        float* dst = reinterpret_cast<float*>(c_base) + batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col0;
-        static_for<4>([&](auto cq) {
-          constexpr int q = decltype(cq)::value;
-          if constexpr (INT) {
-            const auto a4 = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
-            f32x4 out;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(a4[e]) + static_cast<uint32_t>(corr[q][e]));
-              const float t = static_cast<float>(v) * rs[i];  // row scale first, then column scale:
-              out[e] = t * cs[q][e];                          // two separately rounded multiplies
-            }
-            *reinterpret_cast<f32x4*>(dst + q * 8) = out;
-          }
-        });
-      });
-    });
-  } else {
-    static_for<WM>([&](auto ci) {
-      constexpr int i = decltype(ci)::value;
-      static_for<WN>([&](auto cj) {
-        constexpr int j = decltype(cj)::value;
-        store_tile_general<INT>(p, batch, split, m0 + (wm * WM + i) * 32 + frag_row,
-                                n0 + (wn * WN + j) * 32 + frag_half * 4, acc[i][j]);
-      });
-    });
-  }
+  store_accumulators<SRC, WAVES_M, WAVES_N, WM, WN, kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>()>(
+      p, lds, acc, batch, split, m0, n0, wm, wn, wave, lane);
 }
 
 // Sums the split-K partials and applies the same epilogue as the tile kernel.
