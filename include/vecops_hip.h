@@ -141,6 +141,68 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t l
                                                         const float* scales, void* y, int64_t ldy, int64_t m,
                                                         int64_t n, int64_t k, int64_t group, void* stream);
 
+/*
+ * Prepacked B operand - the GPU counterpart of ops::matmul_pack with side B and
+ * matmul::packed_layout (ops/MatmulPack.h:9-117; x86 block format
+ * matmul/details/packing/amx/Format.h:27-58).  Packing is a permutation plus
+ * zero padding, so a matmul on the packed operand returns exactly what the
+ * plain one returns; weights that are multiplied many times are packed once and
+ * the multiplication then fetches them straight into matrix-core registers.
+ *
+ * Layout (EPC = elements per 16 bytes: 8 for bf16, 16 for i8; KS = k-steps of
+ * 2*EPC elements, K rounded up to a multiple of 8*EPC):
+ *   dim order [ panel (N/32) ][ k-step (KS) ][ k-half (2) ][ row (32) ][ k (EPC) ]
+ * i.e. element B[n,k] sits at byte
+ *   ((n/32 * KS + k/(2*EPC)) * 64 + (k/EPC % 2) * 32 + n % 32) * 16 + (k % EPC) * sizeof(element);
+ * rows past N and k past K are zero.
+ *
+ * packed dtypes: 11 bf16 (from a bf16 or f32 source; f32 is rounded to nearest
+ * even, as the matmul itself rounds it) and 2 i8.
+ */
+
+/* Bytes of the packed form of a [N,K] operand; 0 for an unsupported dtype. */
+VECOPS_HIP_EXPORT uint64_t vecops_hip_packed_b_bytes(uint32_t packed_dtype, int64_t n, int64_t k);
+
+/* Packs b (rank 2, [N,K], any strides; bf16, f32 or i8) into `packed`
+ * (16-byte aligned, at least vecops_hip_packed_b_bytes).  Replaces
+ * ops::MatmulPack<MatmulPackConfig<Atom, Operand::B>>::operator()
+ * (ops/MatmulPack.h:132-190). */
+VECOPS_HIP_EXPORT int32_t vecops_hip_pack_b(const VecopsHipOperand* b, void* packed, uint64_t packed_size,
+                                            void* stream);
+
+/* Packs an int8 b and also writes compensation[n] = -a_zero_point * sum_k b[n,k]
+ * (wrapping int32), the C-input row that corrects an asymmetrically quantised
+ * A - replaces ops::MatmulPackBCompensated (ops/MatmulPack.h:25-33,100-117). */
+VECOPS_HIP_EXPORT int32_t vecops_hip_pack_b_compensated(const VecopsHipOperand* b, int32_t a_zero_point, void* packed,
+                                                        uint64_t packed_size, int32_t* compensation, void* stream);
+
+/* vecops_hip_plan_matmul for a packed b of `n` rows (family, split-K, workspace). */
+VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul_packed_b(const VecopsHipOperand* a, uint32_t packed_dtype, int64_t n,
+                                                          const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                          VecopsHipPlan* plan);
+
+/*
+ * C[..,M,N] = C_in + A[..,M,K] . B[N,K]^T with B prepacked; the one packed
+ * operand serves every batch of a rank-3 A (vecops: a packed tensor passed as B
+ * lets the planner skip the packing stage, ops/MatmulPack.h:22-24).
+ *   packed bf16: a bf16 or f32 (rounded to bf16), c f32|bf16
+ *   packed i8  : a i8, c i32
+ * Same results, bit for bit, as vecops_hip_matmul on the unpacked operand when
+ * that runs its tile kernels.
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_packed_b(const VecopsHipOperand* a, const void* packed_b,
+                                                     uint32_t packed_dtype, int64_t n, const VecopsHipOperand* c_in,
+                                                     const VecopsHipOperand* c, void* workspace,
+                                                     uint64_t workspace_size, void* stream);
+
+/* vecops_hip_matmul_i8_dequant with b prepacked (i8); workspace as for the
+ * plain call with the same extents. */
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_i8_dequant_packed_b(const int8_t* a, int64_t lda, const void* packed_b,
+                                                                const float* row_scales, const float* column_scales,
+                                                                const int32_t* correction, float* c, int64_t ldc,
+                                                                int64_t m, int64_t n, int64_t k, void* workspace,
+                                                                uint64_t workspace_size, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

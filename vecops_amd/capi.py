@@ -21,7 +21,8 @@ STATUS_NAMES = {0: "Ok", 1: "InvalidArgument", 2: "NotApplicable", 3: "NotFound"
 EXPORTS = [
     "vecops_hip_abi_version", "vecops_hip_last_error", "vecops_hip_device_count", "vecops_hip_plan_matmul",
     "vecops_hip_matmul", "vecops_hip_matmul_i8_dequant", "vecops_hip_matmul_i8_dequant_workspace",
-    "vecops_hip_matmul_w8a16_group",
+    "vecops_hip_matmul_w8a16_group", "vecops_hip_packed_b_bytes", "vecops_hip_pack_b", "vecops_hip_pack_b_compensated",
+    "vecops_hip_plan_matmul_packed_b", "vecops_hip_matmul_packed_b", "vecops_hip_matmul_i8_dequant_packed_b",
 ]
 
 
@@ -65,6 +66,16 @@ def lib() -> C.CDLL:
         L.vecops_hip_matmul_w8a16_group.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p,
                                                     C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
                                                     C.c_int64, C.c_void_p]
+        L.vecops_hip_packed_b_bytes.restype = C.c_uint64
+        L.vecops_hip_packed_b_bytes.argtypes = [C.c_uint32, C.c_int64, C.c_int64]
+        L.vecops_hip_pack_b.argtypes = [P, C.c_void_p, C.c_uint64, C.c_void_p]
+        L.vecops_hip_pack_b_compensated.argtypes = [P, C.c_int32, C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]
+        L.vecops_hip_plan_matmul_packed_b.argtypes = [P, C.c_uint32, C.c_int64, P, P, C.POINTER(Plan)]
+        L.vecops_hip_matmul_packed_b.argtypes = [P, C.c_void_p, C.c_uint32, C.c_int64, P, P, C.c_void_p, C.c_uint64,
+                                                 C.c_void_p]
+        L.vecops_hip_matmul_i8_dequant_packed_b.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                            C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
+                                                            C.c_int64, C.c_void_p, C.c_uint64, C.c_void_p]
         _lib = L
     return _lib
 
@@ -153,3 +164,77 @@ def matmul_w8a16_group(x, w, scales, y, group: int, stream=None):
                                                scales.data_ptr(), y.data_ptr(), y.stride(0), m, n, k, group,
                                                _stream_handle(stream)))
     return y
+
+
+class PackedB:
+    """A [N,K] operand in the packed layout of ``vecops_hip_pack_b``: ``storage`` (uint8 tensor),
+    ``dtype`` (BF16 or I8), ``n`` and ``k`` - the counterpart of a tensor over
+    ``matmul::packed_layout<Atom, Operand::B>``."""
+
+    def __init__(self, storage, dtype: int, n: int, k: int) -> None:
+        self.storage, self.dtype, self.n, self.k = storage, dtype, n, k
+
+
+def pack_b(b, a_zero_point=None, stream=None):
+    """Pack b ([N,K]; bf16, f32 or int8) once for any number of ``matmul_packed_b`` calls.
+
+    With ``a_zero_point`` (int8 b only) also returns the int32[N] compensation row
+    ``-a_zero_point * sum_k b[n,k]`` (``ops::matmul_pack_b_compensated``).
+    """
+    import torch
+    n, k = b.shape
+    dtype = I8 if b.dtype == torch.int8 else BF16
+    size = lib().vecops_hip_packed_b_bytes(dtype, n, k)
+    storage = torch.empty(max(size, 16), dtype=torch.uint8, device=b.device)
+    ob = operand(b)
+    if a_zero_point is None:
+        _check(lib().vecops_hip_pack_b(C.byref(ob), storage.data_ptr(), size, _stream_handle(stream)))
+        return PackedB(storage, dtype, n, k)
+    comp = torch.empty(n, dtype=torch.int32, device=b.device)
+    _check(lib().vecops_hip_pack_b_compensated(C.byref(ob), a_zero_point, storage.data_ptr(), size, comp.data_ptr(),
+                                               _stream_handle(stream)))
+    return PackedB(storage, dtype, n, k), comp
+
+
+def plan_matmul_packed_b(a, packed: PackedB, c, c_in=None) -> Plan:
+    plan = Plan()
+    oa, oc = operand(a), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    _check(lib().vecops_hip_plan_matmul_packed_b(C.byref(oa), packed.dtype, packed.n,
+                                                 C.byref(oi) if oi is not None else None, C.byref(oc), C.byref(plan)))
+    return plan
+
+
+def matmul_packed_b(a, packed: PackedB, c, c_in=None, workspace=None, stream=None):
+    """c[..,M,N] = c_in + a[..,M,K] . B^T with B packed by ``pack_b``; returns c."""
+    import torch
+    plan = plan_matmul_packed_b(a, packed, c, c_in)
+    if plan.workspace_bytes and (workspace is None or workspace.numel() * workspace.element_size()
+                                 < plan.workspace_bytes):
+        workspace = torch.empty(plan.workspace_bytes, dtype=torch.uint8, device=c.device)
+    oa, oc = operand(a), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_packed_b(C.byref(oa), packed.storage.data_ptr(), packed.dtype, packed.n,
+                                            C.byref(oi) if oi is not None else None, C.byref(oc), ws_ptr, ws_size,
+                                            _stream_handle(stream)))
+    return c
+
+
+def matmul_i8_dequant_packed_b(a, packed: PackedB, row_scales, column_scales, c, correction=None, workspace=None,
+                               stream=None):
+    import torch
+    m, k = a.shape
+    n = packed.n
+    assert a.stride(1) == 1 and c.stride(1) == 1 and packed.dtype == I8 and packed.k == k
+    need = lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k)
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=c.device)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_i8_dequant_packed_b(
+        a.data_ptr(), a.stride(0), packed.storage.data_ptr(), row_scales.data_ptr(), column_scales.data_ptr(),
+        correction.data_ptr() if correction is not None else None, c.data_ptr(), c.stride(0), m, n, k, ws_ptr,
+        ws_size, _stream_handle(stream)))
+    return c

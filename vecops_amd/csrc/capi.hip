@@ -9,6 +9,7 @@
 #include "skinny_dense.h"
 #include "skinny_w8a16.h"
 #include "tile_gemm_launch.h"
+#include "tile_gemm_packed.h"
 #include "vecops_hip.h"
 
 namespace {
@@ -87,6 +88,7 @@ struct Problem {
   int out_kind;  // OutKind
   int cin_kind;
   int64_t batch, m, n, k;
+  bool packed_b;  // b.data addresses a prepacked operand (vecops_hip_pack_b), shared by every batch
 };
 
 // Same rules as vecops' validate() (planning/families/ArchitectureFamily.h:1590-1652,
@@ -95,6 +97,7 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
                  const VecopsHipOperand* c, uint32_t compute, Problem* pr) {
   if (!normalise(a, &pr->a) || !normalise(b, &pr->b) || !normalise(c, &pr->c))
     return fail(ST_INVALID, "matmul: operands must be rank 2 or 3 with non-negative extents");
+  pr->packed_b = false;
   pr->has_cin = cin != nullptr;
   if (pr->has_cin && !normalise(cin, &pr->cin)) return fail(ST_INVALID, "matmul: malformed c_in");
   if (a->rank != b->rank || a->rank != c->rank || (pr->has_cin && cin->rank != c->rank))
@@ -162,7 +165,7 @@ constexpr int kComputeUnits = 256;
 
 // bf16 x bf16 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
 bool skinny_applies(const Problem& pr) {
-  if (pr.src != SRC_BF16 || pr.has_cin) return false;
+  if (pr.src != SRC_BF16 || pr.has_cin || pr.packed_b) return false;
   if (!k_vector_ok(pr.a) || !k_vector_ok(pr.b) || pr.k % 8 != 0 || pr.k < 64) return false;
   const int64_t narrow = pr.m < pr.n ? pr.m : pr.n, wide = pr.m < pr.n ? pr.n : pr.m;
   return narrow <= 16 && wide >= 512 && pr.batch <= 65535;
@@ -190,7 +193,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     return;
   }
   plan->vector_a = k_vector_ok(pr.a) ? 1 : 0;
-  plan->vector_b = (k_vector_ok(pr.b) || (pr.b.rs == 1 && pr.b.cs != 1 && n_vector_ok(pr.b) && dtype_bytes(pr.b.dtype) != 1)) ? 1 : 0;
+  plan->vector_b = pr.packed_b || (k_vector_ok(pr.b) || (pr.b.rs == 1 && pr.b.cs != 1 && n_vector_ok(pr.b) && dtype_bytes(pr.b.dtype) != 1)) ? 1 : 0;
   plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
 
   // Skinny family: one operand has at most 16 rows and the other is long - the GPU reading of
@@ -240,6 +243,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   if (plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
   if (pr.a.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: a has no storage");
   if (pr.b.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: b has no storage");
+  if (pr.packed_b && plan.family == VECOPS_HIP_FAMILY_SKINNY) return fail(ST_INVALID, "matmul: plan does not fit a packed b");
   if (pr.c.data == nullptr) return fail(ST_INVALID, "matmul: c has no storage");
   if (plan.workspace_bytes > workspace_size || (plan.workspace_bytes > 0 && workspace == nullptr))
     return fail(ST_INVALID, "matmul: workspace of %llu bytes required, %llu supplied",
@@ -342,7 +346,9 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     }
     if (pr.a_unsigned && pr.b_unsigned) p.const_term = 16384u * static_cast<uint32_t>(pr.k);
   }
-  switch (pr.src) {
+  if (pr.packed_b) {
+    e = launch_tile_gemm_packed_b(pr.src, p, tile, plan.vector_a != 0, stream);
+  } else switch (pr.src) {
     case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile, mode, stream); break;
     case SRC_BF16: e = launch_tile_gemm_bf16(p, tile, mode, stream); break;
     case SRC_F32_AS_BF16: e = launch_tile_gemm_f32_as_bf16(p, tile, mode, stream); break;
@@ -393,9 +399,137 @@ void launch_skinny_mfma_resident(const SkinnyW8A16Params& p, int passes, hipStre
                      stream, p, passes);
 }
 
+// Problem description of a matmul whose B operand is prepacked: b is described as the dense
+// [N,K] operand it was packed from (its strides are never used), with `packed` as its storage.
+int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t packed_dtype, int64_t n,
+                        const VecopsHipOperand* cin, const VecopsHipOperand* c, Problem* pr) {
+  if (a == nullptr || (a->rank != 2 && a->rank != 3)) return fail(ST_INVALID, "matmul_packed_b: malformed a");
+  if (n < 0) return fail(ST_INVALID, "matmul_packed_b: negative n");
+  const uint32_t da = a->dtype;
+  if (packed_dtype == DT_BF16) {
+    if (da != DT_BF16 && da != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: a bf16-packed b needs a bf16 or f32 a");
+  } else if (packed_dtype == DT_I8) {
+    if (da != DT_I8) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an i8-packed b needs an i8 a");
+  } else {
+    return fail(ST_NOT_APPLICABLE, "matmul_packed_b: packed dtype %u not supported", packed_dtype);
+  }
+  VecopsHipOperand b;
+  memset(&b, 0, sizeof(b));
+  b.data = const_cast<void*>(packed);
+  b.dtype = da;
+  b.rank = a->rank;
+  const int base = a->rank == 3 ? 1 : 0;
+  const int64_t k = a->sizes[base + 1];
+  if (a->rank == 3) b.sizes[0] = a->sizes[0];  // batch stride 0: one packed operand for every batch
+  b.sizes[base] = n;
+  b.sizes[base + 1] = k;
+  b.strides[base] = k;
+  b.strides[base + 1] = 1;
+  int32_t rc = describe(a, &b, cin, c, VECOPS_HIP_COMPUTE_BF16, pr);
+  if (rc != ST_OK) return rc;
+  pr->packed_b = true;
+  // 32-bit offsets inside one workgroup's eight 32-row panels of the packed operand
+  const int64_t ks_total = packed_k_steps(pr->k, pr->src == SRC_I8 ? 16 : 8);
+  if (ks_total * 1024 * 8 >= (int64_t{1} << 31)) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: k too large");
+  return ST_OK;
+}
+
+int src_of_packed_source(uint32_t dtype) {
+  return dtype == DT_BF16 ? SRC_BF16 : dtype == DT_F32 ? SRC_F32_AS_BF16 : dtype == DT_I8 ? SRC_I8 : -1;
+}
+
 }  // namespace
 
 extern "C" {
+
+uint64_t vecops_hip_packed_b_bytes(uint32_t packed_dtype, int64_t n, int64_t k) {
+  if (n < 0 || k < 0 || (packed_dtype != DT_BF16 && packed_dtype != DT_I8)) return 0;
+  return static_cast<uint64_t>(packed_b_bytes(n, k, packed_dtype == DT_I8 ? 16 : 8));
+}
+
+int32_t vecops_hip_pack_b(const VecopsHipOperand* b, void* packed, uint64_t packed_size, void* stream) {
+  View v;
+  if (!normalise(b, &v) || b->rank != 2) return fail(ST_INVALID, "pack_b: b must be a rank-2 [N,K] operand");
+  const int src = src_of_packed_source(v.dtype);
+  if (src < 0) return fail(ST_NOT_APPLICABLE, "pack_b: dtype %u not supported", v.dtype);
+  if (v.rows > INT32_MAX || v.cols > INT32_MAX - 256) return fail(ST_INVALID, "pack_b: extent too large");
+  const uint64_t need = static_cast<uint64_t>(packed_b_bytes(v.rows, v.cols, src == SRC_I8 ? 16 : 8));
+  if (packed_size < need)
+    return fail(ST_INVALID, "pack_b: %llu bytes required, %llu supplied", (unsigned long long)need,
+                (unsigned long long)packed_size);
+  if (need == 0) return ST_OK;
+  if (packed == nullptr || !aligned16(packed)) return fail(ST_INVALID, "pack_b: packed storage must be 16-byte aligned");
+  if (v.data == nullptr) return fail(ST_INVALID, "pack_b: b has no storage");
+  PackBParams q;
+  q.b = v.data;
+  q.packed = packed;
+  q.rs = v.rs;
+  q.ks = v.cs;
+  q.n = static_cast<int32_t>(v.rows);
+  q.k = static_cast<int32_t>(v.cols);
+  hipError_t e = launch_pack_b(src, q, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(ST_EXEC, "pack kernel launch: %s", hipGetErrorString(e));
+  return ST_OK;
+}
+
+int32_t vecops_hip_pack_b_compensated(const VecopsHipOperand* b, int32_t a_zero_point, void* packed,
+                                      uint64_t packed_size, int32_t* compensation, void* stream) {
+  if (b == nullptr || b->dtype != DT_I8) return fail(ST_NOT_APPLICABLE, "pack_b_compensated: b must be int8");
+  int32_t rc = vecops_hip_pack_b(b, packed, packed_size, stream);
+  if (rc != ST_OK) return rc;
+  View v;
+  normalise(b, &v);
+  if (v.rows == 0) return ST_OK;
+  if (compensation == nullptr) return fail(ST_INVALID, "pack_b_compensated: null compensation");
+  // -a_zero_point * sum_k b[n,k], wrapping like every int32 accumulator of the path
+  hipError_t e = launch_byte_row_sums(v.data, 1, static_cast<int32_t>(v.rows), static_cast<int32_t>(v.cols), 0, v.rs, v.cs,
+                                      0u, 0u - static_cast<uint32_t>(a_zero_point), compensation,
+                                      static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
+  return ST_OK;
+}
+
+int32_t vecops_hip_plan_matmul_packed_b(const VecopsHipOperand* a, uint32_t packed_dtype, int64_t n,
+                                        const VecopsHipOperand* c_in, const VecopsHipOperand* c, VecopsHipPlan* plan) {
+  if (plan == nullptr) return fail(ST_INVALID, "plan_matmul_packed_b: null plan");
+  Problem pr;
+  int32_t rc = describe_packed(a, reinterpret_cast<void*>(16), packed_dtype, n, c_in, c, &pr);
+  if (rc != ST_OK) return rc;
+  choose(pr, plan);
+  return ST_OK;
+}
+
+int32_t vecops_hip_matmul_packed_b(const VecopsHipOperand* a, const void* packed_b, uint32_t packed_dtype, int64_t n,
+                                   const VecopsHipOperand* c_in, const VecopsHipOperand* c, void* workspace,
+                                   uint64_t workspace_size, void* stream) {
+  Problem pr;
+  int32_t rc = describe_packed(a, packed_b, packed_dtype, n, c_in, c, &pr);
+  if (rc != ST_OK) return rc;
+  if (pr.k > 0 && pr.n > 0 && !aligned16(packed_b)) return fail(ST_INVALID, "matmul_packed_b: packed b must be 16-byte aligned");
+  VecopsHipPlan plan;
+  choose(pr, &plan);
+  return run_problem(pr, plan, nullptr, nullptr, nullptr, workspace, workspace_size, static_cast<hipStream_t>(stream));
+}
+
+int32_t vecops_hip_matmul_i8_dequant_packed_b(const int8_t* a, int64_t lda, const void* packed_b,
+                                              const float* row_scales, const float* column_scales,
+                                              const int32_t* correction, float* c, int64_t ldc, int64_t m, int64_t n,
+                                              int64_t k, void* workspace, uint64_t workspace_size, void* stream) {
+  if (m < 0 || n < 0 || k < 0) return fail(ST_INVALID, "matmul_i8_dequant_packed_b: negative extent");
+  if (m > 0 && n > 0 && (row_scales == nullptr || column_scales == nullptr))
+    return fail(ST_INVALID, "matmul_i8_dequant_packed_b: scales are required");
+  VecopsHipOperand oa, oc;
+  make_operand(&oa, a, DT_I8, m, k, lda);
+  make_operand(&oc, c, DT_I32, m, n, ldc);  // accumulator class; the epilogue writes fp32
+  Problem pr;
+  int32_t rc = describe_packed(&oa, packed_b, DT_I8, n, nullptr, &oc, &pr);
+  if (rc != ST_OK) return rc;
+  if (pr.k > 0 && pr.n > 0 && !aligned16(packed_b)) return fail(ST_INVALID, "matmul_i8_dequant_packed_b: packed b must be 16-byte aligned");
+  VecopsHipPlan plan;
+  choose(pr, &plan);
+  return run_problem(pr, plan, row_scales, column_scales, correction, workspace, workspace_size,
+                     static_cast<hipStream_t>(stream));
+}
 
 uint32_t vecops_hip_abi_version(void) { return VECOPS_HIP_ABI_VERSION; }
 

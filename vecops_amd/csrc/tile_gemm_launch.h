@@ -28,6 +28,11 @@ hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile, int mode,
 hipError_t launch_byte_row_sums(const void* x, int32_t batch, int32_t rows, int32_t k, int64_t bs, int64_t rs,
                                 int64_t ks, uint32_t flip, uint32_t scale, int32_t* out, hipStream_t stream);
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
+// B prepacked by launch_pack_b (src: SRC_BF16, SRC_F32_AS_BF16 = fp32 A against bf16-packed B, SRC_I8);
+// vector_a: A is K-contiguous and 16-byte aligned
+hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile, bool vector_a, hipStream_t stream);
+struct PackBParams;
+hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream);
 
 // Shared by the per-class translation units.
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB>
