@@ -6,8 +6,9 @@
 A "step" is one pass of the hot path over one batch of synthetic operands that are
 already resident in HBM.  The default workload is the configuration the headline
 metric is quoted on (bf16 GEMM, M=N=K=4096, A[M,K] and B[K,N] row-major, fp32
-accumulate, bf16 output); the int8 quantised matmul and the M=1 weight-only GEMV
-are measured in the same run and reported under "secondary".  Prints ONE JSON line.
+accumulate, bf16 output); the int8 quantised matmul, the M=1 weight-only GEMV and the
+prepacked-weights forms of the two GEMMs are measured in the same run and reported
+under "secondary".  Prints ONE JSON line.
 """
 from __future__ import annotations
 
@@ -33,6 +34,8 @@ PEAK_HBM_GBPS = 8000.0
 TRAFFIC_BF16_4096 = int((102026 * 2.000 + 47616 * 1.000) * 1024)
 TRAFFIC_INT8_DEQUANT = int((103713 * 2.000 + 112200 * 1.000) * 1024)
 TRAFFIC_GEMV_M1 = int((29683.3 * 2.000 + 56.0 * 1.000) * 1024)
+TRAFFIC_BF16_4096_PACKED = None      # not collected yet
+TRAFFIC_INT8_DEQUANT_PACKED = None
 
 
 def _device_tensors_bf16_gemm(dev):
@@ -104,6 +107,52 @@ def bench_int8_dequant(dev, steps, warmup):
             "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                          "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT,
                          "kernel": "vecops_hip::tile_gemm_kernel<int8, 256x256x128, dequant epilogue>",
+                         "algorithmic_ops_per_launch": ops,
+                         "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
+
+
+def bench_bf16_gemm_packed(dev, steps, warmup):
+    """The headline shape with B packed once beforehand (vecops' prepacked-weights mode): the packing is
+    outside the timed region, as in the reference's own prepacked rows."""
+    import torch
+    from vecops_amd import capi
+    n = 4096
+    _, _, ta, tb = _device_tensors_bf16_gemm(dev)
+    packed = capi.pack_b(tb.t())
+    c = torch.empty((n, n), dtype=torch.bfloat16, device=dev)
+    wall_ms, ev_ms = _time_launches(lambda i: capi.matmul_packed_b(ta, packed, c), steps, warmup)
+    flops = 2.0 * n * n * n
+    tflops = flops / (ev_ms * 1e-3) / 1e12
+    return {"metric": "bf16_gemm_4096_prepacked_b_tflops", "workload": "bf16 GEMM M=N=K=4096, B prepacked "
+            "(vecops_hip_pack_b, not timed), fp32 accumulate, bf16 out", "value": tflops, "unit": "TFLOP/s",
+            "ms_per_step": wall_ms, "dtype": "bf16",
+            "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BF16_4096_PACKED,
+                         "kernel": "vecops_hip::tile_gemm_packed_b_kernel<bf16, 256x256x64>",
+                         "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": 3 * 2 * n * n}}
+
+
+def bench_int8_dequant_packed(dev, steps, warmup):
+    import torch
+    from vecops_amd import capi, synth
+    m, k, n = 2048, 4096, 11008
+    a = torch.from_numpy(synth.int8_sym(1, (m, k))).to(dev)
+    packed = capi.pack_b(torch.from_numpy(synth.int8_sym(2, (n, k))).to(dev))
+    rs = torch.from_numpy(synth.scales(3, m)).to(dev)
+    cs = torch.from_numpy(synth.scales(4, n)).to(dev)
+    c = torch.empty((m, n), dtype=torch.float32, device=dev)
+    need = capi.lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    wall_ms, ev_ms = _time_launches(
+        lambda i: capi.matmul_i8_dequant_packed_b(a, packed, rs, cs, c, workspace=ws), steps, warmup)
+    ops = 2.0 * m * n * k
+    tops = ops / (ev_ms * 1e-3) / 1e12
+    return {"metric": "int8_quantized_matmul_prepacked_b_tops", "workload": "int8 2048x4096x11008, weights prepacked "
+            "(not timed), per-token x per-channel dequant fused, fp32 out", "value": tops, "unit": "TOP/s",
+            "ms_per_step": wall_ms, "dtype": "int8",
+            "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                         "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT_PACKED,
+                         "kernel": "vecops_hip::tile_gemm_packed_b_kernel<int8, 256x256x128, dequant epilogue>",
                          "algorithmic_ops_per_launch": ops,
                          "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
 
@@ -189,7 +238,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["bf16", "int8", "gemv", "copy"], help="run a single workload (for profiling)")
+    ap.add_argument("--only", choices=["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed"], help="run a single workload (for profiling)")
     ap.add_argument("--gemv-m", type=int, default=1, help="activation rows of the --only gemv workload (1..16)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -212,6 +261,12 @@ def main() -> int:
     if args.only == "copy":
         print(json.dumps(bench_copy(dev, args.steps, args.warmup)))
         return 0
+    if args.only == "bf16_packed":
+        print(json.dumps(bench_bf16_gemm_packed(dev, args.steps, args.warmup)))
+        return 0
+    if args.only == "int8_packed":
+        print(json.dumps(bench_int8_dequant_packed(dev, args.steps, args.warmup)))
+        return 0
     if args.only == "gemv":
         print(json.dumps(bench_gemv(dev, args.steps, args.warmup, m=args.gemv_m)))
         return 0
@@ -228,7 +283,9 @@ def main() -> int:
     }
     if args.only != "bf16":
         line["secondary"] = [bench_int8_dequant(dev, args.steps, args.warmup),
-                             bench_gemv(dev, max(args.steps, 200), args.warmup, m=1)]
+                             bench_gemv(dev, max(args.steps, 200), args.warmup, m=1),
+                             bench_bf16_gemm_packed(dev, args.steps, args.warmup),
+                             bench_int8_dequant_packed(dev, args.steps, args.warmup)]
     if not args.no_cpu and args.only is None:
         line["cpu_baseline"] = cpu_baseline(a, b_kn)
     print(json.dumps(line))

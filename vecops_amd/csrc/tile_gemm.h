@@ -832,7 +832,9 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
     for (int base = 0; base < TOTAL; base += 64) {
       const int idx = base + lane, r = idx / SEGS, seg = idx % SEGS;
       const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + seg * 16);
-      *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + seg * 8) = v;
+      // whole 128-byte lines per row segment: streamed past L2, so the end of the kernel has no dirty C to
+      // write back (the 16-byte pieces of the 32-bit paths below would turn into partial-line writes: slower)
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + seg * 8));
     }
   } else if (simple && (INT ? (p.out_kind == OUT_I32 && p.row_scales == nullptr && p.correction == nullptr)
                             : p.out_kind == OUT_F32)) {
