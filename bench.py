@@ -31,11 +31,11 @@ PEAK_HBM_GBPS = 8000.0
 # profiles/ (KiB per dispatch x 1024, FETCH scaled by 2.000 and WRITE by 1.000: what the
 # same counters read for a 1 GiB device copy, `--only copy`).  Counters cannot be read
 # from inside this process, so these are the recorded figures for exactly these workloads.
-TRAFFIC_BF16_4096 = int((102026 * 2.000 + 47616 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT = int((103713 * 2.000 + 112200 * 1.000) * 1024)
-TRAFFIC_GEMV_M1 = int((29683.3 * 2.000 + 56.0 * 1.000) * 1024)
-TRAFFIC_BF16_4096_PACKED = None      # not collected yet
-TRAFFIC_INT8_DEQUANT_PACKED = None
+TRAFFIC_BF16_4096 = int((101956 * 2.000 + 47624 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT = int((103564 * 2.000 + 112550 * 1.000) * 1024)
+TRAFFIC_GEMV_M1 = int((29688.5 * 2.000 + 56.1 * 1.000) * 1024)
+TRAFFIC_BF16_4096_PACKED = int((101803 * 2.000 + 47622 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT_PACKED = int((102951 * 2.000 + 112527 * 1.000) * 1024)
 
 
 def _device_tensors_bf16_gemm(dev):
