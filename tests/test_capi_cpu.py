@@ -57,8 +57,15 @@ def test_rule_table_known_answers():
     # one row against a long weight matrix: the skinny family, no workspace
     rc, p = _plan(_operand(capi.BF16, (1, 4096)), _operand(capi.BF16, (14336, 4096)), _operand(capi.BF16, (1, 14336)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "skinny" and p.workspace_bytes == 0
-    # ... but not with a K that 16-byte loads cannot cover, nor for int8
+    # ... but not with a K that 16-byte loads cannot cover
     rc, p = _plan(_operand(capi.BF16, (1, 129)), _operand(capi.BF16, (4097, 129)), _operand(capi.F32, (1, 4097)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] != "skinny"
+    # int8 decode shapes are skinny too (signed bytes, K a multiple of 16); an unsigned side is not
+    rc, p = _plan(_operand(capi.I8, (4, 4096)), _operand(capi.I8, (11008, 4096)), _operand(capi.I32, (4, 11008)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "skinny" and p.workspace_bytes == 0
+    rc, p = _plan(_operand(capi.U8, (4, 4096)), _operand(capi.I8, (11008, 4096)), _operand(capi.I32, (4, 11008)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] != "skinny"
+    rc, p = _plan(_operand(capi.I8, (4, 4104)), _operand(capi.I8, (11008, 4104)), _operand(capi.I32, (4, 11008)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] != "skinny"
     # tiny output, long K (config 3's 255x63x8191): small tile and split-K with workspace
     rc, p = _plan(_operand(capi.BF16, (255, 8191)), _operand(capi.BF16, (63, 8191)), _operand(capi.F32, (255, 63)))

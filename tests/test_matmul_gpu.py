@@ -421,6 +421,58 @@ def test_int8_dequant_bit_exact(device, oracle, m, n, k, corr):
     assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 11008, 4096), (16, 14336, 4096), (4, 4096, 11008), (3, 1000, 528),
+                                   (2048, 7, 272), (5, 513, 128), (16, 600, 8208)])
+def test_skinny_int8_family(device, oracle, m, n, k):
+    """int8 decode shapes on the skinny kernel: int32 accumulators bit-exact, either side narrow."""
+    import torch
+    from vecops_amd import capi
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    c = torch.full((m, n), -1, dtype=torch.int32, device=device)
+    assert capi.FAMILY_NAMES[capi.plan_matmul(ta, tb, c).family] == "skinny"
+    capi.matmul(ta, tb, c)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy(), oracle.matmul_i8_dense(a, b))
+
+
+@pytest.mark.parametrize("m,n,k,corr", [(1, 11008, 4096, False), (16, 11008, 4096, True), (7, 700, 1040, True),
+                                        (2048, 7, 272, True)])
+def test_skinny_int8_dequant_bit_exact(device, oracle, m, n, k, corr):
+    """Decode-shaped quantised matmul (few tokens against the whole weight matrix): the skinny kernel with
+    the dequantising epilogue when A is the narrow side, the tile kernel otherwise - same bits either way."""
+    import torch
+    from vecops_amd import capi
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    rs, cs = synth.scales(3, m), synth.scales(4, n)
+    correction = ((synth.draws(5, n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32) if corr else None
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul_i8_dequant(torch.from_numpy(a).to(device), torch.from_numpy(b).to(device),
+                           torch.from_numpy(rs).to(device), torch.from_numpy(cs).to(device), c,
+                           correction=torch.from_numpy(correction).to(device) if corr else None)
+    torch.cuda.synchronize()
+    want = oracle.matmul_i8_dequant(a, b, rs, cs, correction)
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_skinny_int8_wraps_and_batches(device):
+    """Accumulators wrap mod 2^32 across the K slices of the eight wavefronts; rank-3 with a broadcast A."""
+    import torch
+    from vecops_amd import capi
+    batch, m, n, k = 2, 3, 640, 140000 // 16 * 16
+    a = torch.full((m, k), -128, dtype=torch.int8, device=device)
+    b = torch.full((batch, n, k), -128, dtype=torch.int8, device=device)
+    b[1, :, ::2] = 127
+    c = torch.empty((batch, m, n), dtype=torch.int32, device=device)
+    capi.matmul(a[None].expand(batch, m, k), b, c)
+    torch.cuda.synchronize()
+    want0 = np.int64(16384) * k
+    want1 = np.int64(16384) * (k // 2) + np.int64(-128 * 127) * (k // 2)
+    wrap = lambda v: int(((int(v) + 2 ** 31) % 2 ** 32) - 2 ** 31)
+    assert (c[0] == wrap(want0)).all() and (c[1] == wrap(want1)).all()
+    assert want0 > 2 ** 31  # the case does wrap
+
+
 # --- full BASELINE sizes: size-independent properties -------------------------------------
 
 def test_config2_bf16_4096_sampled_and_linear(device, oracle):

@@ -89,6 +89,7 @@ struct Problem {
   int cin_kind;
   int64_t batch, m, n, k;
   bool packed_b;  // b.data addresses a prepacked operand (vecops_hip_pack_b), shared by every batch
+  bool dequant;   // the int32 accumulators leave through the per-row x per-column dequantisation
 };
 
 // Same rules as vecops' validate() (planning/families/ArchitectureFamily.h:1590-1652,
@@ -98,6 +99,7 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
   if (!normalise(a, &pr->a) || !normalise(b, &pr->b) || !normalise(c, &pr->c))
     return fail(ST_INVALID, "matmul: operands must be rank 2 or 3 with non-negative extents");
   pr->packed_b = false;
+  pr->dequant = false;
   pr->has_cin = cin != nullptr;
   if (pr->has_cin && !normalise(cin, &pr->cin)) return fail(ST_INVALID, "matmul: malformed c_in");
   if (a->rank != b->rank || a->rank != c->rank || (pr->has_cin && cin->rank != c->rank))
@@ -163,10 +165,11 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
 
 constexpr int kComputeUnits = 256;
 
-// bf16 x bf16 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
+// bf16 x bf16 or int8 x int8 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
 bool skinny_applies(const Problem& pr) {
-  if (pr.src != SRC_BF16 || pr.has_cin || pr.packed_b) return false;
-  if (!k_vector_ok(pr.a) || !k_vector_ok(pr.b) || pr.k % 8 != 0 || pr.k < 64) return false;
+  if ((pr.src != SRC_BF16 && pr.src != SRC_I8) || pr.has_cin || pr.packed_b) return false;
+  const int64_t per = pr.src == SRC_I8 ? 16 : 8;  // elements per 16 bytes
+  if (!k_vector_ok(pr.a) || !k_vector_ok(pr.b) || pr.k % per != 0 || pr.k < 8 * per) return false;
   const int64_t narrow = pr.m < pr.n ? pr.m : pr.n, wide = pr.m < pr.n ? pr.n : pr.m;
   return narrow <= 16 && wide >= 512 && pr.batch <= 65535;
 }
@@ -199,7 +202,9 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
   // Skinny family: one operand has at most 16 rows and the other is long - the GPU reading of
   // vecops' small-vector shapes (runtime_dispatch_rules::skinny_at_most / large_m1 / large_n1,
   // matmul/details/kernel/RuntimeDispatch.h:24-83): HBM-bound, the wide operand is read once.
-  if (skinny_applies(pr)) {
+  // (the dequantising epilogue multiplies by A's row scale first: the skinny kernel applies the narrow side's
+  // scale first, so it serves a dequantised product only when A is the narrow side)
+  if (skinny_applies(pr) && !(pr.dequant && pr.m >= pr.n)) {
     plan->family = VECOPS_HIP_FAMILY_SKINNY;
     return;
   }
@@ -283,8 +288,9 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     const View& wide = a_narrow ? pr.b : pr.a;
     const View& narrow = a_narrow ? pr.a : pr.b;
     SkinnyDenseParams q;
-    q.w = static_cast<const uint16_t*>(wide.data);
-    q.x = static_cast<const uint16_t*>(narrow.data);
+    memset(&q, 0, sizeof(q));
+    q.w = wide.data;
+    q.x = narrow.data;
     q.y = pr.c.data;
     q.ldw = wide.rs;
     q.ldx = narrow.rs;
@@ -296,20 +302,32 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     q.rows = static_cast<int32_t>(wide.rows);
     q.s = static_cast<int32_t>(narrow.rows);
     q.k = static_cast<int32_t>(pr.k);
-    q.out_bf16 = pr.out_kind == OUT_BF16 ? 1 : 0;
+    if (is_int) {
+      q.out_kind = row_scales != nullptr ? SKINNY_OUT_DEQUANT_F32 : SKINNY_OUT_I32;
+      q.narrow_scales = row_scales;  // dequantisation comes here only with A as the narrow side
+      q.wide_scales = column_scales;
+      q.wide_term = correction;
+    } else {
+      q.out_kind = pr.out_kind == OUT_BF16 ? SKINNY_OUT_BF16 : SKINNY_OUT_F32;
+    }
     // 64 wide rows per workgroup when that still leaves most compute units a workgroup, else 32 or 16
     const int64_t wgs64 = (wide.rows + 63) / 64 * pr.batch;
     const dim3 block(512);
-    if (wgs64 >= 200) {
-      hipLaunchKernelGGL((skinny_dense_kernel<2, 2>), dim3(static_cast<unsigned>((wide.rows + 63) / 64), p.batch), block, 0,
-                         stream, q);
-    } else if (wgs64 * 2 >= 200) {
-      hipLaunchKernelGGL((skinny_dense_kernel<1, 2>), dim3(static_cast<unsigned>((wide.rows + 31) / 32), p.batch), block, 0,
-                         stream, q);
-    } else {
-      hipLaunchKernelGGL((skinny_dense_kernel<1, 1>), dim3(static_cast<unsigned>((wide.rows + 15) / 16), p.batch), block, 0,
-                         stream, q);
-    }
+    auto launch = [&](auto src_tag) {
+      constexpr int SRC = decltype(src_tag)::value;
+      if (wgs64 >= 200) {
+        hipLaunchKernelGGL((skinny_dense_kernel<SRC, 2, 2>), dim3(static_cast<unsigned>((wide.rows + 63) / 64), p.batch),
+                           block, 0, stream, q);
+      } else if (wgs64 * 2 >= 200) {
+        hipLaunchKernelGGL((skinny_dense_kernel<SRC, 1, 2>), dim3(static_cast<unsigned>((wide.rows + 31) / 32), p.batch),
+                           block, 0, stream, q);
+      } else {
+        hipLaunchKernelGGL((skinny_dense_kernel<SRC, 1, 1>), dim3(static_cast<unsigned>((wide.rows + 15) / 16), p.batch),
+                           block, 0, stream, q);
+      }
+    };
+    if (is_int) launch(std::integral_constant<int, SRC_I8>{});
+    else launch(std::integral_constant<int, SRC_BF16>{});
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(ST_EXEC, "skinny kernel launch: %s", hipGetErrorString(e));
     return ST_OK;
@@ -571,8 +589,11 @@ uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int64_t n, int64_t k)
   make_operand(&a, reinterpret_cast<void*>(16), DT_I8, m, k, k);
   make_operand(&b, reinterpret_cast<void*>(16), DT_I8, n, k, k);
   make_operand(&c, reinterpret_cast<void*>(16), DT_I32, m, n, n);
+  Problem pr;
+  if (describe(&a, &b, nullptr, &c, 0, &pr) != ST_OK) return 0;
+  pr.dequant = true;
   VecopsHipPlan plan;
-  if (vecops_hip_plan_matmul(&a, &b, nullptr, &c, 0, &plan) != ST_OK) return 0;
+  choose(pr, &plan);
   return plan.workspace_bytes;
 }
 
@@ -590,6 +611,7 @@ int32_t vecops_hip_matmul_i8_dequant(const int8_t* a, int64_t lda, const int8_t*
   Problem pr;
   int32_t rc = describe(&oa, &ob, nullptr, &oc, 0, &pr);
   if (rc != ST_OK) return rc;
+  pr.dequant = true;
   VecopsHipPlan plan;
   choose(pr, &plan);
   return run_problem(pr, plan, row_scales, column_scales, correction, workspace, workspace_size,

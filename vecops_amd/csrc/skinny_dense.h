@@ -1,19 +1,21 @@
-// Skinny bf16 matmul for gfx950 (HBM-bound): one operand has at most 16 rows.
+// Skinny matmul for gfx950 (HBM-bound): one operand has at most 16 rows.
 //   y[s, r] = sum_k x[s, k] * w[r, k]      w: the wide operand [R, K], x: the narrow one [S <= 16, K]
-// fp32 accumulation, both operands bf16 with K contiguous.  This is the GPU
-// counterpart of vecops' small-vector leaves (small_vector_dense_matmul /
-// small_vector_tall_matmul, matmul/details/kernel/amx/Backend.h:767-1151): the wide
-// operand is read exactly once, the narrow one is kept in registers.
+// bf16 x bf16 with fp32 accumulation, or int8 x int8 with wrapping int32 accumulation
+// (optionally followed by the per-row x per-column dequantisation); both operands K
+// contiguous.  This is the GPU counterpart of vecops' small-vector leaves
+// (small_vector_dense_matmul / small_vector_tall_matmul,
+// matmul/details/kernel/amx/Backend.h:767-1151): the wide operand is read exactly
+// once, the narrow one is kept in registers.
 //
-// One v_mfma_f32_16x16x32_bf16 multiplies 16 wide rows x 32 k by 32 k x 16 narrow rows
-// (S padded to 16 with zeros).  Lane l holds wide row l % 16 and the 8 consecutive k
-// of quarter l / 16 of a 32-element step (one 16-byte load); the narrow operand uses the
-// same k order.  A workgroup of 8 wavefronts owns PASSES x TILES blocks of 16 wide
-// rows; its wavefronts split K step by step (step t belongs to wavefront t % 8), so K
-// need only be a multiple of 8.  K is walked in blocks of 4096: a wavefront loads the
-// narrow fragments of its 16 steps of the block once (64 registers) and reuses them
-// for every row block.  Loads of the wide operand run D = 4 steps ahead.  The K
-// slices are summed through LDS at the end.
+// One v_mfma_f32_16x16x32_bf16 (v_mfma_i32_16x16x64_i8) multiplies 16 wide rows by 16
+// narrow rows (S padded to 16 with zeros) over a step of 32 (64) k.  Lane l holds wide
+// row l % 16 and the 16 consecutive bytes of quarter l / 16 of the step (one 16-byte
+// load); the narrow operand uses the same k order.  A workgroup of 8 wavefronts owns
+// PASSES x TILES blocks of 16 wide rows; its wavefronts split K step by step (step t
+// belongs to wavefront t % 8), so K need only be a multiple of 16 bytes.  K is walked
+// in blocks of 128 steps: a wavefront loads the narrow fragments of its 16 steps of the
+// block once (64 registers) and reuses them for every row block.  Loads of the wide
+// operand run D = 4 steps ahead.  The K slices are summed through LDS at the end.
 #ifndef VECOPS_HIP_SKINNY_DENSE_H
 #define VECOPS_HIP_SKINNY_DENSE_H
 
@@ -24,53 +26,65 @@
 
 namespace vecops_hip {
 
+enum SkinnyOut : int { SKINNY_OUT_F32 = 0, SKINNY_OUT_BF16 = 1, SKINNY_OUT_I32 = 2, SKINNY_OUT_DEQUANT_F32 = 3 };
+
 struct SkinnyDenseParams {
-  const uint16_t* w;  // wide operand, bf16 bits
-  const uint16_t* x;  // narrow operand, bf16 bits
-  void* y;            // fp32 or bf16
+  const void* w;      // wide operand (bf16 bits or int8)
+  const void* x;      // narrow operand
+  void* y;            // fp32, bf16 or int32
   int64_t ldw, ldx;   // row strides in elements
   int64_t w_bs, x_bs, y_bs;  // batch strides in elements (0 broadcasts an operand)
   int64_t y_stride_r;  // elements between consecutive wide rows in y
   int64_t y_stride_s;  // elements between consecutive narrow rows in y
+  // dequantisation (SKINNY_OUT_DEQUANT_F32): y = (float(acc + wide_term[r]) * narrow_scales[s]) * wide_scales[r]
+  const float* narrow_scales;
+  const float* wide_scales;
+  const int32_t* wide_term;  // null = none
   int32_t rows;        // R
   int32_t s;           // S, 1..16
-  int32_t k;           // multiple of 8
-  int32_t out_bf16;
+  int32_t k;           // multiple of 16 bytes of elements
+  int32_t out_kind;    // SkinnyOut
 };
 
-template <int PASSES, int TILES>
+template <int SRC, int PASSES, int TILES>
 __global__ __launch_bounds__(512) void skinny_dense_kernel(const SkinnyDenseParams p) {
-  constexpr int WAVES = 8, XS = 16, D = 4;  // XS steps of 32 k per wavefront and K block
+  constexpr bool INT = SrcTraits<SRC>::kInt;
+  constexpr int EPL = SrcTraits<SRC>::kElemsPerChunk;  // elements per lane and step (16 bytes)
+  constexpr int EPS = 4 * EPL;                         // elements per step
+  constexpr int EB = SrcTraits<SRC>::kSrcBytes;
+  using AccScalar = typename std::conditional<INT, int32_t, float>::type;
+  using Acc4 = typename std::conditional<INT, i32x4, f32x4>::type;
+  constexpr int WAVES = 8, XS = 16, D = 4;  // XS steps per wavefront and K block
   constexpr int BLOCKS = PASSES * TILES;    // 16-row blocks of this workgroup
-  __shared__ float red[WAVES][BLOCKS][16 * 16];
+  __shared__ AccScalar red[WAVES][BLOCKS][16 * 16];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int row = lane & 15, quarter = lane >> 4;
   const int batch = blockIdx.y;
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * (16 * BLOCKS);
   const int64_t last_row = static_cast<int64_t>(p.rows) - 1;
-  const VECOPS_GLOBAL uint16_t* wbase = (const VECOPS_GLOBAL uint16_t*)p.w + batch * p.w_bs;
-  const VECOPS_GLOBAL uint16_t* xrow =
-      (const VECOPS_GLOBAL uint16_t*)p.x + batch * p.x_bs + static_cast<int64_t>(min(row, p.s - 1)) * p.ldx;
+  const VECOPS_GLOBAL char* wbase = (const VECOPS_GLOBAL char*)p.w + batch * p.w_bs * EB;
+  const VECOPS_GLOBAL char* xrow =
+      (const VECOPS_GLOBAL char*)p.x + (batch * p.x_bs + static_cast<int64_t>(min(row, p.s - 1)) * p.ldx) * EB;
   // rows past R are clamped: computed, never stored
-  const VECOPS_GLOBAL uint16_t* wrow[BLOCKS];
+  const VECOPS_GLOBAL char* wrow[BLOCKS];
 #pragma unroll
-  for (int b = 0; b < BLOCKS; ++b) wrow[b] = wbase + min(row0 + b * 16 + row, last_row) * p.ldw;
+  for (int b = 0; b < BLOCKS; ++b) wrow[b] = wbase + min(row0 + b * 16 + row, last_row) * p.ldw * EB;
 
-  f32x4 acc[BLOCKS];
+  Acc4 acc[BLOCKS];
 #pragma unroll
-  for (int b = 0; b < BLOCKS; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int b = 0; b < BLOCKS; ++b) acc[b] = Acc4{0, 0, 0, 0};
 
-  const int k_blocks = (p.k + 4095) / 4096;
+  const int k_blocks = (p.k + 128 * EPS - 1) / (128 * EPS);
   for (int kb = 0; kb < k_blocks; ++kb) {
     // k of (step s of this wavefront, this lane's quarter) in this K block
-    auto k_of = [&](int s) { return (kb * 128 + s * WAVES + wave) * 32 + quarter * 8; };
+    auto k_of = [&](int s) { return (kb * 128 + s * WAVES + wave) * EPS + quarter * EPL; };
     u32x4 xq[XS];
 #pragma unroll
     for (int s = 0; s < XS; ++s) {
       const int k0 = k_of(s);
       xq[s] = u32x4{0u, 0u, 0u, 0u};
-      if (row < p.s && k0 < p.k) xq[s] = *(const VECOPS_GLOBAL u32x4*)(xrow + k0);
+      if (row < p.s && k0 < p.k) xq[s] = *(const VECOPS_GLOBAL u32x4*)(xrow + static_cast<int64_t>(k0) * EB);
     }
     // flat sequence of (block, step) with the wide loads D ahead; a load past K reads as zero
     u32x4 wq[D];
@@ -79,7 +93,7 @@ __global__ __launch_bounds__(512) void skinny_dense_kernel(const SkinnyDensePara
       if constexpr (b < BLOCKS) {
         const int k0 = k_of(s);
         wq[slot] = u32x4{0u, 0u, 0u, 0u};
-        if (k0 < p.k) wq[slot] = *(const VECOPS_GLOBAL u32x4*)(wrow[b] + k0);
+        if (k0 < p.k) wq[slot] = *(const VECOPS_GLOBAL u32x4*)(wrow[b] + static_cast<int64_t>(k0) * EB);
       }
     };
     static_for<D>([&](auto u) { issue(u, std::integral_constant<int, 0>{}, u); });
@@ -87,8 +101,12 @@ __global__ __launch_bounds__(512) void skinny_dense_kernel(const SkinnyDensePara
       constexpr int b = decltype(cb)::value;
       static_for<XS>([&](auto cs) {
         constexpr int s = decltype(cs)::value, slot = s % D;
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wq[slot]),
-                                                         __builtin_bit_cast(bf16x8, xq[s]), acc[b], 0, 0, 0);
+        if constexpr (INT)
+          acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, wq[slot]),
+                                                         __builtin_bit_cast(i32x4, xq[s]), acc[b], 0, 0, 0);
+        else
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wq[slot]),
+                                                           __builtin_bit_cast(bf16x8, xq[s]), acc[b], 0, 0, 0);
         constexpr int ns = s + D;  // the step that takes over this slot
         issue(std::integral_constant<int, slot>{}, std::integral_constant<int, b + ns / XS>{},
               std::integral_constant<int, ns % XS>{});
@@ -106,14 +124,27 @@ __global__ __launch_bounds__(512) void skinny_dense_kernel(const SkinnyDensePara
   for (int b = wave; b < BLOCKS; b += WAVES) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float total = 0.0f;
+      AccScalar total = 0;
 #pragma unroll
-      for (int w = 0; w < WAVES; ++w) total += red[w][b][(quarter * 4 + r) * 16 + row];
+      for (int w = 0; w < WAVES; ++w) {
+        if constexpr (INT) total = static_cast<int32_t>(static_cast<uint32_t>(total) + static_cast<uint32_t>(red[w][b][(quarter * 4 + r) * 16 + row]));
+        else total += red[w][b][(quarter * 4 + r) * 16 + row];
+      }
       const int64_t n = row0 + b * 16 + quarter * 4 + r;
       if (row < p.s && n < p.rows) {
         const int64_t at = batch * p.y_bs + n * p.y_stride_r + row * p.y_stride_s;
-        if (p.out_bf16) static_cast<uint16_t*>(p.y)[at] = static_cast<uint16_t>(bf16_bits_rne(total));
-        else static_cast<float*>(p.y)[at] = total;
+        if constexpr (INT) {
+          if (p.out_kind == SKINNY_OUT_DEQUANT_F32) {
+            const uint32_t term = p.wide_term ? static_cast<uint32_t>(p.wide_term[n]) : 0u;
+            const float t = static_cast<float>(static_cast<int32_t>(static_cast<uint32_t>(total) + term)) * p.narrow_scales[row];
+            static_cast<float*>(p.y)[at] = t * p.wide_scales[n];  // two separately rounded multiplies, row scale first
+          } else {
+            static_cast<int32_t*>(p.y)[at] = total;
+          }
+        } else {
+          if (p.out_kind == SKINNY_OUT_BF16) static_cast<uint16_t*>(p.y)[at] = static_cast<uint16_t>(bf16_bits_rne(total));
+          else static_cast<float*>(p.y)[at] = total;
+        }
       }
     }
   }
