@@ -191,6 +191,41 @@ def test_batched_and_broadcast(device, oracle):
                 torch.empty((0, m, n), dtype=torch.float32, device=device))
 
 
+def test_shared_b_batch_is_folded(device, oracle):
+    """One B for every batch and A / C rows running on from batch to batch: planned and run as a single
+    [batch * M, K] x B product (tests/ops/MatmulBatchTest.cpp:301-335), with a per-batch C input, a bias
+    row, and - rows not running on - the unfolded path giving the same values."""
+    import torch
+    from vecops_amd import capi
+    batch, m, n, k = 64, 32, 1024, 264
+    a = synth.bf16_round(synth.uniform_pm1(1, (batch, m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    cin = synth.uniform_pm1(3, (batch, m, n))
+    ta, tb = dev_bf16(a, device), dev_bf16(b, device)[None].expand(batch, n, k)
+    c = torch.full((batch, m, n), float("nan"), dtype=torch.float32, device=device)
+    folded = capi.plan_matmul(ta, tb, c)
+    apart = capi.plan_matmul(ta, dev_bf16(np.broadcast_to(b, (batch, n, k)).copy(), device), c)
+    assert capi.FAMILY_NAMES[folded.family] == "tile_128" and capi.FAMILY_NAMES[apart.family] == "tile_64"
+    hb = np.broadcast_to(b, (batch, n, k))
+    for c_in, h_in in ((None, None), (torch.from_numpy(cin).to(device), cin),
+                       (torch.from_numpy(cin[0, 0].copy()).to(device).expand(batch, m, n),
+                        np.broadcast_to(cin[0, 0], (batch, m, n)))):
+        c.fill_(float("nan"))
+        capi.matmul(ta, tb, c, c_in=c_in)
+        torch.cuda.synchronize()
+        want = np.zeros((batch, m, n), np.float32)
+        oracle.matmul(a, hb, want, cin=h_in, acc_f64=True)
+        assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+    # C with padded rows between batches: not foldable, same values
+    c_store = torch.full((batch, m + 3, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul(ta, tb, c_store[:, :m])
+    torch.cuda.synchronize()
+    want = np.zeros((batch, m, n), np.float32)
+    oracle.matmul(a, hb, want, acc_f64=True)
+    assert rel_err(c_store[:, :m].cpu().numpy(), want) <= fp32_tol(k)
+    assert torch.isnan(c_store[:, m:]).all()
+
+
 @pytest.mark.parametrize("m,n,k", [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)])
 def test_config3_irregular_batch8(device, oracle, m, n, k):
     """BASELINE config 3 at full size: batch 8, bf16 in, fp32 out.  All eight

@@ -146,6 +146,22 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
     else if (dc == DT_BF16) pr->out_kind = OUT_BF16;
     else return fail(ST_NOT_APPLICABLE, "matmul: floating operands need an f32 or bf16 c");
   }
+  // Rank 3 with one B for every batch and the rows of A and C (and C_in) running on from batch to batch:
+  // the same product as [batch * M, K] x B - folded into one rank-2 problem, which fills bigger tiles
+  // (vecops' shared-operand flattening, planning/families/ArchitectureFamily.h:430-463).
+  auto rows_run_on = [](const View& v) { return v.bs == v.rows * v.rs; };
+  if (pr->batch > 1 && pr->b.bs == 0 && pr->m > 0 && rows_run_on(pr->a) && rows_run_on(pr->c) &&
+      (!pr->has_cin || rows_run_on(pr->cin) || (pr->cin.bs == 0 && pr->cin.rs == 0)) &&
+      pr->batch * pr->m <= INT32_MAX) {
+    for (View* v : {&pr->a, &pr->c, &pr->cin}) {
+      v->rows *= pr->batch;
+      v->batch = 1;
+      v->bs = 0;
+    }
+    pr->b.batch = 1;
+    pr->m *= pr->batch;
+    pr->batch = 1;
+  }
   pr->cin_kind = pr->out_kind;
   if (pr->has_cin) {
     const uint32_t di = pr->cin.dtype;
