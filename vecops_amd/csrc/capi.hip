@@ -61,23 +61,22 @@ bool normalise(const VecopsHipOperand* o, View* v) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// 16-byte loads along K: unit K stride, row and batch strides and base all multiples of 16 bytes.
-// The kernels address a tile through a buffer descriptor based at its first row, with a 32-bit byte
-// offset per lane (up to 256 rows) plus the K offset: together they must stay below 2 GiB.
+// 16-byte loads along K: unit K stride.  Rows need not be 16-byte aligned: global and buffer loads
+// take any byte address on this target (the compiler itself emits dwordx4 loads for under-aligned
+// vectors); a misaligned chunk merely touches one more cache line.  The kernels address a tile
+// through a buffer descriptor based at its first row, with a 32-bit byte offset per lane (up to
+// 256 rows) plus the K offset: together they must stay below 2 GiB.
 bool k_vector_ok(const View& v) {
   const int64_t eb = dtype_bytes(v.dtype);
-  const int64_t per = 16 / eb;
-  return v.cs == 1 && v.rs >= 0 && v.rs % per == 0 && v.bs % per == 0 && aligned16(v.data) &&
-         (v.rs * 256 + v.cols + 256) * eb < (int64_t{1} << 31);
+  return v.cs == 1 && v.rs >= 0 && (v.rs * 256 + v.cols + 256) * eb < (int64_t{1} << 31);
 }
 
-// B stored [K,N] row-major: unit stride along N, N a multiple of 8 elements, K stride,
-// batch stride and base multiples of 16 bytes (16-bit or 32-bit source elements).
+// B stored [K,N] row-major: unit stride along N and N a multiple of 8 elements (the loader has no
+// N tail), 16-bit or 32-bit source elements.
 bool n_vector_ok(const View& v) {
   const int64_t eb = dtype_bytes(v.dtype);
-  const int64_t per = 16 / eb;
-  return v.rs == 1 && v.rows % 8 == 0 && v.rows >= 8 && v.cs > 0 && v.cs % per == 0 && v.bs % per == 0 &&
-         aligned16(v.data) && (v.cs * 64 + 512) * eb < (int64_t{1} << 31);  // 32-bit offsets inside a K tile
+  return v.rs == 1 && v.rows % 8 == 0 && v.rows >= 8 && v.cs > 0 &&
+         (v.cs * 64 + 512) * eb < (int64_t{1} << 31);  // 32-bit offsets inside a K tile
 }
 
 struct Problem {

@@ -280,9 +280,9 @@ __device__ __forceinline__ void mfma_step(typename AccTile<SrcTraits<SRC>::kInt>
 //   int:  v = acc + correction[col] + cin  (wrapping);  c = v  or
 //         c = (float(v) * row_scales[row]) * column_scales[col]
 //         (vecops matmul/Quantization.h:224-231: two multiplies, row first).
+// Returns the 32-bit pattern of the output element (fp32 or int32), or its bf16 bits.
 template <bool INT, typename AccScalar>
-__device__ __forceinline__ void store_output(const TileGemmParams& p, int batch, int row, int col, AccScalar acc) {
-  const int64_t c_off = batch * p.c_bs + row * p.c_rs + col * p.c_cs;
+__device__ __forceinline__ uint32_t output_bits(const TileGemmParams& p, int batch, int row, int col, AccScalar acc) {
   if constexpr (INT) {
     uint32_t v = static_cast<uint32_t>(acc) + p.const_term;
     if (p.row_term) v += static_cast<uint32_t>(p.row_term[static_cast<int64_t>(batch) * p.m + row]);
@@ -293,12 +293,10 @@ __device__ __forceinline__ void store_output(const TileGemmParams& p, int batch,
     const int32_t s = static_cast<int32_t>(v);
     if (p.row_scales) {
       const float t = static_cast<float>(s) * p.row_scales[row];
-      static_cast<float*>(p.c)[c_off] = t * p.column_scales[col];
-    } else if (p.out_kind == OUT_I32) {
-      static_cast<int32_t*>(p.c)[c_off] = s;
-    } else {
-      static_cast<float*>(p.c)[c_off] = static_cast<float>(s);
+      return __float_as_uint(t * p.column_scales[col]);
     }
+    if (p.out_kind == OUT_I32) return v;
+    return __float_as_uint(static_cast<float>(s));
   } else {
     float v = acc;
     if (p.cin) {
@@ -306,34 +304,58 @@ __device__ __forceinline__ void store_output(const TileGemmParams& p, int batch,
       v += (p.cin_kind == OUT_BF16) ? bf16_bits_to_f32(static_cast<const uint16_t*>(p.cin)[ci])
                                     : static_cast<const float*>(p.cin)[ci];
     }
-    if (p.out_kind == OUT_BF16) {
-      static_cast<uint16_t*>(p.c)[c_off] = static_cast<uint16_t>(bf16_bits_rne(v));
-    } else {
-      static_cast<float*>(p.c)[c_off] = v;
-    }
+    return p.out_kind == OUT_BF16 ? bf16_bits_rne(v) : __float_as_uint(v);
   }
 }
 
-// One lane's 16 accumulators of a 32x32 tile through the full epilogue, with
-// bounds checks; out of line to keep the kernels small (edge tiles, split-K
-// partials, C-input and strided C only).  The lane owns output row `row` and
-// columns col0 + (r/4)*8 + r%4.
+template <bool INT, typename AccScalar>
+__device__ __forceinline__ void store_output(const TileGemmParams& p, int batch, int row, int col, AccScalar acc) {
+  const int64_t c_off = batch * p.c_bs + row * p.c_rs + col * p.c_cs;
+  const uint32_t bits = output_bits<INT, AccScalar>(p, batch, row, col, acc);
+  if (!INT && p.out_kind == OUT_BF16) static_cast<uint16_t*>(p.c)[c_off] = static_cast<uint16_t>(bits);
+  else static_cast<uint32_t*>(p.c)[c_off] = bits;
+}
+
+// Four consecutive columns of one output row through the full epilogue, with bounds
+// checks (edge tiles, split-K partials, C-input and strided C): `raw` holds the four
+// accumulators (fp32 or int32 bit patterns) of C[row][col .. col+3].  One 16-byte
+// (bf16: 8-byte) store when the run lies inside C and C's rows are contiguous and
+// aligned, else element by element.
 template <bool INT>
-__device__ __noinline__ void store_tile_general(const TileGemmParams& p, int batch, int split, int row, int col0,
-                                                typename AccTile<INT>::type tile) {
+__device__ __forceinline__ void store_quad_general(const TileGemmParams& p, int batch, int split, int row, int col,
+                                                   const u32x4& raw, bool vec_c, bool vec_partial) {
   using AccScalar = typename std::conditional<INT, int32_t, float>::type;
-  if (row >= p.m) return;
+  if (row >= p.m || col >= p.n) return;
+  auto value = [&](int e) {
+    if constexpr (INT) return static_cast<int32_t>(raw[e]);
+    else return __uint_as_float(raw[e]);
+  };
+  if (p.split_k > 1) {
+    uint32_t* part = static_cast<uint32_t*>(p.partial) +
+                     ((static_cast<int64_t>(split) * p.batch + batch) * p.m + row) * p.n + col;
+    if (vec_partial && col + 3 < p.n) {
+      *reinterpret_cast<u32x4*>(part) = raw;
+    } else {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int col = col0 + (r >> 2) * 8 + (r & 3);
-    if (col < p.n) {
-      if (p.split_k > 1) {
-        AccScalar* part = static_cast<AccScalar*>(p.partial);
-        part[((static_cast<int64_t>(split) * p.batch + batch) * p.m + row) * p.n + col] = tile[r];
-      } else {
-        store_output<INT, AccScalar>(p, batch, row, col, tile[r]);
-      }
+      for (int e = 0; e < 4; ++e)
+        if (col + e < p.n) part[e] = raw[e];
     }
+    return;
+  }
+  const bool bf16_out = !INT && p.out_kind == OUT_BF16;
+  if (vec_c && col + 3 < p.n) {
+    uint32_t bits[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bits[e] = output_bits<INT, AccScalar>(p, batch, row, col + e, value(e));
+    const int64_t c_off = batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col;
+    if (bf16_out)
+      *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.c) + c_off) = u32x2{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16)};
+    else
+      *reinterpret_cast<u32x4*>(static_cast<uint32_t*>(p.c) + c_off) = u32x4{bits[0], bits[1], bits[2], bits[3]};
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (col + e < p.n) store_output<INT, AccScalar>(p, batch, row, col + e, value(e));
   }
 }
 
@@ -769,10 +791,19 @@ constexpr int kStageBytes() {
 
 // Dynamic LDS one workgroup is launched with: two staging stages, or the bf16
 // epilogue's row-major tiles if those are larger.
+// LDS the epilogues lay accumulators out in: the bf16 path's row-major tiles, and one 32-row block of
+// 32-bit values per wavefront for the general path.
+template <int WAVES_M, int WAVES_N, int WM, int WN>
+constexpr int kEpilogueLdsBytes() {
+  const int bf16_tiles = (WN * 32 * 2 + 16) * (WM * 32) * WAVES_M * WAVES_N;
+  const int general = 32 * (WN * 32 + 4) * 4 * WAVES_M * WAVES_N;
+  return bf16_tiles > general ? bf16_tiles : general;
+}
+
 template <int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_B>
 constexpr int kTileLdsBytes() {
   const int stages = 2 * kStageBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>();
-  const int epilogue = (WN * 32 * 2 + 16) * (WM * 32) * WAVES_M * WAVES_N;
+  const int epilogue = kEpilogueLdsBytes<WAVES_M, WAVES_N, WM, WN>();
   return stages > epilogue ? stages : epilogue;
 }
 
@@ -887,13 +918,37 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
       });
     });
   } else {
+    // Everything else (edge tiles, C-input, split-K partials, strided or unaligned C, unsigned-operand
+    // terms): each wavefront lays one 32-row block of its accumulators out row-major in LDS and walks it
+    // in a rolled loop, a lane taking four consecutive columns of one row per step - one copy of the
+    // general store code, and stores that run along rows.
+    constexpr int COLS = WN * 32, QUADS = COLS / 4;
+    constexpr int PITCH = COLS + 4;  // 32-bit words; the pad staggers rows across banks
+    static_assert(32 * PITCH * 4 * WAVES_M * WAVES_N <= LDS_BYTES, "general epilogue staging must fit the launch's LDS");
+    __syncthreads();  // every wavefront is done reading fragments
+    uint32_t* mine = reinterpret_cast<uint32_t*>(lds) + wave * (32 * PITCH);
+    const bool bf16_out = !INT && p.out_kind == OUT_BF16;
+    const bool vec_c = p.c_cs == 1 && (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 &&
+                       (reinterpret_cast<uintptr_t>(p.c) & (bf16_out ? 7 : 15)) == 0;
+    const bool vec_partial = (p.n & 3) == 0 && (reinterpret_cast<uintptr_t>(p.partial) & 15) == 0;
     static_for<WM>([&](auto ci) {
       constexpr int i = decltype(ci)::value;
       static_for<WN>([&](auto cj) {
         constexpr int j = decltype(cj)::value;
-        store_tile_general<INT>(p, batch, split, m0 + (wm * WM + i) * 32 + frag_row,
-                                n0 + (wn * WN + j) * 32 + frag_half * 4, acc[i][j]);
+        static_for<4>([&](auto cq) {
+          constexpr int q = decltype(cq)::value;
+          const auto v = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
+          *reinterpret_cast<u32x4*>(mine + frag_row * PITCH + j * 32 + q * 8 + frag_half * 4) = __builtin_bit_cast(u32x4, v);
+        });
       });
+      // the wavefront reads back only what it wrote itself: its own LDS traffic is ordered
+      const int row_base = m0 + (wm * WM + i) * 32, col_base = n0 + wn * COLS;
+#pragma unroll 1
+      for (int idx = lane; idx < 32 * QUADS; idx += 64) {
+        const int r = idx / QUADS, cq = idx % QUADS;
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(mine + r * PITCH + cq * 4);
+        store_quad_general<INT>(p, batch, split, row_base + r, col_base + cq * 4, raw, vec_c, vec_partial);
+      }
     });
   }
 }

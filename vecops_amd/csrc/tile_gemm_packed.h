@@ -90,7 +90,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
   constexpr int BM = 32 * WAVES_M * WM, BN = 32 * WAVES_N * WN;
   constexpr int STAGE_BYTES = BM * 128;
   constexpr int N_MFMA = WM * WN;
-  constexpr int kEpilogueBytes = (WN * 32 * 2 + 16) * (WM * 32) * WAVES_M * WAVES_N;
+  constexpr int kEpilogueBytes = kEpilogueLdsBytes<WAVES_M, WAVES_N, WM, WN>();
   constexpr int kLdsBytes = 2 * STAGE_BYTES > kEpilogueBytes ? 2 * STAGE_BYTES : kEpilogueBytes;
 
   extern __shared__ __attribute__((aligned(16))) char lds[];

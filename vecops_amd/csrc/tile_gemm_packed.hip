@@ -8,7 +8,7 @@ namespace {
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA>
 hipError_t launch_packed_instance(const TileGemmParams& p, hipStream_t stream) {
   constexpr int kStages = 2 * (32 * WAVES_M * WM) * 128;
-  constexpr int kEpilogue = (WN * 32 * 2 + 16) * (WM * 32) * WAVES_M * WAVES_N;
+  constexpr int kEpilogue = kEpilogueLdsBytes<WAVES_M, WAVES_N, WM, WN>();
   constexpr int kLds = kStages > kEpilogue ? kStages : kEpilogue;
   auto kernel = tile_gemm_packed_b_kernel<SRC, WAVES_M, WAVES_N, WM, WN, LA>;
   static thread_local int configured_device = -1;
