@@ -239,6 +239,51 @@ __device__ __noinline__ Staged<SRC> load_chunk_checked(const void* base, int64_t
   }
 }
 
+// A whole K-contiguous operand tile (rows x eight chunks), every element bounds-checked, straight into
+// its LDS tile: the partial last K tile.  Out of line and rolled - it runs once per workgroup - and
+// one call per operand: a call has to wait for its loads before it returns, so chunk-by-chunk calls
+// would pay one memory round trip each.
+template <int SRC>
+__device__ __noinline__ void stage_rows_checked(const void* base, int64_t rs, int64_t kstep, int first_row, int extent,
+                                                int rows, int k0_tile, int k_end, char* lds_tile, int tid,
+                                                int threads, uint32_t flip) {
+  constexpr int EPC = SrcTraits<SRC>::kElemsPerChunk;
+#pragma unroll 2
+  for (int idx = tid; idx < rows * 8; idx += threads) {
+    const int row = idx >> 3, chunk = idx & 7;
+    const int k0 = k0_tile + chunk * EPC;
+    const bool row_ok = first_row + row < extent;
+    const int64_t row_off = static_cast<int64_t>(first_row + row) * rs;
+    u32x4 out;
+    if constexpr (SRC == SRC_F32_AS_BF16) {
+      float f[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int k = k0 + e;
+        f[e] = (row_ok && k < k_end) ? static_cast<const float*>(base)[row_off + k * kstep] : 0.0f;
+      }
+      out = u32x4{cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3]), cvt_pk_bf16(f[4], f[5]), cvt_pk_bf16(f[6], f[7])};
+    } else {
+      uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int e = 0; e < EPC; ++e) {
+        const int k = k0 + e;
+        uint32_t v = flip & 0xffu;  // an element outside the operand: the flip byte, which the xor below turns into 0
+        if (row_ok && k < k_end) {
+          if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
+          else if constexpr (SRC == SRC_F32) v = __float_as_uint(static_cast<const float*>(base)[row_off + k * kstep]);
+          else v = static_cast<const uint8_t*>(base)[row_off + k * kstep];
+        }
+        constexpr int per_word = EPC / 4;
+        w[e / per_word] |= v << ((e % per_word) * (32 / per_word));
+      }
+      out = u32x4{w[0], w[1], w[2], w[3]};
+      if constexpr (SRC == SRC_I8_FLIP) out ^= u32x4{flip, flip, flip, flip};
+    }
+    *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(row, chunk)) = out;
+  }
+}
+
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
   if constexpr (N > 0) {
@@ -470,7 +515,15 @@ struct Stager {
     }
   }
 
-  // Whole tile, every element bounds-checked: the partial last K tile.
+  // The partial last K tile, bounds-checked, straight into its LDS tile (no registers involved).
+  // (not for fp32 held as loaded: its 256x256 instances have no register to spare for the extra path)
+  static constexpr bool kStagesChecked = SRC != SRC_F32_AS_BF16;
+  __device__ __forceinline__ void stage_checked(int kt, char* lds_tile) const {
+    stage_rows_checked<SRC>(base, rs, ks, first_row, extent, ROWS, kt * 8 * T::kElemsPerChunk, k_end, lds_tile,
+                            ld_row * 8 + ld_chunk, THREADS, flip);
+  }
+
+  // Whole tile, every element bounds-checked, into the staging registers.
   __device__ __forceinline__ void fetch_checked(int kt) {
     const int k0 = kt * 8 * T::kElemsPerChunk + ld_chunk * T::kElemsPerChunk;
 #pragma unroll
@@ -525,6 +578,8 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
   static constexpr int kStoreOps = 1;
   static constexpr int kLoadOps = 1;
   static constexpr bool kHasSpare = SRC != SRC_F32_AS_BF16;
+  static constexpr bool kStagesChecked = false;
+  __device__ __forceinline__ void stage_checked(int, char*) const {}
   const char* base;
   const VECOPS_GLOBAL char* tile_base;  // (k = 0, first n of the tile), wavefront-uniform
   static_assert(THREADS % CHUNKS_PER_ROW == 0, "every part of a thread is the same chunk, THREADS / CHUNKS_PER_ROW k rows on");
@@ -643,6 +698,8 @@ struct Stager<SRC_F32, LOAD_NVEC, ROWS, THREADS> {
   static constexpr int kStoreOps = 4;
   static constexpr int kLoadOps = 4;
   static constexpr bool kHasSpare = false;
+  static constexpr bool kStagesChecked = false;
+  __device__ __forceinline__ void stage_checked(int, char*) const {}
   struct Spare {};
   const char* base;
   const VECOPS_GLOBAL char* tile_base;
@@ -1083,12 +1140,15 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
     // (scalar tile indices: a load whose uniform offset sits in a vector register is wrapped in a loop)
     const int first = __builtin_amdgcn_readfirstlane(seq(0));
     const int second = __builtin_amdgcn_readfirstlane(seq(nk > 1 ? 1 : 0));
-    if (first < full_k_tiles) {
+    const bool tail_first = first >= full_k_tiles;
+    if (!tail_first) {
       stager_a.fetch_full(first);
       stager_b.fetch_full(first);
     } else {
-      stager_a.fetch_checked(first);
-      stager_b.fetch_checked(first);
+      if constexpr (SA::kStagesChecked) stager_a.stage_checked(first, lds);
+      else stager_a.fetch_checked(first);
+      if constexpr (SB::kStagesChecked) stager_b.stage_checked(first, lds + BM * 128);
+      else stager_b.fetch_checked(first);
     }
     typename SA::Spare spare_a;
     typename SB::Spare spare_b;
@@ -1096,8 +1156,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
       if constexpr (SA::kHasSpare) stager_a.fetch_full_spare(spare_a, second);
       if constexpr (SB::kHasSpare) stager_b.fetch_full_spare(spare_b, second);
     }
-    stager_a.commit(lds);
-    stager_b.commit(lds + BM * 128);
+    if (!(SA::kStagesChecked && tail_first)) stager_a.commit(lds);
+    if (!(SB::kStagesChecked && tail_first)) stager_b.commit(lds + BM * 128);
     if (nk > 1) {
       if constexpr (SA::kHasSpare) stager_a.take_spare(spare_a);
       else stager_a.fetch_full(second);
@@ -1116,7 +1176,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
 
   if (nk > 0) {
     const int full_in_range = nk - has_tail;  // whole K tiles this workgroup owns
-    if constexpr (SRC == SRC_F32_AS_BF16) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    // Every load of the start-up has landed before the loop is entered: the compiler's wait insertion
+    // merges the start-up's branches without knowing which conditions coincide, and would otherwise
+    // carry loads "still in flight" into the loop and wait for them in every iteration.
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
     lds_barrier();  // tile 0 is in LDS
     read_frags(0, lds, 0);
 

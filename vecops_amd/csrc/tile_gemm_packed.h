@@ -156,14 +156,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
   if (nk > 0) {
     const int first = __builtin_amdgcn_readfirstlane(seq(0));
     const int second = __builtin_amdgcn_readfirstlane(seq(nk > 1 ? 1 : 0));
-    if (first < full_k_tiles) stager_a.fetch_full(first);
+    const bool tail_first = first >= full_k_tiles;
+    if (!tail_first) stager_a.fetch_full(first);
+    else if constexpr (SA::kStagesChecked) stager_a.stage_checked(first, lds);
     else stager_a.fetch_checked(first);
     static_for<4>([&](auto cks) { static_for<WN>([&](auto cj) { load_b(cks, cj, first); }); });
     typename SA::Spare spare_a;
     if (nk > 1) {
       if constexpr (SA::kHasSpare) stager_a.fetch_full_spare(spare_a, second);
     }
-    stager_a.commit(lds);
+    if (!(SA::kStagesChecked && tail_first)) stager_a.commit(lds);
     if (nk > 1) {
       if constexpr (SA::kHasSpare) stager_a.take_spare(spare_a);
       else stager_a.fetch_full(second);
