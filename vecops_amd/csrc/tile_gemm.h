@@ -974,6 +974,23 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
         });
       });
     });
+  } else if (interior && p.split_k > 1 && (p.n & 3) == 0 && (reinterpret_cast<uintptr_t>(p.partial) & 15) == 0) {
+    // split-K partial sums of an interior tile: raw accumulators, 16 bytes per store
+    static_for<WM>([&](auto ci) {
+      constexpr int i = decltype(ci)::value;
+      const int row = m0 + (wm * WM + i) * 32 + frag_row;
+      uint32_t* dst_row = static_cast<uint32_t*>(p.partial) +
+                          ((static_cast<int64_t>(split) * p.batch + batch) * p.m + row) * p.n;
+      static_for<WN>([&](auto cj) {
+        constexpr int j = decltype(cj)::value;
+        uint32_t* dst = dst_row + n0 + (wn * WN + j) * 32 + frag_half * 4;
+        static_for<4>([&](auto cq) {
+          constexpr int q = decltype(cq)::value;
+          const auto v = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
+          *reinterpret_cast<typename std::remove_const<decltype(v)>::type*>(dst + q * 8) = v;
+        });
+      });
+    });
   } else {
     // Everything else (edge tiles, C-input, split-K partials, strided or unaligned C, unsigned-operand
     // terms): each wavefront lays one 32-row block of its accumulators out row-major in LDS and walks it
@@ -1259,6 +1276,30 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const TileGemmParams
   const int64_t per_batch = static_cast<int64_t>(p.m) * p.n;
   const int64_t total = per_batch * p.batch;
   const AccScalar* part = static_cast<const AccScalar*>(p.partial);
+  // four consecutive columns of a row per thread when rows hold whole quads (16-byte loads of the
+  // partials, one 16-byte or 8-byte store), else element by element
+  const bool quads = (p.n & 3) == 0 && (reinterpret_cast<uintptr_t>(p.partial) & 15) == 0;
+  if (quads) {
+    const bool bf16_out = !INT && p.out_kind == OUT_BF16;
+    const bool vec_c = p.c_cs == 1 && (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 &&
+                       (reinterpret_cast<uintptr_t>(p.c) & (bf16_out ? 7 : 15)) == 0;
+    typedef AccScalar Vec4 __attribute__((ext_vector_type(4)));
+    TileGemmParams q = p;  // split_k is > 1 here, or 0 (the empty sum): the sums leave through the final epilogue
+    q.split_k = 1;
+    for (int64_t idx = (blockIdx.x * 256ll + threadIdx.x) * 4; idx < total; idx += gridDim.x * 1024ll) {
+      const int batch = static_cast<int>(idx / per_batch);
+      const int64_t rem = idx - batch * per_batch;
+      const int row = static_cast<int>(rem / p.n), col = static_cast<int>(rem - static_cast<int64_t>(row) * p.n);
+      Vec4 sum = {0, 0, 0, 0};
+      for (int s = 0; s < p.split_k; ++s) {
+        const Vec4 v = *reinterpret_cast<const Vec4*>(part + s * total + idx);
+        if constexpr (INT) sum = __builtin_bit_cast(Vec4, __builtin_bit_cast(u32x4, sum) + __builtin_bit_cast(u32x4, v));
+        else sum += v;
+      }
+      store_quad_general<INT>(q, batch, 0, row, col, __builtin_bit_cast(u32x4, sum), vec_c, false);
+    }
+    return;
+  }
   for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += gridDim.x * 256ll) {
     const int batch = static_cast<int>(idx / per_batch);
     const int64_t rem = idx - batch * per_batch;
