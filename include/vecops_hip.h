@@ -58,7 +58,9 @@ typedef enum VecopsHipKernelFamily {
   VECOPS_HIP_FAMILY_TILE_128 = 2,      /* 128x128 workgroup tile, MFMA */
   VECOPS_HIP_FAMILY_TILE_64 = 3,       /* 64x64 workgroup tile, MFMA */
   VECOPS_HIP_FAMILY_SKINNY = 4,        /* one side <= 16 rows: wavefronts split K, the wide operand is read once */
-  VECOPS_HIP_FAMILY_ZERO_K = 5         /* K == 0: C = Cin or zeros */
+  VECOPS_HIP_FAMILY_ZERO_K = 5,        /* K == 0: C = Cin or zeros */
+  VECOPS_HIP_FAMILY_TILE_256X128 = 6,  /* 256 (M) x 128 (N) workgroup tile, MFMA */
+  VECOPS_HIP_FAMILY_TILE_128X256 = 7   /* 128 (M) x 256 (N) workgroup tile, MFMA */
 } VecopsHipKernelFamily;
 
 typedef struct VecopsHipPlan {

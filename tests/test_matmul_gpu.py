@@ -205,7 +205,8 @@ def test_shared_b_batch_is_folded(device, oracle):
     c = torch.full((batch, m, n), float("nan"), dtype=torch.float32, device=device)
     folded = capi.plan_matmul(ta, tb, c)
     apart = capi.plan_matmul(ta, dev_bf16(np.broadcast_to(b, (batch, n, k)).copy(), device), c)
-    assert capi.FAMILY_NAMES[folded.family] == "tile_128" and capi.FAMILY_NAMES[apart.family] == "tile_64"
+    assert capi.FAMILY_NAMES[folded.family] in ("tile_128", "tile_256x128", "tile_128x256")
+    assert capi.FAMILY_NAMES[apart.family] == "tile_64"
     hb = np.broadcast_to(b, (batch, n, k))
     for c_in, h_in in ((None, None), (torch.from_numpy(cin).to(device), cin),
                        (torch.from_numpy(cin[0, 0].copy()).to(device).expand(batch, m, n),

@@ -179,6 +179,7 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
 }
 
 constexpr int kComputeUnits = 256;
+constexpr int64_t kQuality256x128 = 880, kQuality128 = 770;  // see choose()
 
 // bf16 x bf16 or int8 x int8 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
 bool skinny_applies(const Problem& pr) {
@@ -224,36 +225,44 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     return;
   }
 
-  auto tiles = [&](int64_t t) { return ((pr.m + t - 1) / t) * ((pr.n + t - 1) / t) * pr.batch; };
-  uint32_t family;
-  int64_t tile;
-  // share of the compute-unit rounds a tiling fills: tiles / (rounds * 256)
-  auto fill_per_mille = [&](int64_t t) {
-    const int64_t count = tiles(t), rounds = (count + kComputeUnits - 1) / kComputeUnits;
-    return count * 1000 / (rounds * kComputeUnits);
-  };
-  // A 128x128 tile does 0.77 of the 256x256 tile's work per compute unit and second (measured, bf16
-  // 2048x2048x4096 against 4096^3); it is preferred when its fuller rounds outweigh that by 10 %
-  // (4096x4224: 272 big tiles fill 53 % of two rounds, 1056 small ones 83 % of five).
-  const bool small_fills_better = fill_per_mille(128) * 77 > fill_per_mille(256) * 110;
-  if (pr.m > 128 && pr.n > 128 && tiles(256) >= kComputeUnits * 3 / 4 && !small_fills_better) {
-    family = VECOPS_HIP_FAMILY_TILE_256;
-    tile = 256;
-  } else if (pr.m > 64 && pr.n > 64 && tiles(128) >= kComputeUnits / 2) {
-    family = VECOPS_HIP_FAMILY_TILE_128;
-    tile = 128;
-  } else {
-    family = VECOPS_HIP_FAMILY_TILE_64;
-    tile = 64;
-    if (pr.m > 64 && pr.n > 64 && tiles(64) > 4 * kComputeUnits) {
-      family = VECOPS_HIP_FAMILY_TILE_128;
-      tile = 128;
+  auto tiles2 = [&](int64_t tm, int64_t tn) { return ((pr.m + tm - 1) / tm) * ((pr.n + tn - 1) / tn) * pr.batch; };
+  auto tiles = [&](int64_t t) { return tiles2(t, t); };
+  // Candidate workgroup tiles with the work each does per compute unit and second relative to 256x256
+  // (per mille; measured on bf16 problems that fill exactly one round).  A candidate must keep at least
+  // half the compute units busy; among those the cheapest wins, cost = rounds x tile area / quality -
+  // so a part-filled last round, rows or columns of padding and a less efficient small tile are all
+  // priced in one number (4096^3: 256 tiles of 256x256, one round; 2048x11008: 688 tiles of 256x128 in
+  // three rounds instead of 344 big ones in two; 8 x 777x1000: 256 tiles of 256x128, one round).
+  struct Candidate { uint32_t family; int64_t tm, tn, quality; };
+  const Candidate candidates[] = {{VECOPS_HIP_FAMILY_TILE_256, 256, 256, 1000},
+                                  {VECOPS_HIP_FAMILY_TILE_256X128, 256, 128, kQuality256x128},
+                                  {VECOPS_HIP_FAMILY_TILE_128X256, 128, 256, kQuality256x128},
+                                  {VECOPS_HIP_FAMILY_TILE_128, 128, 128, kQuality128}};
+  uint32_t family = VECOPS_HIP_FAMILY_TILE_64;
+  int64_t tile_m = 64, tile_n = 64, best_cost = INT64_MAX;
+  for (const Candidate& c : candidates) {
+    if (pr.m <= c.tm / 2 || pr.n <= c.tn / 2) continue;  // a tile more than half empty in one direction
+    const int64_t count = tiles2(c.tm, c.tn);
+    if (count < kComputeUnits / 2) continue;
+    const int64_t rounds = (count + kComputeUnits - 1) / kComputeUnits;
+    const int64_t cost = rounds * c.tm * c.tn * 1000 / c.quality;
+    // a smaller tile has to be 10 % cheaper: a part-filled round of big tiles runs faster than the count
+    // says (the chip is power-limited; 3000^3 as 144 big tiles beats 576 small ones in three rounds)
+    if (best_cost == INT64_MAX || cost * 11 < best_cost * 10) {
+      best_cost = cost;
+      family = c.family;
+      tile_m = c.tm;
+      tile_n = c.tn;
     }
+  }
+  if (family == VECOPS_HIP_FAMILY_TILE_64 && pr.m > 64 && pr.n > 64 && tiles(64) > 4 * kComputeUnits) {
+    family = VECOPS_HIP_FAMILY_TILE_128;
+    tile_m = tile_n = 128;
   }
   plan->family = family;
   const int64_t ktile = k_tile_elements(pr.src);
   const int64_t k_tiles = (pr.k + ktile - 1) / ktile;
-  const int64_t wgs = tiles(tile);
+  const int64_t wgs = tiles2(tile_m, tile_n);
   int64_t split = 1;
   if (wgs < kComputeUnits / 2 && k_tiles >= 8) {
     split = kComputeUnits / wgs;
@@ -357,10 +366,17 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     return ST_OK;
   }
 
-  const int tile = plan.family == VECOPS_HIP_FAMILY_TILE_256 ? 256 : plan.family == VECOPS_HIP_FAMILY_TILE_128 ? 128 : 64;
+  int tile_m = 64, tile_n = 64;
+  switch (plan.family) {
+    case VECOPS_HIP_FAMILY_TILE_256: tile_m = tile_n = 256; break;
+    case VECOPS_HIP_FAMILY_TILE_256X128: tile_m = 256; tile_n = 128; break;
+    case VECOPS_HIP_FAMILY_TILE_128X256: tile_m = 128; tile_n = 256; break;
+    case VECOPS_HIP_FAMILY_TILE_128: tile_m = tile_n = 128; break;
+    default: break;
+  }
   const int ktile = k_tile_elements(pr.src);
-  p.tiles_m = static_cast<int32_t>((pr.m + tile - 1) / tile);
-  p.tiles_n = static_cast<int32_t>((pr.n + tile - 1) / tile);
+  p.tiles_m = static_cast<int32_t>((pr.m + tile_m - 1) / tile_m);
+  p.tiles_n = static_cast<int32_t>((pr.n + tile_n - 1) / tile_n);
   const int k_tiles = static_cast<int>((pr.k + ktile - 1) / ktile);
   p.split_k = static_cast<int32_t>(plan.split_k);
   p.k_tiles_per_split = (k_tiles + p.split_k - 1) / p.split_k;
@@ -389,13 +405,13 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     if (pr.a_unsigned && pr.b_unsigned) p.const_term = 16384u * static_cast<uint32_t>(pr.k);
   }
   if (pr.packed_b) {
-    e = launch_tile_gemm_packed_b(pr.src, p, tile, plan.vector_a != 0, stream);
+    e = launch_tile_gemm_packed_b(pr.src, p, tile_m, tile_n, plan.vector_a != 0, stream);
   } else switch (pr.src) {
-    case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile, mode, stream); break;
-    case SRC_BF16: e = launch_tile_gemm_bf16(p, tile, mode, stream); break;
-    case SRC_F32_AS_BF16: e = launch_tile_gemm_f32_as_bf16(p, tile, mode, stream); break;
-    case SRC_F32: e = launch_tile_gemm_f32(p, tile, mode, stream); break;
-    default: e = launch_tile_gemm_i8(p, tile, mode, stream); break;
+    case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile_m, tile_n, mode, stream); break;
+    case SRC_BF16: e = launch_tile_gemm_bf16(p, tile_m, tile_n, mode, stream); break;
+    case SRC_F32_AS_BF16: e = launch_tile_gemm_f32_as_bf16(p, tile_m, tile_n, mode, stream); break;
+    case SRC_F32: e = launch_tile_gemm_f32(p, tile_m, tile_n, mode, stream); break;
+    default: e = launch_tile_gemm_i8(p, tile_m, tile_n, mode, stream); break;
   }
   if (e != hipSuccess) return fail(ST_EXEC, "tile kernel launch: %s", hipGetErrorString(e));
   if (p.split_k > 1) {

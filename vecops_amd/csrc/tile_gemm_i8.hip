@@ -1,8 +1,8 @@
 // int8 x int8 -> int32 tile GEMM instances and the split-K reduction kernels.
 #include "tile_gemm_launch.h"
 namespace vecops_hip {
-hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile, int mode, hipStream_t stream) {
-  return launch_tile_class<SRC_I8>(p, tile, mode, stream);
+hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream) {
+  return launch_tile_class<SRC_I8>(p, tile_m, tile_n, mode, stream);
 }
 
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream) {

@@ -16,21 +16,22 @@ enum LoadMode : int {
   MODE_NVEC_B = 2    // A K-contiguous; B stored [K,N] row-major, 16-byte aligned (16- and 32-bit compute types)
 };
 
-// tile: 256, 128 or 64 (workgroup tile edge).  Returns the HIP error of the
-// launch (hipSuccess when enqueued).
-hipError_t launch_tile_gemm_bf16(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
-hipError_t launch_tile_gemm_f32_as_bf16(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
-hipError_t launch_tile_gemm_f32(const TileGemmParams& p, int tile, int mode, hipStream_t stream);  // fp32 compute
-hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
+// tile_m x tile_n: 256x256, 256x128, 128x256, 128x128 or 64x64 (the workgroup tile).  Returns the HIP
+// error of the launch (hipSuccess when enqueued).
+hipError_t launch_tile_gemm_bf16(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
+hipError_t launch_tile_gemm_f32_as_bf16(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
+hipError_t launch_tile_gemm_f32(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);  // fp32 compute
+hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
 // 8-bit operands of which at least one is unsigned (p.a_flip / p.b_flip and the epilogue terms set)
-hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile, int mode, hipStream_t stream);
+hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
 // out[b][r] = scale * sum_k int8(x[b][r][k] xor flip): the epilogue terms of an unsigned operand
 hipError_t launch_byte_row_sums(const void* x, int32_t batch, int32_t rows, int32_t k, int64_t bs, int64_t rs,
                                 int64_t ks, uint32_t flip, uint32_t scale, int32_t* out, hipStream_t stream);
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
 // B prepacked by launch_pack_b (src: SRC_BF16, SRC_F32_AS_BF16 = fp32 A against bf16-packed B, SRC_I8);
 // vector_a: A is K-contiguous and 16-byte aligned
-hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile, bool vector_a, hipStream_t stream);
+hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_m, int tile_n, bool vector_a,
+                                     hipStream_t stream);
 struct PackBParams;
 hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream);
 
@@ -70,14 +71,15 @@ hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t strea
 }
 
 template <int SRC>
-hipError_t launch_tile_class(const TileGemmParams& p, int tile, int mode, hipStream_t stream) {
-  if (tile == 256) {
-    // 4 wavefronts of 128x128, one per SIMD: a third less LDS read traffic than 8 wavefronts of 128x64,
-    // which matters because the LDS pipe, not the MFMA pipe, is what the 8-wavefront shape saturates
-    return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
-  }
-  if (tile == 128) return launch_tile_mode<SRC, 2, 2, 2, 2>(p, mode, stream);  // 4 wavefronts of 64x64
-  return launch_tile_mode<SRC, 2, 2, 1, 1>(p, mode, stream);                    // 4 wavefronts of 32x32
+hipError_t launch_tile_class(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream) {
+  // Every shape runs 4 wavefronts (2 x 2), one per SIMD.  256x256: 128x128 per wavefront - a third less LDS
+  // read traffic than 8 wavefronts of 128x64, which matters because the LDS pipe, not the MFMA pipe, is
+  // what the 8-wavefront shape saturates.
+  if (tile_m == 256 && tile_n == 256) return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
+  if (tile_m == 256 && tile_n == 128) return launch_tile_mode<SRC, 2, 2, 4, 2>(p, mode, stream);
+  if (tile_m == 128 && tile_n == 256) return launch_tile_mode<SRC, 2, 2, 2, 4>(p, mode, stream);
+  if (tile_m == 128 && tile_n == 128) return launch_tile_mode<SRC, 2, 2, 2, 2>(p, mode, stream);
+  return launch_tile_mode<SRC, 2, 2, 1, 1>(p, mode, stream);
 }
 
 }  // namespace vecops_hip

@@ -27,27 +27,30 @@ hipError_t launch_packed_instance(const TileGemmParams& p, hipStream_t stream) {
 }
 
 template <int SRC, int LA>
-hipError_t launch_packed_tile(const TileGemmParams& p, int tile, hipStream_t stream) {
-  // (1 x 4 wavefronts of 256x64, which load no B fragment twice but read A from LDS twice as often,
-  // measured the same as 2 x 2 of 128x128)
-  if (tile == 256) return launch_packed_instance<SRC, 2, 2, 4, 4, LA>(p, stream);
-  if (tile == 128) return launch_packed_instance<SRC, 2, 2, 2, 2, LA>(p, stream);
+hipError_t launch_packed_tile(const TileGemmParams& p, int tile_m, int tile_n, hipStream_t stream) {
+  // (for 256x256, 1 x 4 wavefronts of 256x64, which load no B fragment twice but read A from LDS twice as
+  // often, measured the same as 2 x 2 of 128x128)
+  if (tile_m == 256 && tile_n == 256) return launch_packed_instance<SRC, 2, 2, 4, 4, LA>(p, stream);
+  if (tile_m == 256 && tile_n == 128) return launch_packed_instance<SRC, 2, 2, 4, 2, LA>(p, stream);
+  if (tile_m == 128 && tile_n == 256) return launch_packed_instance<SRC, 2, 2, 2, 4, LA>(p, stream);
+  if (tile_m == 128 && tile_n == 128) return launch_packed_instance<SRC, 2, 2, 2, 2, LA>(p, stream);
   return launch_packed_instance<SRC, 2, 2, 1, 1, LA>(p, stream);
 }
 
 template <int SRC>
-hipError_t launch_packed_class(const TileGemmParams& p, int tile, bool vector_a, hipStream_t stream) {
-  return vector_a ? launch_packed_tile<SRC, LOAD_KVEC>(p, tile, stream)
-                  : launch_packed_tile<SRC, LOAD_GENERIC>(p, tile, stream);
+hipError_t launch_packed_class(const TileGemmParams& p, int tile_m, int tile_n, bool vector_a, hipStream_t stream) {
+  return vector_a ? launch_packed_tile<SRC, LOAD_KVEC>(p, tile_m, tile_n, stream)
+                  : launch_packed_tile<SRC, LOAD_GENERIC>(p, tile_m, tile_n, stream);
 }
 
 }  // namespace
 
-hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile, bool vector_a, hipStream_t stream) {
+hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_m, int tile_n, bool vector_a,
+                                     hipStream_t stream) {
   switch (src) {
-    case SRC_BF16: return launch_packed_class<SRC_BF16>(p, tile, vector_a, stream);
-    case SRC_F32_AS_BF16: return launch_packed_class<SRC_F32_AS_BF16>(p, tile, vector_a, stream);
-    case SRC_I8: return launch_packed_class<SRC_I8>(p, tile, vector_a, stream);
+    case SRC_BF16: return launch_packed_class<SRC_BF16>(p, tile_m, tile_n, vector_a, stream);
+    case SRC_F32_AS_BF16: return launch_packed_class<SRC_F32_AS_BF16>(p, tile_m, tile_n, vector_a, stream);
+    case SRC_I8: return launch_packed_class<SRC_I8>(p, tile_m, tile_n, vector_a, stream);
     default: return hipErrorInvalidValue;
   }
 }

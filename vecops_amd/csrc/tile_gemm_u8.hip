@@ -2,8 +2,8 @@
 // row-sum kernel that produces their epilogue terms.
 #include "tile_gemm_launch.h"
 namespace vecops_hip {
-hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile, int mode, hipStream_t stream) {
-  return launch_tile_class<SRC_I8_FLIP>(p, tile, mode, stream);
+hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream) {
+  return launch_tile_class<SRC_I8_FLIP>(p, tile_m, tile_n, mode, stream);
 }
 
 // out[b][r] = scale * sum_k int8(x[b][r][k] xor flip)  (wrapping): the per-row and
