@@ -31,11 +31,11 @@ PEAK_HBM_GBPS = 8000.0
 # profiles/ (KiB per dispatch x 1024, FETCH scaled by 2.000 and WRITE by 1.000: what the
 # same counters read for a 1 GiB device copy, `--only copy`).  Counters cannot be read
 # from inside this process, so these are the recorded figures for exactly these workloads.
-TRAFFIC_BF16_4096 = int((101956 * 2.000 + 47624 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT = int((103564 * 2.000 + 112550 * 1.000) * 1024)
-TRAFFIC_GEMV_M1 = int((29688.5 * 2.000 + 56.1 * 1.000) * 1024)
-TRAFFIC_BF16_4096_PACKED = int((101803 * 2.000 + 47622 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT_PACKED = int((102951 * 2.000 + 112527 * 1.000) * 1024)
+TRAFFIC_BF16_4096 = int((98424 * 2.000 + 32782 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT = int((125307 * 2.000 + 90524 * 1.000) * 1024)
+TRAFFIC_GEMV_M1 = int((29729.8 * 2.000 + 56.0 * 1.000) * 1024)
+TRAFFIC_BF16_4096_PACKED = int((98420 * 2.000 + 32783 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT_PACKED = int((125143 * 2.000 + 90061 * 1.000) * 1024)
 
 
 def _device_tensors_bf16_gemm(dev):
@@ -106,7 +106,7 @@ def bench_int8_dequant(dev, steps, warmup):
             "dequant fused, fp32 out", "value": tops, "unit": "TOP/s", "ms_per_step": wall_ms, "dtype": "int8",
             "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                          "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT,
-                         "kernel": "vecops_hip::tile_gemm_kernel<int8, 256x256x128, dequant epilogue>",
+                         "kernel": "vecops_hip::tile_gemm_kernel<int8, 256x128x128, dequant epilogue>",
                          "algorithmic_ops_per_launch": ops,
                          "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
 
@@ -152,7 +152,7 @@ def bench_int8_dequant_packed(dev, steps, warmup):
             "ms_per_step": wall_ms, "dtype": "int8",
             "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                          "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT_PACKED,
-                         "kernel": "vecops_hip::tile_gemm_packed_b_kernel<int8, 256x256x128, dequant epilogue>",
+                         "kernel": "vecops_hip::tile_gemm_packed_b_kernel<int8, 256x128x128, dequant epilogue>",
                          "algorithmic_ops_per_launch": ops,
                          "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
 
