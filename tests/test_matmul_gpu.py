@@ -191,6 +191,31 @@ def test_batched_and_broadcast(device, oracle):
                 torch.empty((0, m, n), dtype=torch.float32, device=device))
 
 
+@pytest.mark.parametrize("m,n,k,family", [(4187, 900, 72, "tile_256x128"), (2111, 3643, 72, "tile_128x256"),
+                                          (1938, 900, 72, "tile_128"), (2457, 3221, 72, "tile_256"),
+                                          (900, 900, 72, "tile_64")])
+def test_every_tile_family_ragged(device, oracle, m, n, k, family):
+    """Each workgroup tile shape of the rule table on extents that leave partial tiles in M, N and K,
+    with a bf16 C input and a bf16 output (RNE of the fp32 result of the same launch sequence)."""
+    import torch
+    from vecops_amd import capi
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    cin = synth.bf16_round(synth.uniform_pm1(3, (m, n)))
+    ta, tb, tci = dev_bf16(a, device), dev_bf16(b, device), dev_bf16(cin, device)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    assert capi.FAMILY_NAMES[capi.plan_matmul(ta, tb, c, c_in=tci).family] == family
+    capi.matmul(ta, tb, c, c_in=tci)
+    c16 = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    capi.matmul(ta, tb, c16, c_in=tci)
+    torch.cuda.synchronize()
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, cin=cin, acc_f64=True)
+    got = c.cpu().numpy()
+    assert rel_err(got, want) <= fp32_tol(k)
+    assert np.array_equal(host_bits(c16), oracle.bf16_from_f32(got))
+
+
 def test_shared_b_batch_is_folded(device, oracle):
     """One B for every batch and A / C rows running on from batch to batch: planned and run as a single
     [batch * M, K] x B product (tests/ops/MatmulBatchTest.cpp:301-335), with a per-batch C input, a bias
