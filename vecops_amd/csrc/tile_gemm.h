@@ -18,6 +18,7 @@
 #ifndef VECOPS_HIP_TILE_GEMM_H
 #define VECOPS_HIP_TILE_GEMM_H
 
+
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -854,7 +855,9 @@ template <int WAVES_M, int WAVES_N, int WM, int WN>
 constexpr int kEpilogueLdsBytes() {
   const int bf16_tiles = (WN * 32 * 2 + 16) * (WM * 32) * WAVES_M * WAVES_N;
   const int general = 32 * (WN * 32 + 4) * 4 * WAVES_M * WAVES_N;
-  return bf16_tiles > general ? bf16_tiles : general;
+  const int columns32 = WM * 32 * 36 * 4 * WAVES_M * WAVES_N;
+  const int most = bf16_tiles > general ? bf16_tiles : general;
+  return most > columns32 ? most : columns32;
 }
 
 template <int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_B>
@@ -920,59 +923,63 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
     for (int base = 0; base < TOTAL; base += 64) {
       const int idx = base + lane, r = idx / SEGS, seg = idx % SEGS;
       const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + seg * 16);
-      // whole 128-byte lines per row segment: streamed past L2, so the end of the kernel has no dirty C to
-      // write back (the 16-byte pieces of the 32-bit paths below would turn into partial-line writes: slower)
-      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + seg * 8));
+      // (the non-temporal hint was measured on these whole-line stores: no gain at 4096^3, and 13 % slower
+      // when the output dominates, 8192 x 8192 x 64)
+      *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + seg * 8) = v;
     }
-  } else if (simple && (INT ? (p.out_kind == OUT_I32 && p.row_scales == nullptr && p.correction == nullptr)
-                            : p.out_kind == OUT_F32)) {
-    static_for<WM>([&](auto ci) {
-      constexpr int i = decltype(ci)::value;
-      const int row = m0 + (wm * WM + i) * 32 + frag_row;
-      static_for<WN>([&](auto cj) {
-        constexpr int j = decltype(cj)::value;
-        const int col0 = n0 + (wn * WN + j) * 32 + frag_half * 4;
-        uint32_t* dst = reinterpret_cast<uint32_t*>(c_base) + batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col0;
-        static_for<4>([&](auto cq) {
-          constexpr int q = decltype(cq)::value;
-          // four consecutive accumulator registers as one 16-byte vector of their own type
-          const auto v = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
-          *reinterpret_cast<typename std::remove_const<decltype(v)>::type*>(dst + q * 8) = v;
-        });
-      });
-    });
-  } else if (simple && INT && p.row_scales != nullptr) {
+  } else if (simple && (INT ? (p.out_kind == OUT_I32 || p.row_scales != nullptr) : p.out_kind == OUT_F32)) {
+    // 32-bit outputs: one 32-column block of the wavefront's tile at a time goes row-major through LDS
+    // (128 rows x 128 bytes) and leaves as whole cache lines (16-byte pieces scattered over 32 rows, straight
+    // from the accumulator layout, wrote 8192 x 8192 fp32 at 3.9 TB/s; whole lines at 4.9 TB/s).
+    constexpr int ROWS = WM * 32, PITCH = 36;  // words
+    static_assert(ROWS * PITCH * 4 * WAVES_M * WAVES_N <= LDS_BYTES, "32-bit epilogue staging must fit the launch's LDS");
+    __syncthreads();  // every wavefront is done reading fragments
+    uint32_t* mine = reinterpret_cast<uint32_t*>(lds) + wave * (ROWS * PITCH);
+    const bool dequant = INT && p.row_scales != nullptr;
     float rs[WM];
-    static_for<WM>([&](auto ci) { rs[decltype(ci)::value] = p.row_scales[m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row]; });
+    static_for<WM>([&](auto ci) {
+      rs[decltype(ci)::value] = dequant ? p.row_scales[m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row] : 1.0f;
+    });
+    uint32_t* out = reinterpret_cast<uint32_t*>(c_base) + batch * p.c_bs + static_cast<int64_t>(m0 + wm * ROWS) * p.c_rs;
     static_for<WN>([&](auto cj) {
       constexpr int j = decltype(cj)::value;
-      const int col0 = n0 + (wn * WN + j) * 32 + frag_half * 4;
+      const int col_block = n0 + (wn * WN + j) * 32;
       f32x4 cs[4];
       i32x4 corr[4];
       static_for<4>([&](auto cq) {
         constexpr int q = decltype(cq)::value;
-        cs[q] = *reinterpret_cast<const f32x4*>(p.column_scales + col0 + q * 8);
-        corr[q] = p.correction ? *reinterpret_cast<const i32x4*>(p.correction + col0 + q * 8) : i32x4{0, 0, 0, 0};
+        const int col0 = col_block + frag_half * 4 + q * 8;
+        cs[q] = dequant ? *reinterpret_cast<const f32x4*>(p.column_scales + col0) : f32x4{1.f, 1.f, 1.f, 1.f};
+        corr[q] = (INT && p.correction) ? *reinterpret_cast<const i32x4*>(p.correction + col0) : i32x4{0, 0, 0, 0};
       });
       static_for<WM>([&](auto ci) {
         constexpr int i = decltype(ci)::value;
-        const int row = m0 + (wm * WM + i) * 32 + frag_row;
-        float* dst = reinterpret_cast<float*>(c_base) + batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col0;
         static_for<4>([&](auto cq) {
           constexpr int q = decltype(cq)::value;
+          const auto a4 = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
+          u32x4 bits = __builtin_bit_cast(u32x4, a4);
           if constexpr (INT) {
-            const auto a4 = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
-            f32x4 out;
+            bits += __builtin_bit_cast(u32x4, corr[q]);
+            if (dequant) {
+              f32x4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(a4[e]) + static_cast<uint32_t>(corr[q][e]));
-              const float t = static_cast<float>(v) * rs[i];  // row scale first, then column scale:
-              out[e] = t * cs[q][e];                          // two separately rounded multiplies
+              for (int e = 0; e < 4; ++e) {
+                const float t = static_cast<float>(static_cast<int32_t>(bits[e])) * rs[i];  // row scale first, then
+                o[e] = t * cs[q][e];                                                         // column scale
+              }
+              bits = __builtin_bit_cast(u32x4, o);
             }
-            *reinterpret_cast<f32x4*>(dst + q * 8) = out;
           }
+          *reinterpret_cast<u32x4*>(mine + (i * 32 + frag_row) * PITCH + q * 8 + frag_half * 4) = bits;
         });
       });
+      // the wavefront reads back only what it wrote itself: its own LDS traffic is ordered
+#pragma unroll
+      for (int base = 0; base < ROWS * 8; base += 64) {
+        const int idx = base + lane, r = idx >> 3, cq = idx & 7;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + cq * 4);
+        *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + col_block + cq * 4) = v;
+      }
     });
   } else if (interior && p.split_k > 1 && (p.n & 3) == 0 && (reinterpret_cast<uintptr_t>(p.partial) & 15) == 0) {
     // split-K partial sums of an interior tile: raw accumulators, 16 bytes per store
