@@ -886,7 +886,9 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
   // out-of-line routine.
   const bool interior = m0 + BM <= p.m && n0 + BN <= p.n;
   const bool aligned = (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
-  const bool simple = interior && aligned && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1 && SRC != SRC_I8_FLIP;
+  // the two fast paths take edge tiles too: their stores (and scale loads) are guarded per row and per run
+  // of columns, which costs an interior tile a few compares
+  const bool simple = aligned && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1 && SRC != SRC_I8_FLIP;
   char* c_base = static_cast<char*>(p.c);
   if (simple && !INT && p.out_kind == OUT_BF16) {
     // bf16: 8-byte pieces scattered over 32 rows would waste most of every memory
@@ -925,7 +927,17 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
       const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + seg * 16);
       // (the non-temporal hint was measured on these whole-line stores: no gain at 4096^3, and 13 % slower
       // when the output dominates, 8192 x 8192 x 64)
-      *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + seg * 8) = v;
+      uint16_t* dst = out + static_cast<int64_t>(r) * p.c_rs + seg * 8;
+      const int cols_left = p.n - (n0 + wn * TILE_COLS + seg * 8);
+      if (m0 + wm * TILE_ROWS + r < p.m) {
+        if (cols_left >= 8) {
+          *reinterpret_cast<u32x4*>(dst) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (e < cols_left) dst[e] = static_cast<uint16_t>(v[e >> 1] >> ((e & 1) * 16));
+        }
+      }
     }
   } else if (simple && (INT ? (p.out_kind == OUT_I32 || p.row_scales != nullptr) : p.out_kind == OUT_F32)) {
     // 32-bit outputs: one 32-column block of the wavefront's tile at a time goes row-major through LDS
@@ -938,7 +950,8 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
     const bool dequant = INT && p.row_scales != nullptr;
     float rs[WM];
     static_for<WM>([&](auto ci) {
-      rs[decltype(ci)::value] = dequant ? p.row_scales[m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row] : 1.0f;
+      const int row = m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row;
+      rs[decltype(ci)::value] = (dequant && row < p.m) ? p.row_scales[row] : 1.0f;
     });
     uint32_t* out = reinterpret_cast<uint32_t*>(c_base) + batch * p.c_bs + static_cast<int64_t>(m0 + wm * ROWS) * p.c_rs;
     static_for<WN>([&](auto cj) {
@@ -949,8 +962,20 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
       static_for<4>([&](auto cq) {
         constexpr int q = decltype(cq)::value;
         const int col0 = col_block + frag_half * 4 + q * 8;
-        cs[q] = dequant ? *reinterpret_cast<const f32x4*>(p.column_scales + col0) : f32x4{1.f, 1.f, 1.f, 1.f};
-        corr[q] = (INT && p.correction) ? *reinterpret_cast<const i32x4*>(p.correction + col0) : i32x4{0, 0, 0, 0};
+        cs[q] = f32x4{1.f, 1.f, 1.f, 1.f};
+        corr[q] = i32x4{0, 0, 0, 0};
+        if (col0 + 3 < p.n) {
+          if (dequant) cs[q] = *reinterpret_cast<const f32x4*>(p.column_scales + col0);
+          if (INT && p.correction) corr[q] = *reinterpret_cast<const i32x4*>(p.correction + col0);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (col0 + e < p.n) {
+              if (dequant) cs[q][e] = p.column_scales[col0 + e];
+              if (INT && p.correction) corr[q][e] = p.correction[col0 + e];
+            }
+          }
+        }
       });
       static_for<WM>([&](auto ci) {
         constexpr int i = decltype(ci)::value;
@@ -978,7 +1003,17 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
       for (int base = 0; base < ROWS * 8; base += 64) {
         const int idx = base + lane, r = idx >> 3, cq = idx & 7;
         const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + cq * 4);
-        *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(r) * p.c_rs + col_block + cq * 4) = v;
+        uint32_t* dst = out + static_cast<int64_t>(r) * p.c_rs + col_block + cq * 4;
+        const int cols_left = p.n - (col_block + cq * 4);
+        if (m0 + wm * ROWS + r < p.m) {
+          if (cols_left >= 4) {
+            *reinterpret_cast<u32x4*>(dst) = v;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (e < cols_left) dst[e] = v[e];
+          }
+        }
       }
     });
   } else if (interior && p.split_k > 1 && (p.n & 3) == 0 && (reinterpret_cast<uintptr_t>(p.partial) & 15) == 0) {
