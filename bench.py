@@ -177,7 +177,7 @@ def bench_gemv(dev, steps, warmup, m=1):
             "us_per_step": wall_ms * 1e3, "dtype": "int8 x bf16 -> f32",
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                          "frac": gbps / PEAK_HBM_GBPS, "traffic": TRAFFIC_GEMV_M1 if m == 1 else None,
-                         "kernel": "vecops_hip::skinny_w8a16_kernel" if m == 1 else
+                         "kernel": "vecops_hip::skinny_w8a16_stream_kernel" if m == 1 else
                                    "vecops_hip::skinny_w8a16_mfma_resident_kernel",
                          "algorithmic_bytes_per_launch": nbytes}}
 

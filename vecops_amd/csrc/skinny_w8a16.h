@@ -132,6 +132,84 @@ __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const SkinnyW8A16Para
   }
 }
 
+// ---- M = 1, streaming: a wavefront walks many weight rows with the next row's loads in flight --------
+// K = CH x 1024: lane l owns the 16-element chunks u * 64 + l (u < CH) of every row, exactly as in the
+// dot-product kernel above, so the sums are taken in the same order and the results are the same
+// bits.  The activations of the lane's chunks (widened to fp32) and their sums stay in registers for
+// the whole kernel; wavefront w takes rows w, w + W, w + 2W, ... (W wavefronts in the grid), so that at
+// any moment the grid reads one contiguous run of rows; a row's CH weight loads and CH scale loads are
+// issued one row ahead of its arithmetic (two rows ahead measured 10 % slower).  The dot-product
+// kernel's grid starts every wavefront at the same moment - all of them load, then all of them
+// compute; here each wavefront overlaps the two.
+template <int CH>
+__global__ __launch_bounds__(256) void skinny_w8a16_stream_kernel(const SkinnyW8A16Params p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int64_t waves = static_cast<int64_t>(gridDim.x) * 4;
+  const VECOPS_GLOBAL char* wbase = (const VECOPS_GLOBAL char*)p.w;
+  const VECOPS_GLOBAL uint16_t* xbase = (const VECOPS_GLOBAL uint16_t*)p.x;
+  const VECOPS_GLOBAL float* sbase = (const VECOPS_GLOBAL float*)p.scales;
+
+  float xf[CH][16], xsum[CH];
+  int group_of[CH];
+#pragma unroll
+  for (int u = 0; u < CH; ++u) {
+    const int k0 = (u * 64 + lane) << 4;
+    group_of[u] = k0 / p.group;
+    const VECOPS_GLOBAL u32x4* px = (const VECOPS_GLOBAL u32x4*)(xbase + k0);
+    const u32x4 lo = px[0], hi = px[1];
+    const uint32_t words[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    float s = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      xf[u][2 * e] = __uint_as_float(words[e] << 16);
+      xf[u][2 * e + 1] = __uint_as_float(words[e] & 0xffff0000u);
+      s += xf[u][2 * e];
+      s += xf[u][2 * e + 1];
+    }
+    xsum[u] = s;
+  }
+
+  u32x4 wq[2][CH];
+  float sc[2][CH];
+  auto fetch = [&](int set, int64_t n) {
+    // rows past N are clamped: computed, never stored
+    const int64_t row = n < p.n ? n : p.n - 1;
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      wq[set][u] = *(const VECOPS_GLOBAL u32x4*)(wbase + row * p.ldw + (static_cast<int64_t>(u * 64 + lane) << 4));
+      sc[set][u] = sbase[row * p.groups + group_of[u]];
+    }
+  };
+  auto finish = [&](int set, int64_t n) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      const uint32_t words[4] = {wq[set][u].x ^ 0x80808080u, wq[set][u].y ^ 0x80808080u, wq[set][u].z ^ 0x80808080u,
+                                 wq[set][u].w ^ 0x80808080u};
+      float part = -128.0f * xsum[u];
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        part = fmaf(xf[u][e], static_cast<float>((words[e >> 2] >> ((e & 3) * 8)) & 0xffu), part);
+      acc = fmaf(sc[set][u], part, acc);
+    }
+    const float total = wave_sum(acc);
+    if (lane == 0 && n < p.n) p.y[n] = static_cast<uint16_t>(bf16_bits_rne(total));
+  };
+
+  if (wave >= p.n) return;
+  fetch(0, wave);
+  int64_t n = wave;
+  // two rows per trip so that the register set of a row is a compile-time choice
+  for (; n + waves < p.n; n += 2 * waves) {
+    fetch(1, n + waves);
+    finish(0, n);
+    fetch(0, n + 2 * waves);
+    finish(1, n + waves);
+  }
+  if (n < p.n) finish(0, n);
+}
+
 // ---- matrix-core family: a workgroup owns TILES x 16 weight rows, its WAVES wavefronts
 // split K by scale groups --------------------------------------------------------------------
 // One v_mfma_f32_16x16x32_bf16 multiplies 16 weight rows x 32 k by 32 k x 16
