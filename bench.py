@@ -31,11 +31,11 @@ PEAK_HBM_GBPS = 8000.0
 # profiles/ (KiB per dispatch x 1024, FETCH scaled by 2.000 and WRITE by 1.000: what the
 # same counters read for a 1 GiB device copy, `--only copy`).  Counters cannot be read
 # from inside this process, so these are the recorded figures for exactly these workloads.
-TRAFFIC_BF16_4096 = int((98424 * 2.000 + 32782 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT = int((125307 * 2.000 + 90524 * 1.000) * 1024)
-TRAFFIC_GEMV_M1 = int((29729.8 * 2.000 + 56.0 * 1.000) * 1024)
-TRAFFIC_BF16_4096_PACKED = int((98420 * 2.000 + 32783 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT_PACKED = int((125143 * 2.000 + 90061 * 1.000) * 1024)
+TRAFFIC_BF16_4096 = int((98487 * 2.000 + 32768 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT = int((125552 * 2.000 + 88064 * 1.000) * 1024)
+TRAFFIC_GEMV_M1 = int((29647.4 * 2.000 + 112.0 * 1.000) * 1024)
+TRAFFIC_BF16_4096_PACKED = int((98470 * 2.000 + 32768 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT_PACKED = int((125228 * 2.000 + 88064 * 1.000) * 1024)
 
 
 def _device_tensors_bf16_gemm(dev):
