@@ -113,6 +113,68 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul(const VecopsHipOperand* a, const Vec
                                             void* workspace, uint64_t workspace_size, void* stream);
 
 /*
+ * Fused output transforms - the catalogue that vecops' tests build from
+ * elementwise and lane-local output transforms on tensor::output
+ * (tests/ops/MatmulFusionTest.cpp:29-112; tests/ops/MatmulConversionTestCommon.h:
+ * bias + relu :439-497, runtime and per-column scale :621-702, bias + clamp
+ * :705-760, relu / sigmoid :1028-1092, silu :1095-1168, integer bias with
+ * per-column (re)quantisation :1171-1290).  With acc = C_in + A.B^T (a bias is a
+ * C_in row with row stride 0):
+ *   v = float(acc)                      (int32 accumulators; fp32 ones are v already)
+ *   v = v * row_scales[row]             (row_scales != null)
+ *   v = v * column_scales[col]          (column_scales != null)
+ *   v = v * scale                       (flags & VECOPS_HIP_EPILOGUE_SCALE)
+ *   v = v + shift                       (flags & VECOPS_HIP_EPILOGUE_SHIFT)
+ *   v = activation(v)                   relu max(v,0); clamp min(max(v,lo),hi);
+ *                                       sigmoid 1/(1+exp(-v)); silu v*sigmoid(v)
+ *   c = convert(v)                      fp32; bf16 round-to-nearest-even; u8 / i8:
+ *                                       truncate toward zero, saturate (NaN and
+ *                                       values outside int32 become INT32_MIN before
+ *                                       the saturation, as vecops' x86 vector store
+ *                                       does, vec/details/x86/Conversion.h:522-528)
+ * Every step is one fp32 operation, never contracted.  Scales, shift, relu and
+ * clamp are bit-exact against the reference on int32 accumulators; sigmoid and
+ * silu use the hardware exponential (within 1e-6 relative of the exact value).
+ */
+enum VecopsHipActivation {
+  VECOPS_HIP_ACT_NONE = 0,
+  VECOPS_HIP_ACT_RELU = 1,
+  VECOPS_HIP_ACT_CLAMP = 2,
+  VECOPS_HIP_ACT_SIGMOID = 3,
+  VECOPS_HIP_ACT_SILU = 4
+};
+enum { VECOPS_HIP_EPILOGUE_SCALE = 1u, VECOPS_HIP_EPILOGUE_SHIFT = 2u };
+
+typedef struct VecopsHipEpilogue {
+  uint32_t struct_size;        /* sizeof(VecopsHipEpilogue) */
+  uint32_t activation;         /* VecopsHipActivation */
+  uint32_t flags;              /* VECOPS_HIP_EPILOGUE_* */
+  float scale;
+  float shift;
+  float clamp_lo, clamp_hi;
+  const float* row_scales;     /* device, [M] (rank 3: [batch][M] dense), or null */
+  const float* column_scales;  /* device, [N], or null */
+} VecopsHipEpilogue;
+
+/* vecops_hip_plan_matmul for a call of vecops_hip_matmul_fused. */
+VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul_fused(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                       const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                       uint32_t compute, const VecopsHipEpilogue* epilogue,
+                                                       VecopsHipPlan* plan);
+
+/*
+ * vecops_hip_matmul with the transform above between the accumulator and c.
+ *   a,b bf16 | f32 -> c f32 | bf16      (c_in f32 | bf16)
+ *   a,b i8 | u8    -> c f32 | u8 | i8   (c_in i32)
+ * Operands, strides, batches, zero extents and the workspace rule are those of
+ * vecops_hip_matmul (K == 0 writes transform(C_in or 0)).
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_fused(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                  const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                  uint32_t compute, const VecopsHipEpilogue* epilogue,
+                                                  void* workspace, uint64_t workspace_size, void* stream);
+
+/*
  * c[i,j] = (float(acc[i,j]) * row_scales[i]) * column_scales[j],
  * acc = sum_k a[i,k]*b[j,k] (+ correction[j]) in wrapping int32 - replaces
  * ops::matmul with AMX_I8I32<int8,int8> and an output carrying

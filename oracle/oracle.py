@@ -91,6 +91,8 @@ class Oracle:
         L.vo_matmul_i8_dense.argtypes = [C.c_void_p] * 3 + [C.c_int64] * 3
         L.vo_matmul_i8_dequant.argtypes = [C.c_void_p] * 6 + [C.c_int64] * 3
         L.vo_matmul_w8a16_group.argtypes = [C.c_void_p] * 5 + [C.c_int64] * 4
+        L.vo_fused_outputs.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_uint32,
+                                       C.c_float, C.c_float, C.c_int, C.c_float, C.c_float, C.c_int, C.c_void_p]
         for name in ("vo_amx_small_vector_profitable", "vo_sme_small_vector_profitable"):
             getattr(L, name).argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64]
         L.vo_small_area_profitable.argtypes = [C.c_int64] * 4
@@ -164,6 +166,27 @@ class Oracle:
                                       b.shape[0], a.shape[1])
         return c
 
+    def fused_outputs(self, acc, out_dtype, *, activation=0, scale=None, shift=None, row_scales=None,
+                      column_scales=None, lo=0.0, hi=0.0) -> np.ndarray:
+        """The fused output transform on an [M,N] accumulator matrix (int32 or float32, C-input already
+        added); out_dtype float32, uint16 (bf16 bits), uint8 or int8."""
+        acc = np.ascontiguousarray(acc)
+        assert acc.ndim == 2 and acc.dtype in (np.int32, np.float32)
+        out_dtype = np.dtype(out_dtype)
+        code = {np.dtype(np.float32): 12, np.dtype(np.uint16): 11, np.dtype(np.uint8): 3, np.dtype(np.int8): 2}[out_dtype]
+        rs = np.ascontiguousarray(row_scales, dtype=np.float32) if row_scales is not None else None
+        cs = np.ascontiguousarray(column_scales, dtype=np.float32) if column_scales is not None else None
+        out = np.empty(acc.shape, dtype=out_dtype)
+        rc = self.lib.vo_fused_outputs(acc.ctypes.data, 1 if acc.dtype == np.int32 else 0, acc.shape[0], acc.shape[1],
+                                       rs.ctypes.data if rs is not None else None,
+                                       cs.ctypes.data if cs is not None else None,
+                                       (1 if scale is not None else 0) | (2 if shift is not None else 0),
+                                       0.0 if scale is None else scale, 0.0 if shift is None else shift, activation,
+                                       lo, hi, code, out.ctypes.data)
+        if rc != 0:
+            raise ValueError("vo_fused_outputs rejected its arguments")
+        return out
+
     def matmul_w8a16_group(self, x_bits, w, scales, group: int):
         """Returns (y bf16 bits [M,N], y as float64 [M,N])."""
         x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
@@ -198,6 +221,12 @@ def _strides3(arr: np.ndarray):
     for i in range(arr.ndim):
         s[i] = arr.strides[i] // arr.itemsize
     return s
+
+
+class FusedSpec(C.Structure):
+    """Mirror of FusedSpec in oracle/ref_harness.cpp."""
+    _fields_ = [("activation", C.c_int32), ("flags", C.c_uint32), ("scale", C.c_float), ("shift", C.c_float),
+                ("lo", C.c_float), ("hi", C.c_float), ("column_scales", C.c_void_p)]
 
 
 class Reference:
@@ -281,6 +310,36 @@ class Reference:
             C.c_void_p(c.ctypes.data), C.c_int64(m), C.c_int64(n), C.c_int64(k))
         if rc != 0:
             raise RuntimeError("reference matmul unavailable")
+        return c
+
+    def matmul_fused(self, a, b, bias, out_dtype, *, activation=0, scale=None, column_scales=None, shift=None,
+                     lo=0.0, hi=0.0):
+        """bf16 (uint16 bits) or int8 operands through the reference with a fused output transform:
+        convert(act(((A.B^T + bias) * scale) * column_scales[col] + shift)); out_dtype is a numpy dtype
+        (float32, uint16 = bf16 bits, uint8, int8)."""
+        m, k = a.shape
+        n = b.shape[0]
+        a = np.ascontiguousarray(a)
+        b = np.ascontiguousarray(b)
+        cs = None
+        if column_scales is not None:
+            cs = np.zeros(n + 64, dtype=np.float32)  # unmasked vector load past n
+            cs[:n] = column_scales
+        spec = FusedSpec(activation, (1 if scale is not None else 0) | (2 if shift is not None else 0),
+                         0.0 if scale is None else scale, 0.0 if shift is None else shift, lo, hi,
+                         cs.ctypes.data if cs is not None else None)
+        integer = a.dtype == np.int8
+        if bias is not None:
+            bias = np.ascontiguousarray(bias, dtype=np.int32 if integer else np.float32)
+        out_dtype = np.dtype(out_dtype)
+        kind = {np.dtype(np.float32): 0, np.dtype(np.uint16): 1, np.dtype(np.uint8): 3, np.dtype(np.int8): 4}[out_dtype]
+        c = np.zeros((m, n), dtype=out_dtype)
+        fn = self.lib.vref_matmul_i8_fused if integer else self.lib.vref_matmul_bf16_fused
+        rc = fn(C.c_void_p(a.ctypes.data), C.c_void_p(b.ctypes.data),
+                C.c_void_p(bias.ctypes.data if bias is not None else None), C.c_void_p(c.ctypes.data), C.c_int(kind),
+                C.c_int64(m), C.c_int64(n), C.c_int64(k), C.byref(spec))
+        if rc != 0:
+            raise RuntimeError("reference fused matmul unavailable (rc=%d)" % rc)
         return c
 
     def predicate(self, name: str, *args) -> bool:

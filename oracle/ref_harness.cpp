@@ -89,6 +89,70 @@ int run3(const TA* a, const TB* b, TC* c, int64_t batch, int64_t m, int64_t n, i
   return 0;
 }
 
+// Fused output transforms, built the way the reference's own tests build them
+// (tests/ops/MatmulConversionTestCommon.h: per-column scale :652-660, clamp :735-740,
+// relu :1047-1050, sigmoid :1051-1057, silu :1121-1128, requantisation :1222-1234):
+//   v = A.B^T + bias[col]                (bias = stride-0 C-input row, may be null)
+//   v = float(v)                         (int32 accumulators only)
+//   v = v * scale                        (flags & 1)
+//   v = v * column_scales[col]           (column_scales != null; readable 64 floats past n)
+//   v = v + shift                        (flags & 2)
+//   v = act(v)                           0 none, 1 relu, 2 clamp(lo, hi), 3 sigmoid, 4 silu
+//   c = convert<memory dtype of C>(v)
+struct FusedSpec {
+  int32_t activation;
+  uint32_t flags;
+  float scale, shift, lo, hi;
+  const float* column_scales;
+};
+
+template <typename Domain>
+auto fused_transform(const FusedSpec* spec) {
+  return tensor::make_lane_local_vec_transform<Domain, Domain>(
+    [spec](auto tag, auto value, const auto& context) VECOPS_KERNEL_LAMBDA {
+      const auto coordinate = context.lane_coord(0);
+      const nint_t column = coordinate[coordinate.size() - 1];
+      auto v = value;
+      if (spec->flags & 1u) v = vec::mul(tag, v, vec::fill(tag, Domain{spec->scale}));
+      if (spec->column_scales) v = vec::mul(tag, v, vec::load(tag, spec->column_scales + column));
+      if (spec->flags & 2u) v = vec::add(tag, v, vec::fill(tag, Domain{spec->shift}));
+      const auto one = vec::fill(tag, Domain{1});
+      switch (spec->activation) {
+        case 1: v = vec::max(tag, v, vec::zeros(tag)); break;
+        case 2: v = vec::min(tag, vec::max(tag, v, vec::fill(tag, Domain{spec->lo})), vec::fill(tag, Domain{spec->hi})); break;
+        case 3: v = vec::div(tag, one, vec::add(tag, one, vec::exp(tag, vec::neg(tag, v)))); break;
+        case 4: v = vec::mul(tag, v, vec::div(tag, one, vec::add(tag, one, vec::exp(tag, vec::neg(tag, v))))); break;
+        default: break;
+      }
+      return v;
+    });
+}
+
+template <typename Atom, typename TA, typename TB, typename TBias, typename TC>
+int run_fused(const TA* a, const TB* b, const TBias* bias, TC* c, int64_t m, int64_t n, int64_t k,
+              const FusedSpec* spec) {
+  if (!enable_amx()) return -1;
+  using Acc = typename Atom::TAcc;
+  auto at = view2(const_cast<TA*>(a), m, k, k, 1);
+  auto bt = view2(const_cast<TB*>(b), n, k, k, 1);
+  auto ct = view2(c, m, n, n, 1);
+  auto cout = tensor::output<Acc>(ct, fused_transform<float32_t>(spec));
+  auto op = ops::matmul(ops::MatmulConfig<Atom>{});
+  if (bias) {
+    auto bias_t = tensor::input<Acc>(view2(const_cast<TBias*>(bias), m, n, 0, 1));
+    const nint_t bytes = op.required_workspace(Any{m}, Any{n}, Any{k}, at, bt, bias_t, cout);
+    kernel::Workspace ws(bytes);
+    auto v = ws.view();
+    op(v, Any{m}, Any{n}, Any{k}, at, bt, bias_t, cout);
+  } else {
+    const nint_t bytes = op.required_workspace(Any{m}, Any{n}, Any{k}, at, bt, cout);
+    kernel::Workspace ws(bytes);
+    auto v = ws.view();
+    op(v, Any{m}, Any{n}, Any{k}, at, bt, cout);
+  }
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -164,6 +228,25 @@ VREF_EXPORT int vref_matmul_i8_dequant(const int8_t* a, const int8_t* b, const f
     op(v, Any{m}, Any{n}, Any{k}, at, bt, cout);
   }
   return 0;
+}
+
+// c_kind: 0 fp32, 1 bf16, 3 uint8, 4 int8 (the dtype codes of include/vecops_hip.h are not used here).
+VREF_EXPORT int vref_matmul_bf16_fused(const uint16_t* a, const uint16_t* b, const float* bias, void* c, int c_kind,
+                                       int64_t m, int64_t n, int64_t k, const FusedSpec* spec) {
+  const auto* ab = reinterpret_cast<const bfloat16_t*>(a);
+  const auto* bb = reinterpret_cast<const bfloat16_t*>(b);
+  using Atom = matmul::AMX_BF16F32;
+  if (c_kind == 0) return run_fused<Atom>(ab, bb, bias, static_cast<float*>(c), m, n, k, spec);
+  if (c_kind == 1) return run_fused<Atom>(ab, bb, bias, static_cast<bfloat16_t*>(c), m, n, k, spec);
+  return -2;
+}
+VREF_EXPORT int vref_matmul_i8_fused(const int8_t* a, const int8_t* b, const int32_t* bias, void* c, int c_kind,
+                                     int64_t m, int64_t n, int64_t k, const FusedSpec* spec) {
+  using Atom = matmul::AMX_I8I32<int8_t, int8_t>;
+  if (c_kind == 0) return run_fused<Atom>(a, b, bias, static_cast<float*>(c), m, n, k, spec);
+  if (c_kind == 3) return run_fused<Atom>(a, b, bias, static_cast<uint8_t*>(c), m, n, k, spec);
+  if (c_kind == 4) return run_fused<Atom>(a, b, bias, static_cast<int8_t*>(c), m, n, k, spec);
+  return -2;
 }
 
 // The non-inline dispatch predicates of src/MatmulRuntimeDispatch.cpp:12-32.

@@ -23,6 +23,10 @@
  *       whose products are exact, and oracle/_ref.
  *   vo_matmul_i8_dequant                  - numpy float32 two-step multiply and
  *       oracle/_ref (bit-exact).
+ *   vo_fused_outputs                      - golden vectors of the real reference
+ *       (tests/golden: every step, activation and output dtype, byte outputs with
+ *       out-of-range and NaN values) and oracle/_ref; sigmoid / silu within the
+ *       reference tests' own 8e-4 tolerance, everything else bit for bit.
  *   vo_amx_small_vector_profitable & co   - the static_assert table of
  *       tests/matmul/TilerTest.cpp:86-98.
  *   vo_matmul_w8a16_group                 - PARITY UNPINNED: the reference has
@@ -238,6 +242,61 @@ VO_EXPORT int vo_matmul(const vo_tensor* a, const vo_tensor* b, const vo_tensor*
           }
           store_from_f32(c->data, c->dtype, ci, result);
         }
+      }
+    }
+  }
+  return 0;
+}
+
+/*
+ * Fused output transform on finished accumulators (the accumulator already holds
+ * C_in / the bias row): the restatement of what vecops' tests attach to
+ * tensor::output as elementwise and lane-local transforms
+ * (tests/ops/MatmulConversionTestCommon.h: per-column scale :652-660, runtime scale
+ * :647-651, clamp :735-740, relu :1047-1050, sigmoid :1051-1057, silu :1121-1128,
+ * requantisation :1222-1234), in this order, each step one fp32 operation:
+ *   v = float(acc);  v *= row_scales[row];  v *= column_scales[col];  v *= scale (flags & 1);
+ *   v += shift (flags & 2);  v = activation(v);  c = convert(v)
+ * acc_is_int selects int32 accumulators (converted with a plain int -> float cast).
+ * sigmoid and silu are evaluated in double and rounded once (the tests' own
+ * expectation, :1086-1087, :1157-1160); the reference's vector exp differs from that by
+ * a few ulp, so they are compared with a tolerance, the others bit for bit.
+ * out_dtype: VO_F32, VO_BF16 (round to nearest even), VO_U8 / VO_I8: the x86 vector
+ * store (vec/details/x86/Conversion.h:522-528) = truncating convert to int32, where NaN
+ * and values outside int32 give INT32_MIN, then a saturating narrow.
+ * Pinned by golden vectors of the real reference (tests/golden) for every step and
+ * output dtype, including the out-of-range and NaN cases of the byte outputs.
+ */
+static int32_t cvtt_i32(float v) {
+  if (!(v >= -2147483648.0f && v < 2147483648.0f)) return INT32_MIN;
+  return (int32_t)v;
+}
+
+VO_EXPORT int vo_fused_outputs(const void* acc, int acc_is_int, int64_t M, int64_t N, const float* row_scales,
+                               const float* column_scales, uint32_t flags, float scale, float shift, int activation,
+                               float lo, float hi, int out_dtype, void* out) {
+  if (activation < 0 || activation > 4) return 1;
+  for (int64_t i = 0; i < M; ++i) {
+    for (int64_t j = 0; j < N; ++j) {
+      const int64_t at = i * N + j;
+      float v = acc_is_int ? (float)((const int32_t*)acc)[at] : ((const float*)acc)[at];
+      if (row_scales) v = v * row_scales[i];
+      if (column_scales) v = v * column_scales[j];
+      if (flags & 1u) v = v * scale;
+      if (flags & 2u) v = v + shift;
+      switch (activation) {
+        case 1: v = (v > 0.0f) ? v : 0.0f; break;                        /* max_ps(v, 0): NaN -> 0 */
+        case 2: v = (v > lo) ? v : lo; v = (v < hi) ? v : hi; break;     /* min_ps(max_ps(v, lo), hi) */
+        case 3: v = (float)(1.0 / (1.0 + exp(-(double)v))); break;
+        case 4: v = (float)((double)v / (1.0 + exp(-(double)v))); break;
+        default: break;
+      }
+      switch (out_dtype) {
+        case VO_F32: ((float*)out)[at] = v; break;
+        case VO_BF16: ((uint16_t*)out)[at] = vo_bf16_from_f32(v); break;
+        case VO_U8: { int32_t t = cvtt_i32(v); ((uint8_t*)out)[at] = (uint8_t)(t < 0 ? 0 : t > 255 ? 255 : t); break; }
+        case VO_I8: { int32_t t = cvtt_i32(v); ((int8_t*)out)[at] = (int8_t)(t < -128 ? -128 : t > 127 ? 127 : t); break; }
+        default: return 1;
       }
     }
   }

@@ -99,3 +99,74 @@ def make_inputs(case: dict) -> dict:
         if case.get("correction"):
             out["correction"] = ((synth.draws(5, n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32)
     return out
+
+
+# ---- fused output transforms --------------------------------------------------------------------
+# Outputs of the real vecops matmul with the output transforms its own tests attach
+# (tests/ops/MatmulFusionTest.cpp:29-112; builders in tests/ops/MatmulConversionTestCommon.h).
+# Fields: kind bf16 | i8; out f32 | bf16 | u8 | i8; bias = stride-0 C-input row; act 0 none, 1 relu,
+# 2 clamp, 3 sigmoid, 4 silu; scale / shift = runtime scalars; colscale = per-column fp32 scales.
+FUSED_GOLDEN_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vecops_fused_golden.npz")
+
+FUSED_CASES = [
+    # MatmulFusionTest.RuntimePerColumnScaleAndClampAreFused (19, 23, 65)
+    {"name": "fz_bf16_scale", "kind": "bf16", "m": 19, "n": 23, "k": 65, "scale": 0.75},
+    {"name": "fz_bf16_colscale", "kind": "bf16", "m": 19, "n": 23, "k": 65, "colscale": True},
+    {"name": "fz_bf16_bias_clamp", "kind": "bf16", "m": 19, "n": 23, "k": 65, "bias": True, "act": 2,
+     "clamp": (-0.25, 0.25)},
+    # MatmulFusionTest.MixedBiasNarrowAndActivationsAreFused
+    {"name": "fz_bf16_bias_relu_bf16out", "kind": "bf16", "m": 19, "n": 23, "k": 65, "bias": True, "act": 1,
+     "out": "bf16"},
+    {"name": "fz_bf16_relu", "kind": "bf16", "m": 19, "n": 23, "k": 65, "act": 1},
+    {"name": "fz_bf16_sigmoid", "kind": "bf16", "m": 19, "n": 23, "k": 65, "act": 3},
+    {"name": "fz_bf16_sigmoid_1x8x129", "kind": "bf16", "m": 1, "n": 8, "k": 129, "act": 3},
+    {"name": "fz_bf16_silu_1x8x129", "kind": "bf16", "m": 1, "n": 8, "k": 129, "act": 4},
+    {"name": "fz_bf16_bias_silu_1x8x129", "kind": "bf16", "m": 1, "n": 8, "k": 129, "bias": True, "act": 4},
+    {"name": "fz_bf16_relu_8x1x129", "kind": "bf16", "m": 8, "n": 1, "k": 129, "act": 1},
+    # a shape with whole tiles and edges, every step at once, bf16 out
+    {"name": "fz_bf16_all_130x270x200", "kind": "bf16", "m": 130, "n": 270, "k": 200, "bias": True, "colscale": True,
+     "scale": 0.375, "shift": -0.125, "act": 4, "out": "bf16"},
+    # MatmulFusionTest.IndependentQuantizationAndNativeI8Accumulate: integer bias, per-column scale,
+    # requantisation with an output zero point (1, 8, 129)
+    {"name": "fz_i8_bias_colscale", "kind": "i8", "m": 1, "n": 8, "k": 129, "bias": True, "colscale": True},
+    {"name": "fz_i8_bias_colscale_zp_u8", "kind": "i8", "m": 1, "n": 8, "k": 129, "bias": True, "colscale": True,
+     "shift": 7.0, "out": "u8"},
+    # bigger and ragged, signed and unsigned byte outputs that saturate on both sides
+    {"name": "fz_i8_requant_u8_67x129x515", "kind": "i8", "m": 67, "n": 129, "k": 515, "bias": True, "colscale": True,
+     "shift": 128.0, "out": "u8"},
+    {"name": "fz_i8_requant_i8_67x129x515", "kind": "i8", "m": 67, "n": 129, "k": 515, "bias": True, "colscale": True,
+     "out": "i8"},
+    {"name": "fz_i8_scale_relu_67x129x515", "kind": "i8", "m": 67, "n": 129, "k": 515, "scale": -0.001953125, "act": 1},
+    {"name": "fz_i8_clamp_35x53x257", "kind": "i8", "m": 35, "n": 53, "k": 257, "colscale": True, "act": 2,
+     "clamp": (-20.0, 35.5)},
+    {"name": "fz_i8_sigmoid_35x53x257", "kind": "i8", "m": 35, "n": 53, "k": 257, "scale": 0.0001220703125, "act": 3},
+    {"name": "fz_i8_silu_256x384x1024", "kind": "i8", "m": 256, "n": 384, "k": 1024, "colscale": True, "act": 4},
+    # byte outputs of values outside int32 and of NaN (inf * 0): INT32_MIN before the saturating narrow
+    {"name": "fz_i8_huge_u8", "kind": "i8", "m": 5, "n": 40, "k": 64, "scale": 1.0e6, "out": "u8"},
+    {"name": "fz_i8_huge_i8", "kind": "i8", "m": 5, "n": 40, "k": 64, "scale": 1.0e6, "out": "i8"},
+    {"name": "fz_i8_inf_u8", "kind": "i8", "m": 5, "n": 40, "k": 64, "scale": float("inf"), "out": "u8",
+     "zero_rows": True},
+    {"name": "fz_i8_inf_i8", "kind": "i8", "m": 5, "n": 40, "k": 64, "scale": float("inf"), "out": "i8",
+     "zero_rows": True},
+]
+
+FUSED_OUT_DTYPES = {"f32": np.float32, "bf16": np.uint16, "u8": np.uint8, "i8": np.int8}
+
+
+def make_fused_inputs(case: dict) -> dict:
+    """a, b (bf16 bits as uint16, or int8), bias (fp32 / int32 [n] or None), column_scales (fp32 [n] or None)."""
+    m, n, k = case["m"], case["n"], case["k"]
+    out = {}
+    if case["kind"] == "bf16":
+        out["a"] = synth.bf16_round(synth.uniform_pm1(11, (m, k)))
+        out["b"] = synth.bf16_round(synth.uniform_pm1(12, (n, k)))
+        out["bias"] = synth.uniform_pm1(13, (n,)) if case.get("bias") else None
+    else:
+        out["a"] = synth.int8_sym(11, (m, k))
+        out["b"] = synth.int8_sym(12, (n, k))
+        if case.get("zero_rows"):
+            out["a"][1, :] = 0          # accumulator 0: inf * 0 = NaN
+        out["bias"] = (((synth.draws(13, n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32)
+                       if case.get("bias") else None)
+    out["column_scales"] = synth.scales(14, n) if case.get("colscale") else None
+    return out

@@ -24,7 +24,13 @@ EXPORTS = [
     "vecops_hip_matmul", "vecops_hip_matmul_i8_dequant", "vecops_hip_matmul_i8_dequant_workspace",
     "vecops_hip_matmul_w8a16_group", "vecops_hip_packed_b_bytes", "vecops_hip_pack_b", "vecops_hip_pack_b_compensated",
     "vecops_hip_plan_matmul_packed_b", "vecops_hip_matmul_packed_b", "vecops_hip_matmul_i8_dequant_packed_b",
+    "vecops_hip_plan_matmul_fused", "vecops_hip_matmul_fused",
 ]
+
+ACT_NONE, ACT_RELU, ACT_CLAMP, ACT_SIGMOID, ACT_SILU = 0, 1, 2, 3, 4
+ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "clamp": ACT_CLAMP, "sigmoid": ACT_SIGMOID,
+               "silu": ACT_SILU}
+EPILOGUE_SCALE, EPILOGUE_SHIFT = 1, 2
 
 
 class Operand(C.Structure):
@@ -35,6 +41,12 @@ class Operand(C.Structure):
 class Plan(C.Structure):
     _fields_ = [("family", C.c_uint32), ("split_k", C.c_uint32), ("vector_a", C.c_uint32), ("vector_b", C.c_uint32),
                 ("b_layout", C.c_uint32), ("reserved", C.c_uint32), ("workspace_bytes", C.c_uint64)]
+
+
+class Epilogue(C.Structure):
+    _fields_ = [("struct_size", C.c_uint32), ("activation", C.c_uint32), ("flags", C.c_uint32), ("scale", C.c_float),
+                ("shift", C.c_float), ("clamp_lo", C.c_float), ("clamp_hi", C.c_float), ("row_scales", C.c_void_p),
+                ("column_scales", C.c_void_p)]
 
 
 class VecopsHipError(RuntimeError):
@@ -77,6 +89,9 @@ def lib() -> C.CDLL:
         L.vecops_hip_matmul_i8_dequant_packed_b.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
                                                             C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                                             C.c_int64, C.c_void_p, C.c_uint64, C.c_void_p]
+        E = C.POINTER(Epilogue)
+        L.vecops_hip_plan_matmul_fused.argtypes = [P, P, P, P, C.c_uint32, E, C.POINTER(Plan)]
+        L.vecops_hip_matmul_fused.argtypes = [P, P, P, P, C.c_uint32, E, C.c_void_p, C.c_uint64, C.c_void_p]
         _lib = L
     return _lib
 
@@ -137,6 +152,47 @@ def matmul(a, b, c, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None
     ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
     _check(lib().vecops_hip_matmul(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None, C.byref(oc),
                                    compute, ws_ptr, ws_size, _stream_handle(stream)))
+    return c
+
+
+def epilogue(activation=None, scale=None, shift=None, row_scales=None, column_scales=None, clamp=(0.0, 0.0)) -> Epilogue:
+    """The fused output transform of ``matmul_fused``: ``act(((v * row_scales[row]) * column_scales[col]) * scale
+    + shift)`` on ``v = float(c_in + a . b^T)``; scale tensors are fp32 and live on the device."""
+    e = Epilogue()
+    e.struct_size = C.sizeof(Epilogue)
+    e.activation = ACTIVATIONS[activation] if not isinstance(activation, int) else activation
+    e.flags = (EPILOGUE_SCALE if scale is not None else 0) | (EPILOGUE_SHIFT if shift is not None else 0)
+    e.scale = 0.0 if scale is None else scale
+    e.shift = 0.0 if shift is None else shift
+    e.clamp_lo, e.clamp_hi = clamp
+    e.row_scales = row_scales.data_ptr() if row_scales is not None else None
+    e.column_scales = column_scales.data_ptr() if column_scales is not None else None
+    return e
+
+
+def plan_matmul_fused(a, b, c, ep: Epilogue, c_in=None, compute=COMPUTE_BF16) -> Plan:
+    plan = Plan()
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    _check(lib().vecops_hip_plan_matmul_fused(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None,
+                                              C.byref(oc), compute, C.byref(ep), C.byref(plan)))
+    return plan
+
+
+def matmul_fused(a, b, c, ep: Epilogue, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None):
+    """c = convert(transform(c_in + a . b^T)) with the output transform ``ep`` (see ``epilogue``) fused into the
+    kernel's store; a bias is a ``c_in`` whose row stride is 0.  Mirrors ``tensor::output<Acc>(c, transform)``."""
+    import torch
+    plan = plan_matmul_fused(a, b, c, ep, c_in, compute)
+    if plan.workspace_bytes and (workspace is None or workspace.numel() * workspace.element_size()
+                                 < plan.workspace_bytes):
+        workspace = torch.empty(plan.workspace_bytes, dtype=torch.uint8, device=c.device)
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_fused(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None,
+                                         C.byref(oc), compute, C.byref(ep), ws_ptr, ws_size, _stream_handle(stream)))
     return c
 
 

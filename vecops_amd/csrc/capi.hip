@@ -89,12 +89,14 @@ struct Problem {
   int64_t batch, m, n, k;
   bool packed_b;  // b.data addresses a prepacked operand (vecops_hip_pack_b), shared by every batch
   bool dequant;   // the int32 accumulators leave through the per-row x per-column dequantisation
+  const VecopsHipEpilogue* fused;  // non-null: c is written through the fused output transform
 };
 
 // Same rules as vecops' validate() (planning/families/ArchitectureFamily.h:1590-1652,
 // planning/families/GenericTiled.h:100-154) plus the dtype combinations this library implements.
 int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* cin,
-                 const VecopsHipOperand* c, uint32_t compute, Problem* pr) {
+                 const VecopsHipOperand* c, uint32_t compute, Problem* pr, const VecopsHipEpilogue* fused = nullptr) {
+  pr->fused = fused;
   if (!normalise(a, &pr->a) || !normalise(b, &pr->b) || !normalise(c, &pr->c))
     return fail(ST_INVALID, "matmul: operands must be rank 2 or 3 with non-negative extents");
   pr->packed_b = false;
@@ -137,7 +139,13 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
     return fail(ST_NOT_APPLICABLE, "matmul: operand dtype %u not supported", da);
   }
   const bool is_int = pr->src == SRC_I8 || pr->src == SRC_I8_FLIP;
-  if (is_int) {
+  if (is_int && fused) {
+    // the transform works on float(accumulator); the result is stored as fp32 or as a requantised byte
+    if (dc == DT_F32) pr->out_kind = OUT_F32;
+    else if (dc == DT_U8) pr->out_kind = OUT_U8;
+    else if (dc == DT_I8) pr->out_kind = OUT_I8;
+    else return fail(ST_NOT_APPLICABLE, "matmul_fused: int8 operands need an f32, u8 or i8 c");
+  } else if (is_int) {
     if (dc != DT_I32) return fail(ST_NOT_APPLICABLE, "matmul: int8 operands need an int32 c");
     pr->out_kind = OUT_I32;
   } else {
@@ -161,7 +169,7 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
     pr->m *= pr->batch;
     pr->batch = 1;
   }
-  pr->cin_kind = pr->out_kind;
+  pr->cin_kind = is_int ? OUT_I32 : pr->out_kind;
   if (pr->has_cin) {
     const uint32_t di = pr->cin.dtype;
     if (is_int) {
@@ -184,6 +192,7 @@ constexpr int64_t kQuality256x128 = 880, kQuality128 = 770;  // see choose()
 
 // bf16 x bf16 or int8 x int8 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
 bool skinny_applies(const Problem& pr) {
+  if (pr.fused) return false;  // the skinny kernels have no output transform
   if ((pr.src != SRC_BF16 && pr.src != SRC_I8) || pr.has_cin || pr.packed_b) return false;
   const int64_t per = pr.src == SRC_I8 ? 16 : 8;  // elements per 16 bytes
   if (!k_vector_ok(pr.a) || !k_vector_ok(pr.b) || pr.k % per != 0 || pr.k < 8 * per) return false;
@@ -309,6 +318,24 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   p.c_rs = pr.c.rs; p.c_cs = pr.c.cs; p.c_bs = pr.c.bs;
   if (pr.has_cin) { p.cin_rs = pr.cin.rs; p.cin_cs = pr.cin.cs; p.cin_bs = pr.cin.bs; }
   const bool is_int = pr.src == SRC_I8 || pr.src == SRC_I8_FLIP;
+  if (pr.fused) {
+    const VecopsHipEpilogue& ep = *pr.fused;
+    p.fused = 1;
+    p.ep_act = static_cast<int32_t>(ep.activation);
+    p.ep_flags = ep.flags & (VECOPS_HIP_EPILOGUE_SCALE | VECOPS_HIP_EPILOGUE_SHIFT);
+    p.ep_scale = ep.scale;
+    p.ep_shift = ep.shift;
+    p.ep_lo = ep.clamp_lo;
+    p.ep_hi = ep.clamp_hi;
+    if (is_int && ep.row_scales && ep.column_scales && pr.batch == 1) {
+      // both scales on int32 sums: the dequantisation stage of the kernels, the same two multiplies
+      p.row_scales = ep.row_scales;
+      p.column_scales = ep.column_scales;
+    } else {
+      p.ep_row_scales = ep.row_scales;
+      p.ep_column_scales = ep.column_scales;
+    }
+  }
 
   if (plan.family == VECOPS_HIP_FAMILY_ZERO_K) {
     p.split_k = 0;  // empty sum: the reduce kernel emits epilogue(0)
@@ -612,6 +639,41 @@ int32_t vecops_hip_plan_matmul(const VecopsHipOperand* a, const VecopsHipOperand
   if (rc != ST_OK) return rc;
   choose(pr, plan);
   return ST_OK;
+}
+
+namespace {
+int32_t check_epilogue(const VecopsHipEpilogue* ep) {
+  if (ep == nullptr) return fail(ST_INVALID, "matmul_fused: null epilogue");
+  if (ep->struct_size < sizeof(VecopsHipEpilogue)) return fail(ST_INVALID, "matmul_fused: epilogue record too short");
+  if (ep->activation > VECOPS_HIP_ACT_SILU) return fail(ST_INVALID, "matmul_fused: unknown activation %u", ep->activation);
+  return ST_OK;
+}
+}  // namespace
+
+int32_t vecops_hip_plan_matmul_fused(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                                     const VecopsHipOperand* c, uint32_t compute, const VecopsHipEpilogue* epilogue,
+                                     VecopsHipPlan* plan) {
+  if (plan == nullptr) return fail(ST_INVALID, "plan_matmul_fused: null plan");
+  int32_t rc = check_epilogue(epilogue);
+  if (rc != ST_OK) return rc;
+  Problem pr;
+  rc = describe(a, b, c_in, c, compute, &pr, epilogue);
+  if (rc != ST_OK) return rc;
+  choose(pr, plan);
+  return ST_OK;
+}
+
+int32_t vecops_hip_matmul_fused(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                                const VecopsHipOperand* c, uint32_t compute, const VecopsHipEpilogue* epilogue,
+                                void* workspace, uint64_t workspace_size, void* stream) {
+  int32_t rc = check_epilogue(epilogue);
+  if (rc != ST_OK) return rc;
+  Problem pr;
+  rc = describe(a, b, c_in, c, compute, &pr, epilogue);
+  if (rc != ST_OK) return rc;
+  VecopsHipPlan plan;
+  choose(pr, &plan);
+  return run_problem(pr, plan, nullptr, nullptr, nullptr, workspace, workspace_size, static_cast<hipStream_t>(stream));
 }
 
 int32_t vecops_hip_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,

@@ -45,7 +45,8 @@ typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
 // (v_mfma_f32_32x32x2_f32); a 16-byte chunk holds four k, a k-step (two chunks)
 // feeds four MFMAs per accumulator tile, a K tile is 32 elements.
 enum SrcKind : int { SRC_BF16 = 0, SRC_F32_AS_BF16 = 1, SRC_I8 = 2, SRC_I8_FLIP = 3, SRC_F32 = 4 };
-enum OutKind : int { OUT_F32 = 0, OUT_BF16 = 1, OUT_I32 = 2 };
+enum OutKind : int { OUT_F32 = 0, OUT_BF16 = 1, OUT_I32 = 2, OUT_U8 = 3, OUT_I8 = 4 };
+enum Activation : int { ACT_NONE = 0, ACT_RELU = 1, ACT_CLAMP = 2, ACT_SIGMOID = 3, ACT_SILU = 4 };
 // How an operand tile is fetched from global memory.
 enum LoadKind : int {
   LOAD_KVEC = 0,     // K contiguous, rows and base 16-byte aligned: one 16-byte load per chunk
@@ -81,6 +82,16 @@ struct TileGemmParams {
   int64_t b_rs, b_ks, b_bs;
   int64_t c_rs, c_cs, c_bs;
   int64_t cin_rs, cin_cs, cin_bs;
+  // Fused output transform (fused != 0), applied once the accumulator (+ C-input, + the dequantisation
+  // above) is a float:  v * ep_row_scales[row] * ep_column_scales[col] * ep_scale + ep_shift, then the
+  // activation, then the conversion to the memory dtype of C.
+  const float* ep_row_scales;     // [batch][M]; null = none
+  const float* ep_column_scales;  // null = none
+  float ep_scale, ep_shift;       // used when ep_flags has bit 0 / bit 1
+  float ep_lo, ep_hi;             // ACT_CLAMP bounds
+  uint32_t ep_flags;
+  int32_t ep_act;
+  int32_t fused;
 };
 
 template <int SRC>
@@ -320,6 +331,54 @@ __device__ __forceinline__ void mfma_step(typename AccTile<SrcTraits<SRC>::kInt>
   }
 }
 
+// The fused output transform in the order the header states.  Every step is its own fp32
+// operation (the file is compiled without contraction), as vecops' transforms are separate
+// vector instructions (tests/ops/MatmulConversionTestCommon.h:652-660, 735-740, 1047-1057,
+// 1121-1128, 1222-1234).
+__device__ __forceinline__ float apply_activation(const TileGemmParams& p, float v) {
+  switch (p.ep_act) {
+    // x86 max_ps(a, b) = a > b ? a : b and min_ps(a, b) = a < b ? a : b: NaN and equal zeros give b
+    case ACT_RELU: return v > 0.0f ? v : 0.0f;
+    case ACT_CLAMP: {
+      const float t = v > p.ep_lo ? v : p.ep_lo;
+      return t < p.ep_hi ? t : p.ep_hi;
+    }
+    case ACT_SIGMOID: return __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+    case ACT_SILU: return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+    default: return v;
+  }
+}
+
+__device__ __forceinline__ float finish_value(const TileGemmParams& p, float v, int batch, int row, int col) {
+  if (p.ep_row_scales) v *= p.ep_row_scales[static_cast<int64_t>(batch) * p.m + row];
+  if (p.ep_column_scales) v *= p.ep_column_scales[col];
+  if (p.ep_flags & 1u) v *= p.ep_scale;
+  if (p.ep_flags & 2u) v += p.ep_shift;
+  return apply_activation(p, v);
+}
+
+// fp32 -> 8-bit integer as vecops' x86 store path does it (vec/details/x86/Conversion.h:522-528:
+// a truncating convert to int32 - NaN and anything outside int32 give INT32_MIN - then a saturating
+// narrow).
+__device__ __forceinline__ uint32_t narrow_to_byte(float v, bool is_signed) {
+  const int32_t t = (v >= -2147483648.0f && v < 2147483648.0f) ? static_cast<int32_t>(v) : INT32_MIN;
+  return is_signed ? static_cast<uint32_t>(min(max(t, -128), 127)) & 0xffu : static_cast<uint32_t>(min(max(t, 0), 255));
+}
+
+// A finished fp32 value as the bits of one element of C (fp32, bf16, or an 8-bit integer).
+__device__ __forceinline__ uint32_t float_output_bits(int out_kind, float v) {
+  switch (out_kind) {
+    case OUT_BF16: return bf16_bits_rne(v);
+    case OUT_U8: return narrow_to_byte(v, false);
+    case OUT_I8: return narrow_to_byte(v, true);
+    default: return __float_as_uint(v);
+  }
+}
+
+__device__ __forceinline__ int output_element_bytes(int out_kind) {
+  return out_kind == OUT_BF16 ? 2 : (out_kind == OUT_U8 || out_kind == OUT_I8) ? 1 : 4;
+}
+
 // Final value of one output element: accumulator (+ correction) (+ Cin), then
 // the optional dequantisation, then conversion to the memory dtype of C.
 //   fp :  c = convert(acc + cin)
@@ -337,12 +396,15 @@ __device__ __forceinline__ uint32_t output_bits(const TileGemmParams& p, int bat
     if (p.cin) v += static_cast<uint32_t>(
                  static_cast<const int32_t*>(p.cin)[batch * p.cin_bs + row * p.cin_rs + col * p.cin_cs]);
     const int32_t s = static_cast<int32_t>(v);
+    float f = static_cast<float>(s);
     if (p.row_scales) {
-      const float t = static_cast<float>(s) * p.row_scales[row];
-      return __float_as_uint(t * p.column_scales[col]);
+      const float t = f * p.row_scales[row];
+      f = t * p.column_scales[col];
+    } else if (p.out_kind == OUT_I32) {
+      return v;
     }
-    if (p.out_kind == OUT_I32) return v;
-    return __float_as_uint(static_cast<float>(s));
+    if (p.fused) f = finish_value(p, f, batch, row, col);
+    return float_output_bits(p.out_kind, f);
   } else {
     float v = acc;
     if (p.cin) {
@@ -350,7 +412,8 @@ __device__ __forceinline__ uint32_t output_bits(const TileGemmParams& p, int bat
       v += (p.cin_kind == OUT_BF16) ? bf16_bits_to_f32(static_cast<const uint16_t*>(p.cin)[ci])
                                     : static_cast<const float*>(p.cin)[ci];
     }
-    return p.out_kind == OUT_BF16 ? bf16_bits_rne(v) : __float_as_uint(v);
+    if (p.fused) v = finish_value(p, v, batch, row, col);
+    return float_output_bits(p.out_kind, v);
   }
 }
 
@@ -358,8 +421,140 @@ template <bool INT, typename AccScalar>
 __device__ __forceinline__ void store_output(const TileGemmParams& p, int batch, int row, int col, AccScalar acc) {
   const int64_t c_off = batch * p.c_bs + row * p.c_rs + col * p.c_cs;
   const uint32_t bits = output_bits<INT, AccScalar>(p, batch, row, col, acc);
-  if (!INT && p.out_kind == OUT_BF16) static_cast<uint16_t*>(p.c)[c_off] = static_cast<uint16_t>(bits);
+  const int bytes = output_element_bytes(p.out_kind);
+  if (bytes == 2) static_cast<uint16_t*>(p.c)[c_off] = static_cast<uint16_t>(bits);
+  else if (bytes == 1) static_cast<uint8_t*>(p.c)[c_off] = static_cast<uint8_t>(bits);
   else static_cast<uint32_t*>(p.c)[c_off] = bits;
+}
+
+// Whether four consecutive elements of a row of C can leave as one store: contiguous columns and
+// row / batch strides and base that keep every quad aligned to its own size.
+__device__ __forceinline__ bool c_takes_quads(const TileGemmParams& p) {
+  const uintptr_t quad_bytes = 4u * output_element_bytes(p.out_kind);
+  return p.c_cs == 1 && (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(p.c) & (quad_bytes - 1)) == 0;
+}
+
+__device__ __forceinline__ void store_quad_bits(const TileGemmParams& p, int64_t c_off, const uint32_t (&bits)[4]) {
+  switch (output_element_bytes(p.out_kind)) {
+    case 2:
+      *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.c) + c_off) = u32x2{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16)};
+      break;
+    case 1:
+      *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(p.c) + c_off) = bits[0] | (bits[1] << 8) | (bits[2] << 16) | (bits[3] << 24);
+      break;
+    default:
+      *reinterpret_cast<u32x4*>(static_cast<uint32_t*>(p.c) + c_off) = u32x4{bits[0], bits[1], bits[2], bits[3]};
+  }
+}
+
+// The staged fast path's view of the output transform: the same operations in the same order as
+// output_bits, with every optional step turned into an operation that is exact when the step is absent
+// (x * 1.0f and x + -0.0f return x bit for bit; relu is clamp(0, +inf)), so that the per-element code has
+// no branches.  Built once per kernel from uniform parameters.
+struct Finisher {
+  float scale, shift, lo, hi;
+  bool clamps, smooth, silu, row_scaled;
+  bool int_sums, int_out;  // the staged values are int32 sums; they leave as int32
+  int out_kind;
+};
+
+template <bool INT>
+__device__ __forceinline__ Finisher make_finisher(const TileGemmParams& p, bool dequantised) {
+  Finisher f;
+  const bool on = p.fused != 0;
+  f.scale = (on && (p.ep_flags & 1u)) ? p.ep_scale : 1.0f;
+  f.shift = (on && (p.ep_flags & 2u)) ? p.ep_shift : -0.0f;
+  f.clamps = on && (p.ep_act == ACT_RELU || p.ep_act == ACT_CLAMP);
+  f.lo = p.ep_act == ACT_RELU ? 0.0f : p.ep_lo;
+  f.hi = p.ep_act == ACT_RELU ? __builtin_inff() : p.ep_hi;
+  f.smooth = on && (p.ep_act == ACT_SIGMOID || p.ep_act == ACT_SILU);
+  f.silu = p.ep_act == ACT_SILU;
+  f.row_scaled = on && p.ep_row_scales != nullptr;
+  f.int_sums = INT && !dequantised;
+  f.int_out = f.int_sums && p.out_kind == OUT_I32;
+  f.out_kind = p.out_kind;
+  return f;
+}
+
+// Four consecutive columns of one output row from their staged 32-bit values (int32 sums with the
+// correction added, dequantised fp32, or fp32 sums) to the bits of C.  C-input rows are contiguous and
+// need no alignment; `ecs` are the lane's four fused column scales (ones when there are none).
+typedef uint32_t u32x4_align4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x2_align2 __attribute__((ext_vector_type(2), aligned(2)));
+__device__ __forceinline__ void finish_quad(const TileGemmParams& p, const Finisher& fin, const u32x4& v, int batch,
+                                            int row, int col0, int cols_left, const f32x4& ecs, uint32_t (&bits)[4]) {
+  const uint32_t none = fin.int_sums ? 0u : 0x80000000u;  // adding int 0 or fp32 -0.0 changes nothing
+  u32x4 cin = {none, none, none, none};                   // int32, or fp32 bits (bf16 widened)
+  if (p.cin) {
+    const int64_t ci = batch * p.cin_bs + static_cast<int64_t>(row) * p.cin_rs + col0;
+    if (p.cin_kind == OUT_BF16) {
+      const uint16_t* src = static_cast<const uint16_t*>(p.cin) + ci;
+      if (cols_left >= 4) {
+        const u32x2_align2 h = *reinterpret_cast<const u32x2_align2*>(src);
+        cin = u32x4{h.x << 16, h.x & 0xffff0000u, h.y << 16, h.y & 0xffff0000u};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (e < cols_left) cin[e] = static_cast<uint32_t>(src[e]) << 16;
+      }
+    } else {
+      const uint32_t* src = static_cast<const uint32_t*>(p.cin) + ci;
+      if (cols_left >= 4) {
+        cin = *reinterpret_cast<const u32x4_align4*>(src);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (e < cols_left) cin[e] = src[e];
+      }
+    }
+  }
+  float f[4];
+  if (fin.int_sums) {
+    const u32x4 sum = v + cin;
+    if (fin.int_out) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bits[e] = sum[e];
+      return;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f[e] = static_cast<float>(static_cast<int32_t>(sum[e]));
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f[e] = __uint_as_float(v[e]) + __uint_as_float(cin[e]);
+  }
+  const float row_scale = fin.row_scaled ? p.ep_row_scales[static_cast<int64_t>(batch) * p.m + row] : 1.0f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float x = ((f[e] * row_scale) * ecs[e]) * fin.scale + fin.shift;
+    // x86 max_ps(a, b) = a > b ? a : b, min_ps(a, b) = a < b ? a : b
+    float t = x > fin.lo ? x : fin.lo;
+    t = t < fin.hi ? t : fin.hi;
+    f[e] = fin.clamps ? t : x;
+  }
+  if (fin.smooth) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-f[e]));
+      f[e] = fin.silu ? f[e] * sg : sg;
+    }
+  }
+  switch (fin.out_kind) {
+    case OUT_BF16:
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bits[e] = bf16_bits_rne(f[e]);
+      break;
+    case OUT_U8:
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bits[e] = narrow_to_byte(f[e], false);
+      break;
+    case OUT_I8:
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bits[e] = narrow_to_byte(f[e], true);
+      break;
+    default:
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bits[e] = __float_as_uint(f[e]);
+  }
 }
 
 // Four consecutive columns of one output row through the full epilogue, with bounds
@@ -388,16 +583,11 @@ __device__ __forceinline__ void store_quad_general(const TileGemmParams& p, int 
     }
     return;
   }
-  const bool bf16_out = !INT && p.out_kind == OUT_BF16;
   if (vec_c && col + 3 < p.n) {
     uint32_t bits[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) bits[e] = output_bits<INT, AccScalar>(p, batch, row, col + e, value(e));
-    const int64_t c_off = batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col;
-    if (bf16_out)
-      *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.c) + c_off) = u32x2{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16)};
-    else
-      *reinterpret_cast<u32x4*>(static_cast<uint32_t*>(p.c) + c_off) = u32x4{bits[0], bits[1], bits[2], bits[3]};
+    store_quad_bits(p, batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col, bits);
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e)
@@ -888,9 +1078,14 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
   const bool aligned = (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
   // the two fast paths take edge tiles too: their stores (and scale loads) are guarded per row and per run
   // of columns, which costs an interior tile a few compares
-  const bool simple = aligned && p.split_k == 1 && p.cin == nullptr && p.c_cs == 1 && SRC != SRC_I8_FLIP;
+  const bool dequant = INT && p.row_scales != nullptr;
+  // work that happens on the row-major side of the 32-bit staging: C-input, int32 sums leaving as floats,
+  // the fused output transform, outputs narrower than 32 bits
+  const bool finishing = p.cin != nullptr || p.fused != 0 || (INT ? (!dequant && p.out_kind != OUT_I32) : p.out_kind != OUT_F32);
+  const bool simple = aligned && p.split_k == 1 && p.c_cs == 1 && SRC != SRC_I8_FLIP &&
+                      (p.cin == nullptr || (p.cin_cs == 1 && !dequant));
   char* c_base = static_cast<char*>(p.c);
-  if (simple && !INT && p.out_kind == OUT_BF16) {
+  if (simple && !INT && p.out_kind == OUT_BF16 && p.cin == nullptr && p.fused == 0) {
     // bf16: 8-byte pieces scattered over 32 rows would waste most of every memory
     // transaction, so each wavefront first lays its tile out row-major in LDS (the
     // staging buffers are dead by now) and then stores whole 16-byte row segments.
@@ -939,7 +1134,7 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
         }
       }
     }
-  } else if (simple && (INT ? (p.out_kind == OUT_I32 || p.row_scales != nullptr) : p.out_kind == OUT_F32)) {
+  } else if (simple) {
     // 32-bit outputs: one 32-column block of the wavefront's tile at a time goes row-major through LDS
     // (128 rows x 128 bytes) and leaves as whole cache lines (16-byte pieces scattered over 32 rows, straight
     // from the accumulator layout, wrote 8192 x 8192 fp32 at 3.9 TB/s; whole lines at 4.9 TB/s).
@@ -947,13 +1142,14 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
     static_assert(ROWS * PITCH * 4 * WAVES_M * WAVES_N <= LDS_BYTES, "32-bit epilogue staging must fit the launch's LDS");
     __syncthreads();  // every wavefront is done reading fragments
     uint32_t* mine = reinterpret_cast<uint32_t*>(lds) + wave * (ROWS * PITCH);
-    const bool dequant = INT && p.row_scales != nullptr;
     float rs[WM];
     static_for<WM>([&](auto ci) {
       const int row = m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row;
       rs[decltype(ci)::value] = (dequant && row < p.m) ? p.row_scales[row] : 1.0f;
     });
     uint32_t* out = reinterpret_cast<uint32_t*>(c_base) + batch * p.c_bs + static_cast<int64_t>(m0 + wm * ROWS) * p.c_rs;
+    const int out_bytes = output_element_bytes(p.out_kind);
+    const Finisher fin = make_finisher<INT>(p, dequant);
     static_for<WN>([&](auto cj) {
       constexpr int j = decltype(cj)::value;
       const int col_block = n0 + (wn * WN + j) * 32;
@@ -999,19 +1195,52 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
         });
       });
       // the wavefront reads back only what it wrote itself: its own LDS traffic is ordered
+      if (!finishing) {
 #pragma unroll
-      for (int base = 0; base < ROWS * 8; base += 64) {
-        const int idx = base + lane, r = idx >> 3, cq = idx & 7;
-        const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + cq * 4);
-        uint32_t* dst = out + static_cast<int64_t>(r) * p.c_rs + col_block + cq * 4;
-        const int cols_left = p.n - (col_block + cq * 4);
-        if (m0 + wm * ROWS + r < p.m) {
-          if (cols_left >= 4) {
-            *reinterpret_cast<u32x4*>(dst) = v;
-          } else {
+        for (int base = 0; base < ROWS * 8; base += 64) {
+          const int idx = base + lane, r = idx >> 3, cq = idx & 7;
+          const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + cq * 4);
+          uint32_t* dst = out + static_cast<int64_t>(r) * p.c_rs + col_block + cq * 4;
+          const int cols_left = p.n - (col_block + cq * 4);
+          if (m0 + wm * ROWS + r < p.m) {
+            if (cols_left >= 4) {
+              *reinterpret_cast<u32x4*>(dst) = v;
+            } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (e < cols_left) dst[e] = v[e];
+              for (int e = 0; e < 4; ++e)
+                if (e < cols_left) dst[e] = v[e];
+            }
+          }
+        }
+      } else {
+        // a lane keeps its four columns through the whole block: their fused scales are loaded once
+        const int col0 = col_block + (lane & 7) * 4, cols_left = p.n - col0;
+        f32x4 ecs = {1.f, 1.f, 1.f, 1.f};
+        if (p.fused && p.ep_column_scales) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (e < cols_left) ecs[e] = p.ep_column_scales[col0 + e];
+        }
+#pragma unroll 4
+        for (int base = 0; base < ROWS * 8; base += 64) {
+          const int r = (base + lane) >> 3, row = m0 + wm * ROWS + r;
+          const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * PITCH + (lane & 7) * 4);
+          if (row < p.m && cols_left > 0) {
+            uint32_t bits[4];
+            finish_quad(p, fin, v, batch, row, col0, cols_left, ecs, bits);
+            const int64_t c_off = batch * p.c_bs + static_cast<int64_t>(row) * p.c_rs + col0;
+            if (cols_left >= 4) {
+              store_quad_bits(p, c_off, bits);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                if (e < cols_left) {
+                  if (out_bytes == 2) reinterpret_cast<uint16_t*>(c_base)[c_off + e] = static_cast<uint16_t>(bits[e]);
+                  else if (out_bytes == 1) reinterpret_cast<uint8_t*>(c_base)[c_off + e] = static_cast<uint8_t>(bits[e]);
+                  else reinterpret_cast<uint32_t*>(c_base)[c_off + e] = bits[e];
+                }
+              }
+            }
           }
         }
       }
@@ -1043,9 +1272,7 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
     static_assert(32 * PITCH * 4 * WAVES_M * WAVES_N <= LDS_BYTES, "general epilogue staging must fit the launch's LDS");
     __syncthreads();  // every wavefront is done reading fragments
     uint32_t* mine = reinterpret_cast<uint32_t*>(lds) + wave * (32 * PITCH);
-    const bool bf16_out = !INT && p.out_kind == OUT_BF16;
-    const bool vec_c = p.c_cs == 1 && (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 &&
-                       (reinterpret_cast<uintptr_t>(p.c) & (bf16_out ? 7 : 15)) == 0;
+    const bool vec_c = c_takes_quads(p);
     const bool vec_partial = (p.n & 3) == 0 && (reinterpret_cast<uintptr_t>(p.partial) & 15) == 0;
     static_for<WM>([&](auto ci) {
       constexpr int i = decltype(ci)::value;
@@ -1322,9 +1549,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const TileGemmParams
   // partials, one 16-byte or 8-byte store), else element by element
   const bool quads = (p.n & 3) == 0 && (reinterpret_cast<uintptr_t>(p.partial) & 15) == 0;
   if (quads) {
-    const bool bf16_out = !INT && p.out_kind == OUT_BF16;
-    const bool vec_c = p.c_cs == 1 && (p.c_rs & 3) == 0 && (p.c_bs & 3) == 0 &&
-                       (reinterpret_cast<uintptr_t>(p.c) & (bf16_out ? 7 : 15)) == 0;
+    const bool vec_c = c_takes_quads(p);
     typedef AccScalar Vec4 __attribute__((ext_vector_type(4)));
     TileGemmParams q = p;  // split_k is > 1 here, or 0 (the empty sum): the sums leave through the final epilogue
     q.split_k = 1;
