@@ -276,3 +276,30 @@ def test_gpu_fused_zero_k_and_validation(device):
     with pytest.raises(capi.VecopsHipError) as info:
         capi.matmul_fused(a8, b8, c, bad)
     assert info.value.code == 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(19, 23, 65), (32, 64, 128), (300, 270, 515)], ids=["19x23x65", "32x64x128", "300x270x515"])
+def test_gpu_dual_asymmetric_u8(device, oracle, shape):
+    """Both operands asymmetric uint8 with zero points 3 and 5: the int32 correction matrix
+    -za*sum(b) - zb*sum(a) + k*za*zb comes in as C-input and the sums leave through a fused scale
+    (tests/ops/MatmulConversionTestCommon.h:763-866, MatmulFusionTest.DualAsymmetricU8UsesRowAndColumnCorrection)."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = shape
+    za, zb = 3, 5
+    a = ((synth.draws(31, m * k) % np.uint64(7)).astype(np.int64) + za).astype(np.uint8).reshape(m, k)
+    b = ((synth.draws(32, n * k) % np.uint64(7)).astype(np.int64) + zb).astype(np.uint8).reshape(n, k)
+    sum_a = a.astype(np.int64).sum(axis=1)
+    sum_b = b.astype(np.int64).sum(axis=1)
+    corr = (-za * sum_b[None, :] - zb * sum_a[:, None] + k * za * zb).astype(np.int32)
+    # closed form: the corrected sum is the product of the zero-point-free values
+    exact = (a.astype(np.int64) - za) @ (b.astype(np.int64) - zb).T
+    want = exact.astype(np.float32) * np.float32(0.0625)
+    acc = np.zeros((m, n), np.int32)
+    oracle.matmul(a, b, acc, cin=corr, atom=O.ATOM_I8I32, acc_f64=True, c_bf16=False)
+    assert np.array_equal(oracle.fused_outputs(acc, np.float32, scale=0.0625), want)
+    c = torch.full((m, n), float("nan"), device=device)
+    capi.matmul_fused(_dev(a, device), _dev(b, device), c, capi.epilogue(scale=0.0625), c_in=_dev(corr, device))
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
