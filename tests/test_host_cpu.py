@@ -96,7 +96,7 @@ def test_abi_layout(tmp_path):
 
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
-    assert len(files) == 14
+    assert len(files) == 20
     for f in files:
         name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
         assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
@@ -181,6 +181,40 @@ def test_schema_validation(host):
     with pytest.raises(H.HostError) as e:
         deq.resolve(H.Frame([a, b, np.zeros(3, np.float32), np.zeros(5, np.float32), None, c], outputs=(5,)))
     assert e.value.code == 1 and "row_scales" in e.value.message
+
+
+def test_fused_operator_resolution_and_validation(host):
+    """vecops::matmul_fused: eleven positional values (five of them scalars), one artifact per operand class."""
+    op = host.operator("vecops::matmul_fused")
+    c = np.zeros((4, 5), np.float32)
+    scalars = [1, 1.0, 0.0, 0.0, 0.0]                      # activation relu, no scale, no shift, clamp bounds unused
+    frame = lambda a, b, cin, rs, cs, out, sc=scalars: H.Frame([a, b, cin, rs, cs] + sc + [out], outputs=(10,))  # noqa: E731
+    assert op.resolve(frame(bf16((4, 8)), bf16((5, 8)), None, None, None, c)) == \
+        "vecops::matmul_fused;operands=bf16;memory=host;backend=hip-gfx950"
+    f32 = np.zeros((4, 8), np.float32)
+    assert "operands=f32" in op.resolve(frame(f32, np.zeros((5, 8), np.float32), None, None, None, c))
+    a8, b8 = np.zeros((4, 8), np.int8), np.zeros((5, 8), np.int8)
+    bias = np.zeros((4, 5), np.int32)
+    for out in (c, np.zeros((4, 5), np.uint8), np.zeros((4, 5), np.int8)):
+        assert op.resolve(frame(a8, b8, bias, np.zeros(4, np.float32), np.zeros(5, np.float32), out)) == \
+            "vecops::matmul_fused;operands=i8;memory=host;backend=hip-gfx950"
+    bad = [
+        (frame(a8, b8, None, np.zeros(3, np.float32), None, c), 1, "row_scales"),
+        (frame(a8, b8, None, None, np.zeros(6, np.float32), c), 1, "column_scales"),
+        (frame(a8, b8, None, None, None, c, [7, 1.0, 0.0, 0.0, 0.0]), 1, "activation"),
+        (frame(a8, b8, None, None, None, c, [1.5, 1.0, 0.0, 0.0, 0.0]), 1, "activation"),      # a float where an int goes
+        (frame(bf16((4, 8)), bf16((5, 9)), None, None, None, c), 1, "K"),
+    ]
+    for fr, code, needle in bad:
+        with pytest.raises(H.HostError) as e:
+            op.resolve(fr)
+        assert e.value.code == code and needle in e.value.message, (needle, e.value.message)
+    with pytest.raises(H.HostError) as e:                  # int32 sums cannot leave as bf16: no recipe takes it
+        op.resolve(frame(a8, b8, None, None, None, bf16((4, 5))))
+    assert e.value.code in (2, 3)
+    with pytest.raises(H.HostError) as e:                  # bf16 sums cannot leave as bytes
+        op.resolve(frame(bf16((4, 8)), bf16((5, 8)), None, None, None, np.zeros((4, 5), np.uint8)))
+    assert e.value.code in (2, 3)
 
 
 def test_provider_without_artifacts_reports_not_found(host, tmp_path):

@@ -136,6 +136,52 @@ def test_matmul_i8_dequant_operator(host, oracle, device):
     assert np.array_equal(tc.cpu().numpy().view(np.uint32), oracle.matmul_i8_dequant(a, b, rs, cs).view(np.uint32))
 
 
+def test_matmul_fused_operator(host, oracle, device):
+    """vecops::matmul_fused through the Operator: int8 with an int32 bias row, both scale vectors, a shift and
+    requantisation to uint8 (host tensors, staged); bf16 with a bias row and silu to bf16 (device tensors)."""
+    import torch
+    op = host.operator("vecops::matmul_fused")
+    m, n, k = 67, 129, 515
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    rs, cs = synth.scales(3, m) * np.float32(64), synth.scales(4, n)
+    bias = ((synth.draws(5, n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32)
+    acc = np.zeros((m, n), np.int32)
+    oracle.matmul(a, b, acc, cin=np.broadcast_to(bias, (m, n)), atom=O.ATOM_I8I32, acc_f64=True, c_bf16=False)
+    want = oracle.fused_outputs(acc, np.uint8, row_scales=rs, column_scales=cs, shift=128.0)
+    assert (want == 0).any() and (want == 255).any()
+    c = np.full((m, n), 9, np.uint8)
+    bias_rows = np.broadcast_to(bias, (m, n))                                  # row stride 0
+    frame = H.Frame([a, b, bias_rows, rs, cs, 0, 1.0, 128.0, 0.0, 0.0, c], outputs=(10,))
+    assert op.resolve(frame) == "vecops::matmul_fused;operands=i8;memory=host;backend=hip-gfx950"
+    op.invoke(frame)
+    assert np.array_equal(c, want)
+    # relu on the same sums, fp32 out, device tensors
+    to = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(device)  # noqa: E731
+    want_relu = oracle.fused_outputs(acc, np.float32, column_scales=cs, scale=-0.5, activation=1)
+    tc = torch.full((m, n), float("nan"), device=device)
+    tbias = to(bias).reshape(1, n).expand(m, n)
+    frame = H.Frame([to(a), to(b), tbias, None, to(cs), 1, -0.5, 0.0, 0.0, 0.0, tc], outputs=(10,))
+    assert op.resolve(frame).endswith("operands=i8;memory=device;backend=hip-gfx950")
+    op.invoke(frame)
+    assert np.array_equal(tc.cpu().numpy().view(np.uint32), want_relu.view(np.uint32))
+    # bf16 operands, fp32 bias row, silu, bf16 out
+    m, n, k = 130, 270, 200
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    fbias = synth.uniform_pm1(3, (n,))
+    facc = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, facc, cin=np.broadcast_to(fbias, (m, n)), acc_f64=True, c_bf16=False)
+    want16 = oracle.fused_outputs(facc, np.uint16, activation=4)
+    ta = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+    tb = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
+    tc16 = torch.zeros((m, n), dtype=torch.bfloat16, device=device)
+    frame = H.Frame([ta, tb, to(fbias).reshape(1, n).expand(m, n), None, None, 4, 1.0, 0.0, 0.0, 0.0, tc16], outputs=(10,))
+    assert op.resolve(frame) == "vecops::matmul_fused;operands=bf16;memory=device;backend=hip-gfx950"
+    op.invoke(frame)
+    got16 = tc16.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert rel_err(synth.bf16_to_f32(got16), synth.bf16_to_f32(want16)) <= 2 ** -7
+
+
 def test_matmul_w8a16_group_operator(host, oracle, device):
     import torch
     op = host.operator("vecops::matmul_w8a16_group")

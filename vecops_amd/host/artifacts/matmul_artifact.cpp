@@ -1,8 +1,9 @@
 // Source of the HIP kernel-artifact DSOs for the vecops matmul operators.  One
 // DSO per (operator, operand class, memory placement); the build compiles this
 // file once per artifact with
-//   -DVECOPS_ARTIFACT_KIND=<0..5>   0 matmul bf16, 1 matmul f32 (bf16 compute), 5 matmul f32 (fp32 compute), 2 matmul i8,
-//                                   3 matmul_i8_dequant, 4 matmul_w8a16_group
+//   -DVECOPS_ARTIFACT_KIND=<0..8>   0 matmul bf16, 1 matmul f32 (bf16 compute), 5 matmul f32 (fp32 compute), 2 matmul i8,
+//                                   3 matmul_i8_dequant, 4 matmul_w8a16_group, 6 / 7 / 8 matmul_fused for bf16 / f32 /
+//                                   i8 operands
 //   -DVECOPS_ARTIFACT_DEVICE=<0|1>  0: tensors are host memory, staged through HBM here
 //                                   1: tensors are HIP device pointers, used in place
 //   -DVECOPS_ARTIFACT_GROUP=<G>     group size of kind 4
@@ -427,6 +428,178 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
                                     d.b->strides[0], static_cast<const float*>(rs), static_cast<const float*>(cs),
                                     static_cast<const int32_t*>(corr), static_cast<float*>(c), d.c->strides[0], d.m,
                                     d.n, d.k, ws, ws_size, stream);
+  if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
+  return finish(&staging, stream, error);
+}
+
+// =================================================================================================
+#elif VECOPS_ARTIFACT_KIND >= 6  // vecops::matmul_fused (a, b, c_in?, row_scales?, column_scales?, 5 scalars, c)
+// =================================================================================================
+
+#if VECOPS_ARTIFACT_KIND == 6
+#define OPERANDS "bf16"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16);
+#elif VECOPS_ARTIFACT_KIND == 7
+#define OPERANDS "f32"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
+#else
+#define OPERANDS "i8"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);
+#endif
+#if VECOPS_ARTIFACT_KIND == 8
+constexpr uint64_t kCinMask = bit(VECOPS_DTYPE_I32);
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_U8) | bit(VECOPS_DTYPE_I8);
+#else
+constexpr uint64_t kCinMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
+#endif
+
+constexpr const char* kOperatorName = "vecops::matmul_fused";
+constexpr const char* kKey = "vecops::matmul_fused;operands=" OPERANDS ";memory=" MEMORY_NAME ";backend=hip-gfx950";
+
+#define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
+   {.tensor = {sizeof(VecopsTensorParameter), MASK, kDeviceType, -1, RANK, OPTIONAL,                          \
+               sizeof(VecopsDimensionConstraint), nullptr, nullptr, FLAGS}}}
+#define SCALAR_PARAM(NAME, MASK) \
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_SCALAR, NAME, {.scalar = {sizeof(VecopsScalarParameter), MASK}}}
+
+constexpr uint64_t kRealMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_F64);
+
+const VecopsParameterDescriptor kParameters[] = {
+  TENSOR_PARAM("a", kInMask, -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("b", kInMask, -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("c_in", kCinMask, -1, 1, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("row_scales", bit(VECOPS_DTYPE_F32), -1, 1, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("column_scales", bit(VECOPS_DTYPE_F32), -1, 1, VECOPS_TENSOR_READ),
+  SCALAR_PARAM("activation", bit(VECOPS_DTYPE_I64) | bit(VECOPS_DTYPE_I32)),
+  SCALAR_PARAM("scale", kRealMask),
+  SCALAR_PARAM("shift", kRealMask),
+  SCALAR_PARAM("clamp_lo", kRealMask),
+  SCALAR_PARAM("clamp_hi", kRealMask),
+  TENSOR_PARAM("c", kOutMask, -1, 0, VECOPS_TENSOR_WRITE),
+};
+
+// Scalars travel as 64-bit storage whatever their dtype says (runtime/CallAbi.h: i64 / u64 / f64).
+bool scalar_arg(const VecopsCall* call, uint32_t index, const VecopsScalar** out) {
+  if (index >= call->num_values || call->values[index].kind != VECOPS_VALUE_SCALAR) return false;
+  *out = &call->values[index].value.scalar;
+  return true;
+}
+
+struct FusedArgs {
+  const VecopsTensorView *a, *b, *cin, *rs, *cs, *c;
+  VecopsHipOperand ops[4];  // a, b, c_in, c
+  VecopsHipEpilogue ep;
+};
+
+int32_t decode(const VecopsCall* call, FusedArgs* f, VecopsError* error) {
+  if (int32_t rc = check_call(call, 11, error); rc != VECOPS_STATUS_OK) return rc;
+  f->a = tensor_arg(call, 0);
+  f->b = tensor_arg(call, 1);
+  f->cin = tensor_arg(call, 2);
+  f->rs = tensor_arg(call, 3);
+  f->cs = tensor_arg(call, 4);
+  f->c = tensor_arg(call, 10);
+  if (f->a == nullptr || f->b == nullptr || f->c == nullptr)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "a, b and c must be tensors");
+  const VecopsScalar* s[5];
+  for (uint32_t i = 0; i < 5; ++i)
+    if (!scalar_arg(call, 5 + i, &s[i]))
+      return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "activation, scale, shift, clamp_lo and clamp_hi must be scalars");
+  if (s[0]->value.i64 < 0 || s[0]->value.i64 > VECOPS_HIP_ACT_SILU)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "activation must be 0 (none), 1 relu, 2 clamp, 3 sigmoid or 4 silu");
+  auto unit = [](const VecopsTensorView* t) { return t->rank == 1 && (t->sizes[0] <= 1 || t->strides[0] == 1); };
+  if ((f->rs && !unit(f->rs)) || (f->cs && !unit(f->cs)))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "row_scales and column_scales must be dense rank-1 tensors");
+  memset(&f->ep, 0, sizeof(f->ep));
+  f->ep.struct_size = sizeof(f->ep);
+  f->ep.activation = static_cast<uint32_t>(s[0]->value.i64);
+  const float scale = static_cast<float>(s[1]->value.f64), shift = static_cast<float>(s[2]->value.f64);
+  // a scale of exactly 1 and a shift of exactly 0 stand for "no such step" (the call ABI has no optional scalars)
+  if (scale != 1.0f) f->ep.flags |= VECOPS_HIP_EPILOGUE_SCALE;
+  if (shift != 0.0f) f->ep.flags |= VECOPS_HIP_EPILOGUE_SHIFT;
+  f->ep.scale = scale;
+  f->ep.shift = shift;
+  f->ep.clamp_lo = static_cast<float>(s[3]->value.f64);
+  f->ep.clamp_hi = static_cast<float>(s[4]->value.f64);
+  // 16 is a stand-in address with the alignment real allocations have; planning only reads metadata
+  if (!fill_operand(f->a, reinterpret_cast<void*>(16), &f->ops[0]) || !fill_operand(f->b, reinterpret_cast<void*>(16), &f->ops[1]) ||
+      !fill_operand(f->c, reinterpret_cast<void*>(16), &f->ops[3]) ||
+      (f->cin != nullptr && !fill_operand(f->cin, reinterpret_cast<void*>(16), &f->ops[2])))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "tensors must have rank 2 or 3");
+  const int64_t batch = f->a->rank == 3 ? f->a->sizes[0] : 1;
+  if ((f->rs && f->rs->sizes[0] != batch * f->a->sizes[f->a->rank - 2]) || (f->cs && f->cs->sizes[0] != f->b->sizes[f->b->rank - 2]))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "scale vectors must have one entry per row of a / per row of b");
+#if VECOPS_ARTIFACT_DEVICE
+  f->ops[0].data = origin(f->a);
+  f->ops[1].data = origin(f->b);
+  f->ops[3].data = origin(f->c);
+  if (f->cin != nullptr) f->ops[2].data = origin(f->cin);
+  f->ep.row_scales = f->rs ? reinterpret_cast<const float*>(origin(f->rs)) : nullptr;
+  f->ep.column_scales = f->cs ? reinterpret_cast<const float*>(origin(f->cs)) : nullptr;
+#else
+  // stand-ins so that planning sees which scale vectors exist
+  f->ep.row_scales = f->rs ? reinterpret_cast<const float*>(16) : nullptr;
+  f->ep.column_scales = f->cs ? reinterpret_cast<const float*>(16) : nullptr;
+#endif
+  return VECOPS_STATUS_OK;
+}
+
+int32_t plan(FusedArgs* f, VecopsHipPlan* out, VecopsError* error) {
+  int32_t rc = vecops_hip_plan_matmul_fused(&f->ops[0], &f->ops[1], f->cin ? &f->ops[2] : nullptr, &f->ops[3],
+                                            VECOPS_HIP_COMPUTE_BF16, &f->ep, out);
+  return rc == VECOPS_STATUS_OK ? rc : report_kernel(error, rc);
+}
+
+int32_t workspace_impl(const VecopsCall* call, uint64_t* bytes, VecopsError* error) {
+  FusedArgs f;
+  VecopsHipPlan p;
+  if (int32_t rc = decode(call, &f, error); rc != VECOPS_STATUS_OK) return rc;
+  if (int32_t rc = plan(&f, &p, error); rc != VECOPS_STATUS_OK) return rc;
+#if VECOPS_ARTIFACT_DEVICE
+  *bytes = p.workspace_bytes;
+#else
+  *bytes = 0;
+#endif
+  return VECOPS_STATUS_OK;
+}
+
+int32_t run_impl(const VecopsCall* call, VecopsError* error) {
+  FusedArgs f;
+  VecopsHipPlan p;
+  if (int32_t rc = decode(call, &f, error); rc != VECOPS_STATUS_OK) return rc;
+  if (int32_t rc = plan(&f, &p, error); rc != VECOPS_STATUS_OK) return rc;
+  if (p.family == VECOPS_HIP_FAMILY_NONE) return VECOPS_STATUS_OK;
+  hipStream_t stream = stream_of(call);
+  Staging staging(stream);
+  void* ws = call->workspace;
+  uint64_t ws_size = call->workspace_size;
+#if !VECOPS_ARTIFACT_DEVICE
+  // c first: if c_in aliases c they share the staged buffer and the write-back flag
+  const VecopsTensorView* views[4] = {f.a, f.b, f.cin, f.c};
+  const uint32_t order[4] = {3, 2, 0, 1};
+  for (uint32_t idx : order) {
+    if (views[idx] == nullptr) continue;
+    void* dev = nullptr;
+    if (int32_t rc = device_address(views[idx], idx == 3, &staging, &dev, error); rc != VECOPS_STATUS_OK) return rc;
+    f.ops[idx].data = dev;
+  }
+  void* dev = nullptr;
+  if (f.rs) {
+    if (int32_t rc = device_address(f.rs, false, &staging, &dev, error); rc != VECOPS_STATUS_OK) return rc;
+    f.ep.row_scales = static_cast<const float*>(dev);
+  }
+  if (f.cs) {
+    if (int32_t rc = device_address(f.cs, false, &staging, &dev, error); rc != VECOPS_STATUS_OK) return rc;
+    f.ep.column_scales = static_cast<const float*>(dev);
+  }
+  if (hipError_t e = staging.workspace(p.workspace_bytes, &ws); e != hipSuccess)
+    return report_hip(error, "allocating split-K scratch", e);
+  ws_size = p.workspace_bytes;
+#endif
+  int32_t rc = vecops_hip_matmul_fused(&f.ops[0], &f.ops[1], f.cin ? &f.ops[2] : nullptr, &f.ops[3],
+                                       VECOPS_HIP_COMPUTE_BF16, &f.ep, ws, ws_size, stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
   return finish(&staging, stream, error);
 }

@@ -70,6 +70,32 @@ Status dequant_relations(std::span<const Value> v) {
   return Status::success();
 }
 
+// vecops::matmul_fused: the matmul relations on (a, b, c_in, c = value 10) plus the scale vectors.
+Status fused_relations(std::span<const Value> v) {
+  const TensorView* a = tensor_at(v, 0);
+  const TensorView* b = tensor_at(v, 1);
+  const TensorView* cin = tensor_at(v, 2);
+  const TensorView* rs = tensor_at(v, 3);
+  const TensorView* cs = tensor_at(v, 4);
+  const TensorView* c = tensor_at(v, 10);
+  if (a == nullptr || b == nullptr || c == nullptr) return invalid("vecops::matmul_fused needs a, b and c tensors");
+  const std::size_t rank = a->sizes.size();
+  if (rank != 2 && rank != 3) return invalid("a must have rank 2 or 3");
+  if (b->sizes.size() != rank || c->sizes.size() != rank || (cin && cin->sizes.size() != rank))
+    return invalid("a, b, c_in and c must have the same rank");
+  if (cols(*a) != cols(*b)) return invalid("a and b disagree on K");
+  if (rows(*c) != rows(*a) || cols(*c) != rows(*b)) return invalid("c must be [.., M, N]");
+  if (cin && (rows(*cin) != rows(*c) || cols(*cin) != cols(*c))) return invalid("c_in must be [.., M, N]");
+  if (rank == 3 && (a->sizes[0] != b->sizes[0] || a->sizes[0] != c->sizes[0] || (cin && cin->sizes[0] != c->sizes[0])))
+    return invalid("batch extents differ");
+  const std::int64_t batch = rank == 3 ? a->sizes[0] : 1;
+  if (rs && rs->sizes[0] != batch * rows(*a)) return invalid("row_scales must have one entry per row of a");
+  if (cs && cs->sizes[0] != rows(*b)) return invalid("column_scales must have N entries");
+  const auto* act = std::get_if<rt::Scalar>(&v[5]);
+  if (act == nullptr || act->value.i64 < 0 || act->value.i64 > 4) return invalid("activation must be 0..4");
+  return Status::success();
+}
+
 Status w8a16_relations(std::span<const Value> v) {
   const TensorView* x = tensor_at(v, 0);
   const TensorView* w = tensor_at(v, 1);
@@ -149,6 +175,27 @@ rt::OperatorSchema make_matmul_i8_dequant_schema() {
   params.push_back(tensor_param("correction", dtype_bit(DType::Int32), 1u, VECOPS_TENSOR_READ, /*optional=*/true));
   params.push_back(tensor_param("c", dtype_bit(DType::Float32), 2u, VECOPS_TENSOR_WRITE));
   return rt::OperatorSchema(kMatmulI8DequantName, std::move(params), dequant_relations);
+}
+
+rt::OperatorSchema make_matmul_fused_schema() {
+  using rt::dtype_bit;
+  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8) |
+                           dtype_bit(DType::UInt8);
+  const std::uint64_t cin = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int32);
+  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::UInt8) |
+                            dtype_bit(DType::Int8);
+  const std::uint64_t real = dtype_bit(DType::Float32) | dtype_bit(DType::Float64);
+  std::vector<rt::ParameterSchema> params;
+  params.push_back(tensor_param("a", in, std::nullopt, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("b", in, std::nullopt, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("c_in", cin, std::nullopt, VECOPS_TENSOR_READ, /*optional=*/true));
+  params.push_back(tensor_param("row_scales", dtype_bit(DType::Float32), 1u, VECOPS_TENSOR_READ, /*optional=*/true));
+  params.push_back(tensor_param("column_scales", dtype_bit(DType::Float32), 1u, VECOPS_TENSOR_READ, /*optional=*/true));
+  params.push_back(rt::ParameterSchema{"activation", rt::ScalarConstraint{dtype_bit(DType::Int64) | dtype_bit(DType::Int32)}});
+  for (const char* name : {"scale", "shift", "clamp_lo", "clamp_hi"})
+    params.push_back(rt::ParameterSchema{name, rt::ScalarConstraint{real}});
+  params.push_back(tensor_param("c", out, std::nullopt, VECOPS_TENSOR_WRITE));
+  return rt::OperatorSchema(kMatmulFusedName, std::move(params), fused_relations);
 }
 
 rt::OperatorSchema make_matmul_w8a16_group_schema() {
@@ -246,6 +293,45 @@ rt::Result<rt::BoundKernelRecipe> MatmulI8DequantRecipe::bind(const rt::KernelCa
   return bound;
 }
 
+MatmulFusedRecipe::MatmulFusedRecipe(OperandClass operands) : operands_(operands) {
+  id_ = operands == OperandClass::BF16 ? "hip.matmul_fused.bf16.tile"
+        : operands == OperandClass::F32 ? "hip.matmul_fused.f32.tile"
+                                        : "hip.matmul_fused.i8.tile";
+}
+
+Status MatmulFusedRecipe::match(const rt::KernelCall& call) const {
+  const auto values = call.arguments().values();
+  const TensorView* a = tensor_at(values, 0);
+  const TensorView* b = tensor_at(values, 1);
+  const TensorView* cin = tensor_at(values, 2);
+  const TensorView* c = tensor_at(values, 10);
+  if (a == nullptr || b == nullptr || c == nullptr) return invalid("vecops::matmul_fused needs a, b and c tensors");
+  if (!takes(operands_, a->dtype) || !takes(operands_, b->dtype))
+    return not_applicable("operand dtypes belong to another recipe");
+  // int32 sums leave as fp32 or as requantised bytes; floating sums as fp32 or bf16
+  const bool integer = operands_ == OperandClass::I8;
+  const bool out_ok = integer ? (c->dtype == DType::Float32 || c->dtype == DType::UInt8 || c->dtype == DType::Int8)
+                              : (c->dtype == DType::Float32 || c->dtype == DType::BFloat16);
+  if (!out_ok) return not_applicable("output dtype does not fit these operands");
+  if (cin != nullptr &&
+      (integer ? cin->dtype != DType::Int32 : (cin->dtype != DType::Float32 && cin->dtype != DType::BFloat16)))
+    return not_applicable("c_in dtype does not fit these operands");
+  auto place = placement_of(call);
+  if (!place) return place.status();
+  return Status::success();
+}
+
+rt::Result<rt::BoundKernelRecipe> MatmulFusedRecipe::bind(const rt::KernelCall& call) const {
+  if (Status st = match(call); !st.ok()) return st;
+  const char* operands = operands_ == OperandClass::BF16 ? "bf16" : operands_ == OperandClass::F32 ? "f32" : "i8";
+  rt::BoundKernelRecipe bound;
+  bound.recipe_id = id_;
+  bound.specialization_key = std::string(kMatmulFusedName) + ";operands=" + operands + ";memory=" +
+                             placement_name(placement_of(call).value()) + ";" + kBackend;
+  bound.artifact_key = id_ + ";" + bound.specialization_key;
+  return bound;
+}
+
 Status MatmulW8A16GroupRecipe::match(const rt::KernelCall& call) const {
   auto place = placement_of(call);
   if (!place) return place.status();
@@ -285,6 +371,9 @@ MatmulDispatchPolicy::candidates(const rt::KernelCall& call,
     if (recipes[i] == nullptr) continue;
     if (const auto* mm = dynamic_cast<const MatmulRecipe*>(recipes[i].get()); mm != nullptr && a != nullptr) {
       if (!takes(mm->operands(), a->dtype)) continue;
+    }
+    if (const auto* mf = dynamic_cast<const MatmulFusedRecipe*>(recipes[i].get()); mf != nullptr && a != nullptr) {
+      if (!takes(mf->operands(), a->dtype)) continue;
     }
     order.push_back(i);
   }
@@ -375,6 +464,14 @@ std::shared_ptr<rt::Operator> make_matmul_operator(const std::filesystem::path& 
 
 std::shared_ptr<rt::Operator> make_matmul_i8_dequant_operator(const std::filesystem::path& dir) {
   return assemble(make_matmul_i8_dequant_schema(), {std::make_shared<MatmulI8DequantRecipe>()}, dir);
+}
+
+std::shared_ptr<rt::Operator> make_matmul_fused_operator(const std::filesystem::path& dir) {
+  return assemble(make_matmul_fused_schema(),
+                  {std::make_shared<MatmulFusedRecipe>(OperandClass::BF16),
+                   std::make_shared<MatmulFusedRecipe>(OperandClass::F32),
+                   std::make_shared<MatmulFusedRecipe>(OperandClass::I8)},
+                  dir);
 }
 
 std::shared_ptr<rt::Operator> make_matmul_w8a16_group_operator(const std::filesystem::path& dir) {

@@ -36,6 +36,7 @@ namespace rt = ::vecops::runtime;
 inline constexpr const char* kMatmulName = "vecops::matmul";
 inline constexpr const char* kMatmulI8DequantName = "vecops::matmul_i8_dequant";
 inline constexpr const char* kMatmulW8A16GroupName = "vecops::matmul_w8a16_group";
+inline constexpr const char* kMatmulFusedName = "vecops::matmul_fused";
 
 // Schemas.  Ranks are left open on vecops::matmul (rank 2 and rank 3 go through
 // one operator); the relation validator enforces what the CPU path asserts in
@@ -45,6 +46,12 @@ inline constexpr const char* kMatmulW8A16GroupName = "vecops::matmul_w8a16_group
 rt::OperatorSchema make_matmul_schema();
 rt::OperatorSchema make_matmul_i8_dequant_schema();
 rt::OperatorSchema make_matmul_w8a16_group_schema();
+// vecops::matmul_fused (a, b, c_in?, row_scales?, column_scales?, activation, scale, shift, clamp_lo, clamp_hi,
+// c out): vecops::matmul with a fused output transform, the catalogue that vecops' tests build from
+// tensor::output transforms (tests/ops/MatmulFusionTest.cpp:29-112).  The five scalars are always present
+// (the call ABI has no optional scalars): activation 0 none, 1 relu, 2 clamp, 3 sigmoid, 4 silu; scale 1.0 and
+// shift 0.0 mean "no such step".
+rt::OperatorSchema make_matmul_fused_schema();
 
 // Operand classes of vecops::matmul, one artifact each.
 enum class OperandClass { BF16, F32, I8 };
@@ -80,6 +87,21 @@ public:
   [[nodiscard]] std::string_view id() const override { return "hip.matmul_i8_dequant.tile"; }
   [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
   [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
+};
+
+// vecops::matmul_fused for one operand class (fp32 operands multiply in bf16):
+//   vecops::matmul_fused;operands=<bf16|f32|i8>;memory=<host|device>;backend=hip-gfx950
+class MatmulFusedRecipe final : public rt::KernelRecipe {
+public:
+  explicit MatmulFusedRecipe(OperandClass operands);
+  [[nodiscard]] std::string_view id() const override { return id_; }
+  [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
+  [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
+  [[nodiscard]] OperandClass operands() const { return operands_; }
+
+private:
+  OperandClass operands_;
+  std::string id_;
 };
 
 // vecops::matmul_w8a16_group, skinny family (M <= 16):  ...;G=<group>;memory=..;backend=hip-gfx950
@@ -134,6 +156,7 @@ std::string artifact_file_name(std::string_view specialization_key);
 std::shared_ptr<rt::Operator> make_matmul_operator(const std::filesystem::path& artifact_directory);
 std::shared_ptr<rt::Operator> make_matmul_i8_dequant_operator(const std::filesystem::path& artifact_directory);
 std::shared_ptr<rt::Operator> make_matmul_w8a16_group_operator(const std::filesystem::path& artifact_directory);
+std::shared_ptr<rt::Operator> make_matmul_fused_operator(const std::filesystem::path& artifact_directory);
 
 }  // namespace vecops::hip
 #endif

@@ -71,6 +71,7 @@ void* vecops_hip_host_operator_create(const char* operator_name, const char* art
   if (name == vecops::hip::kMatmulName) op = vecops::hip::make_matmul_operator(artifact_directory);
   else if (name == vecops::hip::kMatmulI8DequantName) op = vecops::hip::make_matmul_i8_dequant_operator(artifact_directory);
   else if (name == vecops::hip::kMatmulW8A16GroupName) op = vecops::hip::make_matmul_w8a16_group_operator(artifact_directory);
+  else if (name == vecops::hip::kMatmulFusedName) op = vecops::hip::make_matmul_fused_operator(artifact_directory);
   else return nullptr;
   return new Handle{std::move(op)};
 }

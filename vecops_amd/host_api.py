@@ -18,6 +18,7 @@ ARTIFACT_DIR = os.path.join(HERE, "lib", "artifacts")
 DEVICE_CPU, DEVICE_PRIVATE = 1, 255
 READ, WRITE = 1, 2
 I8, U8, I32, F16, BF16, F32 = 2, 3, 6, 10, 11, 12
+I64, F64 = 8, 13
 
 
 class TensorView(C.Structure):
@@ -69,6 +70,14 @@ class Frame:
             v.struct_size = C.sizeof(Value)
             if arg is None:
                 v.kind = 0
+                continue
+            if isinstance(arg, (int, float)) and not isinstance(arg, bool):   # scalar argument
+                v.kind = 2
+                v.value.scalar.struct_size = C.sizeof(Scalar)
+                if isinstance(arg, int):
+                    v.value.scalar.dtype, v.value.scalar.value.i64 = I64, arg
+                else:
+                    v.value.scalar.dtype, v.value.scalar.value.f64 = F64, arg
                 continue
             v.kind = 1
             t = v.value.tensor
