@@ -1,0 +1,148 @@
+"""The Torch registration facade (vecops_amd/torch_bridge.py), counterpart of vecops.ops.torch.register
+(python/vecops/ops/torch.py:35-86): name validation, idempotent registration, schemas with mutable outputs,
+Meta dispatch, error mapping without a GPU; on the GPU, results through torch.ops equal the C ABI's."""
+import numpy as np
+import pytest
+import torch
+
+from vecops_amd import host_api as H
+from vecops_amd import synth
+from vecops_amd import torch_bridge as tb
+
+
+def test_name_validation():
+    for bad in ("matmul", "a::b::c"):
+        with pytest.raises(ValueError, match="library::name"):
+            tb.register(bad)
+    for bad in ("::matmul", "lib::"):
+        with pytest.raises(ValueError, match="must not be empty"):
+            tb.register(bad)
+    with pytest.raises(ValueError, match="no HIP operator"):
+        tb.register("vecops_hip_t::transpose")
+    with pytest.raises(TypeError):
+        tb.register("vecops_hip_t::matmul", dispatch=object())
+
+
+def test_registration_is_idempotent_and_schemas_mark_outputs():
+    first = tb.register("vecops_hip_t::matmul")
+    assert tb.register("vecops_hip_t::matmul") is first
+    assert tb.vecops_hip_t.matmul is first
+    with pytest.raises(AttributeError):
+        tb.no_such_library
+    ns = tb.register_all("vecops_hip_t")
+    assert sorted(vars(ns)) == ["matmul", "matmul_fused", "matmul_i8_dequant", "matmul_w8a16_group"]
+    schema = str(torch.ops.vecops_hip_t.matmul.default._schema)
+    assert "Tensor? c_in" in schema and "Tensor(a!) c" in schema and "int ComputeType=-1" in schema
+    assert "-> ()" in schema
+    fused = str(torch.ops.vecops_hip_t.matmul_fused.default._schema)
+    assert "int activation" in fused and "float scale" in fused and "Tensor(a!) c" in fused
+    assert "int G=-1" in str(torch.ops.vecops_hip_t.matmul_w8a16_group.default._schema)
+
+
+def test_meta_tensors_and_argument_checks():
+    mm = tb.register("vecops_hip_t::matmul")
+    a = torch.empty(4, 8, dtype=torch.bfloat16, device="meta")
+    b = torch.empty(5, 8, dtype=torch.bfloat16, device="meta")
+    c = torch.empty(4, 5, device="meta")
+    assert mm(a, b, None, c) is c                        # the caller's own output object comes back
+    with pytest.raises(TypeError, match="positional"):
+        mm(a, b, c)
+    with pytest.raises(TypeError, match="unknown specialization"):
+        mm(a, b, None, c, Group=3)
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="this case is the no-GPU error path")
+def test_host_tensors_without_a_gpu_report_an_execution_error():
+    mm = tb.register("vecops_hip_t::matmul")
+    a, b, c = torch.zeros(4, 8, dtype=torch.bfloat16), torch.zeros(5, 8, dtype=torch.bfloat16), torch.zeros(4, 5)
+    with pytest.raises(H.HostError) as e:                # resolved, loaded, run() stops at "no HIP device"
+        mm(a, b, None, c)
+    assert e.value.code == 6
+    with pytest.raises(H.HostError) as e:                # schema violations surface as InvalidArgument
+        mm(a, torch.zeros(5, 9, dtype=torch.bfloat16), None, c)
+    assert e.value.code == 1 and "K" in e.value.message
+
+
+# ---- GPU ------------------------------------------------------------------------------------------
+
+def _bf16(x, device):
+    return torch.from_numpy(synth.bf16_round(x).view(np.int16)).to(device).view(torch.bfloat16)
+
+
+@pytest.mark.gpu
+def test_torch_ops_matmul_equals_the_c_abi(device):
+    from vecops_amd import capi
+    ns = tb.register_all("vecops_hip_t")
+    m, n, k = 300, 260, 1000
+    a, b = _bf16(synth.uniform_pm1(1, (m, k)), device), _bf16(synth.uniform_pm1(2, (n, k)), device)
+    want = torch.empty(m, n, device=device)
+    capi.matmul(a, b, want)
+    c = torch.full((m, n), float("nan"), device=device)
+    assert ns.matmul(a, b, None, c) is c
+    assert torch.equal(c, want)
+    # the raw torch.ops symbol, on a stream of its own, with a C-input that aliases the output
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        acc = torch.ones(m, n, device=device)
+        torch.ops.vecops_hip_t.matmul(a, b, acc, acc)
+    side.synchronize()
+    want2 = torch.empty(m, n, device=device)
+    capi.matmul(a, b, want2, c_in=torch.ones(m, n, device=device))
+    assert torch.equal(acc, want2)
+    # fp32 operands: the ComputeType specialization picks the artifact (torch dtype or VecopsDType number)
+    a32, b32 = torch.randn(64, 96, device=device), torch.randn(80, 96, device=device)
+    c_bf, c_f32 = torch.empty(64, 80, device=device), torch.empty(64, 80, device=device)
+    ns.matmul(a32, b32, None, c_bf)
+    ns.matmul(a32, b32, None, c_f32, ComputeType=torch.float32)
+    exact = a32.double() @ b32.double().T
+    assert (c_f32.double() - exact).abs().max() < 1e-4 < (c_bf.double() - exact).abs().max()
+    # split-K shape: the workspace comes from torch's allocator, its size is cached per signature
+    a, b = _bf16(synth.uniform_pm1(3, (255, 8191)), device), _bf16(synth.uniform_pm1(4, (63, 8191)), device)
+    c1, c2, want = (torch.empty(255, 63, device=device) for _ in range(3))
+    ns.matmul(a, b, None, c1)
+    ns.matmul(a, b, None, c2)
+    capi.matmul(a, b, want)
+    assert torch.equal(c1, want) and torch.equal(c2, want)
+
+
+@pytest.mark.gpu
+def test_torch_ops_quantised_operators(device, oracle):
+    ns = tb.register_all("vecops_hip_t")
+    m, n, k = 67, 129, 515
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    rs, cs = synth.scales(3, m), synth.scales(4, n)
+    to = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(device)  # noqa: E731
+    c = torch.zeros(m, n, device=device)
+    ns.matmul_i8_dequant(to(a), to(b), to(rs), to(cs), None, c)
+    want = oracle.matmul_i8_dequant(a, b, rs, cs)
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    # fused: dequantisation, silu, fp32 out; and requantisation to uint8
+    acc = oracle.matmul_i8_dense(a, b)
+    y = torch.zeros(m, n, device=device)
+    ns.matmul_fused(to(a), to(b), None, to(rs), to(cs), 1, 1.0, 0.0, 0.0, 0.0, y)
+    want_relu = oracle.fused_outputs(acc, np.float32, row_scales=rs, column_scales=cs, activation=1)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), want_relu.view(np.uint32))
+    q = torch.zeros(m, n, dtype=torch.uint8, device=device)
+    ns.matmul_fused(to(a), to(b), None, None, to(cs), 0, 0.5, 128, 0.0, 0.0, q)      # an int where a float goes
+    assert np.array_equal(q.cpu().numpy(), oracle.fused_outputs(acc, np.uint8, column_scales=cs, scale=0.5, shift=128.0))
+    # weight-only GEMV with the group size as a specialization value
+    k, n = 512, 256
+    x = synth.bf16_round(synth.normal(5, (2, k)))
+    w = synth.int8_sym(6, (n, k))
+    s = synth.scales(7, (n, k // 64))
+    yb = torch.zeros(2, n, dtype=torch.bfloat16, device=device)
+    ns.matmul_w8a16_group(torch.from_numpy(x.view(np.int16)).to(device).view(torch.bfloat16), to(w), to(s), yb, G=64)
+    bits, exact = oracle.matmul_w8a16_group(x, w, s, 64)
+    got = synth.bf16_to_f32(yb.view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
+    assert np.abs(got - exact).max() <= 2 ** -7 * np.abs(exact).max()
+
+
+@pytest.mark.gpu
+def test_torch_ops_host_tensors_are_staged(device):
+    ns = tb.register_all("vecops_hip_t")
+    a = torch.from_numpy(synth.uniform_pm1(1, (33, 70)))
+    b = torch.from_numpy(synth.uniform_pm1(2, (47, 70)))
+    c = torch.zeros(33, 47)
+    ns.matmul(a, b, None, c, ComputeType=torch.float32)
+    assert (c.double() - a.double() @ b.double().T).abs().max() < 1e-4

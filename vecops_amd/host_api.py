@@ -92,10 +92,11 @@ class Frame:
                 t.dtype = arg.view_dtype if hasattr(arg, "view_dtype") else _NP_CODES.get(arg.dtype, BF16)
                 shape, strides = arg.shape, [s // arg.itemsize for s in arg.strides]
                 self._keep.append(arg)
-            else:                               # torch tensor on the GPU
+            else:                               # torch tensor, on the GPU or in host memory
                 import torch
-                t.data, t.device_type = arg.data_ptr(), DEVICE_PRIVATE
-                t.device_index = arg.device.index or 0
+                on_host = arg.device.type == "cpu"
+                t.data, t.device_type = arg.data_ptr(), (DEVICE_CPU if on_host else DEVICE_PRIVATE)
+                t.device_index = 0 if on_host else (arg.device.index or 0)
                 t.dtype = {torch.int8: I8, torch.uint8: U8, torch.int32: I32, torch.bfloat16: BF16,
                            torch.float32: F32, torch.float16: F16}[arg.dtype]
                 shape, strides = tuple(arg.shape), tuple(arg.stride())
