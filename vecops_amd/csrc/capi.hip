@@ -411,6 +411,15 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   int mode = MODE_GENERIC;
   if (plan.vector_a && k_vector_ok(pr.b)) mode = MODE_KVEC;
   else if (plan.vector_a && plan.vector_b && plan.b_layout == 1) mode = MODE_NVEC_B;
+  // 16-byte aligned bases, rows and batches: the loads may write LDS themselves
+  const int64_t elem_bytes = pr.src == SRC_BF16 ? 2 : 1;
+  auto lines_up = [&](const View& v, int64_t line_stride) {
+    return aligned16(v.data) && (line_stride * elem_bytes) % 16 == 0 && (v.bs * elem_bytes) % 16 == 0;
+  };
+  if ((pr.src == SRC_BF16 || pr.src == SRC_I8) && lines_up(pr.a, pr.a.rs)) {
+    if (mode == MODE_KVEC && lines_up(pr.b, pr.b.rs)) mode = MODE_KVEC_DMA;
+    else if (mode == MODE_NVEC_B && lines_up(pr.b, pr.b.cs)) mode = MODE_NVEC_B_DMA;
+  }
 
   hipError_t e;
   if (pr.src == SRC_I8_FLIP) {

@@ -53,9 +53,14 @@ enum LoadKind : int {
   LOAD_GENERIC = 1,  // any strides / alignment: one load per element
   LOAD_NVEC = 2,     // spatial index contiguous (B given as [K,N] row-major), 16-byte aligned rows:
                      // transposed in registers on the way into LDS (32-bit compute elements)
-  LOAD_NTR = 3       // the same operand layout for 16-bit compute elements: stored in LDS as it
+  LOAD_NTR = 3,      // the same operand layout for 16-bit compute elements: stored in LDS as it
                      // lies in memory ([k][n]) and transposed by the LDS read (ds_read_b64_tr_b16)
+  LOAD_KDMA = 4,     // LOAD_KVEC with the loads writing LDS themselves (buffer_load ... lds): no staging
+                     // registers, no LDS store instructions
+  LOAD_NTR_DMA = 5   // LOAD_NTR likewise; rows of the [k][n] tile are packed (no pad) and swizzled instead
 };
+constexpr bool load_is_dma(int load) { return load == LOAD_KDMA || load == LOAD_NTR_DMA; }
+constexpr bool load_is_ntr(int load) { return load == LOAD_NTR || load == LOAD_NTR_DMA; }
 
 struct TileGemmParams {
   const void* a;
@@ -737,7 +742,7 @@ struct Stager {
     commit_part<PART>(lds_tile);
   }
   template <int PART, int OP>
-  __device__ __forceinline__ void load_op(int kt) {
+  __device__ __forceinline__ void load_op(int kt, char* /*lds_tile*/) {
     fetch_part<PART>(kt);
   }
 
@@ -871,8 +876,184 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
     commit_part<PART>(lds_tile);
   }
   template <int PART, int OP>
-  __device__ __forceinline__ void load_op(int kt) {
+  __device__ __forceinline__ void load_op(int kt, char* /*lds_tile*/) {
     fetch_part<PART>(kt);
+  }
+};
+
+// The partial last K tile of an operand stored [k][n] (bf16), bounds-checked, straight into the packed and
+// swizzled LDS tile of the LOAD_NTR_DMA stager: rows k >= K and columns n >= N read as zero.
+__device__ __noinline__ void stage_kn_checked(const void* base, int64_t ks, int first_n, int extent, int cols,
+                                              int k0_tile, int k_end, char* lds_tile, int tid, int threads) {
+  const int chunks_per_row = cols / 8;
+#pragma unroll 2
+  for (int idx = tid; idx < 64 * chunks_per_row; idx += threads) {
+    const int krow = idx / chunks_per_row, chunk = idx % chunks_per_row;
+    const int k = k0_tile + krow;
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    if (k < k_end) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int n = first_n + chunk * 8 + e;
+        if (n < extent)
+          w[e >> 1] |= static_cast<uint32_t>(static_cast<const uint16_t*>(base)[k * ks + n]) << ((e & 1) * 16);
+      }
+    }
+    *reinterpret_cast<u32x4*>(lds_tile + krow * (cols * 2) + ((chunk ^ ((krow & 3) << 2)) << 4)) = u32x4{w[0], w[1], w[2], w[3]};
+  }
+}
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+// The four words of a raw buffer descriptor over [base, base + 2 GiB): what tile_buffer() builds, as scalars.
+__device__ __forceinline__ u32x4 tile_buffer_words(const VECOPS_GLOBAL char* base) {
+  const uint64_t bits = reinterpret_cast<uint64_t>(base);
+  return u32x4{static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits))),
+               static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32) & 0xffffu)),
+               0x7fffffffu, 0x00020000u};
+}
+
+// One buffer load of 16 bytes per lane that writes LDS itself: lane l's bytes land at dst + 16 * l
+// (dst is wavefront-uniform).  Written as an instruction rather than through the compiler's builtin: the
+// compiler orders every later LDS read it cannot tell apart behind such a load - it would wait for the
+// load in front of each transposing fragment read of the tile being multiplied, which lies in the other
+// stage.  The kernel orders them itself: vmcnt(0) and a barrier before a stage filled this way is read.
+// (The instruction exists only in the device pass of the compiler.)
+__device__ __forceinline__ void load_16_bytes_into_lds(const u32x4& descriptor, lds_void_ptr dst, uint32_t lane_offset,
+                                                       uint32_t uniform_offset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t lds_address = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<size_t>(dst)));
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_address), "v"(lane_offset), "s"(descriptor), "s"(uniform_offset)
+               : "memory", "m0");
+#else
+  (void)descriptor; (void)dst; (void)lane_offset; (void)uniform_offset;
+#endif
+}
+
+// LOAD_KDMA: the K-contiguous stager whose loads write LDS themselves.  A load instruction of a
+// wavefront fills 1 KiB of LDS in lane order, which is eight rows of the tile; the swizzle of
+// lds_chunk_offset is kept by permuting which chunk of its row a lane fetches (the eight lanes of a row
+// still cover one contiguous 128 bytes of memory).  Part i is the wavefront's eight rows of pass i.
+template <int SRC, int ROWS, int THREADS>
+struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
+  using T = SrcTraits<SRC>;
+  static_assert(SRC == SRC_BF16 || SRC == SRC_I8, "operands that go into LDS as they are");
+  static constexpr int ROWS_PER_PASS = THREADS / 8;
+  static constexpr int CHUNKS = ROWS / ROWS_PER_PASS;
+  static_assert(CHUNKS >= 1, "tile too small for this many threads");
+  static constexpr int kParts = CHUNKS;
+  static constexpr int kStoreOps = 0;
+  static constexpr int kLoadOps = 1;
+  static constexpr bool kHasSpare = false;
+  static constexpr bool kStagesChecked = true;
+  struct Spare {};
+  const char* base;
+  u32x4 tile_buf;  // descriptor words, based at the first row of the tile, k = 0
+  uint32_t row_bytes[CHUNKS];
+  int64_t rs, ks;
+  int first_row, extent, k_end, tid_, wave_;
+
+  __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
+                                       int k_end_, int tid, uint32_t /*flip*/) {
+    base = static_cast<const char*>(base_);
+    rs = rs_;
+    ks = ks_;
+    first_row = first_row_;
+    extent = extent_;
+    k_end = k_end_;
+    tid_ = tid;
+    wave_ = __builtin_amdgcn_readfirstlane(tid >> 6);
+    tile_buf = tile_buffer_words((const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * rs * T::kSrcBytes));
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int tile_row = (tid >> 3) + i * ROWS_PER_PASS;
+      const int chunk = ((tid & 7) ^ tile_row ^ (tile_row >> 3)) & 7;  // the chunk whose swizzled slot is tid & 7
+      const int row = min(first_row + tile_row, extent - 1) - first_row;
+      row_bytes[i] = static_cast<uint32_t>((static_cast<int64_t>(row) * rs + chunk * T::kElemsPerChunk) * T::kSrcBytes);
+    }
+  }
+  __device__ __forceinline__ void dma_part(int part, int kt, char* lds_tile) const {
+    load_16_bytes_into_lds(tile_buf, (lds_void_ptr)(lds_tile + (part * ROWS_PER_PASS + wave_ * 8) * 128), row_bytes[part],
+                           kt * (8 * T::kElemsPerChunk * T::kSrcBytes));
+  }
+  __device__ __forceinline__ void dma_full(int kt, char* lds_tile) const {
+    static_for<CHUNKS>([&](auto ci) { dma_part(decltype(ci)::value, kt, lds_tile); });
+  }
+  __device__ __forceinline__ void stage_checked(int kt, char* lds_tile) const {
+    stage_rows_checked<SRC>(base, rs, ks, first_row, extent, ROWS, kt * 8 * T::kElemsPerChunk, k_end, lds_tile, tid_,
+                            THREADS, 0u);
+  }
+  template <int PART, int OP>
+  __device__ __forceinline__ void store_op(char*) const {}
+  template <int PART, int OP>
+  __device__ __forceinline__ void load_op(int kt, char* lds_tile) const {
+    dma_part(PART, kt, lds_tile);
+  }
+};
+
+// LOAD_NTR_DMA: the [k][n] stager whose loads write LDS themselves.  The 64 k rows of a tile lie
+// ROWS * 2 bytes apart with no pad, so that the 64 chunks a wavefront's load instruction fills are
+// contiguous; the four rows a transposing read touches are kept in different bank groups by xoring
+// bits 2-3 of the chunk slot with the row's low two bits.  bf16 only; tiles of 128 or more columns.
+template <int SRC, int ROWS, int THREADS>
+struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
+  using T = SrcTraits<SRC>;
+  static_assert(SRC == SRC_BF16, "operands that go into LDS as they are");
+  static constexpr int kPitch = ROWS * 2;
+  static constexpr int CHUNKS_PER_ROW = ROWS / 8;
+  static_assert(CHUNKS_PER_ROW >= 16, "the swizzle needs sixteen chunk slots per row");
+  static constexpr int CHUNKS = 64 * CHUNKS_PER_ROW / THREADS;
+  static_assert(CHUNKS >= 1 && 64 * CHUNKS_PER_ROW % THREADS == 0, "whole chunks per thread");
+  static_assert(THREADS % CHUNKS_PER_ROW == 0 && (THREADS / CHUNKS_PER_ROW) % 4 == 0, "a thread keeps its row's low bits");
+  static constexpr int K_ROWS_PER_PART = THREADS / CHUNKS_PER_ROW;
+  static constexpr int kParts = CHUNKS;
+  static constexpr int kStoreOps = 0;
+  static constexpr int kLoadOps = 1;
+  static constexpr bool kHasSpare = false;
+  static constexpr bool kStagesChecked = true;
+  struct Spare {};
+  const char* base;
+  const VECOPS_GLOBAL char* tile_base;
+  uint32_t chunk_bytes;
+  int64_t ks;
+  int first_row, extent, k_end, tid_, wave_;
+
+  __device__ __forceinline__ void init(const void* base_, int64_t /*rs*/, int64_t ks_, int first_row_, int extent_,
+                                       int k_end_, int tid, uint32_t /*flip*/) {
+    base = static_cast<const char*>(base_);
+    ks = ks_;
+    first_row = first_row_;
+    extent = extent_;
+    k_end = k_end_;
+    tid_ = tid;
+    wave_ = __builtin_amdgcn_readfirstlane(tid >> 6);
+    tile_base = uniform_ptr((const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * T::kSrcBytes));
+    const int krow = tid / CHUNKS_PER_ROW, slot = tid % CHUNKS_PER_ROW;
+    const int chunk = slot ^ ((krow & 3) << 2);  // the chunk whose swizzled slot this lane fills
+    // extent is a multiple of 8 on this path: a chunk past it is clamped onto the last one
+    const int n = min(first_row + chunk * 8, extent - 8) - first_row;
+    chunk_bytes = static_cast<uint32_t>((static_cast<int64_t>(krow) * ks + n) * T::kSrcBytes);
+  }
+  __device__ __forceinline__ uint32_t part_offset(int part) const {
+    return __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(part * K_ROWS_PER_PART * ks * T::kSrcBytes));
+  }
+  __device__ __forceinline__ void dma_part(int part, int kt, char* lds_tile) const {
+    const u32x4 buf = tile_buffer_words(tile_base + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes);
+    load_16_bytes_into_lds(buf, (lds_void_ptr)(lds_tile + (part * THREADS + wave_ * 64) * 16), chunk_bytes, part_offset(part));
+  }
+  __device__ __forceinline__ void dma_full(int kt, char* lds_tile) const {
+    static_for<CHUNKS>([&](auto ci) { dma_part(decltype(ci)::value, kt, lds_tile); });
+  }
+  __device__ __forceinline__ void stage_checked(int kt, char* lds_tile) const {
+    stage_kn_checked(base, ks, first_row, extent, ROWS, kt * 64, k_end, lds_tile, tid_, THREADS);
+  }
+  template <int PART, int OP>
+  __device__ __forceinline__ void store_op(char*) const {}
+  template <int PART, int OP>
+  __device__ __forceinline__ void load_op(int kt, char* lds_tile) const {
+    dma_part(PART, kt, lds_tile);
   }
 };
 
@@ -924,7 +1105,7 @@ struct Stager<SRC_F32, LOAD_NVEC, ROWS, THREADS> {
   }
 
   template <int PART, int R>
-  __device__ __forceinline__ void load_op(int kt) {
+  __device__ __forceinline__ void load_op(int kt, char* /*lds_tile*/) {
     if (!active(PART)) return;
     const VECOPS_GLOBAL char* row = tile_base + (static_cast<int64_t>(kt) * 32 + R) * ks * 4;
     const u32x4 v = *(const VECOPS_GLOBAL u32x4*)(uniform_ptr(row) + unit_bytes[PART]);
@@ -935,7 +1116,7 @@ struct Stager<SRC_F32, LOAD_NVEC, ROWS, THREADS> {
   }
   template <int PART>
   __device__ __forceinline__ void fetch_part(int kt) {
-    static_for<4>([&](auto cr) { load_op<PART, decltype(cr)::value>(kt); });
+    static_for<4>([&](auto cr) { load_op<PART, decltype(cr)::value>(kt, nullptr); });
   }
   __device__ __forceinline__ void fetch_full(int kt) {
     static_for<UNITS>([&](auto cu) { fetch_part<decltype(cu)::value>(kt); });
@@ -988,13 +1169,16 @@ struct StagingOp {
 template <typename SA, typename SB, bool B_TRANSPOSING>
 struct StagingSchedule {
   static constexpr int PARTS_A = SA::kParts, PARTS_B = SB::kParts;
+  static constexpr bool DMA = SA::kStoreOps == 0;  // loads that write LDS: all of them early, in k-steps 0 and 1
   static constexpr int step_a(int part) {
-    if constexpr (!B_TRANSPOSING) return part * 4 / (PARTS_A + PARTS_B);
+    if constexpr (DMA) return part * 2 / (PARTS_A + PARTS_B);
+    else if constexpr (!B_TRANSPOSING) return part * 4 / (PARTS_A + PARTS_B);
     else if constexpr (PARTS_B == 2) return part * 2 < PARTS_A ? 1 : 3;
     else return 1 + part * 3 / PARTS_A;
   }
   static constexpr int step_b(int part) {
-    if constexpr (!B_TRANSPOSING) return (PARTS_A + part) * 4 / (PARTS_A + PARTS_B);
+    if constexpr (DMA) return (PARTS_A + part) * 2 / (PARTS_A + PARTS_B);
+    else if constexpr (!B_TRANSPOSING) return (PARTS_A + part) * 4 / (PARTS_A + PARTS_B);
     else return part * 2;
   }
   // number of operations of k-step `step`
@@ -1034,7 +1218,7 @@ struct StagingSchedule {
 template <int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_B>
 constexpr int kStageBytes() {
   const int bm = 32 * WAVES_M * WM, bn = 32 * WAVES_N * WN;
-  return bm * 128 + (LOAD_B == LOAD_NTR ? 64 * (bn * 2 + 64) : bn * 128);
+  return bm * 128 + (LOAD_B == LOAD_NTR ? 64 * (bn * 2 + 64) : bn * 128);  // LOAD_NTR_DMA: 64 rows of bn * 2 bytes
 }
 
 // Dynamic LDS one workgroup is launched with: two staging stages, or the bf16
@@ -1346,12 +1530,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   for (int i = 0; i < WM; ++i) off_a[i] = lds_chunk_offset((wm * WM + i) * 32 + frag_row, frag_half);
 #pragma unroll
   for (int j = 0; j < WN; ++j) {
-    if constexpr (LOAD_B == LOAD_NTR) {
+    if constexpr (load_is_ntr(LOAD_B)) {
       // transposing read: 16-lane group g = lane / 16 serves columns (g & 1) * 16 .. + 15 of the fragment and
       // the k half g / 2; lane s of the group addresses row s / 4, columns 4 * (s % 4) .. + 3
-      constexpr int PITCH_B = Stager<SRC, LOAD_NTR, BN, THREADS>::kPitch;
+      constexpr int PITCH_B = Stager<SRC, LOAD_B, BN, THREADS>::kPitch;
       const int s = lane & 15, g = lane >> 4;
-      off_b[j] = BM * 128 + ((g >> 1) * 8 + (s >> 2)) * PITCH_B + ((wn * WN + j) * 32 + (g & 1) * 16 + (s & 3) * 4) * 2;
+      int col_bytes = ((wn * WN + j) * 32 + (g & 1) * 16 + (s & 3) * 4) * 2;
+      // packed rows: the 64-byte group is swizzled with the row's low two bits, which are s / 4 for both reads of
+      // every k-step
+      if constexpr (LOAD_B == LOAD_NTR_DMA) col_bytes ^= ((s >> 2) & 3) << 6;
+      off_b[j] = BM * 128 + ((g >> 1) * 8 + (s >> 2)) * PITCH_B + col_bytes;
     } else {
       off_b[j] = BM * 128 + lds_chunk_offset((wn * WN + j) * 32 + frag_row, frag_half);
     }
@@ -1387,9 +1575,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
     constexpr int r = decltype(r_tag)::value;
     if constexpr (r == 0) fa[set][0] = *reinterpret_cast<const u32x4*>(tile + (off_a[0] ^ (ks << 5)));
     else if constexpr (r <= WN) {
-      if constexpr (LOAD_B == LOAD_NTR) {
+      if constexpr (load_is_ntr(LOAD_B)) {
         // k-step ks covers rows 16*ks .. 16*ks+15 of the tile; the two reads give k 0-3 and 4-7 of the lane's half
-        constexpr int PITCH_B = Stager<SRC, LOAD_NTR, BN, THREADS>::kPitch;
+        constexpr int PITCH_B = Stager<SRC, LOAD_B, BN, THREADS>::kPitch;
         typedef __attribute__((ext_vector_type(4))) short s16x4;
         typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
         const char* at = tile + off_b[r - 1] + ks * 16 * PITCH_B;
@@ -1420,7 +1608,22 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   // for it, tile 1 into a spare set (position 1 is never the partial tile: one
   // straight path also keeps the count of loads in flight, which the waits of the
   // loop are derived from, exact); tile 0 to LDS; tile 1 into the staging registers.
-  if (nk > 0) {
+  constexpr bool DMA = load_is_dma(LOAD_A);
+  static_assert(load_is_dma(LOAD_A) == load_is_dma(LOAD_B), "both operands by loads into LDS, or neither");
+  if constexpr (DMA) {
+    // loads that write LDS: tile 0 goes straight into stage 0 (the partial tile through ordinary stores)
+    if (nk > 0) {
+      const int first = __builtin_amdgcn_readfirstlane(seq(0));
+      if (first < full_k_tiles) {
+        stager_a.dma_full(first, lds);
+        stager_b.dma_full(first, lds + BM * 128);
+      } else {
+        stager_a.stage_checked(first, lds);
+        stager_b.stage_checked(first, lds + BM * 128);
+      }
+    }
+  } else if constexpr (!DMA) {
+   if (nk > 0) {
     // one branch for both operands: a wait in front of the out-of-line checked
     // loader must not separate A's loads from B's
     // (scalar tile indices: a load whose uniform offset sits in a vector register is wrapped in a loop)
@@ -1450,6 +1653,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
       if constexpr (SB::kHasSpare) stager_b.take_spare(spare_b);
       else stager_b.fetch_full(second);
     }
+   }
   }
 
   Acc acc[WM][WN];
@@ -1479,14 +1683,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
         const char* tile = lds + (it & 1) * STAGE_BYTES;
         char* other = lds + ((it & 1) ^ 1) * STAGE_BYTES;
         // K tile to prefetch: seq(min(it + 2, nk - 1)), never the tail tile (position 0)
-        const int t2 = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(it + 2, nk - 1)));
+        // (loads that write LDS fetch the next tile, into the other stage)
+        const int t2 = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(it + (DMA ? 1 : 2), nk - 1)));
 
         auto stage_op = [&](auto step_tag, auto g_tag, auto order_tag) {
           constexpr StagingOp o = Sched::op(decltype(step_tag)::value, decltype(g_tag)::value, decltype(order_tag)::value);
+          // (a stager whose loads write LDS has no store operations; the others ignore the load's LDS address)
           if constexpr (o.operand == 0 && o.is_load == 0) stager_a.template store_op<o.part, o.op>(other);
-          if constexpr (o.operand == 0 && o.is_load == 1 && PREFETCH) stager_a.template load_op<o.part, o.op>(t2);
+          if constexpr (o.operand == 0 && o.is_load == 1 && PREFETCH) stager_a.template load_op<o.part, o.op>(t2, other);
           if constexpr (o.operand == 1 && o.is_load == 0) stager_b.template store_op<o.part, o.op>(other + BM * 128);
-          if constexpr (o.operand == 1 && o.is_load == 1 && PREFETCH) stager_b.template load_op<o.part, o.op>(t2);
+          if constexpr (o.operand == 1 && o.is_load == 1 && PREFETCH) stager_b.template load_op<o.part, o.op>(t2, other + BM * 128);
         };
         // Slots [S0, S1) of k-step STEP: MFMA x on fragment set mfma_set, then this
         // slot's share of the N_RD fragment reads (k-step read_ks of read_tile into
@@ -1526,6 +1732,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
         slots(I1{}, I0{}, All{}, Reads{}, std::true_type{}, std::false_type{}, 1, tile, 2);
         slots(I2{}, I0{}, All{}, Reads{}, std::true_type{}, std::false_type{}, 0, tile, 3);
         slots(I3{}, I0{}, Half{}, I0{}, std::true_type{}, std::true_type{}, 1, tile, 0);
+        if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the next tile has landed in the other stage
         lds_barrier();
         slots(I3{}, Half{}, All{}, Reads{}, std::false_type{}, std::false_type{}, 1, other, 0);
       }

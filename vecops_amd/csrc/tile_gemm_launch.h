@@ -13,7 +13,9 @@ namespace vecops_hip {
 enum LoadMode : int {
   MODE_GENERIC = 0,  // element loads, any strides
   MODE_KVEC = 1,     // A and B K-contiguous and 16-byte aligned
-  MODE_NVEC_B = 2    // A K-contiguous; B stored [K,N] row-major, 16-byte aligned (16- and 32-bit compute types)
+  MODE_NVEC_B = 2,   // A K-contiguous; B stored [K,N] row-major, 16-byte aligned (16- and 32-bit compute types)
+  MODE_KVEC_DMA = 3,   // MODE_KVEC with 16-byte aligned rows and bases: loads that write LDS themselves
+  MODE_NVEC_B_DMA = 4  // MODE_NVEC_B likewise
 };
 
 // tile_m x tile_n: 256x256, 256x128, 128x256, 128x128 or 64x64 (the workgroup tile).  Returns the HIP
@@ -59,6 +61,16 @@ hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
 
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN>
 hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t stream) {
+  // loads into LDS: bf16 and int8 operands on the tiles of 128 or more columns
+  if constexpr ((SRC == SRC_BF16 || SRC == SRC_I8) && WAVES_N * WN * 32 >= 128) {
+    if (mode == MODE_KVEC_DMA) return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KDMA, LOAD_KDMA>(p, stream);
+    if constexpr (SRC == SRC_BF16) {
+      if (mode == MODE_NVEC_B_DMA)
+        return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KDMA, LOAD_NTR_DMA>(p, stream);
+    }
+  }
+  if (mode == MODE_KVEC_DMA) mode = MODE_KVEC;
+  if (mode == MODE_NVEC_B_DMA) mode = MODE_NVEC_B;
   if (mode == MODE_KVEC) return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_KVEC>(p, stream);
   if constexpr (SrcTraits<SRC>::kElemsPerChunk == 8) {  // 16-bit compute: B untransposed in LDS, transposing reads
     if (mode == MODE_NVEC_B)

@@ -212,7 +212,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
           auto stage_op = [&](auto cg) {
             constexpr int g = decltype(cg)::value;
             if constexpr (g < NP) stager_a.template store_op<P0 + g, 0>(other);
-            else if constexpr (PREFETCH) stager_a.template load_op<P0 + g - NP, 0>(t2);
+            else if constexpr (PREFETCH) stager_a.template load_op<P0 + g - NP, 0>(t2, nullptr);
           };
           if constexpr (NS == 0) static_for<OPS>(stage_op);
           static_for<NS>([&](auto cs) {
