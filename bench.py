@@ -31,11 +31,11 @@ PEAK_HBM_GBPS = 8000.0
 # profiles/ (KiB per dispatch x 1024, FETCH scaled by 2.000 and WRITE by 1.000: what the
 # same counters read for a 1 GiB device copy, `--only copy`).  Counters cannot be read
 # from inside this process, so these are the recorded figures for exactly these workloads.
-TRAFFIC_BF16_4096 = int((98487 * 2.000 + 32768 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT = int((125552 * 2.000 + 88064 * 1.000) * 1024)
+TRAFFIC_BF16_4096 = int((98487.5 * 2.000 + 32768 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT = int((127024 * 2.000 + 88064 * 1.000) * 1024)
 TRAFFIC_GEMV_M1 = int((29647.4 * 2.000 + 112.0 * 1.000) * 1024)
-TRAFFIC_BF16_4096_PACKED = int((98470 * 2.000 + 32768 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT_PACKED = int((125228 * 2.000 + 88064 * 1.000) * 1024)
+TRAFFIC_BF16_4096_PACKED = int((98477.8 * 2.000 + 32768 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT_PACKED = int((125258 * 2.000 + 88064 * 1.000) * 1024)
 
 
 def _device_tensors_bf16_gemm(dev):
@@ -82,7 +82,7 @@ def bench_bf16_gemm(dev, steps, warmup):
         "wall_ms": wall_ms, "event_ms": ev_ms, "value": flops / (wall_ms * 1e-3) / 1e12,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BF16_4096,
-                     "kernel": "vecops_hip::tile_gemm_kernel<bf16, 256x256x64, B as [K,N]>",
+                     "kernel": "vecops_hip::tile_gemm_kernel<bf16, 256x256x64, loads into LDS, B as [K,N]>",
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": 3 * 2 * n * n},
         "host": (a, b_kn),
     }
@@ -106,7 +106,7 @@ def bench_int8_dequant(dev, steps, warmup):
             "dequant fused, fp32 out", "value": tops, "unit": "TOP/s", "ms_per_step": wall_ms, "dtype": "int8",
             "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                          "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT,
-                         "kernel": "vecops_hip::tile_gemm_kernel<int8, 256x128x128, dequant epilogue>",
+                         "kernel": "vecops_hip::tile_gemm_kernel<int8, 256x128x128, loads into LDS, dequant epilogue>",
                          "algorithmic_ops_per_launch": ops,
                          "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
 
