@@ -442,7 +442,8 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     if (pr.a_unsigned && pr.b_unsigned) p.const_term = 16384u * static_cast<uint32_t>(pr.k);
   }
   if (pr.packed_b) {
-    e = launch_tile_gemm_packed_b(pr.src, p, tile_m, tile_n, plan.vector_a != 0, stream);
+    const int a_mode = plan.vector_a == 0 ? 0 : ((pr.src == SRC_BF16 || pr.src == SRC_I8) && lines_up(pr.a, pr.a.rs)) ? 2 : 1;
+    e = launch_tile_gemm_packed_b(pr.src, p, tile_m, tile_n, a_mode, stream);
   } else switch (pr.src) {
     case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile_m, tile_n, mode, stream); break;
     case SRC_BF16: e = launch_tile_gemm_bf16(p, tile_m, tile_n, mode, stream); break;

@@ -932,6 +932,18 @@ __device__ __forceinline__ void load_16_bytes_into_lds(const u32x4& descriptor, 
 #endif
 }
 
+// The same load through the compiler's builtin, for a kernel that has other loads in flight: the compiler
+// counts it among them (it derives its vmcnt waits from the order of the loads it knows of), at the price
+// described above - fit for loops without transposing reads.
+__device__ __forceinline__ void load_16_bytes_into_lds_counted(__amdgpu_buffer_rsrc_t buffer, lds_void_ptr dst,
+                                                               uint32_t lane_offset, uint32_t uniform_offset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(buffer, dst, 16, lane_offset, uniform_offset, 0, 0);
+#else
+  (void)buffer; (void)dst; (void)lane_offset; (void)uniform_offset;
+#endif
+}
+
 // LOAD_KDMA: the K-contiguous stager whose loads write LDS themselves.  A load instruction of a
 // wavefront fills 1 KiB of LDS in lane order, which is eight rows of the tile; the swizzle of
 // lds_chunk_offset is kept by permuting which chunk of its row a lane fetches (the eight lanes of a row
@@ -951,6 +963,7 @@ struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
   struct Spare {};
   const char* base;
   u32x4 tile_buf;  // descriptor words, based at the first row of the tile, k = 0
+  __amdgpu_buffer_rsrc_t tile_rsrc;  // the same descriptor for the counted form of the load
   uint32_t row_bytes[CHUNKS];
   int64_t rs, ks;
   int first_row, extent, k_end, tid_, wave_;
@@ -966,6 +979,7 @@ struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
     tid_ = tid;
     wave_ = __builtin_amdgcn_readfirstlane(tid >> 6);
     tile_buf = tile_buffer_words((const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * rs * T::kSrcBytes));
+    tile_rsrc = tile_buffer((const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * rs * T::kSrcBytes));
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int tile_row = (tid >> 3) + i * ROWS_PER_PASS;
@@ -980,6 +994,10 @@ struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
   }
   __device__ __forceinline__ void dma_full(int kt, char* lds_tile) const {
     static_for<CHUNKS>([&](auto ci) { dma_part(decltype(ci)::value, kt, lds_tile); });
+  }
+  __device__ __forceinline__ void dma_part_counted(int part, int kt, char* lds_tile) const {
+    load_16_bytes_into_lds_counted(tile_rsrc, (lds_void_ptr)(lds_tile + (part * ROWS_PER_PASS + wave_ * 8) * 128),
+                                   row_bytes[part], kt * (8 * T::kElemsPerChunk * T::kSrcBytes));
   }
   __device__ __forceinline__ void stage_checked(int kt, char* lds_tile) const {
     stage_rows_checked<SRC>(base, rs, ks, first_row, extent, ROWS, kt * 8 * T::kElemsPerChunk, k_end, lds_tile, tid_,

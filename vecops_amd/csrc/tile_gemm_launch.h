@@ -31,8 +31,8 @@ hipError_t launch_byte_row_sums(const void* x, int32_t batch, int32_t rows, int3
                                 int64_t ks, uint32_t flip, uint32_t scale, int32_t* out, hipStream_t stream);
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
 // B prepacked by launch_pack_b (src: SRC_BF16, SRC_F32_AS_BF16 = fp32 A against bf16-packed B, SRC_I8);
-// vector_a: A is K-contiguous and 16-byte aligned
-hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_m, int tile_n, bool vector_a,
+// vector_a: 0 = any strides, 1 = A is K-contiguous, 2 = and its base, rows and batches are 16-byte aligned
+hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_m, int tile_n, int vector_a,
                                      hipStream_t stream);
 struct PackBParams;
 hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream);

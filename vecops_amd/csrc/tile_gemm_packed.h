@@ -152,8 +152,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
     __builtin_amdgcn_s_barrier();
   };
 
+  // LOAD_KDMA: A's loads write LDS themselves (the counted form: B's register loads are in flight beside them)
+  constexpr bool DMA_A = LOAD_A == LOAD_KDMA;
   // Start: A tiles 0 and 1 as in tile_gemm_kernel; the B fragments of tile 0.
-  if (nk > 0) {
+  if constexpr (DMA_A) {
+    if (nk > 0) {
+      const int first = __builtin_amdgcn_readfirstlane(seq(0));
+      if (first < full_k_tiles) static_for<SA::kParts>([&](auto ci) { stager_a.dma_part_counted(decltype(ci)::value, first, lds); });
+      else stager_a.stage_checked(first, lds);
+      static_for<4>([&](auto cks) { static_for<WN>([&](auto cj) { load_b(cks, cj, first); }); });
+    }
+  } else if constexpr (!DMA_A) {
+   if (nk > 0) {
     const int first = __builtin_amdgcn_readfirstlane(seq(0));
     const int second = __builtin_amdgcn_readfirstlane(seq(nk > 1 ? 1 : 0));
     const bool tail_first = first >= full_k_tiles;
@@ -170,6 +180,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
       if constexpr (SA::kHasSpare) stager_a.take_spare(spare_a);
       else stager_a.fetch_full(second);
     }
+   }
   }
 
   Acc acc[WM][WN];
@@ -206,13 +217,19 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
           constexpr int NS = S1 - S0;
           constexpr bool READS = decltype(reads_tag)::value, STAGE = decltype(stage_tag)::value;
           // the staging parts of this k-step: stores, then refills (k-step 3 has the barrier behind its stores)
-          constexpr int P0 = (KS * PARTS + 3) / 4, P1 = ((KS + 1) * PARTS + 3) / 4;
+          // (loads that write LDS: no stores; the parts of tile it + 1 go into the other stage in k-steps 0 and 1)
+          constexpr int P0 = DMA_A ? (KS < 2 ? KS * PARTS / 2 : PARTS) : (KS * PARTS + 3) / 4;
+          constexpr int P1 = DMA_A ? (KS < 2 ? (KS + 1) * PARTS / 2 : PARTS) : ((KS + 1) * PARTS + 3) / 4;
           constexpr int NP = STAGE ? P1 - P0 : 0;
-          constexpr int OPS = NP * 2;
+          constexpr int OPS = DMA_A ? NP : NP * 2;
           auto stage_op = [&](auto cg) {
             constexpr int g = decltype(cg)::value;
-            if constexpr (g < NP) stager_a.template store_op<P0 + g, 0>(other);
-            else if constexpr (PREFETCH) stager_a.template load_op<P0 + g - NP, 0>(t2, nullptr);
+            if constexpr (DMA_A) {
+              if constexpr (PREFETCH) stager_a.dma_part_counted(P0 + g, t1, other);
+            } else {
+              if constexpr (g < NP) stager_a.template store_op<P0 + g, 0>(other);
+              else if constexpr (PREFETCH) stager_a.template load_op<P0 + g - NP, 0>(t2, nullptr);
+            }
           };
           if constexpr (NS == 0) static_for<OPS>(stage_op);
           static_for<NS>([&](auto cs) {
@@ -240,6 +257,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
         slots(std::integral_constant<int, 1>{}, I0{}, All{}, std::true_type{}, std::true_type{});
         slots(std::integral_constant<int, 2>{}, I0{}, All{}, std::true_type{}, std::true_type{});
         slots(std::integral_constant<int, 3>{}, I0{}, Half{}, std::false_type{}, std::true_type{});
+        // A's loads of the next tile have landed once no more loads are in flight than the B fragment loads
+        // issued after them (those of k-step 2 and of the first half of k-step 3)
+        if constexpr (DMA_A) __builtin_amdgcn_s_waitcnt(0x0f70 | (WN + WN / 2));
         lds_barrier();
         slots(std::integral_constant<int, 3>{}, Half{}, All{}, std::true_type{}, std::false_type{});
       }

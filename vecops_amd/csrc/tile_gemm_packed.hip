@@ -38,14 +38,23 @@ hipError_t launch_packed_tile(const TileGemmParams& p, int tile_m, int tile_n, h
 }
 
 template <int SRC>
-hipError_t launch_packed_class(const TileGemmParams& p, int tile_m, int tile_n, bool vector_a, hipStream_t stream) {
+hipError_t launch_packed_class(const TileGemmParams& p, int tile_m, int tile_n, int vector_a, hipStream_t stream) {
+  // vector_a: 0 element loads, 1 16-byte loads, 2 16-byte loads that write LDS themselves (aligned bf16 / int8 A,
+  // the three big tiles)
+  if constexpr (SRC == SRC_BF16 || SRC == SRC_I8) {
+    if (vector_a == 2 && tile_m * tile_n >= 256 * 128) {
+      if (tile_m == 256 && tile_n == 256) return launch_packed_instance<SRC, 2, 2, 4, 4, LOAD_KDMA>(p, stream);
+      if (tile_m == 256 && tile_n == 128) return launch_packed_instance<SRC, 2, 2, 4, 2, LOAD_KDMA>(p, stream);
+      return launch_packed_instance<SRC, 2, 2, 2, 4, LOAD_KDMA>(p, stream);
+    }
+  }
   return vector_a ? launch_packed_tile<SRC, LOAD_KVEC>(p, tile_m, tile_n, stream)
                   : launch_packed_tile<SRC, LOAD_GENERIC>(p, tile_m, tile_n, stream);
 }
 
 }  // namespace
 
-hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_m, int tile_n, bool vector_a,
+hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_m, int tile_n, int vector_a,
                                      hipStream_t stream) {
   switch (src) {
     case SRC_BF16: return launch_packed_class<SRC_BF16>(p, tile_m, tile_n, vector_a, stream);
