@@ -99,6 +99,7 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul(const VecopsHipOperand* a, cons
  * C[..,M,N] = C_in + A[..,M,K] . B[..,N,K]^T  - replaces
  * ops::Matmul<Config>::operator() (ops/Matmul.h:530-570) for
  *   a,b bf16 -> c f32|bf16      (AMX_BF16F32)
+ *   a,b f16  -> c f32|f16       (AMX_F16F32 / SME_F16F32; IEEE half, round to nearest even)
  *   a,b f32  -> c f32|bf16      (bf16 or fp32 compute, see VecopsHipCompute)
  *   a,b i8|u8 -> c i32          (AMX_I8I32<A,B>, either side signed or unsigned;
  *                                accumulators wrap mod 2^32)
@@ -165,6 +166,7 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul_fused(const VecopsHipOperand* a
 /*
  * vecops_hip_matmul with the transform above between the accumulator and c.
  *   a,b bf16 | f32 -> c f32 | bf16      (c_in f32 | bf16)
+ *   a,b f16        -> c f32 | f16       (c_in f32 | f16)
  *   a,b i8 | u8    -> c f32 | u8 | i8   (c_in i32)
  * Operands, strides, batches, zero extents and the workspace rule are those of
  * vecops_hip_matmul (K == 0 writes transform(C_in or 0)).

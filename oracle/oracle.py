@@ -21,7 +21,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 
 # VecopsDType numeric values (runtime/CallAbi.h:62-91)
 I8, U8, I32, F16, BF16, F32 = 2, 3, 6, 10, 11, 12
-ATOM_BF16F32, ATOM_F32F32, ATOM_I8I32 = 0, 1, 2
+ATOM_BF16F32, ATOM_F32F32, ATOM_I8I32, ATOM_F16F32 = 0, 1, 2, 3
 SHAPE_AMX_BF16, SHAPE_AMX_I8_SAME, SHAPE_AMX_I8_MIXED, SHAPE_SME_F16, SHAPE_SME_OTHER = range(5)
 
 
@@ -33,6 +33,8 @@ class _Tensor(C.Structure):
 def _np_dtype_code(arr: np.ndarray, bf16: bool) -> int:
     if arr.dtype == np.float32:
         return F32
+    if arr.dtype == np.float16:
+        return F16
     if arr.dtype == np.uint16:
         return BF16 if bf16 else F16
     if arr.dtype == np.int8:
@@ -85,6 +87,9 @@ class Oracle:
         L.vo_f32_to_i32_sat.restype = C.c_int32
         L.vo_f32_to_i32_sat.argtypes = [C.c_float]
         L.vo_bf16_from_f32_array.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.vo_f16_from_f32_array.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.vo_f32_from_f16.restype = C.c_float
+        L.vo_f32_from_f16.argtypes = [C.c_uint16]
         L.vo_matmul.argtypes = [C.POINTER(_Tensor)] * 4 + [C.c_int, C.c_int]
         L.vo_matmul_sampled.argtypes = [C.POINTER(_Tensor)] * 2 + [C.c_int, C.c_void_p, C.c_void_p, C.c_int64,
                                                                    C.c_void_p]
@@ -105,6 +110,12 @@ class Oracle:
         x = np.ascontiguousarray(x, dtype=np.float32)
         out = np.empty(x.shape, dtype=np.uint16)
         self.lib.vo_bf16_from_f32_array(x.ctypes.data, out.ctypes.data, x.size)
+        return out
+
+    def f16_from_f32(self, x: np.ndarray) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.empty(x.shape, dtype=np.uint16)
+        self.lib.vo_f16_from_f32_array(x.ctypes.data, out.ctypes.data, x.size)
         return out
 
     @staticmethod

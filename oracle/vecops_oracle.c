@@ -12,6 +12,8 @@
  *   vo_bf16_from_f32 / vo_f32_from_bf16   - exhaustive agreement with the
  *       "add 0x7fff + lsb, shift" closed form and with IEEE nearest-even
  *       computed in fp64 (tests/test_oracle.py), NaN -> 0x7fc0.
+ *   vo_f16_from_f32                       - numpy's float16 conversion on random and
+ *       structured inputs, the exhaustive half -> float -> half round trip.
  *   vo_f32_to_i32_sat                     - known answers at the saturation
  *       edges and NaN (tests/test_oracle.py).
  *   vo_matmul (int paths)                 - exact integer arithmetic mod 2^32:
@@ -47,10 +49,13 @@ enum { VO_I8 = 2, VO_U8 = 3, VO_I32 = 6, VO_F16 = 10, VO_BF16 = 11, VO_F32 = 12 
  *   VO_ATOM_BF16F32 : operands rounded to bf16, fp32 accumulate (AMX_BF16F32,
  *                     matmul/details/kernel/amx/Atoms.h:51-60)
  *   VO_ATOM_F32F32  : operands kept in fp32 (SME_F32F32, kernel/sme/Atoms.h:65-76)
+ *   VO_ATOM_F16F32  : operands rounded to IEEE half, fp32 accumulate (AMX_F16F32,
+ *                     matmul/details/kernel/amx/Atoms.h:62-71; the reference build needs AMX-FP16,
+ *                     which the build host lacks: pinned by closed forms only)
  *   VO_ATOM_I8I32   : 8-bit integers, int32 accumulate wrapping mod 2^32
  *                     (AMX_I8I32<A,B>, amx/Atoms.h:73-86; wrap pinned by
  *                     tests/ops/MatmulTest.cpp:1025-1055) */
-enum { VO_ATOM_BF16F32 = 0, VO_ATOM_F32F32 = 1, VO_ATOM_I8I32 = 2 };
+enum { VO_ATOM_BF16F32 = 0, VO_ATOM_F32F32 = 1, VO_ATOM_I8I32 = 2, VO_ATOM_F16F32 = 3 };
 
 typedef struct vo_tensor {
   void* data;
@@ -87,6 +92,34 @@ static float f32_from_f16(uint16_t h) {
   }
   if (exp == 31) return bits_f32(sign | 0x7f800000u | (man << 13));
   return bits_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+/* binary32 -> IEEE binary16, round to nearest even, overflow to infinity, NaN kept quiet: what vecops'
+ * Float16(float) does through F16C (util/Float16.h, _cvtss_sh with nearest rounding).  Pinned against
+ * numpy's float16 conversion on random and structured inputs and by the exhaustive half -> float -> half
+ * round trip (tests/test_oracle.py). */
+VO_EXPORT uint16_t vo_f16_from_f32(float x) {
+  const uint32_t bits = f32_bits(x);
+  const uint32_t sign = (bits >> 16) & 0x8000u;
+  const uint32_t mag = bits & 0x7fffffffu;
+  if (mag > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((mag >> 13) & 0x3ffu));  /* NaN */
+  if (mag >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);  /* >= 65520 rounds to infinity (and infinity) */
+  if (mag < 0x38800000u) {                                     /* below 2^-14: subnormal half or zero */
+    if (mag < 0x33000000u) return (uint16_t)sign;              /* below 2^-25: rounds to zero */
+    const uint32_t man = (mag & 0x7fffffu) | 0x800000u;
+    const uint32_t shift = 126u - (mag >> 23);                 /* 14 .. 24 */
+    const uint32_t kept = man >> shift, rest = man & ((1u << shift) - 1u), half = 1u << (shift - 1u);
+    return (uint16_t)(sign | (kept + ((rest > half || (rest == half && (kept & 1u))) ? 1u : 0u)));
+  }
+  const uint32_t base = ((mag >> 23) - 112u) << 10 | ((mag >> 13) & 0x3ffu);
+  const uint32_t rest = mag & 0x1fffu;
+  return (uint16_t)(sign | (base + ((rest > 0x1000u || (rest == 0x1000u && (base & 1u))) ? 1u : 0u)));
+}
+
+VO_EXPORT float vo_f32_from_f16(uint16_t h);
+
+VO_EXPORT void vo_f16_from_f32_array(const float* in, uint16_t* out, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) out[i] = vo_f16_from_f32(in[i]);
 }
 
 /* util/ScalarConvert.h:60-86: float -> signed int truncates toward zero after a
@@ -142,6 +175,7 @@ static inline void store_from_f32(void* p, int dtype, int64_t off, float v) {
   switch (dtype) {
     case VO_F32: ((float*)p)[off] = v; break;
     case VO_BF16: ((uint16_t*)p)[off] = vo_bf16_from_f32(v); break;
+    case VO_F16: ((uint16_t*)p)[off] = vo_f16_from_f32(v); break;
     case VO_I32: ((int32_t*)p)[off] = vo_f32_to_i32_sat(v); break;
     default: break;
   }
@@ -155,7 +189,10 @@ static inline void store_from_i32(void* p, int dtype, int64_t off, int32_t v) {
   }
 }
 
+VO_EXPORT float vo_f32_from_f16(uint16_t h) { return f32_from_f16(h); }
+
 static inline float to_compute(float v, int atom) {
+  if (atom == VO_ATOM_F16F32) return f32_from_f16(vo_f16_from_f32(v));
   return atom == VO_ATOM_BF16F32 ? vo_f32_from_bf16(vo_bf16_from_f32(v)) : v;
 }
 

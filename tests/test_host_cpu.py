@@ -96,7 +96,7 @@ def test_abi_layout(tmp_path):
 
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
-    assert len(files) == 20
+    assert len(files) == 24
     for f in files:
         name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
         assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
@@ -123,6 +123,13 @@ def test_resolve_picks_recipe_by_dtype_and_placement(host):
         "vecops::matmul;operands=f32;compute=bf16;memory=host;backend=hip-gfx950"
     assert op.resolve(H.Frame([bf16((4, 8)), bf16((5, 8)), None, c32], outputs=(3,))) == \
         "vecops::matmul;operands=bf16;compute=bf16;memory=host;backend=hip-gfx950"
+    ah, bh = np.zeros((4, 8), np.float16), np.zeros((5, 8), np.float16)
+    for ch in (c32, np.zeros((4, 5), np.float16)):          # half operands write fp32 or half
+        assert op.resolve(H.Frame([ah, bh, None, ch], outputs=(3,))) == \
+            "vecops::matmul;operands=f16;compute=f16;memory=host;backend=hip-gfx950"
+    with pytest.raises(H.HostError) as e:                   # ... not bf16
+        op.resolve(H.Frame([ah, bh, None, bf16((4, 5))], outputs=(3,)))
+    assert e.value.code in (2, 3)
     ai, bi, ci = np.zeros((4, 8), np.int8), np.zeros((5, 8), np.int8), np.zeros((4, 5), np.int32)
     assert op.resolve(H.Frame([ai, bi, None, ci], outputs=(3,))) == \
         "vecops::matmul;operands=i8;compute=i32;memory=host;backend=hip-gfx950"
@@ -193,6 +200,8 @@ def test_fused_operator_resolution_and_validation(host):
         "vecops::matmul_fused;operands=bf16;memory=host;backend=hip-gfx950"
     f32 = np.zeros((4, 8), np.float32)
     assert "operands=f32" in op.resolve(frame(f32, np.zeros((5, 8), np.float32), None, None, None, c))
+    assert "operands=f16" in op.resolve(frame(np.zeros((4, 8), np.float16), np.zeros((5, 8), np.float16), None, None,
+                                              None, np.zeros((4, 5), np.float16)))
     a8, b8 = np.zeros((4, 8), np.int8), np.zeros((5, 8), np.int8)
     bias = np.zeros((4, 5), np.int32)
     for out in (c, np.zeros((4, 5), np.uint8), np.zeros((4, 5), np.int8)):

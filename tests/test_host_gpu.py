@@ -136,6 +136,24 @@ def test_matmul_i8_dequant_operator(host, oracle, device):
     assert np.array_equal(tc.cpu().numpy().view(np.uint32), oracle.matmul_i8_dequant(a, b, rs, cs).view(np.uint32))
 
 
+def test_matmul_f16_operator(host, oracle, device):
+    import torch
+    op = host.operator("vecops::matmul")
+    m, n, k = 130, 264, 200
+    a = synth.uniform_pm1(1, (m, k)).astype(np.float16)
+    b = synth.uniform_pm1(2, (n, k)).astype(np.float16)
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, atom=O.ATOM_F16F32, acc_f64=True)
+    c = np.full((m, n), np.nan, np.float32)
+    op.invoke(H.Frame([a, b, None, c], outputs=(3,)))                       # host tensors, staged
+    assert rel_err(c, want) <= fp32_tol(k)
+    th = torch.zeros((m, n), dtype=torch.float16, device=device)
+    frame = H.Frame([torch.from_numpy(a).to(device), torch.from_numpy(b).to(device), None, th], outputs=(3,))
+    assert op.resolve(frame) == "vecops::matmul;operands=f16;compute=f16;memory=device;backend=hip-gfx950"
+    op.invoke(frame)
+    assert rel_err(th.cpu().numpy().astype(np.float32), want) <= 2.0 ** -10
+
+
 def test_matmul_fused_operator(host, oracle, device):
     """vecops::matmul_fused through the Operator: int8 with an int32 bias row, both scale vectors, a shift and
     requantisation to uint8 (host tensors, staged); bf16 with a bias row and silu to bf16 (device tensors)."""

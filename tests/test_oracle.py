@@ -314,3 +314,51 @@ def test_oracle_matches_reference_views(oracle, reference):
     got_c = c.copy()
     oracle.matmul(a, b, got_c, cin=got_c, acc_f64=True)
     assert rel_err(got_c, want_c) <= 2e-6
+
+
+# --- IEEE half -------------------------------------------------------------------
+
+def test_f16_rounding_matches_numpy_and_round_trips(oracle):
+    """vo_f16_from_f32 against numpy's float32 -> float16 (IEEE round to nearest even), which shares no
+    code with it: random bit patterns, every half value's neighbourhood (ties included), the subnormal
+    range, the overflow edge; and half -> float -> half is the identity for every non-NaN half."""
+    rng = np.random.default_rng(3)
+    raw = rng.integers(0, 2 ** 32, size=1 << 20, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    halves = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16).astype(np.float32)
+    ulp = np.spacing(halves.view(np.uint32).view(np.float32))
+    ties = halves + np.float32(0.5) * np.diff(np.append(halves, np.float32(65536.0)))    # exact midpoints
+    near = np.concatenate([halves, ties, np.nextafter(ties, np.float32(0)), np.nextafter(ties, np.float32(1e9))])
+    edge = np.array([65503.9, 65504.0, 65519.9, 65520.0, 65536.0, 1e9, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001,
+                     2.0 ** -26, 0.0, -0.0], np.float32)
+    x = np.concatenate([raw[np.isfinite(raw)], near, -near, edge, -edge]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(oracle.f16_from_f32(x), want)
+    every = np.arange(0, 1 << 16, dtype=np.uint16)
+    not_nan = ~np.isnan(every.view(np.float16))
+    back = oracle.f16_from_f32(every.view(np.float16).astype(np.float32))
+    assert np.array_equal(back[not_nan], every[not_nan])
+    assert oracle.lib.vo_f32_from_f16(0x3C00) == 1.0 and oracle.lib.vo_f32_from_f16(0x0001) == 2.0 ** -24
+    del ulp
+
+
+def test_f16_atom_matches_fp64_product(oracle):
+    """AMX_F16F32 semantics: half operands multiply exactly in fp32; the oracle's fp64-accumulated sums equal a
+    numpy float64 product, the output conversion is the half rounding pinned above."""
+    rng = np.random.default_rng(4)
+    a = rng.uniform(-1, 1, (19, 65)).astype(np.float16)
+    b = rng.uniform(-1, 1, (23, 65)).astype(np.float16)
+    want = a.astype(np.float64) @ b.astype(np.float64).T
+    c = np.zeros((19, 23), np.float32)
+    oracle.matmul(a, b, c, atom=O.ATOM_F16F32, acc_f64=True)
+    assert np.array_equal(c, want.astype(np.float32))
+    ch = np.zeros((19, 23), np.float16)
+    oracle.matmul(a, b, ch, atom=O.ATOM_F16F32, acc_f64=True)
+    assert np.array_equal(ch.view(np.uint16), want.astype(np.float32).astype(np.float16).view(np.uint16))
+    # fp32 memory is rounded to half on the way in
+    a32 = rng.uniform(-1, 1, (5, 33)).astype(np.float32)
+    b32 = rng.uniform(-1, 1, (7, 33)).astype(np.float32)
+    c32 = np.zeros((5, 7), np.float32)
+    oracle.matmul(a32, b32, c32, atom=O.ATOM_F16F32, acc_f64=True)
+    want32 = a32.astype(np.float16).astype(np.float64) @ b32.astype(np.float16).astype(np.float64).T
+    assert np.array_equal(c32, want32.astype(np.float32))

@@ -131,6 +131,8 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
     pr->src = (pr->a_unsigned || pr->b_unsigned) ? SRC_I8_FLIP : SRC_I8;
   } else if (da == DT_BF16) {
     pr->src = SRC_BF16;
+  } else if (da == DT_F16) {
+    pr->src = SRC_F16;  // AMX_F16F32 / SME_F16F32 (matmul/details/kernel/amx/Atoms.h:62-71)
   } else if (da == DT_F32) {
     if (compute != VECOPS_HIP_COMPUTE_BF16 && compute != VECOPS_HIP_COMPUTE_F32)
       return fail(ST_INVALID, "matmul: unknown compute type %u", compute);
@@ -150,8 +152,9 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
     pr->out_kind = OUT_I32;
   } else {
     if (dc == DT_F32) pr->out_kind = OUT_F32;
-    else if (dc == DT_BF16) pr->out_kind = OUT_BF16;
-    else return fail(ST_NOT_APPLICABLE, "matmul: floating operands need an f32 or bf16 c");
+    else if (dc == DT_BF16 && pr->src != SRC_F16) pr->out_kind = OUT_BF16;
+    else if (dc == DT_F16 && pr->src == SRC_F16) pr->out_kind = OUT_F16;
+    else return fail(ST_NOT_APPLICABLE, "matmul: floating operands need an f32 c or one of their own 16-bit type");
   }
   // Rank 3 with one B for every batch and the rows of A and C (and C_in) running on from batch to batch:
   // the same product as [batch * M, K] x B - folded into one rank-2 problem, which fills bigger tiles
@@ -177,10 +180,12 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
       pr->cin_kind = OUT_I32;
     } else if (di == DT_F32) {
       pr->cin_kind = OUT_F32;
-    } else if (di == DT_BF16) {
+    } else if (di == DT_BF16 && pr->src != SRC_F16) {
       pr->cin_kind = OUT_BF16;
+    } else if (di == DT_F16 && pr->src == SRC_F16) {
+      pr->cin_kind = OUT_F16;
     } else {
-      return fail(ST_NOT_APPLICABLE, "matmul: c_in must be f32 or bf16");
+      return fail(ST_NOT_APPLICABLE, "matmul: c_in must be f32 or the operands' 16-bit type");
     }
   }
   return ST_OK;
@@ -412,11 +417,11 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   if (plan.vector_a && k_vector_ok(pr.b)) mode = MODE_KVEC;
   else if (plan.vector_a && plan.vector_b && plan.b_layout == 1) mode = MODE_NVEC_B;
   // 16-byte aligned bases, rows and batches: the loads may write LDS themselves
-  const int64_t elem_bytes = pr.src == SRC_BF16 ? 2 : 1;
+  const int64_t elem_bytes = (pr.src == SRC_BF16 || pr.src == SRC_F16) ? 2 : 1;
   auto lines_up = [&](const View& v, int64_t line_stride) {
     return aligned16(v.data) && (line_stride * elem_bytes) % 16 == 0 && (v.bs * elem_bytes) % 16 == 0;
   };
-  if ((pr.src == SRC_BF16 || pr.src == SRC_I8) && lines_up(pr.a, pr.a.rs)) {
+  if ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr.a, pr.a.rs)) {
     if (mode == MODE_KVEC && lines_up(pr.b, pr.b.rs)) mode = MODE_KVEC_DMA;
     else if (mode == MODE_NVEC_B && lines_up(pr.b, pr.b.cs)) mode = MODE_NVEC_B_DMA;
   }
@@ -447,6 +452,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   } else switch (pr.src) {
     case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile_m, tile_n, mode, stream); break;
     case SRC_BF16: e = launch_tile_gemm_bf16(p, tile_m, tile_n, mode, stream); break;
+    case SRC_F16: e = launch_tile_gemm_f16(p, tile_m, tile_n, mode, stream); break;
     case SRC_F32_AS_BF16: e = launch_tile_gemm_f32_as_bf16(p, tile_m, tile_n, mode, stream); break;
     case SRC_F32: e = launch_tile_gemm_f32(p, tile_m, tile_n, mode, stream); break;
     default: e = launch_tile_gemm_i8(p, tile_m, tile_n, mode, stream); break;

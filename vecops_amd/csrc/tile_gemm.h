@@ -44,8 +44,8 @@ typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
 // SRC_F32: fp32 operands multiplied in fp32 on the fp32 matrix cores
 // (v_mfma_f32_32x32x2_f32); a 16-byte chunk holds four k, a k-step (two chunks)
 // feeds four MFMAs per accumulator tile, a K tile is 32 elements.
-enum SrcKind : int { SRC_BF16 = 0, SRC_F32_AS_BF16 = 1, SRC_I8 = 2, SRC_I8_FLIP = 3, SRC_F32 = 4 };
-enum OutKind : int { OUT_F32 = 0, OUT_BF16 = 1, OUT_I32 = 2, OUT_U8 = 3, OUT_I8 = 4 };
+enum SrcKind : int { SRC_BF16 = 0, SRC_F32_AS_BF16 = 1, SRC_I8 = 2, SRC_I8_FLIP = 3, SRC_F32 = 4, SRC_F16 = 5 };
+enum OutKind : int { OUT_F32 = 0, OUT_BF16 = 1, OUT_I32 = 2, OUT_U8 = 3, OUT_I8 = 4, OUT_F16 = 5 };
 enum Activation : int { ACT_NONE = 0, ACT_RELU = 1, ACT_CLAMP = 2, ACT_SIGMOID = 3, ACT_SILU = 4 };
 // How an operand tile is fetched from global memory.
 enum LoadKind : int {
@@ -108,6 +108,8 @@ struct SrcTraits<SRC_BF16> {
   static constexpr bool kInt = false;
 };
 template <>
+struct SrcTraits<SRC_F16> : SrcTraits<SRC_BF16> {};  // IEEE half: same 16-bit chunks, its own MFMA
+template <>
 struct SrcTraits<SRC_F32_AS_BF16> {
   static constexpr int kElemsPerChunk = 8;
   static constexpr int kSrcBytes = 4;
@@ -140,6 +142,15 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// IEEE binary16 <-> fp32 with the hardware converters (to half: round to nearest even, overflow to infinity -
+// what vecops' Float16 does through F16C, util/Float16.h).
+__device__ __forceinline__ uint32_t f16_bits_rne(float x) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(x));
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
+}
 
 // LDS byte offset of 16-byte chunk `chunk` (0..7) of tile row `row`.  The chunk
 // slot is XOR-swizzled with (row ^ row/8): eight consecutive rows at one logical
@@ -240,7 +251,7 @@ __device__ __noinline__ Staged<SRC> load_chunk_checked(const void* base, int64_t
       const int k = k0 + e;
       uint32_t v = pad;
       if (row_ok && k < k_end) {
-        if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
+        if constexpr (SRC == SRC_BF16 || SRC == SRC_F16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
         else if constexpr (SRC == SRC_F32) v = __float_as_uint(static_cast<const float*>(base)[row_off + k * kstep]);
         else v = static_cast<const uint8_t*>(base)[row_off + k * kstep];
       }
@@ -287,7 +298,7 @@ __device__ __noinline__ void stage_rows_checked(const void* base, int64_t rs, in
         const int k = k0 + e;
         uint32_t v = flip & 0xffu;  // an element outside the operand: the flip byte, which the xor below turns into 0
         if (row_ok && k < k_end) {
-          if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
+          if constexpr (SRC == SRC_BF16 || SRC == SRC_F16) v = static_cast<const uint16_t*>(base)[row_off + k * kstep];
           else if constexpr (SRC == SRC_F32) v = __float_as_uint(static_cast<const float*>(base)[row_off + k * kstep]);
           else v = static_cast<const uint8_t*>(base)[row_off + k * kstep];
         }
@@ -327,6 +338,9 @@ __device__ __forceinline__ void mfma_step(typename AccTile<SrcTraits<SRC>::kInt>
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[e]), __uint_as_float(b[e]), acc, 0, 0, 0);
+  } else if constexpr (SRC == SRC_F16) {
+    typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
   } else if constexpr (SrcTraits<SRC>::kInt) {
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a), __builtin_bit_cast(i32x4, b), acc, 0, 0,
                                                 0);
@@ -374,6 +388,7 @@ __device__ __forceinline__ uint32_t narrow_to_byte(float v, bool is_signed) {
 __device__ __forceinline__ uint32_t float_output_bits(int out_kind, float v) {
   switch (out_kind) {
     case OUT_BF16: return bf16_bits_rne(v);
+    case OUT_F16: return f16_bits_rne(v);
     case OUT_U8: return narrow_to_byte(v, false);
     case OUT_I8: return narrow_to_byte(v, true);
     default: return __float_as_uint(v);
@@ -381,7 +396,7 @@ __device__ __forceinline__ uint32_t float_output_bits(int out_kind, float v) {
 }
 
 __device__ __forceinline__ int output_element_bytes(int out_kind) {
-  return out_kind == OUT_BF16 ? 2 : (out_kind == OUT_U8 || out_kind == OUT_I8) ? 1 : 4;
+  return (out_kind == OUT_BF16 || out_kind == OUT_F16) ? 2 : (out_kind == OUT_U8 || out_kind == OUT_I8) ? 1 : 4;
 }
 
 // Final value of one output element: accumulator (+ correction) (+ Cin), then
@@ -414,8 +429,9 @@ __device__ __forceinline__ uint32_t output_bits(const TileGemmParams& p, int bat
     float v = acc;
     if (p.cin) {
       const int64_t ci = batch * p.cin_bs + row * p.cin_rs + col * p.cin_cs;
-      v += (p.cin_kind == OUT_BF16) ? bf16_bits_to_f32(static_cast<const uint16_t*>(p.cin)[ci])
-                                    : static_cast<const float*>(p.cin)[ci];
+      v += (p.cin_kind == OUT_BF16)  ? bf16_bits_to_f32(static_cast<const uint16_t*>(p.cin)[ci])
+           : (p.cin_kind == OUT_F16) ? f16_bits_to_f32(static_cast<const uint16_t*>(p.cin)[ci])
+                                     : static_cast<const float*>(p.cin)[ci];
     }
     if (p.fused) v = finish_value(p, v, batch, row, col);
     return float_output_bits(p.out_kind, v);
@@ -492,15 +508,20 @@ __device__ __forceinline__ void finish_quad(const TileGemmParams& p, const Finis
   u32x4 cin = {none, none, none, none};                   // int32, or fp32 bits (bf16 widened)
   if (p.cin) {
     const int64_t ci = batch * p.cin_bs + static_cast<int64_t>(row) * p.cin_rs + col0;
-    if (p.cin_kind == OUT_BF16) {
+    if (p.cin_kind == OUT_BF16 || p.cin_kind == OUT_F16) {
       const uint16_t* src = static_cast<const uint16_t*>(p.cin) + ci;
+      uint32_t h[4] = {0u, 0u, 0u, 0u};  // the four 16-bit patterns
       if (cols_left >= 4) {
-        const u32x2_align2 h = *reinterpret_cast<const u32x2_align2*>(src);
-        cin = u32x4{h.x << 16, h.x & 0xffff0000u, h.y << 16, h.y & 0xffff0000u};
+        const u32x2_align2 pair = *reinterpret_cast<const u32x2_align2*>(src);
+        h[0] = pair.x & 0xffffu; h[1] = pair.x >> 16; h[2] = pair.y & 0xffffu; h[3] = pair.y >> 16;
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (e < cols_left) cin[e] = static_cast<uint32_t>(src[e]) << 16;
+          if (e < cols_left) h[e] = src[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (e < cols_left) cin[e] = p.cin_kind == OUT_BF16 ? (h[e] << 16) : __float_as_uint(f16_bits_to_f32(h[e]));
       }
     } else {
       const uint32_t* src = static_cast<const uint32_t*>(p.cin) + ci;
@@ -547,6 +568,10 @@ __device__ __forceinline__ void finish_quad(const TileGemmParams& p, const Finis
     case OUT_BF16:
 #pragma unroll
       for (int e = 0; e < 4; ++e) bits[e] = bf16_bits_rne(f[e]);
+      break;
+    case OUT_F16:
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bits[e] = f16_bits_rne(f[e]);
       break;
     case OUT_U8:
 #pragma unroll
@@ -842,7 +867,7 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int k = kt * 64 + k_row(i, tid_);
-      if constexpr (SRC == SRC_BF16) {
+      if constexpr (SRC == SRC_BF16 || SRC == SRC_F16) {
         uint32_t w[4] = {0u, 0u, 0u, 0u};
         if (k < k_end) {
 #pragma unroll
@@ -951,7 +976,7 @@ __device__ __forceinline__ void load_16_bytes_into_lds_counted(__amdgpu_buffer_r
 template <int SRC, int ROWS, int THREADS>
 struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
   using T = SrcTraits<SRC>;
-  static_assert(SRC == SRC_BF16 || SRC == SRC_I8, "operands that go into LDS as they are");
+  static_assert(SRC == SRC_BF16 || SRC == SRC_F16 || SRC == SRC_I8, "operands that go into LDS as they are");
   static constexpr int ROWS_PER_PASS = THREADS / 8;
   static constexpr int CHUNKS = ROWS / ROWS_PER_PASS;
   static_assert(CHUNKS >= 1, "tile too small for this many threads");
@@ -1018,7 +1043,7 @@ struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
 template <int SRC, int ROWS, int THREADS>
 struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
   using T = SrcTraits<SRC>;
-  static_assert(SRC == SRC_BF16, "operands that go into LDS as they are");
+  static_assert(SRC == SRC_BF16 || SRC == SRC_F16, "operands that go into LDS as they are");
   static constexpr int kPitch = ROWS * 2;
   static constexpr int CHUNKS_PER_ROW = ROWS / 8;
   static_assert(CHUNKS_PER_ROW >= 16, "the swizzle needs sixteen chunk slots per row");

@@ -21,6 +21,7 @@ enum LoadMode : int {
 // tile_m x tile_n: 256x256, 256x128, 128x256, 128x128 or 64x64 (the workgroup tile).  Returns the HIP
 // error of the launch (hipSuccess when enqueued).
 hipError_t launch_tile_gemm_bf16(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
+hipError_t launch_tile_gemm_f16(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_f32_as_bf16(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_f32(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);  // fp32 compute
 hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
@@ -62,9 +63,9 @@ hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN>
 hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t stream) {
   // loads into LDS: bf16 and int8 operands on the tiles of 128 or more columns
-  if constexpr ((SRC == SRC_BF16 || SRC == SRC_I8) && WAVES_N * WN * 32 >= 128) {
+  if constexpr ((SRC == SRC_BF16 || SRC == SRC_F16 || SRC == SRC_I8) && WAVES_N * WN * 32 >= 128) {
     if (mode == MODE_KVEC_DMA) return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KDMA, LOAD_KDMA>(p, stream);
-    if constexpr (SRC == SRC_BF16) {
+    if constexpr (SRC == SRC_BF16 || SRC == SRC_F16) {
       if (mode == MODE_NVEC_B_DMA)
         return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KDMA, LOAD_NTR_DMA>(p, stream);
     }

@@ -2,8 +2,8 @@
 // DSO per (operator, operand class, memory placement); the build compiles this
 // file once per artifact with
 //   -DVECOPS_ARTIFACT_KIND=<0..8>   0 matmul bf16, 1 matmul f32 (bf16 compute), 5 matmul f32 (fp32 compute), 2 matmul i8,
-//                                   3 matmul_i8_dequant, 4 matmul_w8a16_group, 6 / 7 / 8 matmul_fused for bf16 / f32 /
-//                                   i8 operands
+//                                   3 matmul_i8_dequant, 4 matmul_w8a16_group, 6 / 7 / 8 / 10 matmul_fused for bf16 /
+//                                   f32 / i8 / f16 operands, 9 matmul f16
 //   -DVECOPS_ARTIFACT_DEVICE=<0|1>  0: tensors are host memory, staged through HBM here
 //                                   1: tensors are HIP device pointers, used in place
 //   -DVECOPS_ARTIFACT_GROUP=<G>     group size of kind 4
@@ -226,7 +226,7 @@ int32_t check_call(const VecopsCall* call, uint32_t expected, VecopsError* error
 }
 
 // =================================================================================================
-#if VECOPS_ARTIFACT_KIND <= 2 || VECOPS_ARTIFACT_KIND == 5  // vecops::matmul (a, b, c_in?, c)
+#if VECOPS_ARTIFACT_KIND <= 2 || VECOPS_ARTIFACT_KIND == 5 || VECOPS_ARTIFACT_KIND == 9  // vecops::matmul (a, b, c_in?, c)
 // =================================================================================================
 
 #if VECOPS_ARTIFACT_KIND == 0
@@ -234,6 +234,11 @@ int32_t check_call(const VecopsCall* call, uint32_t expected, VecopsError* error
 #define COMPUTE "bf16"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16);
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
+#elif VECOPS_ARTIFACT_KIND == 9
+#define OPERANDS "f16"
+#define COMPUTE "f16"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F16);
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_F16);
 #elif VECOPS_ARTIFACT_KIND == 1
 #define OPERANDS "f32"
 #define COMPUTE "bf16"
@@ -433,7 +438,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
 }
 
 // =================================================================================================
-#elif VECOPS_ARTIFACT_KIND >= 6  // vecops::matmul_fused (a, b, c_in?, row_scales?, column_scales?, 5 scalars, c)
+#elif VECOPS_ARTIFACT_KIND >= 6 && VECOPS_ARTIFACT_KIND != 9  // vecops::matmul_fused (a, b, c_in?, row_scales?, column_scales?, 5 scalars, c)
 // =================================================================================================
 
 #if VECOPS_ARTIFACT_KIND == 6
@@ -442,6 +447,9 @@ constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16);
 #elif VECOPS_ARTIFACT_KIND == 7
 #define OPERANDS "f32"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
+#elif VECOPS_ARTIFACT_KIND == 10
+#define OPERANDS "f16"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F16);
 #else
 #define OPERANDS "i8"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);
@@ -449,6 +457,9 @@ constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);
 #if VECOPS_ARTIFACT_KIND == 8
 constexpr uint64_t kCinMask = bit(VECOPS_DTYPE_I32);
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_U8) | bit(VECOPS_DTYPE_I8);
+#elif VECOPS_ARTIFACT_KIND == 10
+constexpr uint64_t kCinMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_F16);
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_F16);
 #else
 constexpr uint64_t kCinMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);

@@ -154,9 +154,10 @@ std::shared_ptr<rt::Operator> assemble(rt::OperatorSchema schema,
 
 rt::OperatorSchema make_matmul_schema() {
   using rt::dtype_bit;
-  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8) |
-                           dtype_bit(DType::UInt8);
-  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int32);
+  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                           dtype_bit(DType::Int8) | dtype_bit(DType::UInt8);
+  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                            dtype_bit(DType::Int32);
   std::vector<rt::ParameterSchema> params;
   params.push_back(tensor_param("a", in, std::nullopt, VECOPS_TENSOR_READ));
   params.push_back(tensor_param("b", in, std::nullopt, VECOPS_TENSOR_READ));
@@ -179,11 +180,12 @@ rt::OperatorSchema make_matmul_i8_dequant_schema() {
 
 rt::OperatorSchema make_matmul_fused_schema() {
   using rt::dtype_bit;
-  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8) |
-                           dtype_bit(DType::UInt8);
-  const std::uint64_t cin = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int32);
-  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::UInt8) |
-                            dtype_bit(DType::Int8);
+  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                           dtype_bit(DType::Int8) | dtype_bit(DType::UInt8);
+  const std::uint64_t cin = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                            dtype_bit(DType::Int32);
+  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                            dtype_bit(DType::UInt8) | dtype_bit(DType::Int8);
   const std::uint64_t real = dtype_bit(DType::Float32) | dtype_bit(DType::Float64);
   std::vector<rt::ParameterSchema> params;
   params.push_back(tensor_param("a", in, std::nullopt, VECOPS_TENSOR_READ));
@@ -215,6 +217,7 @@ rt::OperatorSchema make_matmul_w8a16_group_schema() {
 static bool takes(OperandClass operands, DType dtype) {
   switch (operands) {
     case OperandClass::BF16: return dtype == DType::BFloat16;
+    case OperandClass::F16: return dtype == DType::Float16;
     case OperandClass::F32: return dtype == DType::Float32;
     default: return dtype == DType::Int8 || dtype == DType::UInt8;
   }
@@ -222,6 +225,7 @@ static bool takes(OperandClass operands, DType dtype) {
 
 MatmulRecipe::MatmulRecipe(OperandClass operands) : operands_(operands) {
   id_ = operands == OperandClass::BF16 ? "hip.matmul.bf16.tile"
+        : operands == OperandClass::F16 ? "hip.matmul.f16.tile"
         : operands == OperandClass::F32 ? "hip.matmul.f32.tile"
                                         : "hip.matmul.i8.tile";
 }
@@ -236,10 +240,11 @@ Status MatmulRecipe::match(const rt::KernelCall& call) const {
   if (!takes(operands_, a->dtype) || !takes(operands_, b->dtype))
     return not_applicable("operand dtypes belong to another recipe");
   const bool int_out = operands_ == OperandClass::I8;
-  if (int_out ? c->dtype != DType::Int32 : (c->dtype != DType::Float32 && c->dtype != DType::BFloat16))
+  // floating sums leave as fp32 or in the operands' own 16-bit type (fp32 operands: bf16)
+  const DType narrow = operands_ == OperandClass::F16 ? DType::Float16 : DType::BFloat16;
+  if (int_out ? c->dtype != DType::Int32 : (c->dtype != DType::Float32 && c->dtype != narrow))
     return not_applicable("output dtype does not fit these operands");
-  if (cin != nullptr &&
-      (int_out ? cin->dtype != DType::Int32 : (cin->dtype != DType::Float32 && cin->dtype != DType::BFloat16)))
+  if (cin != nullptr && (int_out ? cin->dtype != DType::Int32 : (cin->dtype != DType::Float32 && cin->dtype != narrow)))
     return not_applicable("c_in dtype does not fit these operands");
   auto compute = compute_type(call);
   if (!compute) return compute.status();
@@ -250,6 +255,8 @@ Status MatmulRecipe::match(const rt::KernelCall& call) const {
       return not_applicable("ComputeType must be BFloat16 or Float32 for fp32 operands");
   } else if (operands_ == OperandClass::BF16 && compute.value() != DType::BFloat16) {
     return not_applicable("bf16 operands are multiplied in bf16");
+  } else if (operands_ == OperandClass::F16 && compute.value() != DType::BFloat16 && compute.value() != DType::Float16) {
+    return not_applicable("half operands are multiplied in half");  // (BFloat16 is the default of an absent ComputeType)
   }
   auto place = placement_of(call);
   if (!place) return place.status();
@@ -259,9 +266,11 @@ Status MatmulRecipe::match(const rt::KernelCall& call) const {
 rt::Result<rt::BoundKernelRecipe> MatmulRecipe::bind(const rt::KernelCall& call) const {
   if (Status st = match(call); !st.ok()) return st;
   const Placement place = placement_of(call).value();
-  const char* operands = operands_ == OperandClass::BF16 ? "bf16" : operands_ == OperandClass::F32 ? "f32" : "i8";
+  const char* operands = operands_ == OperandClass::BF16 ? "bf16" : operands_ == OperandClass::F16 ? "f16"
+                         : operands_ == OperandClass::F32 ? "f32" : "i8";
   const bool f32_compute = operands_ == OperandClass::F32 && compute_type(call).value() == DType::Float32;
-  const char* compute = operands_ == OperandClass::I8 ? "i32" : f32_compute ? "f32" : "bf16";
+  const char* compute = operands_ == OperandClass::I8 ? "i32" : operands_ == OperandClass::F16 ? "f16"
+                        : f32_compute ? "f32" : "bf16";
   rt::BoundKernelRecipe bound;
   bound.recipe_id = id_;
   bound.specialization_key = std::string(kMatmulName) + ";operands=" + operands + ";compute=" + compute +
@@ -295,6 +304,7 @@ rt::Result<rt::BoundKernelRecipe> MatmulI8DequantRecipe::bind(const rt::KernelCa
 
 MatmulFusedRecipe::MatmulFusedRecipe(OperandClass operands) : operands_(operands) {
   id_ = operands == OperandClass::BF16 ? "hip.matmul_fused.bf16.tile"
+        : operands == OperandClass::F16 ? "hip.matmul_fused.f16.tile"
         : operands == OperandClass::F32 ? "hip.matmul_fused.f32.tile"
                                         : "hip.matmul_fused.i8.tile";
 }
@@ -310,11 +320,11 @@ Status MatmulFusedRecipe::match(const rt::KernelCall& call) const {
     return not_applicable("operand dtypes belong to another recipe");
   // int32 sums leave as fp32 or as requantised bytes; floating sums as fp32 or bf16
   const bool integer = operands_ == OperandClass::I8;
+  const DType narrow = operands_ == OperandClass::F16 ? DType::Float16 : DType::BFloat16;
   const bool out_ok = integer ? (c->dtype == DType::Float32 || c->dtype == DType::UInt8 || c->dtype == DType::Int8)
-                              : (c->dtype == DType::Float32 || c->dtype == DType::BFloat16);
+                              : (c->dtype == DType::Float32 || c->dtype == narrow);
   if (!out_ok) return not_applicable("output dtype does not fit these operands");
-  if (cin != nullptr &&
-      (integer ? cin->dtype != DType::Int32 : (cin->dtype != DType::Float32 && cin->dtype != DType::BFloat16)))
+  if (cin != nullptr && (integer ? cin->dtype != DType::Int32 : (cin->dtype != DType::Float32 && cin->dtype != narrow)))
     return not_applicable("c_in dtype does not fit these operands");
   auto place = placement_of(call);
   if (!place) return place.status();
@@ -323,7 +333,8 @@ Status MatmulFusedRecipe::match(const rt::KernelCall& call) const {
 
 rt::Result<rt::BoundKernelRecipe> MatmulFusedRecipe::bind(const rt::KernelCall& call) const {
   if (Status st = match(call); !st.ok()) return st;
-  const char* operands = operands_ == OperandClass::BF16 ? "bf16" : operands_ == OperandClass::F32 ? "f32" : "i8";
+  const char* operands = operands_ == OperandClass::BF16 ? "bf16" : operands_ == OperandClass::F16 ? "f16"
+                         : operands_ == OperandClass::F32 ? "f32" : "i8";
   rt::BoundKernelRecipe bound;
   bound.recipe_id = id_;
   bound.specialization_key = std::string(kMatmulFusedName) + ";operands=" + operands + ";memory=" +
@@ -457,8 +468,8 @@ rt::Result<std::shared_ptr<rt::Executable>> HipExecutableProvider::resolve(const
 
 std::shared_ptr<rt::Operator> make_matmul_operator(const std::filesystem::path& dir) {
   return assemble(make_matmul_schema(),
-                  {std::make_shared<MatmulRecipe>(OperandClass::BF16), std::make_shared<MatmulRecipe>(OperandClass::F32),
-                   std::make_shared<MatmulRecipe>(OperandClass::I8)},
+                  {std::make_shared<MatmulRecipe>(OperandClass::BF16), std::make_shared<MatmulRecipe>(OperandClass::F16),
+                   std::make_shared<MatmulRecipe>(OperandClass::F32), std::make_shared<MatmulRecipe>(OperandClass::I8)},
                   dir);
 }
 
@@ -469,6 +480,7 @@ std::shared_ptr<rt::Operator> make_matmul_i8_dequant_operator(const std::filesys
 std::shared_ptr<rt::Operator> make_matmul_fused_operator(const std::filesystem::path& dir) {
   return assemble(make_matmul_fused_schema(),
                   {std::make_shared<MatmulFusedRecipe>(OperandClass::BF16),
+                   std::make_shared<MatmulFusedRecipe>(OperandClass::F16),
                    std::make_shared<MatmulFusedRecipe>(OperandClass::F32),
                    std::make_shared<MatmulFusedRecipe>(OperandClass::I8)},
                   dir);

@@ -54,7 +54,7 @@ rt::OperatorSchema make_matmul_w8a16_group_schema();
 rt::OperatorSchema make_matmul_fused_schema();
 
 // Operand classes of vecops::matmul, one artifact each.
-enum class OperandClass { BF16, F32, I8 };
+enum class OperandClass { BF16, F32, I8, F16 };
 
 // Kernel families a recipe stands for: the MFMA workgroup-tile kernels or the
 // wavefront split-K dot-product kernels for skinny shapes.
@@ -67,7 +67,7 @@ enum class Placement { Host, Device };
 
 // Recipe of vecops::matmul for one operand class.  match() is metadata-only:
 // dtype class, ComputeType, uniform placement.  bind() yields
-//   vecops::matmul;operands=<bf16|f32|i8>;compute=<bf16|f32|i32>;memory=<host|device>;backend=hip-gfx950
+//   vecops::matmul;operands=<bf16|f16|f32|i8>;compute=<bf16|f16|f32|i32>;memory=<host|device>;backend=hip-gfx950
 class MatmulRecipe final : public rt::KernelRecipe {
 public:
   explicit MatmulRecipe(OperandClass operands);
@@ -90,7 +90,7 @@ public:
 };
 
 // vecops::matmul_fused for one operand class (fp32 operands multiply in bf16):
-//   vecops::matmul_fused;operands=<bf16|f32|i8>;memory=<host|device>;backend=hip-gfx950
+//   vecops::matmul_fused;operands=<bf16|f16|f32|i8>;memory=<host|device>;backend=hip-gfx950
 class MatmulFusedRecipe final : public rt::KernelRecipe {
 public:
   explicit MatmulFusedRecipe(OperandClass operands);

@@ -56,7 +56,8 @@ class Specialization(C.Structure):
 # layout facts of vecops' runtime/CallAbi.h on LP64, checked by tests/test_host_cpu.py
 ABI_SIZES = {"VecopsTensorView": 64, "VecopsScalar": 16, "VecopsValue": 72, "VecopsExecutionContext": 56}
 
-_NP_CODES = {np.dtype(np.int8): I8, np.dtype(np.uint8): U8, np.dtype(np.int32): I32, np.dtype(np.float32): F32}
+_NP_CODES = {np.dtype(np.int8): I8, np.dtype(np.uint8): U8, np.dtype(np.int32): I32, np.dtype(np.float32): F32,
+             np.dtype(np.float16): F16}
 
 
 class Frame:
