@@ -106,7 +106,7 @@ def bench_int8_dequant(dev, steps, warmup):
             "dequant fused, fp32 out", "value": tops, "unit": "TOP/s", "ms_per_step": wall_ms, "dtype": "int8",
             "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                          "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT,
-                         "kernel": "vecops_hip::tile_gemm_kernel<int8, 256x128x128, loads into LDS, dequant epilogue>",
+                         "kernel": "vecops_hip::tile_gemm_kernel<int8, 256x256x128, loads into LDS, dequant epilogue>",
                          "algorithmic_ops_per_launch": ops,
                          "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
 
@@ -152,7 +152,7 @@ def bench_int8_dequant_packed(dev, steps, warmup):
             "ms_per_step": wall_ms, "dtype": "int8",
             "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                          "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT_PACKED,
-                         "kernel": "vecops_hip::tile_gemm_packed_b_kernel<int8, 256x128x128, dequant epilogue>",
+                         "kernel": "vecops_hip::tile_gemm_packed_b_kernel<int8, 256x256x128, dequant epilogue>",
                          "algorithmic_ops_per_launch": ops,
                          "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
 

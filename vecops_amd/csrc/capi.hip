@@ -193,7 +193,10 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
 
 constexpr int kComputeUnits = 256;
 constexpr int kStreamGroupsPerUnit = 2;  // workgroups of 4 wavefronts per compute unit of the streaming GEMV
-constexpr int64_t kQuality256x128 = 880, kQuality128 = 770;  // see choose()
+// Work per compute unit and second of the smaller tiles relative to 256x256, per mille (see choose()): bf16 4096^3
+// forced onto each tile takes 132 / 167 / 162 / 159 us (256x256, 256x128, 128x256, 128x128; two or three 128x128
+// workgroups share a compute unit).
+constexpr int64_t kQuality256x128 = 800, kQuality128 = 820;
 
 // bf16 x bf16 or int8 x int8 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
 bool skinny_applies(const Problem& pr) {
@@ -246,8 +249,10 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
   // (per mille; measured on bf16 problems that fill exactly one round).  A candidate must keep at least
   // half the compute units busy; among those the cheapest wins, cost = rounds x tile area / quality -
   // so a part-filled last round, rows or columns of padding and a less efficient small tile are all
-  // priced in one number (4096^3: 256 tiles of 256x256, one round; 2048x11008: 688 tiles of 256x128 in
-  // three rounds instead of 344 big ones in two; 8 x 777x1000: 256 tiles of 256x128, one round).
+  // priced in one number (4096^3: 256 tiles of 256x256, one round; 2048x11008: 344 of them in two rounds, which
+  // 688 tiles of 256x128 in three or 1376 of 128x128 in six undercut by less than the margin below - measured
+  // 134 / 141 / 134 us; 4096x4224: 1056 tiles of 128x128, 174 us against 187 for 272 big ones whose second round
+  // is 6 % full; 8 x 777x1000: 256 tiles of 256x128, one round).
   struct Candidate { uint32_t family; int64_t tm, tn, quality; };
   const Candidate candidates[] = {{VECOPS_HIP_FAMILY_TILE_256, 256, 256, 1000},
                                   {VECOPS_HIP_FAMILY_TILE_256X128, 256, 128, kQuality256x128},
