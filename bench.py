@@ -31,11 +31,11 @@ PEAK_HBM_GBPS = 8000.0
 # profiles/ (KiB per dispatch x 1024, FETCH scaled by 2.000 and WRITE by 1.000: what the
 # same counters read for a 1 GiB device copy, `--only copy`).  Counters cannot be read
 # from inside this process, so these are the recorded figures for exactly these workloads.
-TRAFFIC_BF16_4096 = int((98487.5 * 2.000 + 32768 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT = int((127024 * 2.000 + 88064 * 1.000) * 1024)
+TRAFFIC_BF16_4096 = int((98479.5 * 2.000 + 32768 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT = int((95283.3 * 2.000 + 88064 * 1.000) * 1024)
 TRAFFIC_GEMV_M1 = int((29647.4 * 2.000 + 112.0 * 1.000) * 1024)
-TRAFFIC_BF16_4096_PACKED = int((98477.8 * 2.000 + 32768 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT_PACKED = int((125258 * 2.000 + 88064 * 1.000) * 1024)
+TRAFFIC_BF16_4096_PACKED = int((98468.3 * 2.000 + 32768 * 1.000) * 1024)
+TRAFFIC_INT8_DEQUANT_PACKED = int((95160.6 * 2.000 + 88064 * 1.000) * 1024)
 
 
 def _device_tensors_bf16_gemm(dev):
