@@ -96,7 +96,7 @@ def test_abi_layout(tmp_path):
 
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
-    assert len(files) == 24
+    assert len(files) == 34
     for f in files:
         name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
         assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
@@ -224,6 +224,50 @@ def test_fused_operator_resolution_and_validation(host):
     with pytest.raises(H.HostError) as e:                  # bf16 sums cannot leave as bytes
         op.resolve(frame(bf16((4, 8)), bf16((5, 8)), None, None, None, np.zeros((4, 5), np.uint8)))
     assert e.value.code in (2, 3)
+
+
+def test_packed_b_operators_resolution_and_validation(host):
+    """vecops::matmul_pack_b / vecops::matmul_packed_b: the packed operand is an opaque byte tensor; the pack's
+    class follows the source dtype, the multiply's class follows a."""
+    pack = host.operator("vecops::matmul_pack_b")
+    packed = np.zeros(4096, np.uint8)
+    comp = np.zeros(5, np.int32)
+    pf = lambda b, zp, p, c: H.Frame([b, zp, p, c], outputs=(2, 3))  # noqa: E731
+    assert pack.resolve(pf(bf16((5, 8)), 0, packed, None)) == \
+        "vecops::matmul_pack_b;operands=bf16;memory=host;backend=hip-gfx950"
+    assert "operands=bf16" in pack.resolve(pf(np.zeros((5, 8), np.float32), 0, packed, None))   # rounded while packing
+    assert pack.resolve(pf(np.zeros((5, 8), np.int8), 3, packed, comp)) == \
+        "vecops::matmul_pack_b;operands=i8;memory=host;backend=hip-gfx950"
+    for fr, needle in [(pf(bf16((5, 8)), 0, packed, comp), "int8"),
+                       (pf(np.zeros((5, 8), np.int8), 3, packed, np.zeros(4, np.int32)), "N entries"),
+                       (pf(np.zeros((5, 8), np.int8), 1.5, packed, None), "a_zero_point")]:
+        with pytest.raises(H.HostError) as e:
+            pack.resolve(fr)
+        assert e.value.code == 1 and needle in e.value.message, (needle, e.value.message)
+    with pytest.raises(H.HostError) as e:                  # half operands have no packed form
+        pack.resolve(pf(np.zeros((5, 8), np.float16), 0, packed, None))
+    assert e.value.code in (1, 2, 3)
+
+    mul = host.operator("vecops::matmul_packed_b")
+    mf = lambda a, cin, c: H.Frame([a, packed, cin, c], outputs=(3,))  # noqa: E731
+    c = np.zeros((4, 5), np.float32)
+    assert mul.resolve(mf(bf16((4, 8)), None, c)) == "vecops::matmul_packed_b;operands=bf16;memory=host;backend=hip-gfx950"
+    assert "operands=bf16" in mul.resolve(mf(bf16((2, 4, 8)), None, bf16((2, 4, 5))))
+    assert "operands=f32" in mul.resolve(mf(np.zeros((4, 8), np.float32), c, c))
+    assert "operands=i8" in mul.resolve(mf(np.zeros((4, 8), np.int8), None, np.zeros((4, 5), np.int32)))
+    for fr, needle in [(mf(bf16((4, 8)), None, np.zeros((3, 5), np.float32)), "[.., M, N]"),
+                       (mf(bf16((2, 4, 8)), None, np.zeros((3, 4, 5), np.float32)), "batch"),
+                       (mf(bf16((4, 8)), np.zeros((4, 6), np.float32), c), "c_in")]:
+        with pytest.raises(H.HostError) as e:
+            mul.resolve(fr)
+        assert e.value.code == 1 and needle in e.value.message, (needle, e.value.message)
+    with pytest.raises(H.HostError) as e:                  # int32 sums do not leave as fp32 here
+        mul.resolve(mf(np.zeros((4, 8), np.int8), None, c))
+    assert e.value.code in (2, 3)
+    # a packed tensor that is too small for N x K is refused by the artifact's workspace query
+    with pytest.raises(H.HostError) as e:
+        mul.workspace(H.Frame([bf16((4, 8)), np.zeros(16, np.uint8), None, c], outputs=(3,)))
+    assert e.value.code == 1 and "bytes" in e.value.message
 
 
 def test_provider_without_artifacts_reports_not_found(host, tmp_path):

@@ -200,6 +200,65 @@ def test_matmul_fused_operator(host, oracle, device):
     assert rel_err(synth.bf16_to_f32(got16), synth.bf16_to_f32(want16)) <= 2 ** -7
 
 
+def test_packed_b_operators(host, oracle, device):
+    """vecops::matmul_pack_b then vecops::matmul_packed_b through the Operator: results equal vecops::matmul's on
+    the unpacked operand bit for bit (host tensors staged, device tensors in place), the compensation row equals
+    -zp * sum_k b[n,k], and one packed operand serves every batch of a rank-3 a."""
+    import torch
+    from vecops_amd import capi
+    pack, mul, plain = (host.operator("vecops::matmul_pack_b"), host.operator("vecops::matmul_packed_b"),
+                        host.operator("vecops::matmul"))
+    # int8, host tensors, compensated pack
+    m, n, k = 67, 129, 515
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    size = capi.lib().vecops_hip_packed_b_bytes(capi.I8, n, k)
+    packed, comp = np.zeros(size, np.uint8), np.zeros(n, np.int32)
+    frame = H.Frame([b, 7, packed, comp], outputs=(2, 3))
+    assert pack.resolve(frame) == "vecops::matmul_pack_b;operands=i8;memory=host;backend=hip-gfx950"
+    pack.invoke(frame)
+    assert np.array_equal(comp, (-7 * b.astype(np.int64).sum(axis=1)).astype(np.int32))
+    want = np.zeros((m, n), np.int32)
+    oracle.matmul(a, b, want, atom=O.ATOM_I8I32, acc_f64=True, c_bf16=False)
+    c = np.full((m, n), -1, np.int32)
+    mul.invoke(H.Frame([a, packed, None, c], outputs=(3,)))
+    assert np.array_equal(c, want)
+    corr = np.broadcast_to(comp, (m, n))                                      # the sidecar as a stride-0 C-input row
+    mul.invoke(H.Frame([a, packed, corr, c], outputs=(3,)))
+    assert np.array_equal(c, want + comp[None, :])
+    # bf16 from an fp32 source, device tensors, rank-3 a with a workspace when the plan asks for one
+    batch, m, n, k = 3, 50, 200, 1000
+    a = synth.bf16_round(synth.uniform_pm1(1, (batch, m, k)))
+    bf = synth.uniform_pm1(2, (n, k))
+    ta = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+    tbf = torch.from_numpy(bf).to(device)
+    tb = torch.from_numpy(synth.bf16_round(bf).view(np.int16)).to(device).view(torch.bfloat16)
+    tp = torch.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.BF16, n, k), dtype=torch.uint8, device=device)
+    frame = H.Frame([tbf, 0, tp, None], outputs=(2,))
+    assert pack.resolve(frame) == "vecops::matmul_pack_b;operands=bf16;memory=device;backend=hip-gfx950"
+    pack.invoke(frame)
+    tc = torch.full((batch, m, n), float("nan"), device=device)
+    frame = H.Frame([ta, tp, None, tc], outputs=(3,))
+    need = mul.workspace(frame)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    mul.invoke(frame, workspace=ws.data_ptr(), workspace_size=need)
+    tref = torch.full((batch, m, n), float("nan"), device=device)
+    frame = H.Frame([ta, tb.unsqueeze(0).expand(batch, n, k), None, tref], outputs=(3,))
+    need = plain.workspace(frame)
+    ws2 = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    plain.invoke(frame, workspace=ws2.data_ptr(), workspace_size=need)
+    torch.cuda.synchronize()
+    got = tc.cpu().numpy()
+    wantf = np.zeros((batch, m, n), np.float32)
+    for i in range(batch):
+        oracle.matmul(a[i], synth.bf16_round(bf), wantf[i], acc_f64=True, c_bf16=False)
+    assert rel_err(got, wantf) <= fp32_tol(k)
+    assert rel_err(got, tref.cpu().numpy()) <= fp32_tol(k)
+    # a packed tensor of the wrong size is an invalid argument, not a fault
+    with pytest.raises(H.HostError) as e:
+        mul.invoke(H.Frame([ta, tp[:64], None, tc], outputs=(3,)))
+    assert e.value.code == 1
+
+
 def test_matmul_w8a16_group_operator(host, oracle, device):
     import torch
     op = host.operator("vecops::matmul_w8a16_group")

@@ -5,6 +5,7 @@ import numpy as np
 import pytest
 import torch
 
+from vecops_amd import capi
 from vecops_amd import host_api as H
 from vecops_amd import synth
 from vecops_amd import torch_bridge as tb
@@ -30,7 +31,10 @@ def test_registration_is_idempotent_and_schemas_mark_outputs():
     with pytest.raises(AttributeError):
         tb.no_such_library
     ns = tb.register_all("vecops_hip_t")
-    assert sorted(vars(ns)) == ["matmul", "matmul_fused", "matmul_i8_dequant", "matmul_w8a16_group"]
+    assert sorted(vars(ns)) == ["matmul", "matmul_fused", "matmul_i8_dequant", "matmul_pack_b", "matmul_packed_b",
+                                "matmul_w8a16_group"]
+    pack = str(torch.ops.vecops_hip_t.matmul_pack_b.default._schema)
+    assert "int a_zero_point" in pack and "Tensor(a!) packed" in pack and "Tensor(b!)? compensation" in pack
     schema = str(torch.ops.vecops_hip_t.matmul.default._schema)
     assert "Tensor? c_in" in schema and "Tensor(a!) c" in schema and "int ComputeType=-1" in schema
     assert "-> ()" in schema
@@ -136,6 +140,33 @@ def test_torch_ops_quantised_operators(device, oracle):
     bits, exact = oracle.matmul_w8a16_group(x, w, s, 64)
     got = synth.bf16_to_f32(yb.view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
     assert np.abs(got - exact).max() <= 2 ** -7 * np.abs(exact).max()
+
+
+@pytest.mark.gpu
+def test_torch_ops_packed_b(device):
+    """Pack once through torch.ops, multiply twice: bit-equal to vecops::matmul on the unpacked operand."""
+    ns = tb.register_all("vecops_hip_t")
+    to = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(device)  # noqa: E731
+    m, n, k = 70, 300, 520
+    a, b = to(synth.int8_sym(1, (m, k))), to(synth.int8_sym(2, (n, k)))
+    packed = torch.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.I8, n, k), dtype=torch.uint8, device=device)
+    comp = torch.zeros(n, dtype=torch.int32, device=device)
+    outs = ns.matmul_pack_b(b, -3, packed, comp)
+    assert outs[0] is packed and outs[1] is comp
+    assert torch.equal(comp, (3 * b.to(torch.int64).sum(dim=1)).to(torch.int32))
+    assert ns.matmul_pack_b(b, 0, packed, None) is packed                       # without the sidecar
+    c, want = (torch.zeros(m, n, dtype=torch.int32, device=device) for _ in range(2))
+    ns.matmul_packed_b(a, packed, None, c)
+    ns.matmul(a, b, None, want)
+    assert torch.equal(c, want)
+    af, bf = _bf16(synth.uniform_pm1(3, (m, k)), device), _bf16(synth.uniform_pm1(4, (n, k)), device)
+    pf = torch.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.BF16, n, k), dtype=torch.uint8, device=device)
+    ns.matmul_pack_b(bf, 0, pf, None)
+    cin = torch.from_numpy(synth.uniform_pm1(5, (m, n))).to(device)
+    c1, c2 = torch.zeros(m, n, device=device), torch.zeros(m, n, device=device)
+    ns.matmul_packed_b(af, pf, cin, c1)
+    ns.matmul(af, bf, cin, c2)
+    assert torch.equal(c1, c2)
 
 
 @pytest.mark.gpu

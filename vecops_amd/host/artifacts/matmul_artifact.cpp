@@ -3,7 +3,8 @@
 // file once per artifact with
 //   -DVECOPS_ARTIFACT_KIND=<0..8>   0 matmul bf16, 1 matmul f32 (bf16 compute), 5 matmul f32 (fp32 compute), 2 matmul i8,
 //                                   3 matmul_i8_dequant, 4 matmul_w8a16_group, 6 / 7 / 8 / 10 matmul_fused for bf16 /
-//                                   f32 / i8 / f16 operands, 9 matmul f16
+//                                   f32 / i8 / f16 operands, 9 matmul f16, 11 / 12 matmul_pack_b to bf16 / i8,
+//                                   13 / 14 / 15 matmul_packed_b for bf16 / f32 / i8 a
 //   -DVECOPS_ARTIFACT_DEVICE=<0|1>  0: tensors are host memory, staged through HBM here
 //                                   1: tensors are HIP device pointers, used in place
 //   -DVECOPS_ARTIFACT_GROUP=<G>     group size of kind 4
@@ -438,7 +439,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
 }
 
 // =================================================================================================
-#elif VECOPS_ARTIFACT_KIND >= 6 && VECOPS_ARTIFACT_KIND != 9  // vecops::matmul_fused (a, b, c_in?, row_scales?, column_scales?, 5 scalars, c)
+#elif VECOPS_ARTIFACT_KIND >= 6 && VECOPS_ARTIFACT_KIND != 9 && VECOPS_ARTIFACT_KIND < 11  // vecops::matmul_fused (a, b, c_in?, row_scales?, column_scales?, 5 scalars, c)
 // =================================================================================================
 
 #if VECOPS_ARTIFACT_KIND == 6
@@ -611,6 +612,192 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
 #endif
   int32_t rc = vecops_hip_matmul_fused(&f.ops[0], &f.ops[1], f.cin ? &f.ops[2] : nullptr, &f.ops[3],
                                        VECOPS_HIP_COMPUTE_BF16, &f.ep, ws, ws_size, stream);
+  if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
+  return finish(&staging, stream, error);
+}
+
+// =================================================================================================
+#elif VECOPS_ARTIFACT_KIND == 11 || VECOPS_ARTIFACT_KIND == 12  // vecops::matmul_pack_b (b, a_zero_point, packed, compensation?)
+// =================================================================================================
+
+#if VECOPS_ARTIFACT_KIND == 11
+#define OPERANDS "bf16"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16) | bit(VECOPS_DTYPE_F32);  // fp32 sources are rounded to bf16
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_BF16;
+#else
+#define OPERANDS "i8"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8);
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_I8;
+#endif
+constexpr const char* kOperatorName = "vecops::matmul_pack_b";
+constexpr const char* kKey = "vecops::matmul_pack_b;operands=" OPERANDS ";memory=" MEMORY_NAME ";backend=hip-gfx950";
+
+#define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
+   {.tensor = {sizeof(VecopsTensorParameter), MASK, kDeviceType, -1, RANK, OPTIONAL,                          \
+               sizeof(VecopsDimensionConstraint), nullptr, nullptr, FLAGS}}}
+
+const VecopsParameterDescriptor kParameters[] = {
+  TENSOR_PARAM("b", kInMask, -1, 0, VECOPS_TENSOR_READ),
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_SCALAR, "a_zero_point",
+   {.scalar = {sizeof(VecopsScalarParameter), bit(VECOPS_DTYPE_I64) | bit(VECOPS_DTYPE_I32)}}},
+  TENSOR_PARAM("packed", bit(VECOPS_DTYPE_U8), -1, 0, VECOPS_TENSOR_WRITE),
+  TENSOR_PARAM("compensation", bit(VECOPS_DTYPE_I32), -1, 1, VECOPS_TENSOR_WRITE),
+};
+
+int32_t workspace_impl(const VecopsCall* call, uint64_t* bytes, VecopsError* error) {
+  if (int32_t rc = check_call(call, 4, error); rc != VECOPS_STATUS_OK) return rc;
+  *bytes = 0;
+  return VECOPS_STATUS_OK;
+}
+
+int32_t run_impl(const VecopsCall* call, VecopsError* error) {
+  if (int32_t rc = check_call(call, 4, error); rc != VECOPS_STATUS_OK) return rc;
+  const VecopsTensorView* b = tensor_arg(call, 0);
+  const VecopsTensorView* packed = tensor_arg(call, 2);
+  const VecopsTensorView* comp = tensor_arg(call, 3);
+  if (b == nullptr || packed == nullptr || call->values[1].kind != VECOPS_VALUE_SCALAR)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "b and packed must be tensors, a_zero_point a scalar");
+  if (b->rank != 2 || packed->rank != 1 || (packed->sizes[0] > 1 && packed->strides[0] != 1) ||
+      (comp && (comp->rank != 1 || (comp->sizes[0] > 1 && comp->strides[0] != 1))))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "matmul_pack_b takes a rank-2 b and dense rank-1 outputs");
+  const int64_t n = b->sizes[0], k = b->sizes[1];
+  const uint64_t need = vecops_hip_packed_b_bytes(kPackedDtype, n, k);
+  if (static_cast<uint64_t>(packed->sizes[0]) < need)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT,
+                  "packed holds " + std::to_string(packed->sizes[0]) + " bytes, " + std::to_string(need) + " are needed");
+  if (comp && (kPackedDtype != VECOPS_DTYPE_I8 || comp->sizes[0] != n))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "compensation goes with an int8 b and has N entries");
+  if (need == 0) return VECOPS_STATUS_OK;
+  hipStream_t stream = stream_of(call);
+  Staging staging(stream);
+  void *b_dev = nullptr, *p_dev = nullptr, *c_dev = nullptr;
+  int32_t rc;
+  if ((rc = device_address(packed, true, &staging, &p_dev, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(b, false, &staging, &b_dev, error)) != VECOPS_STATUS_OK) return rc;
+  if (comp && (rc = device_address(comp, true, &staging, &c_dev, error)) != VECOPS_STATUS_OK) return rc;
+  VecopsHipOperand ob;
+  if (!fill_operand(b, b_dev, &ob)) return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "b must have rank 2");
+  if (comp)
+    rc = vecops_hip_pack_b_compensated(&ob, static_cast<int32_t>(call->values[1].value.scalar.value.i64), p_dev,
+                                       static_cast<uint64_t>(packed->sizes[0]), static_cast<int32_t*>(c_dev), stream);
+  else
+    rc = vecops_hip_pack_b(&ob, p_dev, static_cast<uint64_t>(packed->sizes[0]), stream);
+  if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
+  return finish(&staging, stream, error);
+}
+
+// =================================================================================================
+#elif VECOPS_ARTIFACT_KIND >= 13 && VECOPS_ARTIFACT_KIND <= 15  // vecops::matmul_packed_b (a, packed_b, c_in?, c)
+// =================================================================================================
+
+#if VECOPS_ARTIFACT_KIND == 13
+#define OPERANDS "bf16"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16);
+#elif VECOPS_ARTIFACT_KIND == 14
+#define OPERANDS "f32"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
+#else
+#define OPERANDS "i8"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8);
+#endif
+#if VECOPS_ARTIFACT_KIND == 15
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_I32);
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_I8;
+#else
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_BF16;
+#endif
+constexpr const char* kOperatorName = "vecops::matmul_packed_b";
+constexpr const char* kKey = "vecops::matmul_packed_b;operands=" OPERANDS ";memory=" MEMORY_NAME ";backend=hip-gfx950";
+
+#define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
+   {.tensor = {sizeof(VecopsTensorParameter), MASK, kDeviceType, -1, RANK, OPTIONAL,                          \
+               sizeof(VecopsDimensionConstraint), nullptr, nullptr, FLAGS}}}
+
+const VecopsParameterDescriptor kParameters[] = {
+  TENSOR_PARAM("a", kInMask, -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("packed_b", bit(VECOPS_DTYPE_U8), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("c_in", kOutMask, -1, 1, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("c", kOutMask, -1, 0, VECOPS_TENSOR_WRITE),
+};
+
+struct PackedArgs {
+  const VecopsTensorView *a, *packed, *cin, *c;
+  VecopsHipOperand oa, ocin, oc;
+  int64_t n;
+};
+
+int32_t decode(const VecopsCall* call, PackedArgs* d, VecopsHipPlan* plan, VecopsError* error) {
+  if (int32_t rc = check_call(call, 4, error); rc != VECOPS_STATUS_OK) return rc;
+  d->a = tensor_arg(call, 0);
+  d->packed = tensor_arg(call, 1);
+  d->cin = tensor_arg(call, 2);
+  d->c = tensor_arg(call, 3);
+  if (d->a == nullptr || d->packed == nullptr || d->c == nullptr)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "a, packed_b and c must be tensors");
+  if (d->packed->rank != 1 || (d->packed->sizes[0] > 1 && d->packed->strides[0] != 1))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "packed_b must be a dense rank-1 byte tensor");
+  if (!fill_operand(d->a, reinterpret_cast<void*>(16), &d->oa) || !fill_operand(d->c, reinterpret_cast<void*>(16), &d->oc) ||
+      (d->cin != nullptr && !fill_operand(d->cin, reinterpret_cast<void*>(16), &d->ocin)))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "tensors must have rank 2 or 3");
+  d->n = d->c->sizes[d->c->rank - 1];
+  const int64_t k = d->a->sizes[d->a->rank - 1];
+  const uint64_t need = vecops_hip_packed_b_bytes(kPackedDtype, d->n, k);
+  if (static_cast<uint64_t>(d->packed->sizes[0]) < need)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT,
+                  "packed_b holds " + std::to_string(d->packed->sizes[0]) + " bytes, " + std::to_string(need) +
+                    " are needed for N = " + std::to_string(d->n) + ", K = " + std::to_string(k));
+#if VECOPS_ARTIFACT_DEVICE
+  d->oa.data = origin(d->a);
+  d->oc.data = origin(d->c);
+  if (d->cin != nullptr) d->ocin.data = origin(d->cin);
+#endif
+  int32_t rc = vecops_hip_plan_matmul_packed_b(&d->oa, kPackedDtype, d->n, d->cin ? &d->ocin : nullptr, &d->oc, plan);
+  return rc == VECOPS_STATUS_OK ? rc : report_kernel(error, rc);
+}
+
+int32_t workspace_impl(const VecopsCall* call, uint64_t* bytes, VecopsError* error) {
+  PackedArgs d;
+  VecopsHipPlan p;
+  if (int32_t rc = decode(call, &d, &p, error); rc != VECOPS_STATUS_OK) return rc;
+#if VECOPS_ARTIFACT_DEVICE
+  *bytes = p.workspace_bytes;
+#else
+  *bytes = 0;
+#endif
+  return VECOPS_STATUS_OK;
+}
+
+int32_t run_impl(const VecopsCall* call, VecopsError* error) {
+  PackedArgs d;
+  VecopsHipPlan p;
+  if (int32_t rc = decode(call, &d, &p, error); rc != VECOPS_STATUS_OK) return rc;
+  if (p.family == VECOPS_HIP_FAMILY_NONE) return VECOPS_STATUS_OK;
+  hipStream_t stream = stream_of(call);
+  Staging staging(stream);
+  void* ws = call->workspace;
+  uint64_t ws_size = call->workspace_size;
+  void* packed_dev = nullptr;
+  int32_t rc;
+#if VECOPS_ARTIFACT_DEVICE
+  packed_dev = origin(d.packed);
+#else
+  void* dev = nullptr;
+  if ((rc = device_address(d.c, true, &staging, &dev, error)) != VECOPS_STATUS_OK) return rc;
+  d.oc.data = dev;
+  if (d.cin && (rc = device_address(d.cin, false, &staging, &dev, error)) != VECOPS_STATUS_OK) return rc;
+  if (d.cin) d.ocin.data = dev;
+  if ((rc = device_address(d.a, false, &staging, &dev, error)) != VECOPS_STATUS_OK) return rc;
+  d.oa.data = dev;
+  if ((rc = device_address(d.packed, false, &staging, &packed_dev, error)) != VECOPS_STATUS_OK) return rc;
+  if (hipError_t e = staging.workspace(p.workspace_bytes, &ws); e != hipSuccess)
+    return report_hip(error, "allocating split-K scratch", e);
+  ws_size = p.workspace_bytes;
+#endif
+  rc = vecops_hip_matmul_packed_b(&d.oa, packed_dev, kPackedDtype, d.n, d.cin ? &d.ocin : nullptr, &d.oc, ws, ws_size,
+                                  stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
   return finish(&staging, stream, error);
 }

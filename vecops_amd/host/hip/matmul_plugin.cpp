@@ -108,6 +108,34 @@ Status w8a16_relations(std::span<const Value> v) {
   return Status::success();
 }
 
+// vecops::matmul_pack_b (b, a_zero_point, packed, compensation?)
+Status pack_b_relations(std::span<const Value> v) {
+  const TensorView* b = tensor_at(v, 0);
+  const TensorView* packed = tensor_at(v, 2);
+  const TensorView* comp = tensor_at(v, 3);
+  if (b == nullptr || packed == nullptr) return invalid("vecops::matmul_pack_b needs b and packed tensors");
+  if (v.size() < 2 || std::get_if<rt::Scalar>(&v[1]) == nullptr) return invalid("a_zero_point must be a scalar");
+  if (comp != nullptr && b->dtype != DType::Int8) return invalid("compensation goes with an int8 b");
+  if (comp != nullptr && comp->sizes[0] != b->sizes[0]) return invalid("compensation must have N entries");
+  return Status::success();
+}
+
+// vecops::matmul_packed_b (a, packed_b, c_in?, c): N is c's last extent, K is a's.
+Status packed_b_relations(std::span<const Value> v) {
+  const TensorView* a = tensor_at(v, 0);
+  const TensorView* packed = tensor_at(v, 1);
+  const TensorView* cin = tensor_at(v, 2);
+  const TensorView* c = tensor_at(v, 3);
+  if (a == nullptr || packed == nullptr || c == nullptr) return invalid("vecops::matmul_packed_b needs a, packed_b and c");
+  const std::size_t rank = a->sizes.size();
+  if (rank != 2 && rank != 3) return invalid("a must have rank 2 or 3");
+  if (c->sizes.size() != rank || (cin && cin->sizes.size() != rank)) return invalid("a, c_in and c must have the same rank");
+  if (rows(*c) != rows(*a)) return invalid("c must be [.., M, N]");
+  if (cin && (rows(*cin) != rows(*c) || cols(*cin) != cols(*c))) return invalid("c_in must be [.., M, N]");
+  if (rank == 3 && (a->sizes[0] != c->sizes[0] || (cin && cin->sizes[0] != c->sizes[0]))) return invalid("batch extents differ");
+  return Status::success();
+}
+
 // Placement of a call: all tensors on the host, or all on the device.
 rt::Result<Placement> placement_of(const rt::KernelCall& call) {
   bool host = false, device = false;
@@ -208,6 +236,29 @@ rt::OperatorSchema make_matmul_w8a16_group_schema() {
   params.push_back(tensor_param("scales", dtype_bit(DType::Float32), 2u, VECOPS_TENSOR_READ));
   params.push_back(tensor_param("y", dtype_bit(DType::BFloat16), 2u, VECOPS_TENSOR_WRITE));
   return rt::OperatorSchema(kMatmulW8A16GroupName, std::move(params), w8a16_relations);
+}
+
+rt::OperatorSchema make_matmul_pack_b_schema() {
+  using rt::dtype_bit;
+  std::vector<rt::ParameterSchema> params;
+  params.push_back(tensor_param("b", dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8), 2u,
+                                VECOPS_TENSOR_READ));
+  params.push_back(rt::ParameterSchema{"a_zero_point", rt::ScalarConstraint{dtype_bit(DType::Int64) | dtype_bit(DType::Int32)}});
+  params.push_back(tensor_param("packed", dtype_bit(DType::UInt8), 1u, VECOPS_TENSOR_WRITE));
+  params.push_back(tensor_param("compensation", dtype_bit(DType::Int32), 1u, VECOPS_TENSOR_WRITE, /*optional=*/true));
+  return rt::OperatorSchema(kMatmulPackBName, std::move(params), pack_b_relations);
+}
+
+rt::OperatorSchema make_matmul_packed_b_schema() {
+  using rt::dtype_bit;
+  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8);
+  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int32);
+  std::vector<rt::ParameterSchema> params;
+  params.push_back(tensor_param("a", in, std::nullopt, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("packed_b", dtype_bit(DType::UInt8), 1u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("c_in", out, std::nullopt, VECOPS_TENSOR_READ, /*optional=*/true));
+  params.push_back(tensor_param("c", out, std::nullopt, VECOPS_TENSOR_WRITE));
+  return rt::OperatorSchema(kMatmulPackedBName, std::move(params), packed_b_relations);
 }
 
 // ---- recipes ------------------------------------------------------------------------------------
@@ -370,6 +421,69 @@ rt::Result<rt::BoundKernelRecipe> MatmulW8A16GroupRecipe::bind(const rt::KernelC
   return bound;
 }
 
+MatmulPackBRecipe::MatmulPackBRecipe(OperandClass packed) : packed_(packed) {
+  id_ = packed == OperandClass::I8 ? "hip.matmul_pack_b.i8" : "hip.matmul_pack_b.bf16";
+}
+
+Status MatmulPackBRecipe::match(const rt::KernelCall& call) const {
+  const auto values = call.arguments().values();
+  const TensorView* b = tensor_at(values, 0);
+  if (b == nullptr) return invalid("vecops::matmul_pack_b needs a b tensor");
+  const bool mine = packed_ == OperandClass::I8 ? b->dtype == DType::Int8
+                                                : (b->dtype == DType::BFloat16 || b->dtype == DType::Float32);
+  if (!mine) return not_applicable("source dtype belongs to another recipe");
+  auto place = placement_of(call);
+  if (!place) return place.status();
+  return Status::success();
+}
+
+rt::Result<rt::BoundKernelRecipe> MatmulPackBRecipe::bind(const rt::KernelCall& call) const {
+  if (Status st = match(call); !st.ok()) return st;
+  rt::BoundKernelRecipe bound;
+  bound.recipe_id = id_;
+  bound.specialization_key = std::string(kMatmulPackBName) + ";operands=" + (packed_ == OperandClass::I8 ? "i8" : "bf16") +
+                             ";memory=" + placement_name(placement_of(call).value()) + ";" + kBackend;
+  bound.artifact_key = id_ + ";" + bound.specialization_key;
+  return bound;
+}
+
+MatmulPackedBRecipe::MatmulPackedBRecipe(OperandClass operands) : operands_(operands) {
+  id_ = operands == OperandClass::BF16 ? "hip.matmul_packed_b.bf16.tile"
+        : operands == OperandClass::F32 ? "hip.matmul_packed_b.f32.tile"
+                                        : "hip.matmul_packed_b.i8.tile";
+}
+
+Status MatmulPackedBRecipe::match(const rt::KernelCall& call) const {
+  const auto values = call.arguments().values();
+  const TensorView* a = tensor_at(values, 0);
+  const TensorView* cin = tensor_at(values, 2);
+  const TensorView* c = tensor_at(values, 3);
+  if (a == nullptr || c == nullptr) return invalid("vecops::matmul_packed_b needs a and c tensors");
+  const bool mine = operands_ == OperandClass::I8 ? a->dtype == DType::Int8
+                    : operands_ == OperandClass::F32 ? a->dtype == DType::Float32
+                                                     : a->dtype == DType::BFloat16;
+  if (!mine) return not_applicable("operand dtype belongs to another recipe");
+  const bool int_out = operands_ == OperandClass::I8;
+  if (int_out ? c->dtype != DType::Int32 : (c->dtype != DType::Float32 && c->dtype != DType::BFloat16))
+    return not_applicable("output dtype does not fit these operands");
+  if (cin != nullptr && (int_out ? cin->dtype != DType::Int32 : (cin->dtype != DType::Float32 && cin->dtype != DType::BFloat16)))
+    return not_applicable("c_in dtype does not fit these operands");
+  auto place = placement_of(call);
+  if (!place) return place.status();
+  return Status::success();
+}
+
+rt::Result<rt::BoundKernelRecipe> MatmulPackedBRecipe::bind(const rt::KernelCall& call) const {
+  if (Status st = match(call); !st.ok()) return st;
+  const char* operands = operands_ == OperandClass::BF16 ? "bf16" : operands_ == OperandClass::F32 ? "f32" : "i8";
+  rt::BoundKernelRecipe bound;
+  bound.recipe_id = id_;
+  bound.specialization_key = std::string(kMatmulPackedBName) + ";operands=" + operands + ";memory=" +
+                             placement_name(placement_of(call).value()) + ";" + kBackend;
+  bound.artifact_key = id_ + ";" + bound.specialization_key;
+  return bound;
+}
+
 // ---- dispatch policy --------------------------------------------------------------------------------
 
 rt::Result<std::vector<std::size_t>>
@@ -385,6 +499,13 @@ MatmulDispatchPolicy::candidates(const rt::KernelCall& call,
     }
     if (const auto* mf = dynamic_cast<const MatmulFusedRecipe*>(recipes[i].get()); mf != nullptr && a != nullptr) {
       if (!takes(mf->operands(), a->dtype)) continue;
+    }
+    if (const auto* mp = dynamic_cast<const MatmulPackedBRecipe*>(recipes[i].get()); mp != nullptr && a != nullptr) {
+      if (mp->operands() == OperandClass::I8 ? a->dtype != DType::Int8
+          : mp->operands() == OperandClass::F32 ? a->dtype != DType::Float32 : a->dtype != DType::BFloat16) continue;
+    }
+    if (const auto* pk = dynamic_cast<const MatmulPackBRecipe*>(recipes[i].get()); pk != nullptr && a != nullptr) {
+      if ((pk->operands() == OperandClass::I8) != (a->dtype == DType::Int8)) continue;
     }
     order.push_back(i);
   }
@@ -483,6 +604,20 @@ std::shared_ptr<rt::Operator> make_matmul_fused_operator(const std::filesystem::
                    std::make_shared<MatmulFusedRecipe>(OperandClass::F16),
                    std::make_shared<MatmulFusedRecipe>(OperandClass::F32),
                    std::make_shared<MatmulFusedRecipe>(OperandClass::I8)},
+                  dir);
+}
+
+std::shared_ptr<rt::Operator> make_matmul_pack_b_operator(const std::filesystem::path& dir) {
+  return assemble(make_matmul_pack_b_schema(),
+                  {std::make_shared<MatmulPackBRecipe>(OperandClass::BF16), std::make_shared<MatmulPackBRecipe>(OperandClass::I8)},
+                  dir);
+}
+
+std::shared_ptr<rt::Operator> make_matmul_packed_b_operator(const std::filesystem::path& dir) {
+  return assemble(make_matmul_packed_b_schema(),
+                  {std::make_shared<MatmulPackedBRecipe>(OperandClass::BF16),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::F32),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::I8)},
                   dir);
 }
 

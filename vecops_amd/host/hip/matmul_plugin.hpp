@@ -16,6 +16,9 @@
 //                                column_scales f32[N], correction? i32[N], c f32[M,N] out)
 //   vecops::matmul_w8a16_group  (x bf16[M,K], w i8[N,K], scales f32[N,K/G], y bf16[M,N] out)
 //       specialization value  G : ConstInt          (128 default)
+//   vecops::matmul_pack_b       (b[N,K], a_zero_point scalar, packed u8[bytes] out, compensation? i32[N] out)
+//       specialization value  PackedType : DType    (the source's own class by default)
+//   vecops::matmul_packed_b     (a[..,M,K], packed_b u8[bytes], c_in?[..,M,N], c[..,M,N] out)
 #ifndef VECOPS_HIP_MATMUL_PLUGIN_HPP
 #define VECOPS_HIP_MATMUL_PLUGIN_HPP
 
@@ -37,6 +40,11 @@ inline constexpr const char* kMatmulName = "vecops::matmul";
 inline constexpr const char* kMatmulI8DequantName = "vecops::matmul_i8_dequant";
 inline constexpr const char* kMatmulW8A16GroupName = "vecops::matmul_w8a16_group";
 inline constexpr const char* kMatmulFusedName = "vecops::matmul_fused";
+inline constexpr const char* kMatmulPackBName = "vecops::matmul_pack_b";
+inline constexpr const char* kMatmulPackedBName = "vecops::matmul_packed_b";
+
+// Operand classes of vecops::matmul, one artifact each.
+enum class OperandClass { BF16, F32, I8, F16 };
 
 // Schemas.  Ranks are left open on vecops::matmul (rank 2 and rank 3 go through
 // one operator); the relation validator enforces what the CPU path asserts in
@@ -52,9 +60,13 @@ rt::OperatorSchema make_matmul_w8a16_group_schema();
 // (the call ABI has no optional scalars): activation 0 none, 1 relu, 2 clamp, 3 sigmoid, 4 silu; scale 1.0 and
 // shift 0.0 mean "no such step".
 rt::OperatorSchema make_matmul_fused_schema();
-
-// Operand classes of vecops::matmul, one artifact each.
-enum class OperandClass { BF16, F32, I8, F16 };
+// vecops::matmul_pack_b (b, a_zero_point, packed out, compensation? out): the B side of ops::matmul_pack
+// (ops/MatmulPack.h:9-117).  `packed` is an opaque byte tensor of at least vecops_hip_packed_b_bytes(dtype, N, K) bytes; with a
+// compensation tensor (int8 only) the pack also writes -a_zero_point * sum_k b[n,k], the sidecar of
+// MatmulPackBCompensated.  vecops::matmul_packed_b (a, packed_b, c_in?, c out) multiplies by such a tensor: N
+// comes from c, K from a, and one packed operand serves every batch of a rank-3 a (ops/MatmulPack.h:22-24).
+rt::OperatorSchema make_matmul_pack_b_schema();
+rt::OperatorSchema make_matmul_packed_b_schema();
 
 // Kernel families a recipe stands for: the MFMA workgroup-tile kernels or the
 // wavefront split-K dot-product kernels for skinny shapes.
@@ -112,6 +124,36 @@ public:
   [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
 };
 
+// vecops::matmul_pack_b for one packed class (BF16 takes bf16 and fp32 sources, I8 takes int8):
+//   vecops::matmul_pack_b;operands=<bf16|i8>;memory=<host|device>;backend=hip-gfx950
+class MatmulPackBRecipe final : public rt::KernelRecipe {
+public:
+  explicit MatmulPackBRecipe(OperandClass packed);
+  [[nodiscard]] std::string_view id() const override { return id_; }
+  [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
+  [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
+  [[nodiscard]] OperandClass operands() const { return packed_; }
+
+private:
+  OperandClass packed_;
+  std::string id_;
+};
+
+// vecops::matmul_packed_b for one class of a (fp32 rows are rounded to bf16 against a bf16 pack):
+//   vecops::matmul_packed_b;operands=<bf16|f32|i8>;memory=<host|device>;backend=hip-gfx950
+class MatmulPackedBRecipe final : public rt::KernelRecipe {
+public:
+  explicit MatmulPackedBRecipe(OperandClass operands);
+  [[nodiscard]] std::string_view id() const override { return id_; }
+  [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
+  [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
+  [[nodiscard]] OperandClass operands() const { return operands_; }
+
+private:
+  OperandClass operands_;
+  std::string id_;
+};
+
 // GPU counterpart of the call sites of vecops' runtime shape predicates
 // (matmul/details/kernel/amx/Backend.h:2724-2757 consulting
 // src/MatmulRuntimeDispatch.cpp:12-32): orders the recipes of an operator for
@@ -157,6 +199,8 @@ std::shared_ptr<rt::Operator> make_matmul_operator(const std::filesystem::path& 
 std::shared_ptr<rt::Operator> make_matmul_i8_dequant_operator(const std::filesystem::path& artifact_directory);
 std::shared_ptr<rt::Operator> make_matmul_w8a16_group_operator(const std::filesystem::path& artifact_directory);
 std::shared_ptr<rt::Operator> make_matmul_fused_operator(const std::filesystem::path& artifact_directory);
+std::shared_ptr<rt::Operator> make_matmul_pack_b_operator(const std::filesystem::path& artifact_directory);
+std::shared_ptr<rt::Operator> make_matmul_packed_b_operator(const std::filesystem::path& artifact_directory);
 
 }  // namespace vecops::hip
 #endif

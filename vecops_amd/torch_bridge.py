@@ -22,7 +22,7 @@ from types import SimpleNamespace
 from . import host_api as H
 
 # Positional parameters of the operators this package ships (name, kind); kind is
-# "in", "in?" (optional tensor), "out", "int" or "float".  Specialization values are
+# "in", "in?" (optional tensor), "out", "out?" (optional output), "int" or "float".  Specialization values are
 # keyword-only integers on the torch operator (-1 = not given); "dtype" ones take a
 # torch dtype or a VecopsDType number on the public callable.
 SIGNATURES = {
@@ -33,6 +33,8 @@ SIGNATURES = {
     "vecops::matmul_fused": ([("a", "in"), ("b", "in"), ("c_in", "in?"), ("row_scales", "in?"),
                               ("column_scales", "in?"), ("activation", "int"), ("scale", "float"), ("shift", "float"),
                               ("clamp_lo", "float"), ("clamp_hi", "float"), ("c", "out")], {}),
+    "vecops::matmul_pack_b": ([("b", "in"), ("a_zero_point", "int"), ("packed", "out"), ("compensation", "out?")], {}),
+    "vecops::matmul_packed_b": ([("a", "in"), ("packed_b", "in"), ("c_in", "in?"), ("c", "out")], {}),
 }
 
 _PREPARED_CALLS = 8          # signatures kept per thread (docs/Runtime.md:196-206)
@@ -66,7 +68,7 @@ class _Registration:
     def __init__(self, library, name, operator, params, specs, return_outputs):
         self.library, self.name, self.operator = library, name, operator
         self.params, self.specs, self.return_outputs = params, specs, return_outputs
-        self.outputs = tuple(i for i, (_, kind) in enumerate(params) if kind == "out")
+        self.outputs = tuple(i for i, (_, kind) in enumerate(params) if kind in ("out", "out?"))
         self.local = threading.local()
         self.torch_op = None
         self.wrapper = None
@@ -76,14 +78,15 @@ class _Registration:
         parts = []
         alias = iter("abcdefgh")
         for pname, kind in self.params:
-            if kind == "out":
-                parts.append(f"Tensor({next(alias)}!) {pname}")
+            if kind in ("out", "out?"):
+                parts.append(f"Tensor({next(alias)}!){'?' if kind == 'out?' else ''} {pname}")
             else:
                 parts.append({"in": "Tensor", "in?": "Tensor?", "int": "int", "float": "float"}[kind] + " " + pname)
         if self.specs:
             parts.append("*")
             parts += [f"int {sname}=-1" for sname in self.specs]
-        returns = "(" + ", ".join("Tensor" for _ in self.outputs) + ")" if self.return_outputs else "()"
+        returns = "(" + ", ".join("Tensor?" if self.params[i][1] == "out?" else "Tensor" for i in self.outputs) + ")" \
+            if self.return_outputs else "()"
         return f"{self.name}({', '.join(parts)}) -> {returns}"
 
     def signature(self, values, spec_values):
@@ -166,7 +169,7 @@ class _Registration:
             if sname in kwargs:
                 spec_ints[sname] = _dtype_code(kwargs[sname]) if skind == "dtype" else int(kwargs[sname])
         self.torch_op(*args, **spec_ints)
-        outs = tuple(args[i] for i in self.outputs)
+        outs = tuple(args[i] for i in self.outputs if args[i] is not None)
         return outs[0] if len(outs) == 1 else outs
 
 
