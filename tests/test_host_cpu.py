@@ -255,6 +255,7 @@ def test_packed_b_operators_resolution_and_validation(host):
     assert "operands=bf16" in mul.resolve(mf(bf16((2, 4, 8)), None, bf16((2, 4, 5))))
     assert "operands=f32" in mul.resolve(mf(np.zeros((4, 8), np.float32), c, c))
     assert "operands=i8" in mul.resolve(mf(np.zeros((4, 8), np.int8), None, np.zeros((4, 5), np.int32)))
+    assert "operands=i8" in mul.resolve(mf(np.zeros((4, 8), np.uint8), None, np.zeros((4, 5), np.int32)))   # u8 x packed s8
     for fr, needle in [(mf(bf16((4, 8)), None, np.zeros((3, 5), np.float32)), "[.., M, N]"),
                        (mf(bf16((2, 4, 8)), None, np.zeros((3, 4, 5), np.float32)), "batch"),
                        (mf(bf16((4, 8)), np.zeros((4, 6), np.float32), c), "c_in")]:

@@ -225,6 +225,9 @@ def test_packed_b_operators(host, oracle, device):
     corr = np.broadcast_to(comp, (m, n))                                      # the sidecar as a stride-0 C-input row
     mul.invoke(H.Frame([a, packed, corr, c], outputs=(3,)))
     assert np.array_equal(c, want + comp[None, :])
+    ua = (a.astype(np.int16) + 7).clip(0, 255).astype(np.uint8)                # asymmetric activations, zero point 7
+    mul.invoke(H.Frame([ua, packed, corr, c], outputs=(3,)))                   # = sum_k (ua - 7) * b
+    assert np.array_equal(c, ((ua.astype(np.int64) - 7) @ b.astype(np.int64).T).astype(np.int32))
     # bf16 from an fp32 source, device tensors, rank-3 a with a workspace when the plan asks for one
     batch, m, n, k = 3, 50, 200, 1000
     a = synth.bf16_round(synth.uniform_pm1(1, (batch, m, k)))

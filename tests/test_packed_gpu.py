@@ -110,6 +110,47 @@ def test_packed_int8_matmul_bit_exact(device, oracle, m, n, k):
     assert np.array_equal(c.cpu().numpy(), oracle.matmul_i8_dense(a, b))
 
 
+@pytest.mark.parametrize("m,n,k", [(19, 21, 69), (1, 128, 65), (35, 53, 257), (256, 256, 128), (300, 520, 1000),
+                                   (1024, 768, 4096), (64, 48, 8191), (2, 33, 262145)])
+def test_packed_int8_b_with_unsigned_a_bit_exact(device, oracle, m, n, k):
+    """uint8 activations against int8-packed weights (the atom AMX_I8I32<uint8_t, int8_t> that
+    ops::matmul_pack_b_compensated exists for): a is staged as a - 128 and 128 * sum_k b[n,k], summed from the
+    packed rows, is added back; every int32 equals the exact integer sum mod 2^32 (tile, split-K, ragged shapes,
+    and a K long enough for the sums of 255 * 127 to wrap)."""
+    import torch
+    from vecops_amd import capi
+    a = (synth.draws(1, m * k) % np.uint64(256)).astype(np.uint8).reshape(m, k)
+    b = synth.int8_sym(2, (n, k))
+    if k > 100000:
+        a[0], b[0] = 255, 127                                   # 262145 * 255 * 127 > 2^31
+    packed = capi.pack_b(torch.from_numpy(b).to(device))
+    c = torch.full((m, n), -1, dtype=torch.int32, device=device)
+    capi.matmul_packed_b(torch.from_numpy(a).to(device), packed, c)
+    torch.cuda.synchronize()
+    exact = a.astype(np.int64) @ b.astype(np.int64).T
+    assert np.array_equal(c.cpu().numpy(), (exact & 0xffffffff).astype(np.uint32).view(np.int32))
+    if k < 100000:
+        want = np.zeros((m, n), np.int32)
+        oracle.matmul(a, b, want, atom=2)
+        assert np.array_equal(c.cpu().numpy(), want)
+
+
+def test_packed_int8_b_with_unsigned_a_batched(device):
+    """One packed operand for every batch of a rank-3 uint8 a, with an int32 C input."""
+    import torch
+    from vecops_amd import capi
+    batch, m, n, k = 3, 70, 200, 300
+    a = (synth.draws(1, batch * m * k) % np.uint64(256)).astype(np.uint8).reshape(batch, m, k)
+    b = synth.int8_sym(2, (n, k))
+    cin = ((synth.draws(3, batch * m * n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32).reshape(batch, m, n)
+    packed = capi.pack_b(torch.from_numpy(b).to(device))
+    c = torch.full((batch, m, n), -1, dtype=torch.int32, device=device)
+    capi.matmul_packed_b(torch.from_numpy(a).to(device), packed, c, c_in=torch.from_numpy(cin).to(device))
+    torch.cuda.synchronize()
+    want = np.einsum("bmk,nk->bmn", a.astype(np.int64), b.astype(np.int64)) + cin
+    assert np.array_equal(c.cpu().numpy(), want.astype(np.int32))
+
+
 @pytest.mark.parametrize("m,n,k,corr", [(67, 129, 515, True), (256, 384, 1024, False), (300, 1000, 2048, True),
                                         (1, 300, 4096, False)])
 def test_packed_int8_dequant_bit_exact(device, oracle, m, n, k, corr):
@@ -206,6 +247,12 @@ def test_pack_b_compensated_reference_case(device):
     torch.cuda.synchronize()
     want_c = (ua.astype(np.int64) - zp) @ logical.astype(np.int64).T
     assert np.array_equal(c.cpu().numpy(), want_c.astype(np.int32))
+    # and the same against the packed operand itself: AMX_I8I32<uint8_t, int8_t> with a packed B and its
+    # sidecar (ops/MatmulPack.h:52-58)
+    c2 = torch.full((m, n), -1, dtype=torch.int32, device=device)
+    capi.matmul_packed_b(torch.from_numpy(ua).to(device), packed, c2, c_in=cin)
+    torch.cuda.synchronize()
+    assert np.array_equal(c2.cpu().numpy(), want_c.astype(np.int32))
 
 
 def test_packed_zero_extents_and_rejections(device):

@@ -444,7 +444,11 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
       if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
       p.row_term = row_term;
     }
-    if (pr.a_unsigned) {  // + 128 * sum_k b'[n,k] per column
+    if (pr.a_unsigned && pr.packed_b) {  // the same term from the packed rows, one copy per batch
+      e = launch_packed_row_sums(pr.b.data, p.n, p.k, p.batch, 128u, col_term, stream);
+      if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
+      p.col_term = col_term;
+    } else if (pr.a_unsigned) {  // + 128 * sum_k b'[n,k] per column
       e = launch_byte_row_sums(pr.b.data, p.batch, p.n, p.k, pr.b.bs, pr.b.rs, pr.b.cs, p.b_flip, 128u, col_term, stream);
       if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
       p.col_term = col_term;
@@ -516,14 +520,14 @@ int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t 
   if (packed_dtype == DT_BF16) {
     if (da != DT_BF16 && da != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: a bf16-packed b needs a bf16 or f32 a");
   } else if (packed_dtype == DT_I8) {
-    if (da != DT_I8) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an i8-packed b needs an i8 a");
+    if (da != DT_I8 && da != DT_U8) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an i8-packed b needs an i8 or u8 a");
   } else {
     return fail(ST_NOT_APPLICABLE, "matmul_packed_b: packed dtype %u not supported", packed_dtype);
   }
   VecopsHipOperand b;
   memset(&b, 0, sizeof(b));
   b.data = const_cast<void*>(packed);
-  b.dtype = da;
+  b.dtype = packed_dtype == DT_I8 ? DT_I8 : da;
   b.rank = a->rank;
   const int base = a->rank == 3 ? 1 : 0;
   const int64_t k = a->sizes[base + 1];
@@ -536,7 +540,7 @@ int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t 
   if (rc != ST_OK) return rc;
   pr->packed_b = true;
   // 32-bit offsets inside one workgroup's eight 32-row panels of the packed operand
-  const int64_t ks_total = packed_k_steps(pr->k, pr->src == SRC_I8 ? 16 : 8);
+  const int64_t ks_total = packed_k_steps(pr->k, packed_dtype == DT_I8 ? 16 : 8);
   if (ks_total * 1024 * 8 >= (int64_t{1} << 31)) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: k too large");
   return ST_OK;
 }

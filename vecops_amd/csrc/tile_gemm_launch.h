@@ -31,10 +31,14 @@ hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile_m, int til
 hipError_t launch_byte_row_sums(const void* x, int32_t batch, int32_t rows, int32_t k, int64_t bs, int64_t rs,
                                 int64_t ks, uint32_t flip, uint32_t scale, int32_t* out, hipStream_t stream);
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
-// B prepacked by launch_pack_b (src: SRC_BF16, SRC_F32_AS_BF16 = fp32 A against bf16-packed B, SRC_I8);
+// B prepacked by launch_pack_b (src: SRC_BF16, SRC_F32_AS_BF16 = fp32 A against bf16-packed B, SRC_I8,
+// SRC_I8_FLIP = unsigned A against int8-packed B with p.a_flip and p.col_term set);
 // vector_a: 0 = any strides, 1 = A is K-contiguous, 2 = and its base, rows and batches are 16-byte aligned
 hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_m, int tile_n, int vector_a,
                                      hipStream_t stream);
+// out[b][n] = scale * sum_k B[n,k] of an int8-packed operand, for b < batch
+hipError_t launch_packed_row_sums(const void* packed, int32_t n, int32_t k, int32_t batch, uint32_t scale, int32_t* out,
+                                  hipStream_t stream);
 struct PackBParams;
 hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream);
 

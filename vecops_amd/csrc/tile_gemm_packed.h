@@ -118,7 +118,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
   auto seq = [&](int j) { return (has_tail && j == 0) ? kt_end - 1 : kt_begin + j - has_tail; };
 
   Stager<SRC, LOAD_A, BM, THREADS> stager_a;
-  stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, tid, 0u);
+  stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, tid, p.a_flip);
   using SA = decltype(stager_a);
 
   // packed B: descriptor at the first 32-row block of this tile; the lane offset picks block row and lane

@@ -699,7 +699,7 @@ constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16);
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
 #else
 #define OPERANDS "i8"
-constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8);
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);
 #endif
 #if VECOPS_ARTIFACT_KIND == 15
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_I32);

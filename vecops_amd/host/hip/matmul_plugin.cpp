@@ -251,7 +251,8 @@ rt::OperatorSchema make_matmul_pack_b_schema() {
 
 rt::OperatorSchema make_matmul_packed_b_schema() {
   using rt::dtype_bit;
-  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8);
+  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8) |
+                           dtype_bit(DType::UInt8);
   const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int32);
   std::vector<rt::ParameterSchema> params;
   params.push_back(tensor_param("a", in, std::nullopt, VECOPS_TENSOR_READ));
@@ -459,7 +460,7 @@ Status MatmulPackedBRecipe::match(const rt::KernelCall& call) const {
   const TensorView* cin = tensor_at(values, 2);
   const TensorView* c = tensor_at(values, 3);
   if (a == nullptr || c == nullptr) return invalid("vecops::matmul_packed_b needs a and c tensors");
-  const bool mine = operands_ == OperandClass::I8 ? a->dtype == DType::Int8
+  const bool mine = operands_ == OperandClass::I8 ? (a->dtype == DType::Int8 || a->dtype == DType::UInt8)
                     : operands_ == OperandClass::F32 ? a->dtype == DType::Float32
                                                      : a->dtype == DType::BFloat16;
   if (!mine) return not_applicable("operand dtype belongs to another recipe");
@@ -501,7 +502,7 @@ MatmulDispatchPolicy::candidates(const rt::KernelCall& call,
       if (!takes(mf->operands(), a->dtype)) continue;
     }
     if (const auto* mp = dynamic_cast<const MatmulPackedBRecipe*>(recipes[i].get()); mp != nullptr && a != nullptr) {
-      if (mp->operands() == OperandClass::I8 ? a->dtype != DType::Int8
+      if (mp->operands() == OperandClass::I8 ? (a->dtype != DType::Int8 && a->dtype != DType::UInt8)
           : mp->operands() == OperandClass::F32 ? a->dtype != DType::Float32 : a->dtype != DType::BFloat16) continue;
     }
     if (const auto* pk = dynamic_cast<const MatmulPackBRecipe*>(recipes[i].get()); pk != nullptr && a != nullptr) {

@@ -139,7 +139,8 @@ private:
   std::string id_;
 };
 
-// vecops::matmul_packed_b for one class of a (fp32 rows are rounded to bf16 against a bf16 pack):
+// vecops::matmul_packed_b for one class of a (fp32 rows are rounded to bf16 against a bf16 pack; the i8 class
+// takes signed and unsigned bytes, AMX_I8I32<uint8_t, int8_t> being what the compensated pack is for):
 //   vecops::matmul_packed_b;operands=<bf16|f32|i8>;memory=<host|device>;backend=hip-gfx950
 class MatmulPackedBRecipe final : public rt::KernelRecipe {
 public:
