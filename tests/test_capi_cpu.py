@@ -61,6 +61,11 @@ def test_rule_table_known_answers():
     # 4096 x 4224: 272 big tiles would leave the second round 6 % full; 1056 of 128x128 are five per compute unit
     rc, p = _plan(_operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (4224, 4096)), _operand(capi.F32, (4096, 4224)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
+    # config 3's 3000 x 3000 x 17: one K tile, the output is the work - several small workgroups per compute unit
+    rc, p = _plan(_operand(capi.BF16, (3000, 17)), _operand(capi.BF16, (3000, 17)), _operand(capi.F32, (3000, 3000)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1
+    rc, p = _plan(_operand(capi.BF16, (8192, 512)), _operand(capi.BF16, (8192, 512)), _operand(capi.F32, (8192, 8192)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"      # from eight K tiles on the big tile is ahead again
     # one row against a long weight matrix: the skinny family, no workspace
     rc, p = _plan(_operand(capi.BF16, (1, 4096)), _operand(capi.BF16, (14336, 4096)), _operand(capi.BF16, (1, 14336)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "skinny" and p.workspace_bytes == 0

@@ -279,9 +279,18 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     family = VECOPS_HIP_FAMILY_TILE_128;
     tile_m = tile_n = 128;
   }
-  plan->family = family;
   const int64_t ktile = k_tile_elements(pr.src);
   const int64_t k_tiles = (pr.k + ktile - 1) / ktile;
+  // At most four K tiles of 16-bit or 8-bit operands: the tile's life is its start-up and its stores, and
+  // two or three 128x128 workgroups on a compute unit overlap one's stores with another's loads, which a
+  // single big tile cannot (batch 8 of 3000x3000x17 to fp32: 93 us against 111; 8 x 1000x1000x100: 17.7
+  // against 21.7; 4096x4096x256 to bf16: 17.9 against 20.2; level at 8192x8192x256, behind from K = 512).
+  if (k_tiles <= 4 && pr.src != SRC_F32 && family != VECOPS_HIP_FAMILY_TILE_64 && family != VECOPS_HIP_FAMILY_TILE_128 &&
+      pr.m > 64 && pr.n > 64 && tiles(128) >= kComputeUnits / 2) {
+    family = VECOPS_HIP_FAMILY_TILE_128;
+    tile_m = tile_n = 128;
+  }
+  plan->family = family;
   const int64_t wgs = tiles2(tile_m, tile_n);
   int64_t split = 1;
   if (wgs < kComputeUnits / 2 && k_tiles >= 8) {
