@@ -785,7 +785,11 @@ int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t ldx, const int8_t* 
   // GPU rule table of the skinny family: matrix cores once the widening of a weight
   // byte can be shared by three or more activation rows
   const bool mfma_ok = group % 64 == 0 && (group == 64 || group == 128 || group == 256);
-  if (m >= 2 && k == 4096 && (group == 128 || group == 256) && n >= 2048) {
+  if (m == 2 && k == 4096 && n >= 4096) {
+    // two rows of activations: the streaming walk of M = 1 with both rows resident (13.9 us at N = 14336 where
+    // the matrix-core kernel takes 17.0)
+    hipLaunchKernelGGL((skinny_w8a16_stream_rows_kernel<2, 4>), dim3(kComputeUnits * kStreamGroupsPerUnit), dim3(256), 0, s, p);
+  } else if (m >= 2 && k == 4096 && (group == 128 || group == 256) && n >= 2048) {
     // activations resident in registers; a workgroup walks two blocks of 32 rows (224 workgroups at
     // N = 14336).  More passes reuse the activations further but leave too few workgroups to pull
     // the bandwidth: 4 passes measured 50 % slower.

@@ -210,6 +210,100 @@ __global__ __launch_bounds__(256) void skinny_w8a16_stream_kernel(const SkinnyW8
   if (n < p.n) finish(0, n);
 }
 
+// ---- M = 2, streaming: the M = 1 walk over the weight rows with MT activation rows resident ----------
+// K = CH x 1024.  The activations of a lane's chunks, widened to fp32, take MT x CH x 16 registers, which
+// is what limits MT to 2 at two wavefronts per SIMD.  A weight byte is widened once (u = w + 128,
+// -128 * sum_k x per 16-element chunk, as in the M = 1 kernel) and multiplied into MT sums.  More rows run
+// into the vector ALU: at N = 14336 one row takes 12.2 us, two 13.9; four rows - K shared between two
+// wavefronts that meet in LDS - took 25 us, and v_dot2c_f32_bf16 on packed activations 19.7 (it issues at
+// a quarter of the rate), so three rows and more stay with the matrix-core kernels below.  The code the
+// compiler makes of this loop is touchy: with the wavefront's number in a vector register (row addresses
+// as vector arithmetic) two rows took 20.4 us, and with a trip count shared by all wavefronts (an eighth,
+// clamped row for each at N = 14336) 15.8.
+template <int MT, int CH>
+__global__ __launch_bounds__(256) void skinny_w8a16_stream_rows_kernel(const SkinnyW8A16Params p) {
+  const int lane = threadIdx.x & 63;
+  // (the wavefront's number in a scalar register: row addresses are then scalar arithmetic)
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t waves = static_cast<int64_t>(gridDim.x) * 4;
+  const VECOPS_GLOBAL char* wbase = (const VECOPS_GLOBAL char*)p.w;
+  const VECOPS_GLOBAL float* sbase = (const VECOPS_GLOBAL float*)p.scales;
+
+  float xf[MT][CH][16], xsum[MT][CH];
+  int group_of[CH];
+#pragma unroll
+  for (int u = 0; u < CH; ++u) {
+    const int k0 = (u * 64 + lane) << 4;
+    group_of[u] = k0 / p.group;
+#pragma unroll
+    for (int mm = 0; mm < MT; ++mm) {
+      const VECOPS_GLOBAL uint16_t* xrow = (const VECOPS_GLOBAL uint16_t*)p.x + static_cast<int64_t>(min(mm, p.m - 1)) * p.ldx;
+      const VECOPS_GLOBAL u32x4* px = (const VECOPS_GLOBAL u32x4*)(xrow + k0);
+      const u32x4 lo = px[0], hi = px[1];
+      const uint32_t words[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      float sum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        xf[mm][u][2 * e] = __uint_as_float(words[e] << 16);
+        xf[mm][u][2 * e + 1] = __uint_as_float(words[e] & 0xffff0000u);
+        sum += xf[mm][u][2 * e];
+        sum += xf[mm][u][2 * e + 1];
+      }
+      xsum[mm][u] = sum;
+    }
+  }
+
+  u32x4 wq[2][CH];
+  float sc[2][CH];
+  auto fetch = [&](int set, int64_t n) {
+    const int64_t row = n < p.n ? n : p.n - 1;  // rows past N are clamped: computed, never stored
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      wq[set][u] = *(const VECOPS_GLOBAL u32x4*)(wbase + row * p.ldw + (static_cast<int64_t>(u * 64 + lane) << 4));
+      sc[set][u] = sbase[row * p.groups + group_of[u]];
+    }
+  };
+  auto finish = [&](int set, int64_t n) {
+    float acc[MT];
+#pragma unroll
+    for (int mm = 0; mm < MT; ++mm) acc[mm] = 0.0f;
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      const uint32_t words[4] = {wq[set][u].x ^ 0x80808080u, wq[set][u].y ^ 0x80808080u, wq[set][u].z ^ 0x80808080u,
+                                 wq[set][u].w ^ 0x80808080u};
+      float part[MT];
+#pragma unroll
+      for (int mm = 0; mm < MT; ++mm) part[mm] = -128.0f * xsum[mm][u];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float wf = static_cast<float>((words[e >> 2] >> ((e & 3) * 8)) & 0xffu);
+#pragma unroll
+        for (int mm = 0; mm < MT; ++mm) part[mm] = fmaf(xf[mm][u][e], wf, part[mm]);
+      }
+#pragma unroll
+      for (int mm = 0; mm < MT; ++mm) acc[mm] = fmaf(sc[set][u], part[mm], acc[mm]);
+    }
+#pragma unroll
+    for (int mm = 0; mm < MT; ++mm) {
+      const float total = wave_sum(acc[mm]);
+      if (lane == 0 && mm < p.m && n < p.n)
+        p.y[static_cast<int64_t>(mm) * p.ldy + n] = static_cast<uint16_t>(bf16_bits_rne(total));
+    }
+  };
+
+  if (wave >= p.n) return;
+  fetch(0, wave);
+  int64_t n = wave;
+  // two rows per trip so that the register set of a row is a compile-time choice
+  for (; n + waves < p.n; n += 2 * waves) {
+    fetch(1, n + waves);
+    finish(0, n);
+    fetch(0, n + 2 * waves);
+    finish(1, n + waves);
+  }
+  if (n < p.n) finish(0, n);
+}
+
 // ---- matrix-core family: a workgroup owns TILES x 16 weight rows, its WAVES wavefronts
 // split K by scale groups --------------------------------------------------------------------
 // One v_mfma_f32_16x16x32_bf16 multiplies 16 weight rows x 32 k by 32 k x 16
