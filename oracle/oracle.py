@@ -100,6 +100,9 @@ class Oracle:
                                        C.c_float, C.c_float, C.c_int, C.c_float, C.c_float, C.c_int, C.c_void_p]
         for name in ("vo_amx_small_vector_profitable", "vo_sme_small_vector_profitable"):
             getattr(L, name).argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64]
+        L.vo_quantize_rows_u8.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_void_p,
+                                          C.c_int64]
+        L.vo_quantize_rows_u8.restype = None
         L.vo_small_area_profitable.argtypes = [C.c_int64] * 4
         L.vo_threads.restype = C.c_int
         L.vo_matmul_bf16_dense.argtypes = [C.c_void_p] * 4 + [C.c_int64] * 3
@@ -176,6 +179,16 @@ class Oracle:
                                       corr.ctypes.data if corr is not None else None, c.ctypes.data, a.shape[0],
                                       b.shape[0], a.shape[1])
         return c
+
+    def quantize_rows(self, a, multipliers, zero_point: int) -> np.ndarray:
+        """uint8 [M,K]: the per-row asymmetric quantisation of fp32 activations (vo_quantize_rows_u8)."""
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        mult = np.ascontiguousarray(multipliers, dtype=np.float32)
+        assert a.ndim == 2 and mult.shape == (a.shape[0],)
+        q = np.empty(a.shape, dtype=np.uint8)
+        self.lib.vo_quantize_rows_u8(a.ctypes.data, a.shape[0], a.shape[1], a.shape[1], mult.ctypes.data,
+                                     int(zero_point), q.ctypes.data, a.shape[1])
+        return q
 
     def fused_outputs(self, acc, out_dtype, *, activation=0, scale=None, shift=None, row_scales=None,
                       column_scales=None, lo=0.0, hi=0.0) -> np.ndarray:
@@ -301,6 +314,32 @@ class Reference:
         rc = self.lib.vref_matmul_bf16_f32_batched(
             C.c_void_p(a.ctypes.data), C.c_void_p(b.ctypes.data), C.c_void_p(c.ctypes.data), C.c_int64(batch),
             C.c_int64(m), C.c_int64(n), C.c_int64(k), _strides3(a), _strides3(b), _strides3(c))
+        if rc != 0:
+            raise RuntimeError("reference matmul unavailable")
+        return c
+
+    def matmul_runtime_quant(self, a, b, multipliers, zero_point, correction, row_scales=None, column_scales=None):
+        """fp32 a quantised on the way in (per-row multiplier, zero point) x int8 b + correction row;
+        int32 sums, or the dequantised fp32 when both scale vectors are given."""
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        b = np.ascontiguousarray(b, dtype=np.int8)
+        m, k = a.shape
+        n = b.shape[0]
+        mult = np.ascontiguousarray(multipliers, dtype=np.float32)
+        corr = np.ascontiguousarray(correction, dtype=np.int32)
+        if row_scales is not None:
+            rs = np.ascontiguousarray(row_scales, dtype=np.float32)
+            cs = np.zeros(n + 64, dtype=np.float32)  # unmasked vector load past n (Quantization.h:229-231)
+            cs[:n] = column_scales
+            c = np.empty((m, n), dtype=np.float32)
+            rs_ptr, cs_ptr = C.c_void_p(rs.ctypes.data), C.c_void_p(cs.ctypes.data)
+        else:
+            c = np.empty((m, n), dtype=np.int32)
+            rs_ptr, cs_ptr = None, None
+        rc = self.lib.vref_matmul_runtime_quant(
+            C.c_void_p(a.ctypes.data), C.c_void_p(b.ctypes.data), C.c_void_p(mult.ctypes.data), C.c_int32(zero_point),
+            rs_ptr, cs_ptr, C.c_void_p(corr.ctypes.data), C.c_void_p(c.ctypes.data), C.c_int64(m), C.c_int64(n),
+            C.c_int64(k))
         if rc != 0:
             raise RuntimeError("reference matmul unavailable")
         return c

@@ -230,6 +230,39 @@ VREF_EXPORT int vref_matmul_i8_dequant(const int8_t* a, const int8_t* b, const f
   return 0;
 }
 
+// fp32 activations quantised on their way in by RuntimePerRowAsymmetricQuantizeTransform
+// (matmul/Quantization.h:91-146: q = x * multipliers[row] + float(zero_point), converted to the
+// atom's uint8), int8 weights, the stride-0 int32 correction row as C input, and either the
+// plain int32 sums (row_scales == null: c is int32) or the per-row x per-column dequantisation
+// (c is fp32) - the pipeline of tests/ops/MatmulConversionTestCommon.h:1437-1540 with B unpacked.
+VREF_EXPORT int vref_matmul_runtime_quant(const float* a, const int8_t* b, const float* multipliers,
+                                          int32_t zero_point, const float* row_scales, const float* column_scales,
+                                          const int32_t* correction, void* c, int64_t m, int64_t n, int64_t k) {
+  if (!enable_amx()) return -1;
+  using Atom = matmul::AMX_I8I32<uint8_t, int8_t>;
+  auto at = view2(const_cast<float*>(a), m, k, k, 1);
+  auto bt = view2(const_cast<int8_t*>(b), n, k, k, 1);
+  auto cit = view2(const_cast<int32_t*>(correction), m, n, 0, 1);
+  auto quantize = matmul::make_runtime_per_row_asymmetric_quantize_transform({multipliers, &zero_point, 0});
+  auto ain = tensor::input<uint8_t>(at, quantize);
+  auto cin = tensor::input<int32_t>(cit);
+  auto op = ops::matmul(ops::MatmulConfig<Atom>{});
+  if (row_scales != nullptr) {
+    auto ct = view2(static_cast<float*>(c), m, n, n, 1);
+    auto deq = matmul::make_runtime_per_row_column_dequantize_transform({row_scales, column_scales, 0});
+    auto cout = tensor::output<int32_t>(ct, deq);
+    kernel::Workspace ws(op.required_workspace(Any{m}, Any{n}, Any{k}, ain, bt, cin, cout));
+    auto v = ws.view();
+    op(v, Any{m}, Any{n}, Any{k}, ain, bt, cin, cout);
+  } else {
+    auto ct = view2(static_cast<int32_t*>(c), m, n, n, 1);
+    kernel::Workspace ws(op.required_workspace(Any{m}, Any{n}, Any{k}, ain, bt, cin, ct));
+    auto v = ws.view();
+    op(v, Any{m}, Any{n}, Any{k}, ain, bt, cin, ct);
+  }
+  return 0;
+}
+
 // c_kind: 0 fp32, 1 bf16, 3 uint8, 4 int8 (the dtype codes of include/vecops_hip.h are not used here).
 VREF_EXPORT int vref_matmul_bf16_fused(const uint16_t* a, const uint16_t* b, const float* bias, void* c, int c_kind,
                                        int64_t m, int64_t n, int64_t k, const FusedSpec* spec) {

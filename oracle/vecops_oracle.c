@@ -340,6 +340,26 @@ VO_EXPORT int vo_fused_outputs(const void* acc, int acc_is_int, int64_t M, int64
   return 0;
 }
 
+/* RuntimePerRowAsymmetricQuantizeTransform (matmul/Quantization.h:91-146, formula :123-128) followed
+ * by the conversion of the transformed fp32 value to the atom's uint8 compute type:
+ *   q[r][k] = u8( a[r][k] * multipliers[r] + (float)zero_point )
+ * - a multiply and an add, each rounded to fp32 (two vector instructions, never fused), then the x86
+ * vector conversion cvtt_i32 above (truncation toward zero; NaN and values outside int32 give
+ * INT32_MIN) and a saturating narrow to 0..255.  Pinned by golden vectors of the real vecops build
+ * (tests/golden/vecops_quant_golden.npz): an edge-value table read back through an identity B, and
+ * elements built so that a fused multiply-add would give a different byte. */
+VO_EXPORT void vo_quantize_rows_u8(const float* a, int64_t M, int64_t K, int64_t lda, const float* multipliers,
+                                   int32_t zero_point, uint8_t* q, int64_t ldq) {
+  const float zp = (float)zero_point;
+  for (int64_t r = 0; r < M; ++r)
+    for (int64_t k = 0; k < K; ++k) {
+      volatile float prod = a[r * lda + k] * multipliers[r];
+      const float t = prod + zp;
+      const int32_t v = cvtt_i32(t);
+      q[r * ldq + k] = (uint8_t)(v < 0 ? 0 : v > 255 ? 255 : v);
+    }
+}
+
 /* Selected outputs of the rank-2 product only: out[s] = acc(rows_idx[s], cols_idx[s])
  * as double (floating atoms) - lets a test check a 4096^3 product in seconds. */
 VO_EXPORT int vo_matmul_sampled(const vo_tensor* a, const vo_tensor* b, int atom, const int64_t* rows_idx,

@@ -170,3 +170,62 @@ def make_fused_inputs(case: dict) -> dict:
                        if case.get("bias") else None)
     out["column_scales"] = synth.scales(14, n) if case.get("colscale") else None
     return out
+
+
+# --- runtime per-row asymmetric quantisation of fp32 activations (matmul/Quantization.h:91-146) ----------
+# fp32 values whose quantised bytes show every branch of the conversion: truncation toward zero on both
+# sides, saturation at 0 and 255, values outside int32, infinities, NaN, denormals.
+QUANT_EDGE_VALUES = [0.0, 0.4, 0.5, 0.99, 1.0, 1.5, 2.5, -0.4, -0.5, -0.99, -1.0, -1.5, -7.0, -7.5, -8.0, -100.0, 247.0,
+                     247.5, 248.0, 248.9, 249.0, 300.0, 1e6, 3e9, -3e9, 1e20, -1e20, float("inf"), float("-inf"),
+                     float("nan"), -0.0, 2147483520.0, -2147483648.0, 4294967040.0, 1e-40, 254.99, 255.0, 255.5, 256.0,
+                     127.5, 128.0]
+QUANT_EDGE_MULTIPLIERS = [1.0, 0.5, 3.0]
+QUANT_EDGE_ZERO_POINTS = [7, 0, -3]
+QUANT_CASES = [
+    {"name": "rq_19x21x69", "m": 19, "n": 21, "k": 69, "zp": 7},
+    {"name": "rq_67x129x515", "m": 67, "n": 129, "k": 515, "zp": 128},
+    {"name": "rq_130x70x1000_zp0", "m": 130, "n": 70, "k": 1000, "zp": 0},
+]
+
+
+def quant_edge_inputs():
+    """a [3,64] (each row the edge values, zero-padded), identity b [64,64]: the int32 sums are the bytes."""
+    import numpy as np
+    vals = np.array(QUANT_EDGE_VALUES, dtype=np.float32)
+    a = np.zeros((len(QUANT_EDGE_MULTIPLIERS), 64), np.float32)
+    a[:, :vals.size] = vals
+    return a, np.eye(64, dtype=np.int8), np.array(QUANT_EDGE_MULTIPLIERS, np.float32)
+
+
+def quant_fma_inputs():
+    """Elements whose product a * multiplier rounds up to 16.0 in fp32 while the exact product lies at
+    least 2^-23 below it: with zero point -15 two roundings give trunc(16 - 15) = 1, one fused rounding
+    trunc(1 - delta) = 0.  Returns (a [1,64], b identity, multipliers [1], zero_point)."""
+    import numpy as np
+    rng = np.random.default_rng(5)
+    found = []
+    while len(found) < 64:
+        x = rng.uniform(15.5, 16.5, 4096).astype(np.float32)
+        mlt = np.float32(rng.uniform(0.97, 1.03))
+        for xv in x:
+            exact = float(xv) * float(mlt)
+            if np.float32(xv) * mlt == np.float32(16.0) and exact < 16.0 - 2.0 ** -22:
+                found.append((xv, mlt))
+                break
+    # one multiplier per row: keep the elements that share the first multiplier, else one row per element
+    a = np.array([[f[0] for f in found]], np.float32).T.copy()        # [64,1] -> one element per row
+    mult = np.array([f[1] for f in found], np.float32)
+    return a, mult
+
+
+def make_quant_inputs(case):
+    import numpy as np
+    from vecops_amd import synth
+    m, n, k = case["m"], case["n"], case["k"]
+    mult = (np.float32(4.0) * (np.float32(1.0) + synth.uniform_pm1(11, (m,)) * np.float32(0.5))).astype(np.float32)
+    # activations spread over a little more than the byte range after quantisation, fractions included
+    a = ((synth.uniform_pm1(12, (m, k)) * np.float32(140.0) + np.float32(128 - case["zp"])) / mult[:, None]).astype(np.float32)
+    b = synth.int8_sym(13, (n, k))
+    correction = (-case["zp"] * b.astype(np.int64).sum(axis=1)).astype(np.int32)
+    return {"a": a, "b": b, "multipliers": mult, "correction": correction,
+            "row_scales": (np.float32(1.0) / mult).astype(np.float32), "column_scales": synth.scales(14, n)}

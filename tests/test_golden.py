@@ -1,6 +1,8 @@
 """The committed golden vectors (outputs of the real vecops CPU matmul, see
 tests/golden/make_golden.py) against the oracle (CPU) and against the gfx950
 kernels through the C ABI (GPU)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -86,3 +88,48 @@ def test_gpu_reproduces_golden(device, case):
         torch.cuda.synchronize()
         got = c.view(torch.int16).cpu().numpy().view(np.uint16) if out_dt == torch.bfloat16 else c.cpu().numpy()
     check(case, got)
+
+
+# --- runtime per-row asymmetric quantisation of fp32 activations -------------------------------------------------
+
+QUANT_GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vecops_quant_golden.npz")
+
+
+def test_quantize_rows_edge_values_match_the_reference(oracle):
+    """Every branch of the fp32 -> uint8 input conversion (truncation toward zero, saturation, NaN, infinities,
+    values outside int32) as the real vecops build produced it, read back through an identity B."""
+    from golden_cases import QUANT_EDGE_ZERO_POINTS, quant_edge_inputs
+    gold = np.load(QUANT_GOLDEN)
+    a, eye, mult = quant_edge_inputs()
+    for zp in QUANT_EDGE_ZERO_POINTS:
+        want = gold[f"edge_zp{zp}"]
+        assert want.min() >= 0 and want.max() == 255
+        assert np.array_equal(oracle.quantize_rows(a, mult, zp).astype(np.int32), want), zp
+
+
+def test_quantize_rows_rounds_twice_like_the_reference(oracle):
+    """Elements built so that one fused rounding of a * multiplier + zero_point gives byte 0 and two roundings
+    give byte 1: the reference gives 1 for every one of them, and so does the oracle."""
+    gold = np.load(QUANT_GOLDEN)
+    a, mult, want = gold["fma_a"], gold["fma_multipliers"], gold["fma_bytes"]
+    fused = np.trunc(a[:, 0].astype(np.float64) * mult.astype(np.float64) - 15.0)
+    assert (fused == 0).all() and (want == 1).all()
+    assert np.array_equal(oracle.quantize_rows(a, mult, -15).astype(np.int32), want)
+
+
+def test_runtime_quant_pipeline_matches_the_reference(oracle):
+    """quantise -> u8 x s8 sums + correction row -> per-row x per-column dequantisation, against the real build
+    (tests/ops/MatmulConversionTestCommon.h:1437-1540): int32 sums and fp32 outputs bit for bit."""
+    from golden_cases import QUANT_CASES, make_quant_inputs
+    from oracle import oracle as O
+    gold = np.load(QUANT_GOLDEN)
+    for case in QUANT_CASES:
+        inp = make_quant_inputs(case)
+        q = oracle.quantize_rows(inp["a"], inp["multipliers"], case["zp"])
+        assert q.min() == 0 and q.max() == 255                     # both ends of the byte range saturate
+        acc = np.zeros((case["m"], case["n"]), np.int32)
+        oracle.matmul(q, inp["b"], acc, cin=np.broadcast_to(inp["correction"], acc.shape), atom=O.ATOM_I8I32,
+                      acc_f64=True, c_bf16=False)
+        assert np.array_equal(acc, gold[case["name"] + "_i32"]), case["name"]
+        out = oracle.fused_outputs(acc, np.float32, row_scales=inp["row_scales"], column_scales=inp["column_scales"])
+        assert np.array_equal(out.view(np.uint32), gold[case["name"] + "_f32"].view(np.uint32)), case["name"]
