@@ -192,6 +192,36 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_i8_dequant(const int8_t* a, int64_t 
                                                        int64_t n, int64_t k, void* workspace, uint64_t workspace_size,
                                                        void* stream);
 
+/*
+ * q[..,r,k] = u8( x[..,r,k] * multipliers[row] + (float)zero_point ), row = batch * M + r:
+ * vecops' RuntimePerRowAsymmetricQuantizeTransform on an fp32 input read as the atom's uint8
+ * (matmul/Quantization.h:91-146, formula :123-128; tensor::input<uint8_t>(a, quantize) in
+ * tests/ops/MatmulConversionTestCommon.h:1503-1506).  The multiply and the add are rounded
+ * separately; the conversion truncates toward zero, sends NaN and values outside int32 to 0 and
+ * saturates at 0 and 255 (the x86 vector conversion, vec/details/x86/Conversion.h:522-528).  x is f32,
+ * q is u8 with the same extents (rank 2 or 3, any strides).  Bit-exact.
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_quantize_rows(const VecopsHipOperand* x, const float* multipliers,
+                                                   int32_t zero_point, const VecopsHipOperand* q, void* stream);
+
+/*
+ * The runtime-quantised product of tests/ops/MatmulConversionTestCommon.h:1437-1540 in one call:
+ *   q = quantize_rows(a);  acc = sum_k q[i,k] * b[j,k] + correction[j]  (AMX_I8I32<uint8_t, int8_t>, wrapping);
+ *   c[i,j] = (float(acc) * row_scales[i]) * column_scales[j].
+ * a f32 [M,K], b i8 [N,K], c f32 [M,N] (rank 2, any strides); correction (int32[N], usually
+ * -zero_point * sum_k b[j,k], see vecops_hip_pack_b_compensated) may be null.  The workspace holds the
+ * quantised activations and the product's own scratch: vecops_hip_matmul_runtime_quant_workspace bytes,
+ * 16-byte aligned.  Bit-exact.
+ */
+VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_runtime_quant_workspace(const VecopsHipOperand* a,
+                                                                     const VecopsHipOperand* b,
+                                                                     const VecopsHipOperand* c);
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* multipliers,
+                                                          int32_t zero_point, const VecopsHipOperand* b,
+                                                          const int32_t* correction, const float* row_scales,
+                                                          const float* column_scales, const VecopsHipOperand* c,
+                                                          void* workspace, uint64_t workspace_size, void* stream);
+
 /* Workspace bytes vecops_hip_matmul_i8_dequant needs for these extents. */
 VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int64_t n, int64_t k);
 

@@ -1,0 +1,112 @@
+"""fp32 activations quantised on the way in (vecops' RuntimePerRowAsymmetricQuantizeTransform,
+matmul/Quantization.h:91-146) through the C ABI: vecops_hip_quantize_rows and the one-call pipeline
+vecops_hip_matmul_runtime_quant (tests/ops/MatmulConversionTestCommon.h:1437-1540), bit for bit against the
+golden vectors of the real vecops build and against the oracle."""
+import os
+
+import numpy as np
+import pytest
+
+from golden_cases import (QUANT_CASES, QUANT_EDGE_ZERO_POINTS, make_quant_inputs, quant_edge_inputs)
+from oracle import oracle as O
+from vecops_amd import synth
+
+pytestmark = pytest.mark.gpu
+GOLD = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vecops_quant_golden.npz"))
+
+
+def dev(x, device):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x)).to(device)
+
+
+def test_quantize_rows_edge_values_and_double_rounding(device):
+    import torch
+    from vecops_amd import capi
+    a, _, mult = quant_edge_inputs()
+    for zp in QUANT_EDGE_ZERO_POINTS:
+        q = torch.full(a.shape, 99, dtype=torch.uint8, device=device)
+        capi.quantize_rows(dev(a, device), dev(mult, device), zp, q)
+        assert np.array_equal(q.cpu().numpy().astype(np.int32), GOLD[f"edge_zp{zp}"]), zp
+    fa, fm = GOLD["fma_a"], GOLD["fma_multipliers"]
+    q = torch.zeros(fa.shape, dtype=torch.uint8, device=device)
+    capi.quantize_rows(dev(fa, device), dev(fm, device), -15, q)
+    assert np.array_equal(q.cpu().numpy().astype(np.int32), GOLD["fma_bytes"])       # 1 everywhere; a fused rounding gives 0
+
+
+@pytest.mark.parametrize("batch,m,k", [(1, 19, 69), (1, 1, 1), (3, 37, 130), (1, 300, 4096), (2, 5, 3)])
+def test_quantize_rows_strided_and_batched(device, oracle, batch, m, k):
+    """Rank 2 and 3, row strides wider than K on both sides, K not a multiple of four, a transposed source."""
+    import torch
+    from vecops_amd import capi
+    mult = (np.float32(3.0) + synth.uniform_pm1(1, (batch * m,))).astype(np.float32)
+    x = (synth.uniform_pm1(2, (batch * m, k)) * np.float32(60.0)).astype(np.float32)
+    want = oracle.quantize_rows(x, mult, 100).reshape(batch, m, k)
+    store = torch.full((batch, m, k + 5), float("nan"), device=device)
+    store[:, :, :k] = dev(x.reshape(batch, m, k), device)
+    qstore = torch.full((batch, m, k + 3), 77, dtype=torch.uint8, device=device)
+    xv, qv = store[:, :, :k], qstore[:, :, :k]
+    if batch == 1:
+        xv, qv = xv[0], qv[0]
+    capi.quantize_rows(xv, dev(mult, device), 100, qv)
+    assert np.array_equal(qstore[:, :, :k].cpu().numpy(), want)
+    assert (qstore[:, :, k:] == 77).all()
+    if batch == 1:                                                   # source stored [K,M]
+        xt = dev(np.ascontiguousarray(x.T), device).t()
+        q2 = torch.zeros((m, k), dtype=torch.uint8, device=device)
+        capi.quantize_rows(xt, dev(mult, device), 100, q2)
+        assert np.array_equal(q2.cpu().numpy(), want[0])
+
+
+@pytest.mark.parametrize("case", QUANT_CASES, ids=lambda c: c["name"])
+def test_runtime_quant_pipeline_golden(device, case):
+    import torch
+    from vecops_amd import capi
+    inp = make_quant_inputs(case)
+    c = torch.full((case["m"], case["n"]), float("nan"), device=device)
+    capi.matmul_runtime_quant(dev(inp["a"], device), dev(inp["multipliers"], device), case["zp"], dev(inp["b"], device),
+                              dev(inp["row_scales"], device), dev(inp["column_scales"], device), c,
+                              correction=dev(inp["correction"], device))
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), GOLD[case["name"] + "_f32"].view(np.uint32))
+
+
+@pytest.mark.parametrize("m,n,k", [(2048, 1100, 4096), (1, 300, 512), (16, 4096, 4096), (255, 63, 8191)])
+def test_runtime_quant_pipeline_against_the_oracle(device, oracle, m, n, k):
+    """Tile, split-K and narrow shapes; B given [K,N]; no correction row."""
+    import torch
+    from vecops_amd import capi
+    mult = (np.float32(2.0) + synth.uniform_pm1(1, (m,))).astype(np.float32)
+    a = ((synth.uniform_pm1(2, (m, k)) * np.float32(140.0) + np.float32(120.0)) / mult[:, None]).astype(np.float32)
+    b = synth.int8_sym(3, (n, k))
+    rs, cs = (np.float32(1.0) / mult).astype(np.float32), synth.scales(4, n)
+    q = oracle.quantize_rows(a, mult, 8)
+    acc = np.zeros((m, n), np.int32)
+    oracle.matmul(q, b, acc, atom=O.ATOM_I8I32, acc_f64=True, c_bf16=False)
+    want = oracle.fused_outputs(acc, np.float32, row_scales=rs, column_scales=cs)
+    bt = dev(np.ascontiguousarray(b.T), device).t()                  # [N,K] view of a [K,N] array
+    c = torch.full((m, n), float("nan"), device=device)
+    capi.matmul_runtime_quant(dev(a, device), dev(mult, device), 8, bt, dev(rs, device), dev(cs, device), c)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_runtime_quant_zero_extents_and_rejections(device):
+    import torch
+    from vecops_amd import capi
+    one = torch.ones(4, device=device)
+    c = torch.full((4, 6), float("nan"), device=device)
+    corr = torch.arange(6, dtype=torch.int32, device=device)
+    capi.matmul_runtime_quant(torch.empty((4, 0), device=device), one, 3, torch.empty((6, 0), dtype=torch.int8, device=device),
+                              one, torch.ones(6, device=device), c, correction=corr)
+    torch.cuda.synchronize()
+    assert torch.equal(c, corr.float().expand(4, 6))                  # K == 0: the correction row, dequantised
+    capi.matmul_runtime_quant(torch.empty((0, 8), device=device), one, 3, torch.zeros((6, 8), dtype=torch.int8, device=device),
+                              one, torch.ones(6, device=device), torch.empty((0, 6), device=device))
+    with pytest.raises(capi.VecopsHipError) as e:                     # bf16 activations are not this entry's business
+        capi.matmul_runtime_quant(torch.zeros((4, 8), dtype=torch.bfloat16, device=device), one, 3,
+                                  torch.zeros((6, 8), dtype=torch.int8, device=device), one, torch.ones(6, device=device), c)
+    assert e.value.code == 2
+    with pytest.raises(capi.VecopsHipError) as e:
+        capi.quantize_rows(torch.zeros((4, 8), device=device), one, 3, torch.zeros((4, 9), dtype=torch.uint8, device=device))
+    assert e.value.code == 1

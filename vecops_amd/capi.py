@@ -24,7 +24,8 @@ EXPORTS = [
     "vecops_hip_matmul", "vecops_hip_matmul_i8_dequant", "vecops_hip_matmul_i8_dequant_workspace",
     "vecops_hip_matmul_w8a16_group", "vecops_hip_packed_b_bytes", "vecops_hip_pack_b", "vecops_hip_pack_b_compensated",
     "vecops_hip_plan_matmul_packed_b", "vecops_hip_matmul_packed_b", "vecops_hip_matmul_i8_dequant_packed_b",
-    "vecops_hip_plan_matmul_fused", "vecops_hip_matmul_fused",
+    "vecops_hip_plan_matmul_fused", "vecops_hip_matmul_fused", "vecops_hip_quantize_rows",
+    "vecops_hip_matmul_runtime_quant_workspace", "vecops_hip_matmul_runtime_quant",
 ]
 
 ACT_NONE, ACT_RELU, ACT_CLAMP, ACT_SIGMOID, ACT_SILU = 0, 1, 2, 3, 4
@@ -90,6 +91,11 @@ def lib() -> C.CDLL:
                                                             C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                                             C.c_int64, C.c_void_p, C.c_uint64, C.c_void_p]
         E = C.POINTER(Epilogue)
+        L.vecops_hip_quantize_rows.argtypes = [P, C.c_void_p, C.c_int32, P, C.c_void_p]
+        L.vecops_hip_matmul_runtime_quant_workspace.restype = C.c_uint64
+        L.vecops_hip_matmul_runtime_quant_workspace.argtypes = [P, P, P]
+        L.vecops_hip_matmul_runtime_quant.argtypes = [P, C.c_void_p, C.c_int32, P, C.c_void_p, C.c_void_p, C.c_void_p, P,
+                                                      C.c_void_p, C.c_uint64, C.c_void_p]
         L.vecops_hip_plan_matmul_fused.argtypes = [P, P, P, P, C.c_uint32, E, C.POINTER(Plan)]
         L.vecops_hip_matmul_fused.argtypes = [P, P, P, P, C.c_uint32, E, C.c_void_p, C.c_uint64, C.c_void_p]
         _lib = L
@@ -210,6 +216,31 @@ def matmul_i8_dequant(a, b, row_scales, column_scales, c, correction=None, works
         a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), row_scales.data_ptr(), column_scales.data_ptr(),
         correction.data_ptr() if correction is not None else None, c.data_ptr(), c.stride(0), m, n, k, ws_ptr,
         ws_size, _stream_handle(stream)))
+    return c
+
+
+def quantize_rows(x, multipliers, zero_point: int, q, stream=None):
+    """q = u8(x * multipliers[row] + zero_point): vecops' per-row asymmetric quantisation of fp32 activations."""
+    ox, oq = operand(x), operand(q)
+    _check(lib().vecops_hip_quantize_rows(C.byref(ox), multipliers.data_ptr(), int(zero_point), C.byref(oq),
+                                          _stream_handle(stream)))
+    return q
+
+
+def matmul_runtime_quant(a, multipliers, zero_point: int, b, row_scales, column_scales, c, correction=None,
+                         workspace=None, stream=None):
+    """c = dequantise(quantise(a) . b^T + correction): fp32 a quantised on the way in, int8 b, fp32 c."""
+    import torch
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    need = lib().vecops_hip_matmul_runtime_quant_workspace(C.byref(oa), C.byref(ob), C.byref(oc))
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=c.device)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_runtime_quant(
+        C.byref(oa), multipliers.data_ptr(), int(zero_point), C.byref(ob),
+        correction.data_ptr() if correction is not None else None, row_scales.data_ptr(), column_scales.data_ptr(),
+        C.byref(oc), ws_ptr, ws_size, _stream_handle(stream)))
     return c
 
 

@@ -651,6 +651,88 @@ int32_t vecops_hip_matmul_i8_dequant_packed_b(const int8_t* a, int64_t lda, cons
                      static_cast<hipStream_t>(stream));
 }
 
+int32_t vecops_hip_quantize_rows(const VecopsHipOperand* x, const float* multipliers, int32_t zero_point,
+                                 const VecopsHipOperand* q, void* stream) {
+  View vx, vq;
+  if (!normalise(x, &vx) || !normalise(q, &vq)) return fail(ST_INVALID, "quantize_rows: operands must be rank 2 or 3");
+  if (vx.dtype != DT_F32 || vq.dtype != DT_U8) return fail(ST_NOT_APPLICABLE, "quantize_rows: x must be f32 and q u8");
+  if (x->rank != q->rank || vx.batch != vq.batch || vx.rows != vq.rows || vx.cols != vq.cols)
+    return fail(ST_INVALID, "quantize_rows: x and q differ in shape");
+  if (vx.batch == 0 || vx.rows == 0 || vx.cols == 0) return ST_OK;
+  if (vx.data == nullptr || vq.data == nullptr || multipliers == nullptr) return fail(ST_INVALID, "quantize_rows: null operand");
+  if (vx.batch * vx.rows > INT32_MAX || vx.rows > INT32_MAX || vx.cols > INT32_MAX)
+    return fail(ST_INVALID, "quantize_rows: extent too large");
+  hipError_t e = launch_quantize_rows(static_cast<const float*>(vx.data), static_cast<int32_t>(vx.batch),
+                                      static_cast<int32_t>(vx.rows), static_cast<int32_t>(vx.cols), vx.bs, vx.rs, vx.cs,
+                                      multipliers, zero_point, static_cast<uint8_t*>(vq.data), vq.bs, vq.rs, vq.cs,
+                                      static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(ST_EXEC, "quantize kernel launch: %s", hipGetErrorString(e));
+  return ST_OK;
+}
+
+namespace {
+// The pieces of vecops_hip_matmul_runtime_quant: the quantised activations sit at the head of the workspace
+// (M x K bytes rounded up to 256), the product's own workspace behind them.
+struct RuntimeQuant {
+  VecopsHipOperand q, cin;
+  VecopsHipEpilogue ep;
+  Problem pr;
+  VecopsHipPlan plan;
+  uint64_t q_bytes;
+};
+
+int32_t describe_runtime_quant(const VecopsHipOperand* a, const VecopsHipOperand* b, const int32_t* correction,
+                               const float* row_scales, const float* column_scales, const VecopsHipOperand* c,
+                               void* workspace, RuntimeQuant* d) {
+  if (a == nullptr || a->rank != 2 || a->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: a must be a rank-2 f32 operand");
+  if (b == nullptr || b->rank != 2 || b->dtype != DT_I8) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: b must be a rank-2 i8 operand");
+  if (c == nullptr || c->rank != 2 || c->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: c must be a rank-2 f32 operand");
+  if (a->sizes[0] < 0 || a->sizes[1] < 0) return fail(ST_INVALID, "matmul_runtime_quant: negative extent");
+  const int64_t m = a->sizes[0], k = a->sizes[1];
+  d->q_bytes = (static_cast<uint64_t>(m) * static_cast<uint64_t>(k) + 255u) & ~uint64_t{255};
+  make_operand(&d->q, workspace, DT_U8, m, k, k);
+  if (correction != nullptr) {
+    make_operand(&d->cin, correction, DT_I32, m, c->sizes[1], 0);  // one row for every row of c
+  }
+  memset(&d->ep, 0, sizeof(d->ep));
+  d->ep.struct_size = sizeof(d->ep);
+  d->ep.row_scales = row_scales;
+  d->ep.column_scales = column_scales;
+  int32_t rc = describe(&d->q, b, correction ? &d->cin : nullptr, c, 0, &d->pr, &d->ep);
+  if (rc != ST_OK) return rc;
+  choose(d->pr, &d->plan);
+  return ST_OK;
+}
+}  // namespace
+
+uint64_t vecops_hip_matmul_runtime_quant_workspace(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                   const VecopsHipOperand* c) {
+  RuntimeQuant d;
+  static const float one = 1.0f;
+  if (describe_runtime_quant(a, b, nullptr, &one, &one, c, reinterpret_cast<void*>(256), &d) != ST_OK) return 0;
+  return d.q_bytes + d.plan.workspace_bytes;
+}
+
+int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* multipliers, int32_t zero_point,
+                                        const VecopsHipOperand* b, const int32_t* correction, const float* row_scales,
+                                        const float* column_scales, const VecopsHipOperand* c, void* workspace,
+                                        uint64_t workspace_size, void* stream) {
+  RuntimeQuant d;
+  int32_t rc = describe_runtime_quant(a, b, correction, row_scales, column_scales, c,
+                                      workspace ? workspace : reinterpret_cast<void*>(256), &d);
+  if (rc != ST_OK) return rc;
+  if (d.plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
+  if (row_scales == nullptr || column_scales == nullptr || multipliers == nullptr)
+    return fail(ST_INVALID, "matmul_runtime_quant: multipliers and both scale vectors are required");
+  if (d.q_bytes + d.plan.workspace_bytes > workspace_size || (d.q_bytes > 0 && (workspace == nullptr || !aligned16(workspace))))
+    return fail(ST_INVALID, "matmul_runtime_quant: %llu bytes of 16-byte aligned workspace required, %llu supplied",
+                (unsigned long long)(d.q_bytes + d.plan.workspace_bytes), (unsigned long long)workspace_size);
+  rc = vecops_hip_quantize_rows(a, multipliers, zero_point, &d.q, stream);
+  if (rc != ST_OK) return rc;
+  return run_problem(d.pr, d.plan, nullptr, nullptr, nullptr, static_cast<char*>(workspace) + d.q_bytes,
+                     workspace_size - d.q_bytes, static_cast<hipStream_t>(stream));
+}
+
 uint32_t vecops_hip_abi_version(void) { return VECOPS_HIP_ABI_VERSION; }
 
 const char* vecops_hip_last_error(void) { return g_error; }
