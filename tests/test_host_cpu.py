@@ -96,7 +96,7 @@ def test_abi_layout(tmp_path):
 
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
-    assert len(files) == 34
+    assert len(files) == 36
     for f in files:
         name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
         assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
@@ -269,6 +269,28 @@ def test_packed_b_operators_resolution_and_validation(host):
     with pytest.raises(H.HostError) as e:
         mul.workspace(H.Frame([bf16((4, 8)), np.zeros(16, np.uint8), None, c], outputs=(3,)))
     assert e.value.code == 1 and "bytes" in e.value.message
+
+
+def test_runtime_quant_operator_resolution_and_validation(host):
+    """vecops::matmul_runtime_quant: eight positional values, the zero point a scalar in the middle."""
+    op = host.operator("vecops::matmul_runtime_quant")
+    a, b, c = np.zeros((4, 8), np.float32), np.zeros((5, 8), np.int8), np.zeros((4, 5), np.float32)
+    m4, n5 = np.ones(4, np.float32), np.ones(5, np.float32)
+    fr = lambda *v: H.Frame(list(v), outputs=(7,))  # noqa: E731
+    assert op.resolve(fr(a, b, m4, 7, m4, n5, None, c)) == \
+        "vecops::matmul_runtime_quant;operands=f32_i8;epilogue=row_col_dequant;memory=host;backend=hip-gfx950"
+    assert op.resolve(fr(a, b, m4, 7, m4, n5, np.zeros(5, np.int32), c)).startswith("vecops::matmul_runtime_quant;")
+    for frame, needle in [(fr(a, b, np.ones(3, np.float32), 7, m4, n5, None, c), "multipliers"),
+                          (fr(a, b, m4, 7, m4, np.ones(6, np.float32), None, c), "column_scales"),
+                          (fr(a, b, m4, 7, m4, n5, np.zeros(4, np.int32), c), "correction"),
+                          (fr(a, b, m4, 7.5, m4, n5, None, c), "zero_point"),
+                          (fr(a, np.zeros((5, 9), np.int8), m4, 7, m4, n5, None, c), "K")]:
+        with pytest.raises(H.HostError) as e:
+            op.resolve(frame)
+        assert e.value.code == 1 and needle in e.value.message, (needle, e.value.message)
+    with pytest.raises(H.HostError) as e:                  # activations that are already bytes go to vecops::matmul_fused
+        op.resolve(fr(np.zeros((4, 8), np.uint8), b, m4, 7, m4, n5, None, c))
+    assert e.value.code in (1, 2, 3)
 
 
 def test_provider_without_artifacts_reports_not_found(host, tmp_path):

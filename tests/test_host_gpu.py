@@ -262,6 +262,38 @@ def test_packed_b_operators(host, oracle, device):
     assert e.value.code == 1
 
 
+def test_matmul_runtime_quant_operator(host, device):
+    """vecops::matmul_runtime_quant through the Operator, host tensors (staged) and device tensors (in place, with
+    the workspace the artifact asks for): the golden case of the real vecops build, bit for bit."""
+    import torch
+    from golden_cases import QUANT_CASES, make_quant_inputs
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vecops_quant_golden.npz"))
+    op = host.operator("vecops::matmul_runtime_quant")
+    case = QUANT_CASES[1]
+    inp = make_quant_inputs(case)
+    want = gold[case["name"] + "_f32"]
+    c = np.full((case["m"], case["n"]), np.nan, np.float32)
+    frame = H.Frame([inp["a"], inp["b"], inp["multipliers"], case["zp"], inp["row_scales"], inp["column_scales"],
+                     inp["correction"], c], outputs=(7,))
+    assert "memory=host" in op.resolve(frame)
+    op.invoke(frame)
+    assert np.array_equal(c.view(np.uint32), want.view(np.uint32))
+    to = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(device)  # noqa: E731
+    tc = torch.full((case["m"], case["n"]), float("nan"), device=device)
+    frame = H.Frame([to(inp["a"]), to(inp["b"]), to(inp["multipliers"]), case["zp"], to(inp["row_scales"]),
+                     to(inp["column_scales"]), to(inp["correction"]), tc], outputs=(7,))
+    assert "memory=device" in op.resolve(frame)
+    need = op.workspace(frame)
+    assert need >= case["m"] * case["k"]                                      # the quantised activations live there
+    ws = torch.empty(need, dtype=torch.uint8, device=device)
+    op.invoke(frame, workspace=ws.data_ptr(), workspace_size=need)
+    torch.cuda.synchronize()
+    assert np.array_equal(tc.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    with pytest.raises(H.HostError) as e:                                      # too little workspace is an error, not a fault
+        op.invoke(frame, workspace=ws.data_ptr(), workspace_size=16)
+    assert e.value.code == 1
+
+
 def test_matmul_w8a16_group_operator(host, oracle, device):
     import torch
     op = host.operator("vecops::matmul_w8a16_group")

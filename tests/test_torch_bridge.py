@@ -32,7 +32,7 @@ def test_registration_is_idempotent_and_schemas_mark_outputs():
         tb.no_such_library
     ns = tb.register_all("vecops_hip_t")
     assert sorted(vars(ns)) == ["matmul", "matmul_fused", "matmul_i8_dequant", "matmul_pack_b", "matmul_packed_b",
-                                "matmul_w8a16_group"]
+                                "matmul_runtime_quant", "matmul_w8a16_group"]
     pack = str(torch.ops.vecops_hip_t.matmul_pack_b.default._schema)
     assert "int a_zero_point" in pack and "Tensor(a!) packed" in pack and "Tensor(b!)? compensation" in pack
     schema = str(torch.ops.vecops_hip_t.matmul.default._schema)
@@ -140,6 +140,23 @@ def test_torch_ops_quantised_operators(device, oracle):
     bits, exact = oracle.matmul_w8a16_group(x, w, s, 64)
     got = synth.bf16_to_f32(yb.view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
     assert np.abs(got - exact).max() <= 2 ** -7 * np.abs(exact).max()
+
+
+@pytest.mark.gpu
+def test_torch_ops_runtime_quant(device, oracle):
+    ns = tb.register_all("vecops_hip_t")
+    to = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(device)  # noqa: E731
+    m, n, k = 70, 130, 260
+    mult = (np.float32(2.0) + synth.uniform_pm1(1, (m,))).astype(np.float32)
+    a = ((synth.uniform_pm1(2, (m, k)) * np.float32(140.0) + np.float32(120.0)) / mult[:, None]).astype(np.float32)
+    b = synth.int8_sym(3, (n, k))
+    rs, cs = (np.float32(1.0) / mult).astype(np.float32), synth.scales(4, n)
+    corr = (-9 * b.astype(np.int64).sum(axis=1)).astype(np.int32)
+    acc = oracle.quantize_rows(a, mult, 9).astype(np.int64) @ b.astype(np.int64).T + corr
+    want = oracle.fused_outputs(acc.astype(np.int32), np.float32, row_scales=rs, column_scales=cs)
+    c = torch.zeros(m, n, device=device)
+    assert ns.matmul_runtime_quant(to(a), to(b), to(mult), 9, to(rs), to(cs), to(corr), c) is c
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
 @pytest.mark.gpu

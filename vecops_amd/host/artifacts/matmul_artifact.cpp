@@ -4,7 +4,7 @@
 //   -DVECOPS_ARTIFACT_KIND=<0..8>   0 matmul bf16, 1 matmul f32 (bf16 compute), 5 matmul f32 (fp32 compute), 2 matmul i8,
 //                                   3 matmul_i8_dequant, 4 matmul_w8a16_group, 6 / 7 / 8 / 10 matmul_fused for bf16 /
 //                                   f32 / i8 / f16 operands, 9 matmul f16, 11 / 12 matmul_pack_b to bf16 / i8,
-//                                   13 / 14 / 15 matmul_packed_b for bf16 / f32 / i8 a
+//                                   13 / 14 / 15 matmul_packed_b for bf16 / f32 / i8 a, 16 matmul_runtime_quant
 //   -DVECOPS_ARTIFACT_DEVICE=<0|1>  0: tensors are host memory, staged through HBM here
 //                                   1: tensors are HIP device pointers, used in place
 //   -DVECOPS_ARTIFACT_GROUP=<G>     group size of kind 4
@@ -798,6 +798,109 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
 #endif
   rc = vecops_hip_matmul_packed_b(&d.oa, packed_dev, kPackedDtype, d.n, d.cin ? &d.ocin : nullptr, &d.oc, ws, ws_size,
                                   stream);
+  if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
+  return finish(&staging, stream, error);
+}
+
+// =================================================================================================
+#elif VECOPS_ARTIFACT_KIND == 16  // vecops::matmul_runtime_quant (a, b, multipliers, zero_point, row_scales, column_scales, correction?, c)
+// =================================================================================================
+
+constexpr const char* kOperatorName = "vecops::matmul_runtime_quant";
+constexpr const char* kKey =
+  "vecops::matmul_runtime_quant;operands=f32_i8;epilogue=row_col_dequant;memory=" MEMORY_NAME ";backend=hip-gfx950";
+
+#define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
+   {.tensor = {sizeof(VecopsTensorParameter), MASK, kDeviceType, -1, RANK, OPTIONAL,                          \
+               sizeof(VecopsDimensionConstraint), nullptr, nullptr, FLAGS}}}
+
+const VecopsParameterDescriptor kParameters[] = {
+  TENSOR_PARAM("a", bit(VECOPS_DTYPE_F32), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("b", bit(VECOPS_DTYPE_I8), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("multipliers", bit(VECOPS_DTYPE_F32), -1, 0, VECOPS_TENSOR_READ),
+  {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_SCALAR, "zero_point",
+   {.scalar = {sizeof(VecopsScalarParameter), bit(VECOPS_DTYPE_I64) | bit(VECOPS_DTYPE_I32)}}},
+  TENSOR_PARAM("row_scales", bit(VECOPS_DTYPE_F32), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("column_scales", bit(VECOPS_DTYPE_F32), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("correction", bit(VECOPS_DTYPE_I32), -1, 1, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("c", bit(VECOPS_DTYPE_F32), -1, 0, VECOPS_TENSOR_WRITE),
+};
+
+struct QuantArgs {
+  const VecopsTensorView *a, *b, *mult, *rs, *cs, *corr, *c;
+  VecopsHipOperand oa, ob, oc;
+  int32_t zero_point;
+};
+
+int32_t decode(const VecopsCall* call, QuantArgs* d, VecopsError* error) {
+  if (int32_t rc = check_call(call, 8, error); rc != VECOPS_STATUS_OK) return rc;
+  d->a = tensor_arg(call, 0);
+  d->b = tensor_arg(call, 1);
+  d->mult = tensor_arg(call, 2);
+  d->rs = tensor_arg(call, 4);
+  d->cs = tensor_arg(call, 5);
+  d->corr = tensor_arg(call, 6);
+  d->c = tensor_arg(call, 7);
+  if (!d->a || !d->b || !d->mult || !d->rs || !d->cs || !d->c || call->values[3].kind != VECOPS_VALUE_SCALAR)
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT,
+                  "a, b, multipliers, row_scales, column_scales and c must be tensors, zero_point a scalar");
+  if (d->a->rank != 2 || d->b->rank != 2 || d->c->rank != 2 || d->mult->rank != 1 || d->rs->rank != 1 ||
+      d->cs->rank != 1 || (d->corr && d->corr->rank != 1))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "matmul_runtime_quant takes rank-2 matrices and rank-1 vectors");
+  const int64_t m = d->a->sizes[0], k = d->a->sizes[1], n = d->b->sizes[0];
+  if (d->b->sizes[1] != k || d->c->sizes[0] != m || d->c->sizes[1] != n || d->mult->sizes[0] != m ||
+      d->rs->sizes[0] != m || d->cs->sizes[0] != n || (d->corr && d->corr->sizes[0] != n))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "matmul_runtime_quant: extents disagree");
+  auto unit = [](const VecopsTensorView* t) { return t->sizes[0] <= 1 || t->strides[0] == 1; };
+  if (!unit(d->mult) || !unit(d->rs) || !unit(d->cs) || (d->corr && !unit(d->corr)))
+    return report(error, VECOPS_STATUS_NOT_APPLICABLE, "matmul_runtime_quant: the vectors must be contiguous");
+  d->zero_point = static_cast<int32_t>(call->values[3].value.scalar.value.i64);
+  void* const probe = reinterpret_cast<void*>(16);
+  if (!fill_operand(d->a, probe, &d->oa) || !fill_operand(d->b, probe, &d->ob) || !fill_operand(d->c, probe, &d->oc))
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "tensors must have rank 2");
+  return VECOPS_STATUS_OK;
+}
+
+int32_t workspace_impl(const VecopsCall* call, uint64_t* bytes, VecopsError* error) {
+  QuantArgs d;
+  if (int32_t rc = decode(call, &d, error); rc != VECOPS_STATUS_OK) return rc;
+#if VECOPS_ARTIFACT_DEVICE
+  *bytes = vecops_hip_matmul_runtime_quant_workspace(&d.oa, &d.ob, &d.oc);
+#else
+  *bytes = 0;
+#endif
+  return VECOPS_STATUS_OK;
+}
+
+int32_t run_impl(const VecopsCall* call, VecopsError* error) {
+  QuantArgs d;
+  if (int32_t rc = decode(call, &d, error); rc != VECOPS_STATUS_OK) return rc;
+  if (d.a->sizes[0] == 0 || d.b->sizes[0] == 0) return VECOPS_STATUS_OK;
+  hipStream_t stream = stream_of(call);
+  Staging staging(stream);
+  void *mult = nullptr, *rs = nullptr, *cs = nullptr, *corr = nullptr, *dev = nullptr;
+  int32_t rc;
+  if ((rc = device_address(d.c, true, &staging, &dev, error)) != VECOPS_STATUS_OK) return rc;
+  d.oc.data = dev;
+  if ((rc = device_address(d.a, false, &staging, &dev, error)) != VECOPS_STATUS_OK) return rc;
+  d.oa.data = dev;
+  if ((rc = device_address(d.b, false, &staging, &dev, error)) != VECOPS_STATUS_OK) return rc;
+  d.ob.data = dev;
+  if ((rc = device_address(d.mult, false, &staging, &mult, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(d.rs, false, &staging, &rs, error)) != VECOPS_STATUS_OK) return rc;
+  if ((rc = device_address(d.cs, false, &staging, &cs, error)) != VECOPS_STATUS_OK) return rc;
+  if (d.corr && (rc = device_address(d.corr, false, &staging, &corr, error)) != VECOPS_STATUS_OK) return rc;
+  void* ws = call->workspace;
+  uint64_t ws_size = call->workspace_size;
+#if !VECOPS_ARTIFACT_DEVICE
+  ws_size = vecops_hip_matmul_runtime_quant_workspace(&d.oa, &d.ob, &d.oc);
+  if (hipError_t e = staging.workspace(ws_size, &ws); e != hipSuccess)
+    return report_hip(error, "allocating the quantised activations", e);
+#endif
+  rc = vecops_hip_matmul_runtime_quant(&d.oa, static_cast<const float*>(mult), d.zero_point, &d.ob,
+                                       static_cast<const int32_t*>(corr), static_cast<const float*>(rs),
+                                       static_cast<const float*>(cs), &d.oc, ws, ws_size, stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
   return finish(&staging, stream, error);
 }

@@ -136,6 +136,27 @@ Status packed_b_relations(std::span<const Value> v) {
   return Status::success();
 }
 
+// vecops::matmul_runtime_quant (a, b, multipliers, zero_point, row_scales, column_scales, correction?, c)
+Status runtime_quant_relations(std::span<const Value> v) {
+  const TensorView* a = tensor_at(v, 0);
+  const TensorView* b = tensor_at(v, 1);
+  const TensorView* mult = tensor_at(v, 2);
+  const TensorView* rs = tensor_at(v, 4);
+  const TensorView* cs = tensor_at(v, 5);
+  const TensorView* corr = tensor_at(v, 6);
+  const TensorView* c = tensor_at(v, 7);
+  if (!a || !b || !mult || !rs || !cs || !c)
+    return invalid("vecops::matmul_runtime_quant needs a, b, multipliers, both scale vectors and c");
+  if (v.size() < 4 || std::get_if<rt::Scalar>(&v[3]) == nullptr) return invalid("zero_point must be a scalar");
+  if (a->sizes[1] != b->sizes[1]) return invalid("a and b disagree on K");
+  if (c->sizes[0] != a->sizes[0] || c->sizes[1] != b->sizes[0]) return invalid("c must be [M, N]");
+  if (mult->sizes[0] != a->sizes[0]) return invalid("multipliers must have M entries");
+  if (rs->sizes[0] != a->sizes[0]) return invalid("row_scales must have M entries");
+  if (cs->sizes[0] != b->sizes[0]) return invalid("column_scales must have N entries");
+  if (corr && corr->sizes[0] != b->sizes[0]) return invalid("correction must have N entries");
+  return Status::success();
+}
+
 // Placement of a call: all tensors on the host, or all on the device.
 rt::Result<Placement> placement_of(const rt::KernelCall& call) {
   bool host = false, device = false;
@@ -260,6 +281,20 @@ rt::OperatorSchema make_matmul_packed_b_schema() {
   params.push_back(tensor_param("c_in", out, std::nullopt, VECOPS_TENSOR_READ, /*optional=*/true));
   params.push_back(tensor_param("c", out, std::nullopt, VECOPS_TENSOR_WRITE));
   return rt::OperatorSchema(kMatmulPackedBName, std::move(params), packed_b_relations);
+}
+
+rt::OperatorSchema make_matmul_runtime_quant_schema() {
+  using rt::dtype_bit;
+  std::vector<rt::ParameterSchema> params;
+  params.push_back(tensor_param("a", dtype_bit(DType::Float32), 2u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("b", dtype_bit(DType::Int8), 2u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("multipliers", dtype_bit(DType::Float32), 1u, VECOPS_TENSOR_READ));
+  params.push_back(rt::ParameterSchema{"zero_point", rt::ScalarConstraint{dtype_bit(DType::Int64) | dtype_bit(DType::Int32)}});
+  params.push_back(tensor_param("row_scales", dtype_bit(DType::Float32), 1u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("column_scales", dtype_bit(DType::Float32), 1u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("correction", dtype_bit(DType::Int32), 1u, VECOPS_TENSOR_READ, /*optional=*/true));
+  params.push_back(tensor_param("c", dtype_bit(DType::Float32), 2u, VECOPS_TENSOR_WRITE));
+  return rt::OperatorSchema(kMatmulRuntimeQuantName, std::move(params), runtime_quant_relations);
 }
 
 // ---- recipes ------------------------------------------------------------------------------------
@@ -485,6 +520,27 @@ rt::Result<rt::BoundKernelRecipe> MatmulPackedBRecipe::bind(const rt::KernelCall
   return bound;
 }
 
+Status MatmulRuntimeQuantRecipe::match(const rt::KernelCall& call) const {
+  auto place = placement_of(call);
+  if (!place) return place.status();
+  const auto values = call.arguments().values();
+  for (std::size_t i : {std::size_t{2}, std::size_t{4}, std::size_t{5}, std::size_t{6}}) {
+    const TensorView* t = tensor_at(values, i);
+    if (t != nullptr && t->sizes[0] > 1 && t->strides[0] != 1) return not_applicable("the vectors must be contiguous");
+  }
+  return Status::success();
+}
+
+rt::Result<rt::BoundKernelRecipe> MatmulRuntimeQuantRecipe::bind(const rt::KernelCall& call) const {
+  if (Status st = match(call); !st.ok()) return st;
+  rt::BoundKernelRecipe bound;
+  bound.recipe_id = std::string(id());
+  bound.specialization_key = std::string(kMatmulRuntimeQuantName) + ";operands=f32_i8;epilogue=row_col_dequant;memory=" +
+                             placement_name(placement_of(call).value()) + ";" + kBackend;
+  bound.artifact_key = bound.recipe_id + ";" + bound.specialization_key;
+  return bound;
+}
+
 // ---- dispatch policy --------------------------------------------------------------------------------
 
 rt::Result<std::vector<std::size_t>>
@@ -620,6 +676,10 @@ std::shared_ptr<rt::Operator> make_matmul_packed_b_operator(const std::filesyste
                    std::make_shared<MatmulPackedBRecipe>(OperandClass::F32),
                    std::make_shared<MatmulPackedBRecipe>(OperandClass::I8)},
                   dir);
+}
+
+std::shared_ptr<rt::Operator> make_matmul_runtime_quant_operator(const std::filesystem::path& dir) {
+  return assemble(make_matmul_runtime_quant_schema(), {std::make_shared<MatmulRuntimeQuantRecipe>()}, dir);
 }
 
 std::shared_ptr<rt::Operator> make_matmul_w8a16_group_operator(const std::filesystem::path& dir) {

@@ -19,6 +19,8 @@
 //   vecops::matmul_pack_b       (b[N,K], a_zero_point scalar, packed u8[bytes] out, compensation? i32[N] out)
 //       specialization value  PackedType : DType    (the source's own class by default)
 //   vecops::matmul_packed_b     (a[..,M,K], packed_b u8[bytes], c_in?[..,M,N], c[..,M,N] out)
+//   vecops::matmul_runtime_quant (a f32[M,K], b i8[N,K], multipliers f32[M], zero_point scalar,
+//                                row_scales f32[M], column_scales f32[N], correction? i32[N], c f32[M,N] out)
 #ifndef VECOPS_HIP_MATMUL_PLUGIN_HPP
 #define VECOPS_HIP_MATMUL_PLUGIN_HPP
 
@@ -42,6 +44,7 @@ inline constexpr const char* kMatmulW8A16GroupName = "vecops::matmul_w8a16_group
 inline constexpr const char* kMatmulFusedName = "vecops::matmul_fused";
 inline constexpr const char* kMatmulPackBName = "vecops::matmul_pack_b";
 inline constexpr const char* kMatmulPackedBName = "vecops::matmul_packed_b";
+inline constexpr const char* kMatmulRuntimeQuantName = "vecops::matmul_runtime_quant";
 
 // Operand classes of vecops::matmul, one artifact each.
 enum class OperandClass { BF16, F32, I8, F16 };
@@ -67,6 +70,11 @@ rt::OperatorSchema make_matmul_fused_schema();
 // comes from c, K from a, and one packed operand serves every batch of a rank-3 a (ops/MatmulPack.h:22-24).
 rt::OperatorSchema make_matmul_pack_b_schema();
 rt::OperatorSchema make_matmul_packed_b_schema();
+// vecops::matmul_runtime_quant: fp32 activations quantised on the way in by vecops'
+// RuntimePerRowAsymmetricQuantizeTransform (q = u8(a * multipliers[row] + zero_point), matmul/Quantization.h:91-146),
+// int8 weights, the int32 correction row as C input and the per-row x per-column dequantisation on the way out -
+// the pipeline of tests/ops/MatmulConversionTestCommon.h:1437-1540 with the transforms' arrays as positional tensors.
+rt::OperatorSchema make_matmul_runtime_quant_schema();
 
 // Kernel families a recipe stands for: the MFMA workgroup-tile kernels or the
 // wavefront split-K dot-product kernels for skinny shapes.
@@ -155,6 +163,14 @@ private:
   std::string id_;
 };
 
+// vecops::matmul_runtime_quant:  ...;operands=f32_i8;epilogue=row_col_dequant;memory=..;backend=hip-gfx950
+class MatmulRuntimeQuantRecipe final : public rt::KernelRecipe {
+public:
+  [[nodiscard]] std::string_view id() const override { return "hip.matmul_runtime_quant.tile"; }
+  [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
+  [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
+};
+
 // GPU counterpart of the call sites of vecops' runtime shape predicates
 // (matmul/details/kernel/amx/Backend.h:2724-2757 consulting
 // src/MatmulRuntimeDispatch.cpp:12-32): orders the recipes of an operator for
@@ -202,6 +218,7 @@ std::shared_ptr<rt::Operator> make_matmul_w8a16_group_operator(const std::filesy
 std::shared_ptr<rt::Operator> make_matmul_fused_operator(const std::filesystem::path& artifact_directory);
 std::shared_ptr<rt::Operator> make_matmul_pack_b_operator(const std::filesystem::path& artifact_directory);
 std::shared_ptr<rt::Operator> make_matmul_packed_b_operator(const std::filesystem::path& artifact_directory);
+std::shared_ptr<rt::Operator> make_matmul_runtime_quant_operator(const std::filesystem::path& artifact_directory);
 
 }  // namespace vecops::hip
 #endif

@@ -35,6 +35,9 @@ SIGNATURES = {
                               ("clamp_lo", "float"), ("clamp_hi", "float"), ("c", "out")], {}),
     "vecops::matmul_pack_b": ([("b", "in"), ("a_zero_point", "int"), ("packed", "out"), ("compensation", "out?")], {}),
     "vecops::matmul_packed_b": ([("a", "in"), ("packed_b", "in"), ("c_in", "in?"), ("c", "out")], {}),
+    "vecops::matmul_runtime_quant": ([("a", "in"), ("b", "in"), ("multipliers", "in"), ("zero_point", "int"),
+                                      ("row_scales", "in"), ("column_scales", "in"), ("correction", "in?"),
+                                      ("c", "out")], {}),
 }
 
 _PREPARED_CALLS = 8          # signatures kept per thread (docs/Runtime.md:196-206)
