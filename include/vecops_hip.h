@@ -210,8 +210,9 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_quantize_rows(const VecopsHipOperand* x, co
  *   c[i,j] = (float(acc) * row_scales[i]) * column_scales[j].
  * a f32 [M,K], b i8 [N,K], c f32 [M,N] (rank 2, any strides); correction (int32[N], usually
  * -zero_point * sum_k b[j,k], see vecops_hip_pack_b_compensated) may be null.  The workspace holds the
- * quantised activations and the product's own scratch: vecops_hip_matmul_runtime_quant_workspace bytes,
- * 16-byte aligned.  Bit-exact.
+ * quantised activations (kept as q - 128 for the signed kernels), the correction row with 128 * sum_k b[j,k]
+ * added, and the product's own scratch: vecops_hip_matmul_runtime_quant_workspace bytes, 16-byte aligned.
+ * Bit-exact (the sums are integers mod 2^32 either way).
  */
 VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_runtime_quant_workspace(const VecopsHipOperand* a,
                                                                      const VecopsHipOperand* b,

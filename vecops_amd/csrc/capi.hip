@@ -449,7 +449,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     p.a_flip = pr.a_unsigned ? 0x80808080u : 0u;
     p.b_flip = pr.b_unsigned ? 0x80808080u : 0u;
     if (pr.b_unsigned) {  // + 128 * sum_k a'[m,k] per row
-      e = launch_byte_row_sums(pr.a.data, p.batch, p.m, p.k, pr.a.bs, pr.a.rs, pr.a.cs, p.a_flip, 128u, row_term, stream);
+      e = launch_byte_row_sums(pr.a.data, p.batch, p.m, p.k, pr.a.bs, pr.a.rs, pr.a.cs, p.a_flip, 128u, nullptr, row_term, stream);
       if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
       p.row_term = row_term;
     }
@@ -458,7 +458,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
       if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
       p.col_term = col_term;
     } else if (pr.a_unsigned) {  // + 128 * sum_k b'[n,k] per column
-      e = launch_byte_row_sums(pr.b.data, p.batch, p.n, p.k, pr.b.bs, pr.b.rs, pr.b.cs, p.b_flip, 128u, col_term, stream);
+      e = launch_byte_row_sums(pr.b.data, p.batch, p.n, p.k, pr.b.bs, pr.b.rs, pr.b.cs, p.b_flip, 128u, nullptr, col_term, stream);
       if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
       p.col_term = col_term;
     }
@@ -603,7 +603,7 @@ int32_t vecops_hip_pack_b_compensated(const VecopsHipOperand* b, int32_t a_zero_
   if (compensation == nullptr) return fail(ST_INVALID, "pack_b_compensated: null compensation");
   // -a_zero_point * sum_k b[n,k], wrapping like every int32 accumulator of the path
   hipError_t e = launch_byte_row_sums(v.data, 1, static_cast<int32_t>(v.rows), static_cast<int32_t>(v.cols), 0, v.rs, v.cs,
-                                      0u, 0u - static_cast<uint32_t>(a_zero_point), compensation,
+                                      0u, 0u - static_cast<uint32_t>(a_zero_point), nullptr, compensation,
                                       static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
   return ST_OK;
@@ -664,42 +664,40 @@ int32_t vecops_hip_quantize_rows(const VecopsHipOperand* x, const float* multipl
     return fail(ST_INVALID, "quantize_rows: extent too large");
   hipError_t e = launch_quantize_rows(static_cast<const float*>(vx.data), static_cast<int32_t>(vx.batch),
                                       static_cast<int32_t>(vx.rows), static_cast<int32_t>(vx.cols), vx.bs, vx.rs, vx.cs,
-                                      multipliers, zero_point, static_cast<uint8_t*>(vq.data), vq.bs, vq.rs, vq.cs,
+                                      multipliers, zero_point, 0u, static_cast<uint8_t*>(vq.data), vq.bs, vq.rs, vq.cs,
                                       static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(ST_EXEC, "quantize kernel launch: %s", hipGetErrorString(e));
   return ST_OK;
 }
 
 namespace {
-// The pieces of vecops_hip_matmul_runtime_quant: the quantised activations sit at the head of the workspace
-// (M x K bytes rounded up to 256), the product's own workspace behind them.
+// The pieces of vecops_hip_matmul_runtime_quant.  The activations are quantised to q - 128 as int8 (the byte
+// xor 0x80), so that the product runs on the signed kernels with their fast dequantising epilogue, and
+//   sum_k q * b = sum_k (q - 128) * b + 128 * sum_k b[n,k]
+// goes into the correction row.  Workspace: M x K bytes of activations, N int32 of that row (both rounded up
+// to 256 bytes), then the product's own scratch.
 struct RuntimeQuant {
-  VecopsHipOperand q, cin;
-  VecopsHipEpilogue ep;
+  VecopsHipOperand q, c_acc;
   Problem pr;
   VecopsHipPlan plan;
-  uint64_t q_bytes;
+  uint64_t q_bytes, row_bytes;
 };
 
-int32_t describe_runtime_quant(const VecopsHipOperand* a, const VecopsHipOperand* b, const int32_t* correction,
-                               const float* row_scales, const float* column_scales, const VecopsHipOperand* c,
+int32_t describe_runtime_quant(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c,
                                void* workspace, RuntimeQuant* d) {
   if (a == nullptr || a->rank != 2 || a->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: a must be a rank-2 f32 operand");
   if (b == nullptr || b->rank != 2 || b->dtype != DT_I8) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: b must be a rank-2 i8 operand");
   if (c == nullptr || c->rank != 2 || c->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: c must be a rank-2 f32 operand");
-  if (a->sizes[0] < 0 || a->sizes[1] < 0) return fail(ST_INVALID, "matmul_runtime_quant: negative extent");
-  const int64_t m = a->sizes[0], k = a->sizes[1];
+  if (a->sizes[0] < 0 || a->sizes[1] < 0 || b->sizes[0] < 0) return fail(ST_INVALID, "matmul_runtime_quant: negative extent");
+  const int64_t m = a->sizes[0], k = a->sizes[1], n = b->sizes[0];
   d->q_bytes = (static_cast<uint64_t>(m) * static_cast<uint64_t>(k) + 255u) & ~uint64_t{255};
-  make_operand(&d->q, workspace, DT_U8, m, k, k);
-  if (correction != nullptr) {
-    make_operand(&d->cin, correction, DT_I32, m, c->sizes[1], 0);  // one row for every row of c
-  }
-  memset(&d->ep, 0, sizeof(d->ep));
-  d->ep.struct_size = sizeof(d->ep);
-  d->ep.row_scales = row_scales;
-  d->ep.column_scales = column_scales;
-  int32_t rc = describe(&d->q, b, correction ? &d->cin : nullptr, c, 0, &d->pr, &d->ep);
+  d->row_bytes = (static_cast<uint64_t>(n) * 4u + 255u) & ~uint64_t{255};
+  make_operand(&d->q, workspace, DT_I8, m, k, k);
+  d->c_acc = *c;
+  d->c_acc.dtype = DT_I32;  // accumulator class; the epilogue writes fp32
+  int32_t rc = describe(&d->q, b, nullptr, &d->c_acc, 0, &d->pr);
   if (rc != ST_OK) return rc;
+  d->pr.dequant = true;
   choose(d->pr, &d->plan);
   return ST_OK;
 }
@@ -708,9 +706,8 @@ int32_t describe_runtime_quant(const VecopsHipOperand* a, const VecopsHipOperand
 uint64_t vecops_hip_matmul_runtime_quant_workspace(const VecopsHipOperand* a, const VecopsHipOperand* b,
                                                    const VecopsHipOperand* c) {
   RuntimeQuant d;
-  static const float one = 1.0f;
-  if (describe_runtime_quant(a, b, nullptr, &one, &one, c, reinterpret_cast<void*>(256), &d) != ST_OK) return 0;
-  return d.q_bytes + d.plan.workspace_bytes;
+  if (describe_runtime_quant(a, b, c, reinterpret_cast<void*>(256), &d) != ST_OK) return 0;
+  return d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
 }
 
 int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* multipliers, int32_t zero_point,
@@ -718,19 +715,31 @@ int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* 
                                         const float* column_scales, const VecopsHipOperand* c, void* workspace,
                                         uint64_t workspace_size, void* stream) {
   RuntimeQuant d;
-  int32_t rc = describe_runtime_quant(a, b, correction, row_scales, column_scales, c,
-                                      workspace ? workspace : reinterpret_cast<void*>(256), &d);
+  int32_t rc = describe_runtime_quant(a, b, c, workspace ? workspace : reinterpret_cast<void*>(256), &d);
   if (rc != ST_OK) return rc;
   if (d.plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
   if (row_scales == nullptr || column_scales == nullptr || multipliers == nullptr)
     return fail(ST_INVALID, "matmul_runtime_quant: multipliers and both scale vectors are required");
-  if (d.q_bytes + d.plan.workspace_bytes > workspace_size || (d.q_bytes > 0 && (workspace == nullptr || !aligned16(workspace))))
+  const uint64_t need = d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
+  if (need > workspace_size || workspace == nullptr || !aligned16(workspace))
     return fail(ST_INVALID, "matmul_runtime_quant: %llu bytes of 16-byte aligned workspace required, %llu supplied",
-                (unsigned long long)(d.q_bytes + d.plan.workspace_bytes), (unsigned long long)workspace_size);
-  rc = vecops_hip_quantize_rows(a, multipliers, zero_point, &d.q, stream);
-  if (rc != ST_OK) return rc;
-  return run_problem(d.pr, d.plan, nullptr, nullptr, nullptr, static_cast<char*>(workspace) + d.q_bytes,
-                     workspace_size - d.q_bytes, static_cast<hipStream_t>(stream));
+                (unsigned long long)need, (unsigned long long)workspace_size);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const View& va = d.pr.a;  // the quantised activations, dense
+  View vx;
+  normalise(a, &vx);
+  hipError_t e = launch_quantize_rows(static_cast<const float*>(vx.data), 1, static_cast<int32_t>(vx.rows),
+                                      static_cast<int32_t>(vx.cols), 0, vx.rs, vx.cs, multipliers, zero_point, 0x80u,
+                                      static_cast<uint8_t*>(va.data), 0, va.rs, va.cs, s);
+  if (e != hipSuccess) return fail(ST_EXEC, "quantize kernel launch: %s", hipGetErrorString(e));
+  // correction[n] + 128 * sum_k b[n,k]
+  int32_t* row = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + d.q_bytes);
+  const View& vb = d.pr.b;
+  e = launch_byte_row_sums(vb.data, 1, static_cast<int32_t>(vb.rows), static_cast<int32_t>(vb.cols), 0, vb.rs, vb.cs, 0u,
+                           128u, correction, row, s);
+  if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
+  return run_problem(d.pr, d.plan, row_scales, column_scales, row, static_cast<char*>(workspace) + d.q_bytes + d.row_bytes,
+                     workspace_size - d.q_bytes - d.row_bytes, s);
 }
 
 uint32_t vecops_hip_abi_version(void) { return VECOPS_HIP_ABI_VERSION; }

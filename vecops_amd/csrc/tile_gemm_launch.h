@@ -27,13 +27,15 @@ hipError_t launch_tile_gemm_f32(const TileGemmParams& p, int tile_m, int tile_n,
 hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
 // 8-bit operands of which at least one is unsigned (p.a_flip / p.b_flip and the epilogue terms set)
 hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
-// out[b][r] = scale * sum_k int8(x[b][r][k] xor flip): the epilogue terms of an unsigned operand
+// out[b][r] = scale * sum_k int8(x[b][r][k] xor flip) (+ add[r], may be null): the epilogue terms of an unsigned operand
 hipError_t launch_byte_row_sums(const void* x, int32_t batch, int32_t rows, int32_t k, int64_t bs, int64_t rs,
-                                int64_t ks, uint32_t flip, uint32_t scale, int32_t* out, hipStream_t stream);
-// q = u8(x * multipliers[row] + zero_point): the per-row asymmetric quantisation of fp32 activations
+                                int64_t ks, uint32_t flip, uint32_t scale, const int32_t* add, int32_t* out,
+                                hipStream_t stream);
+// q = u8(x * multipliers[row] + zero_point) xor flip: the per-row asymmetric quantisation of fp32 activations
+// (flip 0x80 stores the byte as the int8 q - 128)
 hipError_t launch_quantize_rows(const float* x, int32_t batch, int32_t rows, int32_t k, int64_t xbs, int64_t xrs,
-                                int64_t xks, const float* multipliers, int32_t zero_point, uint8_t* q, int64_t qbs,
-                                int64_t qrs, int64_t qks, hipStream_t stream);
+                                int64_t xks, const float* multipliers, int32_t zero_point, uint32_t flip, uint8_t* q,
+                                int64_t qbs, int64_t qrs, int64_t qks, hipStream_t stream);
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
 // B prepacked by launch_pack_b (src: SRC_BF16, SRC_F32_AS_BF16 = fp32 A against bf16-packed B, SRC_I8,
 // SRC_I8_FLIP = unsigned A against int8-packed B with p.a_flip and p.col_term set);

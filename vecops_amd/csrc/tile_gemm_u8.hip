@@ -6,21 +6,35 @@ hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile_m, int til
   return launch_tile_class<SRC_I8_FLIP>(p, tile_m, tile_n, mode, stream);
 }
 
-// out[b][r] = scale * sum_k int8(x[b][r][k] xor flip)  (wrapping): the per-row and
-// per-column terms of SRC_I8_FLIP.  One wavefront per row, any strides.
+// out[b][r] = scale * sum_k int8(x[b][r][k] xor flip) (+ add[r])  (wrapping): the per-row and
+// per-column terms of SRC_I8_FLIP.  One wavefront per row, any strides; 16 bytes per lane and step
+// when the row is contiguous and aligned.
 __global__ __launch_bounds__(256) void byte_row_sums_kernel(const uint8_t* x, int32_t batch, int32_t rows, int32_t k,
                                                             int64_t bs, int64_t rs, int64_t ks, uint32_t flip,
-                                                            uint32_t scale, int32_t* out) {
+                                                            uint32_t scale, const int32_t* add, int32_t* out) {
   const int lane = threadIdx.x & 63;
   const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (row >= static_cast<int64_t>(batch) * rows) return;
   const int64_t b = row / rows, r = row - b * rows;
   const uint8_t* src = x + b * bs + r * rs;
   int32_t sum = 0;
-  for (int kk = lane; kk < k; kk += 64) sum += static_cast<int8_t>(src[kk * ks] ^ static_cast<uint8_t>(flip));
+  int done = 0;
+  if (ks == 1 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0) {
+    const int chunks = k / 16;
+    for (int ch = lane; ch < chunks; ch += 64) {
+      const u32x4 v = reinterpret_cast<const u32x4*>(src)[ch];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const int32_t word = static_cast<int32_t>(v[w] ^ flip);
+        sum += (word << 24 >> 24) + (word << 16 >> 24) + (word << 8 >> 24) + (word >> 24);
+      }
+    }
+    done = chunks * 16;
+  }
+  for (int kk = done + lane; kk < k; kk += 64) sum += static_cast<int8_t>(src[kk * ks] ^ static_cast<uint8_t>(flip));
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
-  if (lane == 0) out[row] = static_cast<int32_t>(static_cast<uint32_t>(sum) * scale);
+  if (lane == 0) out[row] = static_cast<int32_t>(static_cast<uint32_t>(sum) * scale + (add ? static_cast<uint32_t>(add[r]) : 0u));
 }
 
 // q[b][r][k] = u8(x[b][r][k] * multipliers[b * rows + r] + float(zero_point)): vecops'
@@ -28,11 +42,11 @@ __global__ __launch_bounds__(256) void byte_row_sums_kernel(const uint8_t* x, in
 // result to the uint8 compute type - a multiply and an add, each rounded (the file is compiled without
 // contraction), truncation toward zero, NaN and values outside int32 to INT32_MIN, saturation to 0..255.
 // One thread per four consecutive k: one 16-byte load when x is K-contiguous and the quad is aligned, one
-// 4-byte store when q is.
+// 4-byte store when q is.  flip (0 or 0x80) is xored into every byte.
 __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* x, int32_t batch, int32_t rows, int32_t k,
                                                             int64_t xbs, int64_t xrs, int64_t xks,
-                                                            const float* multipliers, float zero_point, uint8_t* q,
-                                                            int64_t qbs, int64_t qrs, int64_t qks) {
+                                                            const float* multipliers, float zero_point, uint32_t flip,
+                                                            uint8_t* q, int64_t qbs, int64_t qrs, int64_t qks) {
   const int64_t quads_per_row = (static_cast<int64_t>(k) + 3) / 4;
   const int64_t total = static_cast<int64_t>(batch) * rows * quads_per_row;
   for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += gridDim.x * 256ll) {
@@ -54,7 +68,7 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* x, int3
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float scaled = v[e] * mult;
-      bytes[e] = narrow_to_byte(scaled + zero_point, false);
+      bytes[e] = narrow_to_byte(scaled + zero_point, false) ^ flip;  // flip 0x80: the byte as q - 128 in int8
     }
     if (left == 4 && qks == 1 && (reinterpret_cast<uintptr_t>(dst) & 3u) == 0) {
       *reinterpret_cast<uint32_t*>(dst) = bytes[0] | (bytes[1] << 8) | (bytes[2] << 16) | (bytes[3] << 24);
@@ -65,25 +79,26 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* x, int3
 }
 
 hipError_t launch_quantize_rows(const float* x, int32_t batch, int32_t rows, int32_t k, int64_t xbs, int64_t xrs,
-                                int64_t xks, const float* multipliers, int32_t zero_point, uint8_t* q, int64_t qbs,
-                                int64_t qrs, int64_t qks, hipStream_t stream) {
+                                int64_t xks, const float* multipliers, int32_t zero_point, uint32_t flip, uint8_t* q,
+                                int64_t qbs, int64_t qrs, int64_t qks, hipStream_t stream) {
   const int64_t total = static_cast<int64_t>(batch) * rows * ((static_cast<int64_t>(k) + 3) / 4);
   if (total <= 0) return hipSuccess;
   int64_t blocks = (total + 255) / 256;
   if (blocks > 256 * 32) blocks = 256 * 32;
   hipLaunchKernelGGL(quantize_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, x, batch, rows, k,
-                     xbs, xrs, xks, multipliers, static_cast<float>(zero_point), q, qbs, qrs, qks);
+                     xbs, xrs, xks, multipliers, static_cast<float>(zero_point), flip & 0xffu, q, qbs, qrs, qks);
   return hipGetLastError();
 }
 
 hipError_t launch_byte_row_sums(const void* x, int32_t batch, int32_t rows, int32_t k, int64_t bs, int64_t rs,
-                                int64_t ks, uint32_t flip, uint32_t scale, int32_t* out, hipStream_t stream) {
+                                int64_t ks, uint32_t flip, uint32_t scale, const int32_t* add, int32_t* out,
+                                hipStream_t stream) {
   const int64_t total = static_cast<int64_t>(batch) * rows;
   if (total <= 0) return hipSuccess;
   const int64_t blocks = (total + 3) / 4;
   if (blocks > INT32_MAX) return hipErrorInvalidConfiguration;
   hipLaunchKernelGGL(byte_row_sums_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
-                     static_cast<const uint8_t*>(x), batch, rows, k, bs, rs, ks, flip, scale, out);
+                     static_cast<const uint8_t*>(x), batch, rows, k, bs, rs, ks, flip, scale, add, out);
   return hipGetLastError();
 }
 }  // namespace vecops_hip
