@@ -1309,7 +1309,10 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
   // work that happens on the row-major side of the 32-bit staging: C-input, int32 sums leaving as floats,
   // the fused output transform, outputs narrower than 32 bits
   const bool finishing = p.cin != nullptr || p.fused != 0 || (INT ? (!dequant && p.out_kind != OUT_I32) : p.out_kind != OUT_F32);
-  const bool simple = aligned && p.split_k == 1 && p.c_cs == 1 && SRC != SRC_I8_FLIP &&
+  // (an unsigned operand's terms go through the general path, unless the launcher has folded them into the
+  // per-column correction: unsigned A, one batch)
+  const bool flip_terms = SRC == SRC_I8_FLIP && (p.row_term != nullptr || p.col_term != nullptr || p.const_term != 0u);
+  const bool simple = aligned && p.split_k == 1 && p.c_cs == 1 && !flip_terms &&
                       (p.cin == nullptr || (p.cin_cs == 1 && !dequant));
   char* c_base = static_cast<char*>(p.c);
   if (simple && !INT && p.out_kind == OUT_BF16 && p.cin == nullptr && p.fused == 0) {
