@@ -111,6 +111,42 @@ def bench_int8_dequant(dev, steps, warmup):
                          "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
 
 
+def bench_runtime_quant(dev, steps, warmup):
+    """fp32 activations quantised per row on the way in (vecops' RuntimePerRowAsymmetricQuantizeTransform), int8
+    weights, correction row, per-token x per-channel dequantisation: three launches (quantise, weight row sums,
+    the int8 product) timed as one step."""
+    import numpy as np
+    import torch
+    from vecops_amd import capi, synth
+    m, k, n, zp = 2048, 4096, 11008, 7
+    mult = (np.float32(4.0) * (np.float32(1.0) + synth.uniform_pm1(11, (m,)) * np.float32(0.5))).astype(np.float32)
+    a_host = ((synth.uniform_pm1(12, (m, k)) * np.float32(140.0) + np.float32(128 - zp)) / mult[:, None]).astype(np.float32)
+    b_host = synth.int8_sym(2, (n, k))
+    a, b = torch.from_numpy(a_host).to(dev), torch.from_numpy(b_host).to(dev)
+    tm = torch.from_numpy(mult).to(dev)
+    rs = torch.from_numpy((np.float32(1.0) / mult).astype(np.float32)).to(dev)
+    cs = torch.from_numpy(synth.scales(4, n)).to(dev)
+    corr = torch.from_numpy((-zp * b_host.astype(np.int64).sum(axis=1)).astype(np.int32)).to(dev)
+    c = torch.empty((m, n), dtype=torch.float32, device=dev)
+    oa, ob, oc = capi.operand(a), capi.operand(b), capi.operand(c)
+    import ctypes as C
+    need = capi.lib().vecops_hip_matmul_runtime_quant_workspace(C.byref(oa), C.byref(ob), C.byref(oc))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    wall_ms, ev_ms = _time_launches(
+        lambda i: capi.matmul_runtime_quant(a, tm, zp, b, rs, cs, c, correction=corr, workspace=ws), steps, warmup)
+    ops = 2.0 * m * n * k
+    tops = ops / (ev_ms * 1e-3) / 1e12
+    return {"metric": "runtime_quantized_matmul_tops", "workload": "fp32 activations 2048x4096 quantised per row to "
+            "uint8 on the way in, int8 weights 11008x4096, correction row, per-token x per-channel dequant, fp32 out",
+            "value": tops, "unit": "TOP/s", "ms_per_step": wall_ms, "dtype": "int8",
+            "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                         "frac": tops / PEAK_INT8_TOPS, "traffic": None,
+                         "kernel": "vecops_hip::quantize_rows_kernel + byte_row_sums_kernel + tile_gemm_kernel<int8, "
+                                   "256x256x128, loads into LDS, dequant epilogue>",
+                         "algorithmic_ops_per_launch": ops,
+                         "algorithmic_bytes_per_launch": 4 * m * k + n * k + 4 * m * n + 4 * (2 * m + 2 * n)}}
+
+
 def bench_bf16_gemm_packed(dev, steps, warmup):
     """The headline shape with B packed once beforehand (vecops' prepacked-weights mode): the packing is
     outside the timed region, as in the reference's own prepacked rows."""
@@ -178,6 +214,7 @@ def bench_gemv(dev, steps, warmup, m=1):
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                          "frac": gbps / PEAK_HBM_GBPS, "traffic": TRAFFIC_GEMV_M1 if m == 1 else None,
                          "kernel": "vecops_hip::skinny_w8a16_stream_kernel" if m == 1 else
+                                   "vecops_hip::skinny_w8a16_stream_rows_kernel" if m == 2 else
                                    "vecops_hip::skinny_w8a16_mfma_resident_kernel",
                          "algorithmic_bytes_per_launch": nbytes}}
 
@@ -238,7 +275,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed"], help="run a single workload (for profiling)")
+    ap.add_argument("--only", choices=["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant"], help="run a single workload (for profiling)")
     ap.add_argument("--gemv-m", type=int, default=1, help="activation rows of the --only gemv workload (1..16)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -267,6 +304,9 @@ def main() -> int:
     if args.only == "int8_packed":
         print(json.dumps(bench_int8_dequant_packed(dev, args.steps, args.warmup)))
         return 0
+    if args.only == "runtime_quant":
+        print(json.dumps(bench_runtime_quant(dev, args.steps, args.warmup)))
+        return 0
     if args.only == "gemv":
         print(json.dumps(bench_gemv(dev, args.steps, args.warmup, m=args.gemv_m)))
         return 0
@@ -284,8 +324,11 @@ def main() -> int:
     if args.only != "bf16":
         line["secondary"] = [bench_int8_dequant(dev, args.steps, args.warmup),
                              bench_gemv(dev, max(args.steps, 200), args.warmup, m=1),
+                             bench_gemv(dev, max(args.steps, 200), args.warmup, m=4),
+                             bench_gemv(dev, max(args.steps, 200), args.warmup, m=16),
                              bench_bf16_gemm_packed(dev, args.steps, args.warmup),
-                             bench_int8_dequant_packed(dev, args.steps, args.warmup)]
+                             bench_int8_dequant_packed(dev, args.steps, args.warmup),
+                             bench_runtime_quant(dev, args.steps, args.warmup)]
     if not args.no_cpu and args.only is None:
         line["cpu_baseline"] = cpu_baseline(a, b_kn)
     print(json.dumps(line))
