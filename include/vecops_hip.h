@@ -208,7 +208,9 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_quantize_rows(const VecopsHipOperand* x, co
  * The runtime-quantised product of tests/ops/MatmulConversionTestCommon.h:1437-1540 in one call:
  *   q = quantize_rows(a);  acc = sum_k q[i,k] * b[j,k] + correction[j]  (AMX_I8I32<uint8_t, int8_t>, wrapping);
  *   c[i,j] = (float(acc) * row_scales[i]) * column_scales[j].
- * a f32 [M,K], b i8 [N,K], c f32 [M,N] (rank 2, any strides); correction (int32[N], usually
+ * a f32 [M,K], b i8 [N,K], c f32 [M,N] (rank 2, any strides), or a [batch,M,K] and c [batch,M,N] whose
+ * rows run on from batch to batch against the one b (multipliers and row_scales then have batch * M
+ * entries: vecops' batch_stride = M); correction (int32[N], usually
  * -zero_point * sum_k b[j,k], see vecops_hip_pack_b_compensated) may be null.  The workspace holds the
  * quantised activations (kept as q - 128 for the signed kernels), the correction row with 128 * sum_k b[j,k]
  * added, and the product's own scratch: vecops_hip_matmul_runtime_quant_workspace bytes, 16-byte aligned.

@@ -91,6 +91,30 @@ def test_runtime_quant_pipeline_against_the_oracle(device, oracle, m, n, k):
     assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+def test_runtime_quant_batched_activations_shared_weights(device, oracle):
+    """Rank-3 a and c against one b (vecops' BroadcastB case, row scales indexed batch * M + row,
+    tests/ops/MatmulConversionTestCommon.h:1277-1434): the batches fold into rows."""
+    import torch
+    from vecops_amd import capi
+    batch, m, n, k = 3, 37, 150, 300
+    mult = (np.float32(2.0) + synth.uniform_pm1(1, (batch * m,))).astype(np.float32)
+    a = ((synth.uniform_pm1(2, (batch * m, k)) * np.float32(140.0) + np.float32(120.0)) / mult[:, None]).astype(np.float32)
+    b = synth.int8_sym(3, (n, k))
+    rs, cs = (np.float32(1.0) / mult).astype(np.float32), synth.scales(4, n)
+    corr = (-8 * b.astype(np.int64).sum(axis=1)).astype(np.int32)
+    acc = (oracle.quantize_rows(a, mult, 8).astype(np.int64) @ b.astype(np.int64).T + corr).astype(np.int32)
+    want = oracle.fused_outputs(acc, np.float32, row_scales=rs, column_scales=cs).reshape(batch, m, n)
+    c = torch.full((batch, m, n), float("nan"), device=device)
+    capi.matmul_runtime_quant(dev(a.reshape(batch, m, k), device), dev(mult, device), 8, dev(b, device), dev(rs, device),
+                              dev(cs, device), c, correction=dev(corr, device))
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    gapped = torch.zeros((batch, m + 1, k), device=device)[:, :m]            # rows do not run on: refused, not wrong
+    with pytest.raises(capi.VecopsHipError) as e:
+        capi.matmul_runtime_quant(gapped, dev(mult, device), 8, dev(b, device), dev(rs, device), dev(cs, device), c)
+    assert e.value.code == 2
+
+
 def test_runtime_quant_zero_extents_and_rejections(device):
     import torch
     from vecops_amd import capi

@@ -683,17 +683,42 @@ namespace {
 // goes into the correction row.  Workspace: M x K bytes of activations, N int32 of that row (both rounded up
 // to 256 bytes), then the product's own scratch.
 struct RuntimeQuant {
-  VecopsHipOperand q, c_acc;
+  VecopsHipOperand q, c_acc, a_flat, c_flat;
   Problem pr;
   VecopsHipPlan plan;
   uint64_t q_bytes, row_bytes;
 };
 
-int32_t describe_runtime_quant(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c,
+// A rank-3 operand whose rows run on from batch to batch (batch stride = M x row stride) as the rank-2
+// [batch * M, cols] matrix it is in memory; rank 2 is passed through.
+bool fold_batches(const VecopsHipOperand* o, VecopsHipOperand* flat) {
+  *flat = *o;
+  if (o->rank != 3) return o->rank == 2;
+  if (o->sizes[0] > 1 && o->strides[0] != o->sizes[1] * o->strides[1]) return false;
+  memset(flat->sizes, 0, sizeof(flat->sizes));
+  memset(flat->strides, 0, sizeof(flat->strides));
+  flat->rank = 2;
+  flat->sizes[0] = o->sizes[0] * o->sizes[1];
+  flat->sizes[1] = o->sizes[2];
+  flat->strides[0] = o->strides[1];
+  flat->strides[1] = o->strides[2];
+  return true;
+}
+
+int32_t describe_runtime_quant(const VecopsHipOperand* a_given, const VecopsHipOperand* b, const VecopsHipOperand* c_given,
                                void* workspace, RuntimeQuant* d) {
-  if (a == nullptr || a->rank != 2 || a->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: a must be a rank-2 f32 operand");
+  if (a_given == nullptr || c_given == nullptr || a_given->rank != c_given->rank ||
+      (a_given->rank == 3 && a_given->sizes[0] != c_given->sizes[0]))
+    return fail(ST_INVALID, "matmul_runtime_quant: a and c must have the same rank and batch extent");
+  // one set of weights for every batch (the serving case; vecops' BroadcastB,
+  // tests/ops/MatmulConversionTestCommon.h:1277-1434): the batches of a and c fold into rows
+  if (!fold_batches(a_given, &d->a_flat) || !fold_batches(c_given, &d->c_flat))
+    return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: rank-3 a and c must have rows that run on from batch to batch");
+  const VecopsHipOperand* a = &d->a_flat;
+  const VecopsHipOperand* c = &d->c_flat;
+  if (a->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: a must be an f32 operand");
   if (b == nullptr || b->rank != 2 || b->dtype != DT_I8) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: b must be a rank-2 i8 operand");
-  if (c == nullptr || c->rank != 2 || c->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: c must be a rank-2 f32 operand");
+  if (c->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: c must be an f32 operand");
   if (a->sizes[0] < 0 || a->sizes[1] < 0 || b->sizes[0] < 0) return fail(ST_INVALID, "matmul_runtime_quant: negative extent");
   const int64_t m = a->sizes[0], k = a->sizes[1], n = b->sizes[0];
   d->q_bytes = (static_cast<uint64_t>(m) * static_cast<uint64_t>(k) + 255u) & ~uint64_t{255};
@@ -733,7 +758,7 @@ int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const View& va = d.pr.a;  // the quantised activations, dense
   View vx;
-  normalise(a, &vx);
+  normalise(&d.a_flat, &vx);
   hipError_t e = launch_quantize_rows(static_cast<const float*>(vx.data), 1, static_cast<int32_t>(vx.rows),
                                       static_cast<int32_t>(vx.cols), 0, vx.rs, vx.cs, multipliers, zero_point, 0x80u,
                                       static_cast<uint8_t*>(va.data), 0, va.rs, va.cs, s);
