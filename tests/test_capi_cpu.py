@@ -66,6 +66,11 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1
     rc, p = _plan(_operand(capi.BF16, (8192, 512)), _operand(capi.BF16, (8192, 512)), _operand(capi.F32, (8192, 8192)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"      # from eight K tiles on the big tile is ahead again
+    # 128 tiles of 128x128 would leave every other compute unit idle and the rest with one workgroup: 512 of 64x64
+    rc, p = _plan(_operand(capi.BF16, (512, 4096)), _operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (512, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 1
+    rc, p = _plan(_operand(capi.BF16, (1024, 4096)), _operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (1024, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
     # one row against a long weight matrix: the skinny family, no workspace
     rc, p = _plan(_operand(capi.BF16, (1, 4096)), _operand(capi.BF16, (14336, 4096)), _operand(capi.BF16, (1, 14336)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "skinny" and p.workspace_bytes == 0

@@ -222,7 +222,7 @@ def test_shared_b_batch_is_folded(device, oracle):
     row, and - rows not running on - the unfolded path giving the same values."""
     import torch
     from vecops_amd import capi
-    batch, m, n, k = 64, 32, 1024, 264
+    batch, m, n, k = 64, 32, 2048, 264
     a = synth.bf16_round(synth.uniform_pm1(1, (batch, m, k)))
     b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
     cin = synth.uniform_pm1(3, (batch, m, n))

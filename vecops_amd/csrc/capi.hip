@@ -290,6 +290,14 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     family = VECOPS_HIP_FAMILY_TILE_128;
     tile_m = tile_n = 128;
   }
+  // Fewer 128x128 tiles than compute units (and more than four K tiles): a unit holds one workgroup and has
+  // nothing to overlap its start-up, barriers and stores with, while four times as many 64x64 tiles put two or
+  // more on every unit (512 x 4096 x 4096: 28.7 us against 45.9; 1536^3: 18.0 against 20.7; 768 x 4096 x 4096:
+  // 42.7 against 46.7; from 256 tiles on - 1024 x 4096 x 4096, 2048^3 - the bigger tile is ahead again).
+  else if (k_tiles > 4 && family == VECOPS_HIP_FAMILY_TILE_128 && pr.src != SRC_F32 && tiles(128) <= 3 * kComputeUnits / 4) {
+    family = VECOPS_HIP_FAMILY_TILE_64;
+    tile_m = tile_n = 64;
+  }
   plan->family = family;
   const int64_t wgs = tiles2(tile_m, tile_n);
   int64_t split = 1;
