@@ -225,6 +225,17 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand
                                                           const float* column_scales, const VecopsHipOperand* c,
                                                           void* workspace, uint64_t workspace_size, void* stream);
 
+/* The same with b packed by vecops_hip_pack_b (int8; n rows) - exactly the operands of
+ * tests/ops/MatmulConversionTestCommon.h:1484-1510, where B is packed first. */
+VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_runtime_quant_packed_b_workspace(const VecopsHipOperand* a, int64_t n,
+                                                                              const VecopsHipOperand* c);
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_runtime_quant_packed_b(const VecopsHipOperand* a, const float* multipliers,
+                                                                   int32_t zero_point, const void* packed_b, int64_t n,
+                                                                   const int32_t* correction, const float* row_scales,
+                                                                   const float* column_scales, const VecopsHipOperand* c,
+                                                                   void* workspace, uint64_t workspace_size,
+                                                                   void* stream);
+
 /* Workspace bytes vecops_hip_matmul_i8_dequant needs for these extents. */
 VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int64_t n, int64_t k);
 

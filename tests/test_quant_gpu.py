@@ -91,6 +91,22 @@ def test_runtime_quant_pipeline_against_the_oracle(device, oracle, m, n, k):
     assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("case", QUANT_CASES, ids=lambda c: c["name"])
+def test_runtime_quant_pipeline_packed_weights_golden(device, case):
+    """The reference test's own operands: B packed first, the compensated pack's sidecar as the correction row
+    (tests/ops/MatmulConversionTestCommon.h:1484-1510, ops/MatmulPack.h:52-58)."""
+    import torch
+    from vecops_amd import capi
+    inp = make_quant_inputs(case)
+    packed, comp = capi.pack_b(dev(inp["b"], device), a_zero_point=case["zp"])
+    assert np.array_equal(comp.cpu().numpy(), inp["correction"])
+    c = torch.full((case["m"], case["n"]), float("nan"), device=device)
+    capi.matmul_runtime_quant_packed_b(dev(inp["a"], device), dev(inp["multipliers"], device), case["zp"], packed,
+                                       dev(inp["row_scales"], device), dev(inp["column_scales"], device), c, correction=comp)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), GOLD[case["name"] + "_f32"].view(np.uint32))
+
+
 def test_runtime_quant_batched_activations_shared_weights(device, oracle):
     """Rank-3 a and c against one b (vecops' BroadcastB case, row scales indexed batch * M + row,
     tests/ops/MatmulConversionTestCommon.h:1277-1434): the batches fold into rows."""

@@ -26,6 +26,7 @@ EXPORTS = [
     "vecops_hip_plan_matmul_packed_b", "vecops_hip_matmul_packed_b", "vecops_hip_matmul_i8_dequant_packed_b",
     "vecops_hip_plan_matmul_fused", "vecops_hip_matmul_fused", "vecops_hip_quantize_rows",
     "vecops_hip_matmul_runtime_quant_workspace", "vecops_hip_matmul_runtime_quant",
+    "vecops_hip_matmul_runtime_quant_packed_b_workspace", "vecops_hip_matmul_runtime_quant_packed_b",
 ]
 
 ACT_NONE, ACT_RELU, ACT_CLAMP, ACT_SIGMOID, ACT_SILU = 0, 1, 2, 3, 4
@@ -96,6 +97,11 @@ def lib() -> C.CDLL:
         L.vecops_hip_matmul_runtime_quant_workspace.argtypes = [P, P, P]
         L.vecops_hip_matmul_runtime_quant.argtypes = [P, C.c_void_p, C.c_int32, P, C.c_void_p, C.c_void_p, C.c_void_p, P,
                                                       C.c_void_p, C.c_uint64, C.c_void_p]
+        L.vecops_hip_matmul_runtime_quant_packed_b_workspace.restype = C.c_uint64
+        L.vecops_hip_matmul_runtime_quant_packed_b_workspace.argtypes = [P, C.c_int64, P]
+        L.vecops_hip_matmul_runtime_quant_packed_b.argtypes = [P, C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p,
+                                                               C.c_void_p, C.c_void_p, P, C.c_void_p, C.c_uint64,
+                                                               C.c_void_p]
         L.vecops_hip_plan_matmul_fused.argtypes = [P, P, P, P, C.c_uint32, E, C.POINTER(Plan)]
         L.vecops_hip_matmul_fused.argtypes = [P, P, P, P, C.c_uint32, E, C.c_void_p, C.c_uint64, C.c_void_p]
         _lib = L
@@ -239,6 +245,23 @@ def matmul_runtime_quant(a, multipliers, zero_point: int, b, row_scales, column_
     ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
     _check(lib().vecops_hip_matmul_runtime_quant(
         C.byref(oa), multipliers.data_ptr(), int(zero_point), C.byref(ob),
+        correction.data_ptr() if correction is not None else None, row_scales.data_ptr(), column_scales.data_ptr(),
+        C.byref(oc), ws_ptr, ws_size, _stream_handle(stream)))
+    return c
+
+
+def matmul_runtime_quant_packed_b(a, multipliers, zero_point: int, packed, row_scales, column_scales, c, correction=None,
+                                  workspace=None, stream=None):
+    """``matmul_runtime_quant`` against weights packed once by ``pack_b`` (int8)."""
+    import torch
+    oa, oc = operand(a), operand(c)
+    need = lib().vecops_hip_matmul_runtime_quant_packed_b_workspace(C.byref(oa), packed.n, C.byref(oc))
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=c.device)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_runtime_quant_packed_b(
+        C.byref(oa), multipliers.data_ptr(), int(zero_point), packed.storage.data_ptr(), packed.n,
         correction.data_ptr() if correction is not None else None, row_scales.data_ptr(), column_scales.data_ptr(),
         C.byref(oc), ws_ptr, ws_size, _stream_handle(stream)))
     return c

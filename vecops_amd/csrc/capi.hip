@@ -462,7 +462,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
       p.row_term = row_term;
     }
     if (pr.a_unsigned && pr.packed_b) {  // the same term from the packed rows, one copy per batch
-      e = launch_packed_row_sums(pr.b.data, p.n, p.k, p.batch, 128u, col_term, stream);
+      e = launch_packed_row_sums(pr.b.data, p.n, p.k, p.batch, 128u, nullptr, col_term, stream);
       if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
       p.col_term = col_term;
     } else if (pr.a_unsigned) {  // + 128 * sum_k b'[n,k] per column
@@ -713,8 +713,9 @@ bool fold_batches(const VecopsHipOperand* o, VecopsHipOperand* flat) {
   return true;
 }
 
-int32_t describe_runtime_quant(const VecopsHipOperand* a_given, const VecopsHipOperand* b, const VecopsHipOperand* c_given,
-                               void* workspace, RuntimeQuant* d) {
+// b is the int8 operand, or null with `packed` / `packed_n` describing weights packed by vecops_hip_pack_b.
+int32_t describe_runtime_quant(const VecopsHipOperand* a_given, const VecopsHipOperand* b, const void* packed,
+                               int64_t packed_n, const VecopsHipOperand* c_given, void* workspace, RuntimeQuant* d) {
   if (a_given == nullptr || c_given == nullptr || a_given->rank != c_given->rank ||
       (a_given->rank == 3 && a_given->sizes[0] != c_given->sizes[0]))
     return fail(ST_INVALID, "matmul_runtime_quant: a and c must have the same rank and batch extent");
@@ -725,16 +726,18 @@ int32_t describe_runtime_quant(const VecopsHipOperand* a_given, const VecopsHipO
   const VecopsHipOperand* a = &d->a_flat;
   const VecopsHipOperand* c = &d->c_flat;
   if (a->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: a must be an f32 operand");
-  if (b == nullptr || b->rank != 2 || b->dtype != DT_I8) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: b must be a rank-2 i8 operand");
+  if (packed == nullptr && (b == nullptr || b->rank != 2 || b->dtype != DT_I8))
+    return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: b must be a rank-2 i8 operand");
   if (c->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: c must be an f32 operand");
-  if (a->sizes[0] < 0 || a->sizes[1] < 0 || b->sizes[0] < 0) return fail(ST_INVALID, "matmul_runtime_quant: negative extent");
-  const int64_t m = a->sizes[0], k = a->sizes[1], n = b->sizes[0];
+  const int64_t m = a->sizes[0], k = a->sizes[1], n = packed ? packed_n : b->sizes[0];
+  if (m < 0 || k < 0 || n < 0) return fail(ST_INVALID, "matmul_runtime_quant: negative extent");
   d->q_bytes = (static_cast<uint64_t>(m) * static_cast<uint64_t>(k) + 255u) & ~uint64_t{255};
   d->row_bytes = (static_cast<uint64_t>(n) * 4u + 255u) & ~uint64_t{255};
   make_operand(&d->q, workspace, DT_I8, m, k, k);
   d->c_acc = *c;
   d->c_acc.dtype = DT_I32;  // accumulator class; the epilogue writes fp32
-  int32_t rc = describe(&d->q, b, nullptr, &d->c_acc, 0, &d->pr);
+  int32_t rc = packed ? describe_packed(&d->q, packed, DT_I8, n, nullptr, &d->c_acc, &d->pr)
+                      : describe(&d->q, b, nullptr, &d->c_acc, 0, &d->pr);
   if (rc != ST_OK) return rc;
   d->pr.dequant = true;
   choose(d->pr, &d->plan);
@@ -742,23 +745,18 @@ int32_t describe_runtime_quant(const VecopsHipOperand* a_given, const VecopsHipO
 }
 }  // namespace
 
-uint64_t vecops_hip_matmul_runtime_quant_workspace(const VecopsHipOperand* a, const VecopsHipOperand* b,
-                                                   const VecopsHipOperand* c) {
+namespace {
+int32_t run_runtime_quant(const VecopsHipOperand* a, const float* multipliers, int32_t zero_point, const VecopsHipOperand* b,
+                          const void* packed, int64_t packed_n, const int32_t* correction, const float* row_scales,
+                          const float* column_scales, const VecopsHipOperand* c, void* workspace, uint64_t workspace_size,
+                          void* stream) {
   RuntimeQuant d;
-  if (describe_runtime_quant(a, b, c, reinterpret_cast<void*>(256), &d) != ST_OK) return 0;
-  return d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
-}
-
-int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* multipliers, int32_t zero_point,
-                                        const VecopsHipOperand* b, const int32_t* correction, const float* row_scales,
-                                        const float* column_scales, const VecopsHipOperand* c, void* workspace,
-                                        uint64_t workspace_size, void* stream) {
-  RuntimeQuant d;
-  int32_t rc = describe_runtime_quant(a, b, c, workspace ? workspace : reinterpret_cast<void*>(256), &d);
+  int32_t rc = describe_runtime_quant(a, b, packed, packed_n, c, workspace ? workspace : reinterpret_cast<void*>(256), &d);
   if (rc != ST_OK) return rc;
   if (d.plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
   if (row_scales == nullptr || column_scales == nullptr || multipliers == nullptr)
     return fail(ST_INVALID, "matmul_runtime_quant: multipliers and both scale vectors are required");
+  if (packed != nullptr && d.pr.k > 0 && !aligned16(packed)) return fail(ST_INVALID, "matmul_runtime_quant: packed b must be 16-byte aligned");
   const uint64_t need = d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
   if (need > workspace_size || workspace == nullptr || !aligned16(workspace))
     return fail(ST_INVALID, "matmul_runtime_quant: %llu bytes of 16-byte aligned workspace required, %llu supplied",
@@ -774,11 +772,49 @@ int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* 
   // correction[n] + 128 * sum_k b[n,k]
   int32_t* row = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + d.q_bytes);
   const View& vb = d.pr.b;
-  e = launch_byte_row_sums(vb.data, 1, static_cast<int32_t>(vb.rows), static_cast<int32_t>(vb.cols), 0, vb.rs, vb.cs, 0u,
-                           128u, correction, row, s);
+  if (packed != nullptr)
+    e = launch_packed_row_sums(packed, static_cast<int32_t>(d.pr.n), static_cast<int32_t>(d.pr.k), 1, 128u, correction, row, s);
+  else
+    e = launch_byte_row_sums(vb.data, 1, static_cast<int32_t>(vb.rows), static_cast<int32_t>(vb.cols), 0, vb.rs, vb.cs, 0u,
+                             128u, correction, row, s);
   if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
   return run_problem(d.pr, d.plan, row_scales, column_scales, row, static_cast<char*>(workspace) + d.q_bytes + d.row_bytes,
                      workspace_size - d.q_bytes - d.row_bytes, s);
+}
+}  // namespace
+
+uint64_t vecops_hip_matmul_runtime_quant_workspace(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                   const VecopsHipOperand* c) {
+  RuntimeQuant d;
+  if (describe_runtime_quant(a, b, nullptr, 0, c, reinterpret_cast<void*>(256), &d) != ST_OK) return 0;
+  return d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
+}
+
+int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* multipliers, int32_t zero_point,
+                                        const VecopsHipOperand* b, const int32_t* correction, const float* row_scales,
+                                        const float* column_scales, const VecopsHipOperand* c, void* workspace,
+                                        uint64_t workspace_size, void* stream) {
+  if (b == nullptr) return fail(ST_INVALID, "matmul_runtime_quant: null b");
+  return run_runtime_quant(a, multipliers, zero_point, b, nullptr, 0, correction, row_scales, column_scales, c, workspace,
+                           workspace_size, stream);
+}
+
+uint64_t vecops_hip_matmul_runtime_quant_packed_b_workspace(const VecopsHipOperand* a, int64_t n, const VecopsHipOperand* c) {
+  RuntimeQuant d;
+  if (describe_runtime_quant(a, nullptr, reinterpret_cast<const void*>(256), n, c, reinterpret_cast<void*>(256), &d) != ST_OK)
+    return 0;
+  return d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
+}
+
+int32_t vecops_hip_matmul_runtime_quant_packed_b(const VecopsHipOperand* a, const float* multipliers, int32_t zero_point,
+                                                 const void* packed_b, int64_t n, const int32_t* correction,
+                                                 const float* row_scales, const float* column_scales,
+                                                 const VecopsHipOperand* c, void* workspace, uint64_t workspace_size,
+                                                 void* stream) {
+  if (packed_b == nullptr && n > 0 && a != nullptr && a->sizes[a->rank - 1] > 0)
+    return fail(ST_INVALID, "matmul_runtime_quant_packed_b: null packed b");
+  return run_runtime_quant(a, multipliers, zero_point, nullptr, packed_b ? packed_b : reinterpret_cast<const void*>(256), n,
+                           correction, row_scales, column_scales, c, workspace, workspace_size, stream);
 }
 
 uint32_t vecops_hip_abi_version(void) { return VECOPS_HIP_ABI_VERSION; }

@@ -42,9 +42,9 @@ hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_
 // vector_a: 0 = any strides, 1 = A is K-contiguous, 2 = and its base, rows and batches are 16-byte aligned
 hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_m, int tile_n, int vector_a,
                                      hipStream_t stream);
-// out[b][n] = scale * sum_k B[n,k] of an int8-packed operand, for b < batch
-hipError_t launch_packed_row_sums(const void* packed, int32_t n, int32_t k, int32_t batch, uint32_t scale, int32_t* out,
-                                  hipStream_t stream);
+// out[b][n] = scale * sum_k B[n,k] (+ add[n], may be null) of an int8-packed operand, for b < batch
+hipError_t launch_packed_row_sums(const void* packed, int32_t n, int32_t k, int32_t batch, uint32_t scale,
+                                  const int32_t* add, int32_t* out, hipStream_t stream);
 struct PackBParams;
 hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream);
 

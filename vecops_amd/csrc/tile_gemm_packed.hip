@@ -66,11 +66,11 @@ hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_
   }
 }
 
-// out[b][n] = scale * sum_k B[n,k] for an int8 packed operand, once per batch b: the per-column term of an
+// out[b][n] = scale * sum_k B[n,k] (+ add[n], may be null) for an int8 packed operand, once per batch b: the per-column term of an
 // unsigned A (a xor 0x80 is multiplied, 128 * sum_k B[n,k] comes back here; wrapping).  One wavefront per
 // 32-row block walks its k-steps as one contiguous stream; lanes l and l + 32 hold the two halves of a row.
 __global__ __launch_bounds__(256) void packed_row_sums_kernel(const void* packed, int32_t n, int32_t k, int32_t batch,
-                                                              uint32_t scale, int32_t* out) {
+                                                              uint32_t scale, const int32_t* add, int32_t* out) {
   const int lane = threadIdx.x & 63;
   const int64_t nb = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (nb * 32 >= n) return;
@@ -88,17 +88,17 @@ __global__ __launch_bounds__(256) void packed_row_sums_kernel(const void* packed
   sum += __shfl_xor(sum, 32, 64);
   const int64_t row = nb * 32 + lane;
   if (lane < 32 && row < n) {
-    const int32_t term = static_cast<int32_t>(static_cast<uint32_t>(sum) * scale);
+    const int32_t term = static_cast<int32_t>(static_cast<uint32_t>(sum) * scale + (add ? static_cast<uint32_t>(add[row]) : 0u));
     for (int32_t b = 0; b < batch; ++b) out[static_cast<int64_t>(b) * n + row] = term;
   }
 }
 
-hipError_t launch_packed_row_sums(const void* packed, int32_t n, int32_t k, int32_t batch, uint32_t scale, int32_t* out,
-                                  hipStream_t stream) {
+hipError_t launch_packed_row_sums(const void* packed, int32_t n, int32_t k, int32_t batch, uint32_t scale,
+                                  const int32_t* add, int32_t* out, hipStream_t stream) {
   if (n <= 0 || batch <= 0) return hipSuccess;
   const int64_t blocks = ((static_cast<int64_t>(n) + 31) / 32 + 3) / 4;
   hipLaunchKernelGGL(packed_row_sums_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, packed, n, k, batch,
-                     scale, out);
+                     scale, add, out);
   return hipGetLastError();
 }
 
