@@ -94,6 +94,23 @@ def test_abi_layout(tmp_path):
         assert ours == theirs
 
 
+def test_host_library_exports_every_declared_symbol(host):
+    import ctypes
+    import re
+    text = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include",
+                             "vecops_hip_host.h")).read()
+    names = sorted(set(re.findall(r"VECOPS_HIP_HOST_EXPORT[^;(]*?\b(vecops_hip_host_\w+)\s*\(", text)))
+    assert len(names) == 7
+    lib = ctypes.CDLL(H.HOST_LIB)
+    for name in names:
+        assert getattr(lib, name) is not None
+    for name in ("vecops::matmul", "vecops::matmul_fused", "vecops::matmul_i8_dequant", "vecops::matmul_runtime_quant",
+                 "vecops::matmul_pack_b", "vecops::matmul_packed_b", "vecops::matmul_w8a16_group"):
+        assert host.operator(name) is not None
+    with pytest.raises(Exception):
+        host.operator("vecops::no_such_operator")
+
+
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
     assert len(files) == 36
