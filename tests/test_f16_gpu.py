@@ -90,3 +90,25 @@ def test_f16_fused_and_dtype_rules(device, oracle):
     with pytest.raises(capi.VecopsHipError) as info:          # nor mix with bf16 operands
         capi.matmul(_dev(a, device), torch.zeros((n, k), dtype=torch.bfloat16, device=device), c)
     assert info.value.code == 2
+
+
+@pytest.mark.parametrize("narrow,wide,k", [(1, 14336, 4096), (4, 4096, 1024), (16, 2048, 4096), (3, 600, 136)])
+@pytest.mark.parametrize("out", ["f32", "f16"])
+def test_f16_skinny_family(device, oracle, narrow, wide, k, out):
+    """Half operands on the skinny kernels (v_mfma_f32_16x16x32_f16), either operand the narrow one."""
+    import torch
+    from vecops_amd import capi
+    for m, n in ((narrow, wide), (wide, narrow)):
+        a, b = _half(1, (m, k)), _half(2, (n, k))
+        ta, tb = _dev(a, device), _dev(b, device)
+        c = torch.full((m, n), float("nan"), dtype=torch.float32 if out == "f32" else torch.float16, device=device)
+        assert capi.FAMILY_NAMES[capi.plan_matmul(ta, tb, c).family] == "skinny"
+        capi.matmul(ta, tb, c)
+        torch.cuda.synchronize()
+        want = np.zeros((m, n), np.float32 if out == "f32" else np.float16)
+        oracle.matmul(a, b, want, atom=O.ATOM_F16F32, acc_f64=True)
+        got = c.cpu().numpy()
+        if out == "f32":
+            assert rel_err(got, want) <= 2e-6 * max(1.0, k / 32)
+        else:
+            assert rel_err(got.astype(np.float32), want.astype(np.float32)) <= 2.0 ** -10

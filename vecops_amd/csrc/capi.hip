@@ -198,10 +198,10 @@ constexpr int kStreamGroupsPerUnit = 2;  // workgroups of 4 wavefronts per compu
 // workgroups share a compute unit).
 constexpr int64_t kQuality256x128 = 800, kQuality128 = 820;
 
-// bf16 x bf16 or int8 x int8 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
+// bf16 x bf16, f16 x f16 or int8 x int8 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
 bool skinny_applies(const Problem& pr) {
   if (pr.fused) return false;  // the skinny kernels have no output transform
-  if ((pr.src != SRC_BF16 && pr.src != SRC_I8) || pr.has_cin || pr.packed_b) return false;
+  if ((pr.src != SRC_BF16 && pr.src != SRC_F16 && pr.src != SRC_I8) || pr.has_cin || pr.packed_b) return false;
   const int64_t per = pr.src == SRC_I8 ? 16 : 8;  // elements per 16 bytes
   if (!k_vector_ok(pr.a) || !k_vector_ok(pr.b) || pr.k % per != 0 || pr.k < 8 * per) return false;
   const int64_t narrow = pr.m < pr.n ? pr.m : pr.n, wide = pr.m < pr.n ? pr.n : pr.m;
@@ -396,7 +396,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
       q.wide_scales = column_scales;
       q.wide_term = correction;
     } else {
-      q.out_kind = pr.out_kind == OUT_BF16 ? SKINNY_OUT_BF16 : SKINNY_OUT_F32;
+      q.out_kind = pr.out_kind == OUT_BF16 ? SKINNY_OUT_BF16 : pr.out_kind == OUT_F16 ? SKINNY_OUT_F16 : SKINNY_OUT_F32;
     }
     // 64 wide rows per workgroup when that still leaves most compute units a workgroup, else 32 or 16
     const int64_t wgs64 = (wide.rows + 63) / 64 * pr.batch;
@@ -415,6 +415,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
       }
     };
     if (is_int) launch(std::integral_constant<int, SRC_I8>{});
+    else if (pr.src == SRC_F16) launch(std::integral_constant<int, SRC_F16>{});
     else launch(std::integral_constant<int, SRC_BF16>{});
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(ST_EXEC, "skinny kernel launch: %s", hipGetErrorString(e));

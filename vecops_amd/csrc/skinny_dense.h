@@ -7,7 +7,7 @@
 // matmul/details/kernel/amx/Backend.h:767-1151): the wide operand is read exactly
 // once, the narrow one is kept in registers.
 //
-// One v_mfma_f32_16x16x32_bf16 (v_mfma_i32_16x16x64_i8) multiplies 16 wide rows by 16
+// One v_mfma_f32_16x16x32_bf16 (_f16 for half operands; v_mfma_i32_16x16x64_i8) multiplies 16 wide rows by 16
 // narrow rows (S padded to 16 with zeros) over a step of 32 (64) k.  Lane l holds wide
 // row l % 16 and the 16 consecutive bytes of quarter l / 16 of the step (one 16-byte
 // load); the narrow operand uses the same k order.  A workgroup of 8 wavefronts owns
@@ -26,7 +26,7 @@
 
 namespace vecops_hip {
 
-enum SkinnyOut : int { SKINNY_OUT_F32 = 0, SKINNY_OUT_BF16 = 1, SKINNY_OUT_I32 = 2, SKINNY_OUT_DEQUANT_F32 = 3 };
+enum SkinnyOut : int { SKINNY_OUT_F32 = 0, SKINNY_OUT_BF16 = 1, SKINNY_OUT_I32 = 2, SKINNY_OUT_DEQUANT_F32 = 3, SKINNY_OUT_F16 = 4 };
 
 struct SkinnyDenseParams {
   const void* w;      // wide operand (bf16 bits or int8)
@@ -104,7 +104,11 @@ __global__ __launch_bounds__(512) void skinny_dense_kernel(const SkinnyDensePara
         if constexpr (INT)
           acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, wq[slot]),
                                                          __builtin_bit_cast(i32x4, xq[s]), acc[b], 0, 0, 0);
-        else
+        else if constexpr (SRC == SRC_F16) {
+          typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wq[slot]),
+                                                          __builtin_bit_cast(f16x8, xq[s]), acc[b], 0, 0, 0);
+        } else
           acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wq[slot]),
                                                            __builtin_bit_cast(bf16x8, xq[s]), acc[b], 0, 0, 0);
         constexpr int ns = s + D;  // the step that takes over this slot
@@ -143,6 +147,7 @@ __global__ __launch_bounds__(512) void skinny_dense_kernel(const SkinnyDensePara
           }
         } else {
           if (p.out_kind == SKINNY_OUT_BF16) static_cast<uint16_t*>(p.y)[at] = static_cast<uint16_t>(bf16_bits_rne(total));
+          else if (p.out_kind == SKINNY_OUT_F16) static_cast<uint16_t*>(p.y)[at] = static_cast<uint16_t>(f16_bits_rne(total));
           else static_cast<float*>(p.y)[at] = total;
         }
       }
