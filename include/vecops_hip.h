@@ -267,7 +267,7 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t l
  * rows past N and k past K are zero.
  *
  * packed dtypes: 11 bf16 (from a bf16 or f32 source; f32 is rounded to nearest
- * even, as the matmul itself rounds it) and 2 i8.
+ * even, as the matmul itself rounds it), 10 f16 and 2 i8.
  */
 
 /* Bytes of the packed form of a [N,K] operand; 0 for an unsupported dtype. */
@@ -296,6 +296,7 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul_packed_b(const VecopsHipOperand
  * operand serves every batch of a rank-3 A (vecops: a packed tensor passed as B
  * lets the planner skip the packing stage, ops/MatmulPack.h:22-24).
  *   packed bf16: a bf16 or f32 (rounded to bf16), c f32|bf16
+ *   packed f16 : a f16, c f32|f16
  *   packed i8  : a i8 or u8 (AMX_I8I32<uint8_t, int8_t>, the atom the compensated pack serves,
  *                ops/MatmulPack.h:52-58; the workspace then also holds 4 * batch * (M + N) bytes), c i32
  * Same results, bit for bit, as vecops_hip_matmul on the unpacked operand when

@@ -112,3 +112,28 @@ def test_f16_skinny_family(device, oracle, narrow, wide, k, out):
             assert rel_err(got, want) <= 2e-6 * max(1.0, k / 32)
         else:
             assert rel_err(got.astype(np.float32), want.astype(np.float32)) <= 2.0 ** -10
+
+
+@pytest.mark.parametrize("m,n,k", [(300, 260, 1000), (37, 51, 79), (512, 768, 512), (2, 3, 64, 40, 200)][:3] + [(2457, 1221, 72)])
+def test_f16_prepacked_b(device, oracle, m, n, k):
+    """Half weights packed once (the 16-bit permutation of the bf16 pack): bit-equal to the plain product."""
+    import torch
+    from vecops_amd import capi
+    a, b = _half(1, (m, k)), _half(2, (n, k))
+    ta, tb = _dev(a, device), _dev(b, device)
+    packed = capi.pack_b(tb)
+    assert packed.dtype == capi.F16
+    for dt in (torch.float32, torch.float16):
+        c, ref = (torch.full((m, n), float("nan"), dtype=dt, device=device) for _ in range(2))
+        capi.matmul_packed_b(ta, packed, c)
+        capi.matmul(ta, tb, ref)
+        torch.cuda.synchronize()
+        assert torch.equal(c.view(torch.int32 if dt == torch.float32 else torch.int16),
+                           ref.view(torch.int32 if dt == torch.float32 else torch.int16))
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, atom=O.ATOM_F16F32, acc_f64=True)
+    c = torch.empty((m, n), device=device)
+    capi.matmul_packed_b(ta, packed, c)
+    assert rel_err(c.cpu().numpy(), want) <= 2e-6 * max(1.0, k / 32)
+    with pytest.raises(capi.VecopsHipError):                 # a bf16 a against f16-packed weights
+        capi.matmul_packed_b(ta.to(torch.bfloat16), packed, c)

@@ -294,7 +294,7 @@ def pack_b(b, a_zero_point=None, stream=None):
     """
     import torch
     n, k = b.shape
-    dtype = I8 if b.dtype == torch.int8 else BF16
+    dtype = I8 if b.dtype == torch.int8 else F16 if b.dtype == torch.float16 else BF16
     size = lib().vecops_hip_packed_b_bytes(dtype, n, k)
     storage = torch.empty(max(size, 16), dtype=torch.uint8, device=b.device)
     ob = operand(b)

@@ -480,7 +480,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     }
   }
   if (pr.packed_b) {
-    const int a_mode = plan.vector_a == 0 ? 0 : ((pr.src == SRC_BF16 || pr.src == SRC_I8) && lines_up(pr.a, pr.a.rs)) ? 2 : 1;
+    const int a_mode = plan.vector_a == 0 ? 0 : ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr.a, pr.a.rs)) ? 2 : 1;
     e = launch_tile_gemm_packed_b(pr.src, p, tile_m, tile_n, a_mode, stream);
   } else switch (pr.src) {
     case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile_m, tile_n, mode, stream); break;
@@ -543,6 +543,8 @@ int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t 
   const uint32_t da = a->dtype;
   if (packed_dtype == DT_BF16) {
     if (da != DT_BF16 && da != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: a bf16-packed b needs a bf16 or f32 a");
+  } else if (packed_dtype == DT_F16) {
+    if (da != DT_F16) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an f16-packed b needs an f16 a");
   } else if (packed_dtype == DT_I8) {
     if (da != DT_I8 && da != DT_U8) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an i8-packed b needs an i8 or u8 a");
   } else {
@@ -570,7 +572,8 @@ int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t 
 }
 
 int src_of_packed_source(uint32_t dtype) {
-  return dtype == DT_BF16 ? SRC_BF16 : dtype == DT_F32 ? SRC_F32_AS_BF16 : dtype == DT_I8 ? SRC_I8 : -1;
+  // (half operands are packed by the bf16 kernel: a permutation of 16-bit elements either way)
+  return (dtype == DT_BF16 || dtype == DT_F16) ? SRC_BF16 : dtype == DT_F32 ? SRC_F32_AS_BF16 : dtype == DT_I8 ? SRC_I8 : -1;
 }
 
 }  // namespace
@@ -578,7 +581,7 @@ int src_of_packed_source(uint32_t dtype) {
 extern "C" {
 
 uint64_t vecops_hip_packed_b_bytes(uint32_t packed_dtype, int64_t n, int64_t k) {
-  if (n < 0 || k < 0 || (packed_dtype != DT_BF16 && packed_dtype != DT_I8)) return 0;
+  if (n < 0 || k < 0 || (packed_dtype != DT_BF16 && packed_dtype != DT_F16 && packed_dtype != DT_I8)) return 0;
   return static_cast<uint64_t>(packed_b_bytes(n, k, packed_dtype == DT_I8 ? 16 : 8));
 }
 

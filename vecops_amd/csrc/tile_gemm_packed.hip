@@ -41,7 +41,7 @@ template <int SRC>
 hipError_t launch_packed_class(const TileGemmParams& p, int tile_m, int tile_n, int vector_a, hipStream_t stream) {
   // vector_a: 0 element loads, 1 16-byte loads, 2 16-byte loads that write LDS themselves (aligned bf16 / int8 A,
   // the three big tiles)
-  if constexpr (SRC == SRC_BF16 || SRC == SRC_I8) {
+  if constexpr (SRC == SRC_BF16 || SRC == SRC_F16 || SRC == SRC_I8) {
     if (vector_a == 2 && tile_m * tile_n >= 256 * 128) {
       if (tile_m == 256 && tile_n == 256) return launch_packed_instance<SRC, 2, 2, 4, 4, LOAD_KDMA>(p, stream);
       if (tile_m == 256 && tile_n == 128) return launch_packed_instance<SRC, 2, 2, 4, 2, LOAD_KDMA>(p, stream);
@@ -58,6 +58,7 @@ hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_
                                      hipStream_t stream) {
   switch (src) {
     case SRC_BF16: return launch_packed_class<SRC_BF16>(p, tile_m, tile_n, vector_a, stream);
+    case SRC_F16: return launch_packed_class<SRC_F16>(p, tile_m, tile_n, vector_a, stream);
     case SRC_F32_AS_BF16: return launch_packed_class<SRC_F32_AS_BF16>(p, tile_m, tile_n, vector_a, stream);
     case SRC_I8: return launch_packed_class<SRC_I8>(p, tile_m, tile_n, vector_a, stream);
     // unsigned A: xored on its way into LDS, so never by the loads that write LDS themselves
