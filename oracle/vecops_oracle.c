@@ -361,7 +361,8 @@ VO_EXPORT void vo_quantize_rows_u8(const float* a, int64_t M, int64_t K, int64_t
 }
 
 /* Selected outputs of the rank-2 product only: out[s] = acc(rows_idx[s], cols_idx[s])
- * as double (floating atoms) - lets a test check a 4096^3 product in seconds. */
+ * as double (floating atoms) - lets a test check a 4096^3 product in seconds.  Pinned against
+ * vo_matmul's float64 accumulators at the same indices (tests/test_oracle.py). */
 VO_EXPORT int vo_matmul_sampled(const vo_tensor* a, const vo_tensor* b, int atom, const int64_t* rows_idx,
                                 const int64_t* cols_idx, int64_t count, double* out) {
   if (a->rank != 2 || b->rank != 2 || cols(a) != cols(b)) return 1;
@@ -427,6 +428,9 @@ VO_EXPORT void vo_matmul_i8_dequant(const int8_t* a, const int8_t* b, const floa
  *   y[m,n] = bf16_rne( sum_g S[n,g] * sum_{k in group g} float(x[m,k]) * float(W[n,k]) )
  * x bf16 [M,K], W int8 [N,K], S fp32 [N,K/G], y bf16 [M,N].  Accumulated here
  * in double; kernels accumulate in fp32 and are compared with a tolerance.
+ * Pinned (tests/test_oracle.py, test_w8a16_group_*) by a numpy float64 einsum that shares
+ * no loop with this one, by unit scales reducing it to vo_matmul, by one group's scale
+ * moving exactly that group's dot, and by a hand-worked table.
  */
 VO_EXPORT int vo_matmul_w8a16_group(const uint16_t* x, const int8_t* w, const float* scales, uint16_t* y,
                                     double* y_f64, int64_t M, int64_t N, int64_t K, int64_t G) {

@@ -362,3 +362,110 @@ def test_f16_atom_matches_fp64_product(oracle):
     oracle.matmul(a32, b32, c32, atom=O.ATOM_F16F32, acc_f64=True)
     want32 = a32.astype(np.float16).astype(np.float64) @ b32.astype(np.float16).astype(np.float64).T
     assert np.array_equal(c32, want32.astype(np.float32))
+
+
+# --- weight-only int8 with per-group scales (no reference counterpart) -----------------
+
+def _w8a16_inputs(seed, m, n, k, group):
+    rng = np.random.default_rng(seed)
+    x = synth.bf16_to_f32(synth.bf16_round(rng.standard_normal((m, k)).astype(np.float32)))   # bf16-exact fp32
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    s = (2.0 ** -7 * (1.0 + rng.random((n, k // group)))).astype(np.float32)
+    return x, w, s
+
+
+@pytest.mark.parametrize("m,n,k,group", [(1, 5, 32, 16), (3, 7, 128, 128), (4, 9, 256, 64), (16, 33, 384, 128),
+                                         (2, 1, 512, 256), (5, 6, 48, 16)])
+def test_w8a16_group_matches_an_independent_fp64_evaluation(oracle, m, n, k, group):
+    """y = sum_g S[n,g] * sum_{k in g} x[m,k] * W[n,k], evaluated by numpy in float64 through an einsum over the
+    [groups, group] reshaping - shares no code and no loop structure with the oracle; G = 16, one group and
+    N = 1 included.  The bf16 result is the pinned rounding of that float64 sum rounded to fp32."""
+    x, w, s = _w8a16_inputs(10 + m, m, n, k, group)
+    groups = k // group
+    xg = x.astype(np.float64).reshape(m, groups, group)
+    wg = w.astype(np.float64).reshape(n, groups, group)
+    want = np.einsum("mgk,ngk,ng->mn", xg, wg, s.astype(np.float64))
+    y_bits, y64 = oracle.matmul_w8a16_group(synth.bf16_round(x), w, s, group)
+    assert np.allclose(y64, want, rtol=1e-13, atol=1e-13)
+    assert np.array_equal(y_bits, oracle.bf16_from_f32(y64.astype(np.float32)))
+
+
+def test_w8a16_group_with_unit_scales_is_the_pinned_plain_product(oracle):
+    """All scales 1: the contract reduces to x . W^T, which vo_matmul (pinned by the real reference and by fp64
+    products) computes on the weights widened to bf16 (every int8 is a bf16 value)."""
+    m, n, k, group = 4, 21, 256, 128
+    x, w, _ = _w8a16_inputs(3, m, n, k, group)
+    ones = np.ones((n, k // group), np.float32)
+    _, y64 = oracle.matmul_w8a16_group(synth.bf16_round(x), w, ones, group)
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(x, w.astype(np.float32), want, acc_f64=True)   # fp32 memory -> bf16 compute: exact for int8 values
+    assert np.array_equal(y64.astype(np.float32), want)
+
+
+def test_w8a16_group_scale_of_one_group_moves_exactly_that_groups_dot(oracle):
+    """Doubling S[n0, g0] adds S[n0, g0] * (x[:, g0] . W[n0, g0]) to column n0 and nothing anywhere else - fails
+    when the scale index (n * groups + g) or a group boundary is off by one."""
+    m, n, k, group = 3, 8, 512, 128
+    x, w, s = _w8a16_inputs(5, m, n, k, group)
+    _, base = oracle.matmul_w8a16_group(synth.bf16_round(x), w, s, group)
+    for n0, g0 in [(0, 0), (5, 3), (7, 1)]:
+        s2 = s.copy()
+        s2[n0, g0] *= 2.0
+        _, moved = oracle.matmul_w8a16_group(synth.bf16_round(x), w, s2, group)
+        part = np.zeros((m, 1), np.float32)
+        oracle.matmul(np.ascontiguousarray(x[:, g0 * group:(g0 + 1) * group]),
+                      np.ascontiguousarray(w[n0:n0 + 1, g0 * group:(g0 + 1) * group]).astype(np.float32), part, acc_f64=True)
+        want = np.zeros_like(base)
+        want[:, n0] = float(s[n0, g0]) * part[:, 0].astype(np.float64)
+        # the pinned routine hands the group's dot back rounded to fp32: 2^-24 relative
+        assert np.allclose(moved - base, want, rtol=2e-7, atol=1e-9)
+        other = np.ones(n, bool)
+        other[n0] = False
+        assert np.array_equal(moved[:, other], base[:, other])
+
+
+def test_w8a16_group_known_answer(oracle):
+    """Worked by hand.  x[0] = 1 everywhere, x[1] = k % 4 - 1.5 (bf16-exact); W[0] = 1, W[1, k] = k - 16 for K = 32,
+    two groups of 16; S = [[0.5, 2], [0.25, -1]].
+      row 0 of x: W[0] -> 0.5*16 + 2*16 = 40;  W[1]: group sums -136 and 120 -> 0.25*-136 + -1*120 = -154
+      row 1 of x: per 4 elements the pattern sums to 0 against W[0] -> 0; against W[1]: sum over a group of
+      (k%4 - 1.5)(k - 16) = sum (k%4 - 1.5) k = 4 blocks * 5 = 20 per group -> 0.25*20 - 20 = -15."""
+    k = np.arange(32)
+    x = np.stack([np.ones(32), k % 4 - 1.5]).astype(np.float32)
+    w = np.stack([np.ones(32), k - 16]).astype(np.int8)
+    s = np.array([[0.5, 2.0], [0.25, -1.0]], np.float32)
+    y_bits, y64 = oracle.matmul_w8a16_group(synth.bf16_round(x), w, s, 16)
+    assert np.array_equal(y64, np.array([[40.0, -154.0], [0.0, -15.0]]))
+    assert np.array_equal(y_bits, np.array([[0x4220, 0xC31A], [0x0000, 0xC170]], np.uint16))
+
+
+def test_w8a16_group_rejects_a_ragged_group(oracle):
+    x, w, s = _w8a16_inputs(1, 1, 2, 48, 16)
+    with pytest.raises(ValueError):
+        oracle.matmul_w8a16_group(synth.bf16_round(x), w, s, 32)
+
+
+# --- sampled products (the checker of the full-size tests) -----------------------------
+
+@pytest.mark.parametrize("kind", ["bf16_ragged", "f32_memory", "kn_view"])
+def test_sampled_product_equals_the_full_product_at_the_sampled_indices(oracle, kind):
+    """vo_matmul_sampled(i, j) == vo_matmul(acc_f64)[i, j] (the latter pinned above) on a ragged bf16 case, on
+    fp32 memory rounded to bf16 on the way in, and with B handed over as a [K,N] view (strides (1, N))."""
+    m, n, k = 37, 45, 131
+    a = synth.uniform_pm1(21, (m, k))
+    b = synth.uniform_pm1(22, (n, k))
+    if kind != "f32_memory":
+        a, b = synth.bf16_round(a), synth.bf16_round(b)   # bf16 bits
+    if kind == "kn_view":
+        b = np.ascontiguousarray(b.T).T   # [N,K] view of a [K,N] array
+        assert b.strides == (b.itemsize, b.itemsize * n)
+    rng = np.random.default_rng(9)
+    rows = np.concatenate([rng.integers(0, m, 200), [0, m - 1, 0, m - 1]])
+    cols = np.concatenate([rng.integers(0, n, 200), [0, n - 1, n - 1, 0]])
+    got = oracle.matmul_sampled(a, b, rows, cols)
+    full = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, full, acc_f64=True)
+    assert np.array_equal(got.astype(np.float32), full[rows, cols])
+    as_f64 = lambda v: synth.bf16_to_f32(v if v.dtype == np.uint16 else synth.bf16_round(np.ascontiguousarray(v))).astype(np.float64)
+    want64 = as_f64(np.ascontiguousarray(a)) @ as_f64(np.ascontiguousarray(b)).T
+    assert np.allclose(got, want64[rows, cols], rtol=1e-13, atol=1e-13)
