@@ -114,6 +114,24 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul(const VecopsHipOperand* a, const Vec
                                             void* workspace, uint64_t workspace_size, void* stream);
 
 /*
+ * vecops_hip_matmul without a workspace argument, for callers that cannot allocate device memory at all:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
+ * vecops (its callers size and own every workspace, ops/Matmul.h:504-526).  The split-K partial sums and the
+ * unsigned-operand terms live in a buffer of VECOPS_HIP_STATIC_WORKSPACE_BYTES that belongs to the library's
+ * code object on each GPU (8 MiB, held until the process ends; split-K plans need at most 4 MiB, the row
+ * sums of unsigned operands 4 bytes per row of a and b); the call allocates and frees nothing.  A call whose
+ * plan needs more (vecops_hip_plan_matmul(...).workspace_bytes) returns 2 (not applicable) and launches
+ * nothing.  Same kernels and therefore the same results, bit for bit, as vecops_hip_matmul.  Every call on
+ * one GPU shares that GPU's buffer: calls that overlap on one GPU (different streams or host threads) race;
+ * calls on one stream, or otherwise ordered, do not.
+ */
+#define VECOPS_HIP_STATIC_WORKSPACE_BYTES (8u << 20)
+VECOPS_HIP_EXPORT uint64_t vecops_hip_static_workspace_bytes(void);
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_static_workspace(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                             const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                             uint32_t compute, void* stream);
+
+/*
  * Fused output transforms - the catalogue that vecops' tests build from
  * elementwise and lane-local output transforms on tensor::output
  * (tests/ops/MatmulFusionTest.cpp:29-112; tests/ops/MatmulConversionTestCommon.h:

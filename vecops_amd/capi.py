@@ -27,6 +27,7 @@ EXPORTS = [
     "vecops_hip_plan_matmul_fused", "vecops_hip_matmul_fused", "vecops_hip_quantize_rows",
     "vecops_hip_matmul_runtime_quant_workspace", "vecops_hip_matmul_runtime_quant",
     "vecops_hip_matmul_runtime_quant_packed_b_workspace", "vecops_hip_matmul_runtime_quant_packed_b",
+    "vecops_hip_static_workspace_bytes", "vecops_hip_matmul_static_workspace",
 ]
 
 ACT_NONE, ACT_RELU, ACT_CLAMP, ACT_SIGMOID, ACT_SILU = 0, 1, 2, 3, 4
@@ -73,6 +74,8 @@ def lib() -> C.CDLL:
         P = C.POINTER(Operand)
         L.vecops_hip_plan_matmul.argtypes = [P, P, P, P, C.c_uint32, C.POINTER(Plan)]
         L.vecops_hip_matmul.argtypes = [P, P, P, P, C.c_uint32, C.c_void_p, C.c_uint64, C.c_void_p]
+        L.vecops_hip_static_workspace_bytes.restype = C.c_uint64
+        L.vecops_hip_matmul_static_workspace.argtypes = [P, P, P, P, C.c_uint32, C.c_void_p]
         L.vecops_hip_matmul_i8_dequant.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p,
                                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
                                                    C.c_int64, C.c_int64, C.c_void_p, C.c_uint64, C.c_void_p]
@@ -164,6 +167,16 @@ def matmul(a, b, c, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None
     ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
     _check(lib().vecops_hip_matmul(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None, C.byref(oc),
                                    compute, ws_ptr, ws_size, _stream_handle(stream)))
+    return c
+
+
+def matmul_static_workspace(a, b, c, c_in=None, compute=COMPUTE_BF16, stream=None):
+    """``matmul`` for callers that cannot allocate: split-K partials go to the library's own per-GPU buffer
+    (``vecops_hip_matmul_static_workspace``); nothing is allocated here either."""
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    _check(lib().vecops_hip_matmul_static_workspace(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None,
+                                                    C.byref(oc), compute, _stream_handle(stream)))
     return c
 
 

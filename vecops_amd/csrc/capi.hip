@@ -2,6 +2,7 @@
 // validation, the GPU kernel-selection rule table and the kernel launches.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -630,7 +631,7 @@ int32_t vecops_hip_pack_b_compensated(const VecopsHipOperand* b, int32_t a_zero_
 int32_t vecops_hip_plan_matmul_packed_b(const VecopsHipOperand* a, uint32_t packed_dtype, int64_t n,
                                         const VecopsHipOperand* c_in, const VecopsHipOperand* c, VecopsHipPlan* plan) {
   if (plan == nullptr) return fail(ST_INVALID, "plan_matmul_packed_b: null plan");
-  Problem pr;
+  Problem pr{};
   int32_t rc = describe_packed(a, reinterpret_cast<void*>(16), packed_dtype, n, c_in, c, &pr);
   if (rc != ST_OK) return rc;
   choose(pr, plan);
@@ -640,7 +641,7 @@ int32_t vecops_hip_plan_matmul_packed_b(const VecopsHipOperand* a, uint32_t pack
 int32_t vecops_hip_matmul_packed_b(const VecopsHipOperand* a, const void* packed_b, uint32_t packed_dtype, int64_t n,
                                    const VecopsHipOperand* c_in, const VecopsHipOperand* c, void* workspace,
                                    uint64_t workspace_size, void* stream) {
-  Problem pr;
+  Problem pr{};
   int32_t rc = describe_packed(a, packed_b, packed_dtype, n, c_in, c, &pr);
   if (rc != ST_OK) return rc;
   if (pr.k > 0 && pr.n > 0 && !aligned16(packed_b)) return fail(ST_INVALID, "matmul_packed_b: packed b must be 16-byte aligned");
@@ -659,7 +660,7 @@ int32_t vecops_hip_matmul_i8_dequant_packed_b(const int8_t* a, int64_t lda, cons
   VecopsHipOperand oa, oc;
   make_operand(&oa, a, DT_I8, m, k, lda);
   make_operand(&oc, c, DT_I32, m, n, ldc);  // accumulator class; the epilogue writes fp32
-  Problem pr;
+  Problem pr{};
   int32_t rc = describe_packed(&oa, packed_b, DT_I8, n, nullptr, &oc, &pr);
   if (rc != ST_OK) return rc;
   if (pr.k > 0 && pr.n > 0 && !aligned16(packed_b)) return fail(ST_INVALID, "matmul_i8_dequant_packed_b: packed b must be 16-byte aligned");
@@ -696,7 +697,7 @@ namespace {
 // to 256 bytes), then the product's own scratch.
 struct RuntimeQuant {
   VecopsHipOperand q, c_acc, a_flat, c_flat;
-  Problem pr;
+  Problem pr{};
   VecopsHipPlan plan;
   uint64_t q_bytes, row_bytes;
 };
@@ -754,7 +755,7 @@ int32_t run_runtime_quant(const VecopsHipOperand* a, const float* multipliers, i
                           const void* packed, int64_t packed_n, const int32_t* correction, const float* row_scales,
                           const float* column_scales, const VecopsHipOperand* c, void* workspace, uint64_t workspace_size,
                           void* stream) {
-  RuntimeQuant d;
+  RuntimeQuant d{};
   int32_t rc = describe_runtime_quant(a, b, packed, packed_n, c, workspace ? workspace : reinterpret_cast<void*>(256), &d);
   if (rc != ST_OK) return rc;
   if (d.plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
@@ -789,7 +790,7 @@ int32_t run_runtime_quant(const VecopsHipOperand* a, const float* multipliers, i
 
 uint64_t vecops_hip_matmul_runtime_quant_workspace(const VecopsHipOperand* a, const VecopsHipOperand* b,
                                                    const VecopsHipOperand* c) {
-  RuntimeQuant d;
+  RuntimeQuant d{};
   if (describe_runtime_quant(a, b, nullptr, 0, c, reinterpret_cast<void*>(256), &d) != ST_OK) return 0;
   return d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
 }
@@ -804,7 +805,7 @@ int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* 
 }
 
 uint64_t vecops_hip_matmul_runtime_quant_packed_b_workspace(const VecopsHipOperand* a, int64_t n, const VecopsHipOperand* c) {
-  RuntimeQuant d;
+  RuntimeQuant d{};
   if (describe_runtime_quant(a, nullptr, reinterpret_cast<const void*>(256), n, c, reinterpret_cast<void*>(256), &d) != ST_OK)
     return 0;
   return d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
@@ -838,7 +839,7 @@ int32_t vecops_hip_device_count(void) {
 int32_t vecops_hip_plan_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
                                const VecopsHipOperand* c, uint32_t compute, VecopsHipPlan* plan) {
   if (plan == nullptr) return fail(ST_INVALID, "plan_matmul: null plan");
-  Problem pr;
+  Problem pr{};
   int32_t rc = describe(a, b, c_in, c, compute, &pr);
   if (rc != ST_OK) return rc;
   choose(pr, plan);
@@ -860,7 +861,7 @@ int32_t vecops_hip_plan_matmul_fused(const VecopsHipOperand* a, const VecopsHipO
   if (plan == nullptr) return fail(ST_INVALID, "plan_matmul_fused: null plan");
   int32_t rc = check_epilogue(epilogue);
   if (rc != ST_OK) return rc;
-  Problem pr;
+  Problem pr{};
   rc = describe(a, b, c_in, c, compute, &pr, epilogue);
   if (rc != ST_OK) return rc;
   choose(pr, plan);
@@ -872,7 +873,7 @@ int32_t vecops_hip_matmul_fused(const VecopsHipOperand* a, const VecopsHipOperan
                                 void* workspace, uint64_t workspace_size, void* stream) {
   int32_t rc = check_epilogue(epilogue);
   if (rc != ST_OK) return rc;
-  Problem pr;
+  Problem pr{};
   rc = describe(a, b, c_in, c, compute, &pr, epilogue);
   if (rc != ST_OK) return rc;
   VecopsHipPlan plan;
@@ -880,10 +881,68 @@ int32_t vecops_hip_matmul_fused(const VecopsHipOperand* a, const VecopsHipOperan
   return run_problem(pr, plan, nullptr, nullptr, nullptr, workspace, workspace_size, static_cast<hipStream_t>(stream));
 }
 
+}  // extern "C"
+
+// Scratch of the entry point that takes no workspace (vecops_hip_matmul_static_workspace): device memory owned
+// by the library's code object - one copy per GPU, at its own address on each, held until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress; kernels and copies get the address
+// that call returns.
+static __device__ __align__(256) unsigned char scratch[VECOPS_HIP_STATIC_WORKSPACE_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_address[kMaxDevices];
+
+// Address of `scratch` on the current device, looked up once per device.
+int32_t static_workspace(void** address) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail(ST_EXEC, "hipGetDevice: %s", hipGetErrorString(e));
+  if (device < 0 || device >= kMaxDevices) return fail(ST_EXEC, "device ordinal %d out of range", device);
+  void* known = g_scratch_address[device].load(std::memory_order_acquire);
+  if (known == nullptr) {
+    void* found = nullptr;
+    e = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || found == nullptr)
+      return fail(ST_EXEC, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    // two host threads may both look it up: they get the same address
+    g_scratch_address[device].store(found, std::memory_order_release);
+    known = found;
+  }
+  *address = known;
+  return ST_OK;
+}
+}  // namespace
+
+extern "C" {
+
+uint64_t vecops_hip_static_workspace_bytes(void) { return VECOPS_HIP_STATIC_WORKSPACE_BYTES; }
+
+int32_t vecops_hip_matmul_static_workspace(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                           const VecopsHipOperand* c_in, const VecopsHipOperand* c, uint32_t compute,
+                                           void* stream) {
+  Problem pr{};
+  int32_t rc = describe(a, b, c_in, c, compute, &pr);
+  if (rc != ST_OK) return rc;
+  VecopsHipPlan plan;
+  choose(pr, &plan);
+  if (plan.workspace_bytes > VECOPS_HIP_STATIC_WORKSPACE_BYTES)
+    return fail(ST_NOT_APPLICABLE, "matmul_static_workspace: the call needs %llu bytes of scratch, the library holds %llu",
+                (unsigned long long)plan.workspace_bytes, (unsigned long long)VECOPS_HIP_STATIC_WORKSPACE_BYTES);
+  void* address = nullptr;
+  if (plan.workspace_bytes > 0) {
+    rc = static_workspace(&address);
+    if (rc != ST_OK) return rc;
+  }
+  // Nothing in the scratch has to start at zero: every split writes each of its partial sums before the
+  // reduction reads them, and the unsigned-operand terms are written by their own kernels first.
+  return run_problem(pr, plan, nullptr, nullptr, nullptr, address, plan.workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 int32_t vecops_hip_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
                           const VecopsHipOperand* c, uint32_t compute, void* workspace, uint64_t workspace_size,
                           void* stream) {
-  Problem pr;
+  Problem pr{};
   int32_t rc = describe(a, b, c_in, c, compute, &pr);
   if (rc != ST_OK) return rc;
   VecopsHipPlan plan;
@@ -896,7 +955,7 @@ uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int64_t n, int64_t k)
   make_operand(&a, reinterpret_cast<void*>(16), DT_I8, m, k, k);
   make_operand(&b, reinterpret_cast<void*>(16), DT_I8, n, k, k);
   make_operand(&c, reinterpret_cast<void*>(16), DT_I32, m, n, n);
-  Problem pr;
+  Problem pr{};
   if (describe(&a, &b, nullptr, &c, 0, &pr) != ST_OK) return 0;
   pr.dequant = true;
   VecopsHipPlan plan;
@@ -915,7 +974,7 @@ int32_t vecops_hip_matmul_i8_dequant(const int8_t* a, int64_t lda, const int8_t*
   make_operand(&oa, a, DT_I8, m, k, lda);
   make_operand(&ob, b, DT_I8, n, k, ldb);
   make_operand(&oc, c, DT_I32, m, n, ldc);  // accumulator class; the epilogue writes fp32
-  Problem pr;
+  Problem pr{};
   int32_t rc = describe(&oa, &ob, nullptr, &oc, 0, &pr);
   if (rc != ST_OK) return rc;
   pr.dequant = true;
