@@ -333,6 +333,19 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_i8_dequant_packed_b(const int8_t* a,
                                                                 int64_t m, int64_t n, int64_t k, void* workspace,
                                                                 uint64_t workspace_size, void* stream);
 
+/*
+ * Measurement yardstick, no counterpart in vecops: `workgroups` workgroups of four wavefronts (one per SIMD) each
+ * issue iters x 32 independent matrix-core instructions of the tile kernels' shape (dtype 11: v_mfma_f32_32x32x16_bf16,
+ * dtype 2: v_mfma_i32_32x32x32_i8, sixteen 32x32 accumulator tiles per wavefront) on operand registers filled from
+ * `operands` (device memory, 16-byte aligned, operand_bytes of it) - no memory traffic inside the loop.  The rate it
+ * sustains is what a GEMM on those operand values can reach at most on this machine: the clocks follow the power the
+ * multipliers draw.  `out` receives workgroups x 256 words.  vecops_hip_mfma_stream_ops gives the operations one
+ * launch performs (2 per multiply-add).
+ */
+VECOPS_HIP_EXPORT uint64_t vecops_hip_mfma_stream_ops(uint32_t dtype, int32_t workgroups, int32_t iters);
+VECOPS_HIP_EXPORT int32_t vecops_hip_mfma_stream(uint32_t dtype, const void* operands, uint64_t operand_bytes,
+                                                 int32_t workgroups, int32_t iters, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -631,7 +631,8 @@ def test_config4_int8_full_size_checksum(device, oracle):
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 8, 16])
 @pytest.mark.parametrize("n,k,group", [(14336, 4096, 128), (300, 512, 64), (17, 1024, 128), (4096, 11008, 128),
-                                       (2064, 4096, 256), (2100, 4096, 128)])
+                                       (2064, 4096, 256), (2100, 4096, 128), (4100, 4096, 128), (4100, 4096, 256),
+                                       (4100, 4096, 64), (4099, 4096, 32)])
 def test_w8a16_group(device, oracle, m, n, k, group):
     """Checked against the fp64 brute force of the stated contract: fp32 accumulation
     over K=4096 plus the final bf16 rounding stay within one bf16 ulp (2^-7) of it."""
@@ -648,6 +649,29 @@ def test_w8a16_group(device, oracle, m, n, k, group):
     torch.cuda.synchronize()
     _, want = oracle.matmul_w8a16_group(x, w, s, group)
     assert rel_err(synth.bf16_to_f32(host_bits(y)), want) <= 2 ** -7
+
+
+@pytest.mark.parametrize("m", [1, 2, 4, 16])
+@pytest.mark.parametrize("group", [128, 256])
+def test_w8a16_group_strided_operands(device, oracle, m, group):
+    """Rows of x, w and y that are longer than the operand (ldx, ldw, ldy beyond K, K and N) on the decode shape's
+    kernels (K = 4096, N >= 4096, ragged N): the padding must neither be read into the sums nor written."""
+    import torch
+    from vecops_amd import capi
+    n, k = 4100, 4096
+    x = synth.bf16_round(synth.normal(5, (m, k)))
+    w = synth.int8_sym(6, (n, k))
+    s = synth.scales(7, (n, k // group))
+    xp = torch.full((m, k + 64), float("nan"), dtype=torch.bfloat16, device=device)
+    xp[:, :k] = dev_bf16(x, device)
+    wp = torch.full((n, k + 256), 77, dtype=torch.int8, device=device)
+    wp[:, :k] = torch.from_numpy(w).to(device)
+    yp = torch.full((m, n + 24), 3.0, dtype=torch.bfloat16, device=device)
+    capi.matmul_w8a16_group(xp[:, :k], wp[:, :k], torch.from_numpy(s).to(device), yp[:, :n], group)
+    torch.cuda.synchronize()
+    _, want = oracle.matmul_w8a16_group(x, w, s, group)
+    assert rel_err(synth.bf16_to_f32(host_bits(yp[:, :n].contiguous())), want) <= 2 ** -7
+    assert bool((yp[:, n:] == 3.0).all())
 
 
 def test_w8a16_rejects_bad_arguments(device):

@@ -767,7 +767,7 @@ struct Stager {
     commit_part<PART>(lds_tile);
   }
   template <int PART, int OP>
-  __device__ __forceinline__ void load_op(int kt, char* /*lds_tile*/) {
+  __device__ __forceinline__ void load_op(int kt, uint32_t /*lds_tile*/) {
     fetch_part<PART>(kt);
   }
 
@@ -901,7 +901,7 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
     commit_part<PART>(lds_tile);
   }
   template <int PART, int OP>
-  __device__ __forceinline__ void load_op(int kt, char* /*lds_tile*/) {
+  __device__ __forceinline__ void load_op(int kt, uint32_t /*lds_tile*/) {
     fetch_part<PART>(kt);
   }
 };
@@ -938,23 +938,30 @@ __device__ __forceinline__ u32x4 tile_buffer_words(const VECOPS_GLOBAL char* bas
                0x7fffffffu, 0x00020000u};
 }
 
-// One buffer load of 16 bytes per lane that writes LDS itself: lane l's bytes land at dst + 16 * l
-// (dst is wavefront-uniform).  Written as an instruction rather than through the compiler's builtin: the
-// compiler orders every later LDS read it cannot tell apart behind such a load - it would wait for the
-// load in front of each transposing fragment read of the tile being multiplied, which lies in the other
-// stage.  The kernel orders them itself: vmcnt(0) and a barrier before a stage filled this way is read.
+// One buffer load of 16 bytes per lane that writes LDS itself: lane l's bytes land at tile_address + tile_offset +
+// 16 * l (both wavefront-uniform numbers; the low half of a generic pointer into LDS is the LDS address).  Written
+// as an instruction rather than through the compiler's builtin: the compiler orders every later LDS read it cannot
+// tell apart behind such a load - it would wait for the load in front of each transposing fragment read of the
+// tile being multiplied, which lies in the other stage.  The kernel orders them itself: vmcnt(0) and a barrier
+// before a stage filled this way is read.  The LDS address goes into M0 by the one scalar add; handing a pointer
+// over instead cost four more scalar instructions per load (a 64-bit add and the null check of the pointer
+// conversion), and sixteen such sequences per K tile were 3-7 % of the kernel's time.
 // (The instruction exists only in the device pass of the compiler.)
-__device__ __forceinline__ void load_16_bytes_into_lds(const u32x4& descriptor, lds_void_ptr dst, uint32_t lane_offset,
-                                                       uint32_t uniform_offset) {
+__device__ __forceinline__ void load_16_bytes_into_lds(const u32x4& descriptor, uint32_t tile_address, uint32_t tile_offset,
+                                                       uint32_t lane_offset, uint32_t uniform_offset) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  const uint32_t lds_address = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<size_t>(dst)));
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+  asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, %4 offen lds"
                :
-               : "s"(lds_address), "v"(lane_offset), "s"(descriptor), "s"(uniform_offset)
-               : "memory", "m0");
+               : "s"(tile_address), "s"(tile_offset), "v"(lane_offset), "s"(descriptor), "s"(uniform_offset)
+               : "memory", "m0", "scc");
 #else
-  (void)descriptor; (void)dst; (void)lane_offset; (void)uniform_offset;
+  (void)descriptor; (void)tile_address; (void)tile_offset; (void)lane_offset; (void)uniform_offset;
 #endif
+}
+
+// LDS address of a generic pointer into LDS as a wavefront-uniform number: the low half of the pointer.
+__device__ __forceinline__ uint32_t lds_address_of(const char* lds_pointer) {
+  return __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_pointer)));
 }
 
 // The same load through the compiler's builtin, for a kernel that has other loads in flight: the compiler
@@ -1013,12 +1020,14 @@ struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
       row_bytes[i] = static_cast<uint32_t>((static_cast<int64_t>(row) * rs + chunk * T::kElemsPerChunk) * T::kSrcBytes);
     }
   }
-  __device__ __forceinline__ void dma_part(int part, int kt, char* lds_tile) const {
-    load_16_bytes_into_lds(tile_buf, (lds_void_ptr)(lds_tile + (part * ROWS_PER_PASS + wave_ * 8) * 128), row_bytes[part],
-                           kt * (8 * T::kElemsPerChunk * T::kSrcBytes));
+  // lds_tile: LDS address of the operand's tile (lds_address_of)
+  __device__ __forceinline__ void dma_part(int part, int kt, uint32_t lds_tile) const {
+    load_16_bytes_into_lds(tile_buf, lds_tile, __builtin_amdgcn_readfirstlane((part * ROWS_PER_PASS + wave_ * 8) * 128),
+                           row_bytes[part], kt * (8 * T::kElemsPerChunk * T::kSrcBytes));
   }
   __device__ __forceinline__ void dma_full(int kt, char* lds_tile) const {
-    static_for<CHUNKS>([&](auto ci) { dma_part(decltype(ci)::value, kt, lds_tile); });
+    const uint32_t address = lds_address_of(lds_tile);
+    static_for<CHUNKS>([&](auto ci) { dma_part(decltype(ci)::value, kt, address); });
   }
   __device__ __forceinline__ void dma_part_counted(int part, int kt, char* lds_tile) const {
     load_16_bytes_into_lds_counted(tile_rsrc, (lds_void_ptr)(lds_tile + (part * ROWS_PER_PASS + wave_ * 8) * 128),
@@ -1031,7 +1040,7 @@ struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
   template <int PART, int OP>
   __device__ __forceinline__ void store_op(char*) const {}
   template <int PART, int OP>
-  __device__ __forceinline__ void load_op(int kt, char* lds_tile) const {
+  __device__ __forceinline__ void load_op(int kt, uint32_t lds_tile) const {
     dma_part(PART, kt, lds_tile);
   }
 };
@@ -1082,12 +1091,14 @@ struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
   __device__ __forceinline__ uint32_t part_offset(int part) const {
     return __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(part * K_ROWS_PER_PART * ks * T::kSrcBytes));
   }
-  __device__ __forceinline__ void dma_part(int part, int kt, char* lds_tile) const {
+  __device__ __forceinline__ void dma_part(int part, int kt, uint32_t lds_tile) const {
     const u32x4 buf = tile_buffer_words(tile_base + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes);
-    load_16_bytes_into_lds(buf, (lds_void_ptr)(lds_tile + (part * THREADS + wave_ * 64) * 16), chunk_bytes, part_offset(part));
+    load_16_bytes_into_lds(buf, lds_tile, __builtin_amdgcn_readfirstlane((part * THREADS + wave_ * 64) * 16), chunk_bytes,
+                           part_offset(part));
   }
   __device__ __forceinline__ void dma_full(int kt, char* lds_tile) const {
-    static_for<CHUNKS>([&](auto ci) { dma_part(decltype(ci)::value, kt, lds_tile); });
+    const uint32_t address = lds_address_of(lds_tile);
+    static_for<CHUNKS>([&](auto ci) { dma_part(decltype(ci)::value, kt, address); });
   }
   __device__ __forceinline__ void stage_checked(int kt, char* lds_tile) const {
     stage_kn_checked(base, ks, first_row, extent, ROWS, kt * 64, k_end, lds_tile, tid_, THREADS);
@@ -1095,7 +1106,7 @@ struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
   template <int PART, int OP>
   __device__ __forceinline__ void store_op(char*) const {}
   template <int PART, int OP>
-  __device__ __forceinline__ void load_op(int kt, char* lds_tile) const {
+  __device__ __forceinline__ void load_op(int kt, uint32_t lds_tile) const {
     dma_part(PART, kt, lds_tile);
   }
 };
@@ -1148,7 +1159,7 @@ struct Stager<SRC_F32, LOAD_NVEC, ROWS, THREADS> {
   }
 
   template <int PART, int R>
-  __device__ __forceinline__ void load_op(int kt, char* /*lds_tile*/) {
+  __device__ __forceinline__ void load_op(int kt, uint32_t /*lds_tile*/) {
     if (!active(PART)) return;
     const VECOPS_GLOBAL char* row = tile_base + (static_cast<int64_t>(kt) * 32 + R) * ks * 4;
     const u32x4 v = *(const VECOPS_GLOBAL u32x4*)(uniform_ptr(row) + unit_bytes[PART]);
@@ -1159,7 +1170,7 @@ struct Stager<SRC_F32, LOAD_NVEC, ROWS, THREADS> {
   }
   template <int PART>
   __device__ __forceinline__ void fetch_part(int kt) {
-    static_for<4>([&](auto cr) { load_op<PART, decltype(cr)::value>(kt, nullptr); });
+    static_for<4>([&](auto cr) { load_op<PART, decltype(cr)::value>(kt, 0u); });
   }
   __device__ __forceinline__ void fetch_full(int kt) {
     static_for<UNITS>([&](auto cu) { fetch_part<decltype(cu)::value>(kt); });
@@ -1723,11 +1734,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
     // prefetches (tile index clamped to the last one) and the fragment reads of the
     // next tile are issued unconditionally; the surplus ones of the final
     // iterations touch valid memory and are never consumed.
+    const uint32_t lds_address = lds_address_of(lds);
     auto main_loop = [&](auto prefetch_tag) {
       constexpr bool PREFETCH = decltype(prefetch_tag)::value;
       for (int it = 0; it < nk; ++it) {
         const char* tile = lds + (it & 1) * STAGE_BYTES;
         char* other = lds + ((it & 1) ^ 1) * STAGE_BYTES;
+        const uint32_t other_address = lds_address + ((it & 1) ^ 1) * STAGE_BYTES;  // what the loads that write LDS put into M0
         // K tile to prefetch: seq(min(it + 2, nk - 1)), never the tail tile (position 0)
         // (loads that write LDS fetch the next tile, into the other stage)
         const int t2 = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(it + (DMA ? 1 : 2), nk - 1)));
@@ -1736,9 +1749,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
           constexpr StagingOp o = Sched::op(decltype(step_tag)::value, decltype(g_tag)::value, decltype(order_tag)::value);
           // (a stager whose loads write LDS has no store operations; the others ignore the load's LDS address)
           if constexpr (o.operand == 0 && o.is_load == 0) stager_a.template store_op<o.part, o.op>(other);
-          if constexpr (o.operand == 0 && o.is_load == 1 && PREFETCH) stager_a.template load_op<o.part, o.op>(t2, other);
+          if constexpr (o.operand == 0 && o.is_load == 1 && PREFETCH) stager_a.template load_op<o.part, o.op>(t2, other_address);
           if constexpr (o.operand == 1 && o.is_load == 0) stager_b.template store_op<o.part, o.op>(other + BM * 128);
-          if constexpr (o.operand == 1 && o.is_load == 1 && PREFETCH) stager_b.template load_op<o.part, o.op>(t2, other + BM * 128);
+          if constexpr (o.operand == 1 && o.is_load == 1 && PREFETCH) stager_b.template load_op<o.part, o.op>(t2, other_address + BM * 128);
         };
         // Slots [S0, S1) of k-step STEP: MFMA x on fragment set mfma_set, then this
         // slot's share of the N_RD fragment reads (k-step read_ks of read_tile into

@@ -228,7 +228,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
               if constexpr (PREFETCH) stager_a.dma_part_counted(P0 + g, t1, other);
             } else {
               if constexpr (g < NP) stager_a.template store_op<P0 + g, 0>(other);
-              else if constexpr (PREFETCH) stager_a.template load_op<P0 + g - NP, 0>(t2, nullptr);
+              else if constexpr (PREFETCH) stager_a.template load_op<P0 + g - NP, 0>(t2, 0u);
             }
           };
           if constexpr (NS == 0) static_for<OPS>(stage_op);
