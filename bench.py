@@ -1,20 +1,26 @@
 #!/usr/bin/env python3
 """Benchmark of the vecops matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu]
 
-A "step" is one pass of the hot path over one batch of synthetic operands that are
-already resident in HBM.  The default workload is the configuration the headline
-metric is quoted on (bf16 GEMM, M=N=K=4096, A[M,K] and B[K,N] row-major, fp32
-accumulate, bf16 output); the int8 quantised matmul, the M=1 weight-only GEMV and the
-prepacked-weights forms of the two GEMMs are measured in the same run and reported
-under "secondary".  Prints ONE JSON line.
+A "step" is one pass of the hot path over one batch of synthetic operands that are already resident in HBM.  The
+default workload is the configuration the headline metric is quoted on (bf16 GEMM, M=N=K=4096, A[M,K] and B[K,N]
+row-major, fp32 accumulate, bf16 output); every other benchmark configuration - the fp32 1024^3 product on both
+compute strategies, the four irregular batched shapes, the int8 quantised matmul, the weight-only GEMV at M = 1, 4, 16 -
+and the prepacked-weights and runtime-quantised forms are measured in the same run and reported under "secondary",
+together with the matrix-core yardstick (what the machine sustains on the benchmark's operand values with nothing but
+matrix instructions).  Prints ONE JSON line.
+
+Timing: W warm-up launches, then exactly K launches between two device synchronisations give `ms_per_step` and
+`value`; `roofline.achieved` is the median over 7 repetitions of max(K, 50) back-to-back launches timed with HIP
+events on the stream the launches go to (torch's current stream).
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -22,23 +28,82 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# MI355X published peaks
+# MI355X published peaks (dense)
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_INT8_TOPS = 5000.0
+PEAK_FP32_MATRIX_TFLOPS = 157.3
 PEAK_HBM_GBPS = 8000.0
+REPETITIONS = 7
 
-# HBM-side bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes kept under
-# profiles/ (KiB per dispatch x 1024, FETCH scaled by 2.000 and WRITE by 1.000: what the
-# same counters read for a 1 GiB device copy, `--only copy`).  Counters cannot be read
-# from inside this process, so these are the recorded figures for exactly these workloads.
-TRAFFIC_BF16_4096 = int((98479.5 * 2.000 + 32768 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT = int((95283.3 * 2.000 + 88064 * 1.000) * 1024)
-TRAFFIC_GEMV_M1 = int((29647.4 * 2.000 + 112.0 * 1.000) * 1024)
-TRAFFIC_BF16_4096_PACKED = int((98468.3 * 2.000 + 32768 * 1.000) * 1024)
-TRAFFIC_INT8_DEQUANT_PACKED = int((95160.6 * 2.000 + 88064 * 1.000) * 1024)
+# HBM-side bytes per launch recorded with rocprofv3 (FETCH_SIZE and WRITE_SIZE in KiB per dispatch x 1024, FETCH
+# scaled by 2.000 and WRITE by 1.000: what the same counters read for a 1 GiB device copy, `--only copy`).  Counters
+# cannot be read from inside this process: these are the figures of the named summaries, for exactly these workloads.
+RECORDED_TRAFFIC = {
+    "bf16": (int((98479.5 * 2.000 + 32768 * 1.000) * 1024), "profiles/tile_gemm_bf16_4096.md"),
+    "int8": (int((95283.3 * 2.000 + 88064 * 1.000) * 1024), "profiles/tile_gemm_int8_dequant_2048x4096x11008.md"),
+    "gemv_m1": (int((29647.4 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_stream_m1_4096x14336.md"),
+    "bf16_packed": (int((98468.3 * 2.000 + 32768 * 1.000) * 1024),
+                    "profiles/tile_gemm_packed_b_bf16_4096_int8_2048x4096x11008.md"),
+    "int8_packed": (int((95160.6 * 2.000 + 88064 * 1.000) * 1024),
+                    "profiles/tile_gemm_packed_b_bf16_4096_int8_2048x4096x11008.md"),
+}
 
 
-def _device_tensors_bf16_gemm(dev):
+def _traffic(key):
+    if key not in RECORDED_TRAFFIC:
+        return {"traffic": None}
+    nbytes, source = RECORDED_TRAFFIC[key]
+    return {"traffic": nbytes, "traffic_source": "recorded: " + source}
+
+
+def _measure(fn, steps, warmup):
+    """fn(i) enqueues one launch on torch's current stream.  Returns the wall time per step of exactly `steps`
+    launches between two synchronisations, and the median / extremes of HIP-event time per launch over
+    REPETITIONS runs of max(steps, 50) launches."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(i)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    launches = max(steps, 50)
+    per_launch = []
+    for _ in range(REPETITIONS):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(launches):
+            fn(i)
+        stop.record()
+        torch.cuda.synchronize()
+        per_launch.append(start.elapsed_time(stop) / launches)
+    return {"wall_ms": wall_ms, "event_ms": statistics.median(per_launch), "event_ms_min": min(per_launch),
+            "event_ms_max": max(per_launch), "launches_per_repetition": launches, "repetitions": REPETITIONS}
+
+
+def _kernel_label(plan, operands):
+    from vecops_amd import capi
+    family = capi.FAMILY_NAMES.get(plan.family, str(plan.family))
+    loads = "16-byte loads" if plan.vector_a and plan.vector_b else "element loads"
+    b = {0: "B K-contiguous", 1: "B as [K,N]", 2: "B strided"}[plan.b_layout]
+    split = f", split-K {plan.split_k}" if plan.split_k > 1 else ""
+    return f"vecops_hip tile_gemm_kernel<{operands}> family {family}, {loads}, {b}{split}"
+
+
+def _roofline(bound, achieved, peak, unit, **extra):
+    out = {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak}
+    out.update(extra)
+    return out
+
+
+def _timing_fields(t):
+    return {"event_ms": t["event_ms"], "event_ms_min": t["event_ms_min"], "event_ms_max": t["event_ms_max"],
+            "repetitions": t["repetitions"], "launches_per_repetition": t["launches_per_repetition"]}
+
+
+def _bf16_operands(dev):
     import numpy as np
     import torch
     from vecops_amd import synth
@@ -50,45 +115,108 @@ def _device_tensors_bf16_gemm(dev):
     return a, b_kn, ta, tb
 
 
-def _time_launches(fn, steps, warmup):
-    """Returns (wall ms per step, HIP-event ms per launch) for `steps` back-to-back launches
-    on torch's current stream - the stream the launcher is handed."""
+def bench_mfma_ceiling(dev, steps, warmup, which="bf16"):
+    """The matrix-core yardstick: nothing but independent matrix instructions of the tile kernels' shape, one
+    wavefront per SIMD on all compute units, on the benchmark's operand values and on zeros."""
     import torch
-    for i in range(warmup):
-        fn(i)
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    start.record()
-    for i in range(steps):
-        fn(i)
-    stop.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return wall_ms, start.elapsed_time(stop) / steps
+    from vecops_amd import capi, synth
+    out = torch.empty(256 * 256, dtype=torch.int32, device=dev)
+    if which == "bf16":
+        _, _, values, _ = _bf16_operands(dev)
+        label, unit, peak = "v_mfma_f32_32x32x16_bf16", "TFLOP/s", PEAK_BF16_TFLOPS
+        what = "normal(0, 0.02) rounded to bf16 (the GEMM's A operand)"
+    else:
+        values = torch.from_numpy(synth.int8_sym(1, (2048, 4096))).to(dev)
+        label, unit, peak = "v_mfma_i32_32x32x32_i8", "TOP/s", PEAK_INT8_TOPS
+        what = "int8 uniform[-127,127] (the quantised matmul's A operand)"
+    zeros = torch.zeros_like(values)
+    res = {}
+    for name, operands in (("benchmark_operands", values), ("zeros", zeros)):
+        ops_per_launch = [0]
+
+        def launch(i, operands=operands):
+            ops_per_launch[0] = capi.mfma_stream(operands, 256, 512, out)
+        t = _measure(launch, max(5, steps // 10), max(2, warmup // 5))
+        res[name] = ops_per_launch[0] / (t["event_ms"] * 1e-3) / 1e12
+    return {"metric": f"mfma_ceiling_{which}", "workload": f"256 workgroups x 4 wavefronts x 16384 independent {label} "
+            f"(sixteen 32x32 accumulator tiles per wavefront, no memory traffic), operands: {what}; and zeros",
+            "value": res["benchmark_operands"], "unit": unit, "on_zeros": res["zeros"], "peak": peak,
+            "frac_of_peak": res["benchmark_operands"] / peak, "frac_of_peak_on_zeros": res["zeros"] / peak}
 
 
 def bench_bf16_gemm(dev, steps, warmup):
     import torch
     from vecops_amd import capi
     n = 4096
-    a, b_kn, ta, tb = _device_tensors_bf16_gemm(dev)
+    a, b_kn, ta, tb = _bf16_operands(dev)
     tb_view = tb.t()                      # [N,K] view with strides (1, N): vecops' way to pass B[K,N]
     c = torch.empty((n, n), dtype=torch.bfloat16, device=dev)
-    wall_ms, ev_ms = _time_launches(lambda i: capi.matmul(ta, tb_view, c), steps, warmup)
+    plan = capi.plan_matmul(ta, tb_view, c)
+    t = _measure(lambda i: capi.matmul(ta, tb_view, c), steps, warmup)
     flops = 2.0 * n * n * n
-    tflops = flops / (ev_ms * 1e-3) / 1e12
+    tflops = flops / (t["event_ms"] * 1e-3) / 1e12
     return {
-        "wall_ms": wall_ms, "event_ms": ev_ms, "value": flops / (wall_ms * 1e-3) / 1e12,
-        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BF16_4096,
-                     "kernel": "vecops_hip::tile_gemm_kernel<bf16, 256x256x64, loads into LDS, B as [K,N]>",
-                     "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": 3 * 2 * n * n},
+        "wall_ms": t["wall_ms"], "value": flops / (t["wall_ms"] * 1e-3) / 1e12,
+        "roofline": _roofline("mfma", tflops, PEAK_BF16_TFLOPS, "TFLOP/s", kernel=_kernel_label(plan, "bf16"),
+                              algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=3 * 2 * n * n,
+                              **_traffic("bf16"), **_timing_fields(t)),
         "host": (a, b_kn),
     }
 
 
-def bench_int8_dequant(dev, steps, warmup):
+def bench_fp32_gemm(dev, steps, warmup, compute):
+    """BASELINE configs[0]: fp32 1024^3, A[M,K] and B[K,N] row-major, U[-1,1); multiplied as bf16 (vecops' x86
+    behaviour) or in fp32 (its SME_F32F32 atom)."""
+    import torch
+    from vecops_amd import capi, synth
+    n = 1024
+    a = torch.from_numpy(synth.uniform_pm1(1, (n, n))).to(dev)
+    b_kn = torch.from_numpy(synth.uniform_pm1(2, (n, n))).to(dev)
+    c = torch.empty((n, n), dtype=torch.float32, device=dev)
+    code = capi.COMPUTE_F32 if compute == "f32" else capi.COMPUTE_BF16
+    plan = capi.plan_matmul(a, b_kn.t(), c, compute=code)
+    ws = torch.empty(max(int(plan.workspace_bytes), 1), dtype=torch.uint8, device=dev)
+    t = _measure(lambda i: capi.matmul(a, b_kn.t(), c, compute=code, workspace=ws), max(steps, 200), warmup)
+    flops = 2.0 * n ** 3
+    tflops = flops / (t["event_ms"] * 1e-3) / 1e12
+    peak = PEAK_FP32_MATRIX_TFLOPS if compute == "f32" else PEAK_BF16_TFLOPS
+    return {"metric": f"fp32_gemm_1024_{compute}_compute_tflops", "workload": "fp32 GEMM M=N=K=1024, A[M,K] and B[K,N] "
+            f"row-major, uniform[-1,1), multiplied in {'fp32' if compute == 'f32' else 'bf16 (rounded on load)'}, fp32 "
+            "accumulate and output (BASELINE configs[0])", "value": tflops, "unit": "TFLOP/s",
+            "us_per_step": t["wall_ms"] * 1e3, "dtype": "f32" if compute == "f32" else "f32 memory, bf16 compute",
+            "roofline": _roofline("mfma", tflops, peak, "TFLOP/s", kernel=_kernel_label(plan, "f32" if compute == "f32" else "f32 as bf16"),
+                                  algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=3 * 4 * n * n,
+                                  traffic=None, **_timing_fields(t))}
+
+
+def bench_batched(dev, steps, warmup, m, n, k):
+    """BASELINE configs[2]: batch 8, bf16 operands uniform[-1,1), fp32 accumulate and output."""
+    import numpy as np
+    import torch
+    from vecops_amd import capi, synth
+    batch = 8
+    a = torch.from_numpy(synth.bf16_round(synth.uniform_pm1(1, (batch, m, k))).view(np.int16)).to(dev).view(torch.bfloat16)
+    b = torch.from_numpy(synth.bf16_round(synth.uniform_pm1(2, (batch, n, k))).view(np.int16)).to(dev).view(torch.bfloat16)
+    c = torch.empty((batch, m, n), dtype=torch.float32, device=dev)
+    plan = capi.plan_matmul(a, b, c)
+    ws = torch.empty(max(int(plan.workspace_bytes), 1), dtype=torch.uint8, device=dev)
+    t = _measure(lambda i: capi.matmul(a, b, c, workspace=ws), max(steps, 100), warmup)
+    flops = batch * 2.0 * m * n * k
+    nbytes = batch * (2 * m * k + 2 * n * k + 4 * m * n)
+    tflops = flops / (t["event_ms"] * 1e-3) / 1e12
+    gbps = nbytes / (t["event_ms"] * 1e-3) / 1e9
+    # the bound is the one that takes longer at the machine's peaks
+    mfma_bound = flops / (PEAK_BF16_TFLOPS * 1e12) >= nbytes / (PEAK_HBM_GBPS * 1e9)
+    roof = (_roofline("mfma", tflops, PEAK_BF16_TFLOPS, "TFLOP/s") if mfma_bound
+            else _roofline("hbm", gbps, PEAK_HBM_GBPS, "GB/s"))
+    roof.update(kernel=_kernel_label(plan, "bf16"), algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=nbytes,
+                traffic=None, **_timing_fields(t))
+    return {"metric": f"bf16_batched_{m}x{n}x{k}_tflops", "workload": f"batch 8 x bf16 ({m},{n},{k}), A[8,M,K] and "
+            "B[8,N,K], uniform[-1,1), fp32 accumulate and output (BASELINE configs[2])", "value": tflops,
+            "unit": "TFLOP/s", "hbm_gbps": gbps, "us_per_step": t["wall_ms"] * 1e3, "dtype": "bf16", "roofline": roof}
+
+
+def bench_int8_dequant(dev, steps, warmup, ceiling=None):
     import torch
     from vecops_amd import capi, synth
     m, k, n = 2048, 4096, 11008
@@ -99,22 +227,25 @@ def bench_int8_dequant(dev, steps, warmup):
     c = torch.empty((m, n), dtype=torch.float32, device=dev)
     need = capi.lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k)   # the caller owns the scratch
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
-    wall_ms, ev_ms = _time_launches(lambda i: capi.matmul_i8_dequant(a, b, rs, cs, c, workspace=ws), steps, warmup)
+    plan = capi.plan_matmul(a, b, torch.empty((m, n), dtype=torch.int32, device=dev))
+    t = _measure(lambda i: capi.matmul_i8_dequant(a, b, rs, cs, c, workspace=ws), steps, warmup)
     ops = 2.0 * m * n * k
-    tops = ops / (ev_ms * 1e-3) / 1e12
+    tops = ops / (t["event_ms"] * 1e-3) / 1e12
+    roof = _roofline("mfma", tops, PEAK_INT8_TOPS, "TOP/s", kernel=_kernel_label(plan, "int8") + ", dequantising epilogue",
+                     algorithmic_ops_per_launch=ops, algorithmic_bytes_per_launch=m * k + n * k + 4 * m * n + 4 * (m + n),
+                     **_traffic("int8"), **_timing_fields(t))
+    if ceiling:
+        roof.update(measured_ceiling=ceiling, frac_of_ceiling=tops / ceiling)
     return {"metric": "int8_quantized_matmul_tops", "workload": "int8 2048x4096x11008, per-token x per-channel "
-            "dequant fused, fp32 out", "value": tops, "unit": "TOP/s", "ms_per_step": wall_ms, "dtype": "int8",
-            "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                         "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT,
-                         "kernel": "vecops_hip::tile_gemm_kernel<int8, 256x256x128, loads into LDS, dequant epilogue>",
-                         "algorithmic_ops_per_launch": ops,
-                         "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
+            "dequant fused, fp32 out (BASELINE configs[3])", "value": tops, "unit": "TOP/s", "ms_per_step": t["wall_ms"],
+            "dtype": "int8", "roofline": roof}
 
 
 def bench_runtime_quant(dev, steps, warmup):
     """fp32 activations quantised per row on the way in (vecops' RuntimePerRowAsymmetricQuantizeTransform), int8
     weights, correction row, per-token x per-channel dequantisation: three launches (quantise, weight row sums,
     the int8 product) timed as one step."""
+    import ctypes as C
     import numpy as np
     import torch
     from vecops_amd import capi, synth
@@ -129,22 +260,20 @@ def bench_runtime_quant(dev, steps, warmup):
     corr = torch.from_numpy((-zp * b_host.astype(np.int64).sum(axis=1)).astype(np.int32)).to(dev)
     c = torch.empty((m, n), dtype=torch.float32, device=dev)
     oa, ob, oc = capi.operand(a), capi.operand(b), capi.operand(c)
-    import ctypes as C
     need = capi.lib().vecops_hip_matmul_runtime_quant_workspace(C.byref(oa), C.byref(ob), C.byref(oc))
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
-    wall_ms, ev_ms = _time_launches(
-        lambda i: capi.matmul_runtime_quant(a, tm, zp, b, rs, cs, c, correction=corr, workspace=ws), steps, warmup)
+    t = _measure(lambda i: capi.matmul_runtime_quant(a, tm, zp, b, rs, cs, c, correction=corr, workspace=ws), steps, warmup)
     ops = 2.0 * m * n * k
-    tops = ops / (ev_ms * 1e-3) / 1e12
+    tops = ops / (t["event_ms"] * 1e-3) / 1e12
     return {"metric": "runtime_quantized_matmul_tops", "workload": "fp32 activations 2048x4096 quantised per row to "
             "uint8 on the way in, int8 weights 11008x4096, correction row, per-token x per-channel dequant, fp32 out",
-            "value": tops, "unit": "TOP/s", "ms_per_step": wall_ms, "dtype": "int8",
-            "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                         "frac": tops / PEAK_INT8_TOPS, "traffic": None,
-                         "kernel": "vecops_hip::quantize_rows_kernel + byte_row_sums_kernel + tile_gemm_kernel<int8, "
-                                   "256x256x128, loads into LDS, dequant epilogue>",
-                         "algorithmic_ops_per_launch": ops,
-                         "algorithmic_bytes_per_launch": 4 * m * k + n * k + 4 * m * n + 4 * (2 * m + 2 * n)}}
+            "value": tops, "unit": "TOP/s", "ms_per_step": t["wall_ms"], "dtype": "int8",
+            "roofline": _roofline("mfma", tops, PEAK_INT8_TOPS, "TOP/s", traffic=None,
+                                  kernel="vecops_hip quantize_rows_kernel + byte_row_sums_kernel + tile_gemm_kernel<int8> "
+                                         "family tile_256, dequantising epilogue",
+                                  algorithmic_ops_per_launch=ops,
+                                  algorithmic_bytes_per_launch=4 * m * k + n * k + 4 * m * n + 4 * (2 * m + 2 * n),
+                                  **_timing_fields(t))}
 
 
 def bench_bf16_gemm_packed(dev, steps, warmup):
@@ -153,19 +282,19 @@ def bench_bf16_gemm_packed(dev, steps, warmup):
     import torch
     from vecops_amd import capi
     n = 4096
-    _, _, ta, tb = _device_tensors_bf16_gemm(dev)
+    _, _, ta, tb = _bf16_operands(dev)
     packed = capi.pack_b(tb.t())
     c = torch.empty((n, n), dtype=torch.bfloat16, device=dev)
-    wall_ms, ev_ms = _time_launches(lambda i: capi.matmul_packed_b(ta, packed, c), steps, warmup)
+    t = _measure(lambda i: capi.matmul_packed_b(ta, packed, c), steps, warmup)
     flops = 2.0 * n * n * n
-    tflops = flops / (ev_ms * 1e-3) / 1e12
+    tflops = flops / (t["event_ms"] * 1e-3) / 1e12
     return {"metric": "bf16_gemm_4096_prepacked_b_tflops", "workload": "bf16 GEMM M=N=K=4096, B prepacked "
             "(vecops_hip_pack_b, not timed), fp32 accumulate, bf16 out", "value": tflops, "unit": "TFLOP/s",
-            "ms_per_step": wall_ms, "dtype": "bf16",
-            "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BF16_4096_PACKED,
-                         "kernel": "vecops_hip::tile_gemm_packed_b_kernel<bf16, 256x256x64>",
-                         "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": 3 * 2 * n * n}}
+            "ms_per_step": t["wall_ms"], "dtype": "bf16",
+            "roofline": _roofline("mfma", tflops, PEAK_BF16_TFLOPS, "TFLOP/s",
+                                  kernel="vecops_hip tile_gemm_packed_b_kernel<bf16> family tile_256",
+                                  algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=3 * 2 * n * n,
+                                  **_traffic("bf16_packed"), **_timing_fields(t))}
 
 
 def bench_int8_dequant_packed(dev, steps, warmup):
@@ -179,18 +308,17 @@ def bench_int8_dequant_packed(dev, steps, warmup):
     c = torch.empty((m, n), dtype=torch.float32, device=dev)
     need = capi.lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k)
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
-    wall_ms, ev_ms = _time_launches(
-        lambda i: capi.matmul_i8_dequant_packed_b(a, packed, rs, cs, c, workspace=ws), steps, warmup)
+    t = _measure(lambda i: capi.matmul_i8_dequant_packed_b(a, packed, rs, cs, c, workspace=ws), steps, warmup)
     ops = 2.0 * m * n * k
-    tops = ops / (ev_ms * 1e-3) / 1e12
+    tops = ops / (t["event_ms"] * 1e-3) / 1e12
     return {"metric": "int8_quantized_matmul_prepacked_b_tops", "workload": "int8 2048x4096x11008, weights prepacked "
             "(not timed), per-token x per-channel dequant fused, fp32 out", "value": tops, "unit": "TOP/s",
-            "ms_per_step": wall_ms, "dtype": "int8",
-            "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                         "frac": tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_INT8_DEQUANT_PACKED,
-                         "kernel": "vecops_hip::tile_gemm_packed_b_kernel<int8, 256x256x128, dequant epilogue>",
-                         "algorithmic_ops_per_launch": ops,
-                         "algorithmic_bytes_per_launch": m * k + n * k + 4 * m * n + 4 * (m + n)}}
+            "ms_per_step": t["wall_ms"], "dtype": "int8",
+            "roofline": _roofline("mfma", tops, PEAK_INT8_TOPS, "TOP/s",
+                                  kernel="vecops_hip tile_gemm_packed_b_kernel<int8> family tile_256, dequantising epilogue",
+                                  algorithmic_ops_per_launch=ops,
+                                  algorithmic_bytes_per_launch=m * k + n * k + 4 * m * n + 4 * (m + n),
+                                  **_traffic("int8_packed"), **_timing_fields(t))}
 
 
 def bench_gemv(dev, steps, warmup, m=1):
@@ -204,19 +332,16 @@ def bench_gemv(dev, steps, warmup, m=1):
     s = torch.from_numpy(synth.scales(3, (n, k // group))).to(dev)
     ss = [s.clone() for _ in range(copies)]
     y = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
-    wall_ms, ev_ms = _time_launches(
-        lambda i: capi.matmul_w8a16_group(x, ws[i % copies], ss[i % copies], y, group), steps, warmup)
+    t = _measure(lambda i: capi.matmul_w8a16_group(x, ws[i % copies], ss[i % copies], y, group), max(steps, 200), warmup)
     nbytes = n * k + 4 * n * (k // group) + 2 * m * k + 2 * m * n
-    gbps = nbytes / (ev_ms * 1e-3) / 1e9
+    gbps = nbytes / (t["event_ms"] * 1e-3) / 1e9
+    kernel = ("vecops_hip skinny_w8a16_stream_kernel" if m == 1 else "vecops_hip skinny_w8a16_stream_rows_kernel"
+              if m == 2 else "vecops_hip skinny_w8a16_mfma_resident_kernel")
     return {"metric": f"w8a16_gemv_m{m}_hbm_gbps", "workload": f"weight-only int8 GEMV M={m} K=4096 N=14336 group 128, "
-            "bf16 activations, bf16 out, weights rotated through 8 buffers", "value": gbps, "unit": "GB/s",
-            "us_per_step": wall_ms * 1e3, "dtype": "int8 x bf16 -> f32",
-            "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                         "frac": gbps / PEAK_HBM_GBPS, "traffic": TRAFFIC_GEMV_M1 if m == 1 else None,
-                         "kernel": "vecops_hip::skinny_w8a16_stream_kernel" if m == 1 else
-                                   "vecops_hip::skinny_w8a16_stream_rows_kernel" if m == 2 else
-                                   "vecops_hip::skinny_w8a16_mfma_resident_kernel",
-                         "algorithmic_bytes_per_launch": nbytes}}
+            "bf16 activations, bf16 out, weights rotated through 8 buffers (BASELINE configs[4])", "value": gbps,
+            "unit": "GB/s", "us_per_step": t["wall_ms"] * 1e3, "dtype": "int8 x bf16 -> f32",
+            "roofline": _roofline("hbm", gbps, PEAK_HBM_GBPS, "GB/s", kernel=kernel, algorithmic_bytes_per_launch=nbytes,
+                                  **(_traffic("gemv_m1") if m == 1 else {"traffic": None}), **_timing_fields(t))}
 
 
 def bench_copy(dev, steps, warmup):
@@ -226,47 +351,70 @@ def bench_copy(dev, steps, warmup):
     nbytes = 1 << 30
     src = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
     dst = torch.empty_like(src)
-    wall_ms, ev_ms = _time_launches(lambda i: dst.copy_(src), steps, warmup)
+    t = _measure(lambda i: dst.copy_(src), steps, warmup)
     return {"metric": "device_copy_gbps", "workload": "torch copy_ of 1 GiB (reads 1 GiB, writes 1 GiB)",
             "bytes_read_per_launch": nbytes, "bytes_written_per_launch": nbytes,
-            "value": 2.0 * nbytes / (ev_ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall_ms}
+            "value": 2.0 * nbytes / (t["event_ms"] * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": t["wall_ms"]}
+
+
+def recorded_reference():
+    """vecops' own CPU matmul on the headline workload, as timed in the build container by oracle/time_reference.py
+    (the vecops tree is not present where the benchmark runs): figures with their provenance, or None."""
+    path = os.path.join(ROOT, "oracle", "reference_timings.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        doc = json.load(f)
+    rows = [e for e in doc["entries"] if e["config"].startswith("bf16 4096^3")]
+    return {"source": "oracle/reference_timings.json (oracle/time_reference.py, in the build container)",
+            "what": doc["what"], "host": doc["host"],
+            "entries": [{"config": e["config"], "lanes": e["lanes"], "value": e["rate"] / 1e3, "unit": "TFLOP/s",
+                         "ms": e["ms"]} for e in rows]}
 
 
 def cpu_baseline(a, b_kn):
-    """The bf16 4096^3 workload on the host cores: the real vecops CPU matmul when
-    oracle/_ref runs here (AMX host), else the oracle's vectorised all-core port, on a
-    bounded row slab of the same operands."""
+    """The bf16 4096^3 workload on the host cores: the real vecops CPU matmul when oracle/_ref runs here (AMX host),
+    else the oracle's vectorised all-core port, on a bounded row slab of the same operands.  The reference's own
+    figures from the build container ride along either way."""
     import numpy as np
     from oracle.oracle import Oracle, Reference
     n = 4096
-    b_nk = np.ascontiguousarray(b_kn.T)
     ref = Reference.load()
     budget_s = 12.0
     if ref is not None:
         c = np.zeros((n, n), np.uint16)
         reps, t0 = 0, time.perf_counter()
         while reps == 0 or time.perf_counter() - t0 < budget_s:
-            ref.matmul_bf16_bf16(a, b_nk, c)
+            ref.dense_bf16_bf16(a, b_kn, c, b_is_kn=True)
             reps += 1
         dt = (time.perf_counter() - t0) / reps
-        return {"value": 2.0 * n ** 3 / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "reference",
-                "sample": f"full 4096^3 product x {reps}, vecops ops::matmul<AMX_BF16F32> on one thread "
-                          f"({dt * 1e3:.0f} ms each, B pre-transposed to [N,K])"}
-    oracle = Oracle()
-    rows = 256
-    t0 = time.perf_counter()
-    oracle.matmul_bf16_dense(a[:rows], b_nk, out_bf16=True)
-    probe = time.perf_counter() - t0
-    rows = int(min(n, max(256, 256 * (budget_s / max(probe, 1e-3)))))
-    rows -= rows % 256
-    reps, t0 = 0, time.perf_counter()
-    while reps == 0 or time.perf_counter() - t0 < budget_s:
+        out = {"value": 2.0 * n ** 3 / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "reference",
+               "sample": f"full 4096^3 product x {reps}, vecops ops::matmul<AMX_BF16F32> on one thread, dense tensors, "
+                         f"B as the transposed view of [K,N] ({dt * 1e3:.0f} ms each)"}
+    else:
+        oracle = Oracle()
+        b_nk = np.ascontiguousarray(b_kn.T)
+        rows = 256
+        t0 = time.perf_counter()
         oracle.matmul_bf16_dense(a[:rows], b_nk, out_bf16=True)
-        reps += 1
-    dt = (time.perf_counter() - t0) / reps
-    return {"value": 2.0 * rows * n * n / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.threads(), "kind": "port",
-            "sample": f"first {rows} of 4096 rows of A against all of B, {reps} times ({dt:.2f} s each), "
-                      "oracle C port, OpenMP"}
+        probe = time.perf_counter() - t0
+        rows = int(min(n, max(256, 256 * (budget_s / max(probe, 1e-3)))))
+        rows -= rows % 256
+        reps, t0 = 0, time.perf_counter()
+        while reps == 0 or time.perf_counter() - t0 < budget_s:
+            oracle.matmul_bf16_dense(a[:rows], b_nk, out_bf16=True)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        out = {"value": 2.0 * rows * n * n / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.threads(), "kind": "port",
+               "sample": f"first {rows} of 4096 rows of A against all of B, {reps} times ({dt:.2f} s each), "
+                         "oracle C port, OpenMP"}
+    recorded = recorded_reference()
+    if recorded:
+        out["recorded_reference"] = recorded
+    return out
+
+
+ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "fp32", "batched"]
 
 
 def main() -> int:
@@ -275,8 +423,11 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant"], help="run a single workload (for profiling)")
+    ap.add_argument("--only", choices=ONLY, help="run a single workload (for profiling)")
     ap.add_argument("--gemv-m", type=int, default=1, help="activation rows of the --only gemv workload (1..16)")
+    ap.add_argument("--ceiling-dtype", choices=["bf16", "int8"], default="bf16", help="operands of --only mfma_ceiling")
+    ap.add_argument("--fp32-compute", choices=["bf16", "f32"], default="bf16", help="compute type of --only fp32")
+    ap.add_argument("--batched-shape", default="777,1000,3001", help="M,N,K of --only batched")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the matmul path is built and measured on a single MI355X "
@@ -291,44 +442,47 @@ def main() -> int:
     capi.lib()  # fails loudly when the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.synchronize()
+    K, W = args.steps, args.warmup
 
-    if args.only == "int8":
-        print(json.dumps(bench_int8_dequant(dev, args.steps, args.warmup)))
-        return 0
-    if args.only == "copy":
-        print(json.dumps(bench_copy(dev, args.steps, args.warmup)))
-        return 0
-    if args.only == "bf16_packed":
-        print(json.dumps(bench_bf16_gemm_packed(dev, args.steps, args.warmup)))
-        return 0
-    if args.only == "int8_packed":
-        print(json.dumps(bench_int8_dequant_packed(dev, args.steps, args.warmup)))
-        return 0
-    if args.only == "runtime_quant":
-        print(json.dumps(bench_runtime_quant(dev, args.steps, args.warmup)))
-        return 0
-    if args.only == "gemv":
-        print(json.dumps(bench_gemv(dev, args.steps, args.warmup, m=args.gemv_m)))
+    single = {
+        "int8": lambda: bench_int8_dequant(dev, K, W),
+        "copy": lambda: bench_copy(dev, K, W),
+        "bf16_packed": lambda: bench_bf16_gemm_packed(dev, K, W),
+        "int8_packed": lambda: bench_int8_dequant_packed(dev, K, W),
+        "runtime_quant": lambda: bench_runtime_quant(dev, K, W),
+        "gemv": lambda: bench_gemv(dev, K, W, m=args.gemv_m),
+        "mfma_ceiling": lambda: bench_mfma_ceiling(dev, K, W, args.ceiling_dtype),
+        "fp32": lambda: bench_fp32_gemm(dev, K, W, args.fp32_compute),
+        "batched": lambda: bench_batched(dev, K, W, *[int(v) for v in args.batched_shape.split(",")]),
+    }
+    if args.only in single:
+        print(json.dumps(single[args.only]()))
         return 0
 
-    main_res = bench_bf16_gemm(dev, args.steps, args.warmup)
+    main_res = bench_bf16_gemm(dev, K, W)
     a, b_kn = main_res.pop("host")
     line = {
         "metric": "bf16_gemm_4096_tflops", "value": main_res["value"], "unit": "TFLOP/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["wall_ms"], "higher_is_better": True,
+        "steps": K, "warmup": W, "ms_per_step": main_res["wall_ms"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "bf16 GEMM M=N=K=4096, A[M,K] and B[K,N] row-major, normal(0,0.02), fp32 accumulate, "
                                "bf16 output (BASELINE configs[1])", "M": 4096, "N": 4096, "K": 4096},
         "roofline": main_res["roofline"],
     }
     if args.only != "bf16":
-        line["secondary"] = [bench_int8_dequant(dev, args.steps, args.warmup),
-                             bench_gemv(dev, max(args.steps, 200), args.warmup, m=1),
-                             bench_gemv(dev, max(args.steps, 200), args.warmup, m=4),
-                             bench_gemv(dev, max(args.steps, 200), args.warmup, m=16),
-                             bench_bf16_gemm_packed(dev, args.steps, args.warmup),
-                             bench_int8_dequant_packed(dev, args.steps, args.warmup),
-                             bench_runtime_quant(dev, args.steps, args.warmup)]
+        ceiling_bf16 = bench_mfma_ceiling(dev, K, W, "bf16")
+        ceiling_int8 = bench_mfma_ceiling(dev, K, W, "int8")
+        # what the machine sustains on these operand values with nothing but matrix instructions: the practical
+        # ceiling (the clocks follow the power the multipliers draw); `frac` stays against the nominal peak
+        line["roofline"]["measured_ceiling"] = ceiling_bf16["value"]
+        line["roofline"]["frac_of_ceiling"] = line["roofline"]["achieved"] / ceiling_bf16["value"]
+        line["secondary"] = [bench_int8_dequant(dev, K, W, ceiling=ceiling_int8["value"]),
+                             bench_gemv(dev, K, W, m=1), bench_gemv(dev, K, W, m=4), bench_gemv(dev, K, W, m=16),
+                             bench_fp32_gemm(dev, K, W, "bf16"), bench_fp32_gemm(dev, K, W, "f32")]
+        line["secondary"] += [bench_batched(dev, K, W, m, n, k)
+                              for (m, n, k) in [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)]]
+        line["secondary"] += [bench_bf16_gemm_packed(dev, K, W), bench_int8_dequant_packed(dev, K, W),
+                              bench_runtime_quant(dev, K, W), ceiling_bf16, ceiling_int8]
     if not args.no_cpu and args.only is None:
         line["cpu_baseline"] = cpu_baseline(a, b_kn)
     print(json.dumps(line))

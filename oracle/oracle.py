@@ -318,6 +318,18 @@ class Reference:
             raise RuntimeError("reference matmul unavailable")
         return c
 
+    def dense_bf16_bf16(self, a, b, c, b_is_kn: bool = False):
+        """c = a . b^T on dense row-major tensors (the reference's fastest form): a [M,K], b [N,K] - or [K,N] seen
+        through the transposed view when b_is_kn -, c [M,N], all bf16 bits."""
+        m, k = a.shape
+        n = c.shape[1]
+        assert a.flags["C_CONTIGUOUS"] and b.flags["C_CONTIGUOUS"] and c.flags["C_CONTIGUOUS"]
+        rc = self.lib.vref_dense_bf16_bf16(C.c_void_p(a.ctypes.data), C.c_void_p(b.ctypes.data), C.c_void_p(c.ctypes.data),
+                                           C.c_int64(m), C.c_int64(n), C.c_int64(k), 1 if b_is_kn else 0)
+        if rc != 0:
+            raise RuntimeError("reference matmul unavailable")
+        return c
+
     def matmul_runtime_quant(self, a, b, multipliers, zero_point, correction, row_scales=None, column_scales=None):
         """fp32 a quantised on the way in (per-row multiplier, zero point) x int8 b + correction row;
         int32 sums, or the dequantised fp32 when both scale vectors are given."""

@@ -153,6 +153,30 @@ int run_fused(const TA* a, const TB* b, const TBias* bias, TC* c, int64_t m, int
   return 0;
 }
 
+// ---- dense forms, for timing the reference at its best ----------------------------------------------
+// The entry points above describe every tensor with run-time strides, the most general form; vecops plans its
+// kernels from the layout types, and a dense row-major layout (unit inner stride known at compile time) is the
+// form its own benchmarks use (benchmarks/ops/MatmulBenchCommon.h:133-190).  A conventional B[K,N] is the
+// transposed view of a dense [K,N] tensor (tests/ops/MatmulOrientationTest.cpp:65-70).
+template <typename T>
+auto dense2(T* p, int64_t rows, int64_t cols) {
+  return make_tensor(p, make_layout(make_shape(Any{rows}, Any{cols})));
+}
+template <typename T>
+auto dense3(T* p, int64_t batch, int64_t rows, int64_t cols) {
+  return make_tensor(p, make_layout(make_shape(Any{batch}, Any{rows}, Any{cols})));
+}
+template <typename Atom, typename A, typename B, typename Cc>
+int run_dense(A at, B bt, Cc ct, int64_t m, int64_t n, int64_t k) {
+  if (!enable_amx()) return -1;
+  auto op = ops::matmul(ops::MatmulConfig<Atom>{});
+  const nint_t bytes = op.required_workspace(Any{m}, Any{n}, Any{k}, at, bt, ct);
+  kernel::Workspace ws(bytes);
+  auto v = ws.view();
+  op(v, Any{m}, Any{n}, Any{k}, at, bt, ct);
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -283,6 +307,37 @@ VREF_EXPORT int vref_matmul_i8_fused(const int8_t* a, const int8_t* b, const int
 }
 
 // The non-inline dispatch predicates of src/MatmulRuntimeDispatch.cpp:12-32.
+VREF_EXPORT int vref_dense_bf16_bf16(const uint16_t* a, const uint16_t* b, uint16_t* c, int64_t m, int64_t n, int64_t k,
+                                     int b_is_kn) {
+  auto at = dense2(reinterpret_cast<bfloat16_t*>(const_cast<uint16_t*>(a)), m, k);
+  auto ct = dense2(reinterpret_cast<bfloat16_t*>(c), m, n);
+  bfloat16_t* bp = reinterpret_cast<bfloat16_t*>(const_cast<uint16_t*>(b));
+  if (b_is_kn) return run_dense<matmul::AMX_BF16F32>(at, tensor::transpose_view<0, 1>(dense2(bp, k, n)), ct, m, n, k);
+  return run_dense<matmul::AMX_BF16F32>(at, dense2(bp, n, k), ct, m, n, k);
+}
+
+VREF_EXPORT int vref_dense_f32_f32(const float* a, const float* b, float* c, int64_t m, int64_t n, int64_t k, int b_is_kn) {
+  auto at = dense2(const_cast<float*>(a), m, k);
+  auto ct = dense2(c, m, n);
+  float* bp = const_cast<float*>(b);
+  if (b_is_kn) return run_dense<matmul::AMX_BF16F32>(at, tensor::transpose_view<0, 1>(dense2(bp, k, n)), ct, m, n, k);
+  return run_dense<matmul::AMX_BF16F32>(at, dense2(bp, n, k), ct, m, n, k);
+}
+
+VREF_EXPORT int vref_dense_bf16_f32_batched(const uint16_t* a, const uint16_t* b, float* c, int64_t batch, int64_t m,
+                                            int64_t n, int64_t k) {
+  return run_dense<matmul::AMX_BF16F32>(dense3(reinterpret_cast<bfloat16_t*>(const_cast<uint16_t*>(a)), batch, m, k),
+                                        dense3(reinterpret_cast<bfloat16_t*>(const_cast<uint16_t*>(b)), batch, n, k),
+                                        dense3(c, batch, m, n), m, n, k);
+}
+
+VREF_EXPORT int vref_dense_i8_dequant(const int8_t* a, const int8_t* b, const float* row_scales, const float* column_scales,
+                                      float* c, int64_t m, int64_t n, int64_t k) {
+  auto deq = matmul::make_runtime_per_row_column_dequantize_transform({row_scales, column_scales, 0});
+  return run_dense<matmul::AMX_I8I32<int8_t, int8_t>>(dense2(const_cast<int8_t*>(a), m, k), dense2(const_cast<int8_t*>(b), n, k),
+                                                      tensor::output<int32_t>(dense2(c, m, n), deq), m, n, k);
+}
+
 VREF_EXPORT int vref_amx_small_vector_profitable(int shape, int64_t m, int64_t n, int64_t k) {
   return kernel::matmul_details::runtime_amx_small_vector_profitable(
     static_cast<kernel::matmul_details::SmallVectorShape>(shape), m, n, k);
