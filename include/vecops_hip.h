@@ -114,6 +114,38 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul(const VecopsHipOperand* a, const Vec
                                             void* workspace, uint64_t workspace_size, void* stream);
 
 /*
+ * The first tier of vecops' owner selection: an explicit family request (matmul::family_selection::Automatic /
+ * Prefer<F> / Require<F>, matmul/Family.h:216-239; consulted first by Backend<AMX>::run,
+ * matmul/details/kernel/amx/Backend.h:2724-2757).  PREFER takes the family when it can serve the call and the rule
+ * table's choice otherwise; REQUIRE returns 2 (not applicable) and launches nothing when it cannot - the C-ABI form
+ * of the exception of tests/ops/MatmulTest.cpp:514-536.  The tile families serve every non-empty product, the skinny
+ * family only its own shapes.  split_k = 0 leaves the K split to the rule table; another value (tile families only)
+ * fixes it, clamped to the K tiles there are.
+ */
+typedef enum VecopsHipFamilySelection {
+  VECOPS_HIP_SELECT_AUTOMATIC = 0,
+  VECOPS_HIP_SELECT_PREFER = 1,
+  VECOPS_HIP_SELECT_REQUIRE = 2
+} VecopsHipFamilySelection;
+
+typedef struct VecopsHipFamilyRequest {
+  uint32_t struct_size;  /* sizeof(VecopsHipFamilyRequest) */
+  uint32_t selection;    /* VecopsHipFamilySelection */
+  uint32_t family;       /* VecopsHipKernelFamily */
+  uint32_t split_k;      /* 0 = the rule table's */
+} VecopsHipFamilyRequest;
+
+/* vecops_hip_plan_matmul / vecops_hip_matmul under a family request (null = automatic). */
+VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul_family(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                        const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                        uint32_t compute, const VecopsHipFamilyRequest* request,
+                                                        VecopsHipPlan* plan);
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_family(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                   const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                   uint32_t compute, const VecopsHipFamilyRequest* request,
+                                                   void* workspace, uint64_t workspace_size, void* stream);
+
+/*
  * vecops_hip_matmul without a workspace argument, for callers that cannot allocate device memory at all:
  * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
  * vecops (its callers size and own every workspace, ops/Matmul.h:504-526).  The split-K partial sums and the

@@ -118,3 +118,47 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(capi, "LIB_PATH", "/nonexistent/libvecops_hip.so")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         capi.lib()
+
+
+def _plan_family(a, b, c, family, selection, split_k=0):
+    plan = capi.Plan()
+    request = capi.family_request(family, selection, split_k)
+    rc = capi.lib().vecops_hip_plan_matmul_family(C.byref(a), C.byref(b), None, C.byref(c), 0, C.byref(request), C.byref(plan))
+    return rc, plan
+
+
+def test_family_request_known_answers():
+    """The explicit family request (vecops' family_selection::Prefer / Require) is part of the pure planning function."""
+    big = (_operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (4096, 4096)))
+    for family in ("tile_256", "tile_128", "tile_64", "tile_256x128", "tile_128x256"):
+        rc, p = _plan_family(*big, family, capi.SELECT_REQUIRE)
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == 1 and p.workspace_bytes == 0
+    # a required family that cannot serve: not applicable; preferred: the rule table's own answer
+    rc, _ = _plan_family(*big, "skinny", capi.SELECT_REQUIRE)
+    assert rc == 2 and b"skinny" in capi.lib().vecops_hip_last_error()
+    rc, p = _plan_family(*big, "skinny", capi.SELECT_PREFER)
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
+    rc, _ = _plan_family(*big, "zero_k", capi.SELECT_REQUIRE)
+    assert rc == 2
+    # the caller's K split: clamped to the K tiles there are (4096 / 64 = 64), partial sums in the workspace
+    rc, p = _plan_family(*big, "tile_128", capi.SELECT_REQUIRE, split_k=4)
+    assert rc == 0 and p.split_k == 4 and p.workspace_bytes == 4 * 4096 * 4096 * 4
+    rc, p = _plan_family(*big, "tile_128", capi.SELECT_REQUIRE, split_k=1000)
+    assert rc == 0 and p.split_k == 64
+    # the skinny family on a decode shape; a tile family required there instead
+    skinny = (_operand(capi.BF16, (4, 4096)), _operand(capi.BF16, (14336, 4096)), _operand(capi.F32, (4, 14336)))
+    rc, p = _plan_family(*skinny, "skinny", capi.SELECT_REQUIRE)
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "skinny"
+    rc, p = _plan_family(*skinny, "tile_64", capi.SELECT_REQUIRE)
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64"
+    # malformed requests
+    request = capi.family_request(9, capi.SELECT_REQUIRE)
+    plan = capi.Plan()
+    assert capi.lib().vecops_hip_plan_matmul_family(C.byref(big[0]), C.byref(big[1]), None, C.byref(big[2]), 0,
+                                                    C.byref(request), C.byref(plan)) == 1
+    request = capi.family_request("tile_64", 5)
+    assert capi.lib().vecops_hip_plan_matmul_family(C.byref(big[0]), C.byref(big[1]), None, C.byref(big[2]), 0,
+                                                    C.byref(request), C.byref(plan)) == 1
+    # no request = automatic
+    assert capi.lib().vecops_hip_plan_matmul_family(C.byref(big[0]), C.byref(big[1]), None, C.byref(big[2]), 0, None,
+                                                    C.byref(plan)) == 0 and capi.FAMILY_NAMES[plan.family] == "tile_256"

@@ -113,7 +113,7 @@ def test_host_library_exports_every_declared_symbol(host):
 
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
-    assert len(files) == 36
+    assert len(files) == 60   # 36 + (6 required families x {bf16, i8} x {host, device})
     for f in files:
         name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
         assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
@@ -173,6 +173,30 @@ def test_resolve_picks_recipe_by_dtype_and_placement(host):
     with pytest.raises(H.HostError) as e:       # valid call, no artifact for G=32 -> NotFound from the provider
         w.resolve(H.Frame([x, wq, np.zeros((8, 8), np.float32), y], outputs=(3,)), {"G": 32})
     assert e.value.code == 3
+
+
+def test_family_specialization_is_part_of_the_key(host):
+    """`Family` on vecops::matmul: the kernel family the call requires (vecops' family_selection::Require<F> is part
+    of MatmulConfig, i.e. of the specialization); each family has artifacts of its own for bf16 and 8-bit operands."""
+    op = host.operator("vecops::matmul")
+    a, b, c = bf16((4, 8)), bf16((5, 8)), np.zeros((4, 5), np.float32)
+    names = {1: "tile_256", 2: "tile_128", 3: "tile_64", 4: "skinny", 6: "tile_256x128", 7: "tile_128x256"}
+    for code, name in names.items():
+        assert op.resolve(H.Frame([a, b, None, c], outputs=(3,)), {"Family": code}) == \
+            f"vecops::matmul;operands=bf16;compute=bf16;family={name};memory=host;backend=hip-gfx950"
+    ai, bi, ci = np.zeros((4, 8), np.int8), np.zeros((5, 8), np.uint8), np.zeros((4, 5), np.int32)
+    assert op.resolve(H.Frame([ai, bi, None, ci], outputs=(3,)), {"Family": 2}) == \
+        "vecops::matmul;operands=i8;compute=i32;family=tile_128;memory=host;backend=hip-gfx950"
+    # 0 = automatic: the plain artifact
+    assert "family" not in op.resolve(H.Frame([a, b, None, c], outputs=(3,)), {"Family": 0})
+    for bad in (5, 8, -1):                       # zero_k, unknown numbers: nothing a caller can require
+        with pytest.raises(H.HostError) as e:
+            op.resolve(H.Frame([a, b, None, c], outputs=(3,)), {"Family": bad})
+        assert e.value.code in (1, 2, 3)
+    a32, b32, c32 = np.zeros((4, 8), np.float32), np.zeros((5, 8), np.float32), np.zeros((4, 5), np.float32)
+    with pytest.raises(H.HostError) as e:        # fp32 operands: no such artifacts
+        op.resolve(H.Frame([a32, b32, None, c32], outputs=(3,)), {"Family": 2})
+    assert e.value.code in (2, 3)
 
 
 def test_schema_validation(host):

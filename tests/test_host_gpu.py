@@ -83,6 +83,50 @@ def test_matmul_device_tensors_and_workspace(host, oracle, device):
     assert rel_err(got, want) <= fp32_tol(k)
 
 
+def test_matmul_required_family(host, oracle, device):
+    """The `Family` specialization through Operator::invoke: the required family computes the product (host and device
+    tensors); a family that cannot serve the call is "not applicable" from the artifact, nothing is written."""
+    import torch
+    op = host.operator("vecops::matmul")
+    m, n, k = 300, 260, 1000
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, acc_f64=True)
+    for family in (1, 2, 3, 6, 7):
+        c = np.full((m, n), np.nan, np.float32)
+        op.invoke(H.Frame([a, b, None, c], outputs=(3,)), {"Family": family})
+        assert rel_err(c, want) <= fp32_tol(k), family
+    ta = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+    tb = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
+    tc = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    frame = H.Frame([ta, tb, None, tc], outputs=(3,))
+    assert "family=tile_128;memory=device" in op.resolve(frame, {"Family": 2})
+    need = op.workspace(frame, {"Family": 2})
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=device)
+    op.invoke(frame, {"Family": 2}, workspace=ws.data_ptr(), workspace_size=need)
+    assert rel_err(tc.cpu().numpy(), want) <= fp32_tol(k)
+    c = np.full((m, n), 7.0, np.float32)
+    with pytest.raises(H.HostError) as e:        # the skinny family cannot serve 300 x 260 x 1000
+        op.invoke(H.Frame([a, b, None, c], outputs=(3,)), {"Family": 4})
+    assert e.value.code == 2 and "skinny" in e.value.message
+    assert (c == 7.0).all()
+    # ... and serves its own shapes
+    m2, n2, k2 = 4, 1024, 512
+    a2 = synth.bf16_round(synth.uniform_pm1(3, (m2, k2)))
+    b2 = synth.bf16_round(synth.uniform_pm1(4, (n2, k2)))
+    c2 = np.full((m2, n2), np.nan, np.float32)
+    op.invoke(H.Frame([a2, b2, None, c2], outputs=(3,)), {"Family": 4})
+    want2 = np.zeros((m2, n2), np.float32)
+    oracle.matmul(a2, b2, want2, acc_f64=True)
+    assert rel_err(c2, want2) <= fp32_tol(k2)
+    # 8-bit integers, bit-exact
+    ai, bi = synth.int8_sym(5, (m, k)), synth.int8_sym(6, (n, k))
+    ci = np.zeros((m, n), np.int32)
+    op.invoke(H.Frame([ai, bi, None, ci], outputs=(3,)), {"Family": 6})
+    assert np.array_equal(ci, (ai.astype(np.int64) @ bi.astype(np.int64).T).astype(np.int32))
+
+
 def test_matmul_rank3_fp32_and_int8(host, oracle, device):
     import torch
     op = host.operator("vecops::matmul")

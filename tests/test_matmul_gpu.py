@@ -166,6 +166,143 @@ def test_layouts(device, oracle, layout):
     assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
 
 
+@pytest.mark.parametrize("a_t", [False, True])
+@pytest.mark.parametrize("b_t", [False, True])
+@pytest.mark.parametrize("c_t", [False, True])
+@pytest.mark.parametrize("dtype", ["bf16", "i8"])
+def test_eight_orientations(device, oracle, a_t, b_t, c_t, dtype):
+    """Every combination of A, B and C held transposed in memory - the eight orientations of
+    tests/ops/MatmulOrientationTest.cpp:139,249 - gives the values of the dense product, for a floating and an
+    integer atom, on a shape with ragged tiles in every direction."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = 150, 203, 333
+    if dtype == "bf16":
+        a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+        b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+        ta, tb = dev_bf16(a, device), dev_bf16(b, device)
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want, acc_f64=True)
+        out_dtype = torch.float32
+    else:
+        a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+        ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+        want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.int32)
+        out_dtype = torch.int32
+    if a_t:
+        ta = ta.t().contiguous().t()      # [M,K] view of a [K,M] array
+    if b_t:
+        tb = tb.t().contiguous().t()      # [N,K] view of a [K,N] array: the conventional B
+    if c_t:
+        c = torch.zeros((n, m), dtype=out_dtype, device=device).t()
+    else:
+        c = torch.zeros((m, n), dtype=out_dtype, device=device)
+    capi.matmul(ta, tb, c)
+    torch.cuda.synchronize()
+    if dtype == "bf16":
+        assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+    else:
+        assert np.array_equal(c.cpu().numpy(), want)
+
+
+TILE_FAMILIES = ["tile_256", "tile_128", "tile_64", "tile_256x128", "tile_128x256"]
+
+
+@pytest.mark.parametrize("family", TILE_FAMILIES)
+@pytest.mark.parametrize("dtype,layout", [("bf16", "nt"), ("bf16", "nn"), ("i8", "nt"), ("f32", "nn")])
+def test_required_family_equals_the_oracle(device, oracle, family, dtype, layout):
+    """The first tier of the owner selection: every tile family, required by the caller on one ragged shape (where the
+    rule table itself would take 64x64 tiles and split K), gives the oracle's product - and the plan says so."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = 300, 520, 1000
+    request = capi.family_request(family, capi.SELECT_REQUIRE)
+    if dtype == "i8":
+        a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+        ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+        c = torch.zeros((m, n), dtype=torch.int32, device=device)
+        want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.int32)
+    elif dtype == "f32":
+        a, b = synth.uniform_pm1(1, (m, k)), synth.uniform_pm1(2, (n, k))
+        ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+        c = torch.zeros((m, n), dtype=torch.float32, device=device)
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want, acc_f64=True)     # fp32 memory, bf16 compute
+    else:
+        a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+        b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+        ta, tb = dev_bf16(a, device), dev_bf16(b, device)
+        c = torch.zeros((m, n), dtype=torch.float32, device=device)
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want, acc_f64=True)
+    if layout == "nn":
+        tb = tb.t().contiguous().t()
+    plan = capi.plan_matmul_family(ta, tb, c, request)
+    assert capi.FAMILY_NAMES[plan.family] == family
+    capi.matmul_family(ta, tb, c, request)
+    torch.cuda.synchronize()
+    if dtype == "i8":
+        assert np.array_equal(c.cpu().numpy(), want)
+    else:
+        assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+    # and with the K split fixed by the caller (partial sums through the workspace)
+    split = capi.family_request(family, capi.SELECT_REQUIRE, split_k=3)
+    plan = capi.plan_matmul_family(ta, tb, c, split)
+    assert plan.split_k == 3 and plan.workspace_bytes >= 3 * m * n * 4
+    c.zero_()
+    capi.matmul_family(ta, tb, c, split)
+    torch.cuda.synchronize()
+    if dtype == "i8":
+        assert np.array_equal(c.cpu().numpy(), want)
+    else:
+        assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+
+
+def test_required_family_that_cannot_serve_is_rejected(device, oracle):
+    """family_selection::Require on a family that cannot serve the call is an error, not a fallback
+    (tests/ops/MatmulTest.cpp:514-536: RequiredFamilyRuntimeRejectionPropagatesAsException, 128^3 bf16 there too);
+    Prefer falls back to the rule table's choice."""
+    import torch
+    from vecops_amd import capi
+    m = n = k = 128
+    a = synth.bf16_round(synth.uniform_pm1(1, (m, k)))
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    ta, tb = dev_bf16(a, device), dev_bf16(b, device)
+    c = torch.full((m, n), 7.0, dtype=torch.float32, device=device)
+    with pytest.raises(capi.VecopsHipError) as info:
+        capi.matmul_family(ta, tb, c, capi.family_request("skinny", capi.SELECT_REQUIRE))
+    assert info.value.code == 2 and "skinny" in str(info.value)
+    torch.cuda.synchronize()
+    assert bool((c == 7.0).all())                                   # nothing was launched
+    automatic = capi.plan_matmul(ta, tb, c)
+    preferred = capi.plan_matmul_family(ta, tb, c, capi.family_request("skinny", capi.SELECT_PREFER))
+    assert preferred.family == automatic.family and preferred.split_k == automatic.split_k
+    capi.matmul_family(ta, tb, c, capi.family_request("skinny", capi.SELECT_PREFER))
+    torch.cuda.synchronize()
+    want = np.zeros((m, n), np.float32)
+    oracle.matmul(a, b, want, acc_f64=True)
+    assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+    # the skinny family on one of its own shapes, required; and a tile family required on that shape
+    m2, n2, k2 = 4, 1024, 512
+    a2 = synth.bf16_round(synth.uniform_pm1(3, (m2, k2)))
+    b2 = synth.bf16_round(synth.uniform_pm1(4, (n2, k2)))
+    want2 = np.zeros((m2, n2), np.float32)
+    oracle.matmul(a2, b2, want2, acc_f64=True)
+    for family in ("skinny", "tile_64", "tile_128"):
+        c2 = torch.zeros((m2, n2), dtype=torch.float32, device=device)
+        request = capi.family_request(family, capi.SELECT_REQUIRE)
+        assert capi.FAMILY_NAMES[capi.plan_matmul_family(dev_bf16(a2, device), dev_bf16(b2, device), c2, request).family] == family
+        capi.matmul_family(dev_bf16(a2, device), dev_bf16(b2, device), c2, request)
+        torch.cuda.synchronize()
+        assert rel_err(c2.cpu().numpy(), want2) <= fp32_tol(k2), family
+    # nothing to multiply: a tile family cannot be required of an empty product or of K = 0
+    empty = torch.zeros((0, n), dtype=torch.float32, device=device)
+    with pytest.raises(capi.VecopsHipError) as info:
+        capi.matmul_family(ta[:0], tb, empty, capi.family_request("tile_128", capi.SELECT_REQUIRE))
+    assert info.value.code == 2
+    capi.matmul_family(ta[:0], tb, empty, capi.family_request("none", capi.SELECT_REQUIRE))
+
+
 def test_batched_and_broadcast(device, oracle):
     """Rank 3: independent products over the batch; stride 0 broadcasts an operand
     (tests/ops/MatmulBatchTest.cpp:176-335)."""
@@ -254,8 +391,8 @@ def test_shared_b_batch_is_folded(device, oracle):
 
 @pytest.mark.parametrize("m,n,k", [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)])
 def test_config3_irregular_batch8(device, oracle, m, n, k):
-    """BASELINE config 3 at full size: batch 8, bf16 in, fp32 out.  All eight
-    products run on the GPU; the oracle checks batches 0 and 7 in full."""
+    """BASELINE config 3 at full size: batch 8, bf16 in, fp32 out.  All eight products run on the GPU; the oracle
+    checks batches 0 and 7 in full and 302 sampled sums of every batch."""
     import torch
     from vecops_amd import capi
     batch = 8
@@ -270,6 +407,14 @@ def test_config3_irregular_batch8(device, oracle, m, n, k):
         want = np.zeros((m, n), np.float32)
         oracle.matmul(a[bi], b[bi], want, acc_f64=True)
         assert rel_err(got[bi], want) <= fp32_tol(k)
+    # every batch against the oracle's sampled sums (a batch offset by one, a wrong batch stride or a skipped
+    # batch would leave batches 0 and 7 right)
+    rng = np.random.default_rng(m + n + k)
+    for bi in range(batch):
+        rows = np.concatenate([rng.integers(0, m, 300), [0, m - 1]])
+        cols = np.concatenate([rng.integers(0, n, 300), [n - 1, 0]])
+        want = oracle.matmul_sampled(a[bi], b[bi], rows, cols)
+        assert rel_err(got[bi][rows, cols], want) <= fp32_tol(k), f"batch {bi}"
 
 
 def test_explicit_c_input_and_aliasing(device, oracle):

@@ -29,6 +29,7 @@ EXPORTS = [
     "vecops_hip_matmul_runtime_quant_packed_b_workspace", "vecops_hip_matmul_runtime_quant_packed_b",
     "vecops_hip_static_workspace_bytes", "vecops_hip_matmul_static_workspace",
     "vecops_hip_mfma_stream_ops", "vecops_hip_mfma_stream",
+    "vecops_hip_plan_matmul_family", "vecops_hip_matmul_family",
 ]
 
 ACT_NONE, ACT_RELU, ACT_CLAMP, ACT_SIGMOID, ACT_SILU = 0, 1, 2, 3, 4
@@ -51,6 +52,24 @@ class Epilogue(C.Structure):
     _fields_ = [("struct_size", C.c_uint32), ("activation", C.c_uint32), ("flags", C.c_uint32), ("scale", C.c_float),
                 ("shift", C.c_float), ("clamp_lo", C.c_float), ("clamp_hi", C.c_float), ("row_scales", C.c_void_p),
                 ("column_scales", C.c_void_p)]
+
+
+class FamilyRequest(C.Structure):
+    _fields_ = [("struct_size", C.c_uint32), ("selection", C.c_uint32), ("family", C.c_uint32), ("split_k", C.c_uint32)]
+
+
+SELECT_AUTOMATIC, SELECT_PREFER, SELECT_REQUIRE = 0, 1, 2
+FAMILY_CODES = {name: code for code, name in FAMILY_NAMES.items()}
+
+
+def family_request(family, selection=SELECT_REQUIRE, split_k: int = 0) -> FamilyRequest:
+    """`family`: a name of FAMILY_NAMES or its number; the counterpart of family_selection::Require<F> / Prefer<F>."""
+    r = FamilyRequest()
+    r.struct_size = C.sizeof(FamilyRequest)
+    r.selection = selection
+    r.family = FAMILY_CODES[family] if isinstance(family, str) else int(family)
+    r.split_k = split_k
+    return r
 
 
 class VecopsHipError(RuntimeError):
@@ -76,6 +95,9 @@ def lib() -> C.CDLL:
         L.vecops_hip_plan_matmul.argtypes = [P, P, P, P, C.c_uint32, C.POINTER(Plan)]
         L.vecops_hip_matmul.argtypes = [P, P, P, P, C.c_uint32, C.c_void_p, C.c_uint64, C.c_void_p]
         L.vecops_hip_static_workspace_bytes.restype = C.c_uint64
+        R = C.POINTER(FamilyRequest)
+        L.vecops_hip_plan_matmul_family.argtypes = [P, P, P, P, C.c_uint32, R, C.POINTER(Plan)]
+        L.vecops_hip_matmul_family.argtypes = [P, P, P, P, C.c_uint32, R, C.c_void_p, C.c_uint64, C.c_void_p]
         L.vecops_hip_mfma_stream_ops.restype = C.c_uint64
         L.vecops_hip_mfma_stream_ops.argtypes = [C.c_uint32, C.c_int32, C.c_int32]
         L.vecops_hip_mfma_stream.argtypes = [C.c_uint32, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_void_p,
@@ -172,6 +194,31 @@ def matmul(a, b, c, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None
     ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
     _check(lib().vecops_hip_matmul(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None, C.byref(oc),
                                    compute, ws_ptr, ws_size, _stream_handle(stream)))
+    return c
+
+
+def plan_matmul_family(a, b, c, request: FamilyRequest, c_in=None, compute=COMPUTE_BF16) -> Plan:
+    plan = Plan()
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    _check(lib().vecops_hip_plan_matmul_family(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None,
+                                               C.byref(oc), compute, C.byref(request), C.byref(plan)))
+    return plan
+
+
+def matmul_family(a, b, c, request: FamilyRequest, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None):
+    """``matmul`` on the kernel family the caller prefers or requires (``family_request``)."""
+    import torch
+    plan = plan_matmul_family(a, b, c, request, c_in, compute)
+    if plan.workspace_bytes and (workspace is None or workspace.numel() * workspace.element_size()
+                                 < plan.workspace_bytes):
+        workspace = torch.empty(plan.workspace_bytes, dtype=torch.uint8, device=c.device)
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_family(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None,
+                                          C.byref(oc), compute, C.byref(request), ws_ptr, ws_size, _stream_handle(stream)))
     return c
 
 

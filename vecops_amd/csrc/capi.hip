@@ -212,6 +212,42 @@ bool skinny_applies(const Problem& pr) {
 // elements of K in one 128-byte K tile of the compute type
 int k_tile_elements(int src) { return src == SRC_I8 || src == SRC_I8_FLIP ? 128 : src == SRC_F32 ? 32 : 64; }
 
+// Workgroup tile of a tile family (0 x 0 for the others).
+void tile_of_family(uint32_t family, int* tile_m, int* tile_n) {
+  switch (family) {
+    case VECOPS_HIP_FAMILY_TILE_256: *tile_m = *tile_n = 256; break;
+    case VECOPS_HIP_FAMILY_TILE_256X128: *tile_m = 256; *tile_n = 128; break;
+    case VECOPS_HIP_FAMILY_TILE_128X256: *tile_m = 128; *tile_n = 256; break;
+    case VECOPS_HIP_FAMILY_TILE_128: *tile_m = *tile_n = 128; break;
+    case VECOPS_HIP_FAMILY_TILE_64: *tile_m = *tile_n = 64; break;
+    default: *tile_m = *tile_n = 0; break;
+  }
+}
+
+// Split-K factor and workspace of a plan whose family is a tile family: K is split when the tiles leave most
+// compute units idle (forced_split > 0: the caller's factor, clamped to the K tiles there are).
+void finish_tile_plan(const Problem& pr, VecopsHipPlan* plan, uint32_t forced_split) {
+  int tile_m = 0, tile_n = 0;
+  tile_of_family(plan->family, &tile_m, &tile_n);
+  const int64_t ktile = k_tile_elements(pr.src);
+  const int64_t k_tiles = (pr.k + ktile - 1) / ktile;
+  const int64_t wgs = ((pr.m + tile_m - 1) / tile_m) * ((pr.n + tile_n - 1) / tile_n) * pr.batch;
+  int64_t split = 1;
+  if (forced_split > 0) {
+    split = forced_split < k_tiles ? forced_split : k_tiles;
+  } else if (wgs < kComputeUnits / 2 && k_tiles >= 8) {
+    split = kComputeUnits / wgs;
+    if (split > k_tiles / 4) split = k_tiles / 4;
+    if (split > 64) split = 64;
+  }
+  if (split < 1) split = 1;
+  plan->split_k = static_cast<uint32_t>(split);
+  plan->workspace_bytes = 0;
+  if (split > 1) plan->workspace_bytes = static_cast<uint64_t>(split) * pr.batch * pr.m * pr.n * 4u;
+  // an unsigned 8-bit operand needs the sums of the other operand's rows: after the partials
+  if (pr.src == SRC_I8_FLIP) plan->workspace_bytes += static_cast<uint64_t>(pr.batch) * (pr.m + pr.n) * 4u;
+}
+
 // The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure
 // integer function of (operand class, m, n, k); it picks the workgroup tile by
 // how many tiles the problem yields against the 256 compute units and splits K
@@ -300,23 +336,75 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     tile_m = tile_n = 64;
   }
   plan->family = family;
-  const int64_t wgs = tiles2(tile_m, tile_n);
-  int64_t split = 1;
-  if (wgs < kComputeUnits / 2 && k_tiles >= 8) {
-    split = kComputeUnits / wgs;
-    if (split > k_tiles / 4) split = k_tiles / 4;
-    if (split > 64) split = 64;
-    if (split < 1) split = 1;
+  finish_tile_plan(pr, plan, 0);
+}
+
+const char* family_name(uint32_t family) {
+  static const char* const names[] = {"none", "tile_256", "tile_128", "tile_64", "skinny", "zero_k", "tile_256x128", "tile_128x256"};
+  return family < 8 ? names[family] : "unknown";
+}
+
+// The first tier of vecops' owner selection (matmul/details/kernel/amx/Backend.h:2724-2757; matmul/Family.h:216-239):
+// a caller may prefer or require a kernel family.  A family that cannot serve the call is skipped when preferred
+// and is an error when required (family_selection::Require turns an inapplicable family into a hard error,
+// tests/ops/MatmulTest.cpp:514-536).  The tile families serve every non-empty product; the skinny family only its
+// own shapes; none / zero_k only the degenerate problems they name.
+int32_t apply_request(const Problem& pr, const VecopsHipFamilyRequest* request, VecopsHipPlan* plan) {
+  if (request == nullptr || request->selection == VECOPS_HIP_SELECT_AUTOMATIC) return ST_OK;
+  if (request->struct_size < sizeof(VecopsHipFamilyRequest)) return fail(ST_INVALID, "matmul: family request record too short");
+  if (request->selection != VECOPS_HIP_SELECT_PREFER && request->selection != VECOPS_HIP_SELECT_REQUIRE)
+    return fail(ST_INVALID, "matmul: unknown family selection %u", request->selection);
+  if (request->family > VECOPS_HIP_FAMILY_TILE_128X256) return fail(ST_INVALID, "matmul: unknown family %u", request->family);
+  const bool degenerate = plan->family == VECOPS_HIP_FAMILY_NONE || plan->family == VECOPS_HIP_FAMILY_ZERO_K;
+  int tile_m = 0, tile_n = 0;
+  tile_of_family(request->family, &tile_m, &tile_n);
+  bool serves;
+  if (degenerate || tile_m == 0) {
+    // nothing to multiply: only the family that names the case; the skinny family: its own shapes
+    serves = request->family == plan->family ||
+             (request->family == VECOPS_HIP_FAMILY_SKINNY && !degenerate && skinny_applies(pr) && !(pr.dequant && pr.m >= pr.n));
+  } else {
+    serves = true;
   }
-  plan->split_k = static_cast<uint32_t>(split);
-  if (split > 1) plan->workspace_bytes = static_cast<uint64_t>(split) * pr.batch * pr.m * pr.n * 4u;
-  // an unsigned 8-bit operand needs the sums of the other operand's rows: after the partials
-  if (pr.src == SRC_I8_FLIP) plan->workspace_bytes += static_cast<uint64_t>(pr.batch) * (pr.m + pr.n) * 4u;
+  if (!serves) {
+    if (request->selection == VECOPS_HIP_SELECT_PREFER) return ST_OK;  // the rule table's choice stands
+    return fail(ST_NOT_APPLICABLE, "matmul: the required family %s cannot serve this call (the rule table chooses %s)",
+                family_name(request->family), family_name(plan->family));
+  }
+  if (request->family == plan->family && request->split_k == 0) return ST_OK;
+  plan->family = request->family;
+  if (tile_m != 0) {
+    finish_tile_plan(pr, plan, request->split_k);
+  } else {
+    plan->split_k = 1;
+    plan->workspace_bytes = 0;
+  }
+  return ST_OK;
+}
+
+// The rule table and the streaming kernels' grids are calibrated for the 256 compute units of an MI355X: a device
+// with another count (a partitioned one, another gfx950 part) would run correct but mistuned code, so the first
+// launch on each device checks and refuses loudly.
+int32_t check_device() {
+  static std::atomic<int> checked[64];
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail(ST_EXEC, "hipGetDevice: %s", hipGetErrorString(e));
+  if (device < 0 || device >= 64) return fail(ST_EXEC, "device ordinal %d out of range", device);
+  if (checked[device].load(std::memory_order_acquire) == 1) return ST_OK;
+  int units = 0;
+  e = hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device);
+  if (e != hipSuccess) return fail(ST_EXEC, "hipDeviceGetAttribute: %s", hipGetErrorString(e));
+  if (units != kComputeUnits)
+    return fail(ST_EXEC, "this library is calibrated for %d compute units; device %d has %d", kComputeUnits, device, units);
+  checked[device].store(1, std::memory_order_release);
+  return ST_OK;
 }
 
 int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* row_scales, const float* column_scales,
                     const int32_t* correction, void* workspace, uint64_t workspace_size, hipStream_t stream) {
   if (plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
+  if (int32_t rc = check_device(); rc != ST_OK) return rc;
   if (pr.a.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: a has no storage");
   if (pr.b.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: b has no storage");
   if (pr.packed_b && plan.family == VECOPS_HIP_FAMILY_SKINNY) return fail(ST_INVALID, "matmul: plan does not fit a packed b");
@@ -423,14 +511,9 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     return ST_OK;
   }
 
-  int tile_m = 64, tile_n = 64;
-  switch (plan.family) {
-    case VECOPS_HIP_FAMILY_TILE_256: tile_m = tile_n = 256; break;
-    case VECOPS_HIP_FAMILY_TILE_256X128: tile_m = 256; tile_n = 128; break;
-    case VECOPS_HIP_FAMILY_TILE_128X256: tile_m = 128; tile_n = 256; break;
-    case VECOPS_HIP_FAMILY_TILE_128: tile_m = tile_n = 128; break;
-    default: break;
-  }
+  int tile_m = 0, tile_n = 0;
+  tile_of_family(plan.family, &tile_m, &tile_n);
+  if (tile_m == 0) return fail(ST_INVALID, "matmul: plan names no kernel family (%u)", plan.family);
   const int ktile = k_tile_elements(pr.src);
   p.tiles_m = static_cast<int32_t>((pr.m + tile_m - 1) / tile_m);
   p.tiles_n = static_cast<int32_t>((pr.n + tile_n - 1) / tile_n);
@@ -939,6 +1022,30 @@ int32_t vecops_hip_matmul_static_workspace(const VecopsHipOperand* a, const Veco
   return run_problem(pr, plan, nullptr, nullptr, nullptr, address, plan.workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
+int32_t vecops_hip_plan_matmul_family(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                                      const VecopsHipOperand* c, uint32_t compute, const VecopsHipFamilyRequest* request,
+                                      VecopsHipPlan* plan) {
+  if (plan == nullptr) return fail(ST_INVALID, "plan_matmul_family: null plan");
+  Problem pr{};
+  int32_t rc = describe(a, b, c_in, c, compute, &pr);
+  if (rc != ST_OK) return rc;
+  choose(pr, plan);
+  return apply_request(pr, request, plan);
+}
+
+int32_t vecops_hip_matmul_family(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                                 const VecopsHipOperand* c, uint32_t compute, const VecopsHipFamilyRequest* request,
+                                 void* workspace, uint64_t workspace_size, void* stream) {
+  Problem pr{};
+  int32_t rc = describe(a, b, c_in, c, compute, &pr);
+  if (rc != ST_OK) return rc;
+  VecopsHipPlan plan;
+  choose(pr, &plan);
+  rc = apply_request(pr, request, &plan);
+  if (rc != ST_OK) return rc;
+  return run_problem(pr, plan, nullptr, nullptr, nullptr, workspace, workspace_size, static_cast<hipStream_t>(stream));
+}
+
 int32_t vecops_hip_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
                           const VecopsHipOperand* c, uint32_t compute, void* workspace, uint64_t workspace_size,
                           void* stream) {
@@ -1011,6 +1118,7 @@ int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t ldx, const int8_t* 
   p.group = static_cast<int32_t>(group);
   p.groups = static_cast<int32_t>(k / group);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (int32_t rc = check_device(); rc != ST_OK) return rc;
   // GPU rule table of the skinny family: matrix cores once the widening of a weight
   // byte can be shared by three or more activation rows
   const bool mfma_ok = group % 64 == 0 && (group == 64 || group == 128 || group == 256);

@@ -8,6 +8,7 @@
 //   -DVECOPS_ARTIFACT_DEVICE=<0|1>  0: tensors are host memory, staged through HBM here
 //                                   1: tensors are HIP device pointers, used in place
 //   -DVECOPS_ARTIFACT_GROUP=<G>     group size of kind 4
+//   -DVECOPS_ARTIFACT_FAMILY=<F>    vecops::matmul only: the kernel family the artifact's callers require (0: none)
 //
 // Each DSO exports exactly vecops_kernel_query_v1 (vecops runtime/KernelAbi.h:176)
 // and follows the callback contract of runtime/KernelAbi.h:129-131: status codes
@@ -262,8 +263,34 @@ constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_I32);
 #define COMPUTE_CODE VECOPS_HIP_COMPUTE_BF16
 #endif
 constexpr const char* kOperatorName = "vecops::matmul";
+// An artifact built with -DVECOPS_ARTIFACT_FAMILY=<VecopsHipKernelFamily> serves calls that REQUIRE that kernel
+// family (the `Family` specialization value; vecops' family_selection::Require<F>, matmul/Family.h:234-239): the
+// family is part of its key, and a call the family cannot serve fails with "not applicable".
+#ifndef VECOPS_ARTIFACT_FAMILY
+#define VECOPS_ARTIFACT_FAMILY 0
+#endif
+#if VECOPS_ARTIFACT_FAMILY == 0
+#define FAMILY_KEY ""
+#elif VECOPS_ARTIFACT_FAMILY == 1
+#define FAMILY_KEY ";family=tile_256"
+#elif VECOPS_ARTIFACT_FAMILY == 2
+#define FAMILY_KEY ";family=tile_128"
+#elif VECOPS_ARTIFACT_FAMILY == 3
+#define FAMILY_KEY ";family=tile_64"
+#elif VECOPS_ARTIFACT_FAMILY == 4
+#define FAMILY_KEY ";family=skinny"
+#elif VECOPS_ARTIFACT_FAMILY == 6
+#define FAMILY_KEY ";family=tile_256x128"
+#elif VECOPS_ARTIFACT_FAMILY == 7
+#define FAMILY_KEY ";family=tile_128x256"
+#else
+#error "VECOPS_ARTIFACT_FAMILY names no kernel family a caller can require"
+#endif
 constexpr const char* kKey =
-  "vecops::matmul;operands=" OPERANDS ";compute=" COMPUTE ";memory=" MEMORY_NAME ";backend=hip-gfx950";
+  "vecops::matmul;operands=" OPERANDS ";compute=" COMPUTE FAMILY_KEY ";memory=" MEMORY_NAME ";backend=hip-gfx950";
+constexpr VecopsHipFamilyRequest kFamilyRequest = {sizeof(VecopsHipFamilyRequest),
+                                                   VECOPS_ARTIFACT_FAMILY ? VECOPS_HIP_SELECT_REQUIRE : VECOPS_HIP_SELECT_AUTOMATIC,
+                                                   VECOPS_ARTIFACT_FAMILY, 0};
 
 #define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
   {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
@@ -297,7 +324,8 @@ int32_t plan(const VecopsCall* call, VecopsHipOperand ops[4], bool* has_cin, Vec
   ops[3].data = origin(c);
   if (cin != nullptr) ops[2].data = origin(cin);
 #endif
-  int32_t rc = vecops_hip_plan_matmul(&ops[0], &ops[1], *has_cin ? &ops[2] : nullptr, &ops[3], COMPUTE_CODE, out);
+  int32_t rc = vecops_hip_plan_matmul_family(&ops[0], &ops[1], *has_cin ? &ops[2] : nullptr, &ops[3], COMPUTE_CODE,
+                                             &kFamilyRequest, out);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
   return VECOPS_STATUS_OK;
 }
@@ -339,8 +367,8 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
     return report_hip(error, "allocating split-K scratch", e);
   ws_size = p.workspace_bytes;
 #endif
-  int32_t rc = vecops_hip_matmul(&ops[0], &ops[1], has_cin ? &ops[2] : nullptr, &ops[3], COMPUTE_CODE, ws, ws_size,
-                                 stream);
+  int32_t rc = vecops_hip_matmul_family(&ops[0], &ops[1], has_cin ? &ops[2] : nullptr, &ops[3], COMPUTE_CODE,
+                                        &kFamilyRequest, ws, ws_size, stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
   return finish(&staging, stream, error);
 }

@@ -180,6 +180,26 @@ rt::Result<DType> compute_type(const rt::KernelCall& call) {
   return invalid("ComputeType must be a DType");
 }
 
+// The `Family` specialization value of vecops::matmul: the number of a kernel family the call requires (vecops'
+// family_selection::Require<F>, matmul/Family.h:234-239), or absent / 0 for the automatic choice.  Returns the
+// family's name in the specialization key ("" for automatic).
+rt::Result<std::string> required_family(const rt::KernelCall& call) {
+  auto it = call.values().find("Family");
+  if (it == call.values().end()) return std::string();
+  const auto* f = std::get_if<std::int64_t>(&it->second);
+  if (f == nullptr) return invalid("Family must be an integer (a VecopsHipKernelFamily number)");
+  switch (*f) {
+    case 0: return std::string();
+    case 1: return std::string("tile_256");
+    case 2: return std::string("tile_128");
+    case 3: return std::string("tile_64");
+    case 4: return std::string("skinny");
+    case 6: return std::string("tile_256x128");
+    case 7: return std::string("tile_128x256");
+    default: return invalid("Family names no kernel family a caller can require");
+  }
+}
+
 rt::Result<std::int64_t> group_size(const rt::KernelCall& call) {
   auto it = call.values().find("G");
   if (it == call.values().end()) return std::int64_t{128};
@@ -345,6 +365,11 @@ Status MatmulRecipe::match(const rt::KernelCall& call) const {
   } else if (operands_ == OperandClass::F16 && compute.value() != DType::BFloat16 && compute.value() != DType::Float16) {
     return not_applicable("half operands are multiplied in half");  // (BFloat16 is the default of an absent ComputeType)
   }
+  auto family = required_family(call);
+  if (!family) return family.status();
+  // artifacts that require a family exist for the bf16 and the 8-bit integer class
+  if (!family.value().empty() && operands_ != OperandClass::BF16 && operands_ != OperandClass::I8)
+    return not_applicable("a required kernel family is served for bf16 and 8-bit integer operands");
   auto place = placement_of(call);
   if (!place) return place.status();
   return Status::success();
@@ -360,7 +385,9 @@ rt::Result<rt::BoundKernelRecipe> MatmulRecipe::bind(const rt::KernelCall& call)
                         : f32_compute ? "f32" : "bf16";
   rt::BoundKernelRecipe bound;
   bound.recipe_id = id_;
+  const std::string family = required_family(call).value();
   bound.specialization_key = std::string(kMatmulName) + ";operands=" + operands + ";compute=" + compute +
+                             (family.empty() ? std::string() : ";family=" + family) +
                              ";memory=" + placement_name(place) + ";" + kBackend;
   bound.artifact_key = id_ + ";" + bound.specialization_key;
   return bound;
