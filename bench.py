@@ -344,6 +344,32 @@ def bench_gemv(dev, steps, warmup, m=1):
                                   **(_traffic("gemv_m1") if m == 1 else {"traffic": None}), **_timing_fields(t))}
 
 
+def bench_tile_families(dev, steps, warmup):
+    """The measurement the rule table's tile-quality constants come from: bf16 4096^3 (B as [K,N]) and the int8
+    2048 x 4096 x 11008 product, required of every tile family in turn (vecops_hip_matmul_family)."""
+    import torch
+    from vecops_amd import capi, synth
+    families = ["tile_256", "tile_256x128", "tile_128x256", "tile_128", "tile_64"]
+    n = 4096
+    _, _, ta, tb = _bf16_operands(dev)
+    c = torch.empty((n, n), dtype=torch.bfloat16, device=dev)
+    m, k, nn = 2048, 4096, 11008
+    ai = torch.from_numpy(synth.int8_sym(1, (m, k))).to(dev)
+    bi = torch.from_numpy(synth.int8_sym(2, (nn, k))).to(dev)
+    ci = torch.empty((m, nn), dtype=torch.int32, device=dev)
+    rows = []
+    for family in families:
+        request = capi.family_request(family, capi.SELECT_REQUIRE)
+        t16 = _measure(lambda i: capi.matmul_family(ta, tb.t(), c, request), steps, warmup)
+        t8 = _measure(lambda i: capi.matmul_family(ai, bi, ci, request), steps, warmup)
+        rows.append({"family": family, "bf16_4096_us": t16["event_ms"] * 1e3, "int8_2048x4096x11008_us": t8["event_ms"] * 1e3})
+    base = rows[0]["bf16_4096_us"]
+    for r in rows:
+        r["bf16_quality_vs_tile_256"] = base / r["bf16_4096_us"]
+    return {"metric": "tile_family_calibration", "workload": "bf16 4096^3 (B as [K,N]) and int8 2048x4096x11008 -> int32 on "
+            "each required tile family", "unit": "us", "value": base, "families": rows}
+
+
 def bench_copy(dev, steps, warmup):
     """A plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
     counters of the other workloads are scaled by."""
@@ -414,7 +440,8 @@ def cpu_baseline(a, b_kn):
     return out
 
 
-ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "fp32", "batched"]
+ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "fp32", "batched",
+        "families"]
 
 
 def main() -> int:
@@ -454,6 +481,7 @@ def main() -> int:
         "mfma_ceiling": lambda: bench_mfma_ceiling(dev, K, W, args.ceiling_dtype),
         "fp32": lambda: bench_fp32_gemm(dev, K, W, args.fp32_compute),
         "batched": lambda: bench_batched(dev, K, W, *[int(v) for v in args.batched_shape.split(",")]),
+        "families": lambda: bench_tile_families(dev, K, W),
     }
     if args.only in single:
         print(json.dumps(single[args.only]()))

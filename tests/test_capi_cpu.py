@@ -53,8 +53,17 @@ def test_rule_table_known_answers():
     # config 4
     rc, p = _plan(_operand(capi.I8, (2048, 4096)), _operand(capi.I8, (11008, 4096)),
                   _operand(capi.I32, (2048, 11008)))
-    # 344 tiles of 256x256 in two rounds; 688 of 256x128 in three are not enough cheaper to be worth the smaller tile
-    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256" and p.split_k == 1
+    # 344 tiles of 256x256 would take two rounds, the second a third full; 1376 of 128x128 take six short ones
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1
+    # 8 x 777 x 1000: seven rows of 128x256 tiles pad M to 896, four rows of 256-row tiles would pad it to 1024
+    rc, p = _plan(_operand(capi.BF16, (8, 777, 3001)), _operand(capi.BF16, (8, 1000, 3001)),
+                  _operand(capi.F32, (8, 777, 1000)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128x256"
+    # problems of one and a half to two rounds of big tiles keep them
+    rc, p = _plan(_operand(capi.BF16, (5120, 5120)), _operand(capi.BF16, (5120, 5120)), _operand(capi.BF16, (5120, 5120)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
+    rc, p = _plan(_operand(capi.BF16, (2048, 4096)), _operand(capi.BF16, (14336, 4096)), _operand(capi.BF16, (2048, 14336)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
     # 3000^3: 144 big tiles in one part-filled round stay ahead of 576 small ones in three
     rc, p = _plan(_operand(capi.BF16, (3000, 3000)), _operand(capi.BF16, (3000, 3000)), _operand(capi.F32, (3000, 3000)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"

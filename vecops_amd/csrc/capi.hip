@@ -195,9 +195,10 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
 constexpr int kComputeUnits = 256;
 constexpr int kStreamGroupsPerUnit = 2;  // workgroups of 4 wavefronts per compute unit of the streaming GEMV
 // Work per compute unit and second of the smaller tiles relative to 256x256, per mille (see choose()): bf16 4096^3
-// forced onto each tile takes 132 / 167 / 162 / 159 us (256x256, 256x128, 128x256, 128x128; two or three 128x128
-// workgroups share a compute unit).
-constexpr int64_t kQuality256x128 = 800, kQuality128 = 820;
+// required of each tile family (`bench.py --only families`) takes 107 / 133 / 130 / 121 us (256x256, 256x128, 128x256,
+// 128x128; two or three 128x128 workgroups share a compute unit), int8 4096^3 68 / 83 / 84 / 79; the ratio of the
+// small tile falls to 0.78-0.80 at 8192^3.
+constexpr int64_t kQuality256x128 = 800, kQuality128 = 850;
 
 // bf16 x bf16, f16 x f16 or int8 x int8 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
 bool skinny_applies(const Problem& pr) {
@@ -287,9 +288,9 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
   // half the compute units busy; among those the cheapest wins, cost = rounds x tile area / quality -
   // so a part-filled last round, rows or columns of padding and a less efficient small tile are all
   // priced in one number (4096^3: 256 tiles of 256x256, one round; 2048x11008: 344 of them in two rounds, which
-  // 688 tiles of 256x128 in three or 1376 of 128x128 in six undercut by less than the margin below - measured
-  // 134 / 141 / 134 us; 4096x4224: 1056 tiles of 128x128, 174 us against 187 for 272 big ones whose second round
-  // is 6 % full; 8 x 777x1000: 256 tiles of 256x128, one round).
+  // 1376 tiles of 128x128 in six undercut - measured 117 us against 105, 119 for the 688 rectangles; 4096x4224:
+  // 1056 tiles of 128x128, 160 us against 172 for 272 big ones whose second round is 6 % full; 8 x 777x1000: 224
+  // tiles of 128x256 in one round; 5120^3, 2048x14336x4096, 8192^3: big tiles, 19-23 % ahead).
   struct Candidate { uint32_t family; int64_t tm, tn, quality; };
   const Candidate candidates[] = {{VECOPS_HIP_FAMILY_TILE_256, 256, 256, 1000},
                                   {VECOPS_HIP_FAMILY_TILE_256X128, 256, 128, kQuality256x128},
@@ -302,10 +303,15 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     const int64_t count = tiles2(c.tm, c.tn);
     if (count < kComputeUnits / 2) continue;
     const int64_t rounds = (count + kComputeUnits - 1) / kComputeUnits;
-    const int64_t cost = rounds * c.tm * c.tn * 1000 / c.quality;
-    // a smaller tile has to be 10 % cheaper: a part-filled round of big tiles runs faster than the count
-    // says (the chip is power-limited; 3000^3 as 144 big tiles beats 576 small ones in three rounds)
-    if (best_cost == INT64_MAX || cost * 11 < best_cost * 10) {
+    int64_t cost = rounds * c.tm * c.tn * 1000 / c.quality;
+    // a single part-filled round runs faster than a full one (the chip is power-limited: fewer busy compute units
+    // clock higher): half full costs three quarters (3000^3 as 144 big tiles 92 us against 108 for 576 small ones;
+    // 8 x 777 x 1000 x 3001 as 224 tiles of 128x256 65 us, as 256 of 256x128 73, as 128 of 256x256 86)
+    if (rounds == 1) cost = cost * (kComputeUnits + count) / (2 * kComputeUnits);
+    // a smaller tile has to be 10 % cheaper than a bigger one: the round count flatters it (more L2 traffic per
+    // flop, and its quality falls with the problem size)
+    const bool smaller = best_cost != INT64_MAX && c.tm * c.tn < tile_m * tile_n;
+    if (best_cost == INT64_MAX || (smaller ? cost * 11 < best_cost * 10 : cost < best_cost)) {
       best_cost = cost;
       family = c.family;
       tile_m = c.tm;
