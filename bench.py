@@ -40,8 +40,10 @@ REPETITIONS = 7
 # cannot be read from inside this process: these are the figures of the named summaries, for exactly these workloads.
 RECORDED_TRAFFIC = {
     "bf16": (int((98479.5 * 2.000 + 32768 * 1.000) * 1024), "profiles/tile_gemm_bf16_4096.md"),
-    "int8": (int((95283.3 * 2.000 + 88064 * 1.000) * 1024), "profiles/tile_gemm_int8_dequant_2048x4096x11008.md"),
-    "gemv_m1": (int((29647.4 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_stream_m1_4096x14336.md"),
+    "int8": (int((96790.0 * 2.000 + 88060 * 1.000) * 1024), "profiles/tile_gemm_int8_dequant_2048x4096x11008.md"),
+    "gemv_m1": (int((29650.0 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_stream_m1_4096x14336.md"),
+    "gemv_m4": (int((29760.0 * 2.000 + 128.1 * 1.000) * 1024), "profiles/skinny_w8a16_stream_m1_4096x14336.md"),
+    "gemv_m16": (int((30150.0 * 2.000 + 524.8 * 1.000) * 1024), "profiles/skinny_w8a16_stream_m1_4096x14336.md"),
     "bf16_packed": (int((98468.3 * 2.000 + 32768 * 1.000) * 1024),
                     "profiles/tile_gemm_packed_b_bf16_4096_int8_2048x4096x11008.md"),
     "int8_packed": (int((95160.6 * 2.000 + 88064 * 1.000) * 1024),
@@ -341,7 +343,7 @@ def bench_gemv(dev, steps, warmup, m=1):
             "bf16 activations, bf16 out, weights rotated through 8 buffers (BASELINE configs[4])", "value": gbps,
             "unit": "GB/s", "us_per_step": t["wall_ms"] * 1e3, "dtype": "int8 x bf16 -> f32",
             "roofline": _roofline("hbm", gbps, PEAK_HBM_GBPS, "GB/s", kernel=kernel, algorithmic_bytes_per_launch=nbytes,
-                                  **(_traffic("gemv_m1") if m == 1 else {"traffic": None}), **_timing_fields(t))}
+                                  **_traffic(f"gemv_m{m}"), **_timing_fields(t))}
 
 
 def bench_tile_families(dev, steps, warmup):
