@@ -164,6 +164,27 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_static_workspace(const VecopsHipOper
                                                              uint32_t compute, void* stream);
 
 /*
+ * Several independent products in one call: c[i] = c_in[i] + a[i] . b[i]^T for i < count, every group with its own
+ * extents, strides and pointers (irregular batches).  vecops' batch planner serves batches that share an operand by
+ * flattening them into one product (planning/families/ArchitectureBatchPlanner.h:30-160; vecops_hip_matmul does the
+ * same) and everything else batch by batch; this entry point is the form for batches that share nothing, not even
+ * their shapes.  a, b, c (and c_in, which may be null; an entry of rank 0 means "no C input for this group") are
+ * arrays of count descriptors obeying the rules of vecops_hip_matmul group by group.  Groups of bf16 x bf16 or
+ * int8 x int8 operands run as ONE launch over a table of problem records (written into the workspace by small
+ * kernels fed through their arguments: no host buffer has to outlive the call, nothing is allocated); any other
+ * operand class, a mix of classes, and groups with K = 0 run as launches of their own on the same stream.  Results
+ * are those of vecops_hip_matmul on each group (bit-equal when that call would not split K; otherwise equal up to the
+ * order of the fp32 sums).  workspace: vecops_hip_matmul_grouped_workspace bytes, 16-byte aligned.
+ */
+VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_grouped_workspace(uint32_t count, const VecopsHipOperand* a,
+                                                               const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                                                               const VecopsHipOperand* c, uint32_t compute);
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_grouped(uint32_t count, const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                    const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                    uint32_t compute, void* workspace, uint64_t workspace_size,
+                                                    void* stream);
+
+/*
  * Fused output transforms - the catalogue that vecops' tests build from
  * elementwise and lane-local output transforms on tensor::output
  * (tests/ops/MatmulFusionTest.cpp:29-112; tests/ops/MatmulConversionTestCommon.h:
@@ -258,11 +279,15 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_quantize_rows(const VecopsHipOperand* x, co
  * The runtime-quantised product of tests/ops/MatmulConversionTestCommon.h:1437-1540 in one call:
  *   q = quantize_rows(a);  acc = sum_k q[i,k] * b[j,k] + correction[j]  (AMX_I8I32<uint8_t, int8_t>, wrapping);
  *   c[i,j] = (float(acc) * row_scales[i]) * column_scales[j].
- * a f32 [M,K], b i8 [N,K], c f32 [M,N] (rank 2, any strides), or a [batch,M,K] and c [batch,M,N] whose
- * rows run on from batch to batch against the one b (multipliers and row_scales then have batch * M
- * entries: vecops' batch_stride = M); correction (int32[N], usually
+ * a f32 [M,K], b i8 [N,K], c f32 [M,N] (rank 2, any strides), or the batched forms of
+ * tests/ops/MatmulConversionTestCommon.h:1277-1434: a [batch,M,K] and c [batch,M,N] with b either rank 2 (one set of
+ * weights for every batch; when the rows of a and c run on from batch to batch the batches fold into one
+ * [batch * M, K] product) or [batch,N,K]; a batch stride of 0 on a or b shares that operand.  Batch strides of the
+ * vectors follow the reference's tests: multipliers and row_scales have batch * M entries (batch_stride = M) unless a
+ * is shared (then M entries), correction has batch * N entries when b is per batch, else N
+ * (vecops_hip_matmul_runtime_quant_batched takes the strides explicitly).  correction (usually
  * -zero_point * sum_k b[j,k], see vecops_hip_pack_b_compensated) may be null.  The workspace holds the
- * quantised activations (kept as q - 128 for the signed kernels), the correction row with 128 * sum_k b[j,k]
+ * quantised activations (kept as q - 128 for the signed kernels), the correction rows with 128 * sum_k b[j,k]
  * added, and the product's own scratch: vecops_hip_matmul_runtime_quant_workspace bytes, 16-byte aligned.
  * Bit-exact (the sums are integers mod 2^32 either way).
  */
@@ -274,6 +299,24 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand
                                                           const int32_t* correction, const float* row_scales,
                                                           const float* column_scales, const VecopsHipOperand* c,
                                                           void* workspace, uint64_t workspace_size, void* stream);
+
+/*
+ * The same with the batch strides given: batch i quantises with multipliers[i * scale_batch_stride + row], dequantises
+ * with row_scales[i * scale_batch_stride + row] (vecops' `batch_stride` of the two runtime transforms,
+ * matmul/Quantization.h:91-146,195-250) and adds correction[i * correction_batch_stride + col] (the strides {n or 0, 0, 1}
+ * of the reference's correction tensor).  a and c rank 3, b rank 2 or 3.
+ */
+VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_runtime_quant_batched_workspace(const VecopsHipOperand* a,
+                                                                             int64_t scale_batch_stride,
+                                                                             const VecopsHipOperand* b,
+                                                                             int64_t correction_batch_stride,
+                                                                             const VecopsHipOperand* c);
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_runtime_quant_batched(const VecopsHipOperand* a, const float* multipliers,
+                                                                  int32_t zero_point, int64_t scale_batch_stride,
+                                                                  const VecopsHipOperand* b, const int32_t* correction,
+                                                                  int64_t correction_batch_stride, const float* row_scales,
+                                                                  const float* column_scales, const VecopsHipOperand* c,
+                                                                  void* workspace, uint64_t workspace_size, void* stream);
 
 /* The same with b packed by vecops_hip_pack_b (int8; n rows) - exactly the operands of
  * tests/ops/MatmulConversionTestCommon.h:1484-1510, where B is packed first. */

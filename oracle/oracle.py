@@ -356,6 +356,32 @@ class Reference:
             raise RuntimeError("reference matmul unavailable")
         return c
 
+    def matmul_runtime_quant_batched(self, a, b, multipliers, zero_point, row_scales, column_scales, correction,
+                                     batch=None):
+        """The batched runtime-quantised product of tests/ops/MatmulConversionTestCommon.h:1277-1434 on the real
+        vecops build.  a [batch or 1, M, K] f32 and b [batch or 1, N, K] i8 (a leading extent of 1 = shared by every
+        batch, batch stride 0); multipliers / row_scales [a's batches * M]; correction [b's batches * N]."""
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        b = np.ascontiguousarray(b, dtype=np.int8)
+        batch = max(a.shape[0], b.shape[0]) if batch is None else batch
+        m, k = a.shape[1:]
+        n = b.shape[1]
+        mult = np.ascontiguousarray(multipliers, dtype=np.float32)
+        rs = np.ascontiguousarray(row_scales, dtype=np.float32)
+        corr = np.ascontiguousarray(correction, dtype=np.int32)
+        assert mult.size == a.shape[0] * m and rs.size == mult.size and corr.size == b.shape[0] * n
+        cs = np.zeros(n + 64, dtype=np.float32)  # unmasked vector load past n (Quantization.h:229-231)
+        cs[:n] = column_scales
+        c = np.empty((batch, m, n), dtype=np.float32)
+        rc = self.lib.vref_matmul_runtime_quant_batched(
+            C.c_void_p(a.ctypes.data), C.c_void_p(b.ctypes.data), C.c_void_p(mult.ctypes.data), C.c_int32(zero_point),
+            C.c_void_p(rs.ctypes.data), C.c_void_p(cs.ctypes.data), C.c_void_p(corr.ctypes.data),
+            C.c_void_p(c.ctypes.data), C.c_int64(batch), C.c_int64(m), C.c_int64(n), C.c_int64(k),
+            C.c_int(1 if a.shape[0] == 1 and batch > 1 else 0), C.c_int(1 if b.shape[0] == 1 and batch > 1 else 0))
+        if rc != 0:
+            raise RuntimeError("reference matmul unavailable")
+        return c
+
     def matmul_i8_dequant(self, a, b, row_scales, column_scales, correction=None):
         a = np.ascontiguousarray(a, dtype=np.int8)
         b = np.ascontiguousarray(b, dtype=np.int8)

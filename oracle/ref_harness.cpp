@@ -287,6 +287,33 @@ VREF_EXPORT int vref_matmul_runtime_quant(const float* a, const int8_t* b, const
   return 0;
 }
 
+// The batched form of the same pipeline (tests/ops/MatmulConversionTestCommon.h:1277-1434): a [batch,M,K] (batch
+// stride 0 when broadcast_a), b [batch,N,K] (0 when broadcast_b), the correction rows as a C input of strides
+// {N or 0, 0, 1}, multipliers and row_scales with batch stride M or 0, c fp32 [batch,M,N] dense.
+VREF_EXPORT int vref_matmul_runtime_quant_batched(const float* a, const int8_t* b, const float* multipliers,
+                                                  int32_t zero_point, const float* row_scales, const float* column_scales,
+                                                  const int32_t* correction, float* c, int64_t batch, int64_t m, int64_t n,
+                                                  int64_t k, int broadcast_a, int broadcast_b) {
+  if (!enable_amx()) return -1;
+  using Atom = matmul::AMX_I8I32<uint8_t, int8_t>;
+  auto at = view3(const_cast<float*>(a), batch, m, k, broadcast_a ? 0 : m * k, k, 1);
+  auto bt = view3(const_cast<int8_t*>(b), batch, n, k, broadcast_b ? 0 : n * k, k, 1);
+  auto cit = view3(const_cast<int32_t*>(correction), batch, m, n, broadcast_b ? 0 : n, 0, 1);
+  auto ct = view3(c, batch, m, n, m * n, n, 1);
+  const nint_t scale_stride = broadcast_a ? 0 : m;
+  auto quantize = matmul::make_runtime_per_row_asymmetric_quantize_transform({multipliers, &zero_point, scale_stride});
+  auto deq = matmul::make_runtime_per_row_column_dequantize_transform({row_scales, column_scales, scale_stride});
+  auto ain = tensor::input<uint8_t>(at, quantize);
+  auto bin = tensor::input<int8_t>(bt);
+  auto cin = tensor::input<int32_t>(cit);
+  auto cout = tensor::output<int32_t>(ct, deq);
+  auto op = ops::matmul(ops::MatmulConfig<Atom>{});
+  kernel::Workspace ws(op.required_workspace(Any{m}, Any{n}, Any{k}, ain, bin, cin, cout));
+  auto v = ws.view();
+  op(v, Any{m}, Any{n}, Any{k}, ain, bin, cin, cout);
+  return 0;
+}
+
 // c_kind: 0 fp32, 1 bf16, 3 uint8, 4 int8 (the dtype codes of include/vecops_hip.h are not used here).
 VREF_EXPORT int vref_matmul_bf16_fused(const uint16_t* a, const uint16_t* b, const float* bias, void* c, int c_kind,
                                        int64_t m, int64_t n, int64_t k, const FusedSpec* spec) {

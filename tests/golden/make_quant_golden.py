@@ -2,7 +2,8 @@
 activations quantised on the way in by RuntimePerRowAsymmetricQuantizeTransform
 (oracle/_ref/libvecops_ref.so, compiled from the vecops sources in the build container; needs AMX)
 for the inputs of tests/golden_cases.py: the edge-value table and the fused-rounding discriminator read
-back through an identity B, and the seeded pipeline cases QUANT_CASES (int32 sums and dequantised fp32).
+back through an identity B, the seeded pipeline cases QUANT_CASES (int32 sums and dequantised fp32), and the
+batched cases QUANT_BATCHED_CASES (shared or per-batch activations and weights; dequantised fp32).
 
     python tests/golden/make_quant_golden.py
 """
@@ -15,8 +16,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
-from golden_cases import (QUANT_CASES, QUANT_EDGE_ZERO_POINTS, make_quant_inputs, quant_edge_inputs,  # noqa: E402
-                          quant_fma_inputs)
+from golden_cases import (QUANT_BATCHED_CASES, QUANT_CASES, QUANT_EDGE_ZERO_POINTS, make_quant_batched_inputs,  # noqa: E402
+                          make_quant_inputs, quant_edge_inputs, quant_fma_inputs)
 from oracle.oracle import Reference  # noqa: E402
 
 
@@ -38,6 +39,11 @@ def main() -> None:
         out[case["name"] + "_f32"] = ref.matmul_runtime_quant(inp["a"], inp["b"], inp["multipliers"], case["zp"],
                                                               inp["correction"], inp["row_scales"],
                                                               inp["column_scales"])
+    for case in QUANT_BATCHED_CASES:
+        inp = make_quant_batched_inputs(case)
+        out[case["name"] + "_f32"] = ref.matmul_runtime_quant_batched(
+            inp["a"], inp["b"], inp["multipliers"], inp["zero_point"], inp["row_scales"], inp["column_scales"],
+            inp["correction"], batch=case["batch"])
     for name, value in out.items():
         print(f"{name:28s} -> {value.shape} {value.dtype}")
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vecops_quant_golden.npz")

@@ -188,6 +188,67 @@ QUANT_CASES = [
 ]
 
 
+# Batched runtime-quantised products (tests/ops/MatmulConversionTestCommon.h:1277-1434): "ref" cases use that test's own
+# operand formulas and sizes (tests/ops/MatmulFusionTest.cpp:103-108; it instantiates shared b and shared a - the other two
+# combinations are run here on the same formulas), "seeded" cases this repository's generators.
+QUANT_BATCHED_CASES = [
+    {"name": "rqb_ref_3x5x7x65_a_per_batch_b_shared", "kind": "ref", "batch": 3, "m": 5, "n": 7, "k": 65, "shared_a": False, "shared_b": True},
+    {"name": "rqb_ref_3x5x7x65_a_shared_b_per_batch", "kind": "ref", "batch": 3, "m": 5, "n": 7, "k": 65, "shared_a": True, "shared_b": False},
+    {"name": "rqb_ref_3x5x7x65_both_per_batch", "kind": "ref", "batch": 3, "m": 5, "n": 7, "k": 65, "shared_a": False, "shared_b": False},
+    {"name": "rqb_ref_3x5x7x33_both_shared", "kind": "ref", "batch": 3, "m": 5, "n": 7, "k": 33, "shared_a": True, "shared_b": True},
+    {"name": "rqb_4x37x150x300_both_per_batch", "kind": "seeded", "batch": 4, "m": 37, "n": 150, "k": 300, "shared_a": False, "shared_b": False},
+    {"name": "rqb_3x130x70x515_a_shared", "kind": "seeded", "batch": 3, "m": 130, "n": 70, "k": 515, "shared_a": True, "shared_b": False},
+]
+
+
+def make_quant_batched_inputs(case):
+    """a [batch or 1, M, K] f32, b [batch or 1, N, K] i8, multipliers / row_scales [a's batches * M], correction
+    [b's batches * N], column_scales [N], zero_point."""
+    import numpy as np
+    from vecops_amd import synth
+    batch, m, n, k = case["batch"], case["m"], case["n"], case["k"]
+    ab, bb = (1 if case["shared_a"] else batch), (1 if case["shared_b"] else batch)
+    if case["kind"] == "ref":
+        zp = 7
+        idx = np.arange(ab * m)
+        mult = (4 << (idx % 3)).astype(np.float32)
+        rs = (np.float32(1.0) / mult).astype(np.float32)
+        flat = np.arange(ab * m * k).reshape(ab * m, k)
+        a = ((flat % 7 - 3).astype(np.float32) * rs[:, None]).astype(np.float32).reshape(ab, m, k)
+        b = (-3 + (np.arange(bb * n * k) * 5 + 11) % 7).astype(np.int8).reshape(bb, n, k)
+        cs = (np.float32(0.03125) + (np.arange(n) % 5).astype(np.float32) * np.float32(0.0078125)).astype(np.float32)
+    else:
+        zp = 9
+        mult = (np.float32(4.0) * (np.float32(1.0) + synth.uniform_pm1(21, (ab * m,)) * np.float32(0.5))).astype(np.float32)
+        rs = (np.float32(1.0) / mult).astype(np.float32)
+        a = ((synth.uniform_pm1(22, (ab * m, k)) * np.float32(140.0) + np.float32(128 - zp)) / mult[:, None]).astype(np.float32)
+        a = a.reshape(ab, m, k)
+        b = synth.int8_sym(23, (bb * n, k)).reshape(bb, n, k)
+        cs = synth.scales(24, n)
+    correction = (-zp * b.astype(np.int64).sum(axis=2)).astype(np.int32).reshape(bb * n)
+    return {"a": a, "b": b, "multipliers": mult, "row_scales": rs, "column_scales": cs, "correction": correction,
+            "zero_point": zp}
+
+
+def quant_batched_by_oracle(oracle, inp, batch):
+    """The batched pipeline composed from the oracle's pinned pieces, batch by batch: quantise, u8 x s8 sums plus the
+    batch's correction row, per-row x per-column dequantisation."""
+    import numpy as np
+    from oracle import oracle as O
+    a, b = inp["a"], inp["b"]
+    m, n = a.shape[1], b.shape[1]
+    out = np.empty((batch, m, n), np.float32)
+    for i in range(batch):
+        ia, ib = (0 if a.shape[0] == 1 else i), (0 if b.shape[0] == 1 else i)
+        mult, rs = inp["multipliers"][ia * m:(ia + 1) * m], inp["row_scales"][ia * m:(ia + 1) * m]
+        q = oracle.quantize_rows(a[ia], mult, inp["zero_point"])
+        acc = np.zeros((m, n), np.int32)
+        oracle.matmul(q, b[ib], acc, cin=np.broadcast_to(inp["correction"][ib * n:(ib + 1) * n], acc.shape),
+                      atom=O.ATOM_I8I32, acc_f64=True, c_bf16=False)
+        out[i] = oracle.fused_outputs(acc, np.float32, row_scales=rs, column_scales=inp["column_scales"])
+    return out
+
+
 def quant_edge_inputs():
     """a [3,64] (each row the edge values, zero-padded), identity b [64,64]: the int32 sums are the bytes."""
     import numpy as np

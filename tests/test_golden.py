@@ -133,3 +133,18 @@ def test_runtime_quant_pipeline_matches_the_reference(oracle):
         assert np.array_equal(acc, gold[case["name"] + "_i32"]), case["name"]
         out = oracle.fused_outputs(acc, np.float32, row_scales=inp["row_scales"], column_scales=inp["column_scales"])
         assert np.array_equal(out.view(np.uint32), gold[case["name"] + "_f32"].view(np.uint32)), case["name"]
+
+
+def test_batched_runtime_quant_pipeline_matches_the_reference(oracle):
+    """Shared or per-batch activations and weights (tests/ops/MatmulConversionTestCommon.h:1277-1434, on that test's
+    own operands and on seeded ones): the oracle's pieces composed batch by batch against the real build, bit for bit."""
+    from golden_cases import QUANT_BATCHED_CASES, make_quant_batched_inputs, quant_batched_by_oracle
+    gold = np.load(QUANT_GOLDEN)
+    for case in QUANT_BATCHED_CASES:
+        inp = make_quant_batched_inputs(case)
+        out = quant_batched_by_oracle(oracle, inp, case["batch"])
+        assert np.array_equal(out.view(np.uint32), gold[case["name"] + "_f32"].view(np.uint32)), case["name"]
+    # the reference test's own expectation on its operands: every output an exact small multiple of the scales
+    inp = make_quant_batched_inputs(QUANT_BATCHED_CASES[0])
+    q = oracle.quantize_rows(inp["a"][0], inp["multipliers"][:5], 7)
+    assert np.array_equal(q.astype(np.int64), (np.arange(5 * 65).reshape(5, 65) % 7 - 3) + 7)

@@ -7,7 +7,8 @@ import os
 import numpy as np
 import pytest
 
-from golden_cases import (QUANT_CASES, QUANT_EDGE_ZERO_POINTS, make_quant_inputs, quant_edge_inputs)
+from golden_cases import (QUANT_BATCHED_CASES, QUANT_CASES, QUANT_EDGE_ZERO_POINTS, make_quant_batched_inputs,
+                          make_quant_inputs, quant_batched_by_oracle, quant_edge_inputs)
 from oracle import oracle as O
 from vecops_amd import synth
 
@@ -125,10 +126,79 @@ def test_runtime_quant_batched_activations_shared_weights(device, oracle):
                               dev(cs, device), c, correction=dev(corr, device))
     torch.cuda.synchronize()
     assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
-    gapped = torch.zeros((batch, m + 1, k), device=device)[:, :m]            # rows do not run on: refused, not wrong
-    with pytest.raises(capi.VecopsHipError) as e:
-        capi.matmul_runtime_quant(gapped, dev(mult, device), 8, dev(b, device), dev(rs, device), dev(cs, device), c)
-    assert e.value.code == 2
+    # rows that do not run on from batch to batch in a: quantised from where they are, the product still folds
+    gapped = torch.zeros((batch, m + 1, k), device=device)
+    gapped[:, :m] = dev(a.reshape(batch, m, k), device)
+    c.fill_(float("nan"))
+    capi.matmul_runtime_quant(gapped[:, :m], dev(mult, device), 8, dev(b, device), dev(rs, device), dev(cs, device), c,
+                              correction=dev(corr, device))
+    # ... and in c: batch by batch
+    cg = torch.full((batch, m + 2, n), float("nan"), device=device)
+    capi.matmul_runtime_quant(gapped[:, :m], dev(mult, device), 8, dev(b, device), dev(rs, device), dev(cs, device), cg[:, :m],
+                              correction=dev(corr, device))
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(cg[:, :m].cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert torch.isnan(cg[:, m:]).all()
+
+
+@pytest.mark.parametrize("case", QUANT_BATCHED_CASES, ids=[c["name"] for c in QUANT_BATCHED_CASES])
+def test_runtime_quant_batched_golden(device, case):
+    """Shared or per-batch activations and weights (tests/ops/MatmulConversionTestCommon.h:1277-1434; a batch stride of
+    0 shares an operand): bit for bit against the outputs of the real vecops build."""
+    import torch
+    from vecops_amd import capi
+    inp = make_quant_batched_inputs(case)
+    batch, m, n, k = case["batch"], case["m"], case["n"], case["k"]
+    a = dev(inp["a"], device).expand(batch, m, k)                   # a leading extent of 1 becomes batch stride 0
+    b = dev(inp["b"], device).expand(batch, n, k)
+    c = torch.full((batch, m, n), float("nan"), device=device)
+    capi.matmul_runtime_quant(a, dev(inp["multipliers"], device), inp["zero_point"], b, dev(inp["row_scales"], device),
+                              dev(inp["column_scales"], device), c, correction=dev(inp["correction"], device))
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), GOLD[case["name"] + "_f32"].view(np.uint32))
+
+
+@pytest.mark.parametrize("batch,m,n,k,shared_a,shared_b", [(4, 300, 520, 1030, False, False), (5, 64, 1000, 4096, True, False),
+                                                           (3, 7, 2048, 512, False, False), (6, 130, 130, 129, False, True)])
+def test_runtime_quant_batched_against_the_oracle(device, oracle, batch, m, n, k, shared_a, shared_b):
+    """Bigger batched shapes (several tiles per batch, a skinny M, K with a tail), operands with gaps between rows and
+    batches, and the explicit batch strides of vecops_hip_matmul_runtime_quant_batched - among them one set of scales
+    for per-batch activations (stride 0), which the conventional entry cannot say."""
+    import torch
+    from vecops_amd import capi
+    case = {"kind": "seeded", "batch": batch, "m": m, "n": n, "k": k, "shared_a": shared_a, "shared_b": shared_b}
+    inp = make_quant_batched_inputs(case)
+    want = quant_batched_by_oracle(oracle, inp, batch)
+    ab, bb = inp["a"].shape[0], inp["b"].shape[0]
+    a_store = torch.full((ab, m + 1, k + 4), float("nan"), device=device)
+    a_store[:, :m, :k] = dev(inp["a"], device)
+    b_store = torch.full((bb, n + 2, k + 16), 99, dtype=torch.int8, device=device)
+    b_store[:, :n, :k] = dev(inp["b"], device)
+    a, b = a_store[:, :m, :k].expand(batch, m, k), b_store[:, :n, :k].expand(batch, n, k)
+    c_store = torch.full((batch, m + 3, n + 4), float("nan"), device=device)
+    c = c_store[:, :m, :n]
+    mult, rs, cs = dev(inp["multipliers"], device), dev(inp["row_scales"], device), dev(inp["column_scales"], device)
+    corr = dev(inp["correction"], device)
+    capi.matmul_runtime_quant(a, mult, inp["zero_point"], b, rs, cs, c, correction=corr)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert torch.isnan(c_store[:, m:]).all() and torch.isnan(c_store[:, :, n:]).all()
+    # the same through the explicit strides
+    c_store.fill_(float("nan"))
+    capi.matmul_runtime_quant_batched(a, mult, inp["zero_point"], 0 if shared_a else m, b, rs, cs, c, correction=corr,
+                                      correction_batch_stride=0 if shared_b else n)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    if not shared_a:
+        # per-batch activations under ONE set of multipliers / scales (those of batch 0) and one correction row
+        inp0 = dict(inp, multipliers=np.tile(inp["multipliers"][:m], batch), row_scales=np.tile(inp["row_scales"][:m], batch),
+                    correction=np.tile(inp["correction"][:n], bb))
+        want0 = quant_batched_by_oracle(oracle, inp0, batch)
+        c_store.fill_(float("nan"))
+        capi.matmul_runtime_quant_batched(a, mult, inp["zero_point"], 0, b, rs, cs, c, correction=corr, correction_batch_stride=0)
+        torch.cuda.synchronize()
+        assert np.array_equal(c.cpu().numpy().view(np.uint32), want0.view(np.uint32))
 
 
 def test_runtime_quant_zero_extents_and_rejections(device):

@@ -30,6 +30,8 @@ EXPORTS = [
     "vecops_hip_static_workspace_bytes", "vecops_hip_matmul_static_workspace",
     "vecops_hip_mfma_stream_ops", "vecops_hip_mfma_stream",
     "vecops_hip_plan_matmul_family", "vecops_hip_matmul_family",
+    "vecops_hip_matmul_runtime_quant_batched_workspace", "vecops_hip_matmul_runtime_quant_batched",
+    "vecops_hip_matmul_grouped_workspace", "vecops_hip_matmul_grouped",
 ]
 
 ACT_NONE, ACT_RELU, ACT_CLAMP, ACT_SIGMOID, ACT_SILU = 0, 1, 2, 3, 4
@@ -132,6 +134,13 @@ def lib() -> C.CDLL:
         L.vecops_hip_matmul_runtime_quant_packed_b.argtypes = [P, C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p,
                                                                C.c_void_p, C.c_void_p, P, C.c_void_p, C.c_uint64,
                                                                C.c_void_p]
+        L.vecops_hip_matmul_runtime_quant_batched_workspace.restype = C.c_uint64
+        L.vecops_hip_matmul_runtime_quant_batched_workspace.argtypes = [P, C.c_int64, P, C.c_int64, P]
+        L.vecops_hip_matmul_runtime_quant_batched.argtypes = [P, C.c_void_p, C.c_int32, C.c_int64, P, C.c_void_p, C.c_int64,
+                                                              C.c_void_p, C.c_void_p, P, C.c_void_p, C.c_uint64, C.c_void_p]
+        L.vecops_hip_matmul_grouped_workspace.restype = C.c_uint64
+        L.vecops_hip_matmul_grouped_workspace.argtypes = [C.c_uint32, P, P, P, P, C.c_uint32]
+        L.vecops_hip_matmul_grouped.argtypes = [C.c_uint32, P, P, P, P, C.c_uint32, C.c_void_p, C.c_uint64, C.c_void_p]
         L.vecops_hip_plan_matmul_fused.argtypes = [P, P, P, P, C.c_uint32, E, C.POINTER(Plan)]
         L.vecops_hip_matmul_fused.argtypes = [P, P, P, P, C.c_uint32, E, C.c_void_p, C.c_uint64, C.c_void_p]
         _lib = L
@@ -322,6 +331,46 @@ def matmul_runtime_quant(a, multipliers, zero_point: int, b, row_scales, column_
         correction.data_ptr() if correction is not None else None, row_scales.data_ptr(), column_scales.data_ptr(),
         C.byref(oc), ws_ptr, ws_size, _stream_handle(stream)))
     return c
+
+
+def matmul_runtime_quant_batched(a, multipliers, zero_point: int, scale_batch_stride: int, b, row_scales, column_scales, c,
+                                 correction=None, correction_batch_stride: int = 0, workspace=None, stream=None):
+    """``matmul_runtime_quant`` on rank-3 operands with the batch strides of the scale vectors and of the correction
+    rows given (vecops' ``batch_stride`` of the runtime quantise / dequantise transforms)."""
+    import torch
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    need = lib().vecops_hip_matmul_runtime_quant_batched_workspace(C.byref(oa), int(scale_batch_stride), C.byref(ob),
+                                                                   int(correction_batch_stride), C.byref(oc))
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=c.device)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_runtime_quant_batched(
+        C.byref(oa), multipliers.data_ptr(), int(zero_point), int(scale_batch_stride), C.byref(ob),
+        correction.data_ptr() if correction is not None else None, int(correction_batch_stride), row_scales.data_ptr(),
+        column_scales.data_ptr(), C.byref(oc), ws_ptr, ws_size, _stream_handle(stream)))
+    return c
+
+
+def matmul_grouped(a_list, b_list, c_list, c_in_list=None, compute: int = 0, workspace=None, stream=None):
+    """Several independent products ``c[i] = c_in[i] + a[i] . b[i]^T`` in one call (irregular batches): bf16 or int8
+    groups run as one launch.  ``c_in_list`` entries may be None."""
+    import torch
+    count = len(a_list)
+    if not (len(b_list) == count and len(c_list) == count and (c_in_list is None or len(c_in_list) == count)):
+        raise ValueError("matmul_grouped: lists differ in length")
+    Operands = Operand * max(count, 1)
+    oa, ob, oc = Operands(*map(operand, a_list)), Operands(*map(operand, b_list)), Operands(*map(operand, c_list))
+    oi = None
+    if c_in_list is not None:
+        oi = Operands(*[operand(t) if t is not None else Operand() for t in c_in_list])
+    need = lib().vecops_hip_matmul_grouped_workspace(count, oa, ob, oi, oc, compute)
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=c_list[0].device)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_grouped(count, oa, ob, oi, oc, compute, ws_ptr, ws_size, _stream_handle(stream)))
+    return c_list
 
 
 def matmul_runtime_quant_packed_b(a, multipliers, zero_point: int, packed, row_scales, column_scales, c, correction=None,

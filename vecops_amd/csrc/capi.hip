@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <vector>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -90,14 +91,17 @@ struct Problem {
   int64_t batch, m, n, k;
   bool packed_b;  // b.data addresses a prepacked operand (vecops_hip_pack_b), shared by every batch
   bool dequant;   // the int32 accumulators leave through the per-row x per-column dequantisation
+  int64_t row_scales_bs, correction_bs;  // batch b reads row_scales[b * row_scales_bs + row], correction[b * correction_bs + col]
   const VecopsHipEpilogue* fused;  // non-null: c is written through the fused output transform
 };
 
 // Same rules as vecops' validate() (planning/families/ArchitectureFamily.h:1590-1652,
 // planning/families/GenericTiled.h:100-154) plus the dtype combinations this library implements.
 int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* cin,
-                 const VecopsHipOperand* c, uint32_t compute, Problem* pr, const VecopsHipEpilogue* fused = nullptr) {
+                 const VecopsHipOperand* c, uint32_t compute, Problem* pr, const VecopsHipEpilogue* fused = nullptr,
+                 bool may_fold = true) {
   pr->fused = fused;
+  pr->row_scales_bs = pr->correction_bs = 0;
   if (!normalise(a, &pr->a) || !normalise(b, &pr->b) || !normalise(c, &pr->c))
     return fail(ST_INVALID, "matmul: operands must be rank 2 or 3 with non-negative extents");
   pr->packed_b = false;
@@ -161,7 +165,7 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
   // the same product as [batch * M, K] x B - folded into one rank-2 problem, which fills bigger tiles
   // (vecops' shared-operand flattening, planning/families/ArchitectureFamily.h:430-463).
   auto rows_run_on = [](const View& v) { return v.bs == v.rows * v.rs; };
-  if (pr->batch > 1 && pr->b.bs == 0 && pr->m > 0 && rows_run_on(pr->a) && rows_run_on(pr->c) &&
+  if (may_fold && pr->batch > 1 && pr->b.bs == 0 && pr->m > 0 && rows_run_on(pr->a) && rows_run_on(pr->c) &&
       (!pr->has_cin || rows_run_on(pr->cin) || (pr->cin.bs == 0 && pr->cin.rs == 0)) &&
       pr->batch * pr->m <= INT32_MAX) {
     for (View* v : {&pr->a, &pr->c, &pr->cin}) {
@@ -171,6 +175,22 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
     }
     pr->b.batch = 1;
     pr->m *= pr->batch;
+    pr->batch = 1;
+  }
+  // The mirror case: one row of A for every batch (M = 1, batch stride 0) against weights whose rows run on from
+  // batch to batch, the outputs laid end to end: the [1, batch * N] product of A with [batch * N, K]
+  // (vecops' batch-columns flattening, planning/families/ArchitectureBatchPlanner.h:82-160).  A per-column C input
+  // shared by every batch has no such view and keeps the batched form.
+  auto cols_run_on = [](const View& v) { return v.bs == v.cols * v.cs; };
+  if (may_fold && pr->batch > 1 && pr->m == 1 && pr->a.bs == 0 && pr->n > 0 && rows_run_on(pr->b) && cols_run_on(pr->c) &&
+      (!pr->has_cin || cols_run_on(pr->cin)) && pr->batch * pr->n <= INT32_MAX) {
+    pr->b.rows *= pr->batch;
+    for (View* v : {&pr->c, &pr->cin}) v->cols *= pr->batch;
+    for (View* v : {&pr->a, &pr->b, &pr->c, &pr->cin}) {
+      v->batch = 1;
+      v->bs = 0;
+    }
+    pr->n *= pr->batch;
     pr->batch = 1;
   }
   pr->cin_kind = is_int ? OUT_I32 : pr->out_kind;
@@ -207,6 +227,8 @@ bool skinny_applies(const Problem& pr) {
   const int64_t per = pr.src == SRC_I8 ? 16 : 8;  // elements per 16 bytes
   if (!k_vector_ok(pr.a) || !k_vector_ok(pr.b) || pr.k % per != 0 || pr.k < 8 * per) return false;
   const int64_t narrow = pr.m < pr.n ? pr.m : pr.n, wide = pr.m < pr.n ? pr.n : pr.m;
+  // (the skinny kernels read one set of scales and one correction row for every batch)
+  if (pr.batch > 1 && (pr.row_scales_bs != 0 || pr.correction_bs != 0)) return false;
   return narrow <= 16 && wide >= 512 && pr.batch <= 65535;
 }
 
@@ -407,18 +429,14 @@ int32_t check_device() {
   return ST_OK;
 }
 
-int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* row_scales, const float* column_scales,
-                    const int32_t* correction, void* workspace, uint64_t workspace_size, hipStream_t stream) {
-  if (plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
-  if (int32_t rc = check_device(); rc != ST_OK) return rc;
-  if (pr.a.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: a has no storage");
-  if (pr.b.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: b has no storage");
-  if (pr.packed_b && plan.family == VECOPS_HIP_FAMILY_SKINNY) return fail(ST_INVALID, "matmul: plan does not fit a packed b");
-  if (pr.c.data == nullptr) return fail(ST_INVALID, "matmul: c has no storage");
-  if (plan.workspace_bytes > workspace_size || (plan.workspace_bytes > 0 && workspace == nullptr))
-    return fail(ST_INVALID, "matmul: workspace of %llu bytes required, %llu supplied",
-                (unsigned long long)plan.workspace_bytes, (unsigned long long)workspace_size);
+bool lines_up(const Problem& pr, const View& v, int64_t line_stride) {
+  const int64_t elem_bytes = (pr.src == SRC_BF16 || pr.src == SRC_F16) ? 2 : 1;
+  return aligned16(v.data) && (line_stride * elem_bytes) % 16 == 0 && (v.bs * elem_bytes) % 16 == 0;
+}
 
+// The kernels' parameter record of a problem, before any tiling is chosen.
+TileGemmParams base_params(const Problem& pr, const float* row_scales, const float* column_scales, const int32_t* correction,
+                           void* workspace) {
   TileGemmParams p;
   memset(&p, 0, sizeof(p));
   p.a = pr.a.data;
@@ -429,6 +447,8 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   p.row_scales = row_scales;
   p.column_scales = column_scales;
   p.correction = correction;
+  p.row_scales_bs = pr.batch > 1 ? pr.row_scales_bs : 0;
+  p.correction_bs = pr.batch > 1 ? pr.correction_bs : 0;
   p.m = static_cast<int32_t>(pr.m);
   p.n = static_cast<int32_t>(pr.n);
   p.k = static_cast<int32_t>(pr.k);
@@ -458,6 +478,37 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
       p.ep_column_scales = ep.column_scales;
     }
   }
+
+  return p;
+}
+
+// How a problem's operands can be fetched (LoadMode), from the plan's vector flags and the operands' alignment.
+int fetch_mode(const Problem& pr, const VecopsHipPlan& plan) {
+  int mode = MODE_GENERIC;
+  if (plan.vector_a && k_vector_ok(pr.b)) mode = MODE_KVEC;
+  else if (plan.vector_a && plan.vector_b && plan.b_layout == 1) mode = MODE_NVEC_B;
+  // 16-byte aligned bases, rows and batches: the loads may write LDS themselves
+  if ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr, pr.a, pr.a.rs)) {
+    if (mode == MODE_KVEC && lines_up(pr, pr.b, pr.b.rs)) mode = MODE_KVEC_DMA;
+    else if (mode == MODE_NVEC_B && lines_up(pr, pr.b, pr.b.cs)) mode = MODE_NVEC_B_DMA;
+  }
+  return mode;
+}
+
+int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* row_scales, const float* column_scales,
+                    const int32_t* correction, void* workspace, uint64_t workspace_size, hipStream_t stream) {
+  if (plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
+  if (int32_t rc = check_device(); rc != ST_OK) return rc;
+  if (pr.a.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: a has no storage");
+  if (pr.b.data == nullptr && pr.k > 0) return fail(ST_INVALID, "matmul: b has no storage");
+  if (pr.packed_b && plan.family == VECOPS_HIP_FAMILY_SKINNY) return fail(ST_INVALID, "matmul: plan does not fit a packed b");
+  if (pr.c.data == nullptr) return fail(ST_INVALID, "matmul: c has no storage");
+  if (plan.workspace_bytes > workspace_size || (plan.workspace_bytes > 0 && workspace == nullptr))
+    return fail(ST_INVALID, "matmul: workspace of %llu bytes required, %llu supplied",
+                (unsigned long long)plan.workspace_bytes, (unsigned long long)workspace_size);
+
+  TileGemmParams p = base_params(pr, row_scales, column_scales, correction, workspace);
+  const bool is_int = pr.src == SRC_I8 || pr.src == SRC_I8_FLIP;
 
   if (plan.family == VECOPS_HIP_FAMILY_ZERO_K) {
     p.split_k = 0;  // empty sum: the reduce kernel emits epilogue(0)
@@ -526,18 +577,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   const int k_tiles = static_cast<int>((pr.k + ktile - 1) / ktile);
   p.split_k = static_cast<int32_t>(plan.split_k);
   p.k_tiles_per_split = (k_tiles + p.split_k - 1) / p.split_k;
-  int mode = MODE_GENERIC;
-  if (plan.vector_a && k_vector_ok(pr.b)) mode = MODE_KVEC;
-  else if (plan.vector_a && plan.vector_b && plan.b_layout == 1) mode = MODE_NVEC_B;
-  // 16-byte aligned bases, rows and batches: the loads may write LDS themselves
-  const int64_t elem_bytes = (pr.src == SRC_BF16 || pr.src == SRC_F16) ? 2 : 1;
-  auto lines_up = [&](const View& v, int64_t line_stride) {
-    return aligned16(v.data) && (line_stride * elem_bytes) % 16 == 0 && (v.bs * elem_bytes) % 16 == 0;
-  };
-  if ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr.a, pr.a.rs)) {
-    if (mode == MODE_KVEC && lines_up(pr.b, pr.b.rs)) mode = MODE_KVEC_DMA;
-    else if (mode == MODE_NVEC_B && lines_up(pr.b, pr.b.cs)) mode = MODE_NVEC_B_DMA;
-  }
+  const int mode = fetch_mode(pr, plan);
 
   hipError_t e;
   if (pr.src == SRC_I8_FLIP) {
@@ -548,7 +588,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     p.a_flip = pr.a_unsigned ? 0x80808080u : 0u;
     p.b_flip = pr.b_unsigned ? 0x80808080u : 0u;
     if (pr.b_unsigned) {  // + 128 * sum_k a'[m,k] per row
-      e = launch_byte_row_sums(pr.a.data, p.batch, p.m, p.k, pr.a.bs, pr.a.rs, pr.a.cs, p.a_flip, 128u, nullptr, row_term, stream);
+      e = launch_byte_row_sums(pr.a.data, p.batch, p.m, p.k, pr.a.bs, pr.a.rs, pr.a.cs, p.a_flip, 128u, nullptr, 0, row_term, stream);
       if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
       p.row_term = row_term;
     }
@@ -557,7 +597,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
       if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
       p.col_term = col_term;
     } else if (pr.a_unsigned) {  // + 128 * sum_k b'[n,k] per column
-      e = launch_byte_row_sums(pr.b.data, p.batch, p.n, p.k, pr.b.bs, pr.b.rs, pr.b.cs, p.b_flip, 128u, nullptr, col_term, stream);
+      e = launch_byte_row_sums(pr.b.data, p.batch, p.n, p.k, pr.b.bs, pr.b.rs, pr.b.cs, p.b_flip, 128u, nullptr, 0, col_term, stream);
       if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
       p.col_term = col_term;
     }
@@ -570,7 +610,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     }
   }
   if (pr.packed_b) {
-    const int a_mode = plan.vector_a == 0 ? 0 : ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr.a, pr.a.rs)) ? 2 : 1;
+    const int a_mode = plan.vector_a == 0 ? 0 : ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr, pr.a, pr.a.rs)) ? 2 : 1;
     e = launch_tile_gemm_packed_b(pr.src, p, tile_m, tile_n, a_mode, stream);
   } else switch (pr.src) {
     case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile_m, tile_n, mode, stream); break;
@@ -627,7 +667,7 @@ void launch_skinny_mfma_resident(const SkinnyW8A16Params& p, int passes, hipStre
 // Problem description of a matmul whose B operand is prepacked: b is described as the dense
 // [N,K] operand it was packed from (its strides are never used), with `packed` as its storage.
 int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t packed_dtype, int64_t n,
-                        const VecopsHipOperand* cin, const VecopsHipOperand* c, Problem* pr) {
+                        const VecopsHipOperand* cin, const VecopsHipOperand* c, Problem* pr, bool may_fold = true) {
   if (a == nullptr || (a->rank != 2 && a->rank != 3)) return fail(ST_INVALID, "matmul_packed_b: malformed a");
   if (n < 0) return fail(ST_INVALID, "matmul_packed_b: negative n");
   const uint32_t da = a->dtype;
@@ -652,7 +692,7 @@ int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t 
   b.sizes[base + 1] = k;
   b.strides[base] = k;
   b.strides[base + 1] = 1;
-  int32_t rc = describe(a, &b, cin, c, VECOPS_HIP_COMPUTE_BF16, pr);
+  int32_t rc = describe(a, &b, cin, c, VECOPS_HIP_COMPUTE_BF16, pr, nullptr, may_fold);
   if (rc != ST_OK) return rc;
   pr->packed_b = true;
   // 32-bit offsets inside one workgroup's eight 32-row panels of the packed operand
@@ -711,7 +751,7 @@ int32_t vecops_hip_pack_b_compensated(const VecopsHipOperand* b, int32_t a_zero_
   if (compensation == nullptr) return fail(ST_INVALID, "pack_b_compensated: null compensation");
   // -a_zero_point * sum_k b[n,k], wrapping like every int32 accumulator of the path
   hipError_t e = launch_byte_row_sums(v.data, 1, static_cast<int32_t>(v.rows), static_cast<int32_t>(v.cols), 0, v.rs, v.cs,
-                                      0u, 0u - static_cast<uint32_t>(a_zero_point), nullptr, compensation,
+                                      0u, 0u - static_cast<uint32_t>(a_zero_point), nullptr, 0, compensation,
                                       static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
   return ST_OK;
@@ -772,7 +812,7 @@ int32_t vecops_hip_quantize_rows(const VecopsHipOperand* x, const float* multipl
     return fail(ST_INVALID, "quantize_rows: extent too large");
   hipError_t e = launch_quantize_rows(static_cast<const float*>(vx.data), static_cast<int32_t>(vx.batch),
                                       static_cast<int32_t>(vx.rows), static_cast<int32_t>(vx.cols), vx.bs, vx.rs, vx.cs,
-                                      multipliers, zero_point, 0u, static_cast<uint8_t*>(vq.data), vq.bs, vq.rs, vq.cs,
+                                      multipliers, vx.rows, zero_point, 0u, static_cast<uint8_t*>(vq.data), vq.bs, vq.rs, vq.cs,
                                       static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(ST_EXEC, "quantize kernel launch: %s", hipGetErrorString(e));
   return ST_OK;
@@ -782,105 +822,159 @@ namespace {
 // The pieces of vecops_hip_matmul_runtime_quant.  The activations are quantised to q - 128 as int8 (the byte
 // xor 0x80), so that the product runs on the signed kernels with their fast dequantising epilogue, and
 //   sum_k q * b = sum_k (q - 128) * b + 128 * sum_k b[n,k]
-// goes into the correction row.  Workspace: M x K bytes of activations, N int32 of that row (both rounded up
-// to 256 bytes), then the product's own scratch.
+// goes into the correction rows.  Workspace: the quantised activations (one [M,K] matrix per batch, or a single
+// one when every batch shares activations and multipliers), the correction rows (N int32 per batch, or a single
+// row when every batch shares weights and correction) - both rounded up to 256 bytes - then the product's own
+// scratch.
 struct RuntimeQuant {
-  VecopsHipOperand q, c_acc, a_flat, c_flat;
+  VecopsHipOperand a3, b3, c3, q, c_acc;
   Problem pr{};
   VecopsHipPlan plan;
+  int64_t batch, m, n, k;
+  int64_t q_batches, row_batches;  // distinct quantised matrices / correction rows
+  int64_t scale_bs, correction_bs;
   uint64_t q_bytes, row_bytes;
 };
 
-// A rank-3 operand whose rows run on from batch to batch (batch stride = M x row stride) as the rank-2
-// [batch * M, cols] matrix it is in memory; rank 2 is passed through.
-bool fold_batches(const VecopsHipOperand* o, VecopsHipOperand* flat) {
-  *flat = *o;
-  if (o->rank != 3) return o->rank == 2;
-  if (o->sizes[0] > 1 && o->strides[0] != o->sizes[1] * o->strides[1]) return false;
-  memset(flat->sizes, 0, sizeof(flat->sizes));
-  memset(flat->strides, 0, sizeof(flat->strides));
-  flat->rank = 2;
-  flat->sizes[0] = o->sizes[0] * o->sizes[1];
-  flat->sizes[1] = o->sizes[2];
-  flat->strides[0] = o->strides[1];
-  flat->strides[1] = o->strides[2];
+// Rank 2 as the rank 3 of one batch.
+bool as_rank3(const VecopsHipOperand* o, VecopsHipOperand* out) {
+  if (o == nullptr || (o->rank != 2 && o->rank != 3)) return false;
+  *out = *o;
+  if (o->rank == 3) return true;
+  memset(out->sizes, 0, sizeof(out->sizes));
+  memset(out->strides, 0, sizeof(out->strides));
+  out->rank = 3;
+  out->sizes[0] = 1;
+  for (int i = 0; i < 2; ++i) { out->sizes[i + 1] = o->sizes[i]; out->strides[i + 1] = o->strides[i]; }
   return true;
 }
 
-// b is the int8 operand, or null with `packed` / `packed_n` describing weights packed by vecops_hip_pack_b.
-int32_t describe_runtime_quant(const VecopsHipOperand* a_given, const VecopsHipOperand* b, const void* packed,
-                               int64_t packed_n, const VecopsHipOperand* c_given, void* workspace, RuntimeQuant* d) {
-  if (a_given == nullptr || c_given == nullptr || a_given->rank != c_given->rank ||
-      (a_given->rank == 3 && a_given->sizes[0] != c_given->sizes[0]))
-    return fail(ST_INVALID, "matmul_runtime_quant: a and c must have the same rank and batch extent");
-  // one set of weights for every batch (the serving case; vecops' BroadcastB,
-  // tests/ops/MatmulConversionTestCommon.h:1277-1434): the batches of a and c fold into rows
-  if (!fold_batches(a_given, &d->a_flat) || !fold_batches(c_given, &d->c_flat))
-    return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: rank-3 a and c must have rows that run on from batch to batch");
-  const VecopsHipOperand* a = &d->a_flat;
-  const VecopsHipOperand* c = &d->c_flat;
-  if (a->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: a must be an f32 operand");
-  if (packed == nullptr && (b == nullptr || b->rank != 2 || b->dtype != DT_I8))
-    return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: b must be a rank-2 i8 operand");
-  if (c->dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: c must be an f32 operand");
-  const int64_t m = a->sizes[0], k = a->sizes[1], n = packed ? packed_n : b->sizes[0];
-  if (m < 0 || k < 0 || n < 0) return fail(ST_INVALID, "matmul_runtime_quant: negative extent");
-  d->q_bytes = (static_cast<uint64_t>(m) * static_cast<uint64_t>(k) + 255u) & ~uint64_t{255};
-  d->row_bytes = (static_cast<uint64_t>(n) * 4u + 255u) & ~uint64_t{255};
-  make_operand(&d->q, workspace, DT_I8, m, k, k);
-  d->c_acc = *c;
+// b is the int8 operand (rank 2: one set of weights for every batch; rank 3: its batch stride may be 0), or null with
+// `packed` / `packed_n` describing weights packed by vecops_hip_pack_b.  scale_bs / correction_bs: batch strides of
+// multipliers and row_scales / of the correction row (vecops' batch_stride of the two transforms,
+// matmul/Quantization.h:91-146,195-250; tests/ops/MatmulConversionTestCommon.h:1277-1434 runs M and 0, N and 0).
+int32_t describe_runtime_quant(const VecopsHipOperand* a_given, const VecopsHipOperand* b_given, const void* packed,
+                               int64_t packed_n, const VecopsHipOperand* c_given, int64_t scale_bs, int64_t correction_bs,
+                               void* workspace, RuntimeQuant* d) {
+  if (!as_rank3(a_given, &d->a3) || !as_rank3(c_given, &d->c3) || a_given->rank != c_given->rank)
+    return fail(ST_INVALID, "matmul_runtime_quant: a and c must be rank 2 or both rank 3");
+  if (d->a3.dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: a must be an f32 operand");
+  if (d->c3.dtype != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: c must be an f32 operand");
+  d->batch = d->c3.sizes[0];
+  d->m = d->a3.sizes[1];
+  d->k = d->a3.sizes[2];
+  if (d->a3.sizes[0] != d->batch) return fail(ST_INVALID, "matmul_runtime_quant: a and c differ in batch extent");
+  if (packed == nullptr) {
+    if (b_given == nullptr || b_given->dtype != DT_I8 || !as_rank3(b_given, &d->b3))
+      return fail(ST_NOT_APPLICABLE, "matmul_runtime_quant: b must be a rank-2 or rank-3 i8 operand");
+    if (b_given->rank == 2) {  // one set of weights for every batch
+      d->b3.sizes[0] = d->batch;
+      d->b3.strides[0] = 0;
+    } else if (a_given->rank != 3 || d->b3.sizes[0] != d->batch) {
+      return fail(ST_INVALID, "matmul_runtime_quant: a rank-3 b needs rank-3 a and c of the same batch extent");
+    }
+    d->n = d->b3.sizes[1];
+  } else {
+    d->n = packed_n;
+  }
+  if (d->batch < 0 || d->m < 0 || d->k < 0 || d->n < 0) return fail(ST_INVALID, "matmul_runtime_quant: negative extent");
+  if (scale_bs < 0 || correction_bs < 0) return fail(ST_INVALID, "matmul_runtime_quant: negative batch stride");
+  if (d->batch <= 1) scale_bs = correction_bs = 0;
+  d->scale_bs = scale_bs;
+  d->correction_bs = correction_bs;
+  const bool shared_b = packed != nullptr || d->b3.strides[0] == 0 || d->batch <= 1;
+  d->q_batches = (d->batch > 1 && (d->a3.strides[0] != 0 || scale_bs != 0)) ? d->batch : 1;
+  d->row_batches = (d->batch > 1 && (!shared_b || correction_bs != 0)) ? d->batch : 1;
+  d->q_bytes = (static_cast<uint64_t>(d->q_batches) * d->m * d->k + 255u) & ~uint64_t{255};
+  d->row_bytes = (static_cast<uint64_t>(d->row_batches) * d->n * 4u + 255u) & ~uint64_t{255};
+  // the quantised activations: dense [batch, M, K], every batch the same matrix when there is only one
+  memset(&d->q, 0, sizeof(d->q));
+  d->q.data = workspace;
+  d->q.dtype = DT_I8;
+  d->q.rank = a_given->rank;
+  const int base = a_given->rank == 3 ? 1 : 0;
+  if (base) { d->q.sizes[0] = d->batch; d->q.strides[0] = d->q_batches > 1 ? d->m * d->k : 0; }
+  d->q.sizes[base] = d->m; d->q.strides[base] = d->k;
+  d->q.sizes[base + 1] = d->k; d->q.strides[base + 1] = 1;
+  d->c_acc = *c_given;
   d->c_acc.dtype = DT_I32;  // accumulator class; the epilogue writes fp32
-  int32_t rc = packed ? describe_packed(&d->q, packed, DT_I8, n, nullptr, &d->c_acc, &d->pr)
-                      : describe(&d->q, b, nullptr, &d->c_acc, 0, &d->pr);
+  // Batches fold into rows ([batch * M, K] x the one B) only when the scales run on with the rows and one
+  // correction row serves every batch.
+  const bool may_fold = d->q_batches > 1 && scale_bs == d->m && d->row_batches == 1;
+  int32_t rc;
+  if (packed != nullptr) {
+    rc = describe_packed(&d->q, packed, DT_I8, d->n, nullptr, &d->c_acc, &d->pr, may_fold);
+  } else {
+    const VecopsHipOperand* b = a_given->rank == 3 ? &d->b3 : b_given;
+    rc = describe(&d->q, b, nullptr, &d->c_acc, 0, &d->pr, nullptr, may_fold);
+  }
   if (rc != ST_OK) return rc;
   d->pr.dequant = true;
+  if (d->pr.batch > 1) {
+    d->pr.row_scales_bs = scale_bs;
+    d->pr.correction_bs = d->row_batches > 1 ? d->n : 0;
+  }
   choose(d->pr, &d->plan);
   return ST_OK;
 }
-}  // namespace
 
-namespace {
-int32_t run_runtime_quant(const VecopsHipOperand* a, const float* multipliers, int32_t zero_point, const VecopsHipOperand* b,
-                          const void* packed, int64_t packed_n, const int32_t* correction, const float* row_scales,
-                          const float* column_scales, const VecopsHipOperand* c, void* workspace, uint64_t workspace_size,
-                          void* stream) {
+int32_t run_runtime_quant(const VecopsHipOperand* a, const float* multipliers, int32_t zero_point, int64_t scale_bs,
+                          const VecopsHipOperand* b, const void* packed, int64_t packed_n, const int32_t* correction,
+                          int64_t correction_bs, const float* row_scales, const float* column_scales,
+                          const VecopsHipOperand* c, void* workspace, uint64_t workspace_size, void* stream) {
   RuntimeQuant d{};
-  int32_t rc = describe_runtime_quant(a, b, packed, packed_n, c, workspace ? workspace : reinterpret_cast<void*>(256), &d);
+  int32_t rc = describe_runtime_quant(a, b, packed, packed_n, c, scale_bs, correction_bs,
+                                      workspace ? workspace : reinterpret_cast<void*>(256), &d);
   if (rc != ST_OK) return rc;
   if (d.plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
   if (row_scales == nullptr || column_scales == nullptr || multipliers == nullptr)
     return fail(ST_INVALID, "matmul_runtime_quant: multipliers and both scale vectors are required");
   if (packed != nullptr && d.pr.k > 0 && !aligned16(packed)) return fail(ST_INVALID, "matmul_runtime_quant: packed b must be 16-byte aligned");
+  if (d.batch * d.m > INT32_MAX || d.batch * d.n > INT32_MAX) return fail(ST_INVALID, "matmul_runtime_quant: extent too large");
   const uint64_t need = d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
   if (need > workspace_size || workspace == nullptr || !aligned16(workspace))
     return fail(ST_INVALID, "matmul_runtime_quant: %llu bytes of 16-byte aligned workspace required, %llu supplied",
                 (unsigned long long)need, (unsigned long long)workspace_size);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const View& va = d.pr.a;  // the quantised activations, dense
   View vx;
-  normalise(&d.a_flat, &vx);
-  hipError_t e = launch_quantize_rows(static_cast<const float*>(vx.data), 1, static_cast<int32_t>(vx.rows),
-                                      static_cast<int32_t>(vx.cols), 0, vx.rs, vx.cs, multipliers, zero_point, 0x80u,
-                                      static_cast<uint8_t*>(va.data), 0, va.rs, va.cs, s);
+  normalise(&d.a3, &vx);
+  hipError_t e = launch_quantize_rows(static_cast<const float*>(vx.data), static_cast<int32_t>(d.q_batches),
+                                      static_cast<int32_t>(d.m), static_cast<int32_t>(d.k), vx.bs, vx.rs, vx.cs,
+                                      multipliers, d.scale_bs, zero_point, 0x80u, static_cast<uint8_t*>(workspace),
+                                      d.m * d.k, d.k, 1, s);
   if (e != hipSuccess) return fail(ST_EXEC, "quantize kernel launch: %s", hipGetErrorString(e));
-  // correction[n] + 128 * sum_k b[n,k]
-  int32_t* row = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + d.q_bytes);
-  const View& vb = d.pr.b;
-  if (packed != nullptr)
-    e = launch_packed_row_sums(packed, static_cast<int32_t>(d.pr.n), static_cast<int32_t>(d.pr.k), 1, 128u, correction, row, s);
-  else
-    e = launch_byte_row_sums(vb.data, 1, static_cast<int32_t>(vb.rows), static_cast<int32_t>(vb.cols), 0, vb.rs, vb.cs, 0u,
-                             128u, correction, row, s);
+  // correction[batch][n] + 128 * sum_k b[batch][n,k]
+  int32_t* rows = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + d.q_bytes);
+  if (packed != nullptr) {
+    // one packed operand: the same sums for every batch, the caller's correction per batch
+    for (int64_t bi = 0; bi < d.row_batches && e == hipSuccess; ++bi)
+      e = launch_packed_row_sums(packed, static_cast<int32_t>(d.n), static_cast<int32_t>(d.k), 1, 128u,
+                                 correction ? correction + bi * d.correction_bs : nullptr, rows + bi * d.n, s);
+  } else {
+    View vb;
+    normalise(&d.b3, &vb);
+    e = launch_byte_row_sums(vb.data, static_cast<int32_t>(d.row_batches), static_cast<int32_t>(d.n),
+                             static_cast<int32_t>(d.k), vb.bs, vb.rs, vb.cs, 0u, 128u, correction, d.correction_bs, rows, s);
+  }
   if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
-  return run_problem(d.pr, d.plan, row_scales, column_scales, row, static_cast<char*>(workspace) + d.q_bytes + d.row_bytes,
+  return run_problem(d.pr, d.plan, row_scales, column_scales, rows, static_cast<char*>(workspace) + d.q_bytes + d.row_bytes,
                      workspace_size - d.q_bytes - d.row_bytes, s);
+}
+
+// The batch strides of the reference's tests: scales run on with the rows of a ([batch * M]) unless every batch
+// shares a, the correction rows run on ([batch * N]) when the weights are per batch.
+void conventional_strides(const VecopsHipOperand* a, const VecopsHipOperand* b, int64_t* scale_bs, int64_t* correction_bs) {
+  *scale_bs = (a != nullptr && a->rank == 3 && a->strides[0] != 0) ? a->sizes[1] : 0;
+  *correction_bs = (b != nullptr && b->rank == 3 && b->strides[0] != 0) ? b->sizes[1] : 0;
 }
 }  // namespace
 
 uint64_t vecops_hip_matmul_runtime_quant_workspace(const VecopsHipOperand* a, const VecopsHipOperand* b,
                                                    const VecopsHipOperand* c) {
   RuntimeQuant d{};
-  if (describe_runtime_quant(a, b, nullptr, 0, c, reinterpret_cast<void*>(256), &d) != ST_OK) return 0;
+  int64_t scale_bs = 0, correction_bs = 0;
+  conventional_strides(a, b, &scale_bs, &correction_bs);
+  if (describe_runtime_quant(a, b, nullptr, 0, c, scale_bs, correction_bs, reinterpret_cast<void*>(256), &d) != ST_OK) return 0;
   return d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
 }
 
@@ -889,13 +983,38 @@ int32_t vecops_hip_matmul_runtime_quant(const VecopsHipOperand* a, const float* 
                                         const float* column_scales, const VecopsHipOperand* c, void* workspace,
                                         uint64_t workspace_size, void* stream) {
   if (b == nullptr) return fail(ST_INVALID, "matmul_runtime_quant: null b");
-  return run_runtime_quant(a, multipliers, zero_point, b, nullptr, 0, correction, row_scales, column_scales, c, workspace,
-                           workspace_size, stream);
+  int64_t scale_bs = 0, correction_bs = 0;
+  conventional_strides(a, b, &scale_bs, &correction_bs);
+  return run_runtime_quant(a, multipliers, zero_point, scale_bs, b, nullptr, 0, correction, correction_bs, row_scales,
+                           column_scales, c, workspace, workspace_size, stream);
+}
+
+uint64_t vecops_hip_matmul_runtime_quant_batched_workspace(const VecopsHipOperand* a, int64_t scale_batch_stride,
+                                                           const VecopsHipOperand* b, int64_t correction_batch_stride,
+                                                           const VecopsHipOperand* c) {
+  RuntimeQuant d{};
+  if (describe_runtime_quant(a, b, nullptr, 0, c, scale_batch_stride, correction_batch_stride, reinterpret_cast<void*>(256),
+                             &d) != ST_OK)
+    return 0;
+  return d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
+}
+
+int32_t vecops_hip_matmul_runtime_quant_batched(const VecopsHipOperand* a, const float* multipliers, int32_t zero_point,
+                                                int64_t scale_batch_stride, const VecopsHipOperand* b,
+                                                const int32_t* correction, int64_t correction_batch_stride,
+                                                const float* row_scales, const float* column_scales,
+                                                const VecopsHipOperand* c, void* workspace, uint64_t workspace_size,
+                                                void* stream) {
+  if (b == nullptr) return fail(ST_INVALID, "matmul_runtime_quant_batched: null b");
+  return run_runtime_quant(a, multipliers, zero_point, scale_batch_stride, b, nullptr, 0, correction, correction_batch_stride,
+                           row_scales, column_scales, c, workspace, workspace_size, stream);
 }
 
 uint64_t vecops_hip_matmul_runtime_quant_packed_b_workspace(const VecopsHipOperand* a, int64_t n, const VecopsHipOperand* c) {
   RuntimeQuant d{};
-  if (describe_runtime_quant(a, nullptr, reinterpret_cast<const void*>(256), n, c, reinterpret_cast<void*>(256), &d) != ST_OK)
+  int64_t scale_bs = 0, correction_bs = 0;
+  conventional_strides(a, nullptr, &scale_bs, &correction_bs);
+  if (describe_runtime_quant(a, nullptr, reinterpret_cast<const void*>(256), n, c, scale_bs, 0, reinterpret_cast<void*>(256), &d) != ST_OK)
     return 0;
   return d.q_bytes + d.row_bytes + d.plan.workspace_bytes;
 }
@@ -907,8 +1026,210 @@ int32_t vecops_hip_matmul_runtime_quant_packed_b(const VecopsHipOperand* a, cons
                                                  void* stream) {
   if (packed_b == nullptr && n > 0 && a != nullptr && a->sizes[a->rank - 1] > 0)
     return fail(ST_INVALID, "matmul_runtime_quant_packed_b: null packed b");
-  return run_runtime_quant(a, multipliers, zero_point, nullptr, packed_b ? packed_b : reinterpret_cast<const void*>(256), n,
-                           correction, row_scales, column_scales, c, workspace, workspace_size, stream);
+  int64_t scale_bs = 0, correction_bs = 0;
+  conventional_strides(a, nullptr, &scale_bs, &correction_bs);
+  return run_runtime_quant(a, multipliers, zero_point, scale_bs, nullptr, packed_b ? packed_b : reinterpret_cast<const void*>(256),
+                           n, correction, 0, row_scales, column_scales, c, workspace, workspace_size, stream);
+}
+
+}  // extern "C"
+
+namespace vecops_hip {
+// Table set-up of a grouped launch.  The records travel as kernel arguments, so no host buffer has to outlive the call.
+__global__ __launch_bounds__(64) void write_groups_kernel(const GroupChunk chunk, int32_t* __restrict__ first,
+                                                          TileGemmParams* __restrict__ groups) {
+  const int lane = threadIdx.x;
+  constexpr int kWords = sizeof(TileGemmParams) / 4;
+  for (int g = 0; g < chunk.count; ++g) {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(&chunk.params[g]);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(&groups[chunk.offset + g]);
+    for (int w = lane; w < kWords; w += 64) dst[w] = src[w];
+  }
+  if (lane <= chunk.count) first[chunk.offset + lane] = chunk.first[lane];
+}
+
+// group_of[w] = the group whose run of workgroups holds w (binary search over first[0 .. groups])
+__global__ __launch_bounds__(256) void expand_groups_kernel(const int32_t* __restrict__ first, int32_t groups,
+                                                            int32_t* __restrict__ group_of) {
+  const int total = first[groups];
+  for (int w = blockIdx.x * 256 + threadIdx.x; w < total; w += gridDim.x * 256) {
+    int lo = 0, hi = groups - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (first[mid] <= w) lo = mid;
+      else hi = mid - 1;
+    }
+    group_of[w] = lo;
+  }
+}
+}  // namespace vecops_hip
+
+namespace {
+// A grouped call: several independent products (irregular batches - every group with its own extents, strides and
+// pointers).  bf16 and int8 groups that all multiply run as ONE launch of tile_gemm_grouped_kernel over a table of
+// problem records in the workspace; other operand classes, and groups with K = 0, run as launches of their own on
+// the same stream.
+struct Grouped {
+  std::vector<Problem> problems;
+  std::vector<VecopsHipPlan> plans;
+  std::vector<int> table_groups;  // indices of the groups served by the one grouped launch
+  bool one_launch = false;
+  int src = -1, tile = 0, mode = 0;
+  std::vector<int32_t> first;     // first workgroup of each table group, and the end
+  uint64_t first_bytes = 0, record_bytes = 0, map_bytes = 0, loop_workspace = 0;
+};
+
+uint64_t round_up_256(uint64_t v) { return (v + 255u) & ~uint64_t{255}; }
+
+int32_t describe_grouped(uint32_t count, const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                         const VecopsHipOperand* c, uint32_t compute, Grouped* g) {
+  if (count > 0 && (a == nullptr || b == nullptr || c == nullptr)) return fail(ST_INVALID, "matmul_grouped: null operand array");
+  if (count > 65536) return fail(ST_INVALID, "matmul_grouped: more than 65536 groups");
+  g->problems.resize(count);
+  g->plans.resize(count);
+  bool same_class = true;
+  for (uint32_t i = 0; i < count; ++i) {
+    const VecopsHipOperand* cin = (c_in != nullptr && c_in[i].rank != 0) ? &c_in[i] : nullptr;
+    // the groups are independent problems: nothing folds across them, each may fold its own batches
+    int32_t rc = describe(&a[i], &b[i], cin, &c[i], compute, &g->problems[i]);
+    if (rc != ST_OK) return rc;
+    choose(g->problems[i], &g->plans[i]);
+    const VecopsHipPlan& plan = g->plans[i];
+    if (plan.family == VECOPS_HIP_FAMILY_NONE) continue;
+    if (plan.workspace_bytes > g->loop_workspace) g->loop_workspace = plan.workspace_bytes;
+    if (plan.family == VECOPS_HIP_FAMILY_ZERO_K) continue;
+    if (g->src < 0) g->src = g->problems[i].src;
+    else if (g->src != g->problems[i].src) same_class = false;
+    g->table_groups.push_back(static_cast<int>(i));
+  }
+  g->one_launch = same_class && (g->src == SRC_BF16 || g->src == SRC_I8) && g->table_groups.size() > 1;
+  if (!g->one_launch) return ST_OK;
+  // One workgroup tile for every group: the biggest square tile that still yields two rounds' worth of
+  // workgroups over all groups together (priced like the rule table's candidates), else 64 x 64.
+  auto tiles = [&](int64_t t) {
+    int64_t total = 0;
+    for (int i : g->table_groups) {
+      const Problem& pr = g->problems[i];
+      total += ((pr.m + t - 1) / t) * ((pr.n + t - 1) / t) * pr.batch;
+    }
+    return total;
+  };
+  g->tile = 64;
+  int64_t best = INT64_MAX;
+  const struct { int tile; int64_t quality; } candidates[] = {{256, 1000}, {128, kQuality128}};
+  for (const auto& cand : candidates) {
+    const int64_t n_tiles = tiles(cand.tile);
+    if (n_tiles < kComputeUnits / 2) continue;
+    const int64_t rounds = (n_tiles + kComputeUnits - 1) / kComputeUnits;
+    int64_t cost = rounds * cand.tile * cand.tile * 1000 / cand.quality;
+    if (rounds == 1) cost = cost * (kComputeUnits + n_tiles) / (2 * kComputeUnits);
+    if (best == INT64_MAX || cost * 11 < best * 10) {
+      best = cost;
+      g->tile = cand.tile;
+    }
+  }
+  // the weakest fetch mode any group needs serves them all
+  bool all_k = true, all_n = true, all_dma = true;
+  for (int i : g->table_groups) {
+    const int mode = fetch_mode(g->problems[i], g->plans[i]);
+    all_k = all_k && (mode == MODE_KVEC || mode == MODE_KVEC_DMA);
+    all_n = all_n && (mode == MODE_NVEC_B || mode == MODE_NVEC_B_DMA);
+    all_dma = all_dma && (mode == MODE_KVEC_DMA || mode == MODE_NVEC_B_DMA);
+  }
+  g->mode = all_k ? (all_dma ? MODE_KVEC_DMA : MODE_KVEC) : all_n ? (all_dma ? MODE_NVEC_B_DMA : MODE_NVEC_B) : MODE_GENERIC;
+  int64_t next = 0;
+  for (int i : g->table_groups) {
+    const Problem& pr = g->problems[i];
+    g->first.push_back(static_cast<int32_t>(next));
+    const int64_t wgs = ((pr.m + g->tile - 1) / g->tile) * ((pr.n + g->tile - 1) / g->tile) * pr.batch;
+    next += (wgs + 7) & ~int64_t{7};  // a multiple of eight: the XCD renumbering then works per group
+    if (next > INT32_MAX) return fail(ST_INVALID, "matmul_grouped: too many workgroups");
+  }
+  g->first.push_back(static_cast<int32_t>(next));
+  g->first_bytes = round_up_256(g->first.size() * 4u);
+  g->record_bytes = round_up_256(g->table_groups.size() * sizeof(TileGemmParams));
+  g->map_bytes = round_up_256(static_cast<uint64_t>(next) * 4u);
+  return ST_OK;
+}
+
+uint64_t grouped_workspace(const Grouped& g) {
+  const uint64_t table = g.one_launch ? g.first_bytes + g.record_bytes + g.map_bytes : 0;
+  // (the loop's scratch serves one launch at a time; with a table only the K = 0 groups loop, and they need none)
+  return g.one_launch ? table : g.loop_workspace;
+}
+}  // namespace
+
+extern "C" {
+
+uint64_t vecops_hip_matmul_grouped_workspace(uint32_t count, const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                             const VecopsHipOperand* c_in, const VecopsHipOperand* c, uint32_t compute) {
+  Grouped g;
+  if (describe_grouped(count, a, b, c_in, c, compute, &g) != ST_OK) return 0;
+  return grouped_workspace(g);
+}
+
+int32_t vecops_hip_matmul_grouped(uint32_t count, const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                  const VecopsHipOperand* c_in, const VecopsHipOperand* c, uint32_t compute, void* workspace,
+                                  uint64_t workspace_size, void* stream) {
+  Grouped g;
+  int32_t rc = describe_grouped(count, a, b, c_in, c, compute, &g);
+  if (rc != ST_OK) return rc;
+  const uint64_t need = grouped_workspace(g);
+  if (need > workspace_size || (need > 0 && (workspace == nullptr || !aligned16(workspace))))
+    return fail(ST_INVALID, "matmul_grouped: %llu bytes of 16-byte aligned workspace required, %llu supplied",
+                (unsigned long long)need, (unsigned long long)workspace_size);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (!g.one_launch) {
+    for (uint32_t i = 0; i < count; ++i) {
+      rc = run_problem(g.problems[i], g.plans[i], nullptr, nullptr, nullptr, workspace, workspace_size, s);
+      if (rc != ST_OK) return rc;
+    }
+    return ST_OK;
+  }
+  if (int32_t device_rc = check_device(); device_rc != ST_OK) return device_rc;
+  // K = 0 groups: c = c_in (or zero), a launch each
+  for (uint32_t i = 0; i < count; ++i) {
+    if (g.plans[i].family != VECOPS_HIP_FAMILY_ZERO_K) continue;
+    rc = run_problem(g.problems[i], g.plans[i], nullptr, nullptr, nullptr, nullptr, 0, s);
+    if (rc != ST_OK) return rc;
+  }
+  char* base = static_cast<char*>(workspace);
+  int32_t* first = reinterpret_cast<int32_t*>(base);
+  TileGemmParams* records = reinterpret_cast<TileGemmParams*>(base + g.first_bytes);
+  int32_t* group_of = reinterpret_cast<int32_t*>(base + g.first_bytes + g.record_bytes);
+  const int groups = static_cast<int>(g.table_groups.size());
+  const int ktile = k_tile_elements(g.src);
+  for (int offset = 0; offset < groups; offset += kGroupChunk) {
+    GroupChunk chunk;
+    memset(&chunk, 0, sizeof(chunk));
+    chunk.offset = offset;
+    chunk.count = groups - offset < kGroupChunk ? groups - offset : kGroupChunk;
+    for (int j = 0; j < chunk.count; ++j) {
+      const Problem& pr = g.problems[g.table_groups[offset + j]];
+      if (pr.a.data == nullptr || pr.b.data == nullptr || pr.c.data == nullptr)
+        return fail(ST_INVALID, "matmul_grouped: group %d has an operand without storage", g.table_groups[offset + j]);
+      TileGemmParams& p = chunk.params[j];
+      p = base_params(pr, nullptr, nullptr, nullptr, nullptr);
+      p.tiles_m = static_cast<int32_t>((pr.m + g.tile - 1) / g.tile);
+      p.tiles_n = static_cast<int32_t>((pr.n + g.tile - 1) / g.tile);
+      p.split_k = 1;
+      p.k_tiles_per_split = static_cast<int32_t>((pr.k + ktile - 1) / ktile);
+    }
+    for (int j = 0; j <= chunk.count; ++j) chunk.first[j] = g.first[offset + j];
+    hipLaunchKernelGGL(write_groups_kernel, dim3(1), dim3(64), 0, s, chunk, first, records);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(ST_EXEC, "group table launch: %s", hipGetErrorString(e));
+  }
+  const int32_t workgroups = g.first.back();
+  int blocks = (workgroups + 255) / 256;
+  if (blocks > 1024) blocks = 1024;
+  hipLaunchKernelGGL(expand_groups_kernel, dim3(blocks), dim3(256), 0, s, first, groups, group_of);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(ST_EXEC, "group map launch: %s", hipGetErrorString(e));
+  GroupedTables t{group_of, first, records, workgroups};
+  e = g.src == SRC_BF16 ? launch_tile_gemm_grouped_bf16(t, g.tile, g.mode, s) : launch_tile_gemm_grouped_i8(t, g.tile, g.mode, s);
+  if (e != hipSuccess) return fail(ST_EXEC, "grouped tile kernel launch: %s", hipGetErrorString(e));
+  return ST_OK;
 }
 
 uint32_t vecops_hip_abi_version(void) { return VECOPS_HIP_ABI_VERSION; }

@@ -68,9 +68,10 @@ struct TileGemmParams {
   const void* cin;  // null = zero accumulator
   void* c;
   void* partial;    // split-K partial sums [split][batch][M][N] in accumulator type
-  const float* row_scales;     // int8 dequant epilogue (null = none)
+  const float* row_scales;     // int8 dequant epilogue (null = none); batch b reads row_scales[b * row_scales_bs + row]
   const float* column_scales;
-  const int32_t* correction;   // int32 row added to every accumulator row (null = none)
+  const int32_t* correction;   // int32 row added to every accumulator row (null = none): correction[b * correction_bs + col]
+  int64_t row_scales_bs, correction_bs;  // 0 = one set for every batch
   // unsigned-operand terms (SRC_I8_FLIP; null / zero = none), added to the accumulator first
   const int32_t* row_term;     // [batch][M]
   const int32_t* col_term;     // [batch][N]
@@ -412,13 +413,13 @@ __device__ __forceinline__ uint32_t output_bits(const TileGemmParams& p, int bat
     uint32_t v = static_cast<uint32_t>(acc) + p.const_term;
     if (p.row_term) v += static_cast<uint32_t>(p.row_term[static_cast<int64_t>(batch) * p.m + row]);
     if (p.col_term) v += static_cast<uint32_t>(p.col_term[static_cast<int64_t>(batch) * p.n + col]);
-    if (p.correction) v += static_cast<uint32_t>(p.correction[col]);
+    if (p.correction) v += static_cast<uint32_t>(p.correction[batch * p.correction_bs + col]);
     if (p.cin) v += static_cast<uint32_t>(
                  static_cast<const int32_t*>(p.cin)[batch * p.cin_bs + row * p.cin_rs + col * p.cin_cs]);
     const int32_t s = static_cast<int32_t>(v);
     float f = static_cast<float>(s);
     if (p.row_scales) {
-      const float t = f * p.row_scales[row];
+      const float t = f * p.row_scales[batch * p.row_scales_bs + row];
       f = t * p.column_scales[col];
     } else if (p.out_kind == OUT_I32) {
       return v;
@@ -629,9 +630,9 @@ __device__ __forceinline__ void store_quad_general(const TileGemmParams& p, int 
 // eight XCDs round-robin, each XCD with its own L2: renumber so that an XCD
 // receives a contiguous run of tiles, then walk tiles in bands of 8 tile rows so
 // that a run shares A rows and B columns.
-__device__ __forceinline__ void map_workgroup(const TileGemmParams& p, int& batch, int& split, int& tm, int& tn) {
-  int pid = blockIdx.x;
-  const int total = gridDim.x;
+// `pid` of `total`: the workgroup's number within its launch (or within its group's run of a grouped launch).
+__device__ __forceinline__ void map_workgroup(const TileGemmParams& p, int pid, int total, int& batch, int& split, int& tm,
+                                              int& tn) {
   if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
   const int tiles = p.tiles_m * p.tiles_n;
   const int tile = pid % tiles;
@@ -1386,7 +1387,7 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
     float rs[WM];
     static_for<WM>([&](auto ci) {
       const int row = m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row;
-      rs[decltype(ci)::value] = (dequant && row < p.m) ? p.row_scales[row] : 1.0f;
+      rs[decltype(ci)::value] = (dequant && row < p.m) ? p.row_scales[batch * p.row_scales_bs + row] : 1.0f;
     });
     uint32_t* out = reinterpret_cast<uint32_t*>(c_base) + batch * p.c_bs + static_cast<int64_t>(m0 + wm * ROWS) * p.c_rs;
     const int out_bytes = output_element_bytes(p.out_kind);
@@ -1403,13 +1404,13 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
         corr[q] = i32x4{0, 0, 0, 0};
         if (col0 + 3 < p.n) {
           if (dequant) cs[q] = *reinterpret_cast<const f32x4*>(p.column_scales + col0);
-          if (INT && p.correction) corr[q] = *reinterpret_cast<const i32x4*>(p.correction + col0);
+          if (INT && p.correction) corr[q] = *reinterpret_cast<const i32x4*>(p.correction + batch * p.correction_bs + col0);
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             if (col0 + e < p.n) {
               if (dequant) cs[q][e] = p.column_scales[col0 + e];
-              if (INT && p.correction) corr[q][e] = p.correction[col0 + e];
+              if (INT && p.correction) corr[q][e] = p.correction[batch * p.correction_bs + col0 + e];
             }
           }
         }
@@ -1541,8 +1542,10 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
 // tiles of 32x32.  Every shape in use runs 4 wavefronts, one per SIMD: the 256x256
 // tile with 128x128 per wavefront (256 accumulator registers in the AGPR half of
 // the unified file), the small tiles with 64x64 or 32x32.
+//
+// The work of one workgroup: number `pid` of the `total` that serve the problem `p`.
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const TileGemmParams p) {
+__device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int pid, int total) {
   using T = SrcTraits<SRC>;
   constexpr bool INT = T::kInt;
   using Acc = typename AccTile<INT>::type;
@@ -1560,10 +1563,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
   int batch, split, tm, tn;
-  map_workgroup(p, batch, split, tm, tn);
+  map_workgroup(p, pid, total, batch, split, tm, tn);
   // workgroup-uniform by construction; say so, or every loop bound derived from
   // them is treated as divergent
   batch = __builtin_amdgcn_readfirstlane(batch);
+  if (batch >= p.batch) return;  // a grouped launch rounds each group's run of workgroups up to a multiple of eight
   split = __builtin_amdgcn_readfirstlane(split);
   tm = __builtin_amdgcn_readfirstlane(tm);
   tn = __builtin_amdgcn_readfirstlane(tn);
@@ -1803,6 +1807,36 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
   store_accumulators<SRC, WAVES_M, WAVES_N, WM, WN, kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>()>(
       p, lds, acc, batch, split, m0, n0, wm, wn, wave, lane);
 }
+
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const TileGemmParams p) {
+  tile_gemm_workgroup<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_A, LOAD_B>(p, blockIdx.x, gridDim.x);
+}
+
+// Several independent problems in one launch (irregular batches: every group has its own extents, strides and
+// pointers; all share the operand class, the workgroup tile and the loaders).  Workgroups first[g] .. first[g + 1] - 1
+// serve group g (each run a multiple of eight long, so that a group's workgroups are dealt to the XCDs like a
+// launch of its own); group_of[w] names the group of workgroup w.  No group splits K.
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_grouped_kernel(
+    const int32_t* __restrict__ group_of, const int32_t* __restrict__ first, const TileGemmParams* __restrict__ groups) {
+  const int g = __builtin_amdgcn_readfirstlane(group_of[blockIdx.x]);
+  const TileGemmParams p = groups[g];
+  const int begin = __builtin_amdgcn_readfirstlane(first[g]);
+  const int end = __builtin_amdgcn_readfirstlane(first[g + 1]);
+  tile_gemm_workgroup<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_A, LOAD_B>(p, static_cast<int>(blockIdx.x) - begin, end - begin);
+}
+
+// Table set-up of a grouped launch is fed through kernel arguments, so that no host buffer has to outlive the
+// call: one chunk carries up to kGroupChunk problem records and their first workgroups.
+constexpr int kGroupChunk = 12;
+struct GroupChunk {
+  TileGemmParams params[kGroupChunk];
+  int32_t first[kGroupChunk + 1];  // first[count] = end of the last group of this chunk
+  int32_t count, offset;           // groups in this chunk, index of its first group
+};
+static_assert(sizeof(GroupChunk) <= 4096, "a chunk travels as kernel arguments");
+static_assert(sizeof(TileGemmParams) % 8 == 0, "records are copied word by word and stored back to back");
 
 // Sums the split-K partials and applies the same epilogue as the tile kernel.
 template <bool INT>

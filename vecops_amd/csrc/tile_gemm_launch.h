@@ -5,6 +5,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "tile_gemm.h"
 
 namespace vecops_hip {
@@ -27,15 +29,16 @@ hipError_t launch_tile_gemm_f32(const TileGemmParams& p, int tile_m, int tile_n,
 hipError_t launch_tile_gemm_i8(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
 // 8-bit operands of which at least one is unsigned (p.a_flip / p.b_flip and the epilogue terms set)
 hipError_t launch_tile_gemm_i8_flip(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
-// out[b][r] = scale * sum_k int8(x[b][r][k] xor flip) (+ add[r], may be null): the epilogue terms of an unsigned operand
+// out[b][r] = scale * sum_k int8(x[b][r][k] xor flip) (+ add[b * add_bs + r], add may be null): the epilogue terms of an
+// unsigned operand
 hipError_t launch_byte_row_sums(const void* x, int32_t batch, int32_t rows, int32_t k, int64_t bs, int64_t rs,
-                                int64_t ks, uint32_t flip, uint32_t scale, const int32_t* add, int32_t* out,
+                                int64_t ks, uint32_t flip, uint32_t scale, const int32_t* add, int64_t add_bs, int32_t* out,
                                 hipStream_t stream);
-// q = u8(x * multipliers[row] + zero_point) xor flip: the per-row asymmetric quantisation of fp32 activations
-// (flip 0x80 stores the byte as the int8 q - 128)
+// q = u8(x * multipliers[batch * mult_bs + row] + zero_point) xor flip: the per-row asymmetric quantisation of fp32
+// activations (flip 0x80 stores the byte as the int8 q - 128)
 hipError_t launch_quantize_rows(const float* x, int32_t batch, int32_t rows, int32_t k, int64_t xbs, int64_t xrs,
-                                int64_t xks, const float* multipliers, int32_t zero_point, uint32_t flip, uint8_t* q,
-                                int64_t qbs, int64_t qrs, int64_t qks, hipStream_t stream);
+                                int64_t xks, const float* multipliers, int64_t mult_bs, int32_t zero_point, uint32_t flip,
+                                uint8_t* q, int64_t qbs, int64_t qrs, int64_t qks, hipStream_t stream);
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
 // B prepacked by launch_pack_b (src: SRC_BF16, SRC_F32_AS_BF16 = fp32 A against bf16-packed B, SRC_I8,
 // SRC_I8_FLIP = unsigned A against int8-packed B with p.a_flip and p.col_term set);
@@ -70,27 +73,34 @@ hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN>
-hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t stream) {
+// Calls f(load of A, load of B) with the loader pair of a fetch mode, as integral constants.
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, typename F>
+hipError_t with_loaders(int mode, F&& f) {
+  auto pair = [&](auto la, auto lb) { return f(la, lb); };
+  using std::integral_constant;
   // loads into LDS: bf16 and int8 operands on the tiles of 128 or more columns
   if constexpr ((SRC == SRC_BF16 || SRC == SRC_F16 || SRC == SRC_I8) && WAVES_N * WN * 32 >= 128) {
-    if (mode == MODE_KVEC_DMA) return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KDMA, LOAD_KDMA>(p, stream);
+    if (mode == MODE_KVEC_DMA) return pair(integral_constant<int, LOAD_KDMA>{}, integral_constant<int, LOAD_KDMA>{});
     if constexpr (SRC == SRC_BF16 || SRC == SRC_F16) {
-      if (mode == MODE_NVEC_B_DMA)
-        return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KDMA, LOAD_NTR_DMA>(p, stream);
+      if (mode == MODE_NVEC_B_DMA) return pair(integral_constant<int, LOAD_KDMA>{}, integral_constant<int, LOAD_NTR_DMA>{});
     }
   }
   if (mode == MODE_KVEC_DMA) mode = MODE_KVEC;
   if (mode == MODE_NVEC_B_DMA) mode = MODE_NVEC_B;
-  if (mode == MODE_KVEC) return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_KVEC>(p, stream);
+  if (mode == MODE_KVEC) return pair(integral_constant<int, LOAD_KVEC>{}, integral_constant<int, LOAD_KVEC>{});
   if constexpr (SrcTraits<SRC>::kElemsPerChunk == 8) {  // 16-bit compute: B untransposed in LDS, transposing reads
-    if (mode == MODE_NVEC_B)
-      return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_NTR>(p, stream);
+    if (mode == MODE_NVEC_B) return pair(integral_constant<int, LOAD_KVEC>{}, integral_constant<int, LOAD_NTR>{});
   } else if constexpr (SRC == SRC_F32) {                // 32-bit compute: transposed in registers
-    if (mode == MODE_NVEC_B)
-      return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_KVEC, LOAD_NVEC>(p, stream);
+    if (mode == MODE_NVEC_B) return pair(integral_constant<int, LOAD_KVEC>{}, integral_constant<int, LOAD_NVEC>{});
   }
-  return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_GENERIC, LOAD_GENERIC>(p, stream);
+  return pair(integral_constant<int, LOAD_GENERIC>{}, integral_constant<int, LOAD_GENERIC>{});
+}
+
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN>
+hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t stream) {
+  return with_loaders<SRC, WAVES_M, WAVES_N, WM, WN>(mode, [&](auto la, auto lb) {
+    return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, decltype(la)::value, decltype(lb)::value>(p, stream);
+  });
 }
 
 template <int SRC>
@@ -104,6 +114,50 @@ hipError_t launch_tile_class(const TileGemmParams& p, int tile_m, int tile_n, in
   if (tile_m == 128 && tile_n == 128) return launch_tile_mode<SRC, 2, 2, 2, 2>(p, mode, stream);
   return launch_tile_mode<SRC, 2, 2, 1, 1>(p, mode, stream);
 }
+
+// A grouped launch: the device tables written by launch_group_tables, `workgroups` = first[groups].
+struct GroupedTables {
+  const int32_t* group_of;
+  const int32_t* first;
+  const TileGemmParams* groups;
+  int32_t workgroups;
+};
+
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB>
+hipError_t launch_grouped_instance(const GroupedTables& t, hipStream_t stream) {
+  constexpr int kLds = kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LB>();
+  constexpr int kThreads = 64 * WAVES_M * WAVES_N;
+  auto kernel = tile_gemm_grouped_kernel<SRC, WAVES_M, WAVES_N, WM, WN, LA, LB>;
+  static thread_local int configured_device = -1;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  if (configured_device != device) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return e;
+    configured_device = device;
+  }
+  if (t.workgroups <= 0) return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(t.workgroups)), dim3(kThreads), kLds, stream, t.group_of, t.first,
+                     t.groups);
+  return hipGetLastError();
+}
+
+// Square tiles of 256, 128 or 64.
+template <int SRC>
+hipError_t launch_grouped_class(const GroupedTables& t, int tile, int mode, hipStream_t stream) {
+  auto go = [&](auto wm_tag) {
+    constexpr int W = decltype(wm_tag)::value;
+    return with_loaders<SRC, 2, 2, W, W>(mode, [&](auto la, auto lb) {
+      return launch_grouped_instance<SRC, 2, 2, W, W, decltype(la)::value, decltype(lb)::value>(t, stream);
+    });
+  };
+  if (tile == 256) return go(std::integral_constant<int, 4>{});
+  if (tile == 128) return go(std::integral_constant<int, 2>{});
+  return go(std::integral_constant<int, 1>{});
+}
+hipError_t launch_tile_gemm_grouped_bf16(const GroupedTables& t, int tile, int mode, hipStream_t stream);
+hipError_t launch_tile_gemm_grouped_i8(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 
 }  // namespace vecops_hip
 #endif

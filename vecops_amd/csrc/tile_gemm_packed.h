@@ -101,7 +101,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
   int batch, split, tm, tn;
-  map_workgroup(p, batch, split, tm, tn);
+  map_workgroup(p, blockIdx.x, gridDim.x, batch, split, tm, tn);
   batch = __builtin_amdgcn_readfirstlane(batch);
   split = __builtin_amdgcn_readfirstlane(split);
   tm = __builtin_amdgcn_readfirstlane(tm);
