@@ -218,6 +218,38 @@ def bench_batched(dev, steps, warmup, m, n, k):
             "unit": "TFLOP/s", "hbm_gbps": gbps, "us_per_step": t["wall_ms"] * 1e3, "dtype": "bf16", "roofline": roof}
 
 
+GROUPED_SHAPES = [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17), (1300, 700, 520), (64, 5000, 1030),
+                  (2000, 2000, 264), (500, 300, 4100)]
+
+
+def bench_grouped(dev, steps, warmup):
+    """Irregular batches: eight bf16 products of unlike shapes (BASELINE configs[2]'s four among them, unbatched) as one
+    vecops_hip_matmul_grouped call, and the same eight as separate vecops_hip_matmul calls."""
+    import numpy as np
+    import torch
+    from vecops_amd import capi, synth
+    a_list, b_list, c_list = [], [], []
+    for i, (m, n, k) in enumerate(GROUPED_SHAPES):
+        a_list.append(torch.from_numpy(synth.bf16_round(synth.uniform_pm1(10 + i, (m, k))).view(np.int16)).to(dev).view(torch.bfloat16))
+        b_list.append(torch.from_numpy(synth.bf16_round(synth.uniform_pm1(40 + i, (n, k))).view(np.int16)).to(dev).view(torch.bfloat16))
+        c_list.append(torch.empty((m, n), dtype=torch.float32, device=dev))
+    ws = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    grouped = _measure(lambda i: capi.matmul_grouped(a_list, b_list, c_list, workspace=ws), max(steps, 50), warmup)
+
+    def one_by_one(i):
+        for a, b, c in zip(a_list, b_list, c_list):
+            capi.matmul(a, b, c, workspace=ws)
+    looped = _measure(one_by_one, max(steps, 50), warmup)
+    flops = sum(2.0 * m * n * k for m, n, k in GROUPED_SHAPES)
+    tflops = flops / (grouped["event_ms"] * 1e-3) / 1e12
+    roof = _roofline("mfma", tflops, PEAK_BF16_TFLOPS, "TFLOP/s", kernel="vecops_hip tile_gemm_grouped_kernel<bf16>",
+                     algorithmic_flops_per_launch=flops, traffic=None, **_timing_fields(grouped))
+    return {"metric": "bf16_grouped_irregular_tflops", "workload": "eight bf16 products of unlike shapes "
+            f"{GROUPED_SHAPES}, fp32 out, one vecops_hip_matmul_grouped call", "value": tflops, "unit": "TFLOP/s",
+            "us_per_step": grouped["wall_ms"] * 1e3, "separate_calls_event_us": looped["event_ms"] * 1e3,
+            "separate_calls_wall_us": looped["wall_ms"] * 1e3, "dtype": "bf16", "roofline": roof}
+
+
 def bench_int8_dequant(dev, steps, warmup, ceiling=None):
     import torch
     from vecops_amd import capi, synth
@@ -443,7 +475,7 @@ def cpu_baseline(a, b_kn):
 
 
 ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "fp32", "batched",
-        "families"]
+        "families", "grouped"]
 
 
 def main() -> int:
@@ -484,6 +516,7 @@ def main() -> int:
         "fp32": lambda: bench_fp32_gemm(dev, K, W, args.fp32_compute),
         "batched": lambda: bench_batched(dev, K, W, *[int(v) for v in args.batched_shape.split(",")]),
         "families": lambda: bench_tile_families(dev, K, W),
+        "grouped": lambda: bench_grouped(dev, K, W),
     }
     if args.only in single:
         print(json.dumps(single[args.only]()))

@@ -360,13 +360,20 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t l
  * rows past N and k past K are zero.
  *
  * packed dtypes: 11 bf16 (from a bf16 or f32 source; f32 is rounded to nearest
- * even, as the matmul itself rounds it), 10 f16 and 2 i8.
+ * even, as the matmul itself rounds it), 10 f16, 2 i8 and 3 u8.  An unsigned operand is stored as the signed
+ * b - 128 (its bytes xor 0x80, padding still zero), so that the product runs on the signed matrix-core instruction and
+ * adds 128 * sum_k a[m,k] back in its epilogue: AMX_I8I32<int8_t, uint8_t> and <uint8_t, uint8_t> with a packed B
+ * (tests/ops/MatmulMixedPackingTest.cpp:137-153).
+ *
+ * The [M,K] operand packs into the same 32-row panels (vecops_hip_pack_a; vecops keeps a format per side,
+ * ops/MatmulPack.h:63-65 - here one format serves both, but a packed operand still has to be passed as the side it was
+ * packed for).
  */
 
 /* Bytes of the packed form of a [N,K] operand; 0 for an unsupported dtype. */
 VECOPS_HIP_EXPORT uint64_t vecops_hip_packed_b_bytes(uint32_t packed_dtype, int64_t n, int64_t k);
 
-/* Packs b (rank 2, [N,K], any strides; bf16, f32 or i8) into `packed`
+/* Packs b (rank 2, [N,K], any strides; bf16, f16, f32, i8 or u8) into `packed`
  * (16-byte aligned, at least vecops_hip_packed_b_bytes).  Replaces
  * ops::MatmulPack<MatmulPackConfig<Atom, Operand::B>>::operator()
  * (ops/MatmulPack.h:132-190). */
@@ -392,6 +399,7 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul_packed_b(const VecopsHipOperand
  *   packed f16 : a f16, c f32|f16
  *   packed i8  : a i8 or u8 (AMX_I8I32<uint8_t, int8_t>, the atom the compensated pack serves,
  *                ops/MatmulPack.h:52-58; the workspace then also holds 4 * batch * (M + N) bytes), c i32
+ *   packed u8  : a i8 or u8, c i32 (the same workspace term)
  * Same results, bit for bit, as vecops_hip_matmul on the unpacked operand when
  * that runs its tile kernels.
  */
@@ -399,6 +407,39 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_packed_b(const VecopsHipOperand* a, 
                                                      uint32_t packed_dtype, int64_t n, const VecopsHipOperand* c_in,
                                                      const VecopsHipOperand* c, void* workspace,
                                                      uint64_t workspace_size, void* stream);
+
+/*
+ * Side A: ops::MatmulPack<MatmulPackConfig<Atom, Operand::A>> (ops/MatmulPack.h:81-96,132-190) and the product with a
+ * packed A (tests/ops/MatmulMixedPackingTest.cpp:24-28).  C = C_in + A . B^T with A[M,K] prepacked runs as
+ * C^T = C_in^T + B . A^T on the packed-operand kernels: b is then the operand that travels through LDS and the
+ * packed a the one fetched straight into registers; c and c_in are written and read through their transposed views
+ * (any strides are legal, the stores of a row-major c are element-wise).  Same sums in the same order as the plain
+ * product.  b rank 2 or 3 (the one packed a serves every batch), dtypes as for vecops_hip_matmul_packed_b with the
+ * sides exchanged.
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_pack_a(const VecopsHipOperand* a, void* packed, uint64_t packed_size, void* stream);
+VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul_packed_a(uint32_t packed_dtype, int64_t m, const VecopsHipOperand* b,
+                                                          const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                          VecopsHipPlan* plan);
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_packed_a(const void* packed_a, uint32_t packed_dtype, int64_t m,
+                                                     const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                                                     const VecopsHipOperand* c, void* workspace, uint64_t workspace_size,
+                                                     void* stream);
+
+/*
+ * Both operands packed (tests/ops/MatmulMixedPackingTest.cpp:31-108, check_both_packed): c[M,N] = c_in + A . B^T with
+ * A packed by vecops_hip_pack_a ([M,K], a_dtype) and B by vecops_hip_pack_b ([N,K], b_dtype).  The matrix cores take one
+ * operand from registers and one through LDS, so A is first written back to a dense [M,K] matrix at the front of the
+ * workspace (a permutation) and then multiplied with the packed B.  c rank 2.  workspace:
+ * vecops_hip_matmul_packed_ab_workspace bytes, 16-byte aligned.
+ */
+VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_packed_ab_workspace(uint32_t a_dtype, int64_t m, uint32_t b_dtype, int64_t n,
+                                                                 int64_t k, const VecopsHipOperand* c_in,
+                                                                 const VecopsHipOperand* c);
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_packed_ab(const void* packed_a, uint32_t a_dtype, int64_t m, const void* packed_b,
+                                                      uint32_t b_dtype, int64_t n, int64_t k, const VecopsHipOperand* c_in,
+                                                      const VecopsHipOperand* c, void* workspace, uint64_t workspace_size,
+                                                      void* stream);
 
 /* vecops_hip_matmul_i8_dequant with b prepacked (i8); workspace as for the
  * plain call with the same extents. */

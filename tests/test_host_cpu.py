@@ -113,7 +113,7 @@ def test_host_library_exports_every_declared_symbol(host):
 
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
-    assert len(files) == 60   # 36 + (6 required families x {bf16, i8} x {host, device})
+    assert len(files) == 64   # 40 + (6 required families x {bf16, i8} x {host, device})
     for f in files:
         name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
         assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
@@ -285,8 +285,10 @@ def test_packed_b_operators_resolution_and_validation(host):
         with pytest.raises(H.HostError) as e:
             pack.resolve(fr)
         assert e.value.code == 1 and needle in e.value.message, (needle, e.value.message)
-    with pytest.raises(H.HostError) as e:                  # half operands have no packed form
-        pack.resolve(pf(np.zeros((5, 8), np.float16), 0, packed, None))
+    assert pack.resolve(pf(np.zeros((5, 8), np.float16), 0, packed, None)) == \
+        "vecops::matmul_pack_b;operands=f16;memory=host;backend=hip-gfx950"        # half operands: a recipe of their own
+    with pytest.raises(H.HostError) as e:                  # unsigned weights have no recipe in the host layer
+        pack.resolve(pf(np.zeros((5, 8), np.uint8), 0, packed, None))
     assert e.value.code in (1, 2, 3)
 
     mul = host.operator("vecops::matmul_packed_b")
@@ -297,6 +299,10 @@ def test_packed_b_operators_resolution_and_validation(host):
     assert "operands=f32" in mul.resolve(mf(np.zeros((4, 8), np.float32), c, c))
     assert "operands=i8" in mul.resolve(mf(np.zeros((4, 8), np.int8), None, np.zeros((4, 5), np.int32)))
     assert "operands=i8" in mul.resolve(mf(np.zeros((4, 8), np.uint8), None, np.zeros((4, 5), np.int32)))   # u8 x packed s8
+    assert "operands=f16" in mul.resolve(mf(np.zeros((4, 8), np.float16), None, np.zeros((4, 5), np.float16)))
+    with pytest.raises(H.HostError) as e:                  # half operands write fp32 or half, not bf16
+        mul.resolve(mf(np.zeros((4, 8), np.float16), None, bf16((4, 5))))
+    assert e.value.code in (2, 3)
     for fr, needle in [(mf(bf16((4, 8)), None, np.zeros((3, 5), np.float32)), "[.., M, N]"),
                        (mf(bf16((2, 4, 8)), None, np.zeros((3, 4, 5), np.float32)), "batch"),
                        (mf(bf16((4, 8)), np.zeros((4, 6), np.float32), c), "c_in")]:

@@ -304,6 +304,30 @@ def test_packed_b_operators(host, oracle, device):
     with pytest.raises(H.HostError) as e:
         mul.invoke(H.Frame([ta, tp[:64], None, tc], outputs=(3,)))
     assert e.value.code == 1
+    # half operands (AMX_F16F32): their own recipes and artifacts, f32 and f16 outputs, host and device tensors
+    m, n, k = 70, 130, 264
+    ah, bh = synth.uniform_pm1(5, (m, k)).astype(np.float16), synth.uniform_pm1(6, (n, k)).astype(np.float16)
+    wanth = ah.astype(np.float64) @ bh.astype(np.float64).T
+    packed = np.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.F16, n, k), np.uint8)
+    frame = H.Frame([bh, 0, packed, None], outputs=(2,))
+    assert pack.resolve(frame) == "vecops::matmul_pack_b;operands=f16;memory=host;backend=hip-gfx950"
+    pack.invoke(frame)
+    ch = np.full((m, n), np.nan, np.float32)
+    frame = H.Frame([ah, packed, None, ch], outputs=(3,))
+    assert mul.resolve(frame) == "vecops::matmul_packed_b;operands=f16;memory=host;backend=hip-gfx950"
+    mul.invoke(frame)
+    assert rel_err(ch, wanth) <= fp32_tol(k)
+    th, tph = torch.from_numpy(ah).to(device), torch.from_numpy(packed).to(device)
+    tch = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+    frame = H.Frame([th, tph, None, tch], outputs=(3,))
+    assert mul.resolve(frame) == "vecops::matmul_packed_b;operands=f16;memory=device;backend=hip-gfx950"
+    need = mul.workspace(frame)
+    wsh = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    mul.invoke(frame, workspace=wsh.data_ptr(), workspace_size=need)
+    torch.cuda.synchronize()
+    assert np.array_equal(tch.cpu().numpy().view(np.uint16), ch.astype(np.float16).view(np.uint16))   # RNE of the fp32 result
+    with pytest.raises(H.HostError):                                         # a bf16 output does not go with half operands
+        mul.invoke(H.Frame([th, tph, None, torch.empty((m, n), dtype=torch.bfloat16, device=device)], outputs=(3,)))
 
 
 def test_matmul_runtime_quant_operator(host, device):

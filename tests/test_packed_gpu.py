@@ -284,5 +284,6 @@ def test_packed_zero_extents_and_rejections(device):
     import ctypes as C
     rc = capi.lib().vecops_hip_pack_b(C.byref(ob), packed.storage.data_ptr(), 16, None)
     assert rc == 1
-    with pytest.raises(capi.VecopsHipError):               # unsigned bytes have no packed form
-        capi.pack_b(torch.zeros((4, 8), dtype=torch.uint8, device=device))
+    with pytest.raises(capi.VecopsHipError) as err:        # 32-bit integers have no packed form
+        capi.pack_b(torch.zeros((4, 8), dtype=torch.int32, device=device))
+    assert err.value.code == 2

@@ -32,6 +32,8 @@ EXPORTS = [
     "vecops_hip_plan_matmul_family", "vecops_hip_matmul_family",
     "vecops_hip_matmul_runtime_quant_batched_workspace", "vecops_hip_matmul_runtime_quant_batched",
     "vecops_hip_matmul_grouped_workspace", "vecops_hip_matmul_grouped",
+    "vecops_hip_pack_a", "vecops_hip_plan_matmul_packed_a", "vecops_hip_matmul_packed_a",
+    "vecops_hip_matmul_packed_ab_workspace", "vecops_hip_matmul_packed_ab",
 ]
 
 ACT_NONE, ACT_RELU, ACT_CLAMP, ACT_SIGMOID, ACT_SILU = 0, 1, 2, 3, 4
@@ -138,6 +140,14 @@ def lib() -> C.CDLL:
         L.vecops_hip_matmul_runtime_quant_batched_workspace.argtypes = [P, C.c_int64, P, C.c_int64, P]
         L.vecops_hip_matmul_runtime_quant_batched.argtypes = [P, C.c_void_p, C.c_int32, C.c_int64, P, C.c_void_p, C.c_int64,
                                                               C.c_void_p, C.c_void_p, P, C.c_void_p, C.c_uint64, C.c_void_p]
+        L.vecops_hip_pack_a.argtypes = [P, C.c_void_p, C.c_uint64, C.c_void_p]
+        L.vecops_hip_plan_matmul_packed_a.argtypes = [C.c_uint32, C.c_int64, P, P, P, C.POINTER(Plan)]
+        L.vecops_hip_matmul_packed_a.argtypes = [C.c_void_p, C.c_uint32, C.c_int64, P, P, P, C.c_void_p, C.c_uint64,
+                                                 C.c_void_p]
+        L.vecops_hip_matmul_packed_ab_workspace.restype = C.c_uint64
+        L.vecops_hip_matmul_packed_ab_workspace.argtypes = [C.c_uint32, C.c_int64, C.c_uint32, C.c_int64, C.c_int64, P, P]
+        L.vecops_hip_matmul_packed_ab.argtypes = [C.c_void_p, C.c_uint32, C.c_int64, C.c_void_p, C.c_uint32, C.c_int64,
+                                                  C.c_int64, P, P, C.c_void_p, C.c_uint64, C.c_void_p]
         L.vecops_hip_matmul_grouped_workspace.restype = C.c_uint64
         L.vecops_hip_matmul_grouped_workspace.argtypes = [C.c_uint32, P, P, P, P, C.c_uint32]
         L.vecops_hip_matmul_grouped.argtypes = [C.c_uint32, P, P, P, P, C.c_uint32, C.c_void_p, C.c_uint64, C.c_void_p]
@@ -401,9 +411,9 @@ def matmul_w8a16_group(x, w, scales, y, group: int, stream=None):
 
 
 class PackedB:
-    """A [N,K] operand in the packed layout of ``vecops_hip_pack_b``: ``storage`` (uint8 tensor),
-    ``dtype`` (BF16 or I8), ``n`` and ``k`` - the counterpart of a tensor over
-    ``matmul::packed_layout<Atom, Operand::B>``."""
+    """A [N,K] operand (or, from ``pack_a``, an [M,K] one: ``n`` then counts its rows) in the packed layout of
+    ``vecops_hip_pack_b``: ``storage`` (uint8 tensor), ``dtype`` (BF16, F16, I8 or U8), ``n`` and ``k`` - the counterpart
+    of a tensor over ``matmul::packed_layout<Atom, Operand::B>``."""
 
     def __init__(self, storage, dtype: int, n: int, k: int) -> None:
         self.storage, self.dtype, self.n, self.k = storage, dtype, n, k
@@ -417,7 +427,7 @@ def pack_b(b, a_zero_point=None, stream=None):
     """
     import torch
     n, k = b.shape
-    dtype = I8 if b.dtype == torch.int8 else F16 if b.dtype == torch.float16 else BF16
+    dtype = I8 if b.dtype == torch.int8 else U8 if b.dtype == torch.uint8 else F16 if b.dtype == torch.float16 else BF16
     size = lib().vecops_hip_packed_b_bytes(dtype, n, k)
     storage = torch.empty(max(size, 16), dtype=torch.uint8, device=b.device)
     ob = operand(b)
@@ -428,6 +438,48 @@ def pack_b(b, a_zero_point=None, stream=None):
     _check(lib().vecops_hip_pack_b_compensated(C.byref(ob), a_zero_point, storage.data_ptr(), size, comp.data_ptr(),
                                                _stream_handle(stream)))
     return PackedB(storage, dtype, n, k), comp
+
+
+def pack_a(a, stream=None) -> PackedB:
+    """Pack a ([M,K]) for ``matmul_packed_a`` / ``matmul_packed_ab`` (``ops::matmul_pack`` with ``Operand::A``)."""
+    return pack_b(a, stream=stream)
+
+
+def matmul_packed_a(packed: PackedB, b, c, c_in=None, workspace=None, stream=None):
+    """c[..,M,N] = c_in + A . b[..,N,K]^T with A packed by ``pack_a``; returns c."""
+    import torch
+    plan = Plan()
+    ob, oc = operand(b), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    oi_ref = C.byref(oi) if oi is not None else None
+    _check(lib().vecops_hip_plan_matmul_packed_a(packed.dtype, packed.n, C.byref(ob), oi_ref, C.byref(oc), C.byref(plan)))
+    if plan.workspace_bytes and (workspace is None or workspace.numel() * workspace.element_size() < plan.workspace_bytes):
+        workspace = torch.empty(plan.workspace_bytes, dtype=torch.uint8, device=c.device)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_packed_a(packed.storage.data_ptr(), packed.dtype, packed.n, C.byref(ob), oi_ref,
+                                            C.byref(oc), ws_ptr, ws_size, _stream_handle(stream)))
+    return c
+
+
+def matmul_packed_ab(packed_a: PackedB, packed_b: PackedB, c, c_in=None, workspace=None, stream=None):
+    """c[M,N] = c_in + A . B^T with both operands packed (``pack_a``, ``pack_b``); returns c."""
+    import torch
+    if packed_a.k != packed_b.k:
+        raise ValueError("matmul_packed_ab: the packed operands differ in K")
+    oc = operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    oi_ref = C.byref(oi) if oi is not None else None
+    need = lib().vecops_hip_matmul_packed_ab_workspace(packed_a.dtype, packed_a.n, packed_b.dtype, packed_b.n, packed_a.k,
+                                                       oi_ref, C.byref(oc))
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=c.device)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_packed_ab(packed_a.storage.data_ptr(), packed_a.dtype, packed_a.n,
+                                             packed_b.storage.data_ptr(), packed_b.dtype, packed_b.n, packed_a.k, oi_ref,
+                                             C.byref(oc), ws_ptr, ws_size, _stream_handle(stream)))
+    return c
 
 
 def plan_matmul_packed_b(a, packed: PackedB, c, c_in=None) -> Plan:

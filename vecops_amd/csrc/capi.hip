@@ -62,6 +62,7 @@ bool normalise(const VecopsHipOperand* o, View* v) {
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+uint64_t round_up_256(uint64_t v) { return (v + 255u) & ~uint64_t{255}; }
 
 // 16-byte loads along K: unit K stride.  Rows need not be 16-byte aligned: global and buffer loads
 // take any byte address on this target (the compiler itself emits dwordx4 loads for under-aligned
@@ -675,15 +676,16 @@ int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t 
     if (da != DT_BF16 && da != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: a bf16-packed b needs a bf16 or f32 a");
   } else if (packed_dtype == DT_F16) {
     if (da != DT_F16) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an f16-packed b needs an f16 a");
-  } else if (packed_dtype == DT_I8) {
-    if (da != DT_I8 && da != DT_U8) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an i8-packed b needs an i8 or u8 a");
+  } else if (packed_dtype == DT_I8 || packed_dtype == DT_U8) {
+    if (da != DT_I8 && da != DT_U8) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an 8-bit packed b needs an i8 or u8 a");
   } else {
     return fail(ST_NOT_APPLICABLE, "matmul_packed_b: packed dtype %u not supported", packed_dtype);
   }
   VecopsHipOperand b;
   memset(&b, 0, sizeof(b));
   b.data = const_cast<void*>(packed);
-  b.dtype = packed_dtype == DT_I8 ? DT_I8 : da;
+  // (an unsigned operand is packed as b - 128, signed: the product's epilogue adds 128 * sum_k a[m,k] back)
+  b.dtype = (packed_dtype == DT_I8 || packed_dtype == DT_U8) ? packed_dtype : da;
   b.rank = a->rank;
   const int base = a->rank == 3 ? 1 : 0;
   const int64_t k = a->sizes[base + 1];
@@ -696,14 +698,17 @@ int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t 
   if (rc != ST_OK) return rc;
   pr->packed_b = true;
   // 32-bit offsets inside one workgroup's eight 32-row panels of the packed operand
-  const int64_t ks_total = packed_k_steps(pr->k, packed_dtype == DT_I8 ? 16 : 8);
+  const int64_t ks_total = packed_k_steps(pr->k, (packed_dtype == DT_I8 || packed_dtype == DT_U8) ? 16 : 8);
   if (ks_total * 1024 * 8 >= (int64_t{1} << 31)) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: k too large");
   return ST_OK;
 }
 
 int src_of_packed_source(uint32_t dtype) {
   // (half operands are packed by the bf16 kernel: a permutation of 16-bit elements either way)
-  return (dtype == DT_BF16 || dtype == DT_F16) ? SRC_BF16 : dtype == DT_F32 ? SRC_F32_AS_BF16 : dtype == DT_I8 ? SRC_I8 : -1;
+  return (dtype == DT_BF16 || dtype == DT_F16) ? SRC_BF16
+         : dtype == DT_F32                     ? SRC_F32_AS_BF16
+         : (dtype == DT_I8 || dtype == DT_U8)  ? SRC_I8
+                                               : -1;
 }
 
 }  // namespace
@@ -711,8 +716,9 @@ int src_of_packed_source(uint32_t dtype) {
 extern "C" {
 
 uint64_t vecops_hip_packed_b_bytes(uint32_t packed_dtype, int64_t n, int64_t k) {
-  if (n < 0 || k < 0 || (packed_dtype != DT_BF16 && packed_dtype != DT_F16 && packed_dtype != DT_I8)) return 0;
-  return static_cast<uint64_t>(packed_b_bytes(n, k, packed_dtype == DT_I8 ? 16 : 8));
+  if (n < 0 || k < 0 || (packed_dtype != DT_BF16 && packed_dtype != DT_F16 && packed_dtype != DT_I8 && packed_dtype != DT_U8))
+    return 0;
+  return static_cast<uint64_t>(packed_b_bytes(n, k, (packed_dtype == DT_I8 || packed_dtype == DT_U8) ? 16 : 8));
 }
 
 int32_t vecops_hip_pack_b(const VecopsHipOperand* b, void* packed, uint64_t packed_size, void* stream) {
@@ -735,6 +741,7 @@ int32_t vecops_hip_pack_b(const VecopsHipOperand* b, void* packed, uint64_t pack
   q.ks = v.cs;
   q.n = static_cast<int32_t>(v.rows);
   q.k = static_cast<int32_t>(v.cols);
+  q.flip = v.dtype == DT_U8 ? 0x80u : 0u;
   hipError_t e = launch_pack_b(src, q, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(ST_EXEC, "pack kernel launch: %s", hipGetErrorString(e));
   return ST_OK;
@@ -777,6 +784,120 @@ int32_t vecops_hip_matmul_packed_b(const VecopsHipOperand* a, const void* packed
   VecopsHipPlan plan;
   choose(pr, &plan);
   return run_problem(pr, plan, nullptr, nullptr, nullptr, workspace, workspace_size, static_cast<hipStream_t>(stream));
+}
+
+int32_t vecops_hip_pack_a(const VecopsHipOperand* a, void* packed, uint64_t packed_size, void* stream) {
+  // the [M,K] operand in the same 32-row panels: the two sides share one format here
+  return vecops_hip_pack_b(a, packed, packed_size, stream);
+}
+
+namespace {
+// The descriptor of the transposed matrix (the last two dimensions swapped).
+VecopsHipOperand transposed(const VecopsHipOperand& o) {
+  VecopsHipOperand t = o;
+  if (o.rank == 2 || o.rank == 3) {
+    const int i = static_cast<int>(o.rank) - 2;
+    t.sizes[i] = o.sizes[i + 1]; t.sizes[i + 1] = o.sizes[i];
+    t.strides[i] = o.strides[i + 1]; t.strides[i + 1] = o.strides[i];
+  }
+  return t;
+}
+
+// A packed: C^T = B . A^T is the product of the plain operand b with the packed operand a.
+int32_t describe_packed_a(const void* packed_a, uint32_t packed_dtype, int64_t m, const VecopsHipOperand* b,
+                          const VecopsHipOperand* c_in, const VecopsHipOperand* c, VecopsHipOperand* ct,
+                          VecopsHipOperand* cint, Problem* pr) {
+  if (b == nullptr || c == nullptr) return fail(ST_INVALID, "matmul_packed_a: null operand");
+  *ct = transposed(*c);
+  if (c_in != nullptr) *cint = transposed(*c_in);
+  return describe_packed(b, packed_a, packed_dtype, m, c_in ? cint : nullptr, ct, pr);
+}
+}  // namespace
+
+int32_t vecops_hip_plan_matmul_packed_a(uint32_t packed_dtype, int64_t m, const VecopsHipOperand* b,
+                                        const VecopsHipOperand* c_in, const VecopsHipOperand* c, VecopsHipPlan* plan) {
+  if (plan == nullptr) return fail(ST_INVALID, "plan_matmul_packed_a: null plan");
+  Problem pr{};
+  VecopsHipOperand ct, cint;
+  int32_t rc = describe_packed_a(reinterpret_cast<void*>(16), packed_dtype, m, b, c_in, c, &ct, &cint, &pr);
+  if (rc != ST_OK) return rc;
+  choose(pr, plan);
+  return ST_OK;
+}
+
+int32_t vecops_hip_matmul_packed_a(const void* packed_a, uint32_t packed_dtype, int64_t m, const VecopsHipOperand* b,
+                                   const VecopsHipOperand* c_in, const VecopsHipOperand* c, void* workspace,
+                                   uint64_t workspace_size, void* stream) {
+  Problem pr{};
+  VecopsHipOperand ct, cint;
+  int32_t rc = describe_packed_a(packed_a, packed_dtype, m, b, c_in, c, &ct, &cint, &pr);
+  if (rc != ST_OK) return rc;
+  if (pr.k > 0 && pr.n > 0 && !aligned16(packed_a)) return fail(ST_INVALID, "matmul_packed_a: packed a must be 16-byte aligned");
+  VecopsHipPlan plan;
+  choose(pr, &plan);
+  return run_problem(pr, plan, nullptr, nullptr, nullptr, workspace, workspace_size, static_cast<hipStream_t>(stream));
+}
+
+namespace {
+// Both operands packed: A is unpacked into the front of the workspace (a dense [M,K] matrix of its own dtype) and
+// multiplied with the packed B.
+struct BothPacked {
+  VecopsHipOperand a;
+  Problem pr{};
+  VecopsHipPlan plan;
+  uint64_t a_bytes;
+};
+int32_t describe_packed_ab(uint32_t a_dtype, int64_t m, uint32_t b_dtype, int64_t n, int64_t k, const VecopsHipOperand* c_in,
+                           const VecopsHipOperand* c, void* workspace, BothPacked* d) {
+  if (m < 0 || n < 0 || k < 0) return fail(ST_INVALID, "matmul_packed_ab: negative extent");
+  if (a_dtype != DT_BF16 && a_dtype != DT_F16 && a_dtype != DT_I8 && a_dtype != DT_U8)
+    return fail(ST_NOT_APPLICABLE, "matmul_packed_ab: packed dtype %u not supported", a_dtype);
+  if (c == nullptr || c->rank != 2) return fail(ST_NOT_APPLICABLE, "matmul_packed_ab: c must be rank 2 (a packed operand has no batches)");
+  make_operand(&d->a, workspace, a_dtype, m, k, k);
+  d->a_bytes = round_up_256(static_cast<uint64_t>(m) * k * dtype_bytes(a_dtype));
+  int32_t rc = describe_packed(&d->a, reinterpret_cast<void*>(16), b_dtype, n, c_in, c, &d->pr);
+  if (rc != ST_OK) return rc;
+  choose(d->pr, &d->plan);
+  return ST_OK;
+}
+}  // namespace
+
+uint64_t vecops_hip_matmul_packed_ab_workspace(uint32_t a_dtype, int64_t m, uint32_t b_dtype, int64_t n, int64_t k,
+                                               const VecopsHipOperand* c_in, const VecopsHipOperand* c) {
+  BothPacked d;
+  if (describe_packed_ab(a_dtype, m, b_dtype, n, k, c_in, c, reinterpret_cast<void*>(256), &d) != ST_OK) return 0;
+  return d.a_bytes + d.plan.workspace_bytes;
+}
+
+int32_t vecops_hip_matmul_packed_ab(const void* packed_a, uint32_t a_dtype, int64_t m, const void* packed_b, uint32_t b_dtype,
+                                    int64_t n, int64_t k, const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                    void* workspace, uint64_t workspace_size, void* stream) {
+  BothPacked d;
+  int32_t rc = describe_packed_ab(a_dtype, m, b_dtype, n, k, c_in, c, workspace ? workspace : reinterpret_cast<void*>(256), &d);
+  if (rc != ST_OK) return rc;
+  if (d.plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
+  const uint64_t need = d.a_bytes + d.plan.workspace_bytes;
+  if (need > workspace_size || (need > 0 && (workspace == nullptr || !aligned16(workspace))))
+    return fail(ST_INVALID, "matmul_packed_ab: %llu bytes of 16-byte aligned workspace required, %llu supplied",
+                (unsigned long long)need, (unsigned long long)workspace_size);
+  if (k > 0 && (packed_a == nullptr || packed_b == nullptr || !aligned16(packed_a) || !aligned16(packed_b)))
+    return fail(ST_INVALID, "matmul_packed_ab: packed operands must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (k > 0 && m > 0) {
+    PackBParams q;
+    q.b = workspace;
+    q.packed = const_cast<void*>(packed_a);
+    q.rs = k;
+    q.ks = 1;
+    q.n = static_cast<int32_t>(m);
+    q.k = static_cast<int32_t>(k);
+    q.flip = a_dtype == DT_U8 ? 0x80u : 0u;
+    hipError_t e = launch_unpack_b((a_dtype == DT_I8 || a_dtype == DT_U8) ? SRC_I8 : SRC_BF16, q, s);
+    if (e != hipSuccess) return fail(ST_EXEC, "unpack kernel launch: %s", hipGetErrorString(e));
+  }
+  d.pr.b.data = const_cast<void*>(packed_b);
+  return run_problem(d.pr, d.plan, nullptr, nullptr, nullptr, static_cast<char*>(workspace) + d.a_bytes,
+                     workspace_size - d.a_bytes, s);
 }
 
 int32_t vecops_hip_matmul_i8_dequant_packed_b(const int8_t* a, int64_t lda, const void* packed_b,
@@ -1078,8 +1199,6 @@ struct Grouped {
   std::vector<int32_t> first;     // first workgroup of each table group, and the end
   uint64_t first_bytes = 0, record_bytes = 0, map_bytes = 0, loop_workspace = 0;
 };
-
-uint64_t round_up_256(uint64_t v) { return (v + 255u) & ~uint64_t{255}; }
 
 int32_t describe_grouped(uint32_t count, const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
                          const VecopsHipOperand* c, uint32_t compute, Grouped* g) {

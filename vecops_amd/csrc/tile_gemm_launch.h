@@ -50,6 +50,8 @@ hipError_t launch_packed_row_sums(const void* packed, int32_t n, int32_t k, int3
                                   const int32_t* add, int32_t* out, hipStream_t stream);
 struct PackBParams;
 hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream);
+// the dense operand back out of its packed form (src: SRC_BF16 for 16-bit elements, SRC_I8 for bytes)
+hipError_t launch_unpack_b(int src, const PackBParams& p, hipStream_t stream);
 
 // Shared by the per-class translation units.
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB>

@@ -31,10 +31,11 @@ __host__ __device__ inline int64_t packed_b_bytes(int64_t n, int64_t k, int elem
 }
 
 struct PackBParams {
-  const void* b;   // [N, K] with element strides rs, ks
+  const void* b;   // [N, K] with element strides rs, ks (unpacking: the destination)
   void* packed;
   int64_t rs, ks;
   int32_t n, k;
+  uint32_t flip;   // bytes only: 0x80 packs an unsigned operand as the signed b - 128 (padding stays zero)
 };
 
 // One thread per 16-byte chunk of the packed operand.  SRC_BF16: bf16 in, bf16
@@ -60,13 +61,43 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const PackBParams p) {
           uint32_t v;
           if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(p.b)[at];
           else if constexpr (SRC == SRC_F32_AS_BF16) v = cvt_pk_bf16(static_cast<const float*>(p.b)[at], 0.0f) & 0xffffu;
-          else v = static_cast<const uint8_t*>(p.b)[at];
+          else v = static_cast<const uint8_t*>(p.b)[at] ^ p.flip;
           constexpr int per_word = EPC / 4;
           w[e / per_word] |= v << ((e % per_word) * (32 / per_word));
         }
       }
     }
     static_cast<u32x4*>(p.packed)[idx] = u32x4{w[0], w[1], w[2], w[3]};
+  }
+}
+
+// The inverse: the dense [N, K] operand (element strides rs, ks) back out of its packed form; 16-bit elements or
+// bytes (SRC_BF16 / SRC_I8), p.flip undone.  Used when both operands of a product arrive packed.
+template <int SRC>
+__global__ __launch_bounds__(256) void unpack_b_kernel(const PackBParams p) {
+  constexpr int EPC = SrcTraits<SRC>::kElemsPerChunk;
+  const int64_t ks_total = packed_k_steps(p.k, EPC);
+  const int64_t chunks = (static_cast<int64_t>(p.n) + 31) / 32 * ks_total * 64;
+  for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < chunks; idx += gridDim.x * 256ll) {
+    const int lane = static_cast<int>(idx & 63);
+    const int64_t block = idx >> 6;
+    const int64_t nb = block / ks_total, ks = block - nb * ks_total;
+    const int64_t n = nb * 32 + (lane & 31);
+    const int64_t k0 = (ks * 2 + (lane >> 5)) * EPC;
+    if (n >= p.n || k0 >= p.k) continue;
+    const u32x4 v = static_cast<const u32x4*>(p.packed)[idx];
+    const uint32_t w[4] = {v[0], v[1], v[2], v[3]};
+    constexpr int per_word = EPC / 4;
+#pragma unroll
+    for (int e = 0; e < EPC; ++e) {
+      const int64_t k = k0 + e;
+      if (k < p.k) {
+        const uint32_t bits = w[e / per_word] >> ((e % per_word) * (32 / per_word));
+        const int64_t at = n * p.rs + k * p.ks;
+        if constexpr (SRC == SRC_BF16) static_cast<uint16_t*>(const_cast<void*>(p.b))[at] = static_cast<uint16_t>(bits);
+        else static_cast<uint8_t*>(const_cast<void*>(p.b))[at] = static_cast<uint8_t>(bits ^ p.flip);
+      }
+    }
   }
 }
 

@@ -119,4 +119,19 @@ hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+hipError_t launch_unpack_b(int src, const PackBParams& p, hipStream_t stream) {
+  const int epc = src == SRC_I8 ? 16 : 8;
+  const int64_t chunks = packed_b_bytes(p.n, p.k, epc) / 16;
+  if (chunks == 0) return hipSuccess;
+  int64_t blocks = (chunks + 255) / 256;
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+  switch (src) {
+    case SRC_BF16: hipLaunchKernelGGL(unpack_b_kernel<SRC_BF16>, grid, block, 0, stream, p); break;
+    case SRC_I8: hipLaunchKernelGGL(unpack_b_kernel<SRC_I8>, grid, block, 0, stream, p); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
 }  // namespace vecops_hip

@@ -645,13 +645,17 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
 }
 
 // =================================================================================================
-#elif VECOPS_ARTIFACT_KIND == 11 || VECOPS_ARTIFACT_KIND == 12  // vecops::matmul_pack_b (b, a_zero_point, packed, compensation?)
+#elif VECOPS_ARTIFACT_KIND == 11 || VECOPS_ARTIFACT_KIND == 12 || VECOPS_ARTIFACT_KIND == 17  // vecops::matmul_pack_b (b, a_zero_point, packed, compensation?)
 // =================================================================================================
 
 #if VECOPS_ARTIFACT_KIND == 11
 #define OPERANDS "bf16"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16) | bit(VECOPS_DTYPE_F32);  // fp32 sources are rounded to bf16
 constexpr uint32_t kPackedDtype = VECOPS_DTYPE_BF16;
+#elif VECOPS_ARTIFACT_KIND == 17
+#define OPERANDS "f16"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F16);
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_F16;
 #else
 #define OPERANDS "i8"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8);
@@ -716,7 +720,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
 }
 
 // =================================================================================================
-#elif VECOPS_ARTIFACT_KIND >= 13 && VECOPS_ARTIFACT_KIND <= 15  // vecops::matmul_packed_b (a, packed_b, c_in?, c)
+#elif (VECOPS_ARTIFACT_KIND >= 13 && VECOPS_ARTIFACT_KIND <= 15) || VECOPS_ARTIFACT_KIND == 18  // vecops::matmul_packed_b (a, packed_b, c_in?, c)
 // =================================================================================================
 
 #if VECOPS_ARTIFACT_KIND == 13
@@ -725,6 +729,9 @@ constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16);
 #elif VECOPS_ARTIFACT_KIND == 14
 #define OPERANDS "f32"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
+#elif VECOPS_ARTIFACT_KIND == 18
+#define OPERANDS "f16"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F16);
 #else
 #define OPERANDS "i8"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);
@@ -732,6 +739,9 @@ constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);
 #if VECOPS_ARTIFACT_KIND == 15
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_I32);
 constexpr uint32_t kPackedDtype = VECOPS_DTYPE_I8;
+#elif VECOPS_ARTIFACT_KIND == 18
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_F16);
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_F16;
 #else
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
 constexpr uint32_t kPackedDtype = VECOPS_DTYPE_BF16;

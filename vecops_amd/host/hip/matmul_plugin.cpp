@@ -282,8 +282,8 @@ rt::OperatorSchema make_matmul_w8a16_group_schema() {
 rt::OperatorSchema make_matmul_pack_b_schema() {
   using rt::dtype_bit;
   std::vector<rt::ParameterSchema> params;
-  params.push_back(tensor_param("b", dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8), 2u,
-                                VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("b", dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                                       dtype_bit(DType::Int8), 2u, VECOPS_TENSOR_READ));
   params.push_back(rt::ParameterSchema{"a_zero_point", rt::ScalarConstraint{dtype_bit(DType::Int64) | dtype_bit(DType::Int32)}});
   params.push_back(tensor_param("packed", dtype_bit(DType::UInt8), 1u, VECOPS_TENSOR_WRITE));
   params.push_back(tensor_param("compensation", dtype_bit(DType::Int32), 1u, VECOPS_TENSOR_WRITE, /*optional=*/true));
@@ -292,9 +292,10 @@ rt::OperatorSchema make_matmul_pack_b_schema() {
 
 rt::OperatorSchema make_matmul_packed_b_schema() {
   using rt::dtype_bit;
-  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int8) |
-                           dtype_bit(DType::UInt8);
-  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float32) | dtype_bit(DType::Int32);
+  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                           dtype_bit(DType::Int8) | dtype_bit(DType::UInt8);
+  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                            dtype_bit(DType::Int32);
   std::vector<rt::ParameterSchema> params;
   params.push_back(tensor_param("a", in, std::nullopt, VECOPS_TENSOR_READ));
   params.push_back(tensor_param("packed_b", dtype_bit(DType::UInt8), 1u, VECOPS_TENSOR_READ));
@@ -485,15 +486,16 @@ rt::Result<rt::BoundKernelRecipe> MatmulW8A16GroupRecipe::bind(const rt::KernelC
 }
 
 MatmulPackBRecipe::MatmulPackBRecipe(OperandClass packed) : packed_(packed) {
-  id_ = packed == OperandClass::I8 ? "hip.matmul_pack_b.i8" : "hip.matmul_pack_b.bf16";
+  id_ = packed == OperandClass::I8 ? "hip.matmul_pack_b.i8" : packed == OperandClass::F16 ? "hip.matmul_pack_b.f16" : "hip.matmul_pack_b.bf16";
 }
 
 Status MatmulPackBRecipe::match(const rt::KernelCall& call) const {
   const auto values = call.arguments().values();
   const TensorView* b = tensor_at(values, 0);
   if (b == nullptr) return invalid("vecops::matmul_pack_b needs a b tensor");
-  const bool mine = packed_ == OperandClass::I8 ? b->dtype == DType::Int8
-                                                : (b->dtype == DType::BFloat16 || b->dtype == DType::Float32);
+  const bool mine = packed_ == OperandClass::I8    ? b->dtype == DType::Int8
+                    : packed_ == OperandClass::F16 ? b->dtype == DType::Float16
+                                                   : (b->dtype == DType::BFloat16 || b->dtype == DType::Float32);
   if (!mine) return not_applicable("source dtype belongs to another recipe");
   auto place = placement_of(call);
   if (!place) return place.status();
@@ -504,7 +506,8 @@ rt::Result<rt::BoundKernelRecipe> MatmulPackBRecipe::bind(const rt::KernelCall& 
   if (Status st = match(call); !st.ok()) return st;
   rt::BoundKernelRecipe bound;
   bound.recipe_id = id_;
-  bound.specialization_key = std::string(kMatmulPackBName) + ";operands=" + (packed_ == OperandClass::I8 ? "i8" : "bf16") +
+  bound.specialization_key = std::string(kMatmulPackBName) + ";operands=" +
+                             (packed_ == OperandClass::I8 ? "i8" : packed_ == OperandClass::F16 ? "f16" : "bf16") +
                              ";memory=" + placement_name(placement_of(call).value()) + ";" + kBackend;
   bound.artifact_key = id_ + ";" + bound.specialization_key;
   return bound;
@@ -512,6 +515,7 @@ rt::Result<rt::BoundKernelRecipe> MatmulPackBRecipe::bind(const rt::KernelCall& 
 
 MatmulPackedBRecipe::MatmulPackedBRecipe(OperandClass operands) : operands_(operands) {
   id_ = operands == OperandClass::BF16 ? "hip.matmul_packed_b.bf16.tile"
+        : operands == OperandClass::F16 ? "hip.matmul_packed_b.f16.tile"
         : operands == OperandClass::F32 ? "hip.matmul_packed_b.f32.tile"
                                         : "hip.matmul_packed_b.i8.tile";
 }
@@ -524,12 +528,14 @@ Status MatmulPackedBRecipe::match(const rt::KernelCall& call) const {
   if (a == nullptr || c == nullptr) return invalid("vecops::matmul_packed_b needs a and c tensors");
   const bool mine = operands_ == OperandClass::I8 ? (a->dtype == DType::Int8 || a->dtype == DType::UInt8)
                     : operands_ == OperandClass::F32 ? a->dtype == DType::Float32
+                    : operands_ == OperandClass::F16 ? a->dtype == DType::Float16
                                                      : a->dtype == DType::BFloat16;
   if (!mine) return not_applicable("operand dtype belongs to another recipe");
   const bool int_out = operands_ == OperandClass::I8;
-  if (int_out ? c->dtype != DType::Int32 : (c->dtype != DType::Float32 && c->dtype != DType::BFloat16))
+  const DType narrow = operands_ == OperandClass::F16 ? DType::Float16 : DType::BFloat16;  // the operands' own 16-bit type
+  if (int_out ? c->dtype != DType::Int32 : (c->dtype != DType::Float32 && c->dtype != narrow))
     return not_applicable("output dtype does not fit these operands");
-  if (cin != nullptr && (int_out ? cin->dtype != DType::Int32 : (cin->dtype != DType::Float32 && cin->dtype != DType::BFloat16)))
+  if (cin != nullptr && (int_out ? cin->dtype != DType::Int32 : (cin->dtype != DType::Float32 && cin->dtype != narrow)))
     return not_applicable("c_in dtype does not fit these operands");
   auto place = placement_of(call);
   if (!place) return place.status();
@@ -538,7 +544,10 @@ Status MatmulPackedBRecipe::match(const rt::KernelCall& call) const {
 
 rt::Result<rt::BoundKernelRecipe> MatmulPackedBRecipe::bind(const rt::KernelCall& call) const {
   if (Status st = match(call); !st.ok()) return st;
-  const char* operands = operands_ == OperandClass::BF16 ? "bf16" : operands_ == OperandClass::F32 ? "f32" : "i8";
+  const char* operands = operands_ == OperandClass::BF16 ? "bf16"
+                         : operands_ == OperandClass::F16 ? "f16"
+                         : operands_ == OperandClass::F32 ? "f32"
+                                                          : "i8";
   rt::BoundKernelRecipe bound;
   bound.recipe_id = id_;
   bound.specialization_key = std::string(kMatmulPackedBName) + ";operands=" + operands + ";memory=" +
@@ -586,10 +595,13 @@ MatmulDispatchPolicy::candidates(const rt::KernelCall& call,
     }
     if (const auto* mp = dynamic_cast<const MatmulPackedBRecipe*>(recipes[i].get()); mp != nullptr && a != nullptr) {
       if (mp->operands() == OperandClass::I8 ? (a->dtype != DType::Int8 && a->dtype != DType::UInt8)
-          : mp->operands() == OperandClass::F32 ? a->dtype != DType::Float32 : a->dtype != DType::BFloat16) continue;
+          : mp->operands() == OperandClass::F32 ? a->dtype != DType::Float32
+          : mp->operands() == OperandClass::F16 ? a->dtype != DType::Float16
+                                                : a->dtype != DType::BFloat16) continue;
     }
     if (const auto* pk = dynamic_cast<const MatmulPackBRecipe*>(recipes[i].get()); pk != nullptr && a != nullptr) {
-      if ((pk->operands() == OperandClass::I8) != (a->dtype == DType::Int8)) continue;
+      if ((pk->operands() == OperandClass::I8) != (a->dtype == DType::Int8) ||
+          (pk->operands() == OperandClass::F16) != (a->dtype == DType::Float16)) continue;
     }
     order.push_back(i);
   }
@@ -693,13 +705,15 @@ std::shared_ptr<rt::Operator> make_matmul_fused_operator(const std::filesystem::
 
 std::shared_ptr<rt::Operator> make_matmul_pack_b_operator(const std::filesystem::path& dir) {
   return assemble(make_matmul_pack_b_schema(),
-                  {std::make_shared<MatmulPackBRecipe>(OperandClass::BF16), std::make_shared<MatmulPackBRecipe>(OperandClass::I8)},
+                  {std::make_shared<MatmulPackBRecipe>(OperandClass::BF16), std::make_shared<MatmulPackBRecipe>(OperandClass::F16),
+                   std::make_shared<MatmulPackBRecipe>(OperandClass::I8)},
                   dir);
 }
 
 std::shared_ptr<rt::Operator> make_matmul_packed_b_operator(const std::filesystem::path& dir) {
   return assemble(make_matmul_packed_b_schema(),
                   {std::make_shared<MatmulPackedBRecipe>(OperandClass::BF16),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::F16),
                    std::make_shared<MatmulPackedBRecipe>(OperandClass::F32),
                    std::make_shared<MatmulPackedBRecipe>(OperandClass::I8)},
                   dir);
