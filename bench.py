@@ -420,13 +420,13 @@ def bench_copy(dev, steps, warmup):
 def recorded_reference():
     """vecops' own CPU matmul on the headline workload, as timed in the build container by oracle/time_reference.py
     (the vecops tree is not present where the benchmark runs): figures with their provenance, or None."""
-    path = os.path.join(ROOT, "oracle", "reference_timings.json")
+    path = os.path.join(ROOT, "baseline", "vecops_cpu_container.json")
     if not os.path.exists(path):
         return None
     with open(path) as f:
         doc = json.load(f)
     rows = [e for e in doc["entries"] if e["config"].startswith("bf16 4096^3")]
-    return {"source": "oracle/reference_timings.json (oracle/time_reference.py, in the build container)",
+    return {"source": "baseline/vecops_cpu_container.json (oracle/time_reference.py, in the build container)",
             "what": doc["what"], "host": doc["host"],
             "entries": [{"config": e["config"], "lanes": e["lanes"], "value": e["rate"] / 1e3, "unit": "TFLOP/s",
                          "ms": e["ms"]} for e in rows]}

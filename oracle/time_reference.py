@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Times the real vecops CPU matmul (oracle/_ref, built from the vecops sources by oracle/Makefile) on the five
-benchmark configurations, on one lane and on eight lanes, and writes oracle/reference_timings.json.
+benchmark configurations, on one lane and on eight lanes, and writes baseline/vecops_cpu_container.json.
 
     python oracle/time_reference.py
 
@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 from oracle.oracle import Reference  # noqa: E402
 from vecops_amd import synth  # noqa: E402
 
-OUT = os.path.join(HERE, "reference_timings.json")
+OUT = os.path.join(os.path.dirname(HERE), "baseline", "vecops_cpu_container.json")
 
 
 def _time(fn, budget_s=4.0, min_reps=2):
