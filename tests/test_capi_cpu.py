@@ -83,6 +83,13 @@ def test_rule_table_known_answers():
     # one row against a long weight matrix: the skinny family, no workspace
     rc, p = _plan(_operand(capi.BF16, (1, 4096)), _operand(capi.BF16, (14336, 4096)), _operand(capi.BF16, (1, 14336)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "skinny" and p.workspace_bytes == 0
+    # fp32 memory takes it too, whichever way it is multiplied (a lane's chunk is 8 elements, 4 in fp32 compute)
+    rc, p = _plan(_operand(capi.F32, (4, 4096)), _operand(capi.F32, (14336, 4096)), _operand(capi.F32, (4, 14336)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "skinny"
+    rc, p = _plan(_operand(capi.F32, (4, 516)), _operand(capi.F32, (14336, 516)), _operand(capi.F32, (4, 14336)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] != "skinny"
+    rc, p = _plan(_operand(capi.F32, (4, 516)), _operand(capi.F32, (14336, 516)), _operand(capi.F32, (4, 14336)), compute=1)
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "skinny"
     # ... but not with a K that 16-byte loads cannot cover
     rc, p = _plan(_operand(capi.BF16, (1, 129)), _operand(capi.BF16, (4097, 129)), _operand(capi.F32, (1, 4097)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] != "skinny"

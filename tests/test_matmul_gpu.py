@@ -501,6 +501,41 @@ def test_skinny_bf16_family(device, oracle, m, n, k):
     assert np.array_equal(host_bits(c16), oracle.bf16_from_f32(got))
 
 
+@pytest.mark.parametrize("compute", ["bf16", "f32"])
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (4, 14336, 1024), (16, 1000, 520), (3000, 7, 264), (1, 513, 64)])
+def test_skinny_f32_operand_family(device, oracle, compute, m, n, k):
+    """fp32 memory on the skinny kernel, rounded to bf16 on the way in (AMX_BF16F32 with fp32 memory) or multiplied in
+    fp32 (SME_F32F32): vecops' small-vector leaves serve every atom (matmul/details/kernel/amx/Backend.h:767-992).
+    Either side narrow, fp32 and bf16 outputs; a K that is not a multiple of the lane's chunk keeps the tile path."""
+    import torch
+    from vecops_amd import capi
+    a, b = synth.uniform_pm1(1, (m, k)).astype(np.float32), synth.uniform_pm1(2, (n, k)).astype(np.float32)
+    ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    code = capi.COMPUTE_F32 if compute == "f32" else capi.COMPUTE_BF16
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    assert capi.FAMILY_NAMES[capi.plan_matmul(ta, tb, c, compute=code).family] == "skinny"
+    capi.matmul(ta, tb, c, compute=code)
+    c16 = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    capi.matmul(ta, tb, c16, compute=code)
+    torch.cuda.synchronize()
+    if compute == "f32":
+        want = (a.astype(np.float64) @ b.astype(np.float64).T).astype(np.float32)
+    else:
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(synth.bf16_round(a), synth.bf16_round(b), want, acc_f64=True)
+    got = c.cpu().numpy()
+    assert rel_err(got, want) <= fp32_tol(k)
+    assert np.array_equal(host_bits(c16), oracle.bf16_from_f32(got))
+    # K + 2: no longer whole chunks per lane - the tile kernels, same values on the common columns
+    a2, b2 = np.pad(a, ((0, 0), (0, 2))), np.pad(b, ((0, 0), (0, 2)))
+    ta2, tb2 = torch.from_numpy(a2).to(device), torch.from_numpy(b2).to(device)
+    assert capi.FAMILY_NAMES[capi.plan_matmul(ta2, tb2, c, compute=code).family] != "skinny"
+    c2 = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul(ta2, tb2, c2, compute=code)
+    torch.cuda.synchronize()
+    assert rel_err(c2.cpu().numpy(), want) <= fp32_tol(k)
+
+
 def test_skinny_bf16_batched_strided(device, oracle):
     """Rank-3 batch with a broadcast narrow operand, padded rows of the wide operand and a
     transposed (column-major) output."""

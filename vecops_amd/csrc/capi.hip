@@ -221,11 +221,12 @@ constexpr int kStreamGroupsPerUnit = 2;  // workgroups of 4 wavefronts per compu
 // small tile falls to 0.78-0.80 at 8192^3.
 constexpr int64_t kQuality256x128 = 800, kQuality128 = 850;
 
-// bf16 x bf16, f16 x f16 or int8 x int8 with K contiguous on both sides, no C input, one side <= 16 rows, the other >= 512
+// Every operand class but the unsigned bytes, with K contiguous on both sides, no C input, one side <= 16 rows, the
+// other >= 512 (vecops' small-vector leaves serve every atom, matmul/details/kernel/amx/Backend.h:767-992)
 bool skinny_applies(const Problem& pr) {
   if (pr.fused) return false;  // the skinny kernels have no output transform
-  if ((pr.src != SRC_BF16 && pr.src != SRC_F16 && pr.src != SRC_I8) || pr.has_cin || pr.packed_b) return false;
-  const int64_t per = pr.src == SRC_I8 ? 16 : 8;  // elements per 16 bytes
+  if (pr.src == SRC_I8_FLIP || pr.has_cin || pr.packed_b) return false;
+  const int64_t per = pr.src == SRC_I8 ? 16 : pr.src == SRC_F32 ? 4 : 8;  // elements a lane takes per step
   if (!k_vector_ok(pr.a) || !k_vector_ok(pr.b) || pr.k % per != 0 || pr.k < 8 * per) return false;
   const int64_t narrow = pr.m < pr.n ? pr.m : pr.n, wide = pr.m < pr.n ? pr.n : pr.m;
   // (the skinny kernels read one set of scales and one correction row for every batch)
@@ -563,6 +564,8 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     };
     if (is_int) launch(std::integral_constant<int, SRC_I8>{});
     else if (pr.src == SRC_F16) launch(std::integral_constant<int, SRC_F16>{});
+    else if (pr.src == SRC_F32_AS_BF16) launch(std::integral_constant<int, SRC_F32_AS_BF16>{});
+    else if (pr.src == SRC_F32) launch(std::integral_constant<int, SRC_F32>{});
     else launch(std::integral_constant<int, SRC_BF16>{});
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(ST_EXEC, "skinny kernel launch: %s", hipGetErrorString(e));

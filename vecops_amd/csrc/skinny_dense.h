@@ -1,8 +1,8 @@
 // Skinny matmul for gfx950 (HBM-bound): one operand has at most 16 rows.
 //   y[s, r] = sum_k x[s, k] * w[r, k]      w: the wide operand [R, K], x: the narrow one [S <= 16, K]
-// bf16 x bf16 with fp32 accumulation, or int8 x int8 with wrapping int32 accumulation
-// (optionally followed by the per-row x per-column dequantisation); both operands K
-// contiguous.  This is the GPU counterpart of vecops' small-vector leaves
+// bf16 x bf16 (f16 x f16) with fp32 accumulation, fp32 operands rounded to bf16 on their way into the registers or
+// multiplied in fp32, or int8 x int8 with wrapping int32 accumulation (optionally followed by the per-row x
+// per-column dequantisation); both operands K contiguous.  This is the GPU counterpart of vecops' small-vector leaves
 // (small_vector_dense_matmul / small_vector_tall_matmul,
 // matmul/details/kernel/amx/Backend.h:767-1151): the wide operand is read exactly
 // once, the narrow one is kept in registers.
@@ -10,7 +10,9 @@
 // One v_mfma_f32_16x16x32_bf16 (_f16 for half operands; v_mfma_i32_16x16x64_i8) multiplies 16 wide rows by 16
 // narrow rows (S padded to 16 with zeros) over a step of 32 (64) k.  Lane l holds wide
 // row l % 16 and the 16 consecutive bytes of quarter l / 16 of the step (one 16-byte
-// load); the narrow operand uses the same k order.  A workgroup of 8 wavefronts owns
+// load; fp32 memory rounded to bf16: two loads, eight floats, converted in front of the MFMA);
+// the narrow operand uses the same k order.  fp32 compute: a step is 16 k, a lane's 16-byte load holds four
+// floats, and four v_mfma_f32_16x16x4_f32 each take one of them (k = 4 * quarter + e for MFMA e on both sides).  A workgroup of 8 wavefronts owns
 // PASSES x TILES blocks of 16 wide rows; its wavefronts split K step by step (step t
 // belongs to wavefront t % 8), so K need only be a multiple of 16 bytes.  K is walked
 // in blocks of 128 steps: a wavefront loads the narrow fragments of its 16 steps of the
@@ -49,9 +51,26 @@ struct SkinnyDenseParams {
 template <int SRC, int PASSES, int TILES>
 __global__ __launch_bounds__(512) void skinny_dense_kernel(const SkinnyDenseParams p) {
   constexpr bool INT = SrcTraits<SRC>::kInt;
-  constexpr int EPL = SrcTraits<SRC>::kElemsPerChunk;  // elements per lane and step (16 bytes)
+  constexpr int EPL = SrcTraits<SRC>::kElemsPerChunk;  // elements per lane and step
   constexpr int EPS = 4 * EPL;                         // elements per step
   constexpr int EB = SrcTraits<SRC>::kSrcBytes;
+  constexpr int LOADS = EPL * EB / 16;                 // 16-byte loads per lane and step (2: fp32 memory, bf16 compute)
+  struct Loaded { u32x4 v[LOADS]; };
+  // the lane's elements of one step as they lie in memory -> the MFMA operand
+  auto operand_of = [](const Loaded& raw) {
+    if constexpr (SRC == SRC_F32_AS_BF16) {
+      return u32x4{cvt_pk_bf16(__uint_as_float(raw.v[0][0]), __uint_as_float(raw.v[0][1])),
+                   cvt_pk_bf16(__uint_as_float(raw.v[0][2]), __uint_as_float(raw.v[0][3])),
+                   cvt_pk_bf16(__uint_as_float(raw.v[1][0]), __uint_as_float(raw.v[1][1])),
+                   cvt_pk_bf16(__uint_as_float(raw.v[1][2]), __uint_as_float(raw.v[1][3]))};
+    } else {
+      return raw.v[0];
+    }
+  };
+  auto load_of = [](const VECOPS_GLOBAL char* at, Loaded& out) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) out.v[i] = *(const VECOPS_GLOBAL u32x4*)(at + 16 * i);
+  };
   using AccScalar = typename std::conditional<INT, int32_t, float>::type;
   using Acc4 = typename std::conditional<INT, i32x4, f32x4>::type;
   constexpr int WAVES = 8, XS = 16, D = 4;  // XS steps per wavefront and K block
@@ -84,16 +103,21 @@ __global__ __launch_bounds__(512) void skinny_dense_kernel(const SkinnyDensePara
     for (int s = 0; s < XS; ++s) {
       const int k0 = k_of(s);
       xq[s] = u32x4{0u, 0u, 0u, 0u};
-      if (row < p.s && k0 < p.k) xq[s] = *(const VECOPS_GLOBAL u32x4*)(xrow + static_cast<int64_t>(k0) * EB);
+      if (row < p.s && k0 < p.k) {
+        Loaded raw;
+        load_of(xrow + static_cast<int64_t>(k0) * EB, raw);
+        xq[s] = operand_of(raw);
+      }
     }
     // flat sequence of (block, step) with the wide loads D ahead; a load past K reads as zero
-    u32x4 wq[D];
+    Loaded wq[D];
     auto issue = [&](auto slot_tag, auto b_tag, auto s_tag) {
       constexpr int slot = decltype(slot_tag)::value, b = decltype(b_tag)::value, s = decltype(s_tag)::value;
       if constexpr (b < BLOCKS) {
         const int k0 = k_of(s);
-        wq[slot] = u32x4{0u, 0u, 0u, 0u};
-        if (k0 < p.k) wq[slot] = *(const VECOPS_GLOBAL u32x4*)(wrow[b] + static_cast<int64_t>(k0) * EB);
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) wq[slot].v[i] = u32x4{0u, 0u, 0u, 0u};
+        if (k0 < p.k) load_of(wrow[b] + static_cast<int64_t>(k0) * EB, wq[slot]);
       }
     };
     static_for<D>([&](auto u) { issue(u, std::integral_constant<int, 0>{}, u); });
@@ -101,15 +125,22 @@ __global__ __launch_bounds__(512) void skinny_dense_kernel(const SkinnyDensePara
       constexpr int b = decltype(cb)::value;
       static_for<XS>([&](auto cs) {
         constexpr int s = decltype(cs)::value, slot = s % D;
+        const u32x4 wv = operand_of(wq[slot]);
         if constexpr (INT)
-          acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, wq[slot]),
+          acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, wv),
                                                          __builtin_bit_cast(i32x4, xq[s]), acc[b], 0, 0, 0);
         else if constexpr (SRC == SRC_F16) {
           typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wq[slot]),
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, wv),
                                                           __builtin_bit_cast(f16x8, xq[s]), acc[b], 0, 0, 0);
+        } else if constexpr (SRC == SRC_F32) {
+          // four floats per lane: MFMA e multiplies element e of every lane (the same k on both sides)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(wv[0]), __uint_as_float(xq[s][0]), acc[b], 0, 0, 0);
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(wv[1]), __uint_as_float(xq[s][1]), acc[b], 0, 0, 0);
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(wv[2]), __uint_as_float(xq[s][2]), acc[b], 0, 0, 0);
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(wv[3]), __uint_as_float(xq[s][3]), acc[b], 0, 0, 0);
         } else
-          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wq[slot]),
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv),
                                                            __builtin_bit_cast(bf16x8, xq[s]), acc[b], 0, 0, 0);
         constexpr int ns = s + D;  // the step that takes over this slot
         issue(std::integral_constant<int, slot>{}, std::integral_constant<int, b + ns / XS>{},
