@@ -31,6 +31,15 @@ extern "C" {
 
 #define VECOPS_HIP_ABI_VERSION 1u
 
+/*
+ * Flag for VecopsExecutionContext::flags of a call that reaches the kernels through vecops' artifact ABI (the field
+ * is "embedding-defined", runtime/CallAbi.h:369-370): the caller orders its own work on context->stream, so an artifact
+ * whose tensors live in device memory returns once its kernels are enqueued.  Without it such an artifact waits for
+ * them (vecops' ABI functions are synchronous, runtime/CallAbi.h:15-16).  Artifacts that stage host tensors always
+ * wait: their results have to be back in host memory on return.
+ */
+#define VECOPS_HIP_CONTEXT_STREAM_ORDERED 1ull
+
 /* One operand of a matmul: `data` addresses logical element zero in device
  * memory.  rank 2 = [rows, cols]; rank 3 = [batch, rows, cols].  Strides are in
  * elements; a zero batch stride broadcasts the operand over the batch

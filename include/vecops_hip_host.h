@@ -25,6 +25,9 @@ extern "C" {
 
 struct VecopsValue;
 struct VecopsExecutionContext;
+struct VecopsCall;
+struct VecopsError;
+struct VecopsSpecializationArgument;
 
 #define VECOPS_HIP_HOST_EXPORT __attribute__((visibility("default")))
 
@@ -66,6 +69,23 @@ VECOPS_HIP_HOST_EXPORT int32_t vecops_hip_host_operator_invoke(void* op, const s
                                                                uint64_t workspace_size,
                                                                const struct VecopsExecutionContext* context,
                                                                char* message, size_t message_capacity);
+
+/*
+ * The process-local bridge of vecops' generated framework adapters (runtime/OperatorBridgeAbi.h:69-71;
+ * implementation python/bindings/module.cpp:1223-1239): an extension holds an opaque handle and enters the Operator
+ * with vecops' own call record.  vecops_operator_bridge_invoke_v1 has the reference's name, signature and error
+ * protocol (VecopsCall, VecopsSpecializationArgument and VecopsError are the records of vecops_rt/abi.h, layout
+ * identical to vecops' headers): it validates the handle and the records, resolves the executable and invokes it
+ * synchronously, in one foreign call that holds no interpreter lock.  A call that brings no workspace gets device
+ * scratch from a per-thread buffer of the bridge, grown on demand and kept.  Handles are never reused: after
+ * vecops_hip_host_bridge_unregister a stale handle is an InvalidArgument (1), not another operator.
+ */
+VECOPS_HIP_HOST_EXPORT uint64_t vecops_hip_host_bridge_register(void* op);
+VECOPS_HIP_HOST_EXPORT void vecops_hip_host_bridge_unregister(uint64_t handle);
+VECOPS_HIP_HOST_EXPORT int32_t vecops_operator_bridge_invoke_v1(uint64_t handle, const struct VecopsCall* call,
+                                                                uint32_t num_specialization_values,
+                                                                const struct VecopsSpecializationArgument* specialization_values,
+                                                                struct VecopsError* error);
 
 /* Executable::load on one file: 0 when it is a valid artifact; writes its operator name and key. */
 VECOPS_HIP_HOST_EXPORT int32_t vecops_hip_host_load_artifact(const char* path, char* operator_name, size_t name_capacity,

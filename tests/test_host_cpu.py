@@ -99,8 +99,8 @@ def test_host_library_exports_every_declared_symbol(host):
     import re
     text = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include",
                              "vecops_hip_host.h")).read()
-    names = sorted(set(re.findall(r"VECOPS_HIP_HOST_EXPORT[^;(]*?\b(vecops_hip_host_\w+)\s*\(", text)))
-    assert len(names) == 7
+    names = sorted(set(re.findall(r"VECOPS_HIP_HOST_EXPORT[^;(]*?\b(vecops_(?:hip_host|operator_bridge)_\w+)\s*\(", text)))
+    assert len(names) == 10 and "vecops_operator_bridge_invoke_v1" in names
     lib = ctypes.CDLL(H.HOST_LIB)
     for name in names:
         assert getattr(lib, name) is not None
@@ -392,3 +392,73 @@ def test_invoke_without_a_gpu_is_an_execution_error(host):
         op.invoke(H.Frame([bf16((4, 8)), bf16((5, 8)), None, c], outputs=(3,)))
     assert e.value.code == 6 and "no HIP device" in e.value.message
     assert (c == 7.0).all()
+
+
+def test_bridge_records_have_the_reference_layout(tmp_path):
+    """VecopsSpecializationArgument and the bridge entry's prototype (runtime/OperatorBridgeAbi.h) as restated in
+    vecops_rt/abi.h: same sizes and offsets as vecops' own header, and the ctypes mirror agrees."""
+    probe = r"""
+#include <stddef.h>
+#include <stdio.h>
+#include HEADER
+int main(void) {
+  printf("%zu %zu %zu %zu %zu %u %u\n", sizeof(VecopsSpecializationArgument), offsetof(VecopsSpecializationArgument, kind),
+         offsetof(VecopsSpecializationArgument, name), offsetof(VecopsSpecializationArgument, value), sizeof(VecopsCall),
+         (unsigned)VECOPS_SPECIALIZATION_CONST_INT, (unsigned)VECOPS_SPECIALIZATION_DTYPE);
+  int32_t (*entry)(uint64_t, const VecopsCall*, uint32_t, const VecopsSpecializationArgument*, VecopsError*) =
+      vecops_operator_bridge_invoke_v1;
+  return entry == 0;
+}
+"""
+    def run(tag, include_dir, header):
+        src = tmp_path / f"bridge_{tag}.c"
+        src.write_text(probe)
+        obj = tmp_path / f"bridge_{tag}.o"
+        # compile only: the prototype must accept the assignment; the numbers come from a second, linkable program
+        subprocess.run(["gcc", "-c", "-I", include_dir, f'-DHEADER="{header}"', str(src), "-o", str(obj)], check=True)
+        src2 = tmp_path / f"bridge_{tag}_sizes.c"
+        src2.write_text(probe.replace("vecops_operator_bridge_invoke_v1;", "0;").replace("return entry == 0;", "return entry != 0;"))
+        exe = tmp_path / f"bridge_{tag}_sizes"
+        subprocess.run(["gcc", "-I", include_dir, f'-DHEADER="{header}"', str(src2), "-o", str(exe)], check=True)
+        return subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    ours = run("ours", os.path.join(ROOT, "vecops_amd", "host", "include"), "vecops_rt/abi.h")
+    sizes = [int(v) for v in ours.split()]
+    assert sizes[0] == C.sizeof(H.SpecializationArgument) and sizes[3] == H.SpecializationArgument.value.offset
+    assert sizes[4] == C.sizeof(H.Call) and sizes[5:] == [1, 2]
+    if os.path.isdir("/root/reference/include/vecops/runtime"):
+        assert ours == run("ref", "/root/reference/include", "vecops/runtime/OperatorBridgeAbi.h")
+
+
+def test_bridge_entry_validates_handles_and_records(host):
+    """vecops_operator_bridge_invoke_v1 without a GPU: unknown and stale handles, malformed records and schema errors
+    come back as status codes with the message in the caller's VecopsError (python/bindings/module.cpp:1223-1239)."""
+    op = host.operator("vecops::matmul")
+    a, b, c = bf16((4, 8)), bf16((5, 8)), np.zeros((4, 5), np.float32)
+    frame = H.Frame([a, b, None, c], outputs=(3,))
+    with pytest.raises(H.HostError) as e:
+        op.bridge_invoke(frame, handle=987654321)
+    assert e.value.code == 1 and "handle" in e.value.message
+    handle = op.bridge_handle()
+    assert handle != 0 and op.bridge_handle() == handle
+    with pytest.raises(H.HostError) as e:                      # K differs: the schema's relation validator, through the bridge
+        op.bridge_invoke(H.Frame([a, bf16((5, 9)), None, c], outputs=(3,)))
+    assert e.value.code == 1 and "K" in e.value.message
+    with pytest.raises(H.HostError) as e:                      # an unknown specialization kind
+        sp = (H.SpecializationArgument * 1)()
+        sp[0].struct_size, sp[0].kind, sp[0].name = C.sizeof(H.SpecializationArgument), 7, b"ComputeType"
+        call = H.Call(C.sizeof(H.Call), len(frame.values), C.cast(frame.values, C.c_void_p), None, 0, None)
+        msg = C.create_string_buffer(256)
+        err = H.Error(C.sizeof(H.Error), 0, C.cast(msg, C.c_void_p), 256, 0)
+        rc = host.lib.vecops_operator_bridge_invoke_v1(handle, C.byref(call), 1, sp, C.byref(err))
+        assert rc == 1 and err.code == 1 and err.message_required == len(msg.value) + 1
+        raise H.HostError(rc, msg.value.decode())
+    assert "specialization" in e.value.message
+    short = H.Call(8, 0, None, None, 0, None)                   # a call record shorter than the ABI's
+    assert host.lib.vecops_operator_bridge_invoke_v1(handle, C.byref(short), 0, None, None) == 1
+    # a handle dies with its registration and is never handed out again
+    host.lib.vecops_hip_host_bridge_unregister(handle)
+    with pytest.raises(H.HostError) as e:
+        op.bridge_invoke(frame, handle=handle)
+    assert e.value.code == 1
+    op._bridge = 0
+    assert op.bridge_handle() > handle

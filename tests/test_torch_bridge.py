@@ -194,3 +194,87 @@ def test_torch_ops_host_tensors_are_staged(device):
     c = torch.zeros(33, 47)
     ns.matmul(a, b, None, c, ComputeType=torch.float32)
     assert (c.double() - a.double() @ b.double().T).abs().max() < 1e-4
+
+
+@pytest.mark.gpu
+def test_bridge_entry_on_device_tensors_with_its_own_scratch(device, oracle):
+    """vecops_operator_bridge_invoke_v1 called directly (what a generated extension does): device tensors, no workspace
+    in the call record - the bridge supplies the split-K scratch from its per-thread buffer - against the oracle; a
+    caller-supplied workspace and the stream-ordered flag give the same bits."""
+    host = H.HostLibrary()
+    op = host.operator("vecops::matmul")
+    for m, n, k in ((255, 63, 8191), (64, 48, 4099), (300, 260, 1000)):
+        a, b = synth.bf16_round(synth.uniform_pm1(1, (m, k))), synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+        ta = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+        tb_ = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want, acc_f64=True)
+        c = torch.full((m, n), float("nan"), device=device)
+        frame = H.Frame([ta, tb_, None, c], outputs=(3,))
+        torch.cuda.synchronize()
+        op.bridge_invoke(frame)                                       # synchronous: the result is there on return
+        got = c.cpu().numpy()
+        assert np.max(np.abs(got - want) / np.maximum(1.0, np.abs(want))) <= 2e-6 * max(1.0, k / 32)
+        need = op.workspace(frame)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+        c2 = torch.full((m, n), float("nan"), device=device)
+        stream = torch.cuda.current_stream().cuda_stream
+        op.bridge_invoke(H.Frame([ta, tb_, None, c2], outputs=(3,)), workspace=ws.data_ptr(), workspace_size=need,
+                         stream=stream, stream_ordered=True)
+        c3 = torch.full((m, n), float("nan"), device=device)
+        op.bridge_invoke(H.Frame([ta, tb_, None, c3], outputs=(3,)), stream=stream, stream_ordered=True)   # bridge scratch: waits
+        assert np.array_equal(c3.cpu().numpy(), got)
+        torch.cuda.synchronize()
+        assert np.array_equal(c2.cpu().numpy(), got)
+    with pytest.raises(H.HostError) as e:                             # a workspace that is too small is refused, not used
+        op.bridge_invoke(H.Frame([ta, tb_, None, c], outputs=(3,)), workspace=ws.data_ptr(), workspace_size=0)
+    assert e.value.code != 0
+
+
+@pytest.mark.gpu
+def test_torch_ops_concurrent_callers_compile_and_the_oracle(device, oracle):
+    """Callers on several host threads (python/tests/test_torch.py:125-134 of vecops), the operator inside a
+    torch.compile'd function (:146-152), and - unlike the comparison with this library's own C ABI - every result
+    against the CPU oracle."""
+    from concurrent.futures import ThreadPoolExecutor
+    ns = tb.register_all("vecops_hip_t")
+    m, n, k = 200, 136, 520
+    b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+    tb_ = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
+
+    def expected(a):
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want, acc_f64=True)
+        return want
+
+    inputs = [synth.bf16_round(synth.uniform_pm1(10 + i, (m, k))) for i in range(4)]
+
+    def threaded_call(i):
+        ta = torch.from_numpy(inputs[i].view(np.int16)).to(device).view(torch.bfloat16)
+        out = torch.full((m, n), float("nan"), device=device)
+        for _ in range(5):
+            ns.matmul(ta, tb_, None, out)
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    with ThreadPoolExecutor(max_workers=4) as executor:
+        results = list(executor.map(threaded_call, range(4)))
+    for i, got in enumerate(results):
+        want = expected(inputs[i])
+        assert np.max(np.abs(got - want) / np.maximum(1.0, np.abs(want))) <= 2e-6 * max(1.0, k / 32), i
+
+    ta = torch.from_numpy(inputs[0].view(np.int16)).to(device).view(torch.bfloat16)
+
+    def compiled_call(x, w, destination):
+        torch.ops.vecops_hip_t.matmul(x, w, None, destination)
+        return destination
+
+    compiled = torch.compile(compiled_call, backend="eager", fullgraph=True)
+    out = torch.full((m, n), float("nan"), device=device)
+    assert compiled(ta, tb_, out) is out
+    torch.cuda.synchronize()
+    want = expected(inputs[0])
+    assert np.max(np.abs(out.cpu().numpy() - want) / np.maximum(1.0, np.abs(want))) <= 2e-6 * max(1.0, k / 32)
+    # fake-tensor propagation of the registered operator (schema, Meta kernel, aliasing of the output)
+    torch.library.opcheck(torch.ops.vecops_hip_t.matmul.default, (ta, tb_, None, torch.empty(m, n, device=device)),
+                          test_utils=("test_schema", "test_faketensor"))

@@ -200,7 +200,9 @@ def matmul(a, b, c, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None
 
     Mirrors ``ops::matmul(config)(workspace, m, n, k, A, B[, Cin], C)``: the caller
     allocates the output; a workspace tensor is allocated here when the plan needs
-    one and none is passed.
+    one and none is passed.  Such a workspace comes from torch's allocator, which orders its reuse on torch's CURRENT
+    stream: pass ``stream`` only when it is that stream (the default), or pass a workspace of your own that outlives
+    the work on the stream you name.
     """
     import torch
     plan = plan_matmul(a, b, c, c_in, compute)

@@ -207,11 +207,21 @@ int32_t device_address(const VecopsTensorView* t, bool is_output, Staging* stagi
 #endif
 }
 
-int32_t finish(Staging* staging, hipStream_t stream, VecopsError* error) {
+// Embedding flag of the execution context (vecops: "embedding-defined flags", runtime/CallAbi.h:369-370): the caller
+// orders its own work on context->stream, so a device-memory artifact returns once its kernels are enqueued
+// instead of waiting for them (the default: ABI functions are synchronous, runtime/CallAbi.h:15-16).
+bool stream_ordered(const VecopsCall* call) {
+  const VecopsExecutionContext* ctx = call->context;
+  return ctx != nullptr && ctx->struct_size >= offsetof(VecopsExecutionContext, flags) + sizeof(uint64_t) &&
+         (ctx->flags & VECOPS_HIP_CONTEXT_STREAM_ORDERED) != 0;
+}
+
+int32_t finish(const VecopsCall* call, Staging* staging, hipStream_t stream, VecopsError* error) {
 #if VECOPS_ARTIFACT_DEVICE
   (void)staging;
-  hipError_t e = hipStreamSynchronize(stream);
+  hipError_t e = stream_ordered(call) ? hipSuccess : hipStreamSynchronize(stream);
 #else
+  (void)call;
   (void)stream;
   hipError_t e = staging->finish();
 #endif
@@ -370,7 +380,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
   int32_t rc = vecops_hip_matmul_family(&ops[0], &ops[1], has_cin ? &ops[2] : nullptr, &ops[3], COMPUTE_CODE,
                                         &kFamilyRequest, ws, ws_size, stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
-  return finish(&staging, stream, error);
+  return finish(call, &staging, stream, error);
 }
 
 // =================================================================================================
@@ -463,7 +473,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
                                     static_cast<const int32_t*>(corr), static_cast<float*>(c), d.c->strides[0], d.m,
                                     d.n, d.k, ws, ws_size, stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
-  return finish(&staging, stream, error);
+  return finish(call, &staging, stream, error);
 }
 
 // =================================================================================================
@@ -641,7 +651,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
   int32_t rc = vecops_hip_matmul_fused(&f.ops[0], &f.ops[1], f.cin ? &f.ops[2] : nullptr, &f.ops[3],
                                        VECOPS_HIP_COMPUTE_BF16, &f.ep, ws, ws_size, stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
-  return finish(&staging, stream, error);
+  return finish(call, &staging, stream, error);
 }
 
 // =================================================================================================
@@ -716,7 +726,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
   else
     rc = vecops_hip_pack_b(&ob, p_dev, static_cast<uint64_t>(packed->sizes[0]), stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
-  return finish(&staging, stream, error);
+  return finish(call, &staging, stream, error);
 }
 
 // =================================================================================================
@@ -837,7 +847,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
   rc = vecops_hip_matmul_packed_b(&d.oa, packed_dev, kPackedDtype, d.n, d.cin ? &d.ocin : nullptr, &d.oc, ws, ws_size,
                                   stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
-  return finish(&staging, stream, error);
+  return finish(call, &staging, stream, error);
 }
 
 // =================================================================================================
@@ -940,7 +950,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
                                        static_cast<const int32_t*>(corr), static_cast<const float*>(rs),
                                        static_cast<const float*>(cs), &d.oc, ws, ws_size, stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
-  return finish(&staging, stream, error);
+  return finish(call, &staging, stream, error);
 }
 
 // =================================================================================================
@@ -996,7 +1006,7 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
   rc = vecops_hip_matmul_w8a16_group(dx, x->strides[0], static_cast<const int8_t*>(dw), w->strides[0],
                                      static_cast<const float*>(ds), dy, y->strides[0], m, n, k, g, stream);
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
-  return finish(&staging, stream, error);
+  return finish(call, &staging, stream, error);
 }
 
 #endif

@@ -204,6 +204,32 @@ typedef const VecopsKernelDescriptorV1* (*VecopsKernelQueryFnV1)(void);
 /* The one symbol an artifact DSO exports. */
 VECOPS_RUNTIME_EXPORT const VecopsKernelDescriptorV1* vecops_kernel_query_v1(void);
 
+/* ---- process-local operator bridge (vecops runtime/OperatorBridgeAbi.h:29-71) --------- */
+/* A framework extension enters an Operator it knows by handle; the records are vecops' own. */
+
+#define VECOPS_OPERATOR_BRIDGE_ABI_VERSION_MAJOR 1u
+#define VECOPS_OPERATOR_BRIDGE_ABI_VERSION_MINOR 0u
+
+typedef enum VecopsSpecializationValueKind {
+  VECOPS_SPECIALIZATION_CONST_INT = 1,
+  VECOPS_SPECIALIZATION_DTYPE = 2
+} VecopsSpecializationValueKind;
+
+typedef struct VecopsSpecializationArgument {
+  uint32_t struct_size;
+  uint32_t kind;      /* VecopsSpecializationValueKind */
+  const char* name;   /* caller-owned, nul-terminated */
+  union {
+    int64_t integer;  /* CONST_INT */
+    uint32_t dtype;   /* DTYPE: a VecopsDType number */
+  } value;
+} VecopsSpecializationArgument;
+
+VECOPS_RUNTIME_EXPORT int32_t vecops_operator_bridge_invoke_v1(uint64_t handle, const VecopsCall* call,
+                                                               uint32_t num_specialization_values,
+                                                               const VecopsSpecializationArgument* specialization_values,
+                                                               VecopsError* error);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,6 +8,7 @@
 #include "vecops/runtime/Executable.h"
 #include "vecops/runtime/KernelDefinition.h"
 #include "vecops/runtime/Operator.h"
+#include "vecops/runtime/OperatorBridgeAbi.h"
 #include "vecops/runtime/Schema.h"
 #include "vecops/runtime/Status.h"
 #else

@@ -1,8 +1,14 @@
 // C entry points over the Operator objects of the HIP drop-in (include/vecops_hip_host.h).
 #include "vecops_hip_host.h"
 
+#include <dlfcn.h>
+
+#include <atomic>
+#include <cstddef>
 #include <cstring>
+#include <mutex>
 #include <string>
+#include <unordered_map>
 
 #include "../hip/matmul_plugin.hpp"
 
@@ -60,9 +66,151 @@ rt::KernelCall make_call(const VecopsValue* values, uint32_t n, const VecopsHost
   return rt::KernelCall(rt::ArgumentMetadata(std::move(erased)), std::move(sv));
 }
 
+// ---- the process-local bridge (vecops runtime/OperatorBridgeAbi.h) ---------------------------------------------
+// Handles are small integers that stay invalid after unregistration (never reused), so a stale handle held by a
+// framework extension is refused rather than served by another operator.
+std::mutex g_bridge_mutex;
+std::unordered_map<std::uint64_t, std::shared_ptr<rt::Operator>> g_bridge_operators;
+std::atomic<std::uint64_t> g_next_handle{1};
+
+// Device workspace of bridge calls that bring none: one buffer per host thread and device, grown on demand and kept
+// (a bridge call is synchronous, so a thread never has two calls using its buffer).  The HIP runtime is looked up at
+// the first need - this library itself does not link it.
+struct HipRuntime {
+  int (*get_device)(int*) = nullptr;
+  int (*malloc_)(void**, size_t) = nullptr;
+  int (*free_)(void*) = nullptr;
+  bool ok = false;
+};
+const HipRuntime& hip_runtime() {
+  static const HipRuntime runtime = [] {
+    HipRuntime r;
+    void* lib = dlopen("libamdhip64.so", RTLD_NOW | RTLD_GLOBAL);
+    if (lib == nullptr) lib = dlopen("/opt/rocm/lib/libamdhip64.so", RTLD_NOW | RTLD_GLOBAL);
+    if (lib == nullptr) return r;
+    r.get_device = reinterpret_cast<int (*)(int*)>(dlsym(lib, "hipGetDevice"));
+    r.malloc_ = reinterpret_cast<int (*)(void**, size_t)>(dlsym(lib, "hipMalloc"));
+    r.free_ = reinterpret_cast<int (*)(void*)>(dlsym(lib, "hipFree"));
+    r.ok = r.get_device != nullptr && r.malloc_ != nullptr && r.free_ != nullptr;
+    return r;
+  }();
+  return runtime;
+}
+struct ThreadWorkspace {
+  static constexpr int kDevices = 64;
+  void* buffer[kDevices] = {};
+  std::uint64_t size[kDevices] = {};
+  ~ThreadWorkspace() {
+    for (int d = 0; d < kDevices; ++d)
+      if (buffer[d] != nullptr) hip_runtime().free_(buffer[d]);
+  }
+  rt::Status get(std::uint64_t bytes, void** out) {
+    const HipRuntime& hip = hip_runtime();
+    if (!hip.ok) return rt::Status(rt::StatusCode::ExecutionError, "bridge workspace: the HIP runtime is not available");
+    int device = 0;
+    if (hip.get_device(&device) != 0 || device < 0 || device >= kDevices)
+      return rt::Status(rt::StatusCode::ExecutionError, "bridge workspace: no current HIP device");
+    if (size[device] < bytes) {
+      if (buffer[device] != nullptr) hip.free_(buffer[device]);
+      buffer[device] = nullptr;
+      size[device] = 0;
+      const std::uint64_t want = (bytes + (std::uint64_t{1} << 20) - 1) & ~((std::uint64_t{1} << 20) - 1);
+      if (hip.malloc_(&buffer[device], want) != 0)
+        return rt::Status(rt::StatusCode::ExecutionError, "bridge workspace: device allocation of " + std::to_string(want) + " bytes failed");
+      size[device] = want;
+    }
+    *out = buffer[device];
+    return rt::Status::success();
+  }
+};
+
+rt::Status bridge_invoke(std::uint64_t handle, const VecopsCall* call, std::uint32_t num_specs,
+                         const VecopsSpecializationArgument* specs) {
+  if (call == nullptr || call->struct_size < sizeof(VecopsCall))
+    return rt::Status(rt::StatusCode::InvalidArgument, "bridge call record is missing or too short");
+  if (call->num_values != 0 && call->values == nullptr)
+    return rt::Status(rt::StatusCode::InvalidArgument, "bridge call has values but no array");
+  if (num_specs != 0 && specs == nullptr)
+    return rt::Status(rt::StatusCode::InvalidArgument, "bridge call has specialization values but no array");
+  std::shared_ptr<rt::Operator> op;
+  {
+    std::lock_guard<std::mutex> lock(g_bridge_mutex);
+    auto it = g_bridge_operators.find(handle);
+    if (it != g_bridge_operators.end()) op = it->second;  // the call keeps the operator alive
+  }
+  if (op == nullptr) return rt::Status(rt::StatusCode::InvalidArgument, "bridge handle " + std::to_string(handle) + " names no operator");
+  std::vector<VecopsHostSpecialization> converted(num_specs);
+  for (std::uint32_t i = 0; i < num_specs; ++i) {
+    const VecopsSpecializationArgument& a = specs[i];
+    if (a.struct_size < sizeof(VecopsSpecializationArgument) || a.name == nullptr)
+      return rt::Status(rt::StatusCode::InvalidArgument, "malformed specialization argument");
+    if (a.kind == VECOPS_SPECIALIZATION_CONST_INT) converted[i] = {a.name, 0, a.value.integer};
+    else if (a.kind == VECOPS_SPECIALIZATION_DTYPE) converted[i] = {a.name, 1, static_cast<std::int64_t>(a.value.dtype)};
+    else return rt::Status(rt::StatusCode::InvalidArgument, "unknown specialization value kind");
+  }
+  const rt::KernelCall kernel_call = make_call(call->values, call->num_values, converted.data(), num_specs);
+  void* workspace = call->workspace;
+  std::uint64_t workspace_size = call->workspace_size;
+  if (workspace == nullptr) {
+    // the bridge owns the scratch of calls that bring none (vecops allocates a host Workspace here,
+    // python/bindings/module.cpp:1186-1203; device tensors need device memory)
+    auto executable = op->resolve(kernel_call, call->context);
+    if (!executable) return executable.status();
+    auto need = executable.value()->workspace_size(kernel_call.arguments(), call->context);
+    if (!need) return need.status();
+    workspace_size = need.value();
+    if (workspace_size != 0) {
+      thread_local ThreadWorkspace cache;
+      if (rt::Status st = cache.get(workspace_size, &workspace); !st.ok()) return st;
+      // the thread's buffer serves its next call too: this one has to be over on return, whatever the caller's
+      // context says about stream order (bit 0 of flags: VECOPS_HIP_CONTEXT_STREAM_ORDERED)
+      if (call->context != nullptr && call->context->struct_size >= offsetof(VecopsExecutionContext, flags) + sizeof(std::uint64_t) &&
+          (call->context->flags & 1u) != 0) {
+        VecopsExecutionContext waiting;
+        memset(&waiting, 0, sizeof(waiting));
+        memcpy(&waiting, call->context, call->context->struct_size < sizeof(waiting) ? call->context->struct_size : sizeof(waiting));
+        waiting.flags &= ~std::uint64_t{1};
+        return op->invoke(kernel_call, &waiting, workspace, workspace_size);
+      }
+    }
+  }
+  return op->invoke(kernel_call, call->context, workspace, workspace_size);
+}
+
 }  // namespace
 
 extern "C" {
+
+uint64_t vecops_hip_host_bridge_register(void* op) {
+  auto* h = static_cast<Handle*>(op);
+  if (h == nullptr || h->op == nullptr) return 0;
+  const std::uint64_t handle = g_next_handle.fetch_add(1);
+  std::lock_guard<std::mutex> lock(g_bridge_mutex);
+  g_bridge_operators.emplace(handle, h->op);
+  return handle;
+}
+
+void vecops_hip_host_bridge_unregister(uint64_t handle) {
+  std::lock_guard<std::mutex> lock(g_bridge_mutex);
+  g_bridge_operators.erase(handle);
+}
+
+int32_t vecops_operator_bridge_invoke_v1(uint64_t handle, const VecopsCall* call, uint32_t num_specialization_values,
+                                         const VecopsSpecializationArgument* specialization_values, VecopsError* error) {
+  const rt::Status result = bridge_invoke(handle, call, num_specialization_values, specialization_values);
+  if (result.ok()) return VECOPS_STATUS_OK;
+  if (error != nullptr && error->struct_size >= sizeof(VecopsError)) {
+    const std::string_view message = result.message();
+    error->code = static_cast<std::int32_t>(result.code());
+    error->message_required = message.size() + 1;
+    if (error->message != nullptr && error->message_capacity != 0) {
+      const size_t copied = message.size() < error->message_capacity - 1 ? message.size() : error->message_capacity - 1;
+      memcpy(error->message, message.data(), copied);
+      error->message[copied] = '\0';
+    }
+  }
+  return static_cast<std::int32_t>(result.code());
+}
 
 void* vecops_hip_host_operator_create(const char* operator_name, const char* artifact_directory) {
   if (operator_name == nullptr || artifact_directory == nullptr) return nullptr;

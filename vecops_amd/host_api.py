@@ -60,6 +60,27 @@ _NP_CODES = {np.dtype(np.int8): I8, np.dtype(np.uint8): U8, np.dtype(np.int32): 
              np.dtype(np.float16): F16}
 
 
+class SpecializationValue(C.Union):
+    _fields_ = [("integer", C.c_int64), ("dtype", C.c_uint32)]
+
+
+class SpecializationArgument(C.Structure):
+    """VecopsSpecializationArgument of the process-local bridge (vecops runtime/OperatorBridgeAbi.h:44-57)."""
+    _fields_ = [("struct_size", C.c_uint32), ("kind", C.c_uint32), ("name", C.c_char_p), ("value", SpecializationValue)]
+
+
+class Call(C.Structure):
+    """VecopsCall (vecops runtime/CallAbi.h): the positional values, the caller's workspace, the context."""
+    _fields_ = [("struct_size", C.c_uint32), ("num_values", C.c_uint32), ("values", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_size", C.c_uint64), ("context", C.c_void_p)]
+
+
+class Error(C.Structure):
+    """VecopsError: code and a caller-owned message buffer."""
+    _fields_ = [("struct_size", C.c_uint32), ("code", C.c_int32), ("message", C.c_void_p),
+                ("message_capacity", C.c_size_t), ("message_required", C.c_size_t)]
+
+
 class Frame:
     """Positional VecopsValue records for one call; keeps the size/stride arrays alive."""
 
@@ -109,6 +130,10 @@ class Frame:
             t.sizes, t.strides = sizes, strd
 
 
+# VECOPS_HIP_CONTEXT_STREAM_ORDERED: device-memory artifacts return once their kernels are enqueued on the stream
+CONTEXT_STREAM_ORDERED = 1
+
+
 class HostError(RuntimeError):
     def __init__(self, code, message):
         super().__init__(f"status {code}: {message}")
@@ -131,6 +156,11 @@ class HostLibrary:
                                                               C.c_char_p, C.c_size_t]
         L.vecops_hip_host_load_artifact.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t,
                                                     C.c_char_p, C.c_size_t]
+        L.vecops_hip_host_bridge_register.restype = C.c_uint64
+        L.vecops_hip_host_bridge_register.argtypes = [C.c_void_p]
+        L.vecops_hip_host_bridge_unregister.argtypes = [C.c_uint64]
+        L.vecops_operator_bridge_invoke_v1.argtypes = [C.c_uint64, C.POINTER(Call), C.c_uint32,
+                                                       C.POINTER(SpecializationArgument), C.POINTER(Error)]
 
     def flavor(self) -> str:
         return self.lib.vecops_hip_host_runtime_flavor().decode()
@@ -147,6 +177,19 @@ class HostLibrary:
         if rc != 0:
             raise HostError(rc, msg.value.decode())
         return name.value.decode(), key.value.decode()
+
+
+def _bridge_specs(specializations):
+    items = list((specializations or {}).items())
+    arr = (SpecializationArgument * max(1, len(items)))()
+    for i, (k, v) in enumerate(items):
+        arr[i].struct_size = C.sizeof(SpecializationArgument)
+        arr[i].name = k.encode()
+        if isinstance(v, tuple):        # ("dtype", code)
+            arr[i].kind, arr[i].value.dtype = 2, v[1]
+        else:
+            arr[i].kind, arr[i].value.integer = 1, int(v)
+    return arr, len(items)
 
 
 def _specs(specializations):
@@ -167,9 +210,37 @@ class HostOperator:
 
     def __del__(self):
         try:
+            if getattr(self, "_bridge", 0):
+                self._lib.lib.vecops_hip_host_bridge_unregister(self._bridge)
             self._lib.lib.vecops_hip_host_operator_destroy(self._h)
         except Exception:
             pass
+
+    def bridge_handle(self) -> int:
+        """Registers the operator with the process-local bridge (once) and returns its handle."""
+        if not getattr(self, "_bridge", 0):
+            self._bridge = self._lib.lib.vecops_hip_host_bridge_register(self._h)
+            if not self._bridge:
+                raise RuntimeError("bridge registration failed")
+        return self._bridge
+
+    def bridge_invoke(self, frame: Frame, specializations=None, workspace=None, workspace_size=0, stream=None,
+                      handle=None, stream_ordered=False):
+        """One foreign call through vecops_operator_bridge_invoke_v1: validation, dispatch, resolution, workspace
+        (the bridge's own scratch when none is given) and the artifact's run callback, synchronous."""
+        ctx = ExecutionContext()
+        ctx.struct_size = C.sizeof(ExecutionContext)
+        ctx.stream = stream
+        ctx.flags = CONTEXT_STREAM_ORDERED if stream_ordered else 0
+        call = Call(C.sizeof(Call), len(frame.values), C.cast(frame.values, C.c_void_p), workspace, workspace_size,
+                    C.cast(C.pointer(ctx), C.c_void_p))
+        msg = C.create_string_buffer(1024)
+        err = Error(C.sizeof(Error), 0, C.cast(msg, C.c_void_p), 1024, 0)
+        sp, n = _bridge_specs(specializations)
+        rc = self._lib.lib.vecops_operator_bridge_invoke_v1(self.bridge_handle() if handle is None else handle,
+                                                            C.byref(call), n, sp, C.byref(err))
+        if rc != 0:
+            raise HostError(rc, msg.value.decode())
 
     def resolve(self, frame: Frame, specializations=None) -> str:
         key, msg = C.create_string_buffer(512), C.create_string_buffer(1024)
@@ -189,12 +260,14 @@ class HostOperator:
             raise HostError(rc, msg.value.decode())
         return size.value
 
-    def invoke(self, frame: Frame, specializations=None, workspace=None, workspace_size=0, stream=None):
+    def invoke(self, frame: Frame, specializations=None, workspace=None, workspace_size=0, stream=None,
+               stream_ordered=False):
         msg = C.create_string_buffer(1024)
         sp, n = _specs(specializations)
         ctx = ExecutionContext()
         ctx.struct_size = C.sizeof(ExecutionContext)
         ctx.stream = stream
+        ctx.flags = CONTEXT_STREAM_ORDERED if stream_ordered else 0
         rc = self._lib.lib.vecops_hip_host_operator_invoke(self._h, frame.values, len(frame.values), sp, n, workspace,
                                                            workspace_size, C.byref(ctx), msg, 1024)
         if rc != 0:

@@ -8,7 +8,10 @@ and returns a public callable that, unlike the raw ``torch.ops`` symbol, accepts
 specialization values and gives back the caller's own output tensors.  Tensors on a ROCm
 device ("cuda" in torch) enter the operator as ``VECOPS_DEVICE_PRIVATE`` views and run on
 ``torch.cuda.current_stream()``; host tensors enter as ``VECOPS_DEVICE_CPU`` views and are
-staged by the artifact.  Device workspace comes from torch's allocator.  Like the
+staged by the artifact.  Device workspace comes from torch's allocator; calls whose tensors all live on the device are
+stream-ordered (they return once enqueued on the current stream), calls with host tensors wait for their results.
+Every call enters the Operator through the native bridge entry ``vecops_operator_bridge_invoke_v1``
+(runtime/OperatorBridgeAbi.h:69-71) of libvecops_hip_host.so.  Like the
 reference's process-local bridge (docs/Runtime.md:196-206) the wrapper keeps up to eight
 call signatures per thread - tensor kind, dtype, device, shape, strides, optional
 presence and specialization values, never addresses or scalar payloads - and reuses the
@@ -137,7 +140,11 @@ class _Registration:
             if need:
                 scratch = torch.empty(need, dtype=torch.uint8, device=device)
                 workspace, workspace_size = scratch.data_ptr(), need
-        self.operator.invoke(frame, specs, workspace=workspace, workspace_size=workspace_size, stream=stream)
+        # One foreign call through the process-local bridge entry (vecops_operator_bridge_invoke_v1); ctypes drops the
+        # interpreter lock for its duration.  Device tensors: the work is ordered on torch's current stream, where
+        # the scratch was allocated, so the call returns once the kernels are enqueued.
+        self.operator.bridge_invoke(frame, specs, workspace=workspace, workspace_size=workspace_size, stream=stream,
+                                    stream_ordered=on_device and not any(not t.is_cuda for t in tensors))
         if self.return_outputs:
             outs = tuple(values[i] for i in self.outputs)
             return outs
