@@ -153,8 +153,9 @@ def bench_bf16_gemm(dev, steps, warmup):
     a, b_kn, ta, tb = _bf16_operands(dev)
     tb_view = tb.t()                      # [N,K] view with strides (1, N): vecops' way to pass B[K,N]
     c = torch.empty((n, n), dtype=torch.bfloat16, device=dev)
-    plan = capi.plan_matmul(ta, tb_view, c)
-    t = _measure(lambda i: capi.matmul(ta, tb_view, c), steps, warmup)
+    run = capi.PreparedMatmul(ta, tb_view, c)       # descriptors and plan built once: a step is one call of the C ABI
+    plan = run.plan
+    t = _measure(lambda i: run(), steps, warmup)
     flops = 2.0 * n * n * n
     tflops = flops / (t["event_ms"] * 1e-3) / 1e12
     return {
@@ -481,8 +482,8 @@ ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_q
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", choices=ONLY, help="run a single workload (for profiling)")
     ap.add_argument("--gemv-m", type=int, default=1, help="activation rows of the --only gemv workload (1..16)")
@@ -545,7 +546,7 @@ def main() -> int:
         line["secondary"] += [bench_batched(dev, K, W, m, n, k)
                               for (m, n, k) in [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)]]
         line["secondary"] += [bench_bf16_gemm_packed(dev, K, W), bench_int8_dequant_packed(dev, K, W),
-                              bench_runtime_quant(dev, K, W), ceiling_bf16, ceiling_int8]
+                              bench_runtime_quant(dev, K, W), bench_grouped(dev, K, W), ceiling_bf16, ceiling_int8]
     if not args.no_cpu and args.only is None:
         line["cpu_baseline"] = cpu_baseline(a, b_kn)
     print(json.dumps(line))

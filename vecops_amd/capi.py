@@ -218,6 +218,34 @@ def matmul(a, b, c, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None
     return c
 
 
+class PreparedMatmul:
+    """``matmul`` on fixed operands with everything but the launch done once: the descriptors, the plan and the
+    workspace are built here, a call is one foreign call (the counterpart of vecops' prepared invocation,
+    ``ops::matmul(config).prepare(...)`` / docs/Runtime.md:196-206).  The tensors must stay alive and in place; the
+    stream is the one that was current at preparation unless ``stream`` is given."""
+
+    def __init__(self, a, b, c, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None):
+        import torch
+        self.plan = plan_matmul(a, b, c, c_in, compute)
+        need = int(self.plan.workspace_bytes)
+        if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+            workspace = torch.empty(need, dtype=torch.uint8, device=c.device)
+        self._keep = (a, b, c, c_in, workspace)
+        self._oa, self._ob, self._oc = operand(a), operand(b), operand(c)
+        self._oi = operand(c_in) if c_in is not None else None
+        ws_ptr = workspace.data_ptr() if workspace is not None else None
+        ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+        self._args = (C.byref(self._oa), C.byref(self._ob), C.byref(self._oi) if self._oi is not None else None,
+                      C.byref(self._oc), compute, ws_ptr, ws_size, _stream_handle(stream))
+        self._fn = lib().vecops_hip_matmul
+
+    def __call__(self):
+        rc = self._fn(*self._args)
+        if rc != 0:
+            _check(rc)
+        return self._keep[2]
+
+
 def plan_matmul_family(a, b, c, request: FamilyRequest, c_in=None, compute=COMPUTE_BF16) -> Plan:
     plan = Plan()
     oa, ob, oc = operand(a), operand(b), operand(c)

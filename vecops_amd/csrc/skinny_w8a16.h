@@ -150,12 +150,29 @@ __global__ __launch_bounds__(256) void skinny_w8a16_stream_kernel(const SkinnyW8
   const VECOPS_GLOBAL uint16_t* xbase = (const VECOPS_GLOBAL uint16_t*)p.x;
   const VECOPS_GLOBAL float* sbase = (const VECOPS_GLOBAL float*)p.scales;
 
-  float xf[CH][16], xsum[CH];
   int group_of[CH];
+#pragma unroll
+  for (int u = 0; u < CH; ++u) group_of[u] = ((u * 64 + lane) << 4) / p.group;
+
+  u32x4 wq[2][CH];
+  float sc[2][CH];
+  auto fetch = [&](int set, int64_t n) {
+    // rows past N are clamped: computed, never stored
+    const int64_t row = n < p.n ? n : p.n - 1;
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      wq[set][u] = *(const VECOPS_GLOBAL u32x4*)(wbase + row * p.ldw + (static_cast<int64_t>(u * 64 + lane) << 4));
+      sc[set][u] = sbase[row * p.groups + group_of[u]];
+    }
+  };
+  if (wave >= p.n) return;
+  // the first row's weights are requested before the activations: they arrive while those are fetched and widened
+  fetch(0, wave);
+
+  float xf[CH][16], xsum[CH];
 #pragma unroll
   for (int u = 0; u < CH; ++u) {
     const int k0 = (u * 64 + lane) << 4;
-    group_of[u] = k0 / p.group;
     const VECOPS_GLOBAL u32x4* px = (const VECOPS_GLOBAL u32x4*)(xbase + k0);
     const u32x4 lo = px[0], hi = px[1];
     const uint32_t words[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
@@ -170,17 +187,6 @@ __global__ __launch_bounds__(256) void skinny_w8a16_stream_kernel(const SkinnyW8
     xsum[u] = s;
   }
 
-  u32x4 wq[2][CH];
-  float sc[2][CH];
-  auto fetch = [&](int set, int64_t n) {
-    // rows past N are clamped: computed, never stored
-    const int64_t row = n < p.n ? n : p.n - 1;
-#pragma unroll
-    for (int u = 0; u < CH; ++u) {
-      wq[set][u] = *(const VECOPS_GLOBAL u32x4*)(wbase + row * p.ldw + (static_cast<int64_t>(u * 64 + lane) << 4));
-      sc[set][u] = sbase[row * p.groups + group_of[u]];
-    }
-  };
   auto finish = [&](int set, int64_t n) {
     float acc = 0.0f;
 #pragma unroll
@@ -197,8 +203,6 @@ __global__ __launch_bounds__(256) void skinny_w8a16_stream_kernel(const SkinnyW8
     if (lane == 0 && n < p.n) p.y[n] = static_cast<uint16_t>(bf16_bits_rne(total));
   };
 
-  if (wave >= p.n) return;
-  fetch(0, wave);
   int64_t n = wave;
   // two rows per trip so that the register set of a row is a compile-time choice
   for (; n + waves < p.n; n += 2 * waves) {
