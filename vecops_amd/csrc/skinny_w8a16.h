@@ -468,7 +468,12 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
   const int64_t wg_row0 = static_cast<int64_t>(blockIdx.x) * passes * (16 * TILES);
   const int64_t last_row = static_cast<int64_t>(p.n) - 1;
   const int g_begin = wave * GPW;
-  const VECOPS_GLOBAL char* wbase = (const VECOPS_GLOBAL char*)p.w + quarter * 16 + static_cast<int64_t>(wave) * S * 64;
+  // Weight loads: lanes 4r .. 4r + 3 fetch the four 16-byte quarters of row r's 64-byte step - one contiguous 64-byte
+  // request per group of four lanes instead of four lines touched by it - and a lane permute
+  // puts the quarters where the matrix cores want them (lane i + 16q: row i, quarter q).
+  const int load_row = lane >> 2;
+  const VECOPS_GLOBAL char* wbase = (const VECOPS_GLOBAL char*)p.w + (lane & 3) * 16 + static_cast<int64_t>(wave) * S * 64;
+  const int from_lane_bytes = (4 * row + quarter) * 4;  // ds_bpermute address of the lane that loaded (row, quarter)
   const VECOPS_GLOBAL float* sbase = (const VECOPS_GLOBAL float*)p.scales;
 
   // activation fragments of this K slice, resident for the whole kernel
@@ -496,6 +501,7 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
 
   // rows past N are clamped: computed, never stored
   auto weight_row = [&](int pass, int t) { return min(wg_row0 + (pass * TILES + t) * 16 + row, last_row); };
+  auto loaded_row = [&](int pass, int t) { return min(wg_row0 + (pass * TILES + t) * 16 + load_row, last_row); };
   auto load_scales = [&](float (&dst)[TILES][NSC], int pass) {
 #pragma unroll
     for (int t = 0; t < TILES; ++t)
@@ -512,7 +518,7 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
       const int pass = step / S, s = step - pass * S;
 #pragma unroll
       for (int t = 0; t < TILES; ++t)
-        wq[slot][t] = *(const VECOPS_GLOBAL u32x4*)(wbase + weight_row(pass, t) * p.ldw + s * 64);
+        wq[slot][t] = *(const VECOPS_GLOBAL u32x4*)(wbase + loaded_row(pass, t) * p.ldw + s * 64);
     }
   };
   // S is a multiple of D: slot `slot` always holds step s = slot or slot + D of its pass
@@ -522,8 +528,11 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       uint32_t a[8];
-      const uint32_t wd[4] = {wq[slot][t].x ^ 0x80808080u, wq[slot][t].y ^ 0x80808080u, wq[slot][t].z ^ 0x80808080u,
-                              wq[slot][t].w ^ 0x80808080u};
+      const uint32_t raw[4] = {wq[slot][t].x, wq[slot][t].y, wq[slot][t].z, wq[slot][t].w};
+      uint32_t wd[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        wd[q] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(from_lane_bytes, static_cast<int>(raw[q]))) ^ 0x80808080u;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const float f0 = static_cast<float>(wd[q] & 0xffu), f1 = static_cast<float>((wd[q] >> 8) & 0xffu);
