@@ -112,8 +112,10 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul(const VecopsHipOperand* a, cons
  *   a,b f32  -> c f32|bf16      (bf16 or fp32 compute, see VecopsHipCompute)
  *   a,b i8|u8 -> c i32          (AMX_I8I32<A,B>, either side signed or unsigned;
  *                                accumulators wrap mod 2^32)
+ *   a,b f64  -> c f64           (SME_F64F64, matmul/details/kernel/sme/Atoms.h:108-112; dtype 13; a kernel of its own
+ *                                on v_mfma_f64_16x16x4_f64: family tile_128, K never split, no fused transform)
  * c_in may be null (zero accumulator); otherwise it has c's dtype class (f32,
- * bf16 or i32) and may alias c element for element.  K == 0 writes zeros or
+ * bf16, i32 or f64) and may alias c element for element.  K == 0 writes zeros or
  * C_in; zero M, N or batch writes nothing (ops/Matmul.h:41-43).  Operand
  * metadata is validated as planning/families/ArchitectureFamily.h:1590-1652
  * does.  `workspace` must hold vecops_hip_plan_matmul(...).workspace_bytes.

@@ -20,8 +20,8 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 # VecopsDType numeric values (runtime/CallAbi.h:62-91)
-I8, U8, I32, F16, BF16, F32 = 2, 3, 6, 10, 11, 12
-ATOM_BF16F32, ATOM_F32F32, ATOM_I8I32, ATOM_F16F32 = 0, 1, 2, 3
+I8, U8, I32, F16, BF16, F32, F64 = 2, 3, 6, 10, 11, 12, 13
+ATOM_BF16F32, ATOM_F32F32, ATOM_I8I32, ATOM_F16F32, ATOM_F64F64 = 0, 1, 2, 3, 4
 SHAPE_AMX_BF16, SHAPE_AMX_I8_SAME, SHAPE_AMX_I8_MIXED, SHAPE_SME_F16, SHAPE_SME_OTHER = range(5)
 
 
@@ -33,6 +33,8 @@ class _Tensor(C.Structure):
 def _np_dtype_code(arr: np.ndarray, bf16: bool) -> int:
     if arr.dtype == np.float32:
         return F32
+    if arr.dtype == np.float64:
+        return F64
     if arr.dtype == np.float16:
         return F16
     if arr.dtype == np.uint16:

@@ -43,7 +43,7 @@
 #define VO_EXPORT __attribute__((visibility("default")))
 
 /* dtype codes = VecopsDType numeric values (runtime/CallAbi.h:62-91). */
-enum { VO_I8 = 2, VO_U8 = 3, VO_I32 = 6, VO_F16 = 10, VO_BF16 = 11, VO_F32 = 12 };
+enum { VO_I8 = 2, VO_U8 = 3, VO_I32 = 6, VO_F16 = 10, VO_BF16 = 11, VO_F32 = 12, VO_F64 = 13 };
 
 /* Compute (atom) selection for vo_matmul.
  *   VO_ATOM_BF16F32 : operands rounded to bf16, fp32 accumulate (AMX_BF16F32,
@@ -52,10 +52,12 @@ enum { VO_I8 = 2, VO_U8 = 3, VO_I32 = 6, VO_F16 = 10, VO_BF16 = 11, VO_F32 = 12 
  *   VO_ATOM_F16F32  : operands rounded to IEEE half, fp32 accumulate (AMX_F16F32,
  *                     matmul/details/kernel/amx/Atoms.h:62-71; the reference build needs AMX-FP16,
  *                     which the build host lacks: pinned by closed forms only)
+ *   VO_ATOM_F64F64  : fp64 operands, fp64 accumulate, one fused multiply-add per k in k order (SME_F64F64,
+ *                     kernel/sme/Atoms.h:108-112: FMOPA .d, one fp64 per K step); a, b, cin and c are VO_F64
  *   VO_ATOM_I8I32   : 8-bit integers, int32 accumulate wrapping mod 2^32
  *                     (AMX_I8I32<A,B>, amx/Atoms.h:73-86; wrap pinned by
  *                     tests/ops/MatmulTest.cpp:1025-1055) */
-enum { VO_ATOM_BF16F32 = 0, VO_ATOM_F32F32 = 1, VO_ATOM_I8I32 = 2, VO_ATOM_F16F32 = 3 };
+enum { VO_ATOM_BF16F32 = 0, VO_ATOM_F32F32 = 1, VO_ATOM_I8I32 = 2, VO_ATOM_F16F32 = 3, VO_ATOM_F64F64 = 4 };
 
 typedef struct vo_tensor {
   void* data;
@@ -143,6 +145,7 @@ static inline int64_t elem_size(int dtype) {
   switch (dtype) {
     case VO_I8: case VO_U8: return 1;
     case VO_F16: case VO_BF16: return 2;
+    case VO_F64: return 8;
     default: return 4;
   }
 }
@@ -238,6 +241,9 @@ static int validate(const vo_tensor* a, const vo_tensor* b, const vo_tensor* cin
 VO_EXPORT int vo_matmul(const vo_tensor* a, const vo_tensor* b, const vo_tensor* cin, const vo_tensor* c,
                         int atom, int acc_f64) {
   if (validate(a, b, cin, c)) return 1;
+  if ((atom == VO_ATOM_F64F64) != (a->dtype == VO_F64) || (a->dtype == VO_F64) != (b->dtype == VO_F64) ||
+      (a->dtype == VO_F64) != (c->dtype == VO_F64) || (cin && (cin->dtype == VO_F64) != (c->dtype == VO_F64)))
+    return 1;  /* fp64 operands go with the fp64 atom and nothing else */
   const int64_t batch = a->rank == 3 ? a->sizes[0] : 1;
   const int64_t M = rows(a), N = rows(b), K = cols(a);
   if (batch == 0 || M == 0 || N == 0) return 0;
@@ -247,7 +253,13 @@ VO_EXPORT int vo_matmul(const vo_tensor* a, const vo_tensor* b, const vo_tensor*
     for (int64_t i = 0; i < M; ++i) {
       for (int64_t j = 0; j < N; ++j) {
         const int64_t ci = co + i * rs(c) + j * cs(c);
-        if (atom == VO_ATOM_I8I32) {
+        if (atom == VO_ATOM_F64F64) {
+          double acc = 0.0;
+          for (int64_t k = 0; k < K; ++k)
+            acc = fma(((const double*)a->data)[ao + i * rs(a) + k * cs(a)], ((const double*)b->data)[bo + j * rs(b) + k * cs(b)], acc);
+          if (cin) acc += ((const double*)cin->data)[cio + i * rs(cin) + j * cs(cin)];
+          ((double*)c->data)[ci] = acc;
+        } else if (atom == VO_ATOM_I8I32) {
           uint32_t acc = 0;
           for (int64_t k = 0; k < K; ++k) {
             int32_t x = load_as_i32(a->data, a->dtype, ao + i * rs(a) + k * cs(a));

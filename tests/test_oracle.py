@@ -469,3 +469,51 @@ def test_sampled_product_equals_the_full_product_at_the_sampled_indices(oracle, 
     as_f64 = lambda v: synth.bf16_to_f32(v if v.dtype == np.uint16 else synth.bf16_round(np.ascontiguousarray(v))).astype(np.float64)
     want64 = as_f64(np.ascontiguousarray(a)) @ as_f64(np.ascontiguousarray(b)).T
     assert np.allclose(got, want64[rows, cols], rtol=1e-13, atol=1e-13)
+
+
+def test_f64_atom_is_the_sequential_fused_sum(oracle):
+    """VO_ATOM_F64F64 (vecops' SME_F64F64: fp64 operands and accumulate, one fused multiply-add per k, in k order) pinned
+    by the mathematics: an independent Python loop of math.fma-free exact arithmetic on small cases (fractions), the
+    reordering bound against numpy's product, exactness on integers, C input, strided views, and the rejection of
+    fp64 operands under any other atom."""
+    from fractions import Fraction
+    from oracle import oracle as O
+    m, n, k = 7, 5, 23
+    a = (synth.uniform_pm1(1, (m, k)).astype(np.float64) + synth.uniform_pm1(2, (m, k)).astype(np.float64) * 2.0 ** -30)
+    b = (synth.uniform_pm1(3, (n, k)).astype(np.float64) + synth.uniform_pm1(4, (n, k)).astype(np.float64) * 2.0 ** -30)
+    cin = synth.uniform_pm1(5, (m, n)).astype(np.float64)
+    got = np.zeros((m, n), np.float64)
+    oracle.matmul(a, b, got, atom=O.ATOM_F64F64)
+    # the fused sequential sum, step by step in exact rational arithmetic rounded once per step
+    def fused(x, y, acc):
+        return float(Fraction(x) * Fraction(y) + Fraction(acc))      # float(Fraction) rounds to nearest even
+    for i in range(m):
+        for j in range(n):
+            acc = 0.0
+            for kk in range(k):
+                acc = fused(a[i, kk], b[j, kk], acc)
+            assert got[i, j] == acc, (i, j)
+    # an unfused product-then-add differs on these operands somewhere: the test would notice a dropped fusion
+    unfused = np.zeros((m, n))
+    for kk in range(k):
+        unfused = unfused + a[:, kk:kk + 1] * b[:, kk][None, :]
+    assert (unfused != got).any()
+    with_c = np.zeros((m, n), np.float64)
+    oracle.matmul(a, b, with_c, cin=cin, atom=O.ATOM_F64F64)
+    assert np.array_equal(with_c, got + cin)
+    # numpy's product: another order of the same sum
+    assert (np.abs(got - a @ b.T) <= k * 2.0 ** -52 * (np.abs(a) @ np.abs(b).T)).all()
+    # integers: exact whatever the order; views with strides
+    ai = (synth.draws(6, 40 * 64) % np.uint64(2 ** 20)).astype(np.float64).reshape(40, 64)
+    bi = (synth.draws(7, 30 * 64) % np.uint64(2 ** 20)).astype(np.float64).reshape(30, 64)
+    exact = (ai.astype(object) @ bi.astype(object).T).astype(np.float64)
+    out = np.zeros((40, 30), np.float64)
+    oracle.matmul(ai, bi, out, atom=O.ATOM_F64F64)
+    assert np.array_equal(out, exact)
+    out_t = np.zeros((30, 40), np.float64)
+    oracle.matmul(np.ascontiguousarray(ai.T).T, np.ascontiguousarray(bi.T).T, out_t.T, atom=O.ATOM_F64F64)
+    assert np.array_equal(out_t.T, exact)
+    with pytest.raises(ValueError):
+        oracle.matmul(ai, bi, out)                                      # fp64 operands under the bf16 atom
+    with pytest.raises(ValueError):
+        oracle.matmul(ai.astype(np.float32), bi.astype(np.float32), out, atom=O.ATOM_F64F64)

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libvecops_hip.so")
 
 # VecopsDType numbers
-I8, U8, I32, F16, BF16, F32 = 2, 3, 6, 10, 11, 12
+I8, U8, I32, F16, BF16, F32, F64 = 2, 3, 6, 10, 11, 12, 13
 COMPUTE_BF16, COMPUTE_F32 = 0, 1
 FAMILY_NAMES = {0: "none", 1: "tile_256", 2: "tile_128", 3: "tile_64", 4: "skinny", 5: "zero_k", 6: "tile_256x128",
                 7: "tile_128x256"}
@@ -165,7 +165,7 @@ def _check(rc: int) -> None:
 def _torch_dtype_code(t) -> int:
     import torch
     return {torch.int8: I8, torch.uint8: U8, torch.int32: I32, torch.float16: F16, torch.bfloat16: BF16,
-            torch.float32: F32}[t.dtype]
+            torch.float32: F32, torch.float64: F64}[t.dtype]
 
 
 def operand(t) -> Operand:

@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstring>
 
+#include "gemm_f64.h"
 #include "skinny_dense.h"
 #include "skinny_w8a16.h"
 #include "tile_gemm_launch.h"
@@ -19,7 +20,9 @@ namespace {
 using namespace vecops_hip;
 
 enum : int32_t { ST_OK = 0, ST_INVALID = 1, ST_NOT_APPLICABLE = 2, ST_EXEC = 6 };
-enum : uint32_t { DT_I8 = 2, DT_U8 = 3, DT_I32 = 6, DT_F16 = 10, DT_BF16 = 11, DT_F32 = 12 };
+enum : uint32_t { DT_I8 = 2, DT_U8 = 3, DT_I32 = 6, DT_F16 = 10, DT_BF16 = 11, DT_F32 = 12, DT_F64 = 13 };
+// fp64 operands run on a kernel of their own (gemm_f64.hip), outside the tile kernels' operand classes and outputs
+constexpr int kSrcF64 = 100, kOutF64 = 100;
 
 thread_local char g_error[512] = "";
 
@@ -36,6 +39,7 @@ int64_t dtype_bytes(uint32_t dt) {
     case DT_I8: case DT_U8: return 1;
     case DT_F16: case DT_BF16: return 2;
     case DT_I32: case DT_F32: return 4;
+    case DT_F64: return 8;
     default: return 0;
   }
 }
@@ -139,6 +143,9 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
     pr->src = SRC_BF16;
   } else if (da == DT_F16) {
     pr->src = SRC_F16;  // AMX_F16F32 / SME_F16F32 (matmul/details/kernel/amx/Atoms.h:62-71)
+  } else if (da == DT_F64) {
+    pr->src = kSrcF64;  // SME_F64F64 (matmul/details/kernel/sme/Atoms.h:108-112)
+    if (fused) return fail(ST_NOT_APPLICABLE, "matmul_fused: fp64 operands have no fused output transform");
   } else if (da == DT_F32) {
     if (compute != VECOPS_HIP_COMPUTE_BF16 && compute != VECOPS_HIP_COMPUTE_F32)
       return fail(ST_INVALID, "matmul: unknown compute type %u", compute);
@@ -156,6 +163,9 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
   } else if (is_int) {
     if (dc != DT_I32) return fail(ST_NOT_APPLICABLE, "matmul: int8 operands need an int32 c");
     pr->out_kind = OUT_I32;
+  } else if (pr->src == kSrcF64) {
+    if (dc != DT_F64) return fail(ST_NOT_APPLICABLE, "matmul: fp64 operands need an fp64 c");
+    pr->out_kind = kOutF64;
   } else {
     if (dc == DT_F32) pr->out_kind = OUT_F32;
     else if (dc == DT_BF16 && pr->src != SRC_F16) pr->out_kind = OUT_BF16;
@@ -200,6 +210,9 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
     if (is_int) {
       if (di != DT_I32) return fail(ST_NOT_APPLICABLE, "matmul: c_in must be int32");
       pr->cin_kind = OUT_I32;
+    } else if (pr->src == kSrcF64) {
+      if (di != DT_F64) return fail(ST_NOT_APPLICABLE, "matmul: c_in must be fp64");
+      pr->cin_kind = kOutF64;
     } else if (di == DT_F32) {
       pr->cin_kind = OUT_F32;
     } else if (di == DT_BF16 && pr->src != SRC_F16) {
@@ -225,7 +238,7 @@ constexpr int64_t kQuality256x128 = 800, kQuality128 = 850;
 // other >= 512 (vecops' small-vector leaves serve every atom, matmul/details/kernel/amx/Backend.h:767-992)
 bool skinny_applies(const Problem& pr) {
   if (pr.fused) return false;  // the skinny kernels have no output transform
-  if (pr.src == SRC_I8_FLIP || pr.has_cin || pr.packed_b) return false;
+  if (pr.src == SRC_I8_FLIP || pr.src == kSrcF64 || pr.has_cin || pr.packed_b) return false;
   const int64_t per = pr.src == SRC_I8 ? 16 : pr.src == SRC_F32 ? 4 : 8;  // elements a lane takes per step
   if (!k_vector_ok(pr.a) || !k_vector_ok(pr.b) || pr.k % per != 0 || pr.k < 8 * per) return false;
   const int64_t narrow = pr.m < pr.n ? pr.m : pr.n, wide = pr.m < pr.n ? pr.n : pr.m;
@@ -295,6 +308,10 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
   plan->vector_b = pr.packed_b || (k_vector_ok(pr.b) || (pr.b.rs == 1 && pr.b.cs != 1 && n_vector_ok(pr.b) && dtype_bytes(pr.b.dtype) != 1)) ? 1 : 0;
   plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
 
+  if (pr.src == kSrcF64) {  // one kernel: 128 x 128 tiles, K never split
+    plan->family = VECOPS_HIP_FAMILY_TILE_128;
+    return;
+  }
   // Skinny family: one operand has at most 16 rows and the other is long - the GPU reading of
   // vecops' small-vector shapes (runtime_dispatch_rules::skinny_at_most / large_m1 / large_n1,
   // matmul/details/kernel/RuntimeDispatch.h:24-83): HBM-bound, the wide operand is read once.
@@ -389,7 +406,10 @@ int32_t apply_request(const Problem& pr, const VecopsHipFamilyRequest* request, 
   int tile_m = 0, tile_n = 0;
   tile_of_family(request->family, &tile_m, &tile_n);
   bool serves;
-  if (degenerate || tile_m == 0) {
+  if (pr.src == kSrcF64 && !degenerate) {
+    serves = request->family == VECOPS_HIP_FAMILY_TILE_128;  // the fp64 kernel's only tile
+    if (serves) return ST_OK;
+  } else if (degenerate || tile_m == 0) {
     // nothing to multiply: only the family that names the case; the skinny family: its own shapes
     serves = request->family == plan->family ||
              (request->family == VECOPS_HIP_FAMILY_SKINNY && !degenerate && skinny_applies(pr) && !(pr.dequant && pr.m >= pr.n));
@@ -512,6 +532,23 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   TileGemmParams p = base_params(pr, row_scales, column_scales, correction, workspace);
   const bool is_int = pr.src == SRC_I8 || pr.src == SRC_I8_FLIP;
 
+  if (pr.src == kSrcF64) {  // (K = 0 included: the kernel then writes C_in or zeros)
+    GemmF64Params q;
+    memset(&q, 0, sizeof(q));
+    q.a = static_cast<const double*>(pr.a.data);
+    q.b = static_cast<const double*>(pr.b.data);
+    q.c = static_cast<double*>(pr.c.data);
+    q.cin = pr.has_cin ? static_cast<const double*>(pr.cin.data) : nullptr;
+    q.m = p.m; q.n = p.n; q.k = p.k; q.batch = p.batch;
+    q.a_rs = pr.a.rs; q.a_ks = pr.a.cs; q.a_bs = pr.a.bs;
+    q.b_rs = pr.b.rs; q.b_ks = pr.b.cs; q.b_bs = pr.b.bs;
+    q.c_rs = pr.c.rs; q.c_cs = pr.c.cs; q.c_bs = pr.c.bs;
+    if (pr.has_cin) { q.cin_rs = pr.cin.rs; q.cin_cs = pr.cin.cs; q.cin_bs = pr.cin.bs; }
+    if (pr.batch > 65535) return fail(ST_INVALID, "matmul: more than 65535 fp64 batches");
+    hipError_t e64 = launch_gemm_f64(q, stream);
+    if (e64 != hipSuccess) return fail(ST_EXEC, "fp64 kernel launch: %s", hipGetErrorString(e64));
+    return ST_OK;
+  }
   if (plan.family == VECOPS_HIP_FAMILY_ZERO_K) {
     p.split_k = 0;  // empty sum: the reduce kernel emits epilogue(0)
     hipError_t e = launch_splitk_reduce(p, is_int, stream);
