@@ -17,6 +17,9 @@ namespace vecops_hip {
 namespace {
 
 typedef __attribute__((ext_vector_type(4))) double f64x4;
+// loads through generic pointers count against the LDS counter too: every wait for a fragment read would then wait
+// for the prefetch of the next K tile as well
+#define GLOBAL_F64 __attribute__((address_space(1))) double
 
 constexpr int kTile = 128, kK = 8, kPitch = kK + 1;
 
@@ -35,8 +38,8 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(const GemmF64Params p) {
   // staging: thread t holds k half (t & 1) of row t >> 1 of both operand tiles (4 doubles each)
   const int s_row = tid >> 1, s_k = (tid & 1) * 4;
   const bool a_row_ok = m0 + s_row < p.m, b_row_ok = n0 + s_row < p.n;
-  const double* a_src = a + static_cast<int64_t>(a_row_ok ? m0 + s_row : 0) * p.a_rs;
-  const double* b_src = b + static_cast<int64_t>(b_row_ok ? n0 + s_row : 0) * p.b_rs;
+  const GLOBAL_F64* a_src = (const GLOBAL_F64*)(a + static_cast<int64_t>(a_row_ok ? m0 + s_row : 0) * p.a_rs);
+  const GLOBAL_F64* b_src = (const GLOBAL_F64*)(b + static_cast<int64_t>(b_row_ok ? n0 + s_row : 0) * p.b_rs);
   double ra[4], rb[4];
   auto fetch = [&](int kt) {
 #pragma unroll
