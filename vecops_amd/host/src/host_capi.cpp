@@ -9,6 +9,7 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <vector>
 
 #include "../hip/matmul_plugin.hpp"
 
@@ -73,13 +74,12 @@ std::mutex g_bridge_mutex;
 std::unordered_map<std::uint64_t, std::shared_ptr<rt::Operator>> g_bridge_operators;
 std::atomic<std::uint64_t> g_next_handle{1};
 
-// Device workspace of bridge calls that bring none: one buffer per host thread and device, grown on demand and kept
+// Device workspace of bridge calls that bring none: one buffer per host thread and device, grown on demand
 // (a bridge call is synchronous, so a thread never has two calls using its buffer).  The HIP runtime is looked up at
 // the first need - this library itself does not link it.
 struct HipRuntime {
   int (*get_device)(int*) = nullptr;
   int (*malloc_)(void**, size_t) = nullptr;
-  int (*free_)(void*) = nullptr;
   bool ok = false;
 };
 const HipRuntime& hip_runtime() {
@@ -90,36 +90,58 @@ const HipRuntime& hip_runtime() {
     if (lib == nullptr) return r;
     r.get_device = reinterpret_cast<int (*)(int*)>(dlsym(lib, "hipGetDevice"));
     r.malloc_ = reinterpret_cast<int (*)(void**, size_t)>(dlsym(lib, "hipMalloc"));
-    r.free_ = reinterpret_cast<int (*)(void*)>(dlsym(lib, "hipFree"));
-    r.ok = r.get_device != nullptr && r.malloc_ != nullptr && r.free_ != nullptr;
+    r.ok = r.get_device != nullptr && r.malloc_ != nullptr;
     return r;
   }();
   return runtime;
 }
+// Buffers are never given back to the device: a thread that ends returns its buffers to a process-wide pool for the
+// next thread to take (no HIP call runs in a thread's or the process's teardown, when the runtime may be gone).
+struct DeviceBuffer {
+  void* data = nullptr;
+  std::uint64_t size = 0;
+};
+constexpr int kBridgeDevices = 64;
+std::mutex g_pool_mutex;
+std::vector<DeviceBuffer> g_buffer_pool[kBridgeDevices];
+
 struct ThreadWorkspace {
-  static constexpr int kDevices = 64;
-  void* buffer[kDevices] = {};
-  std::uint64_t size[kDevices] = {};
+  DeviceBuffer mine[kBridgeDevices];
   ~ThreadWorkspace() {
-    for (int d = 0; d < kDevices; ++d)
-      if (buffer[d] != nullptr) hip_runtime().free_(buffer[d]);
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    for (int d = 0; d < kBridgeDevices; ++d)
+      if (mine[d].data != nullptr) g_buffer_pool[d].push_back(mine[d]);
   }
   rt::Status get(std::uint64_t bytes, void** out) {
     const HipRuntime& hip = hip_runtime();
     if (!hip.ok) return rt::Status(rt::StatusCode::ExecutionError, "bridge workspace: the HIP runtime is not available");
     int device = 0;
-    if (hip.get_device(&device) != 0 || device < 0 || device >= kDevices)
+    if (hip.get_device(&device) != 0 || device < 0 || device >= kBridgeDevices)
       return rt::Status(rt::StatusCode::ExecutionError, "bridge workspace: no current HIP device");
-    if (size[device] < bytes) {
-      if (buffer[device] != nullptr) hip.free_(buffer[device]);
-      buffer[device] = nullptr;
-      size[device] = 0;
-      const std::uint64_t want = (bytes + (std::uint64_t{1} << 20) - 1) & ~((std::uint64_t{1} << 20) - 1);
-      if (hip.malloc_(&buffer[device], want) != 0)
-        return rt::Status(rt::StatusCode::ExecutionError, "bridge workspace: device allocation of " + std::to_string(want) + " bytes failed");
-      size[device] = want;
+    DeviceBuffer& buffer = mine[device];
+    if (buffer.size < bytes) {
+      std::lock_guard<std::mutex> lock(g_pool_mutex);
+      std::vector<DeviceBuffer>& pool = g_buffer_pool[device];
+      if (buffer.data != nullptr) pool.push_back(buffer);  // too small for this call: someone else's next one may fit
+      buffer = DeviceBuffer{};
+      for (size_t i = 0; i < pool.size(); ++i) {
+        if (pool[i].size >= bytes) {
+          buffer = pool[i];
+          pool.erase(pool.begin() + static_cast<std::ptrdiff_t>(i));
+          break;
+        }
+      }
+      if (buffer.data == nullptr) {
+        const std::uint64_t want = (bytes + (std::uint64_t{1} << 20) - 1) & ~((std::uint64_t{1} << 20) - 1);
+        if (hip.malloc_(&buffer.data, want) != 0) {
+          buffer = DeviceBuffer{};
+          return rt::Status(rt::StatusCode::ExecutionError,
+                            "bridge workspace: device allocation of " + std::to_string(want) + " bytes failed");
+        }
+        buffer.size = want;
+      }
     }
-    *out = buffer[device];
+    *out = buffer.data;
     return rt::Status::success();
   }
 };
