@@ -482,8 +482,10 @@ ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_q
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=300,
+                    help="untimed launches before the timed ones (after idling the chip takes about 200 launches of "
+                         "the headline kernel, 25 ms, to settle at its clock under load)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", choices=ONLY, help="run a single workload (for profiling)")
     ap.add_argument("--gemv-m", type=int, default=1, help="activation rows of the --only gemv workload (1..16)")
