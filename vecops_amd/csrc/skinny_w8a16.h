@@ -478,7 +478,7 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
 
   // activation fragments of this K slice, resident for the whole kernel
   u32x4 x1[S], x2[S];
-  {
+  auto load_activations = [&]() {
     const VECOPS_GLOBAL char* xrow = (const VECOPS_GLOBAL char*)(p.x + static_cast<int64_t>(min(row, p.m - 1)) * p.ldx) +
                                      quarter * 32 + static_cast<int64_t>(wave) * S * 128;
 #pragma unroll
@@ -491,7 +491,7 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
         x2[s] = px[1];
       }
     }
-  }
+  };
 
   const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};  // eight bf16 1.0
   u32x4 wq[D][TILES];
@@ -565,8 +565,10 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
     (void)pass;
   };
 
-  load_scales(sc_cur, 0);
+  // the first weights are requested before the activations: they arrive while those are fetched
   static_for<D>([&](auto u) { issue(u, decltype(u)::value); });
+  load_scales(sc_cur, 0);
+  load_activations();
   for (int pass = 0; pass < passes; ++pass) {
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
