@@ -64,6 +64,18 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
     rc, p = _plan(_operand(capi.BF16, (2048, 4096)), _operand(capi.BF16, (14336, 4096)), _operand(capi.BF16, (2048, 14336)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
+    # half a round of big tiles or a round of rectangles against one round of 128x128 pairs (two live on a compute
+    # unit at a time): the small tile, for both classes; int8 also up to eight K tiles
+    for dt, out in ((capi.BF16, capi.BF16), (capi.I8, capi.I32)):
+        for m in (1536, 2048):
+            rc, p = _plan(_operand(dt, (m, 4096)), _operand(dt, (4096, 4096)), _operand(out, (m, 4096)))
+            assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1
+        rc, p = _plan(_operand(dt, (3072, 4096)), _operand(dt, (4096, 4096)), _operand(out, (3072, 4096)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
+    rc, p = _plan(_operand(capi.I8, (4096, 1024)), _operand(capi.I8, (4096, 1024)), _operand(capi.I32, (4096, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
+    rc, p = _plan(_operand(capi.BF16, (4096, 1024)), _operand(capi.BF16, (4096, 1024)), _operand(capi.BF16, (4096, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
     # 3000^3: 144 big tiles in one part-filled round stay ahead of 576 small ones in three
     rc, p = _plan(_operand(capi.BF16, (3000, 3000)), _operand(capi.BF16, (3000, 3000)), _operand(capi.F32, (3000, 3000)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"

@@ -116,7 +116,8 @@ def test_f16_skinny_family(device, oracle, narrow, wide, k, out):
 
 @pytest.mark.parametrize("m,n,k", [(300, 260, 1000), (37, 51, 79), (512, 768, 512), (2, 3, 64, 40, 200)][:3] + [(2457, 1221, 72)])
 def test_f16_prepacked_b(device, oracle, m, n, k):
-    """Half weights packed once (the 16-bit permutation of the bf16 pack): bit-equal to the plain product."""
+    """Half weights packed once (the 16-bit permutation of the bf16 pack): bit-equal to the plain product on the
+    256 x 256 tiles, which multiply in the packed kernel's order (v_mfma_f32_32x32x16_f16)."""
     import torch
     from vecops_amd import capi
     a, b = _half(1, (m, k)), _half(2, (n, k))
@@ -126,7 +127,8 @@ def test_f16_prepacked_b(device, oracle, m, n, k):
     for dt in (torch.float32, torch.float16):
         c, ref = (torch.full((m, n), float("nan"), dtype=dt, device=device) for _ in range(2))
         capi.matmul_packed_b(ta, packed, c)
-        capi.matmul(ta, tb, ref)
+        split_k = capi.plan_matmul_packed_b(ta, packed, c).split_k          # the same partition of K
+        capi.matmul_family(ta, tb, ref, capi.family_request("tile_256", split_k=split_k))
         torch.cuda.synchronize()
         assert torch.equal(c.view(torch.int32 if dt == torch.float32 else torch.int16),
                            ref.view(torch.int32 if dt == torch.float32 else torch.int16))

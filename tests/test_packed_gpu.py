@@ -191,10 +191,12 @@ def test_packed_fp32_a_batched_cin_and_strides(device, oracle):
     oracle.matmul(a, np.ascontiguousarray(b3), want, cin=cin, atom=O.ATOM_BF16F32, acc_f64=True)
     assert rel_err(got, want) <= fp32_tol(k)
     assert torch.isnan(c_store[:, :, n:]).all()
-    # identical, bit for bit, to the plain path on the unpacked operand (same tile kernels' sums)
+    # identical, bit for bit, to the plain path on the unpacked operand on the 256 x 256 tiles (the packed kernel's
+    # MFMA shape and order of sums)
     c_plain = torch.empty((batch, m, n), dtype=torch.float32, device=device)
-    capi.matmul(a_dev[:, :, :k], torch.from_numpy(np.ascontiguousarray(b3)).to(device), c_plain,
-                c_in=dev_bf16(cin, device))
+    capi.matmul_family(a_dev[:, :, :k], torch.from_numpy(np.ascontiguousarray(b3)).to(device), c_plain,
+                       capi.family_request("tile_256", split_k=capi.plan_matmul_packed_b(a_dev[:, :, :k], packed, c).split_k),
+                       c_in=dev_bf16(cin, device))
     torch.cuda.synchronize()
     assert np.array_equal(got, c_plain.cpu().numpy())
 

@@ -229,10 +229,13 @@ int32_t describe(const VecopsHipOperand* a, const VecopsHipOperand* b, const Vec
 constexpr int kComputeUnits = 256;
 constexpr int kStreamGroupsPerUnit = 2;  // workgroups of 4 wavefronts per compute unit of the streaming GEMV
 // Work per compute unit and second of the smaller tiles relative to 256x256, per mille (see choose()): bf16 4096^3
-// required of each tile family (`bench.py --only families`) takes 107 / 133 / 130 / 121 us (256x256, 256x128, 128x256,
-// 128x128; two or three 128x128 workgroups share a compute unit), int8 4096^3 68 / 83 / 84 / 79; the ratio of the
-// small tile falls to 0.78-0.80 at 8192^3.
-constexpr int64_t kQuality256x128 = 800, kQuality128 = 850;
+// required of each tile family (`bench.py --only families`) takes 105 / 133 / 130 / 112 us (256x256, 256x128, 128x256,
+// 128x128; two 128x128 workgroups share a compute unit), 5120^3 221 / 309 / 307 / 255, 2048 x 14336 x 4096
+// 185 / 247 / 246 / 204; int8 4096^3 70 / 83 / 84 / 71.5, 5120^3 142 / 184 / 192 / 150, 2048 x 14336 x 4096
+// 123 / 153 / 159 / 127.
+// Operands whose rows are not 16-byte aligned go through registers into LDS, work that grows with a tile's
+// perimeter: 8 x 777 x 1000 x 3001 takes 64 us on 128x256 tiles and 73.5 on 128x128.
+constexpr int64_t kQuality256x128 = 800, kQuality128 = 900, kQuality128Int8 = 970, kQuality128Staged = 780;
 
 // Every operand class but the unsigned bytes, with K contiguous on both sides, no C input, one side <= 16 rows, the
 // other >= 512 (vecops' small-vector leaves serve every atom, matmul/details/kernel/amx/Backend.h:767-992)
@@ -286,6 +289,8 @@ void finish_tile_plan(const Problem& pr, VecopsHipPlan* plan, uint32_t forced_sp
   if (pr.src == SRC_I8_FLIP) plan->workspace_bytes += static_cast<uint64_t>(pr.batch) * (pr.m + pr.n) * 4u;
 }
 
+int fetch_mode(const Problem& pr, const VecopsHipPlan& plan);
+
 // The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure
 // integer function of (operand class, m, n, k); it picks the workgroup tile by
 // how many tiles the problem yields against the 256 compute units and splits K
@@ -333,25 +338,33 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
   // 1056 tiles of 128x128, 160 us against 172 for 272 big ones whose second round is 6 % full; 8 x 777x1000: 224
   // tiles of 128x256 in one round; 5120^3, 2048x14336x4096, 8192^3: big tiles, 19-23 % ahead).
   struct Candidate { uint32_t family; int64_t tm, tn, quality; };
+  const bool bytes = pr.src == SRC_I8 || pr.src == SRC_I8_FLIP;
+  const int mode = fetch_mode(pr, *plan);
+  const bool direct = mode == MODE_KVEC_DMA || mode == MODE_NVEC_B_DMA;  // loads that write LDS themselves
   const Candidate candidates[] = {{VECOPS_HIP_FAMILY_TILE_256, 256, 256, 1000},
                                   {VECOPS_HIP_FAMILY_TILE_256X128, 256, 128, kQuality256x128},
                                   {VECOPS_HIP_FAMILY_TILE_128X256, 128, 256, kQuality256x128},
-                                  {VECOPS_HIP_FAMILY_TILE_128, 128, 128, kQuality128}};
+                                  {VECOPS_HIP_FAMILY_TILE_128, 128, 128,
+                                   !direct ? kQuality128Staged : bytes ? kQuality128Int8 : kQuality128}};
   uint32_t family = VECOPS_HIP_FAMILY_TILE_64;
   int64_t tile_m = 64, tile_n = 64, best_cost = INT64_MAX;
   for (const Candidate& c : candidates) {
     if (pr.m <= c.tm / 2 || pr.n <= c.tn / 2) continue;  // a tile more than half empty in one direction
     const int64_t count = tiles2(c.tm, c.tn);
     if (count < kComputeUnits / 2) continue;
-    const int64_t rounds = (count + kComputeUnits - 1) / kComputeUnits;
-    int64_t cost = rounds * c.tm * c.tn * 1000 / c.quality;
+    // two 128x128 workgroups live on a compute unit at a time (64 KiB of LDS and at most 256 registers each): a
+    // round of them is 512 tiles
+    const int64_t per_unit = c.family == VECOPS_HIP_FAMILY_TILE_128 ? 2 : 1, slots = per_unit * kComputeUnits;
+    const int64_t rounds = (count + slots - 1) / slots;
+    int64_t cost = rounds * per_unit * c.tm * c.tn * 1000 / c.quality;
     // a single part-filled round runs faster than a full one (the chip is power-limited: fewer busy compute units
-    // clock higher): half full costs three quarters (3000^3 as 144 big tiles 92 us against 108 for 576 small ones;
+    // clock higher): half full costs three quarters (3000^3 as 144 big tiles 87 us against 105 for 576 small ones;
     // 8 x 777 x 1000 x 3001 as 224 tiles of 128x256 65 us, as 256 of 256x128 73, as 128 of 256x256 86)
-    if (rounds == 1) cost = cost * (kComputeUnits + count) / (2 * kComputeUnits);
-    // a smaller tile has to be 10 % cheaper than a bigger one: the round count flatters it (more L2 traffic per
-    // flop, and its quality falls with the problem size)
-    const bool smaller = best_cost != INT64_MAX && c.tm * c.tn < tile_m * tile_n;
+    if (rounds == 1) cost = cost * (slots + count) / (2 * slots);
+    // a rectangle has to be 10 % cheaper than the big tile: the round count flatters it (more L2 traffic per flop,
+    // and its quality falls with the problem size).  The 128x128 tile competes on its cost alone (1536 x 4096 x 4096:
+    // 49 us against 60 for the rectangles, 2048 x 4096 x 4096 58 against 67; int8 31 against 38 and 36 against 42).
+    const bool smaller = best_cost != INT64_MAX && c.tm * c.tn < tile_m * tile_n && c.family != VECOPS_HIP_FAMILY_TILE_128;
     if (best_cost == INT64_MAX || (smaller ? cost * 11 < best_cost * 10 : cost < best_cost)) {
       best_cost = cost;
       family = c.family;
@@ -369,7 +382,8 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
   // two or three 128x128 workgroups on a compute unit overlap one's stores with another's loads, which a
   // single big tile cannot (batch 8 of 3000x3000x17 to fp32: 93 us against 111; 8 x 1000x1000x100: 17.7
   // against 21.7; 4096x4096x256 to bf16: 17.9 against 20.2; level at 8192x8192x256, behind from K = 512).
-  if (k_tiles <= 4 && pr.src != SRC_F32 && family != VECOPS_HIP_FAMILY_TILE_64 && family != VECOPS_HIP_FAMILY_TILE_128 &&
+  // (int8, whose big tile gains least from its size: up to eight, 4096 x 4096 x 1024 29.6 us against 32.9)
+  if (k_tiles <= (bytes ? 8 : 4) && pr.src != SRC_F32 && family != VECOPS_HIP_FAMILY_TILE_64 && family != VECOPS_HIP_FAMILY_TILE_128 &&
       pr.m > 64 && pr.n > 64 && tiles(128) >= kComputeUnits / 2) {
     family = VECOPS_HIP_FAMILY_TILE_128;
     tile_m = tile_n = 128;

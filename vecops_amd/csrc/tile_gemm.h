@@ -331,6 +331,15 @@ struct AccTile<true> {
   using type = i32x16;
 };
 
+template <bool INT>
+struct AccQuad {
+  using type = f32x4;
+};
+template <>
+struct AccQuad<true> {
+  using type = i32x4;
+};
+
 template <int SRC>
 __device__ __forceinline__ void mfma_step(typename AccTile<SrcTraits<SRC>::kInt>::type& acc, const u32x4& a,
                                           const u32x4& b) {
@@ -350,6 +359,75 @@ __device__ __forceinline__ void mfma_step(typename AccTile<SrcTraits<SRC>::kInt>
                                                   0, 0, 0);
   }
 }
+
+// The same product on the 16x16 shapes (v_mfma_f32_16x16x32_bf16 / _f16, v_mfma_i32_16x16x64_i8): lane l
+// supplies 16 bytes of row l % 16, chunk l / 16 of the four 16-byte chunks the instruction consumes along k.
+// On operands with real bit patterns the matrix cores sustain a tenth to a sixth more with this shape than
+// with 32x32 (measured with loops of nothing but independent MFMAs: half the accumulator traffic per
+// multiply-add, and the chip runs against its power limit).
+template <int SRC>
+__device__ __forceinline__ void mfma_step16(typename AccQuad<SrcTraits<SRC>::kInt>::type& acc, const u32x4& a,
+                                            const u32x4& b) {
+  static_assert(SRC != SRC_F32, "the fp32 class stays on 32x32x2");
+  if constexpr (SRC == SRC_F16) {
+    typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
+  } else if constexpr (SrcTraits<SRC>::kInt) {
+    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a), __builtin_bit_cast(i32x4, b), acc, 0, 0,
+                                                0);
+  } else {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc,
+                                                  0, 0, 0);
+  }
+}
+
+// Which tile kernels multiply on the 16x16 shapes: the 128x128 and 64x64 tiles of every class that has them.
+// Measured against the 32x32 shapes in one process on one box (launch to launch, K-contiguous operands): 128x128
+// tiles 1024 x 4096 x 4096 bf16 45.6 against 49.5 us, int8 28.9 against 31.8, int8 2048 x 11008 x 4096 97.6 against
+// 104.7, bf16 2048^3 26.6 against 28.4; 64x64 tiles 512 x 4096 x 4096 33.2 against 36.9 - the short shape draws less
+// power per multiply-add (a loop of nothing but MFMAs sustains 2.06 against 1.75 PFLOP/s on real operands) and its
+// loop below has no address arithmetic.  The 256-row and 256-column tiles stay on 32x32: their 128 to 256
+// accumulator registers need the accumulation half of the register file, where the compiler does not tie an
+// MFMA's result to its addend and permutes the accumulators back at the loop's head (a hundred copies per K tile);
+// with the MFMAs written out as tied instruction text the 256x256 tile gained 1.5-3.5 % for bf16 and lost 4.6 % for
+// int8, and the compiler's hazard tracking does not see through such text - not worth it.  A tile of at most 128x128
+// fits two wavefronts per SIMD, where MFMAs accumulate in place in vector registers.
+template <int SRC, int WM, int WN>
+constexpr bool kShortMfma = SRC != SRC_F32 && WM * WN <= 4;
+
+// The accumulators of one wavefront: WM x WN blocks of 32x32 elements of C, held either as one 32x32 MFMA
+// result per block (M16 = false) or as its four 16x16 quadrants (M16 = true).  Both shapes are issued with the
+// B fragment as first operand, so a lane holds runs of four consecutive columns of one row of C: quad q of a
+// block is the four values at row(lane, q), columns col(lane, q) .. + 3 of the block.
+//   32x32: register r of lane l is C[l % 32][(r / 4) * 8 + (l / 32) * 4 + r % 4], quad q = registers 4q .. 4q + 3
+//   16x16: quadrant (q / 2, q % 2); register r of lane l is C[l % 16][(l / 16) * 4 + r] of the quadrant
+template <bool INT, int WM, int WN, bool M16>
+struct Accumulators {
+  using Quad = typename AccQuad<INT>::type;
+  using Frag = typename std::conditional<M16, Quad, typename AccTile<INT>::type>::type;
+  static constexpr int FM = M16 ? 2 * WM : WM, FN = M16 ? 2 * WN : WN;  // fragments per wavefront tile
+  Frag t[FM][FN];
+  __device__ __forceinline__ void clear() {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int r = 0; r < (M16 ? 4 : 16); ++r) t[i][j][r] = 0;
+  }
+  template <int I, int J, int Q>
+  __device__ __forceinline__ Quad quad() const {
+    if constexpr (M16) return t[2 * I + (Q >> 1)][2 * J + (Q & 1)];
+    else return __builtin_shufflevector(t[I][J], t[I][J], 4 * Q, 4 * Q + 1, 4 * Q + 2, 4 * Q + 3);
+  }
+  static __device__ __forceinline__ int row(int lane, int q) { return M16 ? (q >> 1) * 16 + (lane & 15) : (lane & 31); }
+  static __device__ __forceinline__ int col(int lane, int q) {
+    return M16 ? (q & 1) * 16 + (lane >> 4) * 4 : q * 8 + (lane >> 5) * 4;
+  }
+  // which of the (at most two) different rows a lane has in a block quad q lies in
+  static constexpr int row_slot(int q) { return M16 ? (q >> 1) : 0; }
+  static constexpr int kRowSlots = M16 ? 2 : 1;
+};
 
 // The fused output transform in the order the header states.  Every step is its own fp32
 // operation (the file is compiled without contraction), as vecops' transforms are separate
@@ -1221,18 +1299,25 @@ struct StagingOp {
 // evenly, A's first; a transposing B stager has one or two heavy parts (four
 // writes, eight loads), which take k-steps 0 and 2 while A's chunks share the
 // others.
-template <typename SA, typename SB, bool B_TRANSPOSING>
+//
+// LATE (loads that write LDS, under the loop of the 16x16 shapes, whose barrier stands in the middle of the K
+// tile): the loads are those of the tile after the next, into the stage the barrier has just freed, in phases
+// 4 and 5 = the two quarters of the K tile behind the barrier; a load has half a K tile and more to land.
+template <typename SA, typename SB, bool B_TRANSPOSING, bool LATE = false>
 struct StagingSchedule {
   static constexpr int PARTS_A = SA::kParts, PARTS_B = SB::kParts;
   static constexpr bool DMA = SA::kStoreOps == 0;  // loads that write LDS: all of them early, in k-steps 0 and 1
+  static_assert(DMA || !LATE, "only loads that write LDS can run a tile ahead of the stores");
   static constexpr int step_a(int part) {
-    if constexpr (DMA) return part * 2 / (PARTS_A + PARTS_B);
+    if constexpr (LATE) return 4 + part * 2 / (PARTS_A + PARTS_B);
+    else if constexpr (DMA) return part * 2 / (PARTS_A + PARTS_B);
     else if constexpr (!B_TRANSPOSING) return part * 4 / (PARTS_A + PARTS_B);
     else if constexpr (PARTS_B == 2) return part * 2 < PARTS_A ? 1 : 3;
     else return 1 + part * 3 / PARTS_A;
   }
   static constexpr int step_b(int part) {
-    if constexpr (DMA) return (PARTS_A + part) * 2 / (PARTS_A + PARTS_B);
+    if constexpr (LATE) return 4 + (PARTS_A + part) * 2 / (PARTS_A + PARTS_B);
+    else if constexpr (DMA) return (PARTS_A + part) * 2 / (PARTS_A + PARTS_B);
     else if constexpr (!B_TRANSPOSING) return (PARTS_A + part) * 4 / (PARTS_A + PARTS_B);
     else return part * 2;
   }
@@ -1297,18 +1382,16 @@ constexpr int kTileLdsBytes() {
 }
 
 // Epilogue of the tile kernels: the accumulators of one wavefront to C.
-template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LDS_BYTES>
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LDS_BYTES, bool M16>
 __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char* lds,
-                                                   typename AccTile<SrcTraits<SRC>::kInt>::type (&acc)[WM][WN], int batch,
+                                                   const Accumulators<SrcTraits<SRC>::kInt, WM, WN, M16>& acc, int batch,
                                                    int split, int m0, int n0, int wm, int wn, int wave, int lane) {
   constexpr bool INT = SrcTraits<SRC>::kInt;
   constexpr int BM = 32 * WAVES_M * WM, BN = 32 * WAVES_N * WN;
-  const int frag_row = lane & 31;
-  const int frag_half = lane >> 5;
+  using ACC = Accumulators<INT, WM, WN, M16>;
   // Epilogue.  The MFMAs were issued with the B tile as first operand, so the
-  // accumulators hold C transposed: register r of lane l is
-  //   C[row = l % 32][col = (r/4)*8 + (l/32)*4 + r%4]
-  // of its 32x32 tile, i.e. four consecutive columns per register quad, which
+  // accumulators hold C transposed: a lane holds quads of four consecutive columns
+  // of one row of C (Accumulators::row / col), which
   // become one 8-byte (bf16) or 16-byte (fp32 / int32) store.  Tiles that lie
   // wholly inside C, need no C-input or split-K and have 16-byte aligned rows take
   // one of three inline store loops; everything else goes through the general
@@ -1344,10 +1427,11 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
         static_for<4>([&](auto cq) {
           constexpr int q = decltype(cq)::value;
           if constexpr (!INT) {
+            const auto a4 = acc.template quad<i, j, q>();
             u32x2 v;
-            v.x = cvt_pk_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]);
-            v.y = cvt_pk_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-            *reinterpret_cast<u32x2*>(mine + (i * 32 + frag_row) * PITCH + (j * 32 + q * 8 + frag_half * 4) * 2) = v;
+            v.x = cvt_pk_bf16(a4[0], a4[1]);
+            v.y = cvt_pk_bf16(a4[2], a4[3]);
+            *reinterpret_cast<u32x2*>(mine + (i * 32 + ACC::row(lane, q)) * PITCH + (j * 32 + ACC::col(lane, q)) * 2) = v;
           }
         });
       });
@@ -1384,10 +1468,13 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
     static_assert(ROWS * PITCH * 4 * WAVES_M * WAVES_N <= LDS_BYTES, "32-bit epilogue staging must fit the launch's LDS");
     __syncthreads();  // every wavefront is done reading fragments
     uint32_t* mine = reinterpret_cast<uint32_t*>(lds) + wave * (ROWS * PITCH);
-    float rs[WM];
+    float rs[WM][ACC::kRowSlots];
     static_for<WM>([&](auto ci) {
-      const int row = m0 + (wm * WM + decltype(ci)::value) * 32 + frag_row;
-      rs[decltype(ci)::value] = (dequant && row < p.m) ? p.row_scales[batch * p.row_scales_bs + row] : 1.0f;
+      static_for<ACC::kRowSlots>([&](auto ch) {
+        const int row = m0 + (wm * WM + decltype(ci)::value) * 32 + ACC::row(lane, 2 * decltype(ch)::value);
+        rs[decltype(ci)::value][decltype(ch)::value] =
+            (dequant && row < p.m) ? p.row_scales[batch * p.row_scales_bs + row] : 1.0f;
+      });
     });
     uint32_t* out = reinterpret_cast<uint32_t*>(c_base) + batch * p.c_bs + static_cast<int64_t>(m0 + wm * ROWS) * p.c_rs;
     const int out_bytes = output_element_bytes(p.out_kind);
@@ -1399,7 +1486,7 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
       i32x4 corr[4];
       static_for<4>([&](auto cq) {
         constexpr int q = decltype(cq)::value;
-        const int col0 = col_block + frag_half * 4 + q * 8;
+        const int col0 = col_block + ACC::col(lane, q);
         cs[q] = f32x4{1.f, 1.f, 1.f, 1.f};
         corr[q] = i32x4{0, 0, 0, 0};
         if (col0 + 3 < p.n) {
@@ -1419,7 +1506,7 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
         constexpr int i = decltype(ci)::value;
         static_for<4>([&](auto cq) {
           constexpr int q = decltype(cq)::value;
-          const auto a4 = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
+          const auto a4 = acc.template quad<i, j, q>();
           u32x4 bits = __builtin_bit_cast(u32x4, a4);
           if constexpr (INT) {
             bits += __builtin_bit_cast(u32x4, corr[q]);
@@ -1427,13 +1514,13 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
               f32x4 o;
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
-                const float t = static_cast<float>(static_cast<int32_t>(bits[e])) * rs[i];  // row scale first, then
+                const float t = static_cast<float>(static_cast<int32_t>(bits[e])) * rs[i][ACC::row_slot(q)];  // row scale first, then
                 o[e] = t * cs[q][e];                                                         // column scale
               }
               bits = __builtin_bit_cast(u32x4, o);
             }
           }
-          *reinterpret_cast<u32x4*>(mine + (i * 32 + frag_row) * PITCH + q * 8 + frag_half * 4) = bits;
+          *reinterpret_cast<u32x4*>(mine + (i * 32 + ACC::row(lane, q)) * PITCH + ACC::col(lane, q)) = bits;
         });
       });
       // the wavefront reads back only what it wrote itself: its own LDS traffic is ordered
@@ -1489,18 +1576,17 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
     });
   } else if (interior && p.split_k > 1 && (p.n & 3) == 0 && (reinterpret_cast<uintptr_t>(p.partial) & 15) == 0) {
     // split-K partial sums of an interior tile: raw accumulators, 16 bytes per store
+    uint32_t* partial = static_cast<uint32_t*>(p.partial) + (static_cast<int64_t>(split) * p.batch + batch) * p.m * p.n;
     static_for<WM>([&](auto ci) {
       constexpr int i = decltype(ci)::value;
-      const int row = m0 + (wm * WM + i) * 32 + frag_row;
-      uint32_t* dst_row = static_cast<uint32_t*>(p.partial) +
-                          ((static_cast<int64_t>(split) * p.batch + batch) * p.m + row) * p.n;
       static_for<WN>([&](auto cj) {
         constexpr int j = decltype(cj)::value;
-        uint32_t* dst = dst_row + n0 + (wn * WN + j) * 32 + frag_half * 4;
         static_for<4>([&](auto cq) {
           constexpr int q = decltype(cq)::value;
-          const auto v = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
-          *reinterpret_cast<typename std::remove_const<decltype(v)>::type*>(dst + q * 8) = v;
+          const int row = m0 + (wm * WM + i) * 32 + ACC::row(lane, q);
+          const auto v = acc.template quad<i, j, q>();
+          *reinterpret_cast<typename std::remove_const<decltype(v)>::type*>(
+              partial + static_cast<int64_t>(row) * p.n + n0 + (wn * WN + j) * 32 + ACC::col(lane, q)) = v;
         });
       });
     });
@@ -1522,8 +1608,8 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
         constexpr int j = decltype(cj)::value;
         static_for<4>([&](auto cq) {
           constexpr int q = decltype(cq)::value;
-          const auto v = __builtin_shufflevector(acc[i][j], acc[i][j], 4 * q, 4 * q + 1, 4 * q + 2, 4 * q + 3);
-          *reinterpret_cast<u32x4*>(mine + frag_row * PITCH + j * 32 + q * 8 + frag_half * 4) = __builtin_bit_cast(u32x4, v);
+          const auto v = acc.template quad<i, j, q>();
+          *reinterpret_cast<u32x4*>(mine + ACC::row(lane, q) * PITCH + j * 32 + ACC::col(lane, q)) = __builtin_bit_cast(u32x4, v);
         });
       });
       // the wavefront reads back only what it wrote itself: its own LDS traffic is ordered
@@ -1536,6 +1622,13 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
       }
     });
   }
+}
+
+// Bytes between the k rows of a B tile kept untransposed in LDS (0 for the other layouts).
+template <int SRC, int LOAD_B, int ROWS, int THREADS>
+constexpr int ntr_pitch() {
+  if constexpr (load_is_ntr(LOAD_B)) return Stager<SRC, LOAD_B, ROWS, THREADS>::kPitch;
+  else return 0;
 }
 
 // Workgroup shapes: WAVES_M x WAVES_N wavefronts, each owning WM x WN accumulator
@@ -1554,6 +1647,10 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
   constexpr int THREADS = 64 * WAVES_M * WAVES_N;
   constexpr int BM = 32 * WAVES_M * WM, BN = 32 * WAVES_N * WN;
   constexpr int STAGE_BYTES = kStageBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>();
+  // The 16x16 MFMA shapes (kShortMfma): a K tile is then two k-steps of four 16-byte chunks, and a 32-row block
+  // of a wavefront's tile two fragments
+  constexpr bool M16 = kShortMfma<SRC, WM, WN>;
+  constexpr int FM = M16 ? 2 * WM : WM, FN = M16 ? 2 * WN : WN;
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -1583,26 +1680,60 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
   stager_a.init(static_cast<const char*>(p.a) + batch * p.a_bs * T::kSrcBytes, p.a_rs, p.a_ks, m0, p.m, p.k, tid, p.a_flip);
   stager_b.init(static_cast<const char*>(p.b) + batch * p.b_bs * T::kSrcBytes, p.b_rs, p.b_ks, n0, p.n, p.k, tid, p.b_flip);
 
-  const int frag_row = lane & 31;
-  const int frag_half = lane >> 5;
-  // LDS offsets of this lane's fragments at k-step 0; k-step ks flips bits 5-6: off ^ (ks << 5)
-  int off_a[WM], off_b[WN];
+  // a lane's row of a fragment and its 16-byte chunk within the k-step
+  const int frag_row = M16 ? (lane & 15) : (lane & 31);
+  // (16x16: the four 16-lane groups take the chunks in the order 0, 2, 1, 3 - which k a group multiplies is free as
+  // long as A and B agree, and an LDS read serves lanes l and l + 32 together: their chunks must differ in the
+  // low bit, as they do for the 32x32 shapes, or every fragment read is a two-way bank conflict)
+  const int frag_chunk = M16 ? (((lane >> 4) & 1) << 1 | (lane >> 5)) : (lane >> 5);
+  // 32x32: LDS offsets of this lane's fragments at k-step 0; k-step ks flips chunk bits: off ^ (ks << 5)
+  int off_a[M16 ? 1 : FM], off_b[M16 ? 1 : FN];
+  // 16x16: every fragment read is one of a few per-lane base addresses (per stage) plus a constant, so that a
+  // read costs no vector ALU instruction - with MFMAs of 16 cycles the address arithmetic of the 32x32 loop
+  // (two dependent instructions in front of every read) no longer hides behind the matrix pipe.
+  //   K-contiguous tiles: fragment f, k-step ks lies at row (first + 16 f + lane % 16), chunk slot
+  //   ((4 ks + chunk) ^ row ^ row / 8) & 7 = lane_slot ^ (4 ks ^ 2 f) & 7: four bases by the constant's bits 1-2
+  //   B as k rows: column block j lies (j & 1) * 32 bytes into the 64-byte group ((j >> 1) ^ swizzle)
+  constexpr int PITCH_NTR = ntr_pitch<SRC, LOAD_B, BN, THREADS>();
+  uint32_t base_a[2][4], base_b[2][4];
+  if constexpr (M16) {
+    const uint32_t lds0 = lds_address_of(lds);
+    const int row_a = wm * FM * 16, row_b = wn * FN * 16;
+    const int slot_a = frag_chunk ^ frag_row ^ (frag_row >> 3) ^ (row_a >> 3);
+    const int slot_b = frag_chunk ^ frag_row ^ (frag_row >> 3) ^ (row_b >> 3);
 #pragma unroll
-  for (int i = 0; i < WM; ++i) off_a[i] = lds_chunk_offset((wm * WM + i) * 32 + frag_row, frag_half);
+    for (int st = 0; st < 2; ++st)
 #pragma unroll
-  for (int j = 0; j < WN; ++j) {
-    if constexpr (load_is_ntr(LOAD_B)) {
-      // transposing read: 16-lane group g = lane / 16 serves columns (g & 1) * 16 .. + 15 of the fragment and
-      // the k half g / 2; lane s of the group addresses row s / 4, columns 4 * (s % 4) .. + 3
-      constexpr int PITCH_B = Stager<SRC, LOAD_B, BN, THREADS>::kPitch;
-      const int s = lane & 15, g = lane >> 4;
-      int col_bytes = ((wn * WN + j) * 32 + (g & 1) * 16 + (s & 3) * 4) * 2;
-      // packed rows: the 64-byte group is swizzled with the row's low two bits, which are s / 4 for both reads of
-      // every k-step
-      if constexpr (LOAD_B == LOAD_NTR_DMA) col_bytes ^= ((s >> 2) & 3) << 6;
-      off_b[j] = BM * 128 + ((g >> 1) * 8 + (s >> 2)) * PITCH_B + col_bytes;
-    } else {
-      off_b[j] = BM * 128 + lds_chunk_offset((wn * WN + j) * 32 + frag_row, frag_half);
+      for (int q = 0; q < 4; ++q) {
+        base_a[st][q] = lds0 + st * STAGE_BYTES + (row_a + frag_row) * 128 + (((slot_a ^ (2 * q)) & 7) << 4);
+        if constexpr (load_is_ntr(LOAD_B)) {
+          // transposing read: lane s of the 16-lane group addresses row s / 4 of a block of four k rows, columns
+          // 4 * (s % 4) .. + 3, and receives column s of the block's 16; the group reads chunk frag_chunk of k
+          const int s16 = lane & 15;
+          int col_bytes = ((wn * FN + 2 * q) * 16 + (s16 & 3) * 4) * 2;
+          // packed rows: the 64-byte group is swizzled with the row's low two bits, which are s / 4 for both reads
+          // of every k-step
+          if constexpr (LOAD_B == LOAD_NTR_DMA) col_bytes ^= ((s16 >> 2) & 3) << 6;
+          base_b[st][q] = lds0 + st * STAGE_BYTES + BM * 128 + (frag_chunk * 8 + (s16 >> 2)) * PITCH_NTR + col_bytes;
+        } else {
+          base_b[st][q] = lds0 + st * STAGE_BYTES + BM * 128 + (row_b + frag_row) * 128 + (((slot_b ^ (2 * q)) & 7) << 4);
+        }
+      }
+  } else {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) off_a[i] = lds_chunk_offset((wm * FM + i) * 32 + frag_row, frag_chunk);
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+      if constexpr (load_is_ntr(LOAD_B)) {
+        // transposing read: 16-lane group g = lane / 16 serves columns (g & 1) * 16 .. + 15 of the fragment and
+        // the k half g / 2; lane s of the group addresses row s / 4, columns 4 * (s % 4) .. + 3
+        const int s16 = lane & 15, g = lane >> 4;
+        int col_bytes = ((wn * FN + j) * 32 + (g & 1) * 16 + (s16 & 3) * 4) * 2;
+        if constexpr (LOAD_B == LOAD_NTR_DMA) col_bytes ^= ((s16 >> 2) & 3) << 6;
+        off_b[j] = BM * 128 + ((g >> 1) * 8 + (s16 >> 2)) * PITCH_NTR + col_bytes;
+      } else {
+        off_b[j] = BM * 128 + lds_chunk_offset((wn * FN + j) * 32 + frag_row, frag_chunk);
+      }
     }
   }
 
@@ -1629,30 +1760,56 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
   // MFMAs before, the fragment reads and the other half after.  A global load has a
   // whole K tile of MFMA work to land before its registers are stored; an LDS read
   // has most of a k-step.
-  u32x4 fa[2][WM], fb[2][WN];
-  constexpr int N_MFMA = WM * WN, N_READ = WM + WN;
-  // fragment reads in the order the MFMAs consume them: A fragment 0, every B fragment, the other A fragments
-  auto read_frag = [&](int set, const char* tile, int ks, auto r_tag) {
-    constexpr int r = decltype(r_tag)::value;
-    if constexpr (r == 0) fa[set][0] = *reinterpret_cast<const u32x4*>(tile + (off_a[0] ^ (ks << 5)));
-    else if constexpr (r <= WN) {
-      if constexpr (load_is_ntr(LOAD_B)) {
-        // k-step ks covers rows 16*ks .. 16*ks+15 of the tile; the two reads give k 0-3 and 4-7 of the lane's half
-        constexpr int PITCH_B = Stager<SRC, LOAD_B, BN, THREADS>::kPitch;
-        typedef __attribute__((ext_vector_type(4))) short s16x4;
-        typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-        const char* at = tile + off_b[r - 1] + ks * 16 * PITCH_B;
-        const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at)));
-        const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * PITCH_B)));
-        fb[set][r - 1] = u32x4{lo.x, lo.y, hi.x, hi.y};
-      } else {
-        fb[set][r - 1] = *reinterpret_cast<const u32x4*>(tile + (off_b[r - 1] ^ (ks << 5)));
-      }
+  u32x4 fa[2][FM], fb[2][FN];
+  constexpr int N_MFMA = FM * FN, N_READ = FM + FN;
+  // fragment reads in the order the MFMAs consume them: A fragment 0, every B fragment, the other A fragments;
+  // stage and k-step are compile-time constants
+  typedef __attribute__((ext_vector_type(4))) short s16x4;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+  // (the stage is a compile-time constant under the 16x16 shapes, whose loop is written out for both stages, and a
+  // run-time number otherwise)
+  auto read_a = [&](auto st, auto ks_tag, auto f_tag) -> u32x4 {
+    constexpr int KS = decltype(ks_tag)::value, F = decltype(f_tag)::value;
+    if constexpr (M16) {
+      constexpr int ST = decltype(st)::value;
+      return *reinterpret_cast<const lds_u32x4*>(static_cast<uintptr_t>(base_a[ST][((4 * KS) ^ (2 * F)) >> 1 & 3] + F * 2048));
+    } else {
+      return *reinterpret_cast<const u32x4*>(lds + static_cast<int>(st) * STAGE_BYTES + (off_a[F] ^ (KS << 5)));
     }
-    else fa[set][r - WN] = *reinterpret_cast<const u32x4*>(tile + (off_a[r - WN] ^ (ks << 5)));
   };
-  auto read_frags = [&](int set, const char* tile, int ks) {
-    static_for<N_READ>([&](auto cr) { read_frag(set, tile, ks, cr); });
+  auto read_b = [&](auto st, auto ks_tag, auto f_tag) -> u32x4 {
+    constexpr int KS = decltype(ks_tag)::value, F = decltype(f_tag)::value;
+    if constexpr (load_is_ntr(LOAD_B)) {
+      // k-step KS covers rows 16 KS .. + 15 (16x16: 32 KS .. + 31) of the tile; the two reads give k 0-3 and
+      // 4-7 of the lane's chunk
+      if constexpr (M16) {
+        constexpr int ST = decltype(st)::value;
+        const uint32_t at = base_b[ST][F >> 1] + (F & 1) * 32 + KS * 32 * PITCH_NTR;
+        const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_s16x4*>(static_cast<uintptr_t>(at))));
+        const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_s16x4*>(static_cast<uintptr_t>(at + 4 * PITCH_NTR))));
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+      } else {
+        const char* at = lds + static_cast<int>(st) * STAGE_BYTES + off_b[F] + KS * 16 * PITCH_NTR;
+        const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at)));
+        const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * PITCH_NTR)));
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+      }
+    } else if constexpr (M16) {
+      constexpr int ST = decltype(st)::value;
+      return *reinterpret_cast<const lds_u32x4*>(static_cast<uintptr_t>(base_b[ST][((4 * KS) ^ (2 * F)) >> 1 & 3] + F * 2048));
+    } else {
+      return *reinterpret_cast<const u32x4*>(lds + static_cast<int>(st) * STAGE_BYTES + (off_b[F] ^ (KS << 5)));
+    }
+  };
+  auto read_frag = [&](int set, auto st_tag, auto ks_tag, auto r_tag) {
+    constexpr int r = decltype(r_tag)::value;
+    if constexpr (r == 0) fa[set][0] = read_a(st_tag, ks_tag, std::integral_constant<int, 0>{});
+    else if constexpr (r <= FN) fb[set][r - 1] = read_b(st_tag, ks_tag, std::integral_constant<int, r - 1>{});
+    else fa[set][r - FN] = read_a(st_tag, ks_tag, std::integral_constant<int, r - FN>{});
+  };
+  auto read_frags = [&](int set, auto st_tag, auto ks_tag) {
+    static_for<N_READ>([&](auto cr) { read_frag(set, st_tag, ks_tag, cr); });
   };
   // workgroup barrier that waits only for this wave's LDS traffic, not for the
   // global prefetch in flight
@@ -1663,7 +1820,7 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
 
   using SA = decltype(stager_a);
   using SB = decltype(stager_b);
-  using Sched = StagingSchedule<SA, SB, LOAD_B == LOAD_NVEC>;
+  using Sched = StagingSchedule<SA, SB, LOAD_B == LOAD_NVEC, M16 && load_is_dma(LOAD_A)>;
 
   // Start of the pipeline: tile 0 into the staging registers and, without waiting
   // for it, tile 1 into a spare set (position 1 is never the partial tile: one
@@ -1681,6 +1838,15 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
       } else {
         stager_a.stage_checked(first, lds);
         stager_b.stage_checked(first, lds + BM * 128);
+      }
+      if constexpr (M16) {
+        // the loop of the 16x16 shapes loads two tiles ahead: the second tile (never the partial one) goes into
+        // stage 1 here
+        if (nk - has_tail > 0) {
+          const int second = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(1, nk - 1)));
+          stager_a.dma_full(second, lds + STAGE_BYTES);
+          stager_b.dma_full(second, lds + STAGE_BYTES + BM * 128);
+        }
       }
     }
   } else if constexpr (!DMA) {
@@ -1717,13 +1883,8 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
    }
   }
 
-  Acc acc[WM][WN];
-#pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  Accumulators<INT, WM, WN, M16> acc;
+  acc.clear();
 
   if (nk > 0) {
     const int full_in_range = nk - has_tail;  // whole K tiles this workgroup owns
@@ -1731,50 +1892,66 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
     // merges the start-up's branches without knowing which conditions coincide, and would otherwise
     // carry loads "still in flight" into the loop and wait for them in every iteration.
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-    lds_barrier();  // tile 0 is in LDS
-    read_frags(0, lds, 0);
+    lds_barrier();  // tile 0 is in LDS (and tile 1, where the loop loads two tiles ahead)
+    read_frags(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
 
     // The loop body is one straight-line block: stores into the other stage,
     // prefetches (tile index clamped to the last one) and the fragment reads of the
     // next tile are issued unconditionally; the surplus ones of the final
     // iterations touch valid memory and are never consumed.
     const uint32_t lds_address = lds_address_of(lds);
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
     auto main_loop = [&](auto prefetch_tag) {
       constexpr bool PREFETCH = decltype(prefetch_tag)::value;
-      for (int it = 0; it < nk; ++it) {
-        const char* tile = lds + (it & 1) * STAGE_BYTES;
-        char* other = lds + ((it & 1) ^ 1) * STAGE_BYTES;
-        const uint32_t other_address = lds_address + ((it & 1) ^ 1) * STAGE_BYTES;  // what the loads that write LDS put into M0
+      // One K tile, which lies in stage `this_stage`: an integral constant under the 16x16 shapes (the loop below is
+      // written out for both stages, which makes every fragment address a register plus a constant) and it & 1
+      // otherwise (written out twice, the 32x32 loop loses more to the copies the register allocator then makes
+      // between its two sets of accumulator registers: int8 4096^3 86 us against 70)
+      auto k_tile = [&](auto this_stage, int it) {
+        const int ST = this_stage;
+        auto other_stage = [&]() {
+          if constexpr (std::is_integral<decltype(this_stage)>::value) return this_stage ^ 1;
+          else return std::integral_constant<int, decltype(this_stage)::value ^ 1>{};
+        }();
+        char* other = lds + (ST ^ 1) * STAGE_BYTES;
+        const uint32_t other_address = lds_address + (ST ^ 1) * STAGE_BYTES;  // what the loads that write LDS put into M0
         // K tile to prefetch: seq(min(it + 2, nk - 1)), never the tail tile (position 0)
         // (loads that write LDS fetch the next tile, into the other stage)
-        const int t2 = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(it + (DMA ? 1 : 2), nk - 1)));
+        const int t2 = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(it + (DMA && !M16 ? 1 : 2), nk - 1)));
+        // (the 16x16 loop's loads that write LDS fetch the tile after the next, behind the barrier, into this stage)
+        const uint32_t load_address = (DMA && M16) ? lds_address + ST * STAGE_BYTES : other_address;
 
         auto stage_op = [&](auto step_tag, auto g_tag, auto order_tag) {
           constexpr StagingOp o = Sched::op(decltype(step_tag)::value, decltype(g_tag)::value, decltype(order_tag)::value);
           // (a stager whose loads write LDS has no store operations; the others ignore the load's LDS address)
           if constexpr (o.operand == 0 && o.is_load == 0) stager_a.template store_op<o.part, o.op>(other);
-          if constexpr (o.operand == 0 && o.is_load == 1 && PREFETCH) stager_a.template load_op<o.part, o.op>(t2, other_address);
+          if constexpr (o.operand == 0 && o.is_load == 1 && PREFETCH) stager_a.template load_op<o.part, o.op>(t2, load_address);
           if constexpr (o.operand == 1 && o.is_load == 0) stager_b.template store_op<o.part, o.op>(other + BM * 128);
-          if constexpr (o.operand == 1 && o.is_load == 1 && PREFETCH) stager_b.template load_op<o.part, o.op>(t2, other_address + BM * 128);
+          if constexpr (o.operand == 1 && o.is_load == 1 && PREFETCH) stager_b.template load_op<o.part, o.op>(t2, load_address + BM * 128);
         };
-        // Slots [S0, S1) of k-step STEP: MFMA x on fragment set mfma_set, then this
-        // slot's share of the N_RD fragment reads (k-step read_ks of read_tile into
-        // the other set; dealt front-biased) and of the step's staging operations
-        // (if STAGE).
-        auto slots = [&](auto step_tag, auto s0_tag, auto s1_tag, auto nrd_tag, auto stage_tag, auto order_tag,
-                         int mfma_set, const char* read_tile, int read_ks) {
+        // Slots [S0, S1) of a k-step: MFMA x on fragment set mfma_set, then this
+        // slot's share of the fragment reads RD0 .. RD0 + N_RD - 1 (k-step read_ks of
+        // stage read_st into the other set; dealt front-biased) and of the staging
+        // operations of phase STEP of the K tile (if STAGE).
+        auto slots = [&](auto step_tag, auto s0_tag, auto s1_tag, auto rd0_tag, auto nrd_tag, auto stage_tag,
+                         auto order_tag, int mfma_set, auto read_st, auto read_ks) {
           constexpr int STEP = decltype(step_tag)::value, S0 = decltype(s0_tag)::value, S1 = decltype(s1_tag)::value;
-          constexpr int NS = S1 - S0, N_RD = decltype(nrd_tag)::value;
+          constexpr int NS = S1 - S0, RD0 = decltype(rd0_tag)::value, N_RD = decltype(nrd_tag)::value;
           constexpr int G = decltype(stage_tag)::value ? Sched::ops(STEP) : 0;
           if constexpr (NS == 0) {
             static_for<G>([&](auto cg) { stage_op(step_tag, cg, order_tag); });
           }
           static_for<NS>([&](auto ci) {
             constexpr int i = decltype(ci)::value, x = S0 + i;
-            mfma_step<SRC>(acc[x / WN][x % WN], fb[mfma_set][x % WN], fa[mfma_set][x / WN]);  // B rows first: see the epilogue
+            // B rows first: see the epilogue
+            if constexpr (M16) mfma_step16<SRC>(acc.t[x / FN][x % FN], fb[mfma_set][x % FN], fa[mfma_set][x / FN]);
+            else mfma_step<SRC>(acc.t[x / FN][x % FN], fb[mfma_set][x % FN], fa[mfma_set][x / FN]);
             constexpr int r0 = (i * N_RD + NS - 1) / NS, r1 = ((i + 1) * N_RD + NS - 1) / NS;
             static_for<r1 - r0>([&](auto cr) {
-              read_frag(mfma_set ^ 1, read_tile, read_ks, std::integral_constant<int, r0 + decltype(cr)::value>{});
+              read_frag(mfma_set ^ 1, read_st, read_ks, std::integral_constant<int, RD0 + r0 + decltype(cr)::value>{});
             });
             constexpr int g0 = i * G / NS, g1 = (i + 1) * G / NS;
             static_for<g1 - g0>([&](auto cg) {
@@ -1783,33 +1960,70 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
             __builtin_amdgcn_sched_barrier(0);
           });
         };
-        using I0 = std::integral_constant<int, 0>;
-        using I1 = std::integral_constant<int, 1>;
-        using I2 = std::integral_constant<int, 2>;
-        using I3 = std::integral_constant<int, 3>;
         using All = std::integral_constant<int, N_MFMA>;
         using Half = std::integral_constant<int, N_MFMA / 2>;
         using Reads = std::integral_constant<int, N_READ>;
 
-        slots(I0{}, I0{}, All{}, Reads{}, std::true_type{}, std::false_type{}, 0, tile, 1);
-        slots(I1{}, I0{}, All{}, Reads{}, std::true_type{}, std::false_type{}, 1, tile, 2);
-        slots(I2{}, I0{}, All{}, Reads{}, std::true_type{}, std::false_type{}, 0, tile, 3);
-        slots(I3{}, I0{}, Half{}, I0{}, std::true_type{}, std::true_type{}, 1, tile, 0);
-        if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the next tile has landed in the other stage
-        lds_barrier();
-        slots(I3{}, Half{}, All{}, Reads{}, std::false_type{}, std::false_type{}, 1, other, 0);
+        if constexpr (!M16) {
+          slots(I0{}, I0{}, All{}, I0{}, Reads{}, std::true_type{}, std::false_type{}, 0, this_stage, I1{});
+          slots(I1{}, I0{}, All{}, I0{}, Reads{}, std::true_type{}, std::false_type{}, 1, this_stage, I2{});
+          slots(I2{}, I0{}, All{}, I0{}, Reads{}, std::true_type{}, std::false_type{}, 0, this_stage, I3{});
+          slots(I3{}, I0{}, Half{}, I0{}, I0{}, std::true_type{}, std::true_type{}, 1, this_stage, I0{});
+          if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the next tile has landed in the other stage
+          lds_barrier();
+          slots(I3{}, Half{}, All{}, I0{}, Reads{}, std::false_type{}, std::false_type{}, 1, other_stage, I0{});
+        } else if constexpr (DMA) {
+          // Two k-steps of N_MFMA short MFMAs.  Every fragment of the tile's second k-step is read during the
+          // first, so the barrier stands between the two: behind it this stage is free for the loads of the tile
+          // after the next, and the other stage, complete since those loads were issued half a K tile ago, gives
+          // the next tile's first fragments.
+          using ReadsLo = std::integral_constant<int, N_READ / 2>;
+          using ReadsHi = std::integral_constant<int, N_READ - N_READ / 2>;
+          using I4 = std::integral_constant<int, 4>;
+          using I5 = std::integral_constant<int, 5>;
+          slots(I0{}, I0{}, Half{}, I0{}, ReadsLo{}, std::false_type{}, std::false_type{}, 0, this_stage, I1{});
+          slots(I1{}, Half{}, All{}, ReadsLo{}, ReadsHi{}, std::false_type{}, std::false_type{}, 0, this_stage, I1{});
+          __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the next tile has landed in the other stage
+          lds_barrier();
+          slots(I4{}, I0{}, Half{}, I0{}, ReadsLo{}, std::true_type{}, std::false_type{}, 1, other_stage, I0{});
+          slots(I5{}, Half{}, All{}, ReadsLo{}, ReadsHi{}, std::true_type{}, std::false_type{}, 1, other_stage, I0{});
+        } else {
+          // Register staging under the 16x16 shapes: the four phases of the staging schedule are the halves of
+          // the two k-steps, and the barrier stands behind the last phase's stores.
+          using ReadsLo = std::integral_constant<int, N_READ / 2>;
+          using ReadsHi = std::integral_constant<int, N_READ - N_READ / 2>;
+          using Late = std::integral_constant<int, N_MFMA / 2 + N_MFMA / 4>;
+          slots(I0{}, I0{}, Half{}, I0{}, ReadsLo{}, std::true_type{}, std::false_type{}, 0, this_stage, I1{});
+          slots(I1{}, Half{}, All{}, ReadsLo{}, ReadsHi{}, std::true_type{}, std::false_type{}, 0, this_stage, I1{});
+          slots(I2{}, I0{}, Half{}, I0{}, I0{}, std::true_type{}, std::false_type{}, 1, this_stage, I0{});
+          slots(I3{}, Half{}, Late{}, I0{}, I0{}, std::true_type{}, std::true_type{}, 1, this_stage, I0{});
+          lds_barrier();
+          slots(I3{}, Late{}, All{}, I0{}, Reads{}, std::false_type{}, std::false_type{}, 1, other_stage, I0{});
+        }
+      };
+      if constexpr (M16) {
+        int it = 0;
+        for (; it + 1 < nk; it += 2) {
+          k_tile(I0{}, it);
+          k_tile(I1{}, it + 1);
+        }
+        if (it < nk) k_tile(I0{}, it);
+      } else {
+        for (int it = 0; it < nk; ++it) k_tile(it & 1, it);
       }
     };
     if (full_in_range > 0) main_loop(std::true_type{});
     else main_loop(std::false_type{});
+    // (the last trips' surplus loads into LDS must have landed before the epilogue lays C out there)
+    if constexpr (DMA && M16) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   }
 
-  store_accumulators<SRC, WAVES_M, WAVES_N, WM, WN, kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>()>(
+  store_accumulators<SRC, WAVES_M, WAVES_N, WM, WN, kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>(), M16>(
       p, lds, acc, batch, split, m0, n0, wm, wn, wave, lane);
 }
 
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const TileGemmParams p) {
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (kShortMfma<SRC, WM, WN> ? 2 : 1)) void tile_gemm_kernel(const TileGemmParams p) {
   tile_gemm_workgroup<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_A, LOAD_B>(p, blockIdx.x, gridDim.x);
 }
 
@@ -1818,7 +2032,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_kernel(const
 // serve group g (each run a multiple of eight long, so that a group's workgroups are dealt to the XCDs like a
 // launch of its own); group_of[w] names the group of workgroup w.  No group splits K.
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_grouped_kernel(
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (kShortMfma<SRC, WM, WN> ? 2 : 1)) void tile_gemm_grouped_kernel(
     const int32_t* __restrict__ group_of, const int32_t* __restrict__ first, const TileGemmParams* __restrict__ groups) {
   const int g = __builtin_amdgcn_readfirstlane(group_of[blockIdx.x]);
   const TileGemmParams p = groups[g];

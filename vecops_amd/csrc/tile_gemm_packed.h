@@ -214,7 +214,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
    }
   }
 
-  Acc acc[WM][WN];
+  Accumulators<INT, WM, WN, false> accumulators;  // prepacked fragments are those of the 32x32 shapes
+  auto& acc = accumulators.t;
 #pragma unroll
   for (int i = 0; i < WM; ++i)
 #pragma unroll
@@ -299,7 +300,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void tile_gemm_packed_b_ker
     else main_loop(std::false_type{});
   }
 
-  store_accumulators<SRC, WAVES_M, WAVES_N, WM, WN, kLdsBytes>(p, lds, acc, batch, split, m0, n0, wm, wn, wave, lane);
+  store_accumulators<SRC, WAVES_M, WAVES_N, WM, WN, kLdsBytes, false>(p, lds, accumulators, batch, split, m0, n0, wm, wn, wave,
+                                                                      lane);
 }
 
 }  // namespace vecops_hip
