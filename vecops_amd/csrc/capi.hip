@@ -334,9 +334,10 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
   // half the compute units busy; among those the cheapest wins, cost = rounds x tile area / quality -
   // so a part-filled last round, rows or columns of padding and a less efficient small tile are all
   // priced in one number (4096^3: 256 tiles of 256x256, one round; 2048x11008: 344 of them in two rounds, which
-  // 1376 tiles of 128x128 in six undercut - measured 117 us against 105, 119 for the 688 rectangles; 4096x4224:
-  // 1056 tiles of 128x128, 160 us against 172 for 272 big ones whose second round is 6 % full; 8 x 777x1000: 224
-  // tiles of 128x256 in one round; 5120^3, 2048x14336x4096, 8192^3: big tiles, 19-23 % ahead).
+  // 1376 tiles of 128x128 in three undercut - int8 measured 117-123 us against 92-97, 115-123 for the 688
+  // rectangles; 4096x4224: 1056 tiles of 128x128, 151 us against 176 for 272 big ones whose second round is 6 % full;
+  // 8 x 777x1000: 224 tiles of 128x256 in one round; 3072x4096x4096, 5120^3, 2048x14336x4096, 8192^3: big tiles,
+  // 7-15 % ahead for bf16 and 3-6 % for int8).
   struct Candidate { uint32_t family; int64_t tm, tn, quality; };
   const bool bytes = pr.src == SRC_I8 || pr.src == SRC_I8_FLIP;
   const int mode = fetch_mode(pr, *plan);

@@ -1746,6 +1746,7 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
   auto seq = [&](int j) { return (has_tail && j == 0) ? kt_end - 1 : kt_begin + j - has_tail; };
 
   // Software pipeline over K tiles, two LDS stages, two fragment register sets.
+  // (32x32 shapes; the 16x16 shapes' two k-steps follow the same plan, see the loop.)
   // K tile `it` is multiplied in four k-steps; k-step s
   //   * reads the fragments of k-step s+1 (for s = 3: of k-step 0 of tile it+1, from
   //     the other stage, after the barrier),
