@@ -233,9 +233,10 @@ constexpr int kStreamGroupsPerUnit = 2;  // workgroups of 4 wavefronts per compu
 // 128x128; two 128x128 workgroups share a compute unit), 5120^3 221 / 309 / 307 / 255, 2048 x 14336 x 4096
 // 185 / 247 / 246 / 204; int8 4096^3 70 / 83 / 84 / 71.5, 5120^3 142 / 184 / 192 / 150, 2048 x 14336 x 4096
 // 123 / 153 / 159 / 127.
-// Operands whose rows are not 16-byte aligned go through registers into LDS, work that grows with a tile's
-// perimeter: 8 x 777 x 1000 x 3001 takes 64 us on 128x256 tiles and 73.5 on 128x128.
-constexpr int64_t kQuality256x128 = 800, kQuality128 = 900, kQuality128Int8 = 970, kQuality128Staged = 780;
+// Operands that go through registers into LDS (rows that are not 16-byte aligned, fp32 memory, unsigned bytes) keep
+// the pricing their kernels were calibrated with: 0.85, rounds of 256, and the margin of the rectangles (8 x 777 x
+// 1000 x 3001 64 us on 128x256 tiles against 73.5 on 128x128; fp32 memory 2048^3 32 us on 128x128 against 43).
+constexpr int64_t kQuality256x128 = 800, kQuality128 = 900, kQuality128Int8 = 970, kQuality128Staged = 850;
 
 // Every operand class but the unsigned bytes, with K contiguous on both sides, no C input, one side <= 16 rows, the
 // other >= 512 (vecops' small-vector leaves serve every atom, matmul/details/kernel/amx/Backend.h:767-992)
@@ -355,7 +356,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     if (count < kComputeUnits / 2) continue;
     // two 128x128 workgroups live on a compute unit at a time (64 KiB of LDS and at most 256 registers each): a
     // round of them is 512 tiles
-    const int64_t per_unit = c.family == VECOPS_HIP_FAMILY_TILE_128 ? 2 : 1, slots = per_unit * kComputeUnits;
+    const int64_t per_unit = c.family == VECOPS_HIP_FAMILY_TILE_128 && direct ? 2 : 1, slots = per_unit * kComputeUnits;
     const int64_t rounds = (count + slots - 1) / slots;
     int64_t cost = rounds * per_unit * c.tm * c.tn * 1000 / c.quality;
     // a single part-filled round runs faster than a full one (the chip is power-limited: fewer busy compute units
@@ -365,7 +366,8 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     // a rectangle has to be 10 % cheaper than the big tile: the round count flatters it (more L2 traffic per flop,
     // and its quality falls with the problem size).  The 128x128 tile competes on its cost alone (1536 x 4096 x 4096:
     // 49 us against 60 for the rectangles, 2048 x 4096 x 4096 58 against 67; int8 31 against 38 and 36 against 42).
-    const bool smaller = best_cost != INT64_MAX && c.tm * c.tn < tile_m * tile_n && c.family != VECOPS_HIP_FAMILY_TILE_128;
+    const bool smaller = best_cost != INT64_MAX && c.tm * c.tn < tile_m * tile_n &&
+                         !(c.family == VECOPS_HIP_FAMILY_TILE_128 && direct);
     if (best_cost == INT64_MAX || (smaller ? cost * 11 < best_cost * 10 : cost < best_cost)) {
       best_cost = cost;
       family = c.family;
