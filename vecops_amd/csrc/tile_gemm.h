@@ -1099,10 +1099,14 @@ struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
       row_bytes[i] = static_cast<uint32_t>((static_cast<int64_t>(row) * rs + chunk * T::kElemsPerChunk) * T::kSrcBytes);
     }
   }
-  // lds_tile: LDS address of the operand's tile (lds_address_of)
+  // lds_tile: LDS address of the operand's tile (lds_address_of).  kt < 0: a load that fetches nothing (a buffer of
+  // no records: every lane is out of range, zeros land in LDS and no memory is touched) - for the trips of a loop
+  // that loads ahead of the last tile.
   __device__ __forceinline__ void dma_part(int part, int kt, uint32_t lds_tile) const {
-    load_16_bytes_into_lds(tile_buf, lds_tile, __builtin_amdgcn_readfirstlane((part * ROWS_PER_PASS + wave_ * 8) * 128),
-                           row_bytes[part], kt * (8 * T::kElemsPerChunk * T::kSrcBytes));
+    u32x4 buf = tile_buf;
+    buf[2] = kt < 0 ? 0u : buf[2];
+    load_16_bytes_into_lds(buf, lds_tile, __builtin_amdgcn_readfirstlane((part * ROWS_PER_PASS + wave_ * 8) * 128),
+                           row_bytes[part], max(kt, 0) * (8 * T::kElemsPerChunk * T::kSrcBytes));
   }
   __device__ __forceinline__ void dma_full(int kt, char* lds_tile) const {
     const uint32_t address = lds_address_of(lds_tile);
@@ -1170,8 +1174,10 @@ struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
   __device__ __forceinline__ uint32_t part_offset(int part) const {
     return __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(part * K_ROWS_PER_PART * ks * T::kSrcBytes));
   }
+  // (kt < 0: a load that fetches nothing, as in the K-contiguous stager)
   __device__ __forceinline__ void dma_part(int part, int kt, uint32_t lds_tile) const {
-    const u32x4 buf = tile_buffer_words(tile_base + static_cast<int64_t>(kt) * 64 * ks * T::kSrcBytes);
+    u32x4 buf = tile_buffer_words(tile_base + static_cast<int64_t>(max(kt, 0)) * 64 * ks * T::kSrcBytes);
+    buf[2] = kt < 0 ? 0u : buf[2];
     load_16_bytes_into_lds(buf, lds_tile, __builtin_amdgcn_readfirstlane((part * THREADS + wave_ * 64) * 16), chunk_bytes,
                            part_offset(part));
   }
@@ -1843,8 +1849,8 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
       if constexpr (M16) {
         // the loop of the 16x16 shapes loads two tiles ahead: the second tile (never the partial one) goes into
         // stage 1 here
-        if (nk - has_tail > 0) {
-          const int second = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(1, nk - 1)));
+        if (nk > 1) {
+          const int second = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + 1);
           stager_a.dma_full(second, lds + STAGE_BYTES);
           stager_b.dma_full(second, lds + STAGE_BYTES + BM * 128);
         }
@@ -1921,8 +1927,12 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
         const uint32_t other_address = lds_address + (ST ^ 1) * STAGE_BYTES;  // what the loads that write LDS put into M0
         // K tile to prefetch: seq(min(it + 2, nk - 1)), never the tail tile (position 0)
         // (loads that write LDS fetch the next tile, into the other stage)
-        const int t2 = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(it + (DMA && !M16 ? 1 : 2), nk - 1)));
-        // (the 16x16 loop's loads that write LDS fetch the tile after the next, behind the barrier, into this stage)
+        // (the 16x16 loop's loads that write LDS fetch the tile after the next, behind the barrier, into this stage;
+        // on the last trips of either loop there is no such tile, and loads that write LDS fetch nothing)
+        constexpr int AHEAD = DMA && !M16 ? 1 : 2;
+        const int t2 = (DMA && it + AHEAD >= nk)
+                           ? -1
+                           : __builtin_amdgcn_readfirstlane(kt_begin - has_tail + max(has_tail, min(it + AHEAD, nk - 1)));
         const uint32_t load_address = (DMA && M16) ? lds_address + ST * STAGE_BYTES : other_address;
 
         auto stage_op = [&](auto step_tag, auto g_tag, auto order_tag) {
