@@ -320,6 +320,7 @@ def bench_bf16_gemm_packed(dev, steps, warmup):
     _, _, ta, tb = _bf16_operands(dev)
     packed = capi.pack_b(tb.t())
     c = torch.empty((n, n), dtype=torch.bfloat16, device=dev)
+    family = capi.FAMILY_NAMES.get(capi.plan_matmul_packed_b(ta, packed, c).family)
     t = _measure(lambda i: capi.matmul_packed_b(ta, packed, c), steps, warmup)
     flops = 2.0 * n * n * n
     tflops = flops / (t["event_ms"] * 1e-3) / 1e12
@@ -327,7 +328,7 @@ def bench_bf16_gemm_packed(dev, steps, warmup):
             "(vecops_hip_pack_b, not timed), fp32 accumulate, bf16 out", "value": tflops, "unit": "TFLOP/s",
             "ms_per_step": t["wall_ms"], "dtype": "bf16",
             "roofline": _roofline("mfma", tflops, PEAK_BF16_TFLOPS, "TFLOP/s",
-                                  kernel="vecops_hip tile_gemm_packed_b_kernel<bf16> family tile_256",
+                                  kernel=f"vecops_hip tile_gemm_packed_b_kernel<bf16> family {family}",
                                   algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=3 * 2 * n * n,
                                   **_traffic("bf16_packed"), **_timing_fields(t))}
 
@@ -343,6 +344,7 @@ def bench_int8_dequant_packed(dev, steps, warmup):
     c = torch.empty((m, n), dtype=torch.float32, device=dev)
     need = capi.lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k)
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    family = capi.FAMILY_NAMES.get(capi.plan_matmul_packed_b(a, packed, torch.empty((m, n), dtype=torch.int32, device=dev)).family)
     t = _measure(lambda i: capi.matmul_i8_dequant_packed_b(a, packed, rs, cs, c, workspace=ws), steps, warmup)
     ops = 2.0 * m * n * k
     tops = ops / (t["event_ms"] * 1e-3) / 1e12
@@ -350,7 +352,7 @@ def bench_int8_dequant_packed(dev, steps, warmup):
             "(not timed), per-token x per-channel dequant fused, fp32 out", "value": tops, "unit": "TOP/s",
             "ms_per_step": t["wall_ms"], "dtype": "int8",
             "roofline": _roofline("mfma", tops, PEAK_INT8_TOPS, "TOP/s",
-                                  kernel="vecops_hip tile_gemm_packed_b_kernel<int8> family tile_256, dequantising epilogue",
+                                  kernel=f"vecops_hip tile_gemm_packed_b_kernel<int8> family {family}, dequantising epilogue",
                                   algorithmic_ops_per_launch=ops,
                                   algorithmic_bytes_per_launch=m * k + n * k + 4 * m * n + 4 * (m + n),
                                   **_traffic("int8_packed"), **_timing_fields(t))}
