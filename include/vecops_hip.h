@@ -411,8 +411,9 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul_packed_b(const VecopsHipOperand
  *   packed i8  : a i8 or u8 (AMX_I8I32<uint8_t, int8_t>, the atom the compensated pack serves,
  *                ops/MatmulPack.h:52-58; the workspace then also holds 4 * batch * (M + N) bytes), c i32
  *   packed u8  : a i8 or u8, c i32 (the same workspace term)
- * Same results, bit for bit, as vecops_hip_matmul on the unpacked operand when
- * that runs its tile kernels.
+ * Integer results are those of vecops_hip_matmul on the unpacked operand, bit for bit; floating-point results too
+ * when that call runs its 256-row or 256-column tiles with the same split of K (the packed kernels multiply on the
+ * 32x32 matrix instructions, the small plain tiles on the 16x16 ones: the fp32 sums are then taken in another order).
  */
 VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_packed_b(const VecopsHipOperand* a, const void* packed_b,
                                                      uint32_t packed_dtype, int64_t n, const VecopsHipOperand* c_in,
