@@ -180,10 +180,11 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_static_workspace(const VecopsHipOper
  * flattening them into one product (planning/families/ArchitectureBatchPlanner.h:30-160; vecops_hip_matmul does the
  * same) and everything else batch by batch; this entry point is the form for batches that share nothing, not even
  * their shapes.  a, b, c (and c_in, which may be null; an entry of rank 0 means "no C input for this group") are
- * arrays of count descriptors obeying the rules of vecops_hip_matmul group by group.  Groups of bf16 x bf16 or
- * int8 x int8 operands run as ONE launch over a table of problem records (written into the workspace by small
- * kernels fed through their arguments: no host buffer has to outlive the call, nothing is allocated); any other
- * operand class, a mix of classes, and groups with K = 0 run as launches of their own on the same stream.  Results
+ * arrays of count descriptors obeying the rules of vecops_hip_matmul group by group.  Groups of one operand
+ * class - bf16, f16, int8 x int8, or fp32 in either compute type - run as ONE launch over a table of problem
+ * records (written into the workspace by small kernels fed through their arguments: no host buffer has to outlive
+ * the call, nothing is allocated); unsigned 8-bit and fp64 operands, a mix of classes, and groups with K = 0 run as
+ * launches of their own on the same stream.  Results
  * are those of vecops_hip_matmul on each group (bit-equal when that call runs the same tile shape without splitting K;
  * otherwise equal up to the order of the fp32 sums - integer results are always the same bits).  workspace: vecops_hip_matmul_grouped_workspace bytes, 16-byte aligned.
  */

@@ -139,21 +139,61 @@ def test_grouped_mixed_layouts_and_unaligned_operands(device, oracle):
             assert torch.isnan(stores[i][m:]).all() and torch.isnan(stores[i][:, n:]).all()
 
 
-def test_grouped_other_classes_run_group_by_group(device, oracle):
-    """fp32 operands (no grouped kernel instance) and a mix of classes: the same entry point, launches of their own."""
+@pytest.mark.parametrize("kind", ["f32_as_bf16", "f32", "f16"])
+def test_grouped_floating_classes_in_one_launch(device, oracle, kind):
+    """fp32 operands in both compute types and f16 operands: groups of unlike shapes (ragged, a C input on every
+    other one, enough tiles for the 128 x 128 shape) through the grouped launch, each against the oracle and
+    bit-equal to the single call on one of the three square tile shapes, K unsplit."""
     import torch
-    from oracle import oracle as O
     from vecops_amd import capi
-    a0, b0 = synth.uniform_pm1(1, (70, 200)), synth.uniform_pm1(2, (90, 200))
-    a1, b1 = synth.uniform_pm1(3, (300, 64)), synth.uniform_pm1(4, (20, 64))
-    c0 = torch.full((70, 90), float("nan"), device=device)
-    c1 = torch.full((300, 20), float("nan"), device=device)
-    capi.matmul_grouped([torch.from_numpy(a0).to(device), torch.from_numpy(a1).to(device)],
-                        [torch.from_numpy(b0).to(device), torch.from_numpy(b1).to(device)], [c0, c1], compute=capi.COMPUTE_F32)
+    shapes = [(70, 90, 200), (300, 20, 64), (1000, 1300, 136), (700, 900, 264), (1, 33, 40), (513, 257, 96)]
+    compute = capi.COMPUTE_F32 if kind == "f32" else capi.COMPUTE_BF16
+    ha, hb, hci, ta, tb, tc, tci = [], [], [], [], [], [], []
+    for i, (m, n, k) in enumerate(shapes):
+        a, b = synth.uniform_pm1(10 + i, (m, k)), synth.uniform_pm1(50 + i, (n, k))
+        if kind == "f16":
+            a, b = a.astype(np.float16), b.astype(np.float16)
+        ha.append(a)
+        hb.append(b)
+        hci.append(synth.uniform_pm1(90 + i, (m, n)).astype(np.float32) if i % 2 else None)
+        ta.append(torch.from_numpy(a).to(device))
+        tb.append(torch.from_numpy(b).to(device))
+        tci.append(torch.from_numpy(hci[-1]).to(device) if hci[-1] is not None else None)
+        tc.append(torch.full((m, n), float("nan"), dtype=torch.float32, device=device))
+    capi.matmul_grouped(ta, tb, tc, c_in_list=tci, compute=compute)
     torch.cuda.synchronize()
-    for a, b, c in ((a0, b0, c0), (a1, b1, c1)):
-        want = a.astype(np.float64) @ b.astype(np.float64).T
-        assert rel_err(c.cpu().numpy(), want) <= fp32_tol(a.shape[1])
+    for i, (m, n, k) in enumerate(shapes):
+        if kind == "f32_as_bf16":   # operands rounded to bf16 on the way in, products and sums in fp32
+            a64, b64 = (synth.bf16_to_f32(synth.bf16_round(x)).astype(np.float64) for x in (ha[i], hb[i]))
+        else:
+            a64, b64 = ha[i].astype(np.float64), hb[i].astype(np.float64)
+        want = a64 @ b64.T + (hci[i] if hci[i] is not None else 0.0)
+        assert rel_err(tc[i].cpu().numpy(), want) <= fp32_tol(k), (kind, i)
+        same_bits = []
+        for family in ("tile_256", "tile_128", "tile_64"):
+            alone = torch.empty_like(tc[i])
+            capi.matmul_family(ta[i], tb[i], alone, capi.family_request(family, split_k=1), c_in=tci[i], compute=compute)
+            torch.cuda.synchronize()
+            same_bits.append(np.array_equal(tc[i].cpu().numpy(), alone.cpu().numpy()))
+        assert any(same_bits), (kind, i)
+
+
+def test_grouped_other_classes_run_group_by_group(device, oracle):
+    """Unsigned 8-bit operands (their sign flip needs a pass of its own) and a mix of classes: the same entry point,
+    launches of their own."""
+    import torch
+    from vecops_amd import capi
+    def u8(seed, shape):
+        return (synth.int8_sym(seed, shape).astype(np.int16) + 128).astype(np.uint8)
+    ua, ub = u8(1, (70, 200)), synth.int8_sym(2, (90, 200))
+    va, vb = u8(3, (300, 64)), u8(4, (20, 64))
+    c0 = torch.zeros((70, 90), dtype=torch.int32, device=device)
+    c1 = torch.zeros((300, 20), dtype=torch.int32, device=device)
+    capi.matmul_grouped([torch.from_numpy(ua).to(device), torch.from_numpy(va).to(device)],
+                        [torch.from_numpy(ub).to(device), torch.from_numpy(vb).to(device)], [c0, c1])
+    torch.cuda.synchronize()
+    for a, b, c in ((ua, ub, c0), (va, vb, c1)):
+        assert np.array_equal(c.cpu().numpy(), (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.int32))
     # a bf16 group beside an int8 group
     ha, hb = synth.bf16_round(synth.uniform_pm1(5, (100, 72))), synth.bf16_round(synth.uniform_pm1(6, (50, 72)))
     ia, ib = synth.int8_sym(7, (60, 144)), synth.int8_sym(8, (40, 144))

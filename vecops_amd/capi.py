@@ -393,8 +393,8 @@ def matmul_runtime_quant_batched(a, multipliers, zero_point: int, scale_batch_st
 
 
 def matmul_grouped(a_list, b_list, c_list, c_in_list=None, compute: int = 0, workspace=None, stream=None):
-    """Several independent products ``c[i] = c_in[i] + a[i] . b[i]^T`` in one call (irregular batches): bf16 or int8
-    groups run as one launch.  ``c_in_list`` entries may be None."""
+    """Several independent products ``c[i] = c_in[i] + a[i] . b[i]^T`` in one call (irregular batches): groups of
+    one operand class (bf16, f16, int8, fp32) run as one launch.  ``c_in_list`` entries may be None."""
     import torch
     count = len(a_list)
     if not (len(b_list) == count and len(c_list) == count and (c_in_list is None or len(c_in_list) == count)):

@@ -1245,8 +1245,9 @@ __global__ __launch_bounds__(256) void expand_groups_kernel(const int32_t* __res
 namespace {
 // A grouped call: several independent products (irregular batches - every group with its own extents, strides and
 // pointers).  bf16 and int8 groups that all multiply run as ONE launch of tile_gemm_grouped_kernel over a table of
-// problem records in the workspace; other operand classes, and groups with K = 0, run as launches of their own on
-// the same stream.
+// problem records in the workspace (so do f16 groups and fp32 groups, in either compute type); unsigned 8-bit
+// operands (whose sign flip needs a pass over B first), fp64 operands, groups of mixed classes, and groups with K = 0, run as
+// launches of their own on the same stream.
 struct Grouped {
   std::vector<Problem> problems;
   std::vector<VecopsHipPlan> plans;
@@ -1278,7 +1279,7 @@ int32_t describe_grouped(uint32_t count, const VecopsHipOperand* a, const Vecops
     else if (g->src != g->problems[i].src) same_class = false;
     g->table_groups.push_back(static_cast<int>(i));
   }
-  g->one_launch = same_class && (g->src == SRC_BF16 || g->src == SRC_I8) && g->table_groups.size() > 1;
+  g->one_launch = same_class && g->src != SRC_I8_FLIP && g->src != kSrcF64 && g->table_groups.size() > 1;
   if (!g->one_launch) return ST_OK;
   // One workgroup tile for every group: the biggest square tile that still yields two rounds' worth of
   // workgroups over all groups together (priced like the rule table's candidates), else 64 x 64.
@@ -1403,7 +1404,13 @@ int32_t vecops_hip_matmul_grouped(uint32_t count, const VecopsHipOperand* a, con
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(ST_EXEC, "group map launch: %s", hipGetErrorString(e));
   GroupedTables t{group_of, first, records, workgroups};
-  e = g.src == SRC_BF16 ? launch_tile_gemm_grouped_bf16(t, g.tile, g.mode, s) : launch_tile_gemm_grouped_i8(t, g.tile, g.mode, s);
+  switch (g.src) {
+    case SRC_BF16: e = launch_tile_gemm_grouped_bf16(t, g.tile, g.mode, s); break;
+    case SRC_F16: e = launch_tile_gemm_grouped_f16(t, g.tile, g.mode, s); break;
+    case SRC_F32_AS_BF16: e = launch_tile_gemm_grouped_f32_as_bf16(t, g.tile, g.mode, s); break;
+    case SRC_F32: e = launch_tile_gemm_grouped_f32(t, g.tile, g.mode, s); break;
+    default: e = launch_tile_gemm_grouped_i8(t, g.tile, g.mode, s); break;
+  }
   if (e != hipSuccess) return fail(ST_EXEC, "grouped tile kernel launch: %s", hipGetErrorString(e));
   return ST_OK;
 }
