@@ -185,8 +185,8 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_static_workspace(const VecopsHipOper
  * records (written into the workspace by small kernels fed through their arguments: no host buffer has to outlive
  * the call, nothing is allocated); unsigned 8-bit and fp64 operands, a mix of classes, and groups with K = 0 run as
  * launches of their own on the same stream.  Results
- * are those of vecops_hip_matmul on each group (bit-equal when that call runs the same tile shape without splitting K;
- * otherwise equal up to the order of the fp32 sums - integer results are always the same bits).  workspace: vecops_hip_matmul_grouped_workspace bytes, 16-byte aligned.
+ * are those of vecops_hip_matmul on each group (bit-equal when that call runs the same tile shape without splitting K -
+ * except 16-bit products with K <= 256 on 128 x 128 tiles, where the single call takes the other MFMA shape; otherwise equal up to the order of the fp32 sums - integer results are always the same bits).  workspace: vecops_hip_matmul_grouped_workspace bytes, 16-byte aligned.
  */
 VECOPS_HIP_EXPORT uint64_t vecops_hip_matmul_grouped_workspace(uint32_t count, const VecopsHipOperand* a,
                                                                const VecopsHipOperand* b, const VecopsHipOperand* c_in,

@@ -44,7 +44,9 @@ BF16_GROUPS = {
 def test_grouped_bf16_equals_the_oracle_and_the_single_calls(device, oracle, name):
     """bf16 groups of unlike shapes in one launch: fp32 and bf16 outputs, every other group with a C input; each
     group against the oracle, and bit-equal to vecops_hip_matmul on that group alone on the tile shape the grouped
-    launch took (one of the three square ones), K unsplit: the same kernel body, the same order of sums."""
+    launch took (one of the three square ones), K unsplit: the same kernel body, the same order of sums.  (One
+    exception: with K of 256 or less the single call's 128 x 128 tile multiplies on the 32x32 MFMA shape, the
+    grouped launch's on the 16x16 one - another order of sums inside a K tile.)"""
     import torch
     from vecops_amd import capi
     shapes = BF16_GROUPS[name]
@@ -73,7 +75,7 @@ def test_grouped_bf16_equals_the_oracle_and_the_single_calls(device, oracle, nam
             capi.matmul_family(ta[i], tb[i], alone, capi.family_request(family, split_k=1), c_in=tci[i])
             torch.cuda.synchronize()
             same_bits.append(np.array_equal(host_bits(tc[i]), host_bits(alone)))
-        assert any(same_bits), (name, i)
+        assert any(same_bits) or k <= 256, (name, i)
 
 
 def test_grouped_int8_bit_exact_with_degenerate_groups(device, oracle):
@@ -143,7 +145,8 @@ def test_grouped_mixed_layouts_and_unaligned_operands(device, oracle):
 def test_grouped_floating_classes_in_one_launch(device, oracle, kind):
     """fp32 operands in both compute types and f16 operands: groups of unlike shapes (ragged, a C input on every
     other one, enough tiles for the 128 x 128 shape) through the grouped launch, each against the oracle and
-    bit-equal to the single call on one of the three square tile shapes, K unsplit."""
+    bit-equal to the single call on one of the three square tile shapes, K unsplit (in fp32 compute; with bf16 or
+    f16 compute the single call's 128 x 128 tile takes the other MFMA shape where K is 256 or less)."""
     import torch
     from vecops_amd import capi
     shapes = [(70, 90, 200), (300, 20, 64), (1000, 1300, 136), (700, 900, 264), (1, 33, 40), (513, 257, 96)]
@@ -175,7 +178,7 @@ def test_grouped_floating_classes_in_one_launch(device, oracle, kind):
             capi.matmul_family(ta[i], tb[i], alone, capi.family_request(family, split_k=1), c_in=tci[i], compute=compute)
             torch.cuda.synchronize()
             same_bits.append(np.array_equal(tc[i].cpu().numpy(), alone.cpu().numpy()))
-        assert any(same_bits), (kind, i)
+        assert any(same_bits) or (kind != "f32" and k <= 256), (kind, i)
 
 
 def test_grouped_other_classes_run_group_by_group(device, oracle):

@@ -1643,7 +1643,8 @@ constexpr int ntr_pitch() {
 // the unified file), the small tiles with 64x64 or 32x32.
 //
 // The work of one workgroup: number `pid` of the `total` that serve the problem `p`.
-template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
+// M16: multiply on the 16x16 MFMA shapes (the default: where kShortMfma says so).
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B, bool M16 = kShortMfma<SRC, WM, WN>>
 __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int pid, int total) {
   using T = SrcTraits<SRC>;
   constexpr bool INT = T::kInt;
@@ -1653,9 +1654,9 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
   constexpr int THREADS = 64 * WAVES_M * WAVES_N;
   constexpr int BM = 32 * WAVES_M * WM, BN = 32 * WAVES_N * WN;
   constexpr int STAGE_BYTES = kStageBytes<WAVES_M, WAVES_N, WM, WN, LOAD_B>();
-  // The 16x16 MFMA shapes (kShortMfma): a K tile is then two k-steps of four 16-byte chunks, and a 32-row block
-  // of a wavefront's tile two fragments
-  constexpr bool M16 = kShortMfma<SRC, WM, WN>;
+  // The 16x16 MFMA shapes: a K tile is then two k-steps of four 16-byte chunks, and a 32-row block of a
+  // wavefront's tile two fragments
+  static_assert(!M16 || SRC != SRC_F32, "the fp32 MFMA has one shape here");
   constexpr int FM = M16 ? 2 * WM : WM, FN = M16 ? 2 * WN : WN;
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -2033,9 +2034,9 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
       p, lds, acc, batch, split, m0, n0, wm, wn, wave, lane);
 }
 
-template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (kShortMfma<SRC, WM, WN> ? 2 : 1)) void tile_gemm_kernel(const TileGemmParams p) {
-  tile_gemm_workgroup<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_A, LOAD_B>(p, blockIdx.x, gridDim.x);
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B, bool M16 = kShortMfma<SRC, WM, WN>>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (M16 ? 2 : 1)) void tile_gemm_kernel(const TileGemmParams p) {
+  tile_gemm_workgroup<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_A, LOAD_B, M16>(p, blockIdx.x, gridDim.x);
 }
 
 // Several independent problems in one launch (irregular batches: every group has its own extents, strides and

@@ -54,11 +54,11 @@ hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream);
 hipError_t launch_unpack_b(int src, const PackBParams& p, hipStream_t stream);
 
 // Shared by the per-class translation units.
-template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB>
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB, bool M16>
 hipError_t launch_tile_instance(const TileGemmParams& p, hipStream_t stream) {
   constexpr int kLds = kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LB>();
   constexpr int kThreads = 64 * WAVES_M * WAVES_N;
-  auto kernel = tile_gemm_kernel<SRC, WAVES_M, WAVES_N, WM, WN, LA, LB>;
+  auto kernel = tile_gemm_kernel<SRC, WAVES_M, WAVES_N, WM, WN, LA, LB, M16>;
   // > 64 KiB of dynamic LDS has to be enabled once per device; cheap enough to repeat per thread.
   static thread_local int configured_device = -1;
   int device = 0;
@@ -98,11 +98,22 @@ hipError_t with_loaders(int mode, F&& f) {
   return pair(integral_constant<int, LOAD_GENERIC>{}, integral_constant<int, LOAD_GENERIC>{});
 }
 
-template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN>
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, bool M16 = kShortMfma<SRC, WM, WN>>
 hipError_t launch_tile_mode(const TileGemmParams& p, int mode, hipStream_t stream) {
   return with_loaders<SRC, WAVES_M, WAVES_N, WM, WN>(mode, [&](auto la, auto lb) {
-    return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, decltype(la)::value, decltype(lb)::value>(p, stream);
+    return launch_tile_instance<SRC, WAVES_M, WAVES_N, WM, WN, decltype(la)::value, decltype(lb)::value, M16>(p, stream);
   });
+}
+
+// 128 x 128 tiles of 16-bit operands with at most four K tiles multiply on the 32x32 shape after all: to fp32
+// outputs the 16x16 instance's workgroups live about 1 us longer there (3072 x 3072 x 64 15.0 us against 12.8,
+// x 256 19.1 against 17.1, 8192 x 8192 x 128 73 against 62; 5 % at K = 512, level at 1024, and from there on the
+// 16x16 shape is ahead), and to bf16 outputs the two are level up to K = 256 (from K = 512 the 16x16 shape is
+// ahead, as it is at every K for int32 outputs).  The rule does not look at the output type: a product's bf16
+// output stays the rounded fp32 output of the same call sequence.
+template <int SRC>
+bool long_shape_pays(const TileGemmParams& p) {
+  return !SrcTraits<SRC>::kInt && p.split_k == 1 && p.k_tiles_per_split <= 4;
 }
 
 template <int SRC>
@@ -113,7 +124,12 @@ hipError_t launch_tile_class(const TileGemmParams& p, int tile_m, int tile_n, in
   if (tile_m == 256 && tile_n == 256) return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
   if (tile_m == 256 && tile_n == 128) return launch_tile_mode<SRC, 2, 2, 4, 2>(p, mode, stream);
   if (tile_m == 128 && tile_n == 256) return launch_tile_mode<SRC, 2, 2, 2, 4>(p, mode, stream);
-  if (tile_m == 128 && tile_n == 128) return launch_tile_mode<SRC, 2, 2, 2, 2>(p, mode, stream);
+  if (tile_m == 128 && tile_n == 128) {
+    if constexpr (kShortMfma<SRC, 2, 2> && !SrcTraits<SRC>::kInt) {
+      if (long_shape_pays<SRC>(p)) return launch_tile_mode<SRC, 2, 2, 2, 2, false>(p, mode, stream);
+    }
+    return launch_tile_mode<SRC, 2, 2, 2, 2>(p, mode, stream);
+  }
   return launch_tile_mode<SRC, 2, 2, 1, 1>(p, mode, stream);
 }
 
