@@ -179,7 +179,8 @@ def bench_fp32_gemm(dev, steps, warmup, compute):
     code = capi.COMPUTE_F32 if compute == "f32" else capi.COMPUTE_BF16
     plan = capi.plan_matmul(a, b_kn.t(), c, compute=code)
     ws = torch.empty(max(int(plan.workspace_bytes), 1), dtype=torch.uint8, device=dev)
-    t = _measure(lambda i: capi.matmul(a, b_kn.t(), c, compute=code, workspace=ws), max(steps, 200), warmup)
+    run = capi.PreparedMatmul(a, b_kn.t(), c, compute=code, workspace=ws)   # a step is one call of the C ABI
+    t = _measure(lambda i: run(), max(steps, 200), warmup)
     flops = 2.0 * n ** 3
     tflops = flops / (t["event_ms"] * 1e-3) / 1e12
     peak = PEAK_FP32_MATRIX_TFLOPS if compute == "f32" else PEAK_BF16_TFLOPS
@@ -203,7 +204,8 @@ def bench_batched(dev, steps, warmup, m, n, k):
     c = torch.empty((batch, m, n), dtype=torch.float32, device=dev)
     plan = capi.plan_matmul(a, b, c)
     ws = torch.empty(max(int(plan.workspace_bytes), 1), dtype=torch.uint8, device=dev)
-    t = _measure(lambda i: capi.matmul(a, b, c, workspace=ws), max(steps, 100), warmup)
+    run = capi.PreparedMatmul(a, b, c, workspace=ws)   # a step is one call of the C ABI
+    t = _measure(lambda i: run(), max(steps, 100), warmup)
     flops = batch * 2.0 * m * n * k
     nbytes = batch * (2 * m * k + 2 * n * k + 4 * m * n)
     tflops = flops / (t["event_ms"] * 1e-3) / 1e12
