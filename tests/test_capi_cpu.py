@@ -117,6 +117,10 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k > 1
     assert p.workspace_bytes == p.split_k * 255 * 63 * 4
     assert p.vector_a == 1                                   # rows need not be 16-byte aligned for 16-byte loads
+    # a split must pay for its second kernel: sixteen or thirty-two K tiles are walked in one go, sixty-four are not
+    for (m, n, k), split in (((384, 384, 1024), 1), ((640, 640, 2048), 1), ((512, 512, 4096), 4), ((64, 64, 65536), 64)):
+        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.F32, (m, n)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == split, (m, n, k, p.split_k)
     # empty problems
     rc, p = _plan(_operand(capi.BF16, (0, 64)), _operand(capi.BF16, (8, 64)), _operand(capi.F32, (0, 8)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "none"
