@@ -229,14 +229,25 @@ __device__ __forceinline__ Staged<SRC> load_chunk_fast(__amdgpu_buffer_rsrc_t bu
   }
 }
 
-// Slow path: element by element with bounds checks and arbitrary K stride; used
-// for the K tail of the vector path and for every chunk of the generic path.
+// A whole chunk of K-contiguous source elements that lies inside its row, at any alignment (element-aligned
+// addresses: the memory system takes 16-byte loads at any byte address).
+template <int SRC>
+__device__ __forceinline__ Staged<SRC> load_chunk_whole(const void* base, int64_t first_element) {
+  Staged<SRC> out;
+  __builtin_memcpy(&out, static_cast<const char*>(base) + first_element * SrcTraits<SRC>::kSrcBytes, sizeof(out));
+  return out;
+}
+
+// Slow path: bounds checks and arbitrary K stride; used for the K tail of the vector path and for every chunk
+// of the generic path.  A chunk that lies wholly inside a K-contiguous row is still one load; only the chunk
+// that straddles the end of K (and every chunk of an operand whose K stride is not 1) goes element by element.
 template <int SRC>
 __device__ __noinline__ Staged<SRC> load_chunk_checked(const void* base, int64_t row_off, int64_t kstep, int k0,
                                                        int k_end, bool row_ok, uint32_t pad) {
   // `pad` is what an element outside the operand reads as: 0, or for an operand
   // that is xor-flipped on its way into LDS the flip byte, so that it ends up 0
   constexpr int EPC = SrcTraits<SRC>::kElemsPerChunk;
+  if (kstep == 1 && row_ok && k0 + EPC <= k_end) return load_chunk_whole<SRC>(base, row_off + k0);
   if constexpr (SRC == SRC_F32_AS_BF16) {
     uint32_t w[8];
 #pragma unroll
@@ -268,7 +279,8 @@ __device__ __noinline__ Staged<SRC> load_chunk_checked(const void* base, int64_t
   }
 }
 
-// A whole K-contiguous operand tile (rows x eight chunks), every element bounds-checked, straight into
+// A whole K-contiguous operand tile (rows x eight chunks), bounds-checked (chunk by chunk where the row is
+// K-contiguous, element by element in the chunk that straddles the end of K), straight into
 // its LDS tile: the partial last K tile.  Out of line and rolled - it runs once per workgroup - and
 // one call per operand: a call has to wait for its loads before it returns, so chunk-by-chunk calls
 // would pay one memory round trip each.
@@ -284,7 +296,10 @@ __device__ __noinline__ void stage_rows_checked(const void* base, int64_t rs, in
     const bool row_ok = first_row + row < extent;
     const int64_t row_off = static_cast<int64_t>(first_row + row) * rs;
     u32x4 out;
-    if constexpr (SRC == SRC_F32_AS_BF16) {
+    if (kstep == 1 && row_ok && k0 + EPC <= k_end) {  // a whole chunk inside the row: one load (two for fp32 pairs)
+      out = load_chunk_whole<SRC>(base, row_off + k0).chunk();
+      if constexpr (SRC == SRC_I8_FLIP) out ^= u32x4{flip, flip, flip, flip};
+    } else if constexpr (SRC == SRC_F32_AS_BF16) {
       float f[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
