@@ -233,8 +233,8 @@ __device__ __forceinline__ Staged<SRC> load_chunk_fast(__amdgpu_buffer_rsrc_t bu
 // addresses: the memory system takes 16-byte loads at any byte address).
 template <int SRC>
 __device__ __forceinline__ Staged<SRC> load_chunk_whole(const void* base, int64_t first_element) {
-  Staged<SRC> out;
-  __builtin_memcpy(&out, static_cast<const char*>(base) + first_element * SrcTraits<SRC>::kSrcBytes, sizeof(out));
+  Staged<SRC> out;  // (operands live in global memory: a global load, which LDS traffic does not wait for)
+  __builtin_memcpy(&out, (const VECOPS_GLOBAL char*)base + first_element * SrcTraits<SRC>::kSrcBytes, sizeof(out));
   return out;
 }
 
@@ -279,9 +279,8 @@ __device__ __noinline__ Staged<SRC> load_chunk_checked(const void* base, int64_t
   }
 }
 
-// A whole K-contiguous operand tile (rows x eight chunks), bounds-checked (chunk by chunk where the row is
-// K-contiguous, element by element in the chunk that straddles the end of K), straight into
-// its LDS tile: the partial last K tile.  Out of line and rolled - it runs once per workgroup - and
+// A whole operand tile (rows x eight chunks), bounds-checked (chunk by chunk where the rows are K-contiguous,
+// element by element otherwise), straight into its LDS tile: the partial last K tile.  Out of line and rolled - it runs once per workgroup - and
 // one call per operand: a call has to wait for its loads before it returns, so chunk-by-chunk calls
 // would pay one memory round trip each.
 template <int SRC>
@@ -289,6 +288,48 @@ __device__ __noinline__ void stage_rows_checked(const void* base, int64_t rs, in
                                                 int rows, int k0_tile, int k_end, char* lds_tile, int tid,
                                                 int threads, uint32_t flip) {
   constexpr int EPC = SrcTraits<SRC>::kElemsPerChunk;
+  if (kstep == 1 && k_end >= EPC) {
+    // K-contiguous rows of at least one chunk: every chunk is ONE load and no branch.  A chunk that straddles the
+    // end of K (or lies beyond it) loads the row's last EPC elements instead and shifts them down, so that zeros
+    // fill what lies past the end; a row past the operand loads the last row and shifts everything out.  (Element
+    // loads under per-element conditions, as below, came out as one memory round trip per two elements: a
+    // workgroup's partial tile cost 8 x 777x1000x3000 11 us of 54.)
+    constexpr int ELEM_BITS = 128 / EPC;  // of the compute chunk: 16, 8 (bytes) or 32 (fp32 compute)
+    constexpr int BATCH = 4;              // loads in flight before the first is used
+    const int chunks = rows * 8;
+    for (int idx0 = tid; idx0 < chunks; idx0 += threads * BATCH) {
+      u32x4 v[BATCH];
+#pragma unroll
+      for (int j = 0; j < BATCH; ++j) {
+        const int idx = min(idx0 + j * threads, chunks - 1);
+        const int row_c = min(first_row + (idx >> 3), extent - 1);
+        const int start = min(k0_tile + (idx & 7) * EPC, k_end - EPC);
+        v[j] = load_chunk_whole<SRC>(base, static_cast<int64_t>(row_c) * rs + start).chunk();
+      }
+#pragma unroll
+      for (int j = 0; j < BATCH; ++j) {
+        const int idx = idx0 + j * threads;
+        const int row = idx >> 3, chunk = idx & 7;
+        const int k0 = k0_tile + chunk * EPC;
+        u32x4 w = v[j];
+        if constexpr (SRC == SRC_I8_FLIP) w ^= u32x4{flip, flip, flip, flip};
+        const int shift = (first_row + row < extent) ? min(k0 - min(k0, k_end - EPC), EPC) : EPC;  // in elements
+        const uint32_t bits = static_cast<uint32_t>(shift * ELEM_BITS);                            // 0 .. 128
+        const uint64_t lo = (static_cast<uint64_t>(w.y) << 32) | w.x, hi = (static_cast<uint64_t>(w.w) << 32) | w.z;
+        // (shifts by bits & 63 with the carried half masked out where the count is 0: no branch)
+        const uint32_t b = bits & 63u;
+        const uint64_t carry = b ? hi << (64u - b) : 0;
+        const uint64_t lo_small = (lo >> b) | carry, hi_small = hi >> b;  // bits < 64
+        const uint64_t out_lo = bits >= 128u ? 0 : bits >= 64u ? hi >> b : lo_small;
+        const uint64_t out_hi = bits >= 64u ? 0 : hi_small;
+        if (idx < chunks)
+          *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(row, chunk)) =
+              u32x4{static_cast<uint32_t>(out_lo), static_cast<uint32_t>(out_lo >> 32), static_cast<uint32_t>(out_hi),
+                    static_cast<uint32_t>(out_hi >> 32)};
+      }
+    }
+    return;
+  }
 #pragma unroll 2
   for (int idx = tid; idx < rows * 8; idx += threads) {
     const int row = idx >> 3, chunk = idx & 7;
