@@ -1896,21 +1896,21 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
     // loads that write LDS: tile 0 goes straight into stage 0 (the partial tile through ordinary stores)
     if (nk > 0) {
       const int first = __builtin_amdgcn_readfirstlane(seq(0));
+      if constexpr (M16) {
+        // the loop of the 16x16 shapes loads two tiles ahead: the second tile (never the partial one) goes into
+        // stage 1 here - ahead of a partial first tile, whose out-of-line staging waits for its own loads twice
+        if (nk > 1) {
+          const int second = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + 1);
+          stager_a.dma_full(second, lds + STAGE_BYTES);
+          stager_b.dma_full(second, lds + STAGE_BYTES + BM * 128);
+        }
+      }
       if (first < full_k_tiles) {
         stager_a.dma_full(first, lds);
         stager_b.dma_full(first, lds + BM * 128);
       } else {
         stager_a.stage_checked(first, lds);
         stager_b.stage_checked(first, lds + BM * 128);
-      }
-      if constexpr (M16) {
-        // the loop of the 16x16 shapes loads two tiles ahead: the second tile (never the partial one) goes into
-        // stage 1 here
-        if (nk > 1) {
-          const int second = __builtin_amdgcn_readfirstlane(kt_begin - has_tail + 1);
-          stager_a.dma_full(second, lds + STAGE_BYTES);
-          stager_b.dma_full(second, lds + STAGE_BYTES + BM * 128);
-        }
       }
     }
   } else if constexpr (!DMA) {
