@@ -292,8 +292,8 @@ __device__ __noinline__ void stage_rows_checked(const void* base, int64_t rs, in
     // K-contiguous rows of at least one chunk: every chunk is ONE load and no branch.  A chunk that straddles the
     // end of K (or lies beyond it) loads the row's last EPC elements instead and shifts them down, so that zeros
     // fill what lies past the end; a row past the operand loads the last row and shifts everything out.  (Element
-    // loads under per-element conditions, as below, came out as one memory round trip per two elements: a
-    // workgroup's partial tile cost 8 x 777x1000x3000 11 us of 54.)
+    // loads under per-element conditions, as below, came out as one memory round trip per two elements: batch 8 of
+    // 3000 x 3000 x 17, whose only K tile is a partial one, took 83 us that way and takes 67.)
     constexpr int ELEM_BITS = 128 / EPC;  // of the compute chunk: 16, 8 (bytes) or 32 (fp32 compute)
     constexpr int BATCH = 4;              // loads in flight before the first is used
     const int chunks = rows * 8;
