@@ -49,8 +49,8 @@ enum OutKind : int { OUT_F32 = 0, OUT_BF16 = 1, OUT_I32 = 2, OUT_U8 = 3, OUT_I8 
 enum Activation : int { ACT_NONE = 0, ACT_RELU = 1, ACT_CLAMP = 2, ACT_SIGMOID = 3, ACT_SILU = 4 };
 // How an operand tile is fetched from global memory.
 enum LoadKind : int {
-  LOAD_KVEC = 0,     // K contiguous, rows and base 16-byte aligned: one 16-byte load per chunk
-  LOAD_GENERIC = 1,  // any strides / alignment: one load per element
+  LOAD_KVEC = 0,     // K contiguous (rows at any element alignment): one 16-byte load per chunk
+  LOAD_GENERIC = 1,  // any strides: one load per element
   LOAD_NVEC = 2,     // spatial index contiguous (B given as [K,N] row-major), 16-byte aligned rows:
                      // transposed in registers on the way into LDS (32-bit compute elements)
   LOAD_NTR = 3,      // the same operand layout for 16-bit compute elements: stored in LDS as it
