@@ -237,12 +237,16 @@ def bench_grouped(dev, steps, warmup):
         b_list.append(torch.from_numpy(synth.bf16_round(synth.uniform_pm1(40 + i, (n, k))).view(np.int16)).to(dev).view(torch.bfloat16))
         c_list.append(torch.empty((m, n), dtype=torch.float32, device=dev))
     ws = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
-    grouped = _measure(lambda i: capi.matmul_grouped(a_list, b_list, c_list, workspace=ws), max(steps, 50), warmup)
+    # (a call is seven launches - two groups split K - and a separate-calls step ten: at most 100 steps between
+    # synchronisations, because with thousands of launches queued the HIP runtime's own bookkeeping stalls the host
+    # in the first such loop of a process, 160-200 us per step of wall time where the GPU needs 76)
+    count = min(max(steps, 50), 100)
+    grouped = _measure(lambda i: capi.matmul_grouped(a_list, b_list, c_list, workspace=ws), count, max(warmup, count))
 
     def one_by_one(i):
         for a, b, c in zip(a_list, b_list, c_list):
             capi.matmul(a, b, c, workspace=ws)
-    looped = _measure(one_by_one, max(steps, 50), warmup)
+    looped = _measure(one_by_one, count, max(warmup, count))
     flops = sum(2.0 * m * n * k for m, n, k in GROUPED_SHAPES)
     tflops = flops / (grouped["event_ms"] * 1e-3) / 1e12
     roof = _roofline("mfma", tflops, PEAK_BF16_TFLOPS, "TFLOP/s", kernel="vecops_hip tile_gemm_grouped_kernel<bf16>",

@@ -183,8 +183,9 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_static_workspace(const VecopsHipOper
  * arrays of count descriptors obeying the rules of vecops_hip_matmul group by group.  Groups of one operand
  * class - bf16, f16, int8 x int8, or fp32 in either compute type - run as ONE launch over a table of problem
  * records (written into the workspace by small kernels fed through their arguments: no host buffer has to outlive
- * the call, nothing is allocated); unsigned 8-bit and fp64 operands, a mix of classes, and groups with K = 0 run as
- * launches of their own on the same stream.  Results
+ * the call, nothing is allocated); unsigned 8-bit and fp64 operands, a mix of classes, groups with K = 0 and groups
+ * whose K vecops_hip_matmul would split (few output tiles, long K: they run that call's plan, partial sums behind
+ * the table) run as launches of their own on the same stream.  Results
  * are those of vecops_hip_matmul on each group (bit-equal when that call runs the same tile shape without splitting K -
  * except 16-bit products with K <= 256 on 128 x 128 tiles, where the single call takes the other MFMA shape; otherwise equal up to the order of the fp32 sums - integer results are always the same bits).  workspace: vecops_hip_matmul_grouped_workspace bytes, 16-byte aligned.
  */

@@ -37,6 +37,8 @@ BF16_GROUPS = {
     "large": [(2048, 2048, 520), (3000, 1000, 264), (1024, 4096, 136), (4000, 2000, 72), (2500, 2500, 200)],
     # more groups than one table chunk carries
     "many": [(40 + 7 * i, 300 - 5 * i, 64 + 8 * (i % 5)) for i in range(31)],
+    # groups whose K the rule table splits (launches of their own, partial sums behind the table) among others
+    "long_k": [(255, 63, 8191), (300, 200, 520), (100, 40, 4099), (700, 900, 264), (500, 300, 4100)],
 }
 
 
@@ -75,7 +77,16 @@ def test_grouped_bf16_equals_the_oracle_and_the_single_calls(device, oracle, nam
             capi.matmul_family(ta[i], tb[i], alone, capi.family_request(family, split_k=1), c_in=tci[i])
             torch.cuda.synchronize()
             same_bits.append(np.array_equal(host_bits(tc[i]), host_bits(alone)))
-        assert any(same_bits) or k <= 256, (name, i)
+        plan = capi.plan_matmul(ta[i], tb[i], tc[i], c_in=tci[i])
+        if plan.split_k > 1:       # a group that splits K runs vecops_hip_matmul's own plan
+            alone = torch.empty_like(tc[i])
+            capi.matmul(ta[i], tb[i], alone, c_in=tci[i])
+            torch.cuda.synchronize()
+            assert np.array_equal(host_bits(tc[i]), host_bits(alone)), (name, i)
+        else:
+            assert any(same_bits) or k <= 256, (name, i)
+    if name == "long_k":
+        assert sum(capi.plan_matmul(ta[i], tb[i], tc[i], c_in=tci[i]).split_k > 1 for i in range(len(shapes))) >= 2
 
 
 def test_grouped_int8_bit_exact_with_degenerate_groups(device, oracle):

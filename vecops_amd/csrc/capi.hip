@@ -1258,11 +1258,14 @@ namespace {
 // pointers).  bf16 and int8 groups that all multiply run as ONE launch of tile_gemm_grouped_kernel over a table of
 // problem records in the workspace (so do f16 groups and fp32 groups, in either compute type); unsigned 8-bit
 // operands (whose sign flip needs a pass over B first), fp64 operands, groups of mixed classes, and groups with K = 0, run as
-// launches of their own on the same stream.
+// launches of their own on the same stream.  So do groups whose K the rule table splits (few output tiles, long K):
+// the grouped kernel walks a group's whole K in every workgroup, and two workgroups with 128 K tiles each would
+// be what the whole launch waits for (eight products, 255 x 63 x 8191 among them: 99 us in one launch).
 struct Grouped {
   std::vector<Problem> problems;
   std::vector<VecopsHipPlan> plans;
   std::vector<int> table_groups;  // indices of the groups served by the one grouped launch
+  std::vector<int> split_groups;  // ... and of those that split K: launches of their own
   bool one_launch = false;
   int src = -1, tile = 0, mode = 0;
   std::vector<int32_t> first;     // first workgroup of each table group, and the end
@@ -1288,7 +1291,8 @@ int32_t describe_grouped(uint32_t count, const VecopsHipOperand* a, const Vecops
     if (plan.family == VECOPS_HIP_FAMILY_ZERO_K) continue;
     if (g->src < 0) g->src = g->problems[i].src;
     else if (g->src != g->problems[i].src) same_class = false;
-    g->table_groups.push_back(static_cast<int>(i));
+    if (plan.split_k > 1) g->split_groups.push_back(static_cast<int>(i));
+    else g->table_groups.push_back(static_cast<int>(i));
   }
   g->one_launch = same_class && g->src != SRC_I8_FLIP && g->src != kSrcF64 && g->table_groups.size() > 1;
   if (!g->one_launch) return ST_OK;
@@ -1340,10 +1344,15 @@ int32_t describe_grouped(uint32_t count, const VecopsHipOperand* a, const Vecops
   return ST_OK;
 }
 
+uint64_t grouped_table_bytes(const Grouped& g) { return g.one_launch ? g.first_bytes + g.record_bytes + g.map_bytes : 0; }
+
 uint64_t grouped_workspace(const Grouped& g) {
-  const uint64_t table = g.one_launch ? g.first_bytes + g.record_bytes + g.map_bytes : 0;
-  // (the loop's scratch serves one launch at a time; with a table only the K = 0 groups loop, and they need none)
-  return g.one_launch ? table : g.loop_workspace;
+  // the table, and behind it the scratch of the groups that run as launches of their own (one launch at a time, so
+  // the largest need serves them all: with a table these are the groups that split K - K = 0 groups need none)
+  if (!g.one_launch) return g.loop_workspace;
+  uint64_t most = 0;
+  for (int i : g.split_groups) most = g.plans[i].workspace_bytes > most ? g.plans[i].workspace_bytes : most;
+  return grouped_table_bytes(g) + most;
 }
 }  // namespace
 
@@ -1382,6 +1391,12 @@ int32_t vecops_hip_matmul_grouped(uint32_t count, const VecopsHipOperand* a, con
     if (rc != ST_OK) return rc;
   }
   char* base = static_cast<char*>(workspace);
+  // groups that split K: their own plan, partial sums behind the table
+  for (int i : g.split_groups) {
+    const uint64_t table = grouped_table_bytes(g);
+    rc = run_problem(g.problems[i], g.plans[i], nullptr, nullptr, nullptr, base + table, workspace_size - table, s);
+    if (rc != ST_OK) return rc;
+  }
   int32_t* first = reinterpret_cast<int32_t*>(base);
   TileGemmParams* records = reinterpret_cast<TileGemmParams*>(base + g.first_bytes);
   int32_t* group_of = reinterpret_cast<int32_t*>(base + g.first_bytes + g.record_bytes);
