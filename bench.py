@@ -306,12 +306,14 @@ def bench_runtime_quant(dev, steps, warmup):
     t = _measure(lambda i: capi.matmul_runtime_quant(a, tm, zp, b, rs, cs, c, correction=corr, workspace=ws), steps, warmup)
     ops = 2.0 * m * n * k
     tops = ops / (t["event_ms"] * 1e-3) / 1e12
+    # (the product runs on the quantised bytes: the plan of int8 operands of these extents names its kernel)
+    plan = capi.plan_matmul(torch.empty((m, k), dtype=torch.int8, device=dev), b, torch.empty((m, n), dtype=torch.int32, device=dev))
     return {"metric": "runtime_quantized_matmul_tops", "workload": "fp32 activations 2048x4096 quantised per row to "
             "uint8 on the way in, int8 weights 11008x4096, correction row, per-token x per-channel dequant, fp32 out",
             "value": tops, "unit": "TOP/s", "ms_per_step": t["wall_ms"], "dtype": "int8",
             "roofline": _roofline("mfma", tops, PEAK_INT8_TOPS, "TOP/s", traffic=None,
-                                  kernel="vecops_hip quantize_rows_kernel + byte_row_sums_kernel + tile_gemm_kernel<int8> "
-                                         "family tile_256, dequantising epilogue",
+                                  kernel="vecops_hip quantize_rows_kernel + byte_row_sums_kernel + " +
+                                         _kernel_label(plan, "int8").replace("vecops_hip ", "") + ", dequantising epilogue",
                                   algorithmic_ops_per_launch=ops,
                                   algorithmic_bytes_per_launch=4 * m * k + n * k + 4 * m * n + 4 * (2 * m + 2 * n),
                                   **_timing_fields(t))}
