@@ -46,7 +46,7 @@ RECORDED_TRAFFIC = {
     "gemv_m16": (int((30150.0 * 2.000 + 524.8 * 1.000) * 1024), "profiles/skinny_w8a16_stream_m1_4096x14336.md"),
     "bf16_packed": (int((98468.3 * 2.000 + 32768 * 1.000) * 1024),
                     "profiles/tile_gemm_packed_b_bf16_4096_int8_2048x4096x11008.md"),
-    "int8_packed": (int((95160.6 * 2.000 + 88064 * 1.000) * 1024),
+    "int8_packed": (int((138798.0 * 2.000 + 88064 * 1.000) * 1024),
                     "profiles/tile_gemm_packed_b_bf16_4096_int8_2048x4096x11008.md"),
 }
 
