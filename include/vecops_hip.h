@@ -161,10 +161,13 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_family(const VecopsHipOperand* a, co
  * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
  * vecops (its callers size and own every workspace, ops/Matmul.h:504-526).  The split-K partial sums and the
  * unsigned-operand terms live in a buffer of VECOPS_HIP_STATIC_WORKSPACE_BYTES that belongs to the library's
- * code object on each GPU (8 MiB, held until the process ends; split-K plans need at most 4 MiB, the row
- * sums of unsigned operands 4 bytes per row of a and b); the call allocates and frees nothing.  A call whose
- * plan needs more (vecops_hip_plan_matmul(...).workspace_bytes) returns 2 (not applicable) and launches
- * nothing.  Same kernels and therefore the same results, bit for bit, as vecops_hip_matmul.  Every call on
+ * code object on each GPU (8 MiB, held until the process ends; the K splits of problems with few output tiles
+ * need at most 4 MiB, the row sums of unsigned operands 4 bytes per row of a and b); the call allocates and frees
+ * nothing.  The one plan of vecops_hip_matmul that needs more - K of a problem with 128 to 200 tiles of 128 x 128
+ * split two to four ways, 24-32 MB of partial sums - is not taken here: such a problem runs unsplit (the sums then
+ * differ from vecops_hip_matmul's in their order).  A call whose plan still needs more than the buffer returns 2
+ * (not applicable) and launches nothing.  Otherwise the same kernels and therefore the same results, bit for
+ * bit, as vecops_hip_matmul.  Every call on
  * one GPU shares that GPU's buffer: calls that overlap on one GPU (different streams or host threads) race;
  * calls on one stream, or otherwise ordered, do not.
  */

@@ -117,6 +117,19 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k > 1
     assert p.workspace_bytes == p.split_k * 255 * 63 * 4
     assert p.vector_a == 1                                   # rows need not be 16-byte aligned for 16-byte loads
+    # 128 to 200 tiles of 128 x 128 and twenty K tiles per part or more: K split so that two workgroups sit on
+    # (nearly) every compute unit; shorter K and int8's 128-element K tiles keep the unsplit small tiles
+    for (m, n, k), family, split in (((640, 4096, 4096), "tile_128", 3), ((768, 4096, 4096), "tile_128", 2),
+                                     ((1024, 2048, 8192), "tile_128", 4), ((768, 3072, 12288), "tile_128", 3),
+                                     ((512, 4096, 4096), "tile_64", 1), ((640, 4096, 2048), "tile_64", 1),
+                                     ((896, 4096, 4096), "tile_128", 1)):
+        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
+        assert p.workspace_bytes == (split * m * n * 4 if split > 1 else 0)
+    rc, p = _plan(_operand(capi.I8, (768, 4096)), _operand(capi.I8, (4096, 4096)), _operand(capi.I32, (768, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 1
+    rc, p = _plan(_operand(capi.I8, (768, 12288)), _operand(capi.I8, (3072, 12288)), _operand(capi.I32, (768, 3072)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 3
     # a split must pay for its second kernel: sixteen or thirty-two K tiles are walked in one go, sixty-four are not
     for (m, n, k), split in (((384, 384, 1024), 1), ((640, 640, 2048), 1), ((512, 512, 4096), 4), ((64, 64, 65536), 64)):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.F32, (m, n)))

@@ -869,3 +869,40 @@ def test_w8a16_rejects_bad_arguments(device):
     with pytest.raises(capi.VecopsHipError) as e:
         capi.matmul_w8a16_group(x[:4], w, s, y[:4], 100)
     assert e.value.code == 1
+
+
+@pytest.mark.parametrize("kind,m,n,k", [("bf16", 640, 4096, 4096), ("bf16", 768, 3072, 12288), ("bf16", 1000, 2000, 8200),
+                                        ("i8", 768, 3072, 12288), ("i8", 700, 4000, 8192)])
+def test_mid_band_k_split(device, oracle, kind, m, n, k):
+    """128 to 200 tiles of 128 x 128 with a long K: the rule table splits K two to four ways on 128 x 128 tiles
+    (partial sums in the workspace, summed in the order of the parts).  Against the oracle (int8: exact), with a C
+    input; the entry point that allocates nothing runs the same problem unsplit and agrees within the bound."""
+    import torch
+    from vecops_amd import capi
+    if kind == "bf16":
+        a, b = synth.bf16_round(synth.uniform_pm1(1, (m, k))), synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+        ta, tb = dev_bf16(a, device), dev_bf16(b, device)
+        cin = synth.uniform_pm1(3, (m, n)).astype(np.float32)
+        c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    else:
+        a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+        ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+        cin = (synth.draws(3, m * n) % np.uint64(1 << 20)).astype(np.int32).reshape(m, n)
+        c = torch.full((m, n), -1, dtype=torch.int32, device=device)
+    tci = torch.from_numpy(cin).to(device)
+    plan = capi.plan_matmul(ta, tb, c, c_in=tci)
+    assert capi.FAMILY_NAMES[plan.family] == "tile_128" and 2 <= plan.split_k <= 4
+    capi.matmul(ta, tb, c, c_in=tci)
+    alone = torch.empty_like(c)
+    capi.matmul_static_workspace(ta, tb, alone, c_in=tci)
+    torch.cuda.synchronize()
+    if kind == "bf16":
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want, cin=cin, acc_f64=True)
+        assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+        assert rel_err(alone.cpu().numpy(), want) <= fp32_tol(k)
+    else:
+        want = (a.astype(np.int64) @ b.astype(np.int64).T + cin).astype(np.int64)
+        want = (want & 0xffffffff).astype(np.uint32).view(np.int32)
+        assert np.array_equal(c.cpu().numpy(), want)
+        assert np.array_equal(alone.cpu().numpy(), want)

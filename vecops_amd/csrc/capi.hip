@@ -313,7 +313,8 @@ int fetch_mode(const Problem& pr, const VecopsHipPlan& plan);
 // of big tiles is not worth avoiding: the chip runs against its power limit on real
 // data, a lightly loaded round clocks higher, and narrower tiles (256x192 was
 // measured) cost more LDS and L2 traffic per flop than the better balance saves.
-void choose(const Problem& pr, VecopsHipPlan* plan) {
+// (scratch_limit: partial sums the caller can hold - the mid-band K split below is skipped where it needs more)
+void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UINT64_MAX) {
   memset(plan, 0, sizeof(*plan));
   plan->split_k = 1;
   if (pr.batch == 0 || pr.m == 0 || pr.n == 0) {
@@ -413,8 +414,24 @@ void choose(const Problem& pr, VecopsHipPlan* plan) {
     family = VECOPS_HIP_FAMILY_TILE_64;
     tile_m = tile_n = 64;
   }
+  // 128 to 200 tiles of 128x128 and a long K: half to three quarters of the compute units hold one workgroup each,
+  // and 64x64 tiles fill them with work that is a third less efficient.  K split two to four ways puts two
+  // 128x128 workgroups on (nearly) every unit; it pays from twenty K tiles per part (bf16: 768 x 3072 x 12288 108 us
+  // -> 64, 768 x 4096 x 8192 78 -> 60, 1024 x 2048 x 8192 52 -> 43, 640 x 4096 x 4096 41 -> 34, 768 x 4096 x 4096
+  // 41 -> 39; int8: 768 x 3072 x 12288 58 -> 42; with sixteen per part - 512 x 4096 x 4096, int8 1024 x 2048 x 8192 -
+  // the unsplit small tiles stay ahead, 28.0 against 30.8 and 28.8 against 33.0).  Measured with loads that write
+  // LDS themselves, so only there.
+  uint32_t band_split = 0;
+  if (direct && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) && tiles(128) >= kComputeUnits / 2 &&
+      tiles(128) <= 200) {
+    const int64_t parts = 2 * kComputeUnits / tiles(128);
+    if (k_tiles / parts >= 20 && static_cast<uint64_t>(parts) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
+      family = VECOPS_HIP_FAMILY_TILE_128;
+      band_split = static_cast<uint32_t>(parts);
+    }
+  }
   plan->family = family;
-  finish_tile_plan(pr, plan, 0);
+  finish_tile_plan(pr, plan, band_split);
 }
 
 const char* family_name(uint32_t family) {
@@ -1547,7 +1564,7 @@ int32_t vecops_hip_matmul_static_workspace(const VecopsHipOperand* a, const Veco
   int32_t rc = describe(a, b, c_in, c, compute, &pr);
   if (rc != ST_OK) return rc;
   VecopsHipPlan plan;
-  choose(pr, &plan);
+  choose(pr, &plan, VECOPS_HIP_STATIC_WORKSPACE_BYTES);
   if (plan.workspace_bytes > VECOPS_HIP_STATIC_WORKSPACE_BYTES)
     return fail(ST_NOT_APPLICABLE, "matmul_static_workspace: the call needs %llu bytes of scratch, the library holds %llu",
                 (unsigned long long)plan.workspace_bytes, (unsigned long long)VECOPS_HIP_STATIC_WORKSPACE_BYTES);
