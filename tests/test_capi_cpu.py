@@ -126,6 +126,12 @@ def test_rule_table_known_answers():
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
         assert p.workspace_bytes == (split * m * n * 4 if split > 1 else 0)
+    # ... and from 32 tiles on, one part fewer where that reaches twenty K tiles per part
+    for (m, n, k), family, split in (((512, 2048, 16384), "tile_128", 8), ((384, 3072, 8192), "tile_128", 6),
+                                     ((512, 3072, 8192), "tile_128", 5), ((512, 3072, 4096), "tile_64", 1),
+                                     ((256, 4096, 4096), "tile_64", 1), ((512, 1024, 8192), "tile_64", 2)):
+        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
     rc, p = _plan(_operand(capi.I8, (768, 4096)), _operand(capi.I8, (4096, 4096)), _operand(capi.I32, (768, 4096)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 1
     rc, p = _plan(_operand(capi.I8, (768, 12288)), _operand(capi.I8, (3072, 12288)), _operand(capi.I32, (768, 3072)))

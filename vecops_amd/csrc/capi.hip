@@ -277,7 +277,7 @@ void finish_tile_plan(const Problem& pr, VecopsHipPlan* plan, uint32_t forced_sp
   int64_t split = 1;
   if (forced_split > 0) {
     split = forced_split < k_tiles ? forced_split : k_tiles;
-  } else if (wgs < kComputeUnits / 2 && k_tiles >= 8) {
+  } else if (wgs <= kComputeUnits / 2 && k_tiles >= 8) {
     split = kComputeUnits / wgs;
     if (split > k_tiles / 4) split = k_tiles / 4;
     if (split > 64) split = 64;
@@ -421,10 +421,14 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // 41 -> 39; int8: 768 x 3072 x 12288 58 -> 42; with sixteen per part - 512 x 4096 x 4096, int8 1024 x 2048 x 8192 -
   // the unsplit small tiles stay ahead, 28.0 against 30.8 and 28.8 against 33.0).  Measured with loads that write
   // LDS themselves, so only there.
+  // The same from 32 tiles of 128x128 on, five to sixteen ways (bf16 512 x 2048 x 16384 73 us -> 43, 384 x 3072 x 8192
+  // 46 -> 33, 512 x 3072 x 8192 48 -> 40; the 64x64 tiles the table took there are 128 workgroups or more, which the
+  // rule for few workgroups leaves whole): one part fewer where that reaches the twenty K tiles.
   uint32_t band_split = 0;
-  if (direct && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) && tiles(128) >= kComputeUnits / 2 &&
+  if (direct && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) && tiles(128) >= kComputeUnits / 8 &&
       tiles(128) <= 200) {
-    const int64_t parts = 2 * kComputeUnits / tiles(128);
+    int64_t parts = 2 * kComputeUnits / tiles(128);
+    if (parts >= 6 && k_tiles / parts < 20) --parts;
     if (k_tiles / parts >= 20 && static_cast<uint64_t>(parts) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
       family = VECOPS_HIP_FAMILY_TILE_128;
       band_split = static_cast<uint32_t>(parts);
