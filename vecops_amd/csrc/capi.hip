@@ -423,9 +423,10 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // LDS themselves, so only there.
   // The same from 32 tiles of 128x128 on, five to sixteen ways (bf16 512 x 2048 x 16384 73 us -> 43, 384 x 3072 x 8192
   // 46 -> 33, 512 x 3072 x 8192 48 -> 40; the 64x64 tiles the table took there are 128 workgroups or more, which the
-  // rule for few workgroups leaves whole): one part fewer where that reaches the twenty K tiles.
+  // rule for few workgroups leaves whole): one part fewer where that reaches the twenty K tiles.  (Not for a
+  // prepacked B: its kernels were not measured this way.)
   uint32_t band_split = 0;
-  if (direct && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) && tiles(128) >= kComputeUnits / 8 &&
+  if (direct && !pr.packed_b && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) && tiles(128) >= kComputeUnits / 8 &&
       tiles(128) <= 200) {
     int64_t parts = 2 * kComputeUnits / tiles(128);
     if (parts >= 6 && k_tiles / parts < 20) --parts;
@@ -1618,16 +1619,22 @@ int32_t vecops_hip_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b, 
 }
 
 uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int64_t n, int64_t k) {
-  VecopsHipOperand a, b, c;
-  make_operand(&a, reinterpret_cast<void*>(16), DT_I8, m, k, k);
-  make_operand(&b, reinterpret_cast<void*>(16), DT_I8, n, k, k);
-  make_operand(&c, reinterpret_cast<void*>(16), DT_I32, m, n, n);
-  Problem pr{};
-  if (describe(&a, &b, nullptr, &c, 0, &pr) != ST_OK) return 0;
-  pr.dequant = true;
-  VecopsHipPlan plan;
-  choose(pr, &plan);
-  return plan.workspace_bytes;
+  // The plan depends on how the rows lie (16-byte aligned rows take other kernels, and with them other K splits),
+  // which this query is not told: the larger need of dense rows and of rows padded to 16 bytes.
+  uint64_t most = 0;
+  for (const int64_t ld : {k, (k + 15) & ~int64_t{15}}) {
+    VecopsHipOperand a, b, c;
+    make_operand(&a, reinterpret_cast<void*>(16), DT_I8, m, k, ld);
+    make_operand(&b, reinterpret_cast<void*>(16), DT_I8, n, k, ld);
+    make_operand(&c, reinterpret_cast<void*>(16), DT_I32, m, n, n);
+    Problem pr{};
+    if (describe(&a, &b, nullptr, &c, 0, &pr) != ST_OK) return 0;
+    pr.dequant = true;
+    VecopsHipPlan plan;
+    choose(pr, &plan);
+    most = plan.workspace_bytes > most ? plan.workspace_bytes : most;
+  }
+  return most;
 }
 
 int32_t vecops_hip_matmul_i8_dequant(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
