@@ -902,7 +902,30 @@ def test_mid_band_k_split(device, oracle, kind, m, n, k):
         assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
         assert rel_err(alone.cpu().numpy(), want) <= fp32_tol(k)
     else:
-        want = (a.astype(np.int64) @ b.astype(np.int64).T + cin).astype(np.int64)
+        want = (a.astype(np.float64) @ b.astype(np.float64).T).astype(np.int64) + cin   # exact: sums stay below 2^53
         want = (want & 0xffffffff).astype(np.uint32).view(np.int32)
         assert np.array_equal(c.cpu().numpy(), want)
         assert np.array_equal(alone.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("m,n,k,pad", [(768, 3072, 12288, 0), (768, 3072, 12289, 15)])
+def test_mid_band_k_split_with_dequantisation(device, m, n, k, pad):
+    """The K split of the mid band under the dequantising epilogue (applied by the kernel that sums the parts): bit
+    for bit (float(acc + corr) * rs) * cs.  Rows padded to 16 bytes around an odd K take the split too, and the
+    workspace query, which is told extents only, must have answered for them."""
+    import torch
+    from vecops_amd import capi
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    rs, cs = synth.scales(3, m), synth.scales(4, n)
+    corr = ((synth.draws(5, n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32)
+    ta = torch.zeros(m, k + pad, dtype=torch.int8, device=device)
+    tb = torch.zeros(n, k + pad, dtype=torch.int8, device=device)
+    ta[:, :k], tb[:, :k] = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    assert capi.lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k) >= 2 * m * n * 4
+    c = torch.full((m, n), float("nan"), device=device)
+    capi.matmul_i8_dequant(ta[:, :k], tb[:, :k], torch.from_numpy(rs).to(device), torch.from_numpy(cs).to(device), c,
+                           correction=torch.from_numpy(corr).to(device))
+    torch.cuda.synchronize()
+    acc = ((a.astype(np.float64) @ b.astype(np.float64).T).astype(np.int64) + corr[None, :]).astype(np.int32)   # exact in float64
+    want = (acc.astype(np.float32) * rs[:, None].astype(np.float32)) * cs[None, :].astype(np.float32)
+    assert np.array_equal(c.cpu().numpy(), want)
