@@ -129,13 +129,18 @@ def test_rule_table_known_answers():
     # ... and from 32 tiles on, one part fewer where that reaches twenty K tiles per part
     for (m, n, k), family, split in (((512, 2048, 16384), "tile_128", 8), ((384, 3072, 8192), "tile_128", 6),
                                      ((512, 3072, 8192), "tile_128", 5), ((512, 3072, 4096), "tile_64", 1),
-                                     ((256, 4096, 4096), "tile_64", 1), ((512, 1024, 8192), "tile_64", 2)):
+                                     ((256, 4096, 4096), "tile_64", 1), ((512, 1024, 8192), "tile_128", 6),
+                                     ((128, 8192, 8192), "tile_128", 6)):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
     rc, p = _plan(_operand(capi.I8, (768, 4096)), _operand(capi.I8, (4096, 4096)), _operand(capi.I32, (768, 4096)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 1
     rc, p = _plan(_operand(capi.I8, (768, 12288)), _operand(capi.I8, (3072, 12288)), _operand(capi.I32, (768, 3072)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 3
+    rc, p = _plan(_operand(capi.I8, (512, 16384)), _operand(capi.I8, (2048, 16384)), _operand(capi.I32, (512, 2048)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 6
+    rc, p = _plan(_operand(capi.I8, (512, 8192)), _operand(capi.I8, (1024, 8192)), _operand(capi.I32, (512, 1024)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 1    # exactly 128 workgroups: a split of two does not pay
     # a split must pay for its second kernel: sixteen or thirty-two K tiles are walked in one go, sixty-four are not
     for (m, n, k), split in (((384, 384, 1024), 1), ((640, 640, 2048), 1), ((512, 512, 4096), 4), ((64, 64, 65536), 64)):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.F32, (m, n)))

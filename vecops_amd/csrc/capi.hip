@@ -423,13 +423,14 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // LDS themselves, so only there.
   // The same from 32 tiles of 128x128 on, five to sixteen ways (bf16 512 x 2048 x 16384 73 us -> 43, 384 x 3072 x 8192
   // 46 -> 33, 512 x 3072 x 8192 48 -> 40; the 64x64 tiles the table took there are 128 workgroups or more, which the
-  // rule for few workgroups leaves whole): one part fewer where that reaches the twenty K tiles.  (Not for a
+  // rule for few workgroups leaves whole): fewer parts, down to six, where that reaches the twenty K tiles (int8
+  // 512 x 2048 x 16384 40 -> 31 in six parts; bf16 128 x 8192 x 8192 44 -> 36).  (Not for a
   // prepacked B: its kernels were not measured this way.)
   uint32_t band_split = 0;
   if (direct && !pr.packed_b && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) && tiles(128) >= kComputeUnits / 8 &&
       tiles(128) <= 200) {
     int64_t parts = 2 * kComputeUnits / tiles(128);
-    if (parts >= 6 && k_tiles / parts < 20) --parts;
+    while (parts > 6 && k_tiles / parts < 20) --parts;
     if (k_tiles / parts >= 20 && static_cast<uint64_t>(parts) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
       family = VECOPS_HIP_FAMILY_TILE_128;
       band_split = static_cast<uint32_t>(parts);
