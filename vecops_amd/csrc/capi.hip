@@ -281,14 +281,14 @@ void finish_tile_plan(const Problem& pr, VecopsHipPlan* plan, uint32_t forced_sp
     split = kComputeUnits / wgs;
     if (split > k_tiles / 4) split = k_tiles / 4;
     if (split > 64) split = 64;
-    // A split buys K tiles a workgroup no longer walks (0.2-0.4 us each: one workgroup on a compute unit waits out
+    // A split buys K tiles a workgroup no longer walks (0.2-0.4 us each, 0.3 in the rule: one workgroup on a compute unit waits out
     // every tile's loads) and costs a second kernel plus the partial sums' way to memory and back: about 5 us and
     // 0.75 us per MB (384 x 384 x 1024: 7.3 us unsplit against 10.4 in four parts; 640 x 640 x 2048: 10.4 against
     // 12.7 in two; 512 x 512 x 4096: 24.2 against 13.2 in four).  Halve the factor until it pays.
     // (a K tile of fp32 compute is sixteen 64-cycle MFMAs per 32 x 32 block: about 1 us - 512^3 in fp32 21.2 us
     // unsplit, 13.9 in four parts)
     const int64_t per_split_kb = pr.batch * pr.m * pr.n * 4 / 1024;
-    const int64_t tile_ns = pr.src == SRC_F32 ? 1000 : 250;
+    const int64_t tile_ns = pr.src == SRC_F32 ? 1000 : 300;
     while (split > 1) {
       const int64_t saved_ns = (k_tiles - (k_tiles + split - 1) / split) * tile_ns;
       const int64_t cost_ns = 5000 + split * per_split_kb * 3 / 4;
