@@ -133,6 +133,14 @@ def test_rule_table_known_answers():
                                      ((128, 8192, 8192), "tile_128", 6)):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
+    # ... and up to 256 tiles in two parts, from forty K tiles per part
+    for (m, n, k), split in (((1024, 4096, 11008), 2), ((1024, 4096, 6144), 2), ((1024, 4096, 4096), 1), ((896, 4096, 4096), 1)):
+        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == split, (m, n, k, p.split_k)
+    rc, p = _plan(_operand(capi.I8, (1024, 11008)), _operand(capi.I8, (4096, 11008)), _operand(capi.I32, (1024, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 2
+    rc, p = _plan(_operand(capi.I8, (1024, 8192)), _operand(capi.I8, (4096, 8192)), _operand(capi.I32, (1024, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1
     rc, p = _plan(_operand(capi.I8, (768, 4096)), _operand(capi.I8, (4096, 4096)), _operand(capi.I32, (768, 4096)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 1
     rc, p = _plan(_operand(capi.I8, (768, 12288)), _operand(capi.I8, (3072, 12288)), _operand(capi.I32, (768, 3072)))

@@ -426,12 +426,16 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // rule for few workgroups leaves whole): fewer parts, down to six, where that reaches the twenty K tiles (int8
   // 512 x 2048 x 16384 40 -> 31 in six parts; bf16 128 x 8192 x 8192 44 -> 36).  (Not for a
   // prepacked B: its kernels were not measured this way.)
+  // And up to 256 tiles (one workgroup on every unit) in two parts, from forty K tiles per part (bf16 1024 x 4096 x
+  // 11008 116 us -> 90, 896 x 4096 x 11008 114 -> 81, 1024 x 4096 x 6144 66 -> 58; int8 896 x 4096 x 11008 61 -> 52;
+  // with thirty-two per part - bf16 1024 x 4096 x 4096, int8 ... x 8192 - the unsplit tiles are level or ahead).
   uint32_t band_split = 0;
   if (direct && !pr.packed_b && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) && tiles(128) >= kComputeUnits / 8 &&
-      tiles(128) <= 200) {
+      tiles(128) <= kComputeUnits) {
     int64_t parts = 2 * kComputeUnits / tiles(128);
     while (parts > 6 && k_tiles / parts < 20) --parts;
-    if (k_tiles / parts >= 20 && static_cast<uint64_t>(parts) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
+    const int64_t least = tiles(128) > 200 ? 40 : 20;  // K tiles per part
+    if (k_tiles / parts >= least && static_cast<uint64_t>(parts) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
       family = VECOPS_HIP_FAMILY_TILE_128;
       band_split = static_cast<uint32_t>(parts);
     }
