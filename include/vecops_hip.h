@@ -78,7 +78,8 @@ typedef struct VecopsHipPlan {
   uint32_t vector_a;   /* 1 = 16-byte loads along K usable for A */
   uint32_t vector_b;   /* 1 = 16-byte loads usable for B */
   uint32_t b_layout;   /* 0 = K contiguous, 1 = N contiguous, 2 = generic */
-  uint32_t reserved;
+  uint32_t peeled_columns; /* > 0: the last so many columns of c are a second product with a plan of its own (few
+                              tiles, K split), cut off so that the rest fills whole rounds of workgroups */
   uint64_t workspace_bytes;
 } VecopsHipPlan;
 

@@ -149,6 +149,16 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 6
     rc, p = _plan(_operand(capi.I8, (512, 8192)), _operand(capi.I8, (1024, 8192)), _operand(capi.I32, (512, 1024)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 2    # exactly 128 workgroups: two parts just pay (24 -> 16 us)
+    # two rounds of 128 x 128 tiles and eight more: the last column of tiles is a product of its own (64 x 64 tiles, K in
+    # five parts), the rest fills two rounds; a required family runs the product whole
+    big_n = (_operand(capi.BF16, (1536, 4096)), _operand(capi.BF16, (11008, 4096)), _operand(capi.BF16, (1536, 11008)))
+    rc, p = _plan(*big_n)
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1 and p.peeled_columns == 128
+    assert p.workspace_bytes == 5 * 1536 * 128 * 4
+    rc, p = _plan_family(*big_n, "tile_128", capi.SELECT_REQUIRE)
+    assert rc == 0 and p.peeled_columns == 0 and p.workspace_bytes == 0
+    rc, p = _plan(_operand(capi.BF16, (2048, 4096)), _operand(capi.BF16, (11008, 4096)), _operand(capi.BF16, (2048, 11008)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.peeled_columns == 0   # 1376 tiles: the third round is two thirds full
     # a split must pay for its second kernel: sixteen or thirty-two K tiles are walked in one go, sixty-four are not
     for (m, n, k), split in (((384, 384, 1024), 1), ((640, 640, 2048), 1), ((512, 512, 4096), 4), ((64, 64, 65536), 64)):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.F32, (m, n)))

@@ -929,3 +929,42 @@ def test_mid_band_k_split_with_dequantisation(device, m, n, k, pad):
     acc = ((a.astype(np.float64) @ b.astype(np.float64).T).astype(np.int64) + corr[None, :]).astype(np.int32)   # exact in float64
     want = (acc.astype(np.float32) * rs[:, None].astype(np.float32)) * cs[None, :].astype(np.float32)
     assert np.array_equal(c.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("kind,m,n,k", [("bf16", 1536, 11008, 2048), ("bf16", 1500, 11000, 2056), ("i8", 1536, 11008, 4096)])
+def test_peeled_columns(device, oracle, kind, m, n, k):
+    """Two rounds of 128 x 128 tiles and a few more: the rule table cuts the last columns of tiles off and runs them
+    as a product of their own (few tiles, K split), so that the rest fills whole rounds.  Both parts against the
+    oracle (int8: exact), with a C input; a required family runs the product whole."""
+    import torch
+    from vecops_amd import capi
+    if kind == "bf16":
+        a, b = synth.bf16_round(synth.uniform_pm1(1, (m, k))), synth.bf16_round(synth.uniform_pm1(2, (n, k)))
+        ta, tb = dev_bf16(a, device), dev_bf16(b, device)
+        cin = synth.uniform_pm1(3, (m, n)).astype(np.float32)
+        c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    else:
+        a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+        ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+        cin = (synth.draws(3, m * n) % np.uint64(1 << 20)).astype(np.int32).reshape(m, n)
+        c = torch.full((m, n), -1, dtype=torch.int32, device=device)
+    tci = torch.from_numpy(cin).to(device)
+    plan = capi.plan_matmul(ta, tb, c, c_in=tci)
+    assert capi.FAMILY_NAMES[plan.family] == "tile_128" and plan.split_k == 1 and 0 < plan.peeled_columns <= 256
+    whole_plan = capi.plan_matmul_family(ta, tb, c, capi.family_request("tile_128"), c_in=tci)
+    assert whole_plan.peeled_columns == 0
+    capi.matmul(ta, tb, c, c_in=tci)
+    whole = torch.empty_like(c)
+    capi.matmul_family(ta, tb, whole, capi.family_request("tile_128", split_k=1), c_in=tci)
+    torch.cuda.synchronize()
+    cut = n - plan.peeled_columns
+    if kind == "bf16":
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a, b, want, cin=cin, acc_f64=True)
+        got = c.cpu().numpy()
+        assert rel_err(got[:, :cut], want[:, :cut]) <= fp32_tol(k) and rel_err(got[:, cut:], want[:, cut:]) <= fp32_tol(k)
+        assert np.array_equal(got[:, :cut], whole.cpu().numpy()[:, :cut])   # the same kernel on the same tiles
+    else:
+        want = (a.astype(np.float64) @ b.astype(np.float64).T).astype(np.int64) + cin   # exact: sums stay below 2^53
+        want = (want & 0xffffffff).astype(np.uint32).view(np.int32)
+        assert np.array_equal(c.cpu().numpy(), want)

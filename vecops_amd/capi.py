@@ -49,7 +49,7 @@ class Operand(C.Structure):
 
 class Plan(C.Structure):
     _fields_ = [("family", C.c_uint32), ("split_k", C.c_uint32), ("vector_a", C.c_uint32), ("vector_b", C.c_uint32),
-                ("b_layout", C.c_uint32), ("reserved", C.c_uint32), ("workspace_bytes", C.c_uint64)]
+                ("b_layout", C.c_uint32), ("peeled_columns", C.c_uint32), ("workspace_bytes", C.c_uint64)]
 
 
 class Epilogue(C.Structure):

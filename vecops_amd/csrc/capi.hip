@@ -306,6 +306,21 @@ void finish_tile_plan(const Problem& pr, VecopsHipPlan* plan, uint32_t forced_sp
 
 int fetch_mode(const Problem& pr, const VecopsHipPlan& plan);
 
+// The two halves of a problem cut between columns n_main - 1 and n_main of C: rows of B, columns of C and C_in.
+void cut_columns(const Problem& pr, int64_t n_main, Problem* main, Problem* rest) {
+  *main = pr;
+  *rest = pr;
+  main->n = main->b.rows = main->c.cols = n_main;
+  rest->n = rest->b.rows = rest->c.cols = pr.n - n_main;
+  rest->b.data = static_cast<char*>(pr.b.data) + n_main * pr.b.rs * dtype_bytes(pr.b.dtype);
+  rest->c.data = static_cast<char*>(pr.c.data) + n_main * pr.c.cs * dtype_bytes(pr.c.dtype);
+  if (pr.has_cin) {
+    main->cin.cols = n_main;
+    rest->cin.cols = pr.n - n_main;
+    rest->cin.data = static_cast<char*>(pr.cin.data) + n_main * pr.cin.cs * dtype_bytes(pr.cin.dtype);
+  }
+}
+
 // The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure
 // integer function of (operand class, m, n, k); it picks the workgroup tile by
 // how many tiles the problem yields against the 256 compute units and splits K
@@ -314,7 +329,8 @@ int fetch_mode(const Problem& pr, const VecopsHipPlan& plan);
 // data, a lightly loaded round clocks higher, and narrower tiles (256x192 was
 // measured) cost more LDS and L2 traffic per flop than the better balance saves.
 // (scratch_limit: partial sums the caller can hold - the mid-band K split below is skipped where it needs more)
-void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UINT64_MAX) {
+// (peel_allowed: false for the product of a peel itself)
+void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UINT64_MAX, bool peel_allowed = true) {
   memset(plan, 0, sizeof(*plan));
   plan->split_k = 1;
   if (pr.batch == 0 || pr.m == 0 || pr.n == 0) {
@@ -442,6 +458,30 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   }
   plan->family = family;
   finish_tile_plan(pr, plan, band_split);
+  // Two or more rounds of workgroups and a last one that is nearly empty (1536 x 11008: 1032 tiles of 128x128 are two
+  // rounds of 512 and eight tiles, which cost a third round: 141 us where two would take 95): the last columns of
+  // tiles are cut off, so that the rest fills whole rounds, and run as a product of their own - few tiles and the
+  // whole K, which the rules above split.  peeled_columns = the columns of C that second product computes.
+  if (direct && !pr.packed_b && !pr.dequant && pr.fused == nullptr && pr.src != SRC_I8_FLIP && pr.batch == 1 && plan->split_k == 1 &&
+      (family == VECOPS_HIP_FAMILY_TILE_128 || family == VECOPS_HIP_FAMILY_TILE_256) && k_tiles >= 32 && peel_allowed) {
+    const int64_t slots = family == VECOPS_HIP_FAMILY_TILE_128 ? 2 * kComputeUnits : kComputeUnits;
+    const int64_t tiles_m = (pr.m + tile_m - 1) / tile_m, tiles_n = (pr.n + tile_n - 1) / tile_n;
+    const int64_t count = tiles_m * tiles_n, over = count % slots;
+    if (count > slots && over > 0 && over * 8 <= slots) {
+      const int64_t cut = (over + tiles_m - 1) / tiles_m;  // columns of tiles
+      if (cut * 4 <= tiles_n) {
+        const int64_t n_main = (tiles_n - cut) * tile_n;
+        Problem main, rest;
+        cut_columns(pr, n_main, &main, &rest);
+        VecopsHipPlan rest_plan;
+        choose(rest, &rest_plan, scratch_limit, false);
+        if (rest_plan.workspace_bytes <= scratch_limit) {
+          plan->peeled_columns = static_cast<uint32_t>(pr.n - n_main);
+          plan->workspace_bytes = rest_plan.workspace_bytes;
+        }
+      }
+    }
+  }
 }
 
 const char* family_name(uint32_t family) {
@@ -479,8 +519,15 @@ int32_t apply_request(const Problem& pr, const VecopsHipFamilyRequest* request, 
     return fail(ST_NOT_APPLICABLE, "matmul: the required family %s cannot serve this call (the rule table chooses %s)",
                 family_name(request->family), family_name(plan->family));
   }
-  if (request->family == plan->family && request->split_k == 0) return ST_OK;
+  if (request->family == plan->family && request->split_k == 0) {
+    if (plan->peeled_columns > 0) {  // a requested family runs the whole product (a peel's second product is the table's choice)
+      plan->peeled_columns = 0;
+      finish_tile_plan(pr, plan, 1);
+    }
+    return ST_OK;
+  }
   plan->family = request->family;
+  plan->peeled_columns = 0;  // (the rule table's peel belongs to its own choice of family)
   if (tile_m != 0) {
     finish_tile_plan(pr, plan, request->split_k);
   } else {
@@ -586,6 +633,19 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   if (plan.workspace_bytes > workspace_size || (plan.workspace_bytes > 0 && workspace == nullptr))
     return fail(ST_INVALID, "matmul: workspace of %llu bytes required, %llu supplied",
                 (unsigned long long)plan.workspace_bytes, (unsigned long long)workspace_size);
+
+  if (plan.peeled_columns > 0) {
+    // the last columns of C as a product of their own (choose() planned it with the same limit and found that it fits)
+    Problem main, rest;
+    cut_columns(pr, pr.n - plan.peeled_columns, &main, &rest);
+    VecopsHipPlan main_plan = plan, rest_plan;
+    main_plan.peeled_columns = 0;
+    main_plan.workspace_bytes = 0;
+    choose(rest, &rest_plan, workspace_size, false);
+    int32_t rc = run_problem(main, main_plan, row_scales, column_scales, correction, nullptr, 0, stream);
+    if (rc != ST_OK) return rc;
+    return run_problem(rest, rest_plan, row_scales, column_scales, correction, workspace, workspace_size, stream);
+  }
 
   TileGemmParams p = base_params(pr, row_scales, column_scales, correction, workspace);
   const bool is_int = pr.src == SRC_I8 || pr.src == SRC_I8_FLIP;
