@@ -118,32 +118,38 @@ def _bf16_operands(dev):
 
 
 def bench_mfma_ceiling(dev, steps, warmup, which="bf16"):
-    """The matrix-core yardstick: nothing but independent matrix instructions of the tile kernels' shape, one
-    wavefront per SIMD on all compute units, on the benchmark's operand values and on zeros."""
+    """The matrix-core yardstick: nothing but independent matrix instructions, one wavefront per SIMD on all compute
+    units, on the benchmark's operand values and on zeros - on both instruction shapes the tile kernels use (32x32 and
+    16x16).  `value` is the higher of the two on the benchmark's operands, `shape` names it."""
     import torch
     from vecops_amd import capi, synth
     out = torch.empty(256 * 256, dtype=torch.int32, device=dev)
     if which == "bf16":
         _, _, values, _ = _bf16_operands(dev)
-        label, unit, peak = "v_mfma_f32_32x32x16_bf16", "TFLOP/s", PEAK_BF16_TFLOPS
+        labels, unit, peak = ("v_mfma_f32_32x32x16_bf16", "v_mfma_f32_16x16x32_bf16"), "TFLOP/s", PEAK_BF16_TFLOPS
         what = "normal(0, 0.02) rounded to bf16 (the GEMM's A operand)"
     else:
         values = torch.from_numpy(synth.int8_sym(1, (2048, 4096))).to(dev)
-        label, unit, peak = "v_mfma_i32_32x32x32_i8", "TOP/s", PEAK_INT8_TOPS
+        labels, unit, peak = ("v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8"), "TOP/s", PEAK_INT8_TOPS
         what = "int8 uniform[-127,127] (the quantised matmul's A operand)"
     zeros = torch.zeros_like(values)
     res = {}
-    for name, operands in (("benchmark_operands", values), ("zeros", zeros)):
-        ops_per_launch = [0]
+    for shape in (0, 1):
+        for name, operands in (("benchmark_operands", values), ("zeros", zeros)):
+            ops_per_launch = [0]
 
-        def launch(i, operands=operands):
-            ops_per_launch[0] = capi.mfma_stream(operands, 256, 512, out)
-        t = _measure(launch, max(5, steps // 10), max(2, warmup // 5))
-        res[name] = ops_per_launch[0] / (t["event_ms"] * 1e-3) / 1e12
-    return {"metric": f"mfma_ceiling_{which}", "workload": f"256 workgroups x 4 wavefronts x 16384 independent {label} "
-            f"(sixteen 32x32 accumulator tiles per wavefront, no memory traffic), operands: {what}; and zeros",
-            "value": res["benchmark_operands"], "unit": unit, "on_zeros": res["zeros"], "peak": peak,
-            "frac_of_peak": res["benchmark_operands"] / peak, "frac_of_peak_on_zeros": res["zeros"] / peak}
+            def launch(i, operands=operands, shape=shape):
+                ops_per_launch[0] = capi.mfma_stream(operands, 256, 512 if shape == 0 else 1024, out, shape=shape)
+            t = _measure(launch, max(5, steps // 10), max(2, warmup // 5))
+            res[shape, name] = ops_per_launch[0] / (t["event_ms"] * 1e-3) / 1e12
+    best = max((0, 1), key=lambda shape: res[shape, "benchmark_operands"])
+    return {"metric": f"mfma_ceiling_{which}", "workload": "256 workgroups x 4 wavefronts of nothing but independent matrix "
+            f"instructions (sixteen accumulator tiles per wavefront, no memory traffic), operands: {what}; and zeros",
+            "value": res[best, "benchmark_operands"], "unit": unit, "shape": labels[best],
+            "on_zeros": res[best, "zeros"], "peak": peak,
+            "by_shape": {labels[shape]: {"benchmark_operands": res[shape, "benchmark_operands"], "zeros": res[shape, "zeros"]}
+                         for shape in (0, 1)},
+            "frac_of_peak": res[best, "benchmark_operands"] / peak, "frac_of_peak_on_zeros": res[best, "zeros"] / peak}
 
 
 def bench_bf16_gemm(dev, steps, warmup):
@@ -415,6 +421,62 @@ def bench_tile_families(dev, steps, warmup):
             "each required tile family", "unit": "us", "value": base, "families": rows}
 
 
+RULE_CHECK_SHAPES = [
+    # (class, M, N, K): the shapes the rule table's thresholds were set on, and the known holes
+    ("bf16", 4096, 4096, 4096), ("bf16", 2048, 2048, 2048), ("bf16", 1536, 4096, 4096), ("bf16", 1024, 4096, 4096),
+    ("bf16", 768, 4096, 4096), ("bf16", 512, 4096, 4096), ("bf16", 768, 11008, 4096), ("bf16", 1024, 4096, 11008),
+    ("bf16", 768, 3072, 12288), ("bf16", 512, 2048, 16384), ("bf16", 384, 384, 1024), ("bf16", 512, 512, 4096),
+    ("bf16", 3000, 3000, 3000), ("bf16", 1536, 11008, 4096),
+    ("int8", 2048, 11008, 4096), ("int8", 4096, 4096, 4096), ("int8", 1024, 4096, 4096), ("int8", 768, 3072, 12288),
+    ("int8", 512, 1024, 8192),
+]
+
+
+def bench_rule_check(dev, steps, warmup):
+    """The rule table against what it chooses between: every shape of RULE_CHECK_SHAPES on every tile family with K
+    split 1, 2, 3 and 4 ways (vecops_hip_matmul_family, Require), and as the table plans it.  `regret_us` = the
+    table's time minus the fastest requested combination's."""
+    import numpy as np
+    import torch
+    from vecops_amd import capi, synth
+    families = ["tile_256", "tile_256x128", "tile_128x256", "tile_128", "tile_64"]
+    steps, warmup = max(10, steps // 10), max(10, warmup // 10)
+    ws = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+    rows = []
+    for kind, m, n, k in RULE_CHECK_SHAPES:
+        if kind == "bf16":
+            a = torch.from_numpy(synth.bf16_round(synth.normal(1, (m, k), 0.02)).view(np.int16)).to(dev).view(torch.bfloat16)
+            b = torch.from_numpy(synth.bf16_round(synth.normal(2, (n, k), 0.02)).view(np.int16)).to(dev).view(torch.bfloat16)
+            c = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+        else:
+            a = torch.from_numpy(synth.int8_sym(1, (m, k))).to(dev)
+            b = torch.from_numpy(synth.int8_sym(2, (n, k))).to(dev)
+            c = torch.empty((m, n), dtype=torch.int32, device=dev)
+        plan = capi.plan_matmul(a, b, c)
+        auto = _measure(lambda i: capi.matmul(a, b, c, workspace=ws), steps, warmup)["event_ms"] * 1e3
+        tried = {}
+        for family in families:
+            for split in (1, 2, 3, 4):
+                request = capi.family_request(family, capi.SELECT_REQUIRE, split_k=split)
+                try:
+                    need = capi.plan_matmul_family(a, b, c, request).workspace_bytes
+                    if need > ws.numel():
+                        continue
+                    t = _measure(lambda i: capi.matmul_family(a, b, c, request, workspace=ws), steps, warmup)
+                except capi.VecopsHipError:
+                    continue   # the family cannot serve this problem
+                tried[f"{family}/{split}"] = round(t["event_ms"] * 1e3, 2)
+        best = min(tried, key=tried.get)
+        pick = capi.FAMILY_NAMES.get(plan.family, str(plan.family)) + f"/{max(plan.split_k, 1)}" + (
+            f" (+{plan.peeled_columns} peeled columns)" if plan.peeled_columns else "")
+        rows.append({"shape": f"{kind} {m}x{n}x{k}", "pick": pick, "pick_us": round(auto, 2), "best": best,
+                     "best_us": tried[best], "regret_us": round(auto - tried[best], 2), "tried_us": tried})
+    worst = max(rows, key=lambda r: r["regret_us"])
+    return {"metric": "rule_table_regret", "workload": "every shape of RULE_CHECK_SHAPES on every tile family x K split 1..4 "
+            "against the rule table's own plan (HIP events)", "unit": "us", "value": worst["regret_us"],
+            "worst_shape": worst["shape"], "shapes": rows}
+
+
 def bench_copy(dev, steps, warmup):
     """A plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
     counters of the other workloads are scaled by."""
@@ -486,7 +548,7 @@ def cpu_baseline(a, b_kn):
 
 
 ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "fp32", "batched",
-        "families", "grouped"]
+        "families", "grouped", "rule_check"]
 
 
 def main() -> int:
@@ -530,6 +592,7 @@ def main() -> int:
         "batched": lambda: bench_batched(dev, K, W, *[int(v) for v in args.batched_shape.split(",")]),
         "families": lambda: bench_tile_families(dev, K, W),
         "grouped": lambda: bench_grouped(dev, K, W),
+        "rule_check": lambda: bench_rule_check(dev, K, W),
     }
     if args.only in single:
         print(json.dumps(single[args.only]()))
@@ -537,30 +600,49 @@ def main() -> int:
 
     main_res = bench_bf16_gemm(dev, K, W)
     a, b_kn = main_res.pop("host")
-    line = {
+    head = {
         "metric": "bf16_gemm_4096_tflops", "value": main_res["value"], "unit": "TFLOP/s", "n_gpus": 1,
         "steps": K, "warmup": W, "ms_per_step": main_res["wall_ms"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "bf16 GEMM M=N=K=4096, A[M,K] and B[K,N] row-major, normal(0,0.02), fp32 accumulate, "
                                "bf16 output (BASELINE configs[1])", "M": 4096, "N": 4096, "K": 4096},
-        "roofline": main_res["roofline"],
     }
+    roofline = main_res["roofline"]
+    secondary = None
     if args.only != "bf16":
         ceiling_bf16 = bench_mfma_ceiling(dev, K, W, "bf16")
         ceiling_int8 = bench_mfma_ceiling(dev, K, W, "int8")
-        # what the machine sustains on these operand values with nothing but matrix instructions: the practical
-        # ceiling (the clocks follow the power the multipliers draw); `frac` stays against the nominal peak
-        line["roofline"]["measured_ceiling"] = ceiling_bf16["value"]
-        line["roofline"]["frac_of_ceiling"] = line["roofline"]["achieved"] / ceiling_bf16["value"]
-        line["secondary"] = [bench_int8_dequant(dev, K, W, ceiling=ceiling_int8["value"]),
-                             bench_gemv(dev, K, W, m=1), bench_gemv(dev, K, W, m=4), bench_gemv(dev, K, W, m=16),
-                             bench_fp32_gemm(dev, K, W, "bf16"), bench_fp32_gemm(dev, K, W, "f32")]
-        line["secondary"] += [bench_batched(dev, K, W, m, n, k)
-                              for (m, n, k) in [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)]]
-        line["secondary"] += [bench_bf16_gemm_packed(dev, K, W), bench_int8_dequant_packed(dev, K, W),
-                              bench_runtime_quant(dev, K, W), bench_grouped(dev, K, W), ceiling_bf16, ceiling_int8]
+        # what the machine sustains on these operand values with nothing but matrix instructions (the better of the
+        # two instruction shapes): the practical ceiling - the clocks follow the power the multipliers draw; `frac`
+        # stays against the nominal peak
+        roofline["measured_ceiling"] = ceiling_bf16["value"]
+        roofline["measured_ceiling_shape"] = ceiling_bf16["shape"]
+        roofline["frac_of_ceiling"] = roofline["achieved"] / ceiling_bf16["value"]
+        int8 = bench_int8_dequant(dev, K, W, ceiling=ceiling_int8["value"])
+        gemv = {m: bench_gemv(dev, K, W, m=m) for m in (1, 4, 16)}
+        fp32 = {c: bench_fp32_gemm(dev, K, W, c) for c in ("bf16", "f32")}
+        packed16, packed8 = bench_bf16_gemm_packed(dev, K, W), bench_int8_dequant_packed(dev, K, W)
+        secondary = [bench_batched(dev, K, W, m, n, k)
+                     for (m, n, k) in [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)]]
+        secondary += [bench_runtime_quant(dev, K, W), bench_grouped(dev, K, W), ceiling_bf16, ceiling_int8, packed16, packed8,
+                      fp32["bf16"], fp32["f32"], gemv[16], gemv[4], gemv[1], int8]
+
+        def brief(r):
+            return {"frac": round(r["roofline"]["frac"], 4), "event_us": round(r["roofline"]["event_ms"] * 1e3, 2),
+                    "value": round(r["value"], 1), "unit": r["unit"]}
+        # the other components of the headline metric and the remaining benchmark configurations, in short: the full
+        # records are in `secondary`
+        roofline["also"] = {"int8_cfg4": brief(int8), "int8_cfg4_prepacked": brief(packed8), "gemv_m1": brief(gemv[1]),
+                            "gemv_m4": brief(gemv[4]), "gemv_m16": brief(gemv[16]), "fp32_1024_f32_compute": brief(fp32["f32"]),
+                            "fp32_1024_bf16_compute": brief(fp32["bf16"]), "bf16_4096_prepacked": brief(packed16)}
+    # (the long list first: a reader who sees only the end of the line sees the headline and its roofline)
+    line = {}
+    if secondary is not None:
+        line["secondary"] = secondary
     if not args.no_cpu and args.only is None:
         line["cpu_baseline"] = cpu_baseline(a, b_kn)
+    line.update(head)
+    line["roofline"] = roofline
     print(json.dumps(line))
     return 0
 

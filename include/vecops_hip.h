@@ -479,6 +479,16 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_i8_dequant_packed_b(const int8_t* a,
 VECOPS_HIP_EXPORT uint64_t vecops_hip_mfma_stream_ops(uint32_t dtype, int32_t workgroups, int32_t iters);
 VECOPS_HIP_EXPORT int32_t vecops_hip_mfma_stream(uint32_t dtype, const void* operands, uint64_t operand_bytes,
                                                  int32_t workgroups, int32_t iters, void* out, void* stream);
+/*
+ * The same yardstick on either matrix-instruction shape the tile kernels use.  shape 0: the 32x32 instructions above;
+ * shape 1: v_mfma_f32_16x16x32_bf16 (dtype 11) / v_mfma_i32_16x16x64_i8 (dtype 2), sixteen 16x16 accumulator quads per
+ * wavefront - the shape of the 256x256 tile's written-out K loop and of the small tiles, which draws less power per
+ * multiply-add.  Operations per launch: vecops_hip_mfma_stream_shape_ops.
+ */
+VECOPS_HIP_EXPORT uint64_t vecops_hip_mfma_stream_shape_ops(uint32_t dtype, uint32_t shape, int32_t workgroups, int32_t iters);
+VECOPS_HIP_EXPORT int32_t vecops_hip_mfma_stream_shape(uint32_t dtype, uint32_t shape, const void* operands,
+                                                       uint64_t operand_bytes, int32_t workgroups, int32_t iters, void* out,
+                                                       void* stream);
 
 #ifdef __cplusplus
 }

@@ -116,8 +116,9 @@ def test_f16_skinny_family(device, oracle, narrow, wide, k, out):
 
 @pytest.mark.parametrize("m,n,k", [(300, 260, 1000), (37, 51, 79), (512, 768, 512), (2, 3, 64, 40, 200)][:3] + [(2457, 1221, 72)])
 def test_f16_prepacked_b(device, oracle, m, n, k):
-    """Half weights packed once (the 16-bit permutation of the bf16 pack): bit-equal to the plain product on the
-    256 x 256 tiles, which multiply in the packed kernel's order (v_mfma_f32_32x32x16_f16)."""
+    """Half weights packed once (the 16-bit permutation of the bf16 pack): equal to the plain product on the 256 x 256
+    tiles up to the order of the fp32 sums (the packed kernel multiplies on v_mfma_f32_32x32x16_f16, the plain tile of
+    aligned operands on v_mfma_f32_16x16x32_f16: 16 against 32 k per instruction)."""
     import torch
     from vecops_amd import capi
     a, b = _half(1, (m, k)), _half(2, (n, k))
@@ -130,8 +131,8 @@ def test_f16_prepacked_b(device, oracle, m, n, k):
         split_k = capi.plan_matmul_packed_b(ta, packed, c).split_k          # the same partition of K
         capi.matmul_family(ta, tb, ref, capi.family_request("tile_256", split_k=split_k))
         torch.cuda.synchronize()
-        assert torch.equal(c.view(torch.int32 if dt == torch.float32 else torch.int16),
-                           ref.view(torch.int32 if dt == torch.float32 else torch.int16))
+        tol = 2e-6 * max(1.0, k / 32) if dt == torch.float32 else 2.0 ** -10
+        assert rel_err(c.float().cpu().numpy(), ref.float().cpu().numpy()) <= tol
     want = np.zeros((m, n), np.float32)
     oracle.matmul(a, b, want, atom=O.ATOM_F16F32, acc_f64=True)
     c = torch.empty((m, n), device=device)

@@ -222,7 +222,9 @@ def test_packed_full_size_bf16_sampled(device, oracle):
     want = oracle.matmul_sampled(a, b, rr, cc)
     got = c.cpu().numpy()
     assert rel_err(got[rr, cc], want) <= fp32_tol(k)
-    assert torch.equal(c, c_plain)  # same K order per accumulator: the same bits
+    # (the plain kernel's 256 x 256 tile of aligned bf16 operands sums 32 k per matrix instruction, the packed kernel
+    # 16: the two agree up to the order of the fp32 sums)
+    assert rel_err(got, c_plain.cpu().numpy()) <= fp32_tol(k)
 
 
 def test_pack_b_compensated_reference_case(device):

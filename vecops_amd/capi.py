@@ -29,6 +29,7 @@ EXPORTS = [
     "vecops_hip_matmul_runtime_quant_packed_b_workspace", "vecops_hip_matmul_runtime_quant_packed_b",
     "vecops_hip_static_workspace_bytes", "vecops_hip_matmul_static_workspace",
     "vecops_hip_mfma_stream_ops", "vecops_hip_mfma_stream",
+    "vecops_hip_mfma_stream_shape_ops", "vecops_hip_mfma_stream_shape",
     "vecops_hip_plan_matmul_family", "vecops_hip_matmul_family",
     "vecops_hip_matmul_runtime_quant_batched_workspace", "vecops_hip_matmul_runtime_quant_batched",
     "vecops_hip_matmul_grouped_workspace", "vecops_hip_matmul_grouped",
@@ -106,6 +107,10 @@ def lib() -> C.CDLL:
         L.vecops_hip_mfma_stream_ops.argtypes = [C.c_uint32, C.c_int32, C.c_int32]
         L.vecops_hip_mfma_stream.argtypes = [C.c_uint32, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_void_p,
                                              C.c_void_p]
+        L.vecops_hip_mfma_stream_shape_ops.restype = C.c_uint64
+        L.vecops_hip_mfma_stream_shape_ops.argtypes = [C.c_uint32, C.c_uint32, C.c_int32, C.c_int32]
+        L.vecops_hip_mfma_stream_shape.argtypes = [C.c_uint32, C.c_uint32, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32,
+                                                   C.c_void_p, C.c_void_p]
         L.vecops_hip_matmul_static_workspace.argtypes = [P, P, P, P, C.c_uint32, C.c_void_p]
         L.vecops_hip_matmul_i8_dequant.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p,
                                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
@@ -281,13 +286,13 @@ def matmul_static_workspace(a, b, c, c_in=None, compute=COMPUTE_BF16, stream=Non
     return c
 
 
-def mfma_stream(operands, workgroups: int, iters: int, out, stream=None) -> int:
-    """Launches the matrix-core yardstick on the values of `operands` (bf16 or int8 tensor); returns the
-    operations (2 per multiply-add) the launch performs."""
+def mfma_stream(operands, workgroups: int, iters: int, out, stream=None, shape: int = 0) -> int:
+    """Launches the matrix-core yardstick on the values of `operands` (bf16 or int8 tensor) with the 32x32 (shape 0) or
+    the 16x16 (shape 1) matrix instructions; returns the operations (2 per multiply-add) the launch performs."""
     code = _torch_dtype_code(operands)
-    _check(lib().vecops_hip_mfma_stream(code, operands.data_ptr(), operands.numel() * operands.element_size(),
-                                        workgroups, iters, out.data_ptr(), _stream_handle(stream)))
-    return lib().vecops_hip_mfma_stream_ops(code, workgroups, iters)
+    _check(lib().vecops_hip_mfma_stream_shape(code, shape, operands.data_ptr(), operands.numel() * operands.element_size(),
+                                              workgroups, iters, out.data_ptr(), _stream_handle(stream)))
+    return lib().vecops_hip_mfma_stream_shape_ops(code, shape, workgroups, iters)
 
 
 def epilogue(activation=None, scale=None, shift=None, row_scales=None, column_scales=None, clamp=(0.0, 0.0)) -> Epilogue:

@@ -815,12 +815,12 @@ void launch_skinny_mfma(const SkinnyW8A16Params& p, hipStream_t stream) {
 }
 
 // The register-resident variant: K must be exactly 8 wavefronts x 8 steps x 64.
-template <int SPG, int TILES>
-void launch_skinny_mfma_resident(const SkinnyW8A16Params& p, int passes, hipStream_t stream) {
-  const int64_t rows_per_wg = static_cast<int64_t>(16) * TILES * passes;
+template <int SPG, int TILES, int PASSES>
+void launch_skinny_mfma_resident(const SkinnyW8A16Params& p, hipStream_t stream) {
+  const int64_t rows_per_wg = static_cast<int64_t>(16) * TILES * PASSES;
   const int64_t blocks = (p.n + rows_per_wg - 1) / rows_per_wg;
-  hipLaunchKernelGGL((skinny_w8a16_mfma_resident_kernel<SPG, TILES>), dim3(static_cast<unsigned>(blocks)), dim3(512), 0,
-                     stream, p, passes);
+  hipLaunchKernelGGL((skinny_w8a16_mfma_resident_kernel<SPG, TILES, PASSES>), dim3(static_cast<unsigned>(blocks)), dim3(512),
+                     0, stream, p);
 }
 
 // Problem description of a matmul whose B operand is prepacked: b is described as the dense
@@ -1417,6 +1417,8 @@ int32_t describe_grouped(uint32_t count, const VecopsHipOperand* a, const Vecops
     all_k = all_k && (mode == MODE_KVEC || mode == MODE_KVEC_DMA);
     all_n = all_n && (mode == MODE_NVEC_B || mode == MODE_NVEC_B_DMA);
     all_dma = all_dma && (mode == MODE_KVEC_DMA || mode == MODE_NVEC_B_DMA);
+    // (the 256 x 256 tile's written-out K loop walks a [K,N] operand with 32-bit byte offsets)
+    if (mode == MODE_NVEC_B_DMA && g->problems[i].k * g->problems[i].b.cs * 2 >= (int64_t{1} << 31)) all_dma = false;
   }
   g->mode = all_k ? (all_dma ? MODE_KVEC_DMA : MODE_KVEC) : all_n ? (all_dma ? MODE_NVEC_B_DMA : MODE_NVEC_B) : MODE_GENERIC;
   int64_t next = 0;
@@ -1758,12 +1760,13 @@ int32_t vecops_hip_matmul_w8a16_group(const void* x, int64_t ldx, const int8_t* 
     // two rows of activations: the streaming walk of M = 1 with both rows resident (13.9 us at N = 14336 where
     // the matrix-core kernel takes 17.0)
     hipLaunchKernelGGL((skinny_w8a16_stream_rows_kernel<2, 4>), dim3(kComputeUnits * kStreamGroupsPerUnit), dim3(256), 0, s, p);
-  } else if (m >= 2 && k == 4096 && (group == 128 || group == 256) && n >= 2048) {
+  } else if (m >= 2 && k == 4096 && (group == 128 || group == 256) && n >= 2048 && ldx < (int64_t{1} << 26)) {
+    // (the activation rows are fetched through 32-bit byte offsets)
     // activations resident in registers; a workgroup walks two blocks of 32 rows (224 workgroups at
     // N = 14336).  More passes reuse the activations further but leave too few workgroups to pull
     // the bandwidth: 4 passes measured 50 % slower.
-    if (group == 128) launch_skinny_mfma_resident<2, 2>(p, 2, s);
-    else launch_skinny_mfma_resident<4, 2>(p, 2, s);
+    if (group == 128) launch_skinny_mfma_resident<2, 2, 2>(p, s);
+    else launch_skinny_mfma_resident<4, 2, 2>(p, s);
   } else if (m >= 3 && mfma_ok) {
     const int tiles = m > 4 ? 2 : 1;  // more weight rows per workgroup = fewer activation reloads
     if (group == 64) { if (tiles == 2) launch_skinny_mfma<1, 2>(p, s); else launch_skinny_mfma<1, 1>(p, s); }

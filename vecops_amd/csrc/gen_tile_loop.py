@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""Writes tile_loop_asm.inc: the K loop of the 256x256 workgroup tile on the 16x16 matrix instructions, as one
+instruction stream (inline assembly text).
+
+Why a written-out stream: a wavefront of this tile owns 128x128 of C = 64 accumulator quads = all 256 registers of
+the accumulation half of the register file.  Through the compiler's builtins such a loop gets its accumulators
+renamed on every trip and copied back at the loop's head; written out, every matrix instruction accumulates in
+place, every LDS address is a base register plus an immediate, and the order of issue is exactly the one below.
+
+One K tile (128 bytes of each operand row) = two k-steps of 64 matrix instructions.  The tile in LDS stage S:
+  k-step 0   multiplies fragment set 0 and reads the fragments of k-step 1 (stage S) into set 1
+  barrier    (every wavefront has read stage S for the last time; the next tile's loads have landed in stage S^1)
+  k-step 1   multiplies set 1, reads the fragments of the next tile's k-step 0 (stage S^1) into set 0 and issues
+             the loads (they write LDS themselves) of the tile after the next into stage S
+On the last two trips the loads go out against a descriptor of no records: they fetch nothing.
+
+Fragment registers are fixed (v128..v255: set s, A block i at v[128+64s+4i..], B block j at v[160+64s+4j..]); the
+accumulators, addresses and descriptors are operands of the statement (see asm_k_loop in tile_gemm.h, which
+documents each of them).
+
+    python3 gen_tile_loop.py > tile_loop_asm.inc
+"""
+import os
+import sys
+
+# experiments (not for shipping: results are wrong without the waits): GEN_DROP=vmwait,barrier,dma,reads
+DROP = set(filter(None, os.environ.get("GEN_DROP", "").split(",")))
+
+
+def fa(s, i):
+    return f"v[{128 + 64 * s + 4 * i}:{128 + 64 * s + 4 * i + 3}]"
+
+
+def fb(s, j):
+    return f"v[{160 + 64 * s + 4 * j}:{160 + 64 * s + 4 * j + 3}]"
+
+
+def fb_half(s, j, h):
+    r = 160 + 64 * s + 4 * j + 2 * h
+    return f"v[{r}:{r + 1}]"
+
+
+STAGE = 65536       # bytes of one LDS stage: 256 rows of A and 256 of B (either layout), 128 bytes each
+B_TILE = 32768      # the B tile lies behind the A tile
+PITCH_TR = 512      # bytes between the k rows of a B tile kept as it lies in memory ([k][n], 256 columns)
+
+
+def fragment_reads(tr, st, ks, to_set):
+    """The reads of k-step ks of stage st into fragment set to_set, in the order the matrix instructions consume
+    them: A block 0, every B block, the other A blocks."""
+    out = []
+
+    def a_read(i):
+        q = (2 * ks ^ i) & 3
+        out.append(f"ds_read_b128 {fa(to_set, i)}, %[la{st}{q}] offset:{i * 2048}")
+
+    def b_read(j):
+        if tr:
+            off = (j & 1) * 32 + ks * 32 * PITCH_TR
+            out.append(f"ds_read_b64_tr_b16 {fb_half(to_set, j, 0)}, %[lb{st}{j >> 1}] offset:{off}")
+            out.append(f"ds_read_b64_tr_b16 {fb_half(to_set, j, 1)}, %[lb{st}{j >> 1}] offset:{off + 4 * PITCH_TR}")
+        else:
+            q = (2 * ks ^ j) & 3
+            out.append(f"ds_read_b128 {fb(to_set, j)}, %[lb{st}{q}] offset:{j * 2048}")
+
+    a_read(0)
+    for j in range(8):
+        b_read(j)
+    for i in range(1, 8):
+        a_read(i)
+    return out
+
+
+def loads(tr, st):
+    """The sixteen loads of one K tile into stage st, each as (instructions in front of a matrix instruction,
+    instructions behind it): M0 is written one instruction ahead of the load that uses it."""
+    out = []
+    for p in range(8):
+        out.append(([f"s_add_u32 m0, %[m0w], {st * STAGE + p * 4096}"],
+                    [f"buffer_load_dwordx4 %[ra{p}], s[80:83], %[ka] offen lds"]))
+    for p in range(8):
+        m0 = f"s_add_u32 m0, %[m0w], {st * STAGE + B_TILE + p * 4096}"
+        if tr:
+            pre = [m0] if p == 0 else [m0, "s_add_u32 s88, s88, %[pb]"]
+            if p == 0:
+                pre.append("s_mov_b32 s88, %[kb]")
+            out.append((pre, ["buffer_load_dwordx4 %[rb0], s[84:87], s88 offen lds"]))
+        else:
+            out.append(([m0], [f"buffer_load_dwordx4 %[rb{p}], s[84:87], %[kb] offen lds"]))
+    return out
+
+
+def spread(n_items, n_slots, first=0):
+    """slot -> list of item indices: item r goes behind matrix instruction first + floor(r * n_slots / n_items)"""
+    where = {}
+    for r in range(n_items):
+        where.setdefault(first + (r * n_slots) // n_items, []).append(r)
+    return where
+
+
+def k_tile(tr, st):
+    out = []
+    order = os.environ.get("GEN_ORDER", "a_outer")
+    def mfma(x, s):
+        # x-th instruction of the k-step -> (A block i, B block j)
+        if order == "a_outer":      # A block fixed over eight instructions
+            i, j = x // 8, x % 8
+        elif order == "snake":      # the same, B blocks back and forth
+            i = x // 8
+            j = x % 8 if i % 2 == 0 else 7 - x % 8
+        elif order == "b_outer":
+            j, i = x // 8, x % 8
+        c = i * 8 + j
+        return f"MFMA %[c{c}], {fb(s, j)}, {fa(s, i)}, %[c{c}]"
+    # fetch nothing once no tile is left to fetch: a descriptor of no records
+    out += ["s_cmp_gt_i32 %[left], 0",
+            "s_cselect_b32 s82, 0x7fffffff, 0",
+            "s_cselect_b32 s86, 0x7fffffff, 0",
+            "s_sub_u32 %[left], %[left], 1"]
+    # k-step 0
+    reads = fragment_reads(tr, st, 1, 1)
+    at = spread(len(reads), 40)
+    out.append("s_waitcnt lgkmcnt(0)")
+    for x in range(64):
+        out.append(mfma(x, 0))
+        for r in at.get(x, []):
+            out.append(reads[r])
+    out += ["s_waitcnt lgkmcnt(0)" if "vmwait" in DROP else "s_waitcnt vmcnt(0) lgkmcnt(0)"]
+    if "barrier" not in DROP:
+        out.append("s_barrier")
+    # k-step 1
+    reads = fragment_reads(tr, st ^ 1, 0, 0)
+    at = spread(len(reads), 24, first=1) if not tr else spread(len(reads), 36, first=1)
+    ld = loads(tr, st)
+    every = int(os.environ.get("GEN_LOAD_EVERY", "4"))
+    ld_at = {every * i: i for i in range(16)}   # load i straddles matrix instruction every * i
+    assert max(ld_at) < 64
+    if "dma" in DROP:
+        ld_at = {}
+    for x in range(64):
+        if x in ld_at:
+            out += ld[ld_at[x]][0]
+        out.append(mfma(x, 1))
+        if x in ld_at:
+            out += ld[ld_at[x]][1]
+        for r in at.get(x, []):
+            out.append(reads[r])
+    if "kadvance" not in DROP:
+        out += ["s_add_u32 %[ka], %[ka], 128", "s_add_u32 %[kb], %[kb], %[sb]"]
+    if "reads" in DROP:
+        out = [line for line in out if not line.startswith("ds_read")]
+    return out
+
+
+def loop(tr):
+    out = []
+    # descriptors into fixed scalar registers: word 2 (the record count) is switched inside the loop
+    for w in range(4):
+        out.append(f"s_mov_b32 s{80 + w}, %[da{w}]")
+        out.append(f"s_mov_b32 s{84 + w}, %[db{w}]")
+    out += fragment_reads(tr, 0, 0, 0)
+    out.append("1:")
+    out += ["s_cmp_lt_u32 %[n], 2", "s_cbranch_scc1 2f"]
+    out += k_tile(tr, 0)
+    out += k_tile(tr, 1)
+    out += ["s_sub_u32 %[n], %[n], 2", "s_branch 1b", "2:"]
+    out += ["s_cmp_eq_u32 %[n], 0", "s_cbranch_scc1 3f"]
+    out += k_tile(tr, 0)
+    out.append("3:")
+    # every load has landed (the epilogue lays C out in LDS) and every matrix result is written before the
+    # statement ends: the compiler does not know that these registers come out of the matrix pipe
+    out += ["s_waitcnt vmcnt(0) lgkmcnt(0)", "s_nop 15", "s_nop 15"]
+    return out
+
+
+def as_macro(name, lines):
+    text = f"#define {name}(MFMA) \\\n"
+    body = []
+    for line in lines:
+        if line.startswith("MFMA "):
+            body.append('  MFMA "' + line[4:] + '\\n\\t"')
+        else:
+            body.append('  "' + line + '\\n\\t"')
+    return text + " \\\n".join(body) + "\n"
+
+
+def main():
+    w = sys.stdout.write
+    w("// Generated by gen_tile_loop.py (python3 gen_tile_loop.py > tile_loop_asm.inc): the K loop of the 256x256 tile\n")
+    w("// on the 16x16 matrix instructions.  VECOPS_LOOP256_K: both operands K-contiguous in LDS; VECOPS_LOOP256_TR: B as\n")
+    w("// it lies in memory ([k][n]) and transposed by the LDS reads.  MFMA: the instruction's mnemonic, a string.\n")
+    w(as_macro("VECOPS_LOOP256_K", loop(False)))
+    w("\n")
+    w(as_macro("VECOPS_LOOP256_TR", loop(True)))
+    w("\n// the accumulators as operands: quad x = t[x / 8][x % 8]\n")
+    w("#define VECOPS_LOOP256_ACCUMULATORS(t) \\\n  " +
+      ", \\\n  ".join(", ".join(f'[c{x}] "+a"(t[{x // 8}][{x % 8}])' for x in range(r, r + 4)) for r in range(0, 64, 4)) + "\n")
+    w("\n// registers the loop uses by number\n")
+    w("#define VECOPS_LOOP256_CLOBBERS \\\n  " + ", ".join(f'"s{r}"' for r in range(80, 89)) + ", \\\n  " +
+      ", \\\n  ".join(", ".join(f'"v{r}"' for r in range(b, b + 16)) for b in range(128, 256, 16)) + "\n")
+
+
+if __name__ == "__main__":
+    main()

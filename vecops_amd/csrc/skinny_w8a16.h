@@ -448,20 +448,29 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_mfma_kernel(const Ski
 // Same arithmetic and operand layout as skinny_w8a16_mfma_kernel, for K = 8 wavefronts
 // x 8 steps x 64 (4096).  In that kernel every step carries, besides its weight loads,
 // two activation loads and its share of the scale loads - four of five memory
-// instructions fetch data that is not weights.  Here a wavefront loads the activation
-// fragments of its K slice once (64 registers) and keeps them while the workgroup walks
-// `passes` consecutive blocks of TILES x 16 weight rows; the scales of a block arrive as
-// one coalesced 4-byte load per lane (lane = row + 16 * group) and are handed to the
-// lanes that need them with lane permutes.  The steps of all passes form one flat
-// sequence with loads D = 4 steps ahead; the K slices are summed through LDS once per
-// pass (double-buffered, one barrier per pass).
-template <int SPG, int TILES>
-__global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const SkinnyW8A16Params p, int passes) {
+// instructions fetch data that is not weights.  Here a wavefront fetches the activation
+// rows of its K slice once - one load instruction per row, 1 KiB contiguous, written
+// straight into LDS, from where they come back as matrix-core fragments (64 registers;
+// fetching the fragments themselves, 64 bytes of each of 16 rows per instruction, cost
+// 3 us of 18 at M = 16: twice the cache lines per byte, in a memory pipeline that the
+// weights keep full) - and keeps them while the workgroup walks PASSES consecutive blocks
+// of TILES x 16 weight rows; the scales of a block arrive as one coalesced 4-byte load per
+// lane (lane = row + 16 * group) and are handed to the lanes that need them with lane
+// permutes.  The steps of all passes form one flat sequence with loads D = 4 steps ahead.
+// The K slices of every pass wait in LDS (in the wavefront's own activation rows, which are
+// dead by then) and are summed behind ONE barrier at the end: with a barrier per pass every
+// wavefront waited for the slowest of its workgroup, 1.7 us per pass measured inside the
+// kernel, with no new loads going out meanwhile.
+template <int SPG, int TILES, int PASSES>
+__global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const SkinnyW8A16Params p) {
   constexpr int WAVES = 8, S = 8, D = 4;  // a deeper pipeline (D = 8) measured no faster
   constexpr int GPW = S / SPG;                      // scale groups of a wavefront's K slice
   constexpr int NSC = (16 * GPW + 63) / 64;         // scale registers per tile
   static_assert(S % SPG == 0 && D % SPG == 0, "whole groups per pipeline round");
-  __shared__ float red[2][WAVES][TILES][16 * 16];
+  constexpr int XPITCH = 1024 + 16;   // bytes between the activation rows of a wavefront's K slice in LDS
+  __shared__ __attribute__((aligned(16))) char xlds[WAVES][16 * XPITCH];
+  static_assert(PASSES * TILES * 1024 <= 16 * XPITCH, "a wavefront's partial sums reuse its own staging rows");
+  constexpr int passes = PASSES;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int row = lane & 15, quarter = lane >> 4;
@@ -478,20 +487,6 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
 
   // activation fragments of this K slice, resident for the whole kernel
   u32x4 x1[S], x2[S];
-  auto load_activations = [&]() {
-    const VECOPS_GLOBAL char* xrow = (const VECOPS_GLOBAL char*)(p.x + static_cast<int64_t>(min(row, p.m - 1)) * p.ldx) +
-                                     quarter * 32 + static_cast<int64_t>(wave) * S * 128;
-#pragma unroll
-    for (int s = 0; s < S; ++s) {
-      x1[s] = u32x4{0u, 0u, 0u, 0u};
-      x2[s] = u32x4{0u, 0u, 0u, 0u};
-      if (row < p.m) {
-        const VECOPS_GLOBAL u32x4* px = (const VECOPS_GLOBAL u32x4*)(xrow + s * 128);
-        x1[s] = px[0];
-        x2[s] = px[1];
-      }
-    }
-  };
 
   const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};  // eight bf16 1.0
   u32x4 wq[D][TILES];
@@ -566,9 +561,36 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
   };
 
   // the first weights are requested before the activations: they arrive while those are fetched
-  static_for<D>([&](auto u) { issue(u, decltype(u)::value); });
-  load_scales(sc_cur, 0);
-  load_activations();
+  // start-up: the wavefront's K slice of every activation row goes into LDS by loads that write LDS themselves - one
+  // instruction per row, 1 KiB contiguous - and comes back as matrix-core fragments (lane = row + 16 * quarter)
+  {
+    const __amdgpu_buffer_rsrc_t xbuf = tile_buffer((const VECOPS_GLOBAL char*)p.x);
+    char* mine = xlds[wave];
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      if (r < p.m)
+        load_16_bytes_into_lds_counted(xbuf, (lds_void_ptr)(mine + r * XPITCH), static_cast<uint32_t>(lane * 16),
+                                       __builtin_amdgcn_readfirstlane(static_cast<uint32_t>((r * p.ldx + wave * S * 64) * 2)));
+  }
+  asm volatile("" ::: "memory");  // (the weight loads stay behind the loads above)
+  static_for<D>([&](auto u) {
+    issue(u, decltype(u)::value);
+    if constexpr (decltype(u)::value == 0) load_scales(sc_cur, 0);
+  });
+  {
+    // The loads that write LDS are counted with the loads issued behind them, in order: at least D * TILES weight
+    // loads follow, so "at most D * TILES - TILES still in flight" means the activations (and the first step's
+    // weights) have landed.  Through a statement the compiler moves no memory access across.
+    static_assert(D * TILES - TILES == 6, "the wait below is written for six");
+    asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    const char* mine = xlds[wave] + row * XPITCH + quarter * 32;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      const u32x4 a = *reinterpret_cast<const u32x4*>(mine + s * 128), b = *reinterpret_cast<const u32x4*>(mine + s * 128 + 16);
+      x1[s] = row < p.m ? a : u32x4{0u, 0u, 0u, 0u};
+      x2[s] = row < p.m ? b : u32x4{0u, 0u, 0u, 0u};
+    }
+  }
   for (int pass = 0; pass < passes; ++pass) {
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
@@ -583,30 +605,33 @@ __global__ __launch_bounds__(512) void skinny_w8a16_mfma_resident_kernel(const S
     });
     // Sum the K slices through LDS.  Accumulator register r of lane l is output
     // (weight row quarter*4 + r, activation row l % 16) of its 16x16 tile.
-    float (*mine)[TILES][16 * 16] = red[pass & 1];
+    float (*mine)[16 * 16] = reinterpret_cast<float (*)[16 * 16]>(xlds[wave]) + pass * TILES;
 #pragma unroll
     for (int t = 0; t < TILES; ++t)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) mine[wave][t][(quarter * 4 + r) * 16 + row] = acc[t][r];
-    __syncthreads();
-    if (wave < TILES) {  // wavefront t finishes tile t
-      const int t = wave;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float total_sum = 0.0f;
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w) total_sum += mine[w][t][(quarter * 4 + r) * 16 + row];
-        const int64_t n = wg_row0 + (pass * TILES + t) * 16 + quarter * 4 + r;
-        if (row < p.m && n < p.n)
-          p.y[static_cast<int64_t>(row) * p.ldy + n] = static_cast<uint16_t>(bf16_bits_rne(total_sum));
-      }
-    }
+      for (int r = 0; r < 4; ++r) mine[t][(quarter * 4 + r) * 16 + row] = acc[t][r];
 #pragma unroll
     for (int t = 0; t < TILES; ++t)
 #pragma unroll
       for (int i = 0; i < NSC; ++i) sc_cur[t][i] = sc_nxt[t][i];
   }
+  // One barrier for the whole kernel: the K slices of every pass wait in LDS and are summed at the end (a barrier per
+  // pass held every wavefront until the slowest had finished the pass, with no new loads going out meanwhile).
+  __syncthreads();
+  for (int job = wave; job < passes * TILES; job += WAVES) {
+    const int pass = job / TILES, t = job - pass * TILES;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float total_sum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) total_sum += (reinterpret_cast<const float (*)[16 * 16]>(xlds[w]) + pass * TILES)[t][(quarter * 4 + r) * 16 + row];
+      const int64_t n = wg_row0 + (pass * TILES + t) * 16 + quarter * 4 + r;
+      if (row < p.m && n < p.n)
+        p.y[static_cast<int64_t>(row) * p.ldy + n] = static_cast<uint16_t>(bf16_bits_rne(total_sum));
+    }
+  }
 }
+
 
 }  // namespace vecops_hip
 #endif

@@ -471,10 +471,21 @@ struct Accumulators {
 #pragma unroll
         for (int r = 0; r < (M16 ? 4 : 16); ++r) t[i][j][r] = 0;
   }
+  // The 64 quads of the 256x256 tile's 16x16 form come out of its written-out K loop in the accumulation registers
+  // and stay there until the epilogue takes them one by one: left to itself the compiler copies all 256 values into
+  // vector registers ahead of the branch between the epilogue's paths, spills what does not fit, and reloaded one
+  // spilled value wrongly (ROCm 7.2).  The empty statement pins a quad to its accumulation registers at its use.
+  static constexpr bool kPinned = M16 && WM * WN > 4;
   template <int I, int J, int Q>
   __device__ __forceinline__ Quad quad() const {
-    if constexpr (M16) return t[2 * I + (Q >> 1)][2 * J + (Q & 1)];
-    else return __builtin_shufflevector(t[I][J], t[I][J], 4 * Q, 4 * Q + 1, 4 * Q + 2, 4 * Q + 3);
+    if constexpr (M16) {
+#if defined(__HIP_DEVICE_COMPILE__)
+      if constexpr (kPinned) asm volatile("" : "+a"(const_cast<Frag&>(t[2 * I + (Q >> 1)][2 * J + (Q & 1)])));
+#endif
+      return t[2 * I + (Q >> 1)][2 * J + (Q & 1)];
+    } else {
+      return __builtin_shufflevector(t[I][J], t[I][J], 4 * Q, 4 * Q + 1, 4 * Q + 2, 4 * Q + 3);
+    }
   }
   static __device__ __forceinline__ int row(int lane, int q) { return M16 ? (q >> 1) * 16 + (lane & 15) : (lane & 31); }
   static __device__ __forceinline__ int col(int lane, int q) {
@@ -1691,6 +1702,65 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
   }
 }
 
+// The K loop of the 256x256 tile on the 16x16 matrix instructions, as one written-out instruction stream
+// (tile_loop_asm.inc, generated by gen_tile_loop.py, which describes the schedule).  On entry tile 0 lies in LDS
+// stage 0 and tile 1 (if any) in stage 1, and a barrier has been passed.  Operands:
+//   acc               the 64 accumulator quads (accumulation registers)
+//   lds_a, lds_b      per-lane LDS addresses of the fragment reads, [stage][q] (see tile_gemm_workgroup)
+//   rows_a, rows_b    per-lane byte offsets of the eight loads of a K tile of A and of B (TR: B's one offset)
+//   desc_a, desc_b    buffer descriptors of the operands' tiles (K tile 0)
+//   m0_wave           LDS address of the wavefront's 1 KiB slice of a load's 4 KiB (stage 0, A tile)
+//   k_a, k_b          byte offset of the first K tile the loop fetches (tile 2 of the walk), step_b B's per K tile
+//                     (A's is 128), part_b (TR) the offset between B's eight loads of a K tile
+//   nk                K tiles to multiply
+#include "tile_loop_asm.inc"
+template <int SRC, bool TR, typename ACC>
+__device__ __forceinline__ void asm_k_loop(ACC& acc, const uint32_t (&lds_a)[2][4], const uint32_t (&lds_b)[2][4],
+                                           const uint32_t (&rows_a)[8], const uint32_t (&rows_b)[8], const u32x4& desc_a,
+                                           const u32x4& desc_b, uint32_t m0_wave, uint32_t k_a, uint32_t k_b, uint32_t step_b,
+                                           uint32_t part_b, int nk) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  // (wavefront-uniform by construction; said again here, so that each lives in a scalar register)
+  auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
+  int left = uniform(nk) - 2, n = uniform(nk);
+  k_a = uniform(k_a);
+  k_b = uniform(k_b);
+  const uint32_t da[4] = {uniform(desc_a[0]), uniform(desc_a[1]), uniform(desc_a[2]), uniform(desc_a[3])};
+  const uint32_t db[4] = {uniform(desc_b[0]), uniform(desc_b[1]), uniform(desc_b[2]), uniform(desc_b[3])};
+  m0_wave = uniform(m0_wave);
+  step_b = uniform(step_b);
+  part_b = uniform(part_b);
+#define VECOPS_LOOP256_STATEMENT(TEXT)                                                                                  \
+  asm volatile(TEXT                                                                                                     \
+               : VECOPS_LOOP256_ACCUMULATORS(acc.t), [ka] "+s"(k_a), [kb] "+s"(k_b), [left] "+s"(left), [n] "+s"(n)       \
+               : [la00] "v"(lds_a[0][0]), [la01] "v"(lds_a[0][1]), [la02] "v"(lds_a[0][2]), [la03] "v"(lds_a[0][3]),    \
+                 [la10] "v"(lds_a[1][0]), [la11] "v"(lds_a[1][1]), [la12] "v"(lds_a[1][2]), [la13] "v"(lds_a[1][3]),    \
+                 [lb00] "v"(lds_b[0][0]), [lb01] "v"(lds_b[0][1]), [lb02] "v"(lds_b[0][2]), [lb03] "v"(lds_b[0][3]),    \
+                 [lb10] "v"(lds_b[1][0]), [lb11] "v"(lds_b[1][1]), [lb12] "v"(lds_b[1][2]), [lb13] "v"(lds_b[1][3]),    \
+                 [ra0] "v"(rows_a[0]), [ra1] "v"(rows_a[1]), [ra2] "v"(rows_a[2]), [ra3] "v"(rows_a[3]),                \
+                 [ra4] "v"(rows_a[4]), [ra5] "v"(rows_a[5]), [ra6] "v"(rows_a[6]), [ra7] "v"(rows_a[7]),                \
+                 [rb0] "v"(rows_b[0]), [rb1] "v"(rows_b[1]), [rb2] "v"(rows_b[2]), [rb3] "v"(rows_b[3]),                \
+                 [rb4] "v"(rows_b[4]), [rb5] "v"(rows_b[5]), [rb6] "v"(rows_b[6]), [rb7] "v"(rows_b[7]),                \
+                 [da0] "s"(da[0]), [da1] "s"(da[1]), [da2] "s"(da[2]), [da3] "s"(da[3]),                                \
+                 [db0] "s"(db[0]), [db1] "s"(db[1]), [db2] "s"(db[2]), [db3] "s"(db[3]),                                \
+                 [m0w] "s"(m0_wave), [sb] "s"(step_b), [pb] "s"(part_b)                                                 \
+               : "memory", "m0", "scc", VECOPS_LOOP256_CLOBBERS)
+  if constexpr (TR) {
+    static_assert(SRC == SRC_BF16 || SRC == SRC_F16, "transposing LDS reads move 16-bit elements");
+    if constexpr (SRC == SRC_F16) VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_TR("v_mfma_f32_16x16x32_f16"));
+    else VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_TR("v_mfma_f32_16x16x32_bf16"));
+  } else {
+    if constexpr (SRC == SRC_F16) VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_K("v_mfma_f32_16x16x32_f16"));
+    else if constexpr (SrcTraits<SRC>::kInt) VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_K("v_mfma_i32_16x16x64_i8"));
+    else VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_K("v_mfma_f32_16x16x32_bf16"));
+  }
+#undef VECOPS_LOOP256_STATEMENT
+#else
+  (void)acc; (void)lds_a; (void)lds_b; (void)rows_a; (void)rows_b; (void)desc_a; (void)desc_b; (void)m0_wave;
+  (void)k_a; (void)k_b; (void)step_b; (void)part_b; (void)nk;
+#endif
+}
+
 // Bytes between the k rows of a B tile kept untransposed in LDS (0 for the other layouts).
 template <int SRC, int LOAD_B, int ROWS, int THREADS>
 constexpr int ntr_pitch() {
@@ -1719,6 +1789,11 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
   // wavefront's tile two fragments
   static_assert(!M16 || SRC != SRC_F32, "the fp32 MFMA has one shape here");
   constexpr int FM = M16 ? 2 * WM : WM, FN = M16 ? 2 * WN : WN;
+  // The 256x256 tile on the 16x16 shapes runs its K loop as a written-out instruction stream (asm_k_loop): its 64
+  // accumulator quads fill the accumulation registers, where the compiler's own loop copies them about.
+  constexpr bool ASM_LOOP = M16 && WM == 4 && WN == 4;
+  static_assert(!M16 || WM * WN <= 4 || (ASM_LOOP && load_is_dma(LOAD_A) && load_is_dma(LOAD_B) && WAVES_M == 2 && WAVES_N == 2),
+                "the 16x16 shapes: small tiles, or the 256x256 tile fed by loads that write LDS");
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -1962,6 +2037,21 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
     // carry loads "still in flight" into the loop and wait for them in every iteration.
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
     lds_barrier();  // tile 0 is in LDS (and tile 1, where the loop loads two tiles ahead)
+    if constexpr (ASM_LOOP) {
+      // the loop fetches tile 2 of the walk first (positions 1, 2, ... of the walk are consecutive K tiles)
+      const uint32_t kt2 = static_cast<uint32_t>(kt_begin - has_tail + 2);
+      const uint32_t m0_wave = lds_address_of(lds) + static_cast<uint32_t>(wave) * 1024u;
+      if constexpr (load_is_ntr(LOAD_B)) {
+        const uint32_t step_b = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(64 * stager_b.ks * T::kSrcBytes));
+        const uint32_t rows_b[8] = {stager_b.chunk_bytes, 0, 0, 0, 0, 0, 0, 0};
+        asm_k_loop<SRC, true>(acc, base_a, base_b, stager_a.row_bytes, rows_b, stager_a.tile_buf,
+                              tile_buffer_words(stager_b.tile_base), m0_wave, kt2 * 128u, kt2 * step_b, step_b,
+                              stager_b.part_offset(1), nk);
+      } else {
+        asm_k_loop<SRC, false>(acc, base_a, base_b, stager_a.row_bytes, stager_b.row_bytes, stager_a.tile_buf,
+                               stager_b.tile_buf, m0_wave, kt2 * 128u, kt2 * 128u, 128u, 0u, nk);
+      }
+    } else {
     read_frags(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
 
     // The loop body is one straight-line block: stores into the other stage,
@@ -2087,6 +2177,7 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
     };
     if (full_in_range > 0) main_loop(std::true_type{});
     else main_loop(std::false_type{});
+    }
     // (the last trips' surplus loads into LDS must have landed before the epilogue lays C out there)
     if constexpr (DMA && M16) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   }
@@ -2096,7 +2187,7 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
 }
 
 template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B, bool M16 = kShortMfma<SRC, WM, WN>>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (M16 ? 2 : 1)) void tile_gemm_kernel(const TileGemmParams p) {
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (M16 && WM * WN <= 4 ? 2 : 1)) void tile_gemm_kernel(const TileGemmParams p) {
   tile_gemm_workgroup<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_A, LOAD_B, M16>(p, blockIdx.x, gridDim.x);
 }
 
@@ -2104,14 +2195,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (M16 ? 2 : 1)) void tile_ge
 // pointers; all share the operand class, the workgroup tile and the loaders).  Workgroups first[g] .. first[g + 1] - 1
 // serve group g (each run a multiple of eight long, so that a group's workgroups are dealt to the XCDs like a
 // launch of its own); group_of[w] names the group of workgroup w.  No group splits K.
-template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (kShortMfma<SRC, WM, WN> ? 2 : 1)) void tile_gemm_grouped_kernel(
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_A, int LOAD_B, bool M16 = kShortMfma<SRC, WM, WN>>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (M16 && WM * WN <= 4 ? 2 : 1)) void tile_gemm_grouped_kernel(
     const int32_t* __restrict__ group_of, const int32_t* __restrict__ first, const TileGemmParams* __restrict__ groups) {
   const int g = __builtin_amdgcn_readfirstlane(group_of[blockIdx.x]);
   const TileGemmParams p = groups[g];
   const int begin = __builtin_amdgcn_readfirstlane(first[g]);
   const int end = __builtin_amdgcn_readfirstlane(first[g + 1]);
-  tile_gemm_workgroup<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_A, LOAD_B>(p, static_cast<int>(blockIdx.x) - begin, end - begin);
+  tile_gemm_workgroup<SRC, WAVES_M, WAVES_N, WM, WN, LOAD_A, LOAD_B, M16>(p, static_cast<int>(blockIdx.x) - begin, end - begin);
 }
 
 // Table set-up of a grouped launch is fed through kernel arguments, so that no host buffer has to outlive the

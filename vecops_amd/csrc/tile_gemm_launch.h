@@ -121,7 +121,18 @@ hipError_t launch_tile_class(const TileGemmParams& p, int tile_m, int tile_n, in
   // Every shape runs 4 wavefronts (2 x 2), one per SIMD.  256x256: 128x128 per wavefront - a third less LDS
   // read traffic than 8 wavefronts of 128x64, which matters because the LDS pipe, not the MFMA pipe, is
   // what the 8-wavefront shape saturates.
-  if (tile_m == 256 && tile_n == 256) return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
+  if (tile_m == 256 && tile_n == 256) {
+    // operands whose loads write LDS themselves: the 16x16 shapes under the written-out K loop (asm_k_loop), whose
+    // scalar K offsets are 32-bit
+    if constexpr (SRC == SRC_BF16 || SRC == SRC_F16 || SRC == SRC_I8) {
+      if (mode == MODE_KVEC_DMA) return launch_tile_instance<SRC, 2, 2, 4, 4, LOAD_KDMA, LOAD_KDMA, true>(p, stream);
+      if constexpr (SRC != SRC_I8) {
+        if (mode == MODE_NVEC_B_DMA && static_cast<int64_t>(p.k) * p.b_ks * 2 < (1ll << 31))
+          return launch_tile_instance<SRC, 2, 2, 4, 4, LOAD_KDMA, LOAD_NTR_DMA, true>(p, stream);
+      }
+    }
+    return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
+  }
   if (tile_m == 256 && tile_n == 128) return launch_tile_mode<SRC, 2, 2, 4, 2>(p, mode, stream);
   if (tile_m == 128 && tile_n == 256) return launch_tile_mode<SRC, 2, 2, 2, 4>(p, mode, stream);
   if (tile_m == 128 && tile_n == 128) {
@@ -141,11 +152,11 @@ struct GroupedTables {
   int32_t workgroups;
 };
 
-template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB>
+template <int SRC, int WAVES_M, int WAVES_N, int WM, int WN, int LA, int LB, bool M16 = kShortMfma<SRC, WM, WN>>
 hipError_t launch_grouped_instance(const GroupedTables& t, hipStream_t stream) {
   constexpr int kLds = kTileLdsBytes<WAVES_M, WAVES_N, WM, WN, LB>();
   constexpr int kThreads = 64 * WAVES_M * WAVES_N;
-  auto kernel = tile_gemm_grouped_kernel<SRC, WAVES_M, WAVES_N, WM, WN, LA, LB>;
+  auto kernel = tile_gemm_grouped_kernel<SRC, WAVES_M, WAVES_N, WM, WN, LA, LB, M16>;
   static thread_local int configured_device = -1;
   int device = 0;
   hipError_t e = hipGetDevice(&device);
@@ -170,7 +181,17 @@ hipError_t launch_grouped_class(const GroupedTables& t, int tile, int mode, hipS
       return launch_grouped_instance<SRC, 2, 2, W, W, decltype(la)::value, decltype(lb)::value>(t, stream);
     });
   };
-  if (tile == 256) return go(std::integral_constant<int, 4>{});
+  if (tile == 256) {
+    // as a single product's 256 x 256 tiles: the written-out K loop where the loads write LDS themselves (the table's
+    // mode is that of its weakest group, and none of them then needs more than 32-bit K offsets)
+    if constexpr (SRC == SRC_BF16 || SRC == SRC_F16 || SRC == SRC_I8) {
+      if (mode == MODE_KVEC_DMA) return launch_grouped_instance<SRC, 2, 2, 4, 4, LOAD_KDMA, LOAD_KDMA, true>(t, stream);
+      if constexpr (SRC != SRC_I8) {
+        if (mode == MODE_NVEC_B_DMA) return launch_grouped_instance<SRC, 2, 2, 4, 4, LOAD_KDMA, LOAD_NTR_DMA, true>(t, stream);
+      }
+    }
+    return go(std::integral_constant<int, 4>{});
+  }
   if (tile == 128) return go(std::integral_constant<int, 2>{});
   return go(std::integral_constant<int, 1>{});
 }
