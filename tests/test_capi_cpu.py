@@ -53,8 +53,23 @@ def test_rule_table_known_answers():
     # config 4
     rc, p = _plan(_operand(capi.I8, (2048, 4096)), _operand(capi.I8, (11008, 4096)),
                   _operand(capi.I32, (2048, 11008)))
-    # 344 tiles of 256x256 would take two rounds, the second a third full; 1376 of 128x128 take six short ones
-    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1
+    # 344 tiles of 256x256 would take two rounds, the second a third full; 1376 of 128x128 two and two thirds at two
+    # workgroups per unit; 256 tiles of 256x352 are exactly one round
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256x352" and p.split_k == 1 and p.workspace_bytes == 0
+    # the same extents where that tile cannot serve: bf16 operands, an M that is no multiple of 256, rows of A that are
+    # not 16-byte aligned, a K that is no multiple of 128 - the 128x128 tile as before
+    rc, p = _plan(_operand(capi.BF16, (2048, 4096)), _operand(capi.BF16, (11008, 4096)), _operand(capi.BF16, (2048, 11008)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
+    rc, p = _plan(_operand(capi.I8, (2040, 4096)), _operand(capi.I8, (11008, 4096)), _operand(capi.I32, (2040, 11008)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
+    rc, p = _plan(_operand(capi.I8, (2048, 4096), strides=(4104, 1)), _operand(capi.I8, (11008, 4096)),
+                  _operand(capi.I32, (2048, 11008)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
+    rc, p = _plan(_operand(capi.I8, (2048, 4160)), _operand(capi.I8, (11008, 4160)), _operand(capi.I32, (2048, 11008)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
+    # int8 4096^3 keeps the square tile (192 of the wide ones would leave a quarter of the units idle)
+    rc, p = _plan(_operand(capi.I8, (4096, 4096)), _operand(capi.I8, (4096, 4096)), _operand(capi.I32, (4096, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
     # 8 x 777 x 1000: seven rows of 128x256 tiles pad M to 896, four rows of 256-row tiles would pad it to 1024
     rc, p = _plan(_operand(capi.BF16, (8, 777, 3001)), _operand(capi.BF16, (8, 1000, 3001)),
                   _operand(capi.F32, (8, 777, 1000)))

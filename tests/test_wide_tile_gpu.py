@@ -1,0 +1,102 @@
+"""The 256 x 352 workgroup tile of signed 8-bit operands (family tile_256x352), through the C ABI: int32 sums bit-exact
+against exact integer arithmetic on shapes with one, two, three and more K tiles, ragged N (clamped rows, guarded
+stores), several tile rows and columns; the dequantising epilogue bit-exact against the oracle (the same two
+separately rounded multiplies, vecops matmul/Quantization.h:195-250) on a shape the rule table itself gives to this
+tile; and the family request's error behaviour (a required family that cannot serve the operands is NotApplicable,
+tests/ops/MatmulTest.cpp:514-536)."""
+import numpy as np
+import pytest
+
+from vecops_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 352, 256), (256, 352, 384), (256, 352, 640), (256, 704, 512), (512, 1000, 512),
+                                   (256, 180, 256), (768, 3000, 1024), (256, 356, 2048)])
+def test_wide_tile_int32_sums_are_exact(device, m, n, k):
+    import torch
+    from vecops_amd import capi
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    request = capi.family_request("tile_256x352", capi.SELECT_REQUIRE)
+    c_store = torch.full((m, n + 12), -7, dtype=torch.int32, device=device)   # rows of C with a pad that must stay
+    c = c_store[:, :n]
+    assert capi.FAMILY_NAMES[capi.plan_matmul_family(ta, tb, c, request).family] == "tile_256x352"
+    capi.matmul_family(ta, tb, c, request)
+    torch.cuda.synchronize()
+    want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.int32)
+    assert np.array_equal(c.cpu().numpy(), want)
+    assert bool((c_store[:, n:] == -7).all())
+
+
+def test_wide_tile_extreme_operands_wrap_like_int32(device):
+    """All operands -128: every product 16384, K = 32768 of them = 2^29 per sum... and K = 131072 wraps mod 2^32."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = 256, 352, 131072
+    ta = torch.full((m, k), -128, dtype=torch.int8, device=device)
+    tb = torch.full((n, k), -128, dtype=torch.int8, device=device)
+    c = torch.zeros((m, n), dtype=torch.int32, device=device)
+    capi.matmul_family(ta, tb, c, capi.family_request("tile_256x352", capi.SELECT_REQUIRE))
+    torch.cuda.synchronize()
+    want = np.int64(16384) * k % (1 << 32)
+    assert bool((c.view(torch.int32).cpu().numpy().astype(np.int64) % (1 << 32) == want).all())
+
+
+def test_wide_tile_is_the_tables_choice_and_dequantises_bit_exactly(device, oracle):
+    """2048 x 11008 (the benchmark's extents) with a shorter K: 256 tiles of 256 x 352 = one round, which the rule table
+    takes; per-token x per-channel dequantisation with a correction row, every output against the oracle."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = 2048, 11008, 1152
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    rs, cs = synth.scales(3, m), synth.scales(4, n)
+    correction = ((synth.draws(5, n) % np.uint64(2001)).astype(np.int64) - 1000).astype(np.int32)
+    ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    plan = capi.plan_matmul(ta, tb, torch.empty((m, n), dtype=torch.int32, device=device))
+    assert capi.FAMILY_NAMES[plan.family] == "tile_256x352" and plan.split_k == 1 and plan.workspace_bytes == 0
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul_i8_dequant(ta, tb, torch.from_numpy(rs).to(device), torch.from_numpy(cs).to(device), c,
+                           correction=torch.from_numpy(correction).to(device))
+    torch.cuda.synchronize()
+    want = oracle.matmul_i8_dequant(a, b, rs, cs, correction)
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    # scales and correction at addresses that are not 16-byte aligned: the element-wise loads of the epilogue
+    rs1, cs1, corr1 = (torch.zeros(x.size + 1, dtype=torch.from_numpy(x).dtype, device=device) for x in (rs, cs, correction))
+    rs1[1:], cs1[1:], corr1[1:] = torch.from_numpy(rs).to(device), torch.from_numpy(cs).to(device), torch.from_numpy(correction).to(device)
+    c.fill_(float("nan"))
+    capi.matmul_i8_dequant(ta, tb, rs1[1:], cs1[1:], c, correction=corr1[1:])
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_wide_tile_required_where_it_cannot_serve(device):
+    import torch
+    from vecops_amd import capi
+    request = capi.family_request("tile_256x352", capi.SELECT_REQUIRE)
+    prefer = capi.family_request("tile_256x352", capi.SELECT_PREFER)
+
+    def i8(shape):
+        return torch.zeros(shape, dtype=torch.int8, device=device)
+    cases = {
+        "M not a multiple of 256": (i8((300, 512)), i8((352, 512)), torch.int32),
+        "K not a multiple of 128": (i8((256, 520)), i8((352, 520)), torch.int32),
+        "a single K tile": (i8((256, 128)), i8((352, 128)), torch.int32),
+        "bf16 operands": (torch.zeros((256, 512), dtype=torch.bfloat16, device=device),
+                          torch.zeros((352, 512), dtype=torch.bfloat16, device=device), torch.float32),
+        "unsigned a": (torch.zeros((256, 512), dtype=torch.uint8, device=device), i8((352, 512)), torch.int32),
+    }
+    for name, (a, b, out) in cases.items():
+        c = torch.zeros((a.shape[0], b.shape[0]), dtype=out, device=device)
+        with pytest.raises(capi.VecopsHipError) as err:
+            capi.matmul_family(a, b, c, request)
+        assert err.value.code == 2, name                       # NotApplicable
+        capi.matmul_family(a, b, c, prefer)                    # a preference falls back to the rule table's choice
+        assert capi.FAMILY_NAMES[capi.plan_matmul_family(a, b, c, prefer).family] != "tile_256x352", name
+    # a fixed K split is not this family's either
+    a, b = i8((256, 512)), i8((352, 512))
+    c = torch.zeros((256, 352), dtype=torch.int32, device=device)
+    with pytest.raises(capi.VecopsHipError):
+        capi.matmul_family(a, b, c, capi.family_request("tile_256x352", capi.SELECT_REQUIRE, split_k=2))
+    torch.cuda.synchronize()

@@ -260,6 +260,7 @@ void tile_of_family(uint32_t family, int* tile_m, int* tile_n) {
     case VECOPS_HIP_FAMILY_TILE_256: *tile_m = *tile_n = 256; break;
     case VECOPS_HIP_FAMILY_TILE_256X128: *tile_m = 256; *tile_n = 128; break;
     case VECOPS_HIP_FAMILY_TILE_128X256: *tile_m = 128; *tile_n = 256; break;
+    case VECOPS_HIP_FAMILY_TILE_256X352: *tile_m = 256; *tile_n = 352; break;
     case VECOPS_HIP_FAMILY_TILE_128: *tile_m = *tile_n = 128; break;
     case VECOPS_HIP_FAMILY_TILE_64: *tile_m = *tile_n = 64; break;
     default: *tile_m = *tile_n = 0; break;
@@ -275,6 +276,7 @@ void finish_tile_plan(const Problem& pr, VecopsHipPlan* plan, uint32_t forced_sp
   const int64_t k_tiles = (pr.k + ktile - 1) / ktile;
   const int64_t wgs = ((pr.m + tile_m - 1) / tile_m) * ((pr.n + tile_n - 1) / tile_n) * pr.batch;
   int64_t split = 1;
+  if (plan->family == VECOPS_HIP_FAMILY_TILE_256X352) forced_split = 1;  // its kernel walks the whole K
   if (forced_split > 0) {
     split = forced_split < k_tiles ? forced_split : k_tiles;
   } else if (wgs <= kComputeUnits / 2 && k_tiles >= 8) {
@@ -319,6 +321,19 @@ void cut_columns(const Problem& pr, int64_t n_main, Problem* main, Problem* rest
     rest->cin.cols = pr.n - n_main;
     rest->cin.data = static_cast<char*>(pr.cin.data) + n_main * pr.cin.cs * dtype_bytes(pr.cin.dtype);
   }
+}
+
+// Whether the 256 x 352 tile (tile_gemm_wide_i8.hip) can run a problem: signed 8-bit operands, both K-contiguous with
+// 16-byte aligned bases and rows, K a multiple of 128 (two K tiles or more), M of 256, N of 4, one batch, no C input, no
+// fused transform, a row-major C with 16-byte aligned rows (int32 sums, or fp32 when dequantising).
+bool wide_tile_serves(const Problem& pr) {
+  if (pr.src != SRC_I8 || pr.packed_b || pr.has_cin || pr.fused != nullptr || pr.batch != 1) return false;
+  if (pr.k % 128 != 0 || pr.k < 256 || pr.m % 256 != 0 || pr.n % 4 != 0 || pr.m == 0 || pr.n == 0) return false;
+  if (pr.a.cs != 1 || pr.b.cs != 1 || pr.a.rs % 16 != 0 || pr.b.rs % 16 != 0 || !aligned16(pr.a.data) || !aligned16(pr.b.data)) return false;
+  if (pr.c.cs != 1 || pr.c.rs % 4 != 0 || !aligned16(pr.c.data)) return false;
+  if (256 * pr.a.rs >= (int64_t{1} << 31) || 352 * pr.b.rs >= (int64_t{1} << 31)) return false;
+  // (a dequantised product is described with its accumulator class, int32, and leaves as fp32)
+  return pr.out_kind == OUT_I32 || (pr.dequant && pr.out_kind == OUT_F32);
 }
 
 // The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure
@@ -406,6 +421,22 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
       tile_n = c.tn;
     }
   }
+  // The 256 x 352 tile of 8-bit operands: priced like the big tile (its loop is the same, with a tenth less operand
+  // traffic per multiply-add), it wins where its count fits rounds that the square tiles' counts do not - 2048 x 11008:
+  // 256 tiles in one round against 344 of 256 x 256 (two rounds) and 1376 of 128 x 128 (three).
+  if (wide_tile_serves(pr) && pr.n > 176) {
+    const int64_t count = tiles2(256, 352), rounds = (count + kComputeUnits - 1) / kComputeUnits;
+    if (count >= kComputeUnits / 2) {
+      int64_t cost = rounds * 256 * 352;
+      if (rounds == 1) cost = cost * (kComputeUnits + count) / (2 * kComputeUnits);
+      if (cost < best_cost) {
+        best_cost = cost;
+        family = VECOPS_HIP_FAMILY_TILE_256X352;
+        tile_m = 256;
+        tile_n = 352;
+      }
+    }
+  }
   if (family == VECOPS_HIP_FAMILY_TILE_64 && pr.m > 64 && pr.n > 64 && tiles(64) > 4 * kComputeUnits) {
     family = VECOPS_HIP_FAMILY_TILE_128;
     tile_m = tile_n = 128;
@@ -485,8 +516,9 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
 }
 
 const char* family_name(uint32_t family) {
-  static const char* const names[] = {"none", "tile_256", "tile_128", "tile_64", "skinny", "zero_k", "tile_256x128", "tile_128x256"};
-  return family < 8 ? names[family] : "unknown";
+  static const char* const names[] = {"none", "tile_256", "tile_128", "tile_64", "skinny", "zero_k", "tile_256x128", "tile_128x256",
+                                      "tile_256x352"};
+  return family < 9 ? names[family] : "unknown";
 }
 
 // The first tier of vecops' owner selection (matmul/details/kernel/amx/Backend.h:2724-2757; matmul/Family.h:216-239):
@@ -499,7 +531,7 @@ int32_t apply_request(const Problem& pr, const VecopsHipFamilyRequest* request, 
   if (request->struct_size < sizeof(VecopsHipFamilyRequest)) return fail(ST_INVALID, "matmul: family request record too short");
   if (request->selection != VECOPS_HIP_SELECT_PREFER && request->selection != VECOPS_HIP_SELECT_REQUIRE)
     return fail(ST_INVALID, "matmul: unknown family selection %u", request->selection);
-  if (request->family > VECOPS_HIP_FAMILY_TILE_128X256) return fail(ST_INVALID, "matmul: unknown family %u", request->family);
+  if (request->family > VECOPS_HIP_FAMILY_TILE_256X352) return fail(ST_INVALID, "matmul: unknown family %u", request->family);
   const bool degenerate = plan->family == VECOPS_HIP_FAMILY_NONE || plan->family == VECOPS_HIP_FAMILY_ZERO_K;
   int tile_m = 0, tile_n = 0;
   tile_of_family(request->family, &tile_m, &tile_n);
@@ -512,7 +544,8 @@ int32_t apply_request(const Problem& pr, const VecopsHipFamilyRequest* request, 
     serves = request->family == plan->family ||
              (request->family == VECOPS_HIP_FAMILY_SKINNY && !degenerate && skinny_applies(pr) && !(pr.dequant && pr.m >= pr.n));
   } else {
-    serves = true;
+    // every tile family serves every product, but the 256 x 352 tile its own class of them, K unsplit
+    serves = request->family != VECOPS_HIP_FAMILY_TILE_256X352 || (wide_tile_serves(pr) && request->split_k <= 1);
   }
   if (!serves) {
     if (request->selection == VECOPS_HIP_SELECT_PREFER) return ST_OK;  // the rule table's choice stands
@@ -768,7 +801,11 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
       p.col_term = nullptr;
     }
   }
-  if (pr.packed_b) {
+  if (plan.family == VECOPS_HIP_FAMILY_TILE_256X352) {
+    if (!wide_tile_serves(pr) || !launch_tile_gemm_i8_wide_serves(p, mode))
+      return fail(ST_INVALID, "matmul: the plan's family tile_256x352 cannot serve this call");
+    e = launch_tile_gemm_i8_wide(p, stream);
+  } else if (pr.packed_b) {
     const int a_mode = plan.vector_a == 0 ? 0 : ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr, pr.a, pr.a.rs)) ? 2 : 1;
     e = launch_tile_gemm_packed_b(pr.src, p, tile_m, tile_n, a_mode, stream);
   } else switch (pr.src) {

@@ -173,6 +173,155 @@ def loop(tr):
     return out
 
 
+# ---- the 256 x 352 tile (int8): 8 x 11 accumulator quads per wavefront -------------------------------------
+# A wavefront owns 128 rows x 176 columns: A blocks i = 0..7 (rows wm * 128 + 16 i), B blocks j = 0..10, which are
+# the blocks 2 j + wn of the workgroup's 22 (interleaved, so that the LDS swizzle of a fragment read stays a base
+# register plus a constant).  88 accumulator quads: 64 in accumulation registers, 24 in vector registers.  Fragment
+# registers: A blocks single (v[128 + 4 i ..]), B blocks double (set s at v[160 + 44 s + 4 j ..]).
+#   k-step 0 of a tile multiplies B set 0; it reads B set 1 (this tile's k-step 1) and, behind the last
+#   instruction of each row of blocks, that row's A fragment of k-step 1 into the registers just freed.
+#   The barrier stands one row into k-step 1 (the last of those reads has landed by then); behind it the loads of
+#   the tile after the next go into this stage and the next tile's k-step 0 fragments are read from the other.
+# LDS reads complete in order, so each matrix instruction waits for "at most N reads issued after the one I need":
+# the generator follows the reads through two trips of the loop and writes the counted waits.
+WIDE_FM, WIDE_FN = 8, 11
+WIDE_STAGE = (256 + 352) * 128
+
+
+def wide_fa(i):
+    return f"v[{128 + 4 * i}:{128 + 4 * i + 3}]"
+
+
+def wide_fb(s, j):
+    return f"v[{160 + 44 * s + 4 * j}:{160 + 44 * s + 4 * j + 3}]"
+
+
+class ReadTracker:
+    """Counted LDS waits: reads are numbered in issue order; `done` = every read up to this number has landed."""
+
+    def __init__(self):
+        self.issued = 0
+        self.done = 0
+        self.last_write = {}   # register name -> number of the read that fills it
+
+    def read(self, out, reg, text):
+        out.append(text)
+        self.issued += 1
+        self.last_write[reg] = self.issued
+
+    def need(self, out, regs):
+        upto = max(self.last_write.get(r, 0) for r in regs)
+        if upto > self.done:
+            out.append(f"s_waitcnt lgkmcnt({min(self.issued - upto, 15)})")
+            self.done = upto if self.issued - upto <= 15 else self.issued - 15
+
+    def need_all(self, out):
+        if self.issued > self.done:
+            out.append("s_waitcnt lgkmcnt(0)")
+            self.done = self.issued
+
+
+def wide_k_tile(st, tr):
+    out = []
+    acc = lambda i, j: f"%[c{i * WIDE_FN + j}]"
+
+    def a_read(i, ks, stage):
+        q = (2 * ks ^ i) & 3
+        tr.read(out, ("a", i), f"ds_read_b128 {wide_fa(i)}, %[la{stage}{q}] offset:{i * 2048}")
+
+    def b_read(to_set, j, ks, stage):
+        q = (ks ^ j) & 1
+        tr.read(out, ("b", to_set, j), f"ds_read_b128 {wide_fb(to_set, j)}, %[lb{stage}{q}] offset:{j * 4096}")
+
+    out += ["s_cmp_gt_i32 %[left], 0",
+            "s_cselect_b32 s82, 0x7fffffff, 0",
+            "s_cselect_b32 s86, 0x7fffffff, 0",
+            "s_sub_u32 %[left], %[left], 1"]
+    loads = []
+    for p in range(8):
+        pre = [f"s_add_u32 m0, %[m0w], {st * WIDE_STAGE + p * 4096}"]
+        pre.append("s_mov_b32 s88, %[ka]" if p == 0 else "s_add_u32 s88, s88, %[pa]")
+        loads.append((pre, [f"buffer_load_dwordx4 %[ra{p & 1}], s[80:83], s88 offen lds"]))
+    for p in range(11):
+        loads.append(([f"s_add_u32 m0, %[m0w], {st * WIDE_STAGE + 32768 + p * 4096}"],
+                      [f"buffer_load_dwordx4 %[rb{p}], s[84:87], %[kb] offen lds"]))
+    x = 0
+    for ks in range(2):
+        for i in range(WIDE_FM):
+            for j in range(WIDE_FN):
+                load = None
+                if ks == 1 and x >= 100 and (x - 100) % 4 == 0 and (x - 100) // 4 < len(loads):
+                    load = loads[(x - 100) // 4]
+                    out += load[0]
+                tr.need(out, [("a", i), ("b", ks, j)])
+                out.append(f"MFMA {acc(i, j)}, {wide_fb(ks, j)}, {wide_fa(i)}, {acc(i, j)}")
+                if load:
+                    out += load[1]
+                if ks == 0:
+                    # this tile's k-step 1: B set 1 early, A block i behind its row
+                    if x % 3 == 0 and x // 3 < WIDE_FN:
+                        b_read(1, x // 3, 1, st)
+                    if j == WIDE_FN - 1:
+                        a_read(i, 1, st)
+                else:
+                    if x == 88 + WIDE_FN - 1:
+                        # one row into k-step 1: every read of this stage has landed, every load of the next tile too
+                        tr.need_all(out)
+                        out += ["s_waitcnt vmcnt(0)", "s_barrier"]
+                        a_read(0, 0, st ^ 1)
+                    elif j == WIDE_FN - 1 and i > 0:
+                        a_read(i, 0, st ^ 1)
+                    if x >= 101 and (x - 101) % 3 == 0 and (x - 101) // 3 < WIDE_FN:
+                        b_read(0, (x - 101) // 3, 0, st ^ 1)
+                x += 1
+    assert x == 176
+    out += ["s_add_u32 %[ka], %[ka], 128", "s_add_u32 %[kb], %[kb], 128"]
+    return out
+
+
+def wide_loop():
+    out = []
+    for w in range(4):
+        out.append(f"s_mov_b32 s{80 + w}, %[da{w}]")
+        out.append(f"s_mov_b32 s{84 + w}, %[db{w}]")
+    tr = ReadTracker()
+    # k-step 0 of tile 0: every A block and B set 0
+    dummy = []
+    for j in range(WIDE_FN):
+        q = j & 1
+        tr.read(out, ("b", 0, j), f"ds_read_b128 {wide_fb(0, j)}, %[lb0{q}] offset:{j * 4096}")
+    for i in range(WIDE_FM):
+        tr.read(out, ("a", i), f"ds_read_b128 {wide_fa(i)}, %[la0{i & 3}] offset:{i * 2048}")
+    # The waits of a tile depend on the reads the tile before it left in flight.  Tile 0 follows the reads above; a
+    # tile that follows another tile sees that tile's reads.  The waits written for the first case are the stricter
+    # ones for the A blocks (their reads lie closer) - both cases are generated and compared, and the loop body uses
+    # per-case text: the first trip's tiles are peeled.
+    first0 = wide_k_tile(0, tr)
+    first1 = wide_k_tile(1, tr)
+    steady0 = wide_k_tile(0, tr)
+    steady1 = wide_k_tile(1, tr)
+    again0 = wide_k_tile(0, tr)
+    assert again0 == steady0, "the schedule has not reached its steady state"
+    # walk: tile 0 (first0); tile 1 (first1) if any; then pairs (steady0, steady1); then one more steady0 if odd
+    out += ["s_cmp_lt_u32 %[n], 2", "s_cbranch_scc1 4f"]
+    out += first0
+    out += first1
+    out += ["s_sub_u32 %[n], %[n], 2"]
+    out.append("1:")
+    out += ["s_cmp_lt_u32 %[n], 2", "s_cbranch_scc1 2f"]
+    out += steady0
+    out += steady1
+    out += ["s_sub_u32 %[n], %[n], 2", "s_branch 1b", "2:"]
+    out += ["s_cmp_eq_u32 %[n], 0", "s_cbranch_scc1 3f"]
+    out += steady0
+    out += ["s_branch 3f"]
+    out.append("4:")   # a single tile
+    out += first0
+    out.append("3:")
+    out += ["s_waitcnt vmcnt(0) lgkmcnt(0)", "s_nop 15", "s_nop 15"]
+    return out
+
+
 def as_macro(name, lines):
     text = f"#define {name}(MFMA) \\\n"
     body = []
@@ -192,6 +341,13 @@ def main():
     w(as_macro("VECOPS_LOOP256_K", loop(False)))
     w("\n")
     w(as_macro("VECOPS_LOOP256_TR", loop(True)))
+    w("\n// The K loop of the 256 x 352 tile (8-bit operands, both K-contiguous): see gen_tile_loop.py.\n")
+    w(as_macro("VECOPS_LOOP352_K", wide_loop()))
+    w("\n// its 88 accumulator quads: 64 in accumulation registers, 24 in vector registers\n")
+    w("#define VECOPS_LOOP352_ACCUMULATORS(t) \\\n  " +
+      ", \\\n  ".join(", ".join(f'[c{x}] "+{"a" if x < 64 else "v"}"(t[{x}])' for x in range(r, r + 4)) for r in range(0, 88, 4)) + "\n")
+    w("#define VECOPS_LOOP352_CLOBBERS \\\n  " + ", ".join(f'"s{r}"' for r in range(80, 89)) + ", \\\n  " +
+      ", \\\n  ".join(", ".join(f'"v{r}"' for r in range(b, min(b + 16, 248))) for b in range(128, 248, 16)) + "\n")
     w("\n// the accumulators as operands: quad x = t[x / 8][x % 8]\n")
     w("#define VECOPS_LOOP256_ACCUMULATORS(t) \\\n  " +
       ", \\\n  ".join(", ".join(f'[c{x}] "+a"(t[{x // 8}][{x % 8}])' for x in range(r, r + 4)) for r in range(0, 64, 4)) + "\n")
