@@ -71,6 +71,35 @@ def test_wide_tile_is_the_tables_choice_and_dequantises_bit_exactly(device, orac
     assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+def test_wide_tile_with_prepacked_weights(device, oracle):
+    """The same tile fed from vecops_hip_pack_b's layout (vecops' ops::matmul_pack, ops/MatmulPack.h:9-117), N ragged
+    against the 32-row panels of the pack: dequantised output bit-exact against the oracle and bit-equal to the product
+    with the plain operand."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = 2048, 11004, 1152
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    rs, cs = synth.scales(3, m), synth.scales(4, n)
+    ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    packed = capi.pack_b(tb)
+    plan = capi.plan_matmul_packed_b(ta, packed, torch.empty((m, n), dtype=torch.int32, device=device))
+    assert capi.FAMILY_NAMES[plan.family] == "tile_256x352"
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul_i8_dequant_packed_b(ta, packed, torch.from_numpy(rs).to(device), torch.from_numpy(cs).to(device), c)
+    plain = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    capi.matmul_i8_dequant(ta, tb, torch.from_numpy(rs).to(device), torch.from_numpy(cs).to(device), plain)
+    torch.cuda.synchronize()
+    want = oracle.matmul_i8_dequant(a, b, rs, cs, None)
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert torch.equal(c.view(torch.int32), plain.view(torch.int32))
+    # int32 sums through vecops_hip_matmul_packed_b
+    ci = torch.full((m, n), -1, dtype=torch.int32, device=device)
+    capi.matmul_packed_b(ta, packed, ci)
+    torch.cuda.synchronize()
+    rows = np.arange(0, m, 37)
+    assert np.array_equal(ci.cpu().numpy()[rows], (a[rows].astype(np.int64) @ b.astype(np.int64).T).astype(np.int32))
+
+
 def test_wide_tile_required_where_it_cannot_serve(device):
     import torch
     from vecops_amd import capi

@@ -275,7 +275,7 @@ def wide_k_tile(st, tr):
                         b_read(0, (x - 101) // 3, 0, st ^ 1)
                 x += 1
     assert x == 176
-    out += ["s_add_u32 %[ka], %[ka], 128", "s_add_u32 %[kb], %[kb], 128"]
+    out += ["s_add_u32 %[ka], %[ka], 128", "s_add_u32 %[kb], %[kb], %[sb]"]
     return out
 
 
