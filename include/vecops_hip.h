@@ -128,6 +128,19 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul(const VecopsHipOperand* a, const Vec
                                             void* workspace, uint64_t workspace_size, void* stream);
 
 /*
+ * vecops_hip_matmul with the plan made beforehand - the prepared invocation of vecops (ops::Matmul<Config>::prepare /
+ * Prepared / PatternPrepared, ops/Matmul.h:183-500; the prepared-call cache of docs/Runtime.md:196-206): `plan` is what
+ * vecops_hip_plan_matmul or vecops_hip_plan_matmul_family returned for operands of the same metadata (extents, strides,
+ * dtypes, alignment); the rule table is not consulted again.  The plan is checked against the operands - a family
+ * that cannot serve them, a K split beyond the K tiles or columns peeled where the table peels none is status 1
+ * (invalid argument), nothing is launched - and its workspace need is recomputed, never trusted.
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_planned(const VecopsHipOperand* a, const VecopsHipOperand* b,
+                                                    const VecopsHipOperand* c_in, const VecopsHipOperand* c,
+                                                    uint32_t compute, const VecopsHipPlan* plan, void* workspace,
+                                                    uint64_t workspace_size, void* stream);
+
+/*
  * The first tier of vecops' owner selection: an explicit family request (matmul::family_selection::Automatic /
  * Prefer<F> / Require<F>, matmul/Family.h:216-239; consulted first by Backend<AMX>::run,
  * matmul/details/kernel/amx/Backend.h:2724-2757).  PREFER takes the family when it can serve the call and the rule
@@ -164,15 +177,16 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_family(const VecopsHipOperand* a, co
  * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
  * vecops (its callers size and own every workspace, ops/Matmul.h:504-526).  The split-K partial sums and the
  * unsigned-operand terms live in a buffer of VECOPS_HIP_STATIC_WORKSPACE_BYTES that belongs to the library's
- * code object on each GPU (8 MiB, held until the process ends; the K splits of problems with few output tiles
- * need at most 4 MiB, the row sums of unsigned operands 4 bytes per row of a and b); the call allocates and frees
- * nothing.  The one plan of vecops_hip_matmul that needs more - K of a problem with 128 to 200 tiles of 128 x 128
- * split two to four ways, 24-32 MB of partial sums - is not taken here: such a problem runs unsplit (the sums then
- * differ from vecops_hip_matmul's in their order).  A call whose plan still needs more than the buffer returns 2
- * (not applicable) and launches nothing.  Otherwise the same kernels and therefore the same results, bit for
- * bit, as vecops_hip_matmul.  Every call on
- * one GPU shares that GPU's buffer: calls that overlap on one GPU (different streams or host threads) race;
- * calls on one stream, or otherwise ordered, do not.
+ * code object on each GPU (8 MiB, held until the process ends; the K splits of problems with few output tiles of
+ * 64 x 64 need at most 4 MiB, the row sums of unsigned operands 4 bytes per row of a and b); the call allocates and
+ * frees nothing.  A plan of vecops_hip_matmul whose partial sums would not fit - K of a problem with 128 to 200 tiles
+ * of 128 x 128 split two to four ways (24-32 MB), or of few 128 x 128 tiles of fp32 operands - is not taken here: the
+ * split is halved until the sums fit, down to an unsplit product (the sums then differ from vecops_hip_matmul's in
+ * their order).  A call that still needs more than the buffer - the row sums of an unsigned operand with more than two
+ * million rows - returns 2 (not applicable) and launches nothing.  Otherwise the same kernels and therefore the same
+ * results, bit for bit, as vecops_hip_matmul.  `stream` must belong to the current device (each GPU has its own copy
+ * of the buffer; a stream of another device is status 1).  Every call on one GPU shares that GPU's buffer: calls that
+ * overlap on one GPU (different streams or host threads) race; calls on one stream, or otherwise ordered, do not.
  */
 #define VECOPS_HIP_STATIC_WORKSPACE_BYTES (8u << 20)
 VECOPS_HIP_EXPORT uint64_t vecops_hip_static_workspace_bytes(void);

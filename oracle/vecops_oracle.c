@@ -31,9 +31,11 @@
  *       reference tests' own 8e-4 tolerance, everything else bit for bit.
  *   vo_amx_small_vector_profitable & co   - the static_assert table of
  *       tests/matmul/TilerTest.cpp:86-98.
- *   vo_matmul_w8a16_group                 - PARITY UNPINNED: the reference has
- *       no weight-only group-scaled matmul; the contract is stated here and
- *       checked only against an fp64 brute force of the same formula.
+ *   vo_matmul_w8a16_group                 - the reference has no weight-only
+ *       group-scaled matmul; the contract is stated at the function and pinned by
+ *       the mathematics (tests/test_oracle.py, test_w8a16_group_*): an independent
+ *       float64 einsum, unit scales reducing it to vo_matmul, one group's scale
+ *       moving exactly that group's dot, a hand-worked table.
  */
 #include <math.h>
 #include <stdint.h>

@@ -149,9 +149,12 @@ def test_rule_table_known_answers():
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
     # ... and up to 256 tiles in two parts, from forty K tiles per part
-    for (m, n, k), split in (((1024, 4096, 11008), 2), ((1024, 4096, 6144), 2), ((1024, 4096, 4096), 1), ((896, 4096, 4096), 1)):
+    # (with 160 K tiles or more those 256 tiles become 64 of 256 x 256 in four parts)
+    for (m, n, k), family, split in (((1024, 4096, 11008), "tile_256", 4), ((1024, 4096, 6144), "tile_128", 2),
+                                     ((1024, 4096, 4096), "tile_128", 1), ((896, 4096, 4096), "tile_128", 1),
+                                     ((896, 4096, 11008), "tile_256", 4)):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
-        assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == split, (m, n, k, p.split_k)
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
     rc, p = _plan(_operand(capi.I8, (1024, 11008)), _operand(capi.I8, (4096, 11008)), _operand(capi.I32, (1024, 4096)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 2
     rc, p = _plan(_operand(capi.I8, (1024, 8192)), _operand(capi.I8, (4096, 8192)), _operand(capi.I32, (1024, 4096)))

@@ -14,7 +14,9 @@ from vecops_amd import host_api as H
 from vecops_amd import synth
 
 pytestmark = pytest.mark.gpu
-FLAVORS = [H.HOST_LIB] + ([H.UPSTREAM_LIB] if os.path.exists(H.UPSTREAM_LIB) else [])
+# the same plug-in compiled against the reference's own runtime sources (a checker build: oracle/Makefile, target ref)
+UPSTREAM_LIB = os.path.join(H.ROOT, "oracle", "_ref", "libvecops_hip_host_upstream.so")
+FLAVORS = [H.HOST_LIB] + ([UPSTREAM_LIB] if os.path.exists(UPSTREAM_LIB) else [])
 
 
 @pytest.fixture(scope="module", params=FLAVORS, ids=lambda p: "upstream" if "upstream" in p else "restated")

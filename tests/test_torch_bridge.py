@@ -84,6 +84,9 @@ def test_torch_ops_matmul_equals_the_c_abi(device):
     c = torch.full((m, n), float("nan"), device=device)
     assert ns.matmul(a, b, None, c) is c
     assert torch.equal(c, want)
+    # and against an independent product of the same bf16 values in float64 (not only against the C ABI)
+    exact_bf16 = a.double() @ b.double().T
+    assert float(((c.double() - exact_bf16).abs() / exact_bf16.abs().clamp(min=1.0)).max()) <= 2e-6 * k / 32
     # the raw torch.ops symbol, on a stream of its own, with a C-input that aliases the output
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())

@@ -26,10 +26,17 @@ def test_static_workspace_split_k_twice_in_a_row(device, oracle):
         assert plan.split_k > 1 and 0 < plan.workspace_bytes <= capi.lib().vecops_hip_static_workspace_bytes()
         want = capi.matmul(a, b, torch.empty((m, n), dtype=torch.float32, device=device))
         got = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
-        before = torch.cuda.memory_allocated(device)
-        capi.matmul_static_workspace(a, b, got)
-        assert torch.cuda.memory_allocated(device) == before
+        capi.matmul_static_workspace(a, b, got)      # warm-up: the kernels' code and the scratch address are set up once
         torch.cuda.synchronize()
+        got.fill_(float("nan"))
+        torch.cuda.synchronize()
+        # free device memory as the driver sees it (an allocation inside the library would not show in torch's own
+        # counter, which is kept as a second check)
+        before_driver, before_torch = torch.cuda.mem_get_info(device)[0], torch.cuda.memory_allocated(device)
+        capi.matmul_static_workspace(a, b, got)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info(device)[0] == before_driver
+        assert torch.cuda.memory_allocated(device) == before_torch
         assert torch.equal(got.view(torch.int32), want.view(torch.int32)), f"call {call}: differs from vecops_hip_matmul"
         ref = np.zeros((m, n), np.float32)
         oracle.matmul(a_bits, b_bits, ref, acc_f64=True)
@@ -55,6 +62,23 @@ def test_static_workspace_unsigned_operands_and_c_input(device, oracle):
         ref = np.zeros((m, n), np.int32)
         oracle.matmul(a, b, ref, cin=cin, atom=O.ATOM_I8I32)
         assert np.array_equal(got.cpu().numpy(), ref)
+
+
+def test_static_workspace_shrinks_a_split_that_does_not_fit(device, oracle):
+    """fp32 compute, 128 tiles of 128 x 128 and a long K: vecops_hip_matmul splits K in two (16 MiB of partial sums);
+    this entry point runs the product unsplit instead of refusing it."""
+    import torch
+    m, n, k = 1024, 2048, 4096
+    a, b = synth.uniform_pm1(81, (m, k)), synth.uniform_pm1(82, (n, k))
+    ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    plan = capi.plan_matmul(ta, tb, c, compute=capi.COMPUTE_F32)
+    assert plan.workspace_bytes > capi.lib().vecops_hip_static_workspace_bytes()
+    capi.matmul_static_workspace(ta, tb, c, compute=capi.COMPUTE_F32)
+    torch.cuda.synchronize()
+    rows = np.arange(0, m, 61)
+    want = a[rows].astype(np.float64) @ b.astype(np.float64).T
+    assert rel_err(c.cpu().numpy()[rows], want) <= 2e-6 * max(1, k // 32)
 
 
 def test_static_workspace_rejects_what_does_not_fit(device):

@@ -21,7 +21,7 @@ STATUS_NAMES = {0: "Ok", 1: "InvalidArgument", 2: "NotApplicable", 3: "NotFound"
 
 EXPORTS = [
     "vecops_hip_abi_version", "vecops_hip_last_error", "vecops_hip_device_count", "vecops_hip_plan_matmul",
-    "vecops_hip_matmul", "vecops_hip_matmul_i8_dequant", "vecops_hip_matmul_i8_dequant_workspace",
+    "vecops_hip_matmul", "vecops_hip_matmul_planned", "vecops_hip_matmul_i8_dequant", "vecops_hip_matmul_i8_dequant_workspace",
     "vecops_hip_matmul_w8a16_group", "vecops_hip_packed_b_bytes", "vecops_hip_pack_b", "vecops_hip_pack_b_compensated",
     "vecops_hip_plan_matmul_packed_b", "vecops_hip_matmul_packed_b", "vecops_hip_matmul_i8_dequant_packed_b",
     "vecops_hip_plan_matmul_fused", "vecops_hip_matmul_fused", "vecops_hip_quantize_rows",
@@ -103,6 +103,7 @@ def lib() -> C.CDLL:
         R = C.POINTER(FamilyRequest)
         L.vecops_hip_plan_matmul_family.argtypes = [P, P, P, P, C.c_uint32, R, C.POINTER(Plan)]
         L.vecops_hip_matmul_family.argtypes = [P, P, P, P, C.c_uint32, R, C.c_void_p, C.c_uint64, C.c_void_p]
+        L.vecops_hip_matmul_planned.argtypes = [P, P, P, P, C.c_uint32, C.POINTER(Plan), C.c_void_p, C.c_uint64, C.c_void_p]
         L.vecops_hip_mfma_stream_ops.restype = C.c_uint64
         L.vecops_hip_mfma_stream_ops.argtypes = [C.c_uint32, C.c_int32, C.c_int32]
         L.vecops_hip_mfma_stream.argtypes = [C.c_uint32, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_void_p,
@@ -223,6 +224,21 @@ def matmul(a, b, c, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None
     return c
 
 
+def matmul_planned(a, b, c, plan: Plan, c_in=None, compute=COMPUTE_BF16, workspace=None, stream=None):
+    """``matmul`` with a plan made beforehand (``plan_matmul`` / ``plan_matmul_family`` on operands of the same
+    metadata): ``vecops_hip_matmul_planned``."""
+    import torch
+    if plan.workspace_bytes and (workspace is None or workspace.numel() * workspace.element_size() < plan.workspace_bytes):
+        workspace = torch.empty(plan.workspace_bytes, dtype=torch.uint8, device=c.device)
+    oa, ob, oc = operand(a), operand(b), operand(c)
+    oi = operand(c_in) if c_in is not None else None
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(lib().vecops_hip_matmul_planned(C.byref(oa), C.byref(ob), C.byref(oi) if oi is not None else None, C.byref(oc),
+                                           compute, C.byref(plan), ws_ptr, ws_size, _stream_handle(stream)))
+    return c
+
+
 class PreparedMatmul:
     """``matmul`` on fixed operands with everything but the launch done once: the descriptors, the plan and the
     workspace are built here, a call is one foreign call (the counterpart of vecops' prepared invocation,
@@ -241,8 +257,8 @@ class PreparedMatmul:
         ws_ptr = workspace.data_ptr() if workspace is not None else None
         ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
         self._args = (C.byref(self._oa), C.byref(self._ob), C.byref(self._oi) if self._oi is not None else None,
-                      C.byref(self._oc), compute, ws_ptr, ws_size, _stream_handle(stream))
-        self._fn = lib().vecops_hip_matmul
+                      C.byref(self._oc), compute, C.byref(self.plan), ws_ptr, ws_size, _stream_handle(stream))
+        self._fn = lib().vecops_hip_matmul_planned
 
     def __call__(self):
         rc = self._fn(*self._args)

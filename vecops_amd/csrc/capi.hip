@@ -236,7 +236,11 @@ constexpr int kStreamGroupsPerUnit = 2;  // workgroups of 4 wavefronts per compu
 // Operands that go through registers into LDS (rows that are not 16-byte aligned, fp32 memory, unsigned bytes) keep
 // the pricing their kernels were calibrated with: 0.85, rounds of 256, and the margin of the rectangles (8 x 777 x
 // 1000 x 3001 64 us on 128x256 tiles against 73.5 on 128x128; fp32 memory 2048^3 32 us on 128x128 against 43).
+// Where the loads write LDS themselves the 256x256 tile runs its written-out K loop on the 16x16 matrix instructions,
+// a tenth faster than before, and the smaller tiles are priced against that: bf16 4096^3 94 / 133 / 130 / 113 us,
+// int8 4096^3 59 / 82 / 83 / 70 (`bench.py --only families`, `--only rule_check`).
 constexpr int64_t kQuality256x128 = 800, kQuality128 = 900, kQuality128Int8 = 970, kQuality128Staged = 850;
+constexpr int64_t kQuality256x128Direct = 710, kQuality128Direct = 830, kQuality128Int8Direct = 850;
 
 // Every operand class but the unsigned bytes, with K contiguous on both sides, no C input, one side <= 16 rows, the
 // other >= 512 (vecops' small-vector leaves serve every atom, matmul/details/kernel/amx/Backend.h:767-992)
@@ -341,6 +345,13 @@ bool wide_tile_serves(const Problem& pr) {
   return pr.out_kind == OUT_I32 || (pr.dequant && pr.out_kind == OUT_F32);
 }
 
+// How the operands of a (non-empty) problem can be fetched: the plan's vector flags and B's layout.
+void plan_fetch_flags(const Problem& pr, VecopsHipPlan* plan) {
+  plan->vector_a = k_vector_ok(pr.a) ? 1 : 0;
+  plan->vector_b = pr.packed_b || (k_vector_ok(pr.b) || (pr.b.rs == 1 && pr.b.cs != 1 && n_vector_ok(pr.b) && dtype_bytes(pr.b.dtype) != 1)) ? 1 : 0;
+  plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
+}
+
 // The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure
 // integer function of (operand class, m, n, k); it picks the workgroup tile by
 // how many tiles the problem yields against the 256 compute units and splits K
@@ -361,9 +372,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
     plan->family = VECOPS_HIP_FAMILY_ZERO_K;
     return;
   }
-  plan->vector_a = k_vector_ok(pr.a) ? 1 : 0;
-  plan->vector_b = pr.packed_b || (k_vector_ok(pr.b) || (pr.b.rs == 1 && pr.b.cs != 1 && n_vector_ok(pr.b) && dtype_bytes(pr.b.dtype) != 1)) ? 1 : 0;
-  plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
+  plan_fetch_flags(pr, plan);
 
   if (pr.src == kSrcF64) {  // one kernel: 128 x 128 tiles, K never split
     plan->family = VECOPS_HIP_FAMILY_TILE_128;
@@ -395,10 +404,10 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   const int mode = fetch_mode(pr, *plan);
   const bool direct = mode == MODE_KVEC_DMA || mode == MODE_NVEC_B_DMA;  // loads that write LDS themselves
   const Candidate candidates[] = {{VECOPS_HIP_FAMILY_TILE_256, 256, 256, 1000},
-                                  {VECOPS_HIP_FAMILY_TILE_256X128, 256, 128, kQuality256x128},
-                                  {VECOPS_HIP_FAMILY_TILE_128X256, 128, 256, kQuality256x128},
+                                  {VECOPS_HIP_FAMILY_TILE_256X128, 256, 128, direct ? kQuality256x128Direct : kQuality256x128},
+                                  {VECOPS_HIP_FAMILY_TILE_128X256, 128, 256, direct ? kQuality256x128Direct : kQuality256x128},
                                   {VECOPS_HIP_FAMILY_TILE_128, 128, 128,
-                                   !direct ? kQuality128Staged : bytes ? kQuality128Int8 : kQuality128}};
+                                   !direct ? kQuality128Staged : bytes ? kQuality128Int8Direct : kQuality128Direct}};
   uint32_t family = VECOPS_HIP_FAMILY_TILE_64;
   int64_t tile_m = 64, tile_n = 64, best_cost = INT64_MAX;
   for (const Candidate& c : candidates) {
@@ -491,6 +500,14 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
       family = VECOPS_HIP_FAMILY_TILE_128;
       band_split = static_cast<uint32_t>(parts);
     }
+  }
+  // 256 tiles of 128x128 that are 64 of 256x256, and a K of 160 tiles or more: the big tile in four parts puts one
+  // workgroup of its (faster) loop on every unit (bf16 1024 x 4096 x 11008: 84 us against 89-92 for the two parts of
+  // 128x128 tiles above and 116 unsplit; with a shorter K - 1024 x 4096 x 4096, 16 K tiles per part - it loses, 48 against 44).
+  if (direct && !pr.packed_b && band_split == 2 && tiles(256) * 4 == kComputeUnits && k_tiles / 4 >= 40 &&
+      static_cast<uint64_t>(4) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
+    family = VECOPS_HIP_FAMILY_TILE_256;
+    band_split = 4;
   }
   plan->family = family;
   finish_tile_plan(pr, plan, band_split);
@@ -680,6 +697,10 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     main_plan.peeled_columns = 0;
     main_plan.workspace_bytes = 0;
     choose(rest, &rest_plan, workspace_size, false);
+    // (checked before anything is launched: the main product must not have written C when the call fails)
+    if (rest_plan.workspace_bytes > workspace_size || (rest_plan.workspace_bytes > 0 && workspace == nullptr))
+      return fail(ST_INVALID, "matmul: the peeled columns need a workspace of %llu bytes, %llu supplied",
+                  (unsigned long long)rest_plan.workspace_bytes, (unsigned long long)workspace_size);
     int32_t rc = run_problem(main, main_plan, row_scales, column_scales, correction, nullptr, 0, stream);
     if (rc != ST_OK) return rc;
     return run_problem(rest, rest_plan, row_scales, column_scales, correction, workspace, workspace_size, stream);
@@ -1646,11 +1667,18 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::atomic<void*> g_scratch_address[kMaxDevices];
 
-// Address of `scratch` on the current device, looked up once per device.
-int32_t static_workspace(void** address) {
+// Address of `scratch` on the current device, looked up once per device.  The kernels of a call go to the caller's
+// stream: that stream must belong to the current device (its copy of the array is the one whose address is used).
+int32_t static_workspace(hipStream_t stream, void** address) {
   int device = -1;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return fail(ST_EXEC, "hipGetDevice: %s", hipGetErrorString(e));
+  if (stream != nullptr) {
+    int stream_device = -1;
+    if (hipStreamGetDevice(stream, &stream_device) == hipSuccess && stream_device != device)
+      return fail(ST_INVALID, "matmul_static_workspace: the stream belongs to device %d, the current device is %d",
+                  stream_device, device);
+  }
   if (device < 0 || device >= kMaxDevices) return fail(ST_EXEC, "device ordinal %d out of range", device);
   void* known = g_scratch_address[device].load(std::memory_order_acquire);
   if (known == nullptr) {
@@ -1679,12 +1707,18 @@ int32_t vecops_hip_matmul_static_workspace(const VecopsHipOperand* a, const Veco
   if (rc != ST_OK) return rc;
   VecopsHipPlan plan;
   choose(pr, &plan, VECOPS_HIP_STATIC_WORKSPACE_BYTES);
+  // A K split whose partial sums do not fit the buffer is halved until they do (unsplit, a product needs no scratch
+  // beyond the row sums of an unsigned operand): the call is then slower than with a caller's workspace, not refused.
+  int tile_m = 0, tile_n = 0;
+  tile_of_family(plan.family, &tile_m, &tile_n);
+  while (tile_m != 0 && plan.peeled_columns == 0 && plan.split_k > 1 && plan.workspace_bytes > VECOPS_HIP_STATIC_WORKSPACE_BYTES)
+    finish_tile_plan(pr, &plan, plan.split_k / 2);
   if (plan.workspace_bytes > VECOPS_HIP_STATIC_WORKSPACE_BYTES)
     return fail(ST_NOT_APPLICABLE, "matmul_static_workspace: the call needs %llu bytes of scratch, the library holds %llu",
                 (unsigned long long)plan.workspace_bytes, (unsigned long long)VECOPS_HIP_STATIC_WORKSPACE_BYTES);
   void* address = nullptr;
   if (plan.workspace_bytes > 0) {
-    rc = static_workspace(&address);
+    rc = static_workspace(static_cast<hipStream_t>(stream), &address);
     if (rc != ST_OK) return rc;
   }
   // Nothing in the scratch has to start at zero: every split writes each of its partial sums before the
@@ -1725,6 +1759,48 @@ int32_t vecops_hip_matmul(const VecopsHipOperand* a, const VecopsHipOperand* b, 
   VecopsHipPlan plan;
   choose(pr, &plan);
   return run_problem(pr, plan, nullptr, nullptr, nullptr, workspace, workspace_size, static_cast<hipStream_t>(stream));
+}
+
+int32_t vecops_hip_matmul_planned(const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
+                                  const VecopsHipOperand* c, uint32_t compute, const VecopsHipPlan* plan, void* workspace,
+                                  uint64_t workspace_size, void* stream) {
+  if (plan == nullptr) return fail(ST_INVALID, "matmul_planned: null plan");
+  Problem pr{};
+  int32_t rc = describe(a, b, c_in, c, compute, &pr);
+  if (rc != ST_OK) return rc;
+  // What the plan may say is what the planning entries can return for these operands.  Its family and K split go
+  // through the same check as a required family (which also recomputes the workspace need); columns are peeled only in
+  // the rule table's own plan, so a plan that peels is compared with that - the one case that consults the table.
+  VecopsHipPlan checked;
+  if (plan->peeled_columns != 0) {
+    choose(pr, &checked);
+    if (plan->family != checked.family || plan->split_k != checked.split_k || plan->peeled_columns != checked.peeled_columns)
+      return fail(ST_INVALID, "matmul_planned: the plan peels %u columns, the rule table's own plan for these operands %u",
+                  plan->peeled_columns, checked.peeled_columns);
+  } else {
+    memset(&checked, 0, sizeof(checked));
+    checked.split_k = 1;
+    if (pr.batch == 0 || pr.m == 0 || pr.n == 0) {
+      checked.family = VECOPS_HIP_FAMILY_NONE;
+    } else if (pr.k == 0) {
+      checked.family = VECOPS_HIP_FAMILY_ZERO_K;
+    } else {
+      checked.family = VECOPS_HIP_FAMILY_TILE_64;  // (a stand-in for "some product": the request below decides)
+      plan_fetch_flags(pr, &checked);
+    }
+    if (plan->split_k == 0) return fail(ST_INVALID, "matmul_planned: a finished plan splits K at least one way");
+    VecopsHipFamilyRequest request;
+    request.struct_size = sizeof(request);
+    request.selection = VECOPS_HIP_SELECT_REQUIRE;
+    request.family = plan->family;
+    request.split_k = plan->split_k;
+    if (apply_request(pr, &request, &checked) != ST_OK)
+      return fail(ST_INVALID, "matmul_planned: the plan's family %s cannot serve these operands", family_name(plan->family));
+    checked.family = plan->family;
+    if (checked.split_k != plan->split_k)
+      return fail(ST_INVALID, "matmul_planned: the plan splits K %u ways, these operands allow %u", plan->split_k, checked.split_k);
+  }
+  return run_problem(pr, checked, nullptr, nullptr, nullptr, workspace, workspace_size, static_cast<hipStream_t>(stream));
 }
 
 uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int64_t n, int64_t k) {

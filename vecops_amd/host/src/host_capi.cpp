@@ -80,6 +80,7 @@ std::atomic<std::uint64_t> g_next_handle{1};
 struct HipRuntime {
   int (*get_device)(int*) = nullptr;
   int (*malloc_)(void**, size_t) = nullptr;
+  int (*free_)(void*) = nullptr;
   bool ok = false;
 };
 const HipRuntime& hip_runtime() {
@@ -90,7 +91,8 @@ const HipRuntime& hip_runtime() {
     if (lib == nullptr) return r;
     r.get_device = reinterpret_cast<int (*)(int*)>(dlsym(lib, "hipGetDevice"));
     r.malloc_ = reinterpret_cast<int (*)(void**, size_t)>(dlsym(lib, "hipMalloc"));
-    r.ok = r.get_device != nullptr && r.malloc_ != nullptr;
+    r.free_ = reinterpret_cast<int (*)(void*)>(dlsym(lib, "hipFree"));
+    r.ok = r.get_device != nullptr && r.malloc_ != nullptr && r.free_ != nullptr;
     return r;
   }();
   return runtime;
@@ -122,14 +124,22 @@ struct ThreadWorkspace {
     if (buffer.size < bytes) {
       std::lock_guard<std::mutex> lock(g_pool_mutex);
       std::vector<DeviceBuffer>& pool = g_buffer_pool[device];
-      if (buffer.data != nullptr) pool.push_back(buffer);  // too small for this call: someone else's next one may fit
+      // The buffer that is too small for this call goes back to the pool (someone else's next call may fit), unless
+      // the pool is full: then it is freed (hipFree waits for the device, so no kernel of an earlier call still
+      // uses it).  The pool holds at most kPoolCap buffers per device, which bounds what the bridge keeps.
+      constexpr size_t kPoolCap = 8;
+      if (buffer.data != nullptr) {
+        if (pool.size() < kPoolCap) pool.push_back(buffer);
+        else hip.free_(buffer.data);
+      }
       buffer = DeviceBuffer{};
-      for (size_t i = 0; i < pool.size(); ++i) {
-        if (pool[i].size >= bytes) {
-          buffer = pool[i];
-          pool.erase(pool.begin() + static_cast<std::ptrdiff_t>(i));
-          break;
-        }
+      // the smallest pooled buffer that fits: a small request must not take the largest one
+      size_t best = pool.size();
+      for (size_t i = 0; i < pool.size(); ++i)
+        if (pool[i].size >= bytes && (best == pool.size() || pool[i].size < pool[best].size)) best = i;
+      if (best != pool.size()) {
+        buffer = pool[best];
+        pool.erase(pool.begin() + static_cast<std::ptrdiff_t>(best));
       }
       if (buffer.data == nullptr) {
         const std::uint64_t want = (bytes + (std::uint64_t{1} << 20) - 1) & ~((std::uint64_t{1} << 20) - 1);

@@ -12,7 +12,6 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 HOST_LIB = os.path.join(HERE, "lib", "libvecops_hip_host.so")
-UPSTREAM_LIB = os.path.join(ROOT, "oracle", "_ref", "libvecops_hip_host_upstream.so")
 ARTIFACT_DIR = os.path.join(HERE, "lib", "artifacts")
 
 DEVICE_CPU, DEVICE_PRIVATE = 1, 255
