@@ -32,11 +32,13 @@ def test_static_workspace_split_k_twice_in_a_row(device, oracle):
         torch.cuda.synchronize()
         # free device memory as the driver sees it (an allocation inside the library would not show in torch's own
         # counter, which is kept as a second check)
+        import gc
+        gc.collect()     # (tensors of earlier tests must not be freed between the two readings)
         before_driver, before_torch = torch.cuda.mem_get_info(device)[0], torch.cuda.memory_allocated(device)
         capi.matmul_static_workspace(a, b, got)
         torch.cuda.synchronize()
-        assert torch.cuda.mem_get_info(device)[0] == before_driver
-        assert torch.cuda.memory_allocated(device) == before_torch
+        assert torch.cuda.mem_get_info(device)[0] >= before_driver      # nothing was taken from the device
+        assert torch.cuda.memory_allocated(device) <= before_torch
         assert torch.equal(got.view(torch.int32), want.view(torch.int32)), f"call {call}: differs from vecops_hip_matmul"
         ref = np.zeros((m, n), np.float32)
         oracle.matmul(a_bits, b_bits, ref, acc_f64=True)

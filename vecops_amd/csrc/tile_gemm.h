@@ -51,13 +51,13 @@ enum Activation : int { ACT_NONE = 0, ACT_RELU = 1, ACT_CLAMP = 2, ACT_SIGMOID =
 enum LoadKind : int {
   LOAD_KVEC = 0,     // K contiguous (rows at any element alignment): one 16-byte load per chunk
   LOAD_GENERIC = 1,  // any strides: one load per element
-  LOAD_NVEC = 2,     // spatial index contiguous (B given as [K,N] row-major), 16-byte aligned rows:
-                     // transposed in registers on the way into LDS (32-bit compute elements)
-  LOAD_NTR = 3,      // the same operand layout for 16-bit compute elements: stored in LDS as it
-                     // lies in memory ([k][n]) and transposed by the LDS read (ds_read_b64_tr_b16)
+  LOAD_NTR = 3,      // spatial index contiguous (B given as [K,N] row-major), 16-bit compute elements: stored in
+                     // LDS as it lies in memory ([k][n]) and transposed by the LDS read (ds_read_b64_tr_b16)
   LOAD_KDMA = 4,     // LOAD_KVEC with the loads writing LDS themselves (buffer_load ... lds): no staging
                      // registers, no LDS store instructions
-  LOAD_NTR_DMA = 5   // LOAD_NTR likewise; rows of the [k][n] tile are packed (no pad) and swizzled instead
+  LOAD_NTR_DMA = 5,  // LOAD_NTR likewise; rows of the [k][n] tile are packed (no pad) and swizzled instead
+  LOAD_KN32 = 6      // the same operand layout for 32-bit compute elements (fp32 on the fp32 matrix cores): stored in LDS
+                     // as it lies in memory ([k][n]); a matrix instruction's operand is one 4-byte LDS read per lane
 };
 constexpr bool load_is_dma(int load) { return load == LOAD_KDMA || load == LOAD_NTR_DMA; }
 constexpr bool load_is_ntr(int load) { return load == LOAD_NTR || load == LOAD_NTR_DMA; }
@@ -1268,101 +1268,96 @@ struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
   }
 };
 
-// LOAD_NVEC for 32-bit compute elements: units of 4(k) x 4(n); a thread loads four
-// 16-byte rows along n and writes four K-contiguous chunks, the transposition being
-// a mere choice of registers.
+// LOAD_KN32: fp32 operands multiplied in fp32, stored with the spatial index contiguous (B handed over as [K,N]
+// row-major).  The K tile (32 k rows of ROWS floats) goes into LDS as it lies in memory, kPitch bytes between k rows:
+// 16-byte loads along n, 16-byte LDS writes, no shuffling.  v_mfma_f32_32x32x2_f32 takes ONE float per lane and
+// operand - lane l supplies column l % 32 at k = e (lanes 0-31) or 4 + e (lanes 32-63) of the k-step for instruction
+// e - which is a 4-byte LDS read of 128 contiguous bytes per half wavefront; the pitch (a row plus 32 bytes) puts the
+// two halves' rows, four k rows apart, into different halves of the banks.  (Transposing 4 x 4 units in registers
+// on the way into a K-contiguous tile, four loads and four 16-byte LDS writes per unit with half the threads idle,
+// made the 1024^3 product take 39 us where K-contiguous operands take 23.)
 template <int ROWS, int THREADS>
-struct Stager<SRC_F32, LOAD_NVEC, ROWS, THREADS> {
+struct Stager<SRC_F32, LOAD_KN32, ROWS, THREADS> {
   using T = SrcTraits<SRC_F32>;
-  static constexpr int UNITS_TOTAL = 2 * ROWS;  // (ROWS / 4) along n  x  8 along k
-  static constexpr int UNITS = (UNITS_TOTAL + THREADS - 1) / THREADS;
-  static constexpr bool kAllActive = UNITS_TOTAL % THREADS == 0;
-  static constexpr int kParts = UNITS;
-  static constexpr int kStoreOps = 4;
-  static constexpr int kLoadOps = 4;
+  static constexpr int kPitch = ROWS * 4 + 32;
+  static constexpr int CHUNKS_PER_ROW = ROWS / 4;
+  static constexpr int CHUNKS = 32 * CHUNKS_PER_ROW / THREADS;
+  static_assert(CHUNKS >= 1 && 32 * CHUNKS_PER_ROW % THREADS == 0, "whole chunks per thread");
+  static_assert(THREADS % CHUNKS_PER_ROW == 0, "every part of a thread is the same chunk, THREADS / CHUNKS_PER_ROW k rows on");
+  static constexpr int K_ROWS_PER_PART = THREADS / CHUNKS_PER_ROW;
+  static constexpr int kParts = CHUNKS;
+  static constexpr int kStoreOps = 1;
+  static constexpr int kLoadOps = 1;
   static constexpr bool kHasSpare = false;
   static constexpr bool kStagesChecked = false;
-  __device__ __forceinline__ void stage_checked(int, char*) const {}
   struct Spare {};
+  __device__ __forceinline__ void stage_checked(int, char*) const {}
   const char* base;
-  const VECOPS_GLOBAL char* tile_base;
-  uint32_t unit_bytes[UNITS];
-  int64_t rs, ks;
-  int first_row, extent, k_end;
-  int n_local[UNITS], kb[UNITS];
-  int tid_;
-  uint32_t regs[UNITS][4][4];  // [k row][n]
+  const VECOPS_GLOBAL char* tile_base;  // (k = 0, first n of the tile), wavefront-uniform
+  uint32_t chunk_bytes;                 // byte offset of (k row of part 0, first n of the chunk) from tile_base
+  int64_t ks;                           // elements between consecutive k
+  int first_row, extent, k_end, tid_;
+  u32x4 regs[CHUNKS];
 
-  __device__ __forceinline__ bool active(int u) const { return kAllActive || u * THREADS + tid_ < UNITS_TOTAL; }
+  __device__ __forceinline__ static int k_row(int part, int tid) { return (part * THREADS + tid) / CHUNKS_PER_ROW; }
+  __device__ __forceinline__ static int chunk(int part, int tid) { return (part * THREADS + tid) % CHUNKS_PER_ROW; }
 
-  __device__ __forceinline__ void init(const void* base_, int64_t rs_, int64_t ks_, int first_row_, int extent_,
+  __device__ __forceinline__ void init(const void* base_, int64_t /*rs*/, int64_t ks_, int first_row_, int extent_,
                                        int k_end_, int tid, uint32_t /*flip*/) {
     base = static_cast<const char*>(base_);
-    rs = rs_;
     ks = ks_;
     first_row = first_row_;
     extent = extent_;
     k_end = k_end_;
     tid_ = tid;
-    tile_base = (const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * 4);
-#pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-      const int unit = u * THREADS + tid;
-      n_local[u] = (unit % (ROWS / 4)) * 4;
-      kb[u] = (unit / (ROWS / 4)) & 7;  // chunk of the K tile: k = 4*kb .. 4*kb+3
-      const int n = min(first_row + n_local[u], extent - 4) - first_row;  // extent is a multiple of 4 on this path
-      unit_bytes[u] = static_cast<uint32_t>((static_cast<int64_t>(kb[u]) * 4 * ks + n) * 4);
-    }
+    tile_base = uniform_ptr((const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * 4));
+    // extent is a multiple of 8 on this path: a chunk past it is clamped onto the last one
+    const int n = min(first_row + chunk(0, tid) * 4, extent - 4) - first_row;
+    chunk_bytes = static_cast<uint32_t>((static_cast<int64_t>(k_row(0, tid)) * ks + n) * 4);
   }
-
-  template <int PART, int R>
-  __device__ __forceinline__ void load_op(int kt, uint32_t /*lds_tile*/) {
-    if (!active(PART)) return;
-    const VECOPS_GLOBAL char* row = tile_base + (static_cast<int64_t>(kt) * 32 + R) * ks * 4;
-    const u32x4 v = *(const VECOPS_GLOBAL u32x4*)(uniform_ptr(row) + unit_bytes[PART]);
-    regs[PART][R][0] = v.x;
-    regs[PART][R][1] = v.y;
-    regs[PART][R][2] = v.z;
-    regs[PART][R][3] = v.w;
+  __device__ __forceinline__ uint32_t part_offset(int part) const {
+    return __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(part * K_ROWS_PER_PART * ks * 4));
+  }
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t k_tile_buffer(int kt) const {
+    return tile_buffer(tile_base + static_cast<int64_t>(kt) * 32 * ks * 4);
   }
   template <int PART>
   __device__ __forceinline__ void fetch_part(int kt) {
-    static_for<4>([&](auto cr) { load_op<PART, decltype(cr)::value>(kt, 0u); });
+    regs[PART] = __builtin_amdgcn_raw_buffer_load_b128(k_tile_buffer(kt), chunk_bytes, part_offset(PART), 0);
   }
   __device__ __forceinline__ void fetch_full(int kt) {
-    static_for<UNITS>([&](auto cu) { fetch_part<decltype(cu)::value>(kt); });
+    static_for<CHUNKS>([&](auto ci) { fetch_part<decltype(ci)::value>(kt); });
   }
   __device__ __forceinline__ void fetch_full_spare(Spare&, int) {}
   __device__ __forceinline__ void take_spare(const Spare&) {}
-
+  // Whole tile with bounds checks (the partial last K tile): rows k >= K and columns n >= N read as zero.
   __device__ __forceinline__ void fetch_checked(int kt) {
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-      if (!active(u)) continue;
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int k = kt * 32 + k_row(i, tid_);
+      uint32_t w[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int k = kt * 32 + kb[u] * 4 + r;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int n = first_row + n_local[u] + e;
-          regs[u][r][e] = (k < k_end && n < extent) ? __float_as_uint(reinterpret_cast<const float*>(base)[k * ks + n]) : 0u;
-        }
+      for (int e = 0; e < 4; ++e) {
+        const int n = first_row + chunk(i, tid_) * 4 + e;
+        w[e] = (k < k_end && n < extent) ? __float_as_uint(reinterpret_cast<const float*>(base)[k * ks + n]) : 0u;
       }
+      regs[i] = u32x4{w[0], w[1], w[2], w[3]};
     }
-  }
-
-  template <int PART, int E>
-  __device__ __forceinline__ void store_op(char* lds_tile) const {
-    if (!active(PART)) return;
-    const u32x4 out = {regs[PART][0][E], regs[PART][1][E], regs[PART][2][E], regs[PART][3][E]};
-    *reinterpret_cast<u32x4*>(lds_tile + lds_chunk_offset(n_local[PART] + E, kb[PART])) = out;
   }
   template <int PART>
   __device__ __forceinline__ void commit_part(char* lds_tile) const {
-    static_for<4>([&](auto ce) { store_op<PART, decltype(ce)::value>(lds_tile); });
+    *reinterpret_cast<u32x4*>(lds_tile + k_row(PART, tid_) * kPitch + chunk(PART, tid_) * 16) = regs[PART];
   }
   __device__ __forceinline__ void commit(char* lds_tile) const {
-    static_for<UNITS>([&](auto cu) { commit_part<decltype(cu)::value>(lds_tile); });
+    static_for<CHUNKS>([&](auto ci) { commit_part<decltype(ci)::value>(lds_tile); });
+  }
+  template <int PART, int OP>
+  __device__ __forceinline__ void store_op(char* lds_tile) const {
+    commit_part<PART>(lds_tile);
+  }
+  template <int PART, int OP>
+  __device__ __forceinline__ void load_op(int kt, uint32_t /*lds_tile*/) {
+    fetch_part<PART>(kt);
   }
 };
 
@@ -1373,15 +1368,13 @@ struct StagingOp {
 };
 
 // Which of the four k-steps of a K tile stores (and then refills) which staging
-// parts, and in what order.  Chunk parts (one LDS write, one refill) are dealt out
-// evenly, A's first; a transposing B stager has one or two heavy parts (four
-// writes, eight loads), which take k-steps 0 and 2 while A's chunks share the
-// others.
+// parts, and in what order.  A part is one LDS write and one refill; they are dealt
+// out evenly, A's first.
 //
 // LATE (loads that write LDS, under the loop of the 16x16 shapes, whose barrier stands in the middle of the K
 // tile): the loads are those of the tile after the next, into the stage the barrier has just freed, in phases
 // 4 and 5 = the two quarters of the K tile behind the barrier; a load has half a K tile and more to land.
-template <typename SA, typename SB, bool B_TRANSPOSING, bool LATE = false>
+template <typename SA, typename SB, bool LATE = false>
 struct StagingSchedule {
   static constexpr int PARTS_A = SA::kParts, PARTS_B = SB::kParts;
   static constexpr bool DMA = SA::kStoreOps == 0;  // loads that write LDS: all of them early, in k-steps 0 and 1
@@ -1389,15 +1382,12 @@ struct StagingSchedule {
   static constexpr int step_a(int part) {
     if constexpr (LATE) return 4 + part * 2 / (PARTS_A + PARTS_B);
     else if constexpr (DMA) return part * 2 / (PARTS_A + PARTS_B);
-    else if constexpr (!B_TRANSPOSING) return part * 4 / (PARTS_A + PARTS_B);
-    else if constexpr (PARTS_B == 2) return part * 2 < PARTS_A ? 1 : 3;
-    else return 1 + part * 3 / PARTS_A;
+    else return part * 4 / (PARTS_A + PARTS_B);
   }
   static constexpr int step_b(int part) {
     if constexpr (LATE) return 4 + (PARTS_A + part) * 2 / (PARTS_A + PARTS_B);
     else if constexpr (DMA) return (PARTS_A + part) * 2 / (PARTS_A + PARTS_B);
-    else if constexpr (!B_TRANSPOSING) return (PARTS_A + part) * 4 / (PARTS_A + PARTS_B);
-    else return part * 2;
+    else return (PARTS_A + part) * 4 / (PARTS_A + PARTS_B);
   }
   // number of operations of k-step `step`
   static constexpr int ops(int step) {
@@ -1436,6 +1426,7 @@ struct StagingSchedule {
 template <int WAVES_M, int WAVES_N, int WM, int WN, int LOAD_B>
 constexpr int kStageBytes() {
   const int bm = 32 * WAVES_M * WM, bn = 32 * WAVES_N * WN;
+  if (LOAD_B == LOAD_KN32) return bm * 128 + 32 * (bn * 4 + 32);  // 32 k rows of bn floats and 32 bytes
   return bm * 128 + (LOAD_B == LOAD_NTR ? 64 * (bn * 2 + 64) : bn * 128);  // LOAD_NTR_DMA: 64 rows of bn * 2 bytes
 }
 
@@ -1838,6 +1829,7 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
   //   ((4 ks + chunk) ^ row ^ row / 8) & 7 = lane_slot ^ (4 ks ^ 2 f) & 7: four bases by the constant's bits 1-2
   //   B as k rows: column block j lies (j & 1) * 32 bytes into the 64-byte group ((j >> 1) ^ swizzle)
   constexpr int PITCH_NTR = ntr_pitch<SRC, LOAD_B, BN, THREADS>();
+  constexpr int PITCH_KN32 = BN * 4 + 32;  // (LOAD_KN32: bytes between the k rows of the fp32 B tile)
   uint32_t base_a[2][4], base_b[2][4];
   if constexpr (M16) {
     const uint32_t lds0 = lds_address_of(lds);
@@ -1874,6 +1866,9 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
         int col_bytes = ((wn * FN + j) * 32 + (g & 1) * 16 + (s16 & 3) * 4) * 2;
         if constexpr (LOAD_B == LOAD_NTR_DMA) col_bytes ^= ((s16 >> 2) & 3) << 6;
         off_b[j] = BM * 128 + ((g >> 1) * 8 + (s16 >> 2)) * PITCH_NTR + col_bytes;
+      } else if constexpr (LOAD_B == LOAD_KN32) {
+        // one float per lane and matrix instruction: column lane % 32 of the block, k row e (+ 4 for the upper lanes)
+        off_b[j] = BM * 128 + 4 * (lane >> 5) * PITCH_KN32 + ((wn * FN + j) * 32 + (lane & 31)) * 4;
       } else {
         off_b[j] = BM * 128 + lds_chunk_offset((wn * FN + j) * 32 + frag_row, frag_chunk);
       }
@@ -1939,6 +1934,11 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
         const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * PITCH_NTR)));
         return u32x4{lo.x, lo.y, hi.x, hi.y};
       }
+    } else if constexpr (LOAD_B == LOAD_KN32) {
+      // k-step KS covers rows 8 KS .. + 7 of the tile: instruction e takes rows e and 4 + e
+      const char* at = lds + static_cast<int>(st) * STAGE_BYTES + off_b[F] + KS * 8 * PITCH_KN32;
+      return u32x4{*reinterpret_cast<const uint32_t*>(at), *reinterpret_cast<const uint32_t*>(at + PITCH_KN32),
+                   *reinterpret_cast<const uint32_t*>(at + 2 * PITCH_KN32), *reinterpret_cast<const uint32_t*>(at + 3 * PITCH_KN32)};
     } else if constexpr (M16) {
       constexpr int ST = decltype(st)::value;
       return *reinterpret_cast<const lds_u32x4*>(static_cast<uintptr_t>(base_b[ST][((4 * KS) ^ (2 * F)) >> 1 & 3] + F * 2048));
@@ -1964,7 +1964,7 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
 
   using SA = decltype(stager_a);
   using SB = decltype(stager_b);
-  using Sched = StagingSchedule<SA, SB, LOAD_B == LOAD_NVEC, M16 && load_is_dma(LOAD_A)>;
+  using Sched = StagingSchedule<SA, SB, M16 && load_is_dma(LOAD_A)>;
 
   // Start of the pipeline: tile 0 into the staging registers and, without waiting
   // for it, tile 1 into a spare set (position 1 is never the partial tile: one

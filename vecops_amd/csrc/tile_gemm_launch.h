@@ -97,8 +97,8 @@ hipError_t with_loaders(int mode, F&& f) {
   if (mode == MODE_KVEC) return pair(integral_constant<int, LOAD_KVEC>{}, integral_constant<int, LOAD_KVEC>{});
   if constexpr (SrcTraits<SRC>::kElemsPerChunk == 8) {  // 16-bit compute: B untransposed in LDS, transposing reads
     if (mode == MODE_NVEC_B) return pair(integral_constant<int, LOAD_KVEC>{}, integral_constant<int, LOAD_NTR>{});
-  } else if constexpr (SRC == SRC_F32) {                // 32-bit compute: transposed in registers
-    if (mode == MODE_NVEC_B) return pair(integral_constant<int, LOAD_KVEC>{}, integral_constant<int, LOAD_NVEC>{});
+  } else if constexpr (SRC == SRC_F32) {                // 32-bit compute: B untransposed in LDS, one 4-byte read per operand
+    if (mode == MODE_NVEC_B) return pair(integral_constant<int, LOAD_KVEC>{}, integral_constant<int, LOAD_KN32>{});
   }
   return pair(integral_constant<int, LOAD_GENERIC>{}, integral_constant<int, LOAD_GENERIC>{});
 }
