@@ -39,15 +39,15 @@ REPETITIONS = 7
 # scaled by 2.000 and WRITE by 1.000: what the same counters read for a 1 GiB device copy, `--only copy`).  Counters
 # cannot be read from inside this process: these are the figures of the named summaries, for exactly these workloads.
 RECORDED_TRAFFIC = {
-    "bf16": (int((98479.5 * 2.000 + 32768 * 1.000) * 1024), "profiles/tile_gemm_bf16_4096.md"),
-    "int8": (int((96559.0 * 2.000 + 88064 * 1.000) * 1024), "profiles/tile_gemm_int8_dequant_2048x4096x11008.md"),
-    "gemv_m1": (int((29650.0 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_stream_m1_4096x14336.md"),
-    "gemv_m4": (int((29760.0 * 2.000 + 128.1 * 1.000) * 1024), "profiles/skinny_w8a16_stream_m1_4096x14336.md"),
-    "gemv_m16": (int((30150.0 * 2.000 + 524.8 * 1.000) * 1024), "profiles/skinny_w8a16_stream_m1_4096x14336.md"),
-    "bf16_packed": (int((98468.3 * 2.000 + 32768 * 1.000) * 1024),
-                    "profiles/tile_gemm_packed_b_bf16_4096_int8_2048x4096x11008.md"),
-    "int8_packed": (int((138798.0 * 2.000 + 88064 * 1.000) * 1024),
-                    "profiles/tile_gemm_packed_b_bf16_4096_int8_2048x4096x11008.md"),
+    "bf16": (int((98503.0 * 2.000 + 32768 * 1.000) * 1024), "profiles/tile_gemm_bf16_4096.md"),
+    "int8": (int((55098.0 * 2.000 + 88095 * 1.000) * 1024), "profiles/tile_gemm_wide_i8_dequant_2048x4096x11008.md"),
+    "gemv_m1": (int((29647.0 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
+    "gemv_m4": (int((29761.0 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
+    "gemv_m16": (int((30145.0 * 2.000 + 448.0 * 1.000) * 1024), "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
+    "bf16_packed": (int((98473.0 * 2.000 + 32768 * 1.000) * 1024), "profiles/tile_gemm_packed_b_bf16_4096.md"),
+    "int8_packed": (int((55095.0 * 2.000 + 88108 * 1.000) * 1024),
+                    "profiles/tile_gemm_wide_i8_dequant_2048x4096x11008.md"),
+    "fp32_f32": (int((12360.0 * 2.000 + 4096 * 1.000) * 1024), "profiles/tile_gemm_f32_compute_1024.md"),
 }
 
 
@@ -91,7 +91,8 @@ def _kernel_label(plan, operands):
     loads = "16-byte loads" if plan.vector_a and plan.vector_b else "element loads"
     b = {0: "B K-contiguous", 1: "B as [K,N]", 2: "B strided"}[plan.b_layout]
     split = f", split-K {plan.split_k}" if plan.split_k > 1 else ""
-    return f"vecops_hip tile_gemm_kernel<{operands}> family {family}, {loads}, {b}{split}"
+    kernel = "tile_gemm_wide_i8_kernel" if family == "tile_256x352" else f"tile_gemm_kernel<{operands}>"
+    return f"vecops_hip {kernel} family {family}, {loads}, {b}{split}"
 
 
 def _roofline(bound, achieved, peak, unit, **extra):
@@ -196,7 +197,7 @@ def bench_fp32_gemm(dev, steps, warmup, compute):
             "us_per_step": t["wall_ms"] * 1e3, "dtype": "f32" if compute == "f32" else "f32 memory, bf16 compute",
             "roofline": _roofline("mfma", tflops, peak, "TFLOP/s", kernel=_kernel_label(plan, "f32" if compute == "f32" else "f32 as bf16"),
                                   algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=3 * 4 * n * n,
-                                  traffic=None, **_timing_fields(t))}
+                                  **(_traffic("fp32_f32") if compute == "f32" else {"traffic": None}), **_timing_fields(t))}
 
 
 def bench_batched(dev, steps, warmup, m, n, k):
@@ -366,7 +367,9 @@ def bench_int8_dequant_packed(dev, steps, warmup):
             "(not timed), per-token x per-channel dequant fused, fp32 out", "value": tops, "unit": "TOP/s",
             "ms_per_step": t["wall_ms"], "dtype": "int8",
             "roofline": _roofline("mfma", tops, PEAK_INT8_TOPS, "TOP/s",
-                                  kernel=f"vecops_hip tile_gemm_packed_b_kernel<int8> family {family}, dequantising epilogue",
+                                  kernel=("vecops_hip tile_gemm_wide_i8_kernel<packed B>" if family == "tile_256x352"
+                                          else "vecops_hip tile_gemm_packed_b_kernel<int8>")
+                                  + f" family {family}, dequantising epilogue",
                                   algorithmic_ops_per_launch=ops,
                                   algorithmic_bytes_per_launch=m * k + n * k + 4 * m * n + 4 * (m + n),
                                   **_traffic("int8_packed"), **_timing_fields(t))}
@@ -393,6 +396,26 @@ def bench_gemv(dev, steps, warmup, m=1):
             "unit": "GB/s", "us_per_step": t["wall_ms"] * 1e3, "dtype": "int8 x bf16 -> f32",
             "roofline": _roofline("hbm", gbps, PEAK_HBM_GBPS, "GB/s", kernel=kernel, algorithmic_bytes_per_launch=nbytes,
                                   **_traffic(f"gemv_m{m}"), **_timing_fields(t))}
+
+
+def bench_read_ceiling(dev, steps, warmup):
+    """The read-only yardstick on the GEMV's bytes: the 58.7 MB of one weight matrix, rotated through the same eight
+    buffers, streamed by a kernel that does nothing else.  `value` is the best of a few grid sizes."""
+    import torch
+    from vecops_amd import capi, synth
+    k, n, copies = 4096, 14336, 8
+    w0 = torch.from_numpy(synth.int8_sym(2, (n, k))).to(dev)
+    ws = [w0] + [torch.roll(w0, shifts=i, dims=0) for i in range(1, copies)]
+    out = torch.empty(8192 * 256, dtype=torch.int32, device=dev)
+    by_grid = {}
+    for workgroups in (512, 1024, 2048, 4096):
+        t = _measure(lambda i: capi.read_stream(ws[i % copies], workgroups, out), max(steps, 200), warmup)
+        by_grid[workgroups] = {"us": t["event_ms"] * 1e3, "gbps": n * k / (t["event_ms"] * 1e-3) / 1e9}
+    best = max(by_grid, key=lambda g: by_grid[g]["gbps"])
+    return {"metric": "hbm_read_ceiling_gbps", "workload": f"read-only stream of {n * k} bytes (the GEMV's weights), "
+            "rotated through 8 buffers, launched back to back", "value": by_grid[best]["gbps"], "unit": "GB/s",
+            "us_per_launch": by_grid[best]["us"], "workgroups": best, "by_workgroups": by_grid, "peak": PEAK_HBM_GBPS,
+            "frac_of_peak": by_grid[best]["gbps"] / PEAK_HBM_GBPS}
 
 
 def bench_tile_families(dev, steps, warmup):
@@ -547,8 +570,8 @@ def cpu_baseline(a, b_kn):
     return out
 
 
-ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "fp32", "batched",
-        "families", "grouped", "rule_check"]
+ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "read_ceiling",
+        "fp32", "batched", "families", "grouped", "rule_check"]
 
 
 def main() -> int:
@@ -588,6 +611,7 @@ def main() -> int:
         "runtime_quant": lambda: bench_runtime_quant(dev, K, W),
         "gemv": lambda: bench_gemv(dev, K, W, m=args.gemv_m),
         "mfma_ceiling": lambda: bench_mfma_ceiling(dev, K, W, args.ceiling_dtype),
+        "read_ceiling": lambda: bench_read_ceiling(dev, K, W),
         "fp32": lambda: bench_fp32_gemm(dev, K, W, args.fp32_compute),
         "batched": lambda: bench_batched(dev, K, W, *[int(v) for v in args.batched_shape.split(",")]),
         "families": lambda: bench_tile_families(dev, K, W),
@@ -620,11 +644,16 @@ def main() -> int:
         roofline["frac_of_ceiling"] = roofline["achieved"] / ceiling_bf16["value"]
         int8 = bench_int8_dequant(dev, K, W, ceiling=ceiling_int8["value"])
         gemv = {m: bench_gemv(dev, K, W, m=m) for m in (1, 4, 16)}
+        read_ceiling = bench_read_ceiling(dev, K, W)
+        for r in gemv.values():   # what a kernel that only reads the weights sustains on the same buffers
+            r["roofline"]["measured_read_ceiling"] = read_ceiling["value"]
+            r["roofline"]["frac_of_read_ceiling"] = r["roofline"]["achieved"] / read_ceiling["value"]
         fp32 = {c: bench_fp32_gemm(dev, K, W, c) for c in ("bf16", "f32")}
         packed16, packed8 = bench_bf16_gemm_packed(dev, K, W), bench_int8_dequant_packed(dev, K, W)
         secondary = [bench_batched(dev, K, W, m, n, k)
                      for (m, n, k) in [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)]]
-        secondary += [bench_runtime_quant(dev, K, W), bench_grouped(dev, K, W), ceiling_bf16, ceiling_int8, packed16, packed8,
+        secondary += [bench_runtime_quant(dev, K, W), bench_grouped(dev, K, W), ceiling_bf16, ceiling_int8, read_ceiling, packed16,
+                      packed8,
                       fp32["bf16"], fp32["f32"], gemv[16], gemv[4], gemv[1], int8]
 
         def brief(r):
@@ -634,7 +663,8 @@ def main() -> int:
         # records are in `secondary`
         roofline["also"] = {"int8_cfg4": brief(int8), "int8_cfg4_prepacked": brief(packed8), "gemv_m1": brief(gemv[1]),
                             "gemv_m4": brief(gemv[4]), "gemv_m16": brief(gemv[16]), "fp32_1024_f32_compute": brief(fp32["f32"]),
-                            "fp32_1024_bf16_compute": brief(fp32["bf16"]), "bf16_4096_prepacked": brief(packed16)}
+                            "fp32_1024_bf16_compute": brief(fp32["bf16"]), "bf16_4096_prepacked": brief(packed16),
+                            "hbm_read_ceiling_gbps": round(read_ceiling["value"], 1)}
     # (the long list first: a reader who sees only the end of the line sees the headline and its roofline)
     line = {}
     if secondary is not None:

@@ -506,6 +506,14 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_mfma_stream_shape(uint32_t dtype, uint32_t 
                                                        uint64_t operand_bytes, int32_t workgroups, int32_t iters, void* out,
                                                        void* stream);
 
+/*
+ * Read-only yardstick of the skinny (HBM-bound) kernels, no counterpart in vecops: `workgroups` workgroups of 256 lanes
+ * stream the first bytes / 16 16-byte pieces of `src` (16-byte aligned) with eight loads in flight per lane and write
+ * one word per lane to `out` (workgroups x 256 words).  Launched back to back on a buffer of a GEMV's size it shows the
+ * rate at which this machine delivers that many bytes to any kernel, launch and ramp included.
+ */
+VECOPS_HIP_EXPORT int32_t vecops_hip_read_stream(const void* src, uint64_t bytes, int32_t workgroups, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -29,7 +29,7 @@ EXPORTS = [
     "vecops_hip_matmul_runtime_quant_packed_b_workspace", "vecops_hip_matmul_runtime_quant_packed_b",
     "vecops_hip_static_workspace_bytes", "vecops_hip_matmul_static_workspace",
     "vecops_hip_mfma_stream_ops", "vecops_hip_mfma_stream",
-    "vecops_hip_mfma_stream_shape_ops", "vecops_hip_mfma_stream_shape",
+    "vecops_hip_mfma_stream_shape_ops", "vecops_hip_mfma_stream_shape", "vecops_hip_read_stream",
     "vecops_hip_plan_matmul_family", "vecops_hip_matmul_family",
     "vecops_hip_matmul_runtime_quant_batched_workspace", "vecops_hip_matmul_runtime_quant_batched",
     "vecops_hip_matmul_grouped_workspace", "vecops_hip_matmul_grouped",
@@ -112,6 +112,7 @@ def lib() -> C.CDLL:
         L.vecops_hip_mfma_stream_shape_ops.argtypes = [C.c_uint32, C.c_uint32, C.c_int32, C.c_int32]
         L.vecops_hip_mfma_stream_shape.argtypes = [C.c_uint32, C.c_uint32, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32,
                                                    C.c_void_p, C.c_void_p]
+        L.vecops_hip_read_stream.argtypes = [C.c_void_p, C.c_uint64, C.c_int32, C.c_void_p, C.c_void_p]
         L.vecops_hip_matmul_static_workspace.argtypes = [P, P, P, P, C.c_uint32, C.c_void_p]
         L.vecops_hip_matmul_i8_dequant.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p,
                                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
@@ -309,6 +310,13 @@ def mfma_stream(operands, workgroups: int, iters: int, out, stream=None, shape: 
     _check(lib().vecops_hip_mfma_stream_shape(code, shape, operands.data_ptr(), operands.numel() * operands.element_size(),
                                               workgroups, iters, out.data_ptr(), _stream_handle(stream)))
     return lib().vecops_hip_mfma_stream_shape_ops(code, shape, workgroups, iters)
+
+
+def read_stream(src, workgroups: int, out, stream=None) -> int:
+    """Launches the read-only yardstick over the bytes of `src`; returns the bytes one launch reads."""
+    nbytes = src.numel() * src.element_size() // 16 * 16
+    _check(lib().vecops_hip_read_stream(src.data_ptr(), nbytes, workgroups, out.data_ptr(), _stream_handle(stream)))
+    return nbytes
 
 
 def epilogue(activation=None, scale=None, shift=None, row_scales=None, column_scales=None, clamp=(0.0, 0.0)) -> Epilogue:

@@ -68,6 +68,24 @@ __global__ __launch_bounds__(256) void mfma_stream_kernel(const u32x4* __restric
 }
 
 // The same stream on the 16x16 shapes: 4 x 4 accumulator quads per wavefront, the fragment sets used alternately.
+// The 32 instructions of a trip are ONE asm statement whose accumulators are tied operands in the accumulation
+// registers: written with the builtins the loop came out with three register copies per matrix instruction
+// (a new accumulator on every trip, copied back at the loop's head) and measured 30 % below the pipe's rate.
+#define VECOPS_Y16(INSTR, i, j, s) INSTR " %[c" #i #j "], %[b" #s #j "], %[a" #s #i "], %[c" #i #j "]\n\t"
+#define VECOPS_Y16_ROW(INSTR, i, s) \
+  VECOPS_Y16(INSTR, i, 0, s) VECOPS_Y16(INSTR, i, 1, s) VECOPS_Y16(INSTR, i, 2, s) VECOPS_Y16(INSTR, i, 3, s)
+#define VECOPS_Y16_SET(INSTR, s) \
+  VECOPS_Y16_ROW(INSTR, 0, s) VECOPS_Y16_ROW(INSTR, 1, s) VECOPS_Y16_ROW(INSTR, 2, s) VECOPS_Y16_ROW(INSTR, 3, s)
+#define VECOPS_Y16_ACC(i) \
+  [c##i##0] "+a"(acc[i][0]), [c##i##1] "+a"(acc[i][1]), [c##i##2] "+a"(acc[i][2]), [c##i##3] "+a"(acc[i][3])
+#define VECOPS_Y16_FRAGS(s)                                                                                   \
+  [a##s##0] "v"(a[s][0]), [a##s##1] "v"(a[s][1]), [a##s##2] "v"(a[s][2]), [a##s##3] "v"(a[s][3]),          \
+  [b##s##0] "v"(b[s][0]), [b##s##1] "v"(b[s][1]), [b##s##2] "v"(b[s][2]), [b##s##3] "v"(b[s][3])
+#define VECOPS_Y16_TRIP(INSTR)                                                                               \
+  asm volatile(VECOPS_Y16_SET(INSTR, 0) VECOPS_Y16_SET(INSTR, 1)                                             \
+               : VECOPS_Y16_ACC(0), VECOPS_Y16_ACC(1), VECOPS_Y16_ACC(2), VECOPS_Y16_ACC(3)                  \
+               : VECOPS_Y16_FRAGS(0), VECOPS_Y16_FRAGS(1))
+
 template <bool INT>
 __global__ __launch_bounds__(256) void mfma_stream16_kernel(const u32x4* __restrict__ operands, uint32_t chunks,
                                                            int iters, uint32_t* __restrict__ out) {
@@ -90,20 +108,10 @@ __global__ __launch_bounds__(256) void mfma_stream16_kernel(const u32x4* __restr
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0;
   for (int it = 0; it < iters; ++it) {
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if constexpr (INT)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, b[s][j]),
-                                                              __builtin_bit_cast(i32x4, a[s][i]), acc[i][j], 0, 0, 0);
-          else
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, b[s][j]),
-                                                                __builtin_bit_cast(bf16x8, a[s][i]), acc[i][j], 0, 0, 0);
-        }
+    if constexpr (INT) VECOPS_Y16_TRIP("v_mfma_i32_16x16x64_i8");
+    else VECOPS_Y16_TRIP("v_mfma_f32_16x16x32_bf16");
   }
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the last results are in their registers before they are read
   uint32_t folded = 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -115,6 +123,26 @@ __global__ __launch_bounds__(256) void mfma_stream16_kernel(const u32x4* __restr
         else folded += __float_as_uint(acc[i][j][e]);
       }
   out[tid] = folded;
+}
+
+// Read-only yardstick of the skinny kernels: every workgroup streams its share of `chunks` 16-byte pieces with eight
+// loads in flight per lane and folds them into one word per lane.  Nothing is computed and 1 KiB per workgroup is
+// written: what it sustains on a buffer of the GEMV's size is the rate at which this machine delivers that many bytes
+// to a kernel launched back to back, launch and ramp included.
+__global__ __launch_bounds__(256) void read_stream_kernel(const u32x4* __restrict__ src, uint64_t chunks,
+                                                         uint32_t* __restrict__ out) {
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * 256u;
+  uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+  u32x4 f = {0u, 0u, 0u, 0u};
+  for (; i + 7 * stride < chunks; i += 8 * stride) {
+    u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) f ^= v[u];
+  }
+  for (; i < chunks; i += stride) f ^= __builtin_nontemporal_load(src + i);
+  out[blockIdx.x * 256u + threadIdx.x] = f.x ^ f.y ^ f.z ^ f.w;
 }
 
 }  // namespace
@@ -164,6 +192,14 @@ int32_t vecops_hip_mfma_stream(uint32_t dtype, const void* operands, uint64_t op
   else
     hipLaunchKernelGGL(mfma_stream_kernel<false>, dim3(workgroups), dim3(256), 0, s, static_cast<const u32x4*>(operands),
                        chunks, iters, static_cast<uint32_t*>(out));
+  return hipGetLastError() == hipSuccess ? 0 : 6;
+}
+
+int32_t vecops_hip_read_stream(const void* src, uint64_t bytes, int32_t workgroups, void* out, void* stream) {
+  if (src == nullptr || out == nullptr || bytes < 16 || workgroups <= 0 || (reinterpret_cast<uintptr_t>(src) & 15u) != 0)
+    return 1;
+  hipLaunchKernelGGL(read_stream_kernel, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const u32x4*>(src), bytes / 16, static_cast<uint32_t*>(out));
   return hipGetLastError() == hipSuccess ? 0 : 6;
 }
 
