@@ -201,11 +201,13 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_matmul_static_workspace(const VecopsHipOper
  * same) and everything else batch by batch; this entry point is the form for batches that share nothing, not even
  * their shapes.  a, b, c (and c_in, which may be null; an entry of rank 0 means "no C input for this group") are
  * arrays of count descriptors obeying the rules of vecops_hip_matmul group by group.  Groups of one operand
- * class - bf16, f16, int8 x int8, or fp32 in either compute type - run as ONE launch over a table of problem
- * records (written into the workspace by small kernels fed through their arguments: no host buffer has to outlive
- * the call, nothing is allocated); unsigned 8-bit and fp64 operands, a mix of classes, groups with K = 0 and groups
- * whose K vecops_hip_matmul would split (few output tiles, long K: they run that call's plan, partial sums behind
- * the table) run as launches of their own on the same stream.  Results
+ * class - bf16, f16, int8 x int8, 8-bit integers with an unsigned side, or fp32 in either compute type - run as ONE
+ * launch over a table of problem records (written into the workspace by small kernels fed through their arguments: no
+ * host buffer has to outlive the call, nothing is allocated; the row-sum terms of unsigned sides are computed group by
+ * group into the workspace first); fp64 operands, a mix of classes (signed x signed bytes beside groups with an
+ * unsigned side count as a mix), groups with K = 0 and groups whose K vecops_hip_matmul would split (few output tiles,
+ * long K: they run that call's plan, partial sums behind the table) run as launches of their own on the same stream.
+ * Results
  * are those of vecops_hip_matmul on each group (bit-equal when that call runs the same tile shape without splitting K -
  * except 16-bit products with K <= 256 on 128 x 128 tiles, where the single call takes the other MFMA shape; otherwise equal up to the order of the fp32 sums - integer results are always the same bits).  workspace: vecops_hip_matmul_grouped_workspace bytes, 16-byte aligned.
  */
@@ -412,6 +414,14 @@ VECOPS_HIP_EXPORT uint64_t vecops_hip_packed_b_bytes(uint32_t packed_dtype, int6
  * (ops/MatmulPack.h:132-190). */
 VECOPS_HIP_EXPORT int32_t vecops_hip_pack_b(const VecopsHipOperand* b, void* packed, uint64_t packed_size,
                                             void* stream);
+/* The same with the packed dtype named by the caller: what vecops_hip_pack_b chooses (bf16 for a bf16 or f32 source,
+ * the source's own dtype otherwise), or 12 (f32) for an f32 source whose elements stay fp32 - the pack of the
+ * fp32-compute atom (ops::MatmulPack is generic over atoms, ops/MatmulPack.h:9-117; SME_F32F32,
+ * matmul/details/kernel/sme/Atoms.h): 4 elements per 16-byte chunk, the same 32-row panels; products against it
+ * (vecops_hip_matmul_packed_b / _packed_a / _packed_ab with packed dtype 12, an f32 dense operand, f32 c) multiply in
+ * fp32.  Serves either side. */
+VECOPS_HIP_EXPORT int32_t vecops_hip_pack_as(const VecopsHipOperand* b, uint32_t packed_dtype, void* packed,
+                                             uint64_t packed_size, void* stream);
 
 /* Packs an int8 b and also writes compensation[n] = -a_zero_point * sum_k b[n,k]
  * (wrapping int32), the C-input row that corrects an asymmetrically quantised
@@ -433,6 +443,7 @@ VECOPS_HIP_EXPORT int32_t vecops_hip_plan_matmul_packed_b(const VecopsHipOperand
  *   packed i8  : a i8 or u8 (AMX_I8I32<uint8_t, int8_t>, the atom the compensated pack serves,
  *                ops/MatmulPack.h:52-58; the workspace then also holds 4 * batch * (M + N) bytes), c i32
  *   packed u8  : a i8 or u8, c i32 (the same workspace term)
+ *   packed f32 : a f32, c f32, products in fp32 (vecops_hip_pack_as)
  * Integer results are those of vecops_hip_matmul on the unpacked operand, bit for bit; floating-point results too
  * when that call runs its 256-row or 256-column tiles with the same split of K (the packed kernels multiply on the
  * 32x32 matrix instructions, the small plain tiles on the 16x16 ones: the fp32 sums are then taken in another order).

@@ -39,8 +39,8 @@ typedef struct VecopsHostSpecialization {
 } VecopsHostSpecialization;
 
 /* operator_name: "vecops::matmul", "vecops::matmul_fused", "vecops::matmul_i8_dequant",
- * "vecops::matmul_runtime_quant", "vecops::matmul_pack_b", "vecops::matmul_packed_b" or
- * "vecops::matmul_w8a16_group".  Returns null for an unknown name. */
+ * "vecops::matmul_runtime_quant", "vecops::matmul_pack_b", "vecops::matmul_packed_b", "vecops::matmul_pack_a",
+ * "vecops::matmul_packed_a" or "vecops::matmul_w8a16_group".  Returns null for an unknown name. */
 VECOPS_HIP_HOST_EXPORT void* vecops_hip_host_operator_create(const char* operator_name, const char* artifact_directory);
 VECOPS_HIP_HOST_EXPORT void vecops_hip_host_operator_destroy(void* op);
 

@@ -192,9 +192,48 @@ def test_grouped_floating_classes_in_one_launch(device, oracle, kind):
         assert any(same_bits) or (kind != "f32" and k <= 256), (kind, i)
 
 
+def test_grouped_unsigned_sides_in_one_launch(device):
+    """Groups with an unsigned 8-bit side (AMX_I8I32<uint8_t, int8_t>, <int8_t, uint8_t>, <uint8_t, uint8_t>; the
+    reference's batch planner serves every atom alike, planning/families/ArchitectureFamily.h:430-463): one table,
+    every group with its own sign flips and row-sum terms in the workspace.  Exact sums mod 2^32, ragged shapes, a
+    C input on every other group, bytes of the full range; and the result of each group equals its single call's."""
+    import torch
+    from vecops_amd import capi
+
+    def raw(seed, shape, unsigned):
+        x = (synth.draws(seed, int(np.prod(shape))) % np.uint64(256)).astype(np.uint8).reshape(shape)
+        return x if unsigned else x.view(np.int8)
+    cases = [((70, 90, 200), True, False), ((300, 20, 64), True, True), ((1000, 1300, 136), False, True),
+             ((513, 257, 96), True, True), ((1, 33, 40), True, False), ((700, 900, 1100), False, True)]
+    ha, hb, hci, ta, tb, tc, tci = [], [], [], [], [], [], []
+    for i, ((m, n, k), au, bu) in enumerate(cases):
+        ha.append(raw(10 + i, (m, k), au))
+        hb.append(raw(50 + i, (n, k), bu))
+        hci.append(synth.int8_sym(90 + i, (m, n)).astype(np.int32) * 1000 if i % 2 else None)
+        ta.append(torch.from_numpy(ha[-1]).to(device))
+        tb.append(torch.from_numpy(hb[-1]).to(device))
+        tci.append(torch.from_numpy(hci[-1]).to(device) if hci[-1] is not None else None)
+        tc.append(torch.full((m, n), -1, dtype=torch.int32, device=device))
+    capi.matmul_grouped(ta, tb, tc, c_in_list=tci)
+    torch.cuda.synchronize()
+    for i in range(len(cases)):
+        want = ha[i].astype(np.int64) @ hb[i].astype(np.int64).T + (hci[i] if hci[i] is not None else 0)
+        assert np.array_equal(tc[i].cpu().numpy(), (want & 0xffffffff).astype(np.uint32).view(np.int32)), cases[i]
+        alone = torch.full_like(tc[i], -1)
+        capi.matmul(ta[i], tb[i], alone, c_in=tci[i])
+        torch.cuda.synchronize()
+        assert torch.equal(alone, tc[i])
+    # too small a workspace is refused before anything runs
+    Operands = capi.Operand * len(cases)
+    oa, ob, oc = (Operands(*map(capi.operand, xs)) for xs in (ta, tb, tc))
+    need = capi.lib().vecops_hip_matmul_grouped_workspace(len(cases), oa, ob, None, oc, 0)
+    assert need >= sum(4 * (m + n) for (m, n, _), _, _ in cases)
+    ws = torch.empty(need, dtype=torch.uint8, device=device)
+    assert capi.lib().vecops_hip_matmul_grouped(len(cases), oa, ob, None, oc, 0, ws.data_ptr(), need - 256, None) == 1
+
+
 def test_grouped_other_classes_run_group_by_group(device, oracle):
-    """Unsigned 8-bit operands (their sign flip needs a pass of its own) and a mix of classes: the same entry point,
-    launches of their own."""
+    """Two unsigned-side groups, then a mix of classes (launches of their own): the same entry point."""
     import torch
     from vecops_amd import capi
     def u8(seed, shape):

@@ -115,7 +115,7 @@ def test_host_library_exports_every_declared_symbol(host):
 
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
-    assert len(files) == 64   # 40 + (6 required families x {bf16, i8} x {host, device})
+    assert len(files) == 94   # 40 + (6 required families x {bf16, i8} + 15 unsigned-weight, side-A and fp32-pack kinds) x {host, device}
     for f in files:
         name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
         assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
@@ -289,9 +289,11 @@ def test_packed_b_operators_resolution_and_validation(host):
         assert e.value.code == 1 and needle in e.value.message, (needle, e.value.message)
     assert pack.resolve(pf(np.zeros((5, 8), np.float16), 0, packed, None)) == \
         "vecops::matmul_pack_b;operands=f16;memory=host;backend=hip-gfx950"        # half operands: a recipe of their own
-    with pytest.raises(H.HostError) as e:                  # unsigned weights have no recipe in the host layer
-        pack.resolve(pf(np.zeros((5, 8), np.uint8), 0, packed, None))
-    assert e.value.code in (1, 2, 3)
+    assert pack.resolve(pf(np.zeros((5, 8), np.uint8), 0, packed, None)) == \
+        "vecops::matmul_pack_b;operands=u8;memory=host;backend=hip-gfx950"         # unsigned weights (AMX_I8I32<.., uint8_t>)
+    with pytest.raises(H.HostError) as e:                  # the compensated pack is the signed-weights atom's
+        pack.resolve(pf(np.zeros((5, 8), np.uint8), 3, packed, comp))
+    assert e.value.code == 1 and "int8" in e.value.message
 
     mul = host.operator("vecops::matmul_packed_b")
     mf = lambda a, cin, c: H.Frame([a, packed, cin, c], outputs=(3,))  # noqa: E731
@@ -317,6 +319,84 @@ def test_packed_b_operators_resolution_and_validation(host):
     # a packed tensor that is too small for N x K is refused by the artifact's workspace query
     with pytest.raises(H.HostError) as e:
         mul.workspace(H.Frame([bf16((4, 8)), np.zeros(16, np.uint8), None, c], outputs=(3,)))
+    assert e.value.code == 1 and "bytes" in e.value.message
+    # unsigned packed weights: the PackedType specialization value names what the opaque bytes hold
+    i32 = np.zeros((4, 5), np.int32)
+    u8 = {"PackedType": ("dtype", H.U8)}
+    assert mul.resolve(mf(np.zeros((4, 8), np.int8), None, i32), u8) == \
+        "vecops::matmul_packed_b;operands=i8;packed=u8;memory=host;backend=hip-gfx950"
+    assert "packed=u8" in mul.resolve(mf(np.zeros((4, 8), np.uint8), None, i32), u8)
+    assert "packed=" not in mul.resolve(mf(np.zeros((4, 8), np.int8), None, i32), {"PackedType": ("dtype", H.I8)})
+    for fr, spec, needle in [(mf(bf16((4, 8)), None, c), u8, "8-bit"),
+                             (mf(np.zeros((4, 8), np.int8), None, i32), {"PackedType": 3}, "DType")]:
+        with pytest.raises(H.HostError) as e:
+            mul.resolve(fr, spec)
+        assert e.value.code == 1 and needle in e.value.message, (needle, e.value.message)
+
+
+def test_fp32_compute_pack_resolution(host):
+    """The pack of the fp32-compute atom (ops::MatmulPack over SME_F32F32): ComputeType = Float32 on the pack keeps an
+    fp32 source's elements fp32, and on the product selects the recipe that multiplies in fp32; either side."""
+    f32 = {"ComputeType": ("dtype", H.F32)}
+    packed = np.zeros(4096, np.uint8)
+    src = np.zeros((5, 8), np.float32)
+    pack_b, pack_a = host.operator("vecops::matmul_pack_b"), host.operator("vecops::matmul_pack_a")
+    assert pack_b.resolve(H.Frame([src, 0, packed, None], outputs=(2,)), f32) == \
+        "vecops::matmul_pack_b;operands=f32;memory=host;backend=hip-gfx950"
+    assert "operands=bf16" in pack_b.resolve(H.Frame([src, 0, packed, None], outputs=(2,)))
+    assert "operands=bf16" in pack_b.resolve(H.Frame([src, 0, packed, None], outputs=(2,)), {"ComputeType": ("dtype", H.BF16)})
+    assert pack_a.resolve(H.Frame([src, packed], outputs=(1,)), f32) == \
+        "vecops::matmul_pack_a;operands=f32;memory=host;backend=hip-gfx950"
+    assert "operands=bf16" in pack_b.resolve(H.Frame([bf16((5, 8)), 0, packed, None], outputs=(2,)), f32)   # bf16 stays bf16
+    c = np.zeros((4, 5), np.float32)
+    mul_b, mul_a = host.operator("vecops::matmul_packed_b"), host.operator("vecops::matmul_packed_a")
+    assert mul_b.resolve(H.Frame([np.zeros((4, 8), np.float32), packed, None, c], outputs=(3,)), f32) == \
+        "vecops::matmul_packed_b;operands=f32;compute=f32;memory=host;backend=hip-gfx950"
+    assert mul_b.resolve(H.Frame([np.zeros((4, 8), np.float32), packed, None, c], outputs=(3,))) == \
+        "vecops::matmul_packed_b;operands=f32;memory=host;backend=hip-gfx950"              # fp32 rows against a bf16 pack
+    assert mul_a.resolve(H.Frame([packed, np.zeros((5, 8), np.float32), c, c], outputs=(3,)), f32) == \
+        "vecops::matmul_packed_a;operands=f32;compute=f32;memory=host;backend=hip-gfx950"
+    with pytest.raises(H.HostError) as e:                  # fp32 products leave as fp32
+        mul_b.resolve(H.Frame([np.zeros((4, 8), np.float32), packed, None, bf16((4, 5))], outputs=(3,)), f32)
+    assert e.value.code in (2, 3)
+
+
+def test_packed_a_operators_resolution_and_validation(host):
+    """vecops::matmul_pack_a / vecops::matmul_packed_a (ops::matmul_pack with Operand::A, ops/MatmulPack.h:81-96):
+    the packed operand comes first, M is taken from c and K from b; every class of the B side has its mirror."""
+    pack = host.operator("vecops::matmul_pack_a")
+    packed = np.zeros(4096, np.uint8)
+    pf = lambda a: H.Frame([a, packed], outputs=(1,))  # noqa: E731
+    for src, name in [(bf16((5, 8)), "bf16"), (np.zeros((5, 8), np.float32), "bf16"), (np.zeros((5, 8), np.float16), "f16"),
+                      (np.zeros((5, 8), np.int8), "i8"), (np.zeros((5, 8), np.uint8), "u8")]:
+        assert pack.resolve(pf(src)) == f"vecops::matmul_pack_a;operands={name};memory=host;backend=hip-gfx950"
+    with pytest.raises(H.HostError) as e:
+        pack.resolve(pf(np.zeros((5, 8), np.int32)))
+    assert e.value.code in (1, 2, 3)
+
+    mul = host.operator("vecops::matmul_packed_a")
+    mf = lambda b, cin, c: H.Frame([packed, b, cin, c], outputs=(3,))  # noqa: E731
+    c = np.zeros((4, 5), np.float32)
+    key = "vecops::matmul_packed_a;operands={};memory=host;backend=hip-gfx950"
+    assert mul.resolve(mf(bf16((5, 8)), None, c)) == key.format("bf16")
+    assert mul.resolve(mf(bf16((2, 5, 8)), None, bf16((2, 4, 5)))) == key.format("bf16")   # one packed a, every batch of b
+    assert mul.resolve(mf(np.zeros((5, 8), np.float32), c, c)) == key.format("f32")
+    assert mul.resolve(mf(np.zeros((5, 8), np.float16), None, np.zeros((4, 5), np.float16))) == key.format("f16")
+    i32 = np.zeros((4, 5), np.int32)
+    assert mul.resolve(mf(np.zeros((5, 8), np.int8), None, i32)) == key.format("i8")
+    assert mul.resolve(mf(np.zeros((5, 8), np.uint8), None, i32)) == key.format("i8")       # s8-packed a x u8 b
+    assert mul.resolve(mf(np.zeros((5, 8), np.int8), None, i32), {"PackedType": ("dtype", H.U8)}) == key.format("i8;packed=u8")
+    for fr, needle in [(mf(bf16((5, 8)), None, np.zeros((4, 6), np.float32)), "[.., M, N]"),
+                       (mf(bf16((2, 5, 8)), None, np.zeros((3, 4, 5), np.float32)), "batch"),
+                       (mf(bf16((5, 8)), np.zeros((3, 5), np.float32), c), "c_in")]:
+        with pytest.raises(H.HostError) as e:
+            mul.resolve(fr)
+        assert e.value.code == 1 and needle in e.value.message, (needle, e.value.message)
+    with pytest.raises(H.HostError) as e:                  # int32 sums do not leave as fp32 here
+        mul.resolve(mf(np.zeros((5, 8), np.int8), None, c))
+    assert e.value.code in (2, 3)
+    with pytest.raises(H.HostError) as e:                  # too small for M x K
+        mul.workspace(H.Frame([np.zeros(16, np.uint8), bf16((5, 8)), None, c], outputs=(3,)))
     assert e.value.code == 1 and "bytes" in e.value.message
 
 

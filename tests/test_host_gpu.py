@@ -395,3 +395,145 @@ def test_mixed_placement_is_refused(host, device):
     with pytest.raises(H.HostError) as e:
         op.invoke(H.Frame([a, tb, None, np.zeros((4, 5), np.float32)], outputs=(3,)))
     assert e.value.code in (2, 3)
+
+
+def _conversion_value(count, seed, unsigned):
+    """tests/ops/MatmulConversionTestCommon.h:62-70 for the integral types: the operands of the reference's tests."""
+    low = 0 if unsigned else -3
+    return (low + (np.arange(count, dtype=np.int64) * 5 + seed) % 7).astype(np.uint8 if unsigned else np.int8)
+
+
+@pytest.mark.parametrize("a_unsigned,b_unsigned", [(False, False), (False, True), (True, False), (True, True)])
+def test_mixed_packing_case_through_the_operators(host, a_unsigned, b_unsigned):
+    """tests/ops/MatmulMixedPackingTest.cpp:24-28 through the Operator surface: the reference's own 19 x 21 x 65 case with
+    its conversion_value operands, for each signedness, with A packed (vecops::matmul_pack_a / matmul_packed_a) and
+    with B packed (vecops::matmul_pack_b / matmul_packed_b); a packed operand of unsigned bytes is announced by the
+    PackedType specialization value.  Exact int32 sums."""
+    from vecops_amd import capi
+    m, n, k = 19, 21, 65
+    a = _conversion_value(m * k, 3, a_unsigned).reshape(m, k)
+    b = _conversion_value(n * k, 11, b_unsigned).reshape(n, k)
+    want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.int32)
+    u8 = {"PackedType": ("dtype", H.U8)}
+    # B packed
+    packed_b = np.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.U8 if b_unsigned else capi.I8, n, k), np.uint8)
+    frame = H.Frame([b, 0, packed_b, None], outputs=(2,))
+    pack_b = host.operator("vecops::matmul_pack_b")
+    assert f"operands={'u8' if b_unsigned else 'i8'};" in pack_b.resolve(frame)
+    pack_b.invoke(frame)
+    c = np.full((m, n), -1, np.int32)
+    mul_b = host.operator("vecops::matmul_packed_b")
+    frame = H.Frame([a, packed_b, None, c], outputs=(3,))
+    assert ("packed=u8" in mul_b.resolve(frame, u8 if b_unsigned else None)) == b_unsigned
+    mul_b.invoke(frame, u8 if b_unsigned else None)
+    assert np.array_equal(c, want)
+    # A packed
+    packed_a = np.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.U8 if a_unsigned else capi.I8, m, k), np.uint8)
+    frame = H.Frame([a, packed_a], outputs=(1,))
+    pack_a = host.operator("vecops::matmul_pack_a")
+    assert pack_a.resolve(frame) == f"vecops::matmul_pack_a;operands={'u8' if a_unsigned else 'i8'};memory=host;backend=hip-gfx950"
+    pack_a.invoke(frame)
+    c = np.full((m, n), -1, np.int32)
+    mul_a = host.operator("vecops::matmul_packed_a")
+    frame = H.Frame([packed_a, b, None, c], outputs=(3,))
+    assert ("packed=u8" in mul_a.resolve(frame, u8 if a_unsigned else None)) == a_unsigned
+    mul_a.invoke(frame, u8 if a_unsigned else None)
+    assert np.array_equal(c, want)
+    # with the wrong announcement the bytes are read as the other signedness: the sums differ by 128 * the row sums
+    if a_unsigned:
+        mul_a.invoke(frame)
+        assert np.array_equal(c, want - 128 * b.astype(np.int64).sum(axis=1)[None, :].astype(np.int32))
+
+
+def test_packed_a_operators(host, oracle, device):
+    """vecops::matmul_pack_a then vecops::matmul_packed_a on larger shapes: int8 bit for bit against vecops::matmul
+    (host tensors), bf16 from an fp32 source on device tensors with one packed a serving every batch of a rank-3 b and
+    a C-input, half operands to a half output; too small a packed buffer is an invalid argument."""
+    import torch
+    from vecops_amd import capi
+    pack, mul, plain = (host.operator("vecops::matmul_pack_a"), host.operator("vecops::matmul_packed_a"),
+                        host.operator("vecops::matmul"))
+    m, n, k = 129, 67, 515
+    a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
+    packed = np.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.I8, m, k), np.uint8)
+    pack.invoke(H.Frame([a, packed], outputs=(1,)))
+    want = np.zeros((m, n), np.int32)
+    plain.invoke(H.Frame([a, b, None, want], outputs=(3,)))
+    assert np.array_equal(want, (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.int32))
+    c = np.full((m, n), -1, np.int32)
+    mul.invoke(H.Frame([packed, b, None, c], outputs=(3,)))
+    assert np.array_equal(c, want)
+    cin = synth.int8_sym(3, (m, n)).astype(np.int32)
+    mul.invoke(H.Frame([packed, b, cin, c], outputs=(3,)))
+    assert np.array_equal(c, want + cin)
+    with pytest.raises(H.HostError) as e:
+        pack.invoke(H.Frame([a, np.zeros(16, np.uint8)], outputs=(1,)))
+    assert e.value.code == 1 and "bytes" in e.value.message
+    with pytest.raises(H.HostError) as e:
+        mul.invoke(H.Frame([packed[:64], b, None, c], outputs=(3,)))
+    assert e.value.code == 1
+    # bf16 packed from fp32, device tensors, rank-3 b
+    batch, m, n, k = 3, 200, 50, 1000
+    af = synth.uniform_pm1(1, (m, k))
+    b = synth.bf16_round(synth.uniform_pm1(2, (batch, n, k)))
+    taf = torch.from_numpy(af).to(device)
+    tb = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
+    tp = torch.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.BF16, m, k), dtype=torch.uint8, device=device)
+    frame = H.Frame([taf, tp], outputs=(1,))
+    assert pack.resolve(frame) == "vecops::matmul_pack_a;operands=bf16;memory=device;backend=hip-gfx950"
+    pack.invoke(frame)
+    cin = synth.uniform_pm1(4, (batch, m, n))
+    tcin = torch.from_numpy(cin).to(device)
+    tc = torch.full((batch, m, n), float("nan"), device=device)
+    frame = H.Frame([tp, tb, tcin, tc], outputs=(3,))
+    assert mul.resolve(frame) == "vecops::matmul_packed_a;operands=bf16;memory=device;backend=hip-gfx950"
+    need = mul.workspace(frame)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    mul.invoke(frame, workspace=ws.data_ptr(), workspace_size=need)
+    torch.cuda.synchronize()
+    wantf = np.zeros((batch, m, n), np.float32)
+    for i in range(batch):
+        oracle.matmul(synth.bf16_round(af), b[i], wantf[i], cin=cin[i], acc_f64=True, c_bf16=False)
+    assert rel_err(tc.cpu().numpy(), wantf) <= fp32_tol(k)
+    # half operands, host tensors, half output
+    m, n, k = 130, 70, 264
+    ah, bh = synth.uniform_pm1(5, (m, k)).astype(np.float16), synth.uniform_pm1(6, (n, k)).astype(np.float16)
+    packed = np.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.F16, m, k), np.uint8)
+    pack.invoke(H.Frame([ah, packed], outputs=(1,)))
+    ch = np.full((m, n), np.nan, np.float16)
+    frame = H.Frame([packed, bh, None, ch], outputs=(3,))
+    assert mul.resolve(frame) == "vecops::matmul_packed_a;operands=f16;memory=host;backend=hip-gfx950"
+    mul.invoke(frame)
+    wanth = ah.astype(np.float64) @ bh.astype(np.float64).T
+    assert rel_err(ch.astype(np.float64), wanth) <= 2e-3
+
+
+def test_fp32_compute_pack_through_the_operators(host, device):
+    """ComputeType = Float32 on the pack and on the product: fp32 operands packed as fp32 and multiplied in fp32, B
+    side on host tensors and A side on device tensors, against fp64 far inside what bf16 rounding would leave."""
+    import torch
+    from vecops_amd import capi
+    f32 = {"ComputeType": ("dtype", H.F32)}
+    m, n, k = 70, 130, 520
+    a, b = synth.uniform_pm1(1, (m, k)), synth.uniform_pm1(2, (n, k))
+    want = a.astype(np.float64) @ b.astype(np.float64).T
+    packed = np.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.F32, n, k), np.uint8)
+    host.operator("vecops::matmul_pack_b").invoke(H.Frame([b, 0, packed, None], outputs=(2,)), f32)
+    c = np.full((m, n), np.nan, np.float32)
+    host.operator("vecops::matmul_packed_b").invoke(H.Frame([a, packed, None, c], outputs=(3,)), f32)
+    assert rel_err(c, want) <= 1e-5
+    ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    tp = torch.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.F32, m, k), dtype=torch.uint8, device=device)
+    host.operator("vecops::matmul_pack_a").invoke(H.Frame([ta, tp], outputs=(1,)), f32)
+    tc = torch.full((m, n), float("nan"), device=device)
+    mul_a = host.operator("vecops::matmul_packed_a")
+    frame = H.Frame([tp, tb, None, tc], outputs=(3,))
+    need = mul_a.workspace(frame, f32)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    mul_a.invoke(frame, f32, workspace=ws.data_ptr(), workspace_size=need)
+    torch.cuda.synchronize()
+    assert rel_err(tc.cpu().numpy(), want) <= 1e-5
+    # the bf16 pack of the same source, for contrast: the rounding of the weights is visible
+    host.operator("vecops::matmul_pack_b").invoke(H.Frame([b, 0, packed, None], outputs=(2,)))
+    host.operator("vecops::matmul_packed_b").invoke(H.Frame([a, packed, None, c], outputs=(3,)))
+    assert rel_err(c, want) > 1e-4

@@ -31,8 +31,8 @@ def test_registration_is_idempotent_and_schemas_mark_outputs():
     with pytest.raises(AttributeError):
         tb.no_such_library
     ns = tb.register_all("vecops_hip_t")
-    assert sorted(vars(ns)) == ["matmul", "matmul_fused", "matmul_i8_dequant", "matmul_pack_b", "matmul_packed_b",
-                                "matmul_runtime_quant", "matmul_w8a16_group"]
+    assert sorted(vars(ns)) == ["matmul", "matmul_fused", "matmul_i8_dequant", "matmul_pack_a", "matmul_pack_b",
+                                "matmul_packed_a", "matmul_packed_b", "matmul_runtime_quant", "matmul_w8a16_group"]
     pack = str(torch.ops.vecops_hip_t.matmul_pack_b.default._schema)
     assert "int a_zero_point" in pack and "Tensor(a!) packed" in pack and "Tensor(b!)? compensation" in pack
     schema = str(torch.ops.vecops_hip_t.matmul.default._schema)
@@ -192,6 +192,28 @@ def test_torch_ops_packed_b(device):
     c3 = torch.zeros(m, n, device=device)
     capi.matmul_packed_b(af, capi.pack_b(bf), c3, c_in=cin)
     assert torch.equal(c1, c3)
+
+
+@pytest.mark.gpu
+def test_torch_ops_packed_a_and_unsigned_weights(device):
+    """Side A and unsigned weights through torch.ops: pack A once, multiply by dense B; pack uint8 weights and announce
+    them with PackedType - int32 sums exact against the plain operator."""
+    ns = tb.register_all("vecops_hip_t")
+    to = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(device)  # noqa: E731
+    m, n, k = 300, 70, 520
+    a, b = to(synth.int8_sym(1, (m, k))), to(synth.int8_sym(2, (n, k)))
+    packed = torch.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.I8, m, k), dtype=torch.uint8, device=device)
+    assert ns.matmul_pack_a(a, packed) is packed
+    c, want = (torch.zeros(m, n, dtype=torch.int32, device=device) for _ in range(2))
+    ns.matmul_packed_a(packed, b, None, c)
+    ns.matmul(a, b, None, want)
+    assert torch.equal(c, want)
+    ub = to((synth.int8_sym(3, (n, k)).astype(np.int16) + 128).astype(np.uint8))
+    pu = torch.zeros(capi.lib().vecops_hip_packed_b_bytes(capi.U8, n, k), dtype=torch.uint8, device=device)
+    ns.matmul_pack_b(ub, 0, pu, None)
+    ns.matmul_packed_b(a, pu, None, c, PackedType=torch.uint8)
+    ns.matmul(a, ub, None, want)
+    assert torch.equal(c, want)
 
 
 @pytest.mark.gpu

@@ -23,7 +23,7 @@ EXPORTS = [
     "vecops_hip_abi_version", "vecops_hip_last_error", "vecops_hip_device_count", "vecops_hip_plan_matmul",
     "vecops_hip_matmul", "vecops_hip_matmul_planned", "vecops_hip_matmul_i8_dequant", "vecops_hip_matmul_i8_dequant_workspace",
     "vecops_hip_matmul_w8a16_group", "vecops_hip_packed_b_bytes", "vecops_hip_pack_b", "vecops_hip_pack_b_compensated",
-    "vecops_hip_plan_matmul_packed_b", "vecops_hip_matmul_packed_b", "vecops_hip_matmul_i8_dequant_packed_b",
+    "vecops_hip_pack_as", "vecops_hip_plan_matmul_packed_b", "vecops_hip_matmul_packed_b", "vecops_hip_matmul_i8_dequant_packed_b",
     "vecops_hip_plan_matmul_fused", "vecops_hip_matmul_fused", "vecops_hip_quantize_rows",
     "vecops_hip_matmul_runtime_quant_workspace", "vecops_hip_matmul_runtime_quant",
     "vecops_hip_matmul_runtime_quant_packed_b_workspace", "vecops_hip_matmul_runtime_quant_packed_b",
@@ -126,6 +126,7 @@ def lib() -> C.CDLL:
         L.vecops_hip_packed_b_bytes.argtypes = [C.c_uint32, C.c_int64, C.c_int64]
         L.vecops_hip_pack_b.argtypes = [P, C.c_void_p, C.c_uint64, C.c_void_p]
         L.vecops_hip_pack_b_compensated.argtypes = [P, C.c_int32, C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]
+        L.vecops_hip_pack_as.argtypes = [P, C.c_uint32, C.c_void_p, C.c_uint64, C.c_void_p]
         L.vecops_hip_plan_matmul_packed_b.argtypes = [P, C.c_uint32, C.c_int64, P, P, C.POINTER(Plan)]
         L.vecops_hip_matmul_packed_b.argtypes = [P, C.c_void_p, C.c_uint32, C.c_int64, P, P, C.c_void_p, C.c_uint64,
                                                  C.c_void_p]
@@ -478,20 +479,22 @@ class PackedB:
         self.storage, self.dtype, self.n, self.k = storage, dtype, n, k
 
 
-def pack_b(b, a_zero_point=None, stream=None):
-    """Pack b ([N,K]; bf16, f32 or int8) once for any number of ``matmul_packed_b`` calls.
+def pack_b(b, a_zero_point=None, stream=None, compute: int = 0):
+    """Pack b ([N,K]; bf16, f16, f32, int8 or uint8) once for any number of ``matmul_packed_b`` calls.  An fp32 source
+    is rounded to bf16 unless ``compute`` is ``COMPUTE_F32``, which keeps fp32 elements (the fp32-compute atom).
 
     With ``a_zero_point`` (int8 b only) also returns the int32[N] compensation row
     ``-a_zero_point * sum_k b[n,k]`` (``ops::matmul_pack_b_compensated``).
     """
     import torch
     n, k = b.shape
-    dtype = I8 if b.dtype == torch.int8 else U8 if b.dtype == torch.uint8 else F16 if b.dtype == torch.float16 else BF16
+    dtype = (I8 if b.dtype == torch.int8 else U8 if b.dtype == torch.uint8 else F16 if b.dtype == torch.float16
+             else F32 if b.dtype == torch.float32 and compute == COMPUTE_F32 else BF16)
     size = lib().vecops_hip_packed_b_bytes(dtype, n, k)
     storage = torch.empty(max(size, 16), dtype=torch.uint8, device=b.device)
     ob = operand(b)
     if a_zero_point is None:
-        _check(lib().vecops_hip_pack_b(C.byref(ob), storage.data_ptr(), size, _stream_handle(stream)))
+        _check(lib().vecops_hip_pack_as(C.byref(ob), dtype, storage.data_ptr(), size, _stream_handle(stream)))
         return PackedB(storage, dtype, n, k)
     comp = torch.empty(n, dtype=torch.int32, device=b.device)
     _check(lib().vecops_hip_pack_b_compensated(C.byref(ob), a_zero_point, storage.data_ptr(), size, comp.data_ptr(),
@@ -499,9 +502,9 @@ def pack_b(b, a_zero_point=None, stream=None):
     return PackedB(storage, dtype, n, k), comp
 
 
-def pack_a(a, stream=None) -> PackedB:
+def pack_a(a, stream=None, compute: int = 0) -> PackedB:
     """Pack a ([M,K]) for ``matmul_packed_a`` / ``matmul_packed_ab`` (``ops::matmul_pack`` with ``Operand::A``)."""
-    return pack_b(a, stream=stream)
+    return pack_b(a, stream=stream, compute=compute)
 
 
 def matmul_packed_a(packed: PackedB, b, c, c_in=None, workspace=None, stream=None):

@@ -677,6 +677,41 @@ int fetch_mode(const Problem& pr, const VecopsHipPlan& plan) {
   return mode;
 }
 
+// Unsigned 8-bit sides (SRC_I8_FLIP): the kernels multiply the signed images x - 128 (bytes xor 0x80) and the epilogue
+// restores the sum with 128 * (row sums of the other operand's image) per row / column (+ 16384 K when both sides are
+// unsigned).  Launches the row-sum kernels into `terms` (batch * (m + n) int32) and fills the flips and term pointers
+// of `p`.
+int32_t unsigned_side_terms(const Problem& pr, TileGemmParams* params, int32_t* terms, hipStream_t stream) {
+  TileGemmParams& p = *params;
+  hipError_t e;
+  int32_t* row_term = terms;
+  int32_t* col_term = row_term + pr.batch * pr.m;
+  p.a_flip = pr.a_unsigned ? 0x80808080u : 0u;
+  p.b_flip = pr.b_unsigned ? 0x80808080u : 0u;
+  if (pr.b_unsigned) {  // + 128 * sum_k a'[m,k] per row
+    e = launch_byte_row_sums(pr.a.data, p.batch, p.m, p.k, pr.a.bs, pr.a.rs, pr.a.cs, p.a_flip, 128u, nullptr, 0, row_term, stream);
+    if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
+    p.row_term = row_term;
+  }
+  if (pr.a_unsigned && pr.packed_b) {  // the same term from the packed rows, one copy per batch
+    e = launch_packed_row_sums(pr.b.data, p.n, p.k, p.batch, 128u, nullptr, col_term, stream);
+    if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
+    p.col_term = col_term;
+  } else if (pr.a_unsigned) {  // + 128 * sum_k b'[n,k] per column
+    e = launch_byte_row_sums(pr.b.data, p.batch, p.n, p.k, pr.b.bs, pr.b.rs, pr.b.cs, p.b_flip, 128u, nullptr, 0, col_term, stream);
+    if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
+    p.col_term = col_term;
+  }
+  if (pr.a_unsigned && pr.b_unsigned) p.const_term = 16384u * static_cast<uint32_t>(pr.k);
+  // u8 x s8 (AMX_I8I32<uint8_t, int8_t>), one batch, no correction row of the caller's: the column term is
+  // a correction row, which every fast epilogue adds (the general path took 450 us at 2048 x 4096 x 11008)
+  if (pr.a_unsigned && !pr.b_unsigned && p.batch == 1 && p.correction == nullptr) {
+    p.correction = p.col_term;
+    p.col_term = nullptr;
+  }
+  return ST_OK;
+}
+
 int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* row_scales, const float* column_scales,
                     const int32_t* correction, void* workspace, uint64_t workspace_size, hipStream_t stream) {
   if (plan.family == VECOPS_HIP_FAMILY_NONE) return ST_OK;
@@ -801,31 +836,8 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   if (pr.src == SRC_I8_FLIP) {
     // terms of the unsigned side(s), kept behind the split-K partials in the workspace
     const uint64_t partial_bytes = plan.split_k > 1 ? static_cast<uint64_t>(plan.split_k) * pr.batch * pr.m * pr.n * 4u : 0;
-    int32_t* row_term = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + partial_bytes);
-    int32_t* col_term = row_term + pr.batch * pr.m;
-    p.a_flip = pr.a_unsigned ? 0x80808080u : 0u;
-    p.b_flip = pr.b_unsigned ? 0x80808080u : 0u;
-    if (pr.b_unsigned) {  // + 128 * sum_k a'[m,k] per row
-      e = launch_byte_row_sums(pr.a.data, p.batch, p.m, p.k, pr.a.bs, pr.a.rs, pr.a.cs, p.a_flip, 128u, nullptr, 0, row_term, stream);
-      if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
-      p.row_term = row_term;
-    }
-    if (pr.a_unsigned && pr.packed_b) {  // the same term from the packed rows, one copy per batch
-      e = launch_packed_row_sums(pr.b.data, p.n, p.k, p.batch, 128u, nullptr, col_term, stream);
-      if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
-      p.col_term = col_term;
-    } else if (pr.a_unsigned) {  // + 128 * sum_k b'[n,k] per column
-      e = launch_byte_row_sums(pr.b.data, p.batch, p.n, p.k, pr.b.bs, pr.b.rs, pr.b.cs, p.b_flip, 128u, nullptr, 0, col_term, stream);
-      if (e != hipSuccess) return fail(ST_EXEC, "row-sum kernel launch: %s", hipGetErrorString(e));
-      p.col_term = col_term;
-    }
-    if (pr.a_unsigned && pr.b_unsigned) p.const_term = 16384u * static_cast<uint32_t>(pr.k);
-    // u8 x s8 (AMX_I8I32<uint8_t, int8_t>), one batch, no correction row of the caller's: the column term is
-    // a correction row, which every fast epilogue adds (the general path took 450 us at 2048 x 4096 x 11008)
-    if (pr.a_unsigned && !pr.b_unsigned && p.batch == 1 && p.correction == nullptr) {
-      p.correction = p.col_term;
-      p.col_term = nullptr;
-    }
+    int32_t rc = unsigned_side_terms(pr, &p, reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + partial_bytes), stream);
+    if (rc != ST_OK) return rc;
   }
   if (plan.family == VECOPS_HIP_FAMILY_TILE_256X352) {
     if (!wide_tile_serves(pr) || !launch_tile_gemm_i8_wide_serves(p, mode, pr.packed_b))
@@ -886,6 +898,12 @@ void launch_skinny_mfma_resident(const SkinnyW8A16Params& p, hipStream_t stream)
                      0, stream, p);
 }
 
+// Elements per 16-byte chunk of a packed operand of this dtype (0: no such pack).
+int packed_elems_per_chunk(uint32_t packed_dtype) {
+  return (packed_dtype == DT_I8 || packed_dtype == DT_U8) ? 16 : (packed_dtype == DT_BF16 || packed_dtype == DT_F16) ? 8
+         : packed_dtype == DT_F32 ? 4 : 0;
+}
+
 // Problem description of a matmul whose B operand is prepacked: b is described as the dense
 // [N,K] operand it was packed from (its strides are never used), with `packed` as its storage.
 int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t packed_dtype, int64_t n,
@@ -899,6 +917,8 @@ int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t 
     if (da != DT_F16) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an f16-packed b needs an f16 a");
   } else if (packed_dtype == DT_I8 || packed_dtype == DT_U8) {
     if (da != DT_I8 && da != DT_U8) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an 8-bit packed b needs an i8 or u8 a");
+  } else if (packed_dtype == DT_F32) {  // the fp32-compute atom: operands stay fp32
+    if (da != DT_F32) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: an f32-packed b needs an f32 a");
   } else {
     return fail(ST_NOT_APPLICABLE, "matmul_packed_b: packed dtype %u not supported", packed_dtype);
   }
@@ -915,21 +935,25 @@ int32_t describe_packed(const VecopsHipOperand* a, const void* packed, uint32_t 
   b.sizes[base + 1] = k;
   b.strides[base] = k;
   b.strides[base + 1] = 1;
-  int32_t rc = describe(a, &b, cin, c, VECOPS_HIP_COMPUTE_BF16, pr, nullptr, may_fold);
+  int32_t rc = describe(a, &b, cin, c, packed_dtype == DT_F32 ? VECOPS_HIP_COMPUTE_F32 : VECOPS_HIP_COMPUTE_BF16, pr, nullptr,
+                        may_fold);
   if (rc != ST_OK) return rc;
   pr->packed_b = true;
   // 32-bit offsets inside one workgroup's eight 32-row panels of the packed operand
-  const int64_t ks_total = packed_k_steps(pr->k, (packed_dtype == DT_I8 || packed_dtype == DT_U8) ? 16 : 8);
+  const int64_t ks_total = packed_k_steps(pr->k, packed_elems_per_chunk(packed_dtype));
   if (ks_total * 1024 * 8 >= (int64_t{1} << 31)) return fail(ST_NOT_APPLICABLE, "matmul_packed_b: k too large");
   return ST_OK;
 }
 
-int src_of_packed_source(uint32_t dtype) {
-  // (half operands are packed by the bf16 kernel: a permutation of 16-bit elements either way)
-  return (dtype == DT_BF16 || dtype == DT_F16) ? SRC_BF16
-         : dtype == DT_F32                     ? SRC_F32_AS_BF16
-         : (dtype == DT_I8 || dtype == DT_U8)  ? SRC_I8
-                                               : -1;
+// The pack kernel for a source dtype and the dtype it is packed as (half operands are packed by the bf16 kernel: a
+// permutation of 16-bit elements either way); -1: no such pack.
+int src_of_pack(uint32_t source, uint32_t packed_dtype) {
+  if (source == DT_BF16 && packed_dtype == DT_BF16) return SRC_BF16;
+  if (source == DT_F16 && packed_dtype == DT_F16) return SRC_BF16;
+  if (source == DT_F32 && packed_dtype == DT_BF16) return SRC_F32_AS_BF16;
+  if (source == DT_F32 && packed_dtype == DT_F32) return SRC_F32;
+  if ((source == DT_I8 || source == DT_U8) && packed_dtype == source) return SRC_I8;
+  return -1;
 }
 
 }  // namespace
@@ -937,18 +961,18 @@ int src_of_packed_source(uint32_t dtype) {
 extern "C" {
 
 uint64_t vecops_hip_packed_b_bytes(uint32_t packed_dtype, int64_t n, int64_t k) {
-  if (n < 0 || k < 0 || (packed_dtype != DT_BF16 && packed_dtype != DT_F16 && packed_dtype != DT_I8 && packed_dtype != DT_U8))
-    return 0;
-  return static_cast<uint64_t>(packed_b_bytes(n, k, (packed_dtype == DT_I8 || packed_dtype == DT_U8) ? 16 : 8));
+  const int epc = packed_elems_per_chunk(packed_dtype);
+  if (n < 0 || k < 0 || epc == 0) return 0;
+  return static_cast<uint64_t>(packed_b_bytes(n, k, epc));
 }
 
-int32_t vecops_hip_pack_b(const VecopsHipOperand* b, void* packed, uint64_t packed_size, void* stream) {
+int32_t vecops_hip_pack_as(const VecopsHipOperand* b, uint32_t packed_dtype, void* packed, uint64_t packed_size, void* stream) {
   View v;
-  if (!normalise(b, &v) || b->rank != 2) return fail(ST_INVALID, "pack_b: b must be a rank-2 [N,K] operand");
-  const int src = src_of_packed_source(v.dtype);
-  if (src < 0) return fail(ST_NOT_APPLICABLE, "pack_b: dtype %u not supported", v.dtype);
+  if (!normalise(b, &v) || b->rank != 2) return fail(ST_INVALID, "pack: the source must be a rank-2 [rows, K] operand");
+  const int src = src_of_pack(v.dtype, packed_dtype);
+  if (src < 0) return fail(ST_NOT_APPLICABLE, "pack: dtype %u cannot be packed as dtype %u", v.dtype, packed_dtype);
   if (v.rows > INT32_MAX || v.cols > INT32_MAX - 256) return fail(ST_INVALID, "pack_b: extent too large");
-  const uint64_t need = static_cast<uint64_t>(packed_b_bytes(v.rows, v.cols, src == SRC_I8 ? 16 : 8));
+  const uint64_t need = static_cast<uint64_t>(packed_b_bytes(v.rows, v.cols, packed_elems_per_chunk(packed_dtype)));
   if (packed_size < need)
     return fail(ST_INVALID, "pack_b: %llu bytes required, %llu supplied", (unsigned long long)need,
                 (unsigned long long)packed_size);
@@ -966,6 +990,12 @@ int32_t vecops_hip_pack_b(const VecopsHipOperand* b, void* packed, uint64_t pack
   hipError_t e = launch_pack_b(src, q, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(ST_EXEC, "pack kernel launch: %s", hipGetErrorString(e));
   return ST_OK;
+}
+
+int32_t vecops_hip_pack_b(const VecopsHipOperand* b, void* packed, uint64_t packed_size, void* stream) {
+  if (b == nullptr) return fail(ST_INVALID, "pack_b: b must be a rank-2 [N,K] operand");
+  // the default pack of a dtype: fp32 sources are rounded to bf16 (the x86 reference's behaviour), the others keep theirs
+  return vecops_hip_pack_as(b, b->dtype == DT_F32 ? DT_BF16 : b->dtype, packed, packed_size, stream);
 }
 
 int32_t vecops_hip_pack_b_compensated(const VecopsHipOperand* b, int32_t a_zero_point, void* packed,
@@ -1071,7 +1101,7 @@ struct BothPacked {
 int32_t describe_packed_ab(uint32_t a_dtype, int64_t m, uint32_t b_dtype, int64_t n, int64_t k, const VecopsHipOperand* c_in,
                            const VecopsHipOperand* c, void* workspace, BothPacked* d) {
   if (m < 0 || n < 0 || k < 0) return fail(ST_INVALID, "matmul_packed_ab: negative extent");
-  if (a_dtype != DT_BF16 && a_dtype != DT_F16 && a_dtype != DT_I8 && a_dtype != DT_U8)
+  if (packed_elems_per_chunk(a_dtype) == 0)
     return fail(ST_NOT_APPLICABLE, "matmul_packed_ab: packed dtype %u not supported", a_dtype);
   if (c == nullptr || c->rank != 2) return fail(ST_NOT_APPLICABLE, "matmul_packed_ab: c must be rank 2 (a packed operand has no batches)");
   make_operand(&d->a, workspace, a_dtype, m, k, k);
@@ -1113,7 +1143,7 @@ int32_t vecops_hip_matmul_packed_ab(const void* packed_a, uint32_t a_dtype, int6
     q.n = static_cast<int32_t>(m);
     q.k = static_cast<int32_t>(k);
     q.flip = a_dtype == DT_U8 ? 0x80u : 0u;
-    hipError_t e = launch_unpack_b((a_dtype == DT_I8 || a_dtype == DT_U8) ? SRC_I8 : SRC_BF16, q, s);
+    hipError_t e = launch_unpack_b((a_dtype == DT_I8 || a_dtype == DT_U8) ? SRC_I8 : a_dtype == DT_F32 ? SRC_F32 : SRC_BF16, q, s);
     if (e != hipSuccess) return fail(ST_EXEC, "unpack kernel launch: %s", hipGetErrorString(e));
   }
   d.pr.b.data = const_cast<void*>(packed_b);
@@ -1409,9 +1439,9 @@ __global__ __launch_bounds__(256) void expand_groups_kernel(const int32_t* __res
 namespace {
 // A grouped call: several independent products (irregular batches - every group with its own extents, strides and
 // pointers).  bf16 and int8 groups that all multiply run as ONE launch of tile_gemm_grouped_kernel over a table of
-// problem records in the workspace (so do f16 groups and fp32 groups, in either compute type); unsigned 8-bit
-// operands (whose sign flip needs a pass over B first), fp64 operands, groups of mixed classes, and groups with K = 0, run as
-// launches of their own on the same stream.  So do groups whose K the rule table splits (few output tiles, long K):
+// problem records in the workspace (so do f16 groups and fp32 groups, in either compute type, and groups with an
+// unsigned 8-bit side, whose row-sum terms are computed group by group into the workspace first); fp64 operands,
+// groups of mixed classes, and groups with K = 0, run as launches of their own on the same stream.  So do groups whose K the rule table splits (few output tiles, long K):
 // the grouped kernel walks a group's whole K in every workgroup, and two workgroups with 128 K tiles each would
 // be what the whole launch waits for (eight products, 255 x 63 x 8191 among them: 99 us in one launch).
 struct Grouped {
@@ -1422,7 +1452,8 @@ struct Grouped {
   bool one_launch = false;
   int src = -1, tile = 0, mode = 0;
   std::vector<int32_t> first;     // first workgroup of each table group, and the end
-  uint64_t first_bytes = 0, record_bytes = 0, map_bytes = 0, loop_workspace = 0;
+  uint64_t first_bytes = 0, record_bytes = 0, map_bytes = 0, term_bytes = 0, loop_workspace = 0;
+  std::vector<uint64_t> term_offset;  // unsigned 8-bit sides: where a table group's row and column terms lie
 };
 
 int32_t describe_grouped(uint32_t count, const VecopsHipOperand* a, const VecopsHipOperand* b, const VecopsHipOperand* c_in,
@@ -1447,7 +1478,7 @@ int32_t describe_grouped(uint32_t count, const VecopsHipOperand* a, const Vecops
     if (plan.split_k > 1) g->split_groups.push_back(static_cast<int>(i));
     else g->table_groups.push_back(static_cast<int>(i));
   }
-  g->one_launch = same_class && g->src != SRC_I8_FLIP && g->src != kSrcF64 && g->table_groups.size() > 1;
+  g->one_launch = same_class && g->src != kSrcF64 && g->table_groups.size() > 1;
   if (!g->one_launch) return ST_OK;
   // One workgroup tile for every group: the biggest square tile that still yields two rounds' worth of
   // workgroups over all groups together (priced like the rule table's candidates), else 64 x 64.
@@ -1496,10 +1527,19 @@ int32_t describe_grouped(uint32_t count, const VecopsHipOperand* a, const Vecops
   g->first_bytes = round_up_256(g->first.size() * 4u);
   g->record_bytes = round_up_256(g->table_groups.size() * sizeof(TileGemmParams));
   g->map_bytes = round_up_256(static_cast<uint64_t>(next) * 4u);
+  if (g->src == SRC_I8_FLIP) {
+    for (int i : g->table_groups) {
+      const Problem& pr = g->problems[i];
+      g->term_offset.push_back(g->term_bytes);
+      g->term_bytes += round_up_256(static_cast<uint64_t>(pr.batch) * (pr.m + pr.n) * 4u);
+    }
+  }
   return ST_OK;
 }
 
-uint64_t grouped_table_bytes(const Grouped& g) { return g.one_launch ? g.first_bytes + g.record_bytes + g.map_bytes : 0; }
+uint64_t grouped_table_bytes(const Grouped& g) {
+  return g.one_launch ? g.first_bytes + g.record_bytes + g.map_bytes + g.term_bytes : 0;
+}
 
 uint64_t grouped_workspace(const Grouped& g) {
   // the table, and behind it the scratch of the groups that run as launches of their own (one launch at a time, so
@@ -1568,6 +1608,11 @@ int32_t vecops_hip_matmul_grouped(uint32_t count, const VecopsHipOperand* a, con
         return fail(ST_INVALID, "matmul_grouped: group %d has an operand without storage", g.table_groups[offset + j]);
       TileGemmParams& p = chunk.params[j];
       p = base_params(pr, nullptr, nullptr, nullptr, nullptr);
+      if (g.src == SRC_I8_FLIP) {
+        char* terms = base + g.first_bytes + g.record_bytes + g.map_bytes + g.term_offset[offset + j];
+        rc = unsigned_side_terms(pr, &p, reinterpret_cast<int32_t*>(terms), s);
+        if (rc != ST_OK) return rc;
+      }
       p.tiles_m = static_cast<int32_t>((pr.m + g.tile - 1) / g.tile);
       p.tiles_n = static_cast<int32_t>((pr.n + g.tile - 1) / g.tile);
       p.split_k = 1;
@@ -1590,6 +1635,7 @@ int32_t vecops_hip_matmul_grouped(uint32_t count, const VecopsHipOperand* a, con
     case SRC_F16: e = launch_tile_gemm_grouped_f16(t, g.tile, g.mode, s); break;
     case SRC_F32_AS_BF16: e = launch_tile_gemm_grouped_f32_as_bf16(t, g.tile, g.mode, s); break;
     case SRC_F32: e = launch_tile_gemm_grouped_f32(t, g.tile, g.mode, s); break;
+    case SRC_I8_FLIP: e = launch_tile_gemm_grouped_i8_flip(t, g.tile, g.mode, s); break;
     default: e = launch_tile_gemm_grouped_i8(t, g.tile, g.mode, s); break;
   }
   if (e != hipSuccess) return fail(ST_EXEC, "grouped tile kernel launch: %s", hipGetErrorString(e));

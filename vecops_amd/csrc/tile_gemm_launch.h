@@ -202,6 +202,7 @@ hipError_t launch_grouped_class(const GroupedTables& t, int tile, int mode, hipS
 }
 hipError_t launch_tile_gemm_grouped_bf16(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_i8(const GroupedTables& t, int tile, int mode, hipStream_t stream);
+hipError_t launch_tile_gemm_grouped_i8_flip(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_f16(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_f32_as_bf16(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_f32(const GroupedTables& t, int tile, int mode, hipStream_t stream);

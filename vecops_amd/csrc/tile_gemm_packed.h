@@ -7,7 +7,8 @@
 // into MFMA operand registers.  B then bypasses LDS entirely: the LDS pipe, which
 // the plain kernel keeps three quarters busy, carries only A.
 //
-// Packed layout (bytes; EPC = elements per 16-byte chunk: 8 for bf16, 16 for int8).
+// Packed layout (bytes; EPC = elements per 16-byte chunk: 8 for bf16 and f16, 16 for int8, 4 for fp32 kept as fp32 -
+// the fp32-compute atom, whose matrix instruction takes one float per lane: a lane's chunk feeds four of them).
 // B[N, K] is cut into blocks of 32 rows (n) x one MFMA k-step (2 * EPC elements of
 // k); block (nb, ks) is 1 KiB at ((nb * KS) + ks) * 1024, KS = k-steps of K rounded
 // up to whole K tiles (4 k-steps); inside it lane l of a wavefront owns the 16 bytes
@@ -39,7 +40,7 @@ struct PackBParams {
 };
 
 // One thread per 16-byte chunk of the packed operand.  SRC_BF16: bf16 in, bf16
-// packed; SRC_F32_AS_BF16: fp32 in, rounded to bf16 (nearest even); SRC_I8: bytes.
+// packed; SRC_F32_AS_BF16: fp32 in, rounded to bf16 (nearest even); SRC_F32: fp32 in, fp32 packed; SRC_I8: bytes.
 template <int SRC>
 __global__ __launch_bounds__(256) void pack_b_kernel(const PackBParams p) {
   constexpr int EPC = SrcTraits<SRC>::kElemsPerChunk;
@@ -61,6 +62,7 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const PackBParams p) {
           uint32_t v;
           if constexpr (SRC == SRC_BF16) v = static_cast<const uint16_t*>(p.b)[at];
           else if constexpr (SRC == SRC_F32_AS_BF16) v = cvt_pk_bf16(static_cast<const float*>(p.b)[at], 0.0f) & 0xffffu;
+          else if constexpr (SRC == SRC_F32) v = static_cast<const uint32_t*>(p.b)[at];
           else v = static_cast<const uint8_t*>(p.b)[at] ^ p.flip;
           constexpr int per_word = EPC / 4;
           w[e / per_word] |= v << ((e % per_word) * (32 / per_word));
@@ -71,8 +73,8 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const PackBParams p) {
   }
 }
 
-// The inverse: the dense [N, K] operand (element strides rs, ks) back out of its packed form; 16-bit elements or
-// bytes (SRC_BF16 / SRC_I8), p.flip undone.  Used when both operands of a product arrive packed.
+// The inverse: the dense [N, K] operand (element strides rs, ks) back out of its packed form; 16-bit elements,
+// bytes or fp32 (SRC_BF16 / SRC_I8 / SRC_F32), p.flip undone.  Used when both operands of a product arrive packed.
 template <int SRC>
 __global__ __launch_bounds__(256) void unpack_b_kernel(const PackBParams p) {
   constexpr int EPC = SrcTraits<SRC>::kElemsPerChunk;
@@ -95,6 +97,7 @@ __global__ __launch_bounds__(256) void unpack_b_kernel(const PackBParams p) {
         const uint32_t bits = w[e / per_word] >> ((e % per_word) * (32 / per_word));
         const int64_t at = n * p.rs + k * p.ks;
         if constexpr (SRC == SRC_BF16) static_cast<uint16_t*>(const_cast<void*>(p.b))[at] = static_cast<uint16_t>(bits);
+        else if constexpr (SRC == SRC_F32) static_cast<uint32_t*>(const_cast<void*>(p.b))[at] = bits;
         else static_cast<uint8_t*>(const_cast<void*>(p.b))[at] = static_cast<uint8_t>(bits ^ p.flip);
       }
     }

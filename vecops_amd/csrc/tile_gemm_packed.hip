@@ -60,6 +60,7 @@ hipError_t launch_tile_gemm_packed_b(int src, const TileGemmParams& p, int tile_
     case SRC_BF16: return launch_packed_class<SRC_BF16>(p, tile_m, tile_n, vector_a, stream);
     case SRC_F16: return launch_packed_class<SRC_F16>(p, tile_m, tile_n, vector_a, stream);
     case SRC_F32_AS_BF16: return launch_packed_class<SRC_F32_AS_BF16>(p, tile_m, tile_n, vector_a, stream);
+    case SRC_F32: return launch_packed_class<SRC_F32>(p, tile_m, tile_n, vector_a, stream);
     case SRC_I8: return launch_packed_class<SRC_I8>(p, tile_m, tile_n, vector_a, stream);
     // unsigned A: xored on its way into LDS, so never by the loads that write LDS themselves
     case SRC_I8_FLIP: return launch_packed_class<SRC_I8_FLIP>(p, tile_m, tile_n, vector_a ? 1 : 0, stream);
@@ -104,7 +105,7 @@ hipError_t launch_packed_row_sums(const void* packed, int32_t n, int32_t k, int3
 }
 
 hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream) {
-  const int epc = src == SRC_I8 ? 16 : 8;
+  const int epc = src == SRC_I8 ? 16 : src == SRC_F32 ? 4 : 8;
   const int64_t chunks = packed_b_bytes(p.n, p.k, epc) / 16;
   if (chunks == 0) return hipSuccess;
   int64_t blocks = (chunks + 255) / 256;
@@ -113,6 +114,7 @@ hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream) {
   switch (src) {
     case SRC_BF16: hipLaunchKernelGGL(pack_b_kernel<SRC_BF16>, grid, block, 0, stream, p); break;
     case SRC_F32_AS_BF16: hipLaunchKernelGGL(pack_b_kernel<SRC_F32_AS_BF16>, grid, block, 0, stream, p); break;
+    case SRC_F32: hipLaunchKernelGGL(pack_b_kernel<SRC_F32>, grid, block, 0, stream, p); break;
     case SRC_I8: hipLaunchKernelGGL(pack_b_kernel<SRC_I8>, grid, block, 0, stream, p); break;
     default: return hipErrorInvalidValue;
   }
@@ -120,7 +122,7 @@ hipError_t launch_pack_b(int src, const PackBParams& p, hipStream_t stream) {
 }
 
 hipError_t launch_unpack_b(int src, const PackBParams& p, hipStream_t stream) {
-  const int epc = src == SRC_I8 ? 16 : 8;
+  const int epc = src == SRC_I8 ? 16 : src == SRC_F32 ? 4 : 8;
   const int64_t chunks = packed_b_bytes(p.n, p.k, epc) / 16;
   if (chunks == 0) return hipSuccess;
   int64_t blocks = (chunks + 255) / 256;
@@ -128,6 +130,7 @@ hipError_t launch_unpack_b(int src, const PackBParams& p, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>(blocks)), block(256);
   switch (src) {
     case SRC_BF16: hipLaunchKernelGGL(unpack_b_kernel<SRC_BF16>, grid, block, 0, stream, p); break;
+    case SRC_F32: hipLaunchKernelGGL(unpack_b_kernel<SRC_F32>, grid, block, 0, stream, p); break;
     case SRC_I8: hipLaunchKernelGGL(unpack_b_kernel<SRC_I8>, grid, block, 0, stream, p); break;
     default: return hipErrorInvalidValue;
   }

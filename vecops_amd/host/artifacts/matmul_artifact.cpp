@@ -4,7 +4,12 @@
 //   -DVECOPS_ARTIFACT_KIND=<0..8>   0 matmul bf16, 1 matmul f32 (bf16 compute), 5 matmul f32 (fp32 compute), 2 matmul i8,
 //                                   3 matmul_i8_dequant, 4 matmul_w8a16_group, 6 / 7 / 8 / 10 matmul_fused for bf16 /
 //                                   f32 / i8 / f16 operands, 9 matmul f16, 11 / 12 matmul_pack_b to bf16 / i8,
-//                                   13 / 14 / 15 matmul_packed_b for bf16 / f32 / i8 a, 16 matmul_runtime_quant
+//                                   13 / 14 / 15 matmul_packed_b for bf16 / f32 / i8 a, 16 matmul_runtime_quant,
+//                                   17 / 18 matmul_pack_b / matmul_packed_b for f16, 19 matmul_pack_b of u8 weights,
+//                                   20 matmul_packed_b for i8 a against u8-packed weights, 21..24 matmul_pack_a to
+//                                   bf16 / f16 / i8 / u8, 25..28 matmul_packed_a for bf16 / f32 / f16 / i8 b,
+//                                   29 matmul_packed_a for i8 b against a u8-packed a, 30 / 31 matmul_pack_b / _a of
+//                                   fp32 kept fp32, 32 / 33 matmul_packed_b / _a in fp32 compute
 //   -DVECOPS_ARTIFACT_DEVICE=<0|1>  0: tensors are host memory, staged through HBM here
 //                                   1: tensors are HIP device pointers, used in place
 //   -DVECOPS_ARTIFACT_GROUP=<G>     group size of kind 4
@@ -655,30 +660,57 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
 }
 
 // =================================================================================================
-#elif VECOPS_ARTIFACT_KIND == 11 || VECOPS_ARTIFACT_KIND == 12 || VECOPS_ARTIFACT_KIND == 17  // vecops::matmul_pack_b (b, a_zero_point, packed, compensation?)
+#elif VECOPS_ARTIFACT_KIND == 11 || VECOPS_ARTIFACT_KIND == 12 || VECOPS_ARTIFACT_KIND == 17 || VECOPS_ARTIFACT_KIND == 19 || \
+  (VECOPS_ARTIFACT_KIND >= 21 && VECOPS_ARTIFACT_KIND <= 24) || VECOPS_ARTIFACT_KIND == 30 || VECOPS_ARTIFACT_KIND == 31
+// vecops::matmul_pack_b (b, a_zero_point, packed, compensation?)  /  vecops::matmul_pack_a (a, packed)
 // =================================================================================================
 
-#if VECOPS_ARTIFACT_KIND == 11
+#if (VECOPS_ARTIFACT_KIND >= 21 && VECOPS_ARTIFACT_KIND <= 24) || VECOPS_ARTIFACT_KIND == 31
+#define VECOPS_PACK_SIDE_A 1
+#else
+#define VECOPS_PACK_SIDE_A 0
+#endif
+#if VECOPS_ARTIFACT_KIND == 30 || VECOPS_ARTIFACT_KIND == 31
+#define OPERANDS "f32"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);  // elements stay fp32: the pack of the fp32-compute atom
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_F32;
+#elif VECOPS_ARTIFACT_KIND == 11 || VECOPS_ARTIFACT_KIND == 21
 #define OPERANDS "bf16"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16) | bit(VECOPS_DTYPE_F32);  // fp32 sources are rounded to bf16
 constexpr uint32_t kPackedDtype = VECOPS_DTYPE_BF16;
-#elif VECOPS_ARTIFACT_KIND == 17
+#elif VECOPS_ARTIFACT_KIND == 17 || VECOPS_ARTIFACT_KIND == 22
 #define OPERANDS "f16"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F16);
 constexpr uint32_t kPackedDtype = VECOPS_DTYPE_F16;
+#elif VECOPS_ARTIFACT_KIND == 19 || VECOPS_ARTIFACT_KIND == 24
+#define OPERANDS "u8"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_U8);
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_U8;
 #else
 #define OPERANDS "i8"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8);
 constexpr uint32_t kPackedDtype = VECOPS_DTYPE_I8;
 #endif
-constexpr const char* kOperatorName = "vecops::matmul_pack_b";
-constexpr const char* kKey = "vecops::matmul_pack_b;operands=" OPERANDS ";memory=" MEMORY_NAME ";backend=hip-gfx950";
+#if VECOPS_PACK_SIDE_A
+#define PACK_OPERATOR "vecops::matmul_pack_a"
+#else
+#define PACK_OPERATOR "vecops::matmul_pack_b"
+#endif
+constexpr const char* kOperatorName = PACK_OPERATOR;
+constexpr const char* kKey = PACK_OPERATOR ";operands=" OPERANDS ";memory=" MEMORY_NAME ";backend=hip-gfx950";
 
 #define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
   {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
    {.tensor = {sizeof(VecopsTensorParameter), MASK, kDeviceType, -1, RANK, OPTIONAL,                          \
                sizeof(VecopsDimensionConstraint), nullptr, nullptr, FLAGS}}}
 
+#if VECOPS_PACK_SIDE_A
+const VecopsParameterDescriptor kParameters[] = {
+  TENSOR_PARAM("a", kInMask, -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("packed", bit(VECOPS_DTYPE_U8), -1, 0, VECOPS_TENSOR_WRITE),
+};
+constexpr uint32_t kArguments = 2, kPackedAt = 1;
+#else
 const VecopsParameterDescriptor kParameters[] = {
   TENSOR_PARAM("b", kInMask, -1, 0, VECOPS_TENSOR_READ),
   {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_SCALAR, "a_zero_point",
@@ -686,25 +718,32 @@ const VecopsParameterDescriptor kParameters[] = {
   TENSOR_PARAM("packed", bit(VECOPS_DTYPE_U8), -1, 0, VECOPS_TENSOR_WRITE),
   TENSOR_PARAM("compensation", bit(VECOPS_DTYPE_I32), -1, 1, VECOPS_TENSOR_WRITE),
 };
+constexpr uint32_t kArguments = 4, kPackedAt = 2;
+#endif
 
 int32_t workspace_impl(const VecopsCall* call, uint64_t* bytes, VecopsError* error) {
-  if (int32_t rc = check_call(call, 4, error); rc != VECOPS_STATUS_OK) return rc;
+  if (int32_t rc = check_call(call, kArguments, error); rc != VECOPS_STATUS_OK) return rc;
   *bytes = 0;
   return VECOPS_STATUS_OK;
 }
 
 int32_t run_impl(const VecopsCall* call, VecopsError* error) {
-  if (int32_t rc = check_call(call, 4, error); rc != VECOPS_STATUS_OK) return rc;
+  if (int32_t rc = check_call(call, kArguments, error); rc != VECOPS_STATUS_OK) return rc;
   const VecopsTensorView* b = tensor_arg(call, 0);
-  const VecopsTensorView* packed = tensor_arg(call, 2);
+  const VecopsTensorView* packed = tensor_arg(call, kPackedAt);
+#if VECOPS_PACK_SIDE_A
+  const VecopsTensorView* comp = nullptr;
+  if (b == nullptr || packed == nullptr) return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "a and packed must be tensors");
+#else
   const VecopsTensorView* comp = tensor_arg(call, 3);
   if (b == nullptr || packed == nullptr || call->values[1].kind != VECOPS_VALUE_SCALAR)
     return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "b and packed must be tensors, a_zero_point a scalar");
+#endif
   if (b->rank != 2 || packed->rank != 1 || (packed->sizes[0] > 1 && packed->strides[0] != 1) ||
       (comp && (comp->rank != 1 || (comp->sizes[0] > 1 && comp->strides[0] != 1))))
-    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "matmul_pack_b takes a rank-2 b and dense rank-1 outputs");
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, PACK_OPERATOR " takes a rank-2 source and dense rank-1 outputs");
   const int64_t n = b->sizes[0], k = b->sizes[1];
-  const uint64_t need = vecops_hip_packed_b_bytes(kPackedDtype, n, k);
+  const uint64_t need = vecops_hip_packed_b_bytes(kPackedDtype, n, k);   // (one format serves both sides)
   if (static_cast<uint64_t>(packed->sizes[0]) < need)
     return report(error, VECOPS_STATUS_INVALID_ARGUMENT,
                   "packed holds " + std::to_string(packed->sizes[0]) + " bytes, " + std::to_string(need) + " are needed");
@@ -719,45 +758,75 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
   if ((rc = device_address(b, false, &staging, &b_dev, error)) != VECOPS_STATUS_OK) return rc;
   if (comp && (rc = device_address(comp, true, &staging, &c_dev, error)) != VECOPS_STATUS_OK) return rc;
   VecopsHipOperand ob;
-  if (!fill_operand(b, b_dev, &ob)) return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "b must have rank 2");
+  if (!fill_operand(b, b_dev, &ob)) return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "the source must have rank 2");
+#if VECOPS_PACK_SIDE_A || VECOPS_ARTIFACT_KIND == 30
+  rc = vecops_hip_pack_as(&ob, kPackedDtype, p_dev, static_cast<uint64_t>(packed->sizes[0]), stream);
+#else
   if (comp)
     rc = vecops_hip_pack_b_compensated(&ob, static_cast<int32_t>(call->values[1].value.scalar.value.i64), p_dev,
                                        static_cast<uint64_t>(packed->sizes[0]), static_cast<int32_t*>(c_dev), stream);
   else
     rc = vecops_hip_pack_b(&ob, p_dev, static_cast<uint64_t>(packed->sizes[0]), stream);
+#endif
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
   return finish(call, &staging, stream, error);
 }
 
 // =================================================================================================
-#elif (VECOPS_ARTIFACT_KIND >= 13 && VECOPS_ARTIFACT_KIND <= 15) || VECOPS_ARTIFACT_KIND == 18  // vecops::matmul_packed_b (a, packed_b, c_in?, c)
+#elif (VECOPS_ARTIFACT_KIND >= 13 && VECOPS_ARTIFACT_KIND <= 15) || VECOPS_ARTIFACT_KIND == 18 || VECOPS_ARTIFACT_KIND == 20 || \
+  (VECOPS_ARTIFACT_KIND >= 25 && VECOPS_ARTIFACT_KIND <= 29) || VECOPS_ARTIFACT_KIND == 32 || VECOPS_ARTIFACT_KIND == 33
+// vecops::matmul_packed_b (a, packed_b, c_in?, c)  /  vecops::matmul_packed_a (packed_a, b, c_in?, c)
 // =================================================================================================
 
-#if VECOPS_ARTIFACT_KIND == 13
+#if (VECOPS_ARTIFACT_KIND >= 25 && VECOPS_ARTIFACT_KIND <= 29) || VECOPS_ARTIFACT_KIND == 33
+#define VECOPS_PACK_SIDE_A 1
+#else
+#define VECOPS_PACK_SIDE_A 0
+#endif
+#if VECOPS_ARTIFACT_KIND == 32 || VECOPS_ARTIFACT_KIND == 33
+#define OPERANDS "f32;compute=f32"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
+#elif VECOPS_ARTIFACT_KIND == 13 || VECOPS_ARTIFACT_KIND == 25
 #define OPERANDS "bf16"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_BF16);
-#elif VECOPS_ARTIFACT_KIND == 14
+#elif VECOPS_ARTIFACT_KIND == 14 || VECOPS_ARTIFACT_KIND == 26
 #define OPERANDS "f32"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F32);
-#elif VECOPS_ARTIFACT_KIND == 18
+#elif VECOPS_ARTIFACT_KIND == 18 || VECOPS_ARTIFACT_KIND == 27
 #define OPERANDS "f16"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_F16);
+#elif VECOPS_ARTIFACT_KIND == 20 || VECOPS_ARTIFACT_KIND == 29
+#define OPERANDS "i8;packed=u8"
+constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);
 #else
 #define OPERANDS "i8"
 constexpr uint64_t kInMask = bit(VECOPS_DTYPE_I8) | bit(VECOPS_DTYPE_U8);
 #endif
-#if VECOPS_ARTIFACT_KIND == 15
+#if VECOPS_ARTIFACT_KIND == 32 || VECOPS_ARTIFACT_KIND == 33
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32);
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_F32;
+#elif VECOPS_ARTIFACT_KIND == 15 || VECOPS_ARTIFACT_KIND == 28
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_I32);
 constexpr uint32_t kPackedDtype = VECOPS_DTYPE_I8;
-#elif VECOPS_ARTIFACT_KIND == 18
+#elif VECOPS_ARTIFACT_KIND == 20 || VECOPS_ARTIFACT_KIND == 29
+constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_I32);
+constexpr uint32_t kPackedDtype = VECOPS_DTYPE_U8;
+#elif VECOPS_ARTIFACT_KIND == 18 || VECOPS_ARTIFACT_KIND == 27
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_F16);
 constexpr uint32_t kPackedDtype = VECOPS_DTYPE_F16;
 #else
 constexpr uint64_t kOutMask = bit(VECOPS_DTYPE_F32) | bit(VECOPS_DTYPE_BF16);
 constexpr uint32_t kPackedDtype = VECOPS_DTYPE_BF16;
 #endif
-constexpr const char* kOperatorName = "vecops::matmul_packed_b";
-constexpr const char* kKey = "vecops::matmul_packed_b;operands=" OPERANDS ";memory=" MEMORY_NAME ";backend=hip-gfx950";
+#if VECOPS_PACK_SIDE_A
+#define PACKED_OPERATOR "vecops::matmul_packed_a"
+constexpr uint32_t kDenseAt = 1, kPackedAt = 0;
+#else
+#define PACKED_OPERATOR "vecops::matmul_packed_b"
+constexpr uint32_t kDenseAt = 0, kPackedAt = 1;
+#endif
+constexpr const char* kOperatorName = PACKED_OPERATOR;
+constexpr const char* kKey = PACKED_OPERATOR ";operands=" OPERANDS ";memory=" MEMORY_NAME ";backend=hip-gfx950";
 
 #define TENSOR_PARAM(NAME, MASK, RANK, OPTIONAL, FLAGS)                                                       \
   {sizeof(VecopsParameterDescriptor), VECOPS_VALUE_TENSOR, NAME,                                              \
@@ -765,44 +834,59 @@ constexpr const char* kKey = "vecops::matmul_packed_b;operands=" OPERANDS ";memo
                sizeof(VecopsDimensionConstraint), nullptr, nullptr, FLAGS}}}
 
 const VecopsParameterDescriptor kParameters[] = {
+#if VECOPS_PACK_SIDE_A
+  TENSOR_PARAM("packed_a", bit(VECOPS_DTYPE_U8), -1, 0, VECOPS_TENSOR_READ),
+  TENSOR_PARAM("b", kInMask, -1, 0, VECOPS_TENSOR_READ),
+#else
   TENSOR_PARAM("a", kInMask, -1, 0, VECOPS_TENSOR_READ),
   TENSOR_PARAM("packed_b", bit(VECOPS_DTYPE_U8), -1, 0, VECOPS_TENSOR_READ),
+#endif
   TENSOR_PARAM("c_in", kOutMask, -1, 1, VECOPS_TENSOR_READ),
   TENSOR_PARAM("c", kOutMask, -1, 0, VECOPS_TENSOR_WRITE),
 };
 
+// `a` is the dense operand ([..,M,K] of matmul_packed_b, [..,N,K] of matmul_packed_a), `n` the rows of the packed one
+// (N resp. M), taken from c.
 struct PackedArgs {
   const VecopsTensorView *a, *packed, *cin, *c;
   VecopsHipOperand oa, ocin, oc;
   int64_t n;
 };
 
+int32_t plan_packed(const PackedArgs& d, VecopsHipPlan* plan) {
+#if VECOPS_PACK_SIDE_A
+  return vecops_hip_plan_matmul_packed_a(kPackedDtype, d.n, &d.oa, d.cin ? &d.ocin : nullptr, &d.oc, plan);
+#else
+  return vecops_hip_plan_matmul_packed_b(&d.oa, kPackedDtype, d.n, d.cin ? &d.ocin : nullptr, &d.oc, plan);
+#endif
+}
+
 int32_t decode(const VecopsCall* call, PackedArgs* d, VecopsHipPlan* plan, VecopsError* error) {
   if (int32_t rc = check_call(call, 4, error); rc != VECOPS_STATUS_OK) return rc;
-  d->a = tensor_arg(call, 0);
-  d->packed = tensor_arg(call, 1);
+  d->a = tensor_arg(call, kDenseAt);
+  d->packed = tensor_arg(call, kPackedAt);
   d->cin = tensor_arg(call, 2);
   d->c = tensor_arg(call, 3);
   if (d->a == nullptr || d->packed == nullptr || d->c == nullptr)
-    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "a, packed_b and c must be tensors");
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "the dense operand, the packed operand and c must be tensors");
   if (d->packed->rank != 1 || (d->packed->sizes[0] > 1 && d->packed->strides[0] != 1))
-    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "packed_b must be a dense rank-1 byte tensor");
+    return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "the packed operand must be a dense rank-1 byte tensor");
   if (!fill_operand(d->a, reinterpret_cast<void*>(16), &d->oa) || !fill_operand(d->c, reinterpret_cast<void*>(16), &d->oc) ||
       (d->cin != nullptr && !fill_operand(d->cin, reinterpret_cast<void*>(16), &d->ocin)))
     return report(error, VECOPS_STATUS_INVALID_ARGUMENT, "tensors must have rank 2 or 3");
-  d->n = d->c->sizes[d->c->rank - 1];
+  d->n = d->c->sizes[d->c->rank - (VECOPS_PACK_SIDE_A ? 2 : 1)];
   const int64_t k = d->a->sizes[d->a->rank - 1];
   const uint64_t need = vecops_hip_packed_b_bytes(kPackedDtype, d->n, k);
   if (static_cast<uint64_t>(d->packed->sizes[0]) < need)
     return report(error, VECOPS_STATUS_INVALID_ARGUMENT,
-                  "packed_b holds " + std::to_string(d->packed->sizes[0]) + " bytes, " + std::to_string(need) +
-                    " are needed for N = " + std::to_string(d->n) + ", K = " + std::to_string(k));
+                  "the packed operand holds " + std::to_string(d->packed->sizes[0]) + " bytes, " + std::to_string(need) +
+                    " are needed for " + std::to_string(d->n) + " rows, K = " + std::to_string(k));
 #if VECOPS_ARTIFACT_DEVICE
   d->oa.data = origin(d->a);
   d->oc.data = origin(d->c);
   if (d->cin != nullptr) d->ocin.data = origin(d->cin);
 #endif
-  int32_t rc = vecops_hip_plan_matmul_packed_b(&d->oa, kPackedDtype, d->n, d->cin ? &d->ocin : nullptr, &d->oc, plan);
+  int32_t rc = plan_packed(*d, plan);
   return rc == VECOPS_STATUS_OK ? rc : report_kernel(error, rc);
 }
 
@@ -844,8 +928,12 @@ int32_t run_impl(const VecopsCall* call, VecopsError* error) {
     return report_hip(error, "allocating split-K scratch", e);
   ws_size = p.workspace_bytes;
 #endif
+#if VECOPS_PACK_SIDE_A
+  rc = vecops_hip_matmul_packed_a(packed_dev, kPackedDtype, d.n, &d.oa, d.cin ? &d.ocin : nullptr, &d.oc, ws, ws_size, stream);
+#else
   rc = vecops_hip_matmul_packed_b(&d.oa, packed_dev, kPackedDtype, d.n, d.cin ? &d.ocin : nullptr, &d.oc, ws, ws_size,
                                   stream);
+#endif
   if (rc != VECOPS_STATUS_OK) return report_kernel(error, rc);
   return finish(call, &staging, stream, error);
 }

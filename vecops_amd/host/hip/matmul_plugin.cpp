@@ -120,6 +120,28 @@ Status pack_b_relations(std::span<const Value> v) {
   return Status::success();
 }
 
+// vecops::matmul_pack_a (a, packed)
+Status pack_a_relations(std::span<const Value> v) {
+  if (tensor_at(v, 0) == nullptr || tensor_at(v, 1) == nullptr) return invalid("vecops::matmul_pack_a needs a and packed tensors");
+  return Status::success();
+}
+
+// vecops::matmul_packed_a (packed_a, b, c_in?, c): M is c's second-to-last extent, K is b's last.
+Status packed_a_relations(std::span<const Value> v) {
+  const TensorView* packed = tensor_at(v, 0);
+  const TensorView* b = tensor_at(v, 1);
+  const TensorView* cin = tensor_at(v, 2);
+  const TensorView* c = tensor_at(v, 3);
+  if (packed == nullptr || b == nullptr || c == nullptr) return invalid("vecops::matmul_packed_a needs packed_a, b and c");
+  const std::size_t rank = b->sizes.size();
+  if (rank != 2 && rank != 3) return invalid("b must have rank 2 or 3");
+  if (c->sizes.size() != rank || (cin && cin->sizes.size() != rank)) return invalid("b, c_in and c must have the same rank");
+  if (cols(*c) != rows(*b)) return invalid("c must be [.., M, N]");
+  if (cin && (rows(*cin) != rows(*c) || cols(*cin) != cols(*c))) return invalid("c_in must be [.., M, N]");
+  if (rank == 3 && (b->sizes[0] != c->sizes[0] || (cin && cin->sizes[0] != c->sizes[0]))) return invalid("batch extents differ");
+  return Status::success();
+}
+
 // vecops::matmul_packed_b (a, packed_b, c_in?, c): N is c's last extent, K is a's.
 Status packed_b_relations(std::span<const Value> v) {
   const TensorView* a = tensor_at(v, 0);
@@ -178,6 +200,15 @@ rt::Result<DType> compute_type(const rt::KernelCall& call) {
   if (it == call.values().end()) return DType::BFloat16;
   if (const auto* d = std::get_if<DType>(&it->second)) return *d;
   return invalid("ComputeType must be a DType");
+}
+
+// The `PackedType` specialization value of vecops::matmul_packed_a / _b: the element type of the packed operand where the
+// dense operand does not fix it - UInt8 for packs of unsigned bytes; absent (or the class's own type) otherwise.
+rt::Result<bool> packed_is_unsigned(const rt::KernelCall& call) {
+  auto it = call.values().find("PackedType");
+  if (it == call.values().end()) return false;
+  if (const auto* d = std::get_if<DType>(&it->second)) return *d == DType::UInt8;
+  return invalid("PackedType must be a DType");
 }
 
 // The `Family` specialization value of vecops::matmul: the number of a kernel family the call requires (vecops'
@@ -283,7 +314,7 @@ rt::OperatorSchema make_matmul_pack_b_schema() {
   using rt::dtype_bit;
   std::vector<rt::ParameterSchema> params;
   params.push_back(tensor_param("b", dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
-                                       dtype_bit(DType::Int8), 2u, VECOPS_TENSOR_READ));
+                                       dtype_bit(DType::Int8) | dtype_bit(DType::UInt8), 2u, VECOPS_TENSOR_READ));
   params.push_back(rt::ParameterSchema{"a_zero_point", rt::ScalarConstraint{dtype_bit(DType::Int64) | dtype_bit(DType::Int32)}});
   params.push_back(tensor_param("packed", dtype_bit(DType::UInt8), 1u, VECOPS_TENSOR_WRITE));
   params.push_back(tensor_param("compensation", dtype_bit(DType::Int32), 1u, VECOPS_TENSOR_WRITE, /*optional=*/true));
@@ -302,6 +333,29 @@ rt::OperatorSchema make_matmul_packed_b_schema() {
   params.push_back(tensor_param("c_in", out, std::nullopt, VECOPS_TENSOR_READ, /*optional=*/true));
   params.push_back(tensor_param("c", out, std::nullopt, VECOPS_TENSOR_WRITE));
   return rt::OperatorSchema(kMatmulPackedBName, std::move(params), packed_b_relations);
+}
+
+rt::OperatorSchema make_matmul_pack_a_schema() {
+  using rt::dtype_bit;
+  std::vector<rt::ParameterSchema> params;
+  params.push_back(tensor_param("a", dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                                       dtype_bit(DType::Int8) | dtype_bit(DType::UInt8), 2u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("packed", dtype_bit(DType::UInt8), 1u, VECOPS_TENSOR_WRITE));
+  return rt::OperatorSchema(kMatmulPackAName, std::move(params), pack_a_relations);
+}
+
+rt::OperatorSchema make_matmul_packed_a_schema() {
+  using rt::dtype_bit;
+  const std::uint64_t in = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                           dtype_bit(DType::Int8) | dtype_bit(DType::UInt8);
+  const std::uint64_t out = dtype_bit(DType::BFloat16) | dtype_bit(DType::Float16) | dtype_bit(DType::Float32) |
+                            dtype_bit(DType::Int32);
+  std::vector<rt::ParameterSchema> params;
+  params.push_back(tensor_param("packed_a", dtype_bit(DType::UInt8), 1u, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("b", in, std::nullopt, VECOPS_TENSOR_READ));
+  params.push_back(tensor_param("c_in", out, std::nullopt, VECOPS_TENSOR_READ, /*optional=*/true));
+  params.push_back(tensor_param("c", out, std::nullopt, VECOPS_TENSOR_WRITE));
+  return rt::OperatorSchema(kMatmulPackedAName, std::move(params), packed_a_relations);
 }
 
 rt::OperatorSchema make_matmul_runtime_quant_schema() {
@@ -485,17 +539,35 @@ rt::Result<rt::BoundKernelRecipe> MatmulW8A16GroupRecipe::bind(const rt::KernelC
   return bound;
 }
 
-MatmulPackBRecipe::MatmulPackBRecipe(OperandClass packed) : packed_(packed) {
-  id_ = packed == OperandClass::I8 ? "hip.matmul_pack_b.i8" : packed == OperandClass::F16 ? "hip.matmul_pack_b.f16" : "hip.matmul_pack_b.bf16";
+namespace {
+const char* class_name(OperandClass c) {
+  switch (c) {
+    case OperandClass::BF16: return "bf16";
+    case OperandClass::F16: return "f16";
+    case OperandClass::F32: return "f32";
+    case OperandClass::I8: return "i8";
+    case OperandClass::U8: return "u8";
+  }
+  return "";
+}
+}  // namespace
+
+MatmulPackBRecipe::MatmulPackBRecipe(OperandClass packed, PackSide side) : packed_(packed), side_(side) {
+  id_ = std::string(side == PackSide::A ? "hip.matmul_pack_a." : "hip.matmul_pack_b.") + class_name(packed);
 }
 
 Status MatmulPackBRecipe::match(const rt::KernelCall& call) const {
   const auto values = call.arguments().values();
-  const TensorView* b = tensor_at(values, 0);
-  if (b == nullptr) return invalid("vecops::matmul_pack_b needs a b tensor");
-  const bool mine = packed_ == OperandClass::I8    ? b->dtype == DType::Int8
-                    : packed_ == OperandClass::F16 ? b->dtype == DType::Float16
-                                                   : (b->dtype == DType::BFloat16 || b->dtype == DType::Float32);
+  const TensorView* src = tensor_at(values, 0);
+  if (src == nullptr) return invalid(std::string(side_ == PackSide::A ? kMatmulPackAName : kMatmulPackBName) + " needs a source tensor");
+  auto compute = compute_type(call);
+  if (!compute) return compute.status();
+  const bool keep_f32 = src->dtype == DType::Float32 && compute.value() == DType::Float32;  // the fp32-compute atom's pack
+  const bool mine = packed_ == OperandClass::I8    ? src->dtype == DType::Int8
+                    : packed_ == OperandClass::U8  ? src->dtype == DType::UInt8
+                    : packed_ == OperandClass::F16 ? src->dtype == DType::Float16
+                    : packed_ == OperandClass::F32 ? keep_f32
+                                                   : (src->dtype == DType::BFloat16 || (src->dtype == DType::Float32 && !keep_f32));
   if (!mine) return not_applicable("source dtype belongs to another recipe");
   auto place = placement_of(call);
   if (!place) return place.status();
@@ -506,31 +578,39 @@ rt::Result<rt::BoundKernelRecipe> MatmulPackBRecipe::bind(const rt::KernelCall& 
   if (Status st = match(call); !st.ok()) return st;
   rt::BoundKernelRecipe bound;
   bound.recipe_id = id_;
-  bound.specialization_key = std::string(kMatmulPackBName) + ";operands=" +
-                             (packed_ == OperandClass::I8 ? "i8" : packed_ == OperandClass::F16 ? "f16" : "bf16") +
-                             ";memory=" + placement_name(placement_of(call).value()) + ";" + kBackend;
+  bound.specialization_key = std::string(side_ == PackSide::A ? kMatmulPackAName : kMatmulPackBName) + ";operands=" +
+                             class_name(packed_) + ";memory=" + placement_name(placement_of(call).value()) + ";" + kBackend;
   bound.artifact_key = id_ + ";" + bound.specialization_key;
   return bound;
 }
 
-MatmulPackedBRecipe::MatmulPackedBRecipe(OperandClass operands) : operands_(operands) {
-  id_ = operands == OperandClass::BF16 ? "hip.matmul_packed_b.bf16.tile"
-        : operands == OperandClass::F16 ? "hip.matmul_packed_b.f16.tile"
-        : operands == OperandClass::F32 ? "hip.matmul_packed_b.f32.tile"
-                                        : "hip.matmul_packed_b.i8.tile";
+MatmulPackedBRecipe::MatmulPackedBRecipe(OperandClass operands, PackSide side, bool packed_unsigned, bool f32_compute)
+  : operands_(operands), side_(side), packed_unsigned_(packed_unsigned), f32_compute_(f32_compute) {
+  id_ = std::string(side == PackSide::A ? "hip.matmul_packed_a." : "hip.matmul_packed_b.") + class_name(operands) +
+        (packed_unsigned ? ".packed_u8" : "") + (f32_compute ? ".f32_compute" : "") + ".tile";
 }
 
 Status MatmulPackedBRecipe::match(const rt::KernelCall& call) const {
   const auto values = call.arguments().values();
-  const TensorView* a = tensor_at(values, 0);
+  const char* op = side_ == PackSide::A ? kMatmulPackedAName : kMatmulPackedBName;
+  const TensorView* dense = tensor_at(values, side_ == PackSide::A ? 1 : 0);
   const TensorView* cin = tensor_at(values, 2);
   const TensorView* c = tensor_at(values, 3);
-  if (a == nullptr || c == nullptr) return invalid("vecops::matmul_packed_b needs a and c tensors");
-  const bool mine = operands_ == OperandClass::I8 ? (a->dtype == DType::Int8 || a->dtype == DType::UInt8)
-                    : operands_ == OperandClass::F32 ? a->dtype == DType::Float32
-                    : operands_ == OperandClass::F16 ? a->dtype == DType::Float16
-                                                     : a->dtype == DType::BFloat16;
+  if (dense == nullptr || c == nullptr) return invalid(std::string(op) + " needs its dense operand and c");
+  const bool mine = operands_ == OperandClass::I8 ? (dense->dtype == DType::Int8 || dense->dtype == DType::UInt8)
+                    : operands_ == OperandClass::F32 ? dense->dtype == DType::Float32
+                    : operands_ == OperandClass::F16 ? dense->dtype == DType::Float16
+                                                     : dense->dtype == DType::BFloat16;
   if (!mine) return not_applicable("operand dtype belongs to another recipe");
+  auto unsigned_pack = packed_is_unsigned(call);
+  if (!unsigned_pack) return unsigned_pack.status();
+  if (unsigned_pack.value() && operands_ != OperandClass::I8) return invalid("PackedType UInt8 goes with 8-bit integer operands");
+  if (unsigned_pack.value() != packed_unsigned_) return not_applicable("the packed operand's signedness belongs to another recipe");
+  auto compute = compute_type(call);
+  if (!compute) return compute.status();
+  const bool wants_f32 = operands_ == OperandClass::F32 && compute.value() == DType::Float32;
+  if (wants_f32 != f32_compute_) return not_applicable("the compute type belongs to another recipe");
+  if (f32_compute_ && c->dtype != DType::Float32) return not_applicable("fp32 products leave as fp32");
   const bool int_out = operands_ == OperandClass::I8;
   const DType narrow = operands_ == OperandClass::F16 ? DType::Float16 : DType::BFloat16;  // the operands' own 16-bit type
   if (int_out ? c->dtype != DType::Int32 : (c->dtype != DType::Float32 && c->dtype != narrow))
@@ -544,13 +624,11 @@ Status MatmulPackedBRecipe::match(const rt::KernelCall& call) const {
 
 rt::Result<rt::BoundKernelRecipe> MatmulPackedBRecipe::bind(const rt::KernelCall& call) const {
   if (Status st = match(call); !st.ok()) return st;
-  const char* operands = operands_ == OperandClass::BF16 ? "bf16"
-                         : operands_ == OperandClass::F16 ? "f16"
-                         : operands_ == OperandClass::F32 ? "f32"
-                                                          : "i8";
   rt::BoundKernelRecipe bound;
   bound.recipe_id = id_;
-  bound.specialization_key = std::string(kMatmulPackedBName) + ";operands=" + operands + ";memory=" +
+  bound.specialization_key = std::string(side_ == PackSide::A ? kMatmulPackedAName : kMatmulPackedBName) + ";operands=" +
+                             class_name(operands_) + (packed_unsigned_ ? ";packed=u8" : "") +
+                             (f32_compute_ ? ";compute=f32" : "") + ";memory=" +
                              placement_name(placement_of(call).value()) + ";" + kBackend;
   bound.artifact_key = id_ + ";" + bound.specialization_key;
   return bound;
@@ -593,15 +671,19 @@ MatmulDispatchPolicy::candidates(const rt::KernelCall& call,
     if (const auto* mf = dynamic_cast<const MatmulFusedRecipe*>(recipes[i].get()); mf != nullptr && a != nullptr) {
       if (!takes(mf->operands(), a->dtype)) continue;
     }
-    if (const auto* mp = dynamic_cast<const MatmulPackedBRecipe*>(recipes[i].get()); mp != nullptr && a != nullptr) {
-      if (mp->operands() == OperandClass::I8 ? (a->dtype != DType::Int8 && a->dtype != DType::UInt8)
-          : mp->operands() == OperandClass::F32 ? a->dtype != DType::Float32
-          : mp->operands() == OperandClass::F16 ? a->dtype != DType::Float16
-                                                : a->dtype != DType::BFloat16) continue;
+    if (const auto* mp = dynamic_cast<const MatmulPackedBRecipe*>(recipes[i].get()); mp != nullptr) {
+      const TensorView* dense = tensor_at(values, mp->side() == PackSide::A ? 1 : 0);   // (packed_a, b, ..) / (a, packed_b, ..)
+      if (dense != nullptr &&
+          (mp->operands() == OperandClass::I8 ? (dense->dtype != DType::Int8 && dense->dtype != DType::UInt8)
+           : mp->operands() == OperandClass::F32 ? dense->dtype != DType::Float32
+           : mp->operands() == OperandClass::F16 ? dense->dtype != DType::Float16
+                                                 : dense->dtype != DType::BFloat16)) continue;
     }
     if (const auto* pk = dynamic_cast<const MatmulPackBRecipe*>(recipes[i].get()); pk != nullptr && a != nullptr) {
       if ((pk->operands() == OperandClass::I8) != (a->dtype == DType::Int8) ||
-          (pk->operands() == OperandClass::F16) != (a->dtype == DType::Float16)) continue;
+          (pk->operands() == OperandClass::U8) != (a->dtype == DType::UInt8) ||
+          (pk->operands() == OperandClass::F16) != (a->dtype == DType::Float16) ||
+          (pk->operands() == OperandClass::F32 && a->dtype != DType::Float32)) continue;   // (fp32: match() reads ComputeType)
     }
     order.push_back(i);
   }
@@ -706,7 +788,29 @@ std::shared_ptr<rt::Operator> make_matmul_fused_operator(const std::filesystem::
 std::shared_ptr<rt::Operator> make_matmul_pack_b_operator(const std::filesystem::path& dir) {
   return assemble(make_matmul_pack_b_schema(),
                   {std::make_shared<MatmulPackBRecipe>(OperandClass::BF16), std::make_shared<MatmulPackBRecipe>(OperandClass::F16),
-                   std::make_shared<MatmulPackBRecipe>(OperandClass::I8)},
+                   std::make_shared<MatmulPackBRecipe>(OperandClass::I8), std::make_shared<MatmulPackBRecipe>(OperandClass::U8),
+                   std::make_shared<MatmulPackBRecipe>(OperandClass::F32)},
+                  dir);
+}
+
+std::shared_ptr<rt::Operator> make_matmul_pack_a_operator(const std::filesystem::path& dir) {
+  return assemble(make_matmul_pack_a_schema(),
+                  {std::make_shared<MatmulPackBRecipe>(OperandClass::BF16, PackSide::A),
+                   std::make_shared<MatmulPackBRecipe>(OperandClass::F16, PackSide::A),
+                   std::make_shared<MatmulPackBRecipe>(OperandClass::I8, PackSide::A),
+                   std::make_shared<MatmulPackBRecipe>(OperandClass::U8, PackSide::A),
+                   std::make_shared<MatmulPackBRecipe>(OperandClass::F32, PackSide::A)},
+                  dir);
+}
+
+std::shared_ptr<rt::Operator> make_matmul_packed_a_operator(const std::filesystem::path& dir) {
+  return assemble(make_matmul_packed_a_schema(),
+                  {std::make_shared<MatmulPackedBRecipe>(OperandClass::BF16, PackSide::A),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::F16, PackSide::A),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::F32, PackSide::A),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::I8, PackSide::A),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::I8, PackSide::A, /*packed_unsigned=*/true),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::F32, PackSide::A, false, /*f32_compute=*/true)},
                   dir);
 }
 
@@ -715,7 +819,9 @@ std::shared_ptr<rt::Operator> make_matmul_packed_b_operator(const std::filesyste
                   {std::make_shared<MatmulPackedBRecipe>(OperandClass::BF16),
                    std::make_shared<MatmulPackedBRecipe>(OperandClass::F16),
                    std::make_shared<MatmulPackedBRecipe>(OperandClass::F32),
-                   std::make_shared<MatmulPackedBRecipe>(OperandClass::I8)},
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::I8),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::I8, PackSide::B, /*packed_unsigned=*/true),
+                   std::make_shared<MatmulPackedBRecipe>(OperandClass::F32, PackSide::B, false, /*f32_compute=*/true)},
                   dir);
 }
 

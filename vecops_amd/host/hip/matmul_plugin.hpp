@@ -44,10 +44,14 @@ inline constexpr const char* kMatmulW8A16GroupName = "vecops::matmul_w8a16_group
 inline constexpr const char* kMatmulFusedName = "vecops::matmul_fused";
 inline constexpr const char* kMatmulPackBName = "vecops::matmul_pack_b";
 inline constexpr const char* kMatmulPackedBName = "vecops::matmul_packed_b";
+inline constexpr const char* kMatmulPackAName = "vecops::matmul_pack_a";
+inline constexpr const char* kMatmulPackedAName = "vecops::matmul_packed_a";
 inline constexpr const char* kMatmulRuntimeQuantName = "vecops::matmul_runtime_quant";
 
-// Operand classes of vecops::matmul, one artifact each.
-enum class OperandClass { BF16, F32, I8, F16 };
+// Operand classes of vecops::matmul, one artifact each (U8: packs of unsigned bytes only).
+enum class OperandClass { BF16, F32, I8, F16, U8 };
+// The side a packed operand was packed for (ops::matmul_pack's Operand::A / Operand::B, ops/MatmulPack.h:63-65).
+enum class PackSide { A, B };
 
 // Schemas.  Ranks are left open on vecops::matmul (rank 2 and rank 3 go through
 // one operator); the relation validator enforces what the CPU path asserts in
@@ -70,6 +74,15 @@ rt::OperatorSchema make_matmul_fused_schema();
 // comes from c, K from a, and one packed operand serves every batch of a rank-3 a (ops/MatmulPack.h:22-24).
 rt::OperatorSchema make_matmul_pack_b_schema();
 rt::OperatorSchema make_matmul_packed_b_schema();
+// Side A (ops::MatmulPack<MatmulPackConfig<Atom, Operand::A>>, ops/MatmulPack.h:81-96; tests/ops/MatmulMixedPackingTest.cpp:24-28):
+// vecops::matmul_pack_a (a[M,K], packed out) and vecops::matmul_packed_a (packed_a, b[..,N,K], c_in?, c out) - M comes
+// from c, K from b, and the one packed a serves every batch of a rank-3 b.
+// Unsigned weights (AMX_I8I32<int8_t, uint8_t>, <uint8_t, uint8_t>): a uint8 source packs like any other; the product
+// is told by the specialization value `PackedType` = UInt8 that its packed operand holds unsigned bytes (a packed
+// tensor is opaque bytes here, where vecops' packed Tensor carries its dtype).  Absent, the packed operand has the
+// class's own type (int8 for the 8-bit class).
+rt::OperatorSchema make_matmul_pack_a_schema();
+rt::OperatorSchema make_matmul_packed_a_schema();
 // vecops::matmul_runtime_quant: fp32 activations quantised on the way in by vecops'
 // RuntimePerRowAsymmetricQuantizeTransform (q = u8(a * multipliers[row] + zero_point), matmul/Quantization.h:91-146),
 // int8 weights, the int32 correction row as C input and the per-row x per-column dequantisation on the way out -
@@ -132,34 +145,48 @@ public:
   [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
 };
 
-// vecops::matmul_pack_b for one packed class (BF16 takes bf16 and fp32 sources, I8 takes int8):
-//   vecops::matmul_pack_b;operands=<bf16|i8>;memory=<host|device>;backend=hip-gfx950
+// vecops::matmul_pack_b / vecops::matmul_pack_a for one packed class (BF16 takes bf16 and fp32 sources, I8 int8,
+// U8 uint8, F16 half; F32 takes fp32 sources when the call's ComputeType is Float32 and keeps their elements fp32 - the
+// pack of the fp32-compute atom):
+//   vecops::matmul_pack_<a|b>;operands=<bf16|f16|f32|i8|u8>;memory=<host|device>;backend=hip-gfx950
 class MatmulPackBRecipe final : public rt::KernelRecipe {
 public:
-  explicit MatmulPackBRecipe(OperandClass packed);
+  explicit MatmulPackBRecipe(OperandClass packed, PackSide side = PackSide::B);
   [[nodiscard]] std::string_view id() const override { return id_; }
   [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
   [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
   [[nodiscard]] OperandClass operands() const { return packed_; }
+  [[nodiscard]] PackSide side() const { return side_; }
 
 private:
   OperandClass packed_;
+  PackSide side_;
   std::string id_;
 };
 
 // vecops::matmul_packed_b for one class of a (fp32 rows are rounded to bf16 against a bf16 pack; the i8 class
 // takes signed and unsigned bytes, AMX_I8I32<uint8_t, int8_t> being what the compensated pack is for):
 //   vecops::matmul_packed_b;operands=<bf16|f32|i8>;memory=<host|device>;backend=hip-gfx950
+// With side A the same for vecops::matmul_packed_a and the class of b; `packed_unsigned` marks the recipe of the 8-bit
+// class that serves PackedType = UInt8:  ...;operands=i8;packed=u8;memory=...; `f32_compute` the recipe of the fp32
+// class that serves ComputeType = Float32 (an fp32-packed operand, products in fp32):  ...;operands=f32;compute=f32;...
 class MatmulPackedBRecipe final : public rt::KernelRecipe {
 public:
-  explicit MatmulPackedBRecipe(OperandClass operands);
+  explicit MatmulPackedBRecipe(OperandClass operands, PackSide side = PackSide::B, bool packed_unsigned = false,
+                               bool f32_compute = false);
   [[nodiscard]] std::string_view id() const override { return id_; }
   [[nodiscard]] rt::Status match(const rt::KernelCall& call) const override;
   [[nodiscard]] rt::Result<rt::BoundKernelRecipe> bind(const rt::KernelCall& call) const override;
   [[nodiscard]] OperandClass operands() const { return operands_; }
+  [[nodiscard]] PackSide side() const { return side_; }
+  [[nodiscard]] bool packed_unsigned() const { return packed_unsigned_; }
+  [[nodiscard]] bool f32_compute() const { return f32_compute_; }
 
 private:
   OperandClass operands_;
+  PackSide side_;
+  bool packed_unsigned_;
+  bool f32_compute_;
   std::string id_;
 };
 
@@ -218,6 +245,8 @@ std::shared_ptr<rt::Operator> make_matmul_w8a16_group_operator(const std::filesy
 std::shared_ptr<rt::Operator> make_matmul_fused_operator(const std::filesystem::path& artifact_directory);
 std::shared_ptr<rt::Operator> make_matmul_pack_b_operator(const std::filesystem::path& artifact_directory);
 std::shared_ptr<rt::Operator> make_matmul_packed_b_operator(const std::filesystem::path& artifact_directory);
+std::shared_ptr<rt::Operator> make_matmul_pack_a_operator(const std::filesystem::path& artifact_directory);
+std::shared_ptr<rt::Operator> make_matmul_packed_a_operator(const std::filesystem::path& artifact_directory);
 std::shared_ptr<rt::Operator> make_matmul_runtime_quant_operator(const std::filesystem::path& artifact_directory);
 
 }  // namespace vecops::hip

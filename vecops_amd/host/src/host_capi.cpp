@@ -254,6 +254,8 @@ void* vecops_hip_host_operator_create(const char* operator_name, const char* art
   else if (name == vecops::hip::kMatmulFusedName) op = vecops::hip::make_matmul_fused_operator(artifact_directory);
   else if (name == vecops::hip::kMatmulPackBName) op = vecops::hip::make_matmul_pack_b_operator(artifact_directory);
   else if (name == vecops::hip::kMatmulPackedBName) op = vecops::hip::make_matmul_packed_b_operator(artifact_directory);
+  else if (name == vecops::hip::kMatmulPackAName) op = vecops::hip::make_matmul_pack_a_operator(artifact_directory);
+  else if (name == vecops::hip::kMatmulPackedAName) op = vecops::hip::make_matmul_packed_a_operator(artifact_directory);
   else if (name == vecops::hip::kMatmulRuntimeQuantName) op = vecops::hip::make_matmul_runtime_quant_operator(artifact_directory);
   else return nullptr;
   return new Handle{std::move(op)};

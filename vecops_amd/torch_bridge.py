@@ -36,8 +36,13 @@ SIGNATURES = {
     "vecops::matmul_fused": ([("a", "in"), ("b", "in"), ("c_in", "in?"), ("row_scales", "in?"),
                               ("column_scales", "in?"), ("activation", "int"), ("scale", "float"), ("shift", "float"),
                               ("clamp_lo", "float"), ("clamp_hi", "float"), ("c", "out")], {}),
-    "vecops::matmul_pack_b": ([("b", "in"), ("a_zero_point", "int"), ("packed", "out"), ("compensation", "out?")], {}),
-    "vecops::matmul_packed_b": ([("a", "in"), ("packed_b", "in"), ("c_in", "in?"), ("c", "out")], {}),
+    "vecops::matmul_pack_b": ([("b", "in"), ("a_zero_point", "int"), ("packed", "out"), ("compensation", "out?")],
+                              {"ComputeType": "dtype"}),
+    "vecops::matmul_packed_b": ([("a", "in"), ("packed_b", "in"), ("c_in", "in?"), ("c", "out")],
+                                {"PackedType": "dtype", "ComputeType": "dtype"}),
+    "vecops::matmul_pack_a": ([("a", "in"), ("packed", "out")], {"ComputeType": "dtype"}),
+    "vecops::matmul_packed_a": ([("packed_a", "in"), ("b", "in"), ("c_in", "in?"), ("c", "out")],
+                                {"PackedType": "dtype", "ComputeType": "dtype"}),
     "vecops::matmul_runtime_quant": ([("a", "in"), ("b", "in"), ("multipliers", "in"), ("zero_point", "int"),
                                       ("row_scales", "in"), ("column_scales", "in"), ("correction", "in?"),
                                       ("c", "out")], {}),
