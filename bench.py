@@ -343,7 +343,8 @@ def bench_bf16_gemm_packed(dev, steps, warmup):
             "(vecops_hip_pack_b, not timed), fp32 accumulate, bf16 out", "value": tflops, "unit": "TFLOP/s",
             "ms_per_step": t["wall_ms"], "dtype": "bf16",
             "roofline": _roofline("mfma", tflops, PEAK_BF16_TFLOPS, "TFLOP/s",
-                                  kernel=f"vecops_hip tile_gemm_packed_b_kernel<bf16> family {family}",
+                                  kernel=("vecops_hip tile_gemm_packed16_kernel<bf16>" if family == "tile_256"   # (aligned A, whole K tiles)
+                                          else "vecops_hip tile_gemm_packed_b_kernel<bf16>") + f" family {family}",
                                   algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=3 * 2 * n * n,
                                   **_traffic("bf16_packed"), **_timing_fields(t))}
 

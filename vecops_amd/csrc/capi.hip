@@ -843,6 +843,8 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     if (!wide_tile_serves(pr) || !launch_tile_gemm_i8_wide_serves(p, mode, pr.packed_b))
       return fail(ST_INVALID, "matmul: the plan's family tile_256x352 cannot serve this call");
     e = launch_tile_gemm_i8_wide(p, pr.packed_b, stream);
+  } else if (pr.packed_b && launch_tile_gemm_packed16_serves(pr.src, p, tile_m, tile_n)) {
+    e = launch_tile_gemm_packed16(pr.src, p, stream);
   } else if (pr.packed_b) {
     const int a_mode = plan.vector_a == 0 ? 0 : ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr, pr.a, pr.a.rs)) ? 2 : 1;
     e = launch_tile_gemm_packed_b(pr.src, p, tile_m, tile_n, a_mode, stream);

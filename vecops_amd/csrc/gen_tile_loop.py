@@ -47,7 +47,10 @@ PITCH_TR = 512      # bytes between the k rows of a B tile kept as it lies in me
 
 def fragment_reads(tr, st, ks, to_set):
     """The reads of k-step ks of stage st into fragment set to_set, in the order the matrix instructions consume
-    them: A block 0, every B block, the other A blocks."""
+    them: A block 0, every B block, the other A blocks.  tr: False (B K-contiguous, swizzled rows of 128 bytes), True
+    (B as [k][n], transposing reads) or "pk" (B prepacked and kept in its pack order: [panel of 32 rows][k-step of two
+    chunks][chunk half][row][16 bytes]; a wavefront's column block j lies in its panel j / 2, rows 16 (j % 2) .. + 15,
+    and the lane's part of the address - its chunk and row - is in the one base register)."""
     out = []
 
     def a_read(i):
@@ -55,7 +58,9 @@ def fragment_reads(tr, st, ks, to_set):
         out.append(f"ds_read_b128 {fa(to_set, i)}, %[la{st}{q}] offset:{i * 2048}")
 
     def b_read(j):
-        if tr:
+        if tr == "pk":
+            out.append(f"ds_read_b128 {fb(to_set, j)}, %[lb{st}0] offset:{(j >> 1) * 4096 + ks * 2048 + (j & 1) * 256}")
+        elif tr:
             off = (j & 1) * 32 + ks * 32 * PITCH_TR
             out.append(f"ds_read_b64_tr_b16 {fb_half(to_set, j, 0)}, %[lb{st}{j >> 1}] offset:{off}")
             out.append(f"ds_read_b64_tr_b16 {fb_half(to_set, j, 1)}, %[lb{st}{j >> 1}] offset:{off + 4 * PITCH_TR}")
@@ -80,7 +85,7 @@ def loads(tr, st):
                     [f"buffer_load_dwordx4 %[ra{p}], s[80:83], %[ka] offen lds"]))
     for p in range(8):
         m0 = f"s_add_u32 m0, %[m0w], {st * STAGE + B_TILE + p * 4096}"
-        if tr:
+        if tr is True:
             pre = [m0] if p == 0 else [m0, "s_add_u32 s88, s88, %[pb]"]
             if p == 0:
                 pre.append("s_mov_b32 s88, %[kb]")
@@ -130,7 +135,7 @@ def k_tile(tr, st):
         out.append("s_barrier")
     # k-step 1
     reads = fragment_reads(tr, st ^ 1, 0, 0)
-    at = spread(len(reads), 24, first=1) if not tr else spread(len(reads), 36, first=1)
+    at = spread(len(reads), 24, first=1) if tr is not True else spread(len(reads), 36, first=1)
     ld = loads(tr, st)
     every = int(os.environ.get("GEN_LOAD_EVERY", "4"))
     ld_at = {every * i: i for i in range(16)}   # load i straddles matrix instruction every * i
@@ -341,6 +346,8 @@ def main():
     w(as_macro("VECOPS_LOOP256_K", loop(False)))
     w("\n")
     w(as_macro("VECOPS_LOOP256_TR", loop(True)))
+    w("\n// VECOPS_LOOP256_PK: B prepacked (vecops_hip_pack_b) and kept in its pack order in LDS.\n")
+    w(as_macro("VECOPS_LOOP256_PK", loop("pk")))
     w("\n// The K loop of the 256 x 352 tile (8-bit operands, both K-contiguous): see gen_tile_loop.py.\n")
     w(as_macro("VECOPS_LOOP352_K", wide_loop()))
     w("\n// its 88 accumulator quads: 64 in accumulation registers, 24 in vector registers\n")

@@ -1705,7 +1705,8 @@ __device__ __forceinline__ void store_accumulators(const TileGemmParams& p, char
 //                     (A's is 128), part_b (TR) the offset between B's eight loads of a K tile
 //   nk                K tiles to multiply
 #include "tile_loop_asm.inc"
-template <int SRC, bool TR, typename ACC>
+// B_MODE: 0 B K-contiguous in LDS, 1 B as [k][n] (transposing reads), 2 B prepacked and kept in its pack order.
+template <int SRC, int B_MODE, typename ACC>
 __device__ __forceinline__ void asm_k_loop(ACC& acc, const uint32_t (&lds_a)[2][4], const uint32_t (&lds_b)[2][4],
                                            const uint32_t (&rows_a)[8], const uint32_t (&rows_b)[8], const u32x4& desc_a,
                                            const u32x4& desc_b, uint32_t m0_wave, uint32_t k_a, uint32_t k_b, uint32_t step_b,
@@ -1736,7 +1737,11 @@ __device__ __forceinline__ void asm_k_loop(ACC& acc, const uint32_t (&lds_a)[2][
                  [db0] "s"(db[0]), [db1] "s"(db[1]), [db2] "s"(db[2]), [db3] "s"(db[3]),                                \
                  [m0w] "s"(m0_wave), [sb] "s"(step_b), [pb] "s"(part_b)                                                 \
                : "memory", "m0", "scc", VECOPS_LOOP256_CLOBBERS)
-  if constexpr (TR) {
+  if constexpr (B_MODE == 2) {
+    if constexpr (SRC == SRC_F16) VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_PK("v_mfma_f32_16x16x32_f16"));
+    else if constexpr (SrcTraits<SRC>::kInt) VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_PK("v_mfma_i32_16x16x64_i8"));
+    else VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_PK("v_mfma_f32_16x16x32_bf16"));
+  } else if constexpr (B_MODE == 1) {
     static_assert(SRC == SRC_BF16 || SRC == SRC_F16, "transposing LDS reads move 16-bit elements");
     if constexpr (SRC == SRC_F16) VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_TR("v_mfma_f32_16x16x32_f16"));
     else VECOPS_LOOP256_STATEMENT(VECOPS_LOOP256_TR("v_mfma_f32_16x16x32_bf16"));
@@ -2044,11 +2049,11 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
       if constexpr (load_is_ntr(LOAD_B)) {
         const uint32_t step_b = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(64 * stager_b.ks * T::kSrcBytes));
         const uint32_t rows_b[8] = {stager_b.chunk_bytes, 0, 0, 0, 0, 0, 0, 0};
-        asm_k_loop<SRC, true>(acc, base_a, base_b, stager_a.row_bytes, rows_b, stager_a.tile_buf,
+        asm_k_loop<SRC, 1>(acc, base_a, base_b, stager_a.row_bytes, rows_b, stager_a.tile_buf,
                               tile_buffer_words(stager_b.tile_base), m0_wave, kt2 * 128u, kt2 * step_b, step_b,
                               stager_b.part_offset(1), nk);
       } else {
-        asm_k_loop<SRC, false>(acc, base_a, base_b, stager_a.row_bytes, stager_b.row_bytes, stager_a.tile_buf,
+        asm_k_loop<SRC, 0>(acc, base_a, base_b, stager_a.row_bytes, stager_b.row_bytes, stager_a.tile_buf,
                                stager_b.tile_buf, m0_wave, kt2 * 128u, kt2 * 128u, 128u, 0u, nk);
       }
     } else {

@@ -200,6 +200,10 @@ hipError_t launch_grouped_class(const GroupedTables& t, int tile, int mode, hipS
   if (tile == 128) return go(std::integral_constant<int, 2>{});
   return go(std::integral_constant<int, 1>{});
 }
+// The 256 x 256 tile on a prepacked B with the written-out K loop (tile_gemm_packed16.hip): whether it serves a
+// launch that the plan gave these tile extents, and the launch.
+bool launch_tile_gemm_packed16_serves(int src, const TileGemmParams& p, int tile_m, int tile_n);
+hipError_t launch_tile_gemm_packed16(int src, const TileGemmParams& p, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_bf16(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_i8(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_i8_flip(const GroupedTables& t, int tile, int mode, hipStream_t stream);
