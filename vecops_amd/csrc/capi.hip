@@ -237,10 +237,11 @@ constexpr int kStreamGroupsPerUnit = 2;  // workgroups of 4 wavefronts per compu
 // the pricing their kernels were calibrated with: 0.85, rounds of 256, and the margin of the rectangles (8 x 777 x
 // 1000 x 3001 64 us on 128x256 tiles against 73.5 on 128x128; fp32 memory 2048^3 32 us on 128x128 against 43).
 // Where the loads write LDS themselves the 256x256 tile runs its written-out K loop on the 16x16 matrix instructions,
-// a tenth faster than before, and the smaller tiles are priced against that: bf16 4096^3 94 / 133 / 130 / 113 us,
-// int8 4096^3 59 / 82 / 83 / 70 (`bench.py --only families`, `--only rule_check`).
+// a tenth faster than before, and the smaller tiles are priced against that: bf16 4096^3 93 / 122 / 118 / 114 us (the
+// rectangles on the 16x16 shapes; 133 / 130 before), int8 4096^3 58 / 75 / 77 / 70 (`bench.py --only families`,
+// `--only rule_check`).
 constexpr int64_t kQuality256x128 = 800, kQuality128 = 900, kQuality128Int8 = 970, kQuality128Staged = 850;
-constexpr int64_t kQuality256x128Direct = 710, kQuality128Direct = 830, kQuality128Int8Direct = 850;
+constexpr int64_t kQuality256x128Direct = 780, kQuality128Direct = 830, kQuality128Int8Direct = 850;
 
 // Every operand class but the unsigned bytes, with K contiguous on both sides, no C input, one side <= 16 rows, the
 // other >= 512 (vecops' small-vector leaves serve every atom, matmul/details/kernel/amx/Backend.h:767-992)

@@ -442,14 +442,15 @@ __device__ __forceinline__ void mfma_step16(typename AccQuad<SrcTraits<SRC>::kIn
 // tiles 1024 x 4096 x 4096 bf16 45.6 against 49.5 us, int8 28.9 against 31.8, int8 2048 x 11008 x 4096 97.6 against
 // 104.7, bf16 2048^3 26.6 against 28.4; 64x64 tiles 512 x 4096 x 4096 33.2 against 36.9 - the short shape draws less
 // power per multiply-add (a loop of nothing but MFMAs sustains 2.06 against 1.75 PFLOP/s on real operands) and its
-// loop below has no address arithmetic.  The 256-row and 256-column tiles stay on 32x32: their 128 to 256
-// accumulator registers need the accumulation half of the register file, where the compiler does not tie an
-// MFMA's result to its addend and permutes the accumulators back at the loop's head (a hundred copies per K tile);
-// with the MFMAs written out as tied instruction text the 256x256 tile gained 1.5-3.5 % for bf16 and lost 4.6 % for
-// int8, and the compiler's hazard tracking does not see through such text - not worth it.  A tile of at most 128x128
-// fits two wavefronts per SIMD, where MFMAs accumulate in place in vector registers.
+// loop below has no address arithmetic.  The rectangular tiles (256x128, 128x256: 32 quads a wavefront) take the
+// short shape too: bf16 4096^3 required of them 119 against 132 us, 1536 x 11008 x 4096 164 against 182, 768 x 4096 x
+// 4096 53 against 59.  The 256x256 tile's 256 accumulator registers need the accumulation half of the register file,
+// where the compiler does not tie an MFMA's result to its addend and permutes the accumulators back at the loop's
+// head (a hundred copies per K tile): on the compiler's loop it stays on 32x32, and takes the 16x16 shapes only under
+// the written-out loop (asm_k_loop).  A tile of at most 128x128 fits two wavefronts per SIMD, where MFMAs accumulate
+// in place in vector registers.
 template <int SRC, int WM, int WN>
-constexpr bool kShortMfma = SRC != SRC_F32 && WM * WN <= 4;
+constexpr bool kShortMfma = SRC != SRC_F32 && WM * WN <= 8;
 
 // The accumulators of one wavefront: WM x WN blocks of 32x32 elements of C, held either as one 32x32 MFMA
 // result per block (M16 = false) or as its four 16x16 quadrants (M16 = true).  Both shapes are issued with the
@@ -475,7 +476,7 @@ struct Accumulators {
   // and stay there until the epilogue takes them one by one: left to itself the compiler copies all 256 values into
   // vector registers ahead of the branch between the epilogue's paths, spills what does not fit, and reloaded one
   // spilled value wrongly (ROCm 7.2).  The empty statement pins a quad to its accumulation registers at its use.
-  static constexpr bool kPinned = M16 && WM * WN > 4;
+  static constexpr bool kPinned = M16 && WM * WN > 8;
   template <int I, int J, int Q>
   __device__ __forceinline__ Quad quad() const {
     if constexpr (M16) {
@@ -1788,8 +1789,8 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
   // The 256x256 tile on the 16x16 shapes runs its K loop as a written-out instruction stream (asm_k_loop): its 64
   // accumulator quads fill the accumulation registers, where the compiler's own loop copies them about.
   constexpr bool ASM_LOOP = M16 && WM == 4 && WN == 4;
-  static_assert(!M16 || WM * WN <= 4 || (ASM_LOOP && load_is_dma(LOAD_A) && load_is_dma(LOAD_B) && WAVES_M == 2 && WAVES_N == 2),
-                "the 16x16 shapes: small tiles, or the 256x256 tile fed by loads that write LDS");
+  static_assert(!M16 || WM * WN <= 8 || (ASM_LOOP && load_is_dma(LOAD_A) && load_is_dma(LOAD_B) && WAVES_M == 2 && WAVES_N == 2),
+                "the 16x16 shapes: tiles up to 256x128, or the 256x256 tile fed by loads that write LDS");
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
