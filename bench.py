@@ -453,6 +453,9 @@ RULE_CHECK_SHAPES = [
     ("bf16", 3000, 3000, 3000), ("bf16", 1536, 11008, 4096),
     ("int8", 2048, 11008, 4096), ("int8", 4096, 4096, 4096), ("int8", 1024, 4096, 4096), ("int8", 768, 3072, 12288),
     ("int8", 512, 1024, 8192),
+    # the band of 32 to 256 tiles of 128 x 128 (one workgroup per compute unit at most)
+    ("bf16", 640, 4096, 4096), ("bf16", 896, 4096, 4096), ("bf16", 1024, 2048, 8192), ("bf16", 384, 3072, 8192),
+    ("bf16", 256, 4096, 4096), ("bf16", 1024, 4096, 6144), ("bf16", 128, 8192, 8192), ("int8", 768, 4096, 4096),
 ]
 
 

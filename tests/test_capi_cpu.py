@@ -102,8 +102,12 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1
     rc, p = _plan(_operand(capi.BF16, (8192, 512)), _operand(capi.BF16, (8192, 512)), _operand(capi.F32, (8192, 8192)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"      # from eight K tiles on the big tile is ahead again
-    # 128 tiles of 128x128 would leave every other compute unit idle and the rest with one workgroup: 512 of 64x64
+    # 128 tiles of 128x128 leave every other compute unit idle, but a lone workgroup of the four-stage kernel does not
+    # wait out its loads (25 us against 28 for 512 tiles of 64x64); operands that kernel does not serve - here a K
+    # that is no whole number of K tiles - still take the small tiles
     rc, p = _plan(_operand(capi.BF16, (512, 4096)), _operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (512, 4096)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1
+    rc, p = _plan(_operand(capi.BF16, (512, 4104)), _operand(capi.BF16, (4096, 4104)), _operand(capi.BF16, (512, 4096)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 1
     rc, p = _plan(_operand(capi.BF16, (1024, 4096)), _operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (1024, 4096)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
@@ -132,41 +136,36 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k > 1
     assert p.workspace_bytes == p.split_k * 255 * 63 * 4
     assert p.vector_a == 1                                   # rows need not be 16-byte aligned for 16-byte loads
-    # 128 to 200 tiles of 128 x 128 and twenty K tiles per part or more: K split so that two workgroups sit on
-    # (nearly) every compute unit; shorter K and int8's 128-element K tiles keep the unsplit small tiles
-    for (m, n, k), family, split in (((640, 4096, 4096), "tile_128", 3), ((768, 4096, 4096), "tile_128", 2),
-                                     ((1024, 2048, 8192), "tile_128", 4), ((768, 3072, 12288), "tile_128", 3),
-                                     ((512, 4096, 4096), "tile_64", 1), ((640, 4096, 2048), "tile_64", 1),
-                                     ((896, 4096, 4096), "tile_128", 1)):
+    # 32 to 256 tiles of 128 x 128, operands the four-stage kernel serves (both K-contiguous and aligned, whole K
+    # tiles): at most one workgroup per compute unit - whole from 96 tiles on (in two parts where the units allow and
+    # the split rule's costs favour it), K split to fill the units once below that; more than half but at most 160
+    # tiles and sixty K tiles per part keep the two-stage kernel's split (two co-resident workgroups on every unit)
+    for (m, n, k), family, split in (((640, 4096, 4096), "tile_128", 1), ((768, 4096, 4096), "tile_128", 1),
+                                     ((1024, 2048, 8192), "tile_128", 2), ((768, 3072, 12288), "tile_128", 3),
+                                     ((512, 4096, 4096), "tile_128", 1), ((640, 4096, 2048), "tile_128", 1),
+                                     ((896, 4096, 4096), "tile_128", 1), ((2048, 2048, 2048), "tile_128", 1),
+                                     ((512, 2048, 16384), "tile_128", 4), ((384, 3072, 8192), "tile_128", 3),
+                                     ((512, 3072, 8192), "tile_128", 2), ((512, 3072, 4096), "tile_128", 1),
+                                     ((256, 4096, 4096), "tile_128", 4), ((512, 1024, 8192), "tile_128", 8),
+                                     ((128, 8192, 8192), "tile_128", 4), ((384, 2048, 4096), "tile_128", 5),
+                                     ((1024, 4096, 11008), "tile_128", 1), ((1024, 4096, 6144), "tile_128", 1),
+                                     ((1024, 4096, 4096), "tile_128", 1), ((896, 4096, 11008), "tile_128", 1)):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
         assert p.workspace_bytes == (split * m * n * 4 if split > 1 else 0)
-    # ... and from 32 tiles on, one part fewer where that reaches twenty K tiles per part
-    for (m, n, k), family, split in (((512, 2048, 16384), "tile_128", 8), ((384, 3072, 8192), "tile_128", 6),
-                                     ((512, 3072, 8192), "tile_128", 5), ((512, 3072, 4096), "tile_64", 1),
-                                     ((256, 4096, 4096), "tile_64", 1), ((512, 1024, 8192), "tile_128", 6),
-                                     ((128, 8192, 8192), "tile_128", 6)):
-        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
+    # operands it does not serve keep the two-stage kernel's rules: B as [K,N] (strides (1, N)) - K split so that two
+    # workgroups sit on (nearly) every unit, from twenty K tiles per part; the big tile in four parts for 64 of them and
+    # a long K
+    for (m, n, k), family, split in (((768, 4096, 4096), "tile_128", 2), ((512, 4096, 4096), "tile_64", 1),
+                                     ((1024, 4096, 11008), "tile_256", 4), ((1024, 4096, 6144), "tile_128", 2),
+                                     ((512, 2048, 16384), "tile_128", 8)):
+        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k), strides=(1, n)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
-    # ... and up to 256 tiles in two parts, from forty K tiles per part
-    # (with 160 K tiles or more those 256 tiles become 64 of 256 x 256 in four parts)
-    for (m, n, k), family, split in (((1024, 4096, 11008), "tile_256", 4), ((1024, 4096, 6144), "tile_128", 2),
-                                     ((1024, 4096, 4096), "tile_128", 1), ((896, 4096, 4096), "tile_128", 1),
-                                     ((896, 4096, 11008), "tile_256", 4)):
-        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
+    for (m, n, k), family, split in (((1024, 4096, 11008), "tile_128", 1), ((1024, 4096, 8192), "tile_128", 1),
+                                     ((768, 4096, 4096), "tile_128", 1), ((768, 3072, 12288), "tile_128", 1),
+                                     ((512, 2048, 16384), "tile_128", 4), ((512, 1024, 8192), "tile_64", 2)):
+        rc, p = _plan(_operand(capi.I8, (m, k)), _operand(capi.I8, (n, k)), _operand(capi.I32, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
-    rc, p = _plan(_operand(capi.I8, (1024, 11008)), _operand(capi.I8, (4096, 11008)), _operand(capi.I32, (1024, 4096)))
-    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 2
-    rc, p = _plan(_operand(capi.I8, (1024, 8192)), _operand(capi.I8, (4096, 8192)), _operand(capi.I32, (1024, 4096)))
-    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1
-    rc, p = _plan(_operand(capi.I8, (768, 4096)), _operand(capi.I8, (4096, 4096)), _operand(capi.I32, (768, 4096)))
-    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 1
-    rc, p = _plan(_operand(capi.I8, (768, 12288)), _operand(capi.I8, (3072, 12288)), _operand(capi.I32, (768, 3072)))
-    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 3
-    rc, p = _plan(_operand(capi.I8, (512, 16384)), _operand(capi.I8, (2048, 16384)), _operand(capi.I32, (512, 2048)))
-    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 6
-    rc, p = _plan(_operand(capi.I8, (512, 8192)), _operand(capi.I8, (1024, 8192)), _operand(capi.I32, (512, 1024)))
-    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64" and p.split_k == 2    # exactly 128 workgroups: two parts just pay (24 -> 16 us)
     # two rounds of 128 x 128 tiles and eight more: the last column of tiles is a product of its own (64 x 64 tiles, K in
     # five parts), the rest fills two rounds; a required family runs the product whole
     big_n = (_operand(capi.BF16, (1536, 4096)), _operand(capi.BF16, (11008, 4096)), _operand(capi.BF16, (1536, 11008)))

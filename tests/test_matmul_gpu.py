@@ -871,12 +871,13 @@ def test_w8a16_rejects_bad_arguments(device):
     assert e.value.code == 1
 
 
-@pytest.mark.parametrize("kind,m,n,k", [("bf16", 640, 4096, 4096), ("bf16", 768, 3072, 12288), ("bf16", 1000, 2000, 8200),
-                                        ("i8", 768, 3072, 12288), ("i8", 700, 4000, 8192)])
-def test_mid_band_k_split(device, oracle, kind, m, n, k):
-    """128 to 200 tiles of 128 x 128 with a long K: the rule table splits K two to four ways on 128 x 128 tiles
-    (partial sums in the workspace, summed in the order of the parts).  Against the oracle (int8: exact), with a C
-    input; the entry point that allocates nothing runs the same problem unsplit and agrees within the bound."""
+@pytest.mark.parametrize("kind,m,n,k,split", [("bf16", 640, 4096, 4096, 1), ("bf16", 768, 3072, 12288, 3), ("bf16", 1000, 2000, 8200, 4),
+                                              ("i8", 768, 3072, 12288, 1), ("i8", 700, 4000, 8192, 1), ("i8", 700, 4000, 8208, 2)])
+def test_mid_band_k_split(device, oracle, kind, m, n, k, split):
+    """128 to 200 tiles of 128 x 128 with a long K: 128 x 128 tiles, whole on the four-stage kernel where it serves
+    (one workgroup per compute unit) and with K split two to four ways otherwise - a K that is no whole number of K
+    tiles, or many idle units and a very long K (partial sums in the workspace, summed in the order of the parts).
+    Against the oracle (int8: exact), with a C input; the entry point that allocates nothing agrees within the bound."""
     import torch
     from vecops_amd import capi
     if kind == "bf16":
@@ -891,7 +892,7 @@ def test_mid_band_k_split(device, oracle, kind, m, n, k):
         c = torch.full((m, n), -1, dtype=torch.int32, device=device)
     tci = torch.from_numpy(cin).to(device)
     plan = capi.plan_matmul(ta, tb, c, c_in=tci)
-    assert capi.FAMILY_NAMES[plan.family] == "tile_128" and 2 <= plan.split_k <= 4
+    assert capi.FAMILY_NAMES[plan.family] == "tile_128" and plan.split_k == split
     capi.matmul(ta, tb, c, c_in=tci)
     alone = torch.empty_like(c)
     capi.matmul_static_workspace(ta, tb, alone, c_in=tci)
@@ -910,9 +911,9 @@ def test_mid_band_k_split(device, oracle, kind, m, n, k):
 
 @pytest.mark.parametrize("m,n,k,pad", [(768, 3072, 12288, 0), (768, 3072, 12289, 15)])
 def test_mid_band_k_split_with_dequantisation(device, m, n, k, pad):
-    """The K split of the mid band under the dequantising epilogue (applied by the kernel that sums the parts): bit
-    for bit (float(acc + corr) * rs) * cs.  Rows padded to 16 bytes around an odd K take the split too, and the
-    workspace query, which is told extents only, must have answered for them."""
+    """The mid band under the dequantising epilogue - unsplit on the four-stage kernel, and split (the epilogue applied
+    by the kernel that sums the parts) for rows padded to 16 bytes around an odd K: bit for bit
+    (float(acc + corr) * rs) * cs.  The workspace query, which is told extents only, must have answered for the split."""
     import torch
     from vecops_amd import capi
     a, b = synth.int8_sym(1, (m, k)), synth.int8_sym(2, (n, k))
@@ -921,7 +922,8 @@ def test_mid_band_k_split_with_dequantisation(device, m, n, k, pad):
     ta = torch.zeros(m, k + pad, dtype=torch.int8, device=device)
     tb = torch.zeros(n, k + pad, dtype=torch.int8, device=device)
     ta[:, :k], tb[:, :k] = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
-    assert capi.lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k) >= 2 * m * n * 4
+    # (whole K tiles and aligned rows run unsplit on the four-stage kernel; the odd K keeps the split)
+    assert capi.lib().vecops_hip_matmul_i8_dequant_workspace(m, n, k) >= (2 * m * n * 4 if pad else 0)
     c = torch.full((m, n), float("nan"), device=device)
     capi.matmul_i8_dequant(ta[:, :k], tb[:, :k], torch.from_numpy(rs).to(device), torch.from_numpy(cs).to(device), c,
                            correction=torch.from_numpy(corr).to(device))

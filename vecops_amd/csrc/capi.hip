@@ -279,6 +279,19 @@ struct RuleConstants {
   //    4096, 512^3 in fp32: `bench.py --only rule_check`)
   int64_t split_min_k_tiles = 8, split_k_tiles_per_part = 4, split_max = 64;
   int64_t k_tile_ns = 300, k_tile_ns_f32 = 1000, split_fixed_ns = 5000, split_ns_per_kb_num = 3, split_ns_per_kb_den = 4;
+  // -- 128x128 tiles that leave a compute unit at most one workgroup run the four-stage kernel (tile_gemm_deep128.hip),
+  //    from this many K tiles per workgroup on (rule_check, 1024 x 4096 x 4096)
+  int64_t deep_max_workgroups = 256, deep_min_k_tiles = 8;
+  // -- planning for that kernel (operands it serves): from deep_alone_from_tiles tiles of 128x128 on (three eighths of the
+  //    units) the tiles stay whole or split in two, whichever the split rule's costs favour, with deep_k_tile_ns per K
+  //    tile (a lone workgroup of this kernel walks a K tile in 0.3 us) and deep_fixed_ns per launch; between
+  //    deep_fill_from_tiles and that, K is split so that the parts fill the units once, if a part keeps
+  //    deep_fill_k_tiles_per_part K tiles.  Where more than half but at most deep_idle_tiles of the units would hold a
+  //    tile and a part of the two-stage kernel's split keeps deep_idle_k_tiles_per_part K tiles, that split stays (two
+  //    co-resident workgroups on every unit beat one on 56 % of them: bf16 768 x 3072 x 12288 63 against 71 us).
+  //    `bench.py --only rule_check`: 512 / 768 / 1024 x 4096 x 4096, 1024 x 4096 x 11008, 512 x 2048 x 16384.
+  int64_t deep_alone_from_tiles = 96, deep_fill_from_tiles = 32, deep_fill_k_tiles_per_part = 12;
+  int64_t deep_idle_tiles = 160, deep_idle_k_tiles_per_part = 60, deep_k_tile_ns = 300, deep_fixed_ns = 8000;
 };
 constexpr RuleConstants kRules{};
 
@@ -499,6 +512,10 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   }
   const int64_t ktile = k_tile_elements(pr.src);
   const int64_t k_tiles = (pr.k + ktile - 1) / ktile;
+  // operands the four-stage 128x128 kernel (tile_gemm_deep128.hip) serves: both K-contiguous, fetched by loads that
+  // write LDS, K in whole K tiles
+  const bool deep_ok = mode == MODE_KVEC_DMA && !pr.packed_b && pr.k % ktile == 0 && k_tiles >= kRules.deep_min_k_tiles &&
+                       (pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8);
   // At most four K tiles of 16-bit or 8-bit operands: the tile's life is its start-up and its stores, and
   // two or three 128x128 workgroups on a compute unit overlap one's stores with another's loads, which a
   // single big tile cannot (batch 8 of 3000x3000x17 to fp32: 93 us against 111; 8 x 1000x1000x100: 17.7
@@ -514,7 +531,8 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // nothing to overlap its start-up, barriers and stores with, while four times as many 64x64 tiles put two or
   // more on every unit (512 x 4096 x 4096: 28.7 us against 45.9; 1536^3: 18.0 against 20.7; 768 x 4096 x 4096:
   // 42.7 against 46.7; from 256 tiles on - 1024 x 4096 x 4096, 2048^3 - the bigger tile is ahead again).
-  else if (k_tiles > kRules.short_k_tiles_16bit && family == VECOPS_HIP_FAMILY_TILE_128 && pr.src != SRC_F32 &&
+  // (not where the four-stage 128x128 kernel serves: a lone workgroup of it does not wait out its loads)
+  else if (k_tiles > kRules.short_k_tiles_16bit && family == VECOPS_HIP_FAMILY_TILE_128 && pr.src != SRC_F32 && !deep_ok &&
            tiles(128) <= kRules.lonely_tiles_num * kComputeUnits / kRules.lonely_tiles_den) {
     family = VECOPS_HIP_FAMILY_TILE_64;
     tile_m = tile_n = 64;
@@ -535,13 +553,44 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // 11008 116 us -> 90, 896 x 4096 x 11008 114 -> 81, 1024 x 4096 x 6144 66 -> 58; int8 896 x 4096 x 11008 61 -> 52;
   // with thirty-two per part - bf16 1024 x 4096 x 4096, int8 ... x 8192 - the unsplit tiles are level or ahead).
   uint32_t band_split = 0;
+  bool deep_planned = false;
   if (direct && !pr.packed_b && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) && tiles(128) >= kComputeUnits / 8 &&
       tiles(128) <= kComputeUnits) {
-    int64_t parts = kRules.small_tile_workgroups_per_unit * kComputeUnits / tiles(128);
+    const int64_t count = tiles(128);
+    int64_t parts = kRules.small_tile_workgroups_per_unit * kComputeUnits / count;
     while (parts > kRules.band_min_parts && k_tiles / parts < kRules.band_k_tiles_per_part) --parts;
-    const int64_t least = tiles(128) > kRules.band_full_from_tiles ? kRules.band_k_tiles_per_part_full
-                                                                    : kRules.band_k_tiles_per_part;  // K tiles per part
-    if (k_tiles / parts >= least && static_cast<uint64_t>(parts) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
+    const int64_t least = count > kRules.band_full_from_tiles ? kRules.band_k_tiles_per_part_full
+                                                              : kRules.band_k_tiles_per_part;  // K tiles per part
+    const bool fits = static_cast<uint64_t>(parts) * pr.batch * pr.m * pr.n * 4u <= scratch_limit;
+    // Where the four-stage kernel serves, a workgroup alone on its unit is no longer the slow case (1024 x 4096 x 4096
+    // unsplit 31-34 us against 43 on the two-stage kernel, 768 x 4096 x 4096 27 against 38 in two parts, 512 x 4096 x
+    // 4096 25 against 28 on 64x64 tiles, 1024 x 4096 x 11008 79 against 84 on the big tile in four parts; int8
+    // 1024 x 4096 x 4096 21 against 28): at most one workgroup per unit, K split only to fill the units.
+    const bool idle_units_long_k = count > kComputeUnits / 2 && count <= kRules.deep_idle_tiles &&
+                                   k_tiles / parts >= kRules.deep_idle_k_tiles_per_part && fits;
+    if (deep_ok && count >= kRules.deep_alone_from_tiles && !idle_units_long_k) {
+      // whole, or in two parts where the units allow and the split rule's costs favour it
+      int64_t best_parts = 1;
+      if (2 * count <= kRules.deep_max_workgroups && k_tiles / 2 >= kRules.deep_min_k_tiles &&
+          2ull * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
+        const int64_t kb = pr.batch * pr.m * pr.n * 4 / 1024;
+        const int64_t whole_ns = k_tiles * kRules.deep_k_tile_ns + kRules.deep_fixed_ns;
+        const int64_t halves_ns = (k_tiles + 1) / 2 * kRules.deep_k_tile_ns + kRules.deep_fixed_ns + kRules.split_fixed_ns +
+                                  2 * kb * kRules.split_ns_per_kb_num / kRules.split_ns_per_kb_den;
+        if (halves_ns < whole_ns) best_parts = 2;
+      }
+      family = VECOPS_HIP_FAMILY_TILE_128;
+      band_split = static_cast<uint32_t>(best_parts);
+      deep_planned = true;
+    } else if (deep_ok && count >= kRules.deep_fill_from_tiles && count < kRules.deep_alone_from_tiles &&
+               k_tiles / (kRules.deep_max_workgroups / count) >= kRules.deep_fill_k_tiles_per_part &&
+               static_cast<uint64_t>(kRules.deep_max_workgroups / count) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
+      // few tiles and a long K: as many parts as fill the units once (512 x 2048 x 16384: 37 us in four parts against 46
+      // in eight parts of the two-stage kernel)
+      family = VECOPS_HIP_FAMILY_TILE_128;
+      band_split = static_cast<uint32_t>(kRules.deep_max_workgroups / count);
+      deep_planned = true;
+    } else if (k_tiles / parts >= least && fits) {
       family = VECOPS_HIP_FAMILY_TILE_128;
       band_split = static_cast<uint32_t>(parts);
     }
@@ -549,7 +598,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // 256 tiles of 128x128 that are 64 of 256x256, and a K of 160 tiles or more: the big tile in four parts puts one
   // workgroup of its (faster) loop on every unit (bf16 1024 x 4096 x 11008: 84 us against 89-92 for the two parts of
   // 128x128 tiles above and 116 unsplit; with a shorter K - 1024 x 4096 x 4096, 16 K tiles per part - it loses, 48 against 44).
-  if (direct && !pr.packed_b && band_split == 2 && tiles(256) * kRules.big_tile_parts == kComputeUnits &&
+  if (direct && !pr.packed_b && !deep_planned && band_split == 2 && tiles(256) * kRules.big_tile_parts == kComputeUnits &&
       k_tiles / kRules.big_tile_parts >= kRules.big_tile_k_tiles_per_part &&
       static_cast<uint64_t>(kRules.big_tile_parts) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
     family = VECOPS_HIP_FAMILY_TILE_256;
@@ -886,6 +935,11 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
   } else if (pr.packed_b) {
     const int a_mode = plan.vector_a == 0 ? 0 : ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr, pr.a, pr.a.rs)) ? 2 : 1;
     e = launch_tile_gemm_packed_b(pr.src, p, tile_m, tile_n, a_mode, stream);
+  } else if (tile_m == 128 && tile_n == 128 && p.k_tiles_per_split >= kRules.deep_min_k_tiles &&
+             static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.batch * p.split_k <= kRules.deep_max_workgroups &&
+             launch_tile_gemm_deep128_serves(pr.src, p, mode)) {
+    // at most one workgroup per compute unit: the four-stage kernel, whose loads run three K tiles ahead
+    e = launch_tile_gemm_deep128(pr.src, p, stream);
   } else switch (pr.src) {
     case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile_m, tile_n, mode, stream); break;
     case SRC_BF16: e = launch_tile_gemm_bf16(p, tile_m, tile_n, mode, stream); break;
@@ -1891,9 +1945,10 @@ int32_t vecops_hip_matmul_planned(const VecopsHipOperand* a, const VecopsHipOper
 
 uint64_t vecops_hip_matmul_i8_dequant_workspace(int64_t m, int64_t n, int64_t k) {
   // The plan depends on how the rows lie (16-byte aligned rows take other kernels, and with them other K splits),
-  // which this query is not told: the larger need of dense rows and of rows padded to 16 bytes.
+  // which this query is not told: the largest need of dense rows, of rows padded to 16 bytes and of rows that are not
+  // 16-byte aligned.
   uint64_t most = 0;
-  for (const int64_t ld : {k, (k + 15) & ~int64_t{15}}) {
+  for (const int64_t ld : {k, (k + 15) & ~int64_t{15}, k | 1}) {
     VecopsHipOperand a, b, c;
     make_operand(&a, reinterpret_cast<void*>(16), DT_I8, m, k, ld);
     make_operand(&b, reinterpret_cast<void*>(16), DT_I8, n, k, ld);

@@ -327,6 +327,102 @@ def wide_loop():
     return out
 
 
+# ---- the 128 x 128 tile with four LDS stages: one workgroup per compute unit, loads three K tiles ahead -----------
+# A wavefront owns 64 x 64 = 4 x 4 accumulator quads; a stage is 128 rows of A and 128 of B, 128 bytes each = 32 KiB,
+# four of them a ring.  With at most one such workgroup on a compute unit (256 tiles or fewer) nothing else hides the
+# latency of its loads: the two-stage loop of tile_gemm_kernel waits out every tile's loads there (0.67 us per K tile
+# of 0.25 us of matrix instructions).  K tile t lies in stage t % 4:
+#   k-step 0   multiplies fragment set 0, reads k-step 1 (same stage) into set 1
+#   wait for the loads of tile t + 1 (at most those of tile t + 2 still in flight), barrier: every wavefront has read
+#   stage (t - 1) % 4 for the last time and tile t + 1 has landed
+#   k-step 1   multiplies set 1, reads tile t + 1's k-step 0 into set 0, issues the eight loads of tile t + 3 into
+#              stage (t + 3) % 4
+# Fragment registers: set s, A block i at v[128 + 32 s + 4 i ..], B block j at v[144 + 32 s + 4 j ..].  LDS addresses:
+# stages 0 / 1 and 2 / 3 share base registers (la{pair}{q}); the odd stage of a pair lies 32 KiB up, in the offset.
+DEEP_STAGE = 32768
+DEEP_B = 16384
+
+
+def deep_fa(s, i):
+    r = 128 + 32 * s + 4 * i
+    return f"v[{r}:{r + 3}]"
+
+
+def deep_fb(s, j):
+    r = 144 + 32 * s + 4 * j
+    return f"v[{r}:{r + 3}]"
+
+
+def deep_reads(st, ks, to_set):
+    out = []
+    pair, odd = st >> 1, st & 1
+    order = [("a", 0)] + [("b", j) for j in range(4)] + [("a", i) for i in range(1, 4)]
+    for kind, f in order:
+        q = (2 * ks ^ f) & 3
+        if kind == "a":
+            out.append(f"ds_read_b128 {deep_fa(to_set, f)}, %[la{pair}{q}] offset:{odd * DEEP_STAGE + f * 2048}")
+        else:
+            out.append(f"ds_read_b128 {deep_fb(to_set, f)}, %[lb{pair}{q}] offset:{odd * DEEP_STAGE + f * 2048}")
+    return out
+
+
+def deep_k_tile(st):
+    out = ["s_cmp_gt_i32 %[left], 0",
+           "s_cselect_b32 s82, 0x7fffffff, 0",
+           "s_cselect_b32 s86, 0x7fffffff, 0",
+           "s_sub_u32 %[left], %[left], 1"]
+
+    def mfma(x, s):
+        i, j = x // 4, x % 4
+        c = i * 4 + j
+        return f"MFMA %[c{c}], {deep_fb(s, j)}, {deep_fa(s, i)}, %[c{c}]"
+    reads = deep_reads(st, 1, 1)
+    out.append("s_waitcnt lgkmcnt(0)")
+    for x in range(16):
+        out.append(mfma(x, 0))
+        if x < 8:
+            out.append(reads[x])
+    out += ["s_waitcnt vmcnt(8) lgkmcnt(0)", "s_barrier"]
+    reads = deep_reads((st + 1) & 3, 0, 0)
+    target = (st + 3) & 3
+    loads = []
+    for p in range(4):
+        loads.append((f"s_add_u32 m0, %[m0w], {target * DEEP_STAGE + p * 4096}",
+                      f"buffer_load_dwordx4 %[ra{p}], s[80:83], %[ka] offen lds"))
+    for p in range(4):
+        loads.append((f"s_add_u32 m0, %[m0w], {target * DEEP_STAGE + DEEP_B + p * 4096}",
+                      f"buffer_load_dwordx4 %[rb{p}], s[84:87], %[ka] offen lds"))
+    for x in range(16):
+        if x % 2 == 0:
+            out.append(loads[x // 2][0])
+        out.append(mfma(x, 1))
+        if x % 2 == 0:
+            out.append(loads[x // 2][1])
+        if 1 <= x <= 8:
+            out.append(reads[x - 1])
+    out.append("s_add_u32 %[ka], %[ka], 128")
+    return out
+
+
+def deep_loop():
+    out = []
+    for w in range(4):
+        out.append(f"s_mov_b32 s{80 + w}, %[da{w}]")
+        out.append(f"s_mov_b32 s{84 + w}, %[db{w}]")
+    out += deep_reads(0, 0, 0)
+    out.append("1:")
+    out += ["s_cmp_lt_u32 %[n], 4", "s_cbranch_scc1 2f"]
+    for st in range(4):
+        out += deep_k_tile(st)
+    out += ["s_sub_u32 %[n], %[n], 4", "s_branch 1b", "2:"]
+    for st in range(3):
+        out += [f"s_cmp_eq_u32 %[n], {st}", "s_cbranch_scc1 3f"]
+        out += deep_k_tile(st)
+    out.append("3:")
+    out += ["s_waitcnt vmcnt(0) lgkmcnt(0)", "s_nop 15", "s_nop 15"]
+    return out
+
+
 def as_macro(name, lines):
     text = f"#define {name}(MFMA) \\\n"
     body = []
@@ -355,6 +451,12 @@ def main():
       ", \\\n  ".join(", ".join(f'[c{x}] "+{"a" if x < 64 else "v"}"(t[{x}])' for x in range(r, r + 4)) for r in range(0, 88, 4)) + "\n")
     w("#define VECOPS_LOOP352_CLOBBERS \\\n  " + ", ".join(f'"s{r}"' for r in range(80, 89)) + ", \\\n  " +
       ", \\\n  ".join(", ".join(f'"v{r}"' for r in range(b, min(b + 16, 248))) for b in range(128, 248, 16)) + "\n")
+    w("\n// The K loop of the 128 x 128 tile on four LDS stages (one workgroup per compute unit): see gen_tile_loop.py.\n")
+    w(as_macro("VECOPS_LOOP128_DEEP", deep_loop()))
+    w("#define VECOPS_LOOP128_ACCUMULATORS(t) \\\n  " +
+      ", \\\n  ".join(", ".join(f'[c{x}] "+a"(t[{x // 4}][{x % 4}])' for x in range(r, r + 4)) for r in range(0, 16, 4)) + "\n")
+    w("#define VECOPS_LOOP128_CLOBBERS \\\n  " + ", ".join(f'"s{r}"' for r in range(80, 88)) + ", \\\n  " +
+      ", \\\n  ".join(", ".join(f'"v{r}"' for r in range(b, b + 16)) for b in range(128, 192, 16)) + "\n")
     w("\n// the accumulators as operands: quad x = t[x / 8][x % 8]\n")
     w("#define VECOPS_LOOP256_ACCUMULATORS(t) \\\n  " +
       ", \\\n  ".join(", ".join(f'[c{x}] "+a"(t[{x // 8}][{x % 8}])' for x in range(r, r + 4)) for r in range(0, 64, 4)) + "\n")
