@@ -456,6 +456,9 @@ RULE_CHECK_SHAPES = [
     # the band of 32 to 256 tiles of 128 x 128 (one workgroup per compute unit at most)
     ("bf16", 640, 4096, 4096), ("bf16", 896, 4096, 4096), ("bf16", 1024, 2048, 8192), ("bf16", 384, 3072, 8192),
     ("bf16", 256, 4096, 4096), ("bf16", 1024, 4096, 6144), ("bf16", 128, 8192, 8192), ("int8", 768, 4096, 4096),
+    # B stored [K,N] (the layout of the headline line)
+    ("bf16_kn", 1024, 4096, 4096), ("bf16_kn", 512, 4096, 4096), ("bf16_kn", 768, 3072, 12288), ("bf16_kn", 2048, 2048, 2048),
+    ("bf16_kn", 256, 4096, 4096),
 ]
 
 
@@ -471,9 +474,10 @@ def bench_rule_check(dev, steps, warmup):
     ws = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
     rows = []
     for kind, m, n, k in RULE_CHECK_SHAPES:
-        if kind == "bf16":
+        if kind in ("bf16", "bf16_kn"):
             a = torch.from_numpy(synth.bf16_round(synth.normal(1, (m, k), 0.02)).view(np.int16)).to(dev).view(torch.bfloat16)
             b = torch.from_numpy(synth.bf16_round(synth.normal(2, (n, k), 0.02)).view(np.int16)).to(dev).view(torch.bfloat16)
+            b = b.view(k, n).t() if kind == "bf16_kn" else b    # the same bits read as a [K,N] matrix
             c = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
         else:
             a = torch.from_numpy(synth.int8_sym(1, (m, k))).to(dev)

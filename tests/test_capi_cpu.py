@@ -153,13 +153,19 @@ def test_rule_table_known_answers():
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
         assert p.workspace_bytes == (split * m * n * 4 if split > 1 else 0)
-    # operands it does not serve keep the two-stage kernel's rules: B as [K,N] (strides (1, N)) - K split so that two
+    # 16-bit operands with B as [K,N] (strides (1, N)) are served too (the tile lies [k][n] in LDS) and plan alike
+    for (m, n, k), family, split in (((768, 4096, 4096), "tile_128", 1), ((512, 4096, 4096), "tile_128", 1),
+                                     ((1024, 4096, 11008), "tile_128", 1), ((1024, 4096, 6144), "tile_128", 1),
+                                     ((512, 2048, 16384), "tile_128", 4), ((768, 3072, 12288), "tile_128", 3)):
+        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k), strides=(1, n)), _operand(capi.BF16, (m, n)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
+    # operands it does not serve keep the two-stage kernel's rules: a K that is not whole K tiles - K split so that two
     # workgroups sit on (nearly) every unit, from twenty K tiles per part; the big tile in four parts for 64 of them and
     # a long K
-    for (m, n, k), family, split in (((768, 4096, 4096), "tile_128", 2), ((512, 4096, 4096), "tile_64", 1),
-                                     ((1024, 4096, 11008), "tile_256", 4), ((1024, 4096, 6144), "tile_128", 2),
-                                     ((512, 2048, 16384), "tile_128", 8)):
-        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k), strides=(1, n)), _operand(capi.BF16, (m, n)))
+    for (m, n, k), family, split in (((768, 4096, 4104), "tile_128", 2), ((512, 4096, 4104), "tile_64", 1),
+                                     ((1024, 4096, 11016), "tile_256", 4), ((1024, 4096, 6152), "tile_128", 2),
+                                     ((512, 2048, 16392), "tile_128", 8)):
+        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
     for (m, n, k), family, split in (((1024, 4096, 11008), "tile_128", 1), ((1024, 4096, 8192), "tile_128", 1),
                                      ((768, 4096, 4096), "tile_128", 1), ((768, 3072, 12288), "tile_128", 1),

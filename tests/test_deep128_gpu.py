@@ -1,5 +1,6 @@
 """The four-stage 128 x 128 kernel (tile_gemm_deep128.hip): what the library runs when a product gives a compute unit at
-most one 128 x 128 workgroup (256 workgroups or fewer, both operands K-contiguous and aligned, K in whole K tiles).
+most one 128 x 128 workgroup (256 workgroups or fewer, operands aligned and K-contiguous - or, 16-bit ones, B handed
+over as [K,N] -, K in whole K tiles).
 Checked against the oracle, against exact integer sums, and against the two-stage kernel of the same tile - which a
 K that is no whole number of K tiles, or more than 256 workgroups, still selects - on ragged extents, batches, K
 splits, C inputs, bf16 outputs and a transposed C."""
@@ -27,6 +28,34 @@ def test_deep_kernel_bf16_against_the_oracle(device, oracle, m, n, k, split):
     torch.cuda.synchronize()
     want = np.zeros((m, n), np.float32)
     oracle.matmul(a_bits, b_bits, want, acc_f64=True, c_bf16=False)
+    assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n,k,split", [(1024, 1024, 512, 1), (300, 520, 1024, 1), (513, 264, 576, 3), (128, 128, 512, 1),
+                                         (1000, 2000, 640, 1), (700, 904, 2048, 2), (1, 136, 512, 1), (100, 8, 512, 1),
+                                         (2000, 2048, 512, 1)])
+def test_deep_kernel_b_as_k_by_n(device, oracle, kind, m, n, k, split):
+    """B stored [K,N] and handed over as the strided [N,K] view (N a multiple of eight: the rows are 16-byte aligned):
+    the tile lies [k][n] in LDS and the fragment reads transpose.  bf16 against the oracle, f16 against float64 sums of
+    the same operands."""
+    import torch
+    from vecops_amd import capi
+    request = capi.family_request("tile_128", capi.SELECT_REQUIRE, split_k=split)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    if kind == "bf16":
+        a_bits, b_bits = synth.bf16_round(synth.uniform_pm1(1, (m, k))), synth.bf16_round(synth.uniform_pm1(2, (k, n)))
+        a, b = dev_bf16(a_bits, device), dev_bf16(b_bits, device)
+        capi.matmul_family(a, b.t(), c, request)
+        torch.cuda.synchronize()
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a_bits, np.ascontiguousarray(b_bits.T), want, acc_f64=True, c_bf16=False)
+    else:
+        ha, hb = synth.uniform_pm1(1, (m, k)).astype(np.float16), synth.uniform_pm1(2, (k, n)).astype(np.float16)
+        a, b = torch.from_numpy(ha).to(device), torch.from_numpy(hb).to(device)
+        capi.matmul_family(a, b.t(), c, request)
+        torch.cuda.synchronize()
+        want = (ha.astype(np.float64) @ hb.astype(np.float64)).astype(np.float32)
     assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
 
 
@@ -77,9 +106,12 @@ def test_the_table_plans_one_workgroup_per_unit(device):
     result (which a K of one element more, padded operands apart, selects) up to the order of the fp32 sums."""
     import torch
     from vecops_amd import capi
-    for m, n, k in ((1024, 4096, 4096), (768, 4096, 4096), (512, 4096, 4096), (2048, 2048, 2048)):
-        a_bits, b_bits = synth.bf16_round(synth.normal(1, (m, k), 0.02)), synth.bf16_round(synth.normal(2, (n, k), 0.02))
+    for (m, n, k), b_as_kn in (((1024, 4096, 4096), False), ((768, 4096, 4096), False), ((512, 4096, 4096), False),
+                               ((2048, 2048, 2048), False), ((1024, 4096, 4096), True), ((512, 4096, 4096), True)):
+        a_bits = synth.bf16_round(synth.normal(1, (m, k), 0.02))
+        b_bits = synth.bf16_round(synth.normal(2, (k, n) if b_as_kn else (n, k), 0.02))
         a, b = dev_bf16(a_bits, device), dev_bf16(b_bits, device)
+        b = b.t() if b_as_kn else b
         c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
         plan = capi.plan_matmul(a, b, c)
         assert capi.FAMILY_NAMES[plan.family] == "tile_128" and plan.split_k == 1 and plan.workspace_bytes == 0

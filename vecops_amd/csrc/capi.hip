@@ -512,10 +512,12 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   }
   const int64_t ktile = k_tile_elements(pr.src);
   const int64_t k_tiles = (pr.k + ktile - 1) / ktile;
-  // operands the four-stage 128x128 kernel (tile_gemm_deep128.hip) serves: both K-contiguous, fetched by loads that
-  // write LDS, K in whole K tiles
-  const bool deep_ok = mode == MODE_KVEC_DMA && !pr.packed_b && pr.k % ktile == 0 && k_tiles >= kRules.deep_min_k_tiles &&
-                       (pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8);
+  // operands the four-stage 128x128 kernel (tile_gemm_deep128.hip) serves: fetched by loads that write LDS (both
+  // K-contiguous, or 16-bit operands with B as [K,N]), K in whole K tiles
+  const bool deep_tr = mode == MODE_NVEC_B_DMA && (pr.src == SRC_BF16 || pr.src == SRC_F16) && pr.n % 8 == 0 &&
+                       pr.k * pr.b.cs * 2 + 256 < (int64_t{1} << 31);   // B as [K,N]: 16-bit operands, 32-bit K offsets
+  const bool deep_ok = ((mode == MODE_KVEC_DMA && (pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8)) || deep_tr) &&
+                       !pr.packed_b && pr.k % ktile == 0 && k_tiles >= kRules.deep_min_k_tiles;
   // At most four K tiles of 16-bit or 8-bit operands: the tile's life is its start-up and its stores, and
   // two or three 128x128 workgroups on a compute unit overlap one's stores with another's loads, which a
   // single big tile cannot (batch 8 of 3000x3000x17 to fp32: 93 us against 111; 8 x 1000x1000x100: 17.7
@@ -939,7 +941,7 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
              static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.batch * p.split_k <= kRules.deep_max_workgroups &&
              launch_tile_gemm_deep128_serves(pr.src, p, mode)) {
     // at most one workgroup per compute unit: the four-stage kernel, whose loads run three K tiles ahead
-    e = launch_tile_gemm_deep128(pr.src, p, stream);
+    e = launch_tile_gemm_deep128(pr.src, p, mode, stream);
   } else switch (pr.src) {
     case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile_m, tile_n, mode, stream); break;
     case SRC_BF16: e = launch_tile_gemm_bf16(p, tile_m, tile_n, mode, stream); break;

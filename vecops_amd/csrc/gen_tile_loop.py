@@ -337,6 +337,8 @@ def wide_loop():
 #   stage (t - 1) % 4 for the last time and tile t + 1 has landed
 #   k-step 1   multiplies set 1, reads tile t + 1's k-step 0 into set 0, issues the eight loads of tile t + 3 into
 #              stage (t + 3) % 4
+# B either K-contiguous (swizzled rows of 128 bytes, like A) or as it lies in memory ([k][n]: 64 k rows of 256 bytes,
+# swizzled, read by ds_read_b64_tr_b16; one per-lane load offset and a scalar offset per load, as in the 256x256 loop).
 # Fragment registers: set s, A block i at v[128 + 32 s + 4 i ..], B block j at v[144 + 32 s + 4 j ..].  LDS addresses:
 # stages 0 / 1 and 2 / 3 share base registers (la{pair}{q}); the odd stage of a pair lies 32 KiB up, in the offset.
 DEEP_STAGE = 32768
@@ -353,7 +355,15 @@ def deep_fb(s, j):
     return f"v[{r}:{r + 3}]"
 
 
-def deep_reads(st, ks, to_set):
+def deep_fb_half(s, j, h):
+    r = 144 + 32 * s + 4 * j + 2 * h
+    return f"v[{r}:{r + 1}]"
+
+
+DEEP_PITCH_TR = 256   # bytes between the k rows of a B tile kept as it lies in memory ([k][n], 128 columns)
+
+
+def deep_reads(st, ks, to_set, tr):
     out = []
     pair, odd = st >> 1, st & 1
     order = [("a", 0)] + [("b", j) for j in range(4)] + [("a", i) for i in range(1, 4)]
@@ -361,12 +371,18 @@ def deep_reads(st, ks, to_set):
         q = (2 * ks ^ f) & 3
         if kind == "a":
             out.append(f"ds_read_b128 {deep_fa(to_set, f)}, %[la{pair}{q}] offset:{odd * DEEP_STAGE + f * 2048}")
+        elif tr:
+            # B as [k][n]: column block j in base j / 2, 32 bytes on for the odd one; the two reads give k 0-3 and 4-7
+            # of the lane's chunk
+            off = odd * DEEP_STAGE + (f & 1) * 32 + ks * 32 * DEEP_PITCH_TR
+            out.append(f"ds_read_b64_tr_b16 {deep_fb_half(to_set, f, 0)}, %[lb{pair}{f >> 1}] offset:{off}")
+            out.append(f"ds_read_b64_tr_b16 {deep_fb_half(to_set, f, 1)}, %[lb{pair}{f >> 1}] offset:{off + 4 * DEEP_PITCH_TR}")
         else:
             out.append(f"ds_read_b128 {deep_fb(to_set, f)}, %[lb{pair}{q}] offset:{odd * DEEP_STAGE + f * 2048}")
     return out
 
 
-def deep_k_tile(st):
+def deep_k_tile(st, tr):
     out = ["s_cmp_gt_i32 %[left], 0",
            "s_cselect_b32 s82, 0x7fffffff, 0",
            "s_cselect_b32 s86, 0x7fffffff, 0",
@@ -376,48 +392,52 @@ def deep_k_tile(st):
         i, j = x // 4, x % 4
         c = i * 4 + j
         return f"MFMA %[c{c}], {deep_fb(s, j)}, {deep_fa(s, i)}, %[c{c}]"
-    reads = deep_reads(st, 1, 1)
+    reads = deep_reads(st, 1, 1, tr)
     out.append("s_waitcnt lgkmcnt(0)")
     for x in range(16):
         out.append(mfma(x, 0))
-        if x < 8:
+        if x < len(reads):
             out.append(reads[x])
     out += ["s_waitcnt vmcnt(8) lgkmcnt(0)", "s_barrier"]
-    reads = deep_reads((st + 1) & 3, 0, 0)
+    reads = deep_reads((st + 1) & 3, 0, 0, tr)
     target = (st + 3) & 3
     loads = []
     for p in range(4):
-        loads.append((f"s_add_u32 m0, %[m0w], {target * DEEP_STAGE + p * 4096}",
+        loads.append(([f"s_add_u32 m0, %[m0w], {target * DEEP_STAGE + p * 4096}"],
                       f"buffer_load_dwordx4 %[ra{p}], s[80:83], %[ka] offen lds"))
     for p in range(4):
-        loads.append((f"s_add_u32 m0, %[m0w], {target * DEEP_STAGE + DEEP_B + p * 4096}",
-                      f"buffer_load_dwordx4 %[rb{p}], s[84:87], %[ka] offen lds"))
+        m0 = f"s_add_u32 m0, %[m0w], {target * DEEP_STAGE + DEEP_B + p * 4096}"
+        if tr:
+            pre = [m0, "s_mov_b32 s88, %[kb]"] if p == 0 else [m0, "s_add_u32 s88, s88, %[pb]"]
+            loads.append((pre, "buffer_load_dwordx4 %[rb0], s[84:87], s88 offen lds"))
+        else:
+            loads.append(([m0], f"buffer_load_dwordx4 %[rb{p}], s[84:87], %[kb] offen lds"))
     for x in range(16):
         if x % 2 == 0:
-            out.append(loads[x // 2][0])
+            out += loads[x // 2][0]
         out.append(mfma(x, 1))
         if x % 2 == 0:
             out.append(loads[x // 2][1])
-        if 1 <= x <= 8:
+        if 1 <= x <= len(reads):
             out.append(reads[x - 1])
-    out.append("s_add_u32 %[ka], %[ka], 128")
+    out += ["s_add_u32 %[ka], %[ka], 128", "s_add_u32 %[kb], %[kb], %[sb]"]
     return out
 
 
-def deep_loop():
+def deep_loop(tr):
     out = []
     for w in range(4):
         out.append(f"s_mov_b32 s{80 + w}, %[da{w}]")
         out.append(f"s_mov_b32 s{84 + w}, %[db{w}]")
-    out += deep_reads(0, 0, 0)
+    out += deep_reads(0, 0, 0, tr)
     out.append("1:")
     out += ["s_cmp_lt_u32 %[n], 4", "s_cbranch_scc1 2f"]
     for st in range(4):
-        out += deep_k_tile(st)
+        out += deep_k_tile(st, tr)
     out += ["s_sub_u32 %[n], %[n], 4", "s_branch 1b", "2:"]
     for st in range(3):
         out += [f"s_cmp_eq_u32 %[n], {st}", "s_cbranch_scc1 3f"]
-        out += deep_k_tile(st)
+        out += deep_k_tile(st, tr)
     out.append("3:")
     out += ["s_waitcnt vmcnt(0) lgkmcnt(0)", "s_nop 15", "s_nop 15"]
     return out
@@ -452,10 +472,12 @@ def main():
     w("#define VECOPS_LOOP352_CLOBBERS \\\n  " + ", ".join(f'"s{r}"' for r in range(80, 89)) + ", \\\n  " +
       ", \\\n  ".join(", ".join(f'"v{r}"' for r in range(b, min(b + 16, 248))) for b in range(128, 248, 16)) + "\n")
     w("\n// The K loop of the 128 x 128 tile on four LDS stages (one workgroup per compute unit): see gen_tile_loop.py.\n")
-    w(as_macro("VECOPS_LOOP128_DEEP", deep_loop()))
+    w(as_macro("VECOPS_LOOP128_DEEP", deep_loop(False)))
+    w("\n// ... with B as it lies in memory ([k][n]), transposed by the LDS reads\n")
+    w(as_macro("VECOPS_LOOP128_DEEP_TR", deep_loop(True)))
     w("#define VECOPS_LOOP128_ACCUMULATORS(t) \\\n  " +
       ", \\\n  ".join(", ".join(f'[c{x}] "+a"(t[{x // 4}][{x % 4}])' for x in range(r, r + 4)) for r in range(0, 16, 4)) + "\n")
-    w("#define VECOPS_LOOP128_CLOBBERS \\\n  " + ", ".join(f'"s{r}"' for r in range(80, 88)) + ", \\\n  " +
+    w("#define VECOPS_LOOP128_CLOBBERS \\\n  " + ", ".join(f'"s{r}"' for r in range(80, 89)) + ", \\\n  " +
       ", \\\n  ".join(", ".join(f'"v{r}"' for r in range(b, b + 16)) for b in range(128, 192, 16)) + "\n")
     w("\n// the accumulators as operands: quad x = t[x / 8][x % 8]\n")
     w("#define VECOPS_LOOP256_ACCUMULATORS(t) \\\n  " +

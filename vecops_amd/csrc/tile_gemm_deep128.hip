@@ -5,8 +5,10 @@
 // tile's loads (0.67 us per K tile of 0.25 us of matrix instructions at 1024 x 4096 x 4096).
 //
 // What it serves (launch_tile_gemm_deep128_serves): bf16, f16 or signed 8-bit operands, both K-contiguous with 16-byte
-// aligned bases, rows and batches (the loads write LDS themselves); K a whole number of K tiles.  Any M, N, batch
-// count, K split, C input and output type of the class: the epilogue is tile_gemm_kernel's.
+// aligned bases, rows and batches (the loads write LDS themselves), or - 16-bit operands - B handed over as [K,N]
+// (TR: the tile lies [k][n] in LDS, 64 rows of 256 bytes, swizzled as tile_gemm_kernel's, and the fragment reads
+// transpose); K a whole number of K tiles.  Any M, N, batch count, K split, C input and output type of the class: the
+// epilogue is tile_gemm_kernel's.
 #include "tile_gemm_launch.h"
 
 namespace vecops_hip {
@@ -16,7 +18,7 @@ namespace {
 constexpr int kDeepStage = 32768;  // 128 rows of A, then 128 of B, 128 bytes of K each
 constexpr int kDeepStages = 4;
 
-template <int SRC>
+template <int SRC, bool TR>
 __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGemmParams p) {
   using T = SrcTraits<SRC>;
   constexpr bool INT = T::kInt;
@@ -53,9 +55,23 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
       rows_a[i] = static_cast<uint32_t>(static_cast<int64_t>(min(m0 + tile_row, p.m - 1) - m0) * p.a_rs * T::kSrcBytes + chunk * 16);
       rows_b[i] = static_cast<uint32_t>(static_cast<int64_t>(min(n0 + tile_row, p.n - 1) - n0) * p.b_rs * T::kSrcBytes + chunk * 16);
     }
+    if constexpr (TR) {
+      // B as [K,N]: a load instruction of the workgroup fills sixteen k rows of 256 bytes; lane t fetches, of k row
+      // t / 16, the chunk of eight columns whose swizzled slot is t % 16 (slot = chunk xor 4 * (k row % 4): the four
+      // rows a transposing read touches lie in different bank groups).  N is a multiple of eight on this path: a chunk
+      // past it is clamped onto the last one.
+      const int krow = tid >> 4, slot = tid & 15;
+      const int chunk = slot ^ ((krow & 3) << 2);
+      const int col = min(n0 + chunk * 8, p.n - 8) - n0;
+      rows_b[0] = static_cast<uint32_t>((static_cast<int64_t>(krow) * p.b_ks + col) * T::kSrcBytes);
+    }
   }
+  // bytes from one K tile of B to the next, and (TR) from one of its four loads to the next
+  const uint32_t step_b = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(TR ? 64 * p.b_ks * T::kSrcBytes : 128));
+  const uint32_t part_b = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(TR ? 16 * p.b_ks * T::kSrcBytes : 0));
   const u32x4 desc_a = tile_buffer_words((const VECOPS_GLOBAL char*)p.a +
                                          (static_cast<int64_t>(batch) * p.a_bs + static_cast<int64_t>(m0) * p.a_rs) * T::kSrcBytes);
+  // (TR: the rows of the [N,K] view are one element apart)
   const u32x4 desc_b = tile_buffer_words((const VECOPS_GLOBAL char*)p.b +
                                          (static_cast<int64_t>(batch) * p.b_bs + static_cast<int64_t>(n0) * p.b_rs) * T::kSrcBytes);
   const uint32_t lds0 = lds_address_of(lds);
@@ -72,7 +88,8 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
       load_16_bytes_into_lds(da, m0_wave, static_cast<uint32_t>(t * kDeepStage + i * 4096), rows_a[i], k_bytes);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      load_16_bytes_into_lds(db, m0_wave, static_cast<uint32_t>(t * kDeepStage + 16384 + i * 4096), rows_b[i], k_bytes);
+      load_16_bytes_into_lds(db, m0_wave, static_cast<uint32_t>(t * kDeepStage + 16384 + i * 4096), rows_b[TR ? 0 : i],
+                             TR ? static_cast<uint32_t>(kt_begin + t) * step_b + static_cast<uint32_t>(i) * part_b : k_bytes);
   };
   fill(0);
   fill(1);
@@ -90,7 +107,16 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         base_a[pair][q] = lds0 + pair * 2 * kDeepStage + (wm * 64 + frag_row) * 128 + (((slot ^ (2 * q)) & 7) << 4);
-        base_b[pair][q] = lds0 + pair * 2 * kDeepStage + 16384 + (wn * 64 + frag_row) * 128 + (((slot ^ (2 * q)) & 7) << 4);
+        if constexpr (TR) {
+          // transposing read: lane s of the 16-lane group addresses row s / 4 of a block of four k rows, columns
+          // 4 (s % 4) .. + 3 of the column block pair q, and receives column s of the block's 16; the group reads
+          // chunk frag_chunk of k.  The 64-byte group is swizzled with the row's low two bits, which are s / 4.
+          int col_bytes = ((wn * 4 + 2 * q) * 16 + (frag_row & 3) * 4) * 2;
+          col_bytes ^= ((frag_row >> 2) & 3) << 6;
+          base_b[pair][q] = lds0 + pair * 2 * kDeepStage + 16384 + (frag_chunk * 8 + (frag_row >> 2)) * 256 + col_bytes;
+        } else {
+          base_b[pair][q] = lds0 + pair * 2 * kDeepStage + 16384 + (wn * 64 + frag_row) * 128 + (((slot ^ (2 * q)) & 7) << 4);
+        }
       }
   }
 
@@ -103,12 +129,14 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
     auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
     int left = nk - 3, n = nk;
     uint32_t k_a = uniform(static_cast<uint32_t>(kt_begin + 3) * 128u);   // the loop fetches tile 3 of the range first
+    uint32_t k_b = uniform(static_cast<uint32_t>(kt_begin + 3) * step_b);
+    const uint32_t sb = uniform(step_b), pb = uniform(part_b);
     const uint32_t da[4] = {uniform(desc_a[0]), uniform(desc_a[1]), uniform(desc_a[2]), uniform(desc_a[3])};
     const uint32_t db[4] = {uniform(desc_b[0]), uniform(desc_b[1]), uniform(desc_b[2]), uniform(desc_b[3])};
     const uint32_t m0w = uniform(m0_wave);
 #define VECOPS_DEEP_STATEMENT(TEXT)                                                                                  \
     asm volatile(TEXT                                                                                                 \
-                 : VECOPS_LOOP128_ACCUMULATORS(acc.t), [ka] "+s"(k_a), [left] "+s"(left), [n] "+s"(n)                 \
+                 : VECOPS_LOOP128_ACCUMULATORS(acc.t), [ka] "+s"(k_a), [kb] "+s"(k_b), [left] "+s"(left), [n] "+s"(n)  \
                  : [la00] "v"(base_a[0][0]), [la01] "v"(base_a[0][1]), [la02] "v"(base_a[0][2]), [la03] "v"(base_a[0][3]), \
                    [la10] "v"(base_a[1][0]), [la11] "v"(base_a[1][1]), [la12] "v"(base_a[1][2]), [la13] "v"(base_a[1][3]), \
                    [lb00] "v"(base_b[0][0]), [lb01] "v"(base_b[0][1]), [lb02] "v"(base_b[0][2]), [lb03] "v"(base_b[0][3]), \
@@ -116,9 +144,14 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
                    [ra0] "v"(rows_a[0]), [ra1] "v"(rows_a[1]), [ra2] "v"(rows_a[2]), [ra3] "v"(rows_a[3]),            \
                    [rb0] "v"(rows_b[0]), [rb1] "v"(rows_b[1]), [rb2] "v"(rows_b[2]), [rb3] "v"(rows_b[3]),            \
                    [da0] "s"(da[0]), [da1] "s"(da[1]), [da2] "s"(da[2]), [da3] "s"(da[3]),                            \
-                   [db0] "s"(db[0]), [db1] "s"(db[1]), [db2] "s"(db[2]), [db3] "s"(db[3]), [m0w] "s"(m0w)             \
+                   [db0] "s"(db[0]), [db1] "s"(db[1]), [db2] "s"(db[2]), [db3] "s"(db[3]), [m0w] "s"(m0w),            \
+                   [sb] "s"(sb), [pb] "s"(pb)                                                                         \
                  : "memory", "m0", "scc", VECOPS_LOOP128_CLOBBERS)
-    if constexpr (SRC == SRC_F16) VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP("v_mfma_f32_16x16x32_f16"));
+    if constexpr (TR) {
+      static_assert(SRC == SRC_BF16 || SRC == SRC_F16, "transposing LDS reads move 16-bit elements");
+      if constexpr (SRC == SRC_F16) VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP_TR("v_mfma_f32_16x16x32_f16"));
+      else VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP_TR("v_mfma_f32_16x16x32_bf16"));
+    } else if constexpr (SRC == SRC_F16) VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP("v_mfma_f32_16x16x32_f16"));
     else if constexpr (INT) VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP("v_mfma_i32_16x16x64_i8"));
     else VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP("v_mfma_f32_16x16x32_bf16"));
 #undef VECOPS_DEEP_STATEMENT
@@ -130,11 +163,11 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
   store_accumulators<SRC, 2, 2, 2, 2, kLdsBytes, true>(p, lds, acc, batch, split, m0, n0, wm, wn, wave, lane);
 }
 
-template <int SRC>
+template <int SRC, bool TR>
 hipError_t launch(const TileGemmParams& p, hipStream_t stream) {
   constexpr int kEpilogue = kEpilogueLdsBytes<2, 2, 2, 2>();
   constexpr int kLds = kDeepStages * kDeepStage > kEpilogue ? kDeepStages * kDeepStage : kEpilogue;
-  auto kernel = tile_gemm_deep128_kernel<SRC>;
+  auto kernel = tile_gemm_deep128_kernel<SRC, TR>;
   static thread_local int configured_device = -1;
   int device = 0;
   hipError_t e = hipGetDevice(&device);
@@ -154,20 +187,22 @@ hipError_t launch(const TileGemmParams& p, hipStream_t stream) {
 
 bool launch_tile_gemm_deep128_serves(int src, const TileGemmParams& p, int mode) {
   if (src != SRC_BF16 && src != SRC_F16 && src != SRC_I8) return false;
-  if (mode != MODE_KVEC_DMA || p.m <= 0 || p.n <= 0 || p.split_k < 1) return false;
+  const bool tr = mode == MODE_NVEC_B_DMA;
+  if ((mode != MODE_KVEC_DMA && !tr) || (tr && src == SRC_I8) || p.m <= 0 || p.n <= 0 || p.split_k < 1) return false;
   const int elem = src == SRC_I8 ? 1 : 2, ktile = 128 / elem;
   if (p.k < ktile || p.k % ktile != 0) return false;
   // 32-bit byte offsets inside a tile's 128 rows
   if (128 * p.a_rs * elem + static_cast<int64_t>(p.k) * elem >= (int64_t{1} << 31)) return false;
-  if (128 * p.b_rs * elem + static_cast<int64_t>(p.k) * elem >= (int64_t{1} << 31)) return false;
-  return true;
+  if (tr) return p.n % 8 == 0 && p.n >= 8 && p.b_rs == 1 && static_cast<int64_t>(p.k) * p.b_ks * elem + 256 < (int64_t{1} << 31);
+  return 128 * p.b_rs * elem + static_cast<int64_t>(p.k) * elem < (int64_t{1} << 31);
 }
 
-hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, hipStream_t stream) {
+hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, int mode, hipStream_t stream) {
+  const bool tr = mode == MODE_NVEC_B_DMA;
   switch (src) {
-    case SRC_BF16: return launch<SRC_BF16>(p, stream);
-    case SRC_F16: return launch<SRC_F16>(p, stream);
-    case SRC_I8: return launch<SRC_I8>(p, stream);
+    case SRC_BF16: return tr ? launch<SRC_BF16, true>(p, stream) : launch<SRC_BF16, false>(p, stream);
+    case SRC_F16: return tr ? launch<SRC_F16, true>(p, stream) : launch<SRC_F16, false>(p, stream);
+    case SRC_I8: return launch<SRC_I8, false>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }

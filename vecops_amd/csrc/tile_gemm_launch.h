@@ -206,7 +206,7 @@ bool launch_tile_gemm_packed16_serves(int src, const TileGemmParams& p, int tile
 hipError_t launch_tile_gemm_packed16(int src, const TileGemmParams& p, hipStream_t stream);
 // The 128 x 128 tile on four LDS stages for launches of at most one workgroup per compute unit (tile_gemm_deep128.hip).
 bool launch_tile_gemm_deep128_serves(int src, const TileGemmParams& p, int mode);
-hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, hipStream_t stream);
+hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_bf16(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_i8(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_i8_flip(const GroupedTables& t, int tile, int mode, hipStream_t stream);
