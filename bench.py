@@ -44,7 +44,9 @@ RECORDED_TRAFFIC = {
     "gemv_m1": (int((29647.0 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
     "gemv_m4": (int((29761.0 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
     "gemv_m16": (int((30145.0 * 2.000 + 448.0 * 1.000) * 1024), "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
-    "bf16_packed": (int((98473.0 * 2.000 + 32768 * 1.000) * 1024), "profiles/tile_gemm_packed_b_bf16_4096.md"),
+    "bf16_packed": (int((98490.0 * 2.000 + 32768 * 1.000) * 1024), "profiles/tile_gemm_packed16_bf16_4096.md"),
+    "bf16_mid_kn_1024x4096x4096": (int((49256.0 * 2.000 + 8192 * 1.000) * 1024), "profiles/tile_gemm_deep128_bf16_1024x4096x4096.md"),
+    "bf16_mid_nk_1024x4096x4096": (int((49245.0 * 2.000 + 8192 * 1.000) * 1024), "profiles/tile_gemm_deep128_bf16_1024x4096x4096.md"),
     "int8_packed": (int((55095.0 * 2.000 + 88108 * 1.000) * 1024),
                     "profiles/tile_gemm_wide_i8_dequant_2048x4096x11008.md"),
     "fp32_f32": (int((12360.0 * 2.000 + 4096 * 1.000) * 1024), "profiles/tile_gemm_f32_compute_1024.md"),
@@ -198,6 +200,35 @@ def bench_fp32_gemm(dev, steps, warmup, compute):
             "roofline": _roofline("mfma", tflops, peak, "TFLOP/s", kernel=_kernel_label(plan, "f32" if compute == "f32" else "f32 as bf16"),
                                   algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=3 * 4 * n * n,
                                   **(_traffic("fp32_f32") if compute == "f32" else {"traffic": None}), **_timing_fields(t))}
+
+
+def bench_bf16_mid(dev, steps, warmup, m, n, k, b_as_kn):
+    """A product of at most one 128 x 128 workgroup per compute unit (default 1024 x 4096 x 4096: a prefill batch of 1024
+    tokens against a 4096-wide weight), bf16 in and out: the four-stage 128 x 128 kernel's workload."""
+    import numpy as np
+    import torch
+    from vecops_amd import capi, synth
+    a = torch.from_numpy(synth.bf16_round(synth.normal(1, (m, k), 0.02)).view(np.int16)).to(dev).view(torch.bfloat16)
+    b = torch.from_numpy(synth.bf16_round(synth.normal(2, (k, n) if b_as_kn else (n, k), 0.02)).view(np.int16)).to(dev).view(torch.bfloat16)
+    b = b.t() if b_as_kn else b
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+    plan = capi.plan_matmul(a, b, c)
+    ws = torch.empty(max(int(plan.workspace_bytes), 1), dtype=torch.uint8, device=dev)
+    run = capi.PreparedMatmul(a, b, c, workspace=ws)
+    t = _measure(lambda i: run(), steps, warmup)
+    flops = 2.0 * m * n * k
+    tflops = flops / (t["event_ms"] * 1e-3) / 1e12
+    label = _kernel_label(plan, "bf16")
+    split = max(int(plan.split_k), 1)
+    workgroups = -(-m // 128) * -(-n // 128) * split
+    if capi.FAMILY_NAMES.get(plan.family) == "tile_128" and workgroups <= 256 and k % 64 == 0 and k // 64 // split >= 8:
+        label = label.replace("tile_gemm_kernel<bf16>", "tile_gemm_deep128_kernel<bf16>")   # what run_problem launches for such a plan
+    roof = _roofline("mfma", tflops, PEAK_BF16_TFLOPS, "TFLOP/s", kernel=label, algorithmic_flops_per_launch=flops,
+                     algorithmic_bytes_per_launch=2 * (m * k + n * k + m * n),
+                     **_traffic(f"bf16_mid_{'kn' if b_as_kn else 'nk'}_{m}x{n}x{k}"), **_timing_fields(t))
+    return {"metric": f"bf16_gemm_{m}x{n}x{k}_tflops", "workload": f"bf16 ({m},{n},{k}), A[M,K] and B[{'K,N' if b_as_kn else 'N,K'}], "
+            "normal(0,0.02), fp32 accumulate, bf16 output", "value": tflops, "unit": "TFLOP/s",
+            "us_per_step": t["wall_ms"] * 1e3, "dtype": "bf16", "roofline": roof}
 
 
 def bench_batched(dev, steps, warmup, m, n, k):
@@ -579,7 +610,7 @@ def cpu_baseline(a, b_kn):
 
 
 ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "read_ceiling",
-        "fp32", "batched", "families", "grouped", "rule_check"]
+        "fp32", "batched", "bf16_mid", "families", "grouped", "rule_check"]
 
 
 def main() -> int:
@@ -595,6 +626,8 @@ def main() -> int:
     ap.add_argument("--ceiling-dtype", choices=["bf16", "int8"], default="bf16", help="operands of --only mfma_ceiling")
     ap.add_argument("--fp32-compute", choices=["bf16", "f32"], default="bf16", help="compute type of --only fp32")
     ap.add_argument("--batched-shape", default="777,1000,3001", help="M,N,K of --only batched")
+    ap.add_argument("--mid-shape", default="1024,4096,4096", help="M,N,K of --only bf16_mid")
+    ap.add_argument("--mid-layout", choices=["kn", "nk"], default="kn", help="how B is stored for --only bf16_mid")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the matmul path is built and measured on a single MI355X "
@@ -622,6 +655,7 @@ def main() -> int:
         "read_ceiling": lambda: bench_read_ceiling(dev, K, W),
         "fp32": lambda: bench_fp32_gemm(dev, K, W, args.fp32_compute),
         "batched": lambda: bench_batched(dev, K, W, *[int(v) for v in args.batched_shape.split(",")]),
+        "bf16_mid": lambda: bench_bf16_mid(dev, K, W, *[int(v) for v in args.mid_shape.split(",")], args.mid_layout == "kn"),
         "families": lambda: bench_tile_families(dev, K, W),
         "grouped": lambda: bench_grouped(dev, K, W),
         "rule_check": lambda: bench_rule_check(dev, K, W),
@@ -660,6 +694,7 @@ def main() -> int:
         packed16, packed8 = bench_bf16_gemm_packed(dev, K, W), bench_int8_dequant_packed(dev, K, W)
         secondary = [bench_batched(dev, K, W, m, n, k)
                      for (m, n, k) in [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)]]
+        secondary += [bench_bf16_mid(dev, K, W, 1024, 4096, 4096, True), bench_bf16_mid(dev, K, W, 2048, 2048, 2048, False)]
         secondary += [bench_runtime_quant(dev, K, W), bench_grouped(dev, K, W), ceiling_bf16, ceiling_int8, read_ceiling, packed16,
                       packed8,
                       fp32["bf16"], fp32["f32"], gemv[16], gemv[4], gemv[1], int8]
