@@ -176,12 +176,11 @@ def bench_bf16_gemm(dev, steps, warmup):
     }
 
 
-def bench_fp32_gemm(dev, steps, warmup, compute):
+def bench_fp32_gemm(dev, steps, warmup, compute, n=1024):
     """BASELINE configs[0]: fp32 1024^3, A[M,K] and B[K,N] row-major, U[-1,1); multiplied as bf16 (vecops' x86
     behaviour) or in fp32 (its SME_F32F32 atom)."""
     import torch
     from vecops_amd import capi, synth
-    n = 1024
     a = torch.from_numpy(synth.uniform_pm1(1, (n, n))).to(dev)
     b_kn = torch.from_numpy(synth.uniform_pm1(2, (n, n))).to(dev)
     c = torch.empty((n, n), dtype=torch.float32, device=dev)
@@ -189,17 +188,18 @@ def bench_fp32_gemm(dev, steps, warmup, compute):
     plan = capi.plan_matmul(a, b_kn.t(), c, compute=code)
     ws = torch.empty(max(int(plan.workspace_bytes), 1), dtype=torch.uint8, device=dev)
     run = capi.PreparedMatmul(a, b_kn.t(), c, compute=code, workspace=ws)   # a step is one call of the C ABI
-    t = _measure(lambda i: run(), max(steps, 200), warmup)
+    t = _measure(lambda i: run(), max(steps, 200) if n <= 1024 else steps, warmup)
     flops = 2.0 * n ** 3
     tflops = flops / (t["event_ms"] * 1e-3) / 1e12
     peak = PEAK_FP32_MATRIX_TFLOPS if compute == "f32" else PEAK_BF16_TFLOPS
-    return {"metric": f"fp32_gemm_1024_{compute}_compute_tflops", "workload": "fp32 GEMM M=N=K=1024, A[M,K] and B[K,N] "
+    return {"metric": f"fp32_gemm_{n}_{compute}_compute_tflops", "workload": f"fp32 GEMM M=N=K={n}, A[M,K] and B[K,N] "
             f"row-major, uniform[-1,1), multiplied in {'fp32' if compute == 'f32' else 'bf16 (rounded on load)'}, fp32 "
             "accumulate and output (BASELINE configs[0])", "value": tflops, "unit": "TFLOP/s",
             "us_per_step": t["wall_ms"] * 1e3, "dtype": "f32" if compute == "f32" else "f32 memory, bf16 compute",
             "roofline": _roofline("mfma", tflops, peak, "TFLOP/s", kernel=_kernel_label(plan, "f32" if compute == "f32" else "f32 as bf16"),
                                   algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=3 * 4 * n * n,
-                                  **(_traffic("fp32_f32") if compute == "f32" else {"traffic": None}), **_timing_fields(t))}
+                                  **(_traffic("fp32_f32") if compute == "f32" and n == 1024 else {"traffic": None}),
+                                  **_timing_fields(t))}
 
 
 def bench_bf16_mid(dev, steps, warmup, m, n, k, b_as_kn):
@@ -625,6 +625,7 @@ def main() -> int:
     ap.add_argument("--gemv-m", type=int, default=1, help="activation rows of the --only gemv workload (1..16)")
     ap.add_argument("--ceiling-dtype", choices=["bf16", "int8"], default="bf16", help="operands of --only mfma_ceiling")
     ap.add_argument("--fp32-compute", choices=["bf16", "f32"], default="bf16", help="compute type of --only fp32")
+    ap.add_argument("--fp32-size", type=int, default=1024, help="M = N = K of --only fp32 (1024: BASELINE configs[0])")
     ap.add_argument("--batched-shape", default="777,1000,3001", help="M,N,K of --only batched")
     ap.add_argument("--mid-shape", default="1024,4096,4096", help="M,N,K of --only bf16_mid")
     ap.add_argument("--mid-layout", choices=["kn", "nk"], default="kn", help="how B is stored for --only bf16_mid")
@@ -653,7 +654,7 @@ def main() -> int:
         "gemv": lambda: bench_gemv(dev, K, W, m=args.gemv_m),
         "mfma_ceiling": lambda: bench_mfma_ceiling(dev, K, W, args.ceiling_dtype),
         "read_ceiling": lambda: bench_read_ceiling(dev, K, W),
-        "fp32": lambda: bench_fp32_gemm(dev, K, W, args.fp32_compute),
+        "fp32": lambda: bench_fp32_gemm(dev, K, W, args.fp32_compute, args.fp32_size),
         "batched": lambda: bench_batched(dev, K, W, *[int(v) for v in args.batched_shape.split(",")]),
         "bf16_mid": lambda: bench_bf16_mid(dev, K, W, *[int(v) for v in args.mid_shape.split(",")], args.mid_layout == "kn"),
         "families": lambda: bench_tile_families(dev, K, W),
