@@ -49,7 +49,7 @@ RECORDED_TRAFFIC = {
     "bf16_mid_nk_1024x4096x4096": (int((49245.0 * 2.000 + 8192 * 1.000) * 1024), "profiles/tile_gemm_deep128_bf16_1024x4096x4096.md"),
     "int8_packed": (int((55095.0 * 2.000 + 88108 * 1.000) * 1024),
                     "profiles/tile_gemm_wide_i8_dequant_2048x4096x11008.md"),
-    "fp32_f32": (int((12360.0 * 2.000 + 4096 * 1.000) * 1024), "profiles/tile_gemm_f32_compute_1024.md"),
+    "fp32_f32": (int((12357.0 * 2.000 + 4096 * 1.000) * 1024), "profiles/tile_gemm_f32_compute_1024.md"),
 }
 
 
@@ -192,11 +192,16 @@ def bench_fp32_gemm(dev, steps, warmup, compute, n=1024):
     flops = 2.0 * n ** 3
     tflops = flops / (t["event_ms"] * 1e-3) / 1e12
     peak = PEAK_FP32_MATRIX_TFLOPS if compute == "f32" else PEAK_BF16_TFLOPS
+    label = _kernel_label(plan, "f32" if compute == "f32" else "f32 as bf16")
+    family = capi.FAMILY_NAMES.get(plan.family)
+    tile = {"tile_64": 64, "tile_128": 128}.get(family, 0)
+    if compute == "f32" and tile and (-(-n // tile)) ** 2 * max(int(plan.split_k), 1) <= 256 and n % 32 == 0 and n // 32 // max(int(plan.split_k), 1) >= 8:
+        label = label.replace("tile_gemm_kernel<f32>", "tile_gemm_deep_f32_kernel")   # what run_problem launches for such a plan
     return {"metric": f"fp32_gemm_{n}_{compute}_compute_tflops", "workload": f"fp32 GEMM M=N=K={n}, A[M,K] and B[K,N] "
             f"row-major, uniform[-1,1), multiplied in {'fp32' if compute == 'f32' else 'bf16 (rounded on load)'}, fp32 "
             "accumulate and output (BASELINE configs[0])", "value": tflops, "unit": "TFLOP/s",
             "us_per_step": t["wall_ms"] * 1e3, "dtype": "f32" if compute == "f32" else "f32 memory, bf16 compute",
-            "roofline": _roofline("mfma", tflops, peak, "TFLOP/s", kernel=_kernel_label(plan, "f32" if compute == "f32" else "f32 as bf16"),
+            "roofline": _roofline("mfma", tflops, peak, "TFLOP/s", kernel=label,
                                   algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=3 * 4 * n * n,
                                   **(_traffic("fp32_f32") if compute == "f32" and n == 1024 else {"traffic": None}),
                                   **_timing_fields(t))}
@@ -539,6 +544,73 @@ def bench_rule_check(dev, steps, warmup):
             "worst_shape": worst["shape"], "shapes": rows}
 
 
+VENDOR_GRID = [(m, n, k) for (n, k) in ((4096, 4096), (11008, 4096), (4096, 11008)) for m in (512, 768, 1024, 1536, 2048, 4096)] + [
+    (2048, 2048, 2048), (3000, 3000, 3000), (4096, 4224, 4096), (6144, 6144, 6144), (8192, 8192, 8192), (128, 8192, 8192),
+    (256, 4096, 4096), (5000, 5000, 1024), (1000, 1000, 1000)]
+
+
+def bench_vendor_grid(dev, steps, warmup):
+    """This library against the vendor's (hipBLASLt through torch.matmul, torch._int_mm) on a grid of shapes: bf16 -> bf16
+    with B stored [N,K] and [K,N], int8 -> int32 with B [N,K]; one process, HIP events, the median of five runs of as
+    many launches as fill about 20 ms."""
+    import numpy as np
+    import torch
+    from vecops_amd import capi, synth
+
+    def time_us(fn, hint_us):
+        n = max(5, min(200, int(20000 / hint_us)))
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        runs = []
+        for _ in range(5):
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(n):
+                fn()
+            stop.record()
+            torch.cuda.synchronize()
+            runs.append(start.elapsed_time(stop) / n * 1e3)
+        return round(sorted(runs)[2], 1)
+
+    ws = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    rows = []
+    for m, n, k in VENDOR_GRID:
+        hint = max(10.0, 2.0 * m * n * k / 1.2e9)
+        a = torch.from_numpy(synth.bf16_round(synth.normal(1, (m, k), 0.02)).view(np.int16)).to(dev).view(torch.bfloat16)
+        b = torch.from_numpy(synth.bf16_round(synth.normal(2, (n, k), 0.02)).view(np.int16)).to(dev).view(torch.bfloat16)
+        c = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+        row = {"shape": f"{m}x{n}x{k}"}
+        for layout in ("nk", "kn"):
+            ours_b = b if layout == "nk" else b.view(k, n).t()      # the same bits read as a [K,N] matrix
+            theirs_b = b.t() if layout == "nk" else b.view(k, n)
+            plan = capi.plan_matmul(a, ours_b, c)
+            run = capi.PreparedMatmul(a, ours_b, c, workspace=ws)
+            row[f"bf16_{layout}"] = {"ours_us": time_us(lambda: run(), hint),
+                                     "vendor_us": time_us(lambda: torch.matmul(a, theirs_b, out=c), hint),
+                                     "plan": capi.FAMILY_NAMES.get(plan.family, str(plan.family)) + f"/{max(plan.split_k, 1)}" +
+                                             ("+peel" if plan.peeled_columns else "")}
+        ai = torch.from_numpy(synth.int8_sym(1, (m, k))).to(dev)
+        bi = torch.from_numpy(synth.int8_sym(2, (n, k))).to(dev)
+        ci = torch.empty((m, n), dtype=torch.int32, device=dev)
+        plan = capi.plan_matmul(ai, bi, ci)
+        run = capi.PreparedMatmul(ai, bi, ci, workspace=ws)
+        entry = {"ours_us": time_us(lambda: run(), hint / 2),
+                 "plan": capi.FAMILY_NAMES.get(plan.family, str(plan.family)) + f"/{max(plan.split_k, 1)}" +
+                         ("+peel" if plan.peeled_columns else "")}
+        try:
+            entry["vendor_us"] = time_us(lambda: torch._int_mm(ai, bi.t(), out=ci), hint / 2)
+        except RuntimeError:
+            entry["vendor_us"] = None                               # extents torch._int_mm does not take
+        row["int8_nk"] = entry
+        rows.append(row)
+    ratios = [r[key]["ours_us"] / r[key]["vendor_us"] for r in rows for key in ("bf16_nk", "bf16_kn", "int8_nk") if r[key]["vendor_us"]]
+    return {"metric": "time_against_vendor_library", "workload": "VENDOR_GRID: bf16 -> bf16 (B [N,K] and [K,N]) against torch.matmul, "
+            "int8 -> int32 against torch._int_mm, microseconds per product", "unit": "ours / vendor, geometric mean",
+            "value": float(np.exp(np.mean(np.log(ratios)))), "level_or_ahead": sum(r <= 1.02 for r in ratios), "of": len(ratios),
+            "shapes": rows}
+
+
 def bench_copy(dev, steps, warmup):
     """A plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
     counters of the other workloads are scaled by."""
@@ -610,7 +682,7 @@ def cpu_baseline(a, b_kn):
 
 
 ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "read_ceiling",
-        "fp32", "batched", "bf16_mid", "families", "grouped", "rule_check"]
+        "fp32", "batched", "bf16_mid", "families", "grouped", "rule_check", "vendor_grid"]
 
 
 def main() -> int:
@@ -660,6 +732,7 @@ def main() -> int:
         "families": lambda: bench_tile_families(dev, K, W),
         "grouped": lambda: bench_grouped(dev, K, W),
         "rule_check": lambda: bench_rule_check(dev, K, W),
+        "vendor_grid": lambda: bench_vendor_grid(dev, K, W),
     }
     if args.only in single:
         print(json.dumps(single[args.only]()))

@@ -172,6 +172,11 @@ def test_rule_table_known_answers():
                                      ((512, 2048, 16384), "tile_128", 4), ((512, 1024, 8192), "tile_64", 2)):
         rc, p = _plan(_operand(capi.I8, (m, k)), _operand(capi.I8, (n, k)), _operand(capi.I32, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
+    # fp32 compute: a part-filled round of 128 x 128 tiles (up to 192) loses to four times as many 64 x 64 ones - the
+    # fullest unit's tiles times their area decide; a full round keeps the bigger tile
+    for n, family in ((1536, "tile_64"), (1664, "tile_64"), (1792, "tile_128"), (2048, "tile_128"), (1024, "tile_64")):
+        rc, p = _plan(_operand(capi.F32, (n, n)), _operand(capi.F32, (n, n)), _operand(capi.F32, (n, n)), compute=1)
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == 1, (n, p.family, p.split_k)
     # two rounds of 128 x 128 tiles and eight more: the last column of tiles is a product of its own (64 x 64 tiles, K in
     # five parts), the rest fills two rounds; a required family runs the product whole
     big_n = (_operand(capi.BF16, (1536, 4096)), _operand(capi.BF16, (11008, 4096)), _operand(capi.BF16, (1536, 11008)))

@@ -67,19 +67,20 @@ def test_static_workspace_unsigned_operands_and_c_input(device, oracle):
 
 
 def test_static_workspace_shrinks_a_split_that_does_not_fit(device, oracle):
-    """fp32 compute, 128 tiles of 128 x 128 and a long K: vecops_hip_matmul splits K in two (16 MiB of partial sums);
-    this entry point runs the product unsplit instead of refusing it."""
+    """bf16, 64 tiles of 128 x 128 and a long K: vecops_hip_matmul splits K in four (16 MiB of partial sums); this
+    entry point runs the product with a split that fits instead of refusing it."""
     import torch
-    m, n, k = 1024, 2048, 4096
-    a, b = synth.uniform_pm1(81, (m, k)), synth.uniform_pm1(82, (n, k))
-    ta, tb = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+    m, n, k = 512, 2048, 16384
+    a, b = synth.bf16_round(synth.uniform_pm1(81, (m, k))), synth.bf16_round(synth.uniform_pm1(82, (n, k)))
+    ta = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+    tb = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
     c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
-    plan = capi.plan_matmul(ta, tb, c, compute=capi.COMPUTE_F32)
+    plan = capi.plan_matmul(ta, tb, c)
     assert plan.workspace_bytes > capi.lib().vecops_hip_static_workspace_bytes()
-    capi.matmul_static_workspace(ta, tb, c, compute=capi.COMPUTE_F32)
+    capi.matmul_static_workspace(ta, tb, c)
     torch.cuda.synchronize()
     rows = np.arange(0, m, 61)
-    want = a[rows].astype(np.float64) @ b.astype(np.float64).T
+    want = synth.bf16_to_f32(a[rows]).astype(np.float64) @ synth.bf16_to_f32(b).astype(np.float64).T
     assert rel_err(c.cpu().numpy()[rows], want) <= 2e-6 * max(1, k // 32)
 
 

@@ -257,6 +257,10 @@ struct RuleConstants {
   int64_t rectangle_margin_num = 11, rectangle_margin_den = 10;
   // -- more 64x64 tiles than this many rounds of the chip: 128x128 tiles after all
   int64_t many_small_tiles_rounds = 4;
+  // -- fp32 compute (64-cycle matrix instructions, no power limit in sight): time follows the tiles the fullest compute
+  //    unit gets times their area, so up to this many 128x128 tiles (one each on three quarters of the units) lose to
+  //    four times as many 64x64 ones (three each); fp32 1536^3 103 -> 75-78 us
+  int64_t f32_small_tiles_up_to_tiles128 = 192;
   // -- a tile's life is its start-up and its stores when K is this short (K tiles of 16-bit / 8-bit operands): small
   //    tiles, of which two or three overlap on a unit; `bench.py --only batched --batched-shape 3000,3000,17`
   int64_t short_k_tiles_16bit = 4, short_k_tiles_8bit = 8;
@@ -505,6 +509,11 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
         tile_n = 352;
       }
     }
+  }
+  if (pr.src == SRC_F32 && family == VECOPS_HIP_FAMILY_TILE_128 && tiles(128) <= kRules.f32_small_tiles_up_to_tiles128 &&
+      (tiles(64) + kComputeUnits - 1) / kComputeUnits <= 3) {
+    family = VECOPS_HIP_FAMILY_TILE_64;
+    tile_m = tile_n = 64;
   }
   if (family == VECOPS_HIP_FAMILY_TILE_64 && pr.m > 64 && pr.n > 64 && tiles(64) > kRules.many_small_tiles_rounds * kComputeUnits) {
     family = VECOPS_HIP_FAMILY_TILE_128;
@@ -942,6 +951,12 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
              launch_tile_gemm_deep128_serves(pr.src, p, mode)) {
     // at most one workgroup per compute unit: the four-stage kernel, whose loads run three K tiles ahead
     e = launch_tile_gemm_deep128(pr.src, p, mode, stream);
+  } else if (pr.src == SRC_F32 && tile_m == tile_n && (tile_m == 64 || tile_m == 128) && (mode == MODE_KVEC || mode == MODE_NVEC_B) &&
+             p.k_tiles_per_split >= kRules.deep_min_k_tiles &&
+             static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.batch * p.split_k <= kRules.deep_max_workgroups &&
+             launch_tile_gemm_deep_f32_serves(p, tile_m, mode == MODE_NVEC_B)) {
+    // fp32 compute, at most one workgroup per compute unit: the ring of LDS stages (tile_gemm_deep_f32.hip)
+    e = launch_tile_gemm_deep_f32(p, tile_m, mode == MODE_NVEC_B, stream);
   } else switch (pr.src) {
     case SRC_I8_FLIP: e = launch_tile_gemm_i8_flip(p, tile_m, tile_n, mode, stream); break;
     case SRC_BF16: e = launch_tile_gemm_bf16(p, tile_m, tile_n, mode, stream); break;

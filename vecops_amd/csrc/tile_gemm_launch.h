@@ -207,6 +207,10 @@ hipError_t launch_tile_gemm_packed16(int src, const TileGemmParams& p, hipStream
 // The 128 x 128 tile on four LDS stages for launches of at most one workgroup per compute unit (tile_gemm_deep128.hip).
 bool launch_tile_gemm_deep128_serves(int src, const TileGemmParams& p, int mode);
 hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, int mode, hipStream_t stream);
+// fp32 compute on 64 x 64 (tile = 64) or 128 x 128 tiles with a ring of LDS stages, for launches of at most one workgroup
+// per compute unit (tile_gemm_deep_f32.hip); b_as_kn: B handed over as [K,N].
+bool launch_tile_gemm_deep_f32_serves(const TileGemmParams& p, int tile, bool b_as_kn);
+hipError_t launch_tile_gemm_deep_f32(const TileGemmParams& p, int tile, bool b_as_kn, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_bf16(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_i8(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_i8_flip(const GroupedTables& t, int tile, int mode, hipStream_t stream);
