@@ -79,6 +79,41 @@ def test_deep_kernel_int8_exact(device, m, n, k, split):
     assert np.array_equal(c.cpu().numpy()[rows], want)
 
 
+@pytest.mark.parametrize("kind", ["bf16", "f16", "i8"])
+@pytest.mark.parametrize("m,n,k", [(1024, 4096, 1024), (300, 520, 1024), (513, 257, 1152), (128, 100, 512), (256, 4096, 4096),
+                                   (2, 640, 2048)])
+def test_deep_kernel_prepacked_b(device, kind, m, n, k):
+    """B packed by vecops_hip_pack_b: the pack keeps its order in LDS; the product equals the plain operand's bit for
+    bit (the same kernel's loop on the same K order; integer sums in any case), K splits of the plan included."""
+    import torch
+    from vecops_amd import capi
+    gen = torch.Generator().manual_seed(m + n + k)
+    if kind == "i8":
+        a = torch.randint(-128, 128, (m, k), generator=gen, dtype=torch.int8).to(device)
+        b = torch.randint(-128, 128, (n, k), generator=gen, dtype=torch.int8).to(device)
+        c = torch.full((m, n), -1, dtype=torch.int32, device=device)
+    else:
+        dtype = torch.bfloat16 if kind == "bf16" else torch.float16
+        a = (torch.rand((m, k), generator=gen) * 2 - 1).to(dtype).to(device)
+        b = (torch.rand((n, k), generator=gen) * 2 - 1).to(dtype).to(device)
+        c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    packed = capi.pack_b(b)
+    plan = capi.plan_matmul_packed_b(a, packed, c)
+    if m * n >= 128 * 128 * 96:
+        assert capi.FAMILY_NAMES[plan.family] == "tile_128"          # 96 to 256 tiles: whole, on the four-stage kernel
+    capi.matmul_packed_b(a, packed, c)
+    plain = torch.empty_like(c)
+    capi.matmul_family(a, b, plain, capi.family_request("tile_128", capi.SELECT_REQUIRE, split_k=max(int(plan.split_k), 1)))
+    torch.cuda.synchronize()
+    if kind == "i8" or capi.FAMILY_NAMES[plan.family] == "tile_128":
+        assert torch.equal(c, plain)
+    want = a.double() @ b.double().t()
+    if kind == "i8":
+        assert torch.equal(c.to(torch.int64), want.to(torch.int64))
+    else:
+        assert rel_err(c.double().cpu().numpy(), want.cpu().numpy()) <= fp32_tol(k)
+
+
 def test_deep_kernel_batches_cin_bf16_out_transposed_c(device, oracle):
     import torch
     from vecops_amd import capi

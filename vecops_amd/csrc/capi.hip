@@ -368,6 +368,7 @@ void finish_tile_plan(const Problem& pr, VecopsHipPlan* plan, uint32_t forced_sp
 }
 
 int fetch_mode(const Problem& pr, const VecopsHipPlan& plan);
+bool lines_up(const Problem& pr, const View& v, int64_t line_stride);
 
 // The two halves of a problem cut between columns n_main - 1 and n_main of C: rows of B, columns of C and C_in.
 void cut_columns(const Problem& pr, int64_t n_main, Problem* main, Problem* rest) {
@@ -525,8 +526,12 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // K-contiguous, or 16-bit operands with B as [K,N]), K in whole K tiles
   const bool deep_tr = mode == MODE_NVEC_B_DMA && (pr.src == SRC_BF16 || pr.src == SRC_F16) && pr.n % 8 == 0 &&
                        pr.k * pr.b.cs * 2 + 256 < (int64_t{1} << 31);   // B as [K,N]: 16-bit operands, 32-bit K offsets
-  const bool deep_ok = ((mode == MODE_KVEC_DMA && (pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8)) || deep_tr) &&
-                       !pr.packed_b && pr.k % ktile == 0 && k_tiles >= kRules.deep_min_k_tiles;
+  // (a prepacked B keeps its pack order in LDS there: A's alignment decides)
+  const bool deep_pk = pr.packed_b && (pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && plan->vector_a != 0 &&
+                       lines_up(pr, pr.a, pr.a.rs);
+  const bool deep_ok = (pr.packed_b ? deep_pk
+                                    : (mode == MODE_KVEC_DMA && (pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8)) || deep_tr) &&
+                       pr.k % ktile == 0 && k_tiles >= kRules.deep_min_k_tiles;
   // At most four K tiles of 16-bit or 8-bit operands: the tile's life is its start-up and its stores, and
   // two or three 128x128 workgroups on a compute unit overlap one's stores with another's loads, which a
   // single big tile cannot (batch 8 of 3000x3000x17 to fp32: 93 us against 111; 8 x 1000x1000x100: 17.7
@@ -554,7 +559,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // -> 64, 768 x 4096 x 8192 78 -> 60, 1024 x 2048 x 8192 52 -> 43, 640 x 4096 x 4096 41 -> 34, 768 x 4096 x 4096
   // 41 -> 39; int8: 768 x 3072 x 12288 58 -> 42; with sixteen per part - 512 x 4096 x 4096, int8 1024 x 2048 x 8192 -
   // the unsplit small tiles stay ahead, 28.0 against 30.8 and 28.8 against 33.0).  Measured with loads that write
-  // LDS themselves, so only there.
+  // LDS themselves, so only there (a prepacked B: only the four-stage kernel's branches below).
   // The same from 32 tiles of 128x128 on, five to sixteen ways (bf16 512 x 2048 x 16384 73 us -> 43, 384 x 3072 x 8192
   // 46 -> 33, 512 x 3072 x 8192 48 -> 40; the 64x64 tiles the table took there are 128 workgroups or more, which the
   // rule for few workgroups leaves whole): fewer parts, down to six, where that reaches the twenty K tiles (int8
@@ -565,8 +570,8 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // with thirty-two per part - bf16 1024 x 4096 x 4096, int8 ... x 8192 - the unsplit tiles are level or ahead).
   uint32_t band_split = 0;
   bool deep_planned = false;
-  if (direct && !pr.packed_b && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) && tiles(128) >= kComputeUnits / 8 &&
-      tiles(128) <= kComputeUnits) {
+  if (((direct && !pr.packed_b) || (deep_pk && deep_ok)) && (family == VECOPS_HIP_FAMILY_TILE_64 || family == VECOPS_HIP_FAMILY_TILE_128) &&
+      tiles(128) >= kComputeUnits / 8 && tiles(128) <= kComputeUnits) {
     const int64_t count = tiles(128);
     int64_t parts = kRules.small_tile_workgroups_per_unit * kComputeUnits / count;
     while (parts > kRules.band_min_parts && k_tiles / parts < kRules.band_k_tiles_per_part) --parts;
@@ -601,7 +606,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
       family = VECOPS_HIP_FAMILY_TILE_128;
       band_split = static_cast<uint32_t>(kRules.deep_max_workgroups / count);
       deep_planned = true;
-    } else if (k_tiles / parts >= least && fits) {
+    } else if (!pr.packed_b && k_tiles / parts >= least && fits) {
       family = VECOPS_HIP_FAMILY_TILE_128;
       band_split = static_cast<uint32_t>(parts);
     }
@@ -943,14 +948,19 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     e = launch_tile_gemm_i8_wide(p, pr.packed_b, stream);
   } else if (pr.packed_b && launch_tile_gemm_packed16_serves(pr.src, p, tile_m, tile_n)) {
     e = launch_tile_gemm_packed16(pr.src, p, stream);
+  } else if (pr.packed_b && tile_m == 128 && tile_n == 128 && p.k_tiles_per_split >= kRules.deep_min_k_tiles &&
+             static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.batch * p.split_k <= kRules.deep_max_workgroups &&
+             launch_tile_gemm_deep128_serves(pr.src, p, mode, true)) {
+    // at most one workgroup per compute unit: the four-stage kernel with the pack kept in its order in LDS
+    e = launch_tile_gemm_deep128(pr.src, p, mode, true, stream);
   } else if (pr.packed_b) {
     const int a_mode = plan.vector_a == 0 ? 0 : ((pr.src == SRC_BF16 || pr.src == SRC_F16 || pr.src == SRC_I8) && lines_up(pr, pr.a, pr.a.rs)) ? 2 : 1;
     e = launch_tile_gemm_packed_b(pr.src, p, tile_m, tile_n, a_mode, stream);
   } else if (tile_m == 128 && tile_n == 128 && p.k_tiles_per_split >= kRules.deep_min_k_tiles &&
              static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.batch * p.split_k <= kRules.deep_max_workgroups &&
-             launch_tile_gemm_deep128_serves(pr.src, p, mode)) {
+             launch_tile_gemm_deep128_serves(pr.src, p, mode, false)) {
     // at most one workgroup per compute unit: the four-stage kernel, whose loads run three K tiles ahead
-    e = launch_tile_gemm_deep128(pr.src, p, mode, stream);
+    e = launch_tile_gemm_deep128(pr.src, p, mode, false, stream);
   } else if (pr.src == SRC_F32 && tile_m == tile_n && (tile_m == 64 || tile_m == 128) && (mode == MODE_KVEC || mode == MODE_NVEC_B) &&
              p.k_tiles_per_split >= kRules.deep_min_k_tiles &&
              static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.batch * p.split_k <= kRules.deep_max_workgroups &&

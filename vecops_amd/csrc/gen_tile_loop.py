@@ -371,6 +371,11 @@ def deep_reads(st, ks, to_set, tr):
         q = (2 * ks ^ f) & 3
         if kind == "a":
             out.append(f"ds_read_b128 {deep_fa(to_set, f)}, %[la{pair}{q}] offset:{odd * DEEP_STAGE + f * 2048}")
+        elif tr == "pk":
+            # B prepacked and kept in its pack order: block j lies in the wavefront's panel j / 2 (4 KiB a K tile),
+            # rows 16 (j % 2) .. + 15; the matrix k-step reads the pack's k-steps 2 ks and 2 ks + 1 (1 KiB each); the
+            # lane's chunk and row are in the one base register
+            out.append(f"ds_read_b128 {deep_fb(to_set, f)}, %[lb{pair}0] offset:{odd * DEEP_STAGE + (f >> 1) * 4096 + ks * 2048 + (f & 1) * 256}")
         elif tr:
             # B as [k][n]: column block j in base j / 2, 32 bytes on for the odd one; the two reads give k 0-3 and 4-7
             # of the lane's chunk
@@ -407,7 +412,7 @@ def deep_k_tile(st, tr):
                       f"buffer_load_dwordx4 %[ra{p}], s[80:83], %[ka] offen lds"))
     for p in range(4):
         m0 = f"s_add_u32 m0, %[m0w], {target * DEEP_STAGE + DEEP_B + p * 4096}"
-        if tr:
+        if tr is True:
             pre = [m0, "s_mov_b32 s88, %[kb]"] if p == 0 else [m0, "s_add_u32 s88, s88, %[pb]"]
             loads.append((pre, "buffer_load_dwordx4 %[rb0], s[84:87], s88 offen lds"))
         else:
@@ -475,6 +480,8 @@ def main():
     w(as_macro("VECOPS_LOOP128_DEEP", deep_loop(False)))
     w("\n// ... with B as it lies in memory ([k][n]), transposed by the LDS reads\n")
     w(as_macro("VECOPS_LOOP128_DEEP_TR", deep_loop(True)))
+    w("\n// The same with B prepacked (vecops_hip_pack_b's layout, kept in its own order in LDS).\n")
+    w(as_macro("VECOPS_LOOP128_DEEP_PK", deep_loop("pk")))
     w("#define VECOPS_LOOP128_ACCUMULATORS(t) \\\n  " +
       ", \\\n  ".join(", ".join(f'[c{x}] "+a"(t[{x // 4}][{x % 4}])' for x in range(r, r + 4)) for r in range(0, 16, 4)) + "\n")
     w("#define VECOPS_LOOP128_CLOBBERS \\\n  " + ", ".join(f'"s{r}"' for r in range(80, 89)) + ", \\\n  " +

@@ -8,7 +8,9 @@
 // aligned bases, rows and batches (the loads write LDS themselves), or - 16-bit operands - B handed over as [K,N]
 // (TR: the tile lies [k][n] in LDS, 64 rows of 256 bytes, swizzled as tile_gemm_kernel's, and the fragment reads
 // transpose); K a whole number of K tiles.  Any M, N, batch count, K split, C input and output type of the class: the
-// epilogue is tile_gemm_kernel's.
+// epilogue is tile_gemm_kernel's.  PK: B prepacked by vecops_hip_pack_b and kept in its pack order in LDS - a load
+// instruction of a wavefront moves one whole (panel of 32 rows, k-step of two chunks) block, 1 KiB contiguous on both
+// sides, and a fragment read is the stage pair's one per-lane base plus a constant (as in tile_gemm_packed16.hip).
 #include "tile_gemm_launch.h"
 
 namespace vecops_hip {
@@ -18,8 +20,9 @@ namespace {
 constexpr int kDeepStage = 32768;  // 128 rows of A, then 128 of B, 128 bytes of K each
 constexpr int kDeepStages = 4;
 
-template <int SRC, bool TR>
+template <int SRC, bool TR, bool PK>
 __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGemmParams p) {
+  static_assert(!(TR && PK), "one layout of B");
   using T = SrcTraits<SRC>;
   constexpr bool INT = T::kInt;
   constexpr int KTILE = 8 * T::kElemsPerChunk;
@@ -65,15 +68,26 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
       const int col = min(n0 + chunk * 8, p.n - 8) - n0;
       rows_b[0] = static_cast<uint32_t>((static_cast<int64_t>(krow) * p.b_ks + col) * T::kSrcBytes);
     }
+    if constexpr (PK) {
+      // B prepacked: instruction i moves the tile's panel i (clamped onto the operand's last panel), this wavefront the
+      // pack's k-step number `wave` of the K tile's four
+      const int64_t ks_total = static_cast<int64_t>(total_k_tiles) * 4;
+      const int nb0 = n0 / 32, nb_last = (p.n + 31) / 32 - 1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        rows_b[i] = static_cast<uint32_t>(((min(nb0 + i, nb_last) - nb0) * ks_total + wave) * 1024 + lane * 16);
+    }
   }
   // bytes from one K tile of B to the next, and (TR) from one of its four loads to the next
-  const uint32_t step_b = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(TR ? 64 * p.b_ks * T::kSrcBytes : 128));
+  const uint32_t step_b = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(TR ? 64 * p.b_ks * T::kSrcBytes : PK ? 4096 : 128));
   const uint32_t part_b = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(TR ? 16 * p.b_ks * T::kSrcBytes : 0));
   const u32x4 desc_a = tile_buffer_words((const VECOPS_GLOBAL char*)p.a +
                                          (static_cast<int64_t>(batch) * p.a_bs + static_cast<int64_t>(m0) * p.a_rs) * T::kSrcBytes);
   // (TR: the rows of the [N,K] view are one element apart)
+  // (PK: one packed operand for every batch; a panel's K tiles lie 4 KiB apart)
   const u32x4 desc_b = tile_buffer_words((const VECOPS_GLOBAL char*)p.b +
-                                         (static_cast<int64_t>(batch) * p.b_bs + static_cast<int64_t>(n0) * p.b_rs) * T::kSrcBytes);
+                                         (PK ? static_cast<int64_t>(n0 / 32) * total_k_tiles * 4096
+                                             : (static_cast<int64_t>(batch) * p.b_bs + static_cast<int64_t>(n0) * p.b_rs) * T::kSrcBytes));
   const uint32_t lds0 = lds_address_of(lds);
   const uint32_t m0_wave = lds0 + static_cast<uint32_t>(wave) * 1024u;
 
@@ -89,7 +103,8 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       load_16_bytes_into_lds(db, m0_wave, static_cast<uint32_t>(t * kDeepStage + 16384 + i * 4096), rows_b[TR ? 0 : i],
-                             TR ? static_cast<uint32_t>(kt_begin + t) * step_b + static_cast<uint32_t>(i) * part_b : k_bytes);
+                             TR ? static_cast<uint32_t>(kt_begin + t) * step_b + static_cast<uint32_t>(i) * part_b
+                                : PK ? static_cast<uint32_t>(kt_begin + t) * step_b : k_bytes);
   };
   fill(0);
   fill(1);
@@ -114,6 +129,10 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
           int col_bytes = ((wn * 4 + 2 * q) * 16 + (frag_row & 3) * 4) * 2;
           col_bytes ^= ((frag_row >> 2) & 3) << 6;
           base_b[pair][q] = lds0 + pair * 2 * kDeepStage + 16384 + (frag_chunk * 8 + (frag_row >> 2)) * 256 + col_bytes;
+        } else if constexpr (PK) {
+          // [panel][k-step of the pack: chunk / 2][half: chunk % 2][row of the panel][16 bytes]: the wavefront's two panels
+          base_b[pair][q] = lds0 + pair * 2 * kDeepStage + 16384 + wn * 2 * 4096 + (frag_chunk >> 1) * 1024 +
+                            (frag_chunk & 1) * 512 + frag_row * 16;
         } else {
           base_b[pair][q] = lds0 + pair * 2 * kDeepStage + 16384 + (wn * 64 + frag_row) * 128 + (((slot ^ (2 * q)) & 7) << 4);
         }
@@ -147,7 +166,11 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
                    [db0] "s"(db[0]), [db1] "s"(db[1]), [db2] "s"(db[2]), [db3] "s"(db[3]), [m0w] "s"(m0w),            \
                    [sb] "s"(sb), [pb] "s"(pb)                                                                         \
                  : "memory", "m0", "scc", VECOPS_LOOP128_CLOBBERS)
-    if constexpr (TR) {
+    if constexpr (PK) {
+      if constexpr (SRC == SRC_F16) VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP_PK("v_mfma_f32_16x16x32_f16"));
+      else if constexpr (INT) VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP_PK("v_mfma_i32_16x16x64_i8"));
+      else VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP_PK("v_mfma_f32_16x16x32_bf16"));
+    } else if constexpr (TR) {
       static_assert(SRC == SRC_BF16 || SRC == SRC_F16, "transposing LDS reads move 16-bit elements");
       if constexpr (SRC == SRC_F16) VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP_TR("v_mfma_f32_16x16x32_f16"));
       else VECOPS_DEEP_STATEMENT(VECOPS_LOOP128_DEEP_TR("v_mfma_f32_16x16x32_bf16"));
@@ -163,11 +186,11 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
   store_accumulators<SRC, 2, 2, 2, 2, kLdsBytes, true>(p, lds, acc, batch, split, m0, n0, wm, wn, wave, lane);
 }
 
-template <int SRC, bool TR>
+template <int SRC, bool TR, bool PK>
 hipError_t launch(const TileGemmParams& p, hipStream_t stream) {
   constexpr int kEpilogue = kEpilogueLdsBytes<2, 2, 2, 2>();
   constexpr int kLds = kDeepStages * kDeepStage > kEpilogue ? kDeepStages * kDeepStage : kEpilogue;
-  auto kernel = tile_gemm_deep128_kernel<SRC, TR>;
+  auto kernel = tile_gemm_deep128_kernel<SRC, TR, PK>;
   static thread_local int configured_device = -1;
   int device = 0;
   hipError_t e = hipGetDevice(&device);
@@ -185,24 +208,38 @@ hipError_t launch(const TileGemmParams& p, hipStream_t stream) {
 
 }  // namespace
 
-bool launch_tile_gemm_deep128_serves(int src, const TileGemmParams& p, int mode) {
+bool launch_tile_gemm_deep128_serves(int src, const TileGemmParams& p, int mode, bool packed_b) {
   if (src != SRC_BF16 && src != SRC_F16 && src != SRC_I8) return false;
-  const bool tr = mode == MODE_NVEC_B_DMA;
-  if ((mode != MODE_KVEC_DMA && !tr) || (tr && src == SRC_I8) || p.m <= 0 || p.n <= 0 || p.split_k < 1) return false;
+  const bool tr = !packed_b && mode == MODE_NVEC_B_DMA;
+  if (p.m <= 0 || p.n <= 0 || p.split_k < 1) return false;
   const int elem = src == SRC_I8 ? 1 : 2, ktile = 128 / elem;
   if (p.k < ktile || p.k % ktile != 0) return false;
   // 32-bit byte offsets inside a tile's 128 rows
   if (128 * p.a_rs * elem + static_cast<int64_t>(p.k) * elem >= (int64_t{1} << 31)) return false;
+  if (packed_b) {
+    // A: loads that write LDS need 16-byte aligned addresses; B: 32-bit byte offsets inside the tile's four panels
+    if (p.a_ks != 1 || (reinterpret_cast<uintptr_t>(p.a) & 15u) != 0 || (p.a_rs * elem) % 16 != 0 || (p.a_bs * elem) % 16 != 0) return false;
+    return (reinterpret_cast<uintptr_t>(p.b) & 15u) == 0 && 4 * static_cast<int64_t>(p.k / ktile) * 4096 < (int64_t{1} << 31);
+  }
+  if ((mode != MODE_KVEC_DMA && !tr) || (tr && src == SRC_I8)) return false;
   if (tr) return p.n % 8 == 0 && p.n >= 8 && p.b_rs == 1 && static_cast<int64_t>(p.k) * p.b_ks * elem + 256 < (int64_t{1} << 31);
   return 128 * p.b_rs * elem + static_cast<int64_t>(p.k) * elem < (int64_t{1} << 31);
 }
 
-hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, int mode, hipStream_t stream) {
-  const bool tr = mode == MODE_NVEC_B_DMA;
+hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, int mode, bool packed_b, hipStream_t stream) {
+  const bool tr = !packed_b && mode == MODE_NVEC_B_DMA;
+  if (packed_b) {
+    switch (src) {
+      case SRC_BF16: return launch<SRC_BF16, false, true>(p, stream);
+      case SRC_F16: return launch<SRC_F16, false, true>(p, stream);
+      case SRC_I8: return launch<SRC_I8, false, true>(p, stream);
+      default: return hipErrorInvalidValue;
+    }
+  }
   switch (src) {
-    case SRC_BF16: return tr ? launch<SRC_BF16, true>(p, stream) : launch<SRC_BF16, false>(p, stream);
-    case SRC_F16: return tr ? launch<SRC_F16, true>(p, stream) : launch<SRC_F16, false>(p, stream);
-    case SRC_I8: return launch<SRC_I8, false>(p, stream);
+    case SRC_BF16: return tr ? launch<SRC_BF16, true, false>(p, stream) : launch<SRC_BF16, false, false>(p, stream);
+    case SRC_F16: return tr ? launch<SRC_F16, true, false>(p, stream) : launch<SRC_F16, false, false>(p, stream);
+    case SRC_I8: return launch<SRC_I8, false, false>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }

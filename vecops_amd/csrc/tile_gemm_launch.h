@@ -205,8 +205,9 @@ hipError_t launch_grouped_class(const GroupedTables& t, int tile, int mode, hipS
 bool launch_tile_gemm_packed16_serves(int src, const TileGemmParams& p, int tile_m, int tile_n);
 hipError_t launch_tile_gemm_packed16(int src, const TileGemmParams& p, hipStream_t stream);
 // The 128 x 128 tile on four LDS stages for launches of at most one workgroup per compute unit (tile_gemm_deep128.hip).
-bool launch_tile_gemm_deep128_serves(int src, const TileGemmParams& p, int mode);
-hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, int mode, hipStream_t stream);
+// packed_b: p.b is vecops_hip_pack_b's layout (mode is then not consulted).
+bool launch_tile_gemm_deep128_serves(int src, const TileGemmParams& p, int mode, bool packed_b);
+hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, int mode, bool packed_b, hipStream_t stream);
 // fp32 compute on 64 x 64 (tile = 64) or 128 x 128 tiles with a ring of LDS stages, for launches of at most one workgroup
 // per compute unit (tile_gemm_deep_f32.hip); b_as_kn: B handed over as [K,N].
 bool launch_tile_gemm_deep_f32_serves(const TileGemmParams& p, int tile, bool b_as_kn);
