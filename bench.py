@@ -93,7 +93,8 @@ def _kernel_label(plan, operands):
     loads = "16-byte loads" if plan.vector_a and plan.vector_b else "element loads"
     b = {0: "B K-contiguous", 1: "B as [K,N]", 2: "B strided"}[plan.b_layout]
     split = f", split-K {plan.split_k}" if plan.split_k > 1 else ""
-    kernel = "tile_gemm_wide_i8_kernel" if family == "tile_256x352" else f"tile_gemm_kernel<{operands}>"
+    wide = "tile_gemm_wide_i8_kernel" if operands.startswith("int8") else f"tile_gemm_wide_16_kernel<{operands}>"
+    kernel = wide if family == "tile_256x352" else f"tile_gemm_kernel<{operands}>"
     return f"vecops_hip {kernel} family {family}, {loads}, {b}{split}"
 
 
@@ -495,6 +496,9 @@ RULE_CHECK_SHAPES = [
     # B stored [K,N] (the layout of the headline line)
     ("bf16_kn", 1024, 4096, 4096), ("bf16_kn", 512, 4096, 4096), ("bf16_kn", 768, 3072, 12288), ("bf16_kn", 2048, 2048, 2048),
     ("bf16_kn", 256, 4096, 4096),
+    # where the 256 x 352 tile's count fits the units (16-bit operands, B [N,K])
+    ("bf16", 2048, 11008, 4096), ("bf16", 4096, 11008, 4096), ("bf16", 6144, 6144, 6144), ("bf16", 4096, 4224, 4096),
+    ("bf16", 1024, 11008, 4096), ("bf16", 3072, 4096, 4096),
 ]
 
 
@@ -505,7 +509,7 @@ def bench_rule_check(dev, steps, warmup):
     import numpy as np
     import torch
     from vecops_amd import capi, synth
-    families = ["tile_256", "tile_256x128", "tile_128x256", "tile_128", "tile_64"]
+    families = ["tile_256", "tile_256x352", "tile_256x128", "tile_128x256", "tile_128", "tile_64"]
     steps, warmup = max(10, steps // 10), max(10, warmup // 10)
     ws = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
     rows = []
@@ -768,7 +772,8 @@ def main() -> int:
         packed16, packed8 = bench_bf16_gemm_packed(dev, K, W), bench_int8_dequant_packed(dev, K, W)
         secondary = [bench_batched(dev, K, W, m, n, k)
                      for (m, n, k) in [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)]]
-        secondary += [bench_bf16_mid(dev, K, W, 1024, 4096, 4096, True), bench_bf16_mid(dev, K, W, 2048, 2048, 2048, False)]
+        secondary += [bench_bf16_mid(dev, K, W, 1024, 4096, 4096, True), bench_bf16_mid(dev, K, W, 2048, 2048, 2048, False),
+                      bench_bf16_mid(dev, K, W, 2048, 11008, 4096, False)]
         secondary += [bench_runtime_quant(dev, K, W), bench_grouped(dev, K, W), ceiling_bf16, ceiling_int8, read_ceiling, packed16,
                       packed8,
                       fp32["bf16"], fp32["f32"], gemv[16], gemv[4], gemv[1], int8]

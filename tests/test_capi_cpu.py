@@ -56,9 +56,20 @@ def test_rule_table_known_answers():
     # 344 tiles of 256x256 would take two rounds, the second a third full; 1376 of 128x128 two and two thirds at two
     # workgroups per unit; 256 tiles of 256x352 are exactly one round
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256x352" and p.split_k == 1 and p.workspace_bytes == 0
-    # the same extents where that tile cannot serve: bf16 operands, an M that is no multiple of 256, rows of A that are
+    # bf16 and f16 operands take that tile too (the same loop on their 16x16x32 instructions), to their own type or fp32
+    for dtype, out in ((capi.BF16, capi.BF16), (capi.BF16, capi.F32), (capi.F16, capi.F16)):
+        rc, p = _plan(_operand(dtype, (2048, 4096)), _operand(dtype, (11008, 4096)), _operand(out, (2048, 11008)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256x352" and p.split_k == 1 and p.workspace_bytes == 0
+    # 4096 x 11008: 512 of them are two rounds where 688 square ones are three; 6144^3: 432 against 576; 4096^3 and
+    # 8192^3 keep the square tile (192 wide ones leave a quarter of the units idle; 768 are three rounds against four
+    # of less work)
+    for (m, n, k), family in (((4096, 11008, 4096), "tile_256x352"), ((6144, 6144, 6144), "tile_256x352"),
+                              ((4096, 4096, 4096), "tile_256"), ((8192, 8192, 8192), "tile_256"), ((4096, 4096, 11008), "tile_256")):
+        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == family, (m, n, k, p.family)
+    # the same extents where that tile cannot serve: B as [K,N], an M that is no multiple of 256, rows of A that are
     # not 16-byte aligned, a K that is no multiple of 128 - the 128x128 tile as before
-    rc, p = _plan(_operand(capi.BF16, (2048, 4096)), _operand(capi.BF16, (11008, 4096)), _operand(capi.BF16, (2048, 11008)))
+    rc, p = _plan(_operand(capi.BF16, (2048, 4096)), _operand(capi.BF16, (11008, 4096), strides=(1, 11008)), _operand(capi.BF16, (2048, 11008)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
     rc, p = _plan(_operand(capi.I8, (2040, 4096)), _operand(capi.I8, (11008, 4096)), _operand(capi.I32, (2040, 11008)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
@@ -94,8 +105,11 @@ def test_rule_table_known_answers():
     # 3000^3: 144 big tiles in one part-filled round stay ahead of 576 small ones in three
     rc, p = _plan(_operand(capi.BF16, (3000, 3000)), _operand(capi.BF16, (3000, 3000)), _operand(capi.F32, (3000, 3000)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
-    # 4096 x 4224: 272 big tiles would leave the second round 6 % full; 1056 of 128x128 are five per compute unit
+    # 4096 x 4224: 272 big tiles would leave the second round 6 % full; 192 tiles of 256x352 are one round, three
+    # quarters full (1056 of 128x128, five per compute unit, where that tile cannot serve: B as [K,N])
     rc, p = _plan(_operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (4224, 4096)), _operand(capi.F32, (4096, 4224)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256x352"
+    rc, p = _plan(_operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (4224, 4096), strides=(1, 4224)), _operand(capi.F32, (4096, 4224)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
     # config 3's 3000 x 3000 x 17: one K tile, the output is the work - several small workgroups per compute unit
     rc, p = _plan(_operand(capi.BF16, (3000, 17)), _operand(capi.BF16, (3000, 17)), _operand(capi.F32, (3000, 3000)))
@@ -179,13 +193,14 @@ def test_rule_table_known_answers():
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == 1, (n, p.family, p.split_k)
     # two rounds of 128 x 128 tiles and eight more: the last column of tiles is a product of its own (64 x 64 tiles, K in
     # five parts), the rest fills two rounds; a required family runs the product whole
-    big_n = (_operand(capi.BF16, (1536, 4096)), _operand(capi.BF16, (11008, 4096)), _operand(capi.BF16, (1536, 11008)))
+    # (B as [K,N]: with B [N,K] these extents take the 256 x 352 tile, 192 of them in one round)
+    big_n = (_operand(capi.BF16, (1536, 4096)), _operand(capi.BF16, (11008, 4096), strides=(1, 11008)), _operand(capi.BF16, (1536, 11008)))
     rc, p = _plan(*big_n)
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.split_k == 1 and p.peeled_columns == 128
     assert p.workspace_bytes == 5 * 1536 * 128 * 4
     rc, p = _plan_family(*big_n, "tile_128", capi.SELECT_REQUIRE)
     assert rc == 0 and p.peeled_columns == 0 and p.workspace_bytes == 0
-    rc, p = _plan(_operand(capi.BF16, (2048, 4096)), _operand(capi.BF16, (11008, 4096)), _operand(capi.BF16, (2048, 11008)))
+    rc, p = _plan(_operand(capi.BF16, (2048, 4096)), _operand(capi.BF16, (11008, 4096), strides=(1, 11008)), _operand(capi.BF16, (2048, 11008)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128" and p.peeled_columns == 0   # 1376 tiles: the third round is two thirds full
     # a split must pay for its second kernel: sixteen or thirty-two K tiles are walked in one go, sixty-four are not
     for (m, n, k), split in (((384, 384, 1024), 1), ((640, 640, 2048), 1), ((512, 512, 4096), 4), ((64, 64, 65536), 64)):

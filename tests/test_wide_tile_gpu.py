@@ -1,9 +1,10 @@
-"""The 256 x 352 workgroup tile of signed 8-bit operands (family tile_256x352), through the C ABI: int32 sums bit-exact
+"""The 256 x 352 workgroup tile (family tile_256x352), through the C ABI.  Signed 8-bit operands: int32 sums bit-exact
 against exact integer arithmetic on shapes with one, two, three and more K tiles, ragged N (clamped rows, guarded
 stores), several tile rows and columns; the dequantising epilogue bit-exact against the oracle (the same two
 separately rounded multiplies, vecops matmul/Quantization.h:195-250) on a shape the rule table itself gives to this
 tile; and the family request's error behaviour (a required family that cannot serve the operands is NotApplicable,
-tests/ops/MatmulTest.cpp:514-536)."""
+tests/ops/MatmulTest.cpp:514-536).  bf16 and f16 operands on the same tile: against float64 sums of the same
+operands and against the 256 x 256 tile, to fp32 and to the operands' own type."""
 import numpy as np
 import pytest
 
@@ -112,8 +113,10 @@ def test_wide_tile_required_where_it_cannot_serve(device):
         "M not a multiple of 256": (i8((300, 512)), i8((352, 512)), torch.int32),
         "K not a multiple of 128": (i8((256, 520)), i8((352, 520)), torch.int32),
         "a single K tile": (i8((256, 128)), i8((352, 128)), torch.int32),
-        "bf16 operands": (torch.zeros((256, 512), dtype=torch.bfloat16, device=device),
-                          torch.zeros((352, 512), dtype=torch.bfloat16, device=device), torch.float32),
+        "fp32 operands": (torch.zeros((256, 512), dtype=torch.float32, device=device),
+                          torch.zeros((352, 512), dtype=torch.float32, device=device), torch.float32),
+        "bf16 operands, B as [K,N]": (torch.zeros((256, 512), dtype=torch.bfloat16, device=device),
+                                      torch.zeros((512, 352), dtype=torch.bfloat16, device=device).t(), torch.float32),
         "unsigned a": (torch.zeros((256, 512), dtype=torch.uint8, device=device), i8((352, 512)), torch.int32),
     }
     for name, (a, b, out) in cases.items():
@@ -129,3 +132,55 @@ def test_wide_tile_required_where_it_cannot_serve(device):
     with pytest.raises(capi.VecopsHipError):
         capi.matmul_family(a, b, c, capi.family_request("tile_256x352", capi.SELECT_REQUIRE, split_k=2))
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("kind,out", [("bf16", "f32"), ("bf16", "own"), ("f16", "f32"), ("f16", "own")])
+@pytest.mark.parametrize("m,n,k", [(256, 352, 128), (256, 352, 192), (512, 1000, 512), (256, 4, 256), (768, 3000, 1024),
+                                   (256, 356, 2048)])
+def test_wide_tile_16_bit_operands(device, kind, out, m, n, k):
+    import torch
+    from vecops_amd import capi
+    from conftest import rel_err
+    from test_matmul_gpu import fp32_tol
+    dtype = torch.bfloat16 if kind == "bf16" else torch.float16
+    gen = torch.Generator().manual_seed(m + 3 * n + 7 * k)
+    a = (torch.rand((m, k), generator=gen) * 2 - 1).to(dtype).to(device)
+    b = (torch.rand((n, k), generator=gen) * 2 - 1).to(dtype).to(device)
+    out_dtype = torch.float32 if out == "f32" else dtype
+    c_store = torch.full((m, n + 12), -7.0, dtype=out_dtype, device=device)   # rows of C with a pad that must stay
+    c = c_store[:, :n]
+    request = capi.family_request("tile_256x352", capi.SELECT_REQUIRE)
+    assert capi.FAMILY_NAMES[capi.plan_matmul_family(a, b, c, request).family] == "tile_256x352"
+    capi.matmul_family(a, b, c, request)
+    square = torch.empty((m, n), dtype=out_dtype, device=device)
+    capi.matmul_family(a, b, square, capi.family_request("tile_256", capi.SELECT_REQUIRE, split_k=1))
+    torch.cuda.synchronize()
+    want = (a.double() @ b.double().t()).cpu().numpy()
+    tol = fp32_tol(k) + (0.0 if out == "f32" else 2.0 ** (-8 if kind == "bf16" else -11) * 1.01)
+    assert rel_err(c.double().cpu().numpy(), want) <= tol
+    assert rel_err(c.double().cpu().numpy(), square.double().cpu().numpy()) <= tol   # the order of the fp32 sums may differ
+    assert bool((c_store[:, n:] == -7.0).all())
+
+
+def test_wide_tile_bf16_is_the_tables_choice_where_its_count_fits(device):
+    """2048 x 11008 x 4096 in bf16 (B [N,K]): 256 tiles of 256 x 352 are one round; with prepacked weights too.  Every
+    output enters a checksum (C v against A (B^T v) in float64)."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = 2048, 11008, 4096
+    a = torch.from_numpy(synth.bf16_round(synth.normal(1, (m, k), 0.02)).view(np.int16)).to(device).view(torch.bfloat16)
+    b = torch.from_numpy(synth.bf16_round(synth.normal(2, (n, k), 0.02)).view(np.int16)).to(device).view(torch.bfloat16)
+    c = torch.empty((m, n), dtype=torch.float32, device=device)
+    assert capi.FAMILY_NAMES[capi.plan_matmul(a, b, c).family] == "tile_256x352"
+    capi.matmul(a, b, c)
+    packed = capi.pack_b(b)
+    assert capi.FAMILY_NAMES[capi.plan_matmul_packed_b(a, packed, c).family] == "tile_256x352"
+    cp = torch.empty_like(c)
+    capi.matmul_packed_b(a, packed, cp)
+    torch.cuda.synchronize()
+    assert torch.equal(c, cp)                                # the same loop on the same K order
+    v = torch.from_numpy(np.random.default_rng(3).standard_normal(n)).to(device)
+    got = c.double() @ v
+    want = a.double() @ (b.double().t() @ v)
+    scale = (a.double().abs() @ (b.double().abs().t() @ v.abs())).clamp(min=1e-30)
+    assert float(((got - want).abs() / scale).max()) <= 2e-6 * k / 32

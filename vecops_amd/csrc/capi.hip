@@ -385,22 +385,26 @@ void cut_columns(const Problem& pr, int64_t n_main, Problem* main, Problem* rest
   }
 }
 
-// Whether the 256 x 352 tile (tile_gemm_wide_i8.hip) can run a problem: signed 8-bit operands, both K-contiguous with
-// 16-byte aligned bases and rows, K a multiple of 128 (two K tiles or more), M of 256, N of 4, one batch, no C input, no
-// fused transform, a row-major C with 16-byte aligned rows (int32 sums, or fp32 when dequantising).
+// Whether the 256 x 352 tile (tile_gemm_wide_i8.hip) can run a problem: signed 8-bit, bf16 or f16 operands, both
+// K-contiguous with 16-byte aligned bases and rows, K a whole number of K tiles of 128 bytes (two or more), M a multiple
+// of 256, N of 4, one batch, no C input, no fused transform, a row-major C with 16-byte aligned rows (int32 sums, or fp32
+// when dequantising; the 16-bit classes: fp32 or the operands' own type).
 bool wide_tile_serves(const Problem& pr) {
-  if (pr.src != SRC_I8 || pr.has_cin || pr.fused != nullptr || pr.batch != 1) return false;
-  if (pr.k % 128 != 0 || pr.k < 256 || pr.m % 256 != 0 || pr.n % 4 != 0 || pr.m == 0 || pr.n == 0) return false;
-  if (pr.a.cs != 1 || pr.a.rs % 16 != 0 || !aligned16(pr.a.data) || !aligned16(pr.b.data)) return false;
+  const bool bytes = pr.src == SRC_I8;
+  if ((!bytes && pr.src != SRC_BF16 && pr.src != SRC_F16) || pr.has_cin || pr.fused != nullptr || pr.batch != 1) return false;
+  const int64_t elem = bytes ? 1 : 2, ktile = 128 / elem;
+  if (pr.k % ktile != 0 || pr.k < 2 * ktile || pr.m % 256 != 0 || pr.n % 4 != 0 || pr.m == 0 || pr.n == 0) return false;
+  if (pr.a.cs != 1 || (pr.a.rs * elem) % 16 != 0 || !aligned16(pr.a.data) || !aligned16(pr.b.data)) return false;
   if (pr.packed_b) {  // (a prepacked B: its 32-row panels are the tile's parts; 32-bit offsets into it)
-    if ((pr.n + 31) / 32 * (pr.k / 32) * 1024 >= (int64_t{1} << 31)) return false;
-  } else if (pr.b.cs != 1 || pr.b.rs % 16 != 0 || 352 * pr.b.rs >= (int64_t{1} << 31)) {
+    if ((pr.n + 31) / 32 * (pr.k * elem / 32) * 1024 >= (int64_t{1} << 31)) return false;
+  } else if (pr.b.cs != 1 || (pr.b.rs * elem) % 16 != 0 || 352 * pr.b.rs * elem >= (int64_t{1} << 31)) {
     return false;
   }
   if (pr.c.cs != 1 || pr.c.rs % 4 != 0 || !aligned16(pr.c.data)) return false;
-  if (256 * pr.a.rs >= (int64_t{1} << 31)) return false;
+  if (256 * pr.a.rs * elem >= (int64_t{1} << 31)) return false;
   // (a dequantised product is described with its accumulator class, int32, and leaves as fp32)
-  return pr.out_kind == OUT_I32 || (pr.dequant && pr.out_kind == OUT_F32);
+  if (bytes) return pr.out_kind == OUT_I32 || (pr.dequant && pr.out_kind == OUT_F32);
+  return !pr.dequant && (pr.out_kind == OUT_F32 || pr.out_kind == (pr.src == SRC_BF16 ? OUT_BF16 : OUT_F16));
 }
 
 // How the operands of a (non-empty) problem can be fetched: the plan's vector flags and B's layout.
@@ -943,9 +947,9 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     if (rc != ST_OK) return rc;
   }
   if (plan.family == VECOPS_HIP_FAMILY_TILE_256X352) {
-    if (!wide_tile_serves(pr) || !launch_tile_gemm_i8_wide_serves(p, mode, pr.packed_b))
+    if (!wide_tile_serves(pr) || !launch_tile_gemm_wide_serves(pr.src, p, mode, pr.packed_b))
       return fail(ST_INVALID, "matmul: the plan's family tile_256x352 cannot serve this call");
-    e = launch_tile_gemm_i8_wide(p, pr.packed_b, stream);
+    e = launch_tile_gemm_wide(pr.src, p, pr.packed_b, stream);
   } else if (pr.packed_b && launch_tile_gemm_packed16_serves(pr.src, p, tile_m, tile_n)) {
     e = launch_tile_gemm_packed16(pr.src, p, stream);
   } else if (pr.packed_b && tile_m == 128 && tile_n == 128 && p.k_tiles_per_split >= kRules.deep_min_k_tiles &&

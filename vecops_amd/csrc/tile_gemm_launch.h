@@ -42,8 +42,8 @@ hipError_t launch_quantize_rows(const float* x, int32_t batch, int32_t rows, int
 // the 256 x 352 tile of signed 8-bit operands (tile_gemm_wide_i8.hip): p.tiles_m / p.tiles_n count its tiles; `serves`
 // says whether it can run the problem (mode: the operands' LoadMode)
 // (packed_b: p.b is the operand as launch_pack_b lays it out)
-bool launch_tile_gemm_i8_wide_serves(const TileGemmParams& p, int mode, bool packed_b);
-hipError_t launch_tile_gemm_i8_wide(const TileGemmParams& p, bool packed_b, hipStream_t stream);
+bool launch_tile_gemm_wide_serves(int src, const TileGemmParams& p, int mode, bool packed_b);
+hipError_t launch_tile_gemm_wide(int src, const TileGemmParams& p, bool packed_b, hipStream_t stream);
 hipError_t launch_splitk_reduce(const TileGemmParams& p, bool is_int, hipStream_t stream);
 // B prepacked by launch_pack_b (src: SRC_BF16, SRC_F32_AS_BF16 = fp32 A against bf16-packed B, SRC_I8,
 // SRC_I8_FLIP = unsigned A against int8-packed B with p.a_flip and p.col_term set);
