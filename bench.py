@@ -356,7 +356,7 @@ def bench_runtime_quant(dev, steps, warmup):
             "uint8 on the way in, int8 weights 11008x4096, correction row, per-token x per-channel dequant, fp32 out",
             "value": tops, "unit": "TOP/s", "ms_per_step": t["wall_ms"], "dtype": "int8",
             "roofline": _roofline("mfma", tops, PEAK_INT8_TOPS, "TOP/s", traffic=None,
-                                  kernel="vecops_hip quantize_rows_kernel + byte_row_sums_kernel + " +
+                                  kernel="vecops_hip quantize_and_row_sums_kernel + " +
                                          _kernel_label(plan, "int8").replace("vecops_hip ", "") + ", dequantising epilogue",
                                   algorithmic_ops_per_launch=ops,
                                   algorithmic_bytes_per_launch=4 * m * k + n * k + 4 * m * n + 4 * (2 * m + 2 * n),

@@ -1435,13 +1435,26 @@ int32_t run_runtime_quant(const VecopsHipOperand* a, const float* multipliers, i
   hipStream_t s = static_cast<hipStream_t>(stream);
   View vx;
   normalise(&d.a3, &vx);
+  // correction[batch][n] + 128 * sum_k b[batch][n,k]
+  int32_t* rows = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + d.q_bytes);
+  if (packed == nullptr && d.q_batches * d.m * d.k > 0 && d.row_batches * d.n > 0) {
+    // the activations' quantisation and the weight rows' sums in one launch: neither needs the other
+    View vb;
+    normalise(&d.b3, &vb);
+    hipError_t both = launch_quantize_and_row_sums(
+        static_cast<const float*>(vx.data), static_cast<int32_t>(d.q_batches), static_cast<int32_t>(d.m), static_cast<int32_t>(d.k),
+        vx.bs, vx.rs, vx.cs, multipliers, d.scale_bs, zero_point, 0x80u, static_cast<uint8_t*>(workspace), d.m * d.k, d.k, 1,
+        vb.data, static_cast<int32_t>(d.row_batches), static_cast<int32_t>(d.n), vb.bs, vb.rs, vb.cs, 0u, 128u, correction,
+        d.correction_bs, rows, s);
+    if (both != hipSuccess) return fail(ST_EXEC, "quantize and row-sum kernel launch: %s", hipGetErrorString(both));
+    return run_problem(d.pr, d.plan, row_scales, column_scales, rows, static_cast<char*>(workspace) + d.q_bytes + d.row_bytes,
+                       workspace_size - d.q_bytes - d.row_bytes, s);
+  }
   hipError_t e = launch_quantize_rows(static_cast<const float*>(vx.data), static_cast<int32_t>(d.q_batches),
                                       static_cast<int32_t>(d.m), static_cast<int32_t>(d.k), vx.bs, vx.rs, vx.cs,
                                       multipliers, d.scale_bs, zero_point, 0x80u, static_cast<uint8_t*>(workspace),
                                       d.m * d.k, d.k, 1, s);
   if (e != hipSuccess) return fail(ST_EXEC, "quantize kernel launch: %s", hipGetErrorString(e));
-  // correction[batch][n] + 128 * sum_k b[batch][n,k]
-  int32_t* rows = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + d.q_bytes);
   if (packed != nullptr) {
     // one packed operand: the same sums for every batch, the caller's correction per batch
     for (int64_t bi = 0; bi < d.row_batches && e == hipSuccess; ++bi)

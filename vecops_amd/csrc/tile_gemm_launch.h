@@ -39,6 +39,12 @@ hipError_t launch_byte_row_sums(const void* x, int32_t batch, int32_t rows, int3
 hipError_t launch_quantize_rows(const float* x, int32_t batch, int32_t rows, int32_t k, int64_t xbs, int64_t xrs,
                                 int64_t xks, const float* multipliers, int64_t mult_bs, int32_t zero_point, uint32_t flip,
                                 uint8_t* q, int64_t qbs, int64_t qrs, int64_t qks, hipStream_t stream);
+// both of the above as one launch (each must have work to do): what a runtime-quantised product prepares
+hipError_t launch_quantize_and_row_sums(const float* x, int32_t batch, int32_t rows, int32_t k, int64_t xbs, int64_t xrs,
+                                        int64_t xks, const float* multipliers, int64_t mult_bs, int32_t zero_point, uint32_t flip,
+                                        uint8_t* q, int64_t qbs, int64_t qrs, int64_t qks, const void* w, int32_t w_batch,
+                                        int32_t w_rows, int64_t w_bs, int64_t w_rs, int64_t w_ks, uint32_t w_flip, uint32_t scale,
+                                        const int32_t* add, int64_t add_bs, int32_t* out, hipStream_t stream);
 // the 256 x 352 tile of signed 8-bit operands (tile_gemm_wide_i8.hip): p.tiles_m / p.tiles_n count its tiles; `serves`
 // says whether it can run the problem (mode: the operands' LoadMode)
 // (packed_b: p.b is the operand as launch_pack_b lays it out)
