@@ -71,7 +71,7 @@ typedef enum VecopsHipKernelFamily {
   VECOPS_HIP_FAMILY_TILE_256X128 = 6,  /* 256 (M) x 128 (N) workgroup tile, MFMA */
   VECOPS_HIP_FAMILY_TILE_128X256 = 7,  /* 128 (M) x 256 (N) workgroup tile, MFMA */
   VECOPS_HIP_FAMILY_TILE_256X352 = 8   /* 256 (M) x 352 (N) workgroup tile of signed 8-bit, bf16 or f16 operands (aligned,
-                                          K-contiguous, K in whole K tiles of 128 bytes, M a multiple of 256): the tile
+                                          K-contiguous, K in whole K tiles of 128 bytes): the tile
                                           that covers 2048 x 11008 in one round */
 } VecopsHipKernelFamily;
 

@@ -67,12 +67,13 @@ def test_rule_table_known_answers():
                               ((4096, 4096, 4096), "tile_256"), ((8192, 8192, 8192), "tile_256"), ((4096, 4096, 11008), "tile_256")):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family, (m, n, k, p.family)
-    # the same extents where that tile cannot serve: B as [K,N], an M that is no multiple of 256, rows of A that are
-    # not 16-byte aligned, a K that is no multiple of 128 - the 128x128 tile as before
+    # the same extents where that tile cannot serve: B as [K,N], rows of A that are not 16-byte aligned, a K that is no
+    # multiple of 128 - the 128x128 tile as before; an M that is no multiple of 256 is served (rows past M are fetched
+    # as zeros and not stored)
     rc, p = _plan(_operand(capi.BF16, (2048, 4096)), _operand(capi.BF16, (11008, 4096), strides=(1, 11008)), _operand(capi.BF16, (2048, 11008)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
     rc, p = _plan(_operand(capi.I8, (2040, 4096)), _operand(capi.I8, (11008, 4096)), _operand(capi.I32, (2040, 11008)))
-    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256x352"
     rc, p = _plan(_operand(capi.I8, (2048, 4096), strides=(4104, 1)), _operand(capi.I8, (11008, 4096)),
                   _operand(capi.I32, (2048, 11008)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"

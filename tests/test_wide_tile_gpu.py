@@ -14,7 +14,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 352, 256), (256, 352, 384), (256, 352, 640), (256, 704, 512), (512, 1000, 512),
-                                   (256, 180, 256), (768, 3000, 1024), (256, 356, 2048)])
+                                   (256, 180, 256), (768, 3000, 1024), (256, 356, 2048), (300, 352, 512), (1, 704, 256),
+                                   (257, 1000, 384), (1500, 3000, 1024), (129, 356, 256)])
 def test_wide_tile_int32_sums_are_exact(device, m, n, k):
     import torch
     from vecops_amd import capi
@@ -110,7 +111,6 @@ def test_wide_tile_required_where_it_cannot_serve(device):
     def i8(shape):
         return torch.zeros(shape, dtype=torch.int8, device=device)
     cases = {
-        "M not a multiple of 256": (i8((300, 512)), i8((352, 512)), torch.int32),
         "K not a multiple of 128": (i8((256, 520)), i8((352, 520)), torch.int32),
         "a single K tile": (i8((256, 128)), i8((352, 128)), torch.int32),
         "fp32 operands": (torch.zeros((256, 512), dtype=torch.float32, device=device),
@@ -136,7 +136,7 @@ def test_wide_tile_required_where_it_cannot_serve(device):
 
 @pytest.mark.parametrize("kind,out", [("bf16", "f32"), ("bf16", "own"), ("f16", "f32"), ("f16", "own")])
 @pytest.mark.parametrize("m,n,k", [(256, 352, 128), (256, 352, 192), (512, 1000, 512), (256, 4, 256), (768, 3000, 1024),
-                                   (256, 356, 2048)])
+                                   (256, 356, 2048), (300, 352, 256), (1, 704, 128), (1500, 3000, 512)])
 def test_wide_tile_16_bit_operands(device, kind, out, m, n, k):
     import torch
     from vecops_amd import capi

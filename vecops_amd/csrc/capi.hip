@@ -386,14 +386,14 @@ void cut_columns(const Problem& pr, int64_t n_main, Problem* main, Problem* rest
 }
 
 // Whether the 256 x 352 tile (tile_gemm_wide_i8.hip) can run a problem: signed 8-bit, bf16 or f16 operands, both
-// K-contiguous with 16-byte aligned bases and rows, K a whole number of K tiles of 128 bytes (two or more), M a multiple
-// of 256, N of 4, one batch, no C input, no fused transform, a row-major C with 16-byte aligned rows (int32 sums, or fp32
+// K-contiguous with 16-byte aligned bases and rows, K a whole number of K tiles of 128 bytes (two or more), N a multiple
+// of 4, one batch, no C input, no fused transform, a row-major C with 16-byte aligned rows (int32 sums, or fp32
 // when dequantising; the 16-bit classes: fp32 or the operands' own type).
 bool wide_tile_serves(const Problem& pr) {
   const bool bytes = pr.src == SRC_I8;
   if ((!bytes && pr.src != SRC_BF16 && pr.src != SRC_F16) || pr.has_cin || pr.fused != nullptr || pr.batch != 1) return false;
   const int64_t elem = bytes ? 1 : 2, ktile = 128 / elem;
-  if (pr.k % ktile != 0 || pr.k < 2 * ktile || pr.m % 256 != 0 || pr.n % 4 != 0 || pr.m == 0 || pr.n == 0) return false;
+  if (pr.k % ktile != 0 || pr.k < 2 * ktile || pr.n % 4 != 0 || pr.m == 0 || pr.n == 0) return false;
   if (pr.a.cs != 1 || (pr.a.rs * elem) % 16 != 0 || !aligned16(pr.a.data) || !aligned16(pr.b.data)) return false;
   if (pr.packed_b) {  // (a prepacked B: its 32-row panels are the tile's parts; 32-bit offsets into it)
     if ((pr.n + 31) / 32 * (pr.k * elem / 32) * 1024 >= (int64_t{1} << 31)) return false;
@@ -502,7 +502,7 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // The 256 x 352 tile of 8-bit operands: priced like the big tile (its loop is the same, with a tenth less operand
   // traffic per multiply-add), it wins where its count fits rounds that the square tiles' counts do not - 2048 x 11008:
   // 256 tiles in one round against 344 of 256 x 256 (two rounds) and 1376 of 128 x 128 (three).
-  if (wide_tile_serves(pr) && pr.n > 176) {
+  if (wide_tile_serves(pr) && pr.n > 176 && pr.m > 128) {   // (a tile at most half empty in either direction)
     const int64_t count = tiles2(256, 352), rounds = (count + kComputeUnits - 1) / kComputeUnits;
     if (count * kRules.min_busy_den >= kComputeUnits * kRules.min_busy_num) {
       int64_t cost = rounds * 256 * 352;

@@ -187,6 +187,7 @@ def loop(tr):
 #   instruction of each row of blocks, that row's A fragment of k-step 1 into the registers just freed.
 #   The barrier stands one row into k-step 1 (the last of those reads has landed by then); behind it the loads of
 #   the tile after the next go into this stage and the next tile's k-step 0 fragments are read from the other.
+# A's descriptor carries the bytes the tile's rows really have (%[na]: rows past M fetch zeros instead of being clamped).
 # LDS reads complete in order, so each matrix instruction waits for "at most N reads issued after the one I need":
 # the generator follows the reads through two trips of the loop and writes the counted waits.
 WIDE_FM, WIDE_FN = 8, 11
@@ -239,7 +240,7 @@ def wide_k_tile(st, tr):
         tr.read(out, ("b", to_set, j), f"ds_read_b128 {wide_fb(to_set, j)}, %[lb{stage}{q}] offset:{j * 4096}")
 
     out += ["s_cmp_gt_i32 %[left], 0",
-            "s_cselect_b32 s82, 0x7fffffff, 0",
+            "s_cselect_b32 s82, %[na], 0",
             "s_cselect_b32 s86, 0x7fffffff, 0",
             "s_sub_u32 %[left], %[left], 1"]
     loads = []
