@@ -943,6 +943,8 @@ def test_peeled_columns(device, oracle, kind, m, n, k):
     if kind == "bf16":
         a, b = synth.bf16_round(synth.uniform_pm1(1, (m, k))), synth.bf16_round(synth.uniform_pm1(2, (n, k)))
         ta, tb = dev_bf16(a, device), dev_bf16(b, device)
+        if k % 64 == 0:
+            tb = tb.t().contiguous().t()      # B stored [K,N]: with B [N,K] these extents take the 256 x 352 tile, which peels nothing
         cin = synth.uniform_pm1(3, (m, n)).astype(np.float32)
         c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
     else:
@@ -951,6 +953,8 @@ def test_peeled_columns(device, oracle, kind, m, n, k):
         cin = (synth.draws(3, m * n) % np.uint64(1 << 20)).astype(np.int32).reshape(m, n)
         c = torch.full((m, n), -1, dtype=torch.int32, device=device)
     tci = torch.from_numpy(cin).to(device)
+    if kind == "i8":
+        tci = tci.t().contiguous().t()        # (a C input whose rows are not contiguous: not the 256 x 352 tile's)
     plan = capi.plan_matmul(ta, tb, c, c_in=tci)
     assert capi.FAMILY_NAMES[plan.family] == "tile_128" and plan.split_k == 1 and 0 < plan.peeled_columns <= 256
     whole_plan = capi.plan_matmul_family(ta, tb, c, capi.family_request("tile_128"), c_in=tci)

@@ -184,3 +184,64 @@ def test_wide_tile_bf16_is_the_tables_choice_where_its_count_fits(device):
     want = a.double() @ (b.double().t() @ v)
     scale = (a.double().abs() @ (b.double().abs().t() @ v.abs())).clamp(min=1e-30)
     assert float(((got - want).abs() / scale).max()) <= 2e-6 * k / 32
+
+
+@pytest.mark.parametrize("kind,out", [("bf16", "bf16"), ("bf16", "f32"), ("i8", "i32"), ("i8", "u8"), ("i8", "f32")])
+def test_wide_tile_c_input_and_fused_transform(device, kind, out):
+    """A bias row (a C input of row stride 0), per-row and per-column scales, scale, shift and an activation on the
+    256 x 352 tile: the finishing step is tile_gemm_kernel's own, so the result equals the same call with B handed
+    over as [K,N] (which that tile does not serve) - bit for bit on the integer classes, up to the order of the fp32
+    sums otherwise - and the formula of the header on float64 sums."""
+    import torch
+    from vecops_amd import capi
+    from conftest import rel_err
+    m, n = 1500, 11000                            # 6 x 32 = 192 tiles: the table's own choice ...
+    k = 2048 if kind == "i8" else 512             # ... from nine K tiles of bytes on, five of 16-bit elements
+    gen = torch.Generator().manual_seed(11)
+    if kind == "i8":
+        a = torch.randint(-128, 128, (m, k), generator=gen, dtype=torch.int8).to(device)
+        b_kn = torch.randint(-128, 128, (k, n), generator=gen, dtype=torch.int8).to(device)
+        bias = torch.randint(-5000, 5000, (1, n), generator=gen, dtype=torch.int32).to(device)
+    else:
+        a = (torch.rand((m, k), generator=gen) * 2 - 1).to(torch.bfloat16).to(device)
+        b_kn = (torch.rand((k, n), generator=gen) * 2 - 1).to(torch.bfloat16).to(device)
+        bias = (torch.rand((1, n), generator=gen) * 2 - 1).to(torch.bfloat16).to(device)
+    b = b_kn.t().contiguous()                      # [N,K]: the 256 x 352 tile's layout
+    out_dtype = {"bf16": torch.bfloat16, "f32": torch.float32, "i32": torch.int32, "u8": torch.uint8}[out]
+    if out != "i32":
+        rs = (torch.rand(m, generator=gen) * 0.5 + 0.75).to(device)
+        cs = (torch.rand(n, generator=gen) * 0.5 + 0.75).to(device)
+        mag = 2.5e-4 if kind == "i8" else 1.0
+        ep = capi.epilogue(activation="relu" if out == "u8" else "silu", scale=0.5 * mag, shift=0.25, row_scales=rs, column_scales=cs)
+    # (a C input under both scale vectors on int32 sums - the kernels' dequantisation stage - is not this tile's)
+    with_bias = not (kind == "i8" and out != "i32")
+    c_in = bias.expand(m, n) if with_bias else None
+    c = torch.zeros((m, n), dtype=out_dtype, device=device)
+    other = torch.zeros((m, n), dtype=out_dtype, device=device)
+    if out == "i32":                                 # (no transform: the plain entry point with its C input)
+        assert capi.FAMILY_NAMES[capi.plan_matmul(a, b, c, c_in=c_in).family] == "tile_256x352"
+        capi.matmul(a, b, c, c_in=c_in)
+        assert capi.FAMILY_NAMES[capi.plan_matmul(a, b_kn.t(), other, c_in=c_in).family] != "tile_256x352"
+        capi.matmul(a, b_kn.t(), other, c_in=c_in)
+    else:
+        plan = capi.plan_matmul_fused(a, b, c, ep, c_in=c_in)
+        assert capi.FAMILY_NAMES[plan.family] == "tile_256x352"
+        capi.matmul_fused(a, b, c, ep, c_in=c_in)
+        assert capi.FAMILY_NAMES[capi.plan_matmul_fused(a, b_kn.t(), other, ep, c_in=c_in).family] != "tile_256x352"
+        capi.matmul_fused(a, b_kn.t(), other, ep, c_in=c_in)
+    torch.cuda.synchronize()
+    if kind == "i8":
+        assert torch.equal(c, other)
+    else:
+        assert rel_err(c.double().cpu().numpy(), other.double().cpu().numpy()) <= 2e-6 * k / 32 + (2.0 ** -8 if out == "bf16" else 0.0)
+    v = a.double() @ b.double().t() + (bias.double() if with_bias else 0.0)
+    if out == "i32":
+        assert torch.equal(c.to(torch.int64), v.to(torch.int64))
+        return
+    t = ((v * rs.double()[:, None]) * cs.double()[None, :]) * (0.5 * mag) + 0.25
+    want = torch.relu(t) if out == "u8" else t * torch.sigmoid(t)
+    if out == "u8":
+        want = want.clamp(0, 255).floor()
+        assert float((c.double() - want).abs().max()) <= 1.0      # truncation next to an integer boundary
+    else:
+        assert rel_err(c.double().cpu().numpy(), want.cpu().numpy()) <= 1e-4 + (2.0 ** -8 if out == "bf16" else 0.0)

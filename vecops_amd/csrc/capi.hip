@@ -386,12 +386,16 @@ void cut_columns(const Problem& pr, int64_t n_main, Problem* main, Problem* rest
 }
 
 // Whether the 256 x 352 tile (tile_gemm_wide_i8.hip) can run a problem: signed 8-bit, bf16 or f16 operands, both
-// K-contiguous with 16-byte aligned bases and rows, K a whole number of K tiles of 128 bytes (two or more), N a multiple
-// of 4, one batch, no C input, no fused transform, a row-major C with 16-byte aligned rows (int32 sums, or fp32
-// when dequantising; the 16-bit classes: fp32 or the operands' own type).
+// K-contiguous with 16-byte aligned bases and rows, K a whole number of K tiles of 128 bytes (two or more), any M, N a
+// multiple of 4, one batch, a row-major C with 16-byte aligned rows; a C input with contiguous rows (not under the
+// dequantisation), any fused transform and output type of the class.
 bool wide_tile_serves(const Problem& pr) {
   const bool bytes = pr.src == SRC_I8;
-  if ((!bytes && pr.src != SRC_BF16 && pr.src != SRC_F16) || pr.has_cin || pr.fused != nullptr || pr.batch != 1) return false;
+  if ((!bytes && pr.src != SRC_BF16 && pr.src != SRC_F16) || pr.batch != 1) return false;
+  // (a C input: contiguous rows, and not under the kernels' dequantisation stage - which a fused transform's two scale
+  // vectors on int32 sums are too: the C input joins the sums before them)
+  const bool dequant_stage = pr.dequant || (bytes && pr.fused != nullptr && pr.fused->row_scales != nullptr && pr.fused->column_scales != nullptr);
+  if (pr.has_cin && (pr.cin.cs != 1 || dequant_stage)) return false;
   const int64_t elem = bytes ? 1 : 2, ktile = 128 / elem;
   if (pr.k % ktile != 0 || pr.k < 2 * ktile || pr.n % 4 != 0 || pr.m == 0 || pr.n == 0) return false;
   if (pr.a.cs != 1 || (pr.a.rs * elem) % 16 != 0 || !aligned16(pr.a.data) || !aligned16(pr.b.data)) return false;
@@ -402,9 +406,8 @@ bool wide_tile_serves(const Problem& pr) {
   }
   if (pr.c.cs != 1 || pr.c.rs % 4 != 0 || !aligned16(pr.c.data)) return false;
   if (256 * pr.a.rs * elem >= (int64_t{1} << 31)) return false;
-  // (a dequantised product is described with its accumulator class, int32, and leaves as fp32)
-  if (bytes) return pr.out_kind == OUT_I32 || (pr.dequant && pr.out_kind == OUT_F32);
-  return !pr.dequant && (pr.out_kind == OUT_F32 || pr.out_kind == (pr.src == SRC_BF16 ? OUT_BF16 : OUT_F16));
+  // (every output type of the class: straight from the registers or through the epilogue's finishing step)
+  return bytes || !pr.dequant;
 }
 
 // How the operands of a (non-empty) problem can be fetched: the plan's vector flags and B's layout.
