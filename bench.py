@@ -326,6 +326,30 @@ def bench_int8_dequant(dev, steps, warmup, ceiling=None):
             "dtype": "int8", "roofline": roof}
 
 
+def bench_int8_square(dev, steps, warmup, ceiling=None):
+    """int8 4096^3 with the same fused dequantisation: the extents the headline metric names for both operand classes."""
+    import torch
+    from vecops_amd import capi, synth
+    n = 4096
+    a = torch.from_numpy(synth.int8_sym(1, (n, n))).to(dev)
+    b = torch.from_numpy(synth.int8_sym(2, (n, n))).to(dev)
+    rs = torch.from_numpy(synth.scales(3, n)).to(dev)
+    cs = torch.from_numpy(synth.scales(4, n)).to(dev)
+    c = torch.empty((n, n), dtype=torch.float32, device=dev)
+    ws = torch.empty(max(capi.lib().vecops_hip_matmul_i8_dequant_workspace(n, n, n), 1), dtype=torch.uint8, device=dev)
+    plan = capi.plan_matmul(a, b, torch.empty((n, n), dtype=torch.int32, device=dev))
+    t = _measure(lambda i: capi.matmul_i8_dequant(a, b, rs, cs, c, workspace=ws), steps, warmup)
+    ops = 2.0 * n ** 3
+    tops = ops / (t["event_ms"] * 1e-3) / 1e12
+    roof = _roofline("mfma", tops, PEAK_INT8_TOPS, "TOP/s", kernel=_kernel_label(plan, "int8") + ", dequantising epilogue",
+                     algorithmic_ops_per_launch=ops, algorithmic_bytes_per_launch=2 * n * n + 4 * n * n + 8 * n, traffic=None,
+                     **_timing_fields(t))
+    if ceiling:
+        roof.update(measured_ceiling=ceiling, frac_of_ceiling=tops / ceiling)
+    return {"metric": "int8_gemm_4096_tops", "workload": "int8 4096^3, per-token x per-channel dequant fused, fp32 out",
+            "value": tops, "unit": "TOP/s", "ms_per_step": t["wall_ms"], "dtype": "int8", "roofline": roof}
+
+
 def bench_runtime_quant(dev, steps, warmup):
     """fp32 activations quantised per row on the way in (vecops' RuntimePerRowAsymmetricQuantizeTransform), int8
     weights, correction row, per-token x per-channel dequantisation: three launches (quantise, weight row sums,
@@ -685,7 +709,7 @@ def cpu_baseline(a, b_kn):
     return out
 
 
-ONLY = ["bf16", "int8", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "read_ceiling",
+ONLY = ["bf16", "int8", "int8_square", "gemv", "copy", "bf16_packed", "int8_packed", "runtime_quant", "mfma_ceiling", "read_ceiling",
         "fp32", "batched", "bf16_mid", "families", "grouped", "rule_check", "vendor_grid"]
 
 
@@ -723,6 +747,7 @@ def main() -> int:
 
     single = {
         "int8": lambda: bench_int8_dequant(dev, K, W),
+        "int8_square": lambda: bench_int8_square(dev, K, W),
         "copy": lambda: bench_copy(dev, K, W),
         "bf16_packed": lambda: bench_bf16_gemm_packed(dev, K, W),
         "int8_packed": lambda: bench_int8_dequant_packed(dev, K, W),
@@ -763,6 +788,7 @@ def main() -> int:
         roofline["measured_ceiling_shape"] = ceiling_bf16["shape"]
         roofline["frac_of_ceiling"] = roofline["achieved"] / ceiling_bf16["value"]
         int8 = bench_int8_dequant(dev, K, W, ceiling=ceiling_int8["value"])
+        int8_square = bench_int8_square(dev, K, W, ceiling=ceiling_int8["value"])
         gemv = {m: bench_gemv(dev, K, W, m=m) for m in (1, 4, 16)}
         read_ceiling = bench_read_ceiling(dev, K, W)
         for r in gemv.values():   # what a kernel that only reads the weights sustains on the same buffers
@@ -776,14 +802,14 @@ def main() -> int:
                       bench_bf16_mid(dev, K, W, 2048, 11008, 4096, False)]
         secondary += [bench_runtime_quant(dev, K, W), bench_grouped(dev, K, W), ceiling_bf16, ceiling_int8, read_ceiling, packed16,
                       packed8,
-                      fp32["bf16"], fp32["f32"], gemv[16], gemv[4], gemv[1], int8]
+                      fp32["bf16"], fp32["f32"], gemv[16], gemv[4], gemv[1], int8_square, int8]
 
         def brief(r):
             return {"frac": round(r["roofline"]["frac"], 4), "event_us": round(r["roofline"]["event_ms"] * 1e3, 2),
                     "value": round(r["value"], 1), "unit": r["unit"]}
         # the other components of the headline metric and the remaining benchmark configurations, in short: the full
         # records are in `secondary`
-        roofline["also"] = {"int8_cfg4": brief(int8), "int8_cfg4_prepacked": brief(packed8), "gemv_m1": brief(gemv[1]),
+        roofline["also"] = {"int8_cfg4": brief(int8), "int8_4096": brief(int8_square), "int8_cfg4_prepacked": brief(packed8), "gemv_m1": brief(gemv[1]),
                             "gemv_m4": brief(gemv[4]), "gemv_m16": brief(gemv[16]), "fp32_1024_f32_compute": brief(fp32["f32"]),
                             "fp32_1024_bf16_compute": brief(fp32["bf16"]), "bf16_4096_prepacked": brief(packed16),
                             "hbm_read_ceiling_gbps": round(read_ceiling["value"], 1)}
