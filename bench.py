@@ -38,19 +38,22 @@ REPETITIONS = 7
 # HBM-side bytes per launch recorded with rocprofv3 (FETCH_SIZE and WRITE_SIZE in KiB per dispatch x 1024, FETCH
 # scaled by 2.000 and WRITE by 1.000: what the same counters read for a 1 GiB device copy, `--only copy`).  Counters
 # cannot be read from inside this process: these are the figures of the named summaries, for exactly these workloads.
-RECORDED_TRAFFIC = {
-    "bf16": (int((98503.0 * 2.000 + 32768 * 1.000) * 1024), "profiles/tile_gemm_bf16_4096.md"),
-    "int8": (int((55098.0 * 2.000 + 88095 * 1.000) * 1024), "profiles/tile_gemm_wide_i8_dequant_2048x4096x11008.md"),
-    "gemv_m1": (int((29647.0 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
-    "gemv_m4": (int((29761.0 * 2.000 + 112.0 * 1.000) * 1024), "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
-    "gemv_m16": (int((30145.0 * 2.000 + 448.0 * 1.000) * 1024), "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
-    "bf16_packed": (int((98490.0 * 2.000 + 32768 * 1.000) * 1024), "profiles/tile_gemm_packed16_bf16_4096.md"),
-    "bf16_mid_kn_1024x4096x4096": (int((49256.0 * 2.000 + 8192 * 1.000) * 1024), "profiles/tile_gemm_deep128_bf16_1024x4096x4096.md"),
-    "bf16_mid_nk_1024x4096x4096": (int((49245.0 * 2.000 + 8192 * 1.000) * 1024), "profiles/tile_gemm_deep128_bf16_1024x4096x4096.md"),
-    "int8_packed": (int((55095.0 * 2.000 + 88108 * 1.000) * 1024),
-                    "profiles/tile_gemm_wide_i8_dequant_2048x4096x11008.md"),
-    "fp32_f32": (int((12357.0 * 2.000 + 4096 * 1.000) * 1024), "profiles/tile_gemm_f32_compute_1024.md"),
+# (FETCH_SIZE KiB, WRITE_SIZE KiB, the summary that holds them)
+RECORDED_COUNTERS = {
+    "bf16": (98503, 32768, "profiles/tile_gemm_bf16_4096.md"),
+    "int8": (55098, 88095, "profiles/tile_gemm_wide_i8_dequant_2048x4096x11008.md"),
+    "gemv_m1": (29647, 112, "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
+    "gemv_m4": (29761, 112, "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
+    "gemv_m16": (30145, 448, "profiles/skinny_w8a16_m1_m4_m16_4096x14336.md"),
+    "bf16_packed": (98490, 32768, "profiles/tile_gemm_packed16_bf16_4096.md"),
+    "bf16_mid_kn_1024x4096x4096": (49256, 8192, "profiles/tile_gemm_deep128_bf16_1024x4096x4096.md"),
+    "bf16_mid_nk_1024x4096x4096": (49245, 8192, "profiles/tile_gemm_deep128_bf16_1024x4096x4096.md"),
+    "int8_packed": (55095, 88108, "profiles/tile_gemm_wide_i8_dequant_2048x4096x11008.md"),
+    "fp32_f32": (12357, 4096, "profiles/tile_gemm_f32_compute_1024.md"),
+    "bf16_mid_nk_2048x11008x4096": (109918, 48106, "profiles/tile_gemm_wide_16_bf16_2048x11008x4096.md"),
+    "int8_square": (49596, 65536, "profiles/tile_gemm_i8_dequant_4096.md"),
 }
+RECORDED_TRAFFIC = {key: (int((fetch * 2.000 + write * 1.000) * 1024), source) for key, (fetch, write, source) in RECORDED_COUNTERS.items()}
 
 
 def _traffic(key):
@@ -342,8 +345,8 @@ def bench_int8_square(dev, steps, warmup, ceiling=None):
     ops = 2.0 * n ** 3
     tops = ops / (t["event_ms"] * 1e-3) / 1e12
     roof = _roofline("mfma", tops, PEAK_INT8_TOPS, "TOP/s", kernel=_kernel_label(plan, "int8") + ", dequantising epilogue",
-                     algorithmic_ops_per_launch=ops, algorithmic_bytes_per_launch=2 * n * n + 4 * n * n + 8 * n, traffic=None,
-                     **_timing_fields(t))
+                     algorithmic_ops_per_launch=ops, algorithmic_bytes_per_launch=2 * n * n + 4 * n * n + 8 * n,
+                     **_traffic("int8_square"), **_timing_fields(t))
     if ceiling:
         roof.update(measured_ceiling=ceiling, frac_of_ceiling=tops / ceiling)
     return {"metric": "int8_gemm_4096_tops", "workload": "int8 4096^3, per-token x per-channel dequant fused, fp32 out",
