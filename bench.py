@@ -288,7 +288,8 @@ def bench_grouped(dev, steps, warmup):
     # synchronisations, because with thousands of launches queued the HIP runtime's own bookkeeping stalls the host
     # in the first such loop of a process, 160-200 us per step of wall time where the GPU needs 76)
     count = min(max(steps, 50), 100)
-    grouped = _measure(lambda i: capi.matmul_grouped(a_list, b_list, c_list, workspace=ws), count, max(warmup, count))
+    run = capi.PreparedGrouped(a_list, b_list, c_list, workspace=ws)    # a step is one call of the C ABI
+    grouped = _measure(lambda i: run(), count, max(warmup, count))
 
     def one_by_one(i):
         for a, b, c in zip(a_list, b_list, c_list):

@@ -302,3 +302,23 @@ def test_shared_a_row_batch_is_folded(device, oracle, batch, n, k, dtype):
         assert capi.FAMILY_NAMES[folded.family] == "skinny"          # one long GEMV instead of `batch` short ones
     else:
         assert folded.family == unfolded.family or unfolded.split_k >= 1
+
+
+def test_prepared_grouped_call_repeats_the_plain_one(device):
+    """capi.PreparedGrouped: descriptors and workspace built once, every call one foreign call; same bits as
+    matmul_grouped, call after call."""
+    import torch
+    from vecops_amd import capi
+    shapes = [(300, 200, 520), (64, 1000, 136), (1, 77, 64), (1000, 1300, 264)]
+    a_list = [dev_bf16(synth.bf16_round(synth.uniform_pm1(10 + i, (m, k))), device) for i, (m, n, k) in enumerate(shapes)]
+    b_list = [dev_bf16(synth.bf16_round(synth.uniform_pm1(40 + i, (n, k))), device) for i, (m, n, k) in enumerate(shapes)]
+    want = [torch.empty((m, n), dtype=torch.float32, device=device) for m, n, k in shapes]
+    capi.matmul_grouped(a_list, b_list, want)
+    got = [torch.full((m, n), float("nan"), dtype=torch.float32, device=device) for m, n, k in shapes]
+    run = capi.PreparedGrouped(a_list, b_list, got)
+    for _ in range(3):
+        for t in got:
+            t.fill_(float("nan"))
+        run()
+        torch.cuda.synchronize()
+        assert all(torch.equal(g, w) for g, w in zip(got, want))

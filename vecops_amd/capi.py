@@ -443,6 +443,37 @@ def matmul_grouped(a_list, b_list, c_list, c_in_list=None, compute: int = 0, wor
     return c_list
 
 
+class PreparedGrouped:
+    """``matmul_grouped`` on fixed operands with the descriptors and the workspace built once: a call is one foreign
+    call (the library plans the groups anew each time - they are a handful of integer comparisons a group).  The
+    tensors must stay alive and in place."""
+
+    def __init__(self, a_list, b_list, c_list, c_in_list=None, compute: int = 0, workspace=None, stream=None):
+        import torch
+        count = len(a_list)
+        if not (len(b_list) == count and len(c_list) == count and (c_in_list is None or len(c_in_list) == count)):
+            raise ValueError("matmul_grouped: lists differ in length")
+        Operands = Operand * max(count, 1)
+        self._oa, self._ob, self._oc = Operands(*map(operand, a_list)), Operands(*map(operand, b_list)), Operands(*map(operand, c_list))
+        self._oi = None
+        if c_in_list is not None:
+            self._oi = Operands(*[operand(t) if t is not None else Operand() for t in c_in_list])
+        need = lib().vecops_hip_matmul_grouped_workspace(count, self._oa, self._ob, self._oi, self._oc, compute)
+        if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+            workspace = torch.empty(need, dtype=torch.uint8, device=c_list[0].device)
+        self._keep = (a_list, b_list, c_list, c_in_list, workspace)
+        ws_ptr = workspace.data_ptr() if workspace is not None else None
+        ws_size = workspace.numel() * workspace.element_size() if workspace is not None else 0
+        self._args = (count, self._oa, self._ob, self._oi, self._oc, compute, ws_ptr, ws_size, _stream_handle(stream))
+        self._fn = lib().vecops_hip_matmul_grouped
+
+    def __call__(self):
+        rc = self._fn(*self._args)
+        if rc != 0:
+            _check(rc)
+        return self._keep[2]
+
+
 def matmul_runtime_quant_packed_b(a, multipliers, zero_point: int, packed, row_scales, column_scales, c, correction=None,
                                   workspace=None, stream=None):
     """``matmul_runtime_quant`` against weights packed once by ``pack_b`` (int8)."""
