@@ -52,6 +52,7 @@ RECORDED_COUNTERS = {
     "fp32_f32": (12357, 4096, "profiles/tile_gemm_f32_compute_1024.md"),
     "bf16_mid_nk_2048x11008x4096": (109918, 48106, "profiles/tile_gemm_wide_16_bf16_2048x11008x4096.md"),
     "int8_square": (49596, 65536, "profiles/tile_gemm_i8_dequant_4096.md"),
+    "batched_3000x3000x17": (4756, 282920, "profiles/tile_gemm_short_k_bf16_batched_8x3000x3000x17.md"),
 }
 RECORDED_TRAFFIC = {key: (int((fetch * 2.000 + write * 1.000) * 1024), source) for key, (fetch, write, source) in RECORDED_COUNTERS.items()}
 
@@ -261,8 +262,11 @@ def bench_batched(dev, steps, warmup, m, n, k):
     mfma_bound = flops / (PEAK_BF16_TFLOPS * 1e12) >= nbytes / (PEAK_HBM_GBPS * 1e9)
     roof = (_roofline("mfma", tflops, PEAK_BF16_TFLOPS, "TFLOP/s") if mfma_bound
             else _roofline("hbm", gbps, PEAK_HBM_GBPS, "GB/s"))
-    roof.update(kernel=_kernel_label(plan, "bf16"), algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=nbytes,
-                traffic=None, **_timing_fields(t))
+    label = _kernel_label(plan, "bf16")
+    if capi.FAMILY_NAMES[plan.family] == "tile_128" and 8 <= k <= 32:
+        label = "tile_gemm_short_k_kernel<bf16>"   # what run_problem launches for such a plan
+    roof.update(kernel=label, algorithmic_flops_per_launch=flops, algorithmic_bytes_per_launch=nbytes,
+                **_traffic(f"batched_{m}x{n}x{k}"), **_timing_fields(t))
     return {"metric": f"bf16_batched_{m}x{n}x{k}_tflops", "workload": f"batch 8 x bf16 ({m},{n},{k}), A[8,M,K] and "
             "B[8,N,K], uniform[-1,1), fp32 accumulate and output (BASELINE configs[2])", "value": tflops,
             "unit": "TFLOP/s", "hbm_gbps": gbps, "us_per_step": t["wall_ms"] * 1e3, "dtype": "bf16", "roofline": roof}

@@ -296,6 +296,11 @@ struct RuleConstants {
   //    `bench.py --only rule_check`: 512 / 768 / 1024 x 4096 x 4096, 1024 x 4096 x 11008, 512 x 2048 x 16384.
   int64_t deep_alone_from_tiles = 96, deep_fill_from_tiles = 32, deep_fill_k_tiles_per_part = 12;
   int64_t deep_idle_tiles = 160, deep_idle_k_tiles_per_part = 60, deep_k_tile_ns = 300, deep_fixed_ns = 8000;
+  // -- a 128x128 plan of 16-bit compute with K up to this (one matrix instruction deep) runs the kernel that loads its
+  //    fragments straight from memory and overlaps a tile's stores with the next tile's loads (tile_gemm_short_k.hip:
+  //    batch 8 of 3000 x 3000 x 17 to fp32 54 us against 69, to bf16 42 against 53; 8192 x 8192 x 32 43 against 57; with
+  //    a second step along K - its loads are not overlapped - the two-stage kernel is ahead, 65 against 71 us at K = 64)
+  int64_t short_k_direct_max_k = 32;
 };
 constexpr RuleConstants kRules{};
 
@@ -953,6 +958,10 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     if (!wide_tile_serves(pr) || !launch_tile_gemm_wide_serves(pr.src, p, mode, pr.packed_b))
       return fail(ST_INVALID, "matmul: the plan's family tile_256x352 cannot serve this call");
     e = launch_tile_gemm_wide(pr.src, p, pr.packed_b, stream);
+  } else if (!pr.packed_b && tile_m == 128 && tile_n == 128 && pr.k <= kRules.short_k_direct_max_k &&
+             launch_tile_gemm_short_k_serves(pr.src, p)) {
+    // a K tile or two: the kernel that is all stores
+    e = launch_tile_gemm_short_k(pr.src, p, stream);
   } else if (pr.packed_b && launch_tile_gemm_packed16_serves(pr.src, p, tile_m, tile_n)) {
     e = launch_tile_gemm_packed16(pr.src, p, stream);
   } else if (pr.packed_b && tile_m == 128 && tile_n == 128 && p.k_tiles_per_split >= kRules.deep_min_k_tiles &&

@@ -218,6 +218,10 @@ hipError_t launch_tile_gemm_deep128(int src, const TileGemmParams& p, int mode, 
 // per compute unit (tile_gemm_deep_f32.hip); b_as_kn: B handed over as [K,N].
 bool launch_tile_gemm_deep_f32_serves(const TileGemmParams& p, int tile, bool b_as_kn);
 hipError_t launch_tile_gemm_deep_f32(const TileGemmParams& p, int tile, bool b_as_kn, hipStream_t stream);
+// Very short K on 16-bit compute, operands K-contiguous: fragments loaded straight from memory, 64 x 128 of C a workgroup
+// (tile_gemm_short_k.hip).
+bool launch_tile_gemm_short_k_serves(int src, const TileGemmParams& p);
+hipError_t launch_tile_gemm_short_k(int src, TileGemmParams p, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_bf16(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_i8(const GroupedTables& t, int tile, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_grouped_i8_flip(const GroupedTables& t, int tile, int mode, hipStream_t stream);
