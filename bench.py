@@ -531,6 +531,9 @@ RULE_CHECK_SHAPES = [
     # where the 256 x 352 tile's count fits the units (16-bit operands, B [N,K])
     ("bf16", 2048, 11008, 4096), ("bf16", 4096, 11008, 4096), ("bf16", 6144, 6144, 6144), ("bf16", 4096, 4224, 4096),
     ("bf16", 1024, 11008, 4096), ("bf16", 3072, 4096, 4096),
+    # where 192 x 192 tiles fit one round (operands whose loads write LDS, B [N,K]) - and where they only nearly do
+    ("bf16", 3072, 3072, 4096), ("bf16", 1344, 6144, 4096), ("int8", 3000, 3000, 3008), ("int8", 768, 11008, 4096),
+    ("bf16", 2304, 2304, 8192), ("bf16", 1920, 3840, 4096), ("bf16", 2048, 4096, 11008),
 ]
 
 
@@ -541,7 +544,7 @@ def bench_rule_check(dev, steps, warmup):
     import numpy as np
     import torch
     from vecops_amd import capi, synth
-    families = ["tile_256", "tile_256x352", "tile_256x128", "tile_128x256", "tile_128", "tile_64"]
+    families = ["tile_256", "tile_256x352", "tile_192", "tile_256x128", "tile_128x256", "tile_128", "tile_64"]
     steps, warmup = max(10, steps // 10), max(10, warmup // 10)
     ws = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
     rows = []

@@ -103,9 +103,18 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
     rc, p = _plan(_operand(capi.BF16, (4096, 1024)), _operand(capi.BF16, (4096, 1024)), _operand(capi.BF16, (4096, 4096)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
-    # 3000^3: 144 big tiles in one part-filled round stay ahead of 576 small ones in three
+    # 3000^3: 256 tiles of 192 x 192 are one full round, where 144 big tiles leave 112 units idle (B as [K,N], which the
+    # 192 x 192 tile does not take: the big tiles, ahead of 576 small ones in three rounds); so are 232 for 768 x 11008
+    # and 224 for 1344 x 6144; two rounds of them (4096^3: 484) lose to the big tiles, and so does a prepacked B
     rc, p = _plan(_operand(capi.BF16, (3000, 3000)), _operand(capi.BF16, (3000, 3000)), _operand(capi.F32, (3000, 3000)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_192" and p.split_k == 1 and p.workspace_bytes == 0
+    b_kn = _operand(capi.BF16, (3000, 3000))
+    b_kn.strides[0], b_kn.strides[1] = 1, 3000
+    rc, p = _plan(_operand(capi.BF16, (3000, 3000)), b_kn, _operand(capi.F32, (3000, 3000)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
+    for m, n in ((768, 11008), (1344, 6144), (3072, 3072)):
+        rc, p = _plan(_operand(capi.BF16, (m, 4096)), _operand(capi.BF16, (n, 4096)), _operand(capi.BF16, (m, n)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_192", (m, n)
     # 4096 x 4224: 272 big tiles would leave the second round 6 % full; 192 tiles of 256x352 are one round, three
     # quarters full (1056 of 128x128, five per compute unit, where that tile cannot serve: B as [K,N])
     rc, p = _plan(_operand(capi.BF16, (4096, 4096)), _operand(capi.BF16, (4224, 4096)), _operand(capi.F32, (4096, 4224)))
@@ -270,7 +279,7 @@ def test_family_request_known_answers():
     rc, p = _plan_family(*skinny, "tile_64", capi.SELECT_REQUIRE)
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_64"
     # malformed requests
-    request = capi.family_request(9, capi.SELECT_REQUIRE)
+    request = capi.family_request(10, capi.SELECT_REQUIRE)
     plan = capi.Plan()
     assert capi.lib().vecops_hip_plan_matmul_family(C.byref(big[0]), C.byref(big[1]), None, C.byref(big[2]), 0,
                                                     C.byref(request), C.byref(plan)) == 1

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libvecops_hip.so")
 I8, U8, I32, F16, BF16, F32, F64 = 2, 3, 6, 10, 11, 12, 13
 COMPUTE_BF16, COMPUTE_F32 = 0, 1
 FAMILY_NAMES = {0: "none", 1: "tile_256", 2: "tile_128", 3: "tile_64", 4: "skinny", 5: "zero_k", 6: "tile_256x128",
-                7: "tile_128x256", 8: "tile_256x352"}
+                7: "tile_128x256", 8: "tile_256x352", 9: "tile_192"}
 STATUS_NAMES = {0: "Ok", 1: "InvalidArgument", 2: "NotApplicable", 3: "NotFound", 4: "AbiMismatch", 5: "LoadError",
                 6: "ExecutionError", 7: "InternalError"}
 

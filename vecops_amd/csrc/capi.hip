@@ -241,7 +241,7 @@ constexpr int kStreamGroupsPerUnit = 2;  // workgroups of 4 wavefronts per compu
 // rectangles on the 16x16 shapes; 133 / 130 before), int8 4096^3 58 / 75 / 77 / 70 (`bench.py --only families`,
 // `--only rule_check`).
 constexpr int64_t kQuality256x128 = 800, kQuality128 = 900, kQuality128Int8 = 970, kQuality128Staged = 850;
-constexpr int64_t kQuality256x128Direct = 780, kQuality128Direct = 830, kQuality128Int8Direct = 850;
+constexpr int64_t kQuality256x128Direct = 780, kQuality128Direct = 830, kQuality128Int8Direct = 850, kQuality192 = 850;
 
 // Every other number the rule table and the split rule compare against, in one place, each with the mechanism it
 // stands for and the command that measures it.  `bench.py --only rule_check` runs nineteen shapes on every tile family
@@ -327,6 +327,7 @@ void tile_of_family(uint32_t family, int* tile_m, int* tile_n) {
     case VECOPS_HIP_FAMILY_TILE_256X128: *tile_m = 256; *tile_n = 128; break;
     case VECOPS_HIP_FAMILY_TILE_128X256: *tile_m = 128; *tile_n = 256; break;
     case VECOPS_HIP_FAMILY_TILE_256X352: *tile_m = 256; *tile_n = 352; break;
+    case VECOPS_HIP_FAMILY_TILE_192: *tile_m = *tile_n = 192; break;
     case VECOPS_HIP_FAMILY_TILE_128: *tile_m = *tile_n = 128; break;
     case VECOPS_HIP_FAMILY_TILE_64: *tile_m = *tile_n = 64; break;
     default: *tile_m = *tile_n = 0; break;
@@ -422,6 +423,13 @@ void plan_fetch_flags(const Problem& pr, VecopsHipPlan* plan) {
   plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
 }
 
+// Whether the 192 x 192 tile can run a problem: bf16, f16 or signed 8-bit operands, both K-contiguous with 16-byte
+// aligned bases, rows and batches (its only instances are fed by loads that write LDS themselves), B not prepacked.
+bool tile_192_serves(const Problem& pr, const VecopsHipPlan& plan) {
+  if (pr.src != SRC_BF16 && pr.src != SRC_F16 && pr.src != SRC_I8) return false;
+  return !pr.packed_b && fetch_mode(pr, plan) == MODE_KVEC_DMA;
+}
+
 // The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure
 // integer function of (operand class, m, n, k); it picks the workgroup tile by
 // how many tiles the problem yields against the 256 compute units and splits K
@@ -476,11 +484,17 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   const Candidate candidates[] = {{VECOPS_HIP_FAMILY_TILE_256, 256, 256, 1000},
                                   {VECOPS_HIP_FAMILY_TILE_256X128, 256, 128, direct ? kQuality256x128Direct : kQuality256x128},
                                   {VECOPS_HIP_FAMILY_TILE_128X256, 128, 256, direct ? kQuality256x128Direct : kQuality256x128},
+                                  // (256 tiles of 192 x 192 cover 3072 x 3072: one round where 144 big tiles leave 112
+                                  //  units idle - bf16 3000^3 71 us against 81, 768 x 11008 x 4096 64 against 80)
+                                  {VECOPS_HIP_FAMILY_TILE_192, 192, 192, kQuality192},
                                   {VECOPS_HIP_FAMILY_TILE_128, 128, 128,
                                    !direct ? kQuality128Staged : bytes ? kQuality128Int8Direct : kQuality128Direct}};
   uint32_t family = VECOPS_HIP_FAMILY_TILE_64;
   int64_t tile_m = 64, tile_n = 64, best_cost = INT64_MAX;
+  const bool serves_192 = tile_192_serves(pr, *plan);
   for (const Candidate& c : candidates) {
+    // (the 192 x 192 tile: for counts that fit one round - over several rounds the big tiles' loops are ahead)
+    if (c.family == VECOPS_HIP_FAMILY_TILE_192 && (!serves_192 || tiles2(c.tm, c.tn) > kComputeUnits)) continue;
     if (pr.m <= c.tm / 2 || pr.n <= c.tn / 2) continue;  // a tile more than half empty in one direction
     const int64_t count = tiles2(c.tm, c.tn);
     if (count * kRules.min_busy_den < kComputeUnits * kRules.min_busy_num) continue;
@@ -663,8 +677,8 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
 
 const char* family_name(uint32_t family) {
   static const char* const names[] = {"none", "tile_256", "tile_128", "tile_64", "skinny", "zero_k", "tile_256x128", "tile_128x256",
-                                      "tile_256x352"};
-  return family < 9 ? names[family] : "unknown";
+                                      "tile_256x352", "tile_192"};
+  return family < 10 ? names[family] : "unknown";
 }
 
 // The first tier of vecops' owner selection (matmul/details/kernel/amx/Backend.h:2724-2757; matmul/Family.h:216-239):
@@ -677,7 +691,7 @@ int32_t apply_request(const Problem& pr, const VecopsHipFamilyRequest* request, 
   if (request->struct_size < sizeof(VecopsHipFamilyRequest)) return fail(ST_INVALID, "matmul: family request record too short");
   if (request->selection != VECOPS_HIP_SELECT_PREFER && request->selection != VECOPS_HIP_SELECT_REQUIRE)
     return fail(ST_INVALID, "matmul: unknown family selection %u", request->selection);
-  if (request->family > VECOPS_HIP_FAMILY_TILE_256X352) return fail(ST_INVALID, "matmul: unknown family %u", request->family);
+  if (request->family > VECOPS_HIP_FAMILY_TILE_192) return fail(ST_INVALID, "matmul: unknown family %u", request->family);
   const bool degenerate = plan->family == VECOPS_HIP_FAMILY_NONE || plan->family == VECOPS_HIP_FAMILY_ZERO_K;
   int tile_m = 0, tile_n = 0;
   tile_of_family(request->family, &tile_m, &tile_n);
@@ -690,8 +704,11 @@ int32_t apply_request(const Problem& pr, const VecopsHipFamilyRequest* request, 
     serves = request->family == plan->family ||
              (request->family == VECOPS_HIP_FAMILY_SKINNY && !degenerate && skinny_applies(pr) && !(pr.dequant && pr.m >= pr.n));
   } else {
-    // every tile family serves every product, but the 256 x 352 tile its own class of them, K unsplit
-    serves = request->family != VECOPS_HIP_FAMILY_TILE_256X352 || (wide_tile_serves(pr) && request->split_k <= 1);
+    // every tile family serves every product, but the 256 x 352 tile its own class of them, K unsplit,
+    // and the 192 x 192 tile operands whose loads write LDS themselves
+    serves = request->family == VECOPS_HIP_FAMILY_TILE_256X352 ? wide_tile_serves(pr) && request->split_k <= 1
+             : request->family == VECOPS_HIP_FAMILY_TILE_192   ? tile_192_serves(pr, *plan)
+                                                               : true;
   }
   if (!serves) {
     if (request->selection == VECOPS_HIP_SELECT_PREFER) return ST_OK;  // the rule table's choice stands
@@ -954,6 +971,8 @@ int32_t run_problem(const Problem& pr, const VecopsHipPlan& plan, const float* r
     int32_t rc = unsigned_side_terms(pr, &p, reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + partial_bytes), stream);
     if (rc != ST_OK) return rc;
   }
+  if (plan.family == VECOPS_HIP_FAMILY_TILE_192 && !tile_192_serves(pr, plan))
+    return fail(ST_INVALID, "matmul: the plan's family tile_192 cannot serve this call");
   if (plan.family == VECOPS_HIP_FAMILY_TILE_256X352) {
     if (!wide_tile_serves(pr) || !launch_tile_gemm_wide_serves(pr.src, p, mode, pr.packed_b))
       return fail(ST_INVALID, "matmul: the plan's family tile_256x352 cannot serve this call");

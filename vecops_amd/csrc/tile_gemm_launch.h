@@ -20,7 +20,7 @@ enum LoadMode : int {
   MODE_NVEC_B_DMA = 4  // MODE_NVEC_B likewise
 };
 
-// tile_m x tile_n: 256x256, 256x128, 128x256, 128x128 or 64x64 (the workgroup tile).  Returns the HIP
+// tile_m x tile_n: 256x256, 256x128, 128x256, 192x192, 128x128 or 64x64 (the workgroup tile).  Returns the HIP
 // error of the launch (hipSuccess when enqueued).
 hipError_t launch_tile_gemm_bf16(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
 hipError_t launch_tile_gemm_f16(const TileGemmParams& p, int tile_m, int tile_n, int mode, hipStream_t stream);
@@ -143,6 +143,14 @@ hipError_t launch_tile_class(const TileGemmParams& p, int tile_m, int tile_n, in
       }
     }
     return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
+  }
+  if (tile_m == 192 && tile_n == 192) {
+    // 96 x 96 a wavefront on the 16x16 shapes: only for operands whose loads write LDS themselves, both K-contiguous
+    // (what the rule table plans it for, and what a request for it is checked against)
+    if constexpr (SRC == SRC_BF16 || SRC == SRC_F16 || SRC == SRC_I8) {
+      if (mode == MODE_KVEC_DMA) return launch_tile_instance<SRC, 2, 2, 3, 3, LOAD_KDMA, LOAD_KDMA, true>(p, stream);
+    }
+    return hipErrorInvalidConfiguration;
   }
   if (tile_m == 256 && tile_n == 128) return launch_tile_mode<SRC, 2, 2, 4, 2>(p, mode, stream);
   if (tile_m == 128 && tile_n == 256) return launch_tile_mode<SRC, 2, 2, 2, 4>(p, mode, stream);
