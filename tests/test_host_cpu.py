@@ -115,7 +115,7 @@ def test_host_library_exports_every_declared_symbol(host):
 
 def test_every_artifact_loads_with_its_key(host):
     files = sorted(os.listdir(H.ARTIFACT_DIR))
-    assert len(files) == 94   # 40 + (6 required families x {bf16, i8} + 15 unsigned-weight, side-A and fp32-pack kinds) x {host, device}
+    assert len(files) == 102  # 40 + (8 required families x {bf16, i8} + 15 unsigned-weight, side-A and fp32-pack kinds) x {host, device}
     for f in files:
         name, key = host.load_artifact(os.path.join(H.ARTIFACT_DIR, f))
         assert key.startswith(name + ";") and key.endswith(";backend=hip-gfx950")
@@ -182,7 +182,8 @@ def test_family_specialization_is_part_of_the_key(host):
     of MatmulConfig, i.e. of the specialization); each family has artifacts of its own for bf16 and 8-bit operands."""
     op = host.operator("vecops::matmul")
     a, b, c = bf16((4, 8)), bf16((5, 8)), np.zeros((4, 5), np.float32)
-    names = {1: "tile_256", 2: "tile_128", 3: "tile_64", 4: "skinny", 6: "tile_256x128", 7: "tile_128x256"}
+    names = {1: "tile_256", 2: "tile_128", 3: "tile_64", 4: "skinny", 6: "tile_256x128", 7: "tile_128x256", 8: "tile_256x352",
+             9: "tile_192"}
     for code, name in names.items():
         assert op.resolve(H.Frame([a, b, None, c], outputs=(3,)), {"Family": code}) == \
             f"vecops::matmul;operands=bf16;compute=bf16;family={name};memory=host;backend=hip-gfx950"
@@ -191,7 +192,7 @@ def test_family_specialization_is_part_of_the_key(host):
         "vecops::matmul;operands=i8;compute=i32;family=tile_128;memory=host;backend=hip-gfx950"
     # 0 = automatic: the plain artifact
     assert "family" not in op.resolve(H.Frame([a, b, None, c], outputs=(3,)), {"Family": 0})
-    for bad in (5, 8, -1):                       # zero_k, unknown numbers: nothing a caller can require
+    for bad in (5, 10, -1):                      # zero_k, unknown numbers: nothing a caller can require
         with pytest.raises(H.HostError) as e:
             op.resolve(H.Frame([a, b, None, c], outputs=(3,)), {"Family": bad})
         assert e.value.code in (1, 2, 3)

@@ -95,7 +95,7 @@ def test_matmul_required_family(host, oracle, device):
     b = synth.bf16_round(synth.uniform_pm1(2, (n, k)))
     want = np.zeros((m, n), np.float32)
     oracle.matmul(a, b, want, acc_f64=True)
-    for family in (1, 2, 3, 6, 7):
+    for family in (1, 2, 3, 6, 7, 9):
         c = np.full((m, n), np.nan, np.float32)
         op.invoke(H.Frame([a, b, None, c], outputs=(3,)), {"Family": family})
         assert rel_err(c, want) <= fp32_tol(k), family
@@ -113,6 +113,9 @@ def test_matmul_required_family(host, oracle, device):
         op.invoke(H.Frame([a, b, None, c], outputs=(3,)), {"Family": 4})
     assert e.value.code == 2 and "skinny" in e.value.message
     assert (c == 7.0).all()
+    with pytest.raises(H.HostError) as e:        # nor the 256 x 352 tile a K of 1000 (no whole number of K tiles)
+        op.invoke(H.Frame([a, b, None, c], outputs=(3,)), {"Family": 8})
+    assert e.value.code == 2 and (c == 7.0).all()
     # ... and serves its own shapes
     m2, n2, k2 = 4, 1024, 512
     a2 = synth.bf16_round(synth.uniform_pm1(3, (m2, k2)))

@@ -298,6 +298,10 @@ constexpr const char* kOperatorName = "vecops::matmul";
 #define FAMILY_KEY ";family=tile_256x128"
 #elif VECOPS_ARTIFACT_FAMILY == 7
 #define FAMILY_KEY ";family=tile_128x256"
+#elif VECOPS_ARTIFACT_FAMILY == 8
+#define FAMILY_KEY ";family=tile_256x352"
+#elif VECOPS_ARTIFACT_FAMILY == 9
+#define FAMILY_KEY ";family=tile_192"
 #else
 #error "VECOPS_ARTIFACT_FAMILY names no kernel family a caller can require"
 #endif

@@ -227,6 +227,8 @@ rt::Result<std::string> required_family(const rt::KernelCall& call) {
     case 4: return std::string("skinny");
     case 6: return std::string("tile_256x128");
     case 7: return std::string("tile_128x256");
+    case 8: return std::string("tile_256x352");
+    case 9: return std::string("tile_192");
     default: return invalid("Family names no kernel family a caller can require");
   }
 }
