@@ -534,6 +534,7 @@ RULE_CHECK_SHAPES = [
     # where 192 x 192 tiles fit one round (operands whose loads write LDS, B [N,K]) - and where they only nearly do
     ("bf16", 3072, 3072, 4096), ("bf16", 1344, 6144, 4096), ("int8", 3000, 3000, 3008), ("int8", 768, 11008, 4096),
     ("bf16", 2304, 2304, 8192), ("bf16", 1920, 3840, 4096), ("bf16", 2048, 4096, 11008),
+    ("bf16_kn", 3000, 3000, 3000), ("bf16_kn", 768, 11008, 4096), ("bf16_kn", 1344, 6144, 4096),
 ]
 
 

@@ -74,9 +74,9 @@ typedef enum VecopsHipKernelFamily {
   VECOPS_HIP_FAMILY_TILE_256X352 = 8,  /* 256 (M) x 352 (N) workgroup tile of signed 8-bit, bf16 or f16 operands (aligned,
                                           K-contiguous, K in whole K tiles of 128 bytes): the tile
                                           that covers 2048 x 11008 in one round */
-  VECOPS_HIP_FAMILY_TILE_192 = 9       /* 192x192 workgroup tile of bf16, f16 or signed 8-bit operands (both K-contiguous,
-                                          16-byte aligned bases, rows and batches; B not prepacked): the tile that
-                                          covers 3072 x 3072 in one round */
+  VECOPS_HIP_FAMILY_TILE_192 = 9       /* 192x192 workgroup tile of bf16, f16 or signed 8-bit operands (16-byte aligned
+                                          bases, rows and batches; both K-contiguous, or 16-bit ones with B as [K,N];
+                                          B not prepacked): the tile that covers 3072 x 3072 in one round */
 } VecopsHipKernelFamily;
 
 typedef struct VecopsHipPlan {

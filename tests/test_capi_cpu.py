@@ -103,14 +103,16 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_128"
     rc, p = _plan(_operand(capi.BF16, (4096, 1024)), _operand(capi.BF16, (4096, 1024)), _operand(capi.BF16, (4096, 4096)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
-    # 3000^3: 256 tiles of 192 x 192 are one full round, where 144 big tiles leave 112 units idle (B as [K,N], which the
-    # 192 x 192 tile does not take: the big tiles, ahead of 576 small ones in three rounds); so are 232 for 768 x 11008
-    # and 224 for 1344 x 6144; two rounds of them (4096^3: 484) lose to the big tiles, and so does a prepacked B
+    # 3000^3: 256 tiles of 192 x 192 are one full round, where 144 big tiles leave 112 units idle (B as [N,K] or [K,N];
+    # with rows that are not 16-byte aligned, which the 192 x 192 tile does not take: the big tiles, ahead of 576 small
+    # ones in three rounds); so are 232 for 768 x 11008 and 224 for 1344 x 6144
     rc, p = _plan(_operand(capi.BF16, (3000, 3000)), _operand(capi.BF16, (3000, 3000)), _operand(capi.F32, (3000, 3000)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_192" and p.split_k == 1 and p.workspace_bytes == 0
     b_kn = _operand(capi.BF16, (3000, 3000))
     b_kn.strides[0], b_kn.strides[1] = 1, 3000
     rc, p = _plan(_operand(capi.BF16, (3000, 3000)), b_kn, _operand(capi.F32, (3000, 3000)))
+    assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_192"
+    rc, p = _plan(_operand(capi.BF16, (3000, 3000), strides=(3004, 1)), _operand(capi.BF16, (3000, 3000)), _operand(capi.F32, (3000, 3000)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
     for m, n in ((768, 11008), (1344, 6144), (3072, 3072)):
         rc, p = _plan(_operand(capi.BF16, (m, 4096)), _operand(capi.BF16, (n, 4096)), _operand(capi.BF16, (m, n)))

@@ -1,5 +1,6 @@
 """The 192 x 192 workgroup tile (family tile_192), through the C ABI: 96 x 96 a wavefront on the 16x16 matrix instructions,
-for bf16, f16 and signed 8-bit operands whose loads write LDS themselves (both K-contiguous, 16-byte aligned bases and rows).
+for bf16, f16 and signed 8-bit operands whose loads write LDS themselves (16-byte aligned bases and rows; both K-contiguous,
+or 16-bit ones with B handed over as [K,N]).
 The rule table plans it where its count fits one round that the other tiles' counts do not (3000^3: 256 tiles; 768 x 11008:
 232).  bf16 against the oracle, f16 against float64 sums, int8 bit-exact (int32 sums, dequantised fp32); ragged extents, a K
 that is no whole number of K tiles, K splits, batches, C inputs, narrow outputs; refusals where it cannot serve."""
@@ -32,6 +33,34 @@ def test_bf16_against_the_oracle(device, oracle, m, n, k, split):
     torch.cuda.synchronize()
     want = np.zeros((m, n), np.float32)
     oracle.matmul(a_bits, b_bits, want, acc_f64=True, c_bf16=False)
+    assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n,k,split", [(192, 192, 512, 1), (3000, 3000, 264, 1), (500, 392, 1024, 1), (97, 1000, 520, 1),
+                                         (770, 584, 2048, 3), (1, 200, 512, 1), (400, 104, 8, 1), (1000, 1000, 4096, 2),
+                                         (300, 8, 640, 1)])
+def test_b_as_k_by_n(device, oracle, kind, m, n, k, split):
+    """B stored [K,N] and handed over as the strided [N,K] view (N a multiple of eight): the tile lies [k][n] in LDS, 24
+    chunk slots a row, and the fragment reads transpose.  bf16 against the oracle, f16 against float64 sums."""
+    import torch
+    from vecops_amd import capi
+    request = _require(capi, split)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    if kind == "bf16":
+        a_bits, b_bits = synth.bf16_round(synth.uniform_pm1(1, (m, k))), synth.bf16_round(synth.uniform_pm1(2, (k, n)))
+        a, b = dev_bf16(a_bits, device), dev_bf16(b_bits, device)
+        assert capi.FAMILY_NAMES[capi.plan_matmul_family(a, b.t(), c, request).family] == "tile_192"
+        capi.matmul_family(a, b.t(), c, request)
+        torch.cuda.synchronize()
+        want = np.zeros((m, n), np.float32)
+        oracle.matmul(a_bits, np.ascontiguousarray(b_bits.T), want, acc_f64=True, c_bf16=False)
+    else:
+        ha, hb = synth.uniform_pm1(1, (m, k)).astype(np.float16), synth.uniform_pm1(2, (k, n)).astype(np.float16)
+        a, b = torch.from_numpy(ha).to(device), torch.from_numpy(hb).to(device)
+        capi.matmul_family(a, b.t(), c, request)
+        torch.cuda.synchronize()
+        want = (ha.astype(np.float64) @ hb.astype(np.float64)).astype(np.float32)
     assert rel_err(c.cpu().numpy(), want) <= fp32_tol(k)
 
 
@@ -86,7 +115,7 @@ def test_int8_dequantisation_on_the_tables_plan(device, oracle):
 
 
 def test_the_table_plans_one_round_of_them(device):
-    """3000^3 in bf16, B as [N,K]: 256 tiles of 192 x 192; with B as [K,N] (which this tile does not take) the big tiles."""
+    """3000^3 in bf16, B as [N,K] or as [K,N]: 256 tiles of 192 x 192."""
     import torch
     from vecops_amd import capi
     gen = torch.Generator(device="cpu").manual_seed(3)
@@ -95,7 +124,10 @@ def test_the_table_plans_one_round_of_them(device):
     c = torch.full((3000, 3000), float("nan"), dtype=torch.bfloat16, device=device)
     plan = capi.plan_matmul(a, b, c)
     assert capi.FAMILY_NAMES[plan.family] == "tile_192" and plan.split_k == 1 and plan.workspace_bytes == 0
-    assert capi.FAMILY_NAMES[capi.plan_matmul(a, b.t(), c).family] == "tile_256"
+    b_kn = b.t().contiguous()                    # the same matrix stored [K,N]
+    assert capi.FAMILY_NAMES[capi.plan_matmul(a, b_kn.t(), c).family] == "tile_192"
+    from_kn = torch.full((3000, 3000), float("nan"), dtype=torch.bfloat16, device=device)
+    capi.matmul(a, b_kn.t(), from_kn)
     capi.matmul(a, b, c)
     other = torch.full((3000, 3000), float("nan"), dtype=torch.bfloat16, device=device)
     capi.matmul_family(a, b, other, capi.family_request("tile_256", capi.SELECT_REQUIRE, split_k=1))
@@ -104,6 +136,7 @@ def test_the_table_plans_one_round_of_them(device):
     want = torch.matmul(a[rows].double(), b.double().t())
     assert rel_err(c[rows].double().cpu().numpy(), want.cpu().numpy()) <= fp32_tol(3000) + 2.0 ** -8 * 1.01
     assert torch.equal(c, other)      # the same matrix instruction over the same k in the same order
+    assert torch.equal(c, from_kn)
 
 
 def test_required_where_it_cannot_serve(device):
@@ -115,7 +148,8 @@ def test_required_where_it_cannot_serve(device):
         return torch.zeros(shape, dtype=dtype, device=device)
     cases = {
         "fp32 operands": (z((400, 512), torch.float32), z((400, 512), torch.float32), torch.float32),
-        "B as [K,N]": (z((400, 512), torch.bfloat16), z((512, 400), torch.bfloat16).t(), torch.float32),
+        "int8 with B as [K,N]": (z((400, 512), torch.int8), z((512, 400), torch.int8).t(), torch.int32),
+        "B as [K,N] with N no multiple of eight": (z((400, 512), torch.bfloat16), z((512, 404), torch.bfloat16).t(), torch.float32),
         "rows not 16-byte aligned": (z((400, 516), torch.bfloat16)[:, :515], z((400, 516), torch.bfloat16)[:, :515], torch.float32),
         "unsigned a": (z((400, 512), torch.uint8), z((400, 512), torch.int8), torch.int32),
     }

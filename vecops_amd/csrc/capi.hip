@@ -423,11 +423,14 @@ void plan_fetch_flags(const Problem& pr, VecopsHipPlan* plan) {
   plan->b_layout = pr.b.cs == 1 ? 0 : (pr.b.rs == 1 ? 1 : 2);
 }
 
-// Whether the 192 x 192 tile can run a problem: bf16, f16 or signed 8-bit operands, both K-contiguous with 16-byte
-// aligned bases, rows and batches (its only instances are fed by loads that write LDS themselves), B not prepacked.
+// Whether the 192 x 192 tile can run a problem: bf16, f16 or signed 8-bit operands with 16-byte aligned bases, rows
+// and batches (its only instances are fed by loads that write LDS themselves) - both K-contiguous, or 16-bit ones
+// with B handed over as [K,N] -, B not prepacked.
 bool tile_192_serves(const Problem& pr, const VecopsHipPlan& plan) {
   if (pr.src != SRC_BF16 && pr.src != SRC_F16 && pr.src != SRC_I8) return false;
-  return !pr.packed_b && fetch_mode(pr, plan) == MODE_KVEC_DMA;
+  if (pr.packed_b) return false;
+  const int mode = fetch_mode(pr, plan);
+  return mode == MODE_KVEC_DMA || (mode == MODE_NVEC_B_DMA && pr.src != SRC_I8);
 }
 
 // The GPU rule table.  Like vecops' runtime_*_profitable predicates it is a pure

@@ -1060,6 +1060,19 @@ struct Stager<SRC, LOAD_NTR, ROWS, THREADS> {
 
 // The partial last K tile of an operand stored [k][n] (bf16), bounds-checked, straight into the packed and
 // swizzled LDS tile of the LOAD_NTR_DMA stager: rows k >= K and columns n >= N read as zero.
+// Where chunk `chunk` (16 bytes, 8 columns) of k row `krow` lies in its row of a [k][n] tile filled by loads that
+// write LDS (rows packed, cols * 2 bytes apart): the four rows a transposing read touches must lie in different
+// 64-byte groups of the bank period.  A power-of-two count of chunk slots: bits 2-3 of the slot xored with the row's
+// low two bits (rows 512 bytes apart would all start in one bank).  192 columns (24 slots, rows 384 bytes apart): the
+// row's chunks rotated by four slots per row of the four.
+__device__ __forceinline__ int ntr_dma_slot(int cols, int krow, int chunk) {
+  if (cols == 192) {
+    const int slot = chunk + ((krow & 3) << 2);
+    return slot >= 24 ? slot - 24 : slot;
+  }
+  return chunk ^ ((krow & 3) << 2);
+}
+
 __device__ __noinline__ void stage_kn_checked(const void* base, int64_t ks, int first_n, int extent, int cols,
                                               int k0_tile, int k_end, char* lds_tile, int tid, int threads) {
   const int chunks_per_row = cols / 8;
@@ -1076,7 +1089,7 @@ __device__ __noinline__ void stage_kn_checked(const void* base, int64_t ks, int 
           w[e >> 1] |= static_cast<uint32_t>(static_cast<const uint16_t*>(base)[k * ks + n]) << ((e & 1) * 16);
       }
     }
-    *reinterpret_cast<u32x4*>(lds_tile + krow * (cols * 2) + ((chunk ^ ((krow & 3) << 2)) << 4)) = u32x4{w[0], w[1], w[2], w[3]};
+    *reinterpret_cast<u32x4*>(lds_tile + krow * (cols * 2) + (ntr_dma_slot(cols, krow, chunk) << 4)) = u32x4{w[0], w[1], w[2], w[3]};
   }
 }
 
@@ -1203,8 +1216,11 @@ struct Stager<SRC, LOAD_KDMA, ROWS, THREADS> {
 
 // LOAD_NTR_DMA: the [k][n] stager whose loads write LDS themselves.  The 64 k rows of a tile lie
 // ROWS * 2 bytes apart with no pad, so that the 64 chunks a wavefront's load instruction fills are
-// contiguous; the four rows a transposing read touches are kept in different bank groups by xoring
-// bits 2-3 of the chunk slot with the row's low two bits.  bf16 only; tiles of 128 or more columns.
+// contiguous; the four rows a transposing read touches are kept in different bank groups by ntr_dma_slot.
+// bf16 / f16 only; tiles of 128 or more columns.  Part i is chunks i * THREADS .. of the tile's 64 * ROWS / 8, in
+// LDS order: where a row's chunk count divides the thread count a thread keeps its slot and moves
+// THREADS / CHUNKS_PER_ROW k rows on per part (one offset register and a uniform step); else (192 columns: 24 chunks
+// a row) each part has its own row and slot.
 template <int SRC, int ROWS, int THREADS>
 struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
   using T = SrcTraits<SRC>;
@@ -1214,7 +1230,8 @@ struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
   static_assert(CHUNKS_PER_ROW >= 16, "the swizzle needs sixteen chunk slots per row");
   static constexpr int CHUNKS = 64 * CHUNKS_PER_ROW / THREADS;
   static_assert(CHUNKS >= 1 && 64 * CHUNKS_PER_ROW % THREADS == 0, "whole chunks per thread");
-  static_assert(THREADS % CHUNKS_PER_ROW == 0 && (THREADS / CHUNKS_PER_ROW) % 4 == 0, "a thread keeps its row's low bits");
+  static constexpr bool kRegular = THREADS % CHUNKS_PER_ROW == 0 && (THREADS / CHUNKS_PER_ROW) % 4 == 0;  // a thread keeps its row's low bits
+  static_assert(kRegular || ROWS == 192, "a row's chunks divide the threads, or the 192-column tile");
   static constexpr int K_ROWS_PER_PART = THREADS / CHUNKS_PER_ROW;
   static constexpr int kParts = CHUNKS;
   static constexpr int kStoreOps = 0;
@@ -1224,10 +1241,25 @@ struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
   struct Spare {};
   const char* base;
   const VECOPS_GLOBAL char* tile_base;
-  uint32_t chunk_bytes;
+  uint32_t chunk_bytes;                           // (regular) the part-0 chunk's byte offset from tile_base
+  uint32_t part_bytes[kRegular ? 1 : CHUNKS];     // (else) every part's
   int64_t ks;
   int first_row, extent, k_end, tid_, wave_;
 
+  // byte offset from tile_base of the chunk whose LDS place is number `place` of the tile's (k row, slot) places
+  __device__ __forceinline__ uint32_t offset_of_place(int place) const {
+    const int krow = place / CHUNKS_PER_ROW, slot = place % CHUNKS_PER_ROW;
+    int chunk;  // the chunk whose swizzled slot this is
+    if constexpr (ROWS == 192) {
+      chunk = slot - ((krow & 3) << 2);
+      chunk = chunk < 0 ? chunk + CHUNKS_PER_ROW : chunk;
+    } else {
+      chunk = slot ^ ((krow & 3) << 2);
+    }
+    // extent is a multiple of 8 on this path: a chunk past it is clamped onto the last one
+    const int n = min(first_row + chunk * 8, extent - 8) - first_row;
+    return static_cast<uint32_t>((static_cast<int64_t>(krow) * ks + n) * T::kSrcBytes);
+  }
   __device__ __forceinline__ void init(const void* base_, int64_t /*rs*/, int64_t ks_, int first_row_, int extent_,
                                        int k_end_, int tid, uint32_t /*flip*/) {
     base = static_cast<const char*>(base_);
@@ -1238,11 +1270,13 @@ struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
     tid_ = tid;
     wave_ = __builtin_amdgcn_readfirstlane(tid >> 6);
     tile_base = uniform_ptr((const VECOPS_GLOBAL char*)(base + static_cast<int64_t>(first_row) * T::kSrcBytes));
-    const int krow = tid / CHUNKS_PER_ROW, slot = tid % CHUNKS_PER_ROW;
-    const int chunk = slot ^ ((krow & 3) << 2);  // the chunk whose swizzled slot this lane fills
-    // extent is a multiple of 8 on this path: a chunk past it is clamped onto the last one
-    const int n = min(first_row + chunk * 8, extent - 8) - first_row;
-    chunk_bytes = static_cast<uint32_t>((static_cast<int64_t>(krow) * ks + n) * T::kSrcBytes);
+    chunk_bytes = offset_of_place(tid);
+    if constexpr (!kRegular) {
+#pragma unroll
+      for (int part = 0; part < CHUNKS; ++part) part_bytes[part] = offset_of_place(part * THREADS + tid);
+    } else {
+      part_bytes[0] = chunk_bytes;
+    }
   }
   __device__ __forceinline__ uint32_t part_offset(int part) const {
     return __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(part * K_ROWS_PER_PART * ks * T::kSrcBytes));
@@ -1251,8 +1285,12 @@ struct Stager<SRC, LOAD_NTR_DMA, ROWS, THREADS> {
   __device__ __forceinline__ void dma_part(int part, int kt, uint32_t lds_tile) const {
     u32x4 buf = tile_buffer_words(tile_base + static_cast<int64_t>(max(kt, 0)) * 64 * ks * T::kSrcBytes);
     buf[2] = kt < 0 ? 0u : buf[2];
-    load_16_bytes_into_lds(buf, lds_tile, __builtin_amdgcn_readfirstlane((part * THREADS + wave_ * 64) * 16), chunk_bytes,
-                           part_offset(part));
+    if constexpr (kRegular) {
+      load_16_bytes_into_lds(buf, lds_tile, __builtin_amdgcn_readfirstlane((part * THREADS + wave_ * 64) * 16), chunk_bytes,
+                             part_offset(part));
+    } else {
+      load_16_bytes_into_lds(buf, lds_tile, __builtin_amdgcn_readfirstlane((part * THREADS + wave_ * 64) * 16), part_bytes[part], 0u);
+    }
   }
   __device__ __forceinline__ void dma_full(int kt, char* lds_tile) const {
     const uint32_t address = lds_address_of(lds_tile);
@@ -1856,7 +1894,14 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
           int col_bytes = ((wn * FN + 2 * q) * 16 + (s16 & 3) * 4) * 2;
           // packed rows: the 64-byte group is swizzled with the row's low two bits, which are s / 4 for both reads
           // of every k-step
-          if constexpr (LOAD_B == LOAD_NTR_DMA) col_bytes ^= ((s16 >> 2) & 3) << 6;
+          if constexpr (LOAD_B == LOAD_NTR_DMA) {
+            if constexpr (BN == 192) {  // (ntr_dma_slot: the row's 64-byte groups rotated by one per row of the four)
+              const int turned = (col_bytes & ~63) + (((s16 >> 2) & 3) << 6);
+              col_bytes = (turned >= 384 ? turned - 384 : turned) | (col_bytes & 63);
+            } else {
+              col_bytes ^= ((s16 >> 2) & 3) << 6;
+            }
+          }
           base_b[st][q] = lds0 + st * STAGE_BYTES + BM * 128 + (frag_chunk * 8 + (s16 >> 2)) * PITCH_NTR + col_bytes;
         } else {
           base_b[st][q] = lds0 + st * STAGE_BYTES + BM * 128 + (row_b + frag_row) * 128 + (((slot_b ^ (2 * q)) & 7) << 4);
@@ -1872,6 +1917,7 @@ __device__ __forceinline__ void tile_gemm_workgroup(const TileGemmParams& p, int
         // the k half g / 2; lane s of the group addresses row s / 4, columns 4 * (s % 4) .. + 3
         const int s16 = lane & 15, g = lane >> 4;
         int col_bytes = ((wn * FN + j) * 32 + (g & 1) * 16 + (s16 & 3) * 4) * 2;
+        static_assert(!(LOAD_B == LOAD_NTR_DMA && BN == 192), "the 192-column [k][n] tile: the 16x16 shapes' reads only");
         if constexpr (LOAD_B == LOAD_NTR_DMA) col_bytes ^= ((s16 >> 2) & 3) << 6;
         off_b[j] = BM * 128 + ((g >> 1) * 8 + (s16 >> 2)) * PITCH_NTR + col_bytes;
       } else if constexpr (LOAD_B == LOAD_KN32) {

@@ -145,10 +145,13 @@ hipError_t launch_tile_class(const TileGemmParams& p, int tile_m, int tile_n, in
     return launch_tile_mode<SRC, 2, 2, 4, 4>(p, mode, stream);
   }
   if (tile_m == 192 && tile_n == 192) {
-    // 96 x 96 a wavefront on the 16x16 shapes: only for operands whose loads write LDS themselves, both K-contiguous
-    // (what the rule table plans it for, and what a request for it is checked against)
+    // 96 x 96 a wavefront on the 16x16 shapes: only for operands whose loads write LDS themselves (what the rule table
+    // plans it for, and what a request for it is checked against)
     if constexpr (SRC == SRC_BF16 || SRC == SRC_F16 || SRC == SRC_I8) {
       if (mode == MODE_KVEC_DMA) return launch_tile_instance<SRC, 2, 2, 3, 3, LOAD_KDMA, LOAD_KDMA, true>(p, stream);
+      if constexpr (SRC != SRC_I8) {
+        if (mode == MODE_NVEC_B_DMA) return launch_tile_instance<SRC, 2, 2, 3, 3, LOAD_KDMA, LOAD_NTR_DMA, true>(p, stream);
+      }
     }
     return hipErrorInvalidConfiguration;
   }
