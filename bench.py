@@ -535,6 +535,8 @@ RULE_CHECK_SHAPES = [
     ("bf16", 3072, 3072, 4096), ("bf16", 1344, 6144, 4096), ("int8", 3000, 3000, 3008), ("int8", 768, 11008, 4096),
     ("bf16", 2304, 2304, 8192), ("bf16", 1920, 3840, 4096), ("bf16", 2048, 4096, 11008),
     ("bf16_kn", 3000, 3000, 3000), ("bf16_kn", 768, 11008, 4096), ("bf16_kn", 1344, 6144, 4096),
+    # one round of bigger tiles by a K split
+    ("bf16", 1500, 3000, 8192), ("bf16", 2304, 2304, 16384), ("bf16", 2000, 2600, 6144),
 ]
 
 

@@ -114,6 +114,15 @@ def test_rule_table_known_answers():
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_192"
     rc, p = _plan(_operand(capi.BF16, (3000, 3000), strides=(3004, 1)), _operand(capi.BF16, (3000, 3000)), _operand(capi.F32, (3000, 3000)))
     assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_256"
+    # one round of bigger tiles by a K split, where the 128 x 128 pairs fill their round badly or are split already and
+    # K is long: 81 tiles of 256 x 256 in three parts, 64 / 128 of 192 x 192 in four / two; a shorter K, or parts that
+    # would leave a tenth of the units idle, keep the pairs
+    for (m, n, k), family, split in (((2304, 2304, 8192), "tile_256", 3), ((768, 3072, 12288), "tile_192", 4),
+                                     ((1500, 3000, 8192), "tile_192", 2), ((2304, 2304, 4096), "tile_128", 1),
+                                     ((2000, 2600, 6144), "tile_128", 1), ((2048, 4096, 11008), "tile_128", 1)):
+        rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
+        assert p.workspace_bytes == (split * m * n * 4 if split > 1 else 0)
     for m, n in ((768, 11008), (1344, 6144), (3072, 3072)):
         rc, p = _plan(_operand(capi.BF16, (m, 4096)), _operand(capi.BF16, (n, 4096)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_192", (m, n)
@@ -167,7 +176,7 @@ def test_rule_table_known_answers():
     # the split rule's costs favour it), K split to fill the units once below that; more than half but at most 160
     # tiles and sixty K tiles per part keep the two-stage kernel's split (two co-resident workgroups on every unit)
     for (m, n, k), family, split in (((640, 4096, 4096), "tile_128", 1), ((768, 4096, 4096), "tile_128", 1),
-                                     ((1024, 2048, 8192), "tile_128", 2), ((768, 3072, 12288), "tile_128", 3),
+                                     ((1024, 2048, 8192), "tile_128", 2), ((768, 3072, 12288), "tile_192", 4),
                                      ((512, 4096, 4096), "tile_128", 1), ((640, 4096, 2048), "tile_128", 1),
                                      ((896, 4096, 4096), "tile_128", 1), ((2048, 2048, 2048), "tile_128", 1),
                                      ((512, 2048, 16384), "tile_128", 4), ((384, 3072, 8192), "tile_128", 3),
@@ -182,7 +191,7 @@ def test_rule_table_known_answers():
     # 16-bit operands with B as [K,N] (strides (1, N)) are served too (the tile lies [k][n] in LDS) and plan alike
     for (m, n, k), family, split in (((768, 4096, 4096), "tile_128", 1), ((512, 4096, 4096), "tile_128", 1),
                                      ((1024, 4096, 11008), "tile_128", 1), ((1024, 4096, 6144), "tile_128", 1),
-                                     ((512, 2048, 16384), "tile_128", 4), ((768, 3072, 12288), "tile_128", 3)):
+                                     ((512, 2048, 16384), "tile_128", 4), ((768, 3072, 12288), "tile_192", 4)):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k), strides=(1, n)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
     # operands it does not serve keep the two-stage kernel's rules: a K that is not whole K tiles - K split so that two

@@ -871,7 +871,7 @@ def test_w8a16_rejects_bad_arguments(device):
     assert e.value.code == 1
 
 
-@pytest.mark.parametrize("kind,m,n,k,split", [("bf16", 640, 4096, 4096, 1), ("bf16", 768, 3072, 12288, 3), ("bf16", 1000, 2000, 8200, 4),
+@pytest.mark.parametrize("kind,m,n,k,split", [("bf16", 640, 4096, 4096, 1), ("bf16", 896, 2560, 12288, 3), ("bf16", 1000, 2000, 8200, 4),
                                               ("i8", 768, 3072, 12288, 1), ("i8", 700, 4000, 8192, 1), ("i8", 700, 4000, 8208, 2)])
 def test_mid_band_k_split(device, oracle, kind, m, n, k, split):
     """128 to 200 tiles of 128 x 128 with a long K: 128 x 128 tiles, whole on the four-stage kernel where it serves

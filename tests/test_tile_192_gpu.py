@@ -139,6 +139,28 @@ def test_the_table_plans_one_round_of_them(device):
     assert torch.equal(c, from_kn)
 
 
+@pytest.mark.parametrize("m,n,k,b_as_kn,family,split", [(2304, 2304, 8192, False, "tile_256", 3), (768, 3072, 12288, False, "tile_192", 4),
+                                                         (768, 3072, 12288, True, "tile_192", 4), (1500, 3000, 8192, False, "tile_192", 2)])
+def test_one_round_of_bigger_tiles_by_a_k_split(device, m, n, k, b_as_kn, family, split):
+    """Where 128 x 128 pairs fill their round badly and K is long, the table plans one round of 256 x 256 or 192 x 192 tiles
+    in two to four K parts (partial sums in the workspace, summed by the reduce kernel): sampled rows against float64."""
+    import torch
+    from vecops_amd import capi
+    gen = torch.Generator(device="cpu").manual_seed(m + n + k)
+    a = (torch.rand((m, k), generator=gen) * 2 - 1).bfloat16().to(device)
+    b = (torch.rand((k, n) if b_as_kn else (n, k), generator=gen) * 2 - 1).bfloat16().to(device)
+    bv = b.t() if b_as_kn else b
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    plan = capi.plan_matmul(a, bv, c)
+    assert capi.FAMILY_NAMES[plan.family] == family and plan.split_k == split and plan.workspace_bytes == split * m * n * 4
+    capi.matmul(a, bv, c)
+    torch.cuda.synchronize()
+    assert not torch.isnan(c).any()
+    rows = torch.arange(0, m, 41, device=device)
+    want = torch.matmul(a[rows].double(), bv.double().t())
+    assert rel_err(c[rows].double().cpu().numpy(), want.cpu().numpy()) <= fp32_tol(k)
+
+
 def test_required_where_it_cannot_serve(device):
     import torch
     from vecops_amd import capi

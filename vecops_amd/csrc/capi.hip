@@ -273,6 +273,10 @@ struct RuleConstants {
   int64_t band_k_tiles_per_part = 20, band_k_tiles_per_part_full = 40, band_full_from_tiles = 200, band_min_parts = 6;
   // -- the big tile in four parts where 64 of them would fill a quarter of the chip: K tiles a part must keep
   int64_t big_tile_parts = 4, big_tile_k_tiles_per_part = 40;
+  // -- one round of 256x256 or 192x192 tiles by a K split of two to four parts against 128x128 pairs (`bench.py --only
+  //    rule_check`: 2304 x 2304 x 8192, 768 x 3072 x 12288, 2048 x 4096 x 11008)
+  int64_t one_round_max_parts = 4, one_round_k_tiles_per_part = 40, one_round_ps_per_unit = 21600, one_round_split_ns = 3000;
+  int64_t one_round_ns_per_kb_num = 28, one_round_ns_per_kb_den = 100, one_round_margin_num = 104, one_round_margin_den = 100;
   // -- peeling the last columns of tiles: only with this many K tiles (the peeled product splits them), an overhang of
   //    at most 1 / peel_overhang_den of a round, and at most 1 / peel_columns_den of the tile columns cut off
   //    (1536 x 11008 x 4096: 141 -> 125 us)
@@ -648,6 +652,43 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
       static_cast<uint64_t>(kRules.big_tile_parts) * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
     family = VECOPS_HIP_FAMILY_TILE_256;
     band_split = static_cast<uint32_t>(kRules.big_tile_parts);
+  }
+  // One round of bigger tiles by a K split, against 128x128 pairs that fill their round badly or are split already
+  // (16-bit operands, a long K).  Both sides are priced in ns: a workgroup's area / quality per K tile at one_round_ps_per
+  // _unit (a 256x256 workgroup walks a K tile in 1.4 us), the single part-filled round's discount as above, and for a
+  // split one_round_split_ns plus one_round_ns_per_kb for every KiB of partial sums (2304 x 2304 x 8192: 81 tiles of
+  // 256x256 in three parts 80 us against 88-93 for 324 unsplit pairs; 768 x 3072 x 12288: 64 tiles of 192x192 in four
+  // parts 60 against 63-67 for 144 tiles in three).  The parts must fill nine tenths of the units and keep
+  // one_round_k_tiles_per_part K tiles, and the estimate has to be 4 % ahead (2048 x 4096 x 11008, where 128 big tiles in
+  // two parts measure 5 % ahead of 512 pairs, stays as it is: the estimate sees 2 %).
+  if (direct && !pr.packed_b && !deep_planned && pr.batch == 1 && (pr.src == SRC_BF16 || pr.src == SRC_F16) &&
+      family == VECOPS_HIP_FAMILY_TILE_128) {
+    const int64_t c_kb = pr.m * pr.n * 4 / 1024;
+    auto split_ns = [&](int64_t parts) { return parts > 1 ? kRules.one_round_split_ns + parts * c_kb * kRules.one_round_ns_per_kb_num / kRules.one_round_ns_per_kb_den : 0; };
+    auto walk_ns = [&](int64_t units) { return units * k_tiles * kRules.one_round_ps_per_unit / 1000000; };
+    const int64_t own_parts = band_split > 0 ? band_split : 1;
+    const int64_t own_slots = kRules.small_tile_workgroups_per_unit * kComputeUnits, own_wgs = tiles(128) * own_parts;
+    const int64_t own_rounds = (own_wgs + own_slots - 1) / own_slots;
+    int64_t own_units = own_rounds * kRules.small_tile_workgroups_per_unit * 128 * 128 * 1000 / kQuality128Direct / own_parts;
+    if (own_rounds == 1) own_units = own_units * (own_slots + own_wgs) / (2 * own_slots);
+    int64_t best_ns = (walk_ns(own_units) + split_ns(own_parts)) * kRules.one_round_margin_den / kRules.one_round_margin_num;
+    const struct { uint32_t family; int64_t tile, quality; bool serves; } bigger[] = {
+        {VECOPS_HIP_FAMILY_TILE_256, 256, 1000, true}, {VECOPS_HIP_FAMILY_TILE_192, 192, kQuality192, serves_192}};
+    for (const auto& c : bigger) {
+      if (!c.serves) continue;
+      const int64_t count = tiles(c.tile), parts = count > 0 ? kComputeUnits / count : 0;
+      if (parts < 2 || parts > kRules.one_round_max_parts || count * parts * 10 < kComputeUnits * 9 ||
+          k_tiles / parts < kRules.one_round_k_tiles_per_part || static_cast<uint64_t>(parts) * pr.m * pr.n * 4u > scratch_limit)
+        continue;
+      const int64_t units = c.tile * c.tile * 1000 / c.quality / parts * (kComputeUnits + count * parts) / (2 * kComputeUnits);
+      const int64_t ns = walk_ns(units) + split_ns(parts);
+      if (ns < best_ns) {
+        best_ns = ns;
+        family = c.family;
+        tile_m = tile_n = c.tile;
+        band_split = static_cast<uint32_t>(parts);
+      }
+    }
   }
   plan->family = family;
   finish_tile_plan(pr, plan, band_split);
