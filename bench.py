@@ -53,6 +53,7 @@ RECORDED_COUNTERS = {
     "bf16_mid_nk_2048x11008x4096": (109918, 48106, "profiles/tile_gemm_wide_16_bf16_2048x11008x4096.md"),
     "int8_square": (49596, 65536, "profiles/tile_gemm_i8_dequant_4096.md"),
     "batched_3000x3000x17": (4756, 282920, "profiles/tile_gemm_short_k_bf16_batched_8x3000x3000x17.md"),
+    "bf16_mid_kn_3000x3000x3000": (54935, 17770, "profiles/tile_gemm_192_bf16_3000x3000x3000.md"),
 }
 RECORDED_TRAFFIC = {key: (int((fetch * 2.000 + write * 1.000) * 1024), source) for key, (fetch, write, source) in RECORDED_COUNTERS.items()}
 
@@ -813,7 +814,7 @@ def main() -> int:
         secondary = [bench_batched(dev, K, W, m, n, k)
                      for (m, n, k) in [(777, 1000, 3001), (1, 4097, 129), (255, 63, 8191), (3000, 3000, 17)]]
         secondary += [bench_bf16_mid(dev, K, W, 1024, 4096, 4096, True), bench_bf16_mid(dev, K, W, 2048, 2048, 2048, False),
-                      bench_bf16_mid(dev, K, W, 2048, 11008, 4096, False)]
+                      bench_bf16_mid(dev, K, W, 2048, 11008, 4096, False), bench_bf16_mid(dev, K, W, 3000, 3000, 3000, True)]
         secondary += [bench_runtime_quant(dev, K, W), bench_grouped(dev, K, W), ceiling_bf16, ceiling_int8, read_ceiling, packed16,
                       packed8,
                       fp32["bf16"], fp32["f32"], gemv[16], gemv[4], gemv[1], int8_square, int8]
