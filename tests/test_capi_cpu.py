@@ -180,11 +180,14 @@ def test_rule_table_known_answers():
                                      ((512, 4096, 4096), "tile_128", 1), ((640, 4096, 2048), "tile_128", 1),
                                      ((896, 4096, 4096), "tile_128", 1), ((2048, 2048, 2048), "tile_128", 1),
                                      ((512, 2048, 16384), "tile_128", 4), ((384, 3072, 8192), "tile_128", 3),
-                                     ((512, 3072, 8192), "tile_128", 2), ((512, 3072, 4096), "tile_128", 1),
+                                     ((512, 3072, 8192), "tile_128", 2), ((512, 3072, 4096), "tile_128", 2),
                                      ((256, 4096, 4096), "tile_128", 4), ((512, 1024, 8192), "tile_128", 8),
                                      ((128, 8192, 8192), "tile_128", 4), ((384, 2048, 4096), "tile_128", 5),
                                      ((1024, 4096, 11008), "tile_128", 1), ((1024, 4096, 6144), "tile_128", 1),
-                                     ((1024, 4096, 4096), "tile_128", 1), ((896, 4096, 11008), "tile_128", 1)):
+                                     ((1024, 4096, 4096), "tile_128", 1), ((896, 4096, 11008), "tile_128", 1),
+                                     # (96 .. 128 tiles: whole up to 64 K tiles, in two parts from 80 on)
+                                     ((512, 4096, 5120), "tile_128", 2), ((512, 4096, 6144), "tile_128", 2),
+                                     ((512, 4096, 3072), "tile_128", 1)):
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
         assert p.workspace_bytes == (split * m * n * 4 if split > 1 else 0)

@@ -300,6 +300,7 @@ struct RuleConstants {
   //    `bench.py --only rule_check`: 512 / 768 / 1024 x 4096 x 4096, 1024 x 4096 x 11008, 512 x 2048 x 16384.
   int64_t deep_alone_from_tiles = 96, deep_fill_from_tiles = 32, deep_fill_k_tiles_per_part = 12;
   int64_t deep_idle_tiles = 160, deep_idle_k_tiles_per_part = 60, deep_k_tile_ns = 300, deep_fixed_ns = 8000;
+  int64_t deep_halves_ns_per_kb_num = 3, deep_halves_ns_per_kb_den = 10;
   // -- a 128x128 plan of 16-bit compute with K up to this (one matrix instruction deep) runs the kernel that loads its
   //    fragments straight from memory and overlaps a tile's stores with the next tile's loads (tile_gemm_short_k.hip:
   //    batch 8 of 3000 x 3000 x 17 to fp32 54 us against 69, to bf16 42 against 53; 8192 x 8192 x 32 43 against 57; with
@@ -624,8 +625,10 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
           2ull * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
         const int64_t kb = pr.batch * pr.m * pr.n * 4 / 1024;
         const int64_t whole_ns = k_tiles * kRules.deep_k_tile_ns + kRules.deep_fixed_ns;
+        // (the partial sums of two full-chip parts move at 0.3 ns a KiB - int8 512 x 4096 x 11008 33 us in halves against
+        //  37.5 whole, bf16 512 x 4096 x 4096 25.0 whole against 26.2 - where the few-workgroup rule's small launches pay 0.75)
         const int64_t halves_ns = (k_tiles + 1) / 2 * kRules.deep_k_tile_ns + kRules.deep_fixed_ns + kRules.split_fixed_ns +
-                                  2 * kb * kRules.split_ns_per_kb_num / kRules.split_ns_per_kb_den;
+                                  2 * kb * kRules.deep_halves_ns_per_kb_num / kRules.deep_halves_ns_per_kb_den;
         if (halves_ns < whole_ns) best_parts = 2;
       }
       family = VECOPS_HIP_FAMILY_TILE_128;
