@@ -1,9 +1,10 @@
 """Products one matrix instruction deep (8 <= K <= 32, 16-bit compute, both operands K-contiguous) on the kernel that loads
-its fragments straight from memory (tile_gemm_short_k.hip): what the library runs for a 128 x 128 plan of such a product.
-A partial last chunk of K is the row's last eight elements with the overlap zeroed, so K = 8 .. 32 one by one; rows padded
-to odd strides (no alignment is assumed); ragged M and N (N a multiple of four or eight takes the plain stores, others
-the general store); batches; C inputs, fused transforms and narrow outputs.  bf16 against the oracle, everything against
-float64 sums of the same operands, and against the two-stage kernel of the 256 x 256 tile."""
+its fragments straight from memory (tile_gemm_short_k.hip): what the library runs for a 128 x 128 plan of such a product
+whose results leave as they are - fp32, bf16 or f16 into a C with contiguous, aligned rows and N a multiple of four / eight,
+no C input, no fused transform; everything else about such shapes stays with the two-stage tile kernel, and is tested here
+beside it.  A partial last chunk of K is the row's last eight elements with the overlap zeroed, so K = 8 .. 32 one by one;
+rows padded to odd strides (no alignment of the operands is assumed); ragged M and N; batches; narrow outputs.  bf16 against
+the oracle, everything against float64 sums of the same operands, and against the 256 x 256 tile's kernel."""
 import numpy as np
 import pytest
 
@@ -64,8 +65,9 @@ def test_shapes_kinds_and_outputs(device, kind, batch, m, n, k, pad, narrow_out)
     assert rel_err(c.double().cpu().numpy(), want.cpu().numpy()) <= tol
 
 
-@pytest.mark.parametrize("n", [520, 522])          # plain stores with the C input aside / the general store
+@pytest.mark.parametrize("n", [520, 522])
 def test_c_input_fused_transform_and_strided_c(device, n):
+    """What the short-K kernel leaves to the two-stage kernel, on the same shapes."""
     import torch
     from vecops_amd import capi
     m, k = 333, 17
@@ -95,6 +97,33 @@ def test_c_input_fused_transform_and_strided_c(device, n):
     torch.cuda.synchronize()
     fused = torch.clamp(torch.matmul(a2.double(), b2.double().t()) * 0.5 + 0.25, min=0.0)
     assert rel_err(c16.double().cpu().numpy(), fused.cpu().numpy()) <= fp32_tol(k) + 2.0 ** -8 * 1.01
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("narrow_out", [False, True])
+@pytest.mark.parametrize("bias", [False, True])
+def test_c_input_of_cs_type(device, kind, narrow_out, bias):
+    """A C input of C's own element type with rows like C's - or one row for all (a bias: row stride 0) - is added by the
+    short-K kernel itself: batches, ragged M, K = 17."""
+    import torch
+    from vecops_amd import capi
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[kind]
+    batch, m, n, k = 2, 1000, 1032, 17
+    gen = torch.Generator(device="cpu").manual_seed(17 + narrow_out + 2 * bias)
+    a = (torch.rand((batch, m, k), generator=gen) * 2 - 1).to(dtype).to(device)
+    b = (torch.rand((batch, n, k), generator=gen) * 2 - 1).to(dtype).to(device)
+    out_dtype = torch.float32 if not narrow_out else (torch.bfloat16 if kind == "f32" else dtype)
+    if bias:
+        c_in = (torch.rand((batch, 1, n), generator=gen) * 2 - 1).to(out_dtype).to(device).expand(batch, m, n)
+    else:
+        c_in = (torch.rand((batch, m, n), generator=gen) * 2 - 1).to(out_dtype).to(device)
+    c = torch.full((batch, m, n), float("nan"), dtype=out_dtype, device=device)
+    capi.matmul_family(a, b, c, _request(capi), c_in=c_in)
+    torch.cuda.synchronize()
+    ar, br = (a.bfloat16(), b.bfloat16()) if kind == "f32" else (a, b)
+    want = torch.matmul(ar.double(), br.double().transpose(-1, -2)) + c_in.double()
+    tol = fp32_tol(k) + (2.0 ** (-11 if out_dtype == torch.float16 else -8) * 1.01 if narrow_out else 0.0)
+    assert rel_err(c.double().cpu().numpy(), want.cpu().numpy()) <= tol
 
 
 def test_the_table_plans_the_benchmark_shape_on_it(device):

@@ -16,7 +16,6 @@ namespace {
 constexpr int kWaveRows = 32, kWaveCols = 64;    // one wavefront's part of C
 constexpr int kTileRows = 64, kTileCols = 128;   // a workgroup: 2 x 2 wavefronts
 constexpr int kStageRows = 16;                   // rows of C a wavefront lays out in LDS at a time
-constexpr int kResidentWorkgroups = 256 * 4;      // four workgroups on each compute unit (128 registers a lane)
 constexpr int kPitch = kWaveCols + 4;            // 32-bit words per staged row: rows start 16 bytes apart in the bank period
 
 // Eight compute elements of a K-contiguous row of at least eight elements as one 16-byte chunk: elements k0 .. k0+7
@@ -76,17 +75,21 @@ struct ShortKFragments {
   }
 };
 
-// How a launch's results leave: as they are, 32 bits each, in 16-byte runs; narrowed to 16 bits, eight to a 16-byte run
-// (both: no C input, no fused transform, C's rows contiguous and every run inside C and aligned); or through the
-// general store.
-enum ShortKStore : int { STORE_PLAIN32 = 0, STORE_PLAIN_BF16 = 1, STORE_GENERAL = 2, STORE_PLAIN_F16 = 3 };
+// How a launch's results leave: as they are, 32 bits each, in 16-byte runs, or narrowed to 16 bits, eight to a 16-byte
+// run.  Both: no fused transform, C's rows contiguous and every run inside C and aligned, a C input (if any) laid out
+// like C and of its type - anything else is the two-stage tile kernel's.
+enum ShortKStore : int { STORE_PLAIN32 = 0, STORE_PLAIN_BF16 = 1, STORE_PLAIN_F16 = 2, STORE_NONE = -1 };
 
 // A workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...: the fragments of its next tile are on their way
 // while it lays out and stores the tile at hand (a tile's loads and its stores are each a memory round trip, and a
 // compute unit holds four workgroups: without the overlap a wavefront's life was 6 us for 8 KiB written).  The plain
 // stores go through a buffer descriptor and switch a lane off by an offset beyond its range: every tile issues the
 // same stores on every path, so the wait for the next tile's fragments can leave exactly them outstanding.
-template <int SRC, int STORE>
+// CIN: a C input of C's own element type with contiguous, aligned rows (or one row for all: row stride 0) is added to the
+// sums.  Its loads for the whole tile go out behind the next tile's fragment loads and are waited for before the first
+// store: a tile's loads are then one round trip, at the price of the stores of the tile before having to land first
+// (loads and stores complete in the order of their issue) - the other wavefronts of the unit cover that.
+template <int SRC, int STORE, bool CIN>
 __global__ __launch_bounds__(256) void tile_gemm_short_k_kernel(const TileGemmParams p) {
   __shared__ uint32_t staged[4][kStageRows * kPitch];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -98,14 +101,15 @@ __global__ __launch_bounds__(256) void tile_gemm_short_k_kernel(const TileGemmPa
   ShortKFragments<SRC> frags;
   frags.load(p, at, lane, 0);
   uint32_t* mine = staged[wave];
-  const bool quads = STORE == STORE_GENERAL && c_takes_quads(p);
   constexpr bool kNarrow = STORE == STORE_PLAIN_BF16 || STORE == STORE_PLAIN_F16;
   constexpr int kOutBytes = kNarrow ? 2 : 4;
   constexpr int kRun = 16 / kOutBytes;                        // elements of C a lane stores at once (plain paths)
   constexpr int kLanesPerRow = kWaveCols / kRun, kRowsPerStep = 64 / kLanesPerRow;
   const int my_row = lane / kLanesPerRow, my_col = (lane % kLanesPerRow) * kRun;
   const uint32_t row_bytes = static_cast<uint32_t>(p.c_rs) * kOutBytes;
-  if constexpr (STORE != STORE_GENERAL) {
+  const uint32_t cin_row_bytes = static_cast<uint32_t>(p.cin_rs) * kOutBytes;
+  constexpr int kSteps = kStageRows / kRowsPerStep;           // store instructions a block of sixteen rows takes
+  {
     // As many stores as a tile issues, every lane switched off: the first pass of the loop then meets what every
     // later one does - its fragments' loads with one tile's stores behind them - and the wait the compiler places
     // at the loop's head is for the loads alone on every pass.
@@ -131,6 +135,21 @@ __global__ __launch_bounds__(256) void tile_gemm_short_k_kernel(const TileGemmPa
     const bool more = tile < total;
     at = short_k_place(p, min(tile, total - 1), wave);   // (past the last tile: that tile's fragments again, unused)
     frags.load(p, at, lane, 0);
+    u32x4 cin[2][kSteps];
+    if constexpr (CIN) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int row0 = m0 + i * kStageRows;
+        const __amdgpu_buffer_rsrc_t in = tile_buffer(
+            (const VECOPS_GLOBAL char*)p.cin + (batch * p.cin_bs + static_cast<int64_t>(row0) * p.cin_rs + n0) * kOutBytes);
+#pragma unroll
+        for (int step = 0; step < kSteps; ++step) {
+          const int r = step * kRowsPerStep + my_row;
+          const uint32_t offset = (n0 + my_col < p.n && row0 + r < p.m) ? static_cast<uint32_t>(r) * cin_row_bytes + my_col * kOutBytes : 0x80000000u;
+          cin[i][step] = __builtin_amdgcn_raw_buffer_load_b128(in, offset, 0, 0);   // (a lane switched off reads zeros)
+        }
+      }
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int row0 = m0 + i * kStageRows;
@@ -139,72 +158,113 @@ __global__ __launch_bounds__(256) void tile_gemm_short_k_kernel(const TileGemmPa
       for (int j = 0; j < 4; ++j)
         *reinterpret_cast<u32x4*>(mine + frag_row * kPitch + j * 16 + group * 4) = __builtin_bit_cast(u32x4, acc[i][j]);
       __builtin_amdgcn_wave_barrier();
-      if constexpr (STORE != STORE_GENERAL) {
-        // descriptor at C[batch][row0][n0]: a lane's offset is its row and column inside the block
-        const __amdgpu_buffer_rsrc_t out = tile_buffer(
-            (const VECOPS_GLOBAL char*)p.c + (batch * p.c_bs + static_cast<int64_t>(row0) * p.c_rs + n0) * kOutBytes);
-        const bool col_ok = n0 + my_col < p.n;    // N is a multiple of the run: a run lies inside C or outside
+      // descriptor at C[batch][row0][n0]: a lane's offset is its row and column inside the block
+      const __amdgpu_buffer_rsrc_t out = tile_buffer(
+          (const VECOPS_GLOBAL char*)p.c + (batch * p.c_bs + static_cast<int64_t>(row0) * p.c_rs + n0) * kOutBytes);
+      const bool col_ok = n0 + my_col < p.n;    // N is a multiple of the run: a run lies inside C or outside
 #pragma unroll
-        for (int step = 0; step < kStageRows / kRowsPerStep; ++step) {
-          const int r = step * kRowsPerStep + my_row;
-          u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * kPitch + my_col);
-          if constexpr (kNarrow) {
-            const u32x4 hi = *reinterpret_cast<const u32x4*>(mine + r * kPitch + my_col + 4);
-            uint32_t h[8];
+      for (int step = 0; step < kSteps; ++step) {
+        const int r = step * kRowsPerStep + my_row;
+        u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * kPitch + my_col);
+        if constexpr (kNarrow) {
+          constexpr int kKind = STORE == STORE_PLAIN_BF16 ? OUT_BF16 : OUT_F16;
+          const u32x4 hi = *reinterpret_cast<const u32x4*>(mine + r * kPitch + my_col + 4);
+          float f[8];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              h[e] = float_output_bits(STORE == STORE_PLAIN_BF16 ? OUT_BF16 : OUT_F16, __uint_as_float(v[e]));
-              h[4 + e] = float_output_bits(STORE == STORE_PLAIN_BF16 ? OUT_BF16 : OUT_F16, __uint_as_float(hi[e]));
-            }
-            v = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+          for (int e = 0; e < 4; ++e) {
+            f[e] = __uint_as_float(v[e]);
+            f[4 + e] = __uint_as_float(hi[e]);
           }
-          const uint32_t offset = (col_ok && row0 + r < p.m) ? static_cast<uint32_t>(r) * row_bytes + my_col * kOutBytes : 0x80000000u;
-          __builtin_amdgcn_raw_buffer_store_b128(v, out, offset, 0, 0);
-        }
-      } else {
+          if constexpr (CIN) {   // acc + float(cin), then the one rounding to C's type
 #pragma unroll
-        for (int step = 0; step < 4; ++step) {
-          const int r = step * 4 + group;
-          const u32x4 v = *reinterpret_cast<const u32x4*>(mine + r * kPitch + frag_row * 4);
-          store_quad_general<false>(p, batch, 0, row0 + r, n0 + frag_row * 4, v, quads, false);   // (checks the bounds itself)
+            for (int e = 0; e < 8; ++e) {
+              const uint32_t bits = (cin[i][step][e >> 1] >> ((e & 1) * 16)) & 0xffffu;
+              f[e] += kKind == OUT_BF16 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits);
+            }
+          }
+          uint32_t h[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[e] = float_output_bits(kKind, f[e]);
+          v = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+        } else if constexpr (CIN) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = __float_as_uint(__uint_as_float(v[e]) + __uint_as_float(cin[i][step][e]));
         }
+        const uint32_t offset = (col_ok && row0 + r < p.m) ? static_cast<uint32_t>(r) * row_bytes + my_col * kOutBytes : 0x80000000u;
+        __builtin_amdgcn_raw_buffer_store_b128(v, out, offset, 0, 0);
       }
     }
     if (!more) break;
   }
 }
 
+// Launches one instance on as many workgroups as the device holds at once (every workgroup then starts at time zero
+// and walks its share of the tiles: the instances use 104 to 164 registers a lane, three or four workgroups a unit).
+template <auto KERNEL>
+hipError_t launch_resident(const TileGemmParams& p, int64_t tiles, hipStream_t stream) {
+  static thread_local int resident = 0, resident_device = -1;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  if (resident_device != device) {
+    int per_unit = 0, units = 0;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_unit, KERNEL, 256, 0);
+    if (e != hipSuccess) return e;
+    e = hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device);
+    if (e != hipSuccess) return e;
+    resident = (per_unit > 0 ? per_unit : 1) * (units > 0 ? units : 1);
+    resident_device = device;
+  }
+  const dim3 grid(static_cast<unsigned>(tiles < resident ? tiles : resident)), block(256);
+  hipLaunchKernelGGL(KERNEL, grid, block, 0, stream, p);
+  return hipGetLastError();
+}
+
+// Which of the store forms a launch's C takes (STORE_NONE: none of them).
+int store_kind(const TileGemmParams& p) {
+  if (p.fused != 0) return STORE_NONE;
+  const int out_bytes = (p.out_kind == OUT_BF16 || p.out_kind == OUT_F16) ? 2 : (p.out_kind == OUT_F32) ? 4 : 0;
+  if (out_bytes == 0) return STORE_NONE;
+  // every run of 16 bytes lies inside C or outside and starts on a 16-byte boundary; the offsets inside a block of
+  // sixteen rows fit the descriptor's range
+  const int64_t run = 16 / out_bytes;
+  if (p.c_cs != 1 || p.n % run != 0 || p.c_rs % run != 0 || p.c_bs % run != 0 || (reinterpret_cast<uintptr_t>(p.c) & 15u) != 0 ||
+      p.c_rs <= 0 || (kStageRows * p.c_rs + kWaveCols) * out_bytes >= (int64_t{1} << 31))
+    return STORE_NONE;
+  // a C input: C's own element type, rows as C's (a row stride of 0 is one row for all)
+  if (p.cin != nullptr && (p.cin_kind != p.out_kind || p.cin_cs != 1 || p.cin_rs < 0 || p.cin_rs % run != 0 || p.cin_bs % run != 0 ||
+                           (reinterpret_cast<uintptr_t>(p.cin) & 15u) != 0 ||
+                           (kStageRows * p.cin_rs + kWaveCols) * out_bytes >= (int64_t{1} << 31)))
+    return STORE_NONE;
+  return p.out_kind == OUT_F32 ? STORE_PLAIN32 : p.out_kind == OUT_BF16 ? STORE_PLAIN_BF16 : STORE_PLAIN_F16;
+}
+
 template <int SRC>
 hipError_t launch(const TileGemmParams& p, hipStream_t stream) {
   const int64_t tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.batch;
   if (tiles <= 0 || tiles > INT32_MAX) return hipErrorInvalidConfiguration;
-  const dim3 grid(static_cast<unsigned>(tiles < kResidentWorkgroups ? tiles : kResidentWorkgroups)), block(256);
-  const int out_bytes = (p.out_kind == OUT_BF16 || p.out_kind == OUT_F16) ? 2 : (p.out_kind == OUT_U8 || p.out_kind == OUT_I8) ? 1 : 4;
-  // every run of `run` elements (16 bytes) lies inside C or outside and starts on a 16-byte boundary; the offsets
-  // inside a block of sixteen rows fit the descriptor's range
-  auto runs = [&](int64_t run) {
-    return p.c_cs == 1 && p.n % run == 0 && p.c_rs % run == 0 && p.c_bs % run == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15u) == 0 &&
-           p.c_rs > 0 && (kStageRows * p.c_rs + kWaveCols) * out_bytes < (int64_t{1} << 31);
+  auto go = [&](auto store_tag) {
+    constexpr int STORE = decltype(store_tag)::value;
+    return p.cin != nullptr ? launch_resident<tile_gemm_short_k_kernel<SRC, STORE, true>>(p, tiles, stream)
+                            : launch_resident<tile_gemm_short_k_kernel<SRC, STORE, false>>(p, tiles, stream);
   };
-  const bool plain = p.cin == nullptr && p.fused == 0;
-  if (plain && out_bytes == 4 && runs(4))
-    hipLaunchKernelGGL((tile_gemm_short_k_kernel<SRC, STORE_PLAIN32>), grid, block, 0, stream, p);
-  else if (plain && p.out_kind == OUT_BF16 && runs(8))
-    hipLaunchKernelGGL((tile_gemm_short_k_kernel<SRC, STORE_PLAIN_BF16>), grid, block, 0, stream, p);
-  else if (plain && p.out_kind == OUT_F16 && runs(8))
-    hipLaunchKernelGGL((tile_gemm_short_k_kernel<SRC, STORE_PLAIN_F16>), grid, block, 0, stream, p);
-  else
-    hipLaunchKernelGGL((tile_gemm_short_k_kernel<SRC, STORE_GENERAL>), grid, block, 0, stream, p);
-  return hipGetLastError();
+  switch (store_kind(p)) {
+    case STORE_PLAIN32: return go(std::integral_constant<int, STORE_PLAIN32>{});
+    case STORE_PLAIN_BF16: return go(std::integral_constant<int, STORE_PLAIN_BF16>{});
+    case STORE_PLAIN_F16: return go(std::integral_constant<int, STORE_PLAIN_F16>{});
+    default: return hipErrorInvalidConfiguration;
+  }
 }
 
 }  // namespace
 
 // What the kernel takes: 16-bit compute (bf16, f16, fp32 operands multiplied as bf16), both operands K-contiguous with at
-// least eight elements a row, no K split; any extents, row strides and alignment, any C input, output kind and fused transform.
+// least eight elements a row (any extents, row strides and alignment), no K split; fp32, bf16 or f16 results into a C
+// with contiguous, 16-byte aligned rows and N a multiple of four (fp32) or eight, no fused transform; a C input of C's
+// type with rows like C's (or one row for all).
 bool launch_tile_gemm_short_k_serves(int src, const TileGemmParams& p) {
   if (src != SRC_BF16 && src != SRC_F16 && src != SRC_F32_AS_BF16) return false;
-  return p.m > 0 && p.n > 0 && p.k >= 8 && p.split_k == 1 && p.a_ks == 1 && p.b_ks == 1;
+  return p.m > 0 && p.n > 0 && p.k >= 8 && p.split_k == 1 && p.a_ks == 1 && p.b_ks == 1 && store_kind(p) != STORE_NONE;
 }
 
 // (sets the tile counts of its own 64 x 128 tile in its copy of the parameters)
