@@ -96,15 +96,17 @@ __global__ __launch_bounds__(256, 1) void tile_gemm_deep128_kernel(const TileGem
   auto fill = [&](int t) {
     u32x4 da = desc_a, db = desc_b;
     if (t >= nk) da[2] = db[2] = 0u;
-    const uint32_t k_bytes = static_cast<uint32_t>(kt_begin + t) * 128u;
+    // (wavefront-uniform by construction; said so, or the compiler may carry them in vector registers, which the
+    //  load's scalar offset does not take)
+    const uint32_t k_tile = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(kt_begin + t));
+    const uint32_t k_bytes = k_tile * 128u;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       load_16_bytes_into_lds(da, m0_wave, static_cast<uint32_t>(t * kDeepStage + i * 4096), rows_a[i], k_bytes);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       load_16_bytes_into_lds(db, m0_wave, static_cast<uint32_t>(t * kDeepStage + 16384 + i * 4096), rows_b[TR ? 0 : i],
-                             TR ? static_cast<uint32_t>(kt_begin + t) * step_b + static_cast<uint32_t>(i) * part_b
-                                : PK ? static_cast<uint32_t>(kt_begin + t) * step_b : k_bytes);
+                             TR ? k_tile * step_b + static_cast<uint32_t>(i) * part_b : PK ? k_tile * step_b : k_bytes);
   };
   fill(0);
   fill(1);
