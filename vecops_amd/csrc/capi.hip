@@ -663,7 +663,8 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // 256x256 in three parts 80 us against 88-93 for 324 unsplit pairs; 768 x 3072 x 12288: 64 tiles of 192x192 in four
   // parts 60 against 63-67 for 144 tiles in three).  The parts must fill nine tenths of the units and keep
   // one_round_k_tiles_per_part K tiles, and the estimate has to be 4 % ahead (2048 x 4096 x 11008, where 128 big tiles in
-  // two parts measure 5 % ahead of 512 pairs, stays as it is: the estimate sees 2 %).
+  // two parts measure 4 % ahead of 512 pairs, stays as it is: the estimate sees 2 %, and sees the same for 1024 x 8192 x 11008,
+  // where the big tiles in two parts are 7 % behind).
   if (direct && !pr.packed_b && !deep_planned && pr.batch == 1 && (pr.src == SRC_BF16 || pr.src == SRC_F16) &&
       family == VECOPS_HIP_FAMILY_TILE_128) {
     const int64_t c_kb = pr.m * pr.n * 4 / 1024;
