@@ -126,6 +126,51 @@ def test_c_input_of_cs_type(device, kind, narrow_out, bias):
     assert rel_err(c.double().cpu().numpy(), want.cpu().numpy()) <= tol
 
 
+def _random_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        out.append(dict(kind=str(rng.choice(["bf16", "f16", "f32"])), batch=int(rng.choice([1, 1, 2, 5])),
+                        m=int(rng.integers(1, 1400)), n=int(rng.choice([4, 8, 12, 100, 128, 132, 1000, 1016, 1028, 2052, 3000, 777])),
+                        k=int(rng.integers(8, 33)), pad_a=int(rng.choice([0, 1, 8])), pad_b=int(rng.choice([0, 3, 8])),
+                        c_pad=int(rng.choice([0, 0, 8, 5])), narrow=bool(rng.random() < 0.5), c_in=str(rng.choice(["none", "same", "bias", "f32"]))))
+    return out
+
+
+@pytest.mark.parametrize("case", _random_cases(40, 2024), ids=lambda c: "{kind}-{batch}x{m}x{n}x{k}-{c_in}-{out}-pad{pad_a}.{pad_b}.{c_pad}".format(
+    out="narrow" if c["narrow"] else "f32", **c))
+def test_random_short_products(device, case):
+    """Seeded random shapes through the table's own plan (whichever kernel that is): ragged extents, padded operand rows, a
+    C whose rows are padded (aligned or not), C inputs of C's type, as a bias row, or of another type."""
+    import torch
+    from vecops_amd import capi
+    kind, batch, m, n, k = case["kind"], case["batch"], case["m"], case["n"], case["k"]
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[kind]
+    gen = torch.Generator(device="cpu").manual_seed(m * 7919 + n * 31 + k)
+    a = (torch.rand((batch, m, k + case["pad_a"]), generator=gen) * 2 - 1).to(dtype).to(device)[:, :, :k]
+    b = (torch.rand((batch, n, k + case["pad_b"]), generator=gen) * 2 - 1).to(dtype).to(device)[:, :, :k]
+    out_dtype = torch.float32 if not case["narrow"] else (torch.bfloat16 if kind == "f32" else dtype)
+    c = torch.full((batch, m, n + case["c_pad"]), float("nan"), dtype=out_dtype, device=device)[:, :, :n]
+    c_in = None
+    if case["c_in"] == "same":
+        c_in = (torch.rand((batch, m, n), generator=gen) * 2 - 1).to(out_dtype).to(device)
+    elif case["c_in"] == "bias":
+        c_in = (torch.rand((batch, 1, n), generator=gen) * 2 - 1).to(out_dtype).to(device).expand(batch, m, n)
+    elif case["c_in"] == "f32":
+        c_in = (torch.rand((batch, m, n), generator=gen) * 2 - 1).to(device)
+    if batch == 1:
+        a, b, c = a[0], b[0], c[0]
+        c_in = None if c_in is None else c_in[0]
+    capi.matmul(a, b, c, c_in=c_in)
+    torch.cuda.synchronize()
+    ar, br = (a.bfloat16(), b.bfloat16()) if kind == "f32" else (a, b)
+    want = torch.matmul(ar.double(), br.double().transpose(-1, -2))
+    if c_in is not None:
+        want = want + c_in.double()
+    tol = fp32_tol(k) + (2.0 ** (-11 if out_dtype == torch.float16 else -8) * 1.01 if case["narrow"] else 0.0)
+    assert rel_err(c.double().cpu().numpy(), want.cpu().numpy()) <= tol
+
+
 def test_the_table_plans_the_benchmark_shape_on_it(device):
     """Batch 8 of 3000 x 3000 x 17 plans as tile_128 unsplit - the plan this kernel serves - and K = 33 or a B handed
     over as [K,N] still give right results on the two-stage kernel."""
