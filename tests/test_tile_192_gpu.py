@@ -161,6 +161,31 @@ def test_one_round_of_bigger_tiles_by_a_k_split(device, m, n, k, b_as_kn, family
     assert rel_err(c[rows].double().cpu().numpy(), want.cpu().numpy()) <= fp32_tol(k)
 
 
+@pytest.mark.parametrize("b_as_kn", [False, True])
+def test_fused_transform_on_the_tables_plan(device, b_as_kn):
+    """3000 x 3000 x 520 with row and column scales, a shift, silu and a bias row, to bf16: the table plans 192 x 192 tiles;
+    against the same operations in float64 (the bound: bf16's half unit in the last place on top of the sums')."""
+    import torch
+    from vecops_amd import capi
+    m, n, k = 3000, 3000, 520
+    gen = torch.Generator(device="cpu").manual_seed(9)
+    a = (torch.rand((m, k), generator=gen) * 2 - 1).bfloat16().to(device)
+    b = (torch.rand((k, n) if b_as_kn else (n, k), generator=gen) * 2 - 1).bfloat16().to(device)
+    bv = b.t() if b_as_kn else b
+    rs = (torch.rand(m, generator=gen) + 0.5).to(device)
+    cs = (torch.rand(n, generator=gen) + 0.5).to(device)
+    bias = (torch.rand((1, n), generator=gen) * 2 - 1).to(device).expand(m, n)
+    c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=device)
+    ep = capi.epilogue(activation="silu", scale=0.125, shift=0.5, row_scales=rs, column_scales=cs)
+    plan = capi.plan_matmul_fused(a, bv, c, ep, c_in=bias)
+    assert capi.FAMILY_NAMES[plan.family] == "tile_192" and plan.split_k == 1
+    capi.matmul_fused(a, bv, c, ep, c_in=bias)
+    torch.cuda.synchronize()
+    x = (torch.matmul(a.double(), bv.double().t()) + bias.double()) * rs.double()[:, None] * cs.double()[None, :] * 0.125 + 0.5
+    want = x * torch.sigmoid(x)
+    assert rel_err(c.double().cpu().numpy(), want.cpu().numpy()) <= 2.0 ** -8 * 1.01 + 1e-3    # (the fast exp and reciprocal)
+
+
 def test_required_where_it_cannot_serve(device):
     import torch
     from vecops_amd import capi
