@@ -65,7 +65,7 @@ typedef enum VecopsHipKernelFamily {
   VECOPS_HIP_FAMILY_NONE = 0,          /* empty problem: nothing to launch */
   VECOPS_HIP_FAMILY_TILE_256 = 1,      /* 256x256 workgroup tile, MFMA */
   VECOPS_HIP_FAMILY_TILE_128 = 2,      /* 128x128 workgroup tile, MFMA (16-bit compute with 8 <= K <= 32, K-contiguous
-                                          operands and plain fp32 / bf16 / f16 results: a kernel of 64x128 tiles whose
+                                          operands and plain fp32 / bf16 / f16 results: a kernel of 32x256 tiles whose
                                           life is the write of C) */
   VECOPS_HIP_FAMILY_TILE_64 = 3,       /* 64x64 workgroup tile, MFMA */
   VECOPS_HIP_FAMILY_SKINNY = 4,        /* one side <= 16 rows: wavefronts split K, the wide operand is read once */

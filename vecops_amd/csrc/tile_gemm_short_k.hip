@@ -14,7 +14,7 @@ namespace vecops_hip {
 namespace {
 
 constexpr int kWaveRows = 32, kWaveCols = 64;    // one wavefront's part of C
-constexpr int kTileRows = 64, kTileCols = 128;   // a workgroup: 2 x 2 wavefronts
+constexpr int kTileRows = 32, kTileCols = 256;   // a workgroup: four wavefronts side by side along N (1 KiB of a row of fp32 C)
 constexpr int kStageRows = 16;                   // rows of C a wavefront lays out in LDS at a time
 constexpr int kPitch = kWaveCols + 4;            // 32-bit words per staged row: rows start 16 bytes apart in the bank period
 
@@ -43,7 +43,7 @@ __device__ __forceinline__ ShortKPlace short_k_place(const TileGemmParams& p, in
   const int per_batch = p.tiles_m * p.tiles_n;
   const int batch = tile / per_batch, in_batch = tile - batch * per_batch;
   const int tm = in_batch / p.tiles_n, tn = in_batch - tm * p.tiles_n;
-  return ShortKPlace{batch, tm * kTileRows + (wave >> 1) * kWaveRows, tn * kTileCols + (wave & 1) * kWaveCols};
+  return ShortKPlace{batch, tm * kTileRows, tn * kTileCols + wave * kWaveCols};
 }
 
 // The wavefront's operand fragments of one step of 32 along K, as loaded (rows past the operand read its last row:
@@ -267,7 +267,7 @@ bool launch_tile_gemm_short_k_serves(int src, const TileGemmParams& p) {
   return p.m > 0 && p.n > 0 && p.k >= 8 && p.split_k == 1 && p.a_ks == 1 && p.b_ks == 1 && store_kind(p) != STORE_NONE;
 }
 
-// (sets the tile counts of its own 64 x 128 tile in its copy of the parameters)
+// (sets the tile counts of its own 32 x 256 tile in its copy of the parameters)
 hipError_t launch_tile_gemm_short_k(int src, TileGemmParams p, hipStream_t stream) {
   p.tiles_m = (p.m + kTileRows - 1) / kTileRows;
   p.tiles_n = (p.n + kTileCols - 1) / kTileCols;
