@@ -123,6 +123,12 @@ def test_rule_table_known_answers():
         rc, p = _plan(_operand(capi.BF16, (m, k)), _operand(capi.BF16, (n, k)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
         assert p.workspace_bytes == (split * m * n * 4 if split > 1 else 0)
+    # fp32 operands multiplied as bf16 go through staging registers: the small tile only up to half the units' worth of
+    # 128 x 128 tiles, and from 96 tiles and 32 K tiles on two K parts of the 128 x 128 tile
+    for (m, n, k), family, split in (((1024, 1024, 1024), "tile_64", 1), ((1408, 1408, 1408), "tile_64", 1), ((1536, 1536, 1536), "tile_128", 1),
+                                     ((1024, 2048, 4096), "tile_128", 2), ((1280, 1280, 4096), "tile_128", 2), ((1024, 2048, 1024), "tile_64", 1)):
+        rc, p = _plan(_operand(capi.F32, (m, k)), _operand(capi.F32, (n, k)), _operand(capi.F32, (m, n)))
+        assert rc == 0 and capi.FAMILY_NAMES[p.family] == family and p.split_k == split, (m, n, k, p.family, p.split_k)
     for m, n in ((768, 11008), (1344, 6144), (3072, 3072)):
         rc, p = _plan(_operand(capi.BF16, (m, 4096)), _operand(capi.BF16, (n, 4096)), _operand(capi.BF16, (m, n)))
         assert rc == 0 and capi.FAMILY_NAMES[p.family] == "tile_192", (m, n)

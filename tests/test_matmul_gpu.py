@@ -909,6 +909,25 @@ def test_mid_band_k_split(device, oracle, kind, m, n, k, split):
         assert np.array_equal(alone.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("m,n,k,family,split", [(1024, 2048, 4096, "tile_128", 2), (1536, 1536, 1536, "tile_128", 1), (1408, 1408, 1408, "tile_64", 1)])
+def test_fp32_operands_as_bf16_plans(device, m, n, k, family, split):
+    """fp32 operands multiplied as bf16 (register-staged loads) around half the units' worth of 128 x 128 tiles: the table's
+    plan - two K parts from 96 tiles and a long K - against float64 sums of the operands rounded to bf16."""
+    import torch
+    from vecops_amd import capi
+    gen = torch.Generator(device="cpu").manual_seed(m + k)
+    a = (torch.rand((m, k), generator=gen) * 2 - 1).to(device)
+    b = (torch.rand((k, n), generator=gen) * 2 - 1).to(device)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    plan = capi.plan_matmul(a, b.t(), c)
+    assert capi.FAMILY_NAMES[plan.family] == family and plan.split_k == split
+    capi.matmul(a, b.t(), c)
+    torch.cuda.synchronize()
+    rows = torch.arange(0, m, 37, device=device)
+    want = torch.matmul(a[rows].bfloat16().double(), b.bfloat16().double())
+    assert rel_err(c[rows].double().cpu().numpy(), want.cpu().numpy()) <= fp32_tol(k)
+
+
 @pytest.mark.parametrize("m,n,k,pad", [(768, 3072, 12288, 0), (768, 3072, 12289, 15)])
 def test_mid_band_k_split_with_dequantisation(device, m, n, k, pad):
     """The mid band under the dequantising epilogue - unsplit on the four-stage kernel, and split (the epilogue applied

@@ -273,6 +273,8 @@ struct RuleConstants {
   int64_t band_k_tiles_per_part = 20, band_k_tiles_per_part_full = 40, band_full_from_tiles = 200, band_min_parts = 6;
   // -- the big tile in four parts where 64 of them would fill a quarter of the chip: K tiles a part must keep
   int64_t big_tile_parts = 4, big_tile_k_tiles_per_part = 40;
+  // -- fp32 operands multiplied as bf16: 128x128 tiles in two K parts from this many tiles (up to half the units) and K tiles
+  int64_t staged_halves_from_tiles = 96, staged_halves_min_k_tiles = 32;
   // -- one round of 256x256 or 192x192 tiles by a K split of two to four parts against 128x128 pairs (`bench.py --only
   //    rule_check`: 2304 x 2304 x 8192, 768 x 3072 x 12288, 2048 x 4096 x 11008)
   int64_t one_round_max_parts = 4, one_round_k_tiles_per_part = 40, one_round_ps_per_unit = 21600, one_round_split_ns = 3000;
@@ -582,8 +584,11 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
   // more on every unit (512 x 4096 x 4096: 28.7 us against 45.9; 1536^3: 18.0 against 20.7; 768 x 4096 x 4096:
   // 42.7 against 46.7; from 256 tiles on - 1024 x 4096 x 4096, 2048^3 - the bigger tile is ahead again).
   // (not where the four-stage 128x128 kernel serves: a lone workgroup of it does not wait out its loads)
+  // (fp32 operands multiplied as bf16 - twice the bytes through the staging registers, which the small tile fetches twice
+  // as often: only up to half the units - 1536^3, 144 tiles: 23 us on 128x128 against 29; 1408^3, 121 tiles: 20 on 64x64
+  // against 23)
   else if (k_tiles > kRules.short_k_tiles_16bit && family == VECOPS_HIP_FAMILY_TILE_128 && pr.src != SRC_F32 && !deep_ok &&
-           tiles(128) <= kRules.lonely_tiles_num * kComputeUnits / kRules.lonely_tiles_den) {
+           tiles(128) <= (pr.src == SRC_F32_AS_BF16 ? kComputeUnits / 2 : kRules.lonely_tiles_num * kComputeUnits / kRules.lonely_tiles_den)) {
     family = VECOPS_HIP_FAMILY_TILE_64;
     tile_m = tile_n = 64;
   }
@@ -646,6 +651,17 @@ void choose(const Problem& pr, VecopsHipPlan* plan, uint64_t scratch_limit = UIN
       family = VECOPS_HIP_FAMILY_TILE_128;
       band_split = static_cast<uint32_t>(parts);
     }
+  }
+  // fp32 operands multiplied as bf16 (register-staged: none of the rules above), 96 to 128 tiles of 128x128 and 64 K
+  // tiles or more: two K parts of the 128x128 tile fill the units (1024 x 2048 x 4096 37 us against 47 on 64x64 tiles,
+  // 1280 x 1280 x 4096 37 against 49; at K = 2048 - 768 x 2048 x 2048 - 24.6 against 25.7; at K = 1024 the small tiles
+  // stay ahead, 15.7 against 22.6).
+  if (pr.src == SRC_F32_AS_BF16 && !pr.packed_b && band_split == 0 && tiles(128) >= kRules.staged_halves_from_tiles &&
+      tiles(128) <= kComputeUnits / 2 && k_tiles >= kRules.staged_halves_min_k_tiles &&
+      2ull * pr.batch * pr.m * pr.n * 4u <= scratch_limit) {
+    family = VECOPS_HIP_FAMILY_TILE_128;
+    tile_m = tile_n = 128;
+    band_split = 2;
   }
   // 256 tiles of 128x128 that are 64 of 256x256, and a K of 160 tiles or more: the big tile in four parts puts one
   // workgroup of its (faster) loop on every unit (bf16 1024 x 4096 x 11008: 84 us against 89-92 for the two parts of
